@@ -1,0 +1,83 @@
+/* C ABI of libgdn_mi355x.so -- MI355X (gfx950) kernels for the Gated DeltaNet operator path.
+ *
+ * The reference binds this path as Python callables chosen by a config string
+ * (mindspeed_mm/fsdp/models/qwen3_5/modeling_qwen3_5.py:569-633); it has no FFI of its own.  The
+ * entry points below are what a binding for that plugin slot calls: one launcher per operator,
+ * raw device pointers and sizes only.
+ *
+ * Common rules
+ *   - every pointer is device memory, tensors are dense (contiguous) in the stated layout;
+ *   - dtype: 0 = fp32, 1 = bf16 (conv1d also 2 = fp16) and applies to q/k/v/o and their gradients;
+ *     g, beta, states and their gradients are always fp32;
+ *   - `stream` is a hipStream_t; launches are asynchronous, nothing allocates or synchronises;
+ *   - return 0 on success, <0 for an invalid argument (-1 null pointer, -2 bad shape, -3 unsupported
+ *     size, -4 bad dtype, -5 workspace too small), >0 is a hipError_t from the launch;
+ *   - layouts: q,k [B,T,Hqk,K]; v,o [B,T,Hv,V]; g,beta [B,T,Hv]; states [N,Hv,K,V]; Hv % Hqk == 0
+ *     (grouped heads are read in place, no expansion); with cu_seqlens (int64 [N+1], device) B == 1.
+ */
+#ifndef GDN_MI355X_H
+#define GDN_MI355X_H
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* -------- chunked gated delta rule, forward + backward --------------------------------------
+ * replaces chunk_gated_delta_rule_fwd / _bwd, mindspeed_mm/fsdp/ops/gdn/chunk_gated_delta_rule.py:30-174
+ * (semantics of torch_chunk_gated_delta_rule, modeling_qwen3_5.py:398-475). K in {64,128}, V % 64 == 0.
+ *
+ * The workspace keeps what the backward pass needs (cumulative decay, WY factors, per-chunk states);
+ * gdn_chunk_bwd must be given the workspace its forward call filled, unchanged, and that workspace
+ * must have been sized with with_backward = 1.  The workspace must be 256-byte aligned.
+ */
+int64_t gdn_chunk_workspace_bytes(int B, int T, int N, int Hqk, int Hv, int K, int V, int dtype, int with_backward);
+
+int gdn_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const float* beta,
+                  const float* initial_state, const int64_t* cu_seqlens, void* o, float* final_state,
+                  void* workspace, int64_t workspace_bytes, int B, int T, int N, int Hqk, int Hv, int K, int V,
+                  float scale, int use_qk_l2norm, int dtype, void* stream);
+
+int gdn_chunk_bwd(const void* q, const void* k, const void* v, const float* g, const float* beta,
+                  const float* initial_state, const int64_t* cu_seqlens, const void* d_o,
+                  const float* d_final_state, void* dq, void* dk, void* dv, float* dg, float* dbeta,
+                  float* d_initial_state, void* workspace, int64_t workspace_bytes, int B, int T, int N, int Hqk,
+                  int Hv, int K, int V, float scale, int use_qk_l2norm, int dtype, void* stream);
+
+/* -------- fused recurrent gated delta rule (decode) ------------------------------------------
+ * replaces the `recurrent_gated_delta_rule` slot (third-party fla kernel or
+ * torch_recurrent_gated_delta_rule, modeling_qwen3_5.py:478-517, bound at :633, called at :877-886).
+ * state_in may be NULL (zeros); state_out may be NULL or equal to state_in (updated in place).
+ * K in {64,128,256}, V % 64 == 0.
+ */
+int gdn_recurrent_fwd(const void* q, const void* k, const void* v, const float* g, const float* beta,
+                      const float* state_in, float* state_out, void* o, int B, int T, int Hqk, int Hv, int K,
+                      int V, float scale, int use_qk_l2norm, int dtype, void* stream);
+
+/* -------- causal short depthwise conv1d --------------------------------------------------------
+ * replaces causal_conv1d_fwd_impl / causal_conv1d_bwd_impl / causal_conv1d_update_states,
+ * mindspeed_mm/fsdp/ops/gdn/triton/convolution.py:517-588, 591-714, 762-787.
+ * x,y,residual,dy,dx [B,T,D]; weight [W,D]; bias [D]; states [N,D,W]; activation 0 = none, 1 = SiLU.
+ * W in 1..8; D % 8 == 0 (D % 4 for fp32).  dw [W,D] and db [D] are fp32.
+ */
+int gdn_conv1d_fwd(const void* x, const void* weight, const void* bias, const void* residual,
+                   const void* initial_state, const int64_t* cu_seqlens, void* y, void* final_state, int B, int T,
+                   int N, int D, int W, int activation, int dtype, void* stream);
+
+int64_t gdn_conv1d_bwd_workspace_bytes(int B, int T, int D, int W);
+
+int gdn_conv1d_bwd(const void* x, const void* dy, const void* weight, const void* bias, const void* initial_state,
+                   const void* d_final_state, const int64_t* cu_seqlens, void* dx, float* dw, float* db,
+                   void* d_initial_state, void* workspace, int64_t workspace_bytes, int B, int T, int N, int D,
+                   int W, int activation, int dtype, void* stream);
+
+/* decode-time update, replaces the `causal_conv1d_update` slot (torch_causal_conv1d_update,
+ * modeling_qwen3_5.py:373-389, called at :738-744): hidden,out [B,T,D]; conv_state [B,D,state_len]
+ * rolled in place; weight [D,W]; state_len >= W-1. */
+int gdn_conv1d_update(const void* hidden, void* conv_state, const void* weight, const void* bias, void* out, int B,
+                      int T, int D, int W, int state_len, int activation, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,289 @@
+// Device-side building blocks shared by the gated-delta-rule kernels (gfx950 / CDNA4).
+//
+// Conventions
+//   * wavefront = 64 lanes; workgroups are 256 threads (4 waves) unless stated otherwise.
+//   * chunk = 64 tokens.  A "tile" in LDS is [rows][ld] with ld = cols + 16 bytes of padding so that
+//     16-byte fragment reads of consecutive rows fall into different banks.
+//   * every tensor-core contraction goes through mma32<>: one wave accumulates one 32x32 fp32 tile
+//     C[i][j] += sum_k A[i][k] * B[k][j] with operands read from LDS.
+//       bf16: v_mfma_f32_32x32x16_bf16   lane l holds A[l%32][8*(l/32)+0..7] and B[8*(l/32)+0..7][l%32]
+//       fp32: v_mfma_f32_32x32x2_f32     lane l holds A[l%32][l/32]          and B[l/32][l%32]
+//     accumulator register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32].
+//     The k index inside one instruction may be permuted freely as long as A and B agree; the fp32
+//     path uses that to read 4 consecutive k per lane with one 16-byte load.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+// dynamic LDS, one array per workgroup
+extern __shared__ __align__(16) unsigned char gdn_smem[];
+
+namespace gdn {
+
+constexpr int kChunk = 64;
+constexpr int kThreads = 256;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+struct bf16_t { uint16_t bits; };
+struct f16_t { uint16_t bits; };
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {  // round to nearest even; NaN stays NaN
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+  static constexpr int kVec = 4;  // elements per 16 bytes
+  static __device__ __forceinline__ float to_f(float x) { return x; }
+  static __device__ __forceinline__ float from_f(float x) { return x; }
+};
+template <> struct Elem<bf16_t> {
+  static constexpr int kVec = 8;
+  static __device__ __forceinline__ float to_f(bf16_t x) { return bf16_to_f32(x.bits); }
+  static __device__ __forceinline__ bf16_t from_f(float x) { bf16_t r; r.bits = f32_to_bf16(x); return r; }
+};
+template <> struct Elem<f16_t> {
+  static constexpr int kVec = 8;
+  static __device__ __forceinline__ float to_f(f16_t x) { _Float16 h = __builtin_bit_cast(_Float16, x.bits); return (float)h; }
+  static __device__ __forceinline__ f16_t from_f(float x) { _Float16 h = (_Float16)x; f16_t r; r.bits = __builtin_bit_cast(uint16_t, h); return r; }
+};
+
+// padded leading dimension (in elements) of an LDS tile with `cols` columns
+template <typename T> __device__ __host__ constexpr int lds_ld(int cols) { return cols + 16 / (int)sizeof(T); }
+
+__device__ __forceinline__ int imin(int a, int b) { return a < b ? a : b; }
+__device__ __forceinline__ int imax(int a, int b) { return a > b ? a : b; }
+
+// ---------------------------------------------------------------------------------------------
+// 16-byte vectors of T <-> floats
+// ---------------------------------------------------------------------------------------------
+template <typename T> struct Vec16 {
+  u32x4 raw;
+  __device__ __forceinline__ float get(int e) const {
+    if constexpr (sizeof(T) == 4) {
+      return __uint_as_float(raw[e]);
+    } else {
+      uint32_t w = raw[e >> 1];
+      T t; t.bits = (uint16_t)((e & 1) ? (w >> 16) : (w & 0xffffu));
+      return Elem<T>::to_f(t);
+    }
+  }
+  __device__ __forceinline__ void set(int e, float f) {
+    if constexpr (sizeof(T) == 4) {
+      raw[e] = __float_as_uint(f);
+    } else {
+      uint32_t h = Elem<T>::from_f(f).bits;
+      uint32_t w = raw[e >> 1];
+      raw[e >> 1] = (e & 1) ? ((w & 0xffffu) | (h << 16)) : ((w & 0xffff0000u) | h);
+    }
+  }
+};
+
+template <typename T> __device__ __forceinline__ Vec16<T> ld16(const T* p) {
+  Vec16<T> v; v.raw = *reinterpret_cast<const u32x4*>(p); return v;
+}
+template <typename T> __device__ __forceinline__ void st16(T* p, const Vec16<T>& v) {
+  *reinterpret_cast<u32x4*>(p) = v.raw;
+}
+template <typename T> __device__ __forceinline__ Vec16<T> zero16() {
+  Vec16<T> v; v.raw = u32x4{0u, 0u, 0u, 0u}; return v;
+}
+
+// ---------------------------------------------------------------------------------------------
+// global -> LDS tile loads.  The tile has 64 rows (tokens) and COLS columns; rows >= nvalid are
+// zero filled (zero padding of a ragged last chunk is exact for the gated delta rule).
+// ---------------------------------------------------------------------------------------------
+template <typename T, int COLS, int ROWS = kChunk>
+__device__ __forceinline__ void load_tile(T* lds, int ld, const T* g, int64_t row_stride, int nvalid, int tid) {
+  constexpr int V = Elem<T>::kVec, CPR = COLS / V;
+  for (int c = tid; c < ROWS * CPR; c += kThreads) {
+    const int row = c / CPR, cc = c % CPR;
+    Vec16<T> v = row < nvalid ? ld16(g + (int64_t)row * row_stride + cc * V) : zero16<T>();
+    st16(lds + row * ld + cc * V, v);
+  }
+}
+
+// same, each row multiplied by rowscale[row] (fp32, in LDS)
+template <typename T, int COLS>
+__device__ __forceinline__ void load_tile_scaled(T* lds, int ld, const T* g, int64_t row_stride, int nvalid,
+                                                 const float* rowscale, int tid) {
+  constexpr int V = Elem<T>::kVec, CPR = COLS / V;
+  for (int c = tid; c < kChunk * CPR; c += kThreads) {
+    const int row = c / CPR, cc = c % CPR;
+    Vec16<T> v = zero16<T>();
+    if (row < nvalid) {
+      v = ld16(g + (int64_t)row * row_stride + cc * V);
+      const float s = rowscale[row];
+#pragma unroll
+      for (int e = 0; e < V; ++e) v.set(e, v.get(e) * s);
+    }
+    st16(lds + row * ld + cc * V, v);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// MFMA wrappers
+// ---------------------------------------------------------------------------------------------
+// One operand fragment: the 16 bytes a lane feeds to the matrix core for one k-group
+// (bf16: 8 k values -> one 32x32x16 instruction; fp32: 4 k values -> four 32x32x2 instructions).
+template <typename T> struct KGroup { static constexpr int kLen = (sizeof(T) == 2) ? 16 : 8; };
+
+// contiguous: p points at element [row][k0]; the lane reads kVec consecutive k
+template <typename T> __device__ __forceinline__ u32x4 frag_contig(const T* p) {
+  return *reinterpret_cast<const u32x4*>(p);
+}
+// strided: p points at element [k0][col] of a [k][ld] array; the lane gathers kVec values ld apart
+template <typename T> __device__ __forceinline__ u32x4 frag_strided(const T* p, int ld) {
+  u32x4 r;
+  if constexpr (sizeof(T) == 4) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) r[e] = __float_as_uint(p[e * ld]);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      uint32_t lo = p[(2 * e) * ld].bits, hi = p[(2 * e + 1) * ld].bits;
+      r[e] = lo | (hi << 16);
+    }
+  }
+  return r;
+}
+
+template <typename T> __device__ __forceinline__ void mfma_kgroup(f32x16& acc, u32x4 a, u32x4 b) {
+  if constexpr (sizeof(T) == 2) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc,
+                                                  0, 0, 0);
+  } else {
+#pragma unroll
+    for (int m = 0; m < 4; ++m)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[m]), __uint_as_float(b[m]), acc, 0, 0, 0);
+  }
+}
+
+// acc(32x32) += A(32 x KLEN) * B(KLEN x 32), operands in LDS.
+//   A_KC = true : A[i][k] at A[i*lda + k]   (pass A = &tile[i0][k0])
+//   A_KC = false: A[i][k] at A[k*lda + i]   (pass A = &tile[k0][i0])
+//   B_KC = true : B[k][j] at B[j*ldb + k]   (pass B = &tile[j0][k0])
+//   B_KC = false: B[k][j] at B[k*ldb + j]   (pass B = &tile[k0][j0])
+template <typename T, int KLEN, bool A_KC, bool B_KC>
+__device__ __forceinline__ void mma32(f32x16& acc, const T* A, int lda, const T* B, int ldb) {
+  constexpr int G = KGroup<T>::kLen, V = Elem<T>::kVec;
+  static_assert(KLEN % G == 0, "contraction length must be a multiple of the k-group");
+  const int lane = threadIdx.x & 63, r32 = lane & 31, half = lane >> 5;
+#pragma unroll
+  for (int kg = 0; kg < KLEN / G; ++kg) {
+    const int k = kg * G + half * V;
+    u32x4 a, b;
+    if constexpr (A_KC) a = frag_contig(A + r32 * lda + k); else a = frag_strided(A + k * lda + r32, lda);
+    if constexpr (B_KC) b = frag_contig(B + r32 * ldb + k); else b = frag_strided(B + k * ldb + r32, ldb);
+    mfma_kgroup<T>(acc, a, b);
+  }
+}
+
+__device__ __forceinline__ f32x16 acc_zero() {
+  f32x16 z;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) z[r] = 0.f;
+  return z;
+}
+// coordinates of accumulator register r of this lane inside the 32x32 tile
+__device__ __forceinline__ int acc_row(int r) { return 8 * (r >> 2) + 4 * ((threadIdx.x & 63) >> 5) + (r & 3); }
+__device__ __forceinline__ int acc_col() { return threadIdx.x & 31; }
+
+// accumulator tile -> LDS, row-major: dst[(i0+i)*ld + j0 + j]
+template <typename T> __device__ __forceinline__ void acc_to_lds(const f32x16& acc, T* dst, int ld, int i0, int j0) {
+  const int j = j0 + acc_col();
+#pragma unroll
+  for (int r = 0; r < 16; ++r) dst[(i0 + acc_row(r)) * ld + j] = Elem<T>::from_f(acc[r]);
+}
+// accumulator tile -> LDS, transposed: dst[(j0+j)*ld + i0 + i]
+template <typename T> __device__ __forceinline__ void acc_to_lds_t(const f32x16& acc, T* dst, int ld, int i0, int j0) {
+  const int j = j0 + acc_col();
+#pragma unroll
+  for (int r = 0; r < 16; ++r) dst[j * ld + i0 + acc_row(r)] = Elem<T>::from_f(acc[r]);
+}
+// accumulator tile -> global rows (row-major, only rows < nvalid)
+template <typename T>
+__device__ __forceinline__ void acc_to_global(const f32x16& acc, T* g, int64_t row_stride, int i0, int j0, int nvalid) {
+  const int j = j0 + acc_col();
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int i = i0 + acc_row(r);
+    if (i < nvalid) g[(int64_t)i * row_stride + j] = Elem<T>::from_f(acc[r]);
+  }
+}
+// global rows -> accumulator tile (rows >= nvalid read as zero)
+template <typename T>
+__device__ __forceinline__ f32x16 acc_from_global(const T* g, int64_t row_stride, int i0, int j0, int nvalid) {
+  f32x16 a;
+  const int j = j0 + acc_col();
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int i = i0 + acc_row(r);
+    a[r] = i < nvalid ? Elem<T>::to_f(g[(int64_t)i * row_stride + j]) : 0.f;
+  }
+  return a;
+}
+
+// sum over the 32 lanes that share a half-wave (all columns of one accumulator row)
+__device__ __forceinline__ float half_wave_sum(float v) {
+  v += __shfl_xor(v, 16);
+  v += __shfl_xor(v, 8);
+  v += __shfl_xor(v, 4);
+  v += __shfl_xor(v, 2);
+  v += __shfl_xor(v, 1);
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+  v += __shfl_xor(v, 32);
+  return half_wave_sum(v);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Packed-sequence bookkeeping.  chunk_offsets[n] = number of 64-token chunks before sequence n
+// (chunk_offsets[N] = total); built on the device by gdn_chunk_table_kernel so that no host sync is
+// needed.  Without cu_seqlens every batch row is a sequence of T tokens.
+// ---------------------------------------------------------------------------------------------
+struct SeqInfo {
+  int n;        // sequence index
+  int64_t bos;  // first token (index into the flattened [B*T] token axis)
+  int len;      // tokens in this sequence
+  int chunk;    // chunk index inside the sequence
+  int nvalid;   // valid tokens of this chunk (1..64), 0 if the chunk does not exist
+};
+
+__device__ __forceinline__ SeqInfo locate_chunk(int gchunk, const int64_t* cu_seqlens, const int* chunk_offsets,
+                                                int N, int T) {
+  SeqInfo s;
+  if (cu_seqlens == nullptr) {
+    const int nt = (T + kChunk - 1) / kChunk;
+    s.n = gchunk / nt;
+    s.chunk = gchunk % nt;
+    s.bos = (int64_t)s.n * T;
+    s.len = T;
+    s.nvalid = s.n < N ? imin(kChunk, T - s.chunk * kChunk) : 0;
+    return s;
+  }
+  if (gchunk >= chunk_offsets[N]) { s.n = 0; s.bos = 0; s.len = 0; s.chunk = 0; s.nvalid = 0; return s; }
+  int lo = 0, hi = N - 1;  // last n with chunk_offsets[n] <= gchunk
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (chunk_offsets[mid] <= gchunk) lo = mid; else hi = mid - 1;
+  }
+  s.n = lo;
+  s.bos = cu_seqlens[lo];
+  s.len = (int)(cu_seqlens[lo + 1] - s.bos);
+  s.chunk = gchunk - chunk_offsets[lo];
+  s.nvalid = imin(kChunk, s.len - s.chunk * kChunk);
+  return s;
+}
+
+}  // namespace gdn

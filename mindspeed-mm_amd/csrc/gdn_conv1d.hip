@@ -1,0 +1,430 @@
+// Causal short depthwise conv1d (+SiLU) over token-major activations x[B,T,D], weight[W,D]:
+//     y[t,d] = act( sum_{w<W} xpad[t-(W-1)+w, d] * weight[w,d] + bias[d] ) (+ residual[t,d])
+// where xpad reads the sequence's initial_state[n,d,W+tau] for tau = position - sequence start < 0
+// (zero when there is none) and never crosses a cu_seqlens boundary.
+// Reference semantics: mindspeed_mm/fsdp/ops/gdn/triton/convolution.py:41-181 (fwd), :193-514 (bwd),
+// :723-759 (final state); tests/ut_fsdp/models/qwen3_5/test_causal_conv1d/reference_impl.py:18-102;
+// decode update mindspeed_mm/fsdp/models/qwen3_5/modeling_qwen3_5.py:373-389.
+//
+// All kernels are HBM bound (2*W flop per element).  A thread owns 16 bytes of channels (8 bf16 /
+// 4 fp32) and walks a tile of consecutive tokens with the last W inputs in registers, so x is read
+// once; the backward pass recomputes the pre-activation in registers instead of re-reading y.
+#include "gdn_common.h"
+
+namespace gdn {
+
+constexpr int kConvThreads = 128;
+
+struct SeqCursor {  // which sequence a flattened token index belongs to
+  const int64_t* cu; int N; int T; int n; int64_t bos, eos;
+  __device__ __forceinline__ void init(const int64_t* cu_, int N_, int T_, int64_t t) {
+    cu = cu_; N = N_; T = T_;
+    if (cu == nullptr) { n = (int)(t / T); bos = (int64_t)n * T; eos = bos + T; return; }
+    int lo = 0, hi = N - 1;
+    while (lo < hi) { const int mid = (lo + hi + 1) >> 1; if (cu[mid] <= t) lo = mid; else hi = mid - 1; }
+    n = lo; bos = cu[n]; eos = cu[n + 1];
+    while (t >= eos && n + 1 < N) { ++n; bos = eos; eos = cu[n + 1]; }  // skip empty sequences
+  }
+  __device__ __forceinline__ bool advance_to(int64_t t) {  // returns true if a new sequence was entered
+    bool moved = false;
+    while (t >= eos && n + 1 < N) {
+      ++n; bos = eos; eos = (cu == nullptr) ? bos + T : cu[n + 1]; moved = true;
+    }
+    return moved;
+  }
+};
+
+template <typename T, int V> struct ChanVec { float x[V]; };
+
+template <typename T> __device__ __forceinline__ void load_chan(float* dst, const T* p) {
+  const Vec16<T> v = ld16(p);
+#pragma unroll
+  for (int e = 0; e < Elem<T>::kVec; ++e) dst[e] = v.get(e);
+}
+template <typename T> __device__ __forceinline__ void store_chan(T* p, const float* src) {
+  Vec16<T> v = zero16<T>();
+#pragma unroll
+  for (int e = 0; e < Elem<T>::kVec; ++e) v.set(e, src[e]);
+  st16(p, v);
+}
+
+// input at flattened position tau for the sequence described by cur (tau may precede the sequence)
+template <typename T>
+__device__ __forceinline__ void load_hist(float* dst, const T* x, const T* init, int64_t tau, const SeqCursor& cur,
+                                          int D, int W, int d0) {
+  constexpr int V = Elem<T>::kVec;
+  if (tau >= cur.bos) { load_chan(dst, x + tau * D + d0); return; }
+  const int j = W + (int)(tau - cur.bos);
+  if (init != nullptr && j >= 1) {
+#pragma unroll
+    for (int e = 0; e < V; ++e) dst[e] = Elem<T>::to_f(init[((int64_t)cur.n * D + d0 + e) * W + j]);
+  } else {
+#pragma unroll
+    for (int e = 0; e < V; ++e) dst[e] = 0.f;
+  }
+}
+
+__device__ __forceinline__ float sigmoidf_(float p) { return 1.f / (1.f + __expf(-p)); }
+
+template <typename T, int W>
+__global__ __launch_bounds__(kConvThreads) void conv1d_fwd_kernel(
+    const T* __restrict__ x, const T* __restrict__ weight, const T* __restrict__ bias, const T* __restrict__ residual,
+    const T* __restrict__ init, const int64_t* __restrict__ cu, T* __restrict__ y, int64_t total, int T_len, int N,
+    int D, int tile, int silu) {
+  constexpr int V = Elem<T>::kVec;
+  const int d0 = (blockIdx.x * kConvThreads + threadIdx.x) * V;
+  if (d0 >= D) return;
+  const int64_t t0 = (int64_t)blockIdx.y * tile;
+  const int64_t t1 = t0 + tile < total ? t0 + tile : total;
+  float wgt[W][V], bs[V], win[W][V];
+#pragma unroll
+  for (int w = 0; w < W; ++w) load_chan(wgt[w], weight + (int64_t)w * D + d0);
+#pragma unroll
+  for (int e = 0; e < V; ++e) bs[e] = 0.f;
+  if (bias != nullptr) load_chan(bs, bias + d0);
+  SeqCursor cur;
+  cur.init(cu, N, T_len, t0);
+#pragma unroll
+  for (int w = 0; w < W - 1; ++w) load_hist(win[w], x, init, t0 - (W - 1) + w, cur, D, W, d0);
+  for (int64_t t = t0; t < t1; ++t) {
+    if (cur.advance_to(t)) {
+#pragma unroll
+      for (int w = 0; w < W - 1; ++w) load_hist(win[w], x, init, t - (W - 1) + w, cur, D, W, d0);
+    }
+    load_chan(win[W - 1], x + t * D + d0);
+    float out[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      float a = bs[e];
+#pragma unroll
+      for (int w = 0; w < W; ++w) a += win[w][e] * wgt[w][e];
+      out[e] = silu ? a * sigmoidf_(a) : a;
+    }
+    if (residual != nullptr) {
+      float r[V];
+      load_chan(r, residual + t * D + d0);
+#pragma unroll
+      for (int e = 0; e < V; ++e) out[e] += r[e];
+    }
+    store_chan(y + t * D + d0, out);
+#pragma unroll
+    for (int w = 0; w < W - 1; ++w)
+#pragma unroll
+      for (int e = 0; e < V; ++e) win[w][e] = win[w + 1][e];
+  }
+}
+
+// final_state[n,d,w] = x[T_n - W + w] (falls back to the initial state / zero for T_n < W)
+template <typename T>
+__global__ void conv1d_final_state_kernel(const T* __restrict__ x, const T* __restrict__ init,
+                                          const int64_t* __restrict__ cu, T* __restrict__ fs, int T_len, int N, int D,
+                                          int W) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (int64_t)N * D) return;
+  const int n = (int)(idx / D), d = (int)(idx % D);
+  const int64_t bos = cu ? cu[n] : (int64_t)n * T_len;
+  const int len = cu ? (int)(cu[n + 1] - bos) : T_len;
+  for (int w = 0; w < W; ++w) {
+    const int src = len - W + w;
+    T val = Elem<T>::from_f(0.f);
+    if (src >= 0) val = x[(bos + src) * D + d];
+    else if (init != nullptr) val = init[((int64_t)n * D + d) * W + (src + W)];
+    fs[((int64_t)n * D + d) * W + w] = val;
+  }
+}
+
+// Backward.  With p the pre-activation and dyp = dy * act'(p):
+//   dx[s]   = sum_u dyp[s+u] * weight[W-1-u]   (s+u inside the sequence of s)  (+ dht at the last W tokens)
+//   dw[w]   = sum_t dyp[t] * xpad[t-(W-1)+w],   db = sum_t dyp[t]
+// Each thread writes its tile's partial dw/db to part[tile][W+1][D]; conv1d_reduce_kernel sums them.
+template <typename T, int W>
+__global__ __launch_bounds__(kConvThreads) void conv1d_bwd_kernel(
+    const T* __restrict__ x, const T* __restrict__ dy, const T* __restrict__ weight, const T* __restrict__ bias,
+    const T* __restrict__ init, const T* __restrict__ dht, const int64_t* __restrict__ cu, T* __restrict__ dx,
+    float* __restrict__ part, int64_t total, int T_len, int N, int D, int tile, int silu) {
+  constexpr int V = Elem<T>::kVec;
+  const int d0 = (blockIdx.x * kConvThreads + threadIdx.x) * V;
+  if (d0 >= D) return;
+  const int64_t t0 = (int64_t)blockIdx.y * tile;
+  const int64_t t1 = t0 + tile < total ? t0 + tile : total;
+  const int64_t tend = t1 + (W - 1) < total ? t1 + (W - 1) : total;  // halo: dyp of later tokens feeds dx
+  float wgt[W][V], bs[V], win[W][V], dyw[W][V], dwa[W][V], dba[V];
+#pragma unroll
+  for (int w = 0; w < W; ++w) {
+    load_chan(wgt[w], weight + (int64_t)w * D + d0);
+#pragma unroll
+    for (int e = 0; e < V; ++e) { dwa[w][e] = 0.f; dyw[w][e] = 0.f; }
+  }
+#pragma unroll
+  for (int e = 0; e < V; ++e) { bs[e] = 0.f; dba[e] = 0.f; }
+  if (bias != nullptr) load_chan(bs, bias + d0);
+  SeqCursor cur, lag;   // cur follows t (leading), lag follows s = t-(W-1) (the dx being emitted)
+  cur.init(cu, N, T_len, t0);
+  lag.init(cu, N, T_len, t0);
+#pragma unroll
+  for (int w = 0; w < W - 1; ++w) load_hist(win[w], x, init, t0 - (W - 1) + w, cur, D, W, d0);
+  // t runs W-1 steps past the last dyp so that the final dx of the tile are flushed
+  for (int64_t t = t0; t < t1 + (W - 1); ++t) {
+    // dyw[u] will hold dyp[s+u] for s = t-(W-1); shift in dyp[t]
+#pragma unroll
+    for (int w = 0; w < W - 1; ++w)
+#pragma unroll
+      for (int e = 0; e < V; ++e) dyw[w][e] = dyw[w + 1][e];
+    if (t < tend) {
+      if (cur.advance_to(t)) {
+#pragma unroll
+        for (int w = 0; w < W - 1; ++w) load_hist(win[w], x, init, t - (W - 1) + w, cur, D, W, d0);
+      }
+      load_chan(win[W - 1], x + t * D + d0);
+      float g[V];
+      load_chan(g, dy + t * D + d0);
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        if (silu) {
+          float p = bs[e];
+#pragma unroll
+          for (int w = 0; w < W; ++w) p += win[w][e] * wgt[w][e];
+          const float sg = sigmoidf_(p);
+          g[e] *= sg * (1.f + p * (1.f - sg));
+        }
+        dyw[W - 1][e] = g[e];
+      }
+      if (t < t1) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          dba[e] += g[e];
+#pragma unroll
+          for (int w = 0; w < W; ++w) dwa[w][e] += g[e] * win[w][e];
+        }
+      }
+#pragma unroll
+      for (int w = 0; w < W - 1; ++w)
+#pragma unroll
+        for (int e = 0; e < V; ++e) win[w][e] = win[w + 1][e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e) dyw[W - 1][e] = 0.f;
+    }
+    const int64_t s = t - (W - 1);
+    if (s >= t0 && s < t1) {
+      lag.advance_to(s);
+      float out[V];
+#pragma unroll
+      for (int e = 0; e < V; ++e) out[e] = 0.f;
+#pragma unroll
+      for (int u = 0; u < W; ++u) {
+        if (s + u < lag.eos) {
+#pragma unroll
+          for (int e = 0; e < V; ++e) out[e] += dyw[u][e] * wgt[W - 1 - u][e];
+        }
+      }
+      if (dht != nullptr) {
+        const int64_t wq = s - (lag.eos - W);   // final_state[n,d,wq] = x[s]
+        if (wq >= 0) {
+#pragma unroll
+          for (int e = 0; e < V; ++e) out[e] += Elem<T>::to_f(dht[((int64_t)lag.n * D + d0 + e) * W + wq]);
+        }
+      }
+      store_chan(dx + s * D + d0, out);
+    }
+  }
+  float* pp = part + (int64_t)blockIdx.y * (W + 1) * D;
+#pragma unroll
+  for (int w = 0; w < W; ++w)
+#pragma unroll
+    for (int e = 0; e < V; ++e) pp[(int64_t)w * D + d0 + e] = dwa[w][e];
+#pragma unroll
+  for (int e = 0; e < V; ++e) pp[(int64_t)W * D + d0 + e] = dba[e];
+}
+
+__global__ void conv1d_reduce_kernel(const float* __restrict__ part, float* __restrict__ dw, float* __restrict__ db,
+                                     int ntiles, int W, int D) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (int64_t)(W + 1) * D) return;
+  float s = 0.f;
+  for (int i = 0; i < ntiles; ++i) s += part[(int64_t)i * (W + 1) * D + idx];
+  if (idx < (int64_t)W * D) dw[idx] = s;
+  else if (db != nullptr) db[idx - (int64_t)W * D] = s;
+}
+
+// dh0[n,d,j] = sum_{i<=j-1, i<len} dyp[bos+i] * weight[j-1-i]  (j>=1)   (+ dht[n,d,j-len] when len < W)
+template <typename T>
+__global__ void conv1d_dh0_kernel(const T* __restrict__ x, const T* __restrict__ dy, const T* __restrict__ weight,
+                                  const T* __restrict__ bias, const T* __restrict__ init, const T* __restrict__ dht,
+                                  const int64_t* __restrict__ cu, T* __restrict__ dh0, int T_len, int N, int D, int W,
+                                  int silu) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (int64_t)N * D) return;
+  const int n = (int)(idx / D), d = (int)(idx % D);
+  const int64_t bos = cu ? cu[n] : (int64_t)n * T_len;
+  const int len = cu ? (int)(cu[n + 1] - bos) : T_len;
+  float acc[8];
+  for (int j = 0; j < W; ++j) acc[j] = 0.f;
+  for (int i = 0; i < W - 1 && i < len; ++i) {
+    float g = Elem<T>::to_f(dy[(bos + i) * D + d]);
+    if (silu) {
+      float p = bias ? Elem<T>::to_f(bias[d]) : 0.f;
+      for (int w = 0; w < W; ++w) {
+        const int tau = i - (W - 1) + w;
+        float xv = 0.f;
+        if (tau >= 0) xv = Elem<T>::to_f(x[(bos + tau) * D + d]);
+        else if (init != nullptr && W + tau >= 1) xv = Elem<T>::to_f(init[((int64_t)n * D + d) * W + W + tau]);
+        p += xv * Elem<T>::to_f(weight[(int64_t)w * D + d]);
+      }
+      const float sg = sigmoidf_(p);
+      g *= sg * (1.f + p * (1.f - sg));
+    }
+    for (int j = i + 1; j < W; ++j) acc[j] += g * Elem<T>::to_f(weight[(int64_t)(j - 1 - i) * D + d]);
+  }
+  if (dht != nullptr)
+    for (int w = 0; len + w < W; ++w) acc[len + w] += Elem<T>::to_f(dht[((int64_t)n * D + d) * W + w]);
+  for (int j = 0; j < W; ++j) dh0[((int64_t)n * D + d) * W + j] = Elem<T>::from_f(acc[j]);
+}
+
+// Decode update: hidden[B,T,D], conv_state[B,D,S] rolled in place, weight[D,W].
+template <typename T>
+__global__ void conv1d_update_kernel(const T* __restrict__ hidden, T* __restrict__ state, const T* __restrict__ weight,
+                                     const T* __restrict__ bias, T* __restrict__ out, int B, int T_len, int D, int W,
+                                     int S, int silu) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (int64_t)B * D) return;
+  const int b = (int)(idx / D), d = (int)(idx % D);
+  float st[17], wg[8];   // st[0..S-1] = state, st[S] = the incoming token; needs S >= W-1
+  for (int j = 0; j < S; ++j) st[j] = Elem<T>::to_f(state[((int64_t)b * D + d) * S + j]);
+  for (int w = 0; w < W; ++w) wg[w] = Elem<T>::to_f(weight[(int64_t)d * W + w]);
+  const float bs = bias ? Elem<T>::to_f(bias[d]) : 0.f;
+  for (int t = 0; t < T_len; ++t) {
+    st[S] = Elem<T>::to_f(hidden[((int64_t)b * T_len + t) * D + d]);
+    float a = bs;
+    for (int w = 0; w < W; ++w) a += st[S + 1 - W + w] * wg[w];
+    out[((int64_t)b * T_len + t) * D + d] = Elem<T>::from_f(silu ? a * sigmoidf_(a) : a);
+    for (int j = 0; j < S; ++j) st[j] = st[j + 1];   // roll: the state always ends with the newest input
+  }
+  for (int j = 0; j < S; ++j) state[((int64_t)b * D + d) * S + j] = Elem<T>::from_f(st[j]);
+}
+
+template <typename T> struct ConvLaunch {
+  static int fwd(const void* x, const void* weight, const void* bias, const void* residual, const void* init,
+                 const int64_t* cu, void* y, void* fs, int B, int T_len, int N, int D, int W, int silu,
+                 hipStream_t st) {
+    constexpr int V = Elem<T>::kVec;
+    const int64_t total = (int64_t)B * T_len;
+    const int tile = 64;
+    dim3 grid((D / V + kConvThreads - 1) / kConvThreads, (unsigned)((total + tile - 1) / tile));
+    if (total > 0) {
+      switch (W) {
+#define GDN_CASE(W_)                                                                                              \
+  case W_:                                                                                                        \
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(conv1d_fwd_kernel<T, W_>), grid, dim3(kConvThreads), 0, st, (const T*)x,   \
+                       (const T*)weight, (const T*)bias, (const T*)residual, (const T*)init, cu, (T*)y, total,    \
+                       T_len, N, D, tile, silu);                                                                  \
+    break;
+        GDN_CASE(1) GDN_CASE(2) GDN_CASE(3) GDN_CASE(4) GDN_CASE(5) GDN_CASE(6) GDN_CASE(7) GDN_CASE(8)
+#undef GDN_CASE
+        default: return -3;
+      }
+    }
+    if (fs != nullptr) {
+      const int64_t n = (int64_t)N * D;
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(conv1d_final_state_kernel<T>), dim3((unsigned)((n + 255) / 256)), dim3(256),
+                         0, st, (const T*)x, (const T*)init, cu, (T*)fs, T_len, N, D, W);
+    }
+    return (int)hipGetLastError();
+  }
+  static int bwd(const void* x, const void* dy, const void* weight, const void* bias, const void* init,
+                 const void* dht, const int64_t* cu, void* dx, float* dw, float* db, void* dh0, float* workspace,
+                 int B, int T_len, int N, int D, int W, int silu, hipStream_t st) {
+    constexpr int V = Elem<T>::kVec;
+    const int64_t total = (int64_t)B * T_len;
+    const int tile = 256;
+    const int ntiles = (int)((total + tile - 1) / tile);
+    dim3 grid((D / V + kConvThreads - 1) / kConvThreads, (unsigned)ntiles);
+    if (total > 0) {
+      switch (W) {
+#define GDN_CASE(W_)                                                                                              \
+  case W_:                                                                                                        \
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(conv1d_bwd_kernel<T, W_>), grid, dim3(kConvThreads), 0, st, (const T*)x,   \
+                       (const T*)dy, (const T*)weight, (const T*)bias, (const T*)init, (const T*)dht, cu, (T*)dx, \
+                       workspace, total, T_len, N, D, tile, silu);                                                \
+    break;
+        GDN_CASE(1) GDN_CASE(2) GDN_CASE(3) GDN_CASE(4) GDN_CASE(5) GDN_CASE(6) GDN_CASE(7) GDN_CASE(8)
+#undef GDN_CASE
+        default: return -3;
+      }
+    }
+    const int64_t nred = (int64_t)(W + 1) * D;
+    hipLaunchKernelGGL(conv1d_reduce_kernel, dim3((unsigned)((nred + 255) / 256)), dim3(256), 0, st, workspace, dw, db,
+                       ntiles, W, D);
+    if (dh0 != nullptr) {
+      const int64_t n = (int64_t)N * D;
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(conv1d_dh0_kernel<T>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+                         (const T*)x, (const T*)dy, (const T*)weight, (const T*)bias, (const T*)init, (const T*)dht,
+                         cu, (T*)dh0, T_len, N, D, W, silu);
+    }
+    return (int)hipGetLastError();
+  }
+  static int update(const void* hidden, void* state, const void* weight, const void* bias, void* out, int B,
+                    int T_len, int D, int W, int S, int silu, hipStream_t st) {
+    const int64_t n = (int64_t)B * D;
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(conv1d_update_kernel<T>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+                       (const T*)hidden, (T*)state, (const T*)weight, (const T*)bias, (T*)out, B, T_len, D, W, S, silu);
+    return (int)hipGetLastError();
+  }
+};
+
+static int conv_check(int B, int T_len, int N, int D, int W, int dtype) {
+  if (B <= 0 || T_len < 0 || N <= 0 || D <= 0) return -2;
+  if (W < 1 || W > 8) return -3;
+  const int V = dtype == 0 ? 4 : 8;
+  if (D % V != 0) return -3;
+  if (dtype < 0 || dtype > 2) return -4;
+  return 0;
+}
+
+}  // namespace gdn
+
+extern "C" int64_t gdn_conv1d_bwd_workspace_bytes(int B, int T, int D, int W) {
+  const int64_t total = (int64_t)B * T;
+  const int64_t ntiles = (total + 255) / 256;
+  return (ntiles > 0 ? ntiles : 1) * (int64_t)(W + 1) * D * (int64_t)sizeof(float);
+}
+
+extern "C" int gdn_conv1d_fwd(const void* x, const void* weight, const void* bias, const void* residual,
+                              const void* initial_state, const int64_t* cu_seqlens, void* y, void* final_state, int B,
+                              int T, int N, int D, int W, int activation, int dtype, void* stream) {
+  if (!x || !weight || !y) return -1;
+  if (int e = gdn::conv_check(B, T, N, D, W, dtype)) return e;
+  if (cu_seqlens != nullptr && B != 1) return -2;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == 0) return gdn::ConvLaunch<float>::fwd(x, weight, bias, residual, initial_state, cu_seqlens, y, final_state, B, T, N, D, W, activation, s);
+  if (dtype == 1) return gdn::ConvLaunch<gdn::bf16_t>::fwd(x, weight, bias, residual, initial_state, cu_seqlens, y, final_state, B, T, N, D, W, activation, s);
+  return gdn::ConvLaunch<gdn::f16_t>::fwd(x, weight, bias, residual, initial_state, cu_seqlens, y, final_state, B, T, N, D, W, activation, s);
+}
+
+extern "C" int gdn_conv1d_bwd(const void* x, const void* dy, const void* weight, const void* bias,
+                              const void* initial_state, const void* d_final_state, const int64_t* cu_seqlens,
+                              void* dx, float* dw, float* db, void* d_initial_state, void* workspace,
+                              int64_t workspace_bytes, int B, int T, int N, int D, int W, int activation, int dtype,
+                              void* stream) {
+  if (!x || !dy || !weight || !dx || !dw || !workspace) return -1;
+  if (int e = gdn::conv_check(B, T, N, D, W, dtype)) return e;
+  if (cu_seqlens != nullptr && B != 1) return -2;
+  if (workspace_bytes < gdn_conv1d_bwd_workspace_bytes(B, T, D, W)) return -5;
+  hipStream_t s = (hipStream_t)stream;
+  float* ws = (float*)workspace;
+  if (dtype == 0) return gdn::ConvLaunch<float>::bwd(x, dy, weight, bias, initial_state, d_final_state, cu_seqlens, dx, dw, db, d_initial_state, ws, B, T, N, D, W, activation, s);
+  if (dtype == 1) return gdn::ConvLaunch<gdn::bf16_t>::bwd(x, dy, weight, bias, initial_state, d_final_state, cu_seqlens, dx, dw, db, d_initial_state, ws, B, T, N, D, W, activation, s);
+  return gdn::ConvLaunch<gdn::f16_t>::bwd(x, dy, weight, bias, initial_state, d_final_state, cu_seqlens, dx, dw, db, d_initial_state, ws, B, T, N, D, W, activation, s);
+}
+
+extern "C" int gdn_conv1d_update(const void* hidden, void* conv_state, const void* weight, const void* bias, void* out,
+                                 int B, int T, int D, int W, int state_len, int activation, int dtype, void* stream) {
+  if (!hidden || !conv_state || !weight || !out) return -1;
+  if (B <= 0 || T < 0 || D <= 0) return -2;
+  if (W < 1 || W > 8 || state_len < 1 || state_len > 16 || state_len < W - 1) return -3;
+  if (dtype < 0 || dtype > 2) return -4;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == 0) return gdn::ConvLaunch<float>::update(hidden, conv_state, weight, bias, out, B, T, D, W, state_len, activation, s);
+  if (dtype == 1) return gdn::ConvLaunch<gdn::bf16_t>::update(hidden, conv_state, weight, bias, out, B, T, D, W, state_len, activation, s);
+  return gdn::ConvLaunch<gdn::f16_t>::update(hidden, conv_state, weight, bias, out, B, T, D, W, state_len, activation, s);
+}

@@ -1,0 +1,306 @@
+"""Python entry points of the Gated DeltaNet operator path, with the reference's signatures.
+
+    chunk_gated_delta_rule            mindspeed_mm/fsdp/ops/gdn/chunk_gated_delta_rule.py:296-443
+    fused_recurrent_gated_delta_rule  call site mindspeed_mm/fsdp/models/qwen3_5/modeling_qwen3_5.py:877-886
+                                      (semantics of torch_recurrent_gated_delta_rule, :478-517)
+    causal_conv1d                     mindspeed_mm/fsdp/models/qwen3_5/causal_conv1d.py:100-119
+    causal_conv1d_update              modeling_qwen3_5.py:373-389, called at :738-744
+
+Everything here is host glue: validation, output/workspace allocation with torch, and one call into the
+C ABI per operator.  The kernels themselves are the HIP library; nothing in this file computes.
+"""
+import warnings
+from typing import Optional
+
+import torch
+
+from ._lib import DTYPE_CODE, GdnLibrary, default_library, ptr
+
+
+def _act_code(activation):
+    if activation in ("silu", "swish"):
+        return 1
+    if activation is None:
+        return 0
+    raise ValueError(f"unsupported activation {activation!r} (None, 'silu' or 'swish')")
+
+
+class GdnOps:
+    """The operators bound to one loaded kernel library."""
+
+    def __init__(self, lib: GdnLibrary):
+        self.lib = lib
+
+    # ------------------------------------------------------------------ helpers
+    def _need(self, *tensors):
+        for t in tensors:
+            if t is not None and t.device.type != self.lib.device_type:
+                raise RuntimeError(
+                    f"tensor on {t.device}; these operators run only on {self.lib.device_type} tensors "
+                    "(there is no host fallback)")
+
+    @staticmethod
+    def _f32(t):
+        return None if t is None else t.detach().to(torch.float32).contiguous()
+
+    # ------------------------------------------------------------------ chunked rule
+    def chunk_gated_delta_rule(self, q, k, v, g, beta, scale=None, initial_state=None, output_final_state=False,
+                               use_qk_l2norm_in_kernel=False, cu_seqlens=None, chunk_size=64, head_first=False,
+                               skip_recompute=False):
+        if q.dtype != k.dtype or k.dtype != v.dtype:
+            raise ValueError(
+                f"q current type is {q.dtype} , k current type is {k.dtype} ,v current type is {v.dtype} , "
+                "they should are equal")
+        if q.dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"chunk_gated_delta_rule supports bfloat16 and float32, got {q.dtype}")
+        if len(beta.shape) != 3:
+            raise ValueError(
+                f"beta current shape len is {len(beta.shape)}, beta must be of shape [B, T, H] if head_first=False, "
+                "or [B, H, T] otherwise.")
+        if head_first:
+            raise ValueError("head_first=True is deprecated in the reference and not supported here; "
+                             "pass [B, T, H, ...] tensors")
+        if chunk_size != 64:
+            raise ValueError("only chunk_size=64 is supported")
+        if q.shape[1] < q.shape[2]:
+            warnings.warn(
+                f"Input tensor shape suggests potential format mismatch: seq_len ({q.shape[1]}) < num_heads "
+                f"({q.shape[2]}). Please verify your input tensor format matches the expected shape [B, T, H, ...].")
+        if cu_seqlens is not None:
+            if q.shape[0] != 1:
+                raise ValueError(
+                    f"The batch size is expected to be 1 rather than {q.shape[0]} when using `cu_seqlens`."
+                    f"Please flatten variable-length inputs before processing.")
+            if initial_state is not None and initial_state.shape[0] != len(cu_seqlens) - 1:
+                raise ValueError(
+                    f"The number of initial states is expected to be equal to the number of input sequences, "
+                    f"i.e., {len(cu_seqlens) - 1} rather than {initial_state.shape[0]}.")
+        if v.shape[2] % q.shape[2] != 0 or k.shape != q.shape or g.shape != beta.shape or \
+                tuple(g.shape) != tuple(v.shape[:3]):
+            raise ValueError("expected q,k [B,T,Hqk,K], v [B,T,Hv,V], g,beta [B,T,Hv] with Hv % Hqk == 0")
+        if scale is None:
+            scale = k.shape[-1] ** -0.5
+        self._need(q, k, v, g, beta, initial_state, cu_seqlens)
+        return _ChunkGatedDeltaRule.apply(q, k, v, g, beta, float(scale), initial_state, bool(output_final_state),
+                                          cu_seqlens, bool(use_qk_l2norm_in_kernel), self)
+
+    # ------------------------------------------------------------------ decode
+    def fused_recurrent_gated_delta_rule(self, q, k, v, g, beta=None, scale=None, initial_state=None,
+                                         output_final_state=False, cu_seqlens=None, use_qk_l2norm_in_kernel=False,
+                                         inplace_state=False):
+        """One or more decode tokens per sequence.  Returns (o, final_state); final_state is a new fp32 tensor
+        unless inplace_state=True, in which case initial_state (fp32, contiguous) is updated and returned."""
+        if cu_seqlens is not None:
+            raise NotImplementedError("cu_seqlens is not supported by the decode kernel")
+        if q.dtype != k.dtype or k.dtype != v.dtype or q.dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError("q, k, v must share a dtype, bfloat16 or float32")
+        B, T, Hqk, K = q.shape
+        Hv, V = v.shape[2], v.shape[3]
+        if beta is None:
+            beta = torch.ones(B, T, Hv, dtype=torch.float32, device=q.device)
+        self._need(q, k, v, g, beta, initial_state)
+        if scale is None:
+            scale = K ** -0.5
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        o = torch.empty_like(v)
+        s_in = None
+        if initial_state is not None:
+            if inplace_state:
+                if initial_state.dtype != torch.float32 or not initial_state.is_contiguous():
+                    raise ValueError("inplace_state needs a contiguous float32 state")
+                s_in = initial_state
+            else:
+                s_in = self._f32(initial_state)
+        s_out = None
+        if output_final_state or inplace_state:
+            s_out = s_in if (inplace_state and s_in is not None) else \
+                torch.empty(B, Hv, K, V, dtype=torch.float32, device=q.device)
+        g32, b32 = self._f32(g), self._f32(beta)   # named: temporaries must outlive the launch
+        code = self.lib.gdn_recurrent_fwd(ptr(q), ptr(k), ptr(v), ptr(g32), ptr(b32), ptr(s_in),
+                                          ptr(s_out), ptr(o), B, T, Hqk, Hv, K, V, float(scale),
+                                          int(use_qk_l2norm_in_kernel), DTYPE_CODE[q.dtype], self.lib.stream())
+        self.lib.check(code, "gdn_recurrent_fwd")
+        return o, (s_out if output_final_state else None)
+
+    # ------------------------------------------------------------------ conv1d
+    def causal_conv1d(self, x, weight, bias=None, residual=None, initial_state=None, activation=None,
+                      cu_seqlens=None, output_final_state=False):
+        if x.shape[-1] != weight.shape[-1]:
+            raise ValueError("x [B, T, D], weight [W, D], please check.")
+        if cu_seqlens is not None and x.shape[0] != 1:
+            raise ValueError("cu_seqlens needs batch size 1 (packed input)")
+        _act_code(activation)
+        self._need(x, weight, bias, residual, initial_state, cu_seqlens)
+        return _CausalConv1d.apply(x, weight, bias, residual, initial_state, activation, cu_seqlens,
+                                   bool(output_final_state), self)
+
+    def causal_conv1d_update(self, hidden_states, conv_state, weight, bias=None, activation=None):
+        """hidden_states [B,T,D]; conv_state [B,D,S] updated in place; weight [D,W]."""
+        self._need(hidden_states, conv_state, weight, bias)
+        B, T, D = hidden_states.shape
+        W, S = weight.shape[1], conv_state.shape[-1]
+        dt = hidden_states.dtype
+        if not conv_state.is_contiguous():
+            raise ValueError("conv_state must be contiguous (it is updated in place)")
+        x = hidden_states.contiguous()
+        state = conv_state if conv_state.dtype == dt else conv_state.to(dt)
+        out = torch.empty_like(x)
+        wc = weight.to(dt).contiguous()
+        bc = None if bias is None else bias.to(dt).contiguous()
+        code = self.lib.gdn_conv1d_update(ptr(x), ptr(state), ptr(wc), ptr(bc), ptr(out), B, T, D,
+                                          W, S, _act_code(activation), DTYPE_CODE[dt], self.lib.stream())
+        self.lib.check(code, "gdn_conv1d_update")
+        if state is not conv_state:
+            conv_state.copy_(state)
+        return out
+
+
+def _i64(cu, ref):
+    if cu is None:
+        return None
+    return cu.to(device=ref.device, dtype=torch.int64).contiguous()
+
+
+class _ChunkGatedDeltaRule(torch.autograd.Function):
+    """Positional order as ChunkGatedDeltaRuleFunction.forward (chunk_gated_delta_rule.py:182-196)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens,
+                use_qk_l2norm_in_kernel, ops):
+        lib = ops.lib
+        B, T, Hqk, K = q.shape
+        Hv, V = v.shape[2], v.shape[3]
+        N = (len(cu_seqlens) - 1) if cu_seqlens is not None else B
+        need_grad = any(ctx.needs_input_grad[:5]) or (initial_state is not None and ctx.needs_input_grad[6])
+        qc, kc, vc = q.contiguous(), k.contiguous(), v.contiguous()
+        g32, b32, h0 = ops._f32(g), ops._f32(beta), ops._f32(initial_state)
+        cu = _i64(cu_seqlens, q)
+        code = DTYPE_CODE[q.dtype]
+        nbytes = lib.gdn_chunk_workspace_bytes(B, T, N, Hqk, Hv, K, V, code, int(need_grad))
+        ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=q.device)
+        off = (-ws.data_ptr()) % 256
+        ws = ws[off:off + nbytes]
+        o = torch.empty_like(vc)
+        ht = torch.empty(N, Hv, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
+        rc = lib.gdn_chunk_fwd(ptr(qc), ptr(kc), ptr(vc), ptr(g32), ptr(b32), ptr(h0), ptr(cu), ptr(o), ptr(ht),
+                               ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale, int(use_qk_l2norm_in_kernel), code,
+                               lib.stream())
+        lib.check(rc, "gdn_chunk_fwd")
+        if need_grad:
+            ctx.save_for_backward(qc, kc, vc, g32, b32, h0, cu, ws)
+            ctx.meta = (B, T, N, Hqk, Hv, K, V, scale, int(use_qk_l2norm_in_kernel), code, nbytes,
+                        g.dtype, beta.dtype, None if initial_state is None else initial_state.dtype)
+            ctx.ops = ops
+        return o, ht
+
+    @staticmethod
+    def backward(ctx, do, dht):
+        qc, kc, vc, g32, b32, h0, cu, ws = ctx.saved_tensors
+        B, T, N, Hqk, Hv, K, V, scale, l2, code, nbytes, g_dt, b_dt, h_dt = ctx.meta
+        lib = ctx.ops.lib
+        do = do.contiguous()
+        dht = ctx.ops._f32(dht)
+        dq, dk, dv = torch.empty_like(qc), torch.empty_like(kc), torch.empty_like(vc)
+        dg = torch.empty(B, T, Hv, dtype=torch.float32, device=qc.device)
+        db = torch.empty(B, T, Hv, dtype=torch.float32, device=qc.device)
+        dh0 = torch.empty(N, Hv, K, V, dtype=torch.float32, device=qc.device) if h0 is not None else None
+        rc = lib.gdn_chunk_bwd(ptr(qc), ptr(kc), ptr(vc), ptr(g32), ptr(b32), ptr(h0), ptr(cu), ptr(do), ptr(dht),
+                               ptr(dq), ptr(dk), ptr(dv), ptr(dg), ptr(db), ptr(dh0), ptr(ws), nbytes, B, T, N, Hqk,
+                               Hv, K, V, scale, l2, code, lib.stream())
+        lib.check(rc, "gdn_chunk_bwd")
+        return (dq, dk, dv, dg.to(g_dt), db.to(b_dt), None, None if dh0 is None else dh0.to(h_dt), None, None, None,
+                None)
+
+
+class _CausalConv1d(torch.autograd.Function):
+    """Argument order as CausalConv1dFunction.forward (models/qwen3_5/causal_conv1d.py:27-38)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, residual, initial_state, activation, cu_seqlens, output_final_state, ops):
+        lib = ops.lib
+        B, T, D = x.shape
+        W = weight.shape[0]
+        N = (len(cu_seqlens) - 1) if cu_seqlens is not None else B
+        dt = x.dtype
+        xc = x.contiguous()
+        wc = weight.to(dt).contiguous()
+        bc = None if bias is None else bias.to(dt).contiguous()
+        rc_ = None if residual is None else residual.to(dt).contiguous()
+        h0 = None if initial_state is None else initial_state.to(dt).contiguous()
+        cu = _i64(cu_seqlens, x)
+        y = torch.empty_like(xc)
+        fs = torch.empty(N, D, W, dtype=dt, device=x.device) if output_final_state else None
+        code = lib.gdn_conv1d_fwd(ptr(xc), ptr(wc), ptr(bc), ptr(rc_), ptr(h0), ptr(cu), ptr(y), ptr(fs), B, T, N, D,
+                                  W, _act_code(activation), DTYPE_CODE[dt], lib.stream())
+        lib.check(code, "gdn_conv1d_fwd")
+        ctx.save_for_backward(xc, wc, bc, h0, cu)
+        ctx.meta = (B, T, N, D, W, _act_code(activation), dt, weight.dtype, None if bias is None else bias.dtype,
+                    residual is not None, None if residual is None else residual.dtype,
+                    None if initial_state is None else initial_state.dtype)
+        ctx.ops = ops
+        return y, fs
+
+    @staticmethod
+    def backward(ctx, dy, dfs):
+        xc, wc, bc, h0, cu = ctx.saved_tensors
+        B, T, N, D, W, act, dt, w_dt, b_dt, has_res, r_dt, h_dt = ctx.meta
+        lib = ctx.ops.lib
+        dy = dy.to(dt).contiguous()
+        dfs = None if dfs is None else dfs.to(dt).contiguous()
+        dx = torch.empty_like(xc)
+        dw = torch.empty(W, D, dtype=torch.float32, device=xc.device)
+        db = torch.empty(D, dtype=torch.float32, device=xc.device) if bc is not None else None
+        dh0 = torch.empty(N, D, W, dtype=dt, device=xc.device) if h0 is not None else None
+        nbytes = lib.gdn_conv1d_bwd_workspace_bytes(B, T, D, W)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=xc.device)
+        code = lib.gdn_conv1d_bwd(ptr(xc), ptr(dy), ptr(wc), ptr(bc), ptr(h0), ptr(dfs), ptr(cu), ptr(dx), ptr(dw),
+                                  ptr(db), ptr(dh0), ptr(ws), nbytes, B, T, N, D, W, act, DTYPE_CODE[dt], lib.stream())
+        lib.check(code, "gdn_conv1d_bwd")
+        return (dx, dw.to(w_dt), None if db is None else db.to(b_dt), dy.to(r_dt) if has_res else None,
+                None if dh0 is None else dh0.to(h_dt), None, None, None, None)
+
+
+# ---------------------------------------------------------------------- module-level entry points
+_ops: Optional[GdnOps] = None
+
+
+def _default_ops() -> GdnOps:
+    global _ops
+    if _ops is None:
+        _ops = GdnOps(default_library())
+    return _ops
+
+
+@torch.compiler.disable
+def chunk_gated_delta_rule(q, k, v, g, beta, scale=None, initial_state=None, output_final_state=False,
+                           use_qk_l2norm_in_kernel=False, cu_seqlens=None, chunk_size=64, head_first=False,
+                           skip_recompute=False):
+    """Drop-in for mindspeed_mm.fsdp.ops.gdn.chunk_gated_delta_rule.chunk_gated_delta_rule.
+
+    q,k [B,T,Hqk,K]; v [B,T,Hv,V]; g,beta [B,T,Hv]; Hv may be a multiple of Hqk (grouped heads are read in
+    place; dq/dk come back summed over each group).  float32 is accepted as well as bfloat16.
+    `skip_recompute` is accepted and ignored (all backward inputs are kept in the workspace)."""
+    return _default_ops().chunk_gated_delta_rule(q, k, v, g, beta, scale, initial_state, output_final_state,
+                                                 use_qk_l2norm_in_kernel, cu_seqlens, chunk_size, head_first,
+                                                 skip_recompute)
+
+
+@torch.compiler.disable
+def fused_recurrent_gated_delta_rule(q, k, v, g, beta=None, scale=None, initial_state=None,
+                                     output_final_state=False, cu_seqlens=None, use_qk_l2norm_in_kernel=False,
+                                     inplace_state=False):
+    return _default_ops().fused_recurrent_gated_delta_rule(q, k, v, g, beta, scale, initial_state,
+                                                           output_final_state, cu_seqlens, use_qk_l2norm_in_kernel,
+                                                           inplace_state)
+
+
+@torch.compiler.disable
+def causal_conv1d(x, weight, bias=None, residual=None, initial_state=None, activation=None, cu_seqlens=None,
+                  output_final_state=False):
+    return _default_ops().causal_conv1d(x, weight, bias, residual, initial_state, activation, cu_seqlens,
+                                        output_final_state)
+
+
+@torch.compiler.disable
+def causal_conv1d_update(hidden_states, conv_state, weight, bias=None, activation=None):
+    return _default_ops().causal_conv1d_update(hidden_states, conv_state, weight, bias, activation)

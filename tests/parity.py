@@ -1,0 +1,134 @@
+"""Parity checks shared by the GPU tests (HIP library on cuda:0) and the CPU kernel-emulation tests.
+
+Each check runs one operator of the package through the C ABI on seeded inputs and compares it with the
+CPU oracle (oracle/gdn_oracle.py).  Tolerances are the ones the task states:
+    fp32: max relative error (max|x - ref| / max|ref|) <= 1e-4
+    bf16 vs the fp32 oracle on the same (bf16-valued) inputs: max abs error <= 2e-2 on o,
+          <= 5e-2 on dq/dk/dv/dg/dbeta (and on the states, whose magnitude is O(1)).
+"""
+import math
+
+import torch
+import torch.nn.functional as F
+
+from oracle import gdn_oracle as O
+
+FP32_REL = 1e-4
+BF16_ABS_O = 2e-2
+BF16_ABS_GRAD = 5e-2
+
+
+def gdn_inputs(B, T, Hqk, Hv, K, V, dtype, seed=0, N=None, l2norm_in_kernel=True, a_log=(1.0, 16.0),
+               dt_bias=(-4.0, -2.0), h0_std=0.02):
+    """Input recipe of the benchmark configurations: q,k ~ N(0,1) (L2-normalised here if the kernel does not
+    do it), v ~ N(0,1), beta = sigmoid(N(0,1)), g = -exp(A_log) softplus(N(0,1) + dt_bias) with per-head
+    A_log ~ U(log a0, log a1), dt_bias ~ U(b0, b1) (caller-side math: modeling_qwen3_5.py:833-841)."""
+    gen = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=gen)
+    q, k, v = r(B, T, Hqk, K), r(B, T, Hqk, K), r(B, T, Hv, V)
+    if not l2norm_in_kernel:
+        q, k = O.l2norm(q), O.l2norm(k)
+    beta = torch.sigmoid(r(B, T, Hv))
+    A_log = torch.empty(Hv).uniform_(math.log(a_log[0]), math.log(a_log[1]), generator=gen)
+    bias = torch.empty(Hv).uniform_(dt_bias[0], dt_bias[1], generator=gen)
+    g = -A_log.exp() * F.softplus(r(B, T, Hv) + bias)
+    h0 = h0_std * r(N if N is not None else B, Hv, K, V)
+    do = r(B, T, Hv, V)
+    dht = h0_std * r(N if N is not None else B, Hv, K, V)
+    return dict(q=q.to(dtype), k=k.to(dtype), v=v.to(dtype), g=g, beta=beta.to(dtype), h0=h0, do=do.to(dtype), dht=dht)
+
+
+def _err(name, got, ref, dtype, abs_tol, rtol=0.0):
+    """fp32: max|x-ref| <= 1e-4 max|ref|.  Half precision: |x-ref| <= abs_tol + rtol |ref| elementwise."""
+    got, ref = got.detach().float().cpu(), ref.detach().float().cpu()
+    assert got.shape == ref.shape, f"{name}: shape {tuple(got.shape)} vs {tuple(ref.shape)}"
+    assert torch.isfinite(got).all(), f"{name}: non-finite values"
+    diff = (got - ref).abs().max().item() if got.numel() else 0.0
+    scale = ref.abs().max().item() if got.numel() else 0.0
+    if dtype == torch.float32:
+        assert diff <= FP32_REL * max(scale, 1e-30), f"{name}: max rel err {diff / max(scale, 1e-30):.3e} > {FP32_REL}"
+    else:
+        excess = ((got - ref).abs() - rtol * ref.abs()).max().item() if got.numel() else 0.0
+        assert excess <= abs_tol, f"{name}: max abs err {diff:.3e} > {abs_tol} + {rtol}|ref| (ref max {scale:.3f})"
+    return diff
+
+
+def check_chunk(ops, device, B, T, Hqk, Hv, K, V, dtype, l2=True, cu=None, backward=False, seed=0, with_h0=True,
+                scale=None, wrap=lambda t: t, **recipe):
+    N = (len(cu) - 1) if cu is not None else B
+    x = gdn_inputs(B, T, Hqk, Hv, K, V, dtype, seed=seed, N=N, l2norm_in_kernel=l2, **recipe)
+    dev = {n: wrap(t.to(device)) for n, t in x.items()}
+    leaves = {n: dev[n].clone().requires_grad_(backward) for n in ("q", "k", "v", "g", "beta")}
+    h0 = dev["h0"].clone().requires_grad_(backward) if with_h0 else None
+    cu_t = torch.tensor(cu, dtype=torch.int64, device=device) if cu is not None else None
+    o, ht = ops.chunk_gated_delta_rule(leaves["q"], leaves["k"], leaves["v"], leaves["g"], leaves["beta"],
+                                       scale=scale, initial_state=h0, output_final_state=True,
+                                       use_qk_l2norm_in_kernel=l2, cu_seqlens=cu_t)
+    ref_leaves = {n: x[n].float().clone().requires_grad_(backward) for n in ("q", "k", "v", "g", "beta")}
+    rh0 = x["h0"].clone().requires_grad_(backward) if with_h0 else None
+    ro, rht = O.chunk_gated_delta_rule_ref(ref_leaves["q"], ref_leaves["k"], ref_leaves["v"], ref_leaves["g"],
+                                           ref_leaves["beta"], scale=scale, initial_state=rh0,
+                                           output_final_state=True, use_qk_l2norm_in_kernel=l2, cu_seqlens=cu)
+    assert o.dtype == dtype and ht.dtype == torch.float32
+    errs = {"o": _err("o", o, ro, dtype, BF16_ABS_O), "ht": _err("final_state", ht, rht, dtype, BF16_ABS_GRAD)}
+    if backward:
+        ((o.float() * dev["do"].float()).sum() + (ht * dev["dht"]).sum()).backward()
+        ((ro * x["do"].float()).sum() + (rht * x["dht"]).sum()).backward()
+        for n in ("q", "k", "v", "g", "beta"):
+            assert leaves[n].grad.dtype == leaves[n].dtype
+            errs["d" + n] = _err("d" + n, leaves[n].grad, ref_leaves[n].grad, dtype, BF16_ABS_GRAD)
+        if with_h0:
+            errs["dh0"] = _err("dh0", h0.grad, rh0.grad, dtype, BF16_ABS_GRAD)
+    return errs
+
+
+def check_recurrent(ops, device, B, T, Hqk, Hv, K, V, dtype, l2=True, seed=0, with_state=True, wrap=lambda t: t):
+    x = gdn_inputs(B, T, Hqk, Hv, K, V, dtype, seed=seed, l2norm_in_kernel=l2)
+    dev = {n: wrap(t.to(device)) for n, t in x.items()}
+    s0 = dev["h0"] if with_state else None
+    o, s = ops.fused_recurrent_gated_delta_rule(dev["q"], dev["k"], dev["v"], dev["g"], dev["beta"], initial_state=s0,
+                                                output_final_state=True, use_qk_l2norm_in_kernel=l2)
+    ro, rs = O.recurrent_gated_delta_rule_ref(x["q"].float(), x["k"].float(), x["v"].float(), x["g"],
+                                              x["beta"].float(), x["h0"] if with_state else None, True, l2)
+    return {"o": _err("o", o, ro, dtype, BF16_ABS_O), "state": _err("state", s, rs, torch.float32, 0)}
+
+
+def check_conv(ops, device, B, T, D, W, dtype, activation="silu", cu=None, bias=True, residual=False, state=True,
+               backward=True, seed=0, wrap=lambda t: t):
+    gen = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=gen)
+    N = (len(cu) - 1) if cu is not None else B
+    x = dict(x=r(B, T, D), w=r(W, D) / 2, b=r(D) if bias else None, res=r(B, T, D) if residual else None,
+             h0=r(N, D, W) if state else None, dy=r(B, T, D), dfs=r(N, D, W))
+    x = {n: (None if t is None else t.to(dtype)) for n, t in x.items()}
+    cu_t = torch.tensor(cu, dtype=torch.int64, device=device) if cu is not None else None
+    mk = lambda t, grad: None if t is None else wrap(t.to(device)).clone().requires_grad_(grad)
+    dv = dict(x=mk(x["x"], backward), w=mk(x["w"], backward), b=mk(x["b"], backward), res=mk(x["res"], backward),
+              h0=mk(x["h0"], backward))
+    y, fs = ops.causal_conv1d(dv["x"], dv["w"], dv["b"], dv["res"], dv["h0"], activation, cu_t, True)
+    rf = {n: (None if t is None else t.float().clone().requires_grad_(backward)) for n, t in x.items()
+          if n in ("x", "w", "b", "res", "h0")}
+    ry, rfs = O.causal_conv1d_ref(rf["x"], rf["w"], rf["b"], rf["res"], rf["h0"], activation, cu, True)
+    # half precision: the reference's own bounds (test_forward.py:299-305, test_backward.py:88-89), applied as
+    # allclose(atol, rtol) because outputs here reach |y| ~ 6 where one bf16 ulp is already 3e-2
+    tol_f, tol_b, rt = 1e-2, 5e-2, 1e-2
+    errs = {"y": _err("y", y, ry, dtype, tol_f, rt), "final_state": _err("final_state", fs, rfs, dtype, tol_f, rt)}
+    if backward:
+        ((y.float() * x["dy"].to(device).float()).sum() + (fs.float() * x["dfs"].to(device).float()).sum()).backward()
+        ((ry * x["dy"].float()).sum() + (rfs * x["dfs"].float()).sum()).backward()
+        for n in ("x", "w", "b", "res", "h0"):
+            if dv[n] is not None:
+                tol = tol_b * (max(1.0, B * T / 256) if n in ("w", "b") else 1.0)   # test_large_shape.py:156-158
+                errs["d" + n] = _err("d" + n, dv[n].grad, rf[n].grad, dtype, tol, rt)
+    return errs
+
+
+def check_conv_update(ops, device, B, T, D, W, dtype, seed=0, wrap=lambda t: t):
+    gen = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=gen)
+    x, st, w, b = r(B, T, D).to(dtype), r(B, D, W).to(dtype), (r(D, W) / 2).to(dtype), r(D).to(dtype)
+    st_dev = wrap(st.to(device)).clone()
+    y = ops.causal_conv1d_update(wrap(x.to(device)), st_dev, wrap(w.to(device)), wrap(b.to(device)), "silu")
+    st_ref = st.float().clone()
+    ry = O.causal_conv1d_update_ref(x.float(), st_ref, w.float(), b.float(), "silu")
+    return {"y": _err("y", y, ry, dtype, 1e-2, 1e-2), "state": _err("state", st_dev, st_ref, dtype, 1e-2, 1e-2)}

@@ -1,0 +1,51 @@
+"""CPU checks of the HIP kernel sources themselves, compiled for the host against a fiber-based stand-in
+for the HIP runtime (tests/emu).  Same operators, same C ABI, same oracle as the GPU parity tests, on
+small shapes; buffers sit against guard pages so an out-of-range index is a SIGSEGV here rather than a
+GPU fault.  The shipped library is not involved: these tests prove indexing/synchronisation logic, the
+`-m gpu` tests prove the device build."""
+import pytest
+import torch
+
+from tests import parity as P
+from tests.emu.emu_backend import emu_ops, guarded
+
+BF, F32 = torch.bfloat16, torch.float32
+
+
+@pytest.fixture(scope="module")
+def ops():
+    return emu_ops()
+
+
+@pytest.mark.parametrize("dtype,B,T,Hqk,Hv,K,V", [
+    (F32, 2, 3, 1, 2, 64, 64), (BF, 2, 2, 2, 4, 128, 128), (F32, 1, 1, 1, 1, 128, 192), (BF, 1, 4, 1, 2, 256, 128),
+])
+def test_recurrent(ops, dtype, B, T, Hqk, Hv, K, V):
+    P.check_recurrent(ops, "cpu", B, T, Hqk, Hv, K, V, dtype, wrap=guarded)
+    P.check_recurrent(ops, "cpu", B, T, Hqk, Hv, K, V, dtype, l2=False, with_state=False, wrap=guarded)
+
+
+@pytest.mark.parametrize("dtype,B,T,Hqk,Hv,K,V,l2,cu", [
+    (F32, 1, 64, 1, 1, 64, 64, False, None),
+    (F32, 2, 100, 2, 4, 128, 128, True, None),
+    (BF, 1, 200, 1, 2, 128, 128, True, None),
+    (BF, 1, 140, 2, 2, 64, 64, False, [0, 5, 70, 71, 140]),
+    (BF, 1, 128, 1, 1, 128, 256, True, None),
+    (F32, 1, 96, 1, 1, 128, 192, True, [0, 1, 38, 96]),
+])
+def test_chunk_forward(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu):
+    P.check_chunk(ops, "cpu", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu, wrap=guarded, h0_std=0.1)
+
+
+@pytest.mark.parametrize("dtype,B,T,D,W,cu", [
+    (F32, 2, 37, 16, 4, None), (BF, 1, 300, 32, 4, [0, 1, 3, 130, 131, 300]), (F32, 1, 9, 8, 3, [0, 2, 9]),
+    (torch.float16, 2, 5, 8, 2, None), (F32, 3, 2, 8, 4, None), (F32, 1, 600, 8, 4, [0, 255, 257, 600]),
+])
+def test_conv1d(ops, dtype, B, T, D, W, cu):
+    P.check_conv(ops, "cpu", B, T, D, W, dtype, cu=cu, residual=True, wrap=guarded)
+    P.check_conv(ops, "cpu", B, T, D, W, dtype, cu=cu, bias=False, state=False, activation=None, wrap=guarded)
+
+
+@pytest.mark.parametrize("dtype,B,T,D,W", [(F32, 2, 1, 16, 4), (BF, 3, 5, 8, 4), (F32, 1, 3, 8, 2)])
+def test_conv1d_update(ops, dtype, B, T, D, W):
+    P.check_conv_update(ops, "cpu", B, T, D, W, dtype, wrap=guarded)
