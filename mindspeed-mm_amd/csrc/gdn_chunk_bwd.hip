@@ -1,7 +1,661 @@
+// Chunked gated delta rule, backward pass.  Notation as in gdn_chunk_fwd.hip; S is the state BEFORE a
+// chunk, dS' the gradient of the state AFTER it, Gam_ij = e^{G_i - G_j}, everything per (sequence, head):
+//   dv_local = scale tril(Q K^T . Gam)^T dO                                   chunk_dv_local_kernel
+//   dV' = (K dS') . e^{G_last-G} + dv_local                                   chunk_state_bwd_kernel
+//   dS  = e^{G_last} dS' + scale (Q . e^G)^T dO - W^T dV'                       (reverse recurrence)
+//   ds  = scale tril(dO V'^T . Gam);  dQ = scale e^G . (dO S^T) + ds K          chunk_dqkw_kernel
+//   dK1 = e^{G_last-G} . (V' dS'^T) + ds^T Q;  dW = -dV' S^T
+//   dG1_i = <q_i,dQ_i> - <k_i,dK1_i>  (+ e^{G_last}<S,dS'> + sum_j <k_j, dK_inter_j> at the last row)
+//   back through W = Tm (beta e^G K), U = Tm (beta V), Tm = (I+L)^-1:           chunk_wy_bwd_kernel
+//     P = Tm^T dW, R = Tm^T dV', dTm = strict_tril(dW Kb^T + dV' Vb^T), dM = -(Tm^T dTm Tm^T) . Gam
+//     dK2 = P beta e^G + beta (dM K) + dM^T (beta K);  dv = R beta
+//     dbeta = e^G<P,k> + <R,v> + <dM K, k>;  dG2 = beta e^G<P,k> + beta<dM K,k> - <dM^T(beta K),k>
+//   dg = reverse chunk-local cumsum(dG1 + dG2); group sum of dq/dk over grouped heads and the
+//   l2-norm backward dx = (dy - <dy,y> y) rstd                                  qk_grad_finalize_kernel
+// The equations are those of the reference's backward kernels (mindspeed_mm/fsdp/ops/gdn/triton/
+// chunk_o.py:19-284, chunk_delta_h.py:307-513, wy_fast.py:17-141, chunk_gated_delta_rule.py:88-174), with
+// the dG row/column sums rewritten as row dot products with dQ/dK so that Q K^T need not be rebuilt.
 #include "gdn_chunk.h"
 #include "gdn_common.h"
+
+namespace gdn {
+
+// for every accumulator row i of the tile: rowacc[i0+i] += factor * sum_j acc[i][j] * other[(i0+i)*ld + j0+j]
+template <typename T>
+__device__ __forceinline__ void acc_rowdot_add(const f32x16& acc, const T* other, int ld, int i0, int j0, float* rowacc,
+                                               float factor) {
+  const int j = j0 + acc_col();
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int i = i0 + acc_row(r);
+    const float s = half_wave_sum(acc[r] * Elem<T>::to_f(other[i * ld + j]));
+    if (acc_col() == 0) atomicAdd(&rowacc[i], factor * s);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+template <typename T, int DK, int BV> struct DvLocalSmem {
+  static constexpr int LDK = lds_ld<T>(DK), LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
+  static constexpr int off_qs = 0;
+  static constexpr int off_ks = off_qs + 64 * LDK * (int)sizeof(T);
+  static constexpr int off_do = off_ks + 64 * LDK * (int)sizeof(T);
+  static constexpr int off_pt = off_do + 64 * LDV * (int)sizeof(T);
+  static constexpr int off_gs = off_pt + 64 * L64 * (int)sizeof(T);
+  static constexpr int bytes = off_gs + 64 * 4;
+};
+
+template <typename T, int DK, int BV>
+__global__ __launch_bounds__(kThreads) void chunk_dv_local_kernel(
+    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ dO, const float* __restrict__ G,
+    T* __restrict__ dv, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N,
+    int Hqk, int Hv, int V, float scale) {
+  using SM = DvLocalSmem<T, DK, BV>;
+  constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64, MT = BV / 32;
+  T* Qs = reinterpret_cast<T*>(gdn_smem + SM::off_qs);
+  T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
+  T* dOs = reinterpret_cast<T*>(gdn_smem + SM::off_do);
+  T* PT = reinterpret_cast<T*>(gdn_smem + SM::off_pt);
+  float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_gs);
+  const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
+  if (s.nvalid <= 0) return;
+  const int tid = threadIdx.x, wave = tid >> 6;
+  const int h = blockIdx.y, hq = h / (Hv / Hqk), nvalid = s.nvalid, v0 = blockIdx.z * BV;
+  const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk;
+  load_tile<T, DK>(Qs, LDK, q + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
+  load_tile<T, DK>(Ks, LDK, k + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
+  load_tile<T, BV>(dOs, LDV, dO + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
+  if (tid < 64) Gs[tid] = G[(tok0 + imin(tid, nvalid - 1)) * Hv + h];
+  __syncthreads();
+  {  // PT[j][i] = scale (k_j . q_i) e^{G_i - G_j} for i >= j
+    const int tj = wave >> 1, ti = wave & 1;
+    f32x16 acc = acc_zero();
+    if (ti >= tj) mma32<T, DK, true, true>(acc, Ks + 32 * tj * LDK, LDK, Qs + 32 * ti * LDK, LDK);
+    const int i = 32 * ti + acc_col();
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int j = 32 * tj + acc_row(r);
+      PT[j * L64 + i] = Elem<T>::from_f(i >= j ? scale * acc[r] * __expf(Gs[i] - Gs[j]) : 0.f);
+    }
+  }
+  __syncthreads();
+  T* dvg = dv + (tok0 * Hv + h) * V + v0;
+  for (int tt = wave; tt < 2 * MT; tt += 4) {
+    const int ri = tt & 1, cj = tt >> 1;
+    f32x16 acc = acc_zero();
+    mma32<T, 64, true, false>(acc, PT + 32 * ri * L64, L64, dOs + 32 * cj, LDV);
+    acc_to_global(acc, dvg, (int64_t)Hv * V, 32 * ri, 32 * cj, nvalid);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// reverse recurrence; the transposed state-gradient slab dS^T[BV, DK] lives in accumulators
+// ---------------------------------------------------------------------------------------------
+template <typename T, int DK, int BV> struct StateBwdSmem {
+  static constexpr int LDK = lds_ld<T>(DK), LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
+  static constexpr int off_ks = 0;
+  static constexpr int off_qs = off_ks + 64 * LDK * (int)sizeof(T);
+  static constexpr int off_ws = off_qs + 64 * LDK * (int)sizeof(T);
+  static constexpr int off_dsb = off_ws + 64 * LDK * (int)sizeof(T);
+  static constexpr int off_do = off_dsb + BV * LDK * (int)sizeof(T);
+  static constexpr int off_dvt = off_do + 64 * LDV * (int)sizeof(T);
+  static constexpr int off_gs = off_dvt + BV * L64 * (int)sizeof(T);
+  static constexpr int bytes = off_gs + 2 * 64 * 4;
+};
+
+template <typename T, int DK, int BV>
+__global__ __launch_bounds__(kThreads) void chunk_state_bwd_kernel(
+    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ w, const T* __restrict__ dO, T* dv,
+    const float* __restrict__ G, const float* __restrict__ dht, float* __restrict__ dh0, T* __restrict__ dhbuf,
+    const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int Hqk, int Hv, int V,
+    float scale) {
+  using SM = StateBwdSmem<T, DK, BV>;
+  constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64;
+  constexpr int MT = BV / 32, NTC = DK / 32, NS = (MT * NTC + 3) / 4;
+  T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
+  T* Qs = reinterpret_cast<T*>(gdn_smem + SM::off_qs);
+  T* Ws = reinterpret_cast<T*>(gdn_smem + SM::off_ws);
+  T* dSb = reinterpret_cast<T*>(gdn_smem + SM::off_dsb);
+  T* dOs = reinterpret_cast<T*>(gdn_smem + SM::off_do);
+  T* dVT = reinterpret_cast<T*>(gdn_smem + SM::off_dvt);
+  float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_gs);
+  float* qsc = Gs + 64;
+
+  const int tid = threadIdx.x, wave = tid >> 6;
+  const int n = blockIdx.x / Hv, h = blockIdx.x % Hv, hq = h / (Hv / Hqk);
+  const int v0 = blockIdx.y * BV;
+  const int64_t bos = cu ? cu[n] : (int64_t)n * T_len;
+  const int len = cu ? (int)(cu[n + 1] - bos) : T_len;
+  const int nchunks = (len + kChunk - 1) / kChunk;
+  const int64_t chunk_base = cu ? chunk_offsets[n] : (int64_t)n * ((T_len + kChunk - 1) / kChunk);
+
+  f32x16 dS[NS];
+#pragma unroll
+  for (int i = 0; i < NS; ++i) {
+    const int tt = wave + 4 * i;
+    dS[i] = acc_zero();
+    if (tt < MT * NTC && dht != nullptr) {
+      const int mi = tt % MT, ni = tt / MT;
+      const int kcol = 32 * ni + acc_col();
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        dS[i][r] = dht[(((int64_t)n * Hv + h) * DK + kcol) * V + v0 + 32 * mi + acc_row(r)];
+    }
+  }
+
+  for (int c = nchunks - 1; c >= 0; --c) {
+    const int64_t tok0 = bos + (int64_t)c * kChunk;
+    const int nvalid = imin(kChunk, len - c * kChunk);
+    T* dhg = dhbuf + (((chunk_base + c) * Hv + h) * V + v0) * DK;
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+      const int tt = wave + 4 * i;
+      if (tt < MT * NTC) {
+        const int mi = tt % MT, ni = tt / MT;
+        acc_to_lds(dS[i], dSb, LDK, 32 * mi, 32 * ni);
+        acc_to_global(dS[i], dhg, (int64_t)DK, 32 * mi, 32 * ni, BV);
+      }
+    }
+    if (tid < 64) {
+      const float gv = G[(tok0 + imin(tid, nvalid - 1)) * Hv + h];
+      Gs[tid] = gv;
+      qsc[tid] = scale * __expf(gv);
+    }
+    __syncthreads();
+    load_tile<T, DK>(Ks, LDK, k + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
+    load_tile_scaled<T, DK>(Qs, LDK, q + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, qsc, tid);
+    load_tile<T, DK>(Ws, LDK, w + (tok0 * Hv + h) * DK, (int64_t)Hv * DK, nvalid, tid);
+    load_tile<T, BV>(dOs, LDV, dO + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
+    __syncthreads();
+    const float glast = Gs[63];
+    T* dvg = dv + (tok0 * Hv + h) * V + v0;
+    for (int tt = wave; tt < 2 * MT; tt += 4) {
+      const int ri = tt & 1, cj = tt >> 1;
+      f32x16 a = acc_zero();
+      mma32<T, DK, true, true>(a, Ks + 32 * ri * LDK, LDK, dSb + 32 * cj * LDK, LDK);
+      const f32x16 loc = acc_from_global(dvg, (int64_t)Hv * V, 32 * ri, 32 * cj, nvalid);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) a[r] = a[r] * __expf(glast - Gs[32 * ri + acc_row(r)]) + loc[r];
+      acc_to_global(a, dvg, (int64_t)Hv * V, 32 * ri, 32 * cj, nvalid);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) a[r] = (32 * ri + acc_row(r) < nvalid) ? -a[r] : 0.f;
+      acc_to_lds_t(a, dVT, L64, 32 * ri, 32 * cj);
+    }
+    __syncthreads();
+    const float eg = __expf(glast);
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+      const int tt = wave + 4 * i;
+      if (tt < MT * NTC) {
+        const int mi = tt % MT, ni = tt / MT;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dS[i][r] *= eg;
+        mma32<T, 64, false, false>(dS[i], dOs + 32 * mi, LDV, Qs + 32 * ni, LDK);
+        mma32<T, 64, true, false>(dS[i], dVT + 32 * mi * L64, L64, Ws + 32 * ni, LDK);
+      }
+    }
+    __syncthreads();
+  }
+
+  if (dh0 != nullptr) {
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+      const int tt = wave + 4 * i;
+      if (tt < MT * NTC) {
+        const int mi = tt % MT, ni = tt / MT;
+        const int kcol = 32 * ni + acc_col();
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          dh0[(((int64_t)n * Hv + h) * DK + kcol) * V + v0 + 32 * mi + acc_row(r)] = dS[i][r];
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+template <typename T, int DK, int BV> struct DqkwSmem {
+  static constexpr int LDK = lds_ld<T>(DK), LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
+  static constexpr int SR = BV > 64 ? BV : 64;                              // rows of the state tiles / of Q,K
+  static constexpr int off_do = 0;                                          // later ds
+  static constexpr int off_vp = off_do + 64 * LDV * (int)sizeof(T);         // later ds^T
+  static constexpr int off_dv = off_vp + 64 * LDV * (int)sizeof(T);
+  static constexpr int off_sb = off_dv + 64 * LDV * (int)sizeof(T);         // later Q
+  static constexpr int off_dsb = off_sb + SR * LDK * (int)sizeof(T);        // later K
+  static constexpr int off_row = off_dsb + SR * LDK * (int)sizeof(T);
+  static constexpr int bytes = off_row + (4 * 64 + 8) * 4;
+  static_assert(LDV >= L64, "ds reuses the dO tile");
+};
+
+template <typename T, int DK, int BV>
+__global__ __launch_bounds__(kThreads) void chunk_dqkw_kernel(
+    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ vn, const T* __restrict__ dvn,
+    const T* __restrict__ dO, const T* __restrict__ hbuf, const T* __restrict__ dhbuf, const float* __restrict__ G,
+    T* __restrict__ dqh, T* __restrict__ dkh, T* __restrict__ dwb, float* __restrict__ dG,
+    const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V,
+    float scale) {
+  using SM = DqkwSmem<T, DK, BV>;
+  constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64;
+  constexpr int NQ = (2 * (DK / 32) + 3) / 4;
+  T* dOs = reinterpret_cast<T*>(gdn_smem + SM::off_do);
+  T* Vps = reinterpret_cast<T*>(gdn_smem + SM::off_vp);
+  T* dVs = reinterpret_cast<T*>(gdn_smem + SM::off_dv);
+  T* Sb = reinterpret_cast<T*>(gdn_smem + SM::off_sb);
+  T* dSb = reinterpret_cast<T*>(gdn_smem + SM::off_dsb);
+  float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_row);
+  float* rq = Gs + 64;     // <q_i, dQ_i>
+  float* rk = rq + 64;     // <k_i, dK1_i>
+  float* rki = rk + 64;    // <k_i, dK_inter_i>
+  float* wsum = rki + 64;  // per-wave partials of <S, dS'>
+  T* dsm = dOs;
+  T* dsT = Vps;
+  T* Qs = Sb;
+  T* Ks = dSb;
+
+  const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
+  if (s.nvalid <= 0) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int h = blockIdx.y, hq = h / (Hv / Hqk), nvalid = s.nvalid;
+  const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk;
+  const int64_t hoff = ((int64_t)blockIdx.x * Hv + h) * V * DK;
+
+  if (tid < 64) {
+    Gs[tid] = G[(tok0 + imin(tid, nvalid - 1)) * Hv + h];
+    rq[tid] = 0.f; rk[tid] = 0.f; rki[tid] = 0.f;
+  }
+
+  f32x16 ds = acc_zero(), dQi[NQ], dKi[NQ], dWa[NQ];
+#pragma unroll
+  for (int i = 0; i < NQ; ++i) { dQi[i] = acc_zero(); dKi[i] = acc_zero(); dWa[i] = acc_zero(); }
+  float sds = 0.f;
+  const int ti = wave >> 1, tj = wave & 1;
+
+  for (int vb = 0; vb < V / BV; ++vb) {
+    const int v0 = vb * BV;
+    if (vb > 0) __syncthreads();
+    load_tile<T, BV>(dOs, LDV, dO + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
+    load_tile<T, BV>(Vps, LDV, vn + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
+    load_tile<T, BV>(dVs, LDV, dvn + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
+    load_tile<T, DK, BV>(Sb, LDK, hbuf + hoff + (int64_t)v0 * DK, (int64_t)DK, BV, tid);
+    load_tile<T, DK, BV>(dSb, LDK, dhbuf + hoff + (int64_t)v0 * DK, (int64_t)DK, BV, tid);
+    __syncthreads();
+    for (int e = tid; e < BV * DK; e += kThreads) {
+      const int r = e / DK, c = e % DK;
+      sds += Elem<T>::to_f(Sb[r * LDK + c]) * Elem<T>::to_f(dSb[r * LDK + c]);
+    }
+    if (tj <= ti) mma32<T, BV, true, true>(ds, dOs + 32 * ti * LDV, LDV, Vps + 32 * tj * LDV, LDV);
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) {
+      const int tt = wave + 4 * i;
+      if (tt < 2 * (DK / 32)) {
+        const int ri = tt & 1, cj = tt >> 1;
+        mma32<T, BV, true, false>(dQi[i], dOs + 32 * ri * LDV, LDV, Sb + 32 * cj, LDK);
+        mma32<T, BV, true, false>(dKi[i], Vps + 32 * ri * LDV, LDV, dSb + 32 * cj, LDK);
+        mma32<T, BV, true, false>(dWa[i], dVs + 32 * ri * LDV, LDV, Sb + 32 * cj, LDK);
+      }
+    }
+  }
+  sds = wave_sum(sds);
+  if (lane == 0) wsum[wave] = sds;
+  __syncthreads();   // all tiles consumed; their buffers are reused below
+
+  load_tile<T, DK>(Qs, LDK, q + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
+  load_tile<T, DK>(Ks, LDK, k + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
+  {
+    const int j = 32 * tj + acc_col();
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int i = 32 * ti + acc_row(r);
+      const float val = (i >= j) ? scale * ds[r] * __expf(Gs[i] - Gs[j]) : 0.f;
+      dsm[i * L64 + j] = Elem<T>::from_f(val);
+      dsT[j * L64 + i] = Elem<T>::from_f(val);
+    }
+  }
+  __syncthreads();
+  const float glast = Gs[63];
+  T* dqg = dqh + (tok0 * Hv + h) * DK;
+  T* dkg = dkh + (tok0 * Hv + h) * DK;
+  T* dwg = dwb + (tok0 * Hv + h) * DK;
+#pragma unroll
+  for (int i = 0; i < NQ; ++i) {
+    const int tt = wave + 4 * i;
+    if (tt < 2 * (DK / 32)) {
+      const int ri = tt & 1, cj = tt >> 1;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float gi = Gs[32 * ri + acc_row(r)];
+        dQi[i][r] *= scale * __expf(gi);
+        dKi[i][r] *= __expf(glast - gi);
+        dWa[i][r] = -dWa[i][r];
+      }
+      acc_rowdot_add<T>(dKi[i], Ks, LDK, 32 * ri, 32 * cj, rki, 1.f);   // still only the inter-chunk part
+      mma32<T, 64, true, false>(dQi[i], dsm + 32 * ri * L64, L64, Ks + 32 * cj, LDK);
+      mma32<T, 64, true, false>(dKi[i], dsT + 32 * ri * L64, L64, Qs + 32 * cj, LDK);
+      acc_rowdot_add<T>(dQi[i], Qs, LDK, 32 * ri, 32 * cj, rq, 1.f);
+      acc_rowdot_add<T>(dKi[i], Ks, LDK, 32 * ri, 32 * cj, rk, 1.f);
+      acc_to_global(dQi[i], dqg, (int64_t)Hv * DK, 32 * ri, 32 * cj, nvalid);
+      acc_to_global(dKi[i], dkg, (int64_t)Hv * DK, 32 * ri, 32 * cj, nvalid);
+      acc_to_global(dWa[i], dwg, (int64_t)Hv * DK, 32 * ri, 32 * cj, nvalid);
+    }
+  }
+  __syncthreads();
+  if (wave == 0) {
+    float val = rq[lane] - rk[lane];
+    const float tot = wave_sum(rki[lane]);
+    if (lane == nvalid - 1) val += __expf(glast) * (wsum[0] + wsum[1] + wsum[2] + wsum[3]) + tot;
+    if (lane < nvalid) dG[(tok0 + lane) * Hv + h] = val;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+template <typename T, int DK, int BV> struct WySmem {
+  static constexpr int LDK = lds_ld<T>(DK), LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
+  static constexpr int off_tm = 0;
+  static constexpr int off_ks = off_tm + 64 * L64 * (int)sizeof(T);
+  static constexpr int off_dw = off_ks + 64 * LDK * (int)sizeof(T);
+  static constexpr int off_vs = off_dw + 64 * LDK * (int)sizeof(T);          // later (dM . beta)^T
+  static constexpr int off_du = off_vs + 64 * LDV * (int)sizeof(T);
+  static constexpr int off_da = off_du + 64 * LDV * (int)sizeof(T);          // dTm, later dM
+  static constexpr int off_xt = off_da + 64 * L64 * (int)sizeof(T);
+  static constexpr int off_row = off_xt + 64 * L64 * (int)sizeof(T);
+  static constexpr int bytes = off_row + 5 * 64 * 4;
+  static_assert(LDV >= L64, "dM^T reuses the V tile");
+};
+
+template <typename T, int DK, int BV>
+__global__ __launch_bounds__(kThreads) void chunk_wy_bwd_kernel(
+    const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ beta, const float* __restrict__ G,
+    const T* __restrict__ Ai, const T* __restrict__ dwb, const T* __restrict__ dvn, T* dkh, const float* dG1,
+    T* __restrict__ dv_out, float* __restrict__ dbeta, float* __restrict__ dg, const int64_t* __restrict__ cu,
+    const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V) {
+  using SM = WySmem<T, DK, BV>;
+  constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64;
+  constexpr int NQ = (2 * (DK / 32) + 3) / 4, MT = BV / 32, NR = (2 * MT + 3) / 4;
+  T* Tm = reinterpret_cast<T*>(gdn_smem + SM::off_tm);
+  T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
+  T* dWs = reinterpret_cast<T*>(gdn_smem + SM::off_dw);
+  T* Vs = reinterpret_cast<T*>(gdn_smem + SM::off_vs);
+  T* dUs = reinterpret_cast<T*>(gdn_smem + SM::off_du);
+  T* dAs = reinterpret_cast<T*>(gdn_smem + SM::off_da);
+  T* XT = reinterpret_cast<T*>(gdn_smem + SM::off_xt);
+  float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_row);
+  float* bs = Gs + 64;
+  float* rb = bs + 64;     // dbeta
+  float* rg = rb + 64;     // dG2
+  float* egs = rg + 64;    // e^G
+  T* dMs = dAs;
+  T* dMTb = Vs;
+
+  const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
+  if (s.nvalid <= 0) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int h = blockIdx.y, hq = h / (Hv / Hqk), nvalid = s.nvalid;
+  const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk;
+  const int ti = wave >> 1, tj = wave & 1;
+
+  if (tid < 64) {
+    const float gv = G[(tok0 + imin(tid, nvalid - 1)) * Hv + h];
+    Gs[tid] = gv;
+    egs[tid] = __expf(gv);
+    bs[tid] = tid < nvalid ? beta[(tok0 + tid) * Hv + h] : 0.f;
+    rb[tid] = 0.f; rg[tid] = 0.f;
+  }
+  load_tile<T, 64>(Tm, L64, Ai + (tok0 * Hv + h) * 64, (int64_t)Hv * 64, nvalid, tid);
+  load_tile<T, DK>(Ks, LDK, k + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
+  load_tile<T, DK>(dWs, LDK, dwb + (tok0 * Hv + h) * DK, (int64_t)Hv * DK, nvalid, tid);
+  __syncthreads();
+
+  // P = Tm^T dW  ->  dK2 = P beta e^G,  t1 = e^G <P, k>
+  f32x16 dK[NQ];
+#pragma unroll
+  for (int i = 0; i < NQ; ++i) {
+    const int tt = wave + 4 * i;
+    dK[i] = acc_zero();
+    if (tt < 2 * (DK / 32)) {
+      const int ri = tt & 1, cj = tt >> 1;
+      mma32<T, 64, false, false>(dK[i], Tm + 32 * ri, L64, dWs + 32 * cj, LDK);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dK[i][r] *= egs[32 * ri + acc_row(r)];   // now e^G P
+      acc_rowdot_add<T>(dK[i], Ks, LDK, 32 * ri, 32 * cj, rb, 1.f);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dK[i][r] *= bs[32 * ri + acc_row(r)];    // beta e^G P
+      acc_rowdot_add<T>(dK[i], Ks, LDK, 32 * ri, 32 * cj, rg, 1.f);
+    }
+  }
+  // dTm pieces: a1 = dW K^T, a2 = dU V^T (strictly lower tiles only)
+  f32x16 a1 = acc_zero(), a2 = acc_zero();
+  if (tj <= ti) mma32<T, DK, true, true>(a1, dWs + 32 * ti * LDK, LDK, Ks + 32 * tj * LDK, LDK);
+
+  for (int vb = 0; vb < V / BV; ++vb) {
+    const int v0 = vb * BV;
+    if (vb > 0) __syncthreads();
+    load_tile<T, BV>(Vs, LDV, v + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
+    load_tile<T, BV>(dUs, LDV, dvn + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
+    __syncthreads();
+    T* dvg = dv_out + (tok0 * Hv + h) * V + v0;
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      const int tt = wave + 4 * i;
+      if (tt < 2 * MT) {
+        const int ri = tt & 1, cj = tt >> 1;
+        f32x16 R = acc_zero();
+        mma32<T, 64, false, false>(R, Tm + 32 * ri, L64, dUs + 32 * cj, LDV);
+        acc_rowdot_add<T>(R, Vs, LDV, 32 * ri, 32 * cj, rb, 1.f);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) R[r] *= bs[32 * ri + acc_row(r)];
+        acc_to_global(R, dvg, (int64_t)Hv * V, 32 * ri, 32 * cj, nvalid);
+      }
+    }
+    if (tj <= ti) mma32<T, BV, true, true>(a2, dUs + 32 * ti * LDV, LDV, Vs + 32 * tj * LDV, LDV);
+  }
+  {  // dTm[i][j] = beta_j (e^{G_j} a1 + a2), i > j
+    const int j = 32 * tj + acc_col();
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int i = 32 * ti + acc_row(r);
+      dAs[i * L64 + j] = Elem<T>::from_f(i > j ? bs[j] * (egs[j] * a1[r] + a2[r]) : 0.f);
+    }
+  }
+  __syncthreads();
+  {  // X = dTm Tm^T, stored transposed
+    f32x16 x = acc_zero();
+    mma32<T, 64, true, true>(x, dAs + 32 * ti * L64, L64, Tm + 32 * tj * L64, L64);
+    acc_to_lds_t(x, XT, L64, 32 * ti, 32 * tj);
+  }
+  __syncthreads();
+  {  // dM = -(Tm^T X) . Gam, strictly lower;  dMs[i][j] = dM,  dMTb[j][i] = beta_i dM
+    f32x16 y = acc_zero();
+    mma32<T, 64, false, true>(y, Tm + 32 * ti, L64, XT + 32 * tj * L64, L64);
+    const int j = 32 * tj + acc_col();
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int i = 32 * ti + acc_row(r);
+      const float val = i > j ? -y[r] * __expf(Gs[i] - Gs[j]) : 0.f;
+      dMs[i * L64 + j] = Elem<T>::from_f(val);
+      dMTb[j * L64 + i] = Elem<T>::from_f(val * bs[i]);
+    }
+  }
+  __syncthreads();
+  T* dkg = dkh + (tok0 * Hv + h) * DK;
+#pragma unroll
+  for (int i = 0; i < NQ; ++i) {
+    const int tt = wave + 4 * i;
+    if (tt < 2 * (DK / 32)) {
+      const int ri = tt & 1, cj = tt >> 1;
+      f32x16 E = acc_zero(), Fm = acc_zero();
+      mma32<T, 64, true, false>(E, dMs + 32 * ri * L64, L64, Ks + 32 * cj, LDK);
+      mma32<T, 64, true, false>(Fm, dMTb + 32 * ri * L64, L64, Ks + 32 * cj, LDK);
+      acc_rowdot_add<T>(E, Ks, LDK, 32 * ri, 32 * cj, rb, 1.f);
+      acc_rowdot_add<T>(Fm, Ks, LDK, 32 * ri, 32 * cj, rg, -1.f);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) E[r] *= bs[32 * ri + acc_row(r)];
+      acc_rowdot_add<T>(E, Ks, LDK, 32 * ri, 32 * cj, rg, 1.f);
+      const f32x16 k1 = acc_from_global(dkg, (int64_t)Hv * DK, 32 * ri, 32 * cj, nvalid);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dK[i][r] += E[r] + Fm[r] + k1[r];
+      acc_to_global(dK[i], dkg, (int64_t)Hv * DK, 32 * ri, 32 * cj, nvalid);
+    }
+  }
+  __syncthreads();
+  if (wave == 0) {   // d(cumulative G) -> d(g): suffix sum inside the chunk
+    float x = rg[lane] + (lane < nvalid ? dG1[(tok0 + lane) * Hv + h] : 0.f);
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const float t = __shfl_down(x, d);
+      if (lane + d < 64) x += t;
+    }
+    if (lane < nvalid) {
+      dg[(tok0 + lane) * Hv + h] = x;
+      dbeta[(tok0 + lane) * Hv + h] = rb[lane];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// dq/dk: sum over the value heads of a group, then back through the l2 norm if it was applied.
+// ---------------------------------------------------------------------------------------------
+template <typename T, int DK>
+__global__ void qk_grad_finalize_kernel(const T* __restrict__ dqh, const T* __restrict__ dkh, const T* __restrict__ q,
+                                        const T* __restrict__ k, T* __restrict__ dq, T* __restrict__ dk, int64_t rows,
+                                        int Hqk, int Hv, int l2norm) {
+  constexpr int V = Elem<T>::kVec, LPR = DK / V;
+  const T* src = blockIdx.y == 0 ? dqh : dkh;
+  const T* x = blockIdx.y == 0 ? q : k;
+  T* dst = blockIdx.y == 0 ? dq : dk;
+  const int64_t row = (int64_t)blockIdx.x * (kThreads / LPR) + threadIdx.x / LPR;   // (token, qk head)
+  const int c = threadIdx.x % LPR;
+  const bool ok = row < rows;
+  const int grp = Hv / Hqk;
+  const int64_t tok = ok ? row / Hqk : 0;
+  const int hq = ok ? (int)(row % Hqk) : 0;
+  float acc[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) acc[e] = 0.f;
+  if (ok) {
+    for (int gi = 0; gi < grp; ++gi) {
+      const Vec16<T> t = ld16(src + ((tok * Hv + hq * grp + gi) * DK) + c * V);
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] += t.get(e);
+    }
+  }
+  if (l2norm) {   // uniform branch: every lane takes part in the shuffles
+    Vec16<T> xv = ok ? ld16(x + row * DK + c * V) : zero16<T>();
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < V; ++e) { const float f = xv.get(e); ss += f * f; }
+#pragma unroll
+    for (int m = 1; m < LPR; m <<= 1) ss += __shfl_xor(ss, m);
+    const float rstd = rsqrtf(ss + 1e-6f);
+    float dot = 0.f;
+#pragma unroll
+    for (int e = 0; e < V; ++e) dot += acc[e] * xv.get(e) * rstd;
+#pragma unroll
+    for (int m = 1; m < LPR; m <<= 1) dot += __shfl_xor(dot, m);
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc[e] = (acc[e] - dot * xv.get(e) * rstd) * rstd;
+  }
+  if (ok) {
+    Vec16<T> o = zero16<T>();
+#pragma unroll
+    for (int e = 0; e < V; ++e) o.set(e, acc[e]);
+    st16(dst + row * DK + c * V, o);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+template <typename K> static int set_lds_b(K kernel, int bytes) {
+  return (int)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  bytes);
+}
+
+template <typename T, int DK, int BVL, int BVS, int BVQ, int BVW>
+static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const void* q, const void* k, const void* v,
+                            const float* beta, const int64_t* cu, const void* dO, const float* dht, void* dq, void* dk,
+                            void* dv, float* dg, float* dbeta, float* dh0, unsigned char* ws, float scale, int l2norm,
+                            hipStream_t st) {
+  const int64_t tok = d.tokens();
+  const int nc = (int)d.max_chunks();
+  const int* chunk_offsets = reinterpret_cast<const int*>(ws + L.chunk_offsets);
+  const T* qq = l2norm ? reinterpret_cast<const T*>(ws + L.qn) : (const T*)q;
+  const T* kk = l2norm ? reinterpret_cast<const T*>(ws + L.kn) : (const T*)k;
+  const float* G = reinterpret_cast<const float*>(ws + L.G);
+  const T* Ai = reinterpret_cast<const T*>(ws + L.Ai);
+  const T* W = reinterpret_cast<const T*>(ws + L.W);
+  const T* VN = reinterpret_cast<const T*>(ws + L.VN);
+  const T* H = reinterpret_cast<const T*>(ws + L.H);
+  T* DV = reinterpret_cast<T*>(ws + L.DV);
+  T* DH = reinterpret_cast<T*>(ws + L.DH);
+  T* DW = reinterpret_cast<T*>(ws + L.DW);
+  T* DQH = reinterpret_cast<T*>(ws + L.DQH);
+  T* DKH = reinterpret_cast<T*>(ws + L.DKH);
+  float* DG = reinterpret_cast<float*>(ws + L.DG);
+  {
+    auto kern = chunk_dv_local_kernel<T, DK, BVL>;
+    constexpr int smem = DvLocalSmem<T, DK, BVL>::bytes;
+    if (int e = set_lds_b(kern, smem)) return e;
+    hipLaunchKernelGGL(kern, dim3(nc, d.Hv, d.V / BVL), dim3(kThreads), smem, st, qq, kk, (const T*)dO, G, DV, cu,
+                       chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale);
+  }
+  {
+    auto kern = chunk_state_bwd_kernel<T, DK, BVS>;
+    constexpr int smem = StateBwdSmem<T, DK, BVS>::bytes;
+    if (int e = set_lds_b(kern, smem)) return e;
+    hipLaunchKernelGGL(kern, dim3(d.N * d.Hv, d.V / BVS), dim3(kThreads), smem, st, qq, kk, W, (const T*)dO, DV, G,
+                       dht, dh0, DH, cu, chunk_offsets, d.T, d.Hqk, d.Hv, d.V, scale);
+  }
+  {
+    auto kern = chunk_dqkw_kernel<T, DK, BVQ>;
+    constexpr int smem = DqkwSmem<T, DK, BVQ>::bytes;
+    if (int e = set_lds_b(kern, smem)) return e;
+    hipLaunchKernelGGL(kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, VN, (const T*)DV, (const T*)dO, H,
+                       (const T*)DH, G, DQH, DKH, DW, DG, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale);
+  }
+  {
+    auto kern = chunk_wy_bwd_kernel<T, DK, BVW>;
+    constexpr int smem = WySmem<T, DK, BVW>::bytes;
+    if (int e = set_lds_b(kern, smem)) return e;
+    hipLaunchKernelGGL(kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, kk, (const T*)v, beta, G, Ai, (const T*)DW,
+                       (const T*)DV, DKH, (const float*)DG, (T*)dv, dbeta, dg, cu, chunk_offsets, d.T, d.N, d.Hqk,
+                       d.Hv, d.V);
+  }
+  {
+    constexpr int LPR = DK / Elem<T>::kVec;
+    const int64_t rows = tok * d.Hqk;
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(qk_grad_finalize_kernel<T, DK>),
+                       dim3((unsigned)((rows + kThreads / LPR - 1) / (kThreads / LPR)), 2), dim3(kThreads), 0, st,
+                       (const T*)DQH, (const T*)DKH, (const T*)q, (const T*)k, (T*)dq, (T*)dk, rows, d.Hqk, d.Hv,
+                       l2norm);
+  }
+  return (int)hipGetLastError();
+}
+
+}  // namespace gdn
+
 extern "C" int gdn_chunk_bwd(const void* q, const void* k, const void* v, const float* g, const float* beta,
-                  const float* initial_state, const int64_t* cu_seqlens, const void* d_o,
-                  const float* d_final_state, void* dq, void* dk, void* dv, float* dg, float* dbeta,
-                  float* d_initial_state, void* workspace, int64_t workspace_bytes, int B, int T, int N, int Hqk,
-                  int Hv, int K, int V, float scale, int use_qk_l2norm, int dtype, void* stream) { return -100; }
+                             const float* initial_state, const int64_t* cu_seqlens, const void* d_o,
+                             const float* d_final_state, void* dq, void* dk, void* dv, float* dg, float* dbeta,
+                             float* d_initial_state, void* workspace, int64_t workspace_bytes, int B, int T, int N,
+                             int Hqk, int Hv, int K, int V, float scale, int use_qk_l2norm, int dtype, void* stream) {
+  using namespace gdn;
+  (void)g; (void)initial_state;   // their effect is already in the workspace (G, per-chunk states)
+  if (!q || !k || !v || !beta || !d_o || !dq || !dk || !dv || !dg || !dbeta || !workspace) return -1;
+  ChunkDims d{B, T, N, Hqk, Hv, K, V, cu_seqlens != nullptr};
+  if (int e = chunk_check_dims(d, dtype)) return e;
+  ChunkDims dl = d;
+  dl.varlen = true;
+  const ChunkWorkspace L = chunk_workspace_layout(dl, dtype == 0 ? 4 : 2);
+  if (workspace_bytes < L.total_bytes) return -5;
+  if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
+  unsigned char* ws = static_cast<unsigned char*>(workspace);
+  hipStream_t st = (hipStream_t)stream;
+#define GDN_BWD(T_, DK_, BVL_, BVS_, BVQ_, BVW_)                                                                   \
+  return chunk_bwd_launch<T_, DK_, BVL_, BVS_, BVQ_, BVW_>(d, L, q, k, v, beta, cu_seqlens, d_o, d_final_state, dq, \
+                                                            dk, dv, dg, dbeta, d_initial_state, ws, scale,         \
+                                                            use_qk_l2norm, st)
+  if (dtype == 1) {
+    if (K == 128) GDN_BWD(bf16_t, 128, 64, 64, 64, 64);
+    GDN_BWD(bf16_t, 64, 64, 64, 64, 64);
+  } else {
+    if (K == 128) GDN_BWD(float, 128, 64, 32, 64, 64);
+    GDN_BWD(float, 64, 64, 32, 64, 64);
+  }
+#undef GDN_BWD
+}

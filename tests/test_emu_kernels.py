@@ -37,6 +37,21 @@ def test_chunk_forward(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu):
     P.check_chunk(ops, "cpu", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu, wrap=guarded, h0_std=0.1)
 
 
+@pytest.mark.parametrize("dtype,B,T,Hqk,Hv,K,V,l2,cu", [
+    (F32, 1, 130, 1, 2, 64, 64, True, None),
+    (F32, 2, 100, 2, 4, 128, 128, True, None),
+    (BF, 1, 200, 1, 2, 128, 128, True, None),
+    (BF, 1, 140, 2, 2, 64, 64, False, [0, 5, 70, 71, 140]),
+    (F32, 1, 96, 1, 1, 128, 192, True, [0, 1, 38, 96]),
+])
+def test_chunk_backward(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu):
+    P.check_chunk(ops, "cpu", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu, backward=True, wrap=guarded, h0_std=0.1)
+
+
+def test_chunk_backward_without_initial_state(ops):
+    P.check_chunk(ops, "cpu", 1, 70, 1, 1, 64, 64, F32, backward=True, with_h0=False, wrap=guarded)
+
+
 @pytest.mark.parametrize("dtype,B,T,D,W,cu", [
     (F32, 2, 37, 16, 4, None), (BF, 1, 300, 32, 4, [0, 1, 3, 130, 131, 300]), (F32, 1, 9, 8, 3, [0, 2, 9]),
     (torch.float16, 2, 5, 8, 2, None), (F32, 3, 2, 8, 4, None), (F32, 1, 600, 8, 4, [0, 255, 257, 600]),

@@ -66,6 +66,16 @@ def test_chunk_forward(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu):
     P.check_chunk(ops, "cuda", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu)
 
 
+@pytest.mark.parametrize("dtype,B,T,Hqk,Hv,K,V,l2,cu", CHUNK_CASES)
+def test_chunk_backward(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu):
+    print(f"chunk bwd {dtype} B{B} T{T} Hqk{Hqk} Hv{Hv} K{K} V{V} l2={l2} varlen={cu is not None}", flush=True)
+    P.check_chunk(ops, "cuda", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu, backward=True)
+
+
+def test_chunk_backward_without_initial_state(ops):
+    P.check_chunk(ops, "cuda", 1, 200, 2, 2, 128, 128, BF, backward=True, with_h0=False)
+
+
 @pytest.mark.parametrize("dtype,B,T,D,W,cu", [
     (F32, 2, 37, 16, 4, None), (BF, 1, 300, 64, 4, [0, 1, 3, 130, 131, 300]), (F32, 1, 9, 8, 3, [0, 2, 9]),
     (torch.float16, 2, 5, 8, 2, None), (F32, 3, 2, 8, 4, None), (BF, 2, 1024, 512, 4, None),
