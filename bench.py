@@ -1,0 +1,211 @@
+#!/usr/bin/env python3
+"""Benchmark of the GDN operator path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one chunked gated-delta-rule forward + backward over the configuration the metric is quoted on
+(BASELINE.json configs[1]: B=2, T=8192, H_qk=16, H_v=32, d_k=d_v=128, bf16, in-kernel q/k L2 norm, N(0,0.02)
+initial state, upstream grad ~ N(0,1)); inputs are synthetic and already resident in HBM.  Prints ONE JSON line.
+
+  value        tokens/s of fwd+bwd (B*T / step time), measured without per-kernel instrumentation
+  roofline     the kernel with the largest share of the step: its algorithmic matmul FLOP per launch divided by
+               its mean duration, taken live with HIP events on the launch stream in a second, instrumented
+               pass over the same K steps; peak = MI355X dense bf16 MFMA (2.5 PFLOP/s)
+  cpu_baseline the CPU oracle (PyTorch fp32 restatement of the reference's torch path, autograd backward) timed on
+               this box's host cores on a bounded sample of the same workload
+  aux          the whole path against the MFMA peak with the reference's FLOP formula, the per-kernel split,
+               and the HBM-bound siblings (batch-256 decode, the packed conv1d) with their achieved GB/s
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "mindspeed-mm_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+CFG = dict(B=2, T=8192, Hqk=16, Hv=32, K=128, V=128, C=64)
+
+
+def ref_formula_flops(tokens, Hv, K, V, C=64):
+    """fwd+bwd FLOP of the reference's own counter (mindspeed_mm/fsdp/tools/flops_tool/flops_qwen3_5.py:170-204)."""
+    return 3 * 2 * tokens * Hv * (3 * V * C + 2 * K * C + 3 * K * V)
+
+
+def kernel_matmul_flops(K, V, C=64):
+    """Matmul FLOP each kernel performs per (chunk, value head): 2*M*N*K summed over its contractions."""
+    g = lambda m, n, k: 2 * m * n * k
+    return {
+        "chunk_prep_kernel": g(C, C, K) + g(C, K, C) + g(C, V, C),
+        "chunk_state_kernel": g(C, V, K) + g(V, K, C),
+        "chunk_out_kernel": g(C, C, K) + g(C, V, K) + g(C, V, C),
+        "chunk_dv_local_kernel": g(C, C, K) + g(C, V, C),
+        "chunk_state_bwd_kernel": g(C, V, K) + 2 * g(V, K, C),
+        "chunk_dqkw_kernel": g(C, C, V) + 3 * g(C, K, V) + 2 * g(C, K, C),
+        "chunk_wy_bwd_kernel": g(C, K, C) + g(C, C, K) + g(C, V, C) + g(C, C, V) + 2 * g(C, C, C) + 2 * g(C, K, C),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side oracle timing")
+    ap.add_argument("--no-aux", action="store_true", help="skip the decode / conv1d side measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the operator path has no collective and this build runs on a single "
+              "MI355X; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (there is no host execution path for the operators)", file=sys.stderr)
+        sys.exit(1)
+    from mindspeed_mm_amd import _lib
+    from mindspeed_mm_amd.inputs import gdn_inputs, packed_lengths
+    from mindspeed_mm_amd.ops import _default_ops
+
+    ops = _default_ops()
+    lib = ops.lib
+    dev = torch.device("cuda:0")
+    c = CFG
+    tokens = c["B"] * c["T"]
+    x = gdn_inputs(c["B"], c["T"], c["Hqk"], c["Hv"], c["K"], c["V"], torch.bfloat16, seed=0)
+    d = {n: t.to(dev) for n, t in x.items()}
+    leaves = [d[n].requires_grad_(True) for n in ("q", "k", "v", "g", "beta", "h0")]
+
+    def step():
+        o, ht = ops.chunk_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], initial_state=d["h0"],
+                                           output_final_state=True, use_qk_l2norm_in_kernel=True)
+        return torch.autograd.grad([o], leaves, [d["do"]])
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    value = tokens / (ms_per_step * 1e-3)
+
+    # ---- instrumented pass: per-kernel durations from HIP events on the launch stream ----
+    lib.gdn_profile_enable(1)
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    timings = _lib.kernel_timings(lib)
+    lib.gdn_profile_enable(0)
+    nchunk_heads = c["B"] * (c["T"] // c["C"]) * c["Hv"]
+    per_kernel = {}
+    total_kernel_ms = sum(ms for ms, _ in timings.values()) / args.steps
+    flops = kernel_matmul_flops(c["K"], c["V"])
+    for name, (ms, cnt) in timings.items():
+        avg = ms / cnt
+        per_kernel[name] = {"avg_ms": round(avg, 4), "share": round(ms / args.steps / total_kernel_ms, 3)}
+        if name in flops:
+            per_kernel[name]["tflops"] = round(flops[name] * nchunk_heads / (avg * 1e-3) / 1e12, 1)
+    dom = max((n for n in per_kernel if n in flops), key=lambda n: per_kernel[n]["avg_ms"])
+    dom_tflops = flops[dom] * nchunk_heads / (per_kernel[dom]["avg_ms"] * 1e-3) / 1e12
+    roofline = {"kernel": dom, "bound": "mfma", "achieved": round(dom_tflops, 2), "peak": PEAK_BF16_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(dom_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None}
+
+    path_tflops = ref_formula_flops(tokens, c["Hv"], c["K"], c["V"]) / (ms_per_step * 1e-3) / 1e12
+    aux = {"path_tflops_ref_formula": round(path_tflops, 2),
+           "path_frac_of_bf16_mfma_peak": round(path_tflops / PEAK_BF16_TFLOPS, 4),
+           "kernel_ms_sum": round(total_kernel_ms, 3), "kernels": per_kernel}
+
+    if not args.no_aux:
+        # ---- decode: batch 256, 64 consecutive steps, state updated in place (BASELINE.json configs[3]) ----
+        B3 = 256
+        y = gdn_inputs(B3, 64, c["Hqk"], c["Hv"], c["K"], c["V"], torch.bfloat16, seed=3)
+        e = {n: t.to(dev) for n, t in y.items()}
+        state = e["h0"].clone()
+        tok = [{n: e[n][:, t:t + 1].contiguous() for n in ("q", "k", "v", "g", "beta")} for t in range(64)]
+
+        def decode64():
+            for t in tok:
+                ops.fused_recurrent_gated_delta_rule(t["q"], t["k"], t["v"], t["g"], t["beta"], initial_state=state,
+                                                     output_final_state=True, use_qk_l2norm_in_kernel=True,
+                                                     inplace_state=True)
+        decode64()
+        lib.gdn_profile_enable(1)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        decode64()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) / 64
+        tm = _lib.kernel_timings(lib)["recurrent_kernel"]
+        lib.gdn_profile_enable(0)
+        kern_s = tm[0] / tm[1] * 1e-3
+        # per step: fp32 state in + out, bf16 q,k,v,o, fp32 g,beta
+        step_bytes = 2 * B3 * c["Hv"] * c["K"] * c["V"] * 4 + B3 * (2 * c["Hqk"] * c["K"] + 2 * c["Hv"] * c["V"]) * 2 \
+            + 2 * B3 * c["Hv"] * 4
+        aux["decode_b256"] = {"kernel_us": round(kern_s * 1e6, 1), "GBps": round(step_bytes / kern_s / 1e9, 1),
+                              "frac_of_hbm_peak": round(step_bytes / kern_s / 1e9 / PEAK_HBM_GBS, 4),
+                              "tokens_per_s_wall": round(B3 / wall, 1), "bytes_per_step": step_bytes}
+        del e, y, state, tok
+        # ---- packed causal conv1d fwd+bwd (BASELINE.json configs[2]: 32768 tokens, D=8192, W=4, SiLU) ----
+        cu = torch.tensor(packed_lengths(), dtype=torch.int64, device=dev)
+        D = 2 * c["Hqk"] * c["K"] + c["Hv"] * c["V"]
+        gen = torch.Generator().manual_seed(2)
+        xx = torch.randn(1, 32768, D, generator=gen).to(dev, torch.bfloat16).requires_grad_(True)
+        ww = (torch.randn(4, D, generator=gen) / 2).to(dev, torch.bfloat16).requires_grad_(True)
+        dy = torch.randn(1, 32768, D, generator=gen).to(dev, torch.bfloat16)
+
+        def conv_step():
+            yy, _ = ops.causal_conv1d(xx, ww, None, None, None, "silu", cu, False)
+            torch.autograd.grad([yy], [xx, ww], [dy])
+        conv_step()
+        lib.gdn_profile_enable(1)
+        for _ in range(5):
+            conv_step()
+        torch.cuda.synchronize()
+        tm = _lib.kernel_timings(lib)
+        lib.gdn_profile_enable(0)
+        nb = xx.numel() * 2
+        f_s = tm["conv1d_fwd_kernel"][0] / tm["conv1d_fwd_kernel"][1] * 1e-3
+        b_s = tm["conv1d_bwd_kernel"][0] / tm["conv1d_bwd_kernel"][1] * 1e-3
+        aux["conv1d_packed"] = {"fwd_ms": round(f_s * 1e3, 3), "fwd_GBps": round(2 * nb / f_s / 1e9, 1),
+                                "bwd_ms": round(b_s * 1e3, 3), "bwd_GBps": round(3 * nb / b_s / 1e9, 1)}
+        del xx, ww, dy
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import gdn_oracle as O
+        Ts = 8192
+        sample = {n: x[n][:1, :Ts] for n in ("q", "k", "v", "g", "beta", "do")}
+        L = {n: sample[n].float().requires_grad_(True) for n in ("q", "k", "v", "g", "beta")}
+        h0 = x["h0"][:1].clone().requires_grad_(True)
+        t0 = time.perf_counter()
+        o, _ = O.chunk_gated_delta_rule_ref(L["q"], L["k"], L["v"], L["g"], L["beta"], initial_state=h0,
+                                            output_final_state=True, use_qk_l2norm_in_kernel=True)
+        torch.autograd.grad([o], list(L.values()) + [h0], [sample["do"].float()])
+        dt = time.perf_counter() - t0
+        cpu = {"value": round(Ts / dt, 1), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+               "sample": f"one of the two batch rows at full length: B=1, T={Ts}, H_qk=16, H_v=32, d=128, fp32, "
+                         f"fwd+bwd once ({dt:.1f} s)"}
+
+    out = {
+        "metric": "GDN chunk fwd+bwd tokens/sec (H=32,d=128,bf16) on 1 GPU",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "GDN chunk forward+backward, B=2 T=8192 H_qk=16 H_v=32 d_k=d_v=128 chunk=64, "
+                               "use_qk_l2norm_in_kernel, initial state N(0,0.02), native grouped q/k heads",
+                   "global_batch": c["B"], "seq_len": c["T"], "parallelism": "single GPU"},
+        "roofline": roofline, "cpu_baseline": cpu, "aux": aux,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

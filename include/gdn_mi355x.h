@@ -77,6 +77,16 @@ int gdn_conv1d_bwd(const void* x, const void* dy, const void* weight, const void
 int gdn_conv1d_update(const void* hidden, void* conv_state, const void* weight, const void* bias, void* out, int B,
                       int T, int D, int W, int state_len, int activation, int dtype, void* stream);
 
+/* -------- per-kernel timing ------------------------------------------------------------------------
+ * op-level counterpart of the reference's step profiler (mindspeed_mm/fsdp/tools/profiler.py:32-147).
+ * While enabled, every kernel launch of this library is bracketed by HIP events on its stream (this mode
+ * creates events, i.e. it allocates); gdn_profile_collect waits for them and ADDS, per kernel id
+ * (0 .. gdn_profile_kernel_count()-1), the elapsed milliseconds to total_ms[id] and 1 to launches[id]. */
+int gdn_profile_enable(int on);
+int gdn_profile_kernel_count(void);
+const char* gdn_profile_kernel_name(int id);
+int gdn_profile_collect(double* total_ms, int64_t* launches);
+
 #ifdef __cplusplus
 }
 #endif

@@ -17,6 +17,7 @@
 // the dG row/column sums rewritten as row dot products with dQ/dK so that Q K^T need not be rebuilt.
 #include "gdn_chunk.h"
 #include "gdn_common.h"
+#include "gdn_profile.h"
 
 namespace gdn {
 
@@ -591,35 +592,35 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     auto kern = chunk_dv_local_kernel<T, DK, BVL>;
     constexpr int smem = DvLocalSmem<T, DK, BVL>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
-    hipLaunchKernelGGL(kern, dim3(nc, d.Hv, d.V / BVL), dim3(kThreads), smem, st, qq, kk, (const T*)dO, G, DV, cu,
+    GDN_LAUNCH(kKernDvLocal, st, kern, dim3(nc, d.Hv, d.V / BVL), dim3(kThreads), smem, st, qq, kk, (const T*)dO, G, DV, cu,
                        chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale);
   }
   {
     auto kern = chunk_state_bwd_kernel<T, DK, BVS>;
     constexpr int smem = StateBwdSmem<T, DK, BVS>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
-    hipLaunchKernelGGL(kern, dim3(d.N * d.Hv, d.V / BVS), dim3(kThreads), smem, st, qq, kk, W, (const T*)dO, DV, G,
+    GDN_LAUNCH(kKernStateBwd, st, kern, dim3(d.N * d.Hv, d.V / BVS), dim3(kThreads), smem, st, qq, kk, W, (const T*)dO, DV, G,
                        dht, dh0, DH, cu, chunk_offsets, d.T, d.Hqk, d.Hv, d.V, scale);
   }
   {
     auto kern = chunk_dqkw_kernel<T, DK, BVQ>;
     constexpr int smem = DqkwSmem<T, DK, BVQ>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
-    hipLaunchKernelGGL(kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, VN, (const T*)DV, (const T*)dO, H,
+    GDN_LAUNCH(kKernDqkw, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, VN, (const T*)DV, (const T*)dO, H,
                        (const T*)DH, G, DQH, DKH, DW, DG, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale);
   }
   {
     auto kern = chunk_wy_bwd_kernel<T, DK, BVW>;
     constexpr int smem = WySmem<T, DK, BVW>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
-    hipLaunchKernelGGL(kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, kk, (const T*)v, beta, G, Ai, (const T*)DW,
+    GDN_LAUNCH(kKernWyBwd, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, kk, (const T*)v, beta, G, Ai, (const T*)DW,
                        (const T*)DV, DKH, (const float*)DG, (T*)dv, dbeta, dg, cu, chunk_offsets, d.T, d.N, d.Hqk,
                        d.Hv, d.V);
   }
   {
     constexpr int LPR = DK / Elem<T>::kVec;
     const int64_t rows = tok * d.Hqk;
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(qk_grad_finalize_kernel<T, DK>),
+    GDN_LAUNCH(kKernQkFinalize, st, (qk_grad_finalize_kernel<T, DK>),
                        dim3((unsigned)((rows + kThreads / LPR - 1) / (kThreads / LPR)), 2), dim3(kThreads), 0, st,
                        (const T*)DQH, (const T*)DKH, (const T*)q, (const T*)k, (T*)dq, (T*)dk, rows, d.Hqk, d.Hv,
                        l2norm);

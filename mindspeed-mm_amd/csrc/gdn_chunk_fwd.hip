@@ -13,6 +13,7 @@
 // A ragged last chunk is zero padded in LDS (k = v = beta = g = 0 is exact for this recurrence).
 #include "gdn_chunk.h"
 #include "gdn_common.h"
+#include "gdn_profile.h"
 
 namespace gdn {
 
@@ -484,13 +485,13 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   int* chunk_offsets = reinterpret_cast<int*>(ws + L.chunk_offsets);
   const T* qq = (const T*)q;
   const T* kk = (const T*)k;
-  if (cu != nullptr) hipLaunchKernelGGL(chunk_table_kernel, dim3(1), dim3(kThreads), 0, st, cu, chunk_offsets, d.N);
+  if (cu != nullptr) GDN_LAUNCH(kKernChunkTable, st, chunk_table_kernel, dim3(1), dim3(kThreads), 0, st, cu, chunk_offsets, d.N);
   if (l2norm) {
     constexpr int LPR = DK / Elem<T>::kVec;
     const int64_t rows = tok * d.Hqk;
     T* qn = reinterpret_cast<T*>(ws + L.qn);
     T* kn = reinterpret_cast<T*>(ws + L.kn);
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(l2norm_fwd_kernel<T, DK>),
+    GDN_LAUNCH(kKernL2Norm, st, (l2norm_fwd_kernel<T, DK>),
                        dim3((unsigned)((rows + kThreads / LPR - 1) / (kThreads / LPR)), 2), dim3(kThreads), 0, st, qq,
                        kk, qn, kn, rows);
     qq = qn;
@@ -505,21 +506,21 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     auto kern = chunk_prep_kernel<T, DK, BVP>;
     constexpr int smem = PrepSmem<T, DK, BVP>::bytes;
     if (int e = set_lds(kern, smem)) return e;
-    hipLaunchKernelGGL(kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, kk, (const T*)v, g, beta, cu,
+    GDN_LAUNCH(kKernPrep, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, kk, (const T*)v, g, beta, cu,
                        (const int*)chunk_offsets, G, Ai, W, VN, d.T, d.N, d.Hqk, d.Hv, d.V);
   }
   {
     auto kern = chunk_state_kernel<T, DK, BVS>;
     constexpr int smem = StateSmem<T, DK, BVS>::bytes;
     if (int e = set_lds(kern, smem)) return e;
-    hipLaunchKernelGGL(kern, dim3(d.N * d.Hv, d.V / BVS), dim3(kThreads), smem, st, kk, (const T*)W, VN,
+    GDN_LAUNCH(kKernStateFwd, st, kern, dim3(d.N * d.Hv, d.V / BVS), dim3(kThreads), smem, st, kk, (const T*)W, VN,
                        (const float*)G, h0, ht, H, cu, (const int*)chunk_offsets, d.T, d.Hqk, d.Hv, d.V);
   }
   {
     auto kern = chunk_out_kernel<T, DK, BVO>;
     constexpr int smem = OutSmem<T, DK, BVO>::bytes;
     if (int e = set_lds(kern, smem)) return e;
-    hipLaunchKernelGGL(kern, dim3(nc, d.Hv, d.V / BVO), dim3(kThreads), smem, st, qq, kk, (const T*)VN, (const T*)H,
+    GDN_LAUNCH(kKernOut, st, kern, dim3(nc, d.Hv, d.V / BVO), dim3(kThreads), smem, st, qq, kk, (const T*)VN, (const T*)H,
                        (const float*)G, (T*)o, cu, (const int*)chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale);
   }
   return (int)hipGetLastError();

@@ -10,6 +10,7 @@
 // 4 fp32) and walks a tile of consecutive tokens with the last W inputs in registers, so x is read
 // once; the backward pass recomputes the pre-activation in registers instead of re-reading y.
 #include "gdn_common.h"
+#include "gdn_profile.h"
 
 namespace gdn {
 
@@ -315,7 +316,7 @@ template <typename T> struct ConvLaunch {
       switch (W) {
 #define GDN_CASE(W_)                                                                                              \
   case W_:                                                                                                        \
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(conv1d_fwd_kernel<T, W_>), grid, dim3(kConvThreads), 0, st, (const T*)x,   \
+    GDN_LAUNCH(kKernConvFwd, st, (conv1d_fwd_kernel<T, W_>), grid, dim3(kConvThreads), 0, st, (const T*)x,   \
                        (const T*)weight, (const T*)bias, (const T*)residual, (const T*)init, cu, (T*)y, total,    \
                        T_len, N, D, tile, silu);                                                                  \
     break;
@@ -326,7 +327,7 @@ template <typename T> struct ConvLaunch {
     }
     if (fs != nullptr) {
       const int64_t n = (int64_t)N * D;
-      hipLaunchKernelGGL(HIP_KERNEL_NAME(conv1d_final_state_kernel<T>), dim3((unsigned)((n + 255) / 256)), dim3(256),
+      GDN_LAUNCH(kKernConvState, st, (conv1d_final_state_kernel<T>), dim3((unsigned)((n + 255) / 256)), dim3(256),
                          0, st, (const T*)x, (const T*)init, cu, (T*)fs, T_len, N, D, W);
     }
     return (int)hipGetLastError();
@@ -343,7 +344,7 @@ template <typename T> struct ConvLaunch {
       switch (W) {
 #define GDN_CASE(W_)                                                                                              \
   case W_:                                                                                                        \
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(conv1d_bwd_kernel<T, W_>), grid, dim3(kConvThreads), 0, st, (const T*)x,   \
+    GDN_LAUNCH(kKernConvBwd, st, (conv1d_bwd_kernel<T, W_>), grid, dim3(kConvThreads), 0, st, (const T*)x,   \
                        (const T*)dy, (const T*)weight, (const T*)bias, (const T*)init, (const T*)dht, cu, (T*)dx, \
                        workspace, total, T_len, N, D, tile, silu);                                                \
     break;
@@ -353,11 +354,11 @@ template <typename T> struct ConvLaunch {
       }
     }
     const int64_t nred = (int64_t)(W + 1) * D;
-    hipLaunchKernelGGL(conv1d_reduce_kernel, dim3((unsigned)((nred + 255) / 256)), dim3(256), 0, st, workspace, dw, db,
+    GDN_LAUNCH(kKernConvReduce, st, conv1d_reduce_kernel, dim3((unsigned)((nred + 255) / 256)), dim3(256), 0, st, workspace, dw, db,
                        ntiles, W, D);
     if (dh0 != nullptr) {
       const int64_t n = (int64_t)N * D;
-      hipLaunchKernelGGL(HIP_KERNEL_NAME(conv1d_dh0_kernel<T>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+      GDN_LAUNCH(kKernConvDh0, st, (conv1d_dh0_kernel<T>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
                          (const T*)x, (const T*)dy, (const T*)weight, (const T*)bias, (const T*)init, (const T*)dht,
                          cu, (T*)dh0, T_len, N, D, W, silu);
     }
@@ -366,7 +367,7 @@ template <typename T> struct ConvLaunch {
   static int update(const void* hidden, void* state, const void* weight, const void* bias, void* out, int B,
                     int T_len, int D, int W, int S, int silu, hipStream_t st) {
     const int64_t n = (int64_t)B * D;
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(conv1d_update_kernel<T>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+    GDN_LAUNCH(kKernConvUpdate, st, (conv1d_update_kernel<T>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
                        (const T*)hidden, (T*)state, (const T*)weight, (const T*)bias, (T*)out, B, T_len, D, W, S, silu);
     return (int)hipGetLastError();
   }

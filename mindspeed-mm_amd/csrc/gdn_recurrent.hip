@@ -9,6 +9,7 @@
 // so both contractions are taken in ONE pass over the registers, then the rank-1 update is applied.
 // No MFMA: 6 flop per 8 bytes of state traffic, far below the matrix-core ridge.
 #include "gdn_common.h"
+#include "gdn_profile.h"
 
 namespace gdn {
 
@@ -133,7 +134,7 @@ static int launch_recurrent(const void* q, const void* k, const void* v, const f
                             const float* state_in, float* state_out, void* o, int B, int T_len, int Hqk, int Hv, int K,
                             int V, float scale, int use_l2norm, hipStream_t stream) {
 #define GDN_REC(DK_, BV_)                                                                                      \
-  hipLaunchKernelGGL(HIP_KERNEL_NAME(recurrent_kernel<T, DK_, BV_>), dim3(B * Hv, V / BV_), dim3(kThreads), 0, \
+  GDN_LAUNCH(kKernRecurrent, stream, (recurrent_kernel<T, DK_, BV_>), dim3(B * Hv, V / BV_), dim3(kThreads), 0, \
                      stream, (const T*)q, (const T*)k, (const T*)v, g, beta, state_in, state_out, (T*)o, B,    \
                      T_len, Hqk, Hv, V, scale, use_l2norm)
   const bool wide = (V % 128 == 0);

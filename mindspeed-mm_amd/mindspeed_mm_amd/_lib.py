@@ -22,6 +22,10 @@ SIGNATURES = {
     "gdn_conv1d_bwd_workspace_bytes": (L, [I] * 4),
     "gdn_conv1d_bwd": (I, [P] * 12 + [L] + [I] * 7 + [P]),
     "gdn_conv1d_update": (I, [P] * 5 + [I] * 7 + [P]),
+    "gdn_profile_enable": (I, [I]),
+    "gdn_profile_kernel_count": (I, []),
+    "gdn_profile_kernel_name": (ctypes.c_char_p, [I]),
+    "gdn_profile_collect": (I, [P, P]),
 }
 
 DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
@@ -62,6 +66,18 @@ class GdnLibrary:
         if code < 0:
             raise ValueError(f"{what}: {_ERRORS.get(code, 'invalid argument')} (code {code})")
         raise RuntimeError(f"{what}: HIP error {code}")
+
+
+def kernel_timings(lib: "GdnLibrary"):
+    """Collect the per-kernel event timings recorded since profiling was enabled:
+    {kernel name: (total milliseconds, launches)}."""
+    n = lib.gdn_profile_kernel_count()
+    ms = (ctypes.c_double * n)()
+    cnt = (ctypes.c_int64 * n)()
+    rc = lib.gdn_profile_collect(ctypes.cast(ms, c_void_p), ctypes.cast(cnt, c_void_p))
+    if rc != 0:
+        raise RuntimeError("gdn_profile_collect failed")
+    return {lib.gdn_profile_kernel_name(i).decode(): (ms[i], cnt[i]) for i in range(n) if cnt[i] > 0}
 
 
 _default = None

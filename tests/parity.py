@@ -6,36 +6,14 @@ CPU oracle (oracle/gdn_oracle.py).  Tolerances are the ones the task states:
     bf16 vs the fp32 oracle on the same (bf16-valued) inputs: max abs error <= 2e-2 on o,
           <= 5e-2 on dq/dk/dv/dg/dbeta (and on the states, whose magnitude is O(1)).
 """
-import math
-
 import torch
-import torch.nn.functional as F
 
+from mindspeed_mm_amd.inputs import gdn_inputs
 from oracle import gdn_oracle as O
 
 FP32_REL = 1e-4
 BF16_ABS_O = 2e-2
 BF16_ABS_GRAD = 5e-2
-
-
-def gdn_inputs(B, T, Hqk, Hv, K, V, dtype, seed=0, N=None, l2norm_in_kernel=True, a_log=(1.0, 16.0),
-               dt_bias=(-4.0, -2.0), h0_std=0.02):
-    """Input recipe of the benchmark configurations: q,k ~ N(0,1) (L2-normalised here if the kernel does not
-    do it), v ~ N(0,1), beta = sigmoid(N(0,1)), g = -exp(A_log) softplus(N(0,1) + dt_bias) with per-head
-    A_log ~ U(log a0, log a1), dt_bias ~ U(b0, b1) (caller-side math: modeling_qwen3_5.py:833-841)."""
-    gen = torch.Generator().manual_seed(seed)
-    r = lambda *s: torch.randn(*s, generator=gen)
-    q, k, v = r(B, T, Hqk, K), r(B, T, Hqk, K), r(B, T, Hv, V)
-    if not l2norm_in_kernel:
-        q, k = O.l2norm(q), O.l2norm(k)
-    beta = torch.sigmoid(r(B, T, Hv))
-    A_log = torch.empty(Hv).uniform_(math.log(a_log[0]), math.log(a_log[1]), generator=gen)
-    bias = torch.empty(Hv).uniform_(dt_bias[0], dt_bias[1], generator=gen)
-    g = -A_log.exp() * F.softplus(r(B, T, Hv) + bias)
-    h0 = h0_std * r(N if N is not None else B, Hv, K, V)
-    do = r(B, T, Hv, V)
-    dht = h0_std * r(N if N is not None else B, Hv, K, V)
-    return dict(q=q.to(dtype), k=k.to(dtype), v=v.to(dtype), g=g, beta=beta.to(dtype), h0=h0, do=do.to(dtype), dht=dht)
 
 
 def _err(name, got, ref, dtype, abs_tol, rtol=0.0):
