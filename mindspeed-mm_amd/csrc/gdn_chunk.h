@@ -23,11 +23,13 @@ struct ChunkWorkspace {
   int64_t G;              // f32 [tokens,Hv]  chunk-local cumulative log decay
   int64_t Ai;             // T [tokens,Hv,64] rows of (I + A)^-1
   int64_t W;              // T [tokens,Hv,K]
-  int64_t VN;             // T [tokens,Hv,V]  U, overwritten in place by v_new = U - W S
-  int64_t H;              // T [chunks,Hv,V,K] state BEFORE each chunk, stored transposed
+  int64_t AQ;             // T [tokens,Hv,64] rows of tril(Q K^T . Gam) (unscaled)
+  int64_t U;              // T [chunks,Hv,V/32,2,64,16] U in accumulator-fragment order (see chunk_prep_kernel)
+  int64_t VN;             // T [tokens,Hv,V]  v_new = U - W S (kept for the backward pass)
+  int64_t H;              // T [chunks,Hv,K,V] state BEFORE each chunk
   int64_t fwd_bytes;
-  int64_t DV;             // T [tokens,Hv,V]  dv_local, overwritten in place by d(v_new)
-  int64_t DH;             // T [chunks,Hv,V,K] gradient of the state AFTER each chunk, transposed
+  int64_t DV;             // T [tokens,Hv,V]  d(v_new)
+  int64_t DH;             // T [chunks,Hv,K,V] gradient of the state AFTER each chunk
   int64_t DW;             // T [tokens,Hv,K]
   int64_t DQH, DKH;       // T [tokens,Hv,K]  per-value-head dq, dk before the group sum
   int64_t DG;             // f32 [tokens,Hv]  gradient w.r.t. the cumulative decay (two partial terms)
@@ -48,6 +50,8 @@ inline ChunkWorkspace chunk_workspace_layout(const ChunkDims& d, int elem_bytes)
   w.G = take(tok * d.Hv * 4);
   w.Ai = take(tok * d.Hv * 64 * elem_bytes);
   w.W = take(tok * d.Hv * d.K * elem_bytes);
+  w.AQ = take(tok * d.Hv * 64 * elem_bytes);
+  w.U = take(nc * 64 * d.Hv * d.V * elem_bytes);
   w.VN = take(tok * d.Hv * d.V * elem_bytes);
   w.H = take(nc * d.Hv * d.V * d.K * elem_bytes);
   w.fwd_bytes = off;

@@ -146,14 +146,16 @@ __global__ __launch_bounds__(kThreads) void chunk_state_bwd_kernel(
   for (int c = nchunks - 1; c >= 0; --c) {
     const int64_t tok0 = bos + (int64_t)c * kChunk;
     const int nvalid = imin(kChunk, len - c * kChunk);
-    T* dhg = dhbuf + (((chunk_base + c) * Hv + h) * V + v0) * DK;
+    T* dhg = dhbuf + ((chunk_base + c) * Hv + h) * DK * V + v0;      // [K][V]: this slab is columns v0..v0+BV
 #pragma unroll
     for (int i = 0; i < NS; ++i) {
       const int tt = wave + 4 * i;
       if (tt < MT * NTC) {
         const int mi = tt % MT, ni = tt / MT;
         acc_to_lds(dS[i], dSb, LDK, 32 * mi, 32 * ni);
-        acc_to_global(dS[i], dhg, (int64_t)DK, 32 * mi, 32 * ni, BV);
+        const int kcol = 32 * ni + acc_col();
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dhg[(int64_t)kcol * V + 32 * mi + acc_row(r)] = Elem<T>::from_f(dS[i][r]);
       }
     }
     if (tid < 64) {
@@ -215,13 +217,13 @@ __global__ __launch_bounds__(kThreads) void chunk_state_bwd_kernel(
 // ---------------------------------------------------------------------------------------------
 template <typename T, int DK, int BV> struct DqkwSmem {
   static constexpr int LDK = lds_ld<T>(DK), LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
-  static constexpr int SR = BV > 64 ? BV : 64;                              // rows of the state tiles / of Q,K
+  static constexpr int SE = (DK * LDV > 64 * LDK) ? DK * LDV : 64 * LDK;   // state tile [DK][BV] / Q,K tile [64][DK]
   static constexpr int off_do = 0;                                          // later ds
   static constexpr int off_vp = off_do + 64 * LDV * (int)sizeof(T);         // later ds^T
   static constexpr int off_dv = off_vp + 64 * LDV * (int)sizeof(T);
   static constexpr int off_sb = off_dv + 64 * LDV * (int)sizeof(T);         // later Q
-  static constexpr int off_dsb = off_sb + SR * LDK * (int)sizeof(T);        // later K
-  static constexpr int off_row = off_dsb + SR * LDK * (int)sizeof(T);
+  static constexpr int off_dsb = off_sb + SE * (int)sizeof(T);              // later K
+  static constexpr int off_row = off_dsb + SE * (int)sizeof(T);
   static constexpr int bytes = off_row + (4 * 64 + 8) * 4;
   static_assert(LDV >= L64, "ds reuses the dO tile");
 };
@@ -275,12 +277,12 @@ __global__ __launch_bounds__(kThreads) void chunk_dqkw_kernel(
     load_tile<T, BV>(dOs, LDV, dO + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
     load_tile<T, BV>(Vps, LDV, vn + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
     load_tile<T, BV>(dVs, LDV, dvn + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
-    load_tile<T, DK, BV>(Sb, LDK, hbuf + hoff + (int64_t)v0 * DK, (int64_t)DK, BV, tid);
-    load_tile<T, DK, BV>(dSb, LDK, dhbuf + hoff + (int64_t)v0 * DK, (int64_t)DK, BV, tid);
+    load_tile<T, BV, DK>(Sb, LDV, hbuf + hoff + v0, (int64_t)V, DK, tid);       // S[kd][v0..v0+BV)
+    load_tile<T, BV, DK>(dSb, LDV, dhbuf + hoff + v0, (int64_t)V, DK, tid);
     __syncthreads();
-    for (int e = tid; e < BV * DK; e += kThreads) {
-      const int r = e / DK, c = e % DK;
-      sds += Elem<T>::to_f(Sb[r * LDK + c]) * Elem<T>::to_f(dSb[r * LDK + c]);
+    for (int e = tid; e < DK * BV; e += kThreads) {
+      const int r = e / BV, c = e % BV;
+      sds += Elem<T>::to_f(Sb[r * LDV + c]) * Elem<T>::to_f(dSb[r * LDV + c]);
     }
     if (tj <= ti) mma32<T, BV, true, true>(ds, dOs + 32 * ti * LDV, LDV, Vps + 32 * tj * LDV, LDV);
 #pragma unroll
@@ -288,9 +290,9 @@ __global__ __launch_bounds__(kThreads) void chunk_dqkw_kernel(
       const int tt = wave + 4 * i;
       if (tt < 2 * (DK / 32)) {
         const int ri = tt & 1, cj = tt >> 1;
-        mma32<T, BV, true, false>(dQi[i], dOs + 32 * ri * LDV, LDV, Sb + 32 * cj, LDK);
-        mma32<T, BV, true, false>(dKi[i], Vps + 32 * ri * LDV, LDV, dSb + 32 * cj, LDK);
-        mma32<T, BV, true, false>(dWa[i], dVs + 32 * ri * LDV, LDV, Sb + 32 * cj, LDK);
+        mma32<T, BV, true, true>(dQi[i], dOs + 32 * ri * LDV, LDV, Sb + 32 * cj * LDV, LDV);
+        mma32<T, BV, true, true>(dKi[i], Vps + 32 * ri * LDV, LDV, dSb + 32 * cj * LDV, LDV);
+        mma32<T, BV, true, true>(dWa[i], dVs + 32 * ri * LDV, LDV, Sb + 32 * cj * LDV, LDV);
       }
     }
   }

@@ -6,10 +6,9 @@
 //     S <- e^{G_last} S + (e^{G_last - G} . K)^T V'
 // Math: mindspeed_mm/fsdp/models/qwen3_5/modeling_qwen3_5.py:398-475; stage split as in
 // mindspeed_mm/fsdp/ops/gdn/chunk_gated_delta_rule.py:30-85 (cumsum, KK^T, tril solve, W/U, state
-// recurrence, output), fused here into three launches:
-//     chunk_prep_kernel      per (chunk, head):        G, Tm, W, U           -- MFMA + fp32 block solve
-//     chunk_state_kernel     per (sequence, head, V-slab), sequential in chunks: V', S per chunk
-//     chunk_out_kernel       per (chunk, head, V-slab): O
+// recurrence, output), fused here into two launches:
+//     chunk_prep_kernel   per (chunk, head):  G, Tm, W, U, tril(QK^T . Gam)      -- MFMA + fp32 block solve
+//     chunk_fwd_kernel    per (sequence, head, 32-column state slab), sequential in chunks: V', O, S
 // A ragged last chunk is zero padded in LDS (k = v = beta = g = 0 is exact for this recurrence).
 #include "gdn_chunk.h"
 #include "gdn_common.h"
@@ -75,14 +74,18 @@ __global__ void l2norm_fwd_kernel(const T* __restrict__ x0, const T* __restrict_
 }
 
 // ---------------------------------------------------------------------------------------------
-// chunk_prep_kernel
+// chunk_prep_kernel: everything that is independent across chunks.
+//   G (cumulative decay), Tm = (I+L)^-1, W = Tm (beta e^G K), U = Tm (beta V), Aq = tril(Q K^T . Gam)
+// U is written in accumulator-fragment order -- for tile (32-row block ri, 32-column block vb) lane l stores its 16
+// accumulator values as 16/VEC vectors at U[chunk][head][vb][ri][part][l][0..VEC) -- which is exactly how the
+// recurrence kernel reads it back (straight copy to LDS, conflict-free 16-byte fragment reads).
 // ---------------------------------------------------------------------------------------------
 template <typename T, int DK, int BV> struct PrepSmem {
   static constexpr int LDK = lds_ld<T>(DK), LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
   static constexpr int kv_elems = 64 * (LDK > LDV ? LDK : LDV);
-  static constexpr int off_ks = 0;  // K tile, later the (beta V) tile
-  static constexpr int off_kb = off_ks + kv_elems * (int)sizeof(T);
-  static constexpr int off_as = off_kb + 64 * LDK * (int)sizeof(T);
+  static constexpr int off_ks = 0;  // K tile, scaled in place to beta e^G K after the score tiles
+  static constexpr int off_qs = off_ks + 64 * LDK * (int)sizeof(T);  // Q tile, later the (beta V) tile
+  static constexpr int off_as = off_qs + kv_elems * (int)sizeof(T);
   static constexpr int off_ti = off_as + 64 * kLF * 4;
   static constexpr int off_tms = off_ti + 64 * kLF * 4;
   static constexpr int off_misc = off_tms + 64 * L64 * (int)sizeof(T);
@@ -91,14 +94,16 @@ template <typename T, int DK, int BV> struct PrepSmem {
 
 template <typename T, int DK, int BV>
 __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
-    const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ g, const float* __restrict__ beta,
-    const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, float* __restrict__ G_out,
-    T* __restrict__ Ai_out, T* __restrict__ W_out, T* __restrict__ U_out, int T_len, int N, int Hqk, int Hv, int V) {
+    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ g,
+    const float* __restrict__ beta, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets,
+    float* __restrict__ G_out, T* __restrict__ Ai_out, T* __restrict__ W_out, T* __restrict__ U_out,
+    T* __restrict__ Aq_out, int T_len, int N, int Hqk, int Hv, int V) {
   using SM = PrepSmem<T, DK, BV>;
   constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64, VEC = Elem<T>::kVec;
   T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
-  T* Vb = Ks;
-  T* Kb = reinterpret_cast<T*>(gdn_smem + SM::off_kb);
+  T* Kb = Ks;
+  T* Qs = reinterpret_cast<T*>(gdn_smem + SM::off_qs);
+  T* Vb = Qs;
   float* As = reinterpret_cast<float*>(gdn_smem + SM::off_as);
   float* Ti = reinterpret_cast<float*>(gdn_smem + SM::off_ti);
   T* Tms = reinterpret_cast<T*>(gdn_smem + SM::off_tms);
@@ -112,7 +117,7 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
   const int h = blockIdx.y, hq = h / (Hv / Hqk), nvalid = s.nvalid;
   const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk;
 
-  // ---- phase 0: cumulative decay (one lane per token), beta ----
+  // ---- phase 0: cumulative decay (one lane per token), beta; K and Q tiles ----
   if (wave == 0) {
     float x = lane < nvalid ? g[(tok0 + lane) * Hv + h] : 0.f;
 #pragma unroll
@@ -127,46 +132,46 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
     if (lane < nvalid) G_out[(tok0 + lane) * Hv + h] = x;
   }
   for (int i = tid; i < 64 * kLF; i += kThreads) Ti[i] = 0.f;
+  load_tile<T, DK>(Ks, LDK, k + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
+  load_tile<T, DK>(Qs, LDK, q + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
   __syncthreads();
 
-  // ---- phase 1: K tile, plain and scaled by beta e^G ----
-  {
-    constexpr int CPR = DK / VEC;
-    const T* kg = k + (tok0 * Hqk + hq) * DK;
-    for (int c = tid; c < 64 * CPR; c += kThreads) {
-      const int row = c / CPR, cc = c % CPR;
-      Vec16<T> x = zero16<T>(), xs = zero16<T>();
-      if (row < nvalid) {
-        x = ld16(kg + (int64_t)row * Hqk * DK + cc * VEC);
-        const float sc = egs[row];
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) xs.set(e, x.get(e) * sc);
-      }
-      st16(Ks + row * LDK + cc * VEC, x);
-      st16(Kb + row * LDK + cc * VEC, xs);
-    }
-  }
-  __syncthreads();
-
-  // ---- phase 2: A = strict_tril(beta_i k_i.k_j e^{G_i-G_j}), one 32x32 tile per wave ----
+  // ---- phase 1: A = strict_tril(beta_i k_i.k_j Gam_ij) and Aq = tril(q_i.k_j Gam_ij), one 32x32 tile per wave ----
   {
     const int ti = wave >> 1, tj = wave & 1;
-    f32x16 acc = acc_zero();
-    if (tj <= ti) mma32<T, DK, true, true>(acc, Ks + 32 * ti * LDK, LDK, Ks + 32 * tj * LDK, LDK);
+    f32x16 acc = acc_zero(), aq = acc_zero();
+    if (tj <= ti) {
+      mma32<T, DK, true, true>(acc, Ks + 32 * ti * LDK, LDK, Ks + 32 * tj * LDK, LDK);
+      mma32<T, DK, true, true>(aq, Qs + 32 * ti * LDK, LDK, Ks + 32 * tj * LDK, LDK);
+    }
     const int j = 32 * tj + acc_col();
+    T* aqg = Aq_out + (tok0 * Hv + h) * 64;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int i = 32 * ti + acc_row(r);
-      As[i * kLF + j] = i > j ? bs[i] * acc[r] * __expf(Gs[i] - Gs[j]) : 0.f;
+      const float gam = i >= j ? __expf(Gs[i] - Gs[j]) : 0.f;
+      As[i * kLF + j] = i > j ? bs[i] * acc[r] * gam : 0.f;
+      if (i < nvalid) aqg[(int64_t)i * Hv * 64 + j] = Elem<T>::from_f(aq[r] * gam);
     }
   }
   __syncthreads();
 
-  // (beta V) tile of the first V block goes into the dead K tile while the solve runs
+  // K tile -> beta e^G K in place; (beta V) tile of the first V block replaces Q while the solve runs
+  {
+    constexpr int CPR = DK / VEC;
+    for (int c = tid; c < 64 * CPR; c += kThreads) {
+      const int row = c / CPR, cc = c % CPR;
+      Vec16<T> x = ld16(Ks + row * LDK + cc * VEC);
+      const float sc = egs[row];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) x.set(e, x.get(e) * sc);
+      st16(Kb + row * LDK + cc * VEC, x);
+    }
+  }
   const T* vg = v + (tok0 * Hv + h) * V;
   load_tile_scaled<T, BV>(Vb, LDV, vg, (int64_t)Hv * V, nvalid, bs, tid);
 
-  // ---- phase 3a: invert the four 16x16 diagonal blocks by forward substitution (fp32) ----
+  // ---- phase 2a: invert the four 16x16 diagonal blocks by forward substitution (fp32) ----
   if (lane < 16) {
     const int o = 16 * wave, j = lane;
     float tcol[16];
@@ -182,16 +187,15 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
   }
   __syncthreads();
 
-  // ---- phase 3b: 16 -> 32 merges  X = -T22 (A21 T11); the zero upper triangle of As is scratch ----
+  // ---- phase 2b: 16 -> 32 merges  X = -T22 (A21 T11); the zero upper triangle of As is scratch ----
   {
-    const int p = wave & 1;           // waves 0,1 compute; 2,3 repeat the same values (benign)
+    const int p = wave & 1;           // waves 0,1 write; 2,3 repeat the same values (benign)
     const int C0 = 32 * p, R0 = C0 + 16;
     const int li = lane & 15, lk = lane >> 4;
     f32x4 y = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk)
       y = mfma16_f32(y, As[(R0 + li) * kLF + C0 + 4 * kk + lk], Ti[(C0 + 4 * kk + lk) * kLF + C0 + li]);
-    __syncthreads();  // every wave has read its A21 before the scratch next to it is written
     if (wave < 2) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) As[(C0 + 4 * lk + r) * kLF + R0 + li] = y[r];
@@ -208,7 +212,7 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
   }
   __syncthreads();
 
-  // ---- phase 3c: 32 -> 64 merge, one 16x16 tile of the 32x32 block per wave ----
+  // ---- phase 2c: 32 -> 64 merge, one 16x16 tile of the 32x32 block per wave ----
   {
     const int ta = wave >> 1, tb = wave & 1;
     const int li = lane & 15, lk = lane >> 4;
@@ -229,7 +233,7 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
   }
   __syncthreads();
 
-  // ---- phase 4: Tm in operand precision, kept for the backward pass ----
+  // ---- phase 3: Tm in operand precision, kept for the backward pass ----
   {
     constexpr int CPR = 64 / VEC;
     T* ag = Ai_out + (tok0 * Hv + h) * 64;
@@ -244,7 +248,7 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
   }
   __syncthreads();
 
-  // ---- phase 5: W = Tm (beta e^G K) ----
+  // ---- phase 4: W = Tm (beta e^G K) ----
   {
     T* wg = W_out + (tok0 * Hv + h) * DK;
     for (int tt = wave; tt < 2 * (DK / 32); tt += 4) {
@@ -254,217 +258,224 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
       acc_to_global(acc, wg, (int64_t)Hv * DK, 32 * ri, 32 * cj, nvalid);
     }
   }
-  // ---- phase 6: U = Tm (beta V), V block by V block ----
+  // ---- phase 5: U = Tm (beta V), V block by V block, stored in fragment order ----
   for (int vb = 0; vb < V / BV; ++vb) {
     if (vb > 0) {
       __syncthreads();
       load_tile_scaled<T, BV>(Vb, LDV, vg + vb * BV, (int64_t)Hv * V, nvalid, bs, tid);
       __syncthreads();
     }
-    T* ug = U_out + (tok0 * Hv + h) * V + vb * BV;
     for (int tt = wave; tt < 2 * (BV / 32); tt += 4) {
       const int ri = tt & 1, cj = tt >> 1;
       f32x16 acc = acc_zero();
       mma32<T, 64, true, false>(acc, Tms + 32 * ri * L64, L64, Vb + 32 * cj, LDV);
-      acc_to_global(acc, ug, (int64_t)Hv * V, 32 * ri, 32 * cj, nvalid);
+      const int vblk = vb * (BV / 32) + cj;
+      T* ug = U_out + ((((int64_t)blockIdx.x * Hv + h) * (V / 32) + vblk) * 2 + ri) * (64 * 16);
+#pragma unroll
+      for (int c = 0; c < 16 / VEC; ++c) {
+        Vec16<T> x = zero16<T>();
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) x.set(e, acc[c * VEC + e]);
+        st16(ug + (c * 64 + lane) * VEC, x);
+      }
     }
   }
 }
 
 // ---------------------------------------------------------------------------------------------
-// chunk_state_kernel: the inter-chunk recurrence.  The workgroup keeps the transposed state slab
-// S^T[BV, DK] in fp32 accumulators for the whole sequence; a copy in operand precision is staged in
-// LDS once per chunk (B operand of W S) and streamed to HBM for the output and backward kernels.
+// chunk_fwd_kernel: the inter-chunk recurrence fused with the output.  One wave owns a 32-column slab of the
+// state S[K, 32] in fp32 accumulators for the whole sequence, and for every chunk does
+//     V' = U - W S        O = scale [ e^G . (Q S) + Aq V' ]        S <- e^{G_last} S + K^T (e^{G_last-G} . V')
+// Every B operand (S, V') is taken straight from accumulator registers (see frag_b_from_acc), so the waves
+// of a workgroup never exchange data and the chain W S -> V' -> S needs no LDS round trip.  The A operands
+// (W, Q, Aq row-major, K transposed) are staged in LDS by NW dedicated loader waves of the same workgroup; with
+// STAGES = 2 they run one chunk ahead of the NW compute waves and the two roles meet at one barrier per chunk.
 // ---------------------------------------------------------------------------------------------
-template <typename T, int DK, int BV> struct StateSmem {
+template <typename T, int DK, int NW, int STAGES> struct FwdSmem {
   static constexpr int LDK = lds_ld<T>(DK), L64 = lds_ld<T>(64);
   static constexpr int off_ws = 0;
-  static constexpr int off_ks = off_ws + 64 * LDK * (int)sizeof(T);
-  static constexpr int off_sb = off_ks + 64 * LDK * (int)sizeof(T);
-  static constexpr int off_vpt = off_sb + BV * LDK * (int)sizeof(T);
-  static constexpr int off_gs = off_vpt + BV * L64 * (int)sizeof(T);
-  static constexpr int bytes = off_gs + 64 * 4;
+  static constexpr int off_qs = off_ws + 64 * LDK * (int)sizeof(T);
+  static constexpr int off_kt = off_qs + 64 * LDK * (int)sizeof(T);
+  static constexpr int off_aq = off_kt + DK * L64 * (int)sizeof(T);
+  static constexpr int off_uf = off_aq + 64 * L64 * (int)sizeof(T);
+  static constexpr int off_gs = off_uf + NW * 2 * 64 * 16 * (int)sizeof(T);
+  static constexpr int stage = off_gs + 2 * 64 * 4;
+  static constexpr int bytes = STAGES * stage;
 };
 
-template <typename T, int DK, int BV>
-__global__ __launch_bounds__(kThreads) void chunk_state_kernel(
-    const T* __restrict__ k, const T* __restrict__ w, T* vn, const float* __restrict__ G,
-    const float* __restrict__ h0, float* __restrict__ ht, T* __restrict__ hbuf, const int64_t* __restrict__ cu,
-    const int* __restrict__ chunk_offsets, int T_len, int Hqk, int Hv, int V) {
-  using SM = StateSmem<T, DK, BV>;
-  constexpr int LDK = SM::LDK, L64 = SM::L64;
-  constexpr int MT = BV / 32, NTC = DK / 32, NS = (MT * NTC + 3) / 4;  // state tiles per wave
-  T* Ws = reinterpret_cast<T*>(gdn_smem + SM::off_ws);
-  T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
-  T* Sb = reinterpret_cast<T*>(gdn_smem + SM::off_sb);
-  T* VpT = reinterpret_cast<T*>(gdn_smem + SM::off_vpt);
-  float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_gs);
+template <typename T, int DK, int NW, int STAGES>
+__global__ __launch_bounds__(128 * NW) void chunk_fwd_kernel(
+    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ w, const T* __restrict__ ufrag,
+    const T* __restrict__ aqk, const float* __restrict__ G, const float* __restrict__ h0, float* __restrict__ ht,
+    T* __restrict__ o, T* __restrict__ vn, T* __restrict__ hbuf, const int64_t* __restrict__ cu,
+    const int* __restrict__ chunk_offsets, int T_len, int Hqk, int Hv, int V, float scale) {
+  using SM = FwdSmem<T, DK, NW, STAGES>;
+  constexpr int LDK = SM::LDK, L64 = SM::L64, NT = 64 * NW, VEC = Elem<T>::kVec;
+  constexpr int NKT = DK / 32;                                  // state tiles of a compute wave (rows of S)
+  constexpr int CW = 64 * (DK / VEC) / NT, CA = 64 * (64 / VEC) / NT, CU = 16 / VEC;
+  constexpr int CUL = NW * 2 * 64 * 16 / VEC / NT;              // U vectors copied by a loader thread
+  static_assert(64 * (DK / VEC) % NT == 0 && 64 * (64 / VEC) % NT == 0, "tile chunks must divide over the loaders");
 
-  const int tid = threadIdx.x, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31;
   const int n = blockIdx.x / Hv, h = blockIdx.x % Hv, hq = h / (Hv / Hqk);
-  const int v0 = blockIdx.y * BV;
   const int64_t bos = cu ? cu[n] : (int64_t)n * T_len;
   const int len = cu ? (int)(cu[n + 1] - bos) : T_len;
   const int nchunks = (len + kChunk - 1) / kChunk;
   const int64_t chunk_base = cu ? chunk_offsets[n] : (int64_t)n * ((T_len + kChunk - 1) / kChunk);
 
-  // state tile tt of this wave: rows (v) 32*mi.., cols (k) 32*ni..
-  f32x16 S[NS];
+  if (wave >= NW) {
+    // ================= loader waves: global -> LDS stage, one chunk ahead of the compute waves =================
+    const int lt = tid - NT;
+    for (int c = 0; c < nchunks; ++c) {
+      const int buf = (STAGES == 2) ? (c & 1) : 0;
+      if (STAGES == 1 && c > 0) __syncthreads();              // (B) the single stage is free again
+      unsigned char* base = gdn_smem + buf * SM::stage;
+      T* Ws = reinterpret_cast<T*>(base + SM::off_ws);
+      T* Qs = reinterpret_cast<T*>(base + SM::off_qs);
+      T* KT = reinterpret_cast<T*>(base + SM::off_kt);
+      T* Aq = reinterpret_cast<T*>(base + SM::off_aq);
+      T* Uf = reinterpret_cast<T*>(base + SM::off_uf);
+      float* Gs = reinterpret_cast<float*>(base + SM::off_gs);
+      const int64_t tok0 = bos + (int64_t)c * kChunk;
+      const int nvalid = imin(kChunk, len - c * kChunk);
+      Vec16<T> pw[CW], pq[CW], pk[CW], pa[CA], pu[CUL];
+      const float g_last = G[(tok0 + nvalid - 1) * Hv + h];
 #pragma unroll
-  for (int i = 0; i < NS; ++i) {
-    const int tt = wave + 4 * i;
-    S[i] = acc_zero();
-    if (tt < MT * NTC && h0 != nullptr) {
-      const int mi = tt % MT, ni = tt / MT;
-      const int kcol = 32 * ni + acc_col();
+      for (int i = 0; i < CW; ++i) {
+        const int id = lt + i * NT;
+        const int row = id / (DK / VEC), cc = id % (DK / VEC);          // row-major tiles: W, Q
+        pw[i] = row < nvalid ? ld16(w + ((tok0 + row) * Hv + h) * DK + cc * VEC) : zero16<T>();
+        pq[i] = row < nvalid ? ld16(q + ((tok0 + row) * Hqk + hq) * DK + cc * VEC) : zero16<T>();
+        const int rowt = id % kChunk, cct = id / kChunk;                 // K goes in transposed: rows fastest
+        pk[i] = rowt < nvalid ? ld16(k + ((tok0 + rowt) * Hqk + hq) * DK + cct * VEC) : zero16<T>();
+      }
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        S[i][r] = h0[(((int64_t)n * Hv + h) * DK + kcol) * V + v0 + 32 * mi + acc_row(r)];
+      for (int i = 0; i < CA; ++i) {
+        const int id = lt + i * NT;
+        const int row = id / (64 / VEC), cc = id % (64 / VEC);
+        pa[i] = row < nvalid ? ld16(aqk + ((tok0 + row) * Hv + h) * 64 + cc * VEC) : zero16<T>();
+      }
+      const T* ug = ufrag + (((chunk_base + c) * Hv + h) * (V / 32) + blockIdx.y * NW) * (2 * 64 * 16);
+#pragma unroll
+      for (int i = 0; i < CUL; ++i) pu[i] = ld16(ug + (lt + i * NT) * VEC);
+      // every loader lane owns token lt%64 in the transposed K staging: its decay towards the chunk end
+      const float kdec = __expf(g_last - G[(tok0 + imin(lt & 63, nvalid - 1)) * Hv + h]);
+      if (lt < 64) Gs[lt] = G[(tok0 + imin(lt, nvalid - 1)) * Hv + h];
+#pragma unroll
+      for (int i = 0; i < CW; ++i) {
+        const int id = lt + i * NT;
+        const int row = id / (DK / VEC), cc = id % (DK / VEC);
+        st16(Ws + row * LDK + cc * VEC, pw[i]);
+        st16(Qs + row * LDK + cc * VEC, pq[i]);
+        const int rowt = id % kChunk, cct = id / kChunk;      // rowt == lt % 64 because NT is a multiple of 64
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) KT[(cct * VEC + e) * L64 + rowt] = Elem<T>::from_f(pk[i].get(e) * kdec);
+      }
+#pragma unroll
+      for (int i = 0; i < CUL; ++i) st16(Uf + (lt + i * NT) * VEC, pu[i]);
+#pragma unroll
+      for (int i = 0; i < CA; ++i) {
+        const int id = lt + i * NT;
+        const int row = id / (64 / VEC), cc = id % (64 / VEC);
+        st16(Aq + row * L64 + cc * VEC, pa[i]);
+      }
+      __syncthreads();                                         // (A) chunk c is staged
     }
+    return;
   }
 
+  // ================= compute waves: one 32-column slab of the state each =================
+  const int vblk = blockIdx.y * NW + wave, v0 = 32 * vblk;
+  f32x16 S[NKT];
+#pragma unroll
+  for (int kt = 0; kt < NKT; ++kt) {
+    S[kt] = acc_zero();
+    if (h0 != nullptr) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        S[kt][r] = h0[(((int64_t)n * Hv + h) * DK + 32 * kt + acc_row(r)) * V + v0 + acc_col()];
+    }
+  }
   for (int c = 0; c < nchunks; ++c) {
+    const int buf = (STAGES == 2) ? (c & 1) : 0;
+    __syncthreads();                       // (A) stage `buf` holds chunk c
+    unsigned char* base = gdn_smem + buf * SM::stage;
+    const T* Ws = reinterpret_cast<const T*>(base + SM::off_ws);
+    const T* Qs = reinterpret_cast<const T*>(base + SM::off_qs);
+    const T* KT = reinterpret_cast<const T*>(base + SM::off_kt);
+    const T* Aq = reinterpret_cast<const T*>(base + SM::off_aq);
+    const T* Uf = reinterpret_cast<const T*>(base + SM::off_uf) + wave * (2 * 64 * 16);
+    const float* Gs = reinterpret_cast<const float*>(base + SM::off_gs);
     const int64_t tok0 = bos + (int64_t)c * kChunk;
     const int nvalid = imin(kChunk, len - c * kChunk);
-    T* hg = hbuf + (((chunk_base + c) * Hv + h) * V + v0) * DK;
-    // (a) state before this chunk -> LDS (operand precision) and HBM
-#pragma unroll
-    for (int i = 0; i < NS; ++i) {
-      const int tt = wave + 4 * i;
-      if (tt < MT * NTC) {
-        const int mi = tt % MT, ni = tt / MT;
-        acc_to_lds(S[i], Sb, LDK, 32 * mi, 32 * ni);
-        acc_to_global(S[i], hg, (int64_t)DK, 32 * mi, 32 * ni, BV);
-      }
-    }
-    // (b) operands of this chunk
-    load_tile<T, DK>(Ws, LDK, w + (tok0 * Hv + h) * DK, (int64_t)Hv * DK, nvalid, tid);
-    load_tile<T, DK>(Ks, LDK, k + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
-    if (tid < 64) Gs[tid] = G[(tok0 + imin(tid, nvalid - 1)) * Hv + h];
-    __syncthreads();
     const float glast = Gs[63];
-    // (c) V' = U - W S; the copy for the state update is scaled by e^{G_last - G} and transposed
-    T* vg = vn + (tok0 * Hv + h) * V + v0;
-    for (int tt = wave; tt < 2 * MT; tt += 4) {
-      const int ri = tt & 1, cj = tt >> 1;
-      f32x16 ws = acc_zero();
-      mma32<T, DK, true, true>(ws, Ws + 32 * ri * LDK, LDK, Sb + 32 * cj * LDK, LDK);
-      f32x16 vp = acc_from_global(vg, (int64_t)Hv * V, 32 * ri, 32 * cj, nvalid);
+    int64_t row_v = V, row_hv = (int64_t)Hv * V;   // row strides of the h / o,v_new stores
+    GDN_OPAQUE(row_v);
+    GDN_OPAQUE(row_hv);
+
+    AccB<T> Sb[NKT];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) vp[r] -= ws[r];
-      acc_to_global(vp, vg, (int64_t)Hv * V, 32 * ri, 32 * cj, nvalid);
+    for (int kt = 0; kt < NKT; ++kt) Sb[kt].pack(S[kt]);
+    if (hbuf != nullptr) {                 // state before this chunk, for the backward pass
+      T* hg = hbuf + (((chunk_base + c) * Hv + h) * DK) * V + v0;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) vp[r] *= __expf(glast - Gs[32 * ri + acc_row(r)]);
-      acc_to_lds_t(vp, VpT, L64, 32 * ri, 32 * cj);
+      for (int kt = 0; kt < NKT; ++kt) acc_to_global(S[kt], hg, row_v, 32 * kt, 0, DK);
     }
-    __syncthreads();
-    // (d) S^T <- e^{G_last} S^T + V'^T K
+    GDN_PHASE_FENCE();
+    // V' = U - W S, then packed as a B operand (for O and for the state update)
+    AccB<T> Vb[2];
+    T* vg = vn != nullptr ? vn + (tok0 * Hv + h) * V + v0 : nullptr;
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri) {
+      f32x16 p = acc_zero();
+#pragma unroll
+      for (int kt = 0; kt < NKT; ++kt) mma32_accb<T>(p, Ws + (32 * ri + l32) * LDK + 32 * kt, Sb[kt]);
+      f32x16 vp;
+#pragma unroll
+      for (int i = 0; i < CU; ++i) {
+        const Vec16<T> u = ld16(Uf + ((ri * CU + i) * 64 + lane) * VEC);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) vp[i * VEC + e] = u.get(e) - p[i * VEC + e];
+      }
+      if (vg != nullptr) acc_to_global(vp, vg, row_hv, 32 * ri, 0, nvalid);
+      Vb[ri].pack(vp);
+      GDN_PHASE_FENCE();
+    }
+    // O = scale [ e^G . (Q S) + Aq V' ]
+    T* og = o + (tok0 * Hv + h) * V + v0;
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri) {
+      f32x16 oa = acc_zero();
+#pragma unroll
+      for (int kt = 0; kt < NKT; ++kt) mma32_accb<T>(oa, Qs + (32 * ri + l32) * LDK + 32 * kt, Sb[kt]);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oa[r] *= __expf(Gs[32 * ri + acc_row(r)]);
+#pragma unroll
+      for (int tj = 0; tj <= ri; ++tj) mma32_accb<T>(oa, Aq + (32 * ri + l32) * L64 + 32 * tj, Vb[tj]);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oa[r] *= scale;
+      acc_to_global(oa, og, row_hv, 32 * ri, 0, nvalid);
+      GDN_PHASE_FENCE();
+    }
+    // S <- e^{G_last} S + (e^{G_last - G} . K)^T V'   (the loaders staged K already scaled)
     const float eg = __expf(glast);
 #pragma unroll
-    for (int i = 0; i < NS; ++i) {
-      const int tt = wave + 4 * i;
-      if (tt < MT * NTC) {
-        const int mi = tt % MT, ni = tt / MT;
+    for (int kt = 0; kt < NKT; ++kt) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) S[i][r] *= eg;
-        mma32<T, 64, true, false>(S[i], VpT + 32 * mi * L64, L64, Ks + 32 * ni, LDK);
-      }
+      for (int r = 0; r < 16; ++r) S[kt][r] *= eg;
+#pragma unroll
+      for (int tj = 0; tj < 2; ++tj) mma32_accb<T>(S[kt], KT + (32 * kt + l32) * L64 + 32 * tj, Vb[tj]);
+      GDN_PHASE_FENCE();
     }
-    __syncthreads();
+    if (STAGES == 1 && c + 1 < nchunks) __syncthreads();      // (B) done with the single stage
   }
 
   if (ht != nullptr) {
 #pragma unroll
-    for (int i = 0; i < NS; ++i) {
-      const int tt = wave + 4 * i;
-      if (tt < MT * NTC) {
-        const int mi = tt % MT, ni = tt / MT;
-        const int kcol = 32 * ni + acc_col();
+    for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          ht[(((int64_t)n * Hv + h) * DK + kcol) * V + v0 + 32 * mi + acc_row(r)] = S[i][r];
-      }
-    }
-  }
-}
-
-// ---------------------------------------------------------------------------------------------
-// chunk_out_kernel:  O = scale [ e^G . (Q S) + tril(Q K^T . Gam) V' ]
-// ---------------------------------------------------------------------------------------------
-template <typename T, int DK, int BV> struct OutSmem {
-  static constexpr int LDK = lds_ld<T>(DK), LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
-  static constexpr int off_qs = 0;
-  static constexpr int off_ks = off_qs + 64 * LDK * (int)sizeof(T);
-  static constexpr int off_sb = off_ks + 64 * LDK * (int)sizeof(T);
-  static constexpr int off_vp = off_sb + BV * LDK * (int)sizeof(T);
-  static constexpr int off_aq = off_vp + 64 * LDV * (int)sizeof(T);
-  static constexpr int off_gs = off_aq + 64 * L64 * (int)sizeof(T);
-  static constexpr int bytes = off_gs + 64 * 4;
-};
-
-template <typename T, int DK, int BV>
-__global__ __launch_bounds__(kThreads) void chunk_out_kernel(
-    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ vn, const T* __restrict__ hbuf,
-    const float* __restrict__ G, T* __restrict__ o, const int64_t* __restrict__ cu,
-    const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V, float scale) {
-  using SM = OutSmem<T, DK, BV>;
-  constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64, MT = BV / 32;
-  T* Qs = reinterpret_cast<T*>(gdn_smem + SM::off_qs);
-  T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
-  T* Sb = reinterpret_cast<T*>(gdn_smem + SM::off_sb);
-  T* Vp = reinterpret_cast<T*>(gdn_smem + SM::off_vp);
-  T* Aq = reinterpret_cast<T*>(gdn_smem + SM::off_aq);
-  float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_gs);
-
-  const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
-  if (s.nvalid <= 0) return;
-  const int tid = threadIdx.x, wave = tid >> 6;
-  const int h = blockIdx.y, hq = h / (Hv / Hqk), nvalid = s.nvalid, v0 = blockIdx.z * BV;
-  const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk;
-
-  load_tile<T, DK>(Qs, LDK, q + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
-  load_tile<T, DK>(Ks, LDK, k + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
-  load_tile<T, DK, BV>(Sb, LDK, hbuf + (((int64_t)blockIdx.x * Hv + h) * V + v0) * DK, (int64_t)DK, BV, tid);
-  load_tile<T, BV>(Vp, LDV, vn + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
-  if (tid < 64) Gs[tid] = G[(tok0 + imin(tid, nvalid - 1)) * Hv + h];
-  __syncthreads();
-
-  {  // intra-chunk scores, one 32x32 tile per wave
-    const int ti = wave >> 1, tj = wave & 1;
-    f32x16 acc = acc_zero();
-    if (tj <= ti) mma32<T, DK, true, true>(acc, Qs + 32 * ti * LDK, LDK, Ks + 32 * tj * LDK, LDK);
-    const int j = 32 * tj + acc_col();
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int i = 32 * ti + acc_row(r);
-      Aq[i * L64 + j] = Elem<T>::from_f(i >= j ? acc[r] * __expf(Gs[i] - Gs[j]) : 0.f);
-    }
-  }
-  constexpr int NO = (2 * MT + 3) / 4;
-  f32x16 O[NO];
-#pragma unroll
-  for (int i = 0; i < NO; ++i) {
-    const int tt = wave + 4 * i;
-    O[i] = acc_zero();
-    if (tt < 2 * MT) {
-      const int ri = tt & 1, cj = tt >> 1;
-      mma32<T, DK, true, true>(O[i], Qs + 32 * ri * LDK, LDK, Sb + 32 * cj * LDK, LDK);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) O[i][r] *= __expf(Gs[32 * ri + acc_row(r)]);
-    }
-  }
-  __syncthreads();
-  T* og = o + (tok0 * Hv + h) * V + v0;
-#pragma unroll
-  for (int i = 0; i < NO; ++i) {
-    const int tt = wave + 4 * i;
-    if (tt < 2 * MT) {
-      const int ri = tt & 1, cj = tt >> 1;
-      mma32<T, 64, true, false>(O[i], Aq + 32 * ri * L64, L64, Vp + 32 * cj, LDV);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) O[i][r] *= scale;
-      acc_to_global(O[i], og, (int64_t)Hv * V, 32 * ri, 32 * cj, nvalid);
-    }
+      for (int r = 0; r < 16; ++r)
+        ht[(((int64_t)n * Hv + h) * DK + 32 * kt + acc_row(r)) * V + v0 + acc_col()] = S[kt][r];
   }
 }
 
@@ -476,10 +487,10 @@ template <typename K> static int set_lds(K kernel, int bytes) {
                                   bytes);
 }
 
-template <typename T, int DK, int BVP, int BVS, int BVO>
+template <typename T, int DK, int BVP, int NW, int STAGES>
 static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const void* q, const void* k, const void* v,
                             const float* g, const float* beta, const float* h0, const int64_t* cu, void* o, float* ht,
-                            unsigned char* ws, float scale, int l2norm, hipStream_t st) {
+                            unsigned char* ws, float scale, int l2norm, bool keep_for_backward, hipStream_t st) {
   const int64_t tok = d.tokens();
   const int nc = (int)d.max_chunks();
   int* chunk_offsets = reinterpret_cast<int*>(ws + L.chunk_offsets);
@@ -492,36 +503,32 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     T* qn = reinterpret_cast<T*>(ws + L.qn);
     T* kn = reinterpret_cast<T*>(ws + L.kn);
     GDN_LAUNCH(kKernL2Norm, st, (l2norm_fwd_kernel<T, DK>),
-                       dim3((unsigned)((rows + kThreads / LPR - 1) / (kThreads / LPR)), 2), dim3(kThreads), 0, st, qq,
-                       kk, qn, kn, rows);
+               dim3((unsigned)((rows + kThreads / LPR - 1) / (kThreads / LPR)), 2), dim3(kThreads), 0, st, qq, kk, qn,
+               kn, rows);
     qq = qn;
     kk = kn;
   }
   float* G = reinterpret_cast<float*>(ws + L.G);
   T* Ai = reinterpret_cast<T*>(ws + L.Ai);
   T* W = reinterpret_cast<T*>(ws + L.W);
-  T* VN = reinterpret_cast<T*>(ws + L.VN);
-  T* H = reinterpret_cast<T*>(ws + L.H);
+  T* AQ = reinterpret_cast<T*>(ws + L.AQ);
+  T* U = reinterpret_cast<T*>(ws + L.U);
+  T* VN = keep_for_backward ? reinterpret_cast<T*>(ws + L.VN) : nullptr;
+  T* H = keep_for_backward ? reinterpret_cast<T*>(ws + L.H) : nullptr;
   {
     auto kern = chunk_prep_kernel<T, DK, BVP>;
     constexpr int smem = PrepSmem<T, DK, BVP>::bytes;
     if (int e = set_lds(kern, smem)) return e;
-    GDN_LAUNCH(kKernPrep, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, kk, (const T*)v, g, beta, cu,
-                       (const int*)chunk_offsets, G, Ai, W, VN, d.T, d.N, d.Hqk, d.Hv, d.V);
+    GDN_LAUNCH(kKernPrep, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, (const T*)v, g, beta, cu,
+               (const int*)chunk_offsets, G, Ai, W, U, AQ, d.T, d.N, d.Hqk, d.Hv, d.V);
   }
   {
-    auto kern = chunk_state_kernel<T, DK, BVS>;
-    constexpr int smem = StateSmem<T, DK, BVS>::bytes;
+    auto kern = chunk_fwd_kernel<T, DK, NW, STAGES>;
+    constexpr int smem = FwdSmem<T, DK, NW, STAGES>::bytes;
     if (int e = set_lds(kern, smem)) return e;
-    GDN_LAUNCH(kKernStateFwd, st, kern, dim3(d.N * d.Hv, d.V / BVS), dim3(kThreads), smem, st, kk, (const T*)W, VN,
-                       (const float*)G, h0, ht, H, cu, (const int*)chunk_offsets, d.T, d.Hqk, d.Hv, d.V);
-  }
-  {
-    auto kern = chunk_out_kernel<T, DK, BVO>;
-    constexpr int smem = OutSmem<T, DK, BVO>::bytes;
-    if (int e = set_lds(kern, smem)) return e;
-    GDN_LAUNCH(kKernOut, st, kern, dim3(nc, d.Hv, d.V / BVO), dim3(kThreads), smem, st, qq, kk, (const T*)VN, (const T*)H,
-                       (const float*)G, (T*)o, cu, (const int*)chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale);
+    GDN_LAUNCH(kKernStateFwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NW)), dim3(128 * NW), smem, st, qq, kk,
+               (const T*)W, (const T*)U, (const T*)AQ, (const float*)G, h0, ht, (T*)o, VN, H, cu,
+               (const int*)chunk_offsets, d.T, d.Hqk, d.Hv, d.V, scale);
   }
   return (int)hipGetLastError();
 }
@@ -548,20 +555,24 @@ extern "C" int gdn_chunk_fwd(const void* q, const void* k, const void* v, const 
   dl.varlen = true;  // one layout for both modes (the packed bound is the larger)
   const ChunkWorkspace L = chunk_workspace_layout(dl, dtype == 0 ? 4 : 2);
   if (workspace_bytes < L.fwd_bytes) return -5;
+  const bool keep = workspace_bytes >= L.total_bytes;   // a workspace sized for backward also receives v_new and the states
   if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
   unsigned char* ws = static_cast<unsigned char*>(workspace);
   hipStream_t st = (hipStream_t)stream;
-#define GDN_FWD(T_, DK_, BVP_, BVS_, BVO_) \
-  return chunk_fwd_launch<T_, DK_, BVP_, BVS_, BVO_>(d, L, q, k, v, g, beta, initial_state, cu_seqlens, o, final_state, ws, scale, use_qk_l2norm, st)
+#define GDN_FWD(T_, DK_, BVP_, NW_, ST_)                                                                          \
+  return chunk_fwd_launch<T_, DK_, BVP_, NW_, ST_>(d, L, q, k, v, g, beta, initial_state, cu_seqlens, o, final_state, \
+                                                   ws, scale, use_qk_l2norm, keep, st)
   const bool wide = (V % 128 == 0);
   if (dtype == 1) {
-    if (K == 128 && wide) GDN_FWD(bf16_t, 128, 128, 64, 128);
-    if (K == 128) GDN_FWD(bf16_t, 128, 64, 64, 64);
-    if (K == 64 && wide) GDN_FWD(bf16_t, 64, 128, 64, 128);
-    GDN_FWD(bf16_t, 64, 64, 64, 64);
+    if (K == 128 && wide) GDN_FWD(bf16_t, 128, 128, 4, 2);
+    if (K == 128) GDN_FWD(bf16_t, 128, 64, 2, 1);
+    if (K == 64 && wide) GDN_FWD(bf16_t, 64, 128, 4, 2);
+    GDN_FWD(bf16_t, 64, 64, 2, 1);
   } else {
-    if (K == 128) GDN_FWD(float, 128, 64, 64, 64);
-    GDN_FWD(float, 64, 64, 64, 64);
+    if (K == 128 && wide) GDN_FWD(float, 128, 64, 4, 1);
+    if (K == 128) GDN_FWD(float, 128, 64, 2, 1);
+    if (wide) GDN_FWD(float, 64, 64, 4, 1);
+    GDN_FWD(float, 64, 64, 2, 1);
   }
 #undef GDN_FWD
 }

@@ -33,12 +33,14 @@ struct bf16_t { uint16_t bits; };
 struct f16_t { uint16_t bits; };
 
 __device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
-__device__ __forceinline__ uint16_t f32_to_bf16(float f) {  // round to nearest even; NaN stays NaN
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+// round to nearest even; one v_cvt_pk_bf16_f32 on gfx950
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2(float lo, float hi) {
+  const f32x2 f = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
 }
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) { return (uint16_t)(f32x2_to_bf16x2(f, 0.f) & 0xffffu); }
 
 template <typename T> struct Elem;
 template <> struct Elem<float> {
@@ -59,6 +61,13 @@ template <> struct Elem<f16_t> {
 
 // padded leading dimension (in elements) of an LDS tile with `cols` columns
 template <typename T> __device__ __host__ constexpr int lds_ld(int cols) { return cols + 16 / (int)sizeof(T); }
+
+// compiler-only fence: keeps the scheduler from hoisting a later phase's LDS/global loads (and their registers)
+// above it.  No instruction is emitted.
+#define GDN_PHASE_FENCE() asm volatile("" ::: "memory")
+// makes a loop-invariant value opaque inside a loop so that the address arithmetic derived from it is recomputed
+// where it is used instead of being hoisted out of the loop and held in registers for its whole duration
+#define GDN_OPAQUE(x) asm volatile("" : "+r"(x))
 
 __device__ __forceinline__ int imin(int a, int b) { return a < b ? a : b; }
 __device__ __forceinline__ int imax(int a, int b) { return a > b ? a : b; }
@@ -185,6 +194,68 @@ __device__ __forceinline__ void mma32(f32x16& acc, const T* A, int lda, const T*
     if constexpr (A_KC) a = frag_contig(A + r32 * lda + k); else a = frag_strided(A + k * lda + r32, lda);
     if constexpr (B_KC) b = frag_contig(B + r32 * ldb + k); else b = frag_strided(B + k * ldb + r32, ldb);
     mfma_kgroup<T>(acc, a, b);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Chaining two contractions through registers.  An accumulator tile C (rows i in registers, column j = lane%32)
+// already has the lane layout of a B operand whose contraction index is C's row index: D += A * C needs no LDS
+// round trip.  Per k-group the lane's registers cover rows
+//     bf16: r = 8kg..8kg+7  ->  16kg + {4h..4h+3, 8+4h..8+4h+3}      fp32: r = 4kg..4kg+3  ->  8kg + 4h..4h+3
+// (h = lane/32), so the A operand must be gathered with the same k order: frag_a_split.
+// ---------------------------------------------------------------------------------------------
+template <typename T> struct AccK { static constexpr int kGroups = (sizeof(T) == 2) ? 2 : 4; };  // per 32-row tile
+
+template <typename T, int KG> __device__ __forceinline__ u32x4 frag_b_from_acc(const f32x16& c) {
+  u32x4 b;
+  if constexpr (sizeof(T) == 2) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) b[e] = f32x2_to_bf16x2(c[8 * KG + 2 * e], c[8 * KG + 2 * e + 1]);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) b[e] = __float_as_uint(c[4 * KG + e]);
+  }
+  return b;
+}
+// p points at A[row][first contraction index of the k-group]
+template <typename T> __device__ __forceinline__ u32x4 frag_a_split(const T* p) {
+  const int half = (threadIdx.x & 63) >> 5;
+  if constexpr (sizeof(T) == 2) {
+    const u32x2 lo = *reinterpret_cast<const u32x2*>(p + 4 * half);
+    const u32x2 hi = *reinterpret_cast<const u32x2*>(p + 8 + 4 * half);
+    return u32x4{lo[0], lo[1], hi[0], hi[1]};
+  } else {
+    return *reinterpret_cast<const u32x4*>(p + 4 * half);
+  }
+}
+// all k-groups of one 32-row accumulator tile packed as B fragments
+template <typename T> struct AccB {
+  u32x4 f[AccK<T>::kGroups];
+  __device__ __forceinline__ void pack(const f32x16& c) {
+    f[0] = frag_b_from_acc<T, 0>(c);
+    f[1] = frag_b_from_acc<T, 1>(c);
+    if constexpr (sizeof(T) == 4) { f[2] = frag_b_from_acc<T, 2>(c); f[3] = frag_b_from_acc<T, 3>(c); }
+  }
+};
+// d(32x32) += A[32 rows][32 k] * B(32 k x 32) with B packed from an accumulator; arow = &A[row of this lane][k0]
+template <typename T> __device__ __forceinline__ void mma32_accb(f32x16& d, const T* arow, const AccB<T>& b) {
+  constexpr int G = KGroup<T>::kLen;
+#pragma unroll
+  for (int kg = 0; kg < AccK<T>::kGroups; ++kg) mfma_kgroup<T>(d, frag_a_split<T>(arow + G * kg), b.f[kg]);
+}
+
+// global -> LDS transposed staging: tile[64 rows][COLS] in memory becomes lds[COLS][ld] (rows contiguous), each
+// row optionally scaled.  Lanes walk rows fastest so that the 2-byte scattered LDS writes do not conflict.
+template <typename T, int COLS, int NT>
+__device__ __forceinline__ void load_tile_t(T* lds, int ld, const T* g, int64_t row_stride, int nvalid, int tid,
+                                            const float* rowscale = nullptr) {
+  constexpr int V = Elem<T>::kVec, CPR = COLS / V;
+  for (int c = tid; c < kChunk * CPR; c += NT) {
+    const int row = c % kChunk, cc = c / kChunk;
+    Vec16<T> v = row < nvalid ? ld16(g + (int64_t)row * row_stride + cc * V) : zero16<T>();
+    const float s = rowscale ? rowscale[row] : 1.f;
+#pragma unroll
+    for (int e = 0; e < V; ++e) lds[(cc * V + e) * ld + row] = Elem<T>::from_f(rowscale ? v.get(e) * s : v.get(e));
   }
 }
 
