@@ -22,18 +22,24 @@ struct ChunkWorkspace {
   int64_t qn, kn;         // T [tokens,Hqk,K] l2-normalised q,k (only with use_qk_l2norm)
   int64_t G;              // f32 [tokens,Hv]  chunk-local cumulative log decay
   int64_t Ai;             // T [tokens,Hv,64] rows of (I + A)^-1
-  int64_t W;              // T [tokens,Hv,K]
+  int64_t WAF;            // T [chunks,Hv,K/32,2]    W as A operand: tile = (32 tokens) x (32 columns of K), fragment order
   int64_t AQ;             // T [tokens,Hv,64] rows of tril(Q K^T . Gam) (unscaled)
-  int64_t U;              // T [chunks,Hv,V/32,2,64,16] U in accumulator-fragment order (see chunk_prep_kernel)
-  int64_t VN;             // T [tokens,Hv,V]  v_new = U - W S (kept for the backward pass)
-  int64_t H;              // T [chunks,Hv,K,V] state BEFORE each chunk
+  // Tiles exchanged between kernels in fragment order (see AccB<>): 1024 elements per 32x32 tile.
+  int64_t KDF;            // T [chunks,Hv,K/32,2]    (e^{G_last-G} . K)^T as A operand: tile = (32 rows of K) x (32 tokens)
+  int64_t UF;             // T [chunks,Hv,V/32,2]    U,            tile = (32-token block ri) x (32-column block)
+  int64_t VF;             // T [chunks,Hv,V/32,2]    v_new = U - W S
+  int64_t HF;             // T [chunks,Hv,V/32,K/32] state BEFORE each chunk, tile = (32 rows of K) x (32 columns of V)
   int64_t fwd_bytes;
-  int64_t DV;             // T [tokens,Hv,V]  d(v_new)
-  int64_t DH;             // T [chunks,Hv,K,V] gradient of the state AFTER each chunk
+  int64_t WF;             // T [chunks,Hv,K/32,2]    W^T as A operand (written by the forward when a backward follows)
+  int64_t QSF;            // T [chunks,Hv,K/32,2]    (scale e^G . Q)^T as A operand
+  int64_t KAF;            // T [chunks,Hv,K/32,2]    K as A operand: tile = (32 tokens) x (32 columns of K)
+  int64_t DVLF;           // T [chunks,Hv,V/32,2]    dv_local
+  int64_t DOF;            // T [chunks,Hv,V/32,2]    dO
+  int64_t DVF;            // T [chunks,Hv,V/32,2]    d(v_new)
+  int64_t DHF;            // T [chunks,Hv,V/32,K/32] gradient of the state AFTER each chunk
   int64_t DW;             // T [tokens,Hv,K]
   int64_t DQH, DKH;       // T [tokens,Hv,K]  per-value-head dq, dk before the group sum
   int64_t DG;             // f32 [tokens,Hv]  gradient w.r.t. the cumulative decay (two partial terms)
-  int64_t DB;             // f32 [tokens,Hv]
   int64_t total_bytes;
 };
 
@@ -49,19 +55,24 @@ inline ChunkWorkspace chunk_workspace_layout(const ChunkDims& d, int elem_bytes)
   w.kn = take(tok * d.Hqk * d.K * elem_bytes);
   w.G = take(tok * d.Hv * 4);
   w.Ai = take(tok * d.Hv * 64 * elem_bytes);
-  w.W = take(tok * d.Hv * d.K * elem_bytes);
+  w.WAF = take(nc * 64 * d.Hv * d.K * elem_bytes);
   w.AQ = take(tok * d.Hv * 64 * elem_bytes);
-  w.U = take(nc * 64 * d.Hv * d.V * elem_bytes);
-  w.VN = take(tok * d.Hv * d.V * elem_bytes);
-  w.H = take(nc * d.Hv * d.V * d.K * elem_bytes);
+  w.KDF = take(nc * 64 * d.Hv * d.K * elem_bytes);
+  w.UF = take(nc * 64 * d.Hv * d.V * elem_bytes);
+  w.VF = take(nc * 64 * d.Hv * d.V * elem_bytes);
+  w.HF = take(nc * d.Hv * d.V * d.K * elem_bytes);
   w.fwd_bytes = off;
-  w.DV = take(tok * d.Hv * d.V * elem_bytes);
-  w.DH = take(nc * d.Hv * d.V * d.K * elem_bytes);
+  w.WF = take(nc * 64 * d.Hv * d.K * elem_bytes);
+  w.QSF = take(nc * 64 * d.Hv * d.K * elem_bytes);
+  w.KAF = take(nc * 64 * d.Hv * d.K * elem_bytes);
+  w.DVLF = take(nc * 64 * d.Hv * d.V * elem_bytes);
+  w.DOF = take(nc * 64 * d.Hv * d.V * elem_bytes);
+  w.DVF = take(nc * 64 * d.Hv * d.V * elem_bytes);
+  w.DHF = take(nc * d.Hv * d.V * d.K * elem_bytes);
   w.DW = take(tok * d.Hv * d.K * elem_bytes);
   w.DQH = take(tok * d.Hv * d.K * elem_bytes);
   w.DKH = take(tok * d.Hv * d.K * elem_bytes);
   w.DG = take(tok * d.Hv * 4);
-  w.DB = take(tok * d.Hv * 4);
   w.total_bytes = off;
   return w;
 }

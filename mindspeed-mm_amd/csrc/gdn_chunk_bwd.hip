@@ -1,6 +1,6 @@
 // Chunked gated delta rule, backward pass.  Notation as in gdn_chunk_fwd.hip; S is the state BEFORE a
 // chunk, dS' the gradient of the state AFTER it, Gam_ij = e^{G_i - G_j}, everything per (sequence, head):
-//   dv_local = scale tril(Q K^T . Gam)^T dO                                   chunk_dv_local_kernel
+//   dv_local = scale tril(Q K^T . Gam)^T dO                                   chunk_bwd_prep_kernel
 //   dV' = (K dS') . e^{G_last-G} + dv_local                                   chunk_state_bwd_kernel
 //   dS  = e^{G_last} dS' + scale (Q . e^G)^T dO - W^T dV'                       (reverse recurrence)
 //   ds  = scale tril(dO V'^T . Gam);  dQ = scale e^G . (dO S^T) + ds K          chunk_dqkw_kernel
@@ -35,182 +35,295 @@ __device__ __forceinline__ void acc_rowdot_add(const f32x16& acc, const T* other
 }
 
 // ---------------------------------------------------------------------------------------------
-template <typename T, int DK, int BV> struct DvLocalSmem {
-  static constexpr int LDK = lds_ld<T>(DK), LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
+// chunk_bwd_prep_kernel: everything the reverse recurrence needs that is independent across chunks, written in
+// fragment order (AccB<>) so that the sequential kernel only copies contiguous 16-byte pieces:
+//   DVLF  dv_local = scale Aq^T dO                 (accumulator tiles, per 32-column block)
+//   DOF   dO as a B operand                         (lane <-> V column, registers <-> token)
+//   QSF   (scale e^G . Q)^T as an A operand         (lane <-> K column, registers <-> token)
+//   KAF   K as an A operand                         (lane <-> token, registers <-> K column)
+// ---------------------------------------------------------------------------------------------
+constexpr int kLT = 68;   // leading dimension of transposed [*][64] LDS tiles (8-byte fragment reads stay aligned)
+
+template <typename T, int DK, int NW> struct BwdPrepSmem {
+  static constexpr int LDK = lds_ld<T>(DK);
   static constexpr int off_qs = 0;
   static constexpr int off_ks = off_qs + 64 * LDK * (int)sizeof(T);
-  static constexpr int off_do = off_ks + 64 * LDK * (int)sizeof(T);
-  static constexpr int off_pt = off_do + 64 * LDV * (int)sizeof(T);
-  static constexpr int off_gs = off_pt + 64 * L64 * (int)sizeof(T);
+  static constexpr int off_aq = off_ks + 64 * LDK * (int)sizeof(T);
+  static constexpr int off_do = off_aq + 64 * kLT * (int)sizeof(T);
+  static constexpr int off_gs = off_do + 32 * NW * kLT * (int)sizeof(T);
   static constexpr int bytes = off_gs + 64 * 4;
 };
 
-template <typename T, int DK, int BV>
-__global__ __launch_bounds__(kThreads) void chunk_dv_local_kernel(
-    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ dO, const float* __restrict__ G,
-    T* __restrict__ dv, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N,
-    int Hqk, int Hv, int V, float scale) {
-  using SM = DvLocalSmem<T, DK, BV>;
-  constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64, MT = BV / 32;
+template <typename T, int DK, int NW>
+__global__ __launch_bounds__(64 * NW) void chunk_bwd_prep_kernel(
+    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ aqk, const T* __restrict__ dO,
+    const float* __restrict__ G, T* __restrict__ dvlf, T* __restrict__ dof, T* __restrict__ qsf, T* __restrict__ kaf,
+    const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V,
+    float scale) {
+  using SM = BwdPrepSmem<T, DK, NW>;
+  constexpr int LDK = SM::LDK, NT = 64 * NW, VEC = Elem<T>::kVec;
   T* Qs = reinterpret_cast<T*>(gdn_smem + SM::off_qs);
   T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
-  T* dOs = reinterpret_cast<T*>(gdn_smem + SM::off_do);
-  T* PT = reinterpret_cast<T*>(gdn_smem + SM::off_pt);
+  T* AqT = reinterpret_cast<T*>(gdn_smem + SM::off_aq);
+  T* dOT = reinterpret_cast<T*>(gdn_smem + SM::off_do);
   float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_gs);
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
-  const int tid = threadIdx.x, wave = tid >> 6;
-  const int h = blockIdx.y, hq = h / (Hv / Hqk), nvalid = s.nvalid, v0 = blockIdx.z * BV;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31;
+  const int h = blockIdx.y, hq = h / (Hv / Hqk), nvalid = s.nvalid;
+  const int vblk = blockIdx.z * NW + wave;
   const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk;
-  load_tile<T, DK>(Qs, LDK, q + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
-  load_tile<T, DK>(Ks, LDK, k + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
-  load_tile<T, BV>(dOs, LDV, dO + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
-  if (tid < 64) Gs[tid] = G[(tok0 + imin(tid, nvalid - 1)) * Hv + h];
-  __syncthreads();
-  {  // PT[j][i] = scale (k_j . q_i) e^{G_i - G_j} for i >= j
-    const int tj = wave >> 1, ti = wave & 1;
-    f32x16 acc = acc_zero();
-    if (ti >= tj) mma32<T, DK, true, true>(acc, Ks + 32 * tj * LDK, LDK, Qs + 32 * ti * LDK, LDK);
-    const int i = 32 * ti + acc_col();
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int j = 32 * tj + acc_row(r);
-      PT[j * L64 + i] = Elem<T>::from_f(i >= j ? scale * acc[r] * __expf(Gs[i] - Gs[j]) : 0.f);
-    }
+  const int64_t ch = (int64_t)blockIdx.x * Hv + h;
+
+  for (int c = tid; c < 64 * (DK / VEC); c += NT) {
+    const int row = c / (DK / VEC), cc = c % (DK / VEC);
+    const bool ok = row < nvalid;
+    st16(Qs + row * LDK + cc * VEC, ok ? ld16(q + ((tok0 + row) * Hqk + hq) * DK + cc * VEC) : zero16<T>());
+    st16(Ks + row * LDK + cc * VEC, ok ? ld16(k + ((tok0 + row) * Hqk + hq) * DK + cc * VEC) : zero16<T>());
   }
+  load_tile_t<T, 64, NT>(AqT, kLT, aqk + (tok0 * Hv + h) * 64, (int64_t)Hv * 64, nvalid, tid);
+  load_tile_t<T, 32 * NW, NT>(dOT, kLT, dO + (tok0 * Hv + h) * V + 32 * NW * blockIdx.z, (int64_t)Hv * V, nvalid, tid);
+  if (tid < 64) Gs[tid] = scale * __expf(G[(tok0 + imin(tid, nvalid - 1)) * Hv + h]);
   __syncthreads();
-  T* dvg = dv + (tok0 * Hv + h) * V + v0;
-  for (int tt = wave; tt < 2 * MT; tt += 4) {
-    const int ri = tt & 1, cj = tt >> 1;
+
+  AccB<T> df[2];
+#pragma unroll
+  for (int ti = 0; ti < 2; ++ti) {
+    frags_from_lds<T>(df[ti], dOT + (32 * wave + l32) * kLT + 32 * ti);
+    df[ti].store(dof + ((ch * (V / 32) + vblk) * 2 + ti) * 1024);
+  }
+#pragma unroll
+  for (int rj = 0; rj < 2; ++rj) {          // dv_local[j] = scale sum_{i >= j} Aq[i][j] dO[i]
     f32x16 acc = acc_zero();
-    mma32<T, 64, true, false>(acc, PT + 32 * ri * L64, L64, dOs + 32 * cj, LDV);
-    acc_to_global(acc, dvg, (int64_t)Hv * V, 32 * ri, 32 * cj, nvalid);
+#pragma unroll
+    for (int ti = rj; ti < 2; ++ti) mma32_accb<T>(acc, AqT + (32 * rj + l32) * kLT + 32 * ti, df[ti]);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] *= scale;
+    AccB<T> out;
+    out.pack(acc);
+    out.store(dvlf + ((ch * (V / 32) + vblk) * 2 + rj) * 1024);
+  }
+  if (blockIdx.z == 0) {
+    IdentityFrag<T> id;
+    id.init();
+    for (int tt = wave; tt < 2 * (DK / 32); tt += NW) {
+      const int tj = tt & 1, kt = tt >> 1;
+      const int64_t tile = (ch * (DK / 32) + kt) * 2 + tj;
+      AccB<T> f;
+      frags_from_lds<T>(f, Ks + (32 * tj + l32) * LDK + 32 * kt);
+      f.store(kaf + tile * 1024);
+      frags_from_lds<T>(f, Qs + (32 * tj + l32) * LDK + 32 * kt);
+      f32x16 qt = mfma_transpose<T>(f, id);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) qt[r] *= Gs[32 * tj + acc_row(r)];
+      f.pack(qt);
+      f.store(qsf + tile * 1024);
+    }
   }
 }
 
 // ---------------------------------------------------------------------------------------------
-// reverse recurrence; the transposed state-gradient slab dS^T[BV, DK] lives in accumulators
+// chunk_state_bwd_kernel: the reverse recurrence, mirror of chunk_state_kernel.  One compute wave owns a 32-column
+// slab of dS[K, 32] in fp32 accumulators and per chunk (last to first) does
+//     dV' = e^{G_last-G} . (K dS) + dv_local          dS <- e^{G_last} dS + (scale e^G . Q)^T dO - W^T dV'
+// with dS and dV' used as B operands straight from accumulator registers.  dS (gradient of the state AFTER the
+// chunk) and dV' leave in fragment order.  Loader waves copy the A operands (K, Q^T, W^T: `big` stages) and the
+// per-slab dv_local / dO fragments (`small` stage) from contiguous fragment-order blocks.
 // ---------------------------------------------------------------------------------------------
-template <typename T, int DK, int BV> struct StateBwdSmem {
-  static constexpr int LDK = lds_ld<T>(DK), LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
-  static constexpr int off_ks = 0;
-  static constexpr int off_qs = off_ks + 64 * LDK * (int)sizeof(T);
-  static constexpr int off_ws = off_qs + 64 * LDK * (int)sizeof(T);
-  static constexpr int off_dsb = off_ws + 64 * LDK * (int)sizeof(T);
-  static constexpr int off_do = off_dsb + BV * LDK * (int)sizeof(T);
-  static constexpr int off_dvt = off_do + 64 * LDV * (int)sizeof(T);
-  static constexpr int off_gs = off_dvt + BV * L64 * (int)sizeof(T);
-  static constexpr int bytes = off_gs + 2 * 64 * 4;
+template <typename T, int DK, int NW, int STAGES> struct StateBwdSmem {
+  static constexpr int big = 3 * 64 * DK * (int)sizeof(T) + 64 * 4 + 16;   // K, Q^T, W^T images, decay[64], G_last
+  static constexpr int off_small = STAGES * big;
+  static constexpr int bytes = off_small + 2 * NW * 2048 * (int)sizeof(T);
 };
 
-template <typename T, int DK, int BV>
-__global__ __launch_bounds__(kThreads) void chunk_state_bwd_kernel(
-    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ w, const T* __restrict__ dO, T* dv,
-    const float* __restrict__ G, const float* __restrict__ dht, float* __restrict__ dh0, T* __restrict__ dhbuf,
-    const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int Hqk, int Hv, int V,
-    float scale) {
-  using SM = StateBwdSmem<T, DK, BV>;
-  constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64;
-  constexpr int MT = BV / 32, NTC = DK / 32, NS = (MT * NTC + 3) / 4;
-  T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
-  T* Qs = reinterpret_cast<T*>(gdn_smem + SM::off_qs);
-  T* Ws = reinterpret_cast<T*>(gdn_smem + SM::off_ws);
-  T* dSb = reinterpret_cast<T*>(gdn_smem + SM::off_dsb);
-  T* dOs = reinterpret_cast<T*>(gdn_smem + SM::off_do);
-  T* dVT = reinterpret_cast<T*>(gdn_smem + SM::off_dvt);
-  float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_gs);
-  float* qsc = Gs + 64;
+template <typename T, int DK, int NW, int STAGES>
+__global__ __launch_bounds__(128 * NW) void chunk_state_bwd_kernel(
+    const T* __restrict__ kaf, const T* __restrict__ qsf, const T* __restrict__ wf, const T* __restrict__ dvlf,
+    const T* __restrict__ dof, const float* __restrict__ G, const float* __restrict__ dht, float* __restrict__ dh0,
+    T* __restrict__ dvf, T* __restrict__ dhf, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets,
+    int T_len, int Hv, int V) {
+  using SM = StateBwdSmem<T, DK, NW, STAGES>;
+  constexpr int NT = 64 * NW, VEC = Elem<T>::kVec, NKT = DK / 32;
+  constexpr int CW = 64 * (DK / VEC) / NT, CUL = NW * 2048 / VEC / NT, TILE = 64 * DK;
+  static_assert(64 * (DK / VEC) % NT == 0 && (NW * 2048 / VEC) % NT == 0, "tile chunks must divide over the loaders");
+  static_assert(STAGES == 1 || STAGES == 2, "one or two big LDS stages");
 
-  const int tid = threadIdx.x, wave = tid >> 6;
-  const int n = blockIdx.x / Hv, h = blockIdx.x % Hv, hq = h / (Hv / Hqk);
-  const int v0 = blockIdx.y * BV;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n = blockIdx.x / Hv, h = blockIdx.x % Hv;
   const int64_t bos = cu ? cu[n] : (int64_t)n * T_len;
   const int len = cu ? (int)(cu[n + 1] - bos) : T_len;
   const int nchunks = (len + kChunk - 1) / kChunk;
   const int64_t chunk_base = cu ? chunk_offsets[n] : (int64_t)n * ((T_len + kChunk - 1) / kChunk);
+  T* small = reinterpret_cast<T*>(gdn_smem + SM::off_small);   // [dv_local | dO], NW slabs x 2 tiles each
 
-  f32x16 dS[NS];
+  // step s = 0 .. nchunks-1 handles chunk nchunks-1-s
+  if (wave >= NW) {
+    // ================= loader waves =================
+    const int lt = tid - NT;
+    constexpr int DEPTH = (STAGES == 2) ? 2 : 1;
+    Vec16<T> pk[DEPTH][CW], pq[DEPTH][CW], pw[DEPTH][CW], pl[DEPTH][CUL], pd[DEPTH][CUL];
+    float pdec[DEPTH], pgl[DEPTH];
+    auto issue = [&](int st, int set) {
+      const int c = nchunks - 1 - st;
+      const int64_t tok0 = bos + (int64_t)c * kChunk;
+      const int nvalid = imin(kChunk, len - c * kChunk);
+      const int64_t ch = (chunk_base + c) * Hv + h;
 #pragma unroll
-  for (int i = 0; i < NS; ++i) {
-    const int tt = wave + 4 * i;
-    dS[i] = acc_zero();
-    if (tt < MT * NTC && dht != nullptr) {
-      const int mi = tt % MT, ni = tt / MT;
-      const int kcol = 32 * ni + acc_col();
+      for (int i = 0; i < CW; ++i) {
+        const int id = lt + i * NT;
+        pk[set][i] = ld16(kaf + ch * TILE + id * VEC);
+        pq[set][i] = ld16(qsf + ch * TILE + id * VEC);
+        pw[set][i] = ld16(wf + ch * TILE + id * VEC);
+      }
+      const int64_t sl = (ch * (V / 32) + blockIdx.y * NW) * 2048;
+#pragma unroll
+      for (int i = 0; i < CUL; ++i) {
+        pl[set][i] = ld16(dvlf + sl + (lt + i * NT) * VEC);
+        pd[set][i] = ld16(dof + sl + (lt + i * NT) * VEC);
+      }
+      pgl[set] = G[(tok0 + nvalid - 1) * Hv + h];
+      pdec[set] = __expf(pgl[set] - G[(tok0 + imin(lt & 63, nvalid - 1)) * Hv + h]);
+    };
+    auto commit_big = [&](int set, int buf) {
+      unsigned char* base = gdn_smem + buf * SM::big;
+      T* Ka = reinterpret_cast<T*>(base);
+      T* Qa = Ka + TILE;
+      T* Wa = Qa + TILE;
+      float* dec = reinterpret_cast<float*>(Wa + TILE);
+#pragma unroll
+      for (int i = 0; i < CW; ++i) {
+        const int id = lt + i * NT;
+        st16(Ka + id * VEC, pk[set][i]);
+        st16(Qa + id * VEC, pq[set][i]);
+        st16(Wa + id * VEC, pw[set][i]);
+      }
+      if (lt < 64) dec[lt] = pdec[set];
+      if (lt == 0) dec[64] = pgl[set];
+    };
+    auto commit_small = [&](int set) {
+#pragma unroll
+      for (int i = 0; i < CUL; ++i) {
+        st16(small + (lt + i * NT) * VEC, pl[set][i]);
+        st16(small + NW * 2048 + (lt + i * NT) * VEC, pd[set][i]);
+      }
+    };
+    if (STAGES == 2) {
+      if (nchunks > 0) { issue(0, 0); commit_big(0, 0); commit_small(0); }
+#pragma unroll
+      for (int j = 1; j <= DEPTH; ++j)
+        if (j < nchunks) issue(j, j % DEPTH);
+      for (int s0 = 0; s0 < nchunks; s0 += DEPTH) {
+#pragma unroll
+        for (int u = 0; u < DEPTH; ++u) {
+          const int st = s0 + u;
+          if (st < nchunks) {
+            GDN_LDS_BARRIER();              // (A) step st staged
+            if (st + 1 < nchunks) commit_big((u + 1) % DEPTH, (st + 1) & 1);
+            GDN_LDS_BARRIER();              // (B) the compute waves have taken their dv_local / dO fragments
+            if (st + 1 < nchunks) {
+              commit_small((u + 1) % DEPTH);
+              if (st + 1 + DEPTH < nchunks) issue(st + 1 + DEPTH, (u + 1) % DEPTH);
+            }
+          }
+        }
+      }
+    } else {
+      for (int st = 0; st < nchunks; ++st) {
+        if (st > 0) GDN_LDS_BARRIER();      // (C) the single big stage is free again
+        issue(st, 0);
+        commit_big(0, 0);
+        commit_small(0);
+        GDN_LDS_BARRIER();                  // (A)
+        GDN_LDS_BARRIER();                  // (B)
+      }
+    }
+    return;
+  }
+
+  // ================= compute waves =================
+  const int vblk = blockIdx.y * NW + wave, v0 = 32 * vblk;
+  f32x16 dS[NKT];
+#pragma unroll
+  for (int kt = 0; kt < NKT; ++kt) {
+    dS[kt] = acc_zero();
+    if (dht != nullptr) {
 #pragma unroll
       for (int r = 0; r < 16; ++r)
-        dS[i][r] = dht[(((int64_t)n * Hv + h) * DK + kcol) * V + v0 + 32 * mi + acc_row(r)];
+        dS[kt][r] = dht[(((int64_t)n * Hv + h) * DK + 32 * kt + acc_row(r)) * V + v0 + acc_col()];
     }
   }
+  for (int st = 0; st < nchunks; ++st) {
+    const int c = nchunks - 1 - st;
+    const int buf = (STAGES == 2) ? (st & 1) : 0;
+    GDN_LDS_BARRIER();                      // (A)
+    AccB<T> dvl[2], dob[2];
+    dvl[0].load(small + wave * 2048);
+    dvl[1].load(small + wave * 2048 + 1024);
+    dob[0].load(small + NW * 2048 + wave * 2048);
+    dob[1].load(small + NW * 2048 + wave * 2048 + 1024);
+    GDN_LDS_BARRIER();                      // (B)
+    unsigned char* base = gdn_smem + buf * SM::big;
+    const T* Ka = reinterpret_cast<const T*>(base);
+    const T* Qa = Ka + TILE;
+    const T* Wa = Qa + TILE;
+    const float* dec = reinterpret_cast<const float*>(Wa + TILE);
+    const float glast = dec[64];
+    const int64_t tile0 = ((chunk_base + c) * Hv + h) * (V / 32) + vblk;
 
-  for (int c = nchunks - 1; c >= 0; --c) {
-    const int64_t tok0 = bos + (int64_t)c * kChunk;
-    const int nvalid = imin(kChunk, len - c * kChunk);
-    T* dhg = dhbuf + ((chunk_base + c) * Hv + h) * DK * V + v0;      // [K][V]: this slab is columns v0..v0+BV
+    AccB<T> dSb[NKT];
 #pragma unroll
-    for (int i = 0; i < NS; ++i) {
-      const int tt = wave + 4 * i;
-      if (tt < MT * NTC) {
-        const int mi = tt % MT, ni = tt / MT;
-        acc_to_lds(dS[i], dSb, LDK, 32 * mi, 32 * ni);
-        const int kcol = 32 * ni + acc_col();
+    for (int kt = 0; kt < NKT; ++kt) {
+      dSb[kt].pack(dS[kt]);
+      dSb[kt].store(dhf + (tile0 * NKT + kt) * 1024);
+    }
+    // dV' = e^{G_last-G} . (K dS) + dv_local
+    f32x16 a0 = acc_zero(), a1 = acc_zero();
 #pragma unroll
-        for (int r = 0; r < 16; ++r) dhg[(int64_t)kcol * V + 32 * mi + acc_row(r)] = Elem<T>::from_f(dS[i][r]);
+    for (int kt = 0; kt < NKT; ++kt) {
+      AccB<T> ka;
+      ka.load(Ka + (kt * 2 + 0) * 1024);
+      mma32_ff<T>(a0, ka, dSb[kt]);
+      ka.load(Ka + (kt * 2 + 1) * 1024);
+      mma32_ff<T>(a1, ka, dSb[kt]);
+    }
+    AccB<T> dvb[2];
+    {
+      const f32x16 l0 = dvl[0].unpack(), l1 = dvl[1].unpack();
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        a0[r] = a0[r] * dec[acc_row(r)] + l0[r];
+        a1[r] = a1[r] * dec[32 + acc_row(r)] + l1[r];
       }
     }
-    if (tid < 64) {
-      const float gv = G[(tok0 + imin(tid, nvalid - 1)) * Hv + h];
-      Gs[tid] = gv;
-      qsc[tid] = scale * __expf(gv);
-    }
-    __syncthreads();
-    load_tile<T, DK>(Ks, LDK, k + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
-    load_tile_scaled<T, DK>(Qs, LDK, q + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, qsc, tid);
-    load_tile<T, DK>(Ws, LDK, w + (tok0 * Hv + h) * DK, (int64_t)Hv * DK, nvalid, tid);
-    load_tile<T, BV>(dOs, LDV, dO + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
-    __syncthreads();
-    const float glast = Gs[63];
-    T* dvg = dv + (tok0 * Hv + h) * V + v0;
-    for (int tt = wave; tt < 2 * MT; tt += 4) {
-      const int ri = tt & 1, cj = tt >> 1;
-      f32x16 a = acc_zero();
-      mma32<T, DK, true, true>(a, Ks + 32 * ri * LDK, LDK, dSb + 32 * cj * LDK, LDK);
-      const f32x16 loc = acc_from_global(dvg, (int64_t)Hv * V, 32 * ri, 32 * cj, nvalid);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) a[r] = a[r] * __expf(glast - Gs[32 * ri + acc_row(r)]) + loc[r];
-      acc_to_global(a, dvg, (int64_t)Hv * V, 32 * ri, 32 * cj, nvalid);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) a[r] = (32 * ri + acc_row(r) < nvalid) ? -a[r] : 0.f;
-      acc_to_lds_t(a, dVT, L64, 32 * ri, 32 * cj);
-    }
-    __syncthreads();
+    dvb[0].pack(a0);
+    dvb[1].pack(a1);
+    dvb[0].store(dvf + (tile0 * 2 + 0) * 1024);
+    dvb[1].store(dvf + (tile0 * 2 + 1) * 1024);
+    dvb[0].negate();
+    dvb[1].negate();
+    // dS <- e^{G_last} dS + (scale e^G . Q)^T dO - W^T dV'
     const float eg = __expf(glast);
 #pragma unroll
-    for (int i = 0; i < NS; ++i) {
-      const int tt = wave + 4 * i;
-      if (tt < MT * NTC) {
-        const int mi = tt % MT, ni = tt / MT;
+    for (int kt = 0; kt < NKT; ++kt) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) dS[i][r] *= eg;
-        mma32<T, 64, false, false>(dS[i], dOs + 32 * mi, LDV, Qs + 32 * ni, LDK);
-        mma32<T, 64, true, false>(dS[i], dVT + 32 * mi * L64, L64, Ws + 32 * ni, LDK);
+      for (int r = 0; r < 16; ++r) dS[kt][r] *= eg;
+#pragma unroll
+      for (int tj = 0; tj < 2; ++tj) {
+        AccB<T> af;
+        af.load(Qa + (kt * 2 + tj) * 1024);
+        mma32_ff<T>(dS[kt], af, dob[tj]);
+        af.load(Wa + (kt * 2 + tj) * 1024);
+        mma32_ff<T>(dS[kt], af, dvb[tj]);
       }
     }
-    __syncthreads();
+    if (STAGES == 1 && st + 1 < nchunks) GDN_LDS_BARRIER();   // (C)
   }
-
   if (dh0 != nullptr) {
 #pragma unroll
-    for (int i = 0; i < NS; ++i) {
-      const int tt = wave + 4 * i;
-      if (tt < MT * NTC) {
-        const int mi = tt % MT, ni = tt / MT;
-        const int kcol = 32 * ni + acc_col();
+    for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          dh0[(((int64_t)n * Hv + h) * DK + kcol) * V + v0 + 32 * mi + acc_row(r)] = dS[i][r];
-      }
-    }
+      for (int r = 0; r < 16; ++r)
+        dh0[(((int64_t)n * Hv + h) * DK + 32 * kt + acc_row(r)) * V + v0 + acc_col()] = dS[kt][r];
   }
 }
 
@@ -230,8 +343,8 @@ template <typename T, int DK, int BV> struct DqkwSmem {
 
 template <typename T, int DK, int BV>
 __global__ __launch_bounds__(kThreads) void chunk_dqkw_kernel(
-    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ vn, const T* __restrict__ dvn,
-    const T* __restrict__ dO, const T* __restrict__ hbuf, const T* __restrict__ dhbuf, const float* __restrict__ G,
+    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ vf, const T* __restrict__ dvf,
+    const T* __restrict__ dO, const T* __restrict__ hf, const T* __restrict__ dhf, const float* __restrict__ G,
     T* __restrict__ dqh, T* __restrict__ dkh, T* __restrict__ dwb, float* __restrict__ dG,
     const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V,
     float scale) {
@@ -258,7 +371,7 @@ __global__ __launch_bounds__(kThreads) void chunk_dqkw_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int h = blockIdx.y, hq = h / (Hv / Hqk), nvalid = s.nvalid;
   const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk;
-  const int64_t hoff = ((int64_t)blockIdx.x * Hv + h) * V * DK;
+  const int64_t ch = (int64_t)blockIdx.x * Hv + h;
 
   if (tid < 64) {
     Gs[tid] = G[(tok0 + imin(tid, nvalid - 1)) * Hv + h];
@@ -275,10 +388,19 @@ __global__ __launch_bounds__(kThreads) void chunk_dqkw_kernel(
     const int v0 = vb * BV;
     if (vb > 0) __syncthreads();
     load_tile<T, BV>(dOs, LDV, dO + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
-    load_tile<T, BV>(Vps, LDV, vn + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
-    load_tile<T, BV>(dVs, LDV, dvn + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
-    load_tile<T, BV, DK>(Sb, LDV, hbuf + hoff + v0, (int64_t)V, DK, tid);       // S[kd][v0..v0+BV)
-    load_tile<T, BV, DK>(dSb, LDV, dhbuf + hoff + v0, (int64_t)V, DK, tid);
+    // v_new, d(v_new), S and dS' arrive in fragment order: one 32x32 tile per wave at a time into row-major LDS
+    for (int t = wave; t < 2 * (BV / 32); t += 4) {
+      const int ri = t & 1, vb32 = t >> 1;
+      const int64_t tile = ((ch * (V / 32) + v0 / 32 + vb32) * 2 + ri) * 1024;
+      frag_tile_to_lds<T>(Vps, LDV, 32 * ri, 32 * vb32, vf + tile);
+      frag_tile_to_lds<T>(dVs, LDV, 32 * ri, 32 * vb32, dvf + tile);
+    }
+    for (int t = wave; t < (DK / 32) * (BV / 32); t += 4) {
+      const int kt = t % (DK / 32), vb32 = t / (DK / 32);
+      const int64_t tile = ((ch * (V / 32) + v0 / 32 + vb32) * (DK / 32) + kt) * 1024;
+      frag_tile_to_lds<T>(Sb, LDV, 32 * kt, 32 * vb32, hf + tile);
+      frag_tile_to_lds<T>(dSb, LDV, 32 * kt, 32 * vb32, dhf + tile);
+    }
     __syncthreads();
     for (int e = tid; e < DK * BV; e += kThreads) {
       const int r = e / BV, c = e % BV;
@@ -366,7 +488,7 @@ template <typename T, int DK, int BV> struct WySmem {
 template <typename T, int DK, int BV>
 __global__ __launch_bounds__(kThreads) void chunk_wy_bwd_kernel(
     const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ beta, const float* __restrict__ G,
-    const T* __restrict__ Ai, const T* __restrict__ dwb, const T* __restrict__ dvn, T* dkh, const float* dG1,
+    const T* __restrict__ Ai, const T* __restrict__ dwb, const T* __restrict__ dvf, T* dkh, const float* dG1,
     T* __restrict__ dv_out, float* __restrict__ dbeta, float* __restrict__ dg, const int64_t* __restrict__ cu,
     const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V) {
   using SM = WySmem<T, DK, BV>;
@@ -431,7 +553,11 @@ __global__ __launch_bounds__(kThreads) void chunk_wy_bwd_kernel(
     const int v0 = vb * BV;
     if (vb > 0) __syncthreads();
     load_tile<T, BV>(Vs, LDV, v + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
-    load_tile<T, BV>(dUs, LDV, dvn + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
+    for (int t = wave; t < 2 * (BV / 32); t += 4) {      // d(v_new) tiles arrive in fragment order
+      const int ri = t & 1, vb32 = t >> 1;
+      frag_tile_to_lds<T>(dUs, LDV, 32 * ri, 32 * vb32,
+                          dvf + ((((int64_t)blockIdx.x * Hv + h) * (V / 32) + v0 / 32 + vb32) * 2 + ri) * 1024);
+    }
     __syncthreads();
     T* dvg = dv_out + (tok0 * Hv + h) * V + v0;
 #pragma unroll
@@ -569,7 +695,7 @@ template <typename K> static int set_lds_b(K kernel, int bytes) {
                                   bytes);
 }
 
-template <typename T, int DK, int BVL, int BVS, int BVQ, int BVW>
+template <typename T, int DK, int NW, int STAGES, int BVQ, int BVW>
 static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const void* q, const void* k, const void* v,
                             const float* beta, const int64_t* cu, const void* dO, const float* dht, void* dq, void* dk,
                             void* dv, float* dg, float* dbeta, float* dh0, unsigned char* ws, float scale, int l2norm,
@@ -581,51 +707,56 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   const T* kk = l2norm ? reinterpret_cast<const T*>(ws + L.kn) : (const T*)k;
   const float* G = reinterpret_cast<const float*>(ws + L.G);
   const T* Ai = reinterpret_cast<const T*>(ws + L.Ai);
-  const T* W = reinterpret_cast<const T*>(ws + L.W);
-  const T* VN = reinterpret_cast<const T*>(ws + L.VN);
-  const T* H = reinterpret_cast<const T*>(ws + L.H);
-  T* DV = reinterpret_cast<T*>(ws + L.DV);
-  T* DH = reinterpret_cast<T*>(ws + L.DH);
+  const T* AQ = reinterpret_cast<const T*>(ws + L.AQ);
+  const T* WF = reinterpret_cast<const T*>(ws + L.WF);
+  const T* VF = reinterpret_cast<const T*>(ws + L.VF);
+  const T* HF = reinterpret_cast<const T*>(ws + L.HF);
+  T* QSF = reinterpret_cast<T*>(ws + L.QSF);
+  T* KAF = reinterpret_cast<T*>(ws + L.KAF);
+  T* DVLF = reinterpret_cast<T*>(ws + L.DVLF);
+  T* DOF = reinterpret_cast<T*>(ws + L.DOF);
+  T* DVF = reinterpret_cast<T*>(ws + L.DVF);
+  T* DHF = reinterpret_cast<T*>(ws + L.DHF);
   T* DW = reinterpret_cast<T*>(ws + L.DW);
   T* DQH = reinterpret_cast<T*>(ws + L.DQH);
   T* DKH = reinterpret_cast<T*>(ws + L.DKH);
   float* DG = reinterpret_cast<float*>(ws + L.DG);
   {
-    auto kern = chunk_dv_local_kernel<T, DK, BVL>;
-    constexpr int smem = DvLocalSmem<T, DK, BVL>::bytes;
+    auto kern = chunk_bwd_prep_kernel<T, DK, NW>;
+    constexpr int smem = BwdPrepSmem<T, DK, NW>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
-    GDN_LAUNCH(kKernDvLocal, st, kern, dim3(nc, d.Hv, d.V / BVL), dim3(kThreads), smem, st, qq, kk, (const T*)dO, G, DV, cu,
-                       chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale);
+    GDN_LAUNCH(kKernDvLocal, st, kern, dim3(nc, d.Hv, d.V / (32 * NW)), dim3(64 * NW), smem, st, qq, kk, AQ,
+               (const T*)dO, G, DVLF, DOF, QSF, KAF, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale);
   }
   {
-    auto kern = chunk_state_bwd_kernel<T, DK, BVS>;
-    constexpr int smem = StateBwdSmem<T, DK, BVS>::bytes;
+    auto kern = chunk_state_bwd_kernel<T, DK, NW, STAGES>;
+    constexpr int smem = StateBwdSmem<T, DK, NW, STAGES>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
-    GDN_LAUNCH(kKernStateBwd, st, kern, dim3(d.N * d.Hv, d.V / BVS), dim3(kThreads), smem, st, qq, kk, W, (const T*)dO, DV, G,
-                       dht, dh0, DH, cu, chunk_offsets, d.T, d.Hqk, d.Hv, d.V, scale);
+    GDN_LAUNCH(kKernStateBwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NW)), dim3(128 * NW), smem, st, (const T*)KAF,
+               (const T*)QSF, WF, (const T*)DVLF, (const T*)DOF, G, dht, dh0, DVF, DHF, cu, chunk_offsets, d.T, d.Hv,
+               d.V);
   }
   {
     auto kern = chunk_dqkw_kernel<T, DK, BVQ>;
     constexpr int smem = DqkwSmem<T, DK, BVQ>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
-    GDN_LAUNCH(kKernDqkw, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, VN, (const T*)DV, (const T*)dO, H,
-                       (const T*)DH, G, DQH, DKH, DW, DG, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale);
+    GDN_LAUNCH(kKernDqkw, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, VF, (const T*)DVF, (const T*)dO,
+               HF, (const T*)DHF, G, DQH, DKH, DW, DG, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale);
   }
   {
     auto kern = chunk_wy_bwd_kernel<T, DK, BVW>;
     constexpr int smem = WySmem<T, DK, BVW>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
-    GDN_LAUNCH(kKernWyBwd, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, kk, (const T*)v, beta, G, Ai, (const T*)DW,
-                       (const T*)DV, DKH, (const float*)DG, (T*)dv, dbeta, dg, cu, chunk_offsets, d.T, d.N, d.Hqk,
-                       d.Hv, d.V);
+    GDN_LAUNCH(kKernWyBwd, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, kk, (const T*)v, beta, G, Ai,
+               (const T*)DW, (const T*)DVF, DKH, (const float*)DG, (T*)dv, dbeta, dg, cu, chunk_offsets, d.T, d.N,
+               d.Hqk, d.Hv, d.V);
   }
   {
     constexpr int LPR = DK / Elem<T>::kVec;
     const int64_t rows = tok * d.Hqk;
     GDN_LAUNCH(kKernQkFinalize, st, (qk_grad_finalize_kernel<T, DK>),
-                       dim3((unsigned)((rows + kThreads / LPR - 1) / (kThreads / LPR)), 2), dim3(kThreads), 0, st,
-                       (const T*)DQH, (const T*)DKH, (const T*)q, (const T*)k, (T*)dq, (T*)dk, rows, d.Hqk, d.Hv,
-                       l2norm);
+               dim3((unsigned)((rows + kThreads / LPR - 1) / (kThreads / LPR)), 2), dim3(kThreads), 0, st,
+               (const T*)DQH, (const T*)DKH, (const T*)q, (const T*)k, (T*)dq, (T*)dk, rows, d.Hqk, d.Hv, l2norm);
   }
   return (int)hipGetLastError();
 }
@@ -649,16 +780,19 @@ extern "C" int gdn_chunk_bwd(const void* q, const void* k, const void* v, const 
   if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
   unsigned char* ws = static_cast<unsigned char*>(workspace);
   hipStream_t st = (hipStream_t)stream;
-#define GDN_BWD(T_, DK_, BVL_, BVS_, BVQ_, BVW_)                                                                   \
-  return chunk_bwd_launch<T_, DK_, BVL_, BVS_, BVQ_, BVW_>(d, L, q, k, v, beta, cu_seqlens, d_o, d_final_state, dq, \
-                                                            dk, dv, dg, dbeta, d_initial_state, ws, scale,         \
-                                                            use_qk_l2norm, st)
+#define GDN_BWD(T_, DK_, NW_, ST_, BVQ_, BVW_)                                                                     \
+  return chunk_bwd_launch<T_, DK_, NW_, ST_, BVQ_, BVW_>(d, L, q, k, v, beta, cu_seqlens, d_o, d_final_state, dq, \
+                                                          dk, dv, dg, dbeta, d_initial_state, ws, scale,         \
+                                                          use_qk_l2norm, st)
+  const bool wide = (V % 128 == 0);
   if (dtype == 1) {
-    if (K == 128) GDN_BWD(bf16_t, 128, 64, 64, 64, 64);
-    GDN_BWD(bf16_t, 64, 64, 64, 64, 64);
+    if (K == 128 && wide) GDN_BWD(bf16_t, 128, 4, 2, 64, 64);
+    if (K == 128) GDN_BWD(bf16_t, 128, 2, 2, 64, 64);
+    if (wide) GDN_BWD(bf16_t, 64, 4, 2, 64, 64);
+    GDN_BWD(bf16_t, 64, 2, 2, 64, 64);
   } else {
-    if (K == 128) GDN_BWD(float, 128, 64, 32, 64, 64);
-    GDN_BWD(float, 64, 64, 32, 64, 64);
+    if (K == 128) GDN_BWD(float, 128, 2, 1, 64, 64);
+    GDN_BWD(float, 64, 2, 2, 64, 64);
   }
 #undef GDN_BWD
 }

@@ -6,9 +6,10 @@
 //     S <- e^{G_last} S + (e^{G_last - G} . K)^T V'
 // Math: mindspeed_mm/fsdp/models/qwen3_5/modeling_qwen3_5.py:398-475; stage split as in
 // mindspeed_mm/fsdp/ops/gdn/chunk_gated_delta_rule.py:30-85 (cumsum, KK^T, tril solve, W/U, state
-// recurrence, output), fused here into two launches:
+// recurrence, output), fused here into three launches:
 //     chunk_prep_kernel   per (chunk, head):  G, Tm, W, U, tril(QK^T . Gam)      -- MFMA + fp32 block solve
-//     chunk_fwd_kernel    per (sequence, head, 32-column state slab), sequential in chunks: V', O, S
+//     chunk_state_kernel  per (sequence, head, 32-column state slab), sequential in chunks: V', S
+//     chunk_out_kernel    per (chunk, head, 32-column block): O
 // A ragged last chunk is zero padded in LDS (k = v = beta = g = 0 is exact for this recurrence).
 #include "gdn_chunk.h"
 #include "gdn_common.h"
@@ -76,9 +77,8 @@ __global__ void l2norm_fwd_kernel(const T* __restrict__ x0, const T* __restrict_
 // ---------------------------------------------------------------------------------------------
 // chunk_prep_kernel: everything that is independent across chunks.
 //   G (cumulative decay), Tm = (I+L)^-1, W = Tm (beta e^G K), U = Tm (beta V), Aq = tril(Q K^T . Gam)
-// U is written in accumulator-fragment order -- for tile (32-row block ri, 32-column block vb) lane l stores its 16
-// accumulator values as 16/VEC vectors at U[chunk][head][vb][ri][part][l][0..VEC) -- which is exactly how the
-// recurrence kernel reads it back (straight copy to LDS, conflict-free 16-byte fragment reads).
+// U is written in fragment order (AccB<>): tile (32-token block ri) x (32-column block vb) at
+// U[chunk][head][vb][ri][1024], 16 bytes per lane per k-group -- the recurrence kernel copies it straight to LDS.
 // ---------------------------------------------------------------------------------------------
 template <typename T, int DK, int BV> struct PrepSmem {
   static constexpr int LDK = lds_ld<T>(DK), LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
@@ -97,7 +97,7 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ g,
     const float* __restrict__ beta, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets,
     float* __restrict__ G_out, T* __restrict__ Ai_out, T* __restrict__ W_out, T* __restrict__ U_out,
-    T* __restrict__ Aq_out, int T_len, int N, int Hqk, int Hv, int V) {
+    T* __restrict__ Aq_out, T* __restrict__ KD_out, T* __restrict__ WF_out, int T_len, int N, int Hqk, int Hv, int V) {
   using SM = PrepSmem<T, DK, BV>;
   constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64, VEC = Elem<T>::kVec;
   T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
@@ -152,6 +152,23 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
       const float gam = i >= j ? __expf(Gs[i] - Gs[j]) : 0.f;
       As[i * kLF + j] = i > j ? bs[i] * acc[r] * gam : 0.f;
       if (i < nvalid) aqg[(int64_t)i * Hv * 64 + j] = Elem<T>::from_f(aq[r] * gam);
+    }
+  }
+  // (e^{G_last-G} . K)^T as A-operand fragments for the state update: K tile fragments (lane <-> token) turned
+  // through the matrix core into (lane <-> K column, registers <-> token), scaled per token, stored in fragment order
+  {
+    IdentityFrag<T> id;
+    id.init();
+    const float glast = Gs[63];
+    for (int tt = wave; tt < 2 * (DK / 32); tt += 4) {
+      const int tj = tt & 1, kt = tt >> 1;
+      AccB<T> kf;
+      frags_from_lds<T>(kf, Ks + (32 * tj + (lane & 31)) * LDK + 32 * kt);
+      f32x16 kd = mfma_transpose<T>(kf, id);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) kd[r] *= __expf(glast - Gs[32 * tj + acc_row(r)]);
+      kf.pack(kd);
+      kf.store(KD_out + ((((int64_t)blockIdx.x * Hv + h) * (DK / 32) + kt) * 2 + tj) * 1024);
     }
   }
   __syncthreads();
@@ -248,14 +265,21 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
   }
   __syncthreads();
 
-  // ---- phase 4: W = Tm (beta e^G K) ----
+  // ---- phase 4: W = Tm (beta e^G K), handed on in fragment order only ----
   {
-    T* wg = W_out + (tok0 * Hv + h) * DK;
+    IdentityFrag<T> id;
+    id.init();
     for (int tt = wave; tt < 2 * (DK / 32); tt += 4) {
       const int ri = tt & 1, cj = tt >> 1;
       f32x16 acc = acc_zero();
       mma32<T, 64, true, false>(acc, Tms + 32 * ri * L64, L64, Kb + 32 * cj, LDK);
-      acc_to_global(acc, wg, (int64_t)Hv * DK, 32 * ri, 32 * cj, nvalid);
+      const int64_t tile = (((int64_t)blockIdx.x * Hv + h) * (DK / 32) + cj) * 2 + ri;
+      AccB<T> wf;
+      wf.pack(acc);              // (lane <-> K column, registers <-> token): W^T as an A operand, for the backward pass
+      if (WF_out != nullptr) wf.store(WF_out + tile * 1024);
+      const f32x16 wt = mfma_transpose<T>(wf, id);
+      wf.pack(wt);               // (lane <-> token, registers <-> K column): W as an A operand, for W S
+      wf.store(W_out + tile * 1024);
     }
   }
   // ---- phase 5: U = Tm (beta V), V block by V block, stored in fragment order ----
@@ -270,121 +294,122 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
       f32x16 acc = acc_zero();
       mma32<T, 64, true, false>(acc, Tms + 32 * ri * L64, L64, Vb + 32 * cj, LDV);
       const int vblk = vb * (BV / 32) + cj;
-      T* ug = U_out + ((((int64_t)blockIdx.x * Hv + h) * (V / 32) + vblk) * 2 + ri) * (64 * 16);
-#pragma unroll
-      for (int c = 0; c < 16 / VEC; ++c) {
-        Vec16<T> x = zero16<T>();
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) x.set(e, acc[c * VEC + e]);
-        st16(ug + (c * 64 + lane) * VEC, x);
-      }
+      AccB<T> uf;
+      uf.pack(acc);
+      uf.store(U_out + ((((int64_t)blockIdx.x * Hv + h) * (V / 32) + vblk) * 2 + ri) * 1024);
     }
   }
 }
 
 // ---------------------------------------------------------------------------------------------
-// chunk_fwd_kernel: the inter-chunk recurrence fused with the output.  One wave owns a 32-column slab of the
-// state S[K, 32] in fp32 accumulators for the whole sequence, and for every chunk does
-//     V' = U - W S        O = scale [ e^G . (Q S) + Aq V' ]        S <- e^{G_last} S + K^T (e^{G_last-G} . V')
-// Every B operand (S, V') is taken straight from accumulator registers (see frag_b_from_acc), so the waves
-// of a workgroup never exchange data and the chain W S -> V' -> S needs no LDS round trip.  The A operands
-// (W, Q, Aq row-major, K transposed) are staged in LDS by NW dedicated loader waves of the same workgroup; with
-// STAGES = 2 they run one chunk ahead of the NW compute waves and the two roles meet at one barrier per chunk.
+// chunk_state_kernel: the inter-chunk recurrence, kept as lean as possible because it is the only part of the
+// forward pass that is sequential in the chunks.  One compute wave owns a 32-column slab of the state S[K, 32] in
+// fp32 accumulators for the whole sequence and per chunk does
+//     V' = U - W S            S <- e^{G_last} S + (e^{G_last-G} . K)^T V'
+// Both B operands (S, V') are taken straight from accumulator registers (frag_b_from_acc), so the chain
+// W S -> V' -> S never touches LDS and the compute waves of a workgroup never exchange data.  S (before the chunk)
+// and V' leave the kernel in fragment order, 16 bytes per lane per k-group, for chunk_out_kernel and the backward
+// pass.  The A operands (W, the decay-scaled K^T) and U arrive in fragment order, one contiguous 16 KB block per
+// chunk and head prepared by chunk_prep_kernel (token-major tiles would be 64 rows scattered 8 KB apart), and are
+// copied to LDS in 16-byte pieces by NW loader waves of the same workgroup, which run ahead of the NW compute
+// waves: loads for chunk c+2 are in flight in registers while chunk c+1 sits in the other LDS stage; the two roles
+// meet at one barrier per chunk.
 // ---------------------------------------------------------------------------------------------
-template <typename T, int DK, int NW, int STAGES> struct FwdSmem {
-  static constexpr int LDK = lds_ld<T>(DK), L64 = lds_ld<T>(64);
+template <typename T, int DK, int NW, int STAGES> struct StateSmem {
   static constexpr int off_ws = 0;
-  static constexpr int off_qs = off_ws + 64 * LDK * (int)sizeof(T);
-  static constexpr int off_kt = off_qs + 64 * LDK * (int)sizeof(T);
-  static constexpr int off_aq = off_kt + DK * L64 * (int)sizeof(T);
-  static constexpr int off_uf = off_aq + 64 * L64 * (int)sizeof(T);
-  static constexpr int off_gs = off_uf + NW * 2 * 64 * 16 * (int)sizeof(T);
-  static constexpr int stage = off_gs + 2 * 64 * 4;
+  static constexpr int off_kt = off_ws + 64 * DK * (int)sizeof(T);
+  static constexpr int off_uf = off_kt + DK * 64 * (int)sizeof(T);
+  static constexpr int off_gl = off_uf + NW * 2048 * (int)sizeof(T);
+  static constexpr int stage = off_gl + 16;
   static constexpr int bytes = STAGES * stage;
 };
 
 template <typename T, int DK, int NW, int STAGES>
-__global__ __launch_bounds__(128 * NW) void chunk_fwd_kernel(
-    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ w, const T* __restrict__ ufrag,
-    const T* __restrict__ aqk, const float* __restrict__ G, const float* __restrict__ h0, float* __restrict__ ht,
-    T* __restrict__ o, T* __restrict__ vn, T* __restrict__ hbuf, const int64_t* __restrict__ cu,
-    const int* __restrict__ chunk_offsets, int T_len, int Hqk, int Hv, int V, float scale) {
-  using SM = FwdSmem<T, DK, NW, STAGES>;
-  constexpr int LDK = SM::LDK, L64 = SM::L64, NT = 64 * NW, VEC = Elem<T>::kVec;
-  constexpr int NKT = DK / 32;                                  // state tiles of a compute wave (rows of S)
-  constexpr int CW = 64 * (DK / VEC) / NT, CA = 64 * (64 / VEC) / NT, CU = 16 / VEC;
-  constexpr int CUL = NW * 2 * 64 * 16 / VEC / NT;              // U vectors copied by a loader thread
-  static_assert(64 * (DK / VEC) % NT == 0 && 64 * (64 / VEC) % NT == 0, "tile chunks must divide over the loaders");
+__global__ __launch_bounds__(128 * NW) void chunk_state_kernel(
+    const T* __restrict__ kdf, const T* __restrict__ w, const T* __restrict__ uf, const float* __restrict__ G,
+    const float* __restrict__ h0, float* __restrict__ ht, T* __restrict__ vf, T* __restrict__ hf,
+    const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int Hv, int V) {
+  using SM = StateSmem<T, DK, NW, STAGES>;
+  constexpr int NT = 64 * NW, VEC = Elem<T>::kVec;
+  constexpr int NKT = DK / 32;
+  constexpr int CW = 64 * (DK / VEC) / NT, CUL = NW * 2048 / VEC / NT;
+  static_assert(64 * (DK / VEC) % NT == 0 && (NW * 2048 / VEC) % NT == 0, "tile chunks must divide over the loaders");
+  static_assert(STAGES == 1 || STAGES == 2, "one or two LDS stages");
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31;
-  const int n = blockIdx.x / Hv, h = blockIdx.x % Hv, hq = h / (Hv / Hqk);
+  const int n = blockIdx.x / Hv, h = blockIdx.x % Hv;
   const int64_t bos = cu ? cu[n] : (int64_t)n * T_len;
   const int len = cu ? (int)(cu[n + 1] - bos) : T_len;
   const int nchunks = (len + kChunk - 1) / kChunk;
   const int64_t chunk_base = cu ? chunk_offsets[n] : (int64_t)n * ((T_len + kChunk - 1) / kChunk);
 
   if (wave >= NW) {
-    // ================= loader waves: global -> LDS stage, one chunk ahead of the compute waves =================
+    // ================= loader waves: straight 16-byte copies =================
     const int lt = tid - NT;
-    for (int c = 0; c < nchunks; ++c) {
-      const int buf = (STAGES == 2) ? (c & 1) : 0;
-      if (STAGES == 1 && c > 0) __syncthreads();              // (B) the single stage is free again
-      unsigned char* base = gdn_smem + buf * SM::stage;
-      T* Ws = reinterpret_cast<T*>(base + SM::off_ws);
-      T* Qs = reinterpret_cast<T*>(base + SM::off_qs);
-      T* KT = reinterpret_cast<T*>(base + SM::off_kt);
-      T* Aq = reinterpret_cast<T*>(base + SM::off_aq);
-      T* Uf = reinterpret_cast<T*>(base + SM::off_uf);
-      float* Gs = reinterpret_cast<float*>(base + SM::off_gs);
+    // DEPTH register sets: chunk j sits in set j % DEPTH from the iteration that requests it (j - DEPTH - 1) to the
+    // one that copies it to LDS (j - 1), so global loads have DEPTH chunk periods to arrive
+    constexpr int DEPTH = (STAGES == 2) ? 3 : 1;
+    Vec16<T> pw[DEPTH][CW], pk[DEPTH][CW], pu[DEPTH][CUL];
+    float glast[DEPTH];
+    auto issue = [&](int c, int set) {      // global -> registers
       const int64_t tok0 = bos + (int64_t)c * kChunk;
       const int nvalid = imin(kChunk, len - c * kChunk);
-      Vec16<T> pw[CW], pq[CW], pk[CW], pa[CA], pu[CUL];
-      const float g_last = G[(tok0 + nvalid - 1) * Hv + h];
 #pragma unroll
       for (int i = 0; i < CW; ++i) {
         const int id = lt + i * NT;
-        const int row = id / (DK / VEC), cc = id % (DK / VEC);          // row-major tiles: W, Q
-        pw[i] = row < nvalid ? ld16(w + ((tok0 + row) * Hv + h) * DK + cc * VEC) : zero16<T>();
-        pq[i] = row < nvalid ? ld16(q + ((tok0 + row) * Hqk + hq) * DK + cc * VEC) : zero16<T>();
-        const int rowt = id % kChunk, cct = id / kChunk;                 // K goes in transposed: rows fastest
-        pk[i] = rowt < nvalid ? ld16(k + ((tok0 + rowt) * Hqk + hq) * DK + cct * VEC) : zero16<T>();
+        pw[set][i] = ld16(w + ((chunk_base + c) * Hv + h) * (64 * DK) + id * VEC);
+        pk[set][i] = ld16(kdf + ((chunk_base + c) * Hv + h) * (64 * DK) + id * VEC);
       }
+      const T* ug = uf + (((chunk_base + c) * Hv + h) * (V / 32) + blockIdx.y * NW) * 2048;
 #pragma unroll
-      for (int i = 0; i < CA; ++i) {
-        const int id = lt + i * NT;
-        const int row = id / (64 / VEC), cc = id % (64 / VEC);
-        pa[i] = row < nvalid ? ld16(aqk + ((tok0 + row) * Hv + h) * 64 + cc * VEC) : zero16<T>();
-      }
-      const T* ug = ufrag + (((chunk_base + c) * Hv + h) * (V / 32) + blockIdx.y * NW) * (2 * 64 * 16);
-#pragma unroll
-      for (int i = 0; i < CUL; ++i) pu[i] = ld16(ug + (lt + i * NT) * VEC);
-      // every loader lane owns token lt%64 in the transposed K staging: its decay towards the chunk end
-      const float kdec = __expf(g_last - G[(tok0 + imin(lt & 63, nvalid - 1)) * Hv + h]);
-      if (lt < 64) Gs[lt] = G[(tok0 + imin(lt, nvalid - 1)) * Hv + h];
+      for (int i = 0; i < CUL; ++i) pu[set][i] = ld16(ug + (lt + i * NT) * VEC);
+      glast[set] = G[(tok0 + nvalid - 1) * Hv + h];
+    };
+    auto commit = [&](int set, int buf) {   // registers -> LDS stage
+      unsigned char* base = gdn_smem + buf * SM::stage;
+      T* Ws = reinterpret_cast<T*>(base + SM::off_ws);
+      T* KT = reinterpret_cast<T*>(base + SM::off_kt);
+      T* Uf = reinterpret_cast<T*>(base + SM::off_uf);
 #pragma unroll
       for (int i = 0; i < CW; ++i) {
         const int id = lt + i * NT;
-        const int row = id / (DK / VEC), cc = id % (DK / VEC);
-        st16(Ws + row * LDK + cc * VEC, pw[i]);
-        st16(Qs + row * LDK + cc * VEC, pq[i]);
-        const int rowt = id % kChunk, cct = id / kChunk;      // rowt == lt % 64 because NT is a multiple of 64
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) KT[(cct * VEC + e) * L64 + rowt] = Elem<T>::from_f(pk[i].get(e) * kdec);
+        st16(Ws + id * VEC, pw[set][i]);
+        st16(KT + id * VEC, pk[set][i]);
       }
 #pragma unroll
-      for (int i = 0; i < CUL; ++i) st16(Uf + (lt + i * NT) * VEC, pu[i]);
+      for (int i = 0; i < CUL; ++i) st16(Uf + (lt + i * NT) * VEC, pu[set][i]);
+      if (lt == 0) *reinterpret_cast<float*>(base + SM::off_gl) = glast[set];
+    };
+    if (STAGES == 2) {
+      if (nchunks > 0) { issue(0, 0); commit(0, 0); }
 #pragma unroll
-      for (int i = 0; i < CA; ++i) {
-        const int id = lt + i * NT;
-        const int row = id / (64 / VEC), cc = id % (64 / VEC);
-        st16(Aq + row * L64 + cc * VEC, pa[i]);
+      for (int j = 1; j <= DEPTH; ++j)
+        if (j < nchunks) issue(j, j % DEPTH);
+      for (int c0 = 0; c0 < nchunks; c0 += DEPTH) {
+#pragma unroll
+        for (int u = 0; u < DEPTH; ++u) {
+          const int c = c0 + u;
+          if (c < nchunks) {
+            GDN_LDS_BARRIER();              // (A) chunk c staged; the other stage (chunk c-1) is free
+            if (c + 1 < nchunks) {
+              commit((u + 1) % DEPTH, (c + 1) & 1);
+              if (c + 1 + DEPTH < nchunks) issue(c + 1 + DEPTH, (u + 1) % DEPTH);
+            }
+          }
+        }
       }
-      __syncthreads();                                         // (A) chunk c is staged
+    } else {
+      for (int c = 0; c < nchunks; ++c) {
+        if (c > 0) GDN_LDS_BARRIER();       // (B) the single stage is free again
+        issue(c, 0);
+        commit(0, 0);
+        GDN_LDS_BARRIER();                  // (A)
+      }
     }
     return;
   }
 
-  // ================= compute waves: one 32-column slab of the state each =================
+  // ================= compute waves =================
   const int vblk = blockIdx.y * NW + wave, v0 = 32 * vblk;
   f32x16 S[NKT];
 #pragma unroll
@@ -398,84 +423,153 @@ __global__ __launch_bounds__(128 * NW) void chunk_fwd_kernel(
   }
   for (int c = 0; c < nchunks; ++c) {
     const int buf = (STAGES == 2) ? (c & 1) : 0;
-    __syncthreads();                       // (A) stage `buf` holds chunk c
+    GDN_LDS_BARRIER();                        // (A) stage `buf` holds chunk c
     unsigned char* base = gdn_smem + buf * SM::stage;
     const T* Ws = reinterpret_cast<const T*>(base + SM::off_ws);
-    const T* Qs = reinterpret_cast<const T*>(base + SM::off_qs);
     const T* KT = reinterpret_cast<const T*>(base + SM::off_kt);
-    const T* Aq = reinterpret_cast<const T*>(base + SM::off_aq);
-    const T* Uf = reinterpret_cast<const T*>(base + SM::off_uf) + wave * (2 * 64 * 16);
-    const float* Gs = reinterpret_cast<const float*>(base + SM::off_gs);
-    const int64_t tok0 = bos + (int64_t)c * kChunk;
-    const int nvalid = imin(kChunk, len - c * kChunk);
-    const float glast = Gs[63];
-    int64_t row_v = V, row_hv = (int64_t)Hv * V;   // row strides of the h / o,v_new stores
-    GDN_OPAQUE(row_v);
-    GDN_OPAQUE(row_hv);
+    const T* Uf = reinterpret_cast<const T*>(base + SM::off_uf) + wave * 2048;
+    const float glast = *reinterpret_cast<const float*>(base + SM::off_gl);
+    const int64_t tile0 = ((chunk_base + c) * Hv + h) * (V / 32) + vblk;
 
     AccB<T> Sb[NKT];
 #pragma unroll
-    for (int kt = 0; kt < NKT; ++kt) Sb[kt].pack(S[kt]);
-    if (hbuf != nullptr) {                 // state before this chunk, for the backward pass
-      T* hg = hbuf + (((chunk_base + c) * Hv + h) * DK) * V + v0;
-#pragma unroll
-      for (int kt = 0; kt < NKT; ++kt) acc_to_global(S[kt], hg, row_v, 32 * kt, 0, DK);
+    for (int kt = 0; kt < NKT; ++kt) {
+      Sb[kt].pack(S[kt]);
+      Sb[kt].store(hf + (tile0 * NKT + kt) * 1024);
     }
-    GDN_PHASE_FENCE();
-    // V' = U - W S, then packed as a B operand (for O and for the state update)
+    // Hand-made software pipeline over pairs of K tiles: the LDS reads of the next group are issued before the
+    // matrix instructions of the current one (GDN_SCHED_FENCE keeps the order).
+    constexpr int NP = NKT / 2;             // K tiles are processed two at a time
+    AccB<T> Wf[2][2][2];                    // [buffer][32-token block][K tile of the pair]
+    AccB<T> Kf[2][2][2];                    // [buffer][K tile of the pair][32-token block]
+    auto load_w = [&](int b, int kp) {
+#pragma unroll
+      for (int ri = 0; ri < 2; ++ri)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) Wf[b][ri][j].load(Ws + ((2 * kp + j) * 2 + ri) * 1024);
+    };
+    auto load_k = [&](int b, int kp) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int tj = 0; tj < 2; ++tj) Kf[b][j][tj].load(KT + ((2 * kp + j) * 2 + tj) * 1024);
+    };
+    f32x16 p0 = acc_zero(), p1 = acc_zero();
     AccB<T> Vb[2];
-    T* vg = vn != nullptr ? vn + (tok0 * Hv + h) * V + v0 : nullptr;
+    load_w(0, 0);
+    if (NP > 1) load_w(1, 1);
+    GDN_SCHED_FENCE();
 #pragma unroll
-    for (int ri = 0; ri < 2; ++ri) {
-      f32x16 p = acc_zero();
+    for (int kp = 0; kp < NP; ++kp) {
+      // V' = U - W S: the two 32-token blocks are independent accumulation chains
+      if (kp == 0) load_k(0, 0);
+      if (kp == NP - 1) { Vb[0].load(Uf); Vb[1].load(Uf + 1024); if (NP > 1) load_k(1, 1); }
 #pragma unroll
-      for (int kt = 0; kt < NKT; ++kt) mma32_accb<T>(p, Ws + (32 * ri + l32) * LDK + 32 * kt, Sb[kt]);
-      f32x16 vp;
-#pragma unroll
-      for (int i = 0; i < CU; ++i) {
-        const Vec16<T> u = ld16(Uf + ((ri * CU + i) * 64 + lane) * VEC);
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) vp[i * VEC + e] = u.get(e) - p[i * VEC + e];
+      for (int j = 0; j < 2; ++j) {
+        mma32_ff<T>(p0, Wf[kp & 1][0][j], Sb[2 * kp + j]);
+        mma32_ff<T>(p1, Wf[kp & 1][1][j], Sb[2 * kp + j]);
       }
-      if (vg != nullptr) acc_to_global(vp, vg, row_hv, 32 * ri, 0, nvalid);
-      Vb[ri].pack(vp);
-      GDN_PHASE_FENCE();
+      GDN_SCHED_FENCE();
+      if (kp + 2 < NP) { load_w(kp & 1, kp + 2); GDN_SCHED_FENCE(); }
     }
-    // O = scale [ e^G . (Q S) + Aq V' ]
-    T* og = o + (tok0 * Hv + h) * V + v0;
+    {
+      const f32x16 u0 = Vb[0].unpack(), u1 = Vb[1].unpack();
 #pragma unroll
-    for (int ri = 0; ri < 2; ++ri) {
-      f32x16 oa = acc_zero();
-#pragma unroll
-      for (int kt = 0; kt < NKT; ++kt) mma32_accb<T>(oa, Qs + (32 * ri + l32) * LDK + 32 * kt, Sb[kt]);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) oa[r] *= __expf(Gs[32 * ri + acc_row(r)]);
-#pragma unroll
-      for (int tj = 0; tj <= ri; ++tj) mma32_accb<T>(oa, Aq + (32 * ri + l32) * L64 + 32 * tj, Vb[tj]);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) oa[r] *= scale;
-      acc_to_global(oa, og, row_hv, 32 * ri, 0, nvalid);
-      GDN_PHASE_FENCE();
+      for (int r = 0; r < 16; ++r) { p0[r] = u0[r] - p0[r]; p1[r] = u1[r] - p1[r]; }
     }
-    // S <- e^{G_last} S + (e^{G_last - G} . K)^T V'   (the loaders staged K already scaled)
+    Vb[0].pack(p0);
+    Vb[1].pack(p1);
+    Vb[0].store(vf + (tile0 * 2 + 0) * 1024);
+    Vb[1].store(vf + (tile0 * 2 + 1) * 1024);
+    // S <- e^{G_last} S + (e^{G_last - G} . K)^T V'   (K^T arrives already scaled, as A-operand fragments)
     const float eg = __expf(glast);
 #pragma unroll
-    for (int kt = 0; kt < NKT; ++kt) {
+    for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) S[kt][r] *= eg;
+    GDN_SCHED_FENCE();
 #pragma unroll
-      for (int tj = 0; tj < 2; ++tj) mma32_accb<T>(S[kt], KT + (32 * kt + l32) * L64 + 32 * tj, Vb[tj]);
-      GDN_PHASE_FENCE();
+    for (int kp = 0; kp < NP; ++kp) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        mma32_ff<T>(S[2 * kp + j], Kf[kp & 1][j][0], Vb[0]);
+        mma32_ff<T>(S[2 * kp + j], Kf[kp & 1][j][1], Vb[1]);
+      }
+      GDN_SCHED_FENCE();
+      if (kp + 2 < NP) { load_k(kp & 1, kp + 2); GDN_SCHED_FENCE(); }
     }
-    if (STAGES == 1 && c + 1 < nchunks) __syncthreads();      // (B) done with the single stage
+    if (STAGES == 1 && c + 1 < nchunks) GDN_LDS_BARRIER();      // (B) done with the single stage
   }
-
   if (ht != nullptr) {
 #pragma unroll
     for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
       for (int r = 0; r < 16; ++r)
         ht[(((int64_t)n * Hv + h) * DK + 32 * kt + acc_row(r)) * V + v0 + acc_col()] = S[kt][r];
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// chunk_out_kernel:  O = scale [ e^G . (Q S) + Aq V' ], parallel over (chunk, head, 32-column block).
+// S and V' arrive in fragment order and go from global memory straight into B-operand registers.
+// ---------------------------------------------------------------------------------------------
+template <typename T, int DK, int NW> struct OutSmem {
+  static constexpr int LDK = lds_ld<T>(DK), L64 = lds_ld<T>(64);
+  static constexpr int off_qs = 0;
+  static constexpr int off_aq = off_qs + 64 * LDK * (int)sizeof(T);
+  static constexpr int off_eg = off_aq + 64 * L64 * (int)sizeof(T);
+  static constexpr int bytes = off_eg + 64 * 4;
+};
+
+template <typename T, int DK, int NW>
+__global__ __launch_bounds__(64 * NW) void chunk_out_kernel(
+    const T* __restrict__ q, const T* __restrict__ aqk, const T* __restrict__ vf, const T* __restrict__ hf,
+    const float* __restrict__ G, T* __restrict__ o, const int64_t* __restrict__ cu,
+    const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V, float scale) {
+  using SM = OutSmem<T, DK, NW>;
+  constexpr int LDK = SM::LDK, L64 = SM::L64, NT = 64 * NW, VEC = Elem<T>::kVec, NKT = DK / 32;
+  T* Qs = reinterpret_cast<T*>(gdn_smem + SM::off_qs);
+  T* Aq = reinterpret_cast<T*>(gdn_smem + SM::off_aq);
+  float* Eg = reinterpret_cast<float*>(gdn_smem + SM::off_eg);
+  const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
+  if (s.nvalid <= 0) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31;
+  const int h = blockIdx.y, hq = h / (Hv / Hqk), nvalid = s.nvalid;
+  const int vblk = blockIdx.z * NW + wave, v0 = 32 * vblk;
+  const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk;
+  const int64_t tile0 = ((int64_t)blockIdx.x * Hv + h) * (V / 32) + vblk;
+
+  // operands that come in fragment order are requested first, the LDS tiles while they are in flight
+  AccB<T> Sb[NKT], Vb[2];
+#pragma unroll
+  for (int kt = 0; kt < NKT; ++kt) Sb[kt].load(hf + (tile0 * NKT + kt) * 1024);
+  Vb[0].load(vf + tile0 * 2048);
+  Vb[1].load(vf + tile0 * 2048 + 1024);
+  for (int c = tid; c < 64 * (DK / VEC); c += NT) {
+    const int row = c / (DK / VEC), cc = c % (DK / VEC);
+    st16(Qs + row * LDK + cc * VEC,
+         row < nvalid ? ld16(q + ((tok0 + row) * Hqk + hq) * DK + cc * VEC) : zero16<T>());
+  }
+  for (int c = tid; c < 64 * (64 / VEC); c += NT) {
+    const int row = c / (64 / VEC), cc = c % (64 / VEC);
+    st16(Aq + row * L64 + cc * VEC, row < nvalid ? ld16(aqk + ((tok0 + row) * Hv + h) * 64 + cc * VEC) : zero16<T>());
+  }
+  if (tid < 64) Eg[tid] = __expf(G[(tok0 + imin(tid, nvalid - 1)) * Hv + h]);
+  __syncthreads();
+
+  T* og = o + (tok0 * Hv + h) * V + v0;
+#pragma unroll
+  for (int ri = 0; ri < 2; ++ri) {
+    f32x16 oa = acc_zero();
+#pragma unroll
+    for (int kt = 0; kt < NKT; ++kt) mma32_accb<T>(oa, Qs + (32 * ri + l32) * LDK + 32 * kt, Sb[kt]);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oa[r] *= Eg[32 * ri + acc_row(r)];
+#pragma unroll
+    for (int tj = 0; tj <= ri; ++tj) mma32_accb<T>(oa, Aq + (32 * ri + l32) * L64 + 32 * tj, Vb[tj]);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oa[r] *= scale;
+    acc_to_global(oa, og, (int64_t)Hv * V, 32 * ri, 0, nvalid);
   }
 }
 
@@ -490,7 +584,7 @@ template <typename K> static int set_lds(K kernel, int bytes) {
 template <typename T, int DK, int BVP, int NW, int STAGES>
 static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const void* q, const void* k, const void* v,
                             const float* g, const float* beta, const float* h0, const int64_t* cu, void* o, float* ht,
-                            unsigned char* ws, float scale, int l2norm, bool keep_for_backward, hipStream_t st) {
+                            unsigned char* ws, float scale, int l2norm, bool with_backward, hipStream_t st) {
   const int64_t tok = d.tokens();
   const int nc = (int)d.max_chunks();
   int* chunk_offsets = reinterpret_cast<int*>(ws + L.chunk_offsets);
@@ -510,25 +604,35 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   }
   float* G = reinterpret_cast<float*>(ws + L.G);
   T* Ai = reinterpret_cast<T*>(ws + L.Ai);
-  T* W = reinterpret_cast<T*>(ws + L.W);
+  T* W = reinterpret_cast<T*>(ws + L.WAF);
   T* AQ = reinterpret_cast<T*>(ws + L.AQ);
-  T* U = reinterpret_cast<T*>(ws + L.U);
-  T* VN = keep_for_backward ? reinterpret_cast<T*>(ws + L.VN) : nullptr;
-  T* H = keep_for_backward ? reinterpret_cast<T*>(ws + L.H) : nullptr;
+  T* UF = reinterpret_cast<T*>(ws + L.UF);
+  T* KDF = reinterpret_cast<T*>(ws + L.KDF);
+  T* WF = with_backward ? reinterpret_cast<T*>(ws + L.WF) : nullptr;
+  T* VF = reinterpret_cast<T*>(ws + L.VF);
+  T* HF = reinterpret_cast<T*>(ws + L.HF);
   {
     auto kern = chunk_prep_kernel<T, DK, BVP>;
     constexpr int smem = PrepSmem<T, DK, BVP>::bytes;
     if (int e = set_lds(kern, smem)) return e;
     GDN_LAUNCH(kKernPrep, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, (const T*)v, g, beta, cu,
-               (const int*)chunk_offsets, G, Ai, W, U, AQ, d.T, d.N, d.Hqk, d.Hv, d.V);
+               (const int*)chunk_offsets, G, Ai, W, UF, AQ, KDF, WF, d.T, d.N, d.Hqk, d.Hv, d.V);
   }
   {
-    auto kern = chunk_fwd_kernel<T, DK, NW, STAGES>;
-    constexpr int smem = FwdSmem<T, DK, NW, STAGES>::bytes;
+    auto kern = chunk_state_kernel<T, DK, NW, STAGES>;
+    constexpr int smem = StateSmem<T, DK, NW, STAGES>::bytes;
     if (int e = set_lds(kern, smem)) return e;
-    GDN_LAUNCH(kKernStateFwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NW)), dim3(128 * NW), smem, st, qq, kk,
-               (const T*)W, (const T*)U, (const T*)AQ, (const float*)G, h0, ht, (T*)o, VN, H, cu,
-               (const int*)chunk_offsets, d.T, d.Hqk, d.Hv, d.V, scale);
+    GDN_LAUNCH(kKernStateFwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NW)), dim3(128 * NW), smem, st,
+               (const T*)KDF, (const T*)W, (const T*)UF, (const float*)G, h0, ht, VF, HF, cu,
+               (const int*)chunk_offsets, d.T, d.Hv, d.V);
+  }
+  {
+    auto kern = chunk_out_kernel<T, DK, NW>;
+    constexpr int smem = OutSmem<T, DK, NW>::bytes;
+    if (int e = set_lds(kern, smem)) return e;
+    GDN_LAUNCH(kKernOut, st, kern, dim3(nc, d.Hv, d.V / (32 * NW)), dim3(64 * NW), smem, st, qq, (const T*)AQ,
+               (const T*)VF, (const T*)HF, (const float*)G, (T*)o, cu, (const int*)chunk_offsets, d.T, d.N, d.Hqk,
+               d.Hv, d.V, scale);
   }
   return (int)hipGetLastError();
 }
@@ -555,24 +659,24 @@ extern "C" int gdn_chunk_fwd(const void* q, const void* k, const void* v, const 
   dl.varlen = true;  // one layout for both modes (the packed bound is the larger)
   const ChunkWorkspace L = chunk_workspace_layout(dl, dtype == 0 ? 4 : 2);
   if (workspace_bytes < L.fwd_bytes) return -5;
-  const bool keep = workspace_bytes >= L.total_bytes;   // a workspace sized for backward also receives v_new and the states
+  const bool with_bwd = workspace_bytes >= L.total_bytes;   // a workspace sized for backward also receives W^T fragments
   if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
   unsigned char* ws = static_cast<unsigned char*>(workspace);
   hipStream_t st = (hipStream_t)stream;
 #define GDN_FWD(T_, DK_, BVP_, NW_, ST_)                                                                          \
   return chunk_fwd_launch<T_, DK_, BVP_, NW_, ST_>(d, L, q, k, v, g, beta, initial_state, cu_seqlens, o, final_state, \
-                                                   ws, scale, use_qk_l2norm, keep, st)
+                                                   ws, scale, use_qk_l2norm, with_bwd, st)
   const bool wide = (V % 128 == 0);
   if (dtype == 1) {
     if (K == 128 && wide) GDN_FWD(bf16_t, 128, 128, 4, 2);
-    if (K == 128) GDN_FWD(bf16_t, 128, 64, 2, 1);
+    if (K == 128) GDN_FWD(bf16_t, 128, 64, 2, 2);
     if (K == 64 && wide) GDN_FWD(bf16_t, 64, 128, 4, 2);
-    GDN_FWD(bf16_t, 64, 64, 2, 1);
+    GDN_FWD(bf16_t, 64, 64, 2, 2);
   } else {
     if (K == 128 && wide) GDN_FWD(float, 128, 64, 4, 1);
     if (K == 128) GDN_FWD(float, 128, 64, 2, 1);
-    if (wide) GDN_FWD(float, 64, 64, 4, 1);
-    GDN_FWD(float, 64, 64, 2, 1);
+    if (wide) GDN_FWD(float, 64, 64, 4, 2);
+    GDN_FWD(float, 64, 64, 2, 2);
   }
 #undef GDN_FWD
 }

@@ -65,6 +65,19 @@ template <typename T> __device__ __host__ constexpr int lds_ld(int cols) { retur
 // compiler-only fence: keeps the scheduler from hoisting a later phase's LDS/global loads (and their registers)
 // above it.  No instruction is emitted.
 #define GDN_PHASE_FENCE() asm volatile("" ::: "memory")
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding global load
+// and store of the wave (vmcnt(0)), which would serialise a software pipeline whose whole point is to keep global
+// loads in flight across the barrier; kernels that hand data between waves through LDS only use this one.
+#define GDN_LDS_BARRIER()                                             \
+  do {                                                                \
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");   \
+    __builtin_amdgcn_s_barrier();                                     \
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");   \
+  } while (0)
+// Instruction-scheduling fence: nothing is moved across it.  Used to pin hand-made software pipelines (issue the
+// LDS reads of the next group, then the matrix instructions of this group) that the scheduler would otherwise
+// serialise into read -> wait -> multiply.
+#define GDN_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
 // makes a loop-invariant value opaque inside a loop so that the address arithmetic derived from it is recomputed
 // where it is used instead of being hoisted out of the loop and held in registers for its whole duration
 #define GDN_OPAQUE(x) asm volatile("" : "+r"(x))
@@ -204,6 +217,7 @@ __device__ __forceinline__ void mma32(f32x16& acc, const T* A, int lda, const T*
 //     bf16: r = 8kg..8kg+7  ->  16kg + {4h..4h+3, 8+4h..8+4h+3}      fp32: r = 4kg..4kg+3  ->  8kg + 4h..4h+3
 // (h = lane/32), so the A operand must be gathered with the same k order: frag_a_split.
 // ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ f32x16 acc_zero();
 template <typename T> struct AccK { static constexpr int kGroups = (sizeof(T) == 2) ? 2 : 4; };  // per 32-row tile
 
 template <typename T, int KG> __device__ __forceinline__ u32x4 frag_b_from_acc(const f32x16& c) {
@@ -228,13 +242,53 @@ template <typename T> __device__ __forceinline__ u32x4 frag_a_split(const T* p) 
     return *reinterpret_cast<const u32x4*>(p + 4 * half);
   }
 }
-// all k-groups of one 32-row accumulator tile packed as B fragments
+// all k-groups of one 32x32 accumulator tile packed as operand fragments ("fragment order").  The same 1024
+// elements, stored as [k-group][lane][16 bytes], are also the on-memory format in which kernels hand tiles to
+// each other: a lane writes/reads 16 contiguous bytes per k-group and never goes through LDS.
 template <typename T> struct AccB {
-  u32x4 f[AccK<T>::kGroups];
+  static constexpr int kG = AccK<T>::kGroups;
+  static constexpr int kVecElems = 16 / (int)sizeof(T);   // elements per lane per k-group
+  u32x4 f[kG];
   __device__ __forceinline__ void pack(const f32x16& c) {
     f[0] = frag_b_from_acc<T, 0>(c);
     f[1] = frag_b_from_acc<T, 1>(c);
     if constexpr (sizeof(T) == 4) { f[2] = frag_b_from_acc<T, 2>(c); f[3] = frag_b_from_acc<T, 3>(c); }
+  }
+  __device__ __forceinline__ void negate() {
+#pragma unroll
+    for (int g = 0; g < kG; ++g)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) f[g][e] ^= (sizeof(T) == 2 ? 0x80008000u : 0x80000000u);
+  }
+  // accumulator values (fp32) of the tile this fragment set was packed from
+  __device__ __forceinline__ f32x16 unpack() const {
+    f32x16 c;
+    if constexpr (sizeof(T) == 2) {
+#pragma unroll
+      for (int g = 0; g < 2; ++g)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          c[8 * g + 2 * e] = __uint_as_float(f[g][e] << 16);
+          c[8 * g + 2 * e + 1] = __uint_as_float(f[g][e] & 0xffff0000u);
+        }
+    } else {
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) c[4 * g + e] = __uint_as_float(f[g][e]);
+    }
+    return c;
+  }
+  // tile = first element of this 32x32 tile in a fragment-order buffer (1024 elements per tile)
+  __device__ __forceinline__ void store(T* tile) const {
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int g = 0; g < kG; ++g) *reinterpret_cast<u32x4*>(tile + (g * 64 + lane) * kVecElems) = f[g];
+  }
+  __device__ __forceinline__ void load(const T* tile) {
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int g = 0; g < kG; ++g) f[g] = *reinterpret_cast<const u32x4*>(tile + (g * 64 + lane) * kVecElems);
   }
 };
 // d(32x32) += A[32 rows][32 k] * B(32 k x 32) with B packed from an accumulator; arow = &A[row of this lane][k0]
@@ -242,6 +296,66 @@ template <typename T> __device__ __forceinline__ void mma32_accb(f32x16& d, cons
   constexpr int G = KGroup<T>::kLen;
 #pragma unroll
   for (int kg = 0; kg < AccK<T>::kGroups; ++kg) mfma_kgroup<T>(d, frag_a_split<T>(arow + G * kg), b.f[kg]);
+}
+// both operands in fragment order: d += A(32 x 32k) * B(32k x 32)
+template <typename T> __device__ __forceinline__ void mma32_ff(f32x16& d, const AccB<T>& a, const AccB<T>& b) {
+#pragma unroll
+  for (int kg = 0; kg < AccK<T>::kGroups; ++kg) mfma_kgroup<T>(d, a.f[kg], b.f[kg]);
+}
+// fragments of a tile stored in LDS with the contraction index contiguous: row = &tile[row of this lane][k0]
+template <typename T> __device__ __forceinline__ void frags_from_lds(AccB<T>& out, const T* row) {
+  constexpr int G = KGroup<T>::kLen;
+#pragma unroll
+  for (int kg = 0; kg < AccK<T>::kGroups; ++kg) out.f[kg] = frag_a_split<T>(row + G * kg);
+}
+
+// One 32x32 tile in fragment order (global memory) -> LDS, row-major at lds[(row0+i)*ld + col0+j]; one wave.
+template <typename T>
+__device__ __forceinline__ void frag_tile_to_lds(T* lds, int ld, int row0, int col0, const T* tile) {
+  const int lane = threadIdx.x & 63, col = lane & 31, half = lane >> 5;
+  AccB<T> f;
+  f.load(tile);
+#pragma unroll
+  for (int g = 0; g < AccK<T>::kGroups; ++g) {
+    Vec16<T> v;
+    v.raw = f.f[g];
+#pragma unroll
+    for (int e = 0; e < Elem<T>::kVec; ++e) {
+      const int row = (sizeof(T) == 2) ? 16 * g + 8 * (e >> 2) + 4 * half + (e & 3) : 8 * g + 4 * half + e;
+      lds[(row0 + row) * ld + col0 + col] = Elem<T>::from_f(v.get(e));
+    }
+  }
+}
+
+// Cross-lane transpose through the matrix core.  A tile held as fragments with (lane <-> a, registers <-> b)
+// multiplied by the identity comes back as an accumulator with (lane <-> b, registers <-> a): C = X * I read as
+// A operand X[a][b].  Exact (products with 1.0, sums with 0).  Costs kGroups MFMA k-groups per 32x32 tile.
+template <typename T> struct IdentityFrag {
+  u32x4 f[AccK<T>::kGroups];
+  __device__ __forceinline__ void init() {
+    const int lane = threadIdx.x & 63, n = lane & 31, half = lane >> 5;
+#pragma unroll
+    for (int g = 0; g < AccK<T>::kGroups; ++g) {
+      if constexpr (sizeof(T) == 2) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int k0 = 16 * g + 8 * ((2 * e) >> 2) + 4 * half + ((2 * e) & 3);
+          const int k1 = 16 * g + 8 * ((2 * e + 1) >> 2) + 4 * half + ((2 * e + 1) & 3);
+          f[g][e] = (k0 == n ? 0x3f80u : 0u) | (k1 == n ? 0x3f800000u : 0u);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) f[g][e] = (8 * g + 4 * half + e == n) ? 0x3f800000u : 0u;
+      }
+    }
+  }
+};
+template <typename T>
+__device__ __forceinline__ f32x16 mfma_transpose(const AccB<T>& x, const IdentityFrag<T>& id) {
+  f32x16 c = acc_zero();
+#pragma unroll
+  for (int kg = 0; kg < AccK<T>::kGroups; ++kg) mfma_kgroup<T>(c, x.f[kg], id.f[kg]);
+  return c;
 }
 
 // global -> LDS transposed staging: tile[64 rows][COLS] in memory becomes lds[COLS][ld] (rows contiguous), each

@@ -237,6 +237,9 @@ static emu::BdimProxy blockDim;
 static emu::GdimProxy gridDim;
 
 #define __syncthreads() emu::syncthreads()
+#define __builtin_amdgcn_s_barrier() emu::syncthreads()
+#define __builtin_amdgcn_fence(...) ((void)0)
+#define __builtin_amdgcn_sched_barrier(x) ((void)0)
 template <class T> inline T __shfl(T v, int src, int = 64) { return emu::shfl(v, src); }
 template <class T> inline T __shfl_xor(T v, int m, int = 64) { return emu::shfl(v, emu::lane() ^ m); }
 template <class T> inline T __shfl_up(T v, unsigned d, int = 64) {
