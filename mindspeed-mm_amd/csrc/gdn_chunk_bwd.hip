@@ -29,8 +29,8 @@ __device__ __forceinline__ void acc_rowdot_add(const f32x16& acc, const T* other
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int i = i0 + acc_row(r);
-    const float s = half_wave_sum(acc[r] * Elem<T>::to_f(other[i * ld + j]));
-    if (acc_col() == 0) atomicAdd(&rowacc[i], factor * s);
+    const float s = row16_sum(acc[r] * Elem<T>::to_f(other[i * ld + j]));
+    if ((threadIdx.x & 15) == 0) atomicAdd(&rowacc[i], factor * s);
   }
 }
 
@@ -328,18 +328,31 @@ __global__ __launch_bounds__(128 * NW) void chunk_state_bwd_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
+// chunk_dqkw_kernel, per (chunk, head), 4 waves; wave w owns the 32 K-columns [32w, 32w+32) of dQ, dK, dW.
+// v_new, d(v_new), S and dS' arrive in fragment order with (lane <-> V column); the contractions here run over V,
+// so every tile is first turned through the matrix core (mfma_transpose) into (lane <-> token / K column,
+// registers <-> V) and then used from registers: the main loop reads nothing but dO from LDS.
+// ---------------------------------------------------------------------------------------------
 template <typename T, int DK, int BV> struct DqkwSmem {
-  static constexpr int LDK = lds_ld<T>(DK), LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
-  static constexpr int SE = (DK * LDV > 64 * LDK) ? DK * LDV : 64 * LDK;   // state tile [DK][BV] / Q,K tile [64][DK]
-  static constexpr int off_do = 0;                                          // later ds
-  static constexpr int off_vp = off_do + 64 * LDV * (int)sizeof(T);         // later ds^T
-  static constexpr int off_dv = off_vp + 64 * LDV * (int)sizeof(T);
-  static constexpr int off_sb = off_dv + 64 * LDV * (int)sizeof(T);         // later Q
-  static constexpr int off_dsb = off_sb + SE * (int)sizeof(T);              // later K
-  static constexpr int off_row = off_dsb + SE * (int)sizeof(T);
+  static constexpr int LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
+  static constexpr int main_bytes = 64 * LDV * (int)sizeof(T);                       // dO tile
+  static constexpr int post_bytes = (2 * DK * kLT + 2 * 64 * L64) * (int)sizeof(T);  // K^T, Q^T, ds, ds^T
+  static constexpr int off_row = main_bytes > post_bytes ? main_bytes : post_bytes;
   static constexpr int bytes = off_row + (4 * 64 + 8) * 4;
-  static_assert(LDV >= L64, "ds reuses the dO tile");
 };
+
+// rowacc[i0+i] += factor * sum_j acc[i][j] * other_t[(j0+j)*ld + i0+i]   (other given transposed: [column][row])
+template <typename T>
+__device__ __forceinline__ void acc_rowdot_add_t(const f32x16& acc, const T* other_t, int ld, int i0, int j0,
+                                                 float* rowacc, float factor) {
+  const int j = j0 + acc_col();
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int i = i0 + acc_row(r);
+    const float s = row16_sum(acc[r] * Elem<T>::to_f(other_t[j * ld + i]));
+    if ((threadIdx.x & 15) == 0) atomicAdd(&rowacc[i], factor * s);
+  }
+}
 
 template <typename T, int DK, int BV>
 __global__ __launch_bounds__(kThreads) void chunk_dqkw_kernel(
@@ -349,81 +362,87 @@ __global__ __launch_bounds__(kThreads) void chunk_dqkw_kernel(
     const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V,
     float scale) {
   using SM = DqkwSmem<T, DK, BV>;
-  constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64;
-  constexpr int NQ = (2 * (DK / 32) + 3) / 4;
-  T* dOs = reinterpret_cast<T*>(gdn_smem + SM::off_do);
-  T* Vps = reinterpret_cast<T*>(gdn_smem + SM::off_vp);
-  T* dVs = reinterpret_cast<T*>(gdn_smem + SM::off_dv);
-  T* Sb = reinterpret_cast<T*>(gdn_smem + SM::off_sb);
-  T* dSb = reinterpret_cast<T*>(gdn_smem + SM::off_dsb);
+  constexpr int LDV = SM::LDV, L64 = SM::L64, NKT = DK / 32;
+  constexpr int NC = (NKT + 3) / 4;          // K-column blocks per wave (1 for K <= 128)
+  T* dOs = reinterpret_cast<T*>(gdn_smem);
+  T* KT = reinterpret_cast<T*>(gdn_smem);                   // post phase: [DK][kLT]
+  T* QT = KT + DK * kLT;
+  T* dsm = QT + DK * kLT;                                   // [64][L64]
+  T* dsT = dsm + 64 * L64;
   float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_row);
   float* rq = Gs + 64;     // <q_i, dQ_i>
   float* rk = rq + 64;     // <k_i, dK1_i>
   float* rki = rk + 64;    // <k_i, dK_inter_i>
   float* wsum = rki + 64;  // per-wave partials of <S, dS'>
-  T* dsm = dOs;
-  T* dsT = Vps;
-  T* Qs = Sb;
-  T* Ks = dSb;
 
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31;
   const int h = blockIdx.y, hq = h / (Hv / Hqk), nvalid = s.nvalid;
   const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk;
   const int64_t ch = (int64_t)blockIdx.x * Hv + h;
+  const int ti = wave >> 1, tj = wave & 1;
 
   if (tid < 64) {
     Gs[tid] = G[(tok0 + imin(tid, nvalid - 1)) * Hv + h];
     rq[tid] = 0.f; rk[tid] = 0.f; rki[tid] = 0.f;
   }
-
-  f32x16 ds = acc_zero(), dQi[NQ], dKi[NQ], dWa[NQ];
+  IdentityFrag<T> id;
+  id.init();
+  f32x16 ds = acc_zero(), dQi[NC][2], dKi[NC][2], dWa[NC][2];
 #pragma unroll
-  for (int i = 0; i < NQ; ++i) { dQi[i] = acc_zero(); dKi[i] = acc_zero(); dWa[i] = acc_zero(); }
+  for (int c = 0; c < NC; ++c)
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri) { dQi[c][ri] = acc_zero(); dKi[c][ri] = acc_zero(); dWa[c][ri] = acc_zero(); }
   float sds = 0.f;
-  const int ti = wave >> 1, tj = wave & 1;
 
   for (int vb = 0; vb < V / BV; ++vb) {
-    const int v0 = vb * BV;
     if (vb > 0) __syncthreads();
-    load_tile<T, BV>(dOs, LDV, dO + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
-    // v_new, d(v_new), S and dS' arrive in fragment order: one 32x32 tile per wave at a time into row-major LDS
-    for (int t = wave; t < 2 * (BV / 32); t += 4) {
-      const int ri = t & 1, vb32 = t >> 1;
-      const int64_t tile = ((ch * (V / 32) + v0 / 32 + vb32) * 2 + ri) * 1024;
-      frag_tile_to_lds<T>(Vps, LDV, 32 * ri, 32 * vb32, vf + tile);
-      frag_tile_to_lds<T>(dVs, LDV, 32 * ri, 32 * vb32, dvf + tile);
-    }
-    for (int t = wave; t < (DK / 32) * (BV / 32); t += 4) {
-      const int kt = t % (DK / 32), vb32 = t / (DK / 32);
-      const int64_t tile = ((ch * (V / 32) + v0 / 32 + vb32) * (DK / 32) + kt) * 1024;
-      frag_tile_to_lds<T>(Sb, LDV, 32 * kt, 32 * vb32, hf + tile);
-      frag_tile_to_lds<T>(dSb, LDV, 32 * kt, 32 * vb32, dhf + tile);
-    }
+    load_tile<T, BV>(dOs, LDV, dO + (tok0 * Hv + h) * V + vb * BV, (int64_t)Hv * V, nvalid, tid);
     __syncthreads();
-    for (int e = tid; e < DK * BV; e += kThreads) {
-      const int r = e / BV, c = e % BV;
-      sds += Elem<T>::to_f(Sb[r * LDV + c]) * Elem<T>::to_f(dSb[r * LDV + c]);
-    }
-    if (tj <= ti) mma32<T, BV, true, true>(ds, dOs + 32 * ti * LDV, LDV, Vps + 32 * tj * LDV, LDV);
 #pragma unroll
-    for (int i = 0; i < NQ; ++i) {
-      const int tt = wave + 4 * i;
-      if (tt < 2 * (DK / 32)) {
-        const int ri = tt & 1, cj = tt >> 1;
-        mma32<T, BV, true, true>(dQi[i], dOs + 32 * ri * LDV, LDV, Sb + 32 * cj * LDV, LDV);
-        mma32<T, BV, true, true>(dKi[i], Vps + 32 * ri * LDV, LDV, dSb + 32 * cj * LDV, LDV);
-        mma32<T, BV, true, true>(dWa[i], dVs + 32 * ri * LDV, LDV, Sb + 32 * cj * LDV, LDV);
+    for (int v32 = 0; v32 < BV / 32; ++v32) {
+      const int vblk = vb * (BV / 32) + v32;
+      const int64_t t2 = (ch * (V / 32) + vblk) * 2, tk = (ch * (V / 32) + vblk) * NKT;
+      AccB<T> f, Vt[2], dVt[2], dOf[2];
+#pragma unroll
+      for (int ri = 0; ri < 2; ++ri) {       // (lane <-> token, registers <-> V)
+        f.load(vf + (t2 + ri) * 1024);
+        Vt[ri].pack(mfma_transpose<T>(f, id));
+        f.load(dvf + (t2 + ri) * 1024);
+        dVt[ri].pack(mfma_transpose<T>(f, id));
+        frags_from_lds<T>(dOf[ri], dOs + (32 * ri + l32) * LDV + 32 * v32);
+      }
+      if (tj <= ti) mma32_ff<T>(ds, dOf[ti], Vt[tj]);
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const int kt = wave + 4 * c;
+        if (kt < NKT) {
+          AccB<T> Sf, dSf;                   // (lane <-> K column, registers <-> V)
+          f.load(hf + (tk + kt) * 1024);
+          const f32x16 st = mfma_transpose<T>(f, id);
+          Sf.pack(st);
+          f.load(dhf + (tk + kt) * 1024);
+          const f32x16 dst = mfma_transpose<T>(f, id);
+          dSf.pack(dst);
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sds += st[r] * dst[r];
+#pragma unroll
+          for (int ri = 0; ri < 2; ++ri) {
+            mma32_ff<T>(dQi[c][ri], dOf[ri], Sf);
+            mma32_ff<T>(dKi[c][ri], Vt[ri], dSf);
+            mma32_ff<T>(dWa[c][ri], dVt[ri], Sf);
+          }
+        }
       }
     }
   }
   sds = wave_sum(sds);
   if (lane == 0) wsum[wave] = sds;
-  __syncthreads();   // all tiles consumed; their buffers are reused below
+  __syncthreads();   // dO tile consumed; its space is reused below
 
-  load_tile<T, DK>(Qs, LDK, q + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
-  load_tile<T, DK>(Ks, LDK, k + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
+  load_tile_t<T, DK, kThreads>(KT, kLT, k + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
+  load_tile_t<T, DK, kThreads>(QT, kLT, q + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
   {
     const int j = 32 * tj + acc_col();
 #pragma unroll
@@ -438,27 +457,30 @@ __global__ __launch_bounds__(kThreads) void chunk_dqkw_kernel(
   const float glast = Gs[63];
   T* dqg = dqh + (tok0 * Hv + h) * DK;
   T* dkg = dkh + (tok0 * Hv + h) * DK;
-  T* dwg = dwb + (tok0 * Hv + h) * DK;
 #pragma unroll
-  for (int i = 0; i < NQ; ++i) {
-    const int tt = wave + 4 * i;
-    if (tt < 2 * (DK / 32)) {
-      const int ri = tt & 1, cj = tt >> 1;
+  for (int c = 0; c < NC; ++c) {
+    const int cj = wave + 4 * c;
+    if (cj < NKT) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float gi = Gs[32 * ri + acc_row(r)];
-        dQi[i][r] *= scale * __expf(gi);
-        dKi[i][r] *= __expf(glast - gi);
-        dWa[i][r] = -dWa[i][r];
+      for (int ri = 0; ri < 2; ++ri) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float gi = Gs[32 * ri + acc_row(r)];
+          dQi[c][ri][r] *= scale * __expf(gi);
+          dKi[c][ri][r] *= __expf(glast - gi);
+          dWa[c][ri][r] = -dWa[c][ri][r];
+        }
+        acc_rowdot_add_t<T>(dKi[c][ri], KT, kLT, 32 * ri, 32 * cj, rki, 1.f);   // still only the inter-chunk part
+        mma32_ss<T, 64>(dQi[c][ri], dsm + (32 * ri + l32) * L64, KT + (32 * cj + l32) * kLT);
+        mma32_ss<T, 64>(dKi[c][ri], dsT + (32 * ri + l32) * L64, QT + (32 * cj + l32) * kLT);
+        acc_rowdot_add_t<T>(dQi[c][ri], QT, kLT, 32 * ri, 32 * cj, rq, 1.f);
+        acc_rowdot_add_t<T>(dKi[c][ri], KT, kLT, 32 * ri, 32 * cj, rk, 1.f);
+        acc_to_global(dQi[c][ri], dqg, (int64_t)Hv * DK, 32 * ri, 32 * cj, nvalid);
+        acc_to_global(dKi[c][ri], dkg, (int64_t)Hv * DK, 32 * ri, 32 * cj, nvalid);
+        AccB<T> wf;                        // dW as a B operand for the WY backward kernel
+        wf.pack(dWa[c][ri]);
+        wf.store(dwb + ((ch * NKT + cj) * 2 + ri) * 1024);
       }
-      acc_rowdot_add<T>(dKi[i], Ks, LDK, 32 * ri, 32 * cj, rki, 1.f);   // still only the inter-chunk part
-      mma32<T, 64, true, false>(dQi[i], dsm + 32 * ri * L64, L64, Ks + 32 * cj, LDK);
-      mma32<T, 64, true, false>(dKi[i], dsT + 32 * ri * L64, L64, Qs + 32 * cj, LDK);
-      acc_rowdot_add<T>(dQi[i], Qs, LDK, 32 * ri, 32 * cj, rq, 1.f);
-      acc_rowdot_add<T>(dKi[i], Ks, LDK, 32 * ri, 32 * cj, rk, 1.f);
-      acc_to_global(dQi[i], dqg, (int64_t)Hv * DK, 32 * ri, 32 * cj, nvalid);
-      acc_to_global(dKi[i], dkg, (int64_t)Hv * DK, 32 * ri, 32 * cj, nvalid);
-      acc_to_global(dWa[i], dwg, (int64_t)Hv * DK, 32 * ri, 32 * cj, nvalid);
     }
   }
   __syncthreads();
@@ -471,34 +493,47 @@ __global__ __launch_bounds__(kThreads) void chunk_dqkw_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
+// chunk_wy_bwd_kernel, per (chunk, head), 4 waves: back through W = Tm (beta e^G K), U = Tm (beta V), Tm = (I+L)^-1.
+// dW and d(v_new) arrive in fragment order (lane <-> K / V column, registers <-> token): exactly the B operand of
+// P = Tm^T dW and R = Tm^T dU; their transposes through the matrix core are the A operands of dW K^T and dU V^T.
+// Wave w owns the 32 K-columns [32w, 32w+32) of dK and the V blocks w, w+4, ...
+// ---------------------------------------------------------------------------------------------
 template <typename T, int DK, int BV> struct WySmem {
   static constexpr int LDK = lds_ld<T>(DK), LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
-  static constexpr int off_tm = 0;
-  static constexpr int off_ks = off_tm + 64 * L64 * (int)sizeof(T);
-  static constexpr int off_dw = off_ks + 64 * LDK * (int)sizeof(T);
-  static constexpr int off_vs = off_dw + 64 * LDK * (int)sizeof(T);          // later (dM . beta)^T
-  static constexpr int off_du = off_vs + 64 * LDV * (int)sizeof(T);
-  static constexpr int off_da = off_du + 64 * LDV * (int)sizeof(T);          // dTm, later dM
-  static constexpr int off_xt = off_da + 64 * L64 * (int)sizeof(T);
+  static constexpr int off_tmt = 0;                                           // Tm^T  [64][kLT]
+  static constexpr int off_tm = off_tmt + 64 * kLT * (int)sizeof(T);          // Tm    [64][L64]
+  static constexpr int off_ks = off_tm + 64 * L64 * (int)sizeof(T);           // K     [64][LDK]
+  static constexpr int off_vs = off_ks + 64 * LDK * (int)sizeof(T);           // V     [64][LDV], later (beta . dM)^T
+  static constexpr int off_da = off_vs + 64 * LDV * (int)sizeof(T);           // dTm, later dM  [64][L64]
+  static constexpr int off_xt = off_da + 64 * L64 * (int)sizeof(T);           // X^T   [64][L64]
   static constexpr int off_row = off_xt + 64 * L64 * (int)sizeof(T);
   static constexpr int bytes = off_row + 5 * 64 * 4;
   static_assert(LDV >= L64, "dM^T reuses the V tile");
 };
 
+// rowacc[i0+i] += factor * sum_j acc[i][j] * other[i][j] with `other` given as an accumulator tile
+__device__ __forceinline__ void acc_rowdot_add_r(const f32x16& acc, const f32x16& other, int i0, float* rowacc,
+                                                 float factor) {
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const float s = row16_sum(acc[r] * other[r]);
+    if ((threadIdx.x & 15) == 0) atomicAdd(&rowacc[i0 + acc_row(r)], factor * s);
+  }
+}
+
 template <typename T, int DK, int BV>
 __global__ __launch_bounds__(kThreads) void chunk_wy_bwd_kernel(
     const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ beta, const float* __restrict__ G,
-    const T* __restrict__ Ai, const T* __restrict__ dwb, const T* __restrict__ dvf, T* dkh, const float* dG1,
+    const T* __restrict__ Ai, const T* __restrict__ dwf, const T* __restrict__ dvf, T* dkh, const float* dG1,
     T* __restrict__ dv_out, float* __restrict__ dbeta, float* __restrict__ dg, const int64_t* __restrict__ cu,
     const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V) {
   using SM = WySmem<T, DK, BV>;
-  constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64;
-  constexpr int NQ = (2 * (DK / 32) + 3) / 4, MT = BV / 32, NR = (2 * MT + 3) / 4;
+  constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64, NKT = DK / 32;
+  constexpr int NC = (NKT + 3) / 4;
+  T* TmT = reinterpret_cast<T*>(gdn_smem + SM::off_tmt);
   T* Tm = reinterpret_cast<T*>(gdn_smem + SM::off_tm);
   T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
-  T* dWs = reinterpret_cast<T*>(gdn_smem + SM::off_dw);
   T* Vs = reinterpret_cast<T*>(gdn_smem + SM::off_vs);
-  T* dUs = reinterpret_cast<T*>(gdn_smem + SM::off_du);
   T* dAs = reinterpret_cast<T*>(gdn_smem + SM::off_da);
   T* XT = reinterpret_cast<T*>(gdn_smem + SM::off_xt);
   float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_row);
@@ -511,9 +546,10 @@ __global__ __launch_bounds__(kThreads) void chunk_wy_bwd_kernel(
 
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31;
   const int h = blockIdx.y, hq = h / (Hv / Hqk), nvalid = s.nvalid;
   const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk;
+  const int64_t ch = (int64_t)blockIdx.x * Hv + h;
   const int ti = wave >> 1, tj = wave & 1;
 
   if (tid < 64) {
@@ -524,56 +560,87 @@ __global__ __launch_bounds__(kThreads) void chunk_wy_bwd_kernel(
     rb[tid] = 0.f; rg[tid] = 0.f;
   }
   load_tile<T, 64>(Tm, L64, Ai + (tok0 * Hv + h) * 64, (int64_t)Hv * 64, nvalid, tid);
+  load_tile_t<T, 64, kThreads>(TmT, kLT, Ai + (tok0 * Hv + h) * 64, (int64_t)Hv * 64, nvalid, tid);
   load_tile<T, DK>(Ks, LDK, k + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
-  load_tile<T, DK>(dWs, LDK, dwb + (tok0 * Hv + h) * DK, (int64_t)Hv * DK, nvalid, tid);
   __syncthreads();
 
-  // P = Tm^T dW  ->  dK2 = P beta e^G,  t1 = e^G <P, k>
-  f32x16 dK[NQ];
+  IdentityFrag<T> id;
+  id.init();
+  // K columns of this wave as (lane <-> K column, registers <-> token); P = Tm^T dW; dK2 = beta e^G P; t1 = e^G<P,k>
+  AccB<T> KTf[NC][2];
+  f32x16 dK[NC][2];
 #pragma unroll
-  for (int i = 0; i < NQ; ++i) {
-    const int tt = wave + 4 * i;
-    dK[i] = acc_zero();
-    if (tt < 2 * (DK / 32)) {
-      const int ri = tt & 1, cj = tt >> 1;
-      mma32<T, 64, false, false>(dK[i], Tm + 32 * ri, L64, dWs + 32 * cj, LDK);
+  for (int c = 0; c < NC; ++c) {
+    const int cj = wave + 4 * c;
+    dK[c][0] = acc_zero();
+    dK[c][1] = acc_zero();
+    if (cj < NKT) {
+      AccB<T> f, dwb[2];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) dK[i][r] *= egs[32 * ri + acc_row(r)];   // now e^G P
-      acc_rowdot_add<T>(dK[i], Ks, LDK, 32 * ri, 32 * cj, rb, 1.f);
+      for (int t = 0; t < 2; ++t) {
+        frags_from_lds<T>(f, Ks + (32 * t + l32) * LDK + 32 * cj);
+        KTf[c][t].pack(mfma_transpose<T>(f, id));
+        dwb[t].load(dwf + ((ch * NKT + cj) * 2 + t) * 1024);
+      }
 #pragma unroll
-      for (int r = 0; r < 16; ++r) dK[i][r] *= bs[32 * ri + acc_row(r)];    // beta e^G P
-      acc_rowdot_add<T>(dK[i], Ks, LDK, 32 * ri, 32 * cj, rg, 1.f);
+      for (int rj = 0; rj < 2; ++rj) {
+#pragma unroll
+        for (int t = rj; t < 2; ++t) mma32_accb<T>(dK[c][rj], TmT + (32 * rj + l32) * kLT + 32 * t, dwb[t]);
+        const f32x16 kk = KTf[c][rj].unpack();
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dK[c][rj][r] *= egs[32 * rj + acc_row(r)];
+        acc_rowdot_add_r(dK[c][rj], kk, 32 * rj, rb, 1.f);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dK[c][rj][r] *= bs[32 * rj + acc_row(r)];
+        acc_rowdot_add_r(dK[c][rj], kk, 32 * rj, rg, 1.f);
+      }
     }
   }
-  // dTm pieces: a1 = dW K^T, a2 = dU V^T (strictly lower tiles only)
+  // dTm pieces (strictly lower tiles only): a1 = dW K^T, a2 = dU V^T
   f32x16 a1 = acc_zero(), a2 = acc_zero();
-  if (tj <= ti) mma32<T, DK, true, true>(a1, dWs + 32 * ti * LDK, LDK, Ks + 32 * tj * LDK, LDK);
+  if (tj <= ti) {
+#pragma unroll
+    for (int kt = 0; kt < NKT; ++kt) {
+      AccB<T> f, wt, kf;
+      f.load(dwf + ((ch * NKT + kt) * 2 + ti) * 1024);
+      wt.pack(mfma_transpose<T>(f, id));                       // (lane <-> token i, registers <-> K column)
+      frags_from_lds<T>(kf, Ks + (32 * tj + l32) * LDK + 32 * kt);
+      mma32_ff<T>(a1, wt, kf);
+    }
+  }
 
   for (int vb = 0; vb < V / BV; ++vb) {
     const int v0 = vb * BV;
     if (vb > 0) __syncthreads();
     load_tile<T, BV>(Vs, LDV, v + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
-    for (int t = wave; t < 2 * (BV / 32); t += 4) {      // d(v_new) tiles arrive in fragment order
-      const int ri = t & 1, vb32 = t >> 1;
-      frag_tile_to_lds<T>(dUs, LDV, 32 * ri, 32 * vb32,
-                          dvf + ((((int64_t)blockIdx.x * Hv + h) * (V / 32) + v0 / 32 + vb32) * 2 + ri) * 1024);
-    }
     __syncthreads();
-    T* dvg = dv_out + (tok0 * Hv + h) * V + v0;
+    for (int v32 = wave; v32 < BV / 32; v32 += 4) {            // R = Tm^T dU, dv = beta R
+      const int vblk = v0 / 32 + v32;
+      AccB<T> dub[2];
+      dub[0].load(dvf + ((ch * (V / 32) + vblk) * 2 + 0) * 1024);
+      dub[1].load(dvf + ((ch * (V / 32) + vblk) * 2 + 1) * 1024);
+      T* dvg = dv_out + (tok0 * Hv + h) * V + 32 * vblk;
 #pragma unroll
-    for (int i = 0; i < NR; ++i) {
-      const int tt = wave + 4 * i;
-      if (tt < 2 * MT) {
-        const int ri = tt & 1, cj = tt >> 1;
+      for (int rj = 0; rj < 2; ++rj) {
         f32x16 R = acc_zero();
-        mma32<T, 64, false, false>(R, Tm + 32 * ri, L64, dUs + 32 * cj, LDV);
-        acc_rowdot_add<T>(R, Vs, LDV, 32 * ri, 32 * cj, rb, 1.f);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) R[r] *= bs[32 * ri + acc_row(r)];
-        acc_to_global(R, dvg, (int64_t)Hv * V, 32 * ri, 32 * cj, nvalid);
+        for (int t = rj; t < 2; ++t) mma32_accb<T>(R, TmT + (32 * rj + l32) * kLT + 32 * t, dub[t]);
+        acc_rowdot_add<T>(R, Vs, LDV, 32 * rj, 32 * v32, rb, 1.f);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) R[r] *= bs[32 * rj + acc_row(r)];
+        acc_to_global(R, dvg, (int64_t)Hv * V, 32 * rj, 0, nvalid);
       }
     }
-    if (tj <= ti) mma32<T, BV, true, true>(a2, dUs + 32 * ti * LDV, LDV, Vs + 32 * tj * LDV, LDV);
+    if (tj <= ti) {
+#pragma unroll
+      for (int v32 = 0; v32 < BV / 32; ++v32) {
+        AccB<T> f, ut, vfr;
+        f.load(dvf + ((ch * (V / 32) + v0 / 32 + v32) * 2 + ti) * 1024);
+        ut.pack(mfma_transpose<T>(f, id));                     // (lane <-> token i, registers <-> V column)
+        frags_from_lds<T>(vfr, Vs + (32 * tj + l32) * LDV + 32 * v32);
+        mma32_ff<T>(a2, ut, vfr);
+      }
+    }
   }
   {  // dTm[i][j] = beta_j (e^{G_j} a1 + a2), i > j
     const int j = 32 * tj + acc_col();
@@ -592,7 +659,7 @@ __global__ __launch_bounds__(kThreads) void chunk_wy_bwd_kernel(
   __syncthreads();
   {  // dM = -(Tm^T X) . Gam, strictly lower;  dMs[i][j] = dM,  dMTb[j][i] = beta_i dM
     f32x16 y = acc_zero();
-    mma32<T, 64, false, true>(y, Tm + 32 * ti, L64, XT + 32 * tj * L64, L64);
+    mma32_ss<T, 64>(y, TmT + (32 * ti + l32) * kLT, XT + (32 * tj + l32) * L64);
     const int j = 32 * tj + acc_col();
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -605,22 +672,28 @@ __global__ __launch_bounds__(kThreads) void chunk_wy_bwd_kernel(
   __syncthreads();
   T* dkg = dkh + (tok0 * Hv + h) * DK;
 #pragma unroll
-  for (int i = 0; i < NQ; ++i) {
-    const int tt = wave + 4 * i;
-    if (tt < 2 * (DK / 32)) {
-      const int ri = tt & 1, cj = tt >> 1;
-      f32x16 E = acc_zero(), Fm = acc_zero();
-      mma32<T, 64, true, false>(E, dMs + 32 * ri * L64, L64, Ks + 32 * cj, LDK);
-      mma32<T, 64, true, false>(Fm, dMTb + 32 * ri * L64, L64, Ks + 32 * cj, LDK);
-      acc_rowdot_add<T>(E, Ks, LDK, 32 * ri, 32 * cj, rb, 1.f);
-      acc_rowdot_add<T>(Fm, Ks, LDK, 32 * ri, 32 * cj, rg, -1.f);
+  for (int c = 0; c < NC; ++c) {
+    const int cj = wave + 4 * c;
+    if (cj < NKT) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) E[r] *= bs[32 * ri + acc_row(r)];
-      acc_rowdot_add<T>(E, Ks, LDK, 32 * ri, 32 * cj, rg, 1.f);
-      const f32x16 k1 = acc_from_global(dkg, (int64_t)Hv * DK, 32 * ri, 32 * cj, nvalid);
+      for (int ri = 0; ri < 2; ++ri) {
+        f32x16 E = acc_zero(), Fm = acc_zero();
 #pragma unroll
-      for (int r = 0; r < 16; ++r) dK[i][r] += E[r] + Fm[r] + k1[r];
-      acc_to_global(dK[i], dkg, (int64_t)Hv * DK, 32 * ri, 32 * cj, nvalid);
+        for (int t = 0; t < 2; ++t) {
+          mma32_accb<T>(E, dMs + (32 * ri + l32) * L64 + 32 * t, KTf[c][t]);
+          mma32_accb<T>(Fm, dMTb + (32 * ri + l32) * L64 + 32 * t, KTf[c][t]);
+        }
+        const f32x16 kk = KTf[c][ri].unpack();
+        acc_rowdot_add_r(E, kk, 32 * ri, rb, 1.f);
+        acc_rowdot_add_r(Fm, kk, 32 * ri, rg, -1.f);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) E[r] *= bs[32 * ri + acc_row(r)];
+        acc_rowdot_add_r(E, kk, 32 * ri, rg, 1.f);
+        const f32x16 k1 = acc_from_global(dkg, (int64_t)Hv * DK, 32 * ri, 32 * cj, nvalid);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dK[c][ri][r] += E[r] + Fm[r] + k1[r];
+        acc_to_global(dK[c][ri], dkg, (int64_t)Hv * DK, 32 * ri, 32 * cj, nvalid);
+      }
     }
   }
   __syncthreads();
@@ -717,7 +790,7 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   T* DOF = reinterpret_cast<T*>(ws + L.DOF);
   T* DVF = reinterpret_cast<T*>(ws + L.DVF);
   T* DHF = reinterpret_cast<T*>(ws + L.DHF);
-  T* DW = reinterpret_cast<T*>(ws + L.DW);
+  T* DW = reinterpret_cast<T*>(ws + L.DWF);
   T* DQH = reinterpret_cast<T*>(ws + L.DQH);
   T* DKH = reinterpret_cast<T*>(ws + L.DKH);
   float* DG = reinterpret_cast<float*>(ws + L.DG);

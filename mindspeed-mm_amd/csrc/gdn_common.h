@@ -302,6 +302,14 @@ template <typename T> __device__ __forceinline__ void mma32_ff(f32x16& d, const 
 #pragma unroll
   for (int kg = 0; kg < AccK<T>::kGroups; ++kg) mfma_kgroup<T>(d, a.f[kg], b.f[kg]);
 }
+// d(32x32) += A[32 rows][KLEN] * B[32 rows][KLEN]^T, both in LDS with the contraction index contiguous and read with
+// 8-byte (bf16) accesses, so rows only need 8-byte alignment (transposed tiles with a leading dimension of 68)
+template <typename T, int KLEN>
+__device__ __forceinline__ void mma32_ss(f32x16& d, const T* arow, const T* brow) {
+  constexpr int G = KGroup<T>::kLen;
+#pragma unroll
+  for (int kg = 0; kg < KLEN / G; ++kg) mfma_kgroup<T>(d, frag_a_split<T>(arow + G * kg), frag_a_split<T>(brow + G * kg));
+}
 // fragments of a tile stored in LDS with the contraction index contiguous: row = &tile[row of this lane][k0]
 template <typename T> __device__ __forceinline__ void frags_from_lds(AccB<T>& out, const T* row) {
   constexpr int G = KGroup<T>::kLen;
@@ -416,6 +424,19 @@ __device__ __forceinline__ f32x16 acc_from_global(const T* g, int64_t row_stride
     a[r] = i < nvalid ? Elem<T>::to_f(g[(int64_t)i * row_stride + j]) : 0.f;
   }
   return a;
+}
+
+// Sum over the 16 lanes of a DPP row (lanes 16r .. 16r+15), every lane gets the result.  Data-parallel-primitive
+// moves run at VALU speed; wave shuffles (ds_bpermute) go through the LDS crossbar and cost ~10x more.
+template <int CTRL> __device__ __forceinline__ float dpp_mov(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_mov<0xB1>(v);    // quad_perm [1,0,3,2]
+  v += dpp_mov<0x4E>(v);    // quad_perm [2,3,0,1]
+  v += dpp_mov<0x141>(v);   // row_half_mirror
+  v += dpp_mov<0x140>(v);   // row_mirror
+  return v;
 }
 
 // sum over the 32 lanes that share a half-wave (all columns of one accumulator row)

@@ -251,6 +251,17 @@ template <class T> inline T __shfl_down(T v, unsigned d, int = 64) {
   return emu::shfl(v, l + (int)d < emu::kWave ? l + (int)d : l);
 }
 
+inline int emu_update_dpp(int /*old*/, int src, int ctrl) {
+  const int l = emu::lane();
+  int from = l;
+  if (ctrl >= 0 && ctrl <= 0xFF) from = (l & ~3) | ((ctrl >> (2 * (l & 3))) & 3);          // quad_perm
+  else if (ctrl == 0x141) from = (l & ~7) | (7 - (l & 7));                                  // row_half_mirror
+  else if (ctrl == 0x140) from = (l & ~15) | (15 - (l & 15));                               // row_mirror
+  else abort();
+  return emu::shfl(src, from);
+}
+#define __builtin_amdgcn_update_dpp(old, src, ctrl, rm, bm, bc) emu_update_dpp(old, src, ctrl)
+
 #define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) emu::mfma_32x32x16_bf16(a, b, c)
 #define __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, x, y, z) emu::mfma_16x16x32_bf16(a, b, c)
 #define __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, x, y, z) emu::mfma_32x32x2_f32(a, b, c)
