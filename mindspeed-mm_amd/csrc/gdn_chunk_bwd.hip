@@ -355,7 +355,7 @@ __device__ __forceinline__ void acc_rowdot_add_t(const f32x16& acc, const T* oth
 }
 
 template <typename T, int DK, int BV>
-__global__ __launch_bounds__(kThreads) void chunk_dqkw_kernel(
+__global__ __launch_bounds__(kThreads, 2) void chunk_dqkw_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ vf, const T* __restrict__ dvf,
     const T* __restrict__ dO, const T* __restrict__ hf, const T* __restrict__ dhf, const float* __restrict__ G,
     T* __restrict__ dqh, T* __restrict__ dkh, T* __restrict__ dwb, float* __restrict__ dG,
@@ -522,7 +522,7 @@ __device__ __forceinline__ void acc_rowdot_add_r(const f32x16& acc, const f32x16
 }
 
 template <typename T, int DK, int BV>
-__global__ __launch_bounds__(kThreads) void chunk_wy_bwd_kernel(
+__global__ __launch_bounds__(kThreads, 2) void chunk_wy_bwd_kernel(
     const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ beta, const float* __restrict__ G,
     const T* __restrict__ Ai, const T* __restrict__ dwf, const T* __restrict__ dvf, T* dkh, const float* dG1,
     T* __restrict__ dv_out, float* __restrict__ dbeta, float* __restrict__ dg, const int64_t* __restrict__ cu,
