@@ -42,11 +42,11 @@ def kernel_matmul_flops(K, V, C=64):
     """Matmul FLOP each kernel performs per (chunk, value head): 2*M*N*K summed over its contractions."""
     g = lambda m, n, k: 2 * m * n * k
     return {
-        "chunk_prep_kernel": g(C, C, K) + g(C, K, C) + g(C, V, C),
-        "chunk_state_kernel": g(C, V, K) + g(V, K, C),
-        "chunk_out_kernel": g(C, C, K) + g(C, V, K) + g(C, V, C),
-        "chunk_dv_local_kernel": g(C, C, K) + g(C, V, C),
-        "chunk_state_bwd_kernel": g(C, V, K) + 2 * g(V, K, C),
+        "chunk_prep_kernel": 2 * g(C, C, K) + g(C, K, C) + g(C, V, C),     # K K^T, Q K^T, Tm (b e^G K), Tm (b V)
+        "chunk_state_kernel": g(C, V, K) + g(K, V, C),                     # W S, (decayed K)^T V'
+        "chunk_out_kernel": g(C, V, K) + g(C, V, C),                       # Q S, Aq V'
+        "chunk_bwd_prep_kernel": g(C, V, C),                               # Aq^T dO
+        "chunk_state_bwd_kernel": g(C, V, K) + 2 * g(K, V, C),             # K dS, Q^T dO, W^T dV'
         "chunk_dqkw_kernel": g(C, C, V) + 3 * g(C, K, V) + 2 * g(C, K, C),
         "chunk_wy_bwd_kernel": g(C, K, C) + g(C, C, K) + g(C, V, C) + g(C, C, V) + 2 * g(C, C, C) + 2 * g(C, K, C),
     }

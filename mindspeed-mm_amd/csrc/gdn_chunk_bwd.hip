@@ -768,7 +768,7 @@ template <typename K> static int set_lds_b(K kernel, int bytes) {
                                   bytes);
 }
 
-template <typename T, int DK, int NW, int STAGES, int BVQ, int BVW>
+template <typename T, int DK, int NW, int NWS, int STAGES, int BVQ, int BVW>
 static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const void* q, const void* k, const void* v,
                             const float* beta, const int64_t* cu, const void* dO, const float* dht, void* dq, void* dk,
                             void* dv, float* dg, float* dbeta, float* dh0, unsigned char* ws, float scale, int l2norm,
@@ -798,14 +798,14 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     auto kern = chunk_bwd_prep_kernel<T, DK, NW>;
     constexpr int smem = BwdPrepSmem<T, DK, NW>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
-    GDN_LAUNCH(kKernDvLocal, st, kern, dim3(nc, d.Hv, d.V / (32 * NW)), dim3(64 * NW), smem, st, qq, kk, AQ,
+    GDN_LAUNCH(kKernBwdPrep, st, kern, dim3(nc, d.Hv, d.V / (32 * NW)), dim3(64 * NW), smem, st, qq, kk, AQ,
                (const T*)dO, G, DVLF, DOF, QSF, KAF, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale);
   }
   {
-    auto kern = chunk_state_bwd_kernel<T, DK, NW, STAGES>;
-    constexpr int smem = StateBwdSmem<T, DK, NW, STAGES>::bytes;
+    auto kern = chunk_state_bwd_kernel<T, DK, NWS, STAGES>;
+    constexpr int smem = StateBwdSmem<T, DK, NWS, STAGES>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
-    GDN_LAUNCH(kKernStateBwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NW)), dim3(128 * NW), smem, st, (const T*)KAF,
+    GDN_LAUNCH(kKernStateBwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NWS)), dim3(128 * NWS), smem, st, (const T*)KAF,
                (const T*)QSF, WF, (const T*)DVLF, (const T*)DOF, G, dht, dh0, DVF, DHF, cu, chunk_offsets, d.T, d.Hv,
                d.V);
   }
@@ -853,19 +853,19 @@ extern "C" int gdn_chunk_bwd(const void* q, const void* k, const void* v, const 
   if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
   unsigned char* ws = static_cast<unsigned char*>(workspace);
   hipStream_t st = (hipStream_t)stream;
-#define GDN_BWD(T_, DK_, NW_, ST_, BVQ_, BVW_)                                                                     \
-  return chunk_bwd_launch<T_, DK_, NW_, ST_, BVQ_, BVW_>(d, L, q, k, v, beta, cu_seqlens, d_o, d_final_state, dq, \
+#define GDN_BWD(T_, DK_, NW_, NWS_, ST_, BVQ_, BVW_)                                                                   \
+  return chunk_bwd_launch<T_, DK_, NW_, NWS_, ST_, BVQ_, BVW_>(d, L, q, k, v, beta, cu_seqlens, d_o, d_final_state, dq, \
                                                           dk, dv, dg, dbeta, d_initial_state, ws, scale,         \
                                                           use_qk_l2norm, st)
   const bool wide = (V % 128 == 0);
   if (dtype == 1) {
-    if (K == 128 && wide) GDN_BWD(bf16_t, 128, 4, 2, 64, 64);
-    if (K == 128) GDN_BWD(bf16_t, 128, 2, 2, 64, 64);
-    if (wide) GDN_BWD(bf16_t, 64, 4, 2, 64, 64);
-    GDN_BWD(bf16_t, 64, 2, 2, 64, 64);
+    if (K == 128 && wide) GDN_BWD(bf16_t, 128, 4, 2, 2, 64, 64);
+    if (K == 128) GDN_BWD(bf16_t, 128, 2, 2, 2, 64, 64);
+    if (wide) GDN_BWD(bf16_t, 64, 4, 2, 2, 64, 64);
+    GDN_BWD(bf16_t, 64, 2, 2, 2, 64, 64);
   } else {
-    if (K == 128) GDN_BWD(float, 128, 2, 1, 64, 64);
-    GDN_BWD(float, 64, 2, 2, 64, 64);
+    if (K == 128) GDN_BWD(float, 128, 2, 2, 1, 64, 64);
+    GDN_BWD(float, 64, 2, 2, 2, 64, 64);
   }
 #undef GDN_BWD
 }

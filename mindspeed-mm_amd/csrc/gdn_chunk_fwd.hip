@@ -581,7 +581,7 @@ template <typename K> static int set_lds(K kernel, int bytes) {
                                   bytes);
 }
 
-template <typename T, int DK, int BVP, int NW, int STAGES>
+template <typename T, int DK, int BVP, int NW, int NWS, int STAGES>
 static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const void* q, const void* k, const void* v,
                             const float* g, const float* beta, const float* h0, const int64_t* cu, void* o, float* ht,
                             unsigned char* ws, float scale, int l2norm, bool with_backward, hipStream_t st) {
@@ -619,10 +619,10 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
                (const int*)chunk_offsets, G, Ai, W, UF, AQ, KDF, WF, d.T, d.N, d.Hqk, d.Hv, d.V);
   }
   {
-    auto kern = chunk_state_kernel<T, DK, NW, STAGES>;
-    constexpr int smem = StateSmem<T, DK, NW, STAGES>::bytes;
+    auto kern = chunk_state_kernel<T, DK, NWS, STAGES>;
+    constexpr int smem = StateSmem<T, DK, NWS, STAGES>::bytes;
     if (int e = set_lds(kern, smem)) return e;
-    GDN_LAUNCH(kKernStateFwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NW)), dim3(128 * NW), smem, st,
+    GDN_LAUNCH(kKernStateFwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NWS)), dim3(128 * NWS), smem, st,
                (const T*)KDF, (const T*)W, (const T*)UF, (const float*)G, h0, ht, VF, HF, cu,
                (const int*)chunk_offsets, d.T, d.Hv, d.V);
   }
@@ -663,20 +663,20 @@ extern "C" int gdn_chunk_fwd(const void* q, const void* k, const void* v, const 
   if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
   unsigned char* ws = static_cast<unsigned char*>(workspace);
   hipStream_t st = (hipStream_t)stream;
-#define GDN_FWD(T_, DK_, BVP_, NW_, ST_)                                                                          \
-  return chunk_fwd_launch<T_, DK_, BVP_, NW_, ST_>(d, L, q, k, v, g, beta, initial_state, cu_seqlens, o, final_state, \
+#define GDN_FWD(T_, DK_, BVP_, NW_, NWS_, ST_)                                                                        \
+  return chunk_fwd_launch<T_, DK_, BVP_, NW_, NWS_, ST_>(d, L, q, k, v, g, beta, initial_state, cu_seqlens, o, final_state, \
                                                    ws, scale, use_qk_l2norm, with_bwd, st)
   const bool wide = (V % 128 == 0);
   if (dtype == 1) {
-    if (K == 128 && wide) GDN_FWD(bf16_t, 128, 128, 4, 2);
-    if (K == 128) GDN_FWD(bf16_t, 128, 64, 2, 2);
-    if (K == 64 && wide) GDN_FWD(bf16_t, 64, 128, 4, 2);
-    GDN_FWD(bf16_t, 64, 64, 2, 2);
+    if (K == 128 && wide) GDN_FWD(bf16_t, 128, 128, 4, 2, 2);
+    if (K == 128) GDN_FWD(bf16_t, 128, 64, 2, 2, 2);
+    if (K == 64 && wide) GDN_FWD(bf16_t, 64, 128, 4, 2, 2);
+    GDN_FWD(bf16_t, 64, 64, 2, 2, 2);
   } else {
-    if (K == 128 && wide) GDN_FWD(float, 128, 64, 4, 1);
-    if (K == 128) GDN_FWD(float, 128, 64, 2, 1);
-    if (wide) GDN_FWD(float, 64, 64, 4, 2);
-    GDN_FWD(float, 64, 64, 2, 2);
+    if (K == 128 && wide) GDN_FWD(float, 128, 64, 4, 4, 1);
+    if (K == 128) GDN_FWD(float, 128, 64, 2, 2, 1);
+    if (wide) GDN_FWD(float, 64, 64, 4, 4, 2);
+    GDN_FWD(float, 64, 64, 2, 2, 2);
   }
 #undef GDN_FWD
 }

@@ -6,7 +6,7 @@
 namespace gdn {
 
 enum KernelId {
-  kKernChunkTable = 0, kKernL2Norm, kKernPrep, kKernStateFwd, kKernOut, kKernDvLocal, kKernStateBwd, kKernDqkw,
+  kKernChunkTable = 0, kKernL2Norm, kKernPrep, kKernStateFwd, kKernOut, kKernBwdPrep, kKernStateBwd, kKernDqkw,
   kKernWyBwd, kKernQkFinalize, kKernRecurrent, kKernConvFwd, kKernConvState, kKernConvBwd, kKernConvReduce,
   kKernConvDh0, kKernConvUpdate, kKernCount
 };
