@@ -47,8 +47,9 @@ def kernel_matmul_flops(K, V, C=64):
         "chunk_out_kernel": g(C, V, K) + g(C, V, C),                       # Q S, Aq V'
         "chunk_bwd_prep_kernel": g(C, V, C),                               # Aq^T dO
         "chunk_state_bwd_kernel": g(C, V, K) + 2 * g(K, V, C),             # K dS, Q^T dO, W^T dV'
-        "chunk_dqkw_kernel": g(C, C, V) + 3 * g(C, K, V) + 2 * g(C, K, C),
-        "chunk_wy_bwd_kernel": g(C, K, C) + g(C, C, K) + g(C, V, C) + g(C, C, V) + 2 * g(C, C, C) + 2 * g(C, K, C),
+        # dO V'^T, dO S^T, V' dS^T, dV' S^T, ds K, ds^T Q | Tm^T dW, dW K^T, Tm^T dV', dV' V^T, dTm Tm^T, Tm^T X, dM K, dM^T K
+        "chunk_bwd_local_kernel": g(C, C, V) + 3 * g(C, K, V) + 2 * g(C, K, C)
+                                  + g(C, K, C) + g(C, C, K) + g(C, V, C) + g(C, C, V) + 2 * g(C, C, C) + 2 * g(C, K, C),
     }
 
 

@@ -37,9 +37,7 @@ struct ChunkWorkspace {
   int64_t DOF;            // T [chunks,Hv,V/32,2]    dO
   int64_t DVF;            // T [chunks,Hv,V/32,2]    d(v_new)
   int64_t DHF;            // T [chunks,Hv,V/32,K/32] gradient of the state AFTER each chunk
-  int64_t DWF;            // T [chunks,Hv,K/32,2]    dW, tile = (32 tokens) x (32 columns of K)
   int64_t DQH, DKH;       // T [tokens,Hv,K]  per-value-head dq, dk before the group sum
-  int64_t DG;             // f32 [tokens,Hv]  gradient w.r.t. the cumulative decay (two partial terms)
   int64_t total_bytes;
 };
 
@@ -69,10 +67,8 @@ inline ChunkWorkspace chunk_workspace_layout(const ChunkDims& d, int elem_bytes)
   w.DOF = take(nc * 64 * d.Hv * d.V * elem_bytes);
   w.DVF = take(nc * 64 * d.Hv * d.V * elem_bytes);
   w.DHF = take(nc * d.Hv * d.V * d.K * elem_bytes);
-  w.DWF = take(nc * 64 * d.Hv * d.K * elem_bytes);
   w.DQH = take(tok * d.Hv * d.K * elem_bytes);
   w.DKH = take(tok * d.Hv * d.K * elem_bytes);
-  w.DG = take(tok * d.Hv * 4);
   w.total_bytes = off;
   return w;
 }

@@ -3,10 +3,10 @@
 //   dv_local = scale tril(Q K^T . Gam)^T dO                                   chunk_bwd_prep_kernel
 //   dV' = (K dS') . e^{G_last-G} + dv_local                                   chunk_state_bwd_kernel
 //   dS  = e^{G_last} dS' + scale (Q . e^G)^T dO - W^T dV'                       (reverse recurrence)
-//   ds  = scale tril(dO V'^T . Gam);  dQ = scale e^G . (dO S^T) + ds K          chunk_dqkw_kernel
+//   ds  = scale tril(dO V'^T . Gam);  dQ = scale e^G . (dO S^T) + ds K          chunk_bwd_local_kernel
 //   dK1 = e^{G_last-G} . (V' dS'^T) + ds^T Q;  dW = -dV' S^T
 //   dG1_i = <q_i,dQ_i> - <k_i,dK1_i>  (+ e^{G_last}<S,dS'> + sum_j <k_j, dK_inter_j> at the last row)
-//   back through W = Tm (beta e^G K), U = Tm (beta V), Tm = (I+L)^-1:           chunk_wy_bwd_kernel
+//   back through W = Tm (beta e^G K), U = Tm (beta V), Tm = (I+L)^-1:           (same kernel)
 //     P = Tm^T dW, R = Tm^T dV', dTm = strict_tril(dW Kb^T + dV' Vb^T), dM = -(Tm^T dTm Tm^T) . Gam
 //     dK2 = P beta e^G + beta (dM K) + dM^T (beta K);  dv = R beta
 //     dbeta = e^G<P,k> + <R,v> + <dM K, k>;  dG2 = beta e^G<P,k> + beta<dM K,k> - <dM^T(beta K),k>
@@ -328,121 +328,179 @@ __global__ __launch_bounds__(128 * NW) void chunk_state_bwd_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
-// chunk_dqkw_kernel, per (chunk, head), 4 waves; wave w owns the 32 K-columns [32w, 32w+32) of dQ, dK, dW.
-// v_new, d(v_new), S and dS' arrive in fragment order with (lane <-> V column); the contractions here run over V,
-// so every tile is first turned through the matrix core (mfma_transpose) into (lane <-> token / K column,
-// registers <-> V) and then used from registers: the main loop reads nothing but dO from LDS.
+// chunk_bwd_local_kernel, per (chunk, head), 4 waves: everything of the backward pass that is local to a chunk once
+// the reverse recurrence has left dS' and dV' behind.  Wave w owns the 32 K-columns [32w, 32w+32) of dQ, dK, dW and
+// the 32x32 tile (w/2, w%2) of the 64x64 intra-chunk matrices.
+//   main loop over 32-column V blocks (no workgroup barrier, nothing but V in LDS):
+//     v_new, dV', dO, S, dS' arrive in fragment order with (lane <-> V column); the contractions run over V, so each
+//     tile is turned through the matrix core (mfma_transpose) into (lane <-> token / K column, registers <-> V).
+//       ds += dO V'^T   a2 += dV' V^T   dQ += dO S^T   dK += V' dS'^T   dW += dV' S^T   R = Tm^T dV' -> dv, dbeta
+//   epilogue: dQ += ds K, dK += ds^T Q, dG rows as <q,dQ> - <k,dK>; then back through W = Tm (beta e^G K) with dW
+//   still in registers: P = Tm^T dW, a1 = dW K^T, dTm = strict_tril(a1 beta e^G + a2 beta), dM = -(Tm^T dTm Tm^T).Gam,
+//   dK += beta e^G P + beta (dM K) + dM^T (beta K); dbeta, dg.  dQ, dK, dv leave as 16-byte row pieces.
 // ---------------------------------------------------------------------------------------------
-template <typename T, int DK, int BV> struct DqkwSmem {
-  static constexpr int LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
-  static constexpr int main_bytes = 64 * LDV * (int)sizeof(T);                       // dO tile
-  static constexpr int post_bytes = (2 * DK * kLT + 2 * 64 * L64) * (int)sizeof(T);  // K^T, Q^T, ds, ds^T
-  static constexpr int off_row = main_bytes > post_bytes ? main_bytes : post_bytes;
-  static constexpr int bytes = off_row + (4 * 64 + 8) * 4;
+template <typename T, int DK, int BV> struct BwdLocalSmem {
+  static constexpr int LDK = lds_ld<T>(DK), LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
+  static constexpr int vw_elems = 64 * (LDV > LDK ? LDV : LDK);
+  static constexpr int off_ks = 0;                                            // K     [64][LDK]
+  static constexpr int off_tmt = off_ks + 64 * LDK * (int)sizeof(T);          // Tm^T  [64][kLT]
+  static constexpr int off_tm = off_tmt + 64 * kLT * (int)sizeof(T);          // Tm    [64][L64], later (beta . dM)^T
+  static constexpr int off_vw = off_tm + 64 * L64 * (int)sizeof(T);           // V [64][LDV]; later dW [64][LDK]; later store patches
+  static constexpr int off_ds = off_vw + vw_elems * (int)sizeof(T);           // store patches; ds | ds^T; dTm, dM | X^T
+  static constexpr int off_row = off_ds + 2 * 64 * L64 * (int)sizeof(T);
+  static constexpr int bytes = off_row + (6 * 64 + 8) * 4;
+  // store patches: one per wave in the main loop (dv), one per wave that owns K columns afterwards (dq, dk)
+  static_assert(4 * Patch<T>::kElems <= 2 * 64 * L64 && (DK / 32) * Patch<T>::kElems <= vw_elems, "store patches fit");
 };
 
-// rowacc[i0+i] += factor * sum_j acc[i][j] * other_t[(j0+j)*ld + i0+i]   (other given transposed: [column][row])
-template <typename T>
-__device__ __forceinline__ void acc_rowdot_add_t(const f32x16& acc, const T* other_t, int ld, int i0, int j0,
-                                                 float* rowacc, float factor) {
-  const int j = j0 + acc_col();
-#pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int i = i0 + acc_row(r);
-    const float s = row16_sum(acc[r] * Elem<T>::to_f(other_t[j * ld + i]));
-    if ((threadIdx.x & 15) == 0) atomicAdd(&rowacc[i], factor * s);
-  }
-}
-
 template <typename T, int DK, int BV>
-__global__ __launch_bounds__(kThreads, 2) void chunk_dqkw_kernel(
-    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ vf, const T* __restrict__ dvf,
-    const T* __restrict__ dO, const T* __restrict__ hf, const T* __restrict__ dhf, const float* __restrict__ G,
-    T* __restrict__ dqh, T* __restrict__ dkh, T* __restrict__ dwb, float* __restrict__ dG,
+__global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_local_kernel(
+    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ beta,
+    const float* __restrict__ G, const T* __restrict__ Ai, const T* __restrict__ vf, const T* __restrict__ dvf,
+    const T* __restrict__ dof, const T* __restrict__ hf, const T* __restrict__ dhf, T* __restrict__ dqh,
+    T* __restrict__ dkh, T* __restrict__ dv_out, float* __restrict__ dbeta, float* __restrict__ dg,
     const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V,
     float scale) {
-  using SM = DqkwSmem<T, DK, BV>;
-  constexpr int LDV = SM::LDV, L64 = SM::L64, NKT = DK / 32;
-  constexpr int NC = (NKT + 3) / 4;          // K-column blocks per wave (1 for K <= 128)
-  T* dOs = reinterpret_cast<T*>(gdn_smem);
-  T* KT = reinterpret_cast<T*>(gdn_smem);                   // post phase: [DK][kLT]
-  T* QT = KT + DK * kLT;
-  T* dsm = QT + DK * kLT;                                   // [64][L64]
+  using SM = BwdLocalSmem<T, DK, BV>;
+  constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64, NKT = DK / 32;
+  static_assert(NKT <= 4, "one 32-column block of K per wave");
+  T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
+  T* TmT = reinterpret_cast<T*>(gdn_smem + SM::off_tmt);
+  T* Tm = reinterpret_cast<T*>(gdn_smem + SM::off_tm);
+  T* Vs = reinterpret_cast<T*>(gdn_smem + SM::off_vw);
+  T* dsm = reinterpret_cast<T*>(gdn_smem + SM::off_ds);
   T* dsT = dsm + 64 * L64;
   float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_row);
-  float* rq = Gs + 64;     // <q_i, dQ_i>
-  float* rk = rq + 64;     // <k_i, dK1_i>
-  float* rki = rk + 64;    // <k_i, dK_inter_i>
-  float* wsum = rki + 64;  // per-wave partials of <S, dS'>
+  float* egs = Gs + 64;    // e^G
+  float* bs = egs + 64;    // beta
+  float* r1 = bs + 64;     // <q_i,dQ_i> - <k_i,dK1_i>
+  float* rb = r1 + 64;     // dbeta
+  float* rg = rb + 64;     // dG through W, U
+  float* wsum = rg + 64;   // per wave: <S,dS'> [0..3], sum_i <k_i, dK_inter_i> [4..7]
+  T* dWs = Vs;
+  T* dAs = dsm;
+  T* XT = dsT;
+  T* dMs = dsm;
+  T* dMTb = Tm;
 
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31;
+  const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: branches on it are scalar
   const int h = blockIdx.y, hq = h / (Hv / Hqk), nvalid = s.nvalid;
   const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk;
   const int64_t ch = (int64_t)blockIdx.x * Hv + h;
-  const int ti = wave >> 1, tj = wave & 1;
+  const int ti = wave >> 1, tj = wave & 1, cj = wave;
+  const bool lower = tj <= ti, has_k = wave < NKT;
 
   if (tid < 64) {
-    Gs[tid] = G[(tok0 + imin(tid, nvalid - 1)) * Hv + h];
-    rq[tid] = 0.f; rk[tid] = 0.f; rki[tid] = 0.f;
+    const float gv = G[(tok0 + imin(tid, nvalid - 1)) * Hv + h];
+    Gs[tid] = gv;
+    egs[tid] = __expf(gv);
+    bs[tid] = tid < nvalid ? beta[(tok0 + tid) * Hv + h] : 0.f;
+    r1[tid] = 0.f; rb[tid] = 0.f; rg[tid] = 0.f;
   }
+  load_tile<T, 64>(Tm, L64, Ai + (tok0 * Hv + h) * 64, (int64_t)Hv * 64, nvalid, tid);
+  load_tile_t<T, 64, kThreads>(TmT, kLT, Ai + (tok0 * Hv + h) * 64, (int64_t)Hv * 64, nvalid, tid);
+  load_tile<T, DK>(Ks, LDK, k + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
+
   IdentityFrag<T> id;
   id.init();
-  f32x16 ds = acc_zero(), dQi[NC][2], dKi[NC][2], dWa[NC][2];
+  f32x16 ds = acc_zero(), a2 = acc_zero(), dQi[2], dKi[2], dWa[2];
 #pragma unroll
-  for (int c = 0; c < NC; ++c)
-#pragma unroll
-    for (int ri = 0; ri < 2; ++ri) { dQi[c][ri] = acc_zero(); dKi[c][ri] = acc_zero(); dWa[c][ri] = acc_zero(); }
+  for (int ri = 0; ri < 2; ++ri) { dQi[ri] = acc_zero(); dKi[ri] = acc_zero(); dWa[ri] = acc_zero(); }
   float sds = 0.f;
 
   for (int vb = 0; vb < V / BV; ++vb) {
     if (vb > 0) __syncthreads();
-    load_tile<T, BV>(dOs, LDV, dO + (tok0 * Hv + h) * V + vb * BV, (int64_t)Hv * V, nvalid, tid);
+    load_tile<T, BV>(Vs, LDV, v + (tok0 * Hv + h) * V + vb * BV, (int64_t)Hv * V, nvalid, tid);
     __syncthreads();
 #pragma unroll
     for (int v32 = 0; v32 < BV / 32; ++v32) {
       const int vblk = vb * (BV / 32) + v32;
       const int64_t t2 = (ch * (V / 32) + vblk) * 2, tk = (ch * (V / 32) + vblk) * NKT;
-      AccB<T> f, Vt[2], dVt[2], dOf[2];
+      // Operands are brought in one after the other so that few fragments are live at a time; tile indices that
+      // depend on the wave are compared against loop constants (fragments indexed at run time would go to scratch).
+      AccB<T> f, Sf, dSf, dOt[2];
+      if (has_k) {                           // (lane <-> K column, registers <-> V)
+        f.load(hf + (tk + cj) * 1024);
+        const f32x16 st = mfma_transpose<T>(f, id);
+        Sf.pack(st);
+        f.load(dhf + (tk + cj) * 1024);
+        const f32x16 dst = mfma_transpose<T>(f, id);
+        dSf.pack(dst);
 #pragma unroll
-      for (int ri = 0; ri < 2; ++ri) {       // (lane <-> token, registers <-> V)
-        f.load(vf + (t2 + ri) * 1024);
-        Vt[ri].pack(mfma_transpose<T>(f, id));
-        f.load(dvf + (t2 + ri) * 1024);
-        dVt[ri].pack(mfma_transpose<T>(f, id));
-        frags_from_lds<T>(dOf[ri], dOs + (32 * ri + l32) * LDV + 32 * v32);
+        for (int r = 0; r < 16; ++r) sds += st[r] * dst[r];
       }
-      if (tj <= ti) mma32_ff<T>(ds, dOf[ti], Vt[tj]);
 #pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        const int kt = wave + 4 * c;
-        if (kt < NKT) {
-          AccB<T> Sf, dSf;                   // (lane <-> K column, registers <-> V)
-          f.load(hf + (tk + kt) * 1024);
-          const f32x16 st = mfma_transpose<T>(f, id);
-          Sf.pack(st);
-          f.load(dhf + (tk + kt) * 1024);
-          const f32x16 dst = mfma_transpose<T>(f, id);
-          dSf.pack(dst);
+      for (int ri = 0; ri < 2; ++ri) {       // (lane <-> token, registers <-> V) from here on
+        f.load(dof + (t2 + ri) * 1024);
+        dOt[ri].pack(mfma_transpose<T>(f, id));
+        if (has_k) mma32_ff<T>(dQi[ri], dOt[ri], Sf);
+      }
 #pragma unroll
-          for (int r = 0; r < 16; ++r) sds += st[r] * dst[r];
+      for (int ri = 0; ri < 2; ++ri) {
+        AccB<T> Vt;
+        f.load(vf + (t2 + ri) * 1024);
+        Vt.pack(mfma_transpose<T>(f, id));
+        if (has_k) mma32_ff<T>(dKi[ri], Vt, dSf);
+        if (lower && ri == tj) {
+          if (ti == 0) mma32_ff<T>(ds, dOt[0], Vt); else mma32_ff<T>(ds, dOt[1], Vt);
+        }
+      }
 #pragma unroll
-          for (int ri = 0; ri < 2; ++ri) {
-            mma32_ff<T>(dQi[c][ri], dOf[ri], Sf);
-            mma32_ff<T>(dKi[c][ri], Vt[ri], dSf);
-            mma32_ff<T>(dWa[c][ri], dVt[ri], Sf);
-          }
+      for (int ri = 0; ri < 2; ++ri) {
+        AccB<T> dVt;
+        f.load(dvf + (t2 + ri) * 1024);
+        dVt.pack(mfma_transpose<T>(f, id));
+        if (has_k) mma32_ff<T>(dWa[ri], dVt, Sf);
+        if (lower && ri == ti) {
+          frags_from_lds<T>(f, Vs + (32 * tj + l32) * LDV + 32 * v32);
+          mma32_ff<T>(a2, dVt, f);
+        }
+      }
+      if ((vblk & 3) == wave) {              // R = Tm^T dV' for this V block: dv = beta R, dbeta += <R, v>
+        AccB<T> fdv[2];
+        fdv[0].load(dvf + (t2 + 0) * 1024);
+        fdv[1].load(dvf + (t2 + 1) * 1024);
+#pragma unroll
+        for (int rj = 0; rj < 2; ++rj) {
+          f32x16 R = acc_zero(), p;
+#pragma unroll
+          for (int t = rj; t < 2; ++t) mma32_accb<T>(R, TmT + (32 * rj + l32) * kLT + 32 * t, fdv[t]);
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            p[r] = R[r] * Elem<T>::to_f(Vs[(32 * rj + acc_row(r)) * LDV + 32 * v32 + acc_col()]);
+          rows_add(p, rb, 32 * rj);
+#pragma unroll
+          for (int r = 0; r < 16; ++r) R[r] *= bs[32 * rj + acc_row(r)];
+          acc_store_rows<T>(R, dsm + wave * Patch<T>::kElems, dv_out + ((tok0 + 32 * rj) * Hv + h) * V + 32 * vblk,
+                            (int64_t)Hv * V, nvalid - 32 * rj);
         }
       }
     }
   }
   sds = wave_sum(sds);
   if (lane == 0) wsum[wave] = sds;
-  __syncthreads();   // dO tile consumed; its space is reused below
 
-  load_tile_t<T, DK, kThreads>(KT, kLT, k + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
-  load_tile_t<T, DK, kThreads>(QT, kLT, q + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
+  // this wave's K and Q columns as (lane <-> column, registers <-> token): B operands and row-dot partners
+  AccB<T> KTf[2], QTf[2];
+  if (has_k) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      AccB<T> f;
+      frags_from_lds<T>(f, Ks + (32 * t + l32) * LDK + 32 * cj);
+      KTf[t].pack(mfma_transpose<T>(f, id));
+      const int row = 32 * t + l32;
+      frags_from_lds<T>(f, q + ((tok0 + imin(row, nvalid - 1)) * Hqk + hq) * DK + 32 * cj);
+      if (row >= nvalid) {
+#pragma unroll
+        for (int g = 0; g < AccK<T>::kGroups; ++g) f.f[g] = u32x4{0u, 0u, 0u, 0u};
+      }
+      QTf[t].pack(mfma_transpose<T>(f, id));
+    }
+  }
+  __syncthreads();   // every wave is done with the V tile and the main-loop store patches
   {
     const int j = 32 * tj + acc_col();
 #pragma unroll
@@ -453,195 +511,61 @@ __global__ __launch_bounds__(kThreads, 2) void chunk_dqkw_kernel(
       dsT[j * L64 + i] = Elem<T>::from_f(val);
     }
   }
+  AccB<T> dWb[2];
+  if (has_k) {
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dWa[ri][r] = -dWa[ri][r];
+      acc_to_lds(dWa[ri], dWs, LDK, 32 * ri, 32 * cj);
+      dWb[ri].pack(dWa[ri]);
+    }
+  }
   __syncthreads();
   const float glast = Gs[63];
-  T* dqg = dqh + (tok0 * Hv + h) * DK;
-  T* dkg = dkh + (tok0 * Hv + h) * DK;
+  float ski = 0.f;
+  if (has_k) {
 #pragma unroll
-  for (int c = 0; c < NC; ++c) {
-    const int cj = wave + 4 * c;
-    if (cj < NKT) {
+    for (int ri = 0; ri < 2; ++ri) {
+      const f32x16 kk = KTf[ri].unpack(), qq = QTf[ri].unpack();
 #pragma unroll
-      for (int ri = 0; ri < 2; ++ri) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float gi = Gs[32 * ri + acc_row(r)];
-          dQi[c][ri][r] *= scale * __expf(gi);
-          dKi[c][ri][r] *= __expf(glast - gi);
-          dWa[c][ri][r] = -dWa[c][ri][r];
-        }
-        acc_rowdot_add_t<T>(dKi[c][ri], KT, kLT, 32 * ri, 32 * cj, rki, 1.f);   // still only the inter-chunk part
-        mma32_ss<T, 64>(dQi[c][ri], dsm + (32 * ri + l32) * L64, KT + (32 * cj + l32) * kLT);
-        mma32_ss<T, 64>(dKi[c][ri], dsT + (32 * ri + l32) * L64, QT + (32 * cj + l32) * kLT);
-        acc_rowdot_add_t<T>(dQi[c][ri], QT, kLT, 32 * ri, 32 * cj, rq, 1.f);
-        acc_rowdot_add_t<T>(dKi[c][ri], KT, kLT, 32 * ri, 32 * cj, rk, 1.f);
-        acc_to_global(dQi[c][ri], dqg, (int64_t)Hv * DK, 32 * ri, 32 * cj, nvalid);
-        acc_to_global(dKi[c][ri], dkg, (int64_t)Hv * DK, 32 * ri, 32 * cj, nvalid);
-        AccB<T> wf;                        // dW as a B operand for the WY backward kernel
-        wf.pack(dWa[c][ri]);
-        wf.store(dwb + ((ch * NKT + cj) * 2 + ri) * 1024);
-      }
-    }
-  }
-  __syncthreads();
-  if (wave == 0) {
-    float val = rq[lane] - rk[lane];
-    const float tot = wave_sum(rki[lane]);
-    if (lane == nvalid - 1) val += __expf(glast) * (wsum[0] + wsum[1] + wsum[2] + wsum[3]) + tot;
-    if (lane < nvalid) dG[(tok0 + lane) * Hv + h] = val;
-  }
-}
-
-// ---------------------------------------------------------------------------------------------
-// chunk_wy_bwd_kernel, per (chunk, head), 4 waves: back through W = Tm (beta e^G K), U = Tm (beta V), Tm = (I+L)^-1.
-// dW and d(v_new) arrive in fragment order (lane <-> K / V column, registers <-> token): exactly the B operand of
-// P = Tm^T dW and R = Tm^T dU; their transposes through the matrix core are the A operands of dW K^T and dU V^T.
-// Wave w owns the 32 K-columns [32w, 32w+32) of dK and the V blocks w, w+4, ...
-// ---------------------------------------------------------------------------------------------
-template <typename T, int DK, int BV> struct WySmem {
-  static constexpr int LDK = lds_ld<T>(DK), LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
-  static constexpr int off_tmt = 0;                                           // Tm^T  [64][kLT]
-  static constexpr int off_tm = off_tmt + 64 * kLT * (int)sizeof(T);          // Tm    [64][L64]
-  static constexpr int off_ks = off_tm + 64 * L64 * (int)sizeof(T);           // K     [64][LDK]
-  static constexpr int off_vs = off_ks + 64 * LDK * (int)sizeof(T);           // V     [64][LDV], later (beta . dM)^T
-  static constexpr int off_da = off_vs + 64 * LDV * (int)sizeof(T);           // dTm, later dM  [64][L64]
-  static constexpr int off_xt = off_da + 64 * L64 * (int)sizeof(T);           // X^T   [64][L64]
-  static constexpr int off_row = off_xt + 64 * L64 * (int)sizeof(T);
-  static constexpr int bytes = off_row + 5 * 64 * 4;
-  static_assert(LDV >= L64, "dM^T reuses the V tile");
-};
-
-// rowacc[i0+i] += factor * sum_j acc[i][j] * other[i][j] with `other` given as an accumulator tile
-__device__ __forceinline__ void acc_rowdot_add_r(const f32x16& acc, const f32x16& other, int i0, float* rowacc,
-                                                 float factor) {
-#pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const float s = row16_sum(acc[r] * other[r]);
-    if ((threadIdx.x & 15) == 0) atomicAdd(&rowacc[i0 + acc_row(r)], factor * s);
-  }
-}
-
-template <typename T, int DK, int BV>
-__global__ __launch_bounds__(kThreads, 2) void chunk_wy_bwd_kernel(
-    const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ beta, const float* __restrict__ G,
-    const T* __restrict__ Ai, const T* __restrict__ dwf, const T* __restrict__ dvf, T* dkh, const float* dG1,
-    T* __restrict__ dv_out, float* __restrict__ dbeta, float* __restrict__ dg, const int64_t* __restrict__ cu,
-    const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V) {
-  using SM = WySmem<T, DK, BV>;
-  constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64, NKT = DK / 32;
-  constexpr int NC = (NKT + 3) / 4;
-  T* TmT = reinterpret_cast<T*>(gdn_smem + SM::off_tmt);
-  T* Tm = reinterpret_cast<T*>(gdn_smem + SM::off_tm);
-  T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
-  T* Vs = reinterpret_cast<T*>(gdn_smem + SM::off_vs);
-  T* dAs = reinterpret_cast<T*>(gdn_smem + SM::off_da);
-  T* XT = reinterpret_cast<T*>(gdn_smem + SM::off_xt);
-  float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_row);
-  float* bs = Gs + 64;
-  float* rb = bs + 64;     // dbeta
-  float* rg = rb + 64;     // dG2
-  float* egs = rg + 64;    // e^G
-  T* dMs = dAs;
-  T* dMTb = Vs;
-
-  const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
-  if (s.nvalid <= 0) return;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31;
-  const int h = blockIdx.y, hq = h / (Hv / Hqk), nvalid = s.nvalid;
-  const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk;
-  const int64_t ch = (int64_t)blockIdx.x * Hv + h;
-  const int ti = wave >> 1, tj = wave & 1;
-
-  if (tid < 64) {
-    const float gv = G[(tok0 + imin(tid, nvalid - 1)) * Hv + h];
-    Gs[tid] = gv;
-    egs[tid] = __expf(gv);
-    bs[tid] = tid < nvalid ? beta[(tok0 + tid) * Hv + h] : 0.f;
-    rb[tid] = 0.f; rg[tid] = 0.f;
-  }
-  load_tile<T, 64>(Tm, L64, Ai + (tok0 * Hv + h) * 64, (int64_t)Hv * 64, nvalid, tid);
-  load_tile_t<T, 64, kThreads>(TmT, kLT, Ai + (tok0 * Hv + h) * 64, (int64_t)Hv * 64, nvalid, tid);
-  load_tile<T, DK>(Ks, LDK, k + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
-  __syncthreads();
-
-  IdentityFrag<T> id;
-  id.init();
-  // K columns of this wave as (lane <-> K column, registers <-> token); P = Tm^T dW; dK2 = beta e^G P; t1 = e^G<P,k>
-  AccB<T> KTf[NC][2];
-  f32x16 dK[NC][2];
-#pragma unroll
-  for (int c = 0; c < NC; ++c) {
-    const int cj = wave + 4 * c;
-    dK[c][0] = acc_zero();
-    dK[c][1] = acc_zero();
-    if (cj < NKT) {
-      AccB<T> f, dwb[2];
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        frags_from_lds<T>(f, Ks + (32 * t + l32) * LDK + 32 * cj);
-        KTf[c][t].pack(mfma_transpose<T>(f, id));
-        dwb[t].load(dwf + ((ch * NKT + cj) * 2 + t) * 1024);
+      for (int r = 0; r < 16; ++r) {
+        const float gi = Gs[32 * ri + acc_row(r)];
+        dQi[ri][r] *= scale * __expf(gi);
+        dKi[ri][r] *= __expf(glast - gi);
+        ski += dKi[ri][r] * kk[r];           // still only the inter-chunk part
       }
 #pragma unroll
-      for (int rj = 0; rj < 2; ++rj) {
+      for (int t = 0; t <= ri; ++t) mma32_accb<T>(dQi[ri], dsm + (32 * ri + l32) * L64 + 32 * t, KTf[t]);
 #pragma unroll
-        for (int t = rj; t < 2; ++t) mma32_accb<T>(dK[c][rj], TmT + (32 * rj + l32) * kLT + 32 * t, dwb[t]);
-        const f32x16 kk = KTf[c][rj].unpack();
+      for (int t = ri; t < 2; ++t) mma32_accb<T>(dKi[ri], dsT + (32 * ri + l32) * L64 + 32 * t, QTf[t]);
+      f32x16 p;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) dK[c][rj][r] *= egs[32 * rj + acc_row(r)];
-        acc_rowdot_add_r(dK[c][rj], kk, 32 * rj, rb, 1.f);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) dK[c][rj][r] *= bs[32 * rj + acc_row(r)];
-        acc_rowdot_add_r(dK[c][rj], kk, 32 * rj, rg, 1.f);
-      }
+      for (int r = 0; r < 16; ++r) p[r] = dQi[ri][r] * qq[r] - dKi[ri][r] * kk[r];
+      rows_add(p, r1, 32 * ri);
     }
   }
-  // dTm pieces (strictly lower tiles only): a1 = dW K^T, a2 = dU V^T
-  f32x16 a1 = acc_zero(), a2 = acc_zero();
-  if (tj <= ti) {
+  ski = wave_sum(ski);
+  if (lane == 0) wsum[4 + wave] = ski;
+  // dTm pieces (lower tiles only): a1 = dW K^T over all of K, a2 = dV' V^T from the main loop
+  f32x16 a1 = acc_zero();
+  if (lower) mma32<T, DK, true, true>(a1, dWs + 32 * ti * LDK, LDK, Ks + 32 * tj * LDK, LDK);
+  if (has_k) {       // P = Tm^T dW; dK += beta e^G P; dbeta += e^G <P,k>; dG += beta e^G <P,k>
 #pragma unroll
-    for (int kt = 0; kt < NKT; ++kt) {
-      AccB<T> f, wt, kf;
-      f.load(dwf + ((ch * NKT + kt) * 2 + ti) * 1024);
-      wt.pack(mfma_transpose<T>(f, id));                       // (lane <-> token i, registers <-> K column)
-      frags_from_lds<T>(kf, Ks + (32 * tj + l32) * LDK + 32 * kt);
-      mma32_ff<T>(a1, wt, kf);
+    for (int rj = 0; rj < 2; ++rj) {
+      f32x16 P = acc_zero(), p;
+#pragma unroll
+      for (int t = rj; t < 2; ++t) mma32_accb<T>(P, TmT + (32 * rj + l32) * kLT + 32 * t, dWb[t]);
+      const f32x16 kk = KTf[rj].unpack();
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { P[r] *= egs[32 * rj + acc_row(r)]; p[r] = P[r] * kk[r]; }
+      rows_add(p, rb, 32 * rj);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { P[r] *= bs[32 * rj + acc_row(r)]; p[r] = P[r] * kk[r]; dKi[rj][r] += P[r]; }
+      rows_add(p, rg, 32 * rj);
     }
   }
-
-  for (int vb = 0; vb < V / BV; ++vb) {
-    const int v0 = vb * BV;
-    if (vb > 0) __syncthreads();
-    load_tile<T, BV>(Vs, LDV, v + (tok0 * Hv + h) * V + v0, (int64_t)Hv * V, nvalid, tid);
-    __syncthreads();
-    for (int v32 = wave; v32 < BV / 32; v32 += 4) {            // R = Tm^T dU, dv = beta R
-      const int vblk = v0 / 32 + v32;
-      AccB<T> dub[2];
-      dub[0].load(dvf + ((ch * (V / 32) + vblk) * 2 + 0) * 1024);
-      dub[1].load(dvf + ((ch * (V / 32) + vblk) * 2 + 1) * 1024);
-      T* dvg = dv_out + (tok0 * Hv + h) * V + 32 * vblk;
-#pragma unroll
-      for (int rj = 0; rj < 2; ++rj) {
-        f32x16 R = acc_zero();
-#pragma unroll
-        for (int t = rj; t < 2; ++t) mma32_accb<T>(R, TmT + (32 * rj + l32) * kLT + 32 * t, dub[t]);
-        acc_rowdot_add<T>(R, Vs, LDV, 32 * rj, 32 * v32, rb, 1.f);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) R[r] *= bs[32 * rj + acc_row(r)];
-        acc_to_global(R, dvg, (int64_t)Hv * V, 32 * rj, 0, nvalid);
-      }
-    }
-    if (tj <= ti) {
-#pragma unroll
-      for (int v32 = 0; v32 < BV / 32; ++v32) {
-        AccB<T> f, ut, vfr;
-        f.load(dvf + ((ch * (V / 32) + v0 / 32 + v32) * 2 + ti) * 1024);
-        ut.pack(mfma_transpose<T>(f, id));                     // (lane <-> token i, registers <-> V column)
-        frags_from_lds<T>(vfr, Vs + (32 * tj + l32) * LDV + 32 * v32);
-        mma32_ff<T>(a2, ut, vfr);
-      }
-    }
-  }
+  __syncthreads();   // ds, ds^T and the dW tile are consumed
   {  // dTm[i][j] = beta_j (e^{G_j} a1 + a2), i > j
     const int j = 32 * tj + acc_col();
 #pragma unroll
@@ -649,6 +573,13 @@ __global__ __launch_bounds__(kThreads, 2) void chunk_wy_bwd_kernel(
       const int i = 32 * ti + acc_row(r);
       dAs[i * L64 + j] = Elem<T>::from_f(i > j ? bs[j] * (egs[j] * a1[r] + a2[r]) : 0.f);
     }
+  }
+  T* patch = dWs + wave * Patch<T>::kElems;
+  if (has_k) {
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri)
+      acc_store_rows<T>(dQi[ri], patch, dqh + ((tok0 + 32 * ri) * Hv + h) * DK + 32 * cj, (int64_t)Hv * DK,
+                        nvalid - 32 * ri);
   }
   __syncthreads();
   {  // X = dTm Tm^T, stored transposed
@@ -670,35 +601,34 @@ __global__ __launch_bounds__(kThreads, 2) void chunk_wy_bwd_kernel(
     }
   }
   __syncthreads();
-  T* dkg = dkh + (tok0 * Hv + h) * DK;
+  if (has_k) {       // E = dM K, F = dM^T (beta K): dK += beta E + F; dbeta += <E,k>; dG += beta <E,k> - <F,k>
 #pragma unroll
-  for (int c = 0; c < NC; ++c) {
-    const int cj = wave + 4 * c;
-    if (cj < NKT) {
+    for (int ri = 0; ri < 2; ++ri) {
+      f32x16 E = acc_zero(), Fm = acc_zero(), p;
 #pragma unroll
-      for (int ri = 0; ri < 2; ++ri) {
-        f32x16 E = acc_zero(), Fm = acc_zero();
+      for (int t = 0; t <= ri; ++t) mma32_accb<T>(E, dMs + (32 * ri + l32) * L64 + 32 * t, KTf[t]);
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          mma32_accb<T>(E, dMs + (32 * ri + l32) * L64 + 32 * t, KTf[c][t]);
-          mma32_accb<T>(Fm, dMTb + (32 * ri + l32) * L64 + 32 * t, KTf[c][t]);
-        }
-        const f32x16 kk = KTf[c][ri].unpack();
-        acc_rowdot_add_r(E, kk, 32 * ri, rb, 1.f);
-        acc_rowdot_add_r(Fm, kk, 32 * ri, rg, -1.f);
+      for (int t = ri; t < 2; ++t) mma32_accb<T>(Fm, dMTb + (32 * ri + l32) * L64 + 32 * t, KTf[t]);
+      const f32x16 kk = KTf[ri].unpack();
 #pragma unroll
-        for (int r = 0; r < 16; ++r) E[r] *= bs[32 * ri + acc_row(r)];
-        acc_rowdot_add_r(E, kk, 32 * ri, rg, 1.f);
-        const f32x16 k1 = acc_from_global(dkg, (int64_t)Hv * DK, 32 * ri, 32 * cj, nvalid);
+      for (int r = 0; r < 16; ++r) p[r] = E[r] * kk[r];
+      rows_add(p, rb, 32 * ri);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) dK[c][ri][r] += E[r] + Fm[r] + k1[r];
-        acc_to_global(dK[c][ri], dkg, (int64_t)Hv * DK, 32 * ri, 32 * cj, nvalid);
+      for (int r = 0; r < 16; ++r) {
+        E[r] *= bs[32 * ri + acc_row(r)];
+        p[r] = (E[r] - Fm[r]) * kk[r];
+        dKi[ri][r] += E[r] + Fm[r];
       }
+      rows_add(p, rg, 32 * ri);
+      acc_store_rows<T>(dKi[ri], patch, dkh + ((tok0 + 32 * ri) * Hv + h) * DK + 32 * cj, (int64_t)Hv * DK,
+                        nvalid - 32 * ri);
     }
   }
   __syncthreads();
   if (wave == 0) {   // d(cumulative G) -> d(g): suffix sum inside the chunk
-    float x = rg[lane] + (lane < nvalid ? dG1[(tok0 + lane) * Hv + h] : 0.f);
+    float x = rg[lane] + r1[lane];
+    if (lane == nvalid - 1)
+      x += __expf(glast) * (wsum[0] + wsum[1] + wsum[2] + wsum[3]) + (wsum[4] + wsum[5] + wsum[6] + wsum[7]);
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
       const float t = __shfl_down(x, d);
@@ -768,7 +698,7 @@ template <typename K> static int set_lds_b(K kernel, int bytes) {
                                   bytes);
 }
 
-template <typename T, int DK, int NW, int NWS, int STAGES, int BVQ, int BVW>
+template <typename T, int DK, int NW, int NWS, int STAGES, int BVL>
 static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const void* q, const void* k, const void* v,
                             const float* beta, const int64_t* cu, const void* dO, const float* dht, void* dq, void* dk,
                             void* dv, float* dg, float* dbeta, float* dh0, unsigned char* ws, float scale, int l2norm,
@@ -790,10 +720,8 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   T* DOF = reinterpret_cast<T*>(ws + L.DOF);
   T* DVF = reinterpret_cast<T*>(ws + L.DVF);
   T* DHF = reinterpret_cast<T*>(ws + L.DHF);
-  T* DW = reinterpret_cast<T*>(ws + L.DWF);
   T* DQH = reinterpret_cast<T*>(ws + L.DQH);
   T* DKH = reinterpret_cast<T*>(ws + L.DKH);
-  float* DG = reinterpret_cast<float*>(ws + L.DG);
   {
     auto kern = chunk_bwd_prep_kernel<T, DK, NW>;
     constexpr int smem = BwdPrepSmem<T, DK, NW>::bytes;
@@ -810,19 +738,12 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
                d.V);
   }
   {
-    auto kern = chunk_dqkw_kernel<T, DK, BVQ>;
-    constexpr int smem = DqkwSmem<T, DK, BVQ>::bytes;
+    auto kern = chunk_bwd_local_kernel<T, DK, BVL>;
+    constexpr int smem = BwdLocalSmem<T, DK, BVL>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
-    GDN_LAUNCH(kKernDqkw, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, VF, (const T*)DVF, (const T*)dO,
-               HF, (const T*)DHF, G, DQH, DKH, DW, DG, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale);
-  }
-  {
-    auto kern = chunk_wy_bwd_kernel<T, DK, BVW>;
-    constexpr int smem = WySmem<T, DK, BVW>::bytes;
-    if (int e = set_lds_b(kern, smem)) return e;
-    GDN_LAUNCH(kKernWyBwd, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, kk, (const T*)v, beta, G, Ai,
-               (const T*)DW, (const T*)DVF, DKH, (const float*)DG, (T*)dv, dbeta, dg, cu, chunk_offsets, d.T, d.N,
-               d.Hqk, d.Hv, d.V);
+    GDN_LAUNCH(kKernBwdLocal, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, (const T*)v, beta, G, Ai, VF,
+               (const T*)DVF, (const T*)DOF, HF, (const T*)DHF, DQH, DKH, (T*)dv, dbeta, dg, cu, chunk_offsets, d.T,
+               d.N, d.Hqk, d.Hv, d.V, scale);
   }
   {
     constexpr int LPR = DK / Elem<T>::kVec;
@@ -853,19 +774,21 @@ extern "C" int gdn_chunk_bwd(const void* q, const void* k, const void* v, const 
   if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
   unsigned char* ws = static_cast<unsigned char*>(workspace);
   hipStream_t st = (hipStream_t)stream;
-#define GDN_BWD(T_, DK_, NW_, NWS_, ST_, BVQ_, BVW_)                                                                   \
-  return chunk_bwd_launch<T_, DK_, NW_, NWS_, ST_, BVQ_, BVW_>(d, L, q, k, v, beta, cu_seqlens, d_o, d_final_state, dq, \
+#define GDN_BWD(T_, DK_, NW_, NWS_, ST_, BVL_)                                                              \
+  return chunk_bwd_launch<T_, DK_, NW_, NWS_, ST_, BVL_>(d, L, q, k, v, beta, cu_seqlens, d_o, d_final_state, dq, \
                                                           dk, dv, dg, dbeta, d_initial_state, ws, scale,         \
                                                           use_qk_l2norm, st)
   const bool wide = (V % 128 == 0);
   if (dtype == 1) {
-    if (K == 128 && wide) GDN_BWD(bf16_t, 128, 4, 2, 2, 64, 64);
-    if (K == 128) GDN_BWD(bf16_t, 128, 2, 2, 2, 64, 64);
-    if (wide) GDN_BWD(bf16_t, 64, 4, 2, 2, 64, 64);
-    GDN_BWD(bf16_t, 64, 2, 2, 2, 64, 64);
+    if (K == 128 && wide) GDN_BWD(bf16_t, 128, 4, 2, 2, 128);
+    if (K == 128) GDN_BWD(bf16_t, 128, 2, 2, 2, 64);
+    if (wide) GDN_BWD(bf16_t, 64, 4, 2, 2, 128);
+    GDN_BWD(bf16_t, 64, 2, 2, 2, 64);
   } else {
-    if (K == 128) GDN_BWD(float, 128, 2, 2, 1, 64, 64);
-    GDN_BWD(float, 64, 2, 2, 2, 64, 64);
+    if (K == 128 && wide) GDN_BWD(float, 128, 2, 2, 1, 128);
+    if (K == 128) GDN_BWD(float, 128, 2, 2, 1, 64);
+    if (wide) GDN_BWD(float, 64, 2, 2, 2, 128);
+    GDN_BWD(float, 64, 2, 2, 2, 64);
   }
 #undef GDN_BWD
 }

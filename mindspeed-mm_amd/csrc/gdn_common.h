@@ -78,6 +78,14 @@ template <typename T> __device__ __host__ constexpr int lds_ld(int cols) { retur
 // LDS reads of the next group, then the matrix instructions of this group) that the scheduler would otherwise
 // serialise into read -> wait -> multiply.
 #define GDN_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+// Orders the LDS traffic of one wave when its lanes hand data to each other through a wave-private LDS patch.  The
+// hardware already executes a wave's LDS instructions in order; this only stops the compiler from reordering them.
+#define GDN_WAVE_LDS_SYNC()                                           \
+  do {                                                                \
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");   \
+    __builtin_amdgcn_wave_barrier();                                  \
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");   \
+  } while (0)
 // makes a loop-invariant value opaque inside a loop so that the address arithmetic derived from it is recomputed
 // where it is used instead of being hoisted out of the loop and held in registers for its whole duration
 #define GDN_OPAQUE(x) asm volatile("" : "+r"(x))
@@ -437,6 +445,57 @@ __device__ __forceinline__ float row16_sum(float v) {
   v += dpp_mov<0x141>(v);   // row_half_mirror
   v += dpp_mov<0x140>(v);   // row_mirror
   return v;
+}
+
+// Row sums of a 32x32 tile given as per-lane products x[r] (accumulator layout).  A halving butterfly over the 16
+// lanes of a DPP row: at each step a lane keeps the pair sums of the registers whose index bit matches its own lane bit, so 16 sums cost 15 exchanges instead of 64.  Lane l returns the sum over its DPP row of
+// register r = l & 15, i.e. a partial sum (16 of the 32 columns) of tile row acc_row(l & 15).
+__device__ __forceinline__ float rows16_partial(const f32x16& x) {
+  const int lane = threadIdx.x;
+  const bool b0 = lane & 1, b1 = lane & 2, b2 = lane & 4, b3 = lane & 8;
+  // both candidate sums are formed and one is kept: a select between two register elements would be folded into a
+  // dynamically indexed element read, which the backend expands into a 16-way compare/select chain
+  float a[8], b[4], c[2];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float lo = x[2 * i] + dpp_mov<0xB1>(x[2 * i]), hi = x[2 * i + 1] + dpp_mov<0xB1>(x[2 * i + 1]);
+    a[i] = b0 ? hi : lo;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float lo = a[2 * i] + dpp_mov<0x4E>(a[2 * i]), hi = a[2 * i + 1] + dpp_mov<0x4E>(a[2 * i + 1]);
+    b[i] = b1 ? hi : lo;
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {   // row_ror:4
+    const float lo = b[2 * i] + dpp_mov<0x124>(b[2 * i]), hi = b[2 * i + 1] + dpp_mov<0x124>(b[2 * i + 1]);
+    c[i] = b2 ? hi : lo;
+  }
+  const float lo = c[0] + dpp_mov<0x128>(c[0]), hi = c[1] + dpp_mov<0x128>(c[1]);   // row_ror:8
+  return b3 ? hi : lo;
+}
+// rowacc[i0 + i] += sum_j x[i][j] for the 32 rows of the tile (rowacc in LDS; two lanes add into each entry)
+__device__ __forceinline__ void rows_add(const f32x16& x, float* rowacc, int i0) {
+  const float s = rows16_partial(x);
+  atomicAdd(&rowacc[i0 + acc_row(threadIdx.x & 15)], s);
+}
+
+// One wave: 32x32 accumulator tile -> 32 global rows of 32 columns (tile row i at g + i*row_stride), written as
+// 16-byte pieces after a pass through a wave-private LDS patch of 32 x kPatchLd elements.  Element-wise stores of
+// an accumulator tile (2 bytes per lane, 16 instructions) are several times slower than these.
+template <typename T> struct Patch { static constexpr int kLd = 32 + 16 / (int)sizeof(T), kElems = 32 * kLd; };
+template <typename T>
+__device__ __forceinline__ void acc_store_rows(const f32x16& acc, T* patch, T* g, int64_t row_stride, int rows_valid) {
+  constexpr int PLD = Patch<T>::kLd, V = Elem<T>::kVec, PPR = 32 / V;
+  const int lane = threadIdx.x & 63;
+  GDN_WAVE_LDS_SYNC();   // earlier readers of the patch are done
+  acc_to_lds(acc, patch, PLD, 0, 0);
+  GDN_WAVE_LDS_SYNC();
+#pragma unroll
+  for (int p = lane; p < 32 * PPR; p += 64) {
+    const int row = p / PPR, cc = p % PPR;
+    if (row < rows_valid) st16(g + (int64_t)row * row_stride + cc * V, ld16(patch + row * PLD + cc * V));
+  }
 }
 
 // sum over the 32 lanes that share a half-wave (all columns of one accumulator row)

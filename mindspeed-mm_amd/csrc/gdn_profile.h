@@ -6,8 +6,8 @@
 namespace gdn {
 
 enum KernelId {
-  kKernChunkTable = 0, kKernL2Norm, kKernPrep, kKernStateFwd, kKernOut, kKernBwdPrep, kKernStateBwd, kKernDqkw,
-  kKernWyBwd, kKernQkFinalize, kKernRecurrent, kKernConvFwd, kKernConvState, kKernConvBwd, kKernConvReduce,
+  kKernChunkTable = 0, kKernL2Norm, kKernPrep, kKernStateFwd, kKernOut, kKernBwdPrep, kKernStateBwd, kKernBwdLocal,
+  kKernQkFinalize, kKernRecurrent, kKernConvFwd, kKernConvState, kKernConvBwd, kKernConvReduce,
   kKernConvDh0, kKernConvUpdate, kKernCount
 };
 

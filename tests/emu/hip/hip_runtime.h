@@ -128,6 +128,9 @@ template <class T> inline T shfl(T v, int src) {
   return o;
 }
 
+// rendezvous of the lanes of one wave (lanes run as cooperative fibers: a wave-private LDS hand-over needs one)
+inline void wave_sync() { char c = 0; (void)wave_exchange(&c, 1); }
+
 void run_grid(dim3 grid, dim3 block, size_t smem, const std::function<void()>& body);
 
 // ---- MFMA (layouts as on CDNA3/4: see gdn_common.h) ----
@@ -240,6 +243,8 @@ static emu::GdimProxy gridDim;
 #define __builtin_amdgcn_s_barrier() emu::syncthreads()
 #define __builtin_amdgcn_fence(...) ((void)0)
 #define __builtin_amdgcn_sched_barrier(x) ((void)0)
+#define __builtin_amdgcn_wave_barrier() emu::wave_sync()
+#define __builtin_amdgcn_readfirstlane(x) (x)
 template <class T> inline T __shfl(T v, int src, int = 64) { return emu::shfl(v, src); }
 template <class T> inline T __shfl_xor(T v, int m, int = 64) { return emu::shfl(v, emu::lane() ^ m); }
 template <class T> inline T __shfl_up(T v, unsigned d, int = 64) {
@@ -257,6 +262,7 @@ inline int emu_update_dpp(int /*old*/, int src, int ctrl) {
   if (ctrl >= 0 && ctrl <= 0xFF) from = (l & ~3) | ((ctrl >> (2 * (l & 3))) & 3);          // quad_perm
   else if (ctrl == 0x141) from = (l & ~7) | (7 - (l & 7));                                  // row_half_mirror
   else if (ctrl == 0x140) from = (l & ~15) | (15 - (l & 15));                               // row_mirror
+  else if (ctrl > 0x120 && ctrl <= 0x12F) from = (l & ~15) | ((l - (ctrl & 15)) & 15);      // row_ror:n
   else abort();
   return emu::shfl(src, from);
 }
