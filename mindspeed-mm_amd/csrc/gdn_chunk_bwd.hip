@@ -331,29 +331,36 @@ __global__ __launch_bounds__(128 * NW) void chunk_state_bwd_kernel(
 // chunk_bwd_local_kernel, per (chunk, head), 4 waves: everything of the backward pass that is local to a chunk once
 // the reverse recurrence has left dS' and dV' behind.  Wave w owns the 32 K-columns [32w, 32w+32) of dQ, dK, dW and
 // the 32x32 tile (w/2, w%2) of the 64x64 intra-chunk matrices.
-//   main loop over 32-column V blocks (no workgroup barrier, nothing but V in LDS):
+//   main loop over 32-column V blocks:
 //     v_new, dV', dO, S, dS' arrive in fragment order with (lane <-> V column); the contractions run over V, so each
 //     tile is turned through the matrix core (mfma_transpose) into (lane <-> token / K column, registers <-> V).
 //       ds += dO V'^T   a2 += dV' V^T   dQ += dO S^T   dK += V' dS'^T   dW += dV' S^T   R = Tm^T dV' -> dv, dbeta
-//   epilogue: dQ += ds K, dK += ds^T Q, dG rows as <q,dQ> - <k,dK>; then back through W = Tm (beta e^G K) with dW
-//   still in registers: P = Tm^T dW, a1 = dW K^T, dTm = strict_tril(a1 beta e^G + a2 beta), dM = -(Tm^T dTm Tm^T).Gam,
-//   dK += beta e^G P + beta (dM K) + dM^T (beta K); dbeta, dg.  dQ, dK, dv leave as 16-byte row pieces.
+//     All operands of a V block are copied by direct global->LDS loads (no registers in between, fragment order is
+//     exactly the layout such a load produces) into one of two stages, one block ahead of the arithmetic: tiles
+//     shared by the four waves once per workgroup, S and dS' per wave.
+//   epilogue (its LDS tiles reuse the two stages): dQ += ds K, dK += ds^T Q, dG rows as <q,dQ> - <k,dK>; then back
+//   through W = Tm (beta e^G K) with dW still in registers: P = Tm^T dW, a1 = dW K^T,
+//   dTm = strict_tril(a1 beta e^G + a2 beta), dM = -(Tm^T dTm Tm^T).Gam, dK += beta e^G P + beta (dM K) + dM^T (beta K);
+//   dbeta, dg.  dQ, dK, dv leave as 16-byte row pieces.
 // ---------------------------------------------------------------------------------------------
-template <typename T, int DK, int BV> struct BwdLocalSmem {
-  static constexpr int LDK = lds_ld<T>(DK), LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
-  static constexpr int vw_elems = 64 * (LDV > LDK ? LDV : LDK);
+template <typename T, int DK> struct BwdLocalSmem {
+  static constexpr int LDK = lds_ld<T>(DK), L64 = lds_ld<T>(64);
+  // one stage, in elements: [v_new x2 | dV' x2 | dO x2] shared tiles, [S | dS'] per wave, raw V [64][32]
+  static constexpr int st_priv = 6 * 1024, st_vraw = st_priv + 4 * 2048, stage_elems = st_vraw + 64 * 32;
+  // epilogue tiles inside the stage area
   static constexpr int off_ks = 0;                                            // K     [64][LDK]
-  static constexpr int off_tmt = off_ks + 64 * LDK * (int)sizeof(T);          // Tm^T  [64][kLT]
-  static constexpr int off_tm = off_tmt + 64 * kLT * (int)sizeof(T);          // Tm    [64][L64], later (beta . dM)^T
-  static constexpr int off_vw = off_tm + 64 * L64 * (int)sizeof(T);           // V [64][LDV]; later dW [64][LDK]; later store patches
-  static constexpr int off_ds = off_vw + vw_elems * (int)sizeof(T);           // store patches; ds | ds^T; dTm, dM | X^T
-  static constexpr int off_row = off_ds + 2 * 64 * L64 * (int)sizeof(T);
+  static constexpr int off_tm = off_ks + 64 * LDK * (int)sizeof(T);           // Tm    [64][L64], later (beta . dM)^T
+  static constexpr int off_dw = off_tm + 64 * L64 * (int)sizeof(T);           // dW    [64][LDK], later store patches
+  static constexpr int off_ds = off_dw + 64 * LDK * (int)sizeof(T);           // ds | ds^T; dTm, dM | X^T
+  static constexpr int epi_bytes = off_ds + 2 * 64 * L64 * (int)sizeof(T);
+  static constexpr int off_tmt = 2 * stage_elems * (int)sizeof(T);            // Tm^T  [64][kLT]  (whole kernel)
+  static constexpr int off_row = off_tmt + 64 * kLT * (int)sizeof(T);
   static constexpr int bytes = off_row + (6 * 64 + 8) * 4;
-  // store patches: one per wave in the main loop (dv), one per wave that owns K columns afterwards (dq, dk)
-  static_assert(4 * Patch<T>::kElems <= 2 * 64 * L64 && (DK / 32) * Patch<T>::kElems <= vw_elems, "store patches fit");
+  static_assert(epi_bytes <= off_tmt, "epilogue tiles fit in the two stages");
+  static_assert(Patch<T>::kElems <= 2048 && (DK / 32) * Patch<T>::kElems <= 64 * LDK, "store patches fit");
 };
 
-template <typename T, int DK, int BV>
+template <typename T, int DK>
 __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_local_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ beta,
     const float* __restrict__ G, const T* __restrict__ Ai, const T* __restrict__ vf, const T* __restrict__ dvf,
@@ -361,15 +368,16 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     T* __restrict__ dkh, T* __restrict__ dv_out, float* __restrict__ dbeta, float* __restrict__ dg,
     const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V,
     float scale) {
-  using SM = BwdLocalSmem<T, DK, BV>;
-  constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64, NKT = DK / 32;
+  using SM = BwdLocalSmem<T, DK>;
+  constexpr int LDK = SM::LDK, L64 = SM::L64, NKT = DK / 32, VEC = Elem<T>::kVec, KG = AccK<T>::kGroups;
   static_assert(NKT <= 4, "one 32-column block of K per wave");
+  T* stage0 = reinterpret_cast<T*>(gdn_smem);
   T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
-  T* TmT = reinterpret_cast<T*>(gdn_smem + SM::off_tmt);
   T* Tm = reinterpret_cast<T*>(gdn_smem + SM::off_tm);
-  T* Vs = reinterpret_cast<T*>(gdn_smem + SM::off_vw);
+  T* dWs = reinterpret_cast<T*>(gdn_smem + SM::off_dw);
   T* dsm = reinterpret_cast<T*>(gdn_smem + SM::off_ds);
   T* dsT = dsm + 64 * L64;
+  T* TmT = reinterpret_cast<T*>(gdn_smem + SM::off_tmt);
   float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_row);
   float* egs = Gs + 64;    // e^G
   float* bs = egs + 64;    // beta
@@ -377,7 +385,6 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   float* rb = r1 + 64;     // dbeta
   float* rg = rb + 64;     // dG through W, U
   float* wsum = rg + 64;   // per wave: <S,dS'> [0..3], sum_i <k_i, dK_inter_i> [4..7]
-  T* dWs = Vs;
   T* dAs = dsm;
   T* XT = dsT;
   T* dMs = dsm;
@@ -392,6 +399,35 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   const int64_t ch = (int64_t)blockIdx.x * Hv + h;
   const int ti = wave >> 1, tj = wave & 1, cj = wave;
   const bool lower = tj <= ti, has_k = wave < NKT;
+  const int nblk = V / 32;
+
+  // stage `buf` <- operands of V block `vblk`; every load moves 64 x 16 bytes, lane l's piece landing at +16 l
+  auto issue = [&](int vblk, int buf) {
+    T* st = stage0 + buf * SM::stage_elems;
+    const int64_t t2 = (ch * nblk + vblk) * 2, tk = (ch * nblk + vblk) * NKT;
+#pragma unroll
+    for (int j = 0; j < 6 * KG / 4; ++j) {           // shared tiles: k-group pieces dealt round-robin to the waves
+      const int piece = 4 * j + wave, tile = piece / KG, g = piece % KG;
+      const T* src = tile < 2 ? vf + (t2 + tile) * 1024 : tile < 4 ? dvf + (t2 + tile - 2) * 1024 : dof + (t2 + tile - 4) * 1024;
+      load16_to_lds(src + (g * 64 + lane) * VEC, st + tile * 1024 + g * 64 * VEC);
+    }
+#pragma unroll
+    for (int j = 0; j < (int)sizeof(T) / 2; ++j) {   // raw V block [64][32], rows past the end repeat the last row
+      constexpr int LPR = 32 / VEC, RPP = 64 / LPR;  // lanes per row, rows per piece
+      const int piece = 4 * j + wave, row = piece * RPP + lane / LPR, cc = lane % LPR;
+      load16_to_lds(v + ((tok0 + imin(row, nvalid - 1)) * Hv + h) * V + 32 * vblk + cc * VEC,
+                    st + SM::st_vraw + piece * 64 * VEC);
+    }
+    if (has_k) {
+#pragma unroll
+      for (int g = 0; g < KG; ++g) {
+        load16_to_lds(hf + (tk + cj) * 1024 + (g * 64 + lane) * VEC, st + SM::st_priv + wave * 2048 + g * 64 * VEC);
+        load16_to_lds(dhf + (tk + cj) * 1024 + (g * 64 + lane) * VEC,
+                      st + SM::st_priv + wave * 2048 + 1024 + g * 64 * VEC);
+      }
+    }
+  };
+  issue(0, 0);
 
   if (tid < 64) {
     const float gv = G[(tok0 + imin(tid, nvalid - 1)) * Hv + h];
@@ -400,9 +436,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     bs[tid] = tid < nvalid ? beta[(tok0 + tid) * Hv + h] : 0.f;
     r1[tid] = 0.f; rb[tid] = 0.f; rg[tid] = 0.f;
   }
-  load_tile<T, 64>(Tm, L64, Ai + (tok0 * Hv + h) * 64, (int64_t)Hv * 64, nvalid, tid);
   load_tile_t<T, 64, kThreads>(TmT, kLT, Ai + (tok0 * Hv + h) * 64, (int64_t)Hv * 64, nvalid, tid);
-  load_tile<T, DK>(Ks, LDK, k + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
 
   IdentityFrag<T> id;
   id.init();
@@ -411,77 +445,79 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   for (int ri = 0; ri < 2; ++ri) { dQi[ri] = acc_zero(); dKi[ri] = acc_zero(); dWa[ri] = acc_zero(); }
   float sds = 0.f;
 
-  for (int vb = 0; vb < V / BV; ++vb) {
-    if (vb > 0) __syncthreads();
-    load_tile<T, BV>(Vs, LDV, v + (tok0 * Hv + h) * V + vb * BV, (int64_t)Hv * V, nvalid, tid);
-    __syncthreads();
+  for (int vblk = 0; vblk < nblk; ++vblk) {
+    const T* st = stage0 + (vblk & 1) * SM::stage_elems;
+    GDN_WAIT_VMEM();       // this wave's share of the stage has landed ...
+    GDN_LDS_BARRIER();     // ... and so has everybody else's; the other stage is no longer read
+    if (vblk + 1 < nblk) issue(vblk + 1, (vblk + 1) & 1);
+    // Operands are taken one after the other so that few fragments are live at a time; tile indices that depend on
+    // the wave are compared against loop constants (fragments indexed at run time would go to scratch).
+    AccB<T> f, Sf, dSf, dOt[2];
+    if (has_k) {                             // (lane <-> K column, registers <-> V)
+      f.load(st + SM::st_priv + wave * 2048);
+      const f32x16 sv = mfma_transpose<T>(f, id);
+      Sf.pack(sv);
+      f.load(st + SM::st_priv + wave * 2048 + 1024);
+      const f32x16 dsv = mfma_transpose<T>(f, id);
+      dSf.pack(dsv);
 #pragma unroll
-    for (int v32 = 0; v32 < BV / 32; ++v32) {
-      const int vblk = vb * (BV / 32) + v32;
-      const int64_t t2 = (ch * (V / 32) + vblk) * 2, tk = (ch * (V / 32) + vblk) * NKT;
-      // Operands are brought in one after the other so that few fragments are live at a time; tile indices that
-      // depend on the wave are compared against loop constants (fragments indexed at run time would go to scratch).
-      AccB<T> f, Sf, dSf, dOt[2];
-      if (has_k) {                           // (lane <-> K column, registers <-> V)
-        f.load(hf + (tk + cj) * 1024);
-        const f32x16 st = mfma_transpose<T>(f, id);
-        Sf.pack(st);
-        f.load(dhf + (tk + cj) * 1024);
-        const f32x16 dst = mfma_transpose<T>(f, id);
-        dSf.pack(dst);
+      for (int r = 0; r < 16; ++r) sds += sv[r] * dsv[r];
+    }
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sds += st[r] * dst[r];
+    for (int ri = 0; ri < 2; ++ri) {         // (lane <-> token, registers <-> V) from here on
+      f.load(st + (4 + ri) * 1024);
+      dOt[ri].pack(mfma_transpose<T>(f, id));
+      if (has_k) mma32_ff<T>(dQi[ri], dOt[ri], Sf);
+    }
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri) {
+      AccB<T> Vt;
+      f.load(st + ri * 1024);
+      Vt.pack(mfma_transpose<T>(f, id));
+      if (has_k) mma32_ff<T>(dKi[ri], Vt, dSf);
+      if (lower && ri == tj) {
+        if (ti == 0) mma32_ff<T>(ds, dOt[0], Vt); else mma32_ff<T>(ds, dOt[1], Vt);
       }
+    }
 #pragma unroll
-      for (int ri = 0; ri < 2; ++ri) {       // (lane <-> token, registers <-> V) from here on
-        f.load(dof + (t2 + ri) * 1024);
-        dOt[ri].pack(mfma_transpose<T>(f, id));
-        if (has_k) mma32_ff<T>(dQi[ri], dOt[ri], Sf);
+    for (int ri = 0; ri < 2; ++ri) {
+      AccB<T> dVt;
+      f.load(st + (2 + ri) * 1024);
+      dVt.pack(mfma_transpose<T>(f, id));
+      if (has_k) mma32_ff<T>(dWa[ri], dVt, Sf);
+      if (lower && ri == ti) {
+        frags_from_lds<T>(f, st + SM::st_vraw + (32 * tj + l32) * 32);
+        mma32_ff<T>(a2, dVt, f);
       }
+    }
+    if ((vblk & 3) == wave) {                // R = Tm^T dV' for this V block: dv = beta R, dbeta += <R, v>
+      AccB<T> fdv[2];
+      fdv[0].load(st + 2 * 1024);
+      fdv[1].load(st + 3 * 1024);
+      // the wave's S / dS' slots of this stage are consumed: they serve as the store patch
+      T* patch = stage0 + (vblk & 1) * SM::stage_elems + SM::st_priv + wave * 2048;
 #pragma unroll
-      for (int ri = 0; ri < 2; ++ri) {
-        AccB<T> Vt;
-        f.load(vf + (t2 + ri) * 1024);
-        Vt.pack(mfma_transpose<T>(f, id));
-        if (has_k) mma32_ff<T>(dKi[ri], Vt, dSf);
-        if (lower && ri == tj) {
-          if (ti == 0) mma32_ff<T>(ds, dOt[0], Vt); else mma32_ff<T>(ds, dOt[1], Vt);
-        }
-      }
+      for (int rj = 0; rj < 2; ++rj) {
+        f32x16 R = acc_zero(), p;
 #pragma unroll
-      for (int ri = 0; ri < 2; ++ri) {
-        AccB<T> dVt;
-        f.load(dvf + (t2 + ri) * 1024);
-        dVt.pack(mfma_transpose<T>(f, id));
-        if (has_k) mma32_ff<T>(dWa[ri], dVt, Sf);
-        if (lower && ri == ti) {
-          frags_from_lds<T>(f, Vs + (32 * tj + l32) * LDV + 32 * v32);
-          mma32_ff<T>(a2, dVt, f);
-        }
-      }
-      if ((vblk & 3) == wave) {              // R = Tm^T dV' for this V block: dv = beta R, dbeta += <R, v>
-        AccB<T> fdv[2];
-        fdv[0].load(dvf + (t2 + 0) * 1024);
-        fdv[1].load(dvf + (t2 + 1) * 1024);
+        for (int t = rj; t < 2; ++t) mma32_accb<T>(R, TmT + (32 * rj + l32) * kLT + 32 * t, fdv[t]);
 #pragma unroll
-        for (int rj = 0; rj < 2; ++rj) {
-          f32x16 R = acc_zero(), p;
+        for (int r = 0; r < 16; ++r)
+          p[r] = R[r] * Elem<T>::to_f(st[SM::st_vraw + (32 * rj + acc_row(r)) * 32 + acc_col()]);
+        rows_add(p, rb, 32 * rj);
 #pragma unroll
-          for (int t = rj; t < 2; ++t) mma32_accb<T>(R, TmT + (32 * rj + l32) * kLT + 32 * t, fdv[t]);
-#pragma unroll
-          for (int r = 0; r < 16; ++r)
-            p[r] = R[r] * Elem<T>::to_f(Vs[(32 * rj + acc_row(r)) * LDV + 32 * v32 + acc_col()]);
-          rows_add(p, rb, 32 * rj);
-#pragma unroll
-          for (int r = 0; r < 16; ++r) R[r] *= bs[32 * rj + acc_row(r)];
-          acc_store_rows<T>(R, dsm + wave * Patch<T>::kElems, dv_out + ((tok0 + 32 * rj) * Hv + h) * V + 32 * vblk,
-                            (int64_t)Hv * V, nvalid - 32 * rj);
-        }
+        for (int r = 0; r < 16; ++r) R[r] *= bs[32 * rj + acc_row(r)];
+        acc_store_rows<T>(R, patch, dv_out + ((tok0 + 32 * rj) * Hv + h) * V + 32 * vblk, (int64_t)Hv * V,
+                          nvalid - 32 * rj);
       }
     }
   }
   sds = wave_sum(sds);
   if (lane == 0) wsum[wave] = sds;
+  __syncthreads();   // the stages are consumed: their space now takes the epilogue tiles
+  load_tile<T, 64>(Tm, L64, Ai + (tok0 * Hv + h) * 64, (int64_t)Hv * 64, nvalid, tid);
+  load_tile<T, DK>(Ks, LDK, k + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
+  __syncthreads();
 
   // this wave's K and Q columns as (lane <-> column, registers <-> token): B operands and row-dot partners
   AccB<T> KTf[2], QTf[2];
@@ -500,7 +536,6 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       QTf[t].pack(mfma_transpose<T>(f, id));
     }
   }
-  __syncthreads();   // every wave is done with the V tile and the main-loop store patches
   {
     const int j = 32 * tj + acc_col();
 #pragma unroll
@@ -698,7 +733,7 @@ template <typename K> static int set_lds_b(K kernel, int bytes) {
                                   bytes);
 }
 
-template <typename T, int DK, int NW, int NWS, int STAGES, int BVL>
+template <typename T, int DK, int NW, int NWS, int STAGES>
 static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const void* q, const void* k, const void* v,
                             const float* beta, const int64_t* cu, const void* dO, const float* dht, void* dq, void* dk,
                             void* dv, float* dg, float* dbeta, float* dh0, unsigned char* ws, float scale, int l2norm,
@@ -738,8 +773,8 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
                d.V);
   }
   {
-    auto kern = chunk_bwd_local_kernel<T, DK, BVL>;
-    constexpr int smem = BwdLocalSmem<T, DK, BVL>::bytes;
+    auto kern = chunk_bwd_local_kernel<T, DK>;
+    constexpr int smem = BwdLocalSmem<T, DK>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
     GDN_LAUNCH(kKernBwdLocal, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, (const T*)v, beta, G, Ai, VF,
                (const T*)DVF, (const T*)DOF, HF, (const T*)DHF, DQH, DKH, (T*)dv, dbeta, dg, cu, chunk_offsets, d.T,
@@ -774,21 +809,19 @@ extern "C" int gdn_chunk_bwd(const void* q, const void* k, const void* v, const 
   if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
   unsigned char* ws = static_cast<unsigned char*>(workspace);
   hipStream_t st = (hipStream_t)stream;
-#define GDN_BWD(T_, DK_, NW_, NWS_, ST_, BVL_)                                                              \
-  return chunk_bwd_launch<T_, DK_, NW_, NWS_, ST_, BVL_>(d, L, q, k, v, beta, cu_seqlens, d_o, d_final_state, dq, \
+#define GDN_BWD(T_, DK_, NW_, NWS_, ST_)                                                       \
+  return chunk_bwd_launch<T_, DK_, NW_, NWS_, ST_>(d, L, q, k, v, beta, cu_seqlens, d_o, d_final_state, dq, \
                                                           dk, dv, dg, dbeta, d_initial_state, ws, scale,         \
                                                           use_qk_l2norm, st)
   const bool wide = (V % 128 == 0);
   if (dtype == 1) {
-    if (K == 128 && wide) GDN_BWD(bf16_t, 128, 4, 2, 2, 128);
-    if (K == 128) GDN_BWD(bf16_t, 128, 2, 2, 2, 64);
-    if (wide) GDN_BWD(bf16_t, 64, 4, 2, 2, 128);
-    GDN_BWD(bf16_t, 64, 2, 2, 2, 64);
+    if (K == 128 && wide) GDN_BWD(bf16_t, 128, 4, 2, 2);
+    if (K == 128) GDN_BWD(bf16_t, 128, 2, 2, 2);
+    if (wide) GDN_BWD(bf16_t, 64, 4, 2, 2);
+    GDN_BWD(bf16_t, 64, 2, 2, 2);
   } else {
-    if (K == 128 && wide) GDN_BWD(float, 128, 2, 2, 1, 128);
-    if (K == 128) GDN_BWD(float, 128, 2, 2, 1, 64);
-    if (wide) GDN_BWD(float, 64, 2, 2, 2, 128);
-    GDN_BWD(float, 64, 2, 2, 2, 64);
+    if (K == 128) GDN_BWD(float, 128, 2, 2, 1);
+    GDN_BWD(float, 64, 2, 2, 2);
   }
 #undef GDN_BWD
 }

@@ -86,6 +86,15 @@ template <typename T> __device__ __host__ constexpr int lds_ld(int cols) { retur
     __builtin_amdgcn_wave_barrier();                                  \
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");   \
   } while (0)
+// Asynchronous copy global -> LDS that bypasses the registers: each of the 64 lanes of a wave moves 16 bytes from its
+// own address `src`, and lane l's piece lands at lds_wave_base + 16 l (lds_wave_base must be wave-uniform).  A tile
+// in fragment order ([k-group][lane][16 bytes]) is therefore copied verbatim by one such load per k-group.
+// Completion is counted with the vector-memory loads: GDN_WAIT_VMEM() and then a barrier publish the data.
+#define GDN_WAIT_VMEM() __builtin_amdgcn_s_waitcnt(0x0F70)   // vmcnt(0); expcnt and lgkmcnt left alone
+template <typename T> __device__ __forceinline__ void load16_to_lds(const T* src, T* lds_wave_base) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                   (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+}
 // makes a loop-invariant value opaque inside a loop so that the address arithmetic derived from it is recomputed
 // where it is used instead of being hoisted out of the loop and held in registers for its whole duration
 #define GDN_OPAQUE(x) asm volatile("" : "+r"(x))

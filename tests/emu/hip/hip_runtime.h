@@ -245,6 +245,10 @@ static emu::GdimProxy gridDim;
 #define __builtin_amdgcn_sched_barrier(x) ((void)0)
 #define __builtin_amdgcn_wave_barrier() emu::wave_sync()
 #define __builtin_amdgcn_readfirstlane(x) (x)
+#define __builtin_amdgcn_s_waitcnt(x) ((void)0)
+// direct global -> LDS load: lane l's `size` bytes land at dst + l*size (done at once: the emulator has no asynchrony)
+#define __builtin_amdgcn_global_load_lds(src, dst, size, off, aux) \
+  memcpy((unsigned char*)(uintptr_t)(dst) + (off) + emu::lane() * (size), (const void*)(uintptr_t)(src), (size))
 template <class T> inline T __shfl(T v, int src, int = 64) { return emu::shfl(v, src); }
 template <class T> inline T __shfl_xor(T v, int m, int = 64) { return emu::shfl(v, emu::lane() ^ m); }
 template <class T> inline T __shfl_up(T v, unsigned d, int = 64) {
