@@ -438,6 +438,32 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   }
   load_tile_t<T, 64, kThreads>(TmT, kLT, Ai + (tok0 * Hv + h) * 64, (int64_t)Hv * 64, nvalid, tid);
 
+  __syncthreads();
+  // R = Tm^T dV' per 32-column V block (blocks dealt to the waves): dv = beta R, dbeta += <R, v>.  Done before the
+  // accumulators of the main loop exist; the store patch is this wave's S / dS' slot of the stage not yet in use.
+  for (int vblk = wave; vblk < nblk; vblk += 4) {
+    AccB<T> fdv[2];
+    fdv[0].load(dvf + ((ch * nblk + vblk) * 2 + 0) * 1024);
+    fdv[1].load(dvf + ((ch * nblk + vblk) * 2 + 1) * 1024);
+    T* patch = stage0 + SM::stage_elems + SM::st_priv + wave * 2048;
+#pragma unroll
+    for (int rj = 0; rj < 2; ++rj) {
+      f32x16 R = acc_zero(), p;
+#pragma unroll
+      for (int t = rj; t < 2; ++t) mma32_accb<T>(R, TmT + (32 * rj + l32) * kLT + 32 * t, fdv[t]);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = imin(32 * rj + acc_row(r), nvalid - 1);
+        p[r] = R[r] * Elem<T>::to_f(v[((tok0 + row) * Hv + h) * V + 32 * vblk + acc_col()]);
+      }
+      rows_add(p, rb, 32 * rj);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) R[r] *= bs[32 * rj + acc_row(r)];
+      acc_store_rows<T>(R, patch, dv_out + ((tok0 + 32 * rj) * Hv + h) * V + 32 * vblk, (int64_t)Hv * V,
+                        nvalid - 32 * rj);
+    }
+  }
+
   IdentityFrag<T> id;
   id.init();
   f32x16 ds = acc_zero(), a2 = acc_zero(), dQi[2], dKi[2], dWa[2];
@@ -490,34 +516,13 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
         mma32_ff<T>(a2, dVt, f);
       }
     }
-    if ((vblk & 3) == wave) {                // R = Tm^T dV' for this V block: dv = beta R, dbeta += <R, v>
-      AccB<T> fdv[2];
-      fdv[0].load(st + 2 * 1024);
-      fdv[1].load(st + 3 * 1024);
-      // the wave's S / dS' slots of this stage are consumed: they serve as the store patch
-      T* patch = stage0 + (vblk & 1) * SM::stage_elems + SM::st_priv + wave * 2048;
-#pragma unroll
-      for (int rj = 0; rj < 2; ++rj) {
-        f32x16 R = acc_zero(), p;
-#pragma unroll
-        for (int t = rj; t < 2; ++t) mma32_accb<T>(R, TmT + (32 * rj + l32) * kLT + 32 * t, fdv[t]);
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-          p[r] = R[r] * Elem<T>::to_f(st[SM::st_vraw + (32 * rj + acc_row(r)) * 32 + acc_col()]);
-        rows_add(p, rb, 32 * rj);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) R[r] *= bs[32 * rj + acc_row(r)];
-        acc_store_rows<T>(R, patch, dv_out + ((tok0 + 32 * rj) * Hv + h) * V + 32 * vblk, (int64_t)Hv * V,
-                          nvalid - 32 * rj);
-      }
-    }
   }
   sds = wave_sum(sds);
   if (lane == 0) wsum[wave] = sds;
-  __syncthreads();   // the stages are consumed: their space now takes the epilogue tiles
+  GDN_LDS_BARRIER();   // the stages are consumed: their space now takes the epilogue tiles
   load_tile<T, 64>(Tm, L64, Ai + (tok0 * Hv + h) * 64, (int64_t)Hv * 64, nvalid, tid);
   load_tile<T, DK>(Ks, LDK, k + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
-  __syncthreads();
+  GDN_LDS_BARRIER();
 
   // this wave's K and Q columns as (lane <-> column, registers <-> token): B operands and row-dot partners
   AccB<T> KTf[2], QTf[2];
@@ -556,7 +561,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       dWb[ri].pack(dWa[ri]);
     }
   }
-  __syncthreads();
+  GDN_LDS_BARRIER();
   const float glast = Gs[63];
   float ski = 0.f;
   if (has_k) {
@@ -600,7 +605,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       rows_add(p, rg, 32 * rj);
     }
   }
-  __syncthreads();   // ds, ds^T and the dW tile are consumed
+  GDN_LDS_BARRIER();   // ds, ds^T and the dW tile are consumed
   {  // dTm[i][j] = beta_j (e^{G_j} a1 + a2), i > j
     const int j = 32 * tj + acc_col();
 #pragma unroll
@@ -616,13 +621,13 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       acc_store_rows<T>(dQi[ri], patch, dqh + ((tok0 + 32 * ri) * Hv + h) * DK + 32 * cj, (int64_t)Hv * DK,
                         nvalid - 32 * ri);
   }
-  __syncthreads();
+  GDN_LDS_BARRIER();
   {  // X = dTm Tm^T, stored transposed
     f32x16 x = acc_zero();
     mma32<T, 64, true, true>(x, dAs + 32 * ti * L64, L64, Tm + 32 * tj * L64, L64);
     acc_to_lds_t(x, XT, L64, 32 * ti, 32 * tj);
   }
-  __syncthreads();
+  GDN_LDS_BARRIER();
   {  // dM = -(Tm^T X) . Gam, strictly lower;  dMs[i][j] = dM,  dMTb[j][i] = beta_i dM
     f32x16 y = acc_zero();
     mma32_ss<T, 64>(y, TmT + (32 * ti + l32) * kLT, XT + (32 * tj + l32) * L64);
@@ -635,7 +640,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       dMTb[j * L64 + i] = Elem<T>::from_f(val * bs[i]);
     }
   }
-  __syncthreads();
+  GDN_LDS_BARRIER();
   if (has_k) {       // E = dM K, F = dM^T (beta K): dK += beta E + F; dbeta += <E,k>; dG += beta <E,k> - <F,k>
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {
@@ -659,7 +664,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
                         nvalid - 32 * ri);
     }
   }
-  __syncthreads();
+  GDN_LDS_BARRIER();
   if (wave == 0) {   // d(cumulative G) -> d(g): suffix sum inside the chunk
     float x = rg[lane] + r1[lane];
     if (lane == nvalid - 1)
