@@ -438,6 +438,8 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   }
   load_tile_t<T, 64, kThreads>(TmT, kLT, Ai + (tok0 * Hv + h) * 64, (int64_t)Hv * 64, nvalid, tid);
 
+  IdentityFrag<T> id;
+  id.init();
   __syncthreads();
   // R = Tm^T dV' per 32-column V block (blocks dealt to the waves): dv = beta R, dbeta += <R, v>.  Done before the
   // accumulators of the main loop exist; the store patch is this wave's S / dS' slot of the stage not yet in use.
@@ -457,15 +459,14 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
         p[r] = R[r] * Elem<T>::to_f(v[((tok0 + row) * Hv + h) * V + 32 * vblk + acc_col()]);
       }
       rows_add(p, rb, 32 * rj);
+      const f32x16 bsr = rows_ld(bs, 32 * rj);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) R[r] *= bs[32 * rj + acc_row(r)];
-      acc_store_rows<T>(R, patch, dv_out + ((tok0 + 32 * rj) * Hv + h) * V + 32 * vblk, (int64_t)Hv * V,
+      for (int r = 0; r < 16; ++r) R[r] *= bsr[r];
+      acc_store_rows<T>(R, id, patch, dv_out + ((tok0 + 32 * rj) * Hv + h) * V + 32 * vblk, (int64_t)Hv * V,
                         nvalid - 32 * rj);
     }
   }
 
-  IdentityFrag<T> id;
-  id.init();
   f32x16 ds = acc_zero(), a2 = acc_zero(), dQi[2], dKi[2], dWa[2];
 #pragma unroll
   for (int ri = 0; ri < 2; ++ri) { dQi[ri] = acc_zero(); dKi[ri] = acc_zero(); dWa[ri] = acc_zero(); }
@@ -543,13 +544,12 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   }
   {
     const int j = 32 * tj + acc_col();
+    const float gj = Gs[j];
+    const f32x16 gi = rows_ld(Gs, 32 * ti);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int i = 32 * ti + acc_row(r);
-      const float val = (i >= j) ? scale * ds[r] * __expf(Gs[i] - Gs[j]) : 0.f;
-      dsm[i * L64 + j] = Elem<T>::from_f(val);
-      dsT[j * L64 + i] = Elem<T>::from_f(val);
-    }
+    for (int r = 0; r < 16; ++r) ds[r] = (32 * ti + acc_row(r) >= j) ? scale * ds[r] * __expf(gi[r] - gj) : 0.f;
+    acc_to_lds_rm(ds, id, dsm, L64, 32 * ti, 32 * tj);
+    acc_to_lds_t(ds, dsT, L64, 32 * ti, 32 * tj);
   }
   AccB<T> dWb[2];
   if (has_k) {
@@ -557,7 +557,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     for (int ri = 0; ri < 2; ++ri) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) dWa[ri][r] = -dWa[ri][r];
-      acc_to_lds(dWa[ri], dWs, LDK, 32 * ri, 32 * cj);
+      acc_to_lds_rm(dWa[ri], id, dWs, LDK, 32 * ri, 32 * cj);
       dWb[ri].pack(dWa[ri]);
     }
   }
@@ -568,11 +568,11 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {
       const f32x16 kk = KTf[ri].unpack(), qq = QTf[ri].unpack();
+      const f32x16 gi = rows_ld(Gs, 32 * ri);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float gi = Gs[32 * ri + acc_row(r)];
-        dQi[ri][r] *= scale * __expf(gi);
-        dKi[ri][r] *= __expf(glast - gi);
+        dQi[ri][r] *= scale * __expf(gi[r]);
+        dKi[ri][r] *= __expf(glast - gi[r]);
         ski += dKi[ri][r] * kk[r];           // still only the inter-chunk part
       }
 #pragma unroll
@@ -596,29 +596,28 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       f32x16 P = acc_zero(), p;
 #pragma unroll
       for (int t = rj; t < 2; ++t) mma32_accb<T>(P, TmT + (32 * rj + l32) * kLT + 32 * t, dWb[t]);
-      const f32x16 kk = KTf[rj].unpack();
+      const f32x16 kk = KTf[rj].unpack(), er = rows_ld(egs, 32 * rj), br = rows_ld(bs, 32 * rj);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) { P[r] *= egs[32 * rj + acc_row(r)]; p[r] = P[r] * kk[r]; }
+      for (int r = 0; r < 16; ++r) { P[r] *= er[r]; p[r] = P[r] * kk[r]; }
       rows_add(p, rb, 32 * rj);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) { P[r] *= bs[32 * rj + acc_row(r)]; p[r] = P[r] * kk[r]; dKi[rj][r] += P[r]; }
+      for (int r = 0; r < 16; ++r) { P[r] *= br[r]; p[r] = P[r] * kk[r]; dKi[rj][r] += P[r]; }
       rows_add(p, rg, 32 * rj);
     }
   }
   GDN_LDS_BARRIER();   // ds, ds^T and the dW tile are consumed
   {  // dTm[i][j] = beta_j (e^{G_j} a1 + a2), i > j
     const int j = 32 * tj + acc_col();
+    const float bj = bs[j], ej = egs[j];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int i = 32 * ti + acc_row(r);
-      dAs[i * L64 + j] = Elem<T>::from_f(i > j ? bs[j] * (egs[j] * a1[r] + a2[r]) : 0.f);
-    }
+    for (int r = 0; r < 16; ++r) a1[r] = (32 * ti + acc_row(r) > j) ? bj * (ej * a1[r] + a2[r]) : 0.f;
+    acc_to_lds_rm(a1, id, dAs, L64, 32 * ti, 32 * tj);
   }
   T* patch = dWs + wave * Patch<T>::kElems;
   if (has_k) {
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri)
-      acc_store_rows<T>(dQi[ri], patch, dqh + ((tok0 + 32 * ri) * Hv + h) * DK + 32 * cj, (int64_t)Hv * DK,
+      acc_store_rows<T>(dQi[ri], id, patch, dqh + ((tok0 + 32 * ri) * Hv + h) * DK + 32 * cj, (int64_t)Hv * DK,
                         nvalid - 32 * ri);
   }
   GDN_LDS_BARRIER();
@@ -632,13 +631,16 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     f32x16 y = acc_zero();
     mma32_ss<T, 64>(y, TmT + (32 * ti + l32) * kLT, XT + (32 * tj + l32) * L64);
     const int j = 32 * tj + acc_col();
+    const float gj = Gs[j];
+    const f32x16 gi = rows_ld(Gs, 32 * ti), br = rows_ld(bs, 32 * ti);
+    f32x16 yb;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const int i = 32 * ti + acc_row(r);
-      const float val = i > j ? -y[r] * __expf(Gs[i] - Gs[j]) : 0.f;
-      dMs[i * L64 + j] = Elem<T>::from_f(val);
-      dMTb[j * L64 + i] = Elem<T>::from_f(val * bs[i]);
+      y[r] = (32 * ti + acc_row(r) > j) ? -y[r] * __expf(gi[r] - gj) : 0.f;
+      yb[r] = y[r] * br[r];
     }
+    acc_to_lds_rm(y, id, dMs, L64, 32 * ti, 32 * tj);
+    acc_to_lds_t(yb, dMTb, L64, 32 * ti, 32 * tj);
   }
   GDN_LDS_BARRIER();
   if (has_k) {       // E = dM K, F = dM^T (beta K): dK += beta E + F; dbeta += <E,k>; dG += beta <E,k> - <F,k>
@@ -653,14 +655,15 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
 #pragma unroll
       for (int r = 0; r < 16; ++r) p[r] = E[r] * kk[r];
       rows_add(p, rb, 32 * ri);
+      const f32x16 br = rows_ld(bs, 32 * ri);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        E[r] *= bs[32 * ri + acc_row(r)];
+        E[r] *= br[r];
         p[r] = (E[r] - Fm[r]) * kk[r];
         dKi[ri][r] += E[r] + Fm[r];
       }
       rows_add(p, rg, 32 * ri);
-      acc_store_rows<T>(dKi[ri], patch, dkh + ((tok0 + 32 * ri) * Hv + h) * DK + 32 * cj, (int64_t)Hv * DK,
+      acc_store_rows<T>(dKi[ri], id, patch, dkh + ((tok0 + 32 * ri) * Hv + h) * DK + 32 * cj, (int64_t)Hv * DK,
                         nvalid - 32 * ri);
     }
   }

@@ -414,11 +414,38 @@ template <typename T> __device__ __forceinline__ void acc_to_lds(const f32x16& a
 #pragma unroll
   for (int r = 0; r < 16; ++r) dst[(i0 + acc_row(r)) * ld + j] = Elem<T>::from_f(acc[r]);
 }
-// accumulator tile -> LDS, transposed: dst[(j0+j)*ld + i0 + i]
+// accumulator tile -> LDS, transposed: dst[(j0+j)*ld + i0 + i].  Registers 4g..4g+3 are four consecutive rows, so a
+// lane writes four contiguous elements at a time (ld must be a multiple of 4 elements).
 template <typename T> __device__ __forceinline__ void acc_to_lds_t(const f32x16& acc, T* dst, int ld, int i0, int j0) {
-  const int j = j0 + acc_col();
+  T* col = dst + (j0 + acc_col()) * ld + i0 + 4 * ((threadIdx.x & 63) >> 5);
 #pragma unroll
-  for (int r = 0; r < 16; ++r) dst[j * ld + i0 + acc_row(r)] = Elem<T>::from_f(acc[r]);
+  for (int g = 0; g < 4; ++g) {
+    if constexpr (sizeof(T) == 2) {
+      *reinterpret_cast<u32x2*>(col + 8 * g) =
+          u32x2{f32x2_to_bf16x2(acc[4 * g], acc[4 * g + 1]), f32x2_to_bf16x2(acc[4 * g + 2], acc[4 * g + 3])};
+    } else {
+      *reinterpret_cast<f32x4*>(col + 8 * g) = f32x4{acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]};
+    }
+  }
+}
+// accumulator tile -> LDS, row-major, by way of the matrix core: the tile is rounded to T, transposed (exact) and
+// then written like a transposed tile, four contiguous elements per lane and store instead of one.
+template <typename T>
+__device__ __forceinline__ void acc_to_lds_rm(const f32x16& acc, const IdentityFrag<T>& id, T* dst, int ld, int i0, int j0) {
+  AccB<T> b;
+  b.pack(acc);
+  acc_to_lds_t(mfma_transpose<T>(b, id), dst, ld, j0, i0);
+}
+// 16 per-row values (fp32, in LDS at arr[i0 + row]) for the rows of this lane's accumulator registers
+__device__ __forceinline__ f32x16 rows_ld(const float* arr, int i0) {
+  const float* p = arr + i0 + 4 * ((threadIdx.x & 63) >> 5);
+  f32x16 v;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const f32x4 t = *reinterpret_cast<const f32x4*>(p + 8 * g);
+    v[4 * g] = t[0]; v[4 * g + 1] = t[1]; v[4 * g + 2] = t[2]; v[4 * g + 3] = t[3];
+  }
+  return v;
 }
 // accumulator tile -> global rows (row-major, only rows < nvalid)
 template <typename T>
@@ -494,11 +521,12 @@ __device__ __forceinline__ void rows_add(const f32x16& x, float* rowacc, int i0)
 // an accumulator tile (2 bytes per lane, 16 instructions) are several times slower than these.
 template <typename T> struct Patch { static constexpr int kLd = 32 + 16 / (int)sizeof(T), kElems = 32 * kLd; };
 template <typename T>
-__device__ __forceinline__ void acc_store_rows(const f32x16& acc, T* patch, T* g, int64_t row_stride, int rows_valid) {
+__device__ __forceinline__ void acc_store_rows(const f32x16& acc, const IdentityFrag<T>& id, T* patch, T* g,
+                                               int64_t row_stride, int rows_valid) {
   constexpr int PLD = Patch<T>::kLd, V = Elem<T>::kVec, PPR = 32 / V;
   const int lane = threadIdx.x & 63;
   GDN_WAVE_LDS_SYNC();   // earlier readers of the patch are done
-  acc_to_lds(acc, patch, PLD, 0, 0);
+  acc_to_lds_rm(acc, id, patch, PLD, 0, 0);
   GDN_WAVE_LDS_SYNC();
 #pragma unroll
   for (int p = lane; p < 32 * PPR; p += 64) {
