@@ -21,7 +21,7 @@ struct ChunkWorkspace {
   int64_t chunk_offsets;  // int32 [N+1]      chunks before each packed sequence
   int64_t qn, kn;         // T [tokens,Hqk,K] l2-normalised q,k (only with use_qk_l2norm)
   int64_t G;              // f32 [tokens,Hv]  chunk-local cumulative log decay
-  int64_t Ai;             // T [tokens,Hv,64] rows of (I + A)^-1
+  int64_t Ai;             // T [chunks,Hv,2,2]       (I + A)^-1 as A operand: tile = (32 rows) x (32 columns), fragment order
   int64_t WAF;            // T [chunks,Hv,K/32,2]    W as A operand: tile = (32 tokens) x (32 columns of K), fragment order
   int64_t AQ;             // T [tokens,Hv,64] rows of tril(Q K^T . Gam) (unscaled)
   // Tiles exchanged between kernels in fragment order (see AccB<>): 1024 elements per 32x32 tile.
@@ -52,7 +52,7 @@ inline ChunkWorkspace chunk_workspace_layout(const ChunkDims& d, int elem_bytes)
   w.qn = take(tok * d.Hqk * d.K * elem_bytes);
   w.kn = take(tok * d.Hqk * d.K * elem_bytes);
   w.G = take(tok * d.Hv * 4);
-  w.Ai = take(tok * d.Hv * 64 * elem_bytes);
+  w.Ai = take(nc * 64 * d.Hv * 64 * elem_bytes);
   w.WAF = take(nc * 64 * d.Hv * d.K * elem_bytes);
   w.AQ = take(tok * d.Hv * 64 * elem_bytes);
   w.KDF = take(nc * 64 * d.Hv * d.K * elem_bytes);

@@ -331,64 +331,57 @@ __global__ __launch_bounds__(128 * NW) void chunk_state_bwd_kernel(
 // chunk_bwd_local_kernel, per (chunk, head), 4 waves: everything of the backward pass that is local to a chunk once
 // the reverse recurrence has left dS' and dV' behind.  Wave w owns the 32 K-columns [32w, 32w+32) of dQ, dK, dW and
 // the 32x32 tile (w/2, w%2) of the 64x64 intra-chunk matrices.
+//   pre-pass: R = Tm^T dV' per V block -> dv = beta R, dbeta += <R, v>
 //   main loop over 32-column V blocks:
 //     v_new, dV', dO, S, dS' arrive in fragment order with (lane <-> V column); the contractions run over V, so each
 //     tile is turned through the matrix core (mfma_transpose) into (lane <-> token / K column, registers <-> V).
-//       ds += dO V'^T   a2 += dV' V^T   dQ += dO S^T   dK += V' dS'^T   dW += dV' S^T   R = Tm^T dV' -> dv, dbeta
+//       ds += dO V'^T   a2 += dV' V^T   dQ += dO S^T   dK += V' dS'^T   dW += dV' S^T
 //     All operands of a V block are copied by direct global->LDS loads (no registers in between, fragment order is
 //     exactly the layout such a load produces) into one of two stages, one block ahead of the arithmetic: tiles
-//     shared by the four waves once per workgroup, S and dS' per wave.
-//   epilogue (its LDS tiles reuse the two stages): dQ += ds K, dK += ds^T Q, dG rows as <q,dQ> - <k,dK>; then back
-//   through W = Tm (beta e^G K) with dW still in registers: P = Tm^T dW, a1 = dW K^T,
-//   dTm = strict_tril(a1 beta e^G + a2 beta), dM = -(Tm^T dTm Tm^T).Gam, dK += beta e^G P + beta (dM K) + dM^T (beta K);
-//   dbeta, dg.  dQ, dK, dv leave as 16-byte row pieces.
+//     shared by the four waves once per workgroup, S and dS' per wave.  During the last block the idle stage
+//     receives the epilogue's operands (K in fragment order, this wave's Q columns) the same way.
+//   epilogue: dQ += ds K, dK += ds^T Q, dG rows as <q,dQ> - <k,dK>; then back through W = Tm (beta e^G K) with dW
+//   still in registers: P = Tm^T dW, a1 = dW K^T, dTm = strict_tril(a1 beta e^G + a2 beta), dM = -(Tm^T dTm Tm^T).Gam,
+//   dK += beta e^G P + beta (dM K) + dM^T (beta K); dbeta, dg.  The 64x64 intermediates pass between the waves as
+//   fragment-order tiles in LDS, in one or both of two forms of a tile X(i,j) owned as an accumulator:
+//     D ("direct"):      pack(X)                  lane <-> j, registers <-> i
+//     T ("transposed"):  pack(transpose(pack(X)))  lane <-> i, registers <-> j
+//   dQ, dK, dv leave as 16-byte row pieces.
 // ---------------------------------------------------------------------------------------------
 template <typename T, int DK> struct BwdLocalSmem {
-  static constexpr int LDK = lds_ld<T>(DK), L64 = lds_ld<T>(64);
   // one stage, in elements: [v_new x2 | dV' x2 | dO x2] shared tiles, [S | dS'] per wave, raw V [64][32]
   static constexpr int st_priv = 6 * 1024, st_vraw = st_priv + 4 * 2048, stage_elems = st_vraw + 64 * 32;
-  // epilogue tiles inside the stage area
-  static constexpr int off_ks = 0;                                            // K     [64][LDK]
-  static constexpr int off_tm = off_ks + 64 * LDK * (int)sizeof(T);           // Tm    [64][L64], later (beta . dM)^T
-  static constexpr int off_dw = off_tm + 64 * L64 * (int)sizeof(T);           // dW    [64][LDK], later store patches
-  static constexpr int off_ds = off_dw + 64 * LDK * (int)sizeof(T);           // ds | ds^T; dTm, dM | X^T
-  static constexpr int epi_bytes = off_ds + 2 * 64 * L64 * (int)sizeof(T);
-  static constexpr int off_tmt = 2 * stage_elems * (int)sizeof(T);            // Tm^T  [64][kLT]  (whole kernel)
-  static constexpr int off_row = off_tmt + 64 * kLT * (int)sizeof(T);
+  // epilogue, stage that idles during the last block: K tiles [K/32][2] | Q columns of each wave [64][32]
+  static constexpr int ea_q = 8 * 1024;
+  // epilogue, other stage: dW tiles [2][K/32] (later the store patches) | D-form tiles [4] | T-form tiles [4]
+  static constexpr int eb_d = 8 * 1024, eb_t = 12 * 1024;
+  static constexpr int off_tm = 2 * stage_elems * (int)sizeof(T);             // Tm tiles [2][2], whole kernel
+  static constexpr int off_row = off_tm + 4 * 1024 * (int)sizeof(T);
   static constexpr int bytes = off_row + (6 * 64 + 8) * 4;
-  static_assert(epi_bytes <= off_tmt, "epilogue tiles fit in the two stages");
-  static_assert(Patch<T>::kElems <= 2048 && (DK / 32) * Patch<T>::kElems <= 64 * LDK, "store patches fit");
+  static_assert(stage_elems == 16 * 1024, "the epilogue layout fills a stage exactly");
+  static_assert(Patch<T>::kElems <= 2048, "store patches fit");
 };
 
 template <typename T, int DK>
 __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_local_kernel(
-    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ beta,
+    const T* __restrict__ q, const T* __restrict__ kaf, const T* __restrict__ v, const float* __restrict__ beta,
     const float* __restrict__ G, const T* __restrict__ Ai, const T* __restrict__ vf, const T* __restrict__ dvf,
     const T* __restrict__ dof, const T* __restrict__ hf, const T* __restrict__ dhf, T* __restrict__ dqh,
     T* __restrict__ dkh, T* __restrict__ dv_out, float* __restrict__ dbeta, float* __restrict__ dg,
     const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V,
     float scale) {
   using SM = BwdLocalSmem<T, DK>;
-  constexpr int LDK = SM::LDK, L64 = SM::L64, NKT = DK / 32, VEC = Elem<T>::kVec, KG = AccK<T>::kGroups;
+  constexpr int NKT = DK / 32, VEC = Elem<T>::kVec, KG = AccK<T>::kGroups;
   static_assert(NKT <= 4, "one 32-column block of K per wave");
   T* stage0 = reinterpret_cast<T*>(gdn_smem);
-  T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
-  T* Tm = reinterpret_cast<T*>(gdn_smem + SM::off_tm);
-  T* dWs = reinterpret_cast<T*>(gdn_smem + SM::off_dw);
-  T* dsm = reinterpret_cast<T*>(gdn_smem + SM::off_ds);
-  T* dsT = dsm + 64 * L64;
-  T* TmT = reinterpret_cast<T*>(gdn_smem + SM::off_tmt);
+  T* TmF = reinterpret_cast<T*>(gdn_smem + SM::off_tm);
   float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_row);
   float* egs = Gs + 64;    // e^G
   float* bs = egs + 64;    // beta
-  float* r1 = bs + 64;     // <q_i,dQ_i> - <k_i,dK1_i>
-  float* rb = r1 + 64;     // dbeta
-  float* rg = rb + 64;     // dG through W, U
-  float* wsum = rg + 64;   // per wave: <S,dS'> [0..3], sum_i <k_i, dK_inter_i> [4..7]
-  T* dAs = dsm;
-  T* XT = dsT;
-  T* dMs = dsm;
-  T* dMTb = Tm;
+  float* r1 = bs + 64;     // <q_i,dQ_i> - <k_i,dK_i> + <k_i, (beta e^G P + beta E)_i>
+  float* rbk = r1 + 64;    // e^G <P_i,k_i> + <E_i,k_i>: dbeta without the V part; times beta it is part of dG
+  float* rv = rbk + 64;    // <R_i, v_i>
+  float* wsum = rv + 64;   // per wave: <S,dS'> [0..3], sum_i <k_i, dK_inter_i> [4..7]
 
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
@@ -427,6 +420,27 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       }
     }
   };
+  // stage `buf` <- epilogue operands: all K tiles of the chunk (fragment order), this wave's 32 Q columns [64][32]
+  auto issue_epilogue = [&](int buf) {
+    T* st = stage0 + buf * SM::stage_elems;
+#pragma unroll
+    for (int j = 0; j < 2 * NKT * KG / 4; ++j) {
+      const int piece = 4 * j + wave;
+      load16_to_lds(kaf + ch * (NKT * 2048) + (piece * 64 + lane) * VEC, st + piece * 64 * VEC);
+    }
+    if (has_k) {
+      constexpr int LPR = 32 / VEC, RPP = 64 / LPR;
+#pragma unroll
+      for (int piece = 0; piece < LPR; ++piece) {
+        const int row = piece * RPP + lane / LPR, cc = lane % LPR;
+        load16_to_lds(q + ((tok0 + imin(row, nvalid - 1)) * Hqk + hq) * DK + 32 * cj + cc * VEC,
+                      st + SM::ea_q + wave * 2048 + piece * 64 * VEC);
+      }
+    }
+  };
+#pragma unroll
+  for (int j = 0; j < KG; ++j)                        // Tm tiles, fragment order
+    load16_to_lds(Ai + ch * 4096 + ((4 * j + wave) * 64 + lane) * VEC, TmF + (4 * j + wave) * 64 * VEC);
   issue(0, 0);
 
   if (tid < 64) {
@@ -434,14 +448,21 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     Gs[tid] = gv;
     egs[tid] = __expf(gv);
     bs[tid] = tid < nvalid ? beta[(tok0 + tid) * Hv + h] : 0.f;
-    r1[tid] = 0.f; rb[tid] = 0.f; rg[tid] = 0.f;
+    r1[tid] = 0.f; rbk[tid] = 0.f; rv[tid] = 0.f;
   }
-  load_tile_t<T, 64, kThreads>(TmT, kLT, Ai + (tok0 * Hv + h) * 64, (int64_t)Hv * 64, nvalid, tid);
-
   IdentityFrag<T> id;
   id.init();
-  __syncthreads();
-  // R = Tm^T dV' per 32-column V block (blocks dealt to the waves): dv = beta R, dbeta += <R, v>.  Done before the
+  GDN_WAIT_VMEM();
+  GDN_LDS_BARRIER();
+
+  // Tm^T tile (a, b) as an A operand (lane <-> column of Tm, registers <-> row): the stored tile (b, a) turned round
+  auto tm_t = [&](int a, int b) {
+    AccB<T> f, o;
+    f.load(TmF + (2 * b + a) * 1024);
+    o.pack(mfma_transpose<T>(f, id));
+    return o;
+  };
+  // pre-pass: R = Tm^T dV' per 32-column V block (blocks dealt to the waves): dv = beta R, <R, v>.  Done before the
   // accumulators of the main loop exist; the store patch is this wave's S / dS' slot of the stage not yet in use.
   for (int vblk = wave; vblk < nblk; vblk += 4) {
     AccB<T> fdv[2];
@@ -452,13 +473,13 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     for (int rj = 0; rj < 2; ++rj) {
       f32x16 R = acc_zero(), p;
 #pragma unroll
-      for (int t = rj; t < 2; ++t) mma32_accb<T>(R, TmT + (32 * rj + l32) * kLT + 32 * t, fdv[t]);
+      for (int t = rj; t < 2; ++t) mma32_ff<T>(R, tm_t(rj, t), fdv[t]);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = imin(32 * rj + acc_row(r), nvalid - 1);
         p[r] = R[r] * Elem<T>::to_f(v[((tok0 + row) * Hv + h) * V + 32 * vblk + acc_col()]);
       }
-      rows_add(p, rb, 32 * rj);
+      rows_add(p, rv, 32 * rj);
       const f32x16 bsr = rows_ld(bs, 32 * rj);
 #pragma unroll
       for (int r = 0; r < 16; ++r) R[r] *= bsr[r];
@@ -474,9 +495,11 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
 
   for (int vblk = 0; vblk < nblk; ++vblk) {
     const T* st = stage0 + (vblk & 1) * SM::stage_elems;
-    GDN_WAIT_VMEM();       // this wave's share of the stage has landed ...
-    GDN_LDS_BARRIER();     // ... and so has everybody else's; the other stage is no longer read
-    if (vblk + 1 < nblk) issue(vblk + 1, (vblk + 1) & 1);
+    if (vblk > 0) {
+      GDN_WAIT_VMEM();       // this wave's share of the stage has landed ...
+      GDN_LDS_BARRIER();     // ... and so has everybody else's; the other stage is no longer read
+    }
+    if (vblk + 1 < nblk) issue(vblk + 1, (vblk + 1) & 1); else issue_epilogue((vblk + 1) & 1);
     // Operands are taken one after the other so that few fragments are live at a time; tile indices that depend on
     // the wave are compared against loop constants (fragments indexed at run time would go to scratch).
     AccB<T> f, Sf, dSf, dOt[2];
@@ -520,26 +543,38 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   }
   sds = wave_sum(sds);
   if (lane == 0) wsum[wave] = sds;
-  GDN_LDS_BARRIER();   // the stages are consumed: their space now takes the epilogue tiles
-  load_tile<T, 64>(Tm, L64, Ai + (tok0 * Hv + h) * 64, (int64_t)Hv * 64, nvalid, tid);
-  load_tile<T, DK>(Ks, LDK, k + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
-  GDN_LDS_BARRIER();
+  T* EA = stage0 + (nblk & 1) * SM::stage_elems;        // K tiles | Q columns; later (beta dM) D-form tiles over Q
+  T* EB = stage0 + ((nblk - 1) & 1) * SM::stage_elems;  // dW tiles | D-form tiles | T-form tiles
+  T* dWF = EB;
+  T* tileD = EB + SM::eb_d;
+  T* tileT = EB + SM::eb_t;
+  T* dMD = EA + SM::ea_q;
+  GDN_WAIT_VMEM();
+  GDN_LDS_BARRIER();   // the epilogue operands have landed; the last block's stage is consumed
 
   // this wave's K and Q columns as (lane <-> column, registers <-> token): B operands and row-dot partners
-  AccB<T> KTf[2], QTf[2];
+  AccB<T> KTf[2], QTf[2], dWb[2];
   if (has_k) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       AccB<T> f;
-      frags_from_lds<T>(f, Ks + (32 * t + l32) * LDK + 32 * cj);
+      f.load(EA + (2 * cj + t) * 1024);
       KTf[t].pack(mfma_transpose<T>(f, id));
-      const int row = 32 * t + l32;
-      frags_from_lds<T>(f, q + ((tok0 + imin(row, nvalid - 1)) * Hqk + hq) * DK + 32 * cj);
-      if (row >= nvalid) {
+      frags_from_lds<T>(f, EA + SM::ea_q + wave * 2048 + (32 * t + l32) * 32);
+      if (32 * t + l32 >= nvalid) {
 #pragma unroll
-        for (int g = 0; g < AccK<T>::kGroups; ++g) f.f[g] = u32x4{0u, 0u, 0u, 0u};
+        for (int g = 0; g < KG; ++g) f.f[g] = u32x4{0u, 0u, 0u, 0u};
       }
       QTf[t].pack(mfma_transpose<T>(f, id));
+    }
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri) {         // dW = -(dV' S^T): B operand of P in registers, A operand of a1 to LDS
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dWa[ri][r] = -dWa[ri][r];
+      dWb[ri].pack(dWa[ri]);
+      AccB<T> a;
+      a.pack(mfma_transpose<T>(dWb[ri], id));
+      a.store(dWF + (ri * NKT + cj) * 1024);
     }
   }
   {
@@ -548,22 +583,16 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     const f32x16 gi = rows_ld(Gs, 32 * ti);
 #pragma unroll
     for (int r = 0; r < 16; ++r) ds[r] = (32 * ti + acc_row(r) >= j) ? scale * ds[r] * __expf(gi[r] - gj) : 0.f;
-    acc_to_lds_rm(ds, id, dsm, L64, 32 * ti, 32 * tj);
-    acc_to_lds_t(ds, dsT, L64, 32 * ti, 32 * tj);
-  }
-  AccB<T> dWb[2];
-  if (has_k) {
-#pragma unroll
-    for (int ri = 0; ri < 2; ++ri) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) dWa[ri][r] = -dWa[ri][r];
-      acc_to_lds_rm(dWa[ri], id, dWs, LDK, 32 * ri, 32 * cj);
-      dWb[ri].pack(dWa[ri]);
-    }
+    AccB<T> d, t;
+    d.pack(ds);
+    d.store(tileD + wave * 1024);
+    t.pack(mfma_transpose<T>(d, id));
+    t.store(tileT + wave * 1024);
   }
   GDN_LDS_BARRIER();
   const float glast = Gs[63];
   float ski = 0.f;
+  f32x16 p1[2], pb[2];
   if (has_k) {
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {
@@ -575,45 +604,55 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
         dKi[ri][r] *= __expf(glast - gi[r]);
         ski += dKi[ri][r] * kk[r];           // still only the inter-chunk part
       }
+      AccB<T> a;
 #pragma unroll
-      for (int t = 0; t <= ri; ++t) mma32_accb<T>(dQi[ri], dsm + (32 * ri + l32) * L64 + 32 * t, KTf[t]);
+      for (int t = 0; t <= ri; ++t) { a.load(tileT + (2 * ri + t) * 1024); mma32_ff<T>(dQi[ri], a, KTf[t]); }
 #pragma unroll
-      for (int t = ri; t < 2; ++t) mma32_accb<T>(dKi[ri], dsT + (32 * ri + l32) * L64 + 32 * t, QTf[t]);
-      f32x16 p;
+      for (int t = ri; t < 2; ++t) { a.load(tileD + (2 * t + ri) * 1024); mma32_ff<T>(dKi[ri], a, QTf[t]); }
 #pragma unroll
-      for (int r = 0; r < 16; ++r) p[r] = dQi[ri][r] * qq[r] - dKi[ri][r] * kk[r];
-      rows_add(p, r1, 32 * ri);
+      for (int r = 0; r < 16; ++r) p1[ri][r] = dQi[ri][r] * qq[r] - dKi[ri][r] * kk[r];
     }
   }
   ski = wave_sum(ski);
   if (lane == 0) wsum[4 + wave] = ski;
   // dTm pieces (lower tiles only): a1 = dW K^T over all of K, a2 = dV' V^T from the main loop
   f32x16 a1 = acc_zero();
-  if (lower) mma32<T, DK, true, true>(a1, dWs + 32 * ti * LDK, LDK, Ks + 32 * tj * LDK, LDK);
-  if (has_k) {       // P = Tm^T dW; dK += beta e^G P; dbeta += e^G <P,k>; dG += beta e^G <P,k>
+  if (lower) {
 #pragma unroll
-    for (int rj = 0; rj < 2; ++rj) {
-      f32x16 P = acc_zero(), p;
-#pragma unroll
-      for (int t = rj; t < 2; ++t) mma32_accb<T>(P, TmT + (32 * rj + l32) * kLT + 32 * t, dWb[t]);
-      const f32x16 kk = KTf[rj].unpack(), er = rows_ld(egs, 32 * rj), br = rows_ld(bs, 32 * rj);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) { P[r] *= er[r]; p[r] = P[r] * kk[r]; }
-      rows_add(p, rb, 32 * rj);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) { P[r] *= br[r]; p[r] = P[r] * kk[r]; dKi[rj][r] += P[r]; }
-      rows_add(p, rg, 32 * rj);
+    for (int kt = 0; kt < NKT; ++kt) {
+      AccB<T> a, b;
+      a.load(dWF + (ti * NKT + kt) * 1024);
+      b.load(EA + (2 * kt + tj) * 1024);
+      mma32_ff<T>(a1, a, b);
     }
   }
-  GDN_LDS_BARRIER();   // ds, ds^T and the dW tile are consumed
-  {  // dTm[i][j] = beta_j (e^{G_j} a1 + a2), i > j
+  if (has_k) {       // P = Tm^T dW; dK += beta e^G P; e^G <P,k> joins the dbeta / dG row sums
+#pragma unroll
+    for (int rj = 0; rj < 2; ++rj) {
+      f32x16 P = acc_zero();
+#pragma unroll
+      for (int t = rj; t < 2; ++t) mma32_ff<T>(P, tm_t(rj, t), dWb[t]);
+      const f32x16 kk = KTf[rj].unpack(), er = rows_ld(egs, 32 * rj), br = rows_ld(bs, 32 * rj);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        P[r] *= er[r];
+        pb[rj][r] = P[r] * kk[r];
+        dKi[rj][r] += P[r] * br[r];
+      }
+    }
+  }
+  GDN_LDS_BARRIER();   // the ds tiles and the dW tiles are consumed
+  {  // dTm[i][j] = beta_j (e^{G_j} a1 + a2), i > j, handed on in T form
     const int j = 32 * tj + acc_col();
     const float bj = bs[j], ej = egs[j];
 #pragma unroll
     for (int r = 0; r < 16; ++r) a1[r] = (32 * ti + acc_row(r) > j) ? bj * (ej * a1[r] + a2[r]) : 0.f;
-    acc_to_lds_rm(a1, id, dAs, L64, 32 * ti, 32 * tj);
+    AccB<T> d, t;
+    d.pack(a1);
+    t.pack(mfma_transpose<T>(d, id));
+    t.store(tileT + wave * 1024);
   }
-  T* patch = dWs + wave * Patch<T>::kElems;
+  T* patch = dWF + wave * Patch<T>::kElems;
   if (has_k) {
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri)
@@ -621,15 +660,25 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
                         nvalid - 32 * ri);
   }
   GDN_LDS_BARRIER();
-  {  // X = dTm Tm^T, stored transposed
+  {  // X = dTm Tm^T, handed on in D form
     f32x16 x = acc_zero();
-    mma32<T, 64, true, true>(x, dAs + 32 * ti * L64, L64, Tm + 32 * tj * L64, L64);
-    acc_to_lds_t(x, XT, L64, 32 * ti, 32 * tj);
+    AccB<T> a, b;
+    for (int t = 0; t <= imin(ti, tj); ++t) {
+      a.load(tileT + (2 * ti + t) * 1024);
+      b.load(TmF + (2 * tj + t) * 1024);
+      mma32_ff<T>(x, a, b);
+    }
+    a.pack(x);
+    a.store(tileD + wave * 1024);
   }
   GDN_LDS_BARRIER();
-  {  // dM = -(Tm^T X) . Gam, strictly lower;  dMs[i][j] = dM,  dMTb[j][i] = beta_i dM
+  if (lower) {  // dM = -(Tm^T X) . Gam, strictly lower: T form for dM K, D form scaled by beta_i for dM^T (beta K)
     f32x16 y = acc_zero();
-    mma32_ss<T, 64>(y, TmT + (32 * ti + l32) * kLT, XT + (32 * tj + l32) * L64);
+    AccB<T> b;
+    for (int m = ti; m < 2; ++m) {
+      b.load(tileD + (2 * m + tj) * 1024);
+      mma32_ff<T>(y, tm_t(ti, m), b);
+    }
     const int j = 32 * tj + acc_col();
     const float gj = Gs[j];
     const f32x16 gi = rows_ld(Gs, 32 * ti), br = rows_ld(bs, 32 * ti);
@@ -639,37 +688,39 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       y[r] = (32 * ti + acc_row(r) > j) ? -y[r] * __expf(gi[r] - gj) : 0.f;
       yb[r] = y[r] * br[r];
     }
-    acc_to_lds_rm(y, id, dMs, L64, 32 * ti, 32 * tj);
-    acc_to_lds_t(yb, dMTb, L64, 32 * ti, 32 * tj);
+    AccB<T> d, t;
+    d.pack(y);
+    t.pack(mfma_transpose<T>(d, id));
+    t.store(tileT + wave * 1024);
+    d.pack(yb);
+    d.store(dMD + wave * 1024);
   }
   GDN_LDS_BARRIER();
-  if (has_k) {       // E = dM K, F = dM^T (beta K): dK += beta E + F; dbeta += <E,k>; dG += beta <E,k> - <F,k>
+  if (has_k) {       // E = dM K, F = dM^T (beta K): dK += beta E + F; <E,k> and <F,k> complete the row sums
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {
-      f32x16 E = acc_zero(), Fm = acc_zero(), p;
+      f32x16 E = acc_zero(), Fm = acc_zero();
+      AccB<T> a;
 #pragma unroll
-      for (int t = 0; t <= ri; ++t) mma32_accb<T>(E, dMs + (32 * ri + l32) * L64 + 32 * t, KTf[t]);
+      for (int t = 0; t <= ri; ++t) { a.load(tileT + (2 * ri + t) * 1024); mma32_ff<T>(E, a, KTf[t]); }
 #pragma unroll
-      for (int t = ri; t < 2; ++t) mma32_accb<T>(Fm, dMTb + (32 * ri + l32) * L64 + 32 * t, KTf[t]);
-      const f32x16 kk = KTf[ri].unpack();
-#pragma unroll
-      for (int r = 0; r < 16; ++r) p[r] = E[r] * kk[r];
-      rows_add(p, rb, 32 * ri);
-      const f32x16 br = rows_ld(bs, 32 * ri);
+      for (int t = ri; t < 2; ++t) { a.load(dMD + (2 * t + ri) * 1024); mma32_ff<T>(Fm, a, KTf[t]); }
+      const f32x16 kk = KTf[ri].unpack(), br = rows_ld(bs, 32 * ri);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        E[r] *= br[r];
-        p[r] = (E[r] - Fm[r]) * kk[r];
-        dKi[ri][r] += E[r] + Fm[r];
+        pb[ri][r] += E[r] * kk[r];
+        p1[ri][r] -= Fm[r] * kk[r];
+        dKi[ri][r] += E[r] * br[r] + Fm[r];
       }
-      rows_add(p, rg, 32 * ri);
+      rows_add(pb[ri], rbk, 32 * ri);
+      rows_add(p1[ri], r1, 32 * ri);
       acc_store_rows<T>(dKi[ri], id, patch, dkh + ((tok0 + 32 * ri) * Hv + h) * DK + 32 * cj, (int64_t)Hv * DK,
                         nvalid - 32 * ri);
     }
   }
   GDN_LDS_BARRIER();
   if (wave == 0) {   // d(cumulative G) -> d(g): suffix sum inside the chunk
-    float x = rg[lane] + r1[lane];
+    float x = r1[lane] + bs[lane] * rbk[lane];
     if (lane == nvalid - 1)
       x += __expf(glast) * (wsum[0] + wsum[1] + wsum[2] + wsum[3]) + (wsum[4] + wsum[5] + wsum[6] + wsum[7]);
 #pragma unroll
@@ -679,7 +730,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     }
     if (lane < nvalid) {
       dg[(tok0 + lane) * Hv + h] = x;
-      dbeta[(tok0 + lane) * Hv + h] = rb[lane];
+      dbeta[(tok0 + lane) * Hv + h] = rbk[lane] + rv[lane];
     }
   }
 }
@@ -784,7 +835,7 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     auto kern = chunk_bwd_local_kernel<T, DK>;
     constexpr int smem = BwdLocalSmem<T, DK>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
-    GDN_LAUNCH(kKernBwdLocal, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, (const T*)v, beta, G, Ai, VF,
+    GDN_LAUNCH(kKernBwdLocal, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, (const T*)KAF, (const T*)v, beta, G, Ai, VF,
                (const T*)DVF, (const T*)DOF, HF, (const T*)DHF, DQH, DKH, (T*)dv, dbeta, dg, cu, chunk_offsets, d.T,
                d.N, d.Hqk, d.Hv, d.V, scale);
   }

@@ -253,17 +253,20 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
   // ---- phase 3: Tm in operand precision, kept for the backward pass ----
   {
     constexpr int CPR = 64 / VEC;
-    T* ag = Ai_out + (tok0 * Hv + h) * 64;
     for (int c = tid; c < 64 * CPR; c += kThreads) {
       const int row = c / CPR, cc = c % CPR;
       Vec16<T> x = zero16<T>();
 #pragma unroll
       for (int e = 0; e < VEC; ++e) x.set(e, Ti[row * kLF + cc * VEC + e]);
       st16(Tms + row * L64 + cc * VEC, x);
-      if (row < nvalid) st16(ag + (int64_t)row * Hv * 64 + cc * VEC, x);
     }
   }
   __syncthreads();
+  {  // the four 32x32 tiles of Tm as A operands (lane <-> row, registers <-> column), fragment order, for the backward
+    AccB<T> tf;
+    frags_from_lds<T>(tf, Tms + (32 * (wave >> 1) + (lane & 31)) * L64 + 32 * (wave & 1));
+    tf.store(Ai_out + (((int64_t)blockIdx.x * Hv + h) * 4 + wave) * 1024);
+  }
 
   // ---- phase 4: W = Tm (beta e^G K), handed on in fragment order only ----
   {

@@ -533,6 +533,7 @@ __device__ __forceinline__ void acc_store_rows(const f32x16& acc, const Identity
     const int row = p / PPR, cc = p % PPR;
     if (row < rows_valid) st16(g + (int64_t)row * row_stride + cc * V, ld16(patch + row * PLD + cc * V));
   }
+  GDN_WAVE_LDS_SYNC();   // the patch may be overwritten (also by a direct global->LDS load) once every lane has read it
 }
 
 // sum over the 32 lanes that share a half-wave (all columns of one accumulator row)
