@@ -592,7 +592,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   GDN_LDS_BARRIER();
   const float glast = Gs[63];
   float ski = 0.f;
-  f32x16 p1[2], pb[2];
+  f32x16 p1, pb[2];
   if (has_k) {
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {
@@ -610,7 +610,8 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
 #pragma unroll
       for (int t = ri; t < 2; ++t) { a.load(tileD + (2 * t + ri) * 1024); mma32_ff<T>(dKi[ri], a, QTf[t]); }
 #pragma unroll
-      for (int r = 0; r < 16; ++r) p1[ri][r] = dQi[ri][r] * qq[r] - dKi[ri][r] * kk[r];
+      for (int r = 0; r < 16; ++r) p1[r] = dQi[ri][r] * qq[r] - dKi[ri][r] * kk[r];
+      rows_add(p1, r1, 32 * ri);
     }
   }
   ski = wave_sum(ski);
@@ -709,11 +710,11 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         pb[ri][r] += E[r] * kk[r];
-        p1[ri][r] -= Fm[r] * kk[r];
+        p1[r] = -Fm[r] * kk[r];
         dKi[ri][r] += E[r] * br[r] + Fm[r];
       }
       rows_add(pb[ri], rbk, 32 * ri);
-      rows_add(p1[ri], r1, 32 * ri);
+      rows_add(p1, r1, 32 * ri);
       acc_store_rows<T>(dKi[ri], id, patch, dkh + ((tok0 + 32 * ri) * Hv + h) * DK + 32 * cj, (int64_t)Hv * DK,
                         nvalid - 32 * ri);
     }
