@@ -20,6 +20,7 @@ struct ChunkDims {
 struct ChunkWorkspace {
   int64_t chunk_offsets;  // int32 [N+1]      chunks before each packed sequence
   int64_t qn, kn;         // T [tokens,Hqk,K] l2-normalised q,k (only with use_qk_l2norm)
+  int64_t rstd;           // f32 [2][tokens,Hqk] 1/|q|, 1/|k| of that normalisation
   int64_t G;              // f32 [tokens,Hv]  chunk-local cumulative log decay
   int64_t Ai;             // T [chunks,Hv,2,2]       (I + A)^-1 as A operand: tile = (32 rows) x (32 columns), fragment order
   int64_t WAF;            // T [chunks,Hv,K/32,2]    W as A operand: tile = (32 tokens) x (32 columns of K), fragment order
@@ -37,7 +38,6 @@ struct ChunkWorkspace {
   int64_t DOF;            // T [chunks,Hv,V/32,2]    dO
   int64_t DVF;            // T [chunks,Hv,V/32,2]    d(v_new)
   int64_t DHF;            // T [chunks,Hv,V/32,K/32] gradient of the state AFTER each chunk
-  int64_t DQH, DKH;       // T [tokens,Hv,K]  per-value-head dq, dk before the group sum
   int64_t total_bytes;
 };
 
@@ -51,6 +51,7 @@ inline ChunkWorkspace chunk_workspace_layout(const ChunkDims& d, int elem_bytes)
   w.chunk_offsets = take((int64_t)(d.N + 1) * 4);
   w.qn = take(tok * d.Hqk * d.K * elem_bytes);
   w.kn = take(tok * d.Hqk * d.K * elem_bytes);
+  w.rstd = take(2 * tok * d.Hqk * 4);
   w.G = take(tok * d.Hv * 4);
   w.Ai = take(nc * 64 * d.Hv * 64 * elem_bytes);
   w.WAF = take(nc * 64 * d.Hv * d.K * elem_bytes);
@@ -67,8 +68,6 @@ inline ChunkWorkspace chunk_workspace_layout(const ChunkDims& d, int elem_bytes)
   w.DOF = take(nc * 64 * d.Hv * d.V * elem_bytes);
   w.DVF = take(nc * 64 * d.Hv * d.V * elem_bytes);
   w.DHF = take(nc * d.Hv * d.V * d.K * elem_bytes);
-  w.DQH = take(tok * d.Hv * d.K * elem_bytes);
-  w.DKH = take(tok * d.Hv * d.K * elem_bytes);
   w.total_bytes = off;
   return w;
 }

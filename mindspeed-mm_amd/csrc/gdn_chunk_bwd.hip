@@ -11,7 +11,7 @@
 //     dK2 = P beta e^G + beta (dM K) + dM^T (beta K);  dv = R beta
 //     dbeta = e^G<P,k> + <R,v> + <dM K, k>;  dG2 = beta e^G<P,k> + beta<dM K,k> - <dM^T(beta K),k>
 //   dg = reverse chunk-local cumsum(dG1 + dG2); group sum of dq/dk over grouped heads and the
-//   l2-norm backward dx = (dy - <dy,y> y) rstd                                  qk_grad_finalize_kernel
+//   l2-norm backward dx = (dy - <dy,y> y) rstd                                  (same kernel)
 // The equations are those of the reference's backward kernels (mindspeed_mm/fsdp/ops/gdn/triton/
 // chunk_o.py:19-284, chunk_delta_h.py:307-513, wy_fast.py:17-141, chunk_gated_delta_rule.py:88-174), with
 // the dG row/column sums rewritten as row dot products with dQ/dK so that Q K^T need not be rebuilt.
@@ -357,7 +357,7 @@ template <typename T, int DK> struct BwdLocalSmem {
   static constexpr int eb_d = 8 * 1024, eb_t = 12 * 1024;
   static constexpr int off_tm = 2 * stage_elems * (int)sizeof(T);             // Tm tiles [2][2], whole kernel
   static constexpr int off_row = off_tm + 4 * 1024 * (int)sizeof(T);
-  static constexpr int bytes = off_row + (6 * 64 + 8) * 4;
+  static constexpr int bytes = off_row + (11 * 64 + 8) * 4;
   static_assert(stage_elems == 16 * 1024, "the epilogue layout fills a stage exactly");
   static_assert(Patch<T>::kElems <= 2048, "store patches fit");
 };
@@ -366,10 +366,10 @@ template <typename T, int DK>
 __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_local_kernel(
     const T* __restrict__ q, const T* __restrict__ kaf, const T* __restrict__ v, const float* __restrict__ beta,
     const float* __restrict__ G, const T* __restrict__ Ai, const T* __restrict__ vf, const T* __restrict__ dvf,
-    const T* __restrict__ dof, const T* __restrict__ hf, const T* __restrict__ dhf, T* __restrict__ dqh,
-    T* __restrict__ dkh, T* __restrict__ dv_out, float* __restrict__ dbeta, float* __restrict__ dg,
-    const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V,
-    float scale) {
+    const T* __restrict__ dof, const T* __restrict__ hf, const T* __restrict__ dhf, const float* __restrict__ rstd_q,
+    const float* __restrict__ rstd_k, T* dq, T* dk, T* __restrict__ dv_out, float* __restrict__ dbeta,
+    float* __restrict__ dg, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N,
+    int Hqk, int Hv, int V, float scale, int hh) {
   using SM = BwdLocalSmem<T, DK>;
   constexpr int NKT = DK / 32, VEC = Elem<T>::kVec, KG = AccK<T>::kGroups;
   static_assert(NKT <= 4, "one 32-column block of K per wave");
@@ -378,21 +378,32 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_row);
   float* egs = Gs + 64;    // e^G
   float* bs = egs + 64;    // beta
-  float* r1 = bs + 64;     // <q_i,dQ_i> - <k_i,dK_i> + <k_i, (beta e^G P + beta E)_i>
-  float* rbk = r1 + 64;    // e^G <P_i,k_i> + <E_i,k_i>: dbeta without the V part; times beta it is part of dG
-  float* rv = rbk + 64;    // <R_i, v_i>
-  float* wsum = rv + 64;   // per wave: <S,dS'> [0..3], sum_i <k_i, dK_inter_i> [4..7]
+  float* rq = bs + 64;     // <q_i, dQ_i>
+  float* rk1 = rq + 64;    // <k_i, dK_i> before the terms that come back through W
+  float* rbk = rk1 + 64;   // e^G <P_i,k_i> + <E_i,k_i>: dbeta without the V part; times beta it is part of dG and <k,dK>
+  float* rf = rbk + 64;    // <F_i, k_i>
+  float* rv = rf + 64;     // <R_i, v_i>
+  float* rsq = rv + 64;    // 1/|q_i|, 1/|k_i| of the l2 normalisation (1 without it)
+  float* rsk = rsq + 64;
+  float* wsum = rsk + 64;  // per wave: <S,dS'> [0..3], sum_i <k_i, dK_inter_i> [4..7]
 
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: branches on it are scalar
-  const int h = blockIdx.y, hq = h / (Hv / Hqk), nvalid = s.nvalid;
+  const int hq = blockIdx.y, grp = Hv / Hqk, nvalid = s.nvalid;
   const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk;
-  const int64_t ch = (int64_t)blockIdx.x * Hv + h;
   const int ti = wave >> 1, tj = wave & 1, cj = wave;
-  const bool lower = tj <= ti, has_k = wave < NKT;
+  const bool lower = tj <= ti, has_k = wave < NKT, l2 = rstd_q != nullptr;
   const int nblk = V / 32;
+  IdentityFrag<T> id;
+  id.init();
+
+  // One launch per value head of a q/k group (hh = 0 .. Hv/Hqk-1): the first writes dq and dk, the later ones add
+  // to them in place, so no per-value-head copy of dq, dk ever exists.  The l2-norm backward
+  // dx = (dy - <dy,y> y) / |x| is linear in dy and is applied to each head's contribution.
+  const int h = hq * grp + hh;
+  const int64_t ch = (int64_t)blockIdx.x * Hv + h;
 
   // stage `buf` <- operands of V block `vblk`; every load moves 64 x 16 bytes, lane l's piece landing at +16 l
   auto issue = [&](int vblk, int buf) {
@@ -448,10 +459,10 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     Gs[tid] = gv;
     egs[tid] = __expf(gv);
     bs[tid] = tid < nvalid ? beta[(tok0 + tid) * Hv + h] : 0.f;
-    r1[tid] = 0.f; rbk[tid] = 0.f; rv[tid] = 0.f;
+    rq[tid] = 0.f; rk1[tid] = 0.f; rbk[tid] = 0.f; rf[tid] = 0.f; rv[tid] = 0.f;
+    rsq[tid] = l2 ? rstd_q[(tok0 + imin(tid, nvalid - 1)) * Hqk + hq] : 1.f;
+    rsk[tid] = l2 ? rstd_k[(tok0 + imin(tid, nvalid - 1)) * Hqk + hq] : 1.f;
   }
-  IdentityFrag<T> id;
-  id.init();
   GDN_WAIT_VMEM();
   GDN_LDS_BARRIER();
 
@@ -483,7 +494,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       const f32x16 bsr = rows_ld(bs, 32 * rj);
 #pragma unroll
       for (int r = 0; r < 16; ++r) R[r] *= bsr[r];
-      acc_store_rows<T>(R, id, patch, dv_out + ((tok0 + 32 * rj) * Hv + h) * V + 32 * vblk, (int64_t)Hv * V,
+      acc_store_rows<T, false>(R, id, patch, dv_out + ((tok0 + 32 * rj) * Hv + h) * V + 32 * vblk, (int64_t)Hv * V,
                         nvalid - 32 * rj);
     }
   }
@@ -592,7 +603,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   GDN_LDS_BARRIER();
   const float glast = Gs[63];
   float ski = 0.f;
-  f32x16 p1, pb[2];
+  f32x16 pb[2];
   if (has_k) {
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {
@@ -609,9 +620,13 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       for (int t = 0; t <= ri; ++t) { a.load(tileT + (2 * ri + t) * 1024); mma32_ff<T>(dQi[ri], a, KTf[t]); }
 #pragma unroll
       for (int t = ri; t < 2; ++t) { a.load(tileD + (2 * t + ri) * 1024); mma32_ff<T>(dKi[ri], a, QTf[t]); }
+      f32x16 p;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) p1[r] = dQi[ri][r] * qq[r] - dKi[ri][r] * kk[r];
-      rows_add(p1, r1, 32 * ri);
+      for (int r = 0; r < 16; ++r) p[r] = dQi[ri][r] * qq[r];
+      rows_add(p, rq, 32 * ri);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) p[r] = dKi[ri][r] * kk[r];
+      rows_add(p, rk1, 32 * ri);
     }
   }
   ski = wave_sum(ski);
@@ -656,9 +671,16 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   T* patch = dWF + wave * Patch<T>::kElems;
   if (has_k) {
 #pragma unroll
-    for (int ri = 0; ri < 2; ++ri)
-      acc_store_rows<T>(dQi[ri], id, patch, dqh + ((tok0 + 32 * ri) * Hv + h) * DK + 32 * cj, (int64_t)Hv * DK,
-                        nvalid - 32 * ri);
+    for (int ri = 0; ri < 2; ++ri) {
+      if (l2) {
+        const f32x16 qq = QTf[ri].unpack(), dot = rows_ld(rq, 32 * ri), rs = rows_ld(rsq, 32 * ri);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dQi[ri][r] = (dQi[ri][r] - dot[r] * qq[r]) * rs[r];
+      }
+      T* dst = dq + ((tok0 + 32 * ri) * Hqk + hq) * DK + 32 * cj;
+      if (hh == 0) acc_store_rows<T, false>(dQi[ri], id, patch, dst, (int64_t)Hqk * DK, nvalid - 32 * ri);
+      else acc_store_rows<T, true>(dQi[ri], id, patch, dst, (int64_t)Hqk * DK, nvalid - 32 * ri);
+    }
   }
   GDN_LDS_BARRIER();
   {  // X = dTm Tm^T, handed on in D form
@@ -700,7 +722,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   if (has_k) {       // E = dM K, F = dM^T (beta K): dK += beta E + F; <E,k> and <F,k> complete the row sums
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {
-      f32x16 E = acc_zero(), Fm = acc_zero();
+      f32x16 E = acc_zero(), Fm = acc_zero(), p;
       AccB<T> a;
 #pragma unroll
       for (int t = 0; t <= ri; ++t) { a.load(tileT + (2 * ri + t) * 1024); mma32_ff<T>(E, a, KTf[t]); }
@@ -710,18 +732,31 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         pb[ri][r] += E[r] * kk[r];
-        p1[r] = -Fm[r] * kk[r];
+        p[r] = Fm[r] * kk[r];
         dKi[ri][r] += E[r] * br[r] + Fm[r];
       }
       rows_add(pb[ri], rbk, 32 * ri);
-      rows_add(p1, r1, 32 * ri);
-      acc_store_rows<T>(dKi[ri], id, patch, dkh + ((tok0 + 32 * ri) * Hv + h) * DK + 32 * cj, (int64_t)Hv * DK,
-                        nvalid - 32 * ri);
+      rows_add(p, rf, 32 * ri);
     }
   }
-  GDN_LDS_BARRIER();
+  GDN_LDS_BARRIER();   // the row sums are complete
+  if (has_k) {
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri) {
+      if (l2) {          // <k_i, dK_i> = <k,dK1> + beta (e^G <P,k> + <E,k>) + <F,k>
+        const f32x16 kk = KTf[ri].unpack(), d1 = rows_ld(rk1, 32 * ri), db = rows_ld(rbk, 32 * ri),
+                     df = rows_ld(rf, 32 * ri), br = rows_ld(bs, 32 * ri), rs = rows_ld(rsk, 32 * ri);
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          dKi[ri][r] = (dKi[ri][r] - (d1[r] + br[r] * db[r] + df[r]) * kk[r]) * rs[r];
+      }
+      T* dst = dk + ((tok0 + 32 * ri) * Hqk + hq) * DK + 32 * cj;
+      if (hh == 0) acc_store_rows<T, false>(dKi[ri], id, patch, dst, (int64_t)Hqk * DK, nvalid - 32 * ri);
+      else acc_store_rows<T, true>(dKi[ri], id, patch, dst, (int64_t)Hqk * DK, nvalid - 32 * ri);
+    }
+  }
   if (wave == 0) {   // d(cumulative G) -> d(g): suffix sum inside the chunk
-    float x = r1[lane] + bs[lane] * rbk[lane];
+    float x = rq[lane] - rk1[lane] + bs[lane] * rbk[lane] - rf[lane];
     if (lane == nvalid - 1)
       x += __expf(glast) * (wsum[0] + wsum[1] + wsum[2] + wsum[3]) + (wsum[4] + wsum[5] + wsum[6] + wsum[7]);
 #pragma unroll
@@ -733,57 +768,6 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       dg[(tok0 + lane) * Hv + h] = x;
       dbeta[(tok0 + lane) * Hv + h] = rbk[lane] + rv[lane];
     }
-  }
-}
-
-// ---------------------------------------------------------------------------------------------
-// dq/dk: sum over the value heads of a group, then back through the l2 norm if it was applied.
-// ---------------------------------------------------------------------------------------------
-template <typename T, int DK>
-__global__ void qk_grad_finalize_kernel(const T* __restrict__ dqh, const T* __restrict__ dkh, const T* __restrict__ q,
-                                        const T* __restrict__ k, T* __restrict__ dq, T* __restrict__ dk, int64_t rows,
-                                        int Hqk, int Hv, int l2norm) {
-  constexpr int V = Elem<T>::kVec, LPR = DK / V;
-  const T* src = blockIdx.y == 0 ? dqh : dkh;
-  const T* x = blockIdx.y == 0 ? q : k;
-  T* dst = blockIdx.y == 0 ? dq : dk;
-  const int64_t row = (int64_t)blockIdx.x * (kThreads / LPR) + threadIdx.x / LPR;   // (token, qk head)
-  const int c = threadIdx.x % LPR;
-  const bool ok = row < rows;
-  const int grp = Hv / Hqk;
-  const int64_t tok = ok ? row / Hqk : 0;
-  const int hq = ok ? (int)(row % Hqk) : 0;
-  float acc[V];
-#pragma unroll
-  for (int e = 0; e < V; ++e) acc[e] = 0.f;
-  if (ok) {
-    for (int gi = 0; gi < grp; ++gi) {
-      const Vec16<T> t = ld16(src + ((tok * Hv + hq * grp + gi) * DK) + c * V);
-#pragma unroll
-      for (int e = 0; e < V; ++e) acc[e] += t.get(e);
-    }
-  }
-  if (l2norm) {   // uniform branch: every lane takes part in the shuffles
-    Vec16<T> xv = ok ? ld16(x + row * DK + c * V) : zero16<T>();
-    float ss = 0.f;
-#pragma unroll
-    for (int e = 0; e < V; ++e) { const float f = xv.get(e); ss += f * f; }
-#pragma unroll
-    for (int m = 1; m < LPR; m <<= 1) ss += __shfl_xor(ss, m);
-    const float rstd = rsqrtf(ss + 1e-6f);
-    float dot = 0.f;
-#pragma unroll
-    for (int e = 0; e < V; ++e) dot += acc[e] * xv.get(e) * rstd;
-#pragma unroll
-    for (int m = 1; m < LPR; m <<= 1) dot += __shfl_xor(dot, m);
-#pragma unroll
-    for (int e = 0; e < V; ++e) acc[e] = (acc[e] - dot * xv.get(e) * rstd) * rstd;
-  }
-  if (ok) {
-    Vec16<T> o = zero16<T>();
-#pragma unroll
-    for (int e = 0; e < V; ++e) o.set(e, acc[e]);
-    st16(dst + row * DK + c * V, o);
   }
 }
 
@@ -815,8 +799,8 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   T* DOF = reinterpret_cast<T*>(ws + L.DOF);
   T* DVF = reinterpret_cast<T*>(ws + L.DVF);
   T* DHF = reinterpret_cast<T*>(ws + L.DHF);
-  T* DQH = reinterpret_cast<T*>(ws + L.DQH);
-  T* DKH = reinterpret_cast<T*>(ws + L.DKH);
+  const float* rstd_q = l2norm ? reinterpret_cast<const float*>(ws + L.rstd) : nullptr;
+  const float* rstd_k = l2norm ? rstd_q + tok * d.Hqk : nullptr;
   {
     auto kern = chunk_bwd_prep_kernel<T, DK, NW>;
     constexpr int smem = BwdPrepSmem<T, DK, NW>::bytes;
@@ -836,16 +820,10 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     auto kern = chunk_bwd_local_kernel<T, DK>;
     constexpr int smem = BwdLocalSmem<T, DK>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
-    GDN_LAUNCH(kKernBwdLocal, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, (const T*)KAF, (const T*)v, beta, G, Ai, VF,
-               (const T*)DVF, (const T*)DOF, HF, (const T*)DHF, DQH, DKH, (T*)dv, dbeta, dg, cu, chunk_offsets, d.T,
-               d.N, d.Hqk, d.Hv, d.V, scale);
-  }
-  {
-    constexpr int LPR = DK / Elem<T>::kVec;
-    const int64_t rows = tok * d.Hqk;
-    GDN_LAUNCH(kKernQkFinalize, st, (qk_grad_finalize_kernel<T, DK>),
-               dim3((unsigned)((rows + kThreads / LPR - 1) / (kThreads / LPR)), 2), dim3(kThreads), 0, st,
-               (const T*)DQH, (const T*)DKH, (const T*)q, (const T*)k, (T*)dq, (T*)dk, rows, d.Hqk, d.Hv, l2norm);
+    for (int hh = 0; hh < d.Hv / d.Hqk; ++hh)
+      GDN_LAUNCH(kKernBwdLocal, st, kern, dim3(nc, d.Hqk), dim3(kThreads), smem, st, qq, (const T*)KAF, (const T*)v,
+                 beta, G, Ai, VF, (const T*)DVF, (const T*)DOF, HF, (const T*)DHF, rstd_q, rstd_k, (T*)dq, (T*)dk,
+                 (T*)dv, dbeta, dg, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale, hh);
   }
   return (int)hipGetLastError();
 }

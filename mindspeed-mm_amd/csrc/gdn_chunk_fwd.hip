@@ -55,7 +55,7 @@ __global__ void chunk_table_kernel(const int64_t* __restrict__ cu, int* __restri
 // ---------------------------------------------------------------------------------------------
 template <typename T, int DK>
 __global__ void l2norm_fwd_kernel(const T* __restrict__ x0, const T* __restrict__ x1, T* __restrict__ y0,
-                                  T* __restrict__ y1, int64_t rows) {
+                                  T* __restrict__ y1, float* __restrict__ rstd, int64_t rows) {
   constexpr int V = Elem<T>::kVec, LPR = DK / V;  // lanes per row (a power of two <= 32)
   const T* x = blockIdx.y == 0 ? x0 : x1;
   T* y = blockIdx.y == 0 ? y0 : y1;
@@ -72,6 +72,7 @@ __global__ void l2norm_fwd_kernel(const T* __restrict__ x0, const T* __restrict_
 #pragma unroll
   for (int e = 0; e < V; ++e) v.set(e, v.get(e) * r);
   if (ok) st16(y + row * DK + c * V, v);
+  if (ok && c == 0) rstd[blockIdx.y * rows + row] = r;   // kept for the backward pass
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -601,7 +602,7 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     T* kn = reinterpret_cast<T*>(ws + L.kn);
     GDN_LAUNCH(kKernL2Norm, st, (l2norm_fwd_kernel<T, DK>),
                dim3((unsigned)((rows + kThreads / LPR - 1) / (kThreads / LPR)), 2), dim3(kThreads), 0, st, qq, kk, qn,
-               kn, rows);
+               kn, reinterpret_cast<float*>(ws + L.rstd), rows);
     qq = qn;
     kk = kn;
   }

@@ -520,7 +520,8 @@ __device__ __forceinline__ void rows_add(const f32x16& x, float* rowacc, int i0)
 // 16-byte pieces after a pass through a wave-private LDS patch of 32 x kPatchLd elements.  Element-wise stores of
 // an accumulator tile (2 bytes per lane, 16 instructions) are several times slower than these.
 template <typename T> struct Patch { static constexpr int kLd = 32 + 16 / (int)sizeof(T), kElems = 32 * kLd; };
-template <typename T>
+// ADD: the rows are added to what global memory already holds (written earlier by this very thread).
+template <typename T, bool ADD>
 __device__ __forceinline__ void acc_store_rows(const f32x16& acc, const IdentityFrag<T>& id, T* patch, T* g,
                                                int64_t row_stride, int rows_valid) {
   constexpr int PLD = Patch<T>::kLd, V = Elem<T>::kVec, PPR = 32 / V;
@@ -531,7 +532,15 @@ __device__ __forceinline__ void acc_store_rows(const f32x16& acc, const Identity
 #pragma unroll
   for (int p = lane; p < 32 * PPR; p += 64) {
     const int row = p / PPR, cc = p % PPR;
-    if (row < rows_valid) st16(g + (int64_t)row * row_stride + cc * V, ld16(patch + row * PLD + cc * V));
+    if (row < rows_valid) {
+      Vec16<T> x = ld16(patch + row * PLD + cc * V);
+      if constexpr (ADD) {
+        const Vec16<T> y = ld16(g + (int64_t)row * row_stride + cc * V);
+#pragma unroll
+        for (int e = 0; e < V; ++e) x.set(e, x.get(e) + y.get(e));
+      }
+      st16(g + (int64_t)row * row_stride + cc * V, x);
+    }
   }
   GDN_WAVE_LDS_SYNC();   // the patch may be overwritten (also by a direct global->LDS load) once every lane has read it
 }

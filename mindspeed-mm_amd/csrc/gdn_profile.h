@@ -7,7 +7,7 @@ namespace gdn {
 
 enum KernelId {
   kKernChunkTable = 0, kKernL2Norm, kKernPrep, kKernStateFwd, kKernOut, kKernBwdPrep, kKernStateBwd, kKernBwdLocal,
-  kKernQkFinalize, kKernRecurrent, kKernConvFwd, kKernConvState, kKernConvBwd, kKernConvReduce,
+  kKernRecurrent, kKernConvFwd, kKernConvState, kKernConvBwd, kKernConvReduce,
   kKernConvDh0, kKernConvUpdate, kKernCount
 };
 
