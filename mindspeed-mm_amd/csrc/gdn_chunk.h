@@ -24,7 +24,7 @@ struct ChunkWorkspace {
   int64_t G;              // f32 [tokens,Hv]  chunk-local cumulative log decay
   int64_t Ai;             // T [chunks,Hv,2,2]       (I + A)^-1 as A operand: tile = (32 rows) x (32 columns), fragment order
   int64_t WAF;            // T [chunks,Hv,K/32,2]    W as A operand: tile = (32 tokens) x (32 columns of K), fragment order
-  int64_t AQ;             // T [tokens,Hv,64] rows of tril(Q K^T . Gam) (unscaled)
+  int64_t AQ;             // T [chunks,Hv,2,2]       tril(Q K^T . Gam) (unscaled), accumulator tiles: lane <-> column, registers <-> row
   // Tiles exchanged between kernels in fragment order (see AccB<>): 1024 elements per 32x32 tile.
   int64_t KDF;            // T [chunks,Hv,K/32,2]    (e^{G_last-G} . K)^T as A operand: tile = (32 rows of K) x (32 tokens)
   int64_t UF;             // T [chunks,Hv,V/32,2]    U,            tile = (32-token block ri) x (32-column block)
@@ -55,7 +55,7 @@ inline ChunkWorkspace chunk_workspace_layout(const ChunkDims& d, int elem_bytes)
   w.G = take(tok * d.Hv * 4);
   w.Ai = take(nc * 64 * d.Hv * 64 * elem_bytes);
   w.WAF = take(nc * 64 * d.Hv * d.K * elem_bytes);
-  w.AQ = take(tok * d.Hv * 64 * elem_bytes);
+  w.AQ = take(nc * 64 * d.Hv * 64 * elem_bytes);
   w.KDF = take(nc * 64 * d.Hv * d.K * elem_bytes);
   w.UF = take(nc * 64 * d.Hv * d.V * elem_bytes);
   w.VF = take(nc * 64 * d.Hv * d.V * elem_bytes);

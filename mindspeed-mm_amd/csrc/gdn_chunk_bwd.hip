@@ -35,90 +35,55 @@ __device__ __forceinline__ void acc_rowdot_add(const f32x16& acc, const T* other
 }
 
 // ---------------------------------------------------------------------------------------------
-// chunk_bwd_prep_kernel: everything the reverse recurrence needs that is independent across chunks, written in
-// fragment order (AccB<>) so that the sequential kernel only copies contiguous 16-byte pieces:
-//   DVLF  dv_local = scale Aq^T dO                 (accumulator tiles, per 32-column block)
+// chunk_bwd_prep_kernel: what the reverse recurrence needs from dO, written in fragment order (AccB<>) so that the
+// sequential kernel only copies contiguous 16-byte pieces.  One wave per (chunk, head, 32-column V block), no LDS:
 //   DOF   dO as a B operand                         (lane <-> V column, registers <-> token)
-//   QSF   (scale e^G . Q)^T as an A operand         (lane <-> K column, registers <-> token)
-//   KAF   K as an A operand                         (lane <-> token, registers <-> K column)
+//   DVLF  dv_local = scale Aq^T dO                 (accumulator tiles)
+// dO rows are gathered straight from global memory as A-operand fragments (lane <-> token) and turned through the
+// matrix core; Aq^T tiles are the forward pass's tril(Q K^T . Gam) tiles as stored.
 // ---------------------------------------------------------------------------------------------
-constexpr int kLT = 68;   // leading dimension of transposed [*][64] LDS tiles (8-byte fragment reads stay aligned)
 
-template <typename T, int DK, int NW> struct BwdPrepSmem {
-  static constexpr int LDK = lds_ld<T>(DK);
-  static constexpr int off_qs = 0;
-  static constexpr int off_ks = off_qs + 64 * LDK * (int)sizeof(T);
-  static constexpr int off_aq = off_ks + 64 * LDK * (int)sizeof(T);
-  static constexpr int off_do = off_aq + 64 * kLT * (int)sizeof(T);
-  static constexpr int off_gs = off_do + 32 * NW * kLT * (int)sizeof(T);
-  static constexpr int bytes = off_gs + 64 * 4;
-};
-
-template <typename T, int DK, int NW>
+template <typename T, int NW>
 __global__ __launch_bounds__(64 * NW) void chunk_bwd_prep_kernel(
-    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ aqk, const T* __restrict__ dO,
-    const float* __restrict__ G, T* __restrict__ dvlf, T* __restrict__ dof, T* __restrict__ qsf, T* __restrict__ kaf,
-    const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V,
+    const T* __restrict__ aqf, const T* __restrict__ dO, T* __restrict__ dvlf, T* __restrict__ dof,
+    const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N, int Hv, int V,
     float scale) {
-  using SM = BwdPrepSmem<T, DK, NW>;
-  constexpr int LDK = SM::LDK, NT = 64 * NW, VEC = Elem<T>::kVec;
-  T* Qs = reinterpret_cast<T*>(gdn_smem + SM::off_qs);
-  T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
-  T* AqT = reinterpret_cast<T*>(gdn_smem + SM::off_aq);
-  T* dOT = reinterpret_cast<T*>(gdn_smem + SM::off_do);
-  float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_gs);
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31;
-  const int h = blockIdx.y, hq = h / (Hv / Hqk), nvalid = s.nvalid;
+  const int h = blockIdx.y, nvalid = s.nvalid;
   const int vblk = blockIdx.z * NW + wave;
   const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk;
   const int64_t ch = (int64_t)blockIdx.x * Hv + h;
 
-  for (int c = tid; c < 64 * (DK / VEC); c += NT) {
-    const int row = c / (DK / VEC), cc = c % (DK / VEC);
-    const bool ok = row < nvalid;
-    st16(Qs + row * LDK + cc * VEC, ok ? ld16(q + ((tok0 + row) * Hqk + hq) * DK + cc * VEC) : zero16<T>());
-    st16(Ks + row * LDK + cc * VEC, ok ? ld16(k + ((tok0 + row) * Hqk + hq) * DK + cc * VEC) : zero16<T>());
-  }
-  load_tile_t<T, 64, NT>(AqT, kLT, aqk + (tok0 * Hv + h) * 64, (int64_t)Hv * 64, nvalid, tid);
-  load_tile_t<T, 32 * NW, NT>(dOT, kLT, dO + (tok0 * Hv + h) * V + 32 * NW * blockIdx.z, (int64_t)Hv * V, nvalid, tid);
-  if (tid < 64) Gs[tid] = scale * __expf(G[(tok0 + imin(tid, nvalid - 1)) * Hv + h]);
-  __syncthreads();
-
-  AccB<T> df[2];
+  IdentityFrag<T> id;
+  id.init();
+  AccB<T> df[2], aq[3];
+  aq[0].load(aqf + (ch * 4 + 0) * 1024);   // tiles (0,0), (1,0), (1,1)
+  aq[1].load(aqf + (ch * 4 + 2) * 1024);
+  aq[2].load(aqf + (ch * 4 + 3) * 1024);
 #pragma unroll
   for (int ti = 0; ti < 2; ++ti) {
-    frags_from_lds<T>(df[ti], dOT + (32 * wave + l32) * kLT + 32 * ti);
+    const int row = 32 * ti + l32;
+    AccB<T> f;
+    frags_from_lds<T>(f, dO + ((tok0 + imin(row, nvalid - 1)) * Hv + h) * V + 32 * vblk);
+    if (row >= nvalid) {
+#pragma unroll
+      for (int g = 0; g < AccK<T>::kGroups; ++g) f.f[g] = u32x4{0u, 0u, 0u, 0u};
+    }
+    df[ti].pack(mfma_transpose<T>(f, id));
     df[ti].store(dof + ((ch * (V / 32) + vblk) * 2 + ti) * 1024);
   }
 #pragma unroll
   for (int rj = 0; rj < 2; ++rj) {          // dv_local[j] = scale sum_{i >= j} Aq[i][j] dO[i]
     f32x16 acc = acc_zero();
 #pragma unroll
-    for (int ti = rj; ti < 2; ++ti) mma32_accb<T>(acc, AqT + (32 * rj + l32) * kLT + 32 * ti, df[ti]);
+    for (int ti = rj; ti < 2; ++ti) mma32_ff<T>(acc, aq[ti + rj], df[ti]);
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[r] *= scale;
     AccB<T> out;
     out.pack(acc);
     out.store(dvlf + ((ch * (V / 32) + vblk) * 2 + rj) * 1024);
-  }
-  if (blockIdx.z == 0) {
-    IdentityFrag<T> id;
-    id.init();
-    for (int tt = wave; tt < 2 * (DK / 32); tt += NW) {
-      const int tj = tt & 1, kt = tt >> 1;
-      const int64_t tile = (ch * (DK / 32) + kt) * 2 + tj;
-      AccB<T> f;
-      frags_from_lds<T>(f, Ks + (32 * tj + l32) * LDK + 32 * kt);
-      f.store(kaf + tile * 1024);
-      frags_from_lds<T>(f, Qs + (32 * tj + l32) * LDK + 32 * kt);
-      f32x16 qt = mfma_transpose<T>(f, id);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) qt[r] *= Gs[32 * tj + acc_row(r)];
-      f.pack(qt);
-      f.store(qsf + tile * 1024);
-    }
   }
 }
 
@@ -793,8 +758,8 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   const T* WF = reinterpret_cast<const T*>(ws + L.WF);
   const T* VF = reinterpret_cast<const T*>(ws + L.VF);
   const T* HF = reinterpret_cast<const T*>(ws + L.HF);
-  T* QSF = reinterpret_cast<T*>(ws + L.QSF);
-  T* KAF = reinterpret_cast<T*>(ws + L.KAF);
+  const T* QSF = reinterpret_cast<const T*>(ws + L.QSF);
+  const T* KAF = reinterpret_cast<const T*>(ws + L.KAF);
   T* DVLF = reinterpret_cast<T*>(ws + L.DVLF);
   T* DOF = reinterpret_cast<T*>(ws + L.DOF);
   T* DVF = reinterpret_cast<T*>(ws + L.DVF);
@@ -802,11 +767,9 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   const float* rstd_q = l2norm ? reinterpret_cast<const float*>(ws + L.rstd) : nullptr;
   const float* rstd_k = l2norm ? rstd_q + tok * d.Hqk : nullptr;
   {
-    auto kern = chunk_bwd_prep_kernel<T, DK, NW>;
-    constexpr int smem = BwdPrepSmem<T, DK, NW>::bytes;
-    if (int e = set_lds_b(kern, smem)) return e;
-    GDN_LAUNCH(kKernBwdPrep, st, kern, dim3(nc, d.Hv, d.V / (32 * NW)), dim3(64 * NW), smem, st, qq, kk, AQ,
-               (const T*)dO, G, DVLF, DOF, QSF, KAF, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale);
+    auto kern = chunk_bwd_prep_kernel<T, NW>;
+    GDN_LAUNCH(kKernBwdPrep, st, kern, dim3(nc, d.Hv, d.V / (32 * NW)), dim3(64 * NW), 0, st, AQ, (const T*)dO, DVLF,
+               DOF, cu, chunk_offsets, d.T, d.N, d.Hv, d.V, scale);
   }
   {
     auto kern = chunk_state_bwd_kernel<T, DK, NWS, STAGES>;

@@ -98,7 +98,8 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ g,
     const float* __restrict__ beta, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets,
     float* __restrict__ G_out, T* __restrict__ Ai_out, T* __restrict__ W_out, T* __restrict__ U_out,
-    T* __restrict__ Aq_out, T* __restrict__ KD_out, T* __restrict__ WF_out, int T_len, int N, int Hqk, int Hv, int V) {
+    T* __restrict__ Aq_out, T* __restrict__ KD_out, T* __restrict__ WF_out, T* __restrict__ KA_out,
+    T* __restrict__ QS_out, int T_len, int N, int Hqk, int Hv, int V, float scale) {
   using SM = PrepSmem<T, DK, BV>;
   constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64, VEC = Elem<T>::kVec;
   T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
@@ -146,14 +147,18 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
       mma32<T, DK, true, true>(aq, Qs + 32 * ti * LDK, LDK, Ks + 32 * tj * LDK, LDK);
     }
     const int j = 32 * tj + acc_col();
-    T* aqg = Aq_out + (tok0 * Hv + h) * 64;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int i = 32 * ti + acc_row(r);
       const float gam = i >= j ? __expf(Gs[i] - Gs[j]) : 0.f;
       As[i * kLF + j] = i > j ? bs[i] * acc[r] * gam : 0.f;
-      if (i < nvalid) aqg[(int64_t)i * Hv * 64 + j] = Elem<T>::from_f(aq[r] * gam);
+      aq[r] *= gam;
     }
+    // tril(Q K^T . Gam) leaves as four 32x32 tiles in fragment order, packed as they sit in the accumulator
+    // (lane <-> column j, registers <-> row i): the A operand of Aq^T dO as is, of Aq V' after one turn
+    AccB<T> af;
+    af.pack(aq);
+    af.store(Aq_out + (((int64_t)blockIdx.x * Hv + h) * 4 + wave) * 1024);
   }
   // (e^{G_last-G} . K)^T as A-operand fragments for the state update: K tile fragments (lane <-> token) turned
   // through the matrix core into (lane <-> K column, registers <-> token), scaled per token, stored in fragment order
@@ -163,13 +168,23 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
     const float glast = Gs[63];
     for (int tt = wave; tt < 2 * (DK / 32); tt += 4) {
       const int tj = tt & 1, kt = tt >> 1;
+      const int64_t tile = ((((int64_t)blockIdx.x * Hv + h) * (DK / 32) + kt) * 2 + tj) * 1024;
       AccB<T> kf;
       frags_from_lds<T>(kf, Ks + (32 * tj + (lane & 31)) * LDK + 32 * kt);
+      if (KA_out != nullptr) kf.store(KA_out + tile);   // K as an A operand (lane <-> token), for the backward pass
       f32x16 kd = mfma_transpose<T>(kf, id);
 #pragma unroll
       for (int r = 0; r < 16; ++r) kd[r] *= __expf(glast - Gs[32 * tj + acc_row(r)]);
       kf.pack(kd);
-      kf.store(KD_out + ((((int64_t)blockIdx.x * Hv + h) * (DK / 32) + kt) * 2 + tj) * 1024);
+      kf.store(KD_out + tile);
+      if (QS_out != nullptr) {   // (scale e^G . Q)^T as an A operand (lane <-> K column), for the backward pass
+        frags_from_lds<T>(kf, Qs + (32 * tj + (lane & 31)) * LDK + 32 * kt);
+        f32x16 qt = mfma_transpose<T>(kf, id);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) qt[r] *= scale * __expf(Gs[32 * tj + acc_row(r)]);
+        kf.pack(qt);
+        kf.store(QS_out + tile);
+      }
     }
   }
   __syncthreads();
@@ -518,22 +533,21 @@ __global__ __launch_bounds__(128 * NW) void chunk_state_kernel(
 // S and V' arrive in fragment order and go from global memory straight into B-operand registers.
 // ---------------------------------------------------------------------------------------------
 template <typename T, int DK, int NW> struct OutSmem {
-  static constexpr int LDK = lds_ld<T>(DK), L64 = lds_ld<T>(64);
+  static constexpr int LDK = lds_ld<T>(DK);
   static constexpr int off_qs = 0;
-  static constexpr int off_aq = off_qs + 64 * LDK * (int)sizeof(T);
-  static constexpr int off_eg = off_aq + 64 * L64 * (int)sizeof(T);
+  static constexpr int off_patch = off_qs + 64 * LDK * (int)sizeof(T);
+  static constexpr int off_eg = off_patch + NW * Patch<T>::kElems * (int)sizeof(T);
   static constexpr int bytes = off_eg + 64 * 4;
 };
 
 template <typename T, int DK, int NW>
 __global__ __launch_bounds__(64 * NW) void chunk_out_kernel(
-    const T* __restrict__ q, const T* __restrict__ aqk, const T* __restrict__ vf, const T* __restrict__ hf,
+    const T* __restrict__ q, const T* __restrict__ aqf, const T* __restrict__ vf, const T* __restrict__ hf,
     const float* __restrict__ G, T* __restrict__ o, const int64_t* __restrict__ cu,
     const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V, float scale) {
   using SM = OutSmem<T, DK, NW>;
-  constexpr int LDK = SM::LDK, L64 = SM::L64, NT = 64 * NW, VEC = Elem<T>::kVec, NKT = DK / 32;
+  constexpr int LDK = SM::LDK, NT = 64 * NW, VEC = Elem<T>::kVec, NKT = DK / 32;
   T* Qs = reinterpret_cast<T*>(gdn_smem + SM::off_qs);
-  T* Aq = reinterpret_cast<T*>(gdn_smem + SM::off_aq);
   float* Eg = reinterpret_cast<float*>(gdn_smem + SM::off_eg);
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
@@ -541,24 +555,29 @@ __global__ __launch_bounds__(64 * NW) void chunk_out_kernel(
   const int h = blockIdx.y, hq = h / (Hv / Hqk), nvalid = s.nvalid;
   const int vblk = blockIdx.z * NW + wave, v0 = 32 * vblk;
   const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk;
-  const int64_t tile0 = ((int64_t)blockIdx.x * Hv + h) * (V / 32) + vblk;
+  const int64_t ch = (int64_t)blockIdx.x * Hv + h;
+  const int64_t tile0 = ch * (V / 32) + vblk;
+  T* patch = reinterpret_cast<T*>(gdn_smem + SM::off_patch) + wave * Patch<T>::kElems;
 
-  // operands that come in fragment order are requested first, the LDS tiles while they are in flight
-  AccB<T> Sb[NKT], Vb[2];
+  // operands that come in fragment order are requested first, the LDS tile while they are in flight
+  AccB<T> Sb[NKT], Vb[2], Af[3];
 #pragma unroll
   for (int kt = 0; kt < NKT; ++kt) Sb[kt].load(hf + (tile0 * NKT + kt) * 1024);
   Vb[0].load(vf + tile0 * 2048);
   Vb[1].load(vf + tile0 * 2048 + 1024);
+  Af[0].load(aqf + (ch * 4 + 0) * 1024);   // tiles (0,0), (1,0), (1,1) of tril(Q K^T . Gam)
+  Af[1].load(aqf + (ch * 4 + 2) * 1024);
+  Af[2].load(aqf + (ch * 4 + 3) * 1024);
   for (int c = tid; c < 64 * (DK / VEC); c += NT) {
     const int row = c / (DK / VEC), cc = c % (DK / VEC);
     st16(Qs + row * LDK + cc * VEC,
          row < nvalid ? ld16(q + ((tok0 + row) * Hqk + hq) * DK + cc * VEC) : zero16<T>());
   }
-  for (int c = tid; c < 64 * (64 / VEC); c += NT) {
-    const int row = c / (64 / VEC), cc = c % (64 / VEC);
-    st16(Aq + row * L64 + cc * VEC, row < nvalid ? ld16(aqk + ((tok0 + row) * Hv + h) * 64 + cc * VEC) : zero16<T>());
-  }
   if (tid < 64) Eg[tid] = __expf(G[(tok0 + imin(tid, nvalid - 1)) * Hv + h]);
+  IdentityFrag<T> id;
+  id.init();
+#pragma unroll
+  for (int t = 0; t < 3; ++t) Af[t].pack(mfma_transpose<T>(Af[t], id));   // now (lane <-> row i, registers <-> column j)
   __syncthreads();
 
   T* og = o + (tok0 * Hv + h) * V + v0;
@@ -567,13 +586,14 @@ __global__ __launch_bounds__(64 * NW) void chunk_out_kernel(
     f32x16 oa = acc_zero();
 #pragma unroll
     for (int kt = 0; kt < NKT; ++kt) mma32_accb<T>(oa, Qs + (32 * ri + l32) * LDK + 32 * kt, Sb[kt]);
+    const f32x16 eg = rows_ld(Eg, 32 * ri);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) oa[r] *= Eg[32 * ri + acc_row(r)];
+    for (int r = 0; r < 16; ++r) oa[r] *= eg[r];
 #pragma unroll
-    for (int tj = 0; tj <= ri; ++tj) mma32_accb<T>(oa, Aq + (32 * ri + l32) * L64 + 32 * tj, Vb[tj]);
+    for (int tj = 0; tj <= ri; ++tj) mma32_ff<T>(oa, Af[ri + tj], Vb[tj]);
 #pragma unroll
     for (int r = 0; r < 16; ++r) oa[r] *= scale;
-    acc_to_global(oa, og, (int64_t)Hv * V, 32 * ri, 0, nvalid);
+    acc_store_rows<T, false>(oa, id, patch, og + (int64_t)32 * ri * Hv * V, (int64_t)Hv * V, nvalid - 32 * ri);
   }
 }
 
@@ -613,6 +633,8 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   T* UF = reinterpret_cast<T*>(ws + L.UF);
   T* KDF = reinterpret_cast<T*>(ws + L.KDF);
   T* WF = with_backward ? reinterpret_cast<T*>(ws + L.WF) : nullptr;
+  T* KAF = with_backward ? reinterpret_cast<T*>(ws + L.KAF) : nullptr;
+  T* QSF = with_backward ? reinterpret_cast<T*>(ws + L.QSF) : nullptr;
   T* VF = reinterpret_cast<T*>(ws + L.VF);
   T* HF = reinterpret_cast<T*>(ws + L.HF);
   {
@@ -620,7 +642,7 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     constexpr int smem = PrepSmem<T, DK, BVP>::bytes;
     if (int e = set_lds(kern, smem)) return e;
     GDN_LAUNCH(kKernPrep, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, (const T*)v, g, beta, cu,
-               (const int*)chunk_offsets, G, Ai, W, UF, AQ, KDF, WF, d.T, d.N, d.Hqk, d.Hv, d.V);
+               (const int*)chunk_offsets, G, Ai, W, UF, AQ, KDF, WF, KAF, QSF, d.T, d.N, d.Hqk, d.Hv, d.V, scale);
   }
   {
     auto kern = chunk_state_kernel<T, DK, NWS, STAGES>;
