@@ -110,14 +110,19 @@ def main():
     total_kernel_ms = sum(ms for ms, _ in timings.values()) / args.steps
     flops = kernel_matmul_flops(c["K"], c["V"])
     for name, (ms, cnt) in timings.items():
-        avg = ms / cnt
-        per_kernel[name] = {"avg_ms": round(avg, 4), "share": round(ms / args.steps / total_kernel_ms, 3)}
+        # a kernel launched several times per step (one launch per value head of a q/k group) splits the step's work
+        # evenly over its launches: avg_ms is per launch, step_ms per step
+        launches = cnt / args.steps
+        avg, step_ms = ms / cnt, ms / args.steps
+        per_kernel[name] = {"avg_ms": round(avg, 4), "launches_per_step": round(launches, 2),
+                            "step_ms": round(step_ms, 4), "share": round(step_ms / total_kernel_ms, 3)}
         if name in flops:
-            per_kernel[name]["tflops"] = round(flops[name] * nchunk_heads / (avg * 1e-3) / 1e12, 1)
-    dom = max((n for n in per_kernel if n in flops), key=lambda n: per_kernel[n]["avg_ms"])
-    dom_tflops = flops[dom] * nchunk_heads / (per_kernel[dom]["avg_ms"] * 1e-3) / 1e12
+            per_kernel[name]["tflops"] = round(flops[name] * nchunk_heads / (step_ms * 1e-3) / 1e12, 1)
+    dom = max((n for n in per_kernel if n in flops), key=lambda n: per_kernel[n]["step_ms"])
+    dom_tflops = flops[dom] * nchunk_heads / (per_kernel[dom]["step_ms"] * 1e-3) / 1e12
     roofline = {"kernel": dom, "bound": "mfma", "achieved": round(dom_tflops, 2), "peak": PEAK_BF16_TFLOPS,
-                "unit": "TFLOP/s", "frac": round(dom_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None}
+                "unit": "TFLOP/s", "frac": round(dom_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                "launches_per_step": per_kernel[dom]["launches_per_step"], "avg_launch_ms": per_kernel[dom]["avg_ms"]}
 
     path_tflops = ref_formula_flops(tokens, c["Hv"], c["K"], c["V"]) / (ms_per_step * 1e-3) / 1e12
     aux = {"path_tflops_ref_formula": round(path_tflops, 2),
