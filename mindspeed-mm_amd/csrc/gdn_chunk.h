@@ -19,7 +19,7 @@ struct ChunkDims {
 // Byte offsets into the workspace.  Everything the backward pass re-reads is written by the forward.
 struct ChunkWorkspace {
   int64_t chunk_offsets;  // int32 [N+1]      chunks before each packed sequence
-  int64_t qn, kn;         // T [tokens,Hqk,K] l2-normalised q,k (only with use_qk_l2norm)
+  int64_t qn;             // T [tokens,Hqk,K] l2-normalised q (only with use_qk_l2norm)
   int64_t rstd;           // f32 [2][tokens,Hqk] 1/|q|, 1/|k| of that normalisation
   int64_t G;              // f32 [tokens,Hv]  chunk-local cumulative log decay
   int64_t Ai;             // T [chunks,Hv,2,2]       (I + A)^-1 as A operand: tile = (32 rows) x (32 columns), fragment order
@@ -50,7 +50,6 @@ inline ChunkWorkspace chunk_workspace_layout(const ChunkDims& d, int elem_bytes)
   const int64_t tok = d.tokens(), nc = d.max_chunks();
   w.chunk_offsets = take((int64_t)(d.N + 1) * 4);
   w.qn = take(tok * d.Hqk * d.K * elem_bytes);
-  w.kn = take(tok * d.Hqk * d.K * elem_bytes);
   w.rstd = take(2 * tok * d.Hqk * 4);
   w.G = take(tok * d.Hv * 4);
   w.Ai = take(nc * 64 * d.Hv * 64 * elem_bytes);

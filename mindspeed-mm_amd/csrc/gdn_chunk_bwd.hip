@@ -751,7 +751,7 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   const int nc = (int)d.max_chunks();
   const int* chunk_offsets = reinterpret_cast<const int*>(ws + L.chunk_offsets);
   const T* qq = l2norm ? reinterpret_cast<const T*>(ws + L.qn) : (const T*)q;
-  const T* kk = l2norm ? reinterpret_cast<const T*>(ws + L.kn) : (const T*)k;
+  (void)k;   // k reaches the backward kernels as the forward pass's fragment tiles
   const float* G = reinterpret_cast<const float*>(ws + L.G);
   const T* Ai = reinterpret_cast<const T*>(ws + L.Ai);
   const T* AQ = reinterpret_cast<const T*>(ws + L.AQ);

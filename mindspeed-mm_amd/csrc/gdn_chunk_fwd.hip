@@ -51,28 +51,33 @@ __global__ void chunk_table_kernel(const int64_t* __restrict__ cu, int* __restri
 }
 
 // ---------------------------------------------------------------------------------------------
-// y = x * rsqrt(sum(x^2) + 1e-6) over the last axis (modeling_qwen3_5.py:392-395); rows of DK elements
+// global -> LDS tile load (64 rows x DK columns, rows >= nvalid zero) with the optional in-kernel l2 normalisation
+// y = x * rsqrt(sum(x^2) + 1e-6) over the row (modeling_qwen3_5.py:392-395).  The lanes that share a row are
+// neighbours in a wave and combine their partial sums with data-parallel-primitive moves.  y_out / rstd_out (either may be null) receive
+// the normalised rows and 1/|x| for the kernels that come later.
 // ---------------------------------------------------------------------------------------------
 template <typename T, int DK>
-__global__ void l2norm_fwd_kernel(const T* __restrict__ x0, const T* __restrict__ x1, T* __restrict__ y0,
-                                  T* __restrict__ y1, float* __restrict__ rstd, int64_t rows) {
-  constexpr int V = Elem<T>::kVec, LPR = DK / V;  // lanes per row (a power of two <= 32)
-  const T* x = blockIdx.y == 0 ? x0 : x1;
-  T* y = blockIdx.y == 0 ? y0 : y1;
-  const int64_t row = (int64_t)blockIdx.x * (kThreads / LPR) + threadIdx.x / LPR;
-  const int c = threadIdx.x % LPR;
-  const bool ok = row < rows;
-  Vec16<T> v = ok ? ld16(x + row * DK + c * V) : zero16<T>();
-  float ss = 0.f;
+__device__ __forceinline__ void load_tile_qk(T* lds, int ld, const T* g, int64_t row_stride, int nvalid, int tid,
+                                             bool l2norm, T* y_out, float* rstd_out, int64_t rstd_stride) {
+  constexpr int V = Elem<T>::kVec, CPR = DK / V;   // lanes per row: a power of two <= 32
+  static_assert((64 * CPR) % kThreads == 0, "every thread takes the same number of pieces");
+  for (int c = tid; c < 64 * CPR; c += kThreads) {
+    const int row = c / CPR, cc = c % CPR;
+    const bool ok = row < nvalid;
+    Vec16<T> x = ok ? ld16(g + (int64_t)row * row_stride + cc * V) : zero16<T>();
+    if (l2norm) {   // uniform: every lane takes part in the shuffles
+      float ss = 0.f;
 #pragma unroll
-  for (int e = 0; e < V; ++e) { const float f = v.get(e); ss += f * f; }
+      for (int e = 0; e < V; ++e) { const float f = x.get(e); ss += f * f; }
+      ss = lane_group_sum<CPR>(ss);
+      const float r = rsqrtf(ss + 1e-6f);
 #pragma unroll
-  for (int m = 1; m < LPR; m <<= 1) ss += __shfl_xor(ss, m);
-  const float r = rsqrtf(ss + 1e-6f);
-#pragma unroll
-  for (int e = 0; e < V; ++e) v.set(e, v.get(e) * r);
-  if (ok) st16(y + row * DK + c * V, v);
-  if (ok && c == 0) rstd[blockIdx.y * rows + row] = r;   // kept for the backward pass
+      for (int e = 0; e < V; ++e) x.set(e, x.get(e) * r);
+      if (ok && y_out != nullptr) st16(y_out + (int64_t)row * row_stride + cc * V, x);
+      if (ok && rstd_out != nullptr && cc == 0) rstd_out[(int64_t)row * rstd_stride] = r;
+    }
+    st16(lds + row * ld + cc * V, x);
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -99,7 +104,8 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
     const float* __restrict__ beta, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets,
     float* __restrict__ G_out, T* __restrict__ Ai_out, T* __restrict__ W_out, T* __restrict__ U_out,
     T* __restrict__ Aq_out, T* __restrict__ KD_out, T* __restrict__ WF_out, T* __restrict__ KA_out,
-    T* __restrict__ QS_out, int T_len, int N, int Hqk, int Hv, int V, float scale) {
+    T* __restrict__ QS_out, T* __restrict__ qn_out, float* __restrict__ rstd_q_out, float* __restrict__ rstd_k_out,
+    int T_len, int N, int Hqk, int Hv, int V, float scale, int l2norm) {
   using SM = PrepSmem<T, DK, BV>;
   constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64, VEC = Elem<T>::kVec;
   T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
@@ -134,8 +140,16 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
     if (lane < nvalid) G_out[(tok0 + lane) * Hv + h] = x;
   }
   for (int i = tid; i < 64 * kLF; i += kThreads) Ti[i] = 0.f;
-  load_tile<T, DK>(Ks, LDK, k + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
-  load_tile<T, DK>(Qs, LDK, q + (tok0 * Hqk + hq) * DK, (int64_t)Hqk * DK, nvalid, tid);
+  {
+    // q and k arrive raw; with the in-kernel l2 norm they are normalised on the way into LDS.  The first value head
+    // of each q/k group also leaves the normalised q (for the output kernel and the backward pass) and 1/|q|, 1/|k|.
+    const bool keep = l2norm && (h % (Hv / Hqk)) == 0;
+    const int64_t off = (tok0 * Hqk + hq) * DK, roff = tok0 * Hqk + hq;
+    load_tile_qk<T, DK>(Ks, LDK, k + off, (int64_t)Hqk * DK, nvalid, tid, l2norm != 0, nullptr,
+                        keep ? rstd_k_out + roff : nullptr, Hqk);
+    load_tile_qk<T, DK>(Qs, LDK, q + off, (int64_t)Hqk * DK, nvalid, tid, l2norm != 0, keep ? qn_out + off : nullptr,
+                        keep ? rstd_q_out + roff : nullptr, Hqk);
+  }
   __syncthreads();
 
   // ---- phase 1: A = strict_tril(beta_i k_i.k_j Gam_ij) and Aq = tril(q_i.k_j Gam_ij), one 32x32 tile per wave ----
@@ -615,17 +629,8 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   const T* qq = (const T*)q;
   const T* kk = (const T*)k;
   if (cu != nullptr) GDN_LAUNCH(kKernChunkTable, st, chunk_table_kernel, dim3(1), dim3(kThreads), 0, st, cu, chunk_offsets, d.N);
-  if (l2norm) {
-    constexpr int LPR = DK / Elem<T>::kVec;
-    const int64_t rows = tok * d.Hqk;
-    T* qn = reinterpret_cast<T*>(ws + L.qn);
-    T* kn = reinterpret_cast<T*>(ws + L.kn);
-    GDN_LAUNCH(kKernL2Norm, st, (l2norm_fwd_kernel<T, DK>),
-               dim3((unsigned)((rows + kThreads / LPR - 1) / (kThreads / LPR)), 2), dim3(kThreads), 0, st, qq, kk, qn,
-               kn, reinterpret_cast<float*>(ws + L.rstd), rows);
-    qq = qn;
-    kk = kn;
-  }
+  T* qn = l2norm ? reinterpret_cast<T*>(ws + L.qn) : nullptr;   // normalised q, written by the prep kernel
+  float* rstd = reinterpret_cast<float*>(ws + L.rstd);
   float* G = reinterpret_cast<float*>(ws + L.G);
   T* Ai = reinterpret_cast<T*>(ws + L.Ai);
   T* W = reinterpret_cast<T*>(ws + L.WAF);
@@ -642,7 +647,8 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     constexpr int smem = PrepSmem<T, DK, BVP>::bytes;
     if (int e = set_lds(kern, smem)) return e;
     GDN_LAUNCH(kKernPrep, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, (const T*)v, g, beta, cu,
-               (const int*)chunk_offsets, G, Ai, W, UF, AQ, KDF, WF, KAF, QSF, d.T, d.N, d.Hqk, d.Hv, d.V, scale);
+               (const int*)chunk_offsets, G, Ai, W, UF, AQ, KDF, WF, KAF, QSF, qn, rstd, rstd + tok * d.Hqk, d.T, d.N, d.Hqk,
+               d.Hv, d.V, scale, l2norm);
   }
   {
     auto kern = chunk_state_kernel<T, DK, NWS, STAGES>;
@@ -656,8 +662,8 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     auto kern = chunk_out_kernel<T, DK, NW>;
     constexpr int smem = OutSmem<T, DK, NW>::bytes;
     if (int e = set_lds(kern, smem)) return e;
-    GDN_LAUNCH(kKernOut, st, kern, dim3(nc, d.Hv, d.V / (32 * NW)), dim3(64 * NW), smem, st, qq, (const T*)AQ,
-               (const T*)VF, (const T*)HF, (const float*)G, (T*)o, cu, (const int*)chunk_offsets, d.T, d.N, d.Hqk,
+    GDN_LAUNCH(kKernOut, st, kern, dim3(nc, d.Hv, d.V / (32 * NW)), dim3(64 * NW), smem, st, l2norm ? (const T*)qn : qq,
+               (const T*)AQ, (const T*)VF, (const T*)HF, (const float*)G, (T*)o, cu, (const int*)chunk_offsets, d.T, d.N, d.Hqk,
                d.Hv, d.V, scale);
   }
   return (int)hipGetLastError();

@@ -483,6 +483,16 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
+// sum over aligned groups of N neighbouring lanes (N a power of two <= 32), every lane gets the result
+template <int N> __device__ __forceinline__ float lane_group_sum(float v) {
+  if constexpr (N >= 2) v += dpp_mov<0xB1>(v);
+  if constexpr (N >= 4) v += dpp_mov<0x4E>(v);
+  if constexpr (N >= 8) v += dpp_mov<0x141>(v);
+  if constexpr (N >= 16) v += dpp_mov<0x140>(v);
+  if constexpr (N >= 32) v += __shfl_xor(v, 16);
+  return v;
+}
+
 // Row sums of a 32x32 tile given as per-lane products x[r] (accumulator layout).  A halving butterfly over the 16
 // lanes of a DPP row: at each step a lane keeps the pair sums of the registers whose index bit matches its own lane bit, so 16 sums cost 15 exchanges instead of 64.  Lane l returns the sum over its DPP row of
 // register r = l & 15, i.e. a partial sum (16 of the 32 columns) of tile row acc_row(l & 15).

@@ -6,7 +6,7 @@
 namespace gdn {
 
 enum KernelId {
-  kKernChunkTable = 0, kKernL2Norm, kKernPrep, kKernStateFwd, kKernOut, kKernBwdPrep, kKernStateBwd, kKernBwdLocal,
+  kKernChunkTable = 0, kKernPrep, kKernStateFwd, kKernOut, kKernBwdPrep, kKernStateBwd, kKernBwdLocal,
   kKernRecurrent, kKernConvFwd, kKernConvState, kKernConvBwd, kKernConvReduce,
   kKernConvDh0, kKernConvUpdate, kKernCount
 };
