@@ -72,7 +72,7 @@ __global__ __launch_bounds__(64 * NW) void chunk_bwd_prep_kernel(
       for (int g = 0; g < AccK<T>::kGroups; ++g) f.f[g] = u32x4{0u, 0u, 0u, 0u};
     }
     df[ti].pack(mfma_transpose<T>(f, id));
-    df[ti].store(dof + ((ch * (V / 32) + vblk) * 2 + ti) * 1024);
+    df[ti].store_stream(dof + ((ch * (V / 32) + vblk) * 2 + ti) * 1024);
   }
 #pragma unroll
   for (int rj = 0; rj < 2; ++rj) {          // dv_local[j] = scale sum_{i >= j} Aq[i][j] dO[i]
@@ -83,7 +83,7 @@ __global__ __launch_bounds__(64 * NW) void chunk_bwd_prep_kernel(
     for (int r = 0; r < 16; ++r) acc[r] *= scale;
     AccB<T> out;
     out.pack(acc);
-    out.store(dvlf + ((ch * (V / 32) + vblk) * 2 + rj) * 1024);
+    out.store_stream(dvlf + ((ch * (V / 32) + vblk) * 2 + rj) * 1024);
   }
 }
 
@@ -239,7 +239,7 @@ __global__ __launch_bounds__(128 * NW) void chunk_state_bwd_kernel(
 #pragma unroll
     for (int kt = 0; kt < NKT; ++kt) {
       dSb[kt].pack(dS[kt]);
-      dSb[kt].store(dhf + (tile0 * NKT + kt) * 1024);
+      dSb[kt].store_stream(dhf + (tile0 * NKT + kt) * 1024);
     }
     // dV' = e^{G_last-G} . (K dS) + dv_local
     f32x16 a0 = acc_zero(), a1 = acc_zero();
@@ -262,8 +262,8 @@ __global__ __launch_bounds__(128 * NW) void chunk_state_bwd_kernel(
     }
     dvb[0].pack(a0);
     dvb[1].pack(a1);
-    dvb[0].store(dvf + (tile0 * 2 + 0) * 1024);
-    dvb[1].store(dvf + (tile0 * 2 + 1) * 1024);
+    dvb[0].store_stream(dvf + (tile0 * 2 + 0) * 1024);
+    dvb[1].store_stream(dvf + (tile0 * 2 + 1) * 1024);
     dvb[0].negate();
     dvb[1].negate();
     // dS <- e^{G_last} dS + (scale e^G . Q)^T dO - W^T dV'

@@ -172,7 +172,7 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
     // (lane <-> column j, registers <-> row i): the A operand of Aq^T dO as is, of Aq V' after one turn
     AccB<T> af;
     af.pack(aq);
-    af.store(Aq_out + (((int64_t)blockIdx.x * Hv + h) * 4 + wave) * 1024);
+    af.store_stream(Aq_out + (((int64_t)blockIdx.x * Hv + h) * 4 + wave) * 1024);
   }
   // (e^{G_last-G} . K)^T as A-operand fragments for the state update: K tile fragments (lane <-> token) turned
   // through the matrix core into (lane <-> K column, registers <-> token), scaled per token, stored in fragment order
@@ -185,19 +185,19 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
       const int64_t tile = ((((int64_t)blockIdx.x * Hv + h) * (DK / 32) + kt) * 2 + tj) * 1024;
       AccB<T> kf;
       frags_from_lds<T>(kf, Ks + (32 * tj + (lane & 31)) * LDK + 32 * kt);
-      if (KA_out != nullptr) kf.store(KA_out + tile);   // K as an A operand (lane <-> token), for the backward pass
+      if (KA_out != nullptr) kf.store_stream(KA_out + tile);   // K as an A operand (lane <-> token), for the backward pass
       f32x16 kd = mfma_transpose<T>(kf, id);
 #pragma unroll
       for (int r = 0; r < 16; ++r) kd[r] *= __expf(glast - Gs[32 * tj + acc_row(r)]);
       kf.pack(kd);
-      kf.store(KD_out + tile);
+      kf.store_stream(KD_out + tile);
       if (QS_out != nullptr) {   // (scale e^G . Q)^T as an A operand (lane <-> K column), for the backward pass
         frags_from_lds<T>(kf, Qs + (32 * tj + (lane & 31)) * LDK + 32 * kt);
         f32x16 qt = mfma_transpose<T>(kf, id);
 #pragma unroll
         for (int r = 0; r < 16; ++r) qt[r] *= scale * __expf(Gs[32 * tj + acc_row(r)]);
         kf.pack(qt);
-        kf.store(QS_out + tile);
+        kf.store_stream(QS_out + tile);
       }
     }
   }
@@ -295,7 +295,7 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
   {  // the four 32x32 tiles of Tm as A operands (lane <-> row, registers <-> column), fragment order, for the backward
     AccB<T> tf;
     frags_from_lds<T>(tf, Tms + (32 * (wave >> 1) + (lane & 31)) * L64 + 32 * (wave & 1));
-    tf.store(Ai_out + (((int64_t)blockIdx.x * Hv + h) * 4 + wave) * 1024);
+    tf.store_stream(Ai_out + (((int64_t)blockIdx.x * Hv + h) * 4 + wave) * 1024);
   }
 
   // ---- phase 4: W = Tm (beta e^G K), handed on in fragment order only ----
@@ -309,10 +309,10 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
       const int64_t tile = (((int64_t)blockIdx.x * Hv + h) * (DK / 32) + cj) * 2 + ri;
       AccB<T> wf;
       wf.pack(acc);              // (lane <-> K column, registers <-> token): W^T as an A operand, for the backward pass
-      if (WF_out != nullptr) wf.store(WF_out + tile * 1024);
+      if (WF_out != nullptr) wf.store_stream(WF_out + tile * 1024);
       const f32x16 wt = mfma_transpose<T>(wf, id);
       wf.pack(wt);               // (lane <-> token, registers <-> K column): W as an A operand, for W S
-      wf.store(W_out + tile * 1024);
+      wf.store_stream(W_out + tile * 1024);
     }
   }
   // ---- phase 5: U = Tm (beta V), V block by V block, stored in fragment order ----
@@ -329,7 +329,7 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
       const int vblk = vb * (BV / 32) + cj;
       AccB<T> uf;
       uf.pack(acc);
-      uf.store(U_out + ((((int64_t)blockIdx.x * Hv + h) * (V / 32) + vblk) * 2 + ri) * 1024);
+      uf.store_stream(U_out + ((((int64_t)blockIdx.x * Hv + h) * (V / 32) + vblk) * 2 + ri) * 1024);
     }
   }
 }
@@ -468,7 +468,7 @@ __global__ __launch_bounds__(128 * NW) void chunk_state_kernel(
 #pragma unroll
     for (int kt = 0; kt < NKT; ++kt) {
       Sb[kt].pack(S[kt]);
-      Sb[kt].store(hf + (tile0 * NKT + kt) * 1024);
+      Sb[kt].store_stream(hf + (tile0 * NKT + kt) * 1024);
     }
     // Hand-made software pipeline over pairs of K tiles: the LDS reads of the next group are issued before the
     // matrix instructions of the current one (GDN_SCHED_FENCE keeps the order).
@@ -512,8 +512,8 @@ __global__ __launch_bounds__(128 * NW) void chunk_state_kernel(
     }
     Vb[0].pack(p0);
     Vb[1].pack(p1);
-    Vb[0].store(vf + (tile0 * 2 + 0) * 1024);
-    Vb[1].store(vf + (tile0 * 2 + 1) * 1024);
+    Vb[0].store_stream(vf + (tile0 * 2 + 0) * 1024);
+    Vb[1].store_stream(vf + (tile0 * 2 + 1) * 1024);
     // S <- e^{G_last} S + (e^{G_last - G} . K)^T V'   (K^T arrives already scaled, as A-operand fragments)
     const float eg = __expf(glast);
 #pragma unroll

@@ -46,7 +46,8 @@ template <typename T> __device__ __forceinline__ void store_chan(T* p, const flo
   Vec16<T> v = zero16<T>();
 #pragma unroll
   for (int e = 0; e < Elem<T>::kVec; ++e) v.set(e, src[e]);
-  st16(p, v);
+  // streaming store: outputs are not read again by these kernels, the L2 stays with the sliding input window
+  __builtin_nontemporal_store(v.raw, reinterpret_cast<u32x4*>(p));
 }
 
 // input at flattened position tau for the sequence described by cur (tau may precede the sequence)
