@@ -37,11 +37,14 @@ struct SeqCursor {  // which sequence a flattened token index belongs to
 
 template <typename T, int V> struct ChanVec { float x[V]; };
 
-template <typename T> __device__ __forceinline__ void load_chan(float* dst, const T* p) {
-  const Vec16<T> v = ld16(p);
+template <typename T> __device__ __forceinline__ void unpack_chan(float* dst, const Vec16<T>& v) {
 #pragma unroll
   for (int e = 0; e < Elem<T>::kVec; ++e) dst[e] = v.get(e);
 }
+template <typename T> __device__ __forceinline__ void load_chan(float* dst, const T* p) { unpack_chan(dst, ld16(p)); }
+// tokens whose rows are requested together before any of them is used: a thread walks its channels token by token,
+// and without this only one 16-byte load per thread would be in flight
+constexpr int kConvAhead = 4;
 template <typename T> __device__ __forceinline__ void store_chan(T* p, const float* src) {
   Vec16<T> v = zero16<T>();
 #pragma unroll
@@ -88,31 +91,40 @@ __global__ __launch_bounds__(kConvThreads) void conv1d_fwd_kernel(
   cur.init(cu, N, T_len, t0);
 #pragma unroll
   for (int w = 0; w < W - 1; ++w) load_hist(win[w], x, init, t0 - (W - 1) + w, cur, D, W, d0);
-  for (int64_t t = t0; t < t1; ++t) {
-    if (cur.advance_to(t)) {
+  for (int64_t tb = t0; tb < t1; tb += kConvAhead) {
+    Vec16<T> xr[kConvAhead];
 #pragma unroll
-      for (int w = 0; w < W - 1; ++w) load_hist(win[w], x, init, t - (W - 1) + w, cur, D, W, d0);
+    for (int u = 0; u < kConvAhead; ++u)
+      if (tb + u < t1) xr[u] = ld16(x + (tb + u) * D + d0);
+#pragma unroll
+    for (int u = 0; u < kConvAhead; ++u) {
+      const int64_t t = tb + u;
+      if (t >= t1) break;
+      if (cur.advance_to(t)) {
+#pragma unroll
+        for (int w = 0; w < W - 1; ++w) load_hist(win[w], x, init, t - (W - 1) + w, cur, D, W, d0);
+      }
+      unpack_chan(win[W - 1], xr[u]);
+      float out[V];
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        float a = bs[e];
+#pragma unroll
+        for (int w = 0; w < W; ++w) a += win[w][e] * wgt[w][e];
+        out[e] = silu ? a * sigmoidf_(a) : a;
+      }
+      if (residual != nullptr) {
+        float r[V];
+        load_chan(r, residual + t * D + d0);
+#pragma unroll
+        for (int e = 0; e < V; ++e) out[e] += r[e];
+      }
+      store_chan(y + t * D + d0, out);
+#pragma unroll
+      for (int w = 0; w < W - 1; ++w)
+#pragma unroll
+        for (int e = 0; e < V; ++e) win[w][e] = win[w + 1][e];
     }
-    load_chan(win[W - 1], x + t * D + d0);
-    float out[V];
-#pragma unroll
-    for (int e = 0; e < V; ++e) {
-      float a = bs[e];
-#pragma unroll
-      for (int w = 0; w < W; ++w) a += win[w][e] * wgt[w][e];
-      out[e] = silu ? a * sigmoidf_(a) : a;
-    }
-    if (residual != nullptr) {
-      float r[V];
-      load_chan(r, residual + t * D + d0);
-#pragma unroll
-      for (int e = 0; e < V; ++e) out[e] += r[e];
-    }
-    store_chan(y + t * D + d0, out);
-#pragma unroll
-    for (int w = 0; w < W - 1; ++w)
-#pragma unroll
-      for (int e = 0; e < V; ++e) win[w][e] = win[w + 1][e];
   }
 }
 
@@ -166,7 +178,16 @@ __global__ __launch_bounds__(kConvThreads) void conv1d_bwd_kernel(
 #pragma unroll
   for (int w = 0; w < W - 1; ++w) load_hist(win[w], x, init, t0 - (W - 1) + w, cur, D, W, d0);
   // t runs W-1 steps past the last dyp so that the final dx of the tile are flushed
-  for (int64_t t = t0; t < t1 + (W - 1); ++t) {
+  for (int64_t tb = t0; tb < t1 + (W - 1); tb += kConvAhead) {
+    Vec16<T> xr[kConvAhead], gr[kConvAhead];
+#pragma unroll
+    for (int u = 0; u < kConvAhead; ++u) {
+      if (tb + u < tend) { xr[u] = ld16(x + (tb + u) * D + d0); gr[u] = ld16(dy + (tb + u) * D + d0); }
+    }
+#pragma unroll
+    for (int uu = 0; uu < kConvAhead; ++uu) {
+    const int64_t t = tb + uu;
+    if (t >= t1 + (W - 1)) break;
     // dyw[u] will hold dyp[s+u] for s = t-(W-1); shift in dyp[t]
 #pragma unroll
     for (int w = 0; w < W - 1; ++w)
@@ -177,9 +198,9 @@ __global__ __launch_bounds__(kConvThreads) void conv1d_bwd_kernel(
 #pragma unroll
         for (int w = 0; w < W - 1; ++w) load_hist(win[w], x, init, t - (W - 1) + w, cur, D, W, d0);
       }
-      load_chan(win[W - 1], x + t * D + d0);
+      unpack_chan(win[W - 1], xr[uu]);
       float g[V];
-      load_chan(g, dy + t * D + d0);
+      unpack_chan(g, gr[uu]);
 #pragma unroll
       for (int e = 0; e < V; ++e) {
         if (silu) {
@@ -229,6 +250,7 @@ __global__ __launch_bounds__(kConvThreads) void conv1d_bwd_kernel(
       }
       store_chan(dx + s * D + d0, out);
     }
+  }
   }
   float* pp = part + (int64_t)blockIdx.y * (W + 1) * D;
 #pragma unroll
