@@ -45,8 +45,7 @@ def kernel_matmul_flops(K, V, C=64):
         "chunk_prep_kernel": 2 * g(C, C, K) + g(C, K, C) + g(C, V, C),     # K K^T, Q K^T, Tm (b e^G K), Tm (b V)
         "chunk_state_kernel": g(C, V, K) + g(K, V, C),                     # W S, (decayed K)^T V'
         "chunk_out_kernel": g(C, V, K) + g(C, V, C),                       # Q S, Aq V'
-        "chunk_bwd_prep_kernel": g(C, V, C),                               # Aq^T dO
-        "chunk_state_bwd_kernel": g(C, V, K) + 2 * g(K, V, C),             # K dS, Q^T dO, W^T dV'
+        "chunk_state_bwd_kernel": g(C, V, C) + g(C, V, K) + 2 * g(K, V, C),   # Aq^T dO, K dS, Q^T dO, W^T dV'
         # dO V'^T, dO S^T, V' dS^T, dV' S^T, ds K, ds^T Q | Tm^T dW, dW K^T, Tm^T dV', dV' V^T, dTm Tm^T, Tm^T X, dM K, dM^T K
         "chunk_bwd_local_kernel": g(C, C, V) + 3 * g(C, K, V) + 2 * g(C, K, C)
                                   + g(C, K, C) + g(C, C, K) + g(C, V, C) + g(C, C, V) + 2 * g(C, C, C) + 2 * g(C, K, C),

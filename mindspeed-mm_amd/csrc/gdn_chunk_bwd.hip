@@ -1,6 +1,6 @@
 // Chunked gated delta rule, backward pass.  Notation as in gdn_chunk_fwd.hip; S is the state BEFORE a
 // chunk, dS' the gradient of the state AFTER it, Gam_ij = e^{G_i - G_j}, everything per (sequence, head):
-//   dv_local = scale tril(Q K^T . Gam)^T dO                                   chunk_bwd_prep_kernel
+//   dv_local = scale tril(Q K^T . Gam)^T dO                                   chunk_state_bwd_kernel
 //   dV' = (K dS') . e^{G_last-G} + dv_local                                   chunk_state_bwd_kernel
 //   dS  = e^{G_last} dS' + scale (Q . e^G)^T dO - W^T dV'                       (reverse recurrence)
 //   ds  = scale tril(dO V'^T . Gam);  dQ = scale e^G . (dO S^T) + ds K          chunk_bwd_local_kernel
@@ -35,82 +35,32 @@ __device__ __forceinline__ void acc_rowdot_add(const f32x16& acc, const T* other
 }
 
 // ---------------------------------------------------------------------------------------------
-// chunk_bwd_prep_kernel: what the reverse recurrence needs from dO, written in fragment order (AccB<>) so that the
-// sequential kernel only copies contiguous 16-byte pieces.  One wave per (chunk, head, 32-column V block), no LDS:
-//   DOF   dO as a B operand                         (lane <-> V column, registers <-> token)
-//   DVLF  dv_local = scale Aq^T dO                 (accumulator tiles)
-// dO rows are gathered straight from global memory as A-operand fragments (lane <-> token) and turned through the
-// matrix core; Aq^T tiles are the forward pass's tril(Q K^T . Gam) tiles as stored.
-// ---------------------------------------------------------------------------------------------
-
-template <typename T, int NW>
-__global__ __launch_bounds__(64 * NW) void chunk_bwd_prep_kernel(
-    const T* __restrict__ aqf, const T* __restrict__ dO, T* __restrict__ dvlf, T* __restrict__ dof,
-    const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N, int Hv, int V,
-    float scale) {
-  const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
-  if (s.nvalid <= 0) return;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31;
-  const int h = blockIdx.y, nvalid = s.nvalid;
-  const int vblk = blockIdx.z * NW + wave;
-  const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk;
-  const int64_t ch = (int64_t)blockIdx.x * Hv + h;
-
-  IdentityFrag<T> id;
-  id.init();
-  AccB<T> df[2], aq[3];
-  aq[0].load(aqf + (ch * 4 + 0) * 1024);   // tiles (0,0), (1,0), (1,1)
-  aq[1].load(aqf + (ch * 4 + 2) * 1024);
-  aq[2].load(aqf + (ch * 4 + 3) * 1024);
-#pragma unroll
-  for (int ti = 0; ti < 2; ++ti) {
-    const int row = 32 * ti + l32;
-    AccB<T> f;
-    frags_from_lds<T>(f, dO + ((tok0 + imin(row, nvalid - 1)) * Hv + h) * V + 32 * vblk);
-    if (row >= nvalid) {
-#pragma unroll
-      for (int g = 0; g < AccK<T>::kGroups; ++g) f.f[g] = u32x4{0u, 0u, 0u, 0u};
-    }
-    df[ti].pack(mfma_transpose<T>(f, id));
-    df[ti].store_stream(dof + ((ch * (V / 32) + vblk) * 2 + ti) * 1024);
-  }
-#pragma unroll
-  for (int rj = 0; rj < 2; ++rj) {          // dv_local[j] = scale sum_{i >= j} Aq[i][j] dO[i]
-    f32x16 acc = acc_zero();
-#pragma unroll
-    for (int ti = rj; ti < 2; ++ti) mma32_ff<T>(acc, aq[ti + rj], df[ti]);
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] *= scale;
-    AccB<T> out;
-    out.pack(acc);
-    out.store_stream(dvlf + ((ch * (V / 32) + vblk) * 2 + rj) * 1024);
-  }
-}
-
-// ---------------------------------------------------------------------------------------------
 // chunk_state_bwd_kernel: the reverse recurrence, mirror of chunk_state_kernel.  One compute wave owns a 32-column
 // slab of dS[K, 32] in fp32 accumulators and per chunk (last to first) does
 //     dV' = e^{G_last-G} . (K dS) + dv_local          dS <- e^{G_last} dS + (scale e^G . Q)^T dO - W^T dV'
 // with dS and dV' used as B operands straight from accumulator registers.  dS (gradient of the state AFTER the
-// chunk) and dV' leave in fragment order.  Loader waves copy the A operands (K, Q^T, W^T: `big` stages) and the
-// per-slab dv_local / dO fragments (`small` stage) from contiguous fragment-order blocks.
+// chunk) and dV' leave in fragment order.  Loader waves copy the A operands (K, Q^T, W^T: `big` stages) from
+// contiguous fragment-order blocks, and the `small` stage: the slab's dO rows as they lie in memory plus the
+// forward pass's tril(Q K^T . Gam) tiles, from which the compute waves form dv_local = scale Aq^T dO themselves.
 // ---------------------------------------------------------------------------------------------
 template <typename T, int DK, int NW, int STAGES> struct StateBwdSmem {
   static constexpr int big = 3 * 64 * DK * (int)sizeof(T) + 64 * 4 + 16;   // K, Q^T, W^T images, decay[64], G_last
-  static constexpr int off_small = STAGES * big;
-  static constexpr int bytes = off_small + 2 * NW * 2048 * (int)sizeof(T);
+  static constexpr int off_small = STAGES * big;            // dO rows of the slab [64][32 NW] | tril(Q K^T . Gam) tiles [4]
+  static constexpr int bytes = off_small + (NW * 2048 + 4096) * (int)sizeof(T);
 };
 
 template <typename T, int DK, int NW, int STAGES>
 __global__ __launch_bounds__(128 * NW) void chunk_state_bwd_kernel(
-    const T* __restrict__ kaf, const T* __restrict__ qsf, const T* __restrict__ wf, const T* __restrict__ dvlf,
-    const T* __restrict__ dof, const float* __restrict__ G, const float* __restrict__ dht, float* __restrict__ dh0,
+    const T* __restrict__ kaf, const T* __restrict__ qsf, const T* __restrict__ wf, const T* __restrict__ aqf,
+    const T* __restrict__ dO, const float* __restrict__ G, const float* __restrict__ dht, float* __restrict__ dh0,
     T* __restrict__ dvf, T* __restrict__ dhf, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets,
-    int T_len, int Hv, int V) {
+    int T_len, int Hv, int V, float scale) {
   using SM = StateBwdSmem<T, DK, NW, STAGES>;
   constexpr int NT = 64 * NW, VEC = Elem<T>::kVec, NKT = DK / 32;
-  constexpr int CW = 64 * (DK / VEC) / NT, CUL = NW * 2048 / VEC / NT, TILE = 64 * DK;
-  static_assert(64 * (DK / VEC) % NT == 0 && (NW * 2048 / VEC) % NT == 0, "tile chunks must divide over the loaders");
+  constexpr int CW = 64 * (DK / VEC) / NT, CUL = NW * 2048 / VEC / NT, CAQ = 4096 / VEC / NT, TILE = 64 * DK;
+  constexpr int PPR = 32 * NW / VEC;   // 16-byte pieces per dO row of the slab
+  static_assert(64 * (DK / VEC) % NT == 0 && (NW * 2048 / VEC) % NT == 0 && (4096 / VEC) % NT == 0,
+                "tile chunks must divide over the loaders");
   static_assert(STAGES == 1 || STAGES == 2, "one or two big LDS stages");
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -119,14 +69,14 @@ __global__ __launch_bounds__(128 * NW) void chunk_state_bwd_kernel(
   const int len = cu ? (int)(cu[n + 1] - bos) : T_len;
   const int nchunks = (len + kChunk - 1) / kChunk;
   const int64_t chunk_base = cu ? chunk_offsets[n] : (int64_t)n * ((T_len + kChunk - 1) / kChunk);
-  T* small = reinterpret_cast<T*>(gdn_smem + SM::off_small);   // [dv_local | dO], NW slabs x 2 tiles each
+  T* small = reinterpret_cast<T*>(gdn_smem + SM::off_small);   // dO rows of the slab, row-major | Aq tiles
 
   // step s = 0 .. nchunks-1 handles chunk nchunks-1-s
   if (wave >= NW) {
     // ================= loader waves =================
     const int lt = tid - NT;
     constexpr int DEPTH = (STAGES == 2) ? 2 : 1;
-    Vec16<T> pk[DEPTH][CW], pq[DEPTH][CW], pw[DEPTH][CW], pl[DEPTH][CUL], pd[DEPTH][CUL];
+    Vec16<T> pk[DEPTH][CW], pq[DEPTH][CW], pw[DEPTH][CW], pa[DEPTH][CAQ], pd[DEPTH][CUL];
     float pdec[DEPTH], pgl[DEPTH];
     auto issue = [&](int st, int set) {
       const int c = nchunks - 1 - st;
@@ -140,11 +90,13 @@ __global__ __launch_bounds__(128 * NW) void chunk_state_bwd_kernel(
         pq[set][i] = ld16(qsf + ch * TILE + id * VEC);
         pw[set][i] = ld16(wf + ch * TILE + id * VEC);
       }
-      const int64_t sl = (ch * (V / 32) + blockIdx.y * NW) * 2048;
 #pragma unroll
-      for (int i = 0; i < CUL; ++i) {
-        pl[set][i] = ld16(dvlf + sl + (lt + i * NT) * VEC);
-        pd[set][i] = ld16(dof + sl + (lt + i * NT) * VEC);
+      for (int i = 0; i < CAQ; ++i) pa[set][i] = ld16(aqf + ch * 4096 + (lt + i * NT) * VEC);
+#pragma unroll
+      for (int i = 0; i < CUL; ++i) {   // dO rows of this slab, 16-byte pieces; rows past the end are zero
+        const int p = lt + i * NT, row = p / PPR, cc = p % PPR;
+        pd[set][i] = row < nvalid ? ld16(dO + ((tok0 + row) * Hv + h) * V + blockIdx.y * (32 * NW) + cc * VEC)
+                                  : zero16<T>();
       }
       pgl[set] = G[(tok0 + nvalid - 1) * Hv + h];
       pdec[set] = __expf(pgl[set] - G[(tok0 + imin(lt & 63, nvalid - 1)) * Hv + h]);
@@ -167,10 +119,9 @@ __global__ __launch_bounds__(128 * NW) void chunk_state_bwd_kernel(
     };
     auto commit_small = [&](int set) {
 #pragma unroll
-      for (int i = 0; i < CUL; ++i) {
-        st16(small + (lt + i * NT) * VEC, pl[set][i]);
-        st16(small + NW * 2048 + (lt + i * NT) * VEC, pd[set][i]);
-      }
+      for (int i = 0; i < CUL; ++i) st16(small + (lt + i * NT) * VEC, pd[set][i]);
+#pragma unroll
+      for (int i = 0; i < CAQ; ++i) st16(small + NW * 2048 + (lt + i * NT) * VEC, pa[set][i]);
     };
     if (STAGES == 2) {
       if (nchunks > 0) { issue(0, 0); commit_big(0, 0); commit_small(0); }
@@ -184,7 +135,7 @@ __global__ __launch_bounds__(128 * NW) void chunk_state_bwd_kernel(
           if (st < nchunks) {
             GDN_LDS_BARRIER();              // (A) step st staged
             if (st + 1 < nchunks) commit_big((u + 1) % DEPTH, (st + 1) & 1);
-            GDN_LDS_BARRIER();              // (B) the compute waves have taken their dv_local / dO fragments
+            GDN_LDS_BARRIER();              // (B) the compute waves have taken their dO rows and formed dv_local
             if (st + 1 < nchunks) {
               commit_small((u + 1) % DEPTH);
               if (st + 1 + DEPTH < nchunks) issue(st + 1 + DEPTH, (u + 1) % DEPTH);
@@ -207,6 +158,8 @@ __global__ __launch_bounds__(128 * NW) void chunk_state_bwd_kernel(
 
   // ================= compute waves =================
   const int vblk = blockIdx.y * NW + wave, v0 = 32 * vblk;
+  IdentityFrag<T> id;
+  id.init();
   f32x16 dS[NKT];
 #pragma unroll
   for (int kt = 0; kt < NKT; ++kt) {
@@ -221,12 +174,24 @@ __global__ __launch_bounds__(128 * NW) void chunk_state_bwd_kernel(
     const int c = nchunks - 1 - st;
     const int buf = (STAGES == 2) ? (st & 1) : 0;
     GDN_LDS_BARRIER();                      // (A)
-    AccB<T> dvl[2], dob[2];
-    dvl[0].load(small + wave * 2048);
-    dvl[1].load(small + wave * 2048 + 1024);
-    dob[0].load(small + NW * 2048 + wave * 2048);
-    dob[1].load(small + NW * 2048 + wave * 2048 + 1024);
+    // dO of this wave's 32 columns as B operand (lane <-> V column, registers <-> token), turned from the row-major
+    // rows through the matrix core; dv_local = scale tril(Q K^T . Gam)^T dO from the forward pass's accumulator tiles
+    AccB<T> dob[2], aq[3];
+    f32x16 dvl[2];
+    frags_from_lds<T>(dob[0], small + (lane & 31) * (32 * NW) + 32 * wave);
+    frags_from_lds<T>(dob[1], small + (32 + (lane & 31)) * (32 * NW) + 32 * wave);
+    aq[0].load(small + NW * 2048);            // tiles (0,0), (1,0), (1,1)
+    aq[1].load(small + NW * 2048 + 2048);
+    aq[2].load(small + NW * 2048 + 3072);
     GDN_LDS_BARRIER();                      // (B)
+    dob[0].pack(mfma_transpose<T>(dob[0], id));
+    dob[1].pack(mfma_transpose<T>(dob[1], id));
+#pragma unroll
+    for (int rj = 0; rj < 2; ++rj) {
+      dvl[rj] = acc_zero();
+#pragma unroll
+      for (int ti = rj; ti < 2; ++ti) mma32_ff<T>(dvl[rj], aq[ti + rj], dob[ti]);
+    }
     unsigned char* base = gdn_smem + buf * SM::big;
     const T* Ka = reinterpret_cast<const T*>(base);
     const T* Qa = Ka + TILE;
@@ -253,11 +218,10 @@ __global__ __launch_bounds__(128 * NW) void chunk_state_bwd_kernel(
     }
     AccB<T> dvb[2];
     {
-      const f32x16 l0 = dvl[0].unpack(), l1 = dvl[1].unpack();
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        a0[r] = a0[r] * dec[acc_row(r)] + l0[r];
-        a1[r] = a1[r] * dec[32 + acc_row(r)] + l1[r];
+        a0[r] = a0[r] * dec[acc_row(r)] + scale * dvl[0][r];
+        a1[r] = a1[r] * dec[32 + acc_row(r)] + scale * dvl[1][r];
       }
     }
     dvb[0].pack(a0);
@@ -314,8 +278,8 @@ __global__ __launch_bounds__(128 * NW) void chunk_state_bwd_kernel(
 //   dQ, dK, dv leave as 16-byte row pieces.
 // ---------------------------------------------------------------------------------------------
 template <typename T, int DK> struct BwdLocalSmem {
-  // one stage, in elements: [v_new x2 | dV' x2 | dO x2] shared tiles, [S | dS'] per wave, raw V [64][32]
-  static constexpr int st_priv = 6 * 1024, st_vraw = st_priv + 4 * 2048, stage_elems = st_vraw + 64 * 32;
+  // one stage, in elements: [v_new x2 | dV' x2] shared tiles, raw dO [64][32], [S | dS'] per wave, raw V [64][32]
+  static constexpr int st_doraw = 4 * 1024, st_priv = 6 * 1024, st_vraw = st_priv + 4 * 2048, stage_elems = st_vraw + 64 * 32;
   // epilogue, stage that idles during the last block: K tiles [K/32][2] | Q columns of each wave [64][32]
   static constexpr int ea_q = 8 * 1024;
   // epilogue, other stage: dW tiles [2][K/32] (later the store patches) | D-form tiles [4] | T-form tiles [4]
@@ -331,7 +295,7 @@ template <typename T, int DK>
 __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_local_kernel(
     const T* __restrict__ q, const T* __restrict__ kaf, const T* __restrict__ v, const float* __restrict__ beta,
     const float* __restrict__ G, const T* __restrict__ Ai, const T* __restrict__ vf, const T* __restrict__ dvf,
-    const T* __restrict__ dof, const T* __restrict__ hf, const T* __restrict__ dhf, const float* __restrict__ rstd_q,
+    const T* __restrict__ dO, const T* __restrict__ hf, const T* __restrict__ dhf, const float* __restrict__ rstd_q,
     const float* __restrict__ rstd_k, T* dq, T* dk, T* __restrict__ dv_out, float* __restrict__ dbeta,
     float* __restrict__ dg, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N,
     int Hqk, int Hv, int V, float scale, int hh) {
@@ -375,17 +339,18 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     T* st = stage0 + buf * SM::stage_elems;
     const int64_t t2 = (ch * nblk + vblk) * 2, tk = (ch * nblk + vblk) * NKT;
 #pragma unroll
-    for (int j = 0; j < 6 * KG / 4; ++j) {           // shared tiles: k-group pieces dealt round-robin to the waves
+    for (int j = 0; j < 4 * KG / 4; ++j) {           // shared tiles: k-group pieces dealt round-robin to the waves
       const int piece = 4 * j + wave, tile = piece / KG, g = piece % KG;
-      const T* src = tile < 2 ? vf + (t2 + tile) * 1024 : tile < 4 ? dvf + (t2 + tile - 2) * 1024 : dof + (t2 + tile - 4) * 1024;
+      const T* src = tile < 2 ? vf + (t2 + tile) * 1024 : dvf + (t2 + tile - 2) * 1024;
       load16_to_lds(src + (g * 64 + lane) * VEC, st + tile * 1024 + g * 64 * VEC);
     }
 #pragma unroll
-    for (int j = 0; j < (int)sizeof(T) / 2; ++j) {   // raw V block [64][32], rows past the end repeat the last row
+    for (int j = 0; j < (int)sizeof(T) / 2; ++j) {   // raw dO and V blocks [64][32], rows past the end repeat the last row
       constexpr int LPR = 32 / VEC, RPP = 64 / LPR;  // lanes per row, rows per piece
       const int piece = 4 * j + wave, row = piece * RPP + lane / LPR, cc = lane % LPR;
-      load16_to_lds(v + ((tok0 + imin(row, nvalid - 1)) * Hv + h) * V + 32 * vblk + cc * VEC,
-                    st + SM::st_vraw + piece * 64 * VEC);
+      const int64_t off = ((tok0 + imin(row, nvalid - 1)) * Hv + h) * V + 32 * vblk + cc * VEC;
+      load16_to_lds(dO + off, st + SM::st_doraw + piece * 64 * VEC);
+      load16_to_lds(v + off, st + SM::st_vraw + piece * 64 * VEC);
     }
     if (has_k) {
 #pragma unroll
@@ -490,9 +455,12 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       for (int r = 0; r < 16; ++r) sds += sv[r] * dsv[r];
     }
 #pragma unroll
-    for (int ri = 0; ri < 2; ++ri) {         // (lane <-> token, registers <-> V) from here on
-      f.load(st + (4 + ri) * 1024);
-      dOt[ri].pack(mfma_transpose<T>(f, id));
+    for (int ri = 0; ri < 2; ++ri) {         // (lane <-> token, registers <-> V) from here on; dO rows have it already
+      frags_from_lds<T>(dOt[ri], st + SM::st_doraw + (32 * ri + l32) * 32);
+      if (32 * ri + l32 >= nvalid) {
+#pragma unroll
+        for (int g = 0; g < KG; ++g) dOt[ri].f[g] = u32x4{0u, 0u, 0u, 0u};
+      }
       if (has_k) mma32_ff<T>(dQi[ri], dOt[ri], Sf);
     }
 #pragma unroll
@@ -760,24 +728,16 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   const T* HF = reinterpret_cast<const T*>(ws + L.HF);
   const T* QSF = reinterpret_cast<const T*>(ws + L.QSF);
   const T* KAF = reinterpret_cast<const T*>(ws + L.KAF);
-  T* DVLF = reinterpret_cast<T*>(ws + L.DVLF);
-  T* DOF = reinterpret_cast<T*>(ws + L.DOF);
   T* DVF = reinterpret_cast<T*>(ws + L.DVF);
   T* DHF = reinterpret_cast<T*>(ws + L.DHF);
   const float* rstd_q = l2norm ? reinterpret_cast<const float*>(ws + L.rstd) : nullptr;
   const float* rstd_k = l2norm ? rstd_q + tok * d.Hqk : nullptr;
   {
-    auto kern = chunk_bwd_prep_kernel<T, NW>;
-    GDN_LAUNCH(kKernBwdPrep, st, kern, dim3(nc, d.Hv, d.V / (32 * NW)), dim3(64 * NW), 0, st, AQ, (const T*)dO, DVLF,
-               DOF, cu, chunk_offsets, d.T, d.N, d.Hv, d.V, scale);
-  }
-  {
     auto kern = chunk_state_bwd_kernel<T, DK, NWS, STAGES>;
     constexpr int smem = StateBwdSmem<T, DK, NWS, STAGES>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
     GDN_LAUNCH(kKernStateBwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NWS)), dim3(128 * NWS), smem, st, (const T*)KAF,
-               (const T*)QSF, WF, (const T*)DVLF, (const T*)DOF, G, dht, dh0, DVF, DHF, cu, chunk_offsets, d.T, d.Hv,
-               d.V);
+               (const T*)QSF, WF, AQ, (const T*)dO, G, dht, dh0, DVF, DHF, cu, chunk_offsets, d.T, d.Hv, d.V, scale);
   }
   {
     auto kern = chunk_bwd_local_kernel<T, DK>;
@@ -785,7 +745,7 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     if (int e = set_lds_b(kern, smem)) return e;
     for (int hh = 0; hh < d.Hv / d.Hqk; ++hh)
       GDN_LAUNCH(kKernBwdLocal, st, kern, dim3(nc, d.Hqk), dim3(kThreads), smem, st, qq, (const T*)KAF, (const T*)v,
-                 beta, G, Ai, VF, (const T*)DVF, (const T*)DOF, HF, (const T*)DHF, rstd_q, rstd_k, (T*)dq, (T*)dk,
+                 beta, G, Ai, VF, (const T*)DVF, (const T*)dO, HF, (const T*)DHF, rstd_q, rstd_k, (T*)dq, (T*)dk,
                  (T*)dv, dbeta, dg, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale, hh);
   }
   return (int)hipGetLastError();

@@ -6,7 +6,7 @@
 namespace gdn {
 
 enum KernelId {
-  kKernChunkTable = 0, kKernPrep, kKernStateFwd, kKernOut, kKernBwdPrep, kKernStateBwd, kKernBwdLocal,
+  kKernChunkTable = 0, kKernPrep, kKernStateFwd, kKernOut, kKernStateBwd, kKernBwdLocal,
   kKernRecurrent, kKernConvFwd, kKernConvState, kKernConvBwd, kKernConvReduce,
   kKernConvDh0, kKernConvUpdate, kKernCount
 };

@@ -10,7 +10,7 @@ namespace gdn {
 
 static const char* const kNames[kKernCount] = {
     "chunk_table_kernel", "chunk_prep_kernel", "chunk_state_kernel", "chunk_out_kernel",
-    "chunk_bwd_prep_kernel", "chunk_state_bwd_kernel", "chunk_bwd_local_kernel",
+    "chunk_state_bwd_kernel", "chunk_bwd_local_kernel",
     "recurrent_kernel", "conv1d_fwd_kernel", "conv1d_final_state_kernel",
     "conv1d_bwd_kernel", "conv1d_reduce_kernel", "conv1d_dh0_kernel", "conv1d_update_kernel"};
 
