@@ -8,9 +8,10 @@ A step is one chunked gated-delta-rule forward + backward over the configuration
 initial state, upstream grad ~ N(0,1)); inputs are synthetic and already resident in HBM.  Prints ONE JSON line.
 
   value        tokens/s of fwd+bwd (B*T / step time), measured without per-kernel instrumentation
-  roofline     the kernel with the largest share of the step: its algorithmic matmul FLOP per launch divided by
-               its mean duration, taken live with HIP events on the launch stream in a second, instrumented
-               pass over the same K steps; peak = MI355X dense bf16 MFMA (2.5 PFLOP/s)
+  roofline     the kernel with the largest share of the step: its algorithmic HBM bytes per launch divided by its
+               mean launch duration, taken live with HIP events on the launch stream in a second, instrumented
+               pass over the same K steps; peak = MI355X HBM3E (8 TB/s).  Its matmul FLOP rate against the dense
+               bf16 MFMA peak (2.5 PFLOP/s) is given beside it
   cpu_baseline the CPU oracle (PyTorch fp32 restatement of the reference's torch path, autograd backward) timed on
                this box's host cores on a bounded sample of the same workload
   aux          the whole path against the MFMA peak with the reference's FLOP formula, the per-kernel split,
@@ -32,6 +33,14 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 CFG = dict(B=2, T=8192, Hqk=16, Hv=32, K=128, V=128, C=64)
 
+# HBM bytes per launch of each kernel on CFG, read + written, from the hardware counters FETCH_SIZE and WRITE_SIZE
+# (rocprofv3 --pmc, one run per counter, each scaled by what the same counter reads for a 512 MiB copy): the figures
+# of profiles/chunk_fwd_bwd_B2_T8192_bf16_hbm_traffic.md.  Measured offline, reported beside the live timings.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
+    "chunk_prep_kernel": 1328035405, "chunk_state_kernel": 814496928, "chunk_out_kernel": 675852621,
+    "chunk_state_bwd_kernel": 1032402399, "chunk_bwd_local_kernel": 1265262731,
+}
+
 
 def ref_formula_flops(tokens, Hv, K, V, C=64):
     """fwd+bwd FLOP of the reference's own counter (mindspeed_mm/fsdp/tools/flops_tool/flops_qwen3_5.py:170-204)."""
@@ -52,6 +61,24 @@ def kernel_matmul_flops(K, V, C=64):
     }
 
 
+def kernel_algorithmic_bytes(K, V, grp, e=2, C=64):
+    """HBM bytes each kernel has to move per (chunk, value head) given its interface: every input tile read once, every
+    output tile written once (bf16 tiles, fp32 row vectors).  tk = [64,K] tile, tv = [64,V] tile, st = [K,V] state,
+    cc = [64,64] tile, row = 64 fp32 values."""
+    tk, tv, st, cc, row = C * K * e, C * V * e, K * V * e, C * C * e, C * 4
+    return {
+        # q, k, v, g, beta -> G, Tm, W, U, Aq, decayed K^T, W^T, K, scaled Q^T tiles, normalised q and 1/|q|, 1/|k| once per group
+        "chunk_prep_kernel": 2 * tk + tv + 2 * row + row + 2 * cc + tk + tv + tk + 3 * tk + (tk + 2 * row) // grp,
+        "chunk_state_kernel": 2 * tk + tv + row + tv + st,          # W, decayed K^T, U, G -> v_new, state before the chunk
+        "chunk_out_kernel": tk + cc + tv + st + row + tv,            # q, Aq, v_new, state, G -> o
+        "chunk_state_bwd_kernel": 3 * tk + cc + tv + row + tv + st,  # K, Q^T, W^T, Aq, dO, G -> dv_new, dS
+        # v_new, dv_new, dO, S, dS, v, K, q, Tm, row vectors -> dv, dg, dbeta, dq/dk (written by the first head of a
+        # group, read and re-written by the others)
+        "chunk_bwd_local_kernel": 3 * tv + 2 * st + tv + 2 * tk + cc + 5 * row + tv + 2 * row
+                                  + 2 * tk * (2 * grp - 1) // grp,
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -59,6 +86,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side oracle timing")
     ap.add_argument("--no-aux", action="store_true", help="skip the decode / conv1d side measurements")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a 512 MiB device-to-device copy a few times (a kernel of known traffic for scaling "
+                         "hardware counters collected over this command)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the operator path has no collective and this build runs on a single "
@@ -117,11 +147,23 @@ def main():
                             "step_ms": round(step_ms, 4), "share": round(step_ms / total_kernel_ms, 3)}
         if name in flops:
             per_kernel[name]["tflops"] = round(flops[name] * nchunk_heads / (step_ms * 1e-3) / 1e12, 1)
-    dom = max((n for n in per_kernel if n in flops), key=lambda n: per_kernel[n]["step_ms"])
+    abytes = kernel_algorithmic_bytes(c["K"], c["V"], c["Hv"] // c["Hqk"])
+    for name in per_kernel:
+        if name in abytes:
+            per_kernel[name]["GBps"] = round(abytes[name] * nchunk_heads / (per_kernel[name]["step_ms"] * 1e-3) / 1e9, 1)
+    # The dominant kernel's arithmetic intensity (matmul FLOP / algorithmic byte) is far below the ridge of the machine
+    # (2.5 PFLOP/s / 8 TB/s = 312 FLOP/B), like that of every kernel of the path: the roofline that bounds it is HBM.
+    dom = max((n for n in per_kernel if n in abytes), key=lambda n: per_kernel[n]["step_ms"])
+    launches = per_kernel[dom]["launches_per_step"]
+    bytes_per_launch = abytes[dom] * nchunk_heads / launches
+    dom_gbps = bytes_per_launch / (per_kernel[dom]["avg_ms"] * 1e-3) / 1e9
     dom_tflops = flops[dom] * nchunk_heads / (per_kernel[dom]["step_ms"] * 1e-3) / 1e12
-    roofline = {"kernel": dom, "bound": "mfma", "achieved": round(dom_tflops, 2), "peak": PEAK_BF16_TFLOPS,
-                "unit": "TFLOP/s", "frac": round(dom_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None,
-                "launches_per_step": per_kernel[dom]["launches_per_step"], "avg_launch_ms": per_kernel[dom]["avg_ms"]}
+    roofline = {"kernel": dom, "bound": "hbm", "achieved": round(dom_gbps, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": round(dom_gbps / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(dom),
+                "algorithmic_bytes_per_launch": int(bytes_per_launch), "launches_per_step": launches,
+                "avg_launch_ms": per_kernel[dom]["avg_ms"],
+                "flop_per_byte": round(flops[dom] / abytes[dom], 1), "tflops": round(dom_tflops, 1),
+                "frac_of_bf16_mfma_peak": round(dom_tflops / PEAK_BF16_TFLOPS, 4)}
 
     path_tflops = ref_formula_flops(tokens, c["Hv"], c["K"], c["V"]) / (ms_per_step * 1e-3) / 1e12
     aux = {"path_tflops_ref_formula": round(path_tflops, 2),
@@ -182,6 +224,14 @@ def main():
         aux["conv1d_packed"] = {"fwd_ms": round(f_s * 1e3, 3), "fwd_GBps": round(2 * nb / f_s / 1e9, 1),
                                 "bwd_ms": round(b_s * 1e3, 3), "bwd_GBps": round(3 * nb / b_s / 1e9, 1)}
         del xx, ww, dy
+
+    if args.calibrate_copy:
+        src = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     cpu = None
     if not args.no_cpu_baseline:
