@@ -21,19 +21,6 @@
 
 namespace gdn {
 
-// for every accumulator row i of the tile: rowacc[i0+i] += factor * sum_j acc[i][j] * other[(i0+i)*ld + j0+j]
-template <typename T>
-__device__ __forceinline__ void acc_rowdot_add(const f32x16& acc, const T* other, int ld, int i0, int j0, float* rowacc,
-                                               float factor) {
-  const int j = j0 + acc_col();
-#pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int i = i0 + acc_row(r);
-    const float s = row16_sum(acc[r] * Elem<T>::to_f(other[i * ld + j]));
-    if ((threadIdx.x & 15) == 0) atomicAdd(&rowacc[i], factor * s);
-  }
-}
-
 // ---------------------------------------------------------------------------------------------
 // chunk_state_bwd_kernel: the reverse recurrence, mirror of chunk_state_kernel.  One compute wave owns a 32-column
 // slab of dS[K, 32] in fp32 accumulators and per chunk (last to first) does
@@ -286,7 +273,7 @@ template <typename T, int DK> struct BwdLocalSmem {
   static constexpr int eb_d = 8 * 1024, eb_t = 12 * 1024;
   static constexpr int off_tm = 2 * stage_elems * (int)sizeof(T);             // Tm tiles [2][2], whole kernel
   static constexpr int off_row = off_tm + 4 * 1024 * (int)sizeof(T);
-  static constexpr int bytes = off_row + (11 * 64 + 8) * 4;
+  static constexpr int bytes = off_row + (5 * 64 + 5 * 256 + 8) * 4;   // 5 row vectors, 5 per-wave row-sum arrays
   static_assert(stage_elems == 16 * 1024, "the epilogue layout fills a stage exactly");
   static_assert(Patch<T>::kElems <= 2048, "store patches fit");
 };
@@ -307,14 +294,15 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_row);
   float* egs = Gs + 64;    // e^G
   float* bs = egs + 64;    // beta
-  float* rq = bs + 64;     // <q_i, dQ_i>
-  float* rk1 = rq + 64;    // <k_i, dK_i> before the terms that come back through W
-  float* rbk = rk1 + 64;   // e^G <P_i,k_i> + <E_i,k_i>: dbeta without the V part; times beta it is part of dG and <k,dK>
-  float* rf = rbk + 64;    // <F_i, k_i>
-  float* rv = rf + 64;     // <R_i, v_i>
-  float* rsq = rv + 64;    // 1/|q_i|, 1/|k_i| of the l2 normalisation (1 without it)
+  float* rsq = bs + 64;    // 1/|q_i|, 1/|k_i| of the l2 normalisation (1 without it)
   float* rsk = rsq + 64;
-  float* wsum = rsk + 64;  // per wave: <S,dS'> [0..3], sum_i <k_i, dK_inter_i> [4..7]
+  // row sums, one slot of 64 rows per wave (see rows_add):
+  float* rq = rsk + 64;    // <q_i, dQ_i>
+  float* rk1 = rq + 256;   // <k_i, dK_i> before the terms that come back through W
+  float* rbk = rk1 + 256;  // e^G <P_i,k_i> + <E_i,k_i>: dbeta without the V part; times beta it is part of dG and <k,dK>
+  float* rf = rbk + 256;   // <F_i, k_i>
+  float* rv = rf + 256;    // <R_i, v_i>
+  float* wsum = rv + 256;  // per wave: <S,dS'> [0..3], sum_i <k_i, dK_inter_i> [4..7]
 
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
@@ -389,10 +377,10 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     Gs[tid] = gv;
     egs[tid] = __expf(gv);
     bs[tid] = tid < nvalid ? beta[(tok0 + tid) * Hv + h] : 0.f;
-    rq[tid] = 0.f; rk1[tid] = 0.f; rbk[tid] = 0.f; rf[tid] = 0.f; rv[tid] = 0.f;
     rsq[tid] = l2 ? rstd_q[(tok0 + imin(tid, nvalid - 1)) * Hqk + hq] : 1.f;
     rsk[tid] = l2 ? rstd_k[(tok0 + imin(tid, nvalid - 1)) * Hqk + hq] : 1.f;
   }
+  rq[tid] = 0.f; rk1[tid] = 0.f; rbk[tid] = 0.f; rf[tid] = 0.f; rv[tid] = 0.f;   // 256 threads, 256 entries each
   GDN_WAIT_VMEM();
   GDN_LDS_BARRIER();
 
@@ -606,7 +594,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {
       if (l2) {
-        const f32x16 qq = QTf[ri].unpack(), dot = rows_ld(rq, 32 * ri), rs = rows_ld(rsq, 32 * ri);
+        const f32x16 qq = QTf[ri].unpack(), dot = rows_ld4(rq, 32 * ri), rs = rows_ld(rsq, 32 * ri);
 #pragma unroll
         for (int r = 0; r < 16; ++r) dQi[ri][r] = (dQi[ri][r] - dot[r] * qq[r]) * rs[r];
       }
@@ -677,8 +665,8 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {
       if (l2) {          // <k_i, dK_i> = <k,dK1> + beta (e^G <P,k> + <E,k>) + <F,k>
-        const f32x16 kk = KTf[ri].unpack(), d1 = rows_ld(rk1, 32 * ri), db = rows_ld(rbk, 32 * ri),
-                     df = rows_ld(rf, 32 * ri), br = rows_ld(bs, 32 * ri), rs = rows_ld(rsk, 32 * ri);
+        const f32x16 kk = KTf[ri].unpack(), d1 = rows_ld4(rk1, 32 * ri), db = rows_ld4(rbk, 32 * ri),
+                     df = rows_ld4(rf, 32 * ri), br = rows_ld(bs, 32 * ri), rs = rows_ld(rsk, 32 * ri);
 #pragma unroll
         for (int r = 0; r < 16; ++r)
           dKi[ri][r] = (dKi[ri][r] - (d1[r] + br[r] * db[r] + df[r]) * kk[r]) * rs[r];
@@ -689,7 +677,9 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     }
   }
   if (wave == 0) {   // d(cumulative G) -> d(g): suffix sum inside the chunk
-    float x = rq[lane] - rk1[lane] + bs[lane] * rbk[lane] - rf[lane];
+    auto slots = [&](const float* a) { return (a[lane] + a[64 + lane]) + (a[128 + lane] + a[192 + lane]); };
+    const float sbk = slots(rbk);
+    float x = slots(rq) - slots(rk1) + bs[lane] * sbk - slots(rf);
     if (lane == nvalid - 1)
       x += __expf(glast) * (wsum[0] + wsum[1] + wsum[2] + wsum[3]) + (wsum[4] + wsum[5] + wsum[6] + wsum[7]);
 #pragma unroll
@@ -699,7 +689,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     }
     if (lane < nvalid) {
       dg[(tok0 + lane) * Hv + h] = x;
-      dbeta[(tok0 + lane) * Hv + h] = rbk[lane] + rv[lane];
+      dbeta[(tok0 + lane) * Hv + h] = sbk + slots(rv);
     }
   }
 }

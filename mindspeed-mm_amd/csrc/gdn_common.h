@@ -528,10 +528,26 @@ __device__ __forceinline__ float rows16_partial(const f32x16& x) {
   const float lo = c[0] + dpp_mov<0x128>(c[0]), hi = c[1] + dpp_mov<0x128>(c[1]);   // row_ror:8
   return b3 ? hi : lo;
 }
-// rowacc[i0 + i] += sum_j x[i][j] for the 32 rows of the tile (rowacc in LDS; two lanes add into each entry)
+// rowacc[wave][i0 + i] += sum_j x[i][j] for the 32 rows of the tile.  rowacc is an LDS array [4 waves][64 rows]:
+// every wave owns a slot and every row of a slot is always updated by the same lane, so no atomics are needed and the
+// result does not depend on the order in which waves arrive (readers add the four slots in a fixed order).
 __device__ __forceinline__ void rows_add(const f32x16& x, float* rowacc, int i0) {
-  const float s = rows16_partial(x);
-  atomicAdd(&rowacc[i0 + acc_row(threadIdx.x & 15)], s);
+  float s = rows16_partial(x);
+  s += __shfl_xor(s, 16);     // the other half of the 32 columns
+  const int lane = threadIdx.x & 63;
+  if ((lane & 16) == 0) rowacc[(threadIdx.x >> 6) * 64 + i0 + acc_row(lane & 15)] += s;
+}
+// sum over the four wave slots of such an array, for the rows of this lane's accumulator registers
+__device__ __forceinline__ f32x16 rows_ld(const float* arr, int i0);
+__device__ __forceinline__ f32x16 rows_ld4(const float* arr, int i0) {
+  f32x16 a = rows_ld(arr, i0);
+#pragma unroll
+  for (int w = 1; w < 4; ++w) {
+    const f32x16 b = rows_ld(arr + 64 * w, i0);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) a[r] += b[r];
+  }
+  return a;
 }
 
 // One wave: 32x32 accumulator tile -> 32 global rows of 32 columns (tile row i at g + i*row_stride), written as

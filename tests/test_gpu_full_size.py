@@ -1,0 +1,236 @@
+"""The benchmark configurations at their full sizes, on the GPU, through the C ABI.
+
+The CPU oracle cannot run these shapes whole in test time, so each configuration is checked through properties that
+do not depend on the size, plus the oracle on a slice that is cheap because heads and sequences are independent:
+  * split-run continuity: a sequence processed in two calls with the state handed over equals the single call
+    (the split lies on a chunk boundary, so every chunk sees the same operands: bit-exact);
+  * linearity: with q, k, g, beta fixed the operator is linear in (v, h0) and its backward in (dO, dht); a factor of
+    two is exact in binary floating point, so outputs and gradients must double bit for bit;
+  * packed == separate: a packed batch equals its sequences run one by one;
+  * head / batch slices against the fp32 oracle with the tolerances of the small-shape parity tests.
+"""
+import pytest
+import torch
+
+from mindspeed_mm_amd.inputs import gdn_inputs, packed_lengths
+from oracle import gdn_oracle as O
+from parity import BF16_ABS_GRAD, BF16_ABS_O, _err
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+NAMES = ("q", "k", "v", "g", "beta")
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from mindspeed_mm_amd.ops import _default_ops
+    return _default_ops()
+
+
+def _run(ops, d, h0, cu=None, backward=False, do=None, dht=None):
+    leaves = {n: d[n].clone().requires_grad_(backward) for n in NAMES}
+    h = h0.clone().requires_grad_(backward) if h0 is not None else None
+    o, ht = ops.chunk_gated_delta_rule(leaves["q"], leaves["k"], leaves["v"], leaves["g"], leaves["beta"],
+                                       initial_state=h, output_final_state=True, use_qk_l2norm_in_kernel=True,
+                                       cu_seqlens=cu)
+    if not backward:
+        return o, ht
+    outs, gouts = [o], [do]
+    if dht is not None:
+        outs.append(ht)
+        gouts.append(dht)
+    grads = torch.autograd.grad(outs, [leaves[n] for n in NAMES] + [h], gouts)
+    return o, ht, dict(zip(NAMES + ("h0",), grads))
+
+
+def _oracle_slice(x, b, hq, grp, cu=None, n_sel=None):
+    """fp32 oracle on batch row b, q/k head hq and its grp value heads (heads and rows are independent)."""
+    hs = slice(hq * grp, (hq + 1) * grp)
+    L = {"q": x["q"][b:b + 1, :, hq:hq + 1], "k": x["k"][b:b + 1, :, hq:hq + 1], "v": x["v"][b:b + 1, :, hs],
+         "g": x["g"][b:b + 1, :, hs], "beta": x["beta"][b:b + 1, :, hs]}
+    L = {n: t.float().clone().requires_grad_(True) for n, t in L.items()}
+    rows = slice(b, b + 1) if n_sel is None else n_sel
+    h0 = x["h0"][rows, hs].clone().requires_grad_(True)
+    o, ht = O.chunk_gated_delta_rule_ref(L["q"], L["k"], L["v"], L["g"], L["beta"], initial_state=h0,
+                                         output_final_state=True, use_qk_l2norm_in_kernel=True, cu_seqlens=cu)
+    return L, h0, o, ht
+
+
+def test_config1_chunk_fwd_bwd_full_size(ops):
+    """BASELINE configs[1]: B=2, T=8192, H_qk=16, H_v=32, d=128, bf16, fwd+bwd."""
+    B, T, Hqk, Hv, K, V = 2, 8192, 16, 32, 128, 128
+    x = gdn_inputs(B, T, Hqk, Hv, K, V, BF, seed=0)
+    d = {n: t.cuda() for n, t in x.items()}
+    o, ht, gr = _run(ops, d, d["h0"], backward=True, do=d["do"], dht=d["dht"])
+    assert torch.isfinite(o.float()).all() and torch.isfinite(ht).all()
+
+    # split-run continuity at a chunk boundary
+    half = {n: d[n][:, :T // 2].contiguous() for n in NAMES}
+    rest = {n: d[n][:, T // 2:].contiguous() for n in NAMES}
+    o1, s1 = _run(ops, half, d["h0"])
+    o2, s2 = _run(ops, rest, s1)
+    assert torch.equal(torch.cat([o1, o2], 1), o) and torch.equal(s2, ht)
+
+    # linearity in (v, h0) forward and in (dO, dht) backward: exact doubling
+    d2 = dict(d, v=d["v"] * 2)
+    o_2, ht_2 = _run(ops, d2, d["h0"] * 2)
+    assert torch.equal(o_2, o * 2) and torch.equal(ht_2, ht * 2)
+    _, _, gr2 = _run(ops, d, d["h0"], backward=True, do=d["do"] * 2, dht=d["dht"] * 2)
+    for n in gr:
+        assert torch.equal(gr2[n], gr[n] * 2), n
+
+    # oracle on one batch row and one q/k group (2 value heads), all 128 chunks
+    b, hq, grp = 1, 5, Hv // Hqk
+    L, h0, ro, rht = _oracle_slice(x, b, hq, grp)
+    hs = slice(hq * grp, (hq + 1) * grp)
+    rg = torch.autograd.grad([ro, rht], list(L.values()) + [h0], [x["do"][b:b + 1, :, hs].float(), x["dht"][b:b + 1, hs]])
+    rg = dict(zip(NAMES + ("h0",), rg))
+    _err("o", o[b:b + 1, :, hs], ro, BF, BF16_ABS_O)
+    _err("final_state", ht[b:b + 1, hs], rht, BF, BF16_ABS_GRAD)
+    _err("dq", gr["q"][b:b + 1, :, hq:hq + 1], rg["q"], BF, BF16_ABS_GRAD)
+    _err("dk", gr["k"][b:b + 1, :, hq:hq + 1], rg["k"], BF, BF16_ABS_GRAD)
+    for n in ("v", "g", "beta"):
+        _err("d" + n, gr[n][b:b + 1, :, hs], rg[n], BF, BF16_ABS_GRAD)
+    _err("dh0", gr["h0"][b:b + 1, hs], rg["h0"], BF, BF16_ABS_GRAD)
+
+
+def test_config2_packed_sequences_full_size(ops):
+    """BASELINE configs[2]: 32768 packed tokens in 24 sequences of ragged lengths, H_qk=16, H_v=32, d=128, bf16."""
+    cu = packed_lengths()
+    N, total, Hqk, Hv, K, V = len(cu) - 1, cu[-1], 16, 32, 128, 128
+    x = gdn_inputs(1, total, Hqk, Hv, K, V, BF, seed=2, N=N)
+    d = {n: t.cuda() for n, t in x.items()}
+    cu_t = torch.tensor(cu, dtype=torch.int64, device="cuda")
+    o, ht, gr = _run(ops, d, d["h0"], cu=cu_t, backward=True, do=d["do"], dht=d["dht"])
+
+    # packed == every sequence on its own (same chunking inside a sequence: bit-exact)
+    for n in range(N):
+        a, b = cu[n], cu[n + 1]
+        one = {m: d[m][:, a:b].contiguous() for m in NAMES}
+        o_n, ht_n, gr_n = _run(ops, one, d["h0"][n:n + 1], backward=True, do=d["do"][:, a:b].contiguous(),
+                               dht=d["dht"][n:n + 1])
+        assert torch.equal(o_n, o[:, a:b]) and torch.equal(ht_n, ht[n:n + 1]), n
+        for m in NAMES:
+            assert torch.equal(gr_n[m], gr[m][:, a:b]), (n, m)
+        assert torch.equal(gr_n["h0"], gr["h0"][n:n + 1]), n
+
+    # oracle on the two shortest sequences, one q/k group
+    lens = [cu[n + 1] - cu[n] for n in range(N)]
+    for n in sorted(range(N), key=lambda i: lens[i])[:2]:
+        a, b = cu[n], cu[n + 1]
+        hq, grp = 7, Hv // Hqk
+        hs = slice(hq * grp, (hq + 1) * grp)
+        xs = {m: x[m][:, a:b] for m in NAMES}
+        xs["h0"] = x["h0"]
+        L, h0, ro, rht = _oracle_slice(xs, 0, hq, grp, n_sel=slice(n, n + 1))
+        rg = torch.autograd.grad([ro, rht], list(L.values()) + [h0],
+                                 [x["do"][:, a:b, hs].float(), x["dht"][n:n + 1, hs]])
+        rg = dict(zip(NAMES + ("h0",), rg))
+        _err("o", o[:, a:b, hs], ro, BF, BF16_ABS_O)
+        _err("final_state", ht[n:n + 1, hs], rht, BF, BF16_ABS_GRAD)
+        _err("dq", gr["q"][:, a:b, hq:hq + 1], rg["q"], BF, BF16_ABS_GRAD)
+        _err("dk", gr["k"][:, a:b, hq:hq + 1], rg["k"], BF, BF16_ABS_GRAD)
+        for m in ("v", "g", "beta"):
+            _err("d" + m, gr[m][:, a:b, hs], rg[m], BF, BF16_ABS_GRAD)
+
+
+def test_config2_conv1d_packed_full_size(ops):
+    """BASELINE configs[2], conv part: packed [1, 32768, 8192], W=4, SiLU, fwd+bwd; packed == sequences one by one."""
+    cu = packed_lengths()
+    D, W = 8192, 4
+    gen = torch.Generator().manual_seed(2)
+    xx = torch.randn(1, cu[-1], D, generator=gen).to("cuda", BF).requires_grad_(True)
+    ww = (torch.randn(W, D, generator=gen) / 2).to("cuda", BF).requires_grad_(True)
+    dy = torch.randn(1, cu[-1], D, generator=gen).to("cuda", BF)
+    cu_t = torch.tensor(cu, dtype=torch.int64, device="cuda")
+    y, _ = ops.causal_conv1d(xx, ww, None, None, None, "silu", cu_t, False)
+    dx, dw = torch.autograd.grad([y], [xx, ww], [dy])
+    for n in (0, 5, len(cu) - 2):
+        a, b = cu[n], cu[n + 1]
+        xs = xx.detach()[:, a:b].contiguous().requires_grad_(True)
+        ys, _ = ops.causal_conv1d(xs, ww, None, None, None, "silu", None, False)
+        dxs, _ = torch.autograd.grad([ys], [xs, ww], [dy[:, a:b].contiguous()])
+        assert torch.equal(ys, y[:, a:b]) and torch.equal(dxs, dx[:, a:b]), n
+    # dw over the packed batch against the eager definition on a channel slice (fp32)
+    ch = slice(0, 64)
+    xr = xx.detach()[0, :, ch].float().cpu().requires_grad_(True)
+    wr = ww.detach()[:, ch].float().cpu().requires_grad_(True)
+    yr = O.causal_conv1d_ref(xr[None], wr, None, None, None, "silu", cu, False)[0]
+    dxr, dwr = torch.autograd.grad([yr], [xr, wr], [dy[:, :, ch].float().cpu()])
+    _err("y", y[0, :, ch], yr[0], BF, 1e-2, rtol=1e-2)
+    _err("dx", dx[0, :, ch], dxr, BF, 2e-2, rtol=1e-2)
+    _err("dw", dw[:, ch], dwr, BF, 1e-2 * dwr.abs().max().item(), rtol=1e-2)
+
+
+def test_config3_decode_batch256_64_steps(ops):
+    """BASELINE configs[3]: batch 256, one token per sequence per step, 64 steps, state updated in place."""
+    B, S, Hqk, Hv, K, V = 256, 64, 16, 32, 128, 128
+    x = gdn_inputs(B, S, Hqk, Hv, K, V, BF, seed=3)
+    d = {n: t.cuda() for n, t in x.items()}
+    state = d["h0"].clone()
+    outs = []
+    for t in range(S):
+        tok = {n: d[n][:, t:t + 1].contiguous() for n in NAMES}
+        o, s = ops.fused_recurrent_gated_delta_rule(tok["q"], tok["k"], tok["v"], tok["g"], tok["beta"],
+                                                    initial_state=state, output_final_state=True,
+                                                    use_qk_l2norm_in_kernel=True, inplace_state=True)
+        assert s.data_ptr() == state.data_ptr()
+        outs.append(o)
+    o_steps = torch.cat(outs, 1)
+    # 64 single-token calls == one 64-token call (same arithmetic per token: bit-exact)
+    o_all, s_all = ops.fused_recurrent_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"],
+                                                        initial_state=d["h0"], output_final_state=True,
+                                                        use_qk_l2norm_in_kernel=True)
+    assert torch.equal(o_steps, o_all) and torch.equal(state, s_all)
+    # oracle on a batch slice
+    bs = slice(100, 104)
+    ro, rs = O.recurrent_gated_delta_rule_ref(x["q"][bs].float(), x["k"][bs].float(), x["v"][bs].float(), x["g"][bs],
+                                              x["beta"][bs].float(), x["h0"][bs], True, True)
+    _err("o", o_steps[bs], ro, BF, BF16_ABS_O)
+    _err("state", state[bs], rs, torch.float32, 0)
+
+
+def test_config4_long_sequence_wide_heads(ops):
+    """BASELINE configs[4]: B=1, T=65536, H_qk=16, H_v=64, d_k=128, d_v=256, bf16, fwd+bwd (1024 chunks)."""
+    B, T, Hqk, Hv, K, V = 1, 65536, 16, 64, 128, 256
+    x = gdn_inputs(B, T, Hqk, Hv, K, V, BF, seed=4, a_log=(0.5, 2.0), dt_bias=(-6.0, -4.0))
+    d = {n: t.cuda() for n, t in x.items()}
+    o, ht, gr = _run(ops, d, d["h0"], backward=True, do=d["do"], dht=d["dht"])
+    assert torch.isfinite(o.float()).all() and torch.isfinite(ht).all()
+    for n in gr:
+        assert torch.isfinite(gr[n].float()).all(), n
+
+    quarter = T // 4   # four calls with the state handed over == one call
+    s, parts = d["h0"], []
+    for i in range(4):
+        part = {n: d[n][:, i * quarter:(i + 1) * quarter].contiguous() for n in NAMES}
+        oi, s = _run(ops, part, s)
+        parts.append(oi)
+    assert torch.equal(torch.cat(parts, 1), o) and torch.equal(s, ht)
+
+    _, _, gr2 = _run(ops, d, d["h0"], backward=True, do=d["do"] * 2, dht=d["dht"] * 2)
+    for n in gr:
+        assert torch.equal(gr2[n], gr[n] * 2), n
+
+    # backward continuity: the second half's gradient w.r.t. its initial state is the first half's dht
+    half = T // 2
+    first = {n: d[n][:, :half].contiguous() for n in NAMES}
+    second = {n: d[n][:, half:].contiguous() for n in NAMES}
+    _, s_mid = _run(ops, first, d["h0"])
+    _, _, g2 = _run(ops, second, s_mid, backward=True, do=d["do"][:, half:].contiguous(), dht=d["dht"])
+    _, _, g1 = _run(ops, first, d["h0"], backward=True, do=d["do"][:, :half].contiguous(), dht=g2["h0"])
+    for n in NAMES:
+        assert torch.equal(torch.cat([g1[n], g2[n]], 1), gr[n]), n
+    assert torch.equal(g1["h0"], gr["h0"])
+
+    # oracle (forward; its autograd over 1024 chunks takes minutes) on one q/k group of 4 value heads:
+    # o and the final state after 1024 chunks
+    hq, grp = 9, Hv // Hqk
+    hs = slice(hq * grp, (hq + 1) * grp)
+    with torch.no_grad():
+        ro, rht = O.chunk_gated_delta_rule_ref(x["q"][:, :, hq:hq + 1].float(), x["k"][:, :, hq:hq + 1].float(),
+                                               x["v"][:, :, hs].float(), x["g"][:, :, hs], x["beta"][:, :, hs].float(),
+                                               initial_state=x["h0"][:, hs], output_final_state=True,
+                                               use_qk_l2norm_in_kernel=True)
+    _err("o", o[:, :, hs], ro, BF, BF16_ABS_O)
+    _err("final_state", ht[:, hs], rht, BF, BF16_ABS_GRAD)
