@@ -88,13 +88,14 @@ __device__ __forceinline__ void load_tile_qk(T* lds, int ld, const T* g, int64_t
 // ---------------------------------------------------------------------------------------------
 template <typename T, int DK, int BV> struct PrepSmem {
   static constexpr int LDK = lds_ld<T>(DK), LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
-  static constexpr int kv_elems = 64 * (LDK > LDV ? LDK : LDV);
-  static constexpr int off_ks = 0;  // K tile, scaled in place to beta e^G K after the score tiles
-  static constexpr int off_qs = off_ks + 64 * LDK * (int)sizeof(T);  // Q tile, later the (beta V) tile
-  static constexpr int off_as = off_qs + kv_elems * (int)sizeof(T);
-  static constexpr int off_ti = off_as + 64 * kLF * 4;
-  static constexpr int off_tms = off_ti + 64 * kLF * 4;
-  static constexpr int off_misc = off_tms + 64 * L64 * (int)sizeof(T);
+  static constexpr int cmax(int a, int b) { return a > b ? a : b; }
+  // Three regions, each reused once its first tenant is dead, so that three workgroups fit a CU's LDS:
+  static constexpr int off_ks = 0;                                    // K tile, scaled in place to beta e^G K
+  static constexpr int off_qs = off_ks + 64 * LDK * (int)sizeof(T);   // Q tile -> A (fp32, solve input) -> Tm in T
+  static constexpr int qs_bytes = cmax(cmax(64 * LDK * (int)sizeof(T), 64 * kLF * 4), 64 * L64 * (int)sizeof(T));
+  static constexpr int off_ti = off_qs + qs_bytes;                    // Tm (fp32, solve output) -> (beta V) tile
+  static constexpr int ti_bytes = cmax(64 * kLF * 4, 64 * LDV * (int)sizeof(T));
+  static constexpr int off_misc = off_ti + ti_bytes;
   static constexpr int bytes = off_misc + 3 * 64 * 4;
 };
 
@@ -111,10 +112,10 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
   T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
   T* Kb = Ks;
   T* Qs = reinterpret_cast<T*>(gdn_smem + SM::off_qs);
-  T* Vb = Qs;
-  float* As = reinterpret_cast<float*>(gdn_smem + SM::off_as);
+  float* As = reinterpret_cast<float*>(gdn_smem + SM::off_qs);    // after Q
+  T* Tms = reinterpret_cast<T*>(gdn_smem + SM::off_qs);          // after A
   float* Ti = reinterpret_cast<float*>(gdn_smem + SM::off_ti);
-  T* Tms = reinterpret_cast<T*>(gdn_smem + SM::off_tms);
+  T* Vb = reinterpret_cast<T*>(gdn_smem + SM::off_ti);           // after Tm (fp32)
   float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_misc);
   float* bs = Gs + 64;
   float* egs = bs + 64;
@@ -153,11 +154,12 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
   __syncthreads();
 
   // ---- phase 1: A = strict_tril(beta_i k_i.k_j Gam_ij) and Aq = tril(q_i.k_j Gam_ij), one 32x32 tile per wave ----
+  f32x16 a_tile = acc_zero();   // goes to LDS (over the Q tile) once every wave is done with Q
   {
     const int ti = wave >> 1, tj = wave & 1;
-    f32x16 acc = acc_zero(), aq = acc_zero();
+    f32x16 aq = acc_zero();
     if (tj <= ti) {
-      mma32<T, DK, true, true>(acc, Ks + 32 * ti * LDK, LDK, Ks + 32 * tj * LDK, LDK);
+      mma32<T, DK, true, true>(a_tile, Ks + 32 * ti * LDK, LDK, Ks + 32 * tj * LDK, LDK);
       mma32<T, DK, true, true>(aq, Qs + 32 * ti * LDK, LDK, Ks + 32 * tj * LDK, LDK);
     }
     const int j = 32 * tj + acc_col();
@@ -165,7 +167,7 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
     for (int r = 0; r < 16; ++r) {
       const int i = 32 * ti + acc_row(r);
       const float gam = i >= j ? __expf(Gs[i] - Gs[j]) : 0.f;
-      As[i * kLF + j] = i > j ? bs[i] * acc[r] * gam : 0.f;
+      a_tile[r] = i > j ? bs[i] * a_tile[r] * gam : 0.f;
       aq[r] *= gam;
     }
     // tril(Q K^T . Gam) leaves as four 32x32 tiles in fragment order, packed as they sit in the accumulator
@@ -201,9 +203,14 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
       }
     }
   }
-  __syncthreads();
+  __syncthreads();   // Q is consumed: its space takes A
 
-  // K tile -> beta e^G K in place; (beta V) tile of the first V block replaces Q while the solve runs
+  {
+    const int ti = wave >> 1, tj = wave & 1, j = 32 * tj + acc_col();
+#pragma unroll
+    for (int r = 0; r < 16; ++r) As[(32 * ti + acc_row(r)) * kLF + j] = a_tile[r];
+  }
+  // K tile -> beta e^G K in place
   {
     constexpr int CPR = DK / VEC;
     for (int c = tid; c < 64 * CPR; c += kThreads) {
@@ -215,8 +222,16 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
       st16(Kb + row * LDK + cc * VEC, x);
     }
   }
+  // the first V block is requested now and parked in registers until the fp32 Tm has been consumed
   const T* vg = v + (tok0 * Hv + h) * V;
-  load_tile_scaled<T, BV>(Vb, LDV, vg, (int64_t)Hv * V, nvalid, bs, tid);
+  constexpr int VPT = 64 * (BV / VEC) / kThreads;   // 16-byte pieces of the V tile per thread
+  Vec16<T> vreg[VPT];
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int c = tid + i * kThreads, row = c / (BV / VEC), cc = c % (BV / VEC);
+    vreg[i] = row < nvalid ? ld16(vg + (int64_t)row * Hv * V + cc * VEC) : zero16<T>();
+  }
+  __syncthreads();
 
   // ---- phase 2a: invert the four 16x16 diagonal blocks by forward substitution (fp32) ----
   if (lane < 16) {
@@ -292,6 +307,15 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
     }
   }
   __syncthreads();
+  // the fp32 Tm is consumed: its space takes the (beta V) tile parked in registers
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int c = tid + i * kThreads, row = c / (BV / VEC), cc = c % (BV / VEC);
+    const float sc = bs[row];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) vreg[i].set(e, vreg[i].get(e) * sc);
+    st16(Vb + row * LDV + cc * VEC, vreg[i]);
+  }
   {  // the four 32x32 tiles of Tm as A operands (lane <-> row, registers <-> column), fragment order, for the backward
     AccB<T> tf;
     frags_from_lds<T>(tf, Tms + (32 * (wave >> 1) + (lane & 31)) * L64 + 32 * (wave & 1));
@@ -317,8 +341,8 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
   }
   // ---- phase 5: U = Tm (beta V), V block by V block, stored in fragment order ----
   for (int vb = 0; vb < V / BV; ++vb) {
+    __syncthreads();
     if (vb > 0) {
-      __syncthreads();
       load_tile_scaled<T, BV>(Vb, LDV, vg + vb * BV, (int64_t)Hv * V, nvalid, bs, tid);
       __syncthreads();
     }
