@@ -15,7 +15,7 @@ initial state, upstream grad ~ N(0,1)); inputs are synthetic and already residen
   cpu_baseline the CPU oracle (PyTorch fp32 restatement of the reference's torch path, autograd backward) timed on
                this box's host cores on a bounded sample of the same workload
   aux          the whole path against the MFMA peak with the reference's FLOP formula, the per-kernel split,
-               and the HBM-bound siblings (batch-256 decode, the packed conv1d) with their achieved GB/s
+               and the HBM-bound siblings (batch-256 decode, the packed conv1d, the gated RMSNorm) with their achieved GB/s
 """
 import argparse
 import json
@@ -224,6 +224,29 @@ def main():
         aux["conv1d_packed"] = {"fwd_ms": round(f_s * 1e3, 3), "fwd_GBps": round(2 * nb / f_s / 1e9, 1),
                                 "bwd_ms": round(b_s * 1e3, 3), "bwd_GBps": round(3 * nb / b_s / 1e9, 1)}
         del xx, ww, dy
+        # ---- gated RMSNorm on the chunk output of the benchmark shape: [tokens * H_v, d_v] rows, fwd+bwd ----
+        rows = tokens * c["Hv"]
+        xn = torch.randn(rows, c["V"], generator=gen).to(dev, torch.bfloat16).requires_grad_(True)
+        zn = torch.randn(rows, c["V"], generator=gen).to(dev, torch.bfloat16).requires_grad_(True)
+        wn = torch.ones(c["V"], device=dev, dtype=torch.bfloat16, requires_grad=True)
+        dyn = torch.randn(rows, c["V"], generator=gen).to(dev, torch.bfloat16)
+
+        def norm_step():
+            yn = ops.rms_norm_gated(xn, zn, wn, 1e-6)
+            torch.autograd.grad([yn], [xn, zn, wn], [dyn])
+        norm_step()
+        lib.gdn_profile_enable(1)
+        for _ in range(5):
+            norm_step()
+        torch.cuda.synchronize()
+        tm = _lib.kernel_timings(lib)
+        lib.gdn_profile_enable(0)
+        nb = xn.numel() * 2
+        f_s = tm["rmsnorm_gated_fwd_kernel"][0] / tm["rmsnorm_gated_fwd_kernel"][1] * 1e-3
+        b_s = tm["rmsnorm_gated_bwd_kernel"][0] / tm["rmsnorm_gated_bwd_kernel"][1] * 1e-3
+        aux["rmsnorm_gated"] = {"fwd_ms": round(f_s * 1e3, 3), "fwd_GBps": round(3 * nb / f_s / 1e9, 1),
+                                "bwd_ms": round(b_s * 1e3, 3), "bwd_GBps": round(5 * nb / b_s / 1e9, 1)}
+        del xn, zn, dyn
 
     if args.calibrate_copy:
         src = torch.empty(512 << 20, dtype=torch.uint8, device=dev)

@@ -77,6 +77,21 @@ int gdn_conv1d_bwd(const void* x, const void* dy, const void* weight, const void
 int gdn_conv1d_update(const void* hidden, void* conv_state, const void* weight, const void* bias, void* out, int B,
                       int T, int D, int W, int state_len, int activation, int dtype, void* stream);
 
+/* -------- gated RMSNorm (the step after the gated delta rule in the layer) -----------------------------
+ * replaces Qwen3_5RMSNormGated.forward, modeling_qwen3_5.py:330-349 (called on [tokens*Hv, head_v_dim] rows at
+ * :897-900): y = (weight * (x * rsqrt(mean(x^2) + eps))) * silu(gate), intermediate casts to the input dtype as
+ * in the reference.  x, gate, y, dy, dx, dgate [rows, N]; weight [N] in the input dtype (weight_dtype = dtype) or
+ * fp32 (weight_dtype = 0); rstd [rows] fp32 is written by the forward and read by the backward; dweight [N] fp32.
+ * N * element size / 16 must be 4, 8, 16, 32 or 64 (bf16: N = 32 ... 512; fp32: N = 16 ... 256). */
+int gdn_rmsnorm_gated_fwd(const void* x, const void* gate, const void* weight, void* y, float* rstd, int64_t rows,
+                          int N, float eps, int dtype, int weight_dtype, void* stream);
+
+int64_t gdn_rmsnorm_gated_bwd_workspace_bytes(int64_t rows, int N);
+
+int gdn_rmsnorm_gated_bwd(const void* x, const void* gate, const void* weight, const float* rstd, const void* dy,
+                          void* dx, void* dgate, float* dweight, void* workspace, int64_t workspace_bytes,
+                          int64_t rows, int N, int dtype, int weight_dtype, void* stream);
+
 /* -------- per-kernel timing ------------------------------------------------------------------------
  * op-level counterpart of the reference's step profiler (mindspeed_mm/fsdp/tools/profiler.py:32-147).
  * While enabled, every kernel launch of this library is bracketed by HIP events on its stream (this mode

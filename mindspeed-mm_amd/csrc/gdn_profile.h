@@ -8,7 +8,7 @@ namespace gdn {
 enum KernelId {
   kKernChunkTable = 0, kKernPrep, kKernStateFwd, kKernOut, kKernStateBwd, kKernBwdLocal,
   kKernRecurrent, kKernConvFwd, kKernConvState, kKernConvBwd, kKernConvReduce,
-  kKernConvDh0, kKernConvUpdate, kKernCount
+  kKernConvDh0, kKernConvUpdate, kKernRmsNormFwd, kKernRmsNormBwd, kKernRmsNormReduce, kKernCount
 };
 
 bool profile_on();

@@ -22,6 +22,9 @@ SIGNATURES = {
     "gdn_conv1d_bwd_workspace_bytes": (L, [I] * 4),
     "gdn_conv1d_bwd": (I, [P] * 12 + [L] + [I] * 7 + [P]),
     "gdn_conv1d_update": (I, [P] * 5 + [I] * 7 + [P]),
+    "gdn_rmsnorm_gated_fwd": (I, [P] * 5 + [L, I, F, I, I, P]),
+    "gdn_rmsnorm_gated_bwd_workspace_bytes": (L, [L, I]),
+    "gdn_rmsnorm_gated_bwd": (I, [P] * 9 + [L, L, I, I, I, P]),
     "gdn_profile_enable": (I, [I]),
     "gdn_profile_kernel_count": (I, []),
     "gdn_profile_kernel_name": (ctypes.c_char_p, [I]),
@@ -33,7 +36,8 @@ DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 _ERRORS = {
     -1: "null pointer for a required tensor",
     -2: "inconsistent shapes",
-    -3: "unsupported size (K must be 64 or 128 (256 for decode), V a multiple of 64, conv width 1..8, D % 8 == 0)",
+    -3: "unsupported size (K must be 64 or 128 (256 for decode), V a multiple of 64, conv width 1..8, D % 8 == 0, "
+        "norm rows of 4/8/16/32/64 16-byte pieces)",
     -4: "unsupported dtype",
     -5: "workspace too small or misaligned",
 }

@@ -5,6 +5,7 @@
                                       (semantics of torch_recurrent_gated_delta_rule, :478-517)
     causal_conv1d                     mindspeed_mm/fsdp/models/qwen3_5/causal_conv1d.py:100-119
     causal_conv1d_update              modeling_qwen3_5.py:373-389, called at :738-744
+    rms_norm_gated / RMSNormGated     Qwen3_5RMSNormGated, modeling_qwen3_5.py:330-349, called at :897-900
 
 Everything here is host glue: validation, output/workspace allocation with torch, and one call into the
 C ABI per operator.  The kernels themselves are the HIP library; nothing in this file computes.
@@ -154,6 +155,13 @@ class GdnOps:
             conv_state.copy_(state)
         return out
 
+    # ------------------------------------------------------------------ gated RMSNorm
+    def rms_norm_gated(self, hidden_states, gate, weight, eps=1e-6):
+        if gate is None:
+            raise ValueError("rms_norm_gated needs a gate (the reference layer always passes one)")
+        self._need(hidden_states, gate, weight)
+        return _RMSNormGated.apply(hidden_states, gate, weight, eps, self)
+
 
 def _i64(cu, ref):
     if cu is None:
@@ -260,6 +268,52 @@ class _CausalConv1d(torch.autograd.Function):
                 None if dh0 is None else dh0.to(h_dt), None, None, None, None)
 
 
+class _RMSNormGated(torch.autograd.Function):
+    """y = (weight * rmsnorm(x)) * silu(gate) over the last axis."""
+
+    @staticmethod
+    def forward(ctx, x, gate, weight, eps, ops):
+        lib = ops.lib
+        dt = x.dtype
+        if dt not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"rms_norm_gated supports float32 and bfloat16, got {dt}")
+        if gate.shape != x.shape:
+            raise ValueError(f"gate shape {tuple(gate.shape)} differs from hidden_states shape {tuple(x.shape)}")
+        N = x.shape[-1]
+        if weight.shape != (N,):
+            raise ValueError(f"weight shape {tuple(weight.shape)}, expected ({N},)")
+        w_dt = dt if weight.dtype == dt else torch.float32   # same dtype as the input, else fp32 as in the reference
+        xc = x.contiguous().view(-1, N)
+        gc = gate.to(dt).contiguous().view(-1, N)
+        wc = weight.detach().to(w_dt).contiguous()
+        rows = xc.shape[0]
+        y = torch.empty_like(xc)
+        rstd = torch.empty(rows, dtype=torch.float32, device=x.device)
+        code = lib.gdn_rmsnorm_gated_fwd(ptr(xc), ptr(gc), ptr(wc), ptr(y), ptr(rstd), rows, N, float(eps),
+                                         DTYPE_CODE[dt], DTYPE_CODE[w_dt], lib.stream())
+        lib.check(code, "gdn_rmsnorm_gated_fwd")
+        ctx.save_for_backward(xc, gc, wc, rstd)
+        ctx.meta = (rows, N, dt, w_dt, weight.dtype, gate.dtype, x.shape)
+        ctx.ops = ops
+        return y.view(x.shape)
+
+    @staticmethod
+    def backward(ctx, dy):
+        xc, gc, wc, rstd = ctx.saved_tensors
+        rows, N, dt, w_dt, weight_dt, gate_dt, shape = ctx.meta
+        lib = ctx.ops.lib
+        dyc = dy.to(dt).contiguous().view(-1, N)
+        dx = torch.empty_like(xc)
+        dg = torch.empty_like(xc)
+        dw = torch.empty(N, dtype=torch.float32, device=xc.device)
+        nbytes = lib.gdn_rmsnorm_gated_bwd_workspace_bytes(rows, N)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=xc.device)
+        code = lib.gdn_rmsnorm_gated_bwd(ptr(xc), ptr(gc), ptr(wc), ptr(rstd), ptr(dyc), ptr(dx), ptr(dg), ptr(dw),
+                                         ptr(ws), nbytes, rows, N, DTYPE_CODE[dt], DTYPE_CODE[w_dt], lib.stream())
+        lib.check(code, "gdn_rmsnorm_gated_bwd")
+        return dx.view(shape), dg.view(shape).to(gate_dt), dw.to(weight_dt), None, None
+
+
 # ---------------------------------------------------------------------- module-level entry points
 _ops: Optional[GdnOps] = None
 
@@ -304,3 +358,23 @@ def causal_conv1d(x, weight, bias=None, residual=None, initial_state=None, activ
 @torch.compiler.disable
 def causal_conv1d_update(hidden_states, conv_state, weight, bias=None, activation=None):
     return _default_ops().causal_conv1d_update(hidden_states, conv_state, weight, bias, activation)
+
+
+@torch.compiler.disable
+def rms_norm_gated(hidden_states, gate, weight, eps=1e-6):
+    """Functional form of Qwen3_5RMSNormGated.forward (modeling_qwen3_5.py:341-349):
+    (weight * rmsnorm(hidden_states)) * silu(gate) over the last axis, in the input dtype."""
+    return _default_ops().rms_norm_gated(hidden_states, gate, weight, eps)
+
+
+class RMSNormGated(torch.nn.Module):
+    """Drop-in for Qwen3_5RMSNormGated (modeling_qwen3_5.py:330-349): same constructor, parameter and forward."""
+
+    def __init__(self, hidden_size, eps=1e-6, **kwargs):
+        super().__init__()
+        self.weight = torch.nn.Parameter(torch.ones(hidden_size))
+        self.variance_epsilon = eps
+
+    def forward(self, hidden_states, gate=None):
+        return rms_norm_gated(hidden_states, gate, self.weight, self.variance_epsilon)
+

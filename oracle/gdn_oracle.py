@@ -16,6 +16,7 @@ relative to the reference checkout):
 * ``causal_conv1d_final_state_ref`` reference_impl.py:81-102
 * ``causal_conv1d_update_ref``     modeling_qwen3_5.py:373-389
 * ``pad_and_batch``                tests/ut_fsdp/models/qwen3_5/test_chunk_gated_delta_rule.py:14-28
+* ``rms_norm_gated_ref``           Qwen3_5RMSNormGated.forward, modeling_qwen3_5.py:341-349 (the non-NPU branch)
 
 The reference functions take neither ``scale``, ``cu_seqlens`` nor grouped
 (GQA) q/k heads; the operator entry does
@@ -33,6 +34,8 @@ How each function is pinned (tests/test_oracle_*.py):
   continuity, explicit ``(I+A)^-1`` by ``torch.linalg.solve_triangular``;
 * backward == autograd through the fp64 recurrence + ``gradcheck``;
 * conv1d == ``F.conv1d(groups=D)`` library routine and autograd thereof;
+* gated RMSNorm == ``F.rms_norm`` (library routine) times ``F.silu(gate)`` in fp64, the closed form for a constant
+  row, scale invariance in x, ``gradcheck``;
 * committed golden vectors under ``tests/golden`` (made by the fp64
   recurrence) guard against drift.
 
@@ -316,3 +319,19 @@ def causal_conv1d_update_ref(hidden_states, conv_state, weight, bias=None, activ
     out = F.conv1d(cat, weight.unsqueeze(1), bias, padding=0, groups=hs.shape[1])
     out = _act(out[:, :, -Tn:], activation)
     return out.to(hidden_states.dtype).transpose(1, 2).contiguous()
+
+
+# --------------------------------------------------------------------------
+# gated RMSNorm (the step after the gated delta rule in the layer)
+# --------------------------------------------------------------------------
+def rms_norm_gated_ref(hidden_states: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor,
+                       eps: float = 1e-6) -> torch.Tensor:
+    """Qwen3_5RMSNormGated.forward (modeling_qwen3_5.py:341-349): normalise in fp32, cast back to the input dtype,
+    scale by ``weight``, multiply with ``silu(gate)`` taken in fp32, cast to the input dtype.  Differentiable."""
+    input_dtype = hidden_states.dtype
+    x = hidden_states.to(torch.float32)
+    variance = x.pow(2).mean(-1, keepdim=True)
+    x = x * torch.rsqrt(variance + eps)
+    x = weight * x.to(input_dtype)
+    x = x * F.silu(gate.to(torch.float32))
+    return x.to(input_dtype)

@@ -19,7 +19,7 @@ def declared():
 def test_header_declares_the_operator_entry_points():
     names = declared()
     for n in ("gdn_chunk_fwd", "gdn_chunk_bwd", "gdn_recurrent_fwd", "gdn_conv1d_fwd", "gdn_conv1d_bwd",
-              "gdn_conv1d_update", "gdn_chunk_workspace_bytes"):
+              "gdn_conv1d_update", "gdn_chunk_workspace_bytes", "gdn_rmsnorm_gated_fwd", "gdn_rmsnorm_gated_bwd"):
         assert n in names
 
 

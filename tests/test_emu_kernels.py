@@ -64,3 +64,12 @@ def test_conv1d(ops, dtype, B, T, D, W, cu):
 @pytest.mark.parametrize("dtype,B,T,D,W", [(F32, 2, 1, 16, 4), (BF, 3, 5, 8, 4), (F32, 1, 3, 8, 2)])
 def test_conv1d_update(ops, dtype, B, T, D, W):
     P.check_conv_update(ops, "cpu", B, T, D, W, dtype, wrap=guarded)
+
+
+@pytest.mark.parametrize("dtype,shape,N,wdt", [
+    (F32, (3, 5), 64, None), (BF, (70,), 128, None), (BF, (2, 9), 256, torch.float32), (F32, (33,), 16, None),
+    (BF, (5,), 512, None), (F32, (4,), 256, None), (BF, (300,), 32, None),
+])
+def test_rms_norm_gated(ops, dtype, shape, N, wdt):
+    P.check_rms_norm_gated(ops, "cpu", shape, N, dtype, weight_dtype=wdt, wrap=guarded)
+

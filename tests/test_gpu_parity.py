@@ -90,3 +90,24 @@ def test_conv1d(ops, dtype, B, T, D, W, cu):
 @pytest.mark.parametrize("dtype,B,T,D,W", [(F32, 2, 1, 16, 4), (BF, 3, 5, 8, 4), (BF, 16, 1, 8192, 4)])
 def test_conv1d_update(ops, dtype, B, T, D, W):
     P.check_conv_update(ops, "cuda", B, T, D, W, dtype)
+
+
+@pytest.mark.parametrize("dtype,shape,N,wdt", [
+    (F32, (3, 5), 64, None), (BF, (70,), 128, None), (BF, (2, 9), 256, torch.float32), (F32, (33,), 16, None),
+    (BF, (5,), 512, None), (F32, (4,), 256, None), (BF, (2, 1000, 32), 128, None),
+])
+def test_rms_norm_gated(ops, dtype, shape, N, wdt):
+    P.check_rms_norm_gated(ops, "cuda", shape, N, dtype, weight_dtype=wdt)
+
+
+def test_rms_norm_gated_module_matches_functional(ops):
+    from mindspeed_mm_amd import RMSNormGated
+    m = RMSNormGated(128).to("cuda", BF)
+    x = torch.randn(4, 7, 128, device="cuda", dtype=BF)
+    z = torch.randn(4, 7, 128, device="cuda", dtype=BF)
+    assert torch.equal(m(x, z), ops.rms_norm_gated(x, z, m.weight, 1e-6))
+    with pytest.raises(ValueError):
+        ops.rms_norm_gated(x, None, m.weight)
+    with pytest.raises(ValueError):
+        ops.rms_norm_gated(x[..., :100].contiguous(), z[..., :100].contiguous(), m.weight[:100])
+
