@@ -67,6 +67,16 @@ inline ChunkWorkspace chunk_workspace_layout(const ChunkDims& d, int elem_bytes)
   return w;
 }
 
+// The two sequential kernels give one compute wave a 32-column slab of the state.  A workgroup streams its chunk's
+// operand tiles at the rate one CU can pull (~35 GB/s), whatever the number of slabs it serves, so when the whole
+// problem has no more slabs than the device has CUs every slab gets a workgroup (and a CU) of its own; larger
+// problems put two slabs in a workgroup, which share the tiles.
+int device_compute_units();   // defined with the forward launcher
+
+inline bool one_slab_per_workgroup(const ChunkDims& d, int compute_units) {
+  return (int64_t)d.N * d.Hv * (d.V / 32) <= compute_units;
+}
+
 inline int chunk_check_dims(const ChunkDims& d, int dtype) {
   if (d.B <= 0 || d.T <= 0 || d.N <= 0 || d.Hqk <= 0 || d.Hv <= 0 || d.Hv % d.Hqk != 0) return -2;
   if (d.varlen && d.B != 1) return -2;

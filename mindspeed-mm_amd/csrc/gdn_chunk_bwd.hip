@@ -36,14 +36,14 @@ template <typename T, int DK, int NW, int STAGES> struct StateBwdSmem {
   static constexpr int bytes = off_small + (NW * 2048 + 4096) * (int)sizeof(T);
 };
 
-template <typename T, int DK, int NW, int STAGES>
-__global__ __launch_bounds__(128 * NW) void chunk_state_bwd_kernel(
+template <typename T, int DK, int NW, int NL, int STAGES>
+__global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_bwd_kernel(
     const T* __restrict__ kaf, const T* __restrict__ qsf, const T* __restrict__ wf, const T* __restrict__ aqf,
     const T* __restrict__ dO, const float* __restrict__ G, const float* __restrict__ dht, float* __restrict__ dh0,
     T* __restrict__ dvf, T* __restrict__ dhf, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets,
     int T_len, int Hv, int V, float scale) {
   using SM = StateBwdSmem<T, DK, NW, STAGES>;
-  constexpr int NT = 64 * NW, VEC = Elem<T>::kVec, NKT = DK / 32;
+  constexpr int NT = 64 * NL, VEC = Elem<T>::kVec, NKT = DK / 32;   // NT loader threads
   constexpr int CW = 64 * (DK / VEC) / NT, CUL = NW * 2048 / VEC / NT, CAQ = 4096 / VEC / NT, TILE = 64 * DK;
   constexpr int PPR = 32 * NW / VEC;   // 16-byte pieces per dO row of the slab
   static_assert(64 * (DK / VEC) % NT == 0 && (NW * 2048 / VEC) % NT == 0 && (4096 / VEC) % NT == 0,
@@ -61,7 +61,7 @@ __global__ __launch_bounds__(128 * NW) void chunk_state_bwd_kernel(
   // step s = 0 .. nchunks-1 handles chunk nchunks-1-s
   if (wave >= NW) {
     // ================= loader waves =================
-    const int lt = tid - NT;
+    const int lt = tid - 64 * NW;
     constexpr int DEPTH = (STAGES == 2) ? 2 : 1;
     Vec16<T> pk[DEPTH][CW], pq[DEPTH][CW], pw[DEPTH][CW], pa[DEPTH][CAQ], pd[DEPTH][CUL];
     float pdec[DEPTH], pgl[DEPTH];
@@ -700,7 +700,7 @@ template <typename K> static int set_lds_b(K kernel, int bytes) {
                                   bytes);
 }
 
-template <typename T, int DK, int NW, int NWS, int STAGES>
+template <typename T, int DK, int NW, int NWS, int NLS, int STAGES>
 static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const void* q, const void* k, const void* v,
                             const float* beta, const int64_t* cu, const void* dO, const float* dht, void* dq, void* dk,
                             void* dv, float* dg, float* dbeta, float* dh0, unsigned char* ws, float scale, int l2norm,
@@ -723,10 +723,10 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   const float* rstd_q = l2norm ? reinterpret_cast<const float*>(ws + L.rstd) : nullptr;
   const float* rstd_k = l2norm ? rstd_q + tok * d.Hqk : nullptr;
   {
-    auto kern = chunk_state_bwd_kernel<T, DK, NWS, STAGES>;
+    auto kern = chunk_state_bwd_kernel<T, DK, NWS, NLS, STAGES>;
     constexpr int smem = StateBwdSmem<T, DK, NWS, STAGES>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
-    GDN_LAUNCH(kKernStateBwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NWS)), dim3(128 * NWS), smem, st, (const T*)KAF,
+    GDN_LAUNCH(kKernStateBwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NWS)), dim3(64 * (NWS + NLS)), smem, st, (const T*)KAF,
                (const T*)QSF, WF, AQ, (const T*)dO, G, dht, dh0, DVF, DHF, cu, chunk_offsets, d.T, d.Hv, d.V, scale);
   }
   {
@@ -760,19 +760,21 @@ extern "C" int gdn_chunk_bwd(const void* q, const void* k, const void* v, const 
   if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
   unsigned char* ws = static_cast<unsigned char*>(workspace);
   hipStream_t st = (hipStream_t)stream;
-#define GDN_BWD(T_, DK_, NW_, NWS_, ST_)                                                       \
-  return chunk_bwd_launch<T_, DK_, NW_, NWS_, ST_>(d, L, q, k, v, beta, cu_seqlens, d_o, d_final_state, dq, \
+#define GDN_BWD(T_, DK_, NW_, NWS_, NLS_, ST_)                                                       \
+  return chunk_bwd_launch<T_, DK_, NW_, NWS_, NLS_, ST_>(d, L, q, k, v, beta, cu_seqlens, d_o, d_final_state, dq, \
                                                           dk, dv, dg, dbeta, d_initial_state, ws, scale,         \
                                                           use_qk_l2norm, st)
   const bool wide = (V % 128 == 0);
+  const bool solo = one_slab_per_workgroup(d, device_compute_units());
   if (dtype == 1) {
-    if (K == 128 && wide) GDN_BWD(bf16_t, 128, 4, 2, 2);
-    if (K == 128) GDN_BWD(bf16_t, 128, 2, 2, 2);
-    if (wide) GDN_BWD(bf16_t, 64, 4, 2, 2);
-    GDN_BWD(bf16_t, 64, 2, 2, 2);
+    if (K == 128 && wide && solo) GDN_BWD(bf16_t, 128, 4, 1, 2, 2);
+    if (K == 128 && wide) GDN_BWD(bf16_t, 128, 4, 2, 2, 2);
+    if (K == 128) GDN_BWD(bf16_t, 128, 2, 2, 2, 2);
+    if (wide) GDN_BWD(bf16_t, 64, 4, 2, 2, 2);
+    GDN_BWD(bf16_t, 64, 2, 2, 2, 2);
   } else {
-    if (K == 128) GDN_BWD(float, 128, 2, 2, 1);
-    GDN_BWD(float, 64, 2, 2, 2);
+    if (K == 128) GDN_BWD(float, 128, 2, 2, 2, 1);
+    GDN_BWD(float, 64, 2, 2, 2, 2);
   }
 #undef GDN_BWD
 }

@@ -381,13 +381,13 @@ template <typename T, int DK, int NW, int STAGES> struct StateSmem {
   static constexpr int bytes = STAGES * stage;
 };
 
-template <typename T, int DK, int NW, int STAGES>
-__global__ __launch_bounds__(128 * NW) void chunk_state_kernel(
+template <typename T, int DK, int NW, int NL, int STAGES>
+__global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_kernel(
     const T* __restrict__ kdf, const T* __restrict__ w, const T* __restrict__ uf, const float* __restrict__ G,
     const float* __restrict__ h0, float* __restrict__ ht, T* __restrict__ vf, T* __restrict__ hf,
     const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int Hv, int V) {
   using SM = StateSmem<T, DK, NW, STAGES>;
-  constexpr int NT = 64 * NW, VEC = Elem<T>::kVec;
+  constexpr int NT = 64 * NL, VEC = Elem<T>::kVec;   // loader threads
   constexpr int NKT = DK / 32;
   constexpr int CW = 64 * (DK / VEC) / NT, CUL = NW * 2048 / VEC / NT;
   static_assert(64 * (DK / VEC) % NT == 0 && (NW * 2048 / VEC) % NT == 0, "tile chunks must divide over the loaders");
@@ -402,7 +402,7 @@ __global__ __launch_bounds__(128 * NW) void chunk_state_kernel(
 
   if (wave >= NW) {
     // ================= loader waves: straight 16-byte copies =================
-    const int lt = tid - NT;
+    const int lt = tid - 64 * NW;
     // DEPTH register sets: chunk j sits in set j % DEPTH from the iteration that requests it (j - DEPTH - 1) to the
     // one that copies it to LDS (j - 1), so global loads have DEPTH chunk periods to arrive
     constexpr int DEPTH = (STAGES == 2) ? 3 : 1;
@@ -643,7 +643,7 @@ template <typename K> static int set_lds(K kernel, int bytes) {
                                   bytes);
 }
 
-template <typename T, int DK, int BVP, int NW, int NWS, int STAGES>
+template <typename T, int DK, int BVP, int NW, int NWS, int NLS, int STAGES>
 static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const void* q, const void* k, const void* v,
                             const float* g, const float* beta, const float* h0, const int64_t* cu, void* o, float* ht,
                             unsigned char* ws, float scale, int l2norm, bool with_backward, hipStream_t st) {
@@ -675,10 +675,10 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
                d.Hv, d.V, scale, l2norm);
   }
   {
-    auto kern = chunk_state_kernel<T, DK, NWS, STAGES>;
+    auto kern = chunk_state_kernel<T, DK, NWS, NLS, STAGES>;
     constexpr int smem = StateSmem<T, DK, NWS, STAGES>::bytes;
     if (int e = set_lds(kern, smem)) return e;
-    GDN_LAUNCH(kKernStateFwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NWS)), dim3(128 * NWS), smem, st,
+    GDN_LAUNCH(kKernStateFwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NWS)), dim3(64 * (NWS + NLS)), smem, st,
                (const T*)KDF, (const T*)W, (const T*)UF, (const float*)G, h0, ht, VF, HF, cu,
                (const int*)chunk_offsets, d.T, d.Hv, d.V);
   }
@@ -693,6 +693,21 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   return (int)hipGetLastError();
 }
 
+}  // namespace gdn
+
+namespace gdn {
+int device_compute_units() {
+  static int cus = 0;   // one device type per process; a wrong guess only costs speed
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      cus = n;
+    else
+      cus = 256;
+  }
+  return cus;
+}
 }  // namespace gdn
 
 extern "C" int64_t gdn_chunk_workspace_bytes(int B, int T, int N, int Hqk, int Hv, int K, int V, int dtype,
@@ -719,20 +734,22 @@ extern "C" int gdn_chunk_fwd(const void* q, const void* k, const void* v, const 
   if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
   unsigned char* ws = static_cast<unsigned char*>(workspace);
   hipStream_t st = (hipStream_t)stream;
-#define GDN_FWD(T_, DK_, BVP_, NW_, NWS_, ST_)                                                                        \
-  return chunk_fwd_launch<T_, DK_, BVP_, NW_, NWS_, ST_>(d, L, q, k, v, g, beta, initial_state, cu_seqlens, o, final_state, \
+#define GDN_FWD(T_, DK_, BVP_, NW_, NWS_, NLS_, ST_)                                                                        \
+  return chunk_fwd_launch<T_, DK_, BVP_, NW_, NWS_, NLS_, ST_>(d, L, q, k, v, g, beta, initial_state, cu_seqlens, o, final_state, \
                                                    ws, scale, use_qk_l2norm, with_bwd, st)
   const bool wide = (V % 128 == 0);
+  const bool solo = one_slab_per_workgroup(d, device_compute_units());
   if (dtype == 1) {
-    if (K == 128 && wide) GDN_FWD(bf16_t, 128, 128, 4, 2, 2);
-    if (K == 128) GDN_FWD(bf16_t, 128, 64, 2, 2, 2);
-    if (K == 64 && wide) GDN_FWD(bf16_t, 64, 128, 4, 2, 2);
-    GDN_FWD(bf16_t, 64, 64, 2, 2, 2);
+    if (K == 128 && wide && solo) GDN_FWD(bf16_t, 128, 128, 4, 1, 2, 2);
+    if (K == 128 && wide) GDN_FWD(bf16_t, 128, 128, 4, 2, 2, 2);
+    if (K == 128) GDN_FWD(bf16_t, 128, 64, 2, 2, 2, 2);
+    if (K == 64 && wide) GDN_FWD(bf16_t, 64, 128, 4, 2, 2, 2);
+    GDN_FWD(bf16_t, 64, 64, 2, 2, 2, 2);
   } else {
-    if (K == 128 && wide) GDN_FWD(float, 128, 64, 4, 4, 1);
-    if (K == 128) GDN_FWD(float, 128, 64, 2, 2, 1);
-    if (wide) GDN_FWD(float, 64, 64, 4, 4, 2);
-    GDN_FWD(float, 64, 64, 2, 2, 2);
+    if (K == 128 && wide) GDN_FWD(float, 128, 64, 4, 4, 4, 1);
+    if (K == 128) GDN_FWD(float, 128, 64, 2, 2, 2, 1);
+    if (wide) GDN_FWD(float, 64, 64, 4, 4, 4, 2);
+    GDN_FWD(float, 64, 64, 2, 2, 2, 2);
   }
 #undef GDN_FWD
 }
