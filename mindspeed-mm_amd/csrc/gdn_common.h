@@ -4,13 +4,15 @@
 //   * wavefront = 64 lanes; workgroups are 256 threads (4 waves) unless stated otherwise.
 //   * chunk = 64 tokens.  A "tile" in LDS is [rows][ld] with ld = cols + 16 bytes of padding so that
 //     16-byte fragment reads of consecutive rows fall into different banks.
-//   * every tensor-core contraction goes through mma32<>: one wave accumulates one 32x32 fp32 tile
-//     C[i][j] += sum_k A[i][k] * B[k][j] with operands read from LDS.
+//   * every matrix-core contraction accumulates one 32x32 fp32 tile per wave, C[i][j] += sum_k A[i][k] * B[k][j]:
 //       bf16: v_mfma_f32_32x32x16_bf16   lane l holds A[l%32][8*(l/32)+0..7] and B[8*(l/32)+0..7][l%32]
 //       fp32: v_mfma_f32_32x32x2_f32     lane l holds A[l%32][l/32]          and B[l/32][l%32]
 //     accumulator register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32].
 //     The k index inside one instruction may be permuted freely as long as A and B agree; the fp32
 //     path uses that to read 4 consecutive k per lane with one 16-byte load.
+//     Operands come from LDS tiles (mma32<>) or, mostly, as "fragments": the registers a lane feeds to the
+//     instruction, kept together per 32x32 tile (AccB<>).  Tiles travel between kernels, and between waves through
+//     LDS, in that fragment order, and change orientation by a pass through the matrix core (mfma_transpose).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -62,9 +64,6 @@ template <> struct Elem<f16_t> {
 // padded leading dimension (in elements) of an LDS tile with `cols` columns
 template <typename T> __device__ __host__ constexpr int lds_ld(int cols) { return cols + 16 / (int)sizeof(T); }
 
-// compiler-only fence: keeps the scheduler from hoisting a later phase's LDS/global loads (and their registers)
-// above it.  No instruction is emitted.
-#define GDN_PHASE_FENCE() asm volatile("" ::: "memory")
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding global load
 // and store of the wave (vmcnt(0)), which would serialise a software pipeline whose whole point is to keep global
 // loads in flight across the barrier; kernels that hand data between waves through LDS only use this one.
@@ -95,10 +94,6 @@ template <typename T> __device__ __forceinline__ void load16_to_lds(const T* src
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                    (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
 }
-// makes a loop-invariant value opaque inside a loop so that the address arithmetic derived from it is recomputed
-// where it is used instead of being hoisted out of the loop and held in registers for its whole duration
-#define GDN_OPAQUE(x) asm volatile("" : "+r"(x))
-
 __device__ __forceinline__ int imin(int a, int b) { return a < b ? a : b; }
 __device__ __forceinline__ int imax(int a, int b) { return a > b ? a : b; }
 
@@ -141,17 +136,7 @@ template <typename T> __device__ __forceinline__ Vec16<T> zero16() {
 // global -> LDS tile loads.  The tile has 64 rows (tokens) and COLS columns; rows >= nvalid are
 // zero filled (zero padding of a ragged last chunk is exact for the gated delta rule).
 // ---------------------------------------------------------------------------------------------
-template <typename T, int COLS, int ROWS = kChunk>
-__device__ __forceinline__ void load_tile(T* lds, int ld, const T* g, int64_t row_stride, int nvalid, int tid) {
-  constexpr int V = Elem<T>::kVec, CPR = COLS / V;
-  for (int c = tid; c < ROWS * CPR; c += kThreads) {
-    const int row = c / CPR, cc = c % CPR;
-    Vec16<T> v = row < nvalid ? ld16(g + (int64_t)row * row_stride + cc * V) : zero16<T>();
-    st16(lds + row * ld + cc * V, v);
-  }
-}
-
-// same, each row multiplied by rowscale[row] (fp32, in LDS)
+// each row multiplied by rowscale[row] (fp32, in LDS)
 template <typename T, int COLS>
 __device__ __forceinline__ void load_tile_scaled(T* lds, int ld, const T* g, int64_t row_stride, int nvalid,
                                                  const float* rowscale, int tid) {
@@ -327,37 +312,11 @@ template <typename T> __device__ __forceinline__ void mma32_ff(f32x16& d, const 
 #pragma unroll
   for (int kg = 0; kg < AccK<T>::kGroups; ++kg) mfma_kgroup<T>(d, a.f[kg], b.f[kg]);
 }
-// d(32x32) += A[32 rows][KLEN] * B[32 rows][KLEN]^T, both in LDS with the contraction index contiguous and read with
-// 8-byte (bf16) accesses, so rows only need 8-byte alignment (transposed tiles with a leading dimension of 68)
-template <typename T, int KLEN>
-__device__ __forceinline__ void mma32_ss(f32x16& d, const T* arow, const T* brow) {
-  constexpr int G = KGroup<T>::kLen;
-#pragma unroll
-  for (int kg = 0; kg < KLEN / G; ++kg) mfma_kgroup<T>(d, frag_a_split<T>(arow + G * kg), frag_a_split<T>(brow + G * kg));
-}
 // fragments of a tile stored in LDS with the contraction index contiguous: row = &tile[row of this lane][k0]
 template <typename T> __device__ __forceinline__ void frags_from_lds(AccB<T>& out, const T* row) {
   constexpr int G = KGroup<T>::kLen;
 #pragma unroll
   for (int kg = 0; kg < AccK<T>::kGroups; ++kg) out.f[kg] = frag_a_split<T>(row + G * kg);
-}
-
-// One 32x32 tile in fragment order (global memory) -> LDS, row-major at lds[(row0+i)*ld + col0+j]; one wave.
-template <typename T>
-__device__ __forceinline__ void frag_tile_to_lds(T* lds, int ld, int row0, int col0, const T* tile) {
-  const int lane = threadIdx.x & 63, col = lane & 31, half = lane >> 5;
-  AccB<T> f;
-  f.load(tile);
-#pragma unroll
-  for (int g = 0; g < AccK<T>::kGroups; ++g) {
-    Vec16<T> v;
-    v.raw = f.f[g];
-#pragma unroll
-    for (int e = 0; e < Elem<T>::kVec; ++e) {
-      const int row = (sizeof(T) == 2) ? 16 * g + 8 * (e >> 2) + 4 * half + (e & 3) : 8 * g + 4 * half + e;
-      lds[(row0 + row) * ld + col0 + col] = Elem<T>::from_f(v.get(e));
-    }
-  }
 }
 
 // Cross-lane transpose through the matrix core.  A tile held as fragments with (lane <-> a, registers <-> b)
@@ -391,21 +350,6 @@ __device__ __forceinline__ f32x16 mfma_transpose(const AccB<T>& x, const Identit
   return c;
 }
 
-// global -> LDS transposed staging: tile[64 rows][COLS] in memory becomes lds[COLS][ld] (rows contiguous), each
-// row optionally scaled.  Lanes walk rows fastest so that the 2-byte scattered LDS writes do not conflict.
-template <typename T, int COLS, int NT>
-__device__ __forceinline__ void load_tile_t(T* lds, int ld, const T* g, int64_t row_stride, int nvalid, int tid,
-                                            const float* rowscale = nullptr) {
-  constexpr int V = Elem<T>::kVec, CPR = COLS / V;
-  for (int c = tid; c < kChunk * CPR; c += NT) {
-    const int row = c % kChunk, cc = c / kChunk;
-    Vec16<T> v = row < nvalid ? ld16(g + (int64_t)row * row_stride + cc * V) : zero16<T>();
-    const float s = rowscale ? rowscale[row] : 1.f;
-#pragma unroll
-    for (int e = 0; e < V; ++e) lds[(cc * V + e) * ld + row] = Elem<T>::from_f(rowscale ? v.get(e) * s : v.get(e));
-  }
-}
-
 __device__ __forceinline__ f32x16 acc_zero() {
   f32x16 z;
 #pragma unroll
@@ -416,12 +360,6 @@ __device__ __forceinline__ f32x16 acc_zero() {
 __device__ __forceinline__ int acc_row(int r) { return 8 * (r >> 2) + 4 * ((threadIdx.x & 63) >> 5) + (r & 3); }
 __device__ __forceinline__ int acc_col() { return threadIdx.x & 31; }
 
-// accumulator tile -> LDS, row-major: dst[(i0+i)*ld + j0 + j]
-template <typename T> __device__ __forceinline__ void acc_to_lds(const f32x16& acc, T* dst, int ld, int i0, int j0) {
-  const int j = j0 + acc_col();
-#pragma unroll
-  for (int r = 0; r < 16; ++r) dst[(i0 + acc_row(r)) * ld + j] = Elem<T>::from_f(acc[r]);
-}
 // accumulator tile -> LDS, transposed: dst[(j0+j)*ld + i0 + i].  Registers 4g..4g+3 are four consecutive rows, so a
 // lane writes four contiguous elements at a time (ld must be a multiple of 4 elements).
 template <typename T> __device__ __forceinline__ void acc_to_lds_t(const f32x16& acc, T* dst, int ld, int i0, int j0) {
@@ -455,42 +393,11 @@ __device__ __forceinline__ f32x16 rows_ld(const float* arr, int i0) {
   }
   return v;
 }
-// accumulator tile -> global rows (row-major, only rows < nvalid)
-template <typename T>
-__device__ __forceinline__ void acc_to_global(const f32x16& acc, T* g, int64_t row_stride, int i0, int j0, int nvalid) {
-  const int j = j0 + acc_col();
-#pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int i = i0 + acc_row(r);
-    if (i < nvalid) g[(int64_t)i * row_stride + j] = Elem<T>::from_f(acc[r]);
-  }
-}
-// global rows -> accumulator tile (rows >= nvalid read as zero)
-template <typename T>
-__device__ __forceinline__ f32x16 acc_from_global(const T* g, int64_t row_stride, int i0, int j0, int nvalid) {
-  f32x16 a;
-  const int j = j0 + acc_col();
-#pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int i = i0 + acc_row(r);
-    a[r] = i < nvalid ? Elem<T>::to_f(g[(int64_t)i * row_stride + j]) : 0.f;
-  }
-  return a;
-}
-
-// Sum over the 16 lanes of a DPP row (lanes 16r .. 16r+15), every lane gets the result.  Data-parallel-primitive
-// moves run at VALU speed; wave shuffles (ds_bpermute) go through the LDS crossbar and cost ~10x more.
+// Data-parallel-primitive moves between lanes run at VALU speed; wave shuffles (ds_bpermute) go through the LDS
+// crossbar and cost ~10x more.
 template <int CTRL> __device__ __forceinline__ float dpp_mov(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
 }
-__device__ __forceinline__ float row16_sum(float v) {
-  v += dpp_mov<0xB1>(v);    // quad_perm [1,0,3,2]
-  v += dpp_mov<0x4E>(v);    // quad_perm [2,3,0,1]
-  v += dpp_mov<0x141>(v);   // row_half_mirror
-  v += dpp_mov<0x140>(v);   // row_mirror
-  return v;
-}
-
 // sum over aligned groups of N neighbouring lanes (N a power of two <= 32), every lane gets the result
 template <int N> __device__ __forceinline__ float lane_group_sum(float v) {
   if constexpr (N >= 2) v += dpp_mov<0xB1>(v);
