@@ -247,7 +247,7 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_bwd_kernel(
 // chunk_bwd_local_kernel, per (chunk, head), 4 waves: everything of the backward pass that is local to a chunk once
 // the reverse recurrence has left dS' and dV' behind.  Wave w owns the 32 K-columns [32w, 32w+32) of dQ, dK, dW and
 // the 32x32 tile (w/2, w%2) of the 64x64 intra-chunk matrices.
-//   pre-pass: R = Tm^T dV' per V block -> dv = beta R, dbeta += <R, v>
+//   pre-pass: R = Tm^T dV' per V block -> dv = beta R
 //   main loop over 32-column V blocks:
 //     v_new, dV', dO, S, dS' arrive in fragment order with (lane <-> V column); the contractions run over V, so each
 //     tile is turned through the matrix core (mfma_transpose) into (lane <-> token / K column, registers <-> V).
@@ -301,7 +301,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   float* rk1 = rq + 256;   // <k_i, dK_i> before the terms that come back through W
   float* rbk = rk1 + 256;  // e^G <P_i,k_i> + <E_i,k_i>: dbeta without the V part; times beta it is part of dG and <k,dK>
   float* rf = rbk + 256;   // <F_i, k_i>
-  float* rv = rf + 256;    // <R_i, v_i>
+  float* rv = rf + 256;    // <R_i, v_i>, taken as the column sums of Tm . (dV' V^T)
   float* wsum = rv + 256;  // per wave: <S,dS'> [0..3], sum_i <k_i, dK_inter_i> [4..7]
 
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
@@ -391,7 +391,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     o.pack(mfma_transpose<T>(f, id));
     return o;
   };
-  // pre-pass: R = Tm^T dV' per 32-column V block (blocks dealt to the waves): dv = beta R, <R, v>.  Done before the
+  // pre-pass: R = Tm^T dV' per 32-column V block (blocks dealt to the waves): dv = beta R.  Done before the
   // accumulators of the main loop exist; the store patch is this wave's S / dS' slot of the stage not yet in use.
   for (int vblk = wave; vblk < nblk; vblk += 4) {
     AccB<T> fdv[2];
@@ -400,15 +400,9 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     T* patch = stage0 + SM::stage_elems + SM::st_priv + wave * 2048;
 #pragma unroll
     for (int rj = 0; rj < 2; ++rj) {
-      f32x16 R = acc_zero(), p;
+      f32x16 R = acc_zero();
 #pragma unroll
       for (int t = rj; t < 2; ++t) mma32_ff<T>(R, tm_t(rj, t), fdv[t]);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = imin(32 * rj + acc_row(r), nvalid - 1);
-        p[r] = R[r] * Elem<T>::to_f(v[((tok0 + row) * Hv + h) * V + 32 * vblk + acc_col()]);
-      }
-      rows_add(p, rv, 32 * rj);
       const f32x16 bsr = rows_ld(bs, 32 * rj);
 #pragma unroll
       for (int r = 0; r < 16; ++r) R[r] *= bsr[r];
@@ -579,6 +573,14 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     }
   }
   GDN_LDS_BARRIER();   // the ds tiles and the dW tiles are consumed
+  if (lower) {  // <R_t, v_t> = sum_i Tm[i][t] (dV' V^T)[i][t]: column sums of Tm . a2, no second pass over V needed
+    const f32x16 tmv = tm_t(tj, ti).unpack();   // Tm tile (ti, tj) with lane <-> column, registers <-> row
+    float sv = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sv += a2[r] * tmv[r];
+    sv += __shfl_xor(sv, 32);
+    if (lane < 32) rv[wave * 64 + 32 * tj + lane] += sv;
+  }
   {  // dTm[i][j] = beta_j (e^{G_j} a1 + a2), i > j, handed on in T form
     const int j = 32 * tj + acc_col();
     const float bj = bs[j], ej = egs[j];
