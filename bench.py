@@ -67,8 +67,8 @@ def kernel_algorithmic_bytes(K, V, grp, e=2, C=64):
     cc = [64,64] tile, row = 64 fp32 values."""
     tk, tv, st, cc, row = C * K * e, C * V * e, K * V * e, C * C * e, C * 4
     return {
-        # q, k, v, g, beta -> G, Tm, W, U, Aq, decayed K^T, W^T, K, scaled Q^T tiles, normalised q and 1/|q|, 1/|k| once per group
-        "chunk_prep_kernel": 2 * tk + tv + 2 * row + row + 2 * cc + tk + tv + tk + 3 * tk + (tk + 2 * row) // grp,
+        # q, k, v, g, beta -> G, Tm, Aq, W, U, decayed K^T, W^T tiles; once per q/k group: K, Q^T tiles, normalised q, 1/|q|, 1/|k|
+        "chunk_prep_kernel": 2 * tk + tv + 2 * row + row + 2 * cc + tk + tv + tk + tk + (3 * tk + 2 * row) // grp,
         "chunk_state_kernel": 2 * tk + tv + row + tv + st,          # W, decayed K^T, U, G -> v_new, state before the chunk
         "chunk_out_kernel": tk + cc + tv + st + row + tv,            # q, Aq, v_new, state, G -> o
         "chunk_state_bwd_kernel": 3 * tk + cc + tv + row + tv + st,  # K, Q^T, W^T, Aq, dO, G -> dv_new, dS

@@ -32,8 +32,8 @@ struct ChunkWorkspace {
   int64_t HF;             // T [chunks,Hv,V/32,K/32] state BEFORE each chunk, tile = (32 rows of K) x (32 columns of V)
   int64_t fwd_bytes;
   int64_t WF;             // T [chunks,Hv,K/32,2]    W^T as A operand (written by the forward when a backward follows)
-  int64_t QSF;            // T [chunks,Hv,K/32,2]    (scale e^G . Q)^T as A operand
-  int64_t KAF;            // T [chunks,Hv,K/32,2]    K as A operand: tile = (32 tokens) x (32 columns of K)
+  int64_t QTF;            // T [chunks,Hqk,K/32,2]   Q^T as A operand: tile = (32 columns of K) x (32 tokens)
+  int64_t KAF;            // T [chunks,Hqk,K/32,2]   K as A operand: tile = (32 tokens) x (32 columns of K)
   int64_t DVF;            // T [chunks,Hv,V/32,2]    d(v_new)
   int64_t DHF;            // T [chunks,Hv,V/32,K/32] gradient of the state AFTER each chunk
   int64_t total_bytes;
@@ -59,8 +59,8 @@ inline ChunkWorkspace chunk_workspace_layout(const ChunkDims& d, int elem_bytes)
   w.HF = take(nc * d.Hv * d.V * d.K * elem_bytes);
   w.fwd_bytes = off;
   w.WF = take(nc * 64 * d.Hv * d.K * elem_bytes);
-  w.QSF = take(nc * 64 * d.Hv * d.K * elem_bytes);
-  w.KAF = take(nc * 64 * d.Hv * d.K * elem_bytes);
+  w.QTF = take(nc * 64 * d.Hqk * d.K * elem_bytes);
+  w.KAF = take(nc * 64 * d.Hqk * d.K * elem_bytes);
   w.DVF = take(nc * 64 * d.Hv * d.V * elem_bytes);
   w.DHF = take(nc * d.Hv * d.V * d.K * elem_bytes);
   w.total_bytes = off;

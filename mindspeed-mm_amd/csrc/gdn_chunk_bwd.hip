@@ -24,24 +24,24 @@ namespace gdn {
 // ---------------------------------------------------------------------------------------------
 // chunk_state_bwd_kernel: the reverse recurrence, mirror of chunk_state_kernel.  One compute wave owns a 32-column
 // slab of dS[K, 32] in fp32 accumulators and per chunk (last to first) does
-//     dV' = e^{G_last-G} . (K dS) + dv_local          dS <- e^{G_last} dS + (scale e^G . Q)^T dO - W^T dV'
+//     dV' = e^{G_last-G} . (K dS) + dv_local          dS <- e^{G_last} dS + Q^T (scale e^G . dO) - W^T dV'
 // with dS and dV' used as B operands straight from accumulator registers.  dS (gradient of the state AFTER the
 // chunk) and dV' leave in fragment order.  Loader waves copy the A operands (K, Q^T, W^T: `big` stages) from
 // contiguous fragment-order blocks, and the `small` stage: the slab's dO rows as they lie in memory plus the
 // forward pass's tril(Q K^T . Gam) tiles, from which the compute waves form dv_local = scale Aq^T dO themselves.
 // ---------------------------------------------------------------------------------------------
 template <typename T, int DK, int NW, int STAGES> struct StateBwdSmem {
-  static constexpr int big = 3 * 64 * DK * (int)sizeof(T) + 64 * 4 + 16;   // K, Q^T, W^T images, decay[64], G_last
+  static constexpr int big = 3 * 64 * DK * (int)sizeof(T) + 2 * 64 * 4 + 16;   // K, Q^T, W^T images, decay[64], G_last, scale e^G [64]
   static constexpr int off_small = STAGES * big;            // dO rows of the slab [64][32 NW] | tril(Q K^T . Gam) tiles [4]
   static constexpr int bytes = off_small + (NW * 2048 + 4096) * (int)sizeof(T);
 };
 
 template <typename T, int DK, int NW, int NL, int STAGES>
 __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_bwd_kernel(
-    const T* __restrict__ kaf, const T* __restrict__ qsf, const T* __restrict__ wf, const T* __restrict__ aqf,
+    const T* __restrict__ kaf, const T* __restrict__ qtf, const T* __restrict__ wf, const T* __restrict__ aqf,
     const T* __restrict__ dO, const float* __restrict__ G, const float* __restrict__ dht, float* __restrict__ dh0,
     T* __restrict__ dvf, T* __restrict__ dhf, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets,
-    int T_len, int Hv, int V, float scale) {
+    int T_len, int Hqk, int Hv, int V, float scale) {
   using SM = StateBwdSmem<T, DK, NW, STAGES>;
   constexpr int NT = 64 * NL, VEC = Elem<T>::kVec, NKT = DK / 32;   // NT loader threads
   constexpr int CW = 64 * (DK / VEC) / NT, CUL = NW * 2048 / VEC / NT, CAQ = 4096 / VEC / NT, TILE = 64 * DK;
@@ -64,17 +64,17 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_bwd_kernel(
     const int lt = tid - 64 * NW;
     constexpr int DEPTH = (STAGES == 2) ? 2 : 1;
     Vec16<T> pk[DEPTH][CW], pq[DEPTH][CW], pw[DEPTH][CW], pa[DEPTH][CAQ], pd[DEPTH][CUL];
-    float pdec[DEPTH], pgl[DEPTH];
+    float pdec[DEPTH], pgl[DEPTH], pqs[DEPTH];
     auto issue = [&](int st, int set) {
       const int c = nchunks - 1 - st;
       const int64_t tok0 = bos + (int64_t)c * kChunk;
       const int nvalid = imin(kChunk, len - c * kChunk);
-      const int64_t ch = (chunk_base + c) * Hv + h;
+      const int64_t ch = (chunk_base + c) * Hv + h, chq = (chunk_base + c) * Hqk + h / (Hv / Hqk);
 #pragma unroll
       for (int i = 0; i < CW; ++i) {
         const int id = lt + i * NT;
-        pk[set][i] = ld16(kaf + ch * TILE + id * VEC);
-        pq[set][i] = ld16(qsf + ch * TILE + id * VEC);
+        pk[set][i] = ld16(kaf + chq * TILE + id * VEC);
+        pq[set][i] = ld16(qtf + chq * TILE + id * VEC);
         pw[set][i] = ld16(wf + ch * TILE + id * VEC);
       }
 #pragma unroll
@@ -86,7 +86,9 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_bwd_kernel(
                                   : zero16<T>();
       }
       pgl[set] = G[(tok0 + nvalid - 1) * Hv + h];
-      pdec[set] = __expf(pgl[set] - G[(tok0 + imin(lt & 63, nvalid - 1)) * Hv + h]);
+      const float gt = G[(tok0 + imin(lt & 63, nvalid - 1)) * Hv + h];
+      pdec[set] = __expf(pgl[set] - gt);
+      pqs[set] = scale * __expf(gt);
     };
     auto commit_big = [&](int set, int buf) {
       unsigned char* base = gdn_smem + buf * SM::big;
@@ -101,7 +103,7 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_bwd_kernel(
         st16(Qa + id * VEC, pq[set][i]);
         st16(Wa + id * VEC, pw[set][i]);
       }
-      if (lt < 64) dec[lt] = pdec[set];
+      if (lt < 64) { dec[lt] = pdec[set]; dec[68 + lt] = pqs[set]; }
       if (lt == 0) dec[64] = pgl[set];
     };
     auto commit_small = [&](int set) {
@@ -217,7 +219,16 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_bwd_kernel(
     dvb[1].store_stream(dvf + (tile0 * 2 + 1) * 1024);
     dvb[0].negate();
     dvb[1].negate();
-    // dS <- e^{G_last} dS + (scale e^G . Q)^T dO - W^T dV'
+    // dS <- e^{G_last} dS + Q^T (scale e^G . dO) - W^T dV'   (the per-token factor rides on dO, so that the Q^T tiles
+    // are the same for every value head of a q/k group)
+    {
+      const f32x16 q0 = rows_ld(dec + 68, 0), q1 = rows_ld(dec + 68, 32);
+      f32x16 d0 = dob[0].unpack(), d1 = dob[1].unpack();
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { d0[r] *= q0[r]; d1[r] *= q1[r]; }
+      dob[0].pack(d0);
+      dob[1].pack(d1);
+    }
     const float eg = __expf(glast);
 #pragma unroll
     for (int kt = 0; kt < NKT; ++kt) {
@@ -355,7 +366,8 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
 #pragma unroll
     for (int j = 0; j < 2 * NKT * KG / 4; ++j) {
       const int piece = 4 * j + wave;
-      load16_to_lds(kaf + ch * (NKT * 2048) + (piece * 64 + lane) * VEC, st + piece * 64 * VEC);
+      load16_to_lds(kaf + ((int64_t)blockIdx.x * Hqk + hq) * (NKT * 2048) + (piece * 64 + lane) * VEC,
+                    st + piece * 64 * VEC);
     }
     if (has_k) {
       constexpr int LPR = 32 / VEC, RPP = 64 / LPR;
@@ -718,7 +730,7 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   const T* WF = reinterpret_cast<const T*>(ws + L.WF);
   const T* VF = reinterpret_cast<const T*>(ws + L.VF);
   const T* HF = reinterpret_cast<const T*>(ws + L.HF);
-  const T* QSF = reinterpret_cast<const T*>(ws + L.QSF);
+  const T* QTF = reinterpret_cast<const T*>(ws + L.QTF);
   const T* KAF = reinterpret_cast<const T*>(ws + L.KAF);
   T* DVF = reinterpret_cast<T*>(ws + L.DVF);
   T* DHF = reinterpret_cast<T*>(ws + L.DHF);
@@ -729,7 +741,8 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     constexpr int smem = StateBwdSmem<T, DK, NWS, STAGES>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
     GDN_LAUNCH(kKernStateBwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NWS)), dim3(64 * (NWS + NLS)), smem, st, (const T*)KAF,
-               (const T*)QSF, WF, AQ, (const T*)dO, G, dht, dh0, DVF, DHF, cu, chunk_offsets, d.T, d.Hv, d.V, scale);
+               (const T*)QTF, WF, AQ, (const T*)dO, G, dht, dh0, DVF, DHF, cu, chunk_offsets, d.T, d.Hqk, d.Hv, d.V,
+               scale);
   }
   {
     auto kern = chunk_bwd_local_kernel<T, DK>;

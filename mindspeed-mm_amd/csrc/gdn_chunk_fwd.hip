@@ -105,7 +105,7 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
     const float* __restrict__ beta, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets,
     float* __restrict__ G_out, T* __restrict__ Ai_out, T* __restrict__ W_out, T* __restrict__ U_out,
     T* __restrict__ Aq_out, T* __restrict__ KD_out, T* __restrict__ WF_out, T* __restrict__ KA_out,
-    T* __restrict__ QS_out, T* __restrict__ qn_out, float* __restrict__ rstd_q_out, float* __restrict__ rstd_k_out,
+    T* __restrict__ QT_out, T* __restrict__ qn_out, float* __restrict__ rstd_q_out, float* __restrict__ rstd_k_out,
     int T_len, int N, int Hqk, int Hv, int V, float scale, int l2norm) {
   using SM = PrepSmem<T, DK, BV>;
   constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64, VEC = Elem<T>::kVec;
@@ -182,24 +182,23 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
     IdentityFrag<T> id;
     id.init();
     const float glast = Gs[63];
+    const bool group_first = (h % (Hv / Hqk)) == 0;   // K and Q^T tiles are shared by the value heads of a q/k group
     for (int tt = wave; tt < 2 * (DK / 32); tt += 4) {
       const int tj = tt & 1, kt = tt >> 1;
       const int64_t tile = ((((int64_t)blockIdx.x * Hv + h) * (DK / 32) + kt) * 2 + tj) * 1024;
+      const int64_t gtile = ((((int64_t)blockIdx.x * Hqk + hq) * (DK / 32) + kt) * 2 + tj) * 1024;
       AccB<T> kf;
       frags_from_lds<T>(kf, Ks + (32 * tj + (lane & 31)) * LDK + 32 * kt);
-      if (KA_out != nullptr) kf.store_stream(KA_out + tile);   // K as an A operand (lane <-> token), for the backward pass
+      if (KA_out != nullptr && group_first) kf.store_stream(KA_out + gtile);   // K as an A operand (lane <-> token)
       f32x16 kd = mfma_transpose<T>(kf, id);
 #pragma unroll
       for (int r = 0; r < 16; ++r) kd[r] *= __expf(glast - Gs[32 * tj + acc_row(r)]);
       kf.pack(kd);
       kf.store_stream(KD_out + tile);
-      if (QS_out != nullptr) {   // (scale e^G . Q)^T as an A operand (lane <-> K column), for the backward pass
+      if (QT_out != nullptr && group_first) {   // Q^T as an A operand (lane <-> K column), for the backward pass
         frags_from_lds<T>(kf, Qs + (32 * tj + (lane & 31)) * LDK + 32 * kt);
-        f32x16 qt = mfma_transpose<T>(kf, id);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) qt[r] *= scale * __expf(Gs[32 * tj + acc_row(r)]);
-        kf.pack(qt);
-        kf.store_stream(QS_out + tile);
+        kf.pack(mfma_transpose<T>(kf, id));
+        kf.store_stream(QT_out + gtile);
       }
     }
   }
@@ -663,7 +662,7 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   T* KDF = reinterpret_cast<T*>(ws + L.KDF);
   T* WF = with_backward ? reinterpret_cast<T*>(ws + L.WF) : nullptr;
   T* KAF = with_backward ? reinterpret_cast<T*>(ws + L.KAF) : nullptr;
-  T* QSF = with_backward ? reinterpret_cast<T*>(ws + L.QSF) : nullptr;
+  T* QTF = with_backward ? reinterpret_cast<T*>(ws + L.QTF) : nullptr;
   T* VF = reinterpret_cast<T*>(ws + L.VF);
   T* HF = reinterpret_cast<T*>(ws + L.HF);
   {
@@ -671,7 +670,7 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     constexpr int smem = PrepSmem<T, DK, BVP>::bytes;
     if (int e = set_lds(kern, smem)) return e;
     GDN_LAUNCH(kKernPrep, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, (const T*)v, g, beta, cu,
-               (const int*)chunk_offsets, G, Ai, W, UF, AQ, KDF, WF, KAF, QSF, qn, rstd, rstd + tok * d.Hqk, d.T, d.N, d.Hqk,
+               (const int*)chunk_offsets, G, Ai, W, UF, AQ, KDF, WF, KAF, QTF, qn, rstd, rstd + tok * d.Hqk, d.T, d.N, d.Hqk,
                d.Hv, d.V, scale, l2norm);
   }
   {
