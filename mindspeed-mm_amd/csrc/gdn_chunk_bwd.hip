@@ -85,8 +85,9 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_bwd_kernel(
         pd[set][i] = row < nvalid ? ld16(dO + ((tok0 + row) * Hv + h) * V + blockIdx.y * (32 * NW) + cc * VEC)
                                   : zero16<T>();
       }
-      pgl[set] = G[(tok0 + nvalid - 1) * Hv + h];
-      const float gt = G[(tok0 + imin(lt & 63, nvalid - 1)) * Hv + h];
+      const float* gc = G + ch * 64;
+      pgl[set] = gc[nvalid - 1];
+      const float gt = gc[imin(lt & 63, nvalid - 1)];
       pdec[set] = __expf(pgl[set] - gt);
       pqs[set] = scale * __expf(gt);
     };
@@ -385,7 +386,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   issue(0, 0);
 
   if (tid < 64) {
-    const float gv = G[(tok0 + imin(tid, nvalid - 1)) * Hv + h];
+    const float gv = G[ch * 64 + imin(tid, nvalid - 1)];
     Gs[tid] = gv;
     egs[tid] = __expf(gv);
     bs[tid] = tid < nvalid ? beta[(tok0 + tid) * Hv + h] : 0.f;

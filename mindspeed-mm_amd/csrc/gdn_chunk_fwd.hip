@@ -104,7 +104,7 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ g,
     const float* __restrict__ beta, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets,
     float* __restrict__ G_out, T* __restrict__ Ai_out, T* __restrict__ W_out, T* __restrict__ U_out,
-    T* __restrict__ Aq_out, T* __restrict__ KD_out, T* __restrict__ WF_out, T* __restrict__ KA_out,
+    T* __restrict__ Aq_out, T* __restrict__ KT_out, T* __restrict__ WF_out, T* __restrict__ KA_out,
     T* __restrict__ QT_out, T* __restrict__ qn_out, float* __restrict__ rstd_q_out, float* __restrict__ rstd_k_out,
     int T_len, int N, int Hqk, int Hv, int V, float scale, int l2norm) {
   using SM = PrepSmem<T, DK, BV>;
@@ -138,7 +138,7 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
     Gs[lane] = x;
     bs[lane] = b;
     egs[lane] = b * __expf(x);
-    if (lane < nvalid) G_out[(tok0 + lane) * Hv + h] = x;
+    G_out[((int64_t)blockIdx.x * Hv + h) * 64 + lane] = x;   // 64 contiguous values per chunk and head
   }
   for (int i = tid; i < 64 * kLF; i += kThreads) Ti[i] = 0.f;
   {
@@ -181,20 +181,17 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
   {
     IdentityFrag<T> id;
     id.init();
-    const float glast = Gs[63];
     const bool group_first = (h % (Hv / Hqk)) == 0;   // K and Q^T tiles are shared by the value heads of a q/k group
     for (int tt = wave; tt < 2 * (DK / 32); tt += 4) {
       const int tj = tt & 1, kt = tt >> 1;
-      const int64_t tile = ((((int64_t)blockIdx.x * Hv + h) * (DK / 32) + kt) * 2 + tj) * 1024;
       const int64_t gtile = ((((int64_t)blockIdx.x * Hqk + hq) * (DK / 32) + kt) * 2 + tj) * 1024;
       AccB<T> kf;
       frags_from_lds<T>(kf, Ks + (32 * tj + (lane & 31)) * LDK + 32 * kt);
       if (KA_out != nullptr && group_first) kf.store_stream(KA_out + gtile);   // K as an A operand (lane <-> token)
-      f32x16 kd = mfma_transpose<T>(kf, id);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) kd[r] *= __expf(glast - Gs[32 * tj + acc_row(r)]);
-      kf.pack(kd);
-      kf.store_stream(KD_out + tile);
+      if (group_first) {   // K^T as an A operand (lane <-> K column), for the state update
+        kf.pack(mfma_transpose<T>(kf, id));
+        kf.store_stream(KT_out + gtile);
+      }
       if (QT_out != nullptr && group_first) {   // Q^T as an A operand (lane <-> K column), for the backward pass
         frags_from_lds<T>(kf, Qs + (32 * tj + (lane & 31)) * LDK + 32 * kt);
         kf.pack(mfma_transpose<T>(kf, id));
@@ -375,16 +372,16 @@ template <typename T, int DK, int NW, int STAGES> struct StateSmem {
   static constexpr int off_ws = 0;
   static constexpr int off_kt = off_ws + 64 * DK * (int)sizeof(T);
   static constexpr int off_uf = off_kt + DK * 64 * (int)sizeof(T);
-  static constexpr int off_gl = off_uf + NW * 2048 * (int)sizeof(T);
-  static constexpr int stage = off_gl + 16;
+  static constexpr int off_gl = off_uf + NW * 2048 * (int)sizeof(T);   // e^{G_last - G_t} [64], G_last
+  static constexpr int stage = off_gl + 64 * 4 + 16;
   static constexpr int bytes = STAGES * stage;
 };
 
 template <typename T, int DK, int NW, int NL, int STAGES>
 __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_kernel(
-    const T* __restrict__ kdf, const T* __restrict__ w, const T* __restrict__ uf, const float* __restrict__ G,
+    const T* __restrict__ ktf, const T* __restrict__ w, const T* __restrict__ uf, const float* __restrict__ G,
     const float* __restrict__ h0, float* __restrict__ ht, T* __restrict__ vf, T* __restrict__ hf,
-    const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int Hv, int V) {
+    const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int Hqk, int Hv, int V) {
   using SM = StateSmem<T, DK, NW, STAGES>;
   constexpr int NT = 64 * NL, VEC = Elem<T>::kVec;   // loader threads
   constexpr int NKT = DK / 32;
@@ -406,7 +403,7 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_kernel(
     // one that copies it to LDS (j - 1), so global loads have DEPTH chunk periods to arrive
     constexpr int DEPTH = (STAGES == 2) ? 3 : 1;
     Vec16<T> pw[DEPTH][CW], pk[DEPTH][CW], pu[DEPTH][CUL];
-    float glast[DEPTH];
+    float glast[DEPTH], pdec[DEPTH];
     auto issue = [&](int c, int set) {      // global -> registers
       const int64_t tok0 = bos + (int64_t)c * kChunk;
       const int nvalid = imin(kChunk, len - c * kChunk);
@@ -414,12 +411,14 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_kernel(
       for (int i = 0; i < CW; ++i) {
         const int id = lt + i * NT;
         pw[set][i] = ld16(w + ((chunk_base + c) * Hv + h) * (64 * DK) + id * VEC);
-        pk[set][i] = ld16(kdf + ((chunk_base + c) * Hv + h) * (64 * DK) + id * VEC);
+        pk[set][i] = ld16(ktf + ((chunk_base + c) * Hqk + h / (Hv / Hqk)) * (64 * DK) + id * VEC);   // shared by the group
       }
       const T* ug = uf + (((chunk_base + c) * Hv + h) * (V / 32) + blockIdx.y * NW) * 2048;
 #pragma unroll
       for (int i = 0; i < CUL; ++i) pu[set][i] = ld16(ug + (lt + i * NT) * VEC);
-      glast[set] = G[(tok0 + nvalid - 1) * Hv + h];
+      const float* gc = G + ((chunk_base + c) * Hv + h) * 64;
+      glast[set] = gc[nvalid - 1];
+      pdec[set] = __expf(glast[set] - gc[imin(lt & 63, nvalid - 1)]);
     };
     auto commit = [&](int set, int buf) {   // registers -> LDS stage
       unsigned char* base = gdn_smem + buf * SM::stage;
@@ -434,7 +433,9 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_kernel(
       }
 #pragma unroll
       for (int i = 0; i < CUL; ++i) st16(Uf + (lt + i * NT) * VEC, pu[set][i]);
-      if (lt == 0) *reinterpret_cast<float*>(base + SM::off_gl) = glast[set];
+      float* dec = reinterpret_cast<float*>(base + SM::off_gl);
+      if (lt < 64) dec[lt] = pdec[set];
+      if (lt == 0) dec[64] = glast[set];
     };
     if (STAGES == 2) {
       if (nchunks > 0) { issue(0, 0); commit(0, 0); }
@@ -484,7 +485,8 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_kernel(
     const T* Ws = reinterpret_cast<const T*>(base + SM::off_ws);
     const T* KT = reinterpret_cast<const T*>(base + SM::off_kt);
     const T* Uf = reinterpret_cast<const T*>(base + SM::off_uf) + wave * 2048;
-    const float glast = *reinterpret_cast<const float*>(base + SM::off_gl);
+    const float* dec = reinterpret_cast<const float*>(base + SM::off_gl);
+    const float glast = dec[64];
     const int64_t tile0 = ((chunk_base + c) * Hv + h) * (V / 32) + vblk;
 
     AccB<T> Sb[NKT];
@@ -537,7 +539,15 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_kernel(
     Vb[1].pack(p1);
     Vb[0].store_stream(vf + (tile0 * 2 + 0) * 1024);
     Vb[1].store_stream(vf + (tile0 * 2 + 1) * 1024);
-    // S <- e^{G_last} S + (e^{G_last - G} . K)^T V'   (K^T arrives already scaled, as A-operand fragments)
+    {  // the decay of the state update rides on V': (e^{G_last - G} . K)^T V' = K^T (e^{G_last - G} . V'), so that the
+       // K^T tiles are the same for every value head of a q/k group
+      const f32x16 d0 = rows_ld(dec, 0), d1 = rows_ld(dec, 32);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { p0[r] *= d0[r]; p1[r] *= d1[r]; }
+      Vb[0].pack(p0);
+      Vb[1].pack(p1);
+    }
+    // S <- e^{G_last} S + K^T (e^{G_last - G} . V')
     const float eg = __expf(glast);
 #pragma unroll
     for (int kt = 0; kt < NKT; ++kt)
@@ -610,7 +620,7 @@ __global__ __launch_bounds__(64 * NW) void chunk_out_kernel(
     st16(Qs + row * LDK + cc * VEC,
          row < nvalid ? ld16(q + ((tok0 + row) * Hqk + hq) * DK + cc * VEC) : zero16<T>());
   }
-  if (tid < 64) Eg[tid] = __expf(G[(tok0 + imin(tid, nvalid - 1)) * Hv + h]);
+  if (tid < 64) Eg[tid] = __expf(G[ch * 64 + imin(tid, nvalid - 1)]);
   IdentityFrag<T> id;
   id.init();
 #pragma unroll
@@ -659,7 +669,7 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   T* W = reinterpret_cast<T*>(ws + L.WAF);
   T* AQ = reinterpret_cast<T*>(ws + L.AQ);
   T* UF = reinterpret_cast<T*>(ws + L.UF);
-  T* KDF = reinterpret_cast<T*>(ws + L.KDF);
+  T* KTF = reinterpret_cast<T*>(ws + L.KTF);
   T* WF = with_backward ? reinterpret_cast<T*>(ws + L.WF) : nullptr;
   T* KAF = with_backward ? reinterpret_cast<T*>(ws + L.KAF) : nullptr;
   T* QTF = with_backward ? reinterpret_cast<T*>(ws + L.QTF) : nullptr;
@@ -670,7 +680,7 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     constexpr int smem = PrepSmem<T, DK, BVP>::bytes;
     if (int e = set_lds(kern, smem)) return e;
     GDN_LAUNCH(kKernPrep, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, (const T*)v, g, beta, cu,
-               (const int*)chunk_offsets, G, Ai, W, UF, AQ, KDF, WF, KAF, QTF, qn, rstd, rstd + tok * d.Hqk, d.T, d.N, d.Hqk,
+               (const int*)chunk_offsets, G, Ai, W, UF, AQ, KTF, WF, KAF, QTF, qn, rstd, rstd + tok * d.Hqk, d.T, d.N, d.Hqk,
                d.Hv, d.V, scale, l2norm);
   }
   {
@@ -678,8 +688,8 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     constexpr int smem = StateSmem<T, DK, NWS, STAGES>::bytes;
     if (int e = set_lds(kern, smem)) return e;
     GDN_LAUNCH(kKernStateFwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NWS)), dim3(64 * (NWS + NLS)), smem, st,
-               (const T*)KDF, (const T*)W, (const T*)UF, (const float*)G, h0, ht, VF, HF, cu,
-               (const int*)chunk_offsets, d.T, d.Hv, d.V);
+               (const T*)KTF, (const T*)W, (const T*)UF, (const float*)G, h0, ht, VF, HF, cu,
+               (const int*)chunk_offsets, d.T, d.Hqk, d.Hv, d.V);
   }
   {
     auto kern = chunk_out_kernel<T, DK, NW>;
