@@ -24,20 +24,20 @@ namespace gdn {
 // ---------------------------------------------------------------------------------------------
 // chunk_state_bwd_kernel: the reverse recurrence, mirror of chunk_state_kernel.  One compute wave owns a 32-column
 // slab of dS[K, 32] in fp32 accumulators and per chunk (last to first) does
-//     dV' = e^{G_last-G} . (K dS) + dv_local          dS <- e^{G_last} dS + Q^T (scale e^G . dO) - W^T dV'
+//     dV' = (e^{G_last-G} . K) dS + dv_local          dS <- e^{G_last} dS + Q^T (scale e^G . dO) - W^T dV'
 // with dS and dV' used as B operands straight from accumulator registers.  dS (gradient of the state AFTER the
 // chunk) and dV' leave in fragment order.  Loader waves copy the A operands (K, Q^T, W^T: `big` stages) from
 // contiguous fragment-order blocks, and the `small` stage: the slab's dO rows as they lie in memory plus the
 // forward pass's tril(Q K^T . Gam) tiles, from which the compute waves form dv_local = scale Aq^T dO themselves.
 // ---------------------------------------------------------------------------------------------
 template <typename T, int DK, int NW, int STAGES> struct StateBwdSmem {
-  static constexpr int big = 3 * 64 * DK * (int)sizeof(T) + 2 * 64 * 4 + 16;   // K, Q^T, W^T images, decay[64], G_last, scale e^G [64]
+  static constexpr int big = 3 * 64 * DK * (int)sizeof(T) + 2 * 64 * 4 + 16;   // K, Q^T, W^T images, [64 unused], G_last, scale e^G [64]
   static constexpr int off_small = STAGES * big;            // dO rows of the slab [64][32 NW] | tril(Q K^T . Gam) tiles [4]
   static constexpr int bytes = off_small + (NW * 2048 + 4096) * (int)sizeof(T);
 };
 
 template <typename T, int DK, int NW, int NL, int STAGES>
-__global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_bwd_kernel(
+__global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 && NL >= 4) ? 2 : 1) void chunk_state_bwd_kernel(
     const T* __restrict__ kaf, const T* __restrict__ qtf, const T* __restrict__ wf, const T* __restrict__ aqf,
     const T* __restrict__ dO, const float* __restrict__ G, const float* __restrict__ dht, float* __restrict__ dh0,
     T* __restrict__ dvf, T* __restrict__ dhf, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets,
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_bwd_kernel(
     const int lt = tid - 64 * NW;
     constexpr int DEPTH = (STAGES == 2) ? 2 : 1;
     Vec16<T> pk[DEPTH][CW], pq[DEPTH][CW], pw[DEPTH][CW], pa[DEPTH][CAQ], pd[DEPTH][CUL];
-    float pdec[DEPTH], pgl[DEPTH], pqs[DEPTH];
+    float pgt[DEPTH], pgl[DEPTH], pgk[DEPTH][2];
     auto issue = [&](int st, int set) {
       const int c = nchunks - 1 - st;
       const int64_t tok0 = bos + (int64_t)c * kChunk;
@@ -86,10 +86,12 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_bwd_kernel(
                                   : zero16<T>();
       }
       const float* gc = G + ch * 64;
-      pgl[set] = gc[nvalid - 1];
-      const float gt = gc[imin(lt & 63, nvalid - 1)];
-      pdec[set] = __expf(pgl[set] - gt);
-      pqs[set] = scale * __expf(gt);
+      // raw values only: arithmetic here would wait for every load issued so far.  The array repeats G_last past the
+      // end of a short chunk.
+      pgl[set] = gc[63];
+      pgt[set] = gc[lt & 63];
+      pgk[set][0] = gc[lt & 31];
+      pgk[set][1] = gc[32 + (lt & 31)];
     };
     auto commit_big = [&](int set, int buf) {
       unsigned char* base = gdn_smem + buf * SM::big;
@@ -97,14 +99,18 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_bwd_kernel(
       T* Qa = Ka + TILE;
       T* Wa = Qa + TILE;
       float* dec = reinterpret_cast<float*>(Wa + TILE);
+      // K goes to LDS scaled by e^{G_last-G} of its token: in the A-operand tiles (rows = tokens) every 16-byte piece
+      // belongs to one token, 32 (tile & 1) + lane % 32.  The K tiles in memory are shared by the value heads of a
+      // q/k group, the decay is per value head.
+      const float kd[2] = {__expf(pgl[set] - pgk[set][0]), __expf(pgl[set] - pgk[set][1])};
 #pragma unroll
       for (int i = 0; i < CW; ++i) {
         const int id = lt + i * NT;
-        st16(Ka + id * VEC, pk[set][i]);
+        st16(Ka + id * VEC, scale16<T>(pk[set][i], kd[(id / (1024 / VEC)) & 1]));
         st16(Qa + id * VEC, pq[set][i]);
         st16(Wa + id * VEC, pw[set][i]);
       }
-      if (lt < 64) { dec[lt] = pdec[set]; dec[68 + lt] = pqs[set]; }
+      if (lt < 64) dec[68 + lt] = scale * __expf(pgt[set]);
       if (lt == 0) dec[64] = pgl[set];
     };
     auto commit_small = [&](int set) {
@@ -114,23 +120,24 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_bwd_kernel(
       for (int i = 0; i < CAQ; ++i) st16(small + NW * 2048 + (lt + i * NT) * VEC, pa[set][i]);
     };
     if (STAGES == 2) {
-      if (nchunks > 0) { issue(0, 0); commit_big(0, 0); commit_small(0); }
+      // Every path through this loop issues the same loads in the same order (steps past the end are clamped and
+      // their data is never used), so that the number of loads in flight at each wait is a compile-time fact.
+      if (nchunks == 0) return;
+      issue(0, 0);
+      commit_big(0, 0);
+      commit_small(0);
 #pragma unroll
-      for (int j = 1; j <= DEPTH; ++j)
-        if (j < nchunks) issue(j, j % DEPTH);
-      for (int s0 = 0; s0 < nchunks; s0 += DEPTH) {
+      for (int j = 1; j <= DEPTH; ++j) issue(imin(j, nchunks - 1), j % DEPTH);
+      for (int s0 = 0;; s0 += DEPTH) {
 #pragma unroll
         for (int u = 0; u < DEPTH; ++u) {
           const int st = s0 + u;
-          if (st < nchunks) {
-            GDN_LDS_BARRIER();              // (A) step st staged
-            if (st + 1 < nchunks) commit_big((u + 1) % DEPTH, (st + 1) & 1);
-            GDN_LDS_BARRIER();              // (B) the compute waves have taken their dO rows and formed dv_local
-            if (st + 1 < nchunks) {
-              commit_small((u + 1) % DEPTH);
-              if (st + 1 + DEPTH < nchunks) issue(st + 1 + DEPTH, (u + 1) % DEPTH);
-            }
-          }
+          if (st >= nchunks) return;
+          GDN_LDS_BARRIER();                // (A) step st staged
+          commit_big((u + 1) % DEPTH, (st + 1) & 1);
+          GDN_LDS_BARRIER();                // (B) the compute waves have taken their dO rows and the Aq tiles
+          commit_small((u + 1) % DEPTH);
+          issue(imin(st + 1 + DEPTH, nchunks - 1), (u + 1) % DEPTH);
         }
       }
     } else {
@@ -160,90 +167,84 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_bwd_kernel(
         dS[kt][r] = dht[(((int64_t)n * Hv + h) * DK + 32 * kt + acc_row(r)) * V + v0 + acc_col()];
     }
   }
+  // As in the forward recurrence the vector work that does not depend on the running products (decay and packing of
+  // dS) is written between the matrix instructions.
+  AccB<T> dSb[NKT];
+#pragma unroll
+  for (int kt = 0; kt < NKT; ++kt) dSb[kt].pack(dS[kt]);
   for (int st = 0; st < nchunks; ++st) {
     const int c = nchunks - 1 - st;
     const int buf = (STAGES == 2) ? (st & 1) : 0;
     GDN_LDS_BARRIER();                      // (A)
     // dO of this wave's 32 columns as B operand (lane <-> V column, registers <-> token), turned from the row-major
-    // rows through the matrix core; dv_local = scale tril(Q K^T . Gam)^T dO from the forward pass's accumulator tiles
-    AccB<T> dob[2], aq[3];
-    f32x16 dvl[2];
+    // rows through the matrix core; dv_local = (scale tril(Q K^T . Gam))^T dO from the forward pass's tiles
+    AccB<T> dob[2], dos[2], aq[3];
     frags_from_lds<T>(dob[0], small + (lane & 31) * (32 * NW) + 32 * wave);
     frags_from_lds<T>(dob[1], small + (32 + (lane & 31)) * (32 * NW) + 32 * wave);
     aq[0].load(small + NW * 2048);            // tiles (0,0), (1,0), (1,1)
     aq[1].load(small + NW * 2048 + 2048);
     aq[2].load(small + NW * 2048 + 3072);
     GDN_LDS_BARRIER();                      // (B)
-    dob[0].pack(mfma_transpose<T>(dob[0], id));
-    dob[1].pack(mfma_transpose<T>(dob[1], id));
-#pragma unroll
-    for (int rj = 0; rj < 2; ++rj) {
-      dvl[rj] = acc_zero();
-#pragma unroll
-      for (int ti = rj; ti < 2; ++ti) mma32_ff<T>(dvl[rj], aq[ti + rj], dob[ti]);
-    }
     unsigned char* base = gdn_smem + buf * SM::big;
     const T* Ka = reinterpret_cast<const T*>(base);
     const T* Qa = Ka + TILE;
     const T* Wa = Qa + TILE;
     const float* dec = reinterpret_cast<const float*>(Wa + TILE);
-    const float glast = dec[64];
+    const float eg = __expf(dec[64]);
     const int64_t tile0 = ((chunk_base + c) * Hv + h) * (V / 32) + vblk;
-
-    AccB<T> dSb[NKT];
 #pragma unroll
-    for (int kt = 0; kt < NKT; ++kt) {
-      dSb[kt].pack(dS[kt]);
-      dSb[kt].store_stream(dhf + (tile0 * NKT + kt) * 1024);
-    }
-    // dV' = e^{G_last-G} . (K dS) + dv_local
-    f32x16 a0 = acc_zero(), a1 = acc_zero();
-#pragma unroll
-    for (int kt = 0; kt < NKT; ++kt) {
-      AccB<T> ka;
-      ka.load(Ka + (kt * 2 + 0) * 1024);
-      mma32_ff<T>(a0, ka, dSb[kt]);
-      ka.load(Ka + (kt * 2 + 1) * 1024);
-      mma32_ff<T>(a1, ka, dSb[kt]);
-    }
-    AccB<T> dvb[2];
+    for (int kt = 0; kt < NKT; ++kt) dSb[kt].store_stream(dhf + (tile0 * NKT + kt) * 1024);
     {
+      // the per-token factor scale e^G of the Q^T product rides on dO, so that the Q^T tiles are the same for every
+      // value head of a q/k group
+      const f32x16 q0 = rows_ld(dec + 68, 0), q1 = rows_ld(dec + 68, 32);
+      f32x16 t0 = mfma_transpose<T>(dob[0], id), t1 = mfma_transpose<T>(dob[1], id);
+      dob[0].pack(t0);
+      dob[1].pack(t1);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        a0[r] = a0[r] * dec[acc_row(r)] + scale * dvl[0][r];
-        a1[r] = a1[r] * dec[32 + acc_row(r)] + scale * dvl[1][r];
-      }
+      for (int r = 0; r < 16; ++r) { t0[r] *= q0[r]; t1[r] *= q1[r]; }
+      dos[0].pack(t0);
+      dos[1].pack(t1);
     }
+    // dV' = (e^{G_last-G} . K) dS + dv_local, one accumulation chain per 32-token block.  The A-operand tiles come
+    // from LDS two tiles ahead of the matrix instructions that use them; the decay of dS rides in between.
+    f32x16 a0 = acc_zero(), a1 = acc_zero();
+    AccB<T> af[3];
+    af[0].load(Ka);
+    af[1].load(Ka + 1024);
+    mma32_ff<T>(a0, aq[0], dob[0]);
+    mma32_ff<T>(a1, aq[2], dob[1]);
+    mma32_ff<T>(a0, aq[1], dob[1]);
+    GDN_SCHED_FENCE();
+#pragma unroll
+    for (int i = 0; i < 2 * NKT; ++i) {       // tile i = (K tile i / 2, token block i % 2)
+      if (i + 2 < 2 * NKT) af[(i + 2) % 3].load(Ka + (i + 2) * 1024);
+      mma32_ff<T>((i & 1) ? a1 : a0, af[i % 3], dSb[i / 2]);
+#pragma unroll
+      for (int r = 0; r < 8; ++r) dS[i / 2][8 * (i & 1) + r] *= eg;
+      GDN_SCHED_FENCE();
+    }
+    // dS <- e^{G_last} dS + Q^T (scale e^G . dO) - W^T dV'  (the W^T tiles arrive negated); a finished tile of dS is
+    // packed for the next step while the matrix pipe works on the following one
+    auto tile_qw = [&](int i) {               // i = 4 kt + 2 tj + (0: Q^T, 1: W^T)
+      return ((i & 1) ? Wa : Qa) + ((i >> 2) * 2 + ((i >> 1) & 1)) * 1024;
+    };
+    af[0].load(tile_qw(0));
+    af[1].load(tile_qw(1));
+    AccB<T> dvb[2];
     dvb[0].pack(a0);
     dvb[1].pack(a1);
     dvb[0].store_stream(dvf + (tile0 * 2 + 0) * 1024);
     dvb[1].store_stream(dvf + (tile0 * 2 + 1) * 1024);
-    dvb[0].negate();
-    dvb[1].negate();
-    // dS <- e^{G_last} dS + Q^T (scale e^G . dO) - W^T dV'   (the per-token factor rides on dO, so that the Q^T tiles
-    // are the same for every value head of a q/k group)
-    {
-      const f32x16 q0 = rows_ld(dec + 68, 0), q1 = rows_ld(dec + 68, 32);
-      f32x16 d0 = dob[0].unpack(), d1 = dob[1].unpack();
+    GDN_SCHED_FENCE();
 #pragma unroll
-      for (int r = 0; r < 16; ++r) { d0[r] *= q0[r]; d1[r] *= q1[r]; }
-      dob[0].pack(d0);
-      dob[1].pack(d1);
+    for (int i = 0; i < 4 * NKT; ++i) {
+      if (i + 2 < 4 * NKT) af[(i + 2) % 3].load(tile_qw(i + 2));
+      mma32_ff<T>(dS[i >> 2], af[i % 3], (i & 1) ? dvb[(i >> 1) & 1] : dos[(i >> 1) & 1]);
+      if ((i & 3) == 3 && i >= 4) dSb[(i >> 2) - 1].pack(dS[(i >> 2) - 1]);
+      GDN_SCHED_FENCE();
     }
-    const float eg = __expf(glast);
-#pragma unroll
-    for (int kt = 0; kt < NKT; ++kt) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) dS[kt][r] *= eg;
-#pragma unroll
-      for (int tj = 0; tj < 2; ++tj) {
-        AccB<T> af;
-        af.load(Qa + (kt * 2 + tj) * 1024);
-        mma32_ff<T>(dS[kt], af, dob[tj]);
-        af.load(Wa + (kt * 2 + tj) * 1024);
-        mma32_ff<T>(dS[kt], af, dvb[tj]);
-      }
-    }
+    dSb[NKT - 1].pack(dS[NKT - 1]);
     if (STAGES == 1 && st + 1 < nchunks) GDN_LDS_BARRIER();   // (C)
   }
   if (dh0 != nullptr) {
@@ -783,7 +784,7 @@ extern "C" int gdn_chunk_bwd(const void* q, const void* k, const void* v, const 
   const bool wide = (V % 128 == 0);
   const bool solo = one_slab_per_workgroup(d, device_compute_units());
   if (dtype == 1) {
-    if (K == 128 && wide && solo) GDN_BWD(bf16_t, 128, 4, 1, 2, 2);
+    if (K == 128 && wide && solo) GDN_BWD(bf16_t, 128, 4, 1, 4, 2);
     if (K == 128 && wide) GDN_BWD(bf16_t, 128, 4, 2, 2, 2);
     if (K == 128) GDN_BWD(bf16_t, 128, 2, 2, 2, 2);
     if (wide) GDN_BWD(bf16_t, 64, 4, 2, 2, 2);

@@ -15,6 +15,12 @@
 #include "gdn_common.h"
 #include "gdn_profile.h"
 
+#ifndef GDN_PREP_WPS
+#define GDN_PREP_WPS 3
+#endif
+#ifndef GDN_OUT_WPS
+#define GDN_OUT_WPS 2
+#endif
 namespace gdn {
 
 constexpr int kLF = 68;  // leading dimension of the fp32 64x64 solve buffers
@@ -100,7 +106,7 @@ template <typename T, int DK, int BV> struct PrepSmem {
 };
 
 template <typename T, int DK, int BV>
-__global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
+__global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(GDN_PREP_WPS) void chunk_prep_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ g,
     const float* __restrict__ beta, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets,
     float* __restrict__ G_out, T* __restrict__ Ai_out, T* __restrict__ W_out, T* __restrict__ U_out,
@@ -168,9 +174,9 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
       const int i = 32 * ti + acc_row(r);
       const float gam = i >= j ? __expf(Gs[i] - Gs[j]) : 0.f;
       a_tile[r] = i > j ? bs[i] * a_tile[r] * gam : 0.f;
-      aq[r] *= gam;
+      aq[r] *= gam * scale;
     }
-    // tril(Q K^T . Gam) leaves as four 32x32 tiles in fragment order, packed as they sit in the accumulator
+    // scale tril(Q K^T . Gam) leaves as four 32x32 tiles in fragment order, packed as they sit in the accumulator
     // (lane <-> column j, registers <-> row i): the A operand of Aq^T dO as is, of Aq V' after one turn
     AccB<T> af;
     af.pack(aq);
@@ -328,10 +334,11 @@ __global__ __launch_bounds__(kThreads) void chunk_prep_kernel(
       mma32<T, 64, true, false>(acc, Tms + 32 * ri * L64, L64, Kb + 32 * cj, LDK);
       const int64_t tile = (((int64_t)blockIdx.x * Hv + h) * (DK / 32) + cj) * 2 + ri;
       AccB<T> wf;
-      wf.pack(acc);              // (lane <-> K column, registers <-> token): W^T as an A operand, for the backward pass
+      wf.pack(acc);              // (lane <-> K column, registers <-> token): -W^T as an A operand, for the backward pass
+      wf.negate();               // both uses subtract the product (U - W S, dS - W^T dV')
       if (WF_out != nullptr) wf.store_stream(WF_out + tile * 1024);
       const f32x16 wt = mfma_transpose<T>(wf, id);
-      wf.pack(wt);               // (lane <-> token, registers <-> K column): W as an A operand, for W S
+      wf.pack(wt);               // (lane <-> token, registers <-> K column): -W as an A operand, for U - W S
       wf.store_stream(W_out + tile * 1024);
     }
   }
@@ -378,7 +385,7 @@ template <typename T, int DK, int NW, int STAGES> struct StateSmem {
 };
 
 template <typename T, int DK, int NW, int NL, int STAGES>
-__global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_kernel(
+__global__ __launch_bounds__(64 * (NW + NL)) GDN_REGS_256 void chunk_state_kernel(
     const T* __restrict__ ktf, const T* __restrict__ w, const T* __restrict__ uf, const float* __restrict__ G,
     const float* __restrict__ h0, float* __restrict__ ht, T* __restrict__ vf, T* __restrict__ hf,
     const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int Hqk, int Hv, int V) {
@@ -401,7 +408,7 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_kernel(
     const int lt = tid - 64 * NW;
     // DEPTH register sets: chunk j sits in set j % DEPTH from the iteration that requests it (j - DEPTH - 1) to the
     // one that copies it to LDS (j - 1), so global loads have DEPTH chunk periods to arrive
-    constexpr int DEPTH = (STAGES == 2) ? 3 : 1;
+    constexpr int DEPTH = (STAGES == 2) ? 2 : 1;
     Vec16<T> pw[DEPTH][CW], pk[DEPTH][CW], pu[DEPTH][CUL];
     float glast[DEPTH], pdec[DEPTH];
     auto issue = [&](int c, int set) {      // global -> registers
@@ -417,8 +424,8 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_kernel(
 #pragma unroll
       for (int i = 0; i < CUL; ++i) pu[set][i] = ld16(ug + (lt + i * NT) * VEC);
       const float* gc = G + ((chunk_base + c) * Hv + h) * 64;
-      glast[set] = gc[nvalid - 1];
-      pdec[set] = __expf(glast[set] - gc[imin(lt & 63, nvalid - 1)]);
+      glast[set] = gc[nvalid - 1];          // raw values only: arithmetic here would wait for every load issued so far
+      pdec[set] = gc[imin(lt & 63, nvalid - 1)];
     };
     auto commit = [&](int set, int buf) {   // registers -> LDS stage
       unsigned char* base = gdn_smem + buf * SM::stage;
@@ -434,25 +441,26 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_kernel(
 #pragma unroll
       for (int i = 0; i < CUL; ++i) st16(Uf + (lt + i * NT) * VEC, pu[set][i]);
       float* dec = reinterpret_cast<float*>(base + SM::off_gl);
-      if (lt < 64) dec[lt] = pdec[set];
+      if (lt < 64) dec[lt] = __expf(glast[set] - pdec[set]);
       if (lt == 0) dec[64] = glast[set];
     };
     if (STAGES == 2) {
-      if (nchunks > 0) { issue(0, 0); commit(0, 0); }
+      // Every path through this loop issues the same loads in the same order (chunk indices past the end are clamped
+      // and their data is never used), so that the number of loads in flight at each wait is a compile-time fact and
+      // the waits before the LDS writes of one register set leave the younger sets in flight.
+      if (nchunks == 0) return;
+      issue(0, 0);
+      commit(0, 0);
 #pragma unroll
-      for (int j = 1; j <= DEPTH; ++j)
-        if (j < nchunks) issue(j, j % DEPTH);
-      for (int c0 = 0; c0 < nchunks; c0 += DEPTH) {
+      for (int j = 1; j <= DEPTH; ++j) issue(imin(j, nchunks - 1), j % DEPTH);
+      for (int c0 = 0;; c0 += DEPTH) {
 #pragma unroll
         for (int u = 0; u < DEPTH; ++u) {
           const int c = c0 + u;
-          if (c < nchunks) {
-            GDN_LDS_BARRIER();              // (A) chunk c staged; the other stage (chunk c-1) is free
-            if (c + 1 < nchunks) {
-              commit((u + 1) % DEPTH, (c + 1) & 1);
-              if (c + 1 + DEPTH < nchunks) issue(c + 1 + DEPTH, (u + 1) % DEPTH);
-            }
-          }
+          if (c >= nchunks) return;
+          GDN_LDS_BARRIER();                // (A) chunk c staged; the other stage (chunk c-1) is free
+          commit((u + 1) % DEPTH, (c + 1) & 1);
+          issue(imin(c + 1 + DEPTH, nchunks - 1), (u + 1) % DEPTH);
         }
       }
     } else {
@@ -478,6 +486,13 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_kernel(
         S[kt][r] = h0[(((int64_t)n * Hv + h) * DK + 32 * kt + acc_row(r)) * V + v0 + acc_col()];
     }
   }
+  // The wave issues its instructions in order and a matrix instruction occupies the matrix pipe for 32 cycles, in
+  // which eight vector instructions can issue: the loop body is written so that the vector work which does not
+  // depend on the running product (decay of S, packing S for the next chunk, unpacking U) sits between the matrix
+  // instructions instead of before or after them.
+  AccB<T> Sb[NKT];
+#pragma unroll
+  for (int kt = 0; kt < NKT; ++kt) Sb[kt].pack(S[kt]);
   for (int c = 0; c < nchunks; ++c) {
     const int buf = (STAGES == 2) ? (c & 1) : 0;
     GDN_LDS_BARRIER();                        // (A) stage `buf` holds chunk c
@@ -486,17 +501,8 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_kernel(
     const T* KT = reinterpret_cast<const T*>(base + SM::off_kt);
     const T* Uf = reinterpret_cast<const T*>(base + SM::off_uf) + wave * 2048;
     const float* dec = reinterpret_cast<const float*>(base + SM::off_gl);
-    const float glast = dec[64];
     const int64_t tile0 = ((chunk_base + c) * Hv + h) * (V / 32) + vblk;
 
-    AccB<T> Sb[NKT];
-#pragma unroll
-    for (int kt = 0; kt < NKT; ++kt) {
-      Sb[kt].pack(S[kt]);
-      Sb[kt].store_stream(hf + (tile0 * NKT + kt) * 1024);
-    }
-    // Hand-made software pipeline over pairs of K tiles: the LDS reads of the next group are issued before the
-    // matrix instructions of the current one (GDN_SCHED_FENCE keeps the order).
     constexpr int NP = NKT / 2;             // K tiles are processed two at a time
     AccB<T> Wf[2][2][2];                    // [buffer][32-token block][K tile of the pair]
     AccB<T> Kf[2][2][2];                    // [buffer][K tile of the pair][32-token block]
@@ -512,58 +518,62 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_kernel(
 #pragma unroll
         for (int tj = 0; tj < 2; ++tj) Kf[b][j][tj].load(KT + ((2 * kp + j) * 2 + tj) * 1024);
     };
-    f32x16 p0 = acc_zero(), p1 = acc_zero();
     AccB<T> Vb[2];
+    Vb[0].load(Uf);
+    Vb[1].load(Uf + 1024);
     load_w(0, 0);
     if (NP > 1) load_w(1, 1);
+    const float eg = __expf(dec[64]);
+#pragma unroll
+    for (int kt = 0; kt < NKT; ++kt) Sb[kt].store_stream(hf + (tile0 * NKT + kt) * 1024);
+    // V' = U - W S: the accumulators start from U and the W tiles arrive negated; the two 32-token blocks are
+    // independent accumulation chains.  The decay of S rides between the matrix instructions.
+    f32x16 p0 = Vb[0].unpack(), p1 = Vb[1].unpack();
     GDN_SCHED_FENCE();
 #pragma unroll
     for (int kp = 0; kp < NP; ++kp) {
-      // V' = U - W S: the two 32-token blocks are independent accumulation chains
-      if (kp == 0) load_k(0, 0);
-      if (kp == NP - 1) { Vb[0].load(Uf); Vb[1].load(Uf + 1024); if (NP > 1) load_k(1, 1); }
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         mma32_ff<T>(p0, Wf[kp & 1][0][j], Sb[2 * kp + j]);
         mma32_ff<T>(p1, Wf[kp & 1][1][j], Sb[2 * kp + j]);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) S[2 * kp + j][r] *= eg;
+        GDN_INTERLEAVE_MFMA_VALU(2 * AccK<T>::kGroups, 16 / (2 * AccK<T>::kGroups));
       }
       GDN_SCHED_FENCE();
-      if (kp + 2 < NP) { load_w(kp & 1, kp + 2); GDN_SCHED_FENCE(); }
+      if (kp + 2 < NP) load_w(kp & 1, kp + 2);
+      if (kp == (NP > 1 ? NP - 2 : 0)) load_k(0, 0);
+      if (kp == NP - 1 && NP > 1) load_k(1, 1);
+      GDN_SCHED_FENCE();
     }
-    {
-      const f32x16 u0 = Vb[0].unpack(), u1 = Vb[1].unpack();
-#pragma unroll
-      for (int r = 0; r < 16; ++r) { p0[r] = u0[r] - p0[r]; p1[r] = u1[r] - p1[r]; }
-    }
+    const f32x16 d0 = rows_ld(dec, 0), d1 = rows_ld(dec, 32);
     Vb[0].pack(p0);
     Vb[1].pack(p1);
     Vb[0].store_stream(vf + (tile0 * 2 + 0) * 1024);
     Vb[1].store_stream(vf + (tile0 * 2 + 1) * 1024);
-    {  // the decay of the state update rides on V': (e^{G_last - G} . K)^T V' = K^T (e^{G_last - G} . V'), so that the
-       // K^T tiles are the same for every value head of a q/k group
-      const f32x16 d0 = rows_ld(dec, 0), d1 = rows_ld(dec, 32);
+    // the decay of the state update rides on V': (e^{G_last - G} . K)^T V' = K^T (e^{G_last - G} . V'), so that the
+    // K^T tiles are the same for every value head of a q/k group
 #pragma unroll
-      for (int r = 0; r < 16; ++r) { p0[r] *= d0[r]; p1[r] *= d1[r]; }
-      Vb[0].pack(p0);
-      Vb[1].pack(p1);
-    }
-    // S <- e^{G_last} S + K^T (e^{G_last - G} . V')
-    const float eg = __expf(glast);
-#pragma unroll
-    for (int kt = 0; kt < NKT; ++kt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) S[kt][r] *= eg;
+    for (int r = 0; r < 16; ++r) { p0[r] *= d0[r]; p1[r] *= d1[r]; }
+    Vb[0].pack(p0);
+    Vb[1].pack(p1);
     GDN_SCHED_FENCE();
+    // S <- e^{G_last} S + K^T (e^{G_last - G} . V'); a finished tile of S is packed for the next chunk while the
+    // matrix pipe works on the following ones
 #pragma unroll
     for (int kp = 0; kp < NP; ++kp) {
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        mma32_ff<T>(S[2 * kp + j], Kf[kp & 1][j][0], Vb[0]);
-        mma32_ff<T>(S[2 * kp + j], Kf[kp & 1][j][1], Vb[1]);
+        const int kt = 2 * kp + j;
+        mma32_ff<T>(S[kt], Kf[kp & 1][j][0], Vb[0]);
+        mma32_ff<T>(S[kt], Kf[kp & 1][j][1], Vb[1]);
+        if (kt >= 2) Sb[kt - 2].pack(S[kt - 2]);
       }
       GDN_SCHED_FENCE();
       if (kp + 2 < NP) { load_k(kp & 1, kp + 2); GDN_SCHED_FENCE(); }
     }
+#pragma unroll
+    for (int kt = (NKT >= 2 ? NKT - 2 : 0); kt < NKT; ++kt) Sb[kt].pack(S[kt]);
     if (STAGES == 1 && c + 1 < nchunks) GDN_LDS_BARRIER();      // (B) done with the single stage
   }
   if (ht != nullptr) {
@@ -576,7 +586,7 @@ __global__ __launch_bounds__(64 * (NW + NL)) void chunk_state_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
-// chunk_out_kernel:  O = scale [ e^G . (Q S) + Aq V' ], parallel over (chunk, head, 32-column block).
+// chunk_out_kernel:  O = scale e^G . (Q S) + (scale Aq) V', parallel over (chunk, head, 32-column block).
 // S and V' arrive in fragment order and go from global memory straight into B-operand registers.
 // ---------------------------------------------------------------------------------------------
 template <typename T, int DK, int NW> struct OutSmem {
@@ -588,7 +598,7 @@ template <typename T, int DK, int NW> struct OutSmem {
 };
 
 template <typename T, int DK, int NW>
-__global__ __launch_bounds__(64 * NW) void chunk_out_kernel(
+__global__ __launch_bounds__(64 * NW) GDN_WAVES_PER_SIMD(GDN_OUT_WPS) void chunk_out_kernel(
     const T* __restrict__ q, const T* __restrict__ aqf, const T* __restrict__ vf, const T* __restrict__ hf,
     const float* __restrict__ G, T* __restrict__ o, const int64_t* __restrict__ cu,
     const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V, float scale) {
@@ -620,7 +630,7 @@ __global__ __launch_bounds__(64 * NW) void chunk_out_kernel(
     st16(Qs + row * LDK + cc * VEC,
          row < nvalid ? ld16(q + ((tok0 + row) * Hqk + hq) * DK + cc * VEC) : zero16<T>());
   }
-  if (tid < 64) Eg[tid] = __expf(G[ch * 64 + imin(tid, nvalid - 1)]);
+  if (tid < 64) Eg[tid] = scale * __expf(G[ch * 64 + imin(tid, nvalid - 1)]);
   IdentityFrag<T> id;
   id.init();
 #pragma unroll
@@ -638,8 +648,6 @@ __global__ __launch_bounds__(64 * NW) void chunk_out_kernel(
     for (int r = 0; r < 16; ++r) oa[r] *= eg[r];
 #pragma unroll
     for (int tj = 0; tj <= ri; ++tj) mma32_ff<T>(oa, Af[ri + tj], Vb[tj]);
-#pragma unroll
-    for (int r = 0; r < 16; ++r) oa[r] *= scale;
     acc_store_rows<T, false>(oa, id, patch, og + (int64_t)32 * ri * Hv * V, (int64_t)Hv * V, nvalid - 32 * ri);
   }
 }

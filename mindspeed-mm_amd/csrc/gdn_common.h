@@ -15,6 +15,7 @@
 //     LDS, in that fragment order, and change orientation by a pass through the matrix core (mfma_transpose).
 #pragma once
 #include <hip/hip_runtime.h>
+#include <type_traits>
 #include <stdint.h>
 
 // dynamic LDS, one array per workgroup
@@ -77,6 +78,22 @@ template <typename T> __device__ __host__ constexpr int lds_ld(int cols) { retur
 // LDS reads of the next group, then the matrix instructions of this group) that the scheduler would otherwise
 // serialise into read -> wait -> multiply.
 #define GDN_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+// Kernel attribute: at most 256 registers per lane.  With a larger budget the compiler keeps matrix accumulators in
+// the accumulation registers, and every vector instruction that touches them (decay, packing) then costs an extra
+// move in each direction.
+#ifndef GDN_REGS_256
+#define GDN_WAVES_PER_SIMD(n) __attribute__((amdgpu_waves_per_eu(n, n)))   // register budget 512 / n per lane
+#define GDN_REGS_256 GDN_WAVES_PER_SIMD(2)
+#endif
+// Asks the scheduler for the pattern (1 matrix instruction, nvalu vector instructions) x nmfma in the current
+// scheduling region.
+#define GDN_INTERLEAVE_MFMA_VALU(nmfma, nvalu)                        \
+  do {                                                                \
+    _Pragma("unroll") for (int gdn_i_ = 0; gdn_i_ < (nmfma); ++gdn_i_) { \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              \
+      __builtin_amdgcn_sched_group_barrier(0x002, (nvalu), 0);        \
+    }                                                                 \
+  } while (0)
 // Orders the LDS traffic of one wave when its lanes hand data to each other through a wave-private LDS patch.  The
 // hardware already executes a wave's LDS instructions in order; this only stops the compiler from reordering them.
 #define GDN_WAVE_LDS_SYNC()                                           \
@@ -127,6 +144,23 @@ template <typename T> __device__ __forceinline__ Vec16<T> ld16(const T* p) {
 }
 template <typename T> __device__ __forceinline__ void st16(T* p, const Vec16<T>& v) {
   *reinterpret_cast<u32x4*>(p) = v.raw;
+}
+// every element of a 16-byte piece times one factor (bf16: two elements per conversion instruction)
+template <typename T> __device__ __forceinline__ Vec16<T> scale16(const Vec16<T>& v, float s) {
+  Vec16<T> r;
+  if constexpr (sizeof(T) == 4) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) r.raw[e] = __float_as_uint(__uint_as_float(v.raw[e]) * s);
+  } else if constexpr (std::is_same<T, bf16_t>::value) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      r.raw[e] = f32x2_to_bf16x2(__uint_as_float(v.raw[e] << 16) * s, __uint_as_float(v.raw[e] & 0xffff0000u) * s);
+  } else {
+    r = v;
+#pragma unroll
+    for (int e = 0; e < Elem<T>::kVec; ++e) r.set(e, v.get(e) * s);
+  }
+  return r;
 }
 template <typename T> __device__ __forceinline__ Vec16<T> zero16() {
   Vec16<T> v; v.raw = u32x4{0u, 0u, 0u, 0u}; return v;
