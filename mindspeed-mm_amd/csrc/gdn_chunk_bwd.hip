@@ -51,7 +51,7 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
   static_assert(STAGES == 1 || STAGES == 2, "one or two big LDS stages");
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n = blockIdx.x / Hv, h = blockIdx.x % Hv;
+  const int nh = xcd_grouped_head(blockIdx.x, gridDim.x, Hv / Hqk), n = nh / Hv, h = nh % Hv;
   const int64_t bos = cu ? cu[n] : (int64_t)n * T_len;
   const int len = cu ? (int)(cu[n + 1] - bos) : T_len;
   const int nchunks = (len + kChunk - 1) / kChunk;
@@ -785,7 +785,7 @@ extern "C" int gdn_chunk_bwd(const void* q, const void* k, const void* v, const 
   const bool solo = one_slab_per_workgroup(d, device_compute_units());
   if (dtype == 1) {
     if (K == 128 && wide && solo) GDN_BWD(bf16_t, 128, 4, 1, 4, 2);
-    if (K == 128 && wide) GDN_BWD(bf16_t, 128, 4, 2, 2, 2);
+    if (K == 128 && wide) GDN_BWD(bf16_t, 128, 4, 2, 4, 2);
     if (K == 128) GDN_BWD(bf16_t, 128, 2, 2, 2, 2);
     if (wide) GDN_BWD(bf16_t, 64, 4, 2, 2, 2);
     GDN_BWD(bf16_t, 64, 2, 2, 2, 2);

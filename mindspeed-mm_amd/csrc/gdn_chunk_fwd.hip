@@ -397,7 +397,7 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_REGS_256 void chunk_state_kerne
   static_assert(STAGES == 1 || STAGES == 2, "one or two LDS stages");
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31;
-  const int n = blockIdx.x / Hv, h = blockIdx.x % Hv;
+  const int nh = xcd_grouped_head(blockIdx.x, gridDim.x, Hv / Hqk), n = nh / Hv, h = nh % Hv;
   const int64_t bos = cu ? cu[n] : (int64_t)n * T_len;
   const int len = cu ? (int)(cu[n + 1] - bos) : T_len;
   const int nchunks = (len + kChunk - 1) / kChunk;

@@ -78,6 +78,16 @@ template <typename T> __device__ __host__ constexpr int lds_ld(int cols) { retur
 // LDS reads of the next group, then the matrix instructions of this group) that the scheduler would otherwise
 // serialise into read -> wait -> multiply.
 #define GDN_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+// Workgroups are dealt to the 8 XCDs (each with its own L2) round-robin by their linear index.  The recurrence kernels
+// number their workgroups so that the value heads of one q/k group, which read the same K / Q^T tiles, share an XCD:
+// with P = (sequences x q/k groups) a multiple of 8, workgroup b handles pair (b/8/grp) 8 + b % 8, head b/8 % grp of it.
+// Returns the plain index n Hv + h.
+__device__ __forceinline__ int xcd_grouped_head(int b, int total, int grp) {
+  const int pairs = total / grp;
+  if (grp == 1 || pairs % 8 != 0) return b;
+  const int j = b & 7, m = b >> 3;
+  return ((m / grp) * 8 + j) * grp + m % grp;
+}
 // Kernel attribute: at most 256 registers per lane.  With a larger budget the compiler keeps matrix accumulators in
 // the accumulation registers, and every vector instruction that touches them (decay, packing) then costs an extra
 // move in each direction.
