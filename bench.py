@@ -37,8 +37,8 @@ CFG = dict(B=2, T=8192, Hqk=16, Hv=32, K=128, V=128, C=64)
 # (rocprofv3 --pmc, one run per counter, each scaled by what the same counter reads for a 512 MiB copy): the figures
 # of profiles/chunk_fwd_bwd_B2_T8192_bf16_hbm_traffic.md.  Measured offline, reported beside the live timings.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "chunk_prep_kernel": 1328035405, "chunk_state_kernel": 814496928, "chunk_out_kernel": 675852621,
-    "chunk_state_bwd_kernel": 1032402399, "chunk_bwd_local_kernel": 1265262731,
+    "chunk_prep_kernel": 1159219017, "chunk_state_kernel": 816529630, "chunk_out_kernel": 657207758,
+    "chunk_state_bwd_kernel": 1018928506, "chunk_bwd_local_kernel": 1178391908,
 }
 
 
@@ -67,11 +67,12 @@ def kernel_algorithmic_bytes(K, V, grp, e=2, C=64):
     cc = [64,64] tile, row = 64 fp32 values."""
     tk, tv, st, cc, row = C * K * e, C * V * e, K * V * e, C * C * e, C * 4
     return {
-        # q, k, v, g, beta -> G, Tm, Aq, W, U, decayed K^T, W^T tiles; once per q/k group: K, Q^T tiles, normalised q, 1/|q|, 1/|k|
-        "chunk_prep_kernel": 2 * tk + tv + 2 * row + row + 2 * cc + tk + tv + tk + tk + (3 * tk + 2 * row) // grp,
-        "chunk_state_kernel": 2 * tk + tv + row + tv + st,          # W, decayed K^T, U, G -> v_new, state before the chunk
-        "chunk_out_kernel": tk + cc + tv + st + row + tv,            # q, Aq, v_new, state, G -> o
-        "chunk_state_bwd_kernel": 3 * tk + cc + tv + row + tv + st,  # K, Q^T, W^T, Aq, dO, G -> dv_new, dS
+        # v, g, beta -> G, Tm, Aq, -W, U, -W^T tiles; once per q/k group: q, k -> K^T, K, Q^T tiles, normalised q, 1/|q|, 1/|k|
+        "chunk_prep_kernel": tv + 2 * row + row + 2 * cc + tk + tv + tk + (2 * tk + 4 * tk + 2 * row) // grp,
+        "chunk_state_kernel": tk + tk // grp + tv + row + tv + st,   # -W, K^T (per group), U, G -> v_new, state before the chunk
+        "chunk_out_kernel": tk // grp + cc + tv + st + row + tv,     # normalised q (per group), Aq, v_new, state, G -> o
+        # K, Q^T (per group), -W^T, Aq, dO, G -> dv_new, dS
+        "chunk_state_bwd_kernel": 2 * tk // grp + tk + cc + tv + row + tv + st,
         # v_new, dv_new, dO, S, dS, v, K, q, Tm, row vectors -> dv, dg, dbeta, dq/dk (written by the first head of a
         # group, read and re-written by the others)
         "chunk_bwd_local_kernel": 3 * tv + 2 * st + tv + 2 * tk + cc + 5 * row + tv + 2 * row
@@ -247,6 +248,55 @@ def main():
         aux["rmsnorm_gated"] = {"fwd_ms": round(f_s * 1e3, 3), "fwd_GBps": round(3 * nb / f_s / 1e9, 1),
                                 "bwd_ms": round(b_s * 1e3, 3), "bwd_GBps": round(5 * nb / b_s / 1e9, 1)}
         del xn, zn, dyn
+
+        # ---- the rule inside the layer: on the unsplit convolution output (read and written in place) against the
+        # reference's glue (split -> contiguous copies -> rule -> concatenated gradient), and the gate recipe ----
+        nq, nv = c["Hqk"] * c["K"], c["Hv"] * c["V"]
+        mixed = torch.cat([x[n].reshape(c["B"], c["T"], -1) for n in ("q", "k", "v")], dim=-1).to(dev)
+        mixed.requires_grad_(True)
+        gg, bb, hh0 = (d[n].detach().clone().requires_grad_(True) for n in ("g", "beta", "h0"))
+
+        def unsplit_step():
+            o_, _ = ops.chunk_gated_delta_rule_qkv(mixed, gg, bb, c["Hqk"], c["Hv"], c["K"], c["V"], initial_state=hh0,
+                                                   output_final_state=True, use_qk_l2norm_in_kernel=True)
+            torch.autograd.grad([o_], [mixed, gg, bb, hh0], [d["do"]])
+
+        def split_step():
+            q_, k_, v_ = torch.split(mixed, [nq, nq, nv], dim=-1)
+            o_, _ = ops.chunk_gated_delta_rule(q_.reshape(c["B"], c["T"], c["Hqk"], c["K"]).contiguous(),
+                                               k_.reshape(c["B"], c["T"], c["Hqk"], c["K"]).contiguous(),
+                                               v_.reshape(c["B"], c["T"], c["Hv"], c["V"]).contiguous(), gg, bb,
+                                               initial_state=hh0, output_final_state=True, use_qk_l2norm_in_kernel=True)
+            torch.autograd.grad([o_], [mixed, gg, bb, hh0], [d["do"]])
+
+        def wall_ms(fn, n=10):
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n):
+                fn()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / n * 1e3
+        aux["rule_in_layer"] = {"unsplit_qkv_ms": round(wall_ms(unsplit_step), 4),
+                                "split_with_copies_ms": round(wall_ms(split_step), 4)}
+        del mixed
+        aa = torch.randn(c["B"], c["T"], c["Hv"], generator=gen).to(dev, torch.bfloat16).requires_grad_(True)
+        ab = torch.randn(c["B"], c["T"], c["Hv"], generator=gen).to(dev, torch.bfloat16).requires_grad_(True)
+        A_log = torch.zeros(c["Hv"], device=dev, requires_grad=True)
+        dt_b = torch.full((c["Hv"],), -3.0, device=dev, requires_grad=True)
+        dgg = torch.randn(c["B"], c["T"], c["Hv"], generator=gen).to(dev)
+
+        def gates_step():
+            g_, b_ = ops.gdn_gates(aa, ab, A_log, dt_b)
+            torch.autograd.grad([g_, b_], [aa, ab, A_log, dt_b], [dgg, dgg.to(torch.bfloat16)])
+
+        def gates_eager_step():
+            b_ = ab.sigmoid()
+            g_ = -A_log.float().exp() * torch.nn.functional.softplus(aa.float() + dt_b)
+            torch.autograd.grad([g_, b_], [aa, ab, A_log, dt_b], [dgg, dgg.to(torch.bfloat16)])
+        aux["gates"] = {"fused_fwd_bwd_ms": round(wall_ms(gates_step), 4),
+                        "torch_elementwise_fwd_bwd_ms": round(wall_ms(gates_eager_step), 4)}
 
     if args.calibrate_copy:
         src = torch.empty(512 << 20, dtype=torch.uint8, device=dev)

@@ -6,12 +6,14 @@
  * raw device pointers and sizes only.
  *
  * Common rules
- *   - every pointer is device memory, tensors are dense (contiguous) in the stated layout;
+ *   - every pointer is device memory, tensors are dense (contiguous) in the stated layout unless an entry
+ *     point takes strides;
  *   - dtype: 0 = fp32, 1 = bf16 (conv1d also 2 = fp16) and applies to q/k/v/o and their gradients;
  *     g, beta, states and their gradients are always fp32;
  *   - `stream` is a hipStream_t; launches are asynchronous, nothing allocates or synchronises;
  *   - return 0 on success, <0 for an invalid argument (-1 null pointer, -2 bad shape, -3 unsupported
- *     size, -4 bad dtype, -5 workspace too small), >0 is a hipError_t from the launch;
+ *     size, -4 bad dtype, -5 workspace too small, -6 bad stride or a pointer not 16-byte aligned), >0 is a
+ *     hipError_t from the launch;
  *   - layouts: q,k [B,T,Hqk,K]; v,o [B,T,Hv,V]; g,beta [B,T,Hv]; states [N,Hv,K,V]; Hv % Hqk == 0
  *     (grouped heads are read in place, no expansion); with cu_seqlens (int64 [N+1], device) B == 1.
  */
@@ -43,6 +45,25 @@ int gdn_chunk_bwd(const void* q, const void* k, const void* v, const float* g, c
                   const float* d_final_state, void* dq, void* dk, void* dv, float* dg, float* dbeta,
                   float* d_initial_state, void* workspace, int64_t workspace_bytes, int B, int T, int N, int Hqk,
                   int Hv, int K, int V, float scale, int use_qk_l2norm, int dtype, void* stream);
+
+/* The same pair for q, k, v (and dq, dk, dv) that are column slices of a wider token-major tensor, as the layer has
+ * them after `torch.split(mixed_qkv, [key_dim, key_dim, value_dim], dim=-1)` of the convolution's output
+ * (modeling_qwen3_5.py:818-831): x_stride is the distance between consecutive tokens in elements, the heads of a
+ * token stay contiguous; 0 means dense.  Strides must be multiples of 16 bytes and the pointers 16-byte aligned.
+ * The reference's Triton entry makes such views contiguous first (input_guard, triton/utils.py:210-239); reading
+ * and writing them in place saves those copies and the concatenation of dq, dk, dv in the backward pass. */
+int gdn_chunk_fwd_strided(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
+                          int64_t v_stride, const float* g, const float* beta, const float* initial_state,
+                          const int64_t* cu_seqlens, void* o, float* final_state, void* workspace,
+                          int64_t workspace_bytes, int B, int T, int N, int Hqk, int Hv, int K, int V, float scale,
+                          int use_qk_l2norm, int dtype, void* stream);
+
+int gdn_chunk_bwd_strided(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
+                          int64_t v_stride, const float* g, const float* beta, const float* initial_state,
+                          const int64_t* cu_seqlens, const void* d_o, const float* d_final_state, void* dq, void* dk,
+                          void* dv, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride, float* dg, float* dbeta,
+                          float* d_initial_state, void* workspace, int64_t workspace_bytes, int B, int T, int N,
+                          int Hqk, int Hv, int K, int V, float scale, int use_qk_l2norm, int dtype, void* stream);
 
 /* -------- fused recurrent gated delta rule (decode) ------------------------------------------
  * replaces the `recurrent_gated_delta_rule` slot (third-party fla kernel or
@@ -91,6 +112,20 @@ int64_t gdn_rmsnorm_gated_bwd_workspace_bytes(int64_t rows, int N);
 int gdn_rmsnorm_gated_bwd(const void* x, const void* gate, const void* weight, const float* rstd, const void* dy,
                           void* dx, void* dgate, float* dweight, void* workspace, int64_t workspace_bytes,
                           int64_t rows, int N, int dtype, int weight_dtype, void* stream);
+
+/* -------- gates of the rule from the layer's projections -------------------------------------------------
+ * replaces the elementwise chain in Qwen3_5GatedDeltaNet.forward, modeling_qwen3_5.py:833-841:
+ * beta = sigmoid(b) (in b's dtype), g = -exp(A_log) * softplus(a + dt_bias) (fp32).  a, b, beta, da, db, dbeta
+ * [tokens, Hv] in `dtype`; A_log, dt_bias [Hv] in `dtype` (param_dtype = dtype) or fp32 (param_dtype = 0); g, dg
+ * [tokens, Hv] fp32; dA_log, ddt_bias [Hv] fp32.  Hv <= 256. */
+int gdn_gate_fwd(const void* a, const void* b, const void* A_log, const void* dt_bias, float* g, void* beta,
+                 int64_t tokens, int Hv, int dtype, int param_dtype, void* stream);
+
+int64_t gdn_gate_bwd_workspace_bytes(int64_t tokens, int Hv);
+
+int gdn_gate_bwd(const void* a, const void* b, const void* A_log, const void* dt_bias, const float* dg,
+                 const void* dbeta, void* da, void* db, float* dA_log, float* ddt_bias, void* workspace,
+                 int64_t workspace_bytes, int64_t tokens, int Hv, int dtype, int param_dtype, void* stream);
 
 /* -------- per-kernel timing ------------------------------------------------------------------------
  * op-level counterpart of the reference's step profiler (mindspeed_mm/fsdp/tools/profiler.py:32-147).

@@ -4,9 +4,21 @@
 
 namespace gdn {
 
+// Distance between consecutive tokens, in elements, of the token-major tensors the caller hands over.  The heads of a
+// token are contiguous ([Hqk,K] / [Hv,V]); a stride larger than that lets q, k, v (and dq, dk, dv) be slices of one
+// wider [tokens, D] tensor, e.g. the output of the convolution in front of the operator.
+struct TokenStrides {
+  int64_t q, k, v, dq, dk, dv;
+};
+
 struct ChunkDims {
   int B, T, N, Hqk, Hv, K, V;
   bool varlen;
+  TokenStrides ts = {0, 0, 0, 0, 0, 0};   // 0 = contiguous heads
+  TokenStrides strides() const {
+    const int64_t nq = (int64_t)Hqk * K, nv = (int64_t)Hv * V;
+    return {ts.q ? ts.q : nq, ts.k ? ts.k : nq, ts.v ? ts.v : nv, ts.dq ? ts.dq : nq, ts.dk ? ts.dk : nq, ts.dv ? ts.dv : nv};
+  }
   int64_t tokens() const { return (int64_t)B * T; }
   // upper bound on the number of 64-token chunks; exact without cu_seqlens.  Packed sequences add at
   // most one partial chunk each, so the bound needs no look at the (device-resident) lengths.
@@ -23,15 +35,15 @@ struct ChunkWorkspace {
   int64_t rstd;           // f32 [2][tokens,Hqk] 1/|q|, 1/|k| of that normalisation
   int64_t G;              // f32 [chunks,Hv,64]      chunk-local cumulative log decay
   int64_t Ai;             // T [chunks,Hv,2,2]       (I + A)^-1 as A operand: tile = (32 rows) x (32 columns), fragment order
-  int64_t WAF;            // T [chunks,Hv,K/32,2]    W as A operand: tile = (32 tokens) x (32 columns of K), fragment order
-  int64_t AQ;             // T [chunks,Hv,2,2]       tril(Q K^T . Gam) (unscaled), accumulator tiles: lane <-> column, registers <-> row
+  int64_t WAF;            // T [chunks,Hv,K/32,2]    -W as A operand: tile = (32 tokens) x (32 columns of K), fragment order
+  int64_t AQ;             // T [chunks,Hv,2,2]       scale tril(Q K^T . Gam), accumulator tiles: lane <-> column, registers <-> row
   // Tiles exchanged between kernels in fragment order (see AccB<>): 1024 elements per 32x32 tile.
   int64_t KTF;            // T [chunks,Hqk,K/32,2]   K^T as A operand: tile = (32 columns of K) x (32 tokens)
   int64_t UF;             // T [chunks,Hv,V/32,2]    U,            tile = (32-token block ri) x (32-column block)
   int64_t VF;             // T [chunks,Hv,V/32,2]    v_new = U - W S
   int64_t HF;             // T [chunks,Hv,V/32,K/32] state BEFORE each chunk, tile = (32 rows of K) x (32 columns of V)
   int64_t fwd_bytes;
-  int64_t WF;             // T [chunks,Hv,K/32,2]    W^T as A operand (written by the forward when a backward follows)
+  int64_t WF;             // T [chunks,Hv,K/32,2]    -W^T as A operand (written by the forward when a backward follows)
   int64_t QTF;            // T [chunks,Hqk,K/32,2]   Q^T as A operand: tile = (32 columns of K) x (32 tokens)
   int64_t KAF;            // T [chunks,Hqk,K/32,2]   K as A operand: tile = (32 tokens) x (32 columns of K)
   int64_t DVF;            // T [chunks,Hv,V/32,2]    d(v_new)
@@ -84,6 +96,11 @@ inline int chunk_check_dims(const ChunkDims& d, int dtype) {
   if (d.K != 64 && d.K != 128) return -3;
   if (d.V <= 0 || d.V % 64 != 0) return -3;
   if (dtype != 0 && dtype != 1) return -4;
+  // rows are moved in 16-byte pieces: strides must keep them aligned and cannot be shorter than a token's heads
+  const int64_t vec = dtype == 0 ? 4 : 8, nq = (int64_t)d.Hqk * d.K, nv = (int64_t)d.Hv * d.V;
+  const TokenStrides s = d.strides();
+  if (s.q % vec || s.k % vec || s.v % vec || s.dq % vec || s.dk % vec || s.dv % vec) return -6;
+  if (s.q < nq || s.k < nq || s.dq < nq || s.dk < nq || s.v < nv || s.dv < nv) return -6;
   return 0;
 }
 

@@ -298,7 +298,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     const T* __restrict__ dO, const T* __restrict__ hf, const T* __restrict__ dhf, const float* __restrict__ rstd_q,
     const float* __restrict__ rstd_k, T* dq, T* dk, T* __restrict__ dv_out, float* __restrict__ dbeta,
     float* __restrict__ dg, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N,
-    int Hqk, int Hv, int V, float scale, int hh) {
+    int Hqk, int Hv, int V, float scale, int hh, int64_t q_stride, TokenStrides ts) {
   using SM = BwdLocalSmem<T, DK>;
   constexpr int NKT = DK / 32, VEC = Elem<T>::kVec, KG = AccK<T>::kGroups;
   static_assert(NKT <= 4, "one 32-column block of K per wave");
@@ -349,9 +349,9 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     for (int j = 0; j < (int)sizeof(T) / 2; ++j) {   // raw dO and V blocks [64][32], rows past the end repeat the last row
       constexpr int LPR = 32 / VEC, RPP = 64 / LPR;  // lanes per row, rows per piece
       const int piece = 4 * j + wave, row = piece * RPP + lane / LPR, cc = lane % LPR;
-      const int64_t off = ((tok0 + imin(row, nvalid - 1)) * Hv + h) * V + 32 * vblk + cc * VEC;
-      load16_to_lds(dO + off, st + SM::st_doraw + piece * 64 * VEC);
-      load16_to_lds(v + off, st + SM::st_vraw + piece * 64 * VEC);
+      const int64_t tok = tok0 + imin(row, nvalid - 1), col = (int64_t)h * V + 32 * vblk + cc * VEC;
+      load16_to_lds(dO + tok * Hv * V + col, st + SM::st_doraw + piece * 64 * VEC);
+      load16_to_lds(v + tok * ts.v + col, st + SM::st_vraw + piece * 64 * VEC);
     }
     if (has_k) {
 #pragma unroll
@@ -376,7 +376,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
 #pragma unroll
       for (int piece = 0; piece < LPR; ++piece) {
         const int row = piece * RPP + lane / LPR, cc = lane % LPR;
-        load16_to_lds(q + ((tok0 + imin(row, nvalid - 1)) * Hqk + hq) * DK + 32 * cj + cc * VEC,
+        load16_to_lds(q + (tok0 + imin(row, nvalid - 1)) * q_stride + hq * DK + 32 * cj + cc * VEC,
                       st + SM::ea_q + wave * 2048 + piece * 64 * VEC);
       }
     }
@@ -420,7 +420,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       const f32x16 bsr = rows_ld(bs, 32 * rj);
 #pragma unroll
       for (int r = 0; r < 16; ++r) R[r] *= bsr[r];
-      acc_store_rows<T, false>(R, id, patch, dv_out + ((tok0 + 32 * rj) * Hv + h) * V + 32 * vblk, (int64_t)Hv * V,
+      acc_store_rows<T, false>(R, id, patch, dv_out + (tok0 + 32 * rj) * ts.dv + h * V + 32 * vblk, ts.dv,
                         nvalid - 32 * rj);
     }
   }
@@ -614,9 +614,9 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
 #pragma unroll
         for (int r = 0; r < 16; ++r) dQi[ri][r] = (dQi[ri][r] - dot[r] * qq[r]) * rs[r];
       }
-      T* dst = dq + ((tok0 + 32 * ri) * Hqk + hq) * DK + 32 * cj;
-      if (hh == 0) acc_store_rows<T, false>(dQi[ri], id, patch, dst, (int64_t)Hqk * DK, nvalid - 32 * ri);
-      else acc_store_rows<T, true>(dQi[ri], id, patch, dst, (int64_t)Hqk * DK, nvalid - 32 * ri);
+      T* dst = dq + (tok0 + 32 * ri) * ts.dq + hq * DK + 32 * cj;
+      if (hh == 0) acc_store_rows<T, false>(dQi[ri], id, patch, dst, ts.dq, nvalid - 32 * ri);
+      else acc_store_rows<T, true>(dQi[ri], id, patch, dst, ts.dq, nvalid - 32 * ri);
     }
   }
   GDN_LDS_BARRIER();
@@ -687,9 +687,9 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
         for (int r = 0; r < 16; ++r)
           dKi[ri][r] = (dKi[ri][r] - (d1[r] + br[r] * db[r] + df[r]) * kk[r]) * rs[r];
       }
-      T* dst = dk + ((tok0 + 32 * ri) * Hqk + hq) * DK + 32 * cj;
-      if (hh == 0) acc_store_rows<T, false>(dKi[ri], id, patch, dst, (int64_t)Hqk * DK, nvalid - 32 * ri);
-      else acc_store_rows<T, true>(dKi[ri], id, patch, dst, (int64_t)Hqk * DK, nvalid - 32 * ri);
+      T* dst = dk + (tok0 + 32 * ri) * ts.dk + hq * DK + 32 * cj;
+      if (hh == 0) acc_store_rows<T, false>(dKi[ri], id, patch, dst, ts.dk, nvalid - 32 * ri);
+      else acc_store_rows<T, true>(dKi[ri], id, patch, dst, ts.dk, nvalid - 32 * ri);
     }
   }
   if (wave == 0) {   // d(cumulative G) -> d(g): suffix sum inside the chunk
@@ -753,23 +753,28 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     for (int hh = 0; hh < d.Hv / d.Hqk; ++hh)
       GDN_LAUNCH(kKernBwdLocal, st, kern, dim3(nc, d.Hqk), dim3(kThreads), smem, st, qq, (const T*)KAF, (const T*)v,
                  beta, G, Ai, VF, (const T*)DVF, (const T*)dO, HF, (const T*)DHF, rstd_q, rstd_k, (T*)dq, (T*)dk,
-                 (T*)dv, dbeta, dg, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale, hh);
+                 (T*)dv, dbeta, dg, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale, hh,
+                 l2norm ? (int64_t)d.Hqk * d.K : d.strides().q, d.strides());
   }
   return (int)hipGetLastError();
 }
 
 }  // namespace gdn
 
-extern "C" int gdn_chunk_bwd(const void* q, const void* k, const void* v, const float* g, const float* beta,
-                             const float* initial_state, const int64_t* cu_seqlens, const void* d_o,
-                             const float* d_final_state, void* dq, void* dk, void* dv, float* dg, float* dbeta,
-                             float* d_initial_state, void* workspace, int64_t workspace_bytes, int B, int T, int N,
-                             int Hqk, int Hv, int K, int V, float scale, int use_qk_l2norm, int dtype, void* stream) {
+extern "C" int gdn_chunk_bwd_strided(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
+                                     int64_t v_stride, const float* g, const float* beta, const float* initial_state,
+                                     const int64_t* cu_seqlens, const void* d_o, const float* d_final_state, void* dq,
+                                     void* dk, void* dv, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride,
+                                     float* dg, float* dbeta, float* d_initial_state, void* workspace,
+                                     int64_t workspace_bytes, int B, int T, int N, int Hqk, int Hv, int K, int V,
+                                     float scale, int use_qk_l2norm, int dtype, void* stream) {
   using namespace gdn;
   (void)g; (void)initial_state;   // their effect is already in the workspace (G, per-chunk states)
   if (!q || !k || !v || !beta || !d_o || !dq || !dk || !dv || !dg || !dbeta || !workspace) return -1;
   ChunkDims d{B, T, N, Hqk, Hv, K, V, cu_seqlens != nullptr};
+  d.ts = {q_stride, k_stride, v_stride, dq_stride, dk_stride, dv_stride};
   if (int e = chunk_check_dims(d, dtype)) return e;
+  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)d_o | (uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv) & 15) return -6;
   ChunkDims dl = d;
   dl.varlen = true;
   const ChunkWorkspace L = chunk_workspace_layout(dl, dtype == 0 ? 4 : 2);
@@ -794,4 +799,14 @@ extern "C" int gdn_chunk_bwd(const void* q, const void* k, const void* v, const 
     GDN_BWD(float, 64, 2, 2, 2, 2);
   }
 #undef GDN_BWD
+}
+
+extern "C" int gdn_chunk_bwd(const void* q, const void* k, const void* v, const float* g, const float* beta,
+                             const float* initial_state, const int64_t* cu_seqlens, const void* d_o,
+                             const float* d_final_state, void* dq, void* dk, void* dv, float* dg, float* dbeta,
+                             float* d_initial_state, void* workspace, int64_t workspace_bytes, int B, int T, int N,
+                             int Hqk, int Hv, int K, int V, float scale, int use_qk_l2norm, int dtype, void* stream) {
+  return gdn_chunk_bwd_strided(q, k, v, 0, 0, 0, g, beta, initial_state, cu_seqlens, d_o, d_final_state, dq, dk, dv, 0, 0,
+                               0, dg, dbeta, d_initial_state, workspace, workspace_bytes, B, T, N, Hqk, Hv, K, V, scale,
+                               use_qk_l2norm, dtype, stream);
 }

@@ -64,7 +64,8 @@ __global__ void chunk_table_kernel(const int64_t* __restrict__ cu, int* __restri
 // ---------------------------------------------------------------------------------------------
 template <typename T, int DK>
 __device__ __forceinline__ void load_tile_qk(T* lds, int ld, const T* g, int64_t row_stride, int nvalid, int tid,
-                                             bool l2norm, T* y_out, float* rstd_out, int64_t rstd_stride) {
+                                             bool l2norm, T* y_out, int64_t y_stride, float* rstd_out,
+                                             int64_t rstd_stride) {
   constexpr int V = Elem<T>::kVec, CPR = DK / V;   // lanes per row: a power of two <= 32
   static_assert((64 * CPR) % kThreads == 0, "every thread takes the same number of pieces");
   for (int c = tid; c < 64 * CPR; c += kThreads) {
@@ -79,7 +80,7 @@ __device__ __forceinline__ void load_tile_qk(T* lds, int ld, const T* g, int64_t
       const float r = rsqrtf(ss + 1e-6f);
 #pragma unroll
       for (int e = 0; e < V; ++e) x.set(e, x.get(e) * r);
-      if (ok && y_out != nullptr) st16(y_out + (int64_t)row * row_stride + cc * V, x);
+      if (ok && y_out != nullptr) st16(y_out + (int64_t)row * y_stride + cc * V, x);
       if (ok && rstd_out != nullptr && cc == 0) rstd_out[(int64_t)row * rstd_stride] = r;
     }
     st16(lds + row * ld + cc * V, x);
@@ -112,7 +113,7 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(GDN_PREP_WPS) void chu
     float* __restrict__ G_out, T* __restrict__ Ai_out, T* __restrict__ W_out, T* __restrict__ U_out,
     T* __restrict__ Aq_out, T* __restrict__ KT_out, T* __restrict__ WF_out, T* __restrict__ KA_out,
     T* __restrict__ QT_out, T* __restrict__ qn_out, float* __restrict__ rstd_q_out, float* __restrict__ rstd_k_out,
-    int T_len, int N, int Hqk, int Hv, int V, float scale, int l2norm) {
+    int T_len, int N, int Hqk, int Hv, int V, float scale, int l2norm, TokenStrides ts) {
   using SM = PrepSmem<T, DK, BV>;
   constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64, VEC = Elem<T>::kVec;
   T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
@@ -152,10 +153,10 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(GDN_PREP_WPS) void chu
     // of each q/k group also leaves the normalised q (for the output kernel and the backward pass) and 1/|q|, 1/|k|.
     const bool keep = l2norm && (h % (Hv / Hqk)) == 0;
     const int64_t off = (tok0 * Hqk + hq) * DK, roff = tok0 * Hqk + hq;
-    load_tile_qk<T, DK>(Ks, LDK, k + off, (int64_t)Hqk * DK, nvalid, tid, l2norm != 0, nullptr,
+    load_tile_qk<T, DK>(Ks, LDK, k + tok0 * ts.k + hq * DK, ts.k, nvalid, tid, l2norm != 0, nullptr, 0,
                         keep ? rstd_k_out + roff : nullptr, Hqk);
-    load_tile_qk<T, DK>(Qs, LDK, q + off, (int64_t)Hqk * DK, nvalid, tid, l2norm != 0, keep ? qn_out + off : nullptr,
-                        keep ? rstd_q_out + roff : nullptr, Hqk);
+    load_tile_qk<T, DK>(Qs, LDK, q + tok0 * ts.q + hq * DK, ts.q, nvalid, tid, l2norm != 0, keep ? qn_out + off : nullptr,
+                        (int64_t)Hqk * DK, keep ? rstd_q_out + roff : nullptr, Hqk);
   }
   __syncthreads();
 
@@ -225,13 +226,13 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(GDN_PREP_WPS) void chu
     }
   }
   // the first V block is requested now and parked in registers until the fp32 Tm has been consumed
-  const T* vg = v + (tok0 * Hv + h) * V;
+  const T* vg = v + tok0 * ts.v + h * V;
   constexpr int VPT = 64 * (BV / VEC) / kThreads;   // 16-byte pieces of the V tile per thread
   Vec16<T> vreg[VPT];
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
     const int c = tid + i * kThreads, row = c / (BV / VEC), cc = c % (BV / VEC);
-    vreg[i] = row < nvalid ? ld16(vg + (int64_t)row * Hv * V + cc * VEC) : zero16<T>();
+    vreg[i] = row < nvalid ? ld16(vg + row * ts.v + cc * VEC) : zero16<T>();
   }
   __syncthreads();
 
@@ -346,7 +347,7 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(GDN_PREP_WPS) void chu
   for (int vb = 0; vb < V / BV; ++vb) {
     __syncthreads();
     if (vb > 0) {
-      load_tile_scaled<T, BV>(Vb, LDV, vg + vb * BV, (int64_t)Hv * V, nvalid, bs, tid);
+      load_tile_scaled<T, BV>(Vb, LDV, vg + vb * BV, ts.v, nvalid, bs, tid);
       __syncthreads();
     }
     for (int tt = wave; tt < 2 * (BV / 32); tt += 4) {
@@ -601,7 +602,7 @@ template <typename T, int DK, int NW>
 __global__ __launch_bounds__(64 * NW) GDN_WAVES_PER_SIMD(GDN_OUT_WPS) void chunk_out_kernel(
     const T* __restrict__ q, const T* __restrict__ aqf, const T* __restrict__ vf, const T* __restrict__ hf,
     const float* __restrict__ G, T* __restrict__ o, const int64_t* __restrict__ cu,
-    const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V, float scale) {
+    const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V, float scale, int64_t q_stride) {
   using SM = OutSmem<T, DK, NW>;
   constexpr int LDK = SM::LDK, NT = 64 * NW, VEC = Elem<T>::kVec, NKT = DK / 32;
   T* Qs = reinterpret_cast<T*>(gdn_smem + SM::off_qs);
@@ -628,7 +629,7 @@ __global__ __launch_bounds__(64 * NW) GDN_WAVES_PER_SIMD(GDN_OUT_WPS) void chunk
   for (int c = tid; c < 64 * (DK / VEC); c += NT) {
     const int row = c / (DK / VEC), cc = c % (DK / VEC);
     st16(Qs + row * LDK + cc * VEC,
-         row < nvalid ? ld16(q + ((tok0 + row) * Hqk + hq) * DK + cc * VEC) : zero16<T>());
+         row < nvalid ? ld16(q + (tok0 + row) * q_stride + hq * DK + cc * VEC) : zero16<T>());
   }
   if (tid < 64) Eg[tid] = scale * __expf(G[ch * 64 + imin(tid, nvalid - 1)]);
   IdentityFrag<T> id;
@@ -689,7 +690,7 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     if (int e = set_lds(kern, smem)) return e;
     GDN_LAUNCH(kKernPrep, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, (const T*)v, g, beta, cu,
                (const int*)chunk_offsets, G, Ai, W, UF, AQ, KTF, WF, KAF, QTF, qn, rstd, rstd + tok * d.Hqk, d.T, d.N, d.Hqk,
-               d.Hv, d.V, scale, l2norm);
+               d.Hv, d.V, scale, l2norm, d.strides());
   }
   {
     auto kern = chunk_state_kernel<T, DK, NWS, NLS, STAGES>;
@@ -705,7 +706,7 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     if (int e = set_lds(kern, smem)) return e;
     GDN_LAUNCH(kKernOut, st, kern, dim3(nc, d.Hv, d.V / (32 * NW)), dim3(64 * NW), smem, st, l2norm ? (const T*)qn : qq,
                (const T*)AQ, (const T*)VF, (const T*)HF, (const float*)G, (T*)o, cu, (const int*)chunk_offsets, d.T, d.N, d.Hqk,
-               d.Hv, d.V, scale);
+               d.Hv, d.V, scale, l2norm ? (int64_t)d.Hqk * d.K : d.strides().q);
   }
   return (int)hipGetLastError();
 }
@@ -735,14 +736,17 @@ extern "C" int64_t gdn_chunk_workspace_bytes(int B, int T, int N, int Hqk, int H
   return with_backward ? w.total_bytes : w.fwd_bytes;
 }
 
-extern "C" int gdn_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const float* beta,
-                             const float* initial_state, const int64_t* cu_seqlens, void* o, float* final_state,
-                             void* workspace, int64_t workspace_bytes, int B, int T, int N, int Hqk, int Hv, int K,
-                             int V, float scale, int use_qk_l2norm, int dtype, void* stream) {
+extern "C" int gdn_chunk_fwd_strided(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
+                                     int64_t v_stride, const float* g, const float* beta, const float* initial_state,
+                                     const int64_t* cu_seqlens, void* o, float* final_state, void* workspace,
+                                     int64_t workspace_bytes, int B, int T, int N, int Hqk, int Hv, int K, int V,
+                                     float scale, int use_qk_l2norm, int dtype, void* stream) {
   using namespace gdn;
   if (!q || !k || !v || !g || !beta || !o || !workspace) return -1;
   ChunkDims d{B, T, N, Hqk, Hv, K, V, cu_seqlens != nullptr};
+  d.ts = {q_stride, k_stride, v_stride, 0, 0, 0};
   if (int e = chunk_check_dims(d, dtype)) return e;
+  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o) & 15) return -6;
   ChunkDims dl = d;
   dl.varlen = true;  // one layout for both modes (the packed bound is the larger)
   const ChunkWorkspace L = chunk_workspace_layout(dl, dtype == 0 ? 4 : 2);
@@ -769,4 +773,12 @@ extern "C" int gdn_chunk_fwd(const void* q, const void* k, const void* v, const 
     GDN_FWD(float, 64, 64, 2, 2, 2, 2);
   }
 #undef GDN_FWD
+}
+
+extern "C" int gdn_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const float* beta,
+                             const float* initial_state, const int64_t* cu_seqlens, void* o, float* final_state,
+                             void* workspace, int64_t workspace_bytes, int B, int T, int N, int Hqk, int Hv, int K,
+                             int V, float scale, int use_qk_l2norm, int dtype, void* stream) {
+  return gdn_chunk_fwd_strided(q, k, v, 0, 0, 0, g, beta, initial_state, cu_seqlens, o, final_state, workspace,
+                               workspace_bytes, B, T, N, Hqk, Hv, K, V, scale, use_qk_l2norm, dtype, stream);
 }

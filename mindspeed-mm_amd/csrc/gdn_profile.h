@@ -8,7 +8,8 @@ namespace gdn {
 enum KernelId {
   kKernChunkTable = 0, kKernPrep, kKernStateFwd, kKernOut, kKernStateBwd, kKernBwdLocal,
   kKernRecurrent, kKernConvFwd, kKernConvState, kKernConvBwd, kKernConvReduce,
-  kKernConvDh0, kKernConvUpdate, kKernRmsNormFwd, kKernRmsNormBwd, kKernRmsNormReduce, kKernCount
+  kKernConvDh0, kKernConvUpdate, kKernRmsNormFwd, kKernRmsNormBwd, kKernRmsNormReduce,
+  kKernGateFwd, kKernGateBwd, kKernGateReduce, kKernCount
 };
 
 bool profile_on();

@@ -17,6 +17,8 @@ SIGNATURES = {
     "gdn_chunk_workspace_bytes": (L, [I] * 9),
     "gdn_chunk_fwd": (I, [P] * 10 + [L] + [I] * 7 + [F, I, I, P]),
     "gdn_chunk_bwd": (I, [P] * 16 + [L] + [I] * 7 + [F, I, I, P]),
+    "gdn_chunk_fwd_strided": (I, [P] * 3 + [L] * 3 + [P] * 7 + [L] + [I] * 7 + [F, I, I, P]),
+    "gdn_chunk_bwd_strided": (I, [P] * 3 + [L] * 3 + [P] * 9 + [L] * 3 + [P] * 4 + [L] + [I] * 7 + [F, I, I, P]),
     "gdn_recurrent_fwd": (I, [P] * 8 + [I] * 6 + [F, I, I, P]),
     "gdn_conv1d_fwd": (I, [P] * 8 + [I] * 7 + [P]),
     "gdn_conv1d_bwd_workspace_bytes": (L, [I] * 4),
@@ -25,6 +27,9 @@ SIGNATURES = {
     "gdn_rmsnorm_gated_fwd": (I, [P] * 5 + [L, I, F, I, I, P]),
     "gdn_rmsnorm_gated_bwd_workspace_bytes": (L, [L, I]),
     "gdn_rmsnorm_gated_bwd": (I, [P] * 9 + [L, L, I, I, I, P]),
+    "gdn_gate_fwd": (I, [P] * 6 + [L, I, I, I, P]),
+    "gdn_gate_bwd_workspace_bytes": (L, [L, I]),
+    "gdn_gate_bwd": (I, [P] * 11 + [L, L, I, I, I, P]),
     "gdn_profile_enable": (I, [I]),
     "gdn_profile_kernel_count": (I, []),
     "gdn_profile_kernel_name": (ctypes.c_char_p, [I]),
@@ -40,6 +45,7 @@ _ERRORS = {
         "norm rows of 4/8/16/32/64 16-byte pieces)",
     -4: "unsupported dtype",
     -5: "workspace too small or misaligned",
+    -6: "token stride not a multiple of 16 bytes or shorter than a token's heads, or a pointer not 16-byte aligned",
 }
 
 

@@ -6,6 +6,8 @@
     causal_conv1d                     mindspeed_mm/fsdp/models/qwen3_5/causal_conv1d.py:100-119
     causal_conv1d_update              modeling_qwen3_5.py:373-389, called at :738-744
     rms_norm_gated / RMSNormGated     Qwen3_5RMSNormGated, modeling_qwen3_5.py:330-349, called at :897-900
+    gdn_gates                         g / beta recipe of the layer, modeling_qwen3_5.py:833-841
+    chunk_gated_delta_rule_qkv        the rule on the unsplit convolution output (split at :818-831)
 
 Everything here is host glue: validation, output/workspace allocation with torch, and one call into the
 C ABI per operator.  The kernels themselves are the HIP library; nothing in this file computes.
@@ -84,6 +86,44 @@ class GdnOps:
         self._need(q, k, v, g, beta, initial_state, cu_seqlens)
         return _ChunkGatedDeltaRule.apply(q, k, v, g, beta, float(scale), initial_state, bool(output_final_state),
                                           cu_seqlens, bool(use_qk_l2norm_in_kernel), self)
+
+    def chunk_gated_delta_rule_qkv(self, mixed_qkv, g, beta, num_k_heads, num_v_heads, head_k_dim, head_v_dim,
+                                   scale=None, initial_state=None, output_final_state=False,
+                                   use_qk_l2norm_in_kernel=False, cu_seqlens=None):
+        """chunk_gated_delta_rule on the unsplit [B,T,2 Hqk K + Hv V] output of the convolution: equal to splitting it
+        into q, k, v as modeling_qwen3_5.py:818-831 does and calling chunk_gated_delta_rule, without the copies."""
+        if mixed_qkv.dim() != 3 or mixed_qkv.shape[-1] < 2 * num_k_heads * head_k_dim + num_v_heads * head_v_dim:
+            raise ValueError("expected mixed_qkv [B, T, D] with D >= 2 * num_k_heads * head_k_dim + num_v_heads * head_v_dim")
+        if mixed_qkv.dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"chunk_gated_delta_rule supports bfloat16 and float32, got {mixed_qkv.dtype}")
+        if len(beta.shape) != 3 or g.shape != beta.shape or \
+                tuple(g.shape) != (mixed_qkv.shape[0], mixed_qkv.shape[1], num_v_heads) or num_v_heads % num_k_heads:
+            raise ValueError("expected g, beta [B, T, Hv] with Hv % Hqk == 0")
+        if cu_seqlens is not None:
+            if mixed_qkv.shape[0] != 1:
+                raise ValueError(
+                    f"The batch size is expected to be 1 rather than {mixed_qkv.shape[0]} when using `cu_seqlens`."
+                    f"Please flatten variable-length inputs before processing.")
+            if initial_state is not None and initial_state.shape[0] != len(cu_seqlens) - 1:
+                raise ValueError(
+                    f"The number of initial states is expected to be equal to the number of input sequences, "
+                    f"i.e., {len(cu_seqlens) - 1} rather than {initial_state.shape[0]}.")
+        if scale is None:
+            scale = head_k_dim ** -0.5
+        self._need(mixed_qkv, g, beta, initial_state, cu_seqlens)
+        return _ChunkGatedDeltaRuleQKV.apply(mixed_qkv, g, beta, int(num_k_heads), int(num_v_heads), int(head_k_dim),
+                                             int(head_v_dim), float(scale), initial_state, bool(output_final_state),
+                                             cu_seqlens, bool(use_qk_l2norm_in_kernel), self)
+
+    def gdn_gates(self, a, b, A_log, dt_bias):
+        """(g, beta) of the layer from its projections a, b [..., Hv] and parameters A_log, dt_bias [Hv]:
+        beta = b.sigmoid(), g = -A_log.float().exp() * softplus(a.float() + dt_bias) (modeling_qwen3_5.py:833-841)."""
+        if a.shape != b.shape or a.dtype != b.dtype or A_log.shape != (a.shape[-1],) or dt_bias.shape != A_log.shape:
+            raise ValueError("expected a, b [..., Hv] of one dtype and A_log, dt_bias [Hv]")
+        if a.dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"gdn_gates supports bfloat16 and float32, got {a.dtype}")
+        self._need(a, b, A_log, dt_bias)
+        return _GdnGates.apply(a, b, A_log, dt_bias, self)
 
     # ------------------------------------------------------------------ decode
     def fused_recurrent_gated_delta_rule(self, q, k, v, g, beta=None, scale=None, initial_state=None,
@@ -169,6 +209,25 @@ def _i64(cu, ref):
     return cu.to(device=ref.device, dtype=torch.int64).contiguous()
 
 
+def _token_view(x):
+    """(tensor, token stride in elements) for a [B,T,H,D] tensor whose heads are contiguous within a token and whose
+    tokens are evenly spaced (a column slice of a wider [B,T,*] tensor qualifies); anything else is copied."""
+    B, T, H, D = x.shape
+    vec = 16 // x.element_size()
+    ok = (x.stride(3) == 1 and x.stride(2) == D and x.stride(1) >= H * D and x.stride(1) % vec == 0
+          and (B == 1 or x.stride(0) == T * x.stride(1)) and x.data_ptr() % 16 == 0)
+    if not ok:
+        x = x.contiguous()
+    return x, x.stride(1)
+
+
+def _chunk_workspace(lib, device, B, T, N, Hqk, Hv, K, V, code, need_grad):
+    nbytes = lib.gdn_chunk_workspace_bytes(B, T, N, Hqk, Hv, K, V, code, int(need_grad))
+    ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=device)
+    off = (-ws.data_ptr()) % 256
+    return ws[off:off + nbytes], nbytes
+
+
 class _ChunkGatedDeltaRule(torch.autograd.Function):
     """Positional order as ChunkGatedDeltaRuleFunction.forward (chunk_gated_delta_rule.py:182-196)."""
 
@@ -180,44 +239,142 @@ class _ChunkGatedDeltaRule(torch.autograd.Function):
         Hv, V = v.shape[2], v.shape[3]
         N = (len(cu_seqlens) - 1) if cu_seqlens is not None else B
         need_grad = any(ctx.needs_input_grad[:5]) or (initial_state is not None and ctx.needs_input_grad[6])
-        qc, kc, vc = q.contiguous(), k.contiguous(), v.contiguous()
+        (qc, sq), (kc, sk), (vc, sv) = _token_view(q), _token_view(k), _token_view(v)
         g32, b32, h0 = ops._f32(g), ops._f32(beta), ops._f32(initial_state)
         cu = _i64(cu_seqlens, q)
         code = DTYPE_CODE[q.dtype]
-        nbytes = lib.gdn_chunk_workspace_bytes(B, T, N, Hqk, Hv, K, V, code, int(need_grad))
-        ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=q.device)
-        off = (-ws.data_ptr()) % 256
-        ws = ws[off:off + nbytes]
-        o = torch.empty_like(vc)
+        ws, nbytes = _chunk_workspace(lib, q.device, B, T, N, Hqk, Hv, K, V, code, need_grad)
+        o = torch.empty(B, T, Hv, V, dtype=v.dtype, device=v.device)
         ht = torch.empty(N, Hv, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
-        rc = lib.gdn_chunk_fwd(ptr(qc), ptr(kc), ptr(vc), ptr(g32), ptr(b32), ptr(h0), ptr(cu), ptr(o), ptr(ht),
-                               ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale, int(use_qk_l2norm_in_kernel), code,
-                               lib.stream())
-        lib.check(rc, "gdn_chunk_fwd")
+        rc = lib.gdn_chunk_fwd_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(b32), ptr(h0), ptr(cu),
+                                       ptr(o), ptr(ht), ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale,
+                                       int(use_qk_l2norm_in_kernel), code, lib.stream())
+        lib.check(rc, "gdn_chunk_fwd_strided")
         if need_grad:
             ctx.save_for_backward(qc, kc, vc, g32, b32, h0, cu, ws)
             ctx.meta = (B, T, N, Hqk, Hv, K, V, scale, int(use_qk_l2norm_in_kernel), code, nbytes,
-                        g.dtype, beta.dtype, None if initial_state is None else initial_state.dtype)
+                        g.dtype, beta.dtype, None if initial_state is None else initial_state.dtype, sq, sk, sv)
             ctx.ops = ops
         return o, ht
 
     @staticmethod
     def backward(ctx, do, dht):
         qc, kc, vc, g32, b32, h0, cu, ws = ctx.saved_tensors
-        B, T, N, Hqk, Hv, K, V, scale, l2, code, nbytes, g_dt, b_dt, h_dt = ctx.meta
+        B, T, N, Hqk, Hv, K, V, scale, l2, code, nbytes, g_dt, b_dt, h_dt, sq, sk, sv = ctx.meta
         lib = ctx.ops.lib
         do = do.contiguous()
         dht = ctx.ops._f32(dht)
-        dq, dk, dv = torch.empty_like(qc), torch.empty_like(kc), torch.empty_like(vc)
-        dg = torch.empty(B, T, Hv, dtype=torch.float32, device=qc.device)
-        db = torch.empty(B, T, Hv, dtype=torch.float32, device=qc.device)
-        dh0 = torch.empty(N, Hv, K, V, dtype=torch.float32, device=qc.device) if h0 is not None else None
-        rc = lib.gdn_chunk_bwd(ptr(qc), ptr(kc), ptr(vc), ptr(g32), ptr(b32), ptr(h0), ptr(cu), ptr(do), ptr(dht),
-                               ptr(dq), ptr(dk), ptr(dv), ptr(dg), ptr(db), ptr(dh0), ptr(ws), nbytes, B, T, N, Hqk,
-                               Hv, K, V, scale, l2, code, lib.stream())
-        lib.check(rc, "gdn_chunk_bwd")
+        dev = qc.device
+        dq = torch.empty(B, T, Hqk, K, dtype=qc.dtype, device=dev)
+        dk = torch.empty(B, T, Hqk, K, dtype=qc.dtype, device=dev)
+        dv = torch.empty(B, T, Hv, V, dtype=qc.dtype, device=dev)
+        dg = torch.empty(B, T, Hv, dtype=torch.float32, device=dev)
+        db = torch.empty(B, T, Hv, dtype=torch.float32, device=dev)
+        dh0 = torch.empty(N, Hv, K, V, dtype=torch.float32, device=dev) if h0 is not None else None
+        rc = lib.gdn_chunk_bwd_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(b32), ptr(h0), ptr(cu),
+                                       ptr(do), ptr(dht), ptr(dq), ptr(dk), ptr(dv), 0, 0, 0, ptr(dg), ptr(db),
+                                       ptr(dh0), ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale, l2, code,
+                                       lib.stream())
+        lib.check(rc, "gdn_chunk_bwd_strided")
         return (dq, dk, dv, dg.to(g_dt), db.to(b_dt), None, None if dh0 is None else dh0.to(h_dt), None, None, None,
                 None)
+
+
+class _ChunkGatedDeltaRuleQKV(torch.autograd.Function):
+    """The rule on the convolution's output as it is: q, k, v are the column ranges [0, Hqk K), [Hqk K, 2 Hqk K),
+    [2 Hqk K, 2 Hqk K + Hv V) of mixed_qkv [B,T,D] (the split of modeling_qwen3_5.py:818-831), read in place; the
+    backward pass writes dq, dk, dv into one [B,T,D] gradient, so neither the split nor its backward copies."""
+
+    @staticmethod
+    def forward(ctx, qkv, g, beta, Hqk, Hv, K, V, scale, initial_state, output_final_state, cu_seqlens,
+                use_qk_l2norm_in_kernel, ops):
+        lib = ops.lib
+        B, T, D = qkv.shape
+        nq, nv = Hqk * K, Hv * V
+        N = (len(cu_seqlens) - 1) if cu_seqlens is not None else B
+        need_grad = any(ctx.needs_input_grad[:3]) or (initial_state is not None and ctx.needs_input_grad[8])
+        vec = 16 // qkv.element_size()
+        x = qkv if (qkv.is_contiguous() and D % vec == 0 and qkv.data_ptr() % 16 == 0) else qkv.contiguous()
+        g32, b32, h0 = ops._f32(g), ops._f32(beta), ops._f32(initial_state)
+        cu = _i64(cu_seqlens, qkv)
+        code = DTYPE_CODE[qkv.dtype]
+        es = x.element_size()
+        ws, nbytes = _chunk_workspace(lib, qkv.device, B, T, N, Hqk, Hv, K, V, code, need_grad)
+        o = torch.empty(B, T, Hv, V, dtype=qkv.dtype, device=qkv.device)
+        ht = torch.empty(N, Hv, K, V, dtype=torch.float32, device=qkv.device) if output_final_state else None
+        base = x.data_ptr()
+        rc = lib.gdn_chunk_fwd_strided(base, base + nq * es, base + 2 * nq * es, D, D, D, ptr(g32), ptr(b32), ptr(h0),
+                                       ptr(cu), ptr(o), ptr(ht), ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale,
+                                       int(use_qk_l2norm_in_kernel), code, lib.stream())
+        lib.check(rc, "gdn_chunk_fwd_strided")
+        if need_grad:
+            ctx.save_for_backward(x, g32, b32, h0, cu, ws)
+            ctx.meta = (B, T, D, N, Hqk, Hv, K, V, scale, int(use_qk_l2norm_in_kernel), code, nbytes,
+                        g.dtype, beta.dtype, None if initial_state is None else initial_state.dtype)
+            ctx.ops = ops
+        return o, ht
+
+    @staticmethod
+    def backward(ctx, do, dht):
+        x, g32, b32, h0, cu, ws = ctx.saved_tensors
+        B, T, D, N, Hqk, Hv, K, V, scale, l2, code, nbytes, g_dt, b_dt, h_dt = ctx.meta
+        lib = ctx.ops.lib
+        nq, nv, es, dev = Hqk * K, Hv * V, x.element_size(), x.device
+        do = do.contiguous()
+        dht = ctx.ops._f32(dht)
+        # columns past q, k, v (none in the layer) receive no gradient
+        dx = torch.empty_like(x) if D == 2 * nq + nv else torch.zeros_like(x)
+        dg = torch.empty(B, T, Hv, dtype=torch.float32, device=dev)
+        db = torch.empty(B, T, Hv, dtype=torch.float32, device=dev)
+        dh0 = torch.empty(N, Hv, K, V, dtype=torch.float32, device=dev) if h0 is not None else None
+        base, dbase = x.data_ptr(), dx.data_ptr()
+        rc = lib.gdn_chunk_bwd_strided(base, base + nq * es, base + 2 * nq * es, D, D, D, ptr(g32), ptr(b32), ptr(h0),
+                                       ptr(cu), ptr(do), ptr(dht), dbase, dbase + nq * es, dbase + 2 * nq * es, D, D,
+                                       D, ptr(dg), ptr(db), ptr(dh0), ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale,
+                                       l2, code, lib.stream())
+        lib.check(rc, "gdn_chunk_bwd_strided")
+        return (dx, dg.to(g_dt), db.to(b_dt), None, None, None, None, None, None if dh0 is None else dh0.to(h_dt),
+                None, None, None, None)
+
+
+class _GdnGates(torch.autograd.Function):
+    """beta = sigmoid(b), g = -exp(A_log.float()) * softplus(a.float() + dt_bias), modeling_qwen3_5.py:833-841."""
+
+    @staticmethod
+    def forward(ctx, a, b, A_log, dt_bias, ops):
+        lib = ops.lib
+        Hv = a.shape[-1]
+        ac, bc = a.contiguous(), b.contiguous()
+        pdt = a.dtype if (A_log.dtype == a.dtype and dt_bias.dtype == a.dtype) else torch.float32
+        Ac, dc = A_log.detach().to(pdt).contiguous(), dt_bias.detach().to(pdt).contiguous()
+        tokens = ac.numel() // Hv
+        g = torch.empty(ac.shape, dtype=torch.float32, device=a.device)
+        beta = torch.empty_like(bc)
+        rc = lib.gdn_gate_fwd(ptr(ac), ptr(bc), ptr(Ac), ptr(dc), ptr(g), ptr(beta), tokens, Hv, DTYPE_CODE[a.dtype],
+                              DTYPE_CODE[pdt], lib.stream())
+        lib.check(rc, "gdn_gate_fwd")
+        ctx.save_for_backward(ac, bc, Ac, dc)
+        ctx.meta = (tokens, Hv, A_log.dtype, dt_bias.dtype)
+        ctx.ops = ops
+        return g, beta
+
+    @staticmethod
+    def backward(ctx, dg, dbeta):
+        ac, bc, Ac, dc = ctx.saved_tensors
+        tokens, Hv, A_dt, d_dt = ctx.meta
+        lib = ctx.ops.lib
+        dg = dg.to(torch.float32).contiguous()
+        dbeta = dbeta.to(bc.dtype).contiguous()
+        da, db = torch.empty_like(ac), torch.empty_like(bc)
+        dA = torch.empty(Hv, dtype=torch.float32, device=ac.device)
+        dd = torch.empty(Hv, dtype=torch.float32, device=ac.device)
+        nbytes = lib.gdn_gate_bwd_workspace_bytes(tokens, Hv)
+        ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device=ac.device)
+        rc = lib.gdn_gate_bwd(ptr(ac), ptr(bc), ptr(Ac), ptr(dc), ptr(dg), ptr(dbeta), ptr(da), ptr(db), ptr(dA),
+                              ptr(dd), ptr(ws), nbytes, tokens, Hv, DTYPE_CODE[ac.dtype], DTYPE_CODE[Ac.dtype],
+                              lib.stream())
+        lib.check(rc, "gdn_gate_bwd")
+        return da, db, dA.to(A_dt), dd.to(d_dt), None
 
 
 class _CausalConv1d(torch.autograd.Function):
@@ -340,6 +497,18 @@ def chunk_gated_delta_rule(q, k, v, g, beta, scale=None, initial_state=None, out
 
 
 @torch.compiler.disable
+def chunk_gated_delta_rule_qkv(mixed_qkv, g, beta, num_k_heads, num_v_heads, head_k_dim, head_v_dim, scale=None,
+                               initial_state=None, output_final_state=False, use_qk_l2norm_in_kernel=False,
+                               cu_seqlens=None):
+    return _default_ops().chunk_gated_delta_rule_qkv(mixed_qkv, g, beta, num_k_heads, num_v_heads, head_k_dim,
+                                                     head_v_dim, scale, initial_state, output_final_state,
+                                                     use_qk_l2norm_in_kernel, cu_seqlens)
+
+
+def gdn_gates(a, b, A_log, dt_bias):
+    return _default_ops().gdn_gates(a, b, A_log, dt_bias)
+
+
 def fused_recurrent_gated_delta_rule(q, k, v, g, beta=None, scale=None, initial_state=None,
                                      output_final_state=False, cu_seqlens=None, use_qk_l2norm_in_kernel=False,
                                      inplace_state=False):

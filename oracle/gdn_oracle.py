@@ -17,6 +17,7 @@ relative to the reference checkout):
 * ``causal_conv1d_update_ref``     modeling_qwen3_5.py:373-389
 * ``pad_and_batch``                tests/ut_fsdp/models/qwen3_5/test_chunk_gated_delta_rule.py:14-28
 * ``rms_norm_gated_ref``           Qwen3_5RMSNormGated.forward, modeling_qwen3_5.py:341-349 (the non-NPU branch)
+* ``gdn_gates_ref``                g / beta recipe of Qwen3_5GatedDeltaNet.forward, modeling_qwen3_5.py:833-841
 
 The reference functions take neither ``scale``, ``cu_seqlens`` nor grouped
 (GQA) q/k heads; the operator entry does
@@ -36,6 +37,8 @@ How each function is pinned (tests/test_oracle_*.py):
 * conv1d == ``F.conv1d(groups=D)`` library routine and autograd thereof;
 * gated RMSNorm == ``F.rms_norm`` (library routine) times ``F.silu(gate)`` in fp64, the closed form for a constant
   row, scale invariance in x, ``gradcheck``;
+* gate recipe == ``torch.special.expit`` / ``torch.logaddexp(x, 0)`` (library routines other than the ones it
+  calls) in fp64, closed forms at a + dt_bias = 0 and b = 0, the benchmark input generator's own g, ``gradcheck``;
 * committed golden vectors under ``tests/golden`` (made by the fp64
   recurrence) guard against drift.
 
@@ -335,3 +338,14 @@ def rms_norm_gated_ref(hidden_states: torch.Tensor, gate: torch.Tensor, weight: 
     x = weight * x.to(input_dtype)
     x = x * F.silu(gate.to(torch.float32))
     return x.to(input_dtype)
+
+
+def gdn_gates_ref(a: torch.Tensor, b: torch.Tensor, A_log: torch.Tensor,
+                  dt_bias: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(g, beta) as Qwen3_5GatedDeltaNet.forward forms them (modeling_qwen3_5.py:833-841, the branch without sequence
+    parallelism): ``beta = b.sigmoid()`` in b's dtype, ``g = -A_log.float().exp() * softplus(a.float() + dt_bias)``
+    in fp32 (fp64 inputs stay fp64).  Differentiable."""
+    beta = b.sigmoid()
+    up = torch.float64 if a.dtype == torch.float64 else torch.float32
+    g = -A_log.to(up).exp() * F.softplus(a.to(up) + dt_bias)
+    return g, beta

@@ -139,3 +139,82 @@ def check_rms_norm_gated(ops, device, rows_shape, N, dtype, weight_dtype=None, s
         errs["dw"] = _err("dweight", L["w"].grad, R32["w"].grad, dtype, 1e-2 * scale, rtol=1e-2)
     return errs
 
+
+def check_chunk_qkv(ops, device, B, T, Hqk, Hv, K, V, dtype, l2=True, cu=None, backward=True, seed=0, pad=0,
+                    wrap=lambda t: t, **recipe):
+    """The rule on the unsplit [B,T,D] tensor (q | k | v | `pad` unused columns) against the oracle on the split
+    tensors, and bit for bit against the operator on contiguous q, k, v (same kernels, other strides)."""
+    N = (len(cu) - 1) if cu is not None else B
+    x = gdn_inputs(B, T, Hqk, Hv, K, V, dtype, seed=seed, N=N, l2norm_in_kernel=l2, **recipe)
+    nq, nv = Hqk * K, Hv * V
+    mixed = torch.cat([x["q"].reshape(B, T, nq), x["k"].reshape(B, T, nq), x["v"].reshape(B, T, nv),
+                       torch.zeros(B, T, pad, dtype=dtype)], dim=-1)
+    dev = {n: wrap(t.to(device)) for n, t in x.items()}
+    mx = wrap(mixed.to(device)).clone().requires_grad_(backward)
+    g, beta = (dev[n].clone().requires_grad_(backward) for n in ("g", "beta"))
+    h0 = dev["h0"].clone().requires_grad_(backward)
+    cu_t = torch.tensor(cu, dtype=torch.int64, device=device) if cu is not None else None
+    o, ht = ops.chunk_gated_delta_rule_qkv(mx, g, beta, Hqk, Hv, K, V, initial_state=h0, output_final_state=True,
+                                           use_qk_l2norm_in_kernel=l2, cu_seqlens=cu_t)
+    # the same through column slices of the wide tensor (views: read in place) and through contiguous copies
+    mx2 = mx.detach().clone().requires_grad_(backward)
+    q2, k2, v2 = torch.split(mx2, [nq, nq, nv, pad][:3 + (pad > 0)], dim=-1)[:3]
+    leaves2 = [t.clone().requires_grad_(backward) for t in (dev["g"], dev["beta"], dev["h0"])]
+    o2, ht2 = ops.chunk_gated_delta_rule(q2.reshape(B, T, Hqk, K), k2.reshape(B, T, Hqk, K), v2.reshape(B, T, Hv, V),
+                                         leaves2[0], leaves2[1], initial_state=leaves2[2], output_final_state=True,
+                                         use_qk_l2norm_in_kernel=l2, cu_seqlens=cu_t)
+    assert torch.equal(o, o2) and torch.equal(ht, ht2)
+    ref = {n: x[n].float().clone().requires_grad_(backward) for n in ("q", "k", "v", "g", "beta")}
+    rh0 = x["h0"].clone().requires_grad_(backward)
+    ro, rht = O.chunk_gated_delta_rule_ref(ref["q"], ref["k"], ref["v"], ref["g"], ref["beta"], initial_state=rh0,
+                                           output_final_state=True, use_qk_l2norm_in_kernel=l2, cu_seqlens=cu)
+    errs = {"o": _err("o", o, ro, dtype, BF16_ABS_O), "ht": _err("final_state", ht, rht, dtype, BF16_ABS_GRAD)}
+    if backward:
+        ((o.float() * dev["do"].float()).sum() + (ht * dev["dht"]).sum()).backward()
+        ((o2.float() * dev["do"].float()).sum() + (ht2 * dev["dht"]).sum()).backward()
+        ((ro * x["do"].float()).sum() + (rht * x["dht"]).sum()).backward()
+        assert mx.grad.shape == mx.shape and mx.grad.dtype == dtype
+        assert torch.equal(mx.grad, mx2.grad), "packed gradient differs from the gradient through the split views"
+        assert torch.equal(g.grad, leaves2[0].grad) and torch.equal(beta.grad, leaves2[1].grad)
+        assert torch.equal(h0.grad, leaves2[2].grad)
+        dq, dk, dv = mx.grad[..., :nq], mx.grad[..., nq:2 * nq], mx.grad[..., 2 * nq:2 * nq + nv]
+        errs["dq"] = _err("dq", dq.reshape(B, T, Hqk, K), ref["q"].grad, dtype, BF16_ABS_GRAD)
+        errs["dk"] = _err("dk", dk.reshape(B, T, Hqk, K), ref["k"].grad, dtype, BF16_ABS_GRAD)
+        errs["dv"] = _err("dv", dv.reshape(B, T, Hv, V), ref["v"].grad, dtype, BF16_ABS_GRAD)
+        if pad:
+            assert not mx.grad[..., 2 * nq + nv:].any()
+        errs["dg"] = _err("dg", g.grad, ref["g"].grad, dtype, BF16_ABS_GRAD)
+        errs["dbeta"] = _err("dbeta", beta.grad, ref["beta"].grad, dtype, BF16_ABS_GRAD)
+        errs["dh0"] = _err("dh0", h0.grad, rh0.grad, dtype, BF16_ABS_GRAD)
+    return errs
+
+
+def check_gdn_gates(ops, device, shape, Hv, dtype, param_dtype=None, seed=0, backward=True, wrap=lambda t: t):
+    """Gate recipe against the oracle on the same (dtype-valued) inputs.  g is fp32 on both sides (relative 1e-4 of
+    the largest value, the fp32 bar); beta and the gradients in half precision carry one rounding to bf16."""
+    gen = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=gen)
+    param_dtype = param_dtype or dtype
+    x = dict(a=(2.0 * r(*shape, Hv)).to(dtype), b=(2.0 * r(*shape, Hv)).to(dtype),
+             A=torch.empty(Hv).uniform_(0.0, 2.77, generator=gen).to(param_dtype),
+             d=torch.empty(Hv).uniform_(-4.0, -2.0, generator=gen).to(param_dtype),
+             dg=r(*shape, Hv), dbeta=r(*shape, Hv).to(dtype))
+    x["a"].view(-1)[:3] = torch.tensor([30.0, 24.5, -30.0]).to(dtype)    # both softplus branches and the far left
+    dev = {n: wrap(t.to(device)) for n, t in x.items()}
+    L = {n: dev[n].clone().requires_grad_(backward) for n in ("a", "b", "A", "d")}
+    g, beta = ops.gdn_gates(L["a"], L["b"], L["A"], L["d"])
+    R = {n: x[n].float().clone().requires_grad_(backward) for n in ("a", "b", "A", "d")}
+    rg, rbeta = O.gdn_gates_ref(R["a"], R["b"], R["A"], R["d"])
+    assert g.dtype == torch.float32 and beta.dtype == dtype and g.shape == rg.shape
+    errs = {"g": _err("g", g, rg, torch.float32, 0), "beta": _err("beta", beta, rbeta, dtype, 4e-3)}
+    if backward:
+        ((g * dev["dg"]).sum() + (beta.float() * dev["dbeta"].float()).sum()).backward()
+        ((rg * x["dg"]).sum() + (rbeta * x["dbeta"].float()).sum()).backward()
+        for n, m in (("a", "da"), ("b", "db")):
+            assert L[n].grad.dtype == dtype
+            errs[m] = _err(m, L[n].grad, R[n].grad, dtype, 5e-2, rtol=1e-2)
+        for n, m in (("A", "dA_log"), ("d", "ddt_bias")):
+            assert L[n].grad.dtype == param_dtype
+            scale = max(R[n].grad.abs().max().item(), 1.0)
+            errs[m] = _err(m, L[n].grad, R[n].grad, param_dtype, 1e-2 * scale, rtol=1e-2)
+    return errs

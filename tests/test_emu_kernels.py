@@ -73,3 +73,19 @@ def test_conv1d_update(ops, dtype, B, T, D, W):
 def test_rms_norm_gated(ops, dtype, shape, N, wdt):
     P.check_rms_norm_gated(ops, "cpu", shape, N, dtype, weight_dtype=wdt, wrap=guarded)
 
+
+@pytest.mark.parametrize("dtype,B,T,Hqk,Hv,K,V,l2,cu,pad", [
+    (F32, 1, 100, 1, 2, 64, 64, True, None, 0),
+    (BF, 2, 70, 2, 4, 128, 128, True, None, 0),
+    (BF, 1, 140, 2, 2, 64, 64, False, [0, 5, 70, 71, 140], 16),
+])
+def test_chunk_on_unsplit_qkv(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu, pad):
+    P.check_chunk_qkv(ops, "cpu", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu, pad=pad, wrap=guarded, h0_std=0.1)
+
+
+@pytest.mark.parametrize("dtype,shape,Hv,pdt", [
+    (F32, (2, 37), 6, None), (BF, (1, 300), 32, None), (BF, (3, 5), 48, torch.float32), (F32, (1,), 256, None),
+    (BF, (1100,), 4, None),
+])
+def test_gdn_gates(ops, dtype, shape, Hv, pdt):
+    P.check_gdn_gates(ops, "cpu", shape, Hv, dtype, param_dtype=pdt, wrap=guarded)

@@ -3,6 +3,7 @@ oracle on the same seeded inputs.  Run with `-m gpu` on an MI355X."""
 import pytest
 import torch
 
+from oracle import gdn_oracle as O
 from tests import parity as P
 
 pytestmark = pytest.mark.gpu
@@ -111,3 +112,67 @@ def test_rms_norm_gated_module_matches_functional(ops):
     with pytest.raises(ValueError):
         ops.rms_norm_gated(x[..., :100].contiguous(), z[..., :100].contiguous(), m.weight[:100])
 
+
+
+@pytest.mark.parametrize("dtype,B,T,Hqk,Hv,K,V,l2,cu,pad", [
+    (F32, 1, 100, 1, 2, 64, 64, True, None, 0),
+    (BF, 2, 200, 2, 4, 128, 128, True, None, 0),
+    (BF, 1, 140, 2, 2, 64, 64, False, [0, 5, 70, 71, 140], 16),
+    (BF, 1, 512, 4, 8, 128, 128, True, [0, 100, 512], 0),
+])
+def test_chunk_on_unsplit_qkv(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu, pad):
+    print(f"chunk qkv {dtype} B{B} T{T} Hqk{Hqk} Hv{Hv} K{K} V{V} l2={l2} varlen={cu is not None} pad={pad}", flush=True)
+    P.check_chunk_qkv(ops, "cuda", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu, pad=pad, h0_std=0.1)
+
+
+def test_chunk_rejects_bad_strides(ops):
+    """A token stride that breaks 16-byte alignment cannot be read in place: the op copies; the C ABI refuses."""
+    B, T, H, K = 1, 64, 1, 64
+    wide = torch.randn(B, T, 3 * K + 4, device="cuda", dtype=BF)
+    q, k, v = (wide[..., i * K:(i + 1) * K].reshape(B, T, H, K) for i in range(3))
+    g = -torch.rand(B, T, H, device="cuda")
+    beta = torch.rand(B, T, H, device="cuda")
+    o, _ = ops.chunk_gated_delta_rule(q, k, v, g, beta)
+    o2, _ = ops.chunk_gated_delta_rule(q.contiguous(), k.contiguous(), v.contiguous(), g, beta)
+    assert torch.equal(o, o2)
+    lib = ops.lib
+    ws = torch.empty(lib.gdn_chunk_workspace_bytes(B, T, B, H, H, K, K, 1, 0) + 256, dtype=torch.uint8, device="cuda")
+    rc = lib.gdn_chunk_fwd_strided(q.data_ptr(), k.data_ptr(), v.data_ptr(), 3 * K + 4, 3 * K + 4, 3 * K + 4,
+                                   g.data_ptr(), beta.data_ptr(), None, None, o.data_ptr(), None,
+                                   ws.data_ptr() + (-ws.data_ptr()) % 256, ws.numel() - 256, B, T, B, H, H, K, K, 0.125, 0,
+                                   1, lib.stream())
+    assert rc == -6
+
+
+@pytest.mark.parametrize("dtype,shape,Hv,pdt", [
+    (F32, (2, 37), 6, None), (BF, (1, 300), 32, None), (BF, (3, 5), 48, torch.float32), (F32, (1,), 256, None),
+    (BF, (2, 8192), 32, None), (BF, (1, 65536), 64, torch.float32),
+])
+def test_gdn_gates(ops, dtype, shape, Hv, pdt):
+    P.check_gdn_gates(ops, "cuda", shape, Hv, dtype, param_dtype=pdt)
+
+
+def test_gdn_gates_feed_the_rule(ops):
+    """The layer's chain: projections -> gates -> rule, gradients back to the projections and the parameters."""
+    B, T, Hqk, Hv, K, V = 1, 128, 2, 4, 64, 64
+    gen = torch.Generator().manual_seed(1)
+    r = lambda *s: torch.randn(*s, generator=gen)
+    a, b = r(B, T, Hv).to(BF), r(B, T, Hv).to(BF)
+    A_log, dt_bias = torch.empty(Hv).uniform_(0, 2.7, generator=gen), torch.empty(Hv).uniform_(-4, -2, generator=gen)
+    mixed = r(B, T, 2 * Hqk * K + Hv * V).to(BF)
+    do = r(B, T, Hv, V).to(BF)
+    L = [t.cuda().requires_grad_(True) for t in (mixed, a, b, A_log, dt_bias)]
+    g, beta = ops.gdn_gates(L[1], L[2], L[3], L[4])
+    o, _ = ops.chunk_gated_delta_rule_qkv(L[0], g, beta, Hqk, Hv, K, V, use_qk_l2norm_in_kernel=True)
+    o.backward(do.cuda())
+    R = [t.float().requires_grad_(True) for t in (mixed, a, b, A_log, dt_bias)]
+    rg, rbeta = O.gdn_gates_ref(R[1], R[2], R[3], R[4])
+    q, k, v = torch.split(R[0], [Hqk * K, Hqk * K, Hv * V], dim=-1)
+    ro, _ = O.chunk_gated_delta_rule_ref(q.reshape(B, T, Hqk, K), k.reshape(B, T, Hqk, K), v.reshape(B, T, Hv, V), rg,
+                                         rbeta.to(BF).float(), use_qk_l2norm_in_kernel=True)
+    ro.backward(do.float())
+    P._err("o", o, ro, BF, P.BF16_ABS_O)
+    for name, l, rr in zip(("d_mixed", "da", "db"), L[:3], R[:3]):
+        P._err(name, l.grad, rr.grad, BF, P.BF16_ABS_GRAD)
+    for name, l, rr in zip(("dA_log", "ddt_bias"), L[3:], R[3:]):
+        P._err(name, l.grad, rr.grad, BF, 2e-2 * max(rr.grad.abs().max().item(), 1.0), rtol=2e-2)
