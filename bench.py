@@ -200,6 +200,43 @@ def main():
         aux["decode_b256"] = {"kernel_us": round(kern_s * 1e6, 1), "GBps": round(step_bytes / kern_s / 1e9, 1),
                               "frac_of_hbm_peak": round(step_bytes / kern_s / 1e9 / PEAK_HBM_GBS, 4),
                               "tokens_per_s_wall": round(B3 / wall, 1), "bytes_per_step": step_bytes}
+        # ---- one decode step of the layer between the projections and the gated norm, batch 256: convolution update +
+        # rule on its unsplit output with in-kernel gates (2 launches) against the same from separate operators ----
+        nq3, nv3 = c["Hqk"] * c["K"], c["Hv"] * c["V"]
+        D3 = 2 * nq3 + nv3
+        g3 = torch.Generator().manual_seed(4)
+        mx3 = torch.randn(B3, 1, D3, generator=g3).to(dev, torch.bfloat16)
+        a3 = torch.randn(B3, 1, c["Hv"], generator=g3).to(dev, torch.bfloat16)
+        b3 = torch.randn(B3, 1, c["Hv"], generator=g3).to(dev, torch.bfloat16)
+        cw3 = (torch.randn(D3, 4, generator=g3) / 2).to(dev, torch.bfloat16)
+        cb3 = torch.zeros(D3, device=dev, dtype=torch.bfloat16)
+        Al3, db3 = torch.zeros(c["Hv"], device=dev), torch.full((c["Hv"],), -3.0, device=dev)
+        conv3 = torch.zeros(B3, D3, 4, device=dev, dtype=torch.bfloat16)
+
+        def layer_step_fused():
+            ops.decode_step(mx3, a3, b3, conv3, state, cw3, cb3, Al3, db3, c["Hqk"], c["Hv"], c["K"], c["V"])
+
+        def layer_step_separate():
+            y_ = ops.causal_conv1d_update(mx3, conv3, cw3, cb3, "silu")
+            q_, k_, v_ = torch.split(y_, [nq3, nq3, nv3], dim=-1)
+            g_, be_ = ops.gdn_gates(a3, b3, Al3, db3)
+            ops.fused_recurrent_gated_delta_rule(q_.reshape(B3, 1, c["Hqk"], c["K"]), k_.reshape(B3, 1, c["Hqk"], c["K"]),
+                                                 v_.reshape(B3, 1, c["Hv"], c["V"]), g_, be_, initial_state=state,
+                                                 output_final_state=True, use_qk_l2norm_in_kernel=True,
+                                                 inplace_state=True)
+
+        def wall_us(fn, n=64):
+            for _ in range(8):
+                fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n):
+                fn()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / n * 1e6
+        aux["decode_layer_step_b256"] = {"conv_update_plus_rule_us": round(wall_us(layer_step_fused), 1),
+                                         "separate_operators_us": round(wall_us(layer_step_separate), 1)}
+        del mx3, conv3
         del e, y, state, tok
         # ---- packed causal conv1d fwd+bwd (BASELINE.json configs[2]: 32768 tokens, D=8192, W=4, SiLU) ----
         cu = torch.tensor(packed_lengths(), dtype=torch.int64, device=dev)

@@ -75,6 +75,16 @@ int gdn_recurrent_fwd(const void* q, const void* k, const void* v, const float* 
                       const float* state_in, float* state_out, void* o, int B, int T, int Hqk, int Hv, int K,
                       int V, float scale, int use_qk_l2norm, int dtype, void* stream);
 
+/* The same step reading q, k, v in place from the [tokens, D] output of the convolution (column ranges [0, Hqk K),
+ * [Hqk K, 2 Hqk K), [2 Hqk K, 2 Hqk K + Hv V); token_stride >= that width, in elements, a multiple of 16 bytes) and
+ * forming the gates from the layer's projections a, b [tokens, Hv] and parameters A_log, dt_bias [Hv] (in `dtype`
+ * when param_dtype = dtype, fp32 when param_dtype = 0) as modeling_qwen3_5.py:833-841 does: the decode branch of
+ * Qwen3_5GatedDeltaNet.forward (:738-744, :808-848, :877-886) is gdn_conv1d_update followed by this call. */
+int gdn_recurrent_fwd_qkv(const void* qkv, int64_t token_stride, const void* a, const void* b, const void* A_log,
+                          const void* dt_bias, const float* state_in, float* state_out, void* o, int B, int T,
+                          int Hqk, int Hv, int K, int V, float scale, int use_qk_l2norm, int dtype, int param_dtype,
+                          void* stream);
+
 /* -------- causal short depthwise conv1d --------------------------------------------------------
  * replaces causal_conv1d_fwd_impl / causal_conv1d_bwd_impl / causal_conv1d_update_states,
  * mindspeed_mm/fsdp/ops/gdn/triton/convolution.py:517-588, 591-714, 762-787.

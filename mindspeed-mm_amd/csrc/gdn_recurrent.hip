@@ -8,15 +8,29 @@
 //     S^T k = e^g (S_old^T k),   S^T q = e^g (S_old^T q) + (k.q) delta
 // so both contractions are taken in ONE pass over the registers, then the rank-1 update is applied.
 // No MFMA: 6 flop per 8 bytes of state traffic, far below the matrix-core ridge.
+//
+// q, k, v are read with a token stride, so they can be the column ranges of the convolution's [tokens, D] output, and
+// the gates can be formed here from the layer's projections (g = -exp(A_log) softplus(a + dt_bias), beta = sigmoid(b)
+// rounded to b's dtype as the layer's `b.sigmoid()` is; modeling_qwen3_5.py:833-841) instead of being passed in: a
+// decode step of the layer is then the convolution update followed by this kernel, with no copies in between.
 #include "gdn_common.h"
 #include "gdn_profile.h"
 
 namespace gdn {
 
-template <typename T, int DK, int BV>
+struct RecurrentGates {   // either g, beta (fp32 [tokens,Hv]) or the projections a, b [tokens,Hv] and A_log, dt_bias [Hv]
+  const float* g;
+  const float* beta;
+  const void* a;
+  const void* b;
+  const void* A_log;
+  const void* dt_bias;
+};
+
+template <typename T, typename TP, int DK, int BV>
 __global__ __launch_bounds__(256) void recurrent_kernel(
-    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ g,
-    const float* __restrict__ beta, const float* state_in, float* state_out, T* __restrict__ o, int B, int T_len,
+    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, int64_t sq, int64_t sk, int64_t sv,
+    RecurrentGates gates, const float* state_in, float* state_out, T* __restrict__ o, int B, int T_len,
     int Hqk, int Hv, int V, float scale, int use_l2norm) {
   constexpr int CG = BV / 4;            // column groups (4 fp32 = 16 bytes each)
   constexpr int NRG = kThreads / CG;    // row groups
@@ -48,8 +62,8 @@ __global__ __launch_bounds__(256) void recurrent_kernel(
     // ---- q, k of this token: optional l2 norm, q pre-scaled ----
     float kv_ = 0.f, qv_ = 0.f;
     if (tid < DK) {
-      kv_ = Elem<T>::to_f(k[(tok * Hqk + hq) * DK + tid]);
-      qv_ = Elem<T>::to_f(q[(tok * Hqk + hq) * DK + tid]);
+      kv_ = Elem<T>::to_f(k[tok * sk + hq * DK + tid]);
+      qv_ = Elem<T>::to_f(q[tok * sq + hq * DK + tid]);
     }
     const float sk = wave_sum(kv_ * kv_), sq = wave_sum(qv_ * qv_), skq = wave_sum(kv_ * qv_);
     if (lane == 0) { red3[wave][0] = sk; red3[wave][1] = sq; red3[wave][2] = skq; }
@@ -82,13 +96,24 @@ __global__ __launch_bounds__(256) void recurrent_kernel(
     }
     __syncthreads();
 
-    const float eg = __expf(g[tok * Hv + h]), bt = beta[tok * Hv + h];
+    float eg, bt;
+    if (gates.a == nullptr) {
+      eg = __expf(gates.g[tok * Hv + h]);
+      bt = gates.beta[tok * Hv + h];
+    } else {
+      const float x = Elem<T>::to_f(static_cast<const T*>(gates.a)[tok * Hv + h]) +
+                      Elem<TP>::to_f(static_cast<const TP*>(gates.dt_bias)[h]);
+      const float sp = x > 20.f ? x : log1pf(expf(x));
+      eg = __expf(-expf(Elem<TP>::to_f(static_cast<const TP*>(gates.A_log)[h])) * sp);   // as __expf(g) of a passed-in g
+      const float sg = 1.f / (1.f + expf(-Elem<T>::to_f(static_cast<const T*>(gates.b)[tok * Hv + h])));
+      bt = Elem<T>::to_f(Elem<T>::from_f(sg));
+    }
     float delta[4], ov[4];
     Vec16<T> vv;
     if constexpr (sizeof(T) == 4) {
-      vv = ld16(v + (tok * Hv + h) * V + v0);
+      vv = ld16(v + tok * sv + h * V + v0);
     } else {
-      const u32x2 w = *reinterpret_cast<const u32x2*>(v + (tok * Hv + h) * V + v0);
+      const u32x2 w = *reinterpret_cast<const u32x2*>(v + tok * sv + h * V + v0);
       vv.raw = u32x4{w[0], w[1], 0u, 0u};
     }
 #pragma unroll
@@ -132,14 +157,14 @@ __global__ __launch_bounds__(256) void recurrent_kernel(
   (void)RGW; (void)B;
 }
 
-template <typename T>
-static int launch_recurrent(const void* q, const void* k, const void* v, const float* g, const float* beta,
-                            const float* state_in, float* state_out, void* o, int B, int T_len, int Hqk, int Hv, int K,
-                            int V, float scale, int use_l2norm, hipStream_t stream) {
-#define GDN_REC(DK_, BV_)                                                                                      \
-  GDN_LAUNCH(kKernRecurrent, stream, (recurrent_kernel<T, DK_, BV_>), dim3(B * Hv, V / BV_), dim3(kThreads), 0, \
-                     stream, (const T*)q, (const T*)k, (const T*)v, g, beta, state_in, state_out, (T*)o, B,    \
-                     T_len, Hqk, Hv, V, scale, use_l2norm)
+template <typename T, typename TP>
+static int launch_recurrent(const void* q, const void* k, const void* v, int64_t sq, int64_t sk, int64_t sv,
+                            const RecurrentGates& gates, const float* state_in, float* state_out, void* o, int B,
+                            int T_len, int Hqk, int Hv, int K, int V, float scale, int use_l2norm, hipStream_t stream) {
+#define GDN_REC(DK_, BV_)                                                                                          \
+  GDN_LAUNCH(kKernRecurrent, stream, (recurrent_kernel<T, TP, DK_, BV_>), dim3(B * Hv, V / BV_), dim3(kThreads), 0, \
+             stream, (const T*)q, (const T*)k, (const T*)v, sq, sk, sv, gates, state_in, state_out, (T*)o, B, T_len,  \
+             Hqk, Hv, V, scale, use_l2norm)
   const bool wide = (V % 128 == 0);
   if (K == 64 && wide) GDN_REC(64, 128);
   else if (K == 64) GDN_REC(64, 64);
@@ -152,17 +177,55 @@ static int launch_recurrent(const void* q, const void* k, const void* v, const f
   return (int)hipGetLastError();
 }
 
+static int recurrent_check(int B, int T, int Hqk, int Hv, int V) {
+  if (B <= 0 || T < 0 || Hqk <= 0 || Hv <= 0 || Hv % Hqk != 0) return -2;
+  if (V % 64 != 0 || V <= 0) return -3;
+  return 0;
+}
+
 }  // namespace gdn
 
 extern "C" int gdn_recurrent_fwd(const void* q, const void* k, const void* v, const float* g, const float* beta,
                                  const float* state_in, float* state_out, void* o, int B, int T, int Hqk, int Hv,
                                  int K, int V, float scale, int use_qk_l2norm, int dtype, void* stream) {
+  using namespace gdn;
   if (!q || !k || !v || !g || !beta || !o) return -1;
-  if (B <= 0 || T < 0 || Hqk <= 0 || Hv <= 0 || Hv % Hqk != 0) return -2;
-  if (V % 64 != 0 || V <= 0) return -3;
+  if (int e = recurrent_check(B, T, Hqk, Hv, V)) return e;
   if (T == 0 && state_out == nullptr) return 0;
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == 0) return gdn::launch_recurrent<float>(q, k, v, g, beta, state_in, state_out, o, B, T, Hqk, Hv, K, V, scale, use_qk_l2norm, s);
-  if (dtype == 1) return gdn::launch_recurrent<gdn::bf16_t>(q, k, v, g, beta, state_in, state_out, o, B, T, Hqk, Hv, K, V, scale, use_qk_l2norm, s);
+  const RecurrentGates gates{g, beta, nullptr, nullptr, nullptr, nullptr};
+  const int64_t nq = (int64_t)Hqk * K, nv = (int64_t)Hv * V;
+  if (dtype == 0)
+    return launch_recurrent<float, float>(q, k, v, nq, nq, nv, gates, state_in, state_out, o, B, T, Hqk, Hv, K, V, scale,
+                                          use_qk_l2norm, s);
+  if (dtype == 1)
+    return launch_recurrent<bf16_t, float>(q, k, v, nq, nq, nv, gates, state_in, state_out, o, B, T, Hqk, Hv, K, V, scale,
+                                           use_qk_l2norm, s);
   return -4;
+}
+
+extern "C" int gdn_recurrent_fwd_qkv(const void* qkv, int64_t token_stride, const void* a, const void* b,
+                                     const void* A_log, const void* dt_bias, const float* state_in, float* state_out,
+                                     void* o, int B, int T, int Hqk, int Hv, int K, int V, float scale,
+                                     int use_qk_l2norm, int dtype, int param_dtype, void* stream) {
+  using namespace gdn;
+  if (!qkv || !a || !b || !A_log || !dt_bias || !o) return -1;
+  if (int e = recurrent_check(B, T, Hqk, Hv, V)) return e;
+  if (dtype != 0 && dtype != 1) return -4;
+  if (param_dtype != 0 && param_dtype != dtype) return -4;
+  const int64_t nq = (int64_t)Hqk * K, nv = (int64_t)Hv * V, vec = dtype == 0 ? 4 : 8, es = dtype == 0 ? 4 : 2;
+  if (token_stride < 2 * nq + nv || token_stride % vec != 0 || ((uintptr_t)qkv & 15) != 0) return -6;
+  if (T == 0 && state_out == nullptr) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const RecurrentGates gates{nullptr, nullptr, a, b, A_log, dt_bias};
+  const char* base = static_cast<const char*>(qkv);
+  const void *q = base, *k = base + nq * es, *v = base + 2 * nq * es;
+  if (dtype == 0)
+    return launch_recurrent<float, float>(q, k, v, token_stride, token_stride, token_stride, gates, state_in, state_out,
+                                          o, B, T, Hqk, Hv, K, V, scale, use_qk_l2norm, s);
+  if (param_dtype == 1)
+    return launch_recurrent<bf16_t, bf16_t>(q, k, v, token_stride, token_stride, token_stride, gates, state_in,
+                                            state_out, o, B, T, Hqk, Hv, K, V, scale, use_qk_l2norm, s);
+  return launch_recurrent<bf16_t, float>(q, k, v, token_stride, token_stride, token_stride, gates, state_in, state_out,
+                                         o, B, T, Hqk, Hv, K, V, scale, use_qk_l2norm, s);
 }

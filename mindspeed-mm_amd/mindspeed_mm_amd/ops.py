@@ -8,6 +8,9 @@
     rms_norm_gated / RMSNormGated     Qwen3_5RMSNormGated, modeling_qwen3_5.py:330-349, called at :897-900
     gdn_gates                         g / beta recipe of the layer, modeling_qwen3_5.py:833-841
     chunk_gated_delta_rule_qkv        the rule on the unsplit convolution output (split at :818-831)
+    fused_recurrent_gated_delta_rule_qkv / decode_step / GdnDecodeCache
+                                      the layer's decode branch (:738-744, :808-848, :877-890) and the
+                                      linear-attention part of Qwen3_5DynamicCache (:134-221)
 
 Everything here is host glue: validation, output/workspace allocation with torch, and one call into the
 C ABI per operator.  The kernels themselves are the HIP library; nothing in this file computes.
@@ -162,6 +165,65 @@ class GdnOps:
                                           int(use_qk_l2norm_in_kernel), DTYPE_CODE[q.dtype], self.lib.stream())
         self.lib.check(code, "gdn_recurrent_fwd")
         return o, (s_out if output_final_state else None)
+
+    def fused_recurrent_gated_delta_rule_qkv(self, mixed_qkv, a, b, A_log, dt_bias, num_k_heads, num_v_heads,
+                                             head_k_dim, head_v_dim, scale=None, initial_state=None,
+                                             output_final_state=False, use_qk_l2norm_in_kernel=False,
+                                             inplace_state=False):
+        """fused_recurrent_gated_delta_rule on the convolution's unsplit output [B,T,D] with the gates formed in the
+        kernel from the projections a, b [B,T,Hv] and the parameters A_log, dt_bias [Hv]: equal to the layer's chain
+        split -> sigmoid / softplus recipe -> rule (modeling_qwen3_5.py:808-848, 877-886) without its copies."""
+        Hqk, Hv, K, V = int(num_k_heads), int(num_v_heads), int(head_k_dim), int(head_v_dim)
+        if mixed_qkv.dim() != 3 or mixed_qkv.shape[-1] < 2 * Hqk * K + Hv * V:
+            raise ValueError("expected mixed_qkv [B, T, D] with D >= 2 * num_k_heads * head_k_dim + num_v_heads * head_v_dim")
+        B, T, D = mixed_qkv.shape
+        dt = mixed_qkv.dtype
+        if dt not in (torch.float32, torch.bfloat16) or a.dtype != dt or b.dtype != dt:
+            raise ValueError("mixed_qkv, a, b must share a dtype, bfloat16 or float32")
+        if tuple(a.shape) != (B, T, Hv) or a.shape != b.shape or A_log.shape != (Hv,) or dt_bias.shape != (Hv,):
+            raise ValueError("expected a, b [B, T, Hv] and A_log, dt_bias [Hv]")
+        self._need(mixed_qkv, a, b, A_log, dt_bias, initial_state)
+        if scale is None:
+            scale = K ** -0.5
+        vec = 16 // mixed_qkv.element_size()
+        x = mixed_qkv if (mixed_qkv.is_contiguous() and D % vec == 0 and mixed_qkv.data_ptr() % 16 == 0) \
+            else mixed_qkv.contiguous()
+        if D % vec != 0:
+            raise ValueError(f"the width of mixed_qkv must be a multiple of {vec} elements")
+        pdt = dt if (A_log.dtype == dt and dt_bias.dtype == dt) else torch.float32
+        Ac, dc = A_log.detach().to(pdt).contiguous(), dt_bias.detach().to(pdt).contiguous()
+        ac, bc = a.contiguous(), b.contiguous()
+        o = torch.empty(B, T, Hv, V, dtype=dt, device=x.device)
+        s_in = None
+        if initial_state is not None:
+            if inplace_state:
+                if initial_state.dtype != torch.float32 or not initial_state.is_contiguous():
+                    raise ValueError("inplace_state needs a contiguous float32 state")
+                s_in = initial_state
+            else:
+                s_in = self._f32(initial_state)
+        s_out = None
+        if output_final_state or inplace_state:
+            s_out = s_in if (inplace_state and s_in is not None) else \
+                torch.empty(B, Hv, K, V, dtype=torch.float32, device=x.device)
+        code = self.lib.gdn_recurrent_fwd_qkv(ptr(x), D, ptr(ac), ptr(bc), ptr(Ac), ptr(dc), ptr(s_in), ptr(s_out),
+                                              ptr(o), B, T, Hqk, Hv, K, V, float(scale),
+                                              int(use_qk_l2norm_in_kernel), DTYPE_CODE[dt], DTYPE_CODE[pdt],
+                                              self.lib.stream())
+        self.lib.check(code, "gdn_recurrent_fwd_qkv")
+        return o, (s_out if output_final_state else None)
+
+    def decode_step(self, mixed_qkv, a, b, conv_state, recurrent_state, conv_weight, conv_bias, A_log, dt_bias,
+                    num_k_heads, num_v_heads, head_k_dim, head_v_dim, activation="silu"):
+        """The decode branch of Qwen3_5GatedDeltaNet.forward between the input projections and the gated norm
+        (modeling_qwen3_5.py:738-744, 808-848, 877-890) in two launches: convolution update (conv_state [B,D,S] rolled
+        in place), then the rule on its unsplit output with the gates formed in the kernel (recurrent_state
+        [B,Hv,K,V] fp32 updated in place).  mixed_qkv [B,T,D], a, b [B,T,Hv]; conv_weight [D,W].  Returns o [B,T,Hv,V]."""
+        y = self.causal_conv1d_update(mixed_qkv, conv_state, conv_weight, conv_bias, activation)
+        o, _ = self.fused_recurrent_gated_delta_rule_qkv(y, a, b, A_log, dt_bias, num_k_heads, num_v_heads, head_k_dim,
+                                                         head_v_dim, initial_state=recurrent_state,
+                                                         use_qk_l2norm_in_kernel=True, inplace_state=True)
+        return o
 
     # ------------------------------------------------------------------ conv1d
     def causal_conv1d(self, x, weight, bias=None, residual=None, initial_state=None, activation=None,
@@ -518,6 +580,50 @@ def fused_recurrent_gated_delta_rule(q, k, v, g, beta=None, scale=None, initial_
 
 
 @torch.compiler.disable
+def fused_recurrent_gated_delta_rule_qkv(mixed_qkv, a, b, A_log, dt_bias, num_k_heads, num_v_heads, head_k_dim,
+                                         head_v_dim, scale=None, initial_state=None, output_final_state=False,
+                                         use_qk_l2norm_in_kernel=False, inplace_state=False):
+    return _default_ops().fused_recurrent_gated_delta_rule_qkv(
+        mixed_qkv, a, b, A_log, dt_bias, num_k_heads, num_v_heads, head_k_dim, head_v_dim, scale, initial_state,
+        output_final_state, use_qk_l2norm_in_kernel, inplace_state)
+
+
+def decode_step(mixed_qkv, a, b, conv_state, recurrent_state, conv_weight, conv_bias, A_log, dt_bias, num_k_heads,
+                num_v_heads, head_k_dim, head_v_dim, activation="silu"):
+    return _default_ops().decode_step(mixed_qkv, a, b, conv_state, recurrent_state, conv_weight, conv_bias, A_log,
+                                      dt_bias, num_k_heads, num_v_heads, head_k_dim, head_v_dim, activation)
+
+
+class GdnDecodeCache:
+    """The linear-attention half of Qwen3_5DynamicCache (modeling_qwen3_5.py:134-221): per layer a convolution state
+    [B, D, W] and a recurrent state [B, Hv, K, V], created by the prefill, updated in place by decode_step, reordered
+    along the batch for beam search.  Host-side bookkeeping only."""
+
+    def __init__(self, num_layers):
+        self.conv_states = [None] * num_layers
+        self.recurrent_states = [None] * num_layers
+
+    def __len__(self):
+        return len(self.conv_states)
+
+    def set_prefill(self, layer_idx, conv_final_state, recurrent_final_state):
+        """conv_final_state: the final_state causal_conv1d returns with output_final_state=True, which is the layer's
+        zero-left-padded last W inputs (modeling_qwen3_5.py:746-750); recurrent_final_state: the rule's final_state."""
+        self.conv_states[layer_idx] = conv_final_state.contiguous()
+        self.recurrent_states[layer_idx] = recurrent_final_state.to(torch.float32).contiguous()
+
+    def has_previous_state(self, layer_idx):
+        return self.conv_states[layer_idx] is not None
+
+    def reorder_cache(self, beam_idx):
+        """index_select along the batch of every state (modeling_qwen3_5.py:183-196)."""
+        for i, c in enumerate(self.conv_states):
+            if c is not None:
+                idx = beam_idx.to(c.device)
+                self.conv_states[i] = c.index_select(0, idx)
+                self.recurrent_states[i] = self.recurrent_states[i].index_select(0, idx)
+
+
 def causal_conv1d(x, weight, bias=None, residual=None, initial_state=None, activation=None, cu_seqlens=None,
                   output_final_state=False):
     return _default_ops().causal_conv1d(x, weight, bias, residual, initial_state, activation, cu_seqlens,

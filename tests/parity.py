@@ -218,3 +218,48 @@ def check_gdn_gates(ops, device, shape, Hv, dtype, param_dtype=None, seed=0, bac
             scale = max(R[n].grad.abs().max().item(), 1.0)
             errs[m] = _err(m, L[n].grad, R[n].grad, param_dtype, 1e-2 * scale, rtol=1e-2)
     return errs
+
+
+def check_decode_step(ops, device, B, steps, Hqk, Hv, K, V, W, dtype, param_dtype=None, seed=0, wrap=lambda t: t):
+    """`steps` consecutive decode tokens through decode_step (convolution update + rule on its unsplit output with the
+    gates formed in the kernel, both states in place) against the oracle's chain conv update -> split -> gate recipe
+    -> recurrent rule, and bit for bit against this package's own unfused operators."""
+    gen = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=gen)
+    param_dtype = param_dtype or dtype
+    nq, nv = Hqk * K, Hv * V
+    D = 2 * nq + nv
+    x = dict(mixed=r(B, steps, D).to(dtype), a=r(B, steps, Hv).to(dtype), b=r(B, steps, Hv).to(dtype),
+             cw=(r(D, W) / 2).to(dtype), cb=(r(D) / 4).to(dtype),
+             A=torch.empty(Hv).uniform_(0.0, 2.77, generator=gen).to(param_dtype),
+             d=torch.empty(Hv).uniform_(-4.0, -2.0, generator=gen).to(param_dtype),
+             conv=r(B, D, W).to(dtype), S=0.1 * r(B, Hv, K, V))
+    dev = {n: wrap(t.to(device)) for n, t in x.items()}
+    conv1, S1 = dev["conv"].clone(), dev["S"].clone()
+    conv2, S2 = dev["conv"].clone(), dev["S"].clone()
+    rconv, rS = x["conv"].float().clone(), x["S"].clone()
+    errs = {}
+    for t in range(steps):
+        sl = slice(t, t + 1)
+        o = ops.decode_step(dev["mixed"][:, sl], dev["a"][:, sl], dev["b"][:, sl], conv1, S1, dev["cw"], dev["cb"],
+                            dev["A"], dev["d"], Hqk, Hv, K, V)
+        # the same with this package's separate operators
+        y2 = ops.causal_conv1d_update(dev["mixed"][:, sl], conv2, dev["cw"], dev["cb"], "silu")
+        q2, k2, v2 = torch.split(y2, [nq, nq, nv], dim=-1)
+        g2, beta2 = ops.gdn_gates(dev["a"][:, sl], dev["b"][:, sl], dev["A"], dev["d"])
+        o2, _ = ops.fused_recurrent_gated_delta_rule(
+            q2.reshape(B, 1, Hqk, K), k2.reshape(B, 1, Hqk, K), v2.reshape(B, 1, Hv, V), g2, beta2, initial_state=S2,
+            output_final_state=True, use_qk_l2norm_in_kernel=True, inplace_state=True)
+        assert torch.equal(o, o2), f"step {t}: fused decode step differs from the separate operators"
+        # oracle chain, with the layer's dtype flow (the convolution's output is in the activations' dtype)
+        ry = O.causal_conv1d_update_ref(x["mixed"][:, sl].float(), rconv, x["cw"].float(), x["cb"].float(), "silu")
+        ry = ry.to(dtype).float()
+        rq, rk, rv = torch.split(ry, [nq, nq, nv], dim=-1)
+        rg, rbeta = O.gdn_gates_ref(x["a"][:, sl], x["b"][:, sl], x["A"], x["d"])
+        ro, rS = O.recurrent_gated_delta_rule_ref(rq.reshape(B, 1, Hqk, K), rk.reshape(B, 1, Hqk, K),
+                                                  rv.reshape(B, 1, Hv, V), rg, rbeta.float(), rS, True, True)
+        errs["o"] = max(errs.get("o", 0.0), _err(f"o[{t}]", o, ro, dtype, BF16_ABS_O))
+    assert torch.equal(conv1, conv2) and torch.equal(S1, S2)
+    errs["conv_state"] = _err("conv_state", conv1, rconv, dtype, 1e-2, 1e-2)
+    errs["state"] = _err("recurrent_state", S1, rS, dtype, BF16_ABS_GRAD)
+    return errs

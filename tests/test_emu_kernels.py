@@ -89,3 +89,10 @@ def test_chunk_on_unsplit_qkv(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu, pad):
 ])
 def test_gdn_gates(ops, dtype, shape, Hv, pdt):
     P.check_gdn_gates(ops, "cpu", shape, Hv, dtype, param_dtype=pdt, wrap=guarded)
+
+
+@pytest.mark.parametrize("dtype,B,steps,Hqk,Hv,K,V,W,pdt", [
+    (F32, 2, 3, 1, 2, 64, 64, 4, None), (BF, 2, 4, 2, 4, 128, 128, 4, None), (BF, 1, 2, 1, 2, 64, 128, 3, torch.float32),
+])
+def test_decode_step(ops, dtype, B, steps, Hqk, Hv, K, V, W, pdt):
+    P.check_decode_step(ops, "cpu", B, steps, Hqk, Hv, K, V, W, dtype, param_dtype=pdt, wrap=guarded)

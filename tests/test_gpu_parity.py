@@ -176,3 +176,56 @@ def test_gdn_gates_feed_the_rule(ops):
         P._err(name, l.grad, rr.grad, BF, P.BF16_ABS_GRAD)
     for name, l, rr in zip(("dA_log", "ddt_bias"), L[3:], R[3:]):
         P._err(name, l.grad, rr.grad, BF, 2e-2 * max(rr.grad.abs().max().item(), 1.0), rtol=2e-2)
+
+
+@pytest.mark.parametrize("dtype,B,steps,Hqk,Hv,K,V,W,pdt", [
+    (F32, 2, 3, 1, 2, 64, 64, 4, None), (BF, 2, 4, 2, 4, 128, 128, 4, None), (BF, 1, 2, 1, 2, 64, 128, 3, torch.float32),
+    (BF, 16, 8, 16, 32, 128, 128, 4, None),
+])
+def test_decode_step(ops, dtype, B, steps, Hqk, Hv, K, V, W, pdt):
+    print(f"decode step {dtype} B{B} steps{steps} Hqk{Hqk} Hv{Hv} K{K} V{V} W{W}", flush=True)
+    P.check_decode_step(ops, "cuda", B, steps, Hqk, Hv, K, V, W, dtype, param_dtype=pdt)
+
+
+def test_decode_cache_prefill_then_steps(ops):
+    """Prefill with the chunked operators, hand both states to the cache, decode two more tokens, reorder the beams:
+    equal to running the chunked operators over the longer sequences of the reordered batch."""
+    from mindspeed_mm_amd import GdnDecodeCache
+    B, T, Hqk, Hv, K, V, W = 3, 70, 2, 4, 64, 64, 4
+    nq, nv = Hqk * K, Hv * V
+    D = 2 * nq + nv
+    gen = torch.Generator().manual_seed(5)
+    r = lambda *s: torch.randn(*s, generator=gen)
+    xin = r(B, T + 2, D).to(BF).cuda()
+    a, b = r(B, T + 2, Hv).to(BF).cuda(), r(B, T + 2, Hv).to(BF).cuda()
+    cw, cb = (r(D, W) / 2).to(BF).cuda(), (r(D) / 4).to(BF).cuda()
+    A_log, dt_bias = torch.empty(Hv).uniform_(0, 2.7, generator=gen).cuda(), torch.empty(Hv).uniform_(-4, -2, generator=gen).cuda()
+
+    def layer(x, aa, bb):   # chunked path over whole sequences
+        y, conv_fs = ops.causal_conv1d(x, cw.t().contiguous(), cb, activation="silu", output_final_state=True)
+        g, beta = ops.gdn_gates(aa, bb, A_log, dt_bias)
+        o, S = ops.chunk_gated_delta_rule_qkv(y, g, beta, Hqk, Hv, K, V, output_final_state=True,
+                                              use_qk_l2norm_in_kernel=True)
+        return o, conv_fs, S
+    cache = GdnDecodeCache(1)
+    assert not cache.has_previous_state(0)
+    _, conv_fs, S = layer(xin[:, :T], a[:, :T], b[:, :T])
+    cache.set_prefill(0, conv_fs, S)
+    assert cache.has_previous_state(0) and cache.conv_states[0].shape == (B, D, W)
+    o1 = ops.decode_step(xin[:, T:T + 1], a[:, T:T + 1], b[:, T:T + 1], cache.conv_states[0], cache.recurrent_states[0],
+                         cw, cb, A_log, dt_bias, Hqk, Hv, K, V)
+    beam = torch.tensor([2, 0, 0], device="cuda")
+    cache.reorder_cache(beam)
+    x2 = xin[:, T + 1:T + 2]
+    o2 = ops.decode_step(x2, a[:, T + 1:T + 2], b[:, T + 1:T + 2], cache.conv_states[0], cache.recurrent_states[0], cw, cb,
+                         A_log, dt_bias, Hqk, Hv, K, V)
+    # whole-sequence run of the reordered batch: history of beam[i], last token of row i
+    xfull = torch.cat([xin[beam][:, :T + 1], x2], dim=1)
+    afull = torch.cat([a[beam][:, :T + 1], a[:, T + 1:T + 2]], dim=1)
+    bfull = torch.cat([b[beam][:, :T + 1], b[:, T + 1:T + 2]], dim=1)
+    ofull, conv_full, Sfull = layer(xfull, afull, bfull)
+    ofull1, _, _ = layer(xin[:, :T + 1], a[:, :T + 1], b[:, :T + 1])
+    P._err("decode token 1", o1, ofull1[:, T:T + 1], BF, P.BF16_ABS_O)
+    P._err("decode token 2 after reorder", o2, ofull[:, T + 1:T + 2], BF, P.BF16_ABS_O)
+    P._err("recurrent state", cache.recurrent_states[0], Sfull, BF, P.BF16_ABS_GRAD)
+    assert torch.equal(cache.conv_states[0], conv_full)
