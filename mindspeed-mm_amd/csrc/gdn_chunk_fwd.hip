@@ -15,12 +15,6 @@
 #include "gdn_common.h"
 #include "gdn_profile.h"
 
-#ifndef GDN_PREP_WPS
-#define GDN_PREP_WPS 3
-#endif
-#ifndef GDN_OUT_WPS
-#define GDN_OUT_WPS 2
-#endif
 namespace gdn {
 
 constexpr int kLF = 68;  // leading dimension of the fp32 64x64 solve buffers
@@ -107,7 +101,7 @@ template <typename T, int DK, int BV> struct PrepSmem {
 };
 
 template <typename T, int DK, int BV>
-__global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(GDN_PREP_WPS) void chunk_prep_kernel(
+__global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(3) void chunk_prep_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ g,
     const float* __restrict__ beta, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets,
     float* __restrict__ G_out, T* __restrict__ Ai_out, T* __restrict__ W_out, T* __restrict__ U_out,
@@ -599,7 +593,7 @@ template <typename T, int DK, int NW> struct OutSmem {
 };
 
 template <typename T, int DK, int NW>
-__global__ __launch_bounds__(64 * NW) GDN_WAVES_PER_SIMD(GDN_OUT_WPS) void chunk_out_kernel(
+__global__ __launch_bounds__(64 * NW) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 2) void chunk_out_kernel(
     const T* __restrict__ q, const T* __restrict__ aqf, const T* __restrict__ vf, const T* __restrict__ hf,
     const float* __restrict__ G, T* __restrict__ o, const int64_t* __restrict__ cu,
     const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V, float scale, int64_t q_stride) {

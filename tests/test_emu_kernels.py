@@ -48,6 +48,12 @@ def test_chunk_backward(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu):
     P.check_chunk(ops, "cpu", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu, backward=True, wrap=guarded, h0_std=0.1)
 
 
+@pytest.mark.parametrize("cu", [[0, 0, 70], [0, 70, 70], [0, 30, 30, 100], [0, 0, 0, 64]])
+def test_chunk_packed_with_empty_sequences(ops, cu):
+    """A sequence of length 0 has no chunk: its final state is its initial state, its gradients are empty."""
+    P.check_chunk(ops, "cpu", 1, cu[-1], 1, 2, 64, 64, F32, cu=cu, backward=True, wrap=guarded, h0_std=0.1)
+
+
 def test_chunk_backward_without_initial_state(ops):
     P.check_chunk(ops, "cpu", 1, 70, 1, 1, 64, 64, F32, backward=True, with_h0=False, wrap=guarded)
 

@@ -229,3 +229,9 @@ def test_decode_cache_prefill_then_steps(ops):
     P._err("decode token 2 after reorder", o2, ofull[:, T + 1:T + 2], BF, P.BF16_ABS_O)
     P._err("recurrent state", cache.recurrent_states[0], Sfull, BF, P.BF16_ABS_GRAD)
     assert torch.equal(cache.conv_states[0], conv_full)
+
+
+@pytest.mark.parametrize("cu", [[0, 0, 70], [0, 70, 70], [0, 30, 30, 100], [0, 0, 0, 64]])
+def test_chunk_packed_with_empty_sequences(ops, cu):
+    print(f"chunk packed with empty sequences {cu}", flush=True)
+    P.check_chunk(ops, "cuda", 1, cu[-1], 2, 4, 128, 128, BF, cu=cu, backward=True, h0_std=0.1)
