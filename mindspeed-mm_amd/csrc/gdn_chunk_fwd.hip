@@ -67,13 +67,15 @@ __device__ __forceinline__ void load_tile_qk(T* lds, int ld, const T* g, int64_t
     const bool ok = row < nvalid;
     Vec16<T> x = ok ? ld16(g + (int64_t)row * row_stride + cc * V) : zero16<T>();
     if (l2norm) {   // uniform: every lane takes part in the shuffles
-      float ss = 0.f;
+      float f[V], ss = 0.f;
+      unpack16<T>(x, f);
 #pragma unroll
-      for (int e = 0; e < V; ++e) { const float f = x.get(e); ss += f * f; }
+      for (int e = 0; e < V; ++e) ss += f[e] * f[e];
       ss = lane_group_sum<CPR>(ss);
       const float r = rsqrtf(ss + 1e-6f);
 #pragma unroll
-      for (int e = 0; e < V; ++e) x.set(e, x.get(e) * r);
+      for (int e = 0; e < V; ++e) f[e] *= r;
+      x = pack16<T>(f);
       if (ok && y_out != nullptr) st16(y_out + (int64_t)row * y_stride + cc * V, x);
       if (ok && rstd_out != nullptr && cc == 0) rstd_out[(int64_t)row * rstd_stride] = r;
     }
@@ -90,18 +92,20 @@ __device__ __forceinline__ void load_tile_qk(T* lds, int ld, const T* g, int64_t
 template <typename T, int DK, int BV> struct PrepSmem {
   static constexpr int LDK = lds_ld<T>(DK), LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
   static constexpr int cmax(int a, int b) { return a > b ? a : b; }
-  // Three regions, each reused once its first tenant is dead, so that three workgroups fit a CU's LDS:
-  static constexpr int off_ks = 0;                                    // K tile, scaled in place to beta e^G K
-  static constexpr int off_qs = off_ks + 64 * LDK * (int)sizeof(T);   // Q tile -> A (fp32, solve input) -> Tm in T
+  // Two regions, each reused once its tenant is dead, so that four workgroups (bf16) fit a CU's LDS:
+  //   region 1: K tile -> Tm (fp32, solve output) -> beta e^G K (parked in registers during the solve) -> (beta V) tile
+  //   region 2: Q tile -> A (fp32, solve input) -> Tm in T
+  static constexpr int off_ks = 0;
+  static constexpr int r1_bytes = cmax(cmax(64 * LDK * (int)sizeof(T), 64 * kLF * 4), 64 * LDV * (int)sizeof(T));
+  static constexpr int off_qs = off_ks + r1_bytes;
   static constexpr int qs_bytes = cmax(cmax(64 * LDK * (int)sizeof(T), 64 * kLF * 4), 64 * L64 * (int)sizeof(T));
-  static constexpr int off_ti = off_qs + qs_bytes;                    // Tm (fp32, solve output) -> (beta V) tile
-  static constexpr int ti_bytes = cmax(64 * kLF * 4, 64 * LDV * (int)sizeof(T));
-  static constexpr int off_misc = off_ti + ti_bytes;
+  static constexpr int off_ti = off_ks;
+  static constexpr int off_misc = off_qs + qs_bytes;
   static constexpr int bytes = off_misc + 3 * 64 * 4;
 };
 
 template <typename T, int DK, int BV>
-__global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(3) void chunk_prep_kernel(
+__global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3) void chunk_prep_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ g,
     const float* __restrict__ beta, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets,
     float* __restrict__ G_out, T* __restrict__ Ai_out, T* __restrict__ W_out, T* __restrict__ U_out,
@@ -111,12 +115,12 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(3) void chunk_prep_ker
   using SM = PrepSmem<T, DK, BV>;
   constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64, VEC = Elem<T>::kVec;
   T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
-  T* Kb = Ks;
+  T* Kb = Ks;                                                     // after Tm (fp32)
   T* Qs = reinterpret_cast<T*>(gdn_smem + SM::off_qs);
   float* As = reinterpret_cast<float*>(gdn_smem + SM::off_qs);    // after Q
   T* Tms = reinterpret_cast<T*>(gdn_smem + SM::off_qs);          // after A
   float* Ti = reinterpret_cast<float*>(gdn_smem + SM::off_ti);
-  T* Vb = reinterpret_cast<T*>(gdn_smem + SM::off_ti);           // after Tm (fp32)
+  T* Vb = reinterpret_cast<T*>(gdn_smem + SM::off_ti);           // after beta e^G K
   float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_misc);
   float* bs = Gs + 64;
   float* egs = bs + 64;
@@ -141,7 +145,6 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(3) void chunk_prep_ker
     egs[lane] = b * __expf(x);
     G_out[((int64_t)blockIdx.x * Hv + h) * 64 + lane] = x;   // 64 contiguous values per chunk and head
   }
-  for (int i = tid; i < 64 * kLF; i += kThreads) Ti[i] = 0.f;
   {
     // q and k arrive raw; with the in-kernel l2 norm they are normalised on the way into LDS.  The first value head
     // of each q/k group also leaves the normalised q (for the output kernel and the backward pass) and 1/|q|, 1/|k|.
@@ -200,25 +203,22 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(3) void chunk_prep_ker
       }
     }
   }
-  __syncthreads();   // Q is consumed: its space takes A
+  // beta e^G K, this thread's pieces of the K tile, parked in registers: the K tile's space takes the fp32 Tm first
+  constexpr int KPT = 64 * (DK / VEC) / kThreads;
+  Vec16<T> kreg[KPT];
+#pragma unroll
+  for (int i = 0; i < KPT; ++i) {
+    const int c = tid + i * kThreads, row = c / (DK / VEC), cc = c % (DK / VEC);
+    kreg[i] = scale16<T>(ld16(Ks + row * LDK + cc * VEC), egs[row]);
+  }
+  __syncthreads();   // Q and K are consumed: their space takes A and Tm
 
   {
     const int ti = wave >> 1, tj = wave & 1, j = 32 * tj + acc_col();
 #pragma unroll
     for (int r = 0; r < 16; ++r) As[(32 * ti + acc_row(r)) * kLF + j] = a_tile[r];
   }
-  // K tile -> beta e^G K in place
-  {
-    constexpr int CPR = DK / VEC;
-    for (int c = tid; c < 64 * CPR; c += kThreads) {
-      const int row = c / CPR, cc = c % CPR;
-      Vec16<T> x = ld16(Ks + row * LDK + cc * VEC);
-      const float sc = egs[row];
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) x.set(e, x.get(e) * sc);
-      st16(Kb + row * LDK + cc * VEC, x);
-    }
-  }
+  for (int i = tid; i < 64 * kLF; i += kThreads) Ti[i] = 0.f;
   // the first V block is requested now and parked in registers until the fp32 Tm has been consumed
   const T* vg = v + tok0 * ts.v + h * V;
   constexpr int VPT = 64 * (BV / VEC) / kThreads;   // 16-byte pieces of the V tile per thread
@@ -297,27 +297,25 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(3) void chunk_prep_ker
     constexpr int CPR = 64 / VEC;
     for (int c = tid; c < 64 * CPR; c += kThreads) {
       const int row = c / CPR, cc = c % CPR;
-      Vec16<T> x = zero16<T>();
+      float f[VEC];
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) x.set(e, Ti[row * kLF + cc * VEC + e]);
-      st16(Tms + row * L64 + cc * VEC, x);
+      for (int e = 0; e < VEC; ++e) f[e] = Ti[row * kLF + cc * VEC + e];
+      st16(Tms + row * L64 + cc * VEC, pack16<T>(f));
     }
   }
   __syncthreads();
-  // the fp32 Tm is consumed: its space takes the (beta V) tile parked in registers
+  // the fp32 Tm is consumed: its space takes the beta e^G K tile parked in registers
 #pragma unroll
-  for (int i = 0; i < VPT; ++i) {
-    const int c = tid + i * kThreads, row = c / (BV / VEC), cc = c % (BV / VEC);
-    const float sc = bs[row];
-#pragma unroll
-    for (int e = 0; e < VEC; ++e) vreg[i].set(e, vreg[i].get(e) * sc);
-    st16(Vb + row * LDV + cc * VEC, vreg[i]);
+  for (int i = 0; i < KPT; ++i) {
+    const int c = tid + i * kThreads, row = c / (DK / VEC), cc = c % (DK / VEC);
+    st16(Kb + row * LDK + cc * VEC, kreg[i]);
   }
   {  // the four 32x32 tiles of Tm as A operands (lane <-> row, registers <-> column), fragment order, for the backward
     AccB<T> tf;
     frags_from_lds<T>(tf, Tms + (32 * (wave >> 1) + (lane & 31)) * L64 + 32 * (wave & 1));
     tf.store_stream(Ai_out + (((int64_t)blockIdx.x * Hv + h) * 4 + wave) * 1024);
   }
+  __syncthreads();
 
   // ---- phase 4: W = Tm (beta e^G K), handed on in fragment order only ----
   {
@@ -339,11 +337,17 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(3) void chunk_prep_ker
   }
   // ---- phase 5: U = Tm (beta V), V block by V block, stored in fragment order ----
   for (int vb = 0; vb < V / BV; ++vb) {
-    __syncthreads();
-    if (vb > 0) {
+    __syncthreads();   // the tile in region 1 (beta e^G K, or the previous V block) is consumed
+    if (vb == 0) {     // the first (beta V) block was parked in registers
+#pragma unroll
+      for (int i = 0; i < VPT; ++i) {
+        const int c = tid + i * kThreads, row = c / (BV / VEC), cc = c % (BV / VEC);
+        st16(Vb + row * LDV + cc * VEC, scale16<T>(vreg[i], bs[row]));
+      }
+    } else {
       load_tile_scaled<T, BV>(Vb, LDV, vg + vb * BV, ts.v, nvalid, bs, tid);
-      __syncthreads();
     }
+    __syncthreads();
     for (int tt = wave; tt < 2 * (BV / 32); tt += 4) {
       const int ri = tt & 1, cj = tt >> 1;
       f32x16 acc = acc_zero();

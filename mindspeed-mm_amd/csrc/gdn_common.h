@@ -155,6 +155,37 @@ template <typename T> __device__ __forceinline__ Vec16<T> ld16(const T* p) {
 template <typename T> __device__ __forceinline__ void st16(T* p, const Vec16<T>& v) {
   *reinterpret_cast<u32x4*>(p) = v.raw;
 }
+// fp32 values of a 16-byte piece and back (bf16: two elements per 32-bit word, one conversion instruction per word)
+template <typename T> __device__ __forceinline__ void unpack16(const Vec16<T>& v, float* f) {
+  if constexpr (sizeof(T) == 4) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) f[e] = __uint_as_float(v.raw[e]);
+  } else if constexpr (std::is_same<T, bf16_t>::value) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      f[2 * e] = __uint_as_float(v.raw[e] << 16);
+      f[2 * e + 1] = __uint_as_float(v.raw[e] & 0xffff0000u);
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < Elem<T>::kVec; ++e) f[e] = v.get(e);
+  }
+}
+template <typename T> __device__ __forceinline__ Vec16<T> pack16(const float* f) {
+  Vec16<T> r;
+  if constexpr (sizeof(T) == 4) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) r.raw[e] = __float_as_uint(f[e]);
+  } else if constexpr (std::is_same<T, bf16_t>::value) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) r.raw[e] = f32x2_to_bf16x2(f[2 * e], f[2 * e + 1]);
+  } else {
+    r.raw = u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int e = 0; e < Elem<T>::kVec; ++e) r.set(e, f[e]);
+  }
+  return r;
+}
 // every element of a 16-byte piece times one factor (bf16: two elements per conversion instruction)
 template <typename T> __device__ __forceinline__ Vec16<T> scale16(const Vec16<T>& v, float s) {
   Vec16<T> r;
@@ -190,9 +221,7 @@ __device__ __forceinline__ void load_tile_scaled(T* lds, int ld, const T* g, int
     Vec16<T> v = zero16<T>();
     if (row < nvalid) {
       v = ld16(g + (int64_t)row * row_stride + cc * V);
-      const float s = rowscale[row];
-#pragma unroll
-      for (int e = 0; e < V; ++e) v.set(e, v.get(e) * s);
+      v = scale16<T>(v, rowscale[row]);
     }
     st16(lds + row * ld + cc * V, v);
   }
@@ -521,8 +550,12 @@ __device__ __forceinline__ void acc_store_rows(const f32x16& acc, const Identity
       Vec16<T> x = ld16(patch + row * PLD + cc * V);
       if constexpr (ADD) {
         const Vec16<T> y = ld16(g + (int64_t)row * row_stride + cc * V);
+        float fx[V], fy[V];
+        unpack16<T>(x, fx);
+        unpack16<T>(y, fy);
 #pragma unroll
-        for (int e = 0; e < V; ++e) x.set(e, x.get(e) + y.get(e));
+        for (int e = 0; e < V; ++e) fx[e] += fy[e];
+        x = pack16<T>(fx);
       }
       st16(g + (int64_t)row * row_stride + cc * V, x);
     }
