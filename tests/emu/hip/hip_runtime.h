@@ -246,6 +246,7 @@ static emu::GdimProxy gridDim;
 #define __builtin_amdgcn_s_barrier() emu::syncthreads()
 #define __builtin_amdgcn_fence(...) ((void)0)
 #define __builtin_amdgcn_sched_barrier(x) ((void)0)
+#define __builtin_amdgcn_rcpf(x) (1.0f / (x))
 #define GDN_REGS_256
 #define GDN_WAVES_PER_SIMD(n)
 #define __builtin_amdgcn_sched_group_barrier(m, n, s) ((void)0)
