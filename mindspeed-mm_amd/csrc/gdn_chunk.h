@@ -79,10 +79,10 @@ inline ChunkWorkspace chunk_workspace_layout(const ChunkDims& d, int elem_bytes)
   return w;
 }
 
-// The two sequential kernels give one compute wave a 32-column slab of the state.  A workgroup streams its chunk's
-// operand tiles at the rate one CU can pull (~35 GB/s), whatever the number of slabs it serves, so when the whole
-// problem has no more slabs than the device has CUs every slab gets a workgroup (and a CU) of its own; larger
-// problems put two slabs in a workgroup, which share the tiles.
+// The two sequential kernels give one compute wave a 32-column slab of the state.  What limits them is the rate at
+// which one CU gets its requests served (about 35 GB/s measured, loads and stores together), whatever the number of
+// slabs the workgroup serves, so when the whole problem has no more slabs than the device has CUs every slab gets a
+// workgroup (and a CU) of its own; larger problems put two slabs in a workgroup, which share the tiles.
 int device_compute_units();   // defined with the forward launcher
 
 inline bool one_slab_per_workgroup(const ChunkDims& d, int compute_units) {

@@ -85,7 +85,8 @@ __device__ __forceinline__ void load_tile_qk(T* lds, int ld, const T* g, int64_t
 
 // ---------------------------------------------------------------------------------------------
 // chunk_prep_kernel: everything that is independent across chunks.
-//   G (cumulative decay), Tm = (I+L)^-1, W = Tm (beta e^G K), U = Tm (beta V), Aq = tril(Q K^T . Gam)
+//   G (cumulative decay), Tm = (I+L)^-1, -W = -Tm (beta e^G K), U = Tm (beta V), Aq = scale tril(Q K^T . Gam),
+//   per q/k group the K^T, K and Q^T tiles of the recurrence kernels
 // U is written in fragment order (AccB<>): tile (32-token block ri) x (32-column block vb) at
 // U[chunk][head][vb][ri][1024], 16 bytes per lane per k-group -- the recurrence kernel copies it straight to LDS.
 // ---------------------------------------------------------------------------------------------
@@ -180,8 +181,8 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
     af.pack(aq);
     af.store_stream(Aq_out + (((int64_t)blockIdx.x * Hv + h) * 4 + wave) * 1024);
   }
-  // (e^{G_last-G} . K)^T as A-operand fragments for the state update: K tile fragments (lane <-> token) turned
-  // through the matrix core into (lane <-> K column, registers <-> token), scaled per token, stored in fragment order
+  // K^T as A-operand fragments for the state update: K tile fragments (lane <-> token) turned through the matrix
+  // core into (lane <-> K column, registers <-> token), stored in fragment order (the decay is applied by the reader)
   {
     IdentityFrag<T> id;
     id.init();
@@ -363,16 +364,16 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
 // ---------------------------------------------------------------------------------------------
 // chunk_state_kernel: the inter-chunk recurrence, kept as lean as possible because it is the only part of the
 // forward pass that is sequential in the chunks.  One compute wave owns a 32-column slab of the state S[K, 32] in
-// fp32 accumulators for the whole sequence and per chunk does
-//     V' = U - W S            S <- e^{G_last} S + (e^{G_last-G} . K)^T V'
+// fp32 registers for the whole sequence and per chunk does
+//     V' = U - W S            S <- e^{G_last} S + K^T (e^{G_last-G} . V')
 // Both B operands (S, V') are taken straight from accumulator registers (frag_b_from_acc), so the chain
 // W S -> V' -> S never touches LDS and the compute waves of a workgroup never exchange data.  S (before the chunk)
 // and V' leave the kernel in fragment order, 16 bytes per lane per k-group, for chunk_out_kernel and the backward
-// pass.  The A operands (W, the decay-scaled K^T) and U arrive in fragment order, one contiguous 16 KB block per
-// chunk and head prepared by chunk_prep_kernel (token-major tiles would be 64 rows scattered 8 KB apart), and are
-// copied to LDS in 16-byte pieces by NW loader waves of the same workgroup, which run ahead of the NW compute
-// waves: loads for chunk c+2 are in flight in registers while chunk c+1 sits in the other LDS stage; the two roles
-// meet at one barrier per chunk.
+// pass.  The A operands (-W per value head, K^T per q/k group) and U arrive in fragment order, one contiguous 16 KB
+// block per chunk prepared by chunk_prep_kernel (token-major tiles would be 64 rows scattered 8 KB apart), and are
+// copied to LDS in 16-byte pieces by NL loader waves of the same workgroup, which run ahead of the NW compute
+// waves: loads for chunks c+2 and c+3 are in flight in registers while chunk c+1 sits in the other LDS stage; the
+// two roles meet at one barrier per chunk.
 // ---------------------------------------------------------------------------------------------
 template <typename T, int DK, int NW, int STAGES> struct StateSmem {
   static constexpr int off_ws = 0;
