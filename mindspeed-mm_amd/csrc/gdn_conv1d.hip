@@ -324,6 +324,40 @@ __global__ void conv1d_update_kernel(const T* __restrict__ hidden, T* __restrict
   for (int j = 0; j < S; ++j) state[((int64_t)b * D + d) * S + j] = Elem<T>::from_f(st[j]);
 }
 
+// The same for the usual state length S == W with a row of W elements 8 or 16 bytes long: the state row and the
+// weight row of a channel are one vector load each, the window lives in registers with constant indices.
+template <typename T, int W>
+__global__ __launch_bounds__(256) void conv1d_update_rows_kernel(const T* __restrict__ hidden, T* __restrict__ state,
+                                                                 const T* __restrict__ weight, const T* __restrict__ bias,
+                                                                 T* __restrict__ out, int B, int T_len, int D, int silu) {
+  constexpr int kBytes = W * (int)sizeof(T);
+  static_assert(kBytes == 8 || kBytes == 16, "a row is one 8- or 16-byte vector");
+  typedef uint32_t RowVec __attribute__((ext_vector_type(kBytes / 4)));
+  union Row { RowVec v; T e[W]; };
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (int64_t)B * D) return;
+  const int b = (int)(idx / D), d = (int)(idx % D);
+  Row r, wr;
+  r.v = *reinterpret_cast<const RowVec*>(state + idx * W);
+  wr.v = *reinterpret_cast<const RowVec*>(weight + (int64_t)d * W);
+  float st[W + 1], wg[W];
+#pragma unroll
+  for (int j = 0; j < W; ++j) { st[j] = Elem<T>::to_f(r.e[j]); wg[j] = Elem<T>::to_f(wr.e[j]); }
+  const float bs = bias ? Elem<T>::to_f(bias[d]) : 0.f;
+  for (int t = 0; t < T_len; ++t) {
+    st[W] = Elem<T>::to_f(hidden[((int64_t)b * T_len + t) * D + d]);
+    float a = bs;
+#pragma unroll
+    for (int w = 0; w < W; ++w) a += st[1 + w] * wg[w];
+    out[((int64_t)b * T_len + t) * D + d] = Elem<T>::from_f(silu ? a * sigmoidf_(a) : a);
+#pragma unroll
+    for (int j = 0; j < W; ++j) st[j] = st[j + 1];
+  }
+#pragma unroll
+  for (int j = 0; j < W; ++j) r.e[j] = Elem<T>::from_f(st[j]);
+  *reinterpret_cast<RowVec*>(state + idx * W) = r.v;
+}
+
 template <typename T> struct ConvLaunch {
   static int fwd(const void* x, const void* weight, const void* bias, const void* residual, const void* init,
                  const int64_t* cu, void* y, void* fs, int B, int T_len, int N, int D, int W, int silu,
@@ -387,8 +421,18 @@ template <typename T> struct ConvLaunch {
   static int update(const void* hidden, void* state, const void* weight, const void* bias, void* out, int B,
                     int T_len, int D, int W, int S, int silu, hipStream_t st) {
     const int64_t n = (int64_t)B * D;
-    GDN_LAUNCH(kKernConvUpdate, st, (conv1d_update_kernel<T>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
-                       (const T*)hidden, (T*)state, (const T*)weight, (const T*)bias, (T*)out, B, T_len, D, W, S, silu);
+    const dim3 grid((unsigned)((n + 255) / 256));
+    const bool aligned = (((uintptr_t)state | (uintptr_t)weight) & 15) == 0;
+    if (S == W && aligned && W * (int)sizeof(T) == 8) {
+      GDN_LAUNCH(kKernConvUpdate, st, (conv1d_update_rows_kernel<T, 8 / (int)sizeof(T)>), grid, dim3(256), 0, st,
+                 (const T*)hidden, (T*)state, (const T*)weight, (const T*)bias, (T*)out, B, T_len, D, silu);
+    } else if (S == W && aligned && W * (int)sizeof(T) == 16) {
+      GDN_LAUNCH(kKernConvUpdate, st, (conv1d_update_rows_kernel<T, 16 / (int)sizeof(T)>), grid, dim3(256), 0, st,
+                 (const T*)hidden, (T*)state, (const T*)weight, (const T*)bias, (T*)out, B, T_len, D, silu);
+    } else {
+      GDN_LAUNCH(kKernConvUpdate, st, (conv1d_update_kernel<T>), grid, dim3(256), 0, st, (const T*)hidden, (T*)state,
+                 (const T*)weight, (const T*)bias, (T*)out, B, T_len, D, W, S, silu);
+    }
     return (int)hipGetLastError();
   }
 };

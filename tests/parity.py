@@ -101,10 +101,11 @@ def check_conv(ops, device, B, T, D, W, dtype, activation="silu", cu=None, bias=
     return errs
 
 
-def check_conv_update(ops, device, B, T, D, W, dtype, seed=0, wrap=lambda t: t):
+def check_conv_update(ops, device, B, T, D, W, dtype, seed=0, wrap=lambda t: t, S=None):
+    """S: length of the state rows (default W, the layer's; a longer state takes the kernel's general path)."""
     gen = torch.Generator().manual_seed(seed)
     r = lambda *s: torch.randn(*s, generator=gen)
-    x, st, w, b = r(B, T, D).to(dtype), r(B, D, W).to(dtype), (r(D, W) / 2).to(dtype), r(D).to(dtype)
+    x, st, w, b = r(B, T, D).to(dtype), r(B, D, S or W).to(dtype), (r(D, W) / 2).to(dtype), r(D).to(dtype)
     st_dev = wrap(st.to(device)).clone()
     y = ops.causal_conv1d_update(wrap(x.to(device)), st_dev, wrap(w.to(device)), wrap(b.to(device)), "silu")
     st_ref = st.float().clone()

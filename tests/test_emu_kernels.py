@@ -102,3 +102,8 @@ def test_gdn_gates(ops, dtype, shape, Hv, pdt):
 ])
 def test_decode_step(ops, dtype, B, steps, Hqk, Hv, K, V, W, pdt):
     P.check_decode_step(ops, "cpu", B, steps, Hqk, Hv, K, V, W, dtype, param_dtype=pdt, wrap=guarded)
+
+
+@pytest.mark.parametrize("dtype,B,T,D,W,S", [(F32, 2, 3, 16, 4, 6), (BF, 2, 2, 8, 3, 3), (BF, 1, 1, 8, 4, 3)])
+def test_conv1d_update_general_state_length(ops, dtype, B, T, D, W, S):
+    P.check_conv_update(ops, "cpu", B, T, D, W, dtype, S=S, wrap=guarded)

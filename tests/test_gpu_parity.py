@@ -235,3 +235,8 @@ def test_decode_cache_prefill_then_steps(ops):
 def test_chunk_packed_with_empty_sequences(ops, cu):
     print(f"chunk packed with empty sequences {cu}", flush=True)
     P.check_chunk(ops, "cuda", 1, cu[-1], 2, 4, 128, 128, BF, cu=cu, backward=True, h0_std=0.1)
+
+
+@pytest.mark.parametrize("dtype,B,T,D,W,S", [(F32, 2, 3, 16, 4, 6), (BF, 2, 2, 8, 3, 3), (BF, 1, 1, 8, 4, 3)])
+def test_conv1d_update_general_state_length(ops, dtype, B, T, D, W, S):
+    P.check_conv_update(ops, "cuda", B, T, D, W, dtype, S=S)
