@@ -58,6 +58,11 @@ CHUNK_CASES = [
     (BF, 3, 195, 2, 4, 128, 128, True, None),
     (BF, 1, 256, 1, 2, 128, 256, True, None),                    # wide value heads (config 4 head shape)
     (F32, 1, 96, 1, 2, 128, 192, True, [0, 1, 38, 96]),
+    # (sequences x q/k groups) a multiple of 8 with grouped heads: the recurrence kernels renumber their workgroups
+    (BF, 4, 200, 2, 4, 128, 128, True, None),
+    (BF, 2, 130, 4, 16, 128, 128, True, None),
+    (BF, 1, 600, 1, 2, 64, 64, False, [0, 64, 65, 130, 258, 300, 450, 599, 600]),
+    (F32, 8, 70, 1, 2, 64, 64, True, None),
 ]
 
 
