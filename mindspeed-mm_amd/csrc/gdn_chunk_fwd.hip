@@ -385,7 +385,7 @@ template <typename T, int DK, int NW, int STAGES> struct StateSmem {
 };
 
 template <typename T, int DK, int NW, int NL, int STAGES>
-__global__ __launch_bounds__(64 * (NW + NL)) GDN_REGS_256 void chunk_state_kernel(
+__global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 2 : 1) void chunk_state_kernel(
     const T* __restrict__ ktf, const T* __restrict__ w, const T* __restrict__ uf, const float* __restrict__ G,
     const float* __restrict__ h0, float* __restrict__ ht, T* __restrict__ vf, T* __restrict__ hf,
     const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int Hqk, int Hv, int V) {

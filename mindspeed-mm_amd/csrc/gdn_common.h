@@ -88,12 +88,12 @@ __device__ __forceinline__ int xcd_grouped_head(int b, int total, int grp) {
   const int j = b & 7, m = b >> 3;
   return ((m / grp) * 8 + j) * grp + m % grp;
 }
-// Kernel attribute: at most 256 registers per lane.  With a larger budget the compiler keeps matrix accumulators in
-// the accumulation registers, and every vector instruction that touches them (decay, packing) then costs an extra
-// move in each direction.
-#ifndef GDN_REGS_256
-#define GDN_WAVES_PER_SIMD(n) __attribute__((amdgpu_waves_per_eu(n, n)))   // register budget 512 / n per lane
-#define GDN_REGS_256 GDN_WAVES_PER_SIMD(2)
+// Kernel attribute: register budget of 512 / n per lane (n waves per SIMD).  With more than 256 registers allowed the
+// compiler keeps matrix accumulators in the accumulation registers, and every vector instruction that touches them
+// (decay, packing) then costs an extra move in each direction; a budget that allows more workgroups per CU is what
+// the memory-bound kernels gain most from.
+#ifndef GDN_WAVES_PER_SIMD
+#define GDN_WAVES_PER_SIMD(n) __attribute__((amdgpu_waves_per_eu(n, n)))
 #endif
 // Asks the scheduler for the pattern (1 matrix instruction, nvalu vector instructions) x nmfma in the current
 // scheduling region.

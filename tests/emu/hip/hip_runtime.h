@@ -247,7 +247,6 @@ static emu::GdimProxy gridDim;
 #define __builtin_amdgcn_fence(...) ((void)0)
 #define __builtin_amdgcn_sched_barrier(x) ((void)0)
 #define __builtin_amdgcn_rcpf(x) (1.0f / (x))
-#define GDN_REGS_256
 #define GDN_WAVES_PER_SIMD(n)
 #define __builtin_amdgcn_sched_group_barrier(m, n, s) ((void)0)
 #define __builtin_amdgcn_wave_barrier() emu::wave_sync()
