@@ -107,3 +107,25 @@ def test_decode_step(ops, dtype, B, steps, Hqk, Hv, K, V, W, pdt):
 @pytest.mark.parametrize("dtype,B,T,D,W,S", [(F32, 2, 3, 16, 4, 6), (BF, 2, 2, 8, 3, 3), (BF, 1, 1, 8, 4, 3)])
 def test_conv1d_update_general_state_length(ops, dtype, B, T, D, W, S):
     P.check_conv_update(ops, "cpu", B, T, D, W, dtype, S=S, wrap=guarded)
+
+
+def _random_case(seed):
+    import random
+    rng = random.Random(seed)
+    B = rng.choice([1, 1, 2])
+    T = rng.randint(1, 200)
+    Hqk = rng.choice([1, 2])
+    Hv = Hqk * rng.choice([1, 2, 4])
+    K, V = rng.choice([64, 128]), rng.choice([64, 128, 192])
+    cu = None
+    if B == 1 and rng.random() < 0.6:
+        cuts = sorted(rng.sample(range(0, T + 1), min(T + 1, rng.randint(0, 4))))
+        cu = [0] + cuts + [T]
+    return (BF if seed % 2 else F32), B, T, Hqk, Hv, K, V, rng.random() < 0.7, cu
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_chunk_random_shapes(ops, seed):
+    """Seeded random shapes: ragged lengths, packed sequences with empty and one-token members, grouped heads."""
+    dtype, B, T, Hqk, Hv, K, V, l2, cu = _random_case(seed)
+    P.check_chunk(ops, "cpu", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu, backward=True, wrap=guarded, h0_std=0.1, seed=seed)

@@ -245,3 +245,12 @@ def test_chunk_packed_with_empty_sequences(ops, cu):
 @pytest.mark.parametrize("dtype,B,T,D,W,S", [(F32, 2, 3, 16, 4, 6), (BF, 2, 2, 8, 3, 3), (BF, 1, 1, 8, 4, 3)])
 def test_conv1d_update_general_state_length(ops, dtype, B, T, D, W, S):
     P.check_conv_update(ops, "cuda", B, T, D, W, dtype, S=S)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_chunk_random_shapes(ops, seed):
+    """The seeded random shapes of the CPU emulation tests, on the device build."""
+    from tests.test_emu_kernels import _random_case
+    dtype, B, T, Hqk, Hv, K, V, l2, cu = _random_case(seed)
+    print(f"chunk random {seed}: {dtype} B{B} T{T} Hqk{Hqk} Hv{Hv} K{K} V{V} l2={l2} cu={cu}", flush=True)
+    P.check_chunk(ops, "cuda", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu, backward=True, h0_std=0.1, seed=seed)
