@@ -332,8 +332,8 @@ def main():
             b_ = ab.sigmoid()
             g_ = -A_log.float().exp() * torch.nn.functional.softplus(aa.float() + dt_b)
             torch.autograd.grad([g_, b_], [aa, ab, A_log, dt_b], [dgg, dgg.to(torch.bfloat16)])
-        aux["gates"] = {"fused_fwd_bwd_ms": round(wall_ms(gates_step), 4),
-                        "torch_elementwise_fwd_bwd_ms": round(wall_ms(gates_eager_step), 4)}
+        aux["gates"] = {"fused_fwd_bwd_ms": round(wall_ms(gates_step, 100), 4),
+                        "torch_elementwise_fwd_bwd_ms": round(wall_ms(gates_eager_step, 100), 4)}
 
     if args.calibrate_copy:
         src = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
