@@ -33,7 +33,10 @@ namespace gdn {
 template <typename T, int DK, int NW, int STAGES> struct StateBwdSmem {
   static constexpr int big = 3 * 64 * DK * (int)sizeof(T) + 2 * 64 * 4 + 16;   // K, Q^T, W^T images, [64 unused], G_last, scale e^G [64]
   static constexpr int off_small = STAGES * big;            // dO rows of the slab [64][32 NW] | tril(Q K^T . Gam) tiles [4]
-  static constexpr int bytes = off_small + (NW * 2048 + 4096) * (int)sizeof(T);
+  static constexpr int small_elems = NW * 2048 + 4096;
+  // two small stages (and one barrier per step instead of two) where the CU's 160 KB of LDS allow it
+  static constexpr int small_stages = (STAGES == 2 && off_small + 2 * small_elems * (int)sizeof(T) <= 160 * 1024) ? 2 : 1;
+  static constexpr int bytes = off_small + small_stages * small_elems * (int)sizeof(T);
 };
 
 template <typename T, int DK, int NW, int NL, int STAGES>
@@ -56,7 +59,7 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
   const int len = cu ? (int)(cu[n + 1] - bos) : T_len;
   const int nchunks = (len + kChunk - 1) / kChunk;
   const int64_t chunk_base = cu ? chunk_offsets[n] : (int64_t)n * ((T_len + kChunk - 1) / kChunk);
-  T* small = reinterpret_cast<T*>(gdn_smem + SM::off_small);   // dO rows of the slab, row-major | Aq tiles
+  T* small0 = reinterpret_cast<T*>(gdn_smem + SM::off_small);   // per stage: dO rows of the slab, row-major | Aq tiles
 
   // step s = 0 .. nchunks-1 handles chunk nchunks-1-s
   if (wave >= NW) {
@@ -113,7 +116,8 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
       if (lt < 64) dec[68 + lt] = scale * __expf(pgt[set]);
       if (lt == 0) dec[64] = pgl[set];
     };
-    auto commit_small = [&](int set) {
+    auto commit_small = [&](int set, int buf) {
+      T* small = small0 + buf * SM::small_elems;
 #pragma unroll
       for (int i = 0; i < CUL; ++i) st16(small + (lt + i * NT) * VEC, pd[set][i]);
 #pragma unroll
@@ -125,7 +129,7 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
       if (nchunks == 0) return;
       issue(0, 0);
       commit_big(0, 0);
-      commit_small(0);
+      commit_small(0, 0);
 #pragma unroll
       for (int j = 1; j <= DEPTH; ++j) issue(imin(j, nchunks - 1), j % DEPTH);
       for (int s0 = 0;; s0 += DEPTH) {
@@ -133,10 +137,10 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
         for (int u = 0; u < DEPTH; ++u) {
           const int st = s0 + u;
           if (st >= nchunks) return;
-          GDN_LDS_BARRIER();                // (A) step st staged
+          GDN_LDS_BARRIER();                // (A) step st staged; the other stages (step st-1) are free
+          if (SM::small_stages == 1) GDN_LDS_BARRIER();   // (B) the compute waves have taken the single small stage
+          commit_small((u + 1) % DEPTH, (st + 1) & (SM::small_stages - 1));
           commit_big((u + 1) % DEPTH, (st + 1) & 1);
-          GDN_LDS_BARRIER();                // (B) the compute waves have taken their dO rows and the Aq tiles
-          commit_small((u + 1) % DEPTH);
           issue(imin(st + 1 + DEPTH, nchunks - 1), (u + 1) % DEPTH);
         }
       }
@@ -145,9 +149,9 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
         if (st > 0) GDN_LDS_BARRIER();      // (C) the single big stage is free again
         issue(st, 0);
         commit_big(0, 0);
-        commit_small(0);
+        commit_small(0, 0);
         GDN_LDS_BARRIER();                  // (A)
-        GDN_LDS_BARRIER();                  // (B)
+        GDN_LDS_BARRIER();                  // (B) the compute waves have taken their dO rows and the Aq tiles
       }
     }
     return;
@@ -179,12 +183,13 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
     // dO of this wave's 32 columns as B operand (lane <-> V column, registers <-> token), turned from the row-major
     // rows through the matrix core; dv_local = (scale tril(Q K^T . Gam))^T dO from the forward pass's tiles
     AccB<T> dob[2], dos[2], aq[3];
+    const T* small = small0 + (st & (SM::small_stages - 1)) * SM::small_elems;
     frags_from_lds<T>(dob[0], small + (lane & 31) * (32 * NW) + 32 * wave);
     frags_from_lds<T>(dob[1], small + (32 + (lane & 31)) * (32 * NW) + 32 * wave);
     aq[0].load(small + NW * 2048);            // tiles (0,0), (1,0), (1,1)
     aq[1].load(small + NW * 2048 + 2048);
     aq[2].load(small + NW * 2048 + 3072);
-    GDN_LDS_BARRIER();                      // (B)
+    if (SM::small_stages == 1) GDN_LDS_BARRIER();   // (B) the single small stage may be refilled
     unsigned char* base = gdn_smem + buf * SM::big;
     const T* Ka = reinterpret_cast<const T*>(base);
     const T* Qa = Ka + TILE;
