@@ -128,6 +128,18 @@ def main():
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     value = tokens / (ms_per_step * 1e-3)
 
+    # ---- spread of the step time: each of max(steps, 50) further steps bracketed by events on the launch stream ----
+    nspread = max(args.steps, 50)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nspread)]
+    for a, b in evs:
+        a.record()
+        step()
+        b.record()
+    torch.cuda.synchronize()
+    per_step = sorted(a.elapsed_time(b) for a, b in evs)
+    spread = {"n": nspread, "median_ms": round(per_step[nspread // 2], 4), "p10_ms": round(per_step[nspread // 10], 4),
+              "p90_ms": round(per_step[(9 * nspread) // 10], 4)}
+
     # ---- instrumented pass: per-kernel durations from HIP events on the launch stream ----
     lib.gdn_profile_enable(1)
     for _ in range(args.steps):
@@ -169,7 +181,7 @@ def main():
     path_tflops = ref_formula_flops(tokens, c["Hv"], c["K"], c["V"]) / (ms_per_step * 1e-3) / 1e12
     aux = {"path_tflops_ref_formula": round(path_tflops, 2),
            "path_frac_of_bf16_mfma_peak": round(path_tflops / PEAK_BF16_TFLOPS, 4),
-           "kernel_ms_sum": round(total_kernel_ms, 3), "kernels": per_kernel}
+           "kernel_ms_sum": round(total_kernel_ms, 3), "step_time_spread": spread, "kernels": per_kernel}
 
     if not args.no_aux:
         # ---- decode: batch 256, 64 consecutive steps, state updated in place (BASELINE.json configs[3]) ----
