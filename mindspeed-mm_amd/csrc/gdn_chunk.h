@@ -34,7 +34,6 @@ struct ChunkWorkspace {
   int64_t qn;             // T [tokens,Hqk,K] l2-normalised q (only with use_qk_l2norm)
   int64_t rstd;           // f32 [2][tokens,Hqk] 1/|q|, 1/|k| of that normalisation
   int64_t G;              // f32 [chunks,Hv,64]      chunk-local cumulative log decay
-  int64_t Ai;             // T [chunks,Hv,2,2]       (I + A)^-1 as A operand: tile = (32 rows) x (32 columns), fragment order
   int64_t WAF;            // T [chunks,Hv,K/32,2]    -W as A operand: tile = (32 tokens) x (32 columns of K), fragment order
   int64_t AQ;             // T [chunks,Hv,2,2]       scale tril(Q K^T . Gam), accumulator tiles: lane <-> column, registers <-> row
   // Tiles exchanged between kernels in fragment order (see AccB<>): 1024 elements per 32x32 tile.
@@ -43,6 +42,7 @@ struct ChunkWorkspace {
   int64_t VF;             // T [chunks,Hv,V/32,2]    v_new = U - W S
   int64_t HF;             // T [chunks,Hv,V/32,K/32] state BEFORE each chunk, tile = (32 rows of K) x (32 columns of V)
   int64_t fwd_bytes;
+  int64_t Ai;             // T [chunks,Hv,2,2]       (I + A)^-1 as A operand: tile = (32 rows) x (32 columns), fragment order
   int64_t WF;             // T [chunks,Hv,K/32,2]    -W^T as A operand (written by the forward when a backward follows)
   int64_t QTF;            // T [chunks,Hqk,K/32,2]   Q^T as A operand: tile = (32 columns of K) x (32 tokens)
   int64_t KAF;            // T [chunks,Hqk,K/32,2]   K as A operand: tile = (32 tokens) x (32 columns of K)
@@ -62,7 +62,6 @@ inline ChunkWorkspace chunk_workspace_layout(const ChunkDims& d, int elem_bytes)
   w.qn = take(tok * d.Hqk * d.K * elem_bytes);
   w.rstd = take(2 * tok * d.Hqk * 4);
   w.G = take(nc * 64 * d.Hv * 4);
-  w.Ai = take(nc * 64 * d.Hv * 64 * elem_bytes);
   w.WAF = take(nc * 64 * d.Hv * d.K * elem_bytes);
   w.AQ = take(nc * 64 * d.Hv * 64 * elem_bytes);
   w.KTF = take(nc * 64 * d.Hqk * d.K * elem_bytes);
@@ -70,6 +69,7 @@ inline ChunkWorkspace chunk_workspace_layout(const ChunkDims& d, int elem_bytes)
   w.VF = take(nc * 64 * d.Hv * d.V * elem_bytes);
   w.HF = take(nc * d.Hv * d.V * d.K * elem_bytes);
   w.fwd_bytes = off;
+  w.Ai = take(nc * 64 * d.Hv * 64 * elem_bytes);
   w.WF = take(nc * 64 * d.Hv * d.K * elem_bytes);
   w.QTF = take(nc * 64 * d.Hqk * d.K * elem_bytes);
   w.KAF = take(nc * 64 * d.Hqk * d.K * elem_bytes);

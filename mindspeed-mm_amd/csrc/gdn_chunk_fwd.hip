@@ -311,7 +311,7 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
     const int c = tid + i * kThreads, row = c / (DK / VEC), cc = c % (DK / VEC);
     st16(Kb + row * LDK + cc * VEC, kreg[i]);
   }
-  {  // the four 32x32 tiles of Tm as A operands (lane <-> row, registers <-> column), fragment order, for the backward
+  if (Ai_out != nullptr) {  // the four 32x32 tiles of Tm as A operands (lane <-> row, registers <-> column), for the backward
     AccB<T> tf;
     frags_from_lds<T>(tf, Tms + (32 * (wave >> 1) + (lane & 31)) * L64 + 32 * (wave & 1));
     tf.store_stream(Ai_out + (((int64_t)blockIdx.x * Hv + h) * 4 + wave) * 1024);
@@ -673,7 +673,7 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   T* qn = l2norm ? reinterpret_cast<T*>(ws + L.qn) : nullptr;   // normalised q, written by the prep kernel
   float* rstd = reinterpret_cast<float*>(ws + L.rstd);
   float* G = reinterpret_cast<float*>(ws + L.G);
-  T* Ai = reinterpret_cast<T*>(ws + L.Ai);
+  T* Ai = with_backward ? reinterpret_cast<T*>(ws + L.Ai) : nullptr;
   T* W = reinterpret_cast<T*>(ws + L.WAF);
   T* AQ = reinterpret_cast<T*>(ws + L.AQ);
   T* UF = reinterpret_cast<T*>(ws + L.UF);
