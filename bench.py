@@ -327,6 +327,12 @@ def main():
                 fn()
             torch.cuda.synchronize()
             return (time.perf_counter() - t0) / n * 1e3
+        def prefill_step():
+            with torch.no_grad():
+                ops.chunk_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], initial_state=d["h0"],
+                                           output_final_state=True, use_qk_l2norm_in_kernel=True)
+        pf = wall_ms(prefill_step, 20)
+        aux["forward_only"] = {"ms": round(pf, 4), "tokens_per_s": round(tokens / (pf * 1e-3), 1)}
         aux["rule_in_layer"] = {"unsplit_qkv_ms": round(wall_ms(unsplit_step), 4),
                                 "split_with_copies_ms": round(wall_ms(split_step), 4)}
         del mixed
