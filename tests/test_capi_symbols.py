@@ -77,3 +77,44 @@ def test_validation_errors_match_reference():
                                  initial_state=torch.zeros(3, 1, 64, 64))
     with pytest.raises(ValueError):
         M.causal_conv1d(torch.randn(1, 8, 8), torch.randn(4, 16))
+
+
+def test_validation_of_the_layer_level_entry_points():
+    """Shape and dtype errors of the operators around the rule are raised before anything touches a device."""
+    import torch
+    import mindspeed_mm_amd as M
+    BF = torch.bfloat16
+    mixed = torch.randn(1, 64, 2 * 64 + 64, dtype=BF)
+    g, b = torch.zeros(1, 64, 1), torch.ones(1, 64, 1)
+    with pytest.raises(ValueError):          # too narrow for q | k | v
+        M.chunk_gated_delta_rule_qkv(mixed[..., :100], g, b, 1, 1, 64, 64)
+    with pytest.raises(ValueError):          # g, beta of the wrong head count
+        M.chunk_gated_delta_rule_qkv(mixed, torch.zeros(1, 64, 2), torch.ones(1, 64, 2), 1, 1, 64, 64)
+    with pytest.raises(ValueError):          # packed input needs batch 1
+        M.chunk_gated_delta_rule_qkv(torch.cat([mixed, mixed]), torch.zeros(2, 64, 1), torch.ones(2, 64, 1), 1, 1, 64, 64,
+                                     cu_seqlens=torch.tensor([0, 64, 128]))
+    with pytest.raises(RuntimeError, match="no host fallback"):
+        M.chunk_gated_delta_rule_qkv(mixed, g, b, 1, 1, 64, 64)
+    a = torch.randn(2, 5, 4, dtype=BF)
+    with pytest.raises(ValueError):          # parameters of the wrong length
+        M.gdn_gates(a, a, torch.zeros(3), torch.zeros(4))
+    with pytest.raises(ValueError):          # a, b of different dtypes
+        M.gdn_gates(a, a.float(), torch.zeros(4), torch.zeros(4))
+    with pytest.raises(RuntimeError, match="no host fallback"):
+        M.gdn_gates(a, a, torch.zeros(4), torch.zeros(4))
+    with pytest.raises(ValueError):          # projections of the wrong shape for the decode step
+        M.fused_recurrent_gated_delta_rule_qkv(mixed[:, :1], a[:1, :1], a[:1, :1], torch.zeros(4), torch.zeros(4),
+                                               1, 1, 64, 64)
+
+
+def test_decode_cache_bookkeeping():
+    import torch
+    from mindspeed_mm_amd import GdnDecodeCache
+    c = GdnDecodeCache(3)
+    assert len(c) == 3 and not c.has_previous_state(1)
+    conv, rec = torch.arange(2 * 4 * 3.).reshape(2, 4, 3), torch.arange(2 * 1 * 2 * 2.).reshape(2, 1, 2, 2)
+    c.set_prefill(1, conv, rec.to(torch.bfloat16))
+    assert c.has_previous_state(1) and c.recurrent_states[1].dtype == torch.float32
+    c.reorder_cache(torch.tensor([1, 1, 0]))
+    assert torch.equal(c.conv_states[1], conv[[1, 1, 0]]) and torch.equal(c.recurrent_states[1], rec[[1, 1, 0]])
+    assert c.conv_states[0] is None and c.recurrent_states[2] is None
