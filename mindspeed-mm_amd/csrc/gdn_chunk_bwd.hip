@@ -265,11 +265,11 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
 // chunk_bwd_local_kernel, per (chunk, head), 4 waves: everything of the backward pass that is local to a chunk once
 // the reverse recurrence has left dS' and dV' behind.  Wave w owns the 32 K-columns [32w, 32w+32) of dQ, dK, dW and
 // the 32x32 tile (w/2, w%2) of the 64x64 intra-chunk matrices.
-//   pre-pass: R = Tm^T dV' per V block -> dv = beta R
 //   main loop over 32-column V blocks:
 //     v_new, dV', dO, S, dS' arrive in fragment order with (lane <-> V column); the contractions run over V, so each
 //     tile is turned through the matrix core (mfma_transpose) into (lane <-> token / K column, registers <-> V).
 //       ds += dO V'^T   a2 += dV' V^T   dQ += dO S^T   dK += V' dS'^T   dW += dV' S^T
+//     and one wave per block also forms R = Tm^T dV' from the tiles as they lie -> dv = beta R.
 //     All operands of a V block are copied by direct global->LDS loads (no registers in between, fragment order is
 //     exactly the layout such a load produces) into one of two stages, one block ahead of the arithmetic: tiles
 //     shared by the four waves once per workgroup, S and dS' per wave.  During the last block the idle stage
@@ -282,10 +282,33 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
 //     T ("transposed"):  pack(transpose(pack(X)))  lane <-> i, registers <-> j
 //   dQ, dK, dv leave as 16-byte row pieces.
 // ---------------------------------------------------------------------------------------------
+// The raw dO and V blocks [64 tokens][32 columns] sit in LDS with their rows 64 bytes (128 for fp32) apart, so the
+// lanes of one fragment read, one row each, would meet on 8 (4) of the 64 banks.  The 16-byte pieces of row r are
+// therefore stored permuted, piece c at position raw_piece_pos(r, c) (an involution), which spreads such a read over
+// all the banks; the copy that fills the block applies the permutation to its source addresses.
+template <typename T> __device__ __forceinline__ int raw_piece_pos(int r, int c) {
+  return sizeof(T) == 2 ? (c ^ ((r >> 2) & 3)) : (c ^ (((r >> 1) & 3) << 1));
+}
+// A-operand fragments of row r of such a block (lane <-> token r, registers <-> the 32 columns)
+template <typename T> __device__ __forceinline__ void frags_from_raw(AccB<T>& out, const T* blk, int r) {
+  const int half = (threadIdx.x & 63) >> 5;
+  const T* row = blk + r * 32;
+#pragma unroll
+  for (int kg = 0; kg < AccK<T>::kGroups; ++kg) {
+    if constexpr (sizeof(T) == 2) {
+      const u32x2 lo = *reinterpret_cast<const u32x2*>(row + raw_piece_pos<T>(r, 2 * kg) * 8 + 4 * half);
+      const u32x2 hi = *reinterpret_cast<const u32x2*>(row + raw_piece_pos<T>(r, 2 * kg + 1) * 8 + 4 * half);
+      out.f[kg] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+    } else {
+      out.f[kg] = *reinterpret_cast<const u32x4*>(row + raw_piece_pos<T>(r, 2 * kg + half) * 4);
+    }
+  }
+}
+
 template <typename T, int DK> struct BwdLocalSmem {
   // one stage, in elements: [v_new x2 | dV' x2] shared tiles, raw dO [64][32], [S | dS'] per wave, raw V [64][32]
   static constexpr int st_doraw = 4 * 1024, st_priv = 6 * 1024, st_vraw = st_priv + 4 * 2048, stage_elems = st_vraw + 64 * 32;
-  // epilogue, stage that idles during the last block: K tiles [K/32][2] | Q columns of each wave [64][32]
+  // epilogue, stage that idles during the last block: K tiles [K/32][2] | the Q^T tiles [2] of each wave
   static constexpr int ea_q = 8 * 1024;
   // epilogue, other stage: dW tiles [2][K/32] (later the store patches) | D-form tiles [4] | T-form tiles [4]
   static constexpr int eb_d = 8 * 1024, eb_t = 12 * 1024;
@@ -298,12 +321,12 @@ template <typename T, int DK> struct BwdLocalSmem {
 
 template <typename T, int DK>
 __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_local_kernel(
-    const T* __restrict__ q, const T* __restrict__ kaf, const T* __restrict__ v, const float* __restrict__ beta,
+    const T* __restrict__ qtf, const T* __restrict__ kaf, const T* __restrict__ v, const float* __restrict__ beta,
     const float* __restrict__ G, const T* __restrict__ Ai, const T* __restrict__ vf, const T* __restrict__ dvf,
     const T* __restrict__ dO, const T* __restrict__ hf, const T* __restrict__ dhf, const float* __restrict__ rstd_q,
     const float* __restrict__ rstd_k, T* dq, T* dk, T* __restrict__ dv_out, float* __restrict__ dbeta,
     float* __restrict__ dg, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N,
-    int Hqk, int Hv, int V, float scale, int hh, int64_t q_stride, TokenStrides ts) {
+    int Hqk, int Hv, int V, float scale, int hh, TokenStrides ts) {
   using SM = BwdLocalSmem<T, DK>;
   constexpr int NKT = DK / 32, VEC = Elem<T>::kVec, KG = AccK<T>::kGroups;
   static_assert(NKT <= 4, "one 32-column block of K per wave");
@@ -343,7 +366,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   // stage `buf` <- operands of V block `vblk`; every load moves 64 x 16 bytes, lane l's piece landing at +16 l
   auto issue = [&](int vblk, int buf) {
     T* st = stage0 + buf * SM::stage_elems;
-    const int64_t t2 = (ch * nblk + vblk) * 2, tk = (ch * nblk + vblk) * NKT;
+    const int64_t t2 = (ch * nblk + vblk) * 2;
 #pragma unroll
     for (int j = 0; j < 4 * KG / 4; ++j) {           // shared tiles: k-group pieces dealt round-robin to the waves
       const int piece = 4 * j + wave, tile = piece / KG, g = piece % KG;
@@ -353,21 +376,21 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
 #pragma unroll
     for (int j = 0; j < (int)sizeof(T) / 2; ++j) {   // raw dO and V blocks [64][32], rows past the end repeat the last row
       constexpr int LPR = 32 / VEC, RPP = 64 / LPR;  // lanes per row, rows per piece
-      const int piece = 4 * j + wave, row = piece * RPP + lane / LPR, cc = lane % LPR;
+      const int piece = 4 * j + wave, row = piece * RPP + lane / LPR, cc = raw_piece_pos<T>(row, lane % LPR);
       const int64_t tok = tok0 + imin(row, nvalid - 1), col = (int64_t)h * V + 32 * vblk + cc * VEC;
       load16_to_lds(dO + tok * Hv * V + col, st + SM::st_doraw + piece * 64 * VEC);
       load16_to_lds(v + tok * ts.v + col, st + SM::st_vraw + piece * 64 * VEC);
     }
     if (has_k) {
+      const int64_t tile = ((ch * nblk + vblk) * NKT + cj) * 1024;
 #pragma unroll
       for (int g = 0; g < KG; ++g) {
-        load16_to_lds(hf + (tk + cj) * 1024 + (g * 64 + lane) * VEC, st + SM::st_priv + wave * 2048 + g * 64 * VEC);
-        load16_to_lds(dhf + (tk + cj) * 1024 + (g * 64 + lane) * VEC,
-                      st + SM::st_priv + wave * 2048 + 1024 + g * 64 * VEC);
+        load16_to_lds(hf + tile + (g * 64 + lane) * VEC, st + SM::st_priv + wave * 2048 + g * 64 * VEC);
+        load16_to_lds(dhf + tile + (g * 64 + lane) * VEC, st + SM::st_priv + wave * 2048 + 1024 + g * 64 * VEC);
       }
     }
   };
-  // stage `buf` <- epilogue operands: all K tiles of the chunk (fragment order), this wave's 32 Q columns [64][32]
+  // stage `buf` <- epilogue operands: all K tiles of the chunk, this wave's 32 columns of Q^T (both in fragment order)
   auto issue_epilogue = [&](int buf) {
     T* st = stage0 + buf * SM::stage_elems;
 #pragma unroll
@@ -377,13 +400,10 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
                     st + piece * 64 * VEC);
     }
     if (has_k) {
-      constexpr int LPR = 32 / VEC, RPP = 64 / LPR;
 #pragma unroll
-      for (int piece = 0; piece < LPR; ++piece) {
-        const int row = piece * RPP + lane / LPR, cc = lane % LPR;
-        load16_to_lds(q + (tok0 + imin(row, nvalid - 1)) * q_stride + hq * DK + 32 * cj + cc * VEC,
+      for (int piece = 0; piece < 2 * KG; ++piece)
+        load16_to_lds(qtf + (((int64_t)blockIdx.x * Hqk + hq) * NKT + cj) * 2048 + (piece * 64 + lane) * VEC,
                       st + SM::ea_q + wave * 2048 + piece * 64 * VEC);
-      }
     }
   };
 #pragma unroll
@@ -410,26 +430,6 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     o.pack(mfma_transpose<T>(f, id));
     return o;
   };
-  // pre-pass: R = Tm^T dV' per 32-column V block (blocks dealt to the waves): dv = beta R.  Done before the
-  // accumulators of the main loop exist; the store patch is this wave's S / dS' slot of the stage not yet in use.
-  for (int vblk = wave; vblk < nblk; vblk += 4) {
-    AccB<T> fdv[2];
-    fdv[0].load(dvf + ((ch * nblk + vblk) * 2 + 0) * 1024);
-    fdv[1].load(dvf + ((ch * nblk + vblk) * 2 + 1) * 1024);
-    T* patch = stage0 + SM::stage_elems + SM::st_priv + wave * 2048;
-#pragma unroll
-    for (int rj = 0; rj < 2; ++rj) {
-      f32x16 R = acc_zero();
-#pragma unroll
-      for (int t = rj; t < 2; ++t) mma32_ff<T>(R, tm_t(rj, t), fdv[t]);
-      const f32x16 bsr = rows_ld(bs, 32 * rj);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) R[r] *= bsr[r];
-      acc_store_rows<T, false>(R, id, patch, dv_out + (tok0 + 32 * rj) * ts.dv + h * V + 32 * vblk, ts.dv,
-                        nvalid - 32 * rj);
-    }
-  }
-
   f32x16 ds = acc_zero(), a2 = acc_zero(), dQi[2], dKi[2], dWa[2];
 #pragma unroll
   for (int ri = 0; ri < 2; ++ri) { dQi[ri] = acc_zero(); dKi[ri] = acc_zero(); dWa[ri] = acc_zero(); }
@@ -457,7 +457,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     }
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {         // (lane <-> token, registers <-> V) from here on; dO rows have it already
-      frags_from_lds<T>(dOt[ri], st + SM::st_doraw + (32 * ri + l32) * 32);
+      frags_from_raw<T>(dOt[ri], st + SM::st_doraw, 32 * ri + l32);
       if (32 * ri + l32 >= nvalid) {
 #pragma unroll
         for (int g = 0; g < KG; ++g) dOt[ri].f[g] = u32x4{0u, 0u, 0u, 0u};
@@ -481,8 +481,27 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       dVt.pack(mfma_transpose<T>(f, id));
       if (has_k) mma32_ff<T>(dWa[ri], dVt, Sf);
       if (lower && ri == ti) {
-        frags_from_lds<T>(f, st + SM::st_vraw + (32 * tj + l32) * 32);
+        frags_from_raw<T>(f, st + SM::st_vraw, 32 * tj + l32);
         mma32_ff<T>(a2, dVt, f);
+      }
+    }
+    // dv = beta (Tm^T dV') of this V block, the blocks dealt to the waves in turn.  The dV' tiles serve as they lie in
+    // the stage, as the A operand: the product is dv^T (lane <-> token, registers <-> V column), of which every lane
+    // stores four adjacent columns at a time without a detour through LDS.
+    if ((vblk & 3) == wave) {
+#pragma unroll
+      for (int rj = 0; rj < 2; ++rj) {
+        f32x16 Rt = acc_zero();
+#pragma unroll
+        for (int t = rj; t < 2; ++t) {
+          f.load(st + (2 + t) * 1024);
+          mma32_ff<T>(Rt, f, tm_t(rj, t));
+        }
+        const float bj = bs[32 * rj + l32];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) Rt[r] *= bj;
+        if (32 * rj + l32 < nvalid)
+          acc_to_lds_t<T>(Rt, dv_out + (tok0 + 32 * rj + l32) * ts.dv + h * V + 32 * vblk, 0, 0, 0);
       }
     }
   }
@@ -505,12 +524,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       AccB<T> f;
       f.load(EA + (2 * cj + t) * 1024);
       KTf[t].pack(mfma_transpose<T>(f, id));
-      frags_from_lds<T>(f, EA + SM::ea_q + wave * 2048 + (32 * t + l32) * 32);
-      if (32 * t + l32 >= nvalid) {
-#pragma unroll
-        for (int g = 0; g < KG; ++g) f.f[g] = u32x4{0u, 0u, 0u, 0u};
-      }
-      QTf[t].pack(mfma_transpose<T>(f, id));
+      QTf[t].load(EA + SM::ea_q + wave * 2048 + t * 1024);
     }
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {         // dW = -(dV' S^T): B operand of P in registers, A operand of a1 to LDS
@@ -729,8 +743,7 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   const int64_t tok = d.tokens();
   const int nc = (int)d.max_chunks();
   const int* chunk_offsets = reinterpret_cast<const int*>(ws + L.chunk_offsets);
-  const T* qq = l2norm ? reinterpret_cast<const T*>(ws + L.qn) : (const T*)q;
-  (void)k;   // k reaches the backward kernels as the forward pass's fragment tiles
+  (void)q; (void)k;   // q and k reach the backward kernels as the forward pass's fragment tiles
   const float* G = reinterpret_cast<const float*>(ws + L.G);
   const T* Ai = reinterpret_cast<const T*>(ws + L.Ai);
   const T* AQ = reinterpret_cast<const T*>(ws + L.AQ);
@@ -756,10 +769,9 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     constexpr int smem = BwdLocalSmem<T, DK>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
     for (int hh = 0; hh < d.Hv / d.Hqk; ++hh)
-      GDN_LAUNCH(kKernBwdLocal, st, kern, dim3(nc, d.Hqk), dim3(kThreads), smem, st, qq, (const T*)KAF, (const T*)v,
+      GDN_LAUNCH(kKernBwdLocal, st, kern, dim3(nc, d.Hqk), dim3(kThreads), smem, st, QTF, (const T*)KAF, (const T*)v,
                  beta, G, Ai, VF, (const T*)DVF, (const T*)dO, HF, (const T*)DHF, rstd_q, rstd_k, (T*)dq, (T*)dk,
-                 (T*)dv, dbeta, dg, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale, hh,
-                 l2norm ? (int64_t)d.Hqk * d.K : d.strides().q, d.strides());
+                 (T*)dv, dbeta, dg, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale, hh, d.strides());
   }
   return (int)hipGetLastError();
 }

@@ -434,7 +434,8 @@ __device__ __forceinline__ int acc_row(int r) { return 8 * (r >> 2) + 4 * ((thre
 __device__ __forceinline__ int acc_col() { return threadIdx.x & 31; }
 
 // accumulator tile -> LDS, transposed: dst[(j0+j)*ld + i0 + i].  Registers 4g..4g+3 are four consecutive rows, so a
-// lane writes four contiguous elements at a time (ld must be a multiple of 4 elements).
+// lane writes four contiguous elements at a time (ld must be a multiple of 4 elements).  dst may also be global
+// memory; with ld = 0 it is the address of the lane's own row.
 template <typename T> __device__ __forceinline__ void acc_to_lds_t(const f32x16& acc, T* dst, int ld, int i0, int j0) {
   T* col = dst + (j0 + acc_col()) * ld + i0 + 4 * ((threadIdx.x & 63) >> 5);
 #pragma unroll
