@@ -318,8 +318,8 @@ def main():
                                                initial_state=hh0, output_final_state=True, use_qk_l2norm_in_kernel=True)
             torch.autograd.grad([o_], [mixed, gg, bb, hh0], [d["do"]])
 
-        def wall_ms(fn, n=10):
-            for _ in range(3):
+        def wall_ms(fn, n=10, warm=3):
+            for _ in range(warm):
                 fn()
             torch.cuda.synchronize()
             t0 = time.perf_counter()
@@ -333,6 +333,37 @@ def main():
                                            output_final_state=True, use_qk_l2norm_in_kernel=True)
         pf = wall_ms(prefill_step, 20)
         aux["forward_only"] = {"ms": round(pf, 4), "tokens_per_s": round(tokens / (pf * 1e-3), 1)}
+        zg = torch.randn(c["B"], c["T"], c["Hv"], c["V"], generator=gen).to(dev, torch.bfloat16)
+        nw = torch.ones(c["V"], device=dev, dtype=torch.bfloat16)
+
+        def prefill_norm_fused():
+            with torch.no_grad():
+                ops.chunk_gated_delta_rule_norm(d["q"], d["k"], d["v"], d["g"], d["beta"], zg, nw,
+                                                initial_state=d["h0"], output_final_state=True,
+                                                use_qk_l2norm_in_kernel=True)
+
+        def prefill_norm_separate():
+            with torch.no_grad():
+                o_, _ = ops.chunk_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], initial_state=d["h0"],
+                                                   output_final_state=True, use_qk_l2norm_in_kernel=True)
+                ops.rms_norm_gated(o_, zg, nw, 1e-6)
+        def kernel_sum_ms(fn, n=10):
+            """GPU time of one call: the library's per-kernel event timings summed (no launch gaps, no host time)."""
+            torch.cuda.synchronize()
+            lib.gdn_profile_enable(1)
+            for _ in range(n):
+                fn()
+            torch.cuda.synchronize()
+            tm = _lib.kernel_timings(lib)
+            lib.gdn_profile_enable(0)
+            return sum(ms for ms, _ in tm.values()) / n
+        # the host-side generation of the gate above leaves the GPU idle: longer warm-up before these
+        aux["forward_only_with_gated_norm"] = {
+            "separate_operators_ms": round(wall_ms(prefill_norm_separate, 20, 20), 4),
+            "norm_in_output_kernel_ms": round(wall_ms(prefill_norm_fused, 20, 20), 4),
+            "separate_operators_kernel_ms": round(kernel_sum_ms(prefill_norm_separate), 4),
+            "norm_in_output_kernel_kernel_ms": round(kernel_sum_ms(prefill_norm_fused), 4)}
+        del zg
         aux["rule_in_layer"] = {"unsplit_qkv_ms": round(wall_ms(unsplit_step), 4),
                                 "split_with_copies_ms": round(wall_ms(split_step), 4)}
         del mixed

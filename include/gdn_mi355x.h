@@ -58,6 +58,19 @@ int gdn_chunk_fwd_strided(const void* q, const void* k, const void* v, int64_t q
                           int64_t workspace_bytes, int B, int T, int N, int Hqk, int Hv, int K, int V, float scale,
                           int use_qk_l2norm, int dtype, void* stream);
 
+/* gdn_chunk_fwd_strided followed, inside its output kernel, by the layer's gated RMSNorm over head_v_dim
+ * (Qwen3_5RMSNormGated.forward, modeling_qwen3_5.py:330-349, applied to the rule's output at :897-900):
+ * y = (norm_weight * rmsnorm(o, eps)) * silu(gate), with the arithmetic and the bits of gdn_rmsnorm_gated_fwd below.
+ * gate, y [tokens, Hv, V] dense in `dtype`; norm_weight [V] in `dtype` or fp32 (weight_dtype = 0).  o (the rule's
+ * output) and rstd [tokens * Hv] fp32 are written only if non-null: a caller without a backward pass saves one write
+ * and one read of o.  V must be 64 or 128 (a workgroup of the output kernel then holds whole rows), else -3. */
+int gdn_chunk_fwd_norm_strided(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
+                               int64_t v_stride, const float* g, const float* beta, const float* initial_state,
+                               const int64_t* cu_seqlens, const void* gate, const void* norm_weight, void* o, void* y,
+                               float* rstd, float* final_state, void* workspace, int64_t workspace_bytes, int B,
+                               int T, int N, int Hqk, int Hv, int K, int V, float scale, float eps,
+                               int use_qk_l2norm, int dtype, int weight_dtype, void* stream);
+
 int gdn_chunk_bwd_strided(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
                           int64_t v_stride, const float* g, const float* beta, const float* initial_state,
                           const int64_t* cu_seqlens, const void* d_o, const float* d_final_state, void* dq, void* dk,

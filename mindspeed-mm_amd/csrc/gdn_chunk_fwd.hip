@@ -14,6 +14,7 @@
 #include "gdn_chunk.h"
 #include "gdn_common.h"
 #include "gdn_profile.h"
+#include "gdn_rmsnorm_gated.h"
 
 namespace gdn {
 
@@ -588,20 +589,36 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ?
 // ---------------------------------------------------------------------------------------------
 // chunk_out_kernel:  O = scale e^G . (Q S) + (scale Aq) V', parallel over (chunk, head, 32-column block).
 // S and V' arrive in fragment order and go from global memory straight into B-operand registers.
+// NORM: the workgroup's NW waves hold whole rows of a head (V = 32 NW) and the gated RMSNorm that follows the rule
+// in the layer (modeling_qwen3_5.py:897-900) is applied to the rows before they leave: y = norm(o) * silu(gate),
+// with the stand-alone operator's arithmetic on the same 16-byte pieces and its order of additions (pieces of a
+// row: neighbouring lanes pairwise, then the waves pairwise), so both give the same bits.  o itself and 1/rms are
+// written only on request (a backward pass needs them).
 // ---------------------------------------------------------------------------------------------
 template <typename T, int DK, int NW> struct OutSmem {
   static constexpr int LDK = lds_ld<T>(DK);
   static constexpr int off_qs = 0;
   static constexpr int off_patch = off_qs + 64 * LDK * (int)sizeof(T);
   static constexpr int off_eg = off_patch + NW * Patch<T>::kElems * (int)sizeof(T);
-  static constexpr int bytes = off_eg + 64 * 4;
+  static constexpr int off_ss = off_eg + 64 * 4;       // NORM: sums of squares [NW waves][64 rows]
+  static constexpr int bytes = off_ss + NW * 64 * 4;
 };
 
-template <typename T, int DK, int NW>
+// operands of the fused norm: gate and y [tokens, Hv, V] in T, weight [V] in TW; o_opt, rstd_opt may be null
+template <typename T, typename TW> struct OutNorm {
+  const T* gate;
+  const TW* weight;
+  T* y;
+  float* rstd_opt;
+  float eps;
+};
+
+template <typename T, int DK, int NW, bool NORM, typename TW>
 __global__ __launch_bounds__(64 * NW) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 2) void chunk_out_kernel(
     const T* __restrict__ q, const T* __restrict__ aqf, const T* __restrict__ vf, const T* __restrict__ hf,
     const float* __restrict__ G, T* __restrict__ o, const int64_t* __restrict__ cu,
-    const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V, float scale, int64_t q_stride) {
+    const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V, float scale, int64_t q_stride,
+    OutNorm<T, TW> nm) {
   using SM = OutSmem<T, DK, NW>;
   constexpr int LDK = SM::LDK, NT = 64 * NW, VEC = Elem<T>::kVec, NKT = DK / 32;
   T* Qs = reinterpret_cast<T*>(gdn_smem + SM::off_qs);
@@ -637,9 +654,7 @@ __global__ __launch_bounds__(64 * NW) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 2)
   for (int t = 0; t < 3; ++t) Af[t].pack(mfma_transpose<T>(Af[t], id));   // now (lane <-> row i, registers <-> column j)
   __syncthreads();
 
-  T* og = o + (tok0 * Hv + h) * V + v0;
-#pragma unroll
-  for (int ri = 0; ri < 2; ++ri) {
+  auto out_tile = [&](int ri) {
     f32x16 oa = acc_zero();
 #pragma unroll
     for (int kt = 0; kt < NKT; ++kt) mma32_accb<T>(oa, Qs + (32 * ri + l32) * LDK + 32 * kt, Sb[kt]);
@@ -648,7 +663,60 @@ __global__ __launch_bounds__(64 * NW) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 2)
     for (int r = 0; r < 16; ++r) oa[r] *= eg[r];
 #pragma unroll
     for (int tj = 0; tj <= ri; ++tj) mma32_ff<T>(oa, Af[ri + tj], Vb[tj]);
-    acc_store_rows<T, false>(oa, id, patch, og + (int64_t)32 * ri * Hv * V, (int64_t)Hv * V, nvalid - 32 * ri);
+    return oa;
+  };
+  if constexpr (!NORM) {
+    T* og = o + (tok0 * Hv + h) * V + v0;
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri)
+      acc_store_rows<T, false>(out_tile(ri), id, patch, og + (int64_t)32 * ri * Hv * V, (int64_t)Hv * V, nvalid - 32 * ri);
+  } else {
+    // the wave's 32 columns of a row are PPR 16-byte pieces on PPR neighbouring lanes; a lane holds PPL pieces per tile
+    constexpr int PLD = Patch<T>::kLd, PPR = 32 / VEC, PPL = PPR / 2;
+    float* ssw = reinterpret_cast<float*>(gdn_smem + SM::off_ss);
+    const int cc = lane % PPR;
+    Vec16<T> xs[2][PPL], gs[2][PPL];
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri) {
+      const f32x16 oa = out_tile(ri);
+      GDN_WAVE_LDS_SYNC();   // earlier readers of the patch are done
+      acc_to_lds_rm(oa, id, patch, PLD, 0, 0);
+      GDN_WAVE_LDS_SYNC();
+#pragma unroll
+      for (int i = 0; i < PPL; ++i) {
+        const int rowl = (lane + 64 * i) / PPR;
+        xs[ri][i] = ld16(patch + rowl * PLD + cc * VEC);
+        const float ss = lane_group_sum<PPR>(piece_sumsq<T>(xs[ri][i]));
+        if (cc == 0) ssw[wave * 64 + 32 * ri + rowl] = ss;
+      }
+    }
+    // gate and weight are requested only now, when the operands of the products no longer occupy registers
+    float w[VEC];
+    load_weight<T, TW>(w, nm.weight + v0 + cc * VEC);
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri)
+#pragma unroll
+      for (int i = 0; i < PPL; ++i) {
+        const int row = 32 * ri + (lane + 64 * i) / PPR;
+        gs[ri][i] = row < nvalid ? ld16(nm.gate + ((tok0 + row) * Hv + h) * V + v0 + cc * VEC) : zero16<T>();
+      }
+    __syncthreads();
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri)
+#pragma unroll
+      for (int i = 0; i < PPL; ++i) {
+        const int row = 32 * ri + (lane + 64 * i) / PPR;
+        float ss = ssw[row] + ssw[64 + row];
+        if constexpr (NW == 4) ss += ssw[128 + row] + ssw[192 + row];
+        const float rstd = rsqrtf(ss * (1.f / (32 * NW)) + nm.eps);
+        if (row < nvalid) {
+          const int64_t at = ((tok0 + row) * Hv + h) * V + v0 + cc * VEC;
+          const Vec16<T> yv = rmsnorm_gated_piece<T, TW>(xs[ri][i], gs[ri][i], w, rstd);
+          __builtin_nontemporal_store(yv.raw, reinterpret_cast<u32x4*>(nm.y + at));
+          if (o != nullptr) st16(o + at, xs[ri][i]);
+          if (nm.rstd_opt != nullptr && wave == 0 && cc == 0) nm.rstd_opt[(tok0 + row) * Hv + h] = rstd;
+        }
+      }
   }
 }
 
@@ -660,10 +728,21 @@ template <typename K> static int set_lds(K kernel, int bytes) {
                                   bytes);
 }
 
+// the gated RMSNorm applied by the output kernel (null y: none); weight in fp32 or in the rule's dtype
+struct FwdNorm {
+  const void* gate;
+  const void* weight;
+  void* y;
+  float* rstd;
+  float eps;
+  bool weight_fp32;
+};
+
 template <typename T, int DK, int BVP, int NW, int NWS, int NLS, int STAGES>
 static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const void* q, const void* k, const void* v,
                             const float* g, const float* beta, const float* h0, const int64_t* cu, void* o, float* ht,
-                            unsigned char* ws, float scale, int l2norm, bool with_backward, hipStream_t st) {
+                            unsigned char* ws, float scale, int l2norm, bool with_backward, const FwdNorm& fn,
+                            hipStream_t st) {
   const int64_t tok = d.tokens();
   const int nc = (int)d.max_chunks();
   int* chunk_offsets = reinterpret_cast<int*>(ws + L.chunk_offsets);
@@ -699,13 +778,26 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
                (const T*)KTF, (const T*)W, (const T*)UF, (const float*)G, h0, ht, VF, HF, cu,
                (const int*)chunk_offsets, d.T, d.Hqk, d.Hv, d.V);
   }
-  {
-    auto kern = chunk_out_kernel<T, DK, NW>;
+  auto launch_out = [&](auto kern, auto nm) -> int {
     constexpr int smem = OutSmem<T, DK, NW>::bytes;
     if (int e = set_lds(kern, smem)) return e;
     GDN_LAUNCH(kKernOut, st, kern, dim3(nc, d.Hv, d.V / (32 * NW)), dim3(64 * NW), smem, st, l2norm ? (const T*)qn : qq,
                (const T*)AQ, (const T*)VF, (const T*)HF, (const float*)G, (T*)o, cu, (const int*)chunk_offsets, d.T, d.N, d.Hqk,
-               d.Hv, d.V, scale, l2norm ? (int64_t)d.Hqk * d.K : d.strides().q);
+               d.Hv, d.V, scale, l2norm ? (int64_t)d.Hqk * d.K : d.strides().q, nm);
+    return 0;
+  };
+  if (fn.y == nullptr) {
+    if (int e = launch_out(chunk_out_kernel<T, DK, NW, false, T>, OutNorm<T, T>{})) return e;
+  } else if (d.V != 32 * NW) {
+    return -3;   // a workgroup of the output kernel must hold whole rows
+  } else if (fn.weight_fp32) {
+    if (int e = launch_out(chunk_out_kernel<T, DK, NW, true, float>,
+                           OutNorm<T, float>{(const T*)fn.gate, (const float*)fn.weight, (T*)fn.y, fn.rstd, fn.eps}))
+      return e;
+  } else {
+    if (int e = launch_out(chunk_out_kernel<T, DK, NW, true, T>,
+                           OutNorm<T, T>{(const T*)fn.gate, (const T*)fn.weight, (T*)fn.y, fn.rstd, fn.eps}))
+      return e;
   }
   return (int)hipGetLastError();
 }
@@ -735,17 +827,20 @@ extern "C" int64_t gdn_chunk_workspace_bytes(int B, int T, int N, int Hqk, int H
   return with_backward ? w.total_bytes : w.fwd_bytes;
 }
 
-extern "C" int gdn_chunk_fwd_strided(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
-                                     int64_t v_stride, const float* g, const float* beta, const float* initial_state,
-                                     const int64_t* cu_seqlens, void* o, float* final_state, void* workspace,
-                                     int64_t workspace_bytes, int B, int T, int N, int Hqk, int Hv, int K, int V,
-                                     float scale, int use_qk_l2norm, int dtype, void* stream) {
-  using namespace gdn;
-  if (!q || !k || !v || !g || !beta || !o || !workspace) return -1;
+namespace gdn {
+static int chunk_fwd_entry(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
+                           int64_t v_stride, const float* g, const float* beta, const float* initial_state,
+                           const int64_t* cu_seqlens, void* o, float* final_state, void* workspace,
+                           int64_t workspace_bytes, int B, int T, int N, int Hqk, int Hv, int K, int V, float scale,
+                           int use_qk_l2norm, int dtype, const FwdNorm& fn, void* stream) {
+  if (!q || !k || !v || !g || !beta || !workspace) return -1;
+  if (fn.y == nullptr ? !o : (!fn.gate || !fn.weight)) return -1;
   ChunkDims d{B, T, N, Hqk, Hv, K, V, cu_seqlens != nullptr};
   d.ts = {q_stride, k_stride, v_stride, 0, 0, 0};
   if (int e = chunk_check_dims(d, dtype)) return e;
-  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o) & 15) return -6;
+  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o | (uintptr_t)fn.y | (uintptr_t)fn.gate |
+       (uintptr_t)fn.weight) & 15)
+    return -6;
   ChunkDims dl = d;
   dl.varlen = true;  // one layout for both modes (the packed bound is the larger)
   const ChunkWorkspace L = chunk_workspace_layout(dl, dtype == 0 ? 4 : 2);
@@ -756,7 +851,7 @@ extern "C" int gdn_chunk_fwd_strided(const void* q, const void* k, const void* v
   hipStream_t st = (hipStream_t)stream;
 #define GDN_FWD(T_, DK_, BVP_, NW_, NWS_, NLS_, ST_)                                                                        \
   return chunk_fwd_launch<T_, DK_, BVP_, NW_, NWS_, NLS_, ST_>(d, L, q, k, v, g, beta, initial_state, cu_seqlens, o, final_state, \
-                                                   ws, scale, use_qk_l2norm, with_bwd, st)
+                                                   ws, scale, use_qk_l2norm, with_bwd, fn, st)
   const bool wide = (V % 128 == 0);
   const bool solo = one_slab_per_workgroup(d, device_compute_units());
   if (dtype == 1) {
@@ -772,6 +867,32 @@ extern "C" int gdn_chunk_fwd_strided(const void* q, const void* k, const void* v
     GDN_FWD(float, 64, 64, 2, 2, 2, 2);
   }
 #undef GDN_FWD
+}
+}  // namespace gdn
+
+extern "C" int gdn_chunk_fwd_strided(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
+                                     int64_t v_stride, const float* g, const float* beta, const float* initial_state,
+                                     const int64_t* cu_seqlens, void* o, float* final_state, void* workspace,
+                                     int64_t workspace_bytes, int B, int T, int N, int Hqk, int Hv, int K, int V,
+                                     float scale, int use_qk_l2norm, int dtype, void* stream) {
+  return gdn::chunk_fwd_entry(q, k, v, q_stride, k_stride, v_stride, g, beta, initial_state, cu_seqlens, o, final_state,
+                              workspace, workspace_bytes, B, T, N, Hqk, Hv, K, V, scale, use_qk_l2norm, dtype,
+                              gdn::FwdNorm{}, stream);
+}
+
+extern "C" int gdn_chunk_fwd_norm_strided(const void* q, const void* k, const void* v, int64_t q_stride,
+                                          int64_t k_stride, int64_t v_stride, const float* g, const float* beta,
+                                          const float* initial_state, const int64_t* cu_seqlens, const void* gate,
+                                          const void* norm_weight, void* o, void* y, float* rstd, float* final_state,
+                                          void* workspace, int64_t workspace_bytes, int B, int T, int N, int Hqk,
+                                          int Hv, int K, int V, float scale, float eps, int use_qk_l2norm, int dtype,
+                                          int weight_dtype, void* stream) {
+  if (!y) return -1;
+  if (weight_dtype != 0 && weight_dtype != dtype) return -4;
+  if (V != 64 && V != 128) return -3;
+  return gdn::chunk_fwd_entry(q, k, v, q_stride, k_stride, v_stride, g, beta, initial_state, cu_seqlens, o, final_state,
+                              workspace, workspace_bytes, B, T, N, Hqk, Hv, K, V, scale, use_qk_l2norm, dtype,
+                              gdn::FwdNorm{gate, norm_weight, y, rstd, eps, weight_dtype == 0}, stream);
 }
 
 extern "C" int gdn_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const float* beta,

@@ -12,10 +12,9 @@
 // partial row per workgroup; rmsnorm_gated_dw_reduce_kernel adds the partials in a fixed order (bitwise reproducible).
 #include "gdn_common.h"
 #include "gdn_profile.h"
+#include "gdn_rmsnorm_gated.h"
 
 namespace gdn {
-
-__device__ __forceinline__ float sigmoid_(float p) { return 1.f / (1.f + __expf(-p)); }
 
 template <int LPR> __device__ __forceinline__ float row_lanes_sum(float v) {
   if constexpr (LPR <= 32) {
@@ -23,21 +22,6 @@ template <int LPR> __device__ __forceinline__ float row_lanes_sum(float v) {
   } else {
     v = lane_group_sum<32>(v);
     return v + __shfl_xor(v, 32);
-  }
-}
-
-// round to T and back: the reference casts to the input dtype between the steps
-template <typename T> __device__ __forceinline__ float round_to(float x) { return Elem<T>::to_f(Elem<T>::from_f(x)); }
-
-template <typename T, typename TW> __device__ __forceinline__ void load_weight(float* w, const TW* p) {
-  constexpr int V = Elem<T>::kVec;
-  if constexpr (sizeof(TW) == sizeof(T)) {
-    const Vec16<TW> v = ld16(p);
-#pragma unroll
-    for (int e = 0; e < V; ++e) w[e] = v.get(e);
-  } else {
-#pragma unroll
-    for (int e = 0; e < V; ++e) w[e] = Elem<TW>::to_f(p[e]);
   }
 }
 
@@ -56,19 +40,9 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_gated_fwd_kernel(const T* __
     const bool ok = row < rows;      // uniform trip count: every lane takes part in the row sums
     const Vec16<T> xv = ok ? ld16(x + row * N + c * V) : zero16<T>();
     const Vec16<T> gv = ok ? ld16(gate + row * N + c * V) : zero16<T>();
-    float ss = 0.f;
-#pragma unroll
-    for (int e = 0; e < V; ++e) { const float f = xv.get(e); ss += f * f; }
-    ss = row_lanes_sum<LPR>(ss);
+    const float ss = row_lanes_sum<LPR>(piece_sumsq<T>(xv));
     const float rstd = rsqrtf(ss * (1.f / N) + eps);
-    Vec16<T> out = zero16<T>();
-#pragma unroll
-    for (int e = 0; e < V; ++e) {
-      const float xn = round_to<T>(xv.get(e) * rstd);
-      const float t = sizeof(TW) == sizeof(T) ? round_to<T>(w[e] * xn) : w[e] * xn;
-      const float gf = gv.get(e);
-      out.set(e, t * (gf * sigmoid_(gf)));
-    }
+    const Vec16<T> out = rmsnorm_gated_piece<T, TW>(xv, gv, w, rstd);
     if (ok) {
       __builtin_nontemporal_store(out.raw, reinterpret_cast<u32x4*>(y + row * N + c * V));
       if (c == 0) rstd_out[row] = rstd;

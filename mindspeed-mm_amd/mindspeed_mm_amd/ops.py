@@ -49,10 +49,48 @@ class GdnOps:
     def _f32(t):
         return None if t is None else t.detach().to(torch.float32).contiguous()
 
+    @staticmethod
+    def _no_grad_views(*tensors):
+        """Under torch.no_grad() a tensor still reports requires_grad, and an autograd function would take that as a
+        backward pass to prepare for (extra operands written by the forward kernels): hand it detached views then."""
+        if torch.is_grad_enabled():
+            return tensors
+        return tuple(None if t is None else t.detach() for t in tensors)
+
     # ------------------------------------------------------------------ chunked rule
     def chunk_gated_delta_rule(self, q, k, v, g, beta, scale=None, initial_state=None, output_final_state=False,
                                use_qk_l2norm_in_kernel=False, cu_seqlens=None, chunk_size=64, head_first=False,
                                skip_recompute=False):
+        scale = self._check_chunk_args(q, k, v, g, beta, scale, initial_state, cu_seqlens, chunk_size, head_first)
+        q, k, v, g, beta, initial_state = self._no_grad_views(q, k, v, g, beta, initial_state)
+        return _ChunkGatedDeltaRule.apply(q, k, v, g, beta, float(scale), initial_state, bool(output_final_state),
+                                          cu_seqlens, bool(use_qk_l2norm_in_kernel), self)
+
+    def chunk_gated_delta_rule_norm(self, q, k, v, g, beta, gate, norm_weight, eps=1e-6, scale=None,
+                                    initial_state=None, output_final_state=False, use_qk_l2norm_in_kernel=False,
+                                    cu_seqlens=None):
+        """The rule followed by the layer's gated RMSNorm over head_v_dim (modeling_qwen3_5.py:886-900:
+        `core_attn_out = self.norm(core_attn_out.reshape(-1, head_v_dim), z.reshape(-1, head_v_dim))`) in one pass:
+        the output kernel normalises and gates the rows before they leave, so `o` is neither written nor read again
+        when no gradient is needed.  Returns (y [B,T,Hv,V], final_state); same bits as the two operators in sequence.
+        head_v_dim must be 64 or 128."""
+        scale = self._check_chunk_args(q, k, v, g, beta, scale, initial_state, cu_seqlens, 64, False)
+        V = v.shape[-1]
+        if V not in (64, 128):
+            raise ValueError(f"the fused norm needs head_v_dim 64 or 128, got {V}; use the two operators in sequence")
+        if gate.numel() != v.numel():
+            raise ValueError(f"gate has {gate.numel()} elements, expected {v.numel()} (one per element of v)")
+        if tuple(norm_weight.shape) != (V,):
+            raise ValueError(f"norm_weight shape {tuple(norm_weight.shape)}, expected ({V},)")
+        self._need(gate, norm_weight)
+        q, k, v, g, beta, gate, norm_weight, initial_state = self._no_grad_views(q, k, v, g, beta, gate, norm_weight,
+                                                                                 initial_state)
+        return _ChunkGatedDeltaRuleNorm.apply(q, k, v, g, beta, gate, norm_weight, float(eps), float(scale),
+                                              initial_state, bool(output_final_state), cu_seqlens,
+                                              bool(use_qk_l2norm_in_kernel), self)
+
+    def _check_chunk_args(self, q, k, v, g, beta, scale, initial_state, cu_seqlens, chunk_size, head_first):
+        """Argument checks of chunk_gated_delta_rule (chunk_gated_delta_rule.py:379-414); returns the scale."""
         if q.dtype != k.dtype or k.dtype != v.dtype:
             raise ValueError(
                 f"q current type is {q.dtype} , k current type is {k.dtype} ,v current type is {v.dtype} , "
@@ -87,8 +125,7 @@ class GdnOps:
         if scale is None:
             scale = k.shape[-1] ** -0.5
         self._need(q, k, v, g, beta, initial_state, cu_seqlens)
-        return _ChunkGatedDeltaRule.apply(q, k, v, g, beta, float(scale), initial_state, bool(output_final_state),
-                                          cu_seqlens, bool(use_qk_l2norm_in_kernel), self)
+        return scale
 
     def chunk_gated_delta_rule_qkv(self, mixed_qkv, g, beta, num_k_heads, num_v_heads, head_k_dim, head_v_dim,
                                    scale=None, initial_state=None, output_final_state=False,
@@ -114,6 +151,7 @@ class GdnOps:
         if scale is None:
             scale = head_k_dim ** -0.5
         self._need(mixed_qkv, g, beta, initial_state, cu_seqlens)
+        mixed_qkv, g, beta, initial_state = self._no_grad_views(mixed_qkv, g, beta, initial_state)
         return _ChunkGatedDeltaRuleQKV.apply(mixed_qkv, g, beta, int(num_k_heads), int(num_v_heads), int(head_k_dim),
                                              int(head_v_dim), float(scale), initial_state, bool(output_final_state),
                                              cu_seqlens, bool(use_qk_l2norm_in_kernel), self)
@@ -342,6 +380,82 @@ class _ChunkGatedDeltaRule(torch.autograd.Function):
                 None)
 
 
+class _ChunkGatedDeltaRuleNorm(torch.autograd.Function):
+    """Rule + gated RMSNorm in one forward pass; the backward pass is the two operators' backward passes in turn
+    (the forward then also writes `o` and 1/rms, which they need)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, g, beta, gate, norm_weight, eps, scale, initial_state, output_final_state, cu_seqlens,
+                use_qk_l2norm_in_kernel, ops):
+        lib = ops.lib
+        B, T, Hqk, K = q.shape
+        Hv, V = v.shape[2], v.shape[3]
+        N = (len(cu_seqlens) - 1) if cu_seqlens is not None else B
+        rule_grad = any(ctx.needs_input_grad[:5]) or (initial_state is not None and ctx.needs_input_grad[9])
+        need_grad = rule_grad or ctx.needs_input_grad[5] or ctx.needs_input_grad[6]
+        (qc, sq), (kc, sk), (vc, sv) = _token_view(q), _token_view(k), _token_view(v)
+        g32, b32, h0 = ops._f32(g), ops._f32(beta), ops._f32(initial_state)
+        cu = _i64(cu_seqlens, q)
+        dt = q.dtype
+        code = DTYPE_CODE[dt]
+        w_dt = dt if norm_weight.dtype == dt else torch.float32
+        gc = gate.detach().to(dt).contiguous().view(B, T, Hv, V)
+        wc = norm_weight.detach().to(w_dt).contiguous()
+        ws, nbytes = _chunk_workspace(lib, q.device, B, T, N, Hqk, Hv, K, V, code, rule_grad)
+        y = torch.empty(B, T, Hv, V, dtype=dt, device=v.device)
+        o = torch.empty(B, T, Hv, V, dtype=dt, device=v.device) if need_grad else None
+        rstd = torch.empty(B * T * Hv, dtype=torch.float32, device=v.device) if need_grad else None
+        ht = torch.empty(N, Hv, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
+        rc = lib.gdn_chunk_fwd_norm_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(b32), ptr(h0),
+                                            ptr(cu), ptr(gc), ptr(wc), ptr(o), ptr(y), ptr(rstd), ptr(ht), ptr(ws),
+                                            nbytes, B, T, N, Hqk, Hv, K, V, scale, eps,
+                                            int(use_qk_l2norm_in_kernel), code, DTYPE_CODE[w_dt], lib.stream())
+        lib.check(rc, "gdn_chunk_fwd_norm_strided")
+        if need_grad:
+            ctx.save_for_backward(qc, kc, vc, g32, b32, h0, cu, ws if rule_grad else None, o, gc, wc, rstd)
+            ctx.meta = (B, T, N, Hqk, Hv, K, V, scale, int(use_qk_l2norm_in_kernel), code, nbytes, g.dtype,
+                        beta.dtype, None if initial_state is None else initial_state.dtype, sq, sk, sv, w_dt,
+                        norm_weight.dtype, gate.dtype, gate.shape, rule_grad)
+            ctx.ops = ops
+        return y, ht
+
+    @staticmethod
+    def backward(ctx, dy, dht):
+        qc, kc, vc, g32, b32, h0, cu, ws, o, gc, wc, rstd = ctx.saved_tensors
+        (B, T, N, Hqk, Hv, K, V, scale, l2, code, nbytes, g_dt, b_dt, h_dt, sq, sk, sv, w_dt, weight_dt, gate_dt,
+         gate_shape, rule_grad) = ctx.meta
+        lib = ctx.ops.lib
+        dev, dt = qc.device, qc.dtype
+        rows = B * T * Hv
+        dyc = dy.to(dt).contiguous()
+        do = torch.empty_like(o)
+        dgate = torch.empty_like(o)
+        dw = torch.empty(V, dtype=torch.float32, device=dev)
+        nb = lib.gdn_rmsnorm_gated_bwd_workspace_bytes(rows, V)
+        nws = torch.empty(nb, dtype=torch.uint8, device=dev)
+        rc = lib.gdn_rmsnorm_gated_bwd(ptr(o), ptr(gc), ptr(wc), ptr(rstd), ptr(dyc), ptr(do), ptr(dgate), ptr(dw),
+                                       ptr(nws), nb, rows, V, code, DTYPE_CODE[w_dt], lib.stream())
+        lib.check(rc, "gdn_rmsnorm_gated_bwd")
+        dq = dk = dv = dg = db = dh0 = None
+        if rule_grad:
+            dht = ctx.ops._f32(dht)
+            dq = torch.empty(B, T, Hqk, K, dtype=dt, device=dev)
+            dk = torch.empty(B, T, Hqk, K, dtype=dt, device=dev)
+            dv = torch.empty(B, T, Hv, V, dtype=dt, device=dev)
+            dg = torch.empty(B, T, Hv, dtype=torch.float32, device=dev)
+            db = torch.empty(B, T, Hv, dtype=torch.float32, device=dev)
+            dh0 = torch.empty(N, Hv, K, V, dtype=torch.float32, device=dev) if h0 is not None else None
+            rc = lib.gdn_chunk_bwd_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(b32), ptr(h0),
+                                           ptr(cu), ptr(do), ptr(dht), ptr(dq), ptr(dk), ptr(dv), 0, 0, 0, ptr(dg),
+                                           ptr(db), ptr(dh0), ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale, l2,
+                                           code, lib.stream())
+            lib.check(rc, "gdn_chunk_bwd_strided")
+            dg, db = dg.to(g_dt), db.to(b_dt)
+            dh0 = None if dh0 is None else dh0.to(h_dt)
+        return (dq, dk, dv, dg, db, dgate.view(gate_shape).to(gate_dt), dw.to(weight_dt), None, None, dh0, None,
+                None, None, None)
+
+
 class _ChunkGatedDeltaRuleQKV(torch.autograd.Function):
     """The rule on the convolution's output as it is: q, k, v are the column ranges [0, Hqk K), [Hqk K, 2 Hqk K),
     [2 Hqk K, 2 Hqk K + Hv V) of mixed_qkv [B,T,D] (the split of modeling_qwen3_5.py:818-831), read in place; the
@@ -559,6 +673,12 @@ def chunk_gated_delta_rule(q, k, v, g, beta, scale=None, initial_state=None, out
 
 
 @torch.compiler.disable
+def chunk_gated_delta_rule_norm(q, k, v, g, beta, gate, norm_weight, eps=1e-6, scale=None, initial_state=None,
+                                output_final_state=False, use_qk_l2norm_in_kernel=False, cu_seqlens=None):
+    return _default_ops().chunk_gated_delta_rule_norm(q, k, v, g, beta, gate, norm_weight, eps, scale, initial_state,
+                                                      output_final_state, use_qk_l2norm_in_kernel, cu_seqlens)
+
+
 def chunk_gated_delta_rule_qkv(mixed_qkv, g, beta, num_k_heads, num_v_heads, head_k_dim, head_v_dim, scale=None,
                                initial_state=None, output_final_state=False, use_qk_l2norm_in_kernel=False,
                                cu_seqlens=None):

@@ -190,6 +190,63 @@ def check_chunk_qkv(ops, device, B, T, Hqk, Hv, K, V, dtype, l2=True, cu=None, b
     return errs
 
 
+def check_chunk_norm(ops, device, B, T, Hqk, Hv, K, V, dtype, l2=True, cu=None, backward=True, weight_dtype=None,
+                     seed=0, wrap=lambda t: t, **recipe):
+    """Rule + gated RMSNorm in one pass: bit for bit against the two operators in sequence (outputs and every
+    gradient), and against the oracle's rule followed by the oracle's norm.  The norm divides by the row's rms, so an
+    absolute error e on o becomes e / rms on y: the bar on y is the bar on o over the smallest rms of the reference
+    rows (times the largest |weight silu(gate)|), plus the norm's own rounding."""
+    N = (len(cu) - 1) if cu is not None else B
+    x = gdn_inputs(B, T, Hqk, Hv, K, V, dtype, seed=seed, N=N, l2norm_in_kernel=l2, **recipe)
+    gen = torch.Generator().manual_seed(seed + 77)
+    weight_dtype = weight_dtype or dtype
+    z = (1.5 * torch.randn(B, T, Hv * V, generator=gen)).to(dtype)        # the layer's z: [B, T, Hv * V]
+    w = (1.0 + 0.2 * torch.randn(V, generator=gen)).to(weight_dtype)
+    dy = torch.randn(B, T, Hv, V, generator=gen).to(dtype)
+    dev = {n: wrap(t.to(device)) for n, t in x.items()}
+    cu_t = torch.tensor(cu, dtype=torch.int64, device=device) if cu is not None else None
+    names = ("q", "k", "v", "g", "beta", "h0")
+
+    def leaves():
+        L = {n: dev[n].clone().requires_grad_(backward) for n in names}
+        L["z"] = wrap(z.to(device)).clone().requires_grad_(backward)
+        L["w"] = wrap(w.to(device)).clone().requires_grad_(backward)
+        return L
+    A, Bc = leaves(), leaves()
+    y, ht = ops.chunk_gated_delta_rule_norm(A["q"], A["k"], A["v"], A["g"], A["beta"], A["z"], A["w"], eps=1e-6,
+                                            initial_state=A["h0"], output_final_state=True,
+                                            use_qk_l2norm_in_kernel=l2, cu_seqlens=cu_t)
+    o2, ht2 = ops.chunk_gated_delta_rule(Bc["q"], Bc["k"], Bc["v"], Bc["g"], Bc["beta"], initial_state=Bc["h0"],
+                                         output_final_state=True, use_qk_l2norm_in_kernel=l2, cu_seqlens=cu_t)
+    y2 = ops.rms_norm_gated(o2.reshape(-1, V), Bc["z"].reshape(-1, V), Bc["w"], 1e-6).view(B, T, Hv, V)
+    assert y.shape == (B, T, Hv, V) and y.dtype == dtype
+    assert torch.equal(y, y2), "fused norm differs from the two operators in sequence"
+    assert torch.equal(ht, ht2)
+    if not backward:    # without gradients the fused pass writes no o: check that path too
+        with torch.no_grad():
+            y3, _ = ops.chunk_gated_delta_rule_norm(dev["q"], dev["k"], dev["v"], dev["g"], dev["beta"],
+                                                    wrap(z.to(device)), wrap(w.to(device)), initial_state=dev["h0"],
+                                                    use_qk_l2norm_in_kernel=l2, cu_seqlens=cu_t)
+        assert torch.equal(y3, y)
+    ro, rht = O.chunk_gated_delta_rule_ref(x["q"].float(), x["k"].float(), x["v"].float(), x["g"], x["beta"],
+                                           initial_state=x["h0"], output_final_state=True,
+                                           use_qk_l2norm_in_kernel=l2, cu_seqlens=cu)
+    ry = O.rms_norm_gated_ref(ro.reshape(-1, V), z.float().reshape(-1, V), w.float(), 1e-6).view(B, T, Hv, V)
+    rms = ro.pow(2).mean(-1).add(1e-6).sqrt().min().item()
+    amp = (w.float().abs().max() * (z.float() * torch.sigmoid(z.float())).abs().max()).item() / rms
+    o_bar = BF16_ABS_O if dtype == torch.bfloat16 else 1e-4 * ro.abs().max().item()
+    half = dtype == torch.bfloat16
+    # elementwise |err| <= abs_tol + rtol |ref| in both precisions (torch.bfloat16 selects that form of the check)
+    errs = {"y": _err("y", y, ry, torch.bfloat16, o_bar * amp + (2e-2 if half else 1e-5), rtol=1e-2 if half else 1e-4)}
+    if backward:
+        ((y.float() * wrap(dy.to(device)).float()).sum() + (ht * dev["dht"]).sum()).backward()
+        ((y2.float() * wrap(dy.to(device)).float()).sum() + (ht2 * dev["dht"]).sum()).backward()
+        for n in names + ("z", "w"):
+            assert A[n].grad is not None and A[n].grad.dtype == A[n].dtype, n
+            assert torch.equal(A[n].grad, Bc[n].grad), f"gradient of {n} differs from the two operators in sequence"
+    return errs
+
+
 def check_gdn_gates(ops, device, shape, Hv, dtype, param_dtype=None, seed=0, backward=True, wrap=lambda t: t):
     """Gate recipe against the oracle on the same (dtype-valued) inputs.  g is fp32 on both sides (relative 1e-4 of
     the largest value, the fp32 bar); beta and the gradients in half precision carry one rounding to bf16."""

@@ -89,6 +89,17 @@ def test_chunk_on_unsplit_qkv(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu, pad):
     P.check_chunk_qkv(ops, "cpu", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu, pad=pad, wrap=guarded, h0_std=0.1)
 
 
+@pytest.mark.parametrize("dtype,B,T,Hqk,Hv,K,V,l2,cu,wdt,bwd", [
+    (BF, 1, 100, 1, 2, 64, 128, True, None, None, True),
+    (BF, 1, 140, 2, 2, 128, 64, False, [0, 5, 70, 71, 140], torch.float32, True),
+    (F32, 1, 70, 1, 1, 64, 64, True, None, None, True),
+    (BF, 2, 64, 1, 2, 64, 128, True, None, None, False),
+])
+def test_chunk_with_fused_norm(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu, wdt, bwd):
+    P.check_chunk_norm(ops, "cpu", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu, weight_dtype=wdt, backward=bwd,
+                       wrap=guarded, h0_std=0.1)
+
+
 @pytest.mark.parametrize("dtype,shape,Hv,pdt", [
     (F32, (2, 37), 6, None), (BF, (1, 300), 32, None), (BF, (3, 5), 48, torch.float32), (F32, (1,), 256, None),
     (BF, (1100,), 4, None),

@@ -130,6 +130,29 @@ def test_chunk_on_unsplit_qkv(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu, pad):
     P.check_chunk_qkv(ops, "cuda", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu, pad=pad, h0_std=0.1)
 
 
+@pytest.mark.parametrize("dtype,B,T,Hqk,Hv,K,V,l2,cu,wdt,bwd", [
+    (BF, 2, 200, 2, 4, 128, 128, True, None, None, True),
+    (BF, 1, 512, 4, 8, 128, 128, True, [0, 100, 101, 512], torch.float32, True),
+    (BF, 1, 140, 2, 2, 64, 64, False, [0, 5, 70, 71, 140], None, True),
+    (F32, 1, 100, 1, 2, 64, 128, True, None, None, True),
+    (F32, 1, 130, 1, 1, 128, 64, True, None, None, False),
+    (BF, 2, 1024, 4, 8, 128, 128, True, None, None, False),
+])
+def test_chunk_with_fused_norm(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu, wdt, bwd):
+    print(f"chunk+norm {dtype} B{B} T{T} Hqk{Hqk} Hv{Hv} K{K} V{V} l2={l2} varlen={cu is not None} wdt={wdt} bwd={bwd}",
+          flush=True)
+    P.check_chunk_norm(ops, "cuda", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu, weight_dtype=wdt, backward=bwd,
+                       h0_std=0.1)
+
+
+def test_fused_norm_rejects_other_head_dims(ops):
+    q = torch.randn(1, 64, 1, 64, device="cuda", dtype=BF)
+    v = torch.randn(1, 64, 1, 256, device="cuda", dtype=BF)
+    g, b = -torch.rand(1, 64, 1, device="cuda"), torch.rand(1, 64, 1, device="cuda")
+    with pytest.raises(ValueError):
+        ops.chunk_gated_delta_rule_norm(q, q, v, g, b, torch.randn_like(v), torch.ones(256, device="cuda", dtype=BF))
+
+
 def test_chunk_rejects_bad_strides(ops):
     """A token stride that breaks 16-byte alignment cannot be read in place: the op copies; the C ABI refuses."""
     B, T, H, K = 1, 64, 1, 64
@@ -254,3 +277,17 @@ def test_chunk_random_shapes(ops, seed):
     dtype, B, T, Hqk, Hv, K, V, l2, cu = _random_case(seed)
     print(f"chunk random {seed}: {dtype} B{B} T{T} Hqk{Hqk} Hv{Hv} K{K} V{V} l2={l2} cu={cu}", flush=True)
     P.check_chunk(ops, "cuda", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu, backward=True, h0_std=0.1, seed=seed)
+
+
+def test_no_grad_forward_prepares_no_backward(ops):
+    """Under torch.no_grad() inputs that require grad must not make the forward kernels write backward operands:
+    the result is the same and nothing is attached to the graph."""
+    x = P.gdn_inputs(1, 200, 2, 4, 128, 128, BF, seed=3)
+    d = {n: t.cuda().requires_grad_(t.is_floating_point()) for n, t in x.items()}
+    o1, h1 = ops.chunk_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], initial_state=d["h0"],
+                                        output_final_state=True, use_qk_l2norm_in_kernel=True)
+    with torch.no_grad():
+        o2, h2 = ops.chunk_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], initial_state=d["h0"],
+                                            output_final_state=True, use_qk_l2norm_in_kernel=True)
+    assert o1.requires_grad and not o2.requires_grad and o2.grad_fn is None
+    assert torch.equal(o1, o2) and torch.equal(h1, h2)
