@@ -269,7 +269,7 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
 //     v_new, dV', dO, S, dS' arrive in fragment order with (lane <-> V column); the contractions run over V, so each
 //     tile is turned through the matrix core (mfma_transpose) into (lane <-> token / K column, registers <-> V).
 //       ds += dO V'^T   a2 += dV' V^T   dQ += dO S^T   dK += V' dS'^T   dW += dV' S^T
-//     and one wave per block also forms R = Tm^T dV' from the tiles as they lie -> dv = beta R.
+//     and two waves per block also form R = Tm^T dV' from the tiles as they lie -> dv = beta R.
 //     All operands of a V block are copied by direct global->LDS loads (no registers in between, fragment order is
 //     exactly the layout such a load produces) into one of two stages, one block ahead of the arithmetic: tiles
 //     shared by the four waves once per workgroup, S and dS' per wave.  During the last block the idle stage
@@ -485,24 +485,24 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
         mma32_ff<T>(a2, dVt, f);
       }
     }
-    // dv = beta (Tm^T dV') of this V block, the blocks dealt to the waves in turn.  The dV' tiles serve as they lie in
+    // dv = beta (Tm^T dV') of this V block.  The dV' tiles serve as they lie in
     // the stage, as the A operand: the product is dv^T (lane <-> token, registers <-> V column), of which every lane
     // stores four adjacent columns at a time without a detour through LDS.
-    if ((vblk & 3) == wave) {
-#pragma unroll
-      for (int rj = 0; rj < 2; ++rj) {
-        f32x16 Rt = acc_zero();
-#pragma unroll
-        for (int t = rj; t < 2; ++t) {
-          f.load(st + (2 + t) * 1024);
-          mma32_ff<T>(Rt, f, tm_t(rj, t));
-        }
-        const float bj = bs[32 * rj + l32];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) Rt[r] *= bj;
-        if (32 * rj + l32 < nvalid)
-          acc_to_lds_t<T>(Rt, dv_out + (tok0 + 32 * rj + l32) * ts.dv + h * V + 32 * vblk, 0, 0, 0);
+    const int job = (wave - 2 * vblk) & 3;   // the two token halves of a block go to two waves, rotating with the block
+    if (job < 2) {
+      const int rj = job;
+      f32x16 Rt = acc_zero();
+      if (rj == 0) {
+        f.load(st + 2 * 1024);
+        mma32_ff<T>(Rt, f, tm_t(0, 0));
       }
+      f.load(st + 3 * 1024);
+      mma32_ff<T>(Rt, f, tm_t(rj, 1));
+      const float bj = bs[32 * rj + l32];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) Rt[r] *= bj;
+      if (32 * rj + l32 < nvalid)
+        acc_to_lds_t<T>(Rt, dv_out + (tok0 + 32 * rj + l32) * ts.dv + h * V + 32 * vblk, 0, 0, 0);
     }
   }
   sds = wave_sum(sds);
