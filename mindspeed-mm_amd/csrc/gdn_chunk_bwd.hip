@@ -282,31 +282,9 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
 //     T ("transposed"):  pack(transpose(pack(X)))  lane <-> i, registers <-> j
 //   dQ, dK, dv leave as 16-byte row pieces.
 // ---------------------------------------------------------------------------------------------
-// The raw dO and V blocks [64 tokens][32 columns] sit in LDS with their rows 64 bytes (128 for fp32) apart, so the
-// lanes of one fragment read, one row each, would meet on 8 (4) of the 64 banks.  The 16-byte pieces of row r are
-// therefore stored permuted, piece c at position raw_piece_pos(r, c) (an involution), which spreads such a read over
-// all the banks; the copy that fills the block applies the permutation to its source addresses.
-template <typename T> __device__ __forceinline__ int raw_piece_pos(int r, int c) {
-  return sizeof(T) == 2 ? (c ^ ((r >> 2) & 3)) : (c ^ (((r >> 1) & 3) << 1));
-}
-// A-operand fragments of row r of such a block (lane <-> token r, registers <-> the 32 columns)
-template <typename T> __device__ __forceinline__ void frags_from_raw(AccB<T>& out, const T* blk, int r) {
-  const int half = (threadIdx.x & 63) >> 5;
-  const T* row = blk + r * 32;
-#pragma unroll
-  for (int kg = 0; kg < AccK<T>::kGroups; ++kg) {
-    if constexpr (sizeof(T) == 2) {
-      const u32x2 lo = *reinterpret_cast<const u32x2*>(row + raw_piece_pos<T>(r, 2 * kg) * 8 + 4 * half);
-      const u32x2 hi = *reinterpret_cast<const u32x2*>(row + raw_piece_pos<T>(r, 2 * kg + 1) * 8 + 4 * half);
-      out.f[kg] = u32x4{lo[0], lo[1], hi[0], hi[1]};
-    } else {
-      out.f[kg] = *reinterpret_cast<const u32x4*>(row + raw_piece_pos<T>(r, 2 * kg + half) * 4);
-    }
-  }
-}
-
 template <typename T, int DK> struct BwdLocalSmem {
   // one stage, in elements: [v_new x2 | dV' x2] shared tiles, raw dO [64][32], [S | dS'] per wave, raw V [64][32]
+  // (the raw blocks as SwizzledTile<T, 32>)
   static constexpr int st_doraw = 4 * 1024, st_priv = 6 * 1024, st_vraw = st_priv + 4 * 2048, stage_elems = st_vraw + 64 * 32;
   // epilogue, stage that idles during the last block: K tiles [K/32][2] | the Q^T tiles [2] of each wave
   static constexpr int ea_q = 8 * 1024;
@@ -376,7 +354,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
 #pragma unroll
     for (int j = 0; j < (int)sizeof(T) / 2; ++j) {   // raw dO and V blocks [64][32], rows past the end repeat the last row
       constexpr int LPR = 32 / VEC, RPP = 64 / LPR;  // lanes per row, rows per piece
-      const int piece = 4 * j + wave, row = piece * RPP + lane / LPR, cc = raw_piece_pos<T>(row, lane % LPR);
+      const int piece = 4 * j + wave, row = piece * RPP + lane / LPR, cc = SwizzledTile<T, 32>::pos(row, lane % LPR);
       const int64_t tok = tok0 + imin(row, nvalid - 1), col = (int64_t)h * V + 32 * vblk + cc * VEC;
       load16_to_lds(dO + tok * Hv * V + col, st + SM::st_doraw + piece * 64 * VEC);
       load16_to_lds(v + tok * ts.v + col, st + SM::st_vraw + piece * 64 * VEC);
@@ -457,7 +435,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     }
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {         // (lane <-> token, registers <-> V) from here on; dO rows have it already
-      frags_from_raw<T>(dOt[ri], st + SM::st_doraw, 32 * ri + l32);
+      SwizzledTile<T, 32>::frags(dOt[ri], st + SM::st_doraw, 32 * ri + l32, 0);
       if (32 * ri + l32 >= nvalid) {
 #pragma unroll
         for (int g = 0; g < KG; ++g) dOt[ri].f[g] = u32x4{0u, 0u, 0u, 0u};
@@ -481,7 +459,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       dVt.pack(mfma_transpose<T>(f, id));
       if (has_k) mma32_ff<T>(dWa[ri], dVt, Sf);
       if (lower && ri == ti) {
-        frags_from_raw<T>(f, st + SM::st_vraw, 32 * tj + l32);
+        SwizzledTile<T, 32>::frags(f, st + SM::st_vraw, 32 * tj + l32, 0);
         mma32_ff<T>(a2, dVt, f);
       }
     }

@@ -51,22 +51,35 @@ __global__ void chunk_table_kernel(const int64_t* __restrict__ cu, int* __restri
   }
 }
 
-// ---------------------------------------------------------------------------------------------
-// global -> LDS tile load (64 rows x DK columns, rows >= nvalid zero) with the optional in-kernel l2 normalisation
-// y = x * rsqrt(sum(x^2) + 1e-6) over the row (modeling_qwen3_5.py:392-395).  The lanes that share a row are
-// neighbours in a wave and combine their partial sums with data-parallel-primitive moves.  y_out / rstd_out (either may be null) receive
-// the normalised rows and 1/|x| for the kernels that come later.
-// ---------------------------------------------------------------------------------------------
-template <typename T, int DK>
-__device__ __forceinline__ void load_tile_qk(T* lds, int ld, const T* g, int64_t row_stride, int nvalid, int tid,
-                                             bool l2norm, T* y_out, int64_t y_stride, float* rstd_out,
-                                             int64_t rstd_stride) {
-  constexpr int V = Elem<T>::kVec, CPR = DK / V;   // lanes per row: a power of two <= 32
+// A [64, DK] q or k tile on its way into LDS, in two steps so that the requests of both tiles (and of the gates) are
+// in flight together instead of one 16-byte piece at a time: tile_qk_request() issues this thread's loads (rows past
+// the end of the sequence are zero), tile_qk_finish() applies the optional l2 norm (y = x rsqrt(sum x^2 + 1e-6) over
+// the row, modeling_qwen3_5.py:392-395; fp32 arithmetic, result rounded to T; a row sits on DK/VEC neighbouring lanes
+// that combine their partial sums with data-parallel-primitive moves), writes the tile to
+// LDS and, on request, the normalised rows (row stride y_stride) and 1/|x| (stride rstd_stride) to global memory.
+template <typename T, int DK> struct TileQK {
+  static constexpr int V = Elem<T>::kVec, CPR = DK / V, PT = 64 * CPR / kThreads;   // lanes per row; pieces per thread
   static_assert((64 * CPR) % kThreads == 0, "every thread takes the same number of pieces");
-  for (int c = tid; c < 64 * CPR; c += kThreads) {
-    const int row = c / CPR, cc = c % CPR;
+  Vec16<T> x[PT];
+};
+template <typename T, int DK>
+__device__ __forceinline__ void tile_qk_request(TileQK<T, DK>& t, const T* g, int64_t row_stride, int nvalid, int tid) {
+  constexpr int V = TileQK<T, DK>::V, CPR = TileQK<T, DK>::CPR;
+#pragma unroll
+  for (int i = 0; i < TileQK<T, DK>::PT; ++i) {
+    const int c = tid + i * kThreads, row = c / CPR, cc = c % CPR;
+    t.x[i] = ld16(g + (int64_t)imin(row, nvalid - 1) * row_stride + cc * V);   // the same load on every path
+  }
+}
+template <typename T, int DK>
+__device__ __forceinline__ void tile_qk_finish(TileQK<T, DK>& t, T* lds, int ld, int nvalid, int tid, bool l2norm,
+                                               T* y_out, int64_t y_stride, float* rstd_out, int64_t rstd_stride) {
+  constexpr int V = TileQK<T, DK>::V, CPR = TileQK<T, DK>::CPR;
+#pragma unroll
+  for (int i = 0; i < TileQK<T, DK>::PT; ++i) {
+    const int c = tid + i * kThreads, row = c / CPR, cc = c % CPR;
     const bool ok = row < nvalid;
-    Vec16<T> x = ok ? ld16(g + (int64_t)row * row_stride + cc * V) : zero16<T>();
+    Vec16<T> x = ok ? t.x[i] : zero16<T>();
     if (l2norm) {   // uniform: every lane takes part in the shuffles
       float f[V], ss = 0.f;
       unpack16<T>(x, f);
@@ -90,6 +103,8 @@ __device__ __forceinline__ void load_tile_qk(T* lds, int ld, const T* g, int64_t
 //   per q/k group the K^T, K and Q^T tiles of the recurrence kernels
 // U is written in fragment order (AccB<>): tile (32-token block ri) x (32-column block vb) at
 // U[chunk][head][vb][ri][1024], 16 bytes per lane per k-group -- the recurrence kernel copies it straight to LDS.
+// Three quarters of the kernel's traffic are stores, issued all along the way; its barriers order LDS traffic only
+// (GDN_LDS_BARRIER), because a __syncthreads() would also wait until every store issued so far has been acknowledged.
 // ---------------------------------------------------------------------------------------------
 template <typename T, int DK, int BV> struct PrepSmem {
   static constexpr int LDK = lds_ld<T>(DK), LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
@@ -133,15 +148,18 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
   const int h = blockIdx.y, hq = h / (Hv / Hqk), nvalid = s.nvalid;
   const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk;
 
-  // ---- phase 0: cumulative decay (one lane per token), beta; K and Q tiles ----
+  // ---- phase 0: cumulative decay (one lane per token), beta; K and Q tiles.  All requests first. ----
+  TileQK<T, DK> kt, qt;
+  tile_qk_request<T, DK>(kt, k + tok0 * ts.k + hq * DK, ts.k, nvalid, tid);
+  tile_qk_request<T, DK>(qt, q + tok0 * ts.q + hq * DK, ts.q, nvalid, tid);
   if (wave == 0) {
     float x = lane < nvalid ? g[(tok0 + lane) * Hv + h] : 0.f;
+    const float b = lane < nvalid ? beta[(tok0 + lane) * Hv + h] : 0.f;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
       const float t = __shfl_up(x, d);
       if (lane >= d) x += t;
     }
-    const float b = lane < nvalid ? beta[(tok0 + lane) * Hv + h] : 0.f;
     Gs[lane] = x;
     bs[lane] = b;
     egs[lane] = b * __expf(x);
@@ -152,12 +170,11 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
     // of each q/k group also leaves the normalised q (for the output kernel and the backward pass) and 1/|q|, 1/|k|.
     const bool keep = l2norm && (h % (Hv / Hqk)) == 0;
     const int64_t off = (tok0 * Hqk + hq) * DK, roff = tok0 * Hqk + hq;
-    load_tile_qk<T, DK>(Ks, LDK, k + tok0 * ts.k + hq * DK, ts.k, nvalid, tid, l2norm != 0, nullptr, 0,
-                        keep ? rstd_k_out + roff : nullptr, Hqk);
-    load_tile_qk<T, DK>(Qs, LDK, q + tok0 * ts.q + hq * DK, ts.q, nvalid, tid, l2norm != 0, keep ? qn_out + off : nullptr,
-                        (int64_t)Hqk * DK, keep ? rstd_q_out + roff : nullptr, Hqk);
+    tile_qk_finish<T, DK>(kt, Ks, LDK, nvalid, tid, l2norm != 0, nullptr, 0, keep ? rstd_k_out + roff : nullptr, Hqk);
+    tile_qk_finish<T, DK>(qt, Qs, LDK, nvalid, tid, l2norm != 0, keep ? qn_out + off : nullptr, (int64_t)Hqk * DK,
+                          keep ? rstd_q_out + roff : nullptr, Hqk);
   }
-  __syncthreads();
+  GDN_LDS_BARRIER();
 
   // ---- phase 1: A = strict_tril(beta_i k_i.k_j Gam_ij) and Aq = tril(q_i.k_j Gam_ij), one 32x32 tile per wave ----
   f32x16 a_tile = acc_zero();   // goes to LDS (over the Q tile) once every wave is done with Q
@@ -169,11 +186,14 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
       mma32<T, DK, true, true>(aq, Qs + 32 * ti * LDK, LDK, Ks + 32 * tj * LDK, LDK);
     }
     const int j = 32 * tj + acc_col();
+    const float gj = Gs[j];
+    const f32x16 gi = rows_ld(Gs, 32 * ti), bi = rows_ld(bs, 32 * ti);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
+    for (int r = 0; r < 16; ++r) {   // branch-free: where the mask discards the value the exponent is set to 0 first
       const int i = 32 * ti + acc_row(r);
-      const float gam = i >= j ? __expf(Gs[i] - Gs[j]) : 0.f;
-      a_tile[r] = i > j ? bs[i] * a_tile[r] * gam : 0.f;
+      const float e = __expf(i >= j ? gi[r] - gj : 0.f);
+      const float gam = i >= j ? e : 0.f;
+      a_tile[r] = i > j ? bi[r] * a_tile[r] * gam : 0.f;
       aq[r] *= gam * scale;
     }
     // scale tril(Q K^T . Gam) leaves as four 32x32 tiles in fragment order, packed as they sit in the accumulator
@@ -213,7 +233,7 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
     const int c = tid + i * kThreads, row = c / (DK / VEC), cc = c % (DK / VEC);
     kreg[i] = scale16<T>(ld16(Ks + row * LDK + cc * VEC), egs[row]);
   }
-  __syncthreads();   // Q and K are consumed: their space takes A and Tm
+  GDN_LDS_BARRIER();   // Q and K are consumed: their space takes A and Tm
 
   {
     const int ti = wave >> 1, tj = wave & 1, j = 32 * tj + acc_col();
@@ -228,9 +248,9 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
     const int c = tid + i * kThreads, row = c / (BV / VEC), cc = c % (BV / VEC);
-    vreg[i] = row < nvalid ? ld16(vg + row * ts.v + cc * VEC) : zero16<T>();
+    vreg[i] = ld16(vg + imin(row, nvalid - 1) * ts.v + cc * VEC);   // rows past the end: beta = 0 will clear them
   }
-  __syncthreads();
+  GDN_LDS_BARRIER();
 
   // ---- phase 2a: invert the four 16x16 diagonal blocks by forward substitution (fp32) ----
   if (lane < 16) {
@@ -246,7 +266,7 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
 #pragma unroll
     for (int i = 0; i < 16; ++i) Ti[(o + i) * kLF + o + j] = tcol[i];
   }
-  __syncthreads();
+  GDN_LDS_BARRIER();
 
   // ---- phase 2b: 16 -> 32 merges  X = -T22 (A21 T11); the zero upper triangle of As is scratch ----
   {
@@ -261,7 +281,7 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
 #pragma unroll
       for (int r = 0; r < 4; ++r) As[(C0 + 4 * lk + r) * kLF + R0 + li] = y[r];
     }
-    __syncthreads();
+    GDN_LDS_BARRIER();
     f32x4 x = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk)
@@ -271,7 +291,7 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
       for (int r = 0; r < 4; ++r) Ti[(R0 + 4 * lk + r) * kLF + C0 + li] = -x[r];
     }
   }
-  __syncthreads();
+  GDN_LDS_BARRIER();
 
   // ---- phase 2c: 32 -> 64 merge, one 16x16 tile of the 32x32 block per wave ----
   {
@@ -284,7 +304,7 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
     // scratch: upper-right 32x32 quadrant of As (never read as part of A)
 #pragma unroll
     for (int r = 0; r < 4; ++r) As[(16 * ta + 4 * lk + r) * kLF + 32 + 16 * tb + li] = y[r];
-    __syncthreads();
+    GDN_LDS_BARRIER();
     f32x4 x = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int kk = 0; kk < 8; ++kk)
@@ -292,7 +312,7 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
 #pragma unroll
     for (int r = 0; r < 4; ++r) Ti[(32 + 16 * ta + 4 * lk + r) * kLF + 16 * tb + li] = -x[r];
   }
-  __syncthreads();
+  GDN_LDS_BARRIER();
 
   // ---- phase 3: Tm in operand precision, kept for the backward pass ----
   {
@@ -305,19 +325,22 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
       st16(Tms + row * L64 + cc * VEC, pack16<T>(f));
     }
   }
-  __syncthreads();
+  GDN_LDS_BARRIER();
   // the fp32 Tm is consumed: its space takes the beta e^G K tile parked in registers
 #pragma unroll
   for (int i = 0; i < KPT; ++i) {
     const int c = tid + i * kThreads, row = c / (DK / VEC), cc = c % (DK / VEC);
     st16(Kb + row * LDK + cc * VEC, kreg[i]);
   }
+  // The V block requested above has long arrived.  Waiting for it here, before the stores of the next phases are
+  // issued, keeps its first use from waiting for those stores as well (loads and stores are counted in one order).
+  GDN_WAIT_VMEM();
   if (Ai_out != nullptr) {  // the four 32x32 tiles of Tm as A operands (lane <-> row, registers <-> column), for the backward
     AccB<T> tf;
     frags_from_lds<T>(tf, Tms + (32 * (wave >> 1) + (lane & 31)) * L64 + 32 * (wave & 1));
     tf.store_stream(Ai_out + (((int64_t)blockIdx.x * Hv + h) * 4 + wave) * 1024);
   }
-  __syncthreads();
+  GDN_LDS_BARRIER();
 
   // ---- phase 4: W = Tm (beta e^G K), handed on in fragment order only ----
   {
@@ -339,7 +362,7 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
   }
   // ---- phase 5: U = Tm (beta V), V block by V block, stored in fragment order ----
   for (int vb = 0; vb < V / BV; ++vb) {
-    __syncthreads();   // the tile in region 1 (beta e^G K, or the previous V block) is consumed
+    GDN_LDS_BARRIER();   // the tile in region 1 (beta e^G K, or the previous V block) is consumed
     if (vb == 0) {     // the first (beta V) block was parked in registers
 #pragma unroll
       for (int i = 0; i < VPT; ++i) {
@@ -349,7 +372,7 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
     } else {
       load_tile_scaled<T, BV>(Vb, LDV, vg + vb * BV, ts.v, nvalid, bs, tid);
     }
-    __syncthreads();
+    GDN_LDS_BARRIER();
     for (int tt = wave; tt < 2 * (BV / 32); tt += 4) {
       const int ri = tt & 1, cj = tt >> 1;
       f32x16 acc = acc_zero();

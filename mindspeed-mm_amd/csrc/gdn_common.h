@@ -392,6 +392,36 @@ template <typename T> __device__ __forceinline__ void frags_from_lds(AccB<T>& ou
   for (int kg = 0; kg < AccK<T>::kGroups; ++kg) out.f[kg] = frag_a_split<T>(row + G * kg);
 }
 
+// A row-major [rows][COLS] tile in LDS without padding, as a direct global -> LDS copy leaves it (64 lanes x 16 bytes
+// per instruction, contiguous).  Its rows are a multiple of 64 bytes apart, so the lanes of a fragment read, one row
+// each, would meet on a few of the 64 banks.  The 16-byte pieces of row r are therefore stored permuted, piece c at
+// position pos(r, c) = c ^ key(r) (an involution: the copy applies it to its source addresses), with the key chosen so
+// that 16 consecutive rows cover all the banks.
+template <typename T, int COLS> struct SwizzledTile {
+  static constexpr int kVec = 16 / (int)sizeof(T), kPieces = COLS / kVec;   // pieces per row
+  static_assert(kPieces >= 4 && (kPieces & (kPieces - 1)) == 0, "rows of 4, 8, 16, ... pieces");
+  static __device__ __forceinline__ int key(int r) {
+    if constexpr (kPieces >= 16) return r & 15;
+    else return (r / (16 / kPieces)) & (kPieces - 1);
+  }
+  static __device__ __forceinline__ int pos(int r, int c) { return c ^ key(r); }
+  // A-operand fragments of columns [k0, k0 + 32) of row r (lane <-> row r, registers <-> the 32 columns)
+  static __device__ __forceinline__ void frags(AccB<T>& out, const T* tile, int r, int k0) {
+    const int half = (threadIdx.x & 63) >> 5, c0 = k0 / kVec;
+    const T* row = tile + r * COLS;
+#pragma unroll
+    for (int kg = 0; kg < AccK<T>::kGroups; ++kg) {
+      if constexpr (sizeof(T) == 2) {
+        const u32x2 lo = *reinterpret_cast<const u32x2*>(row + pos(r, c0 + 2 * kg) * 8 + 4 * half);
+        const u32x2 hi = *reinterpret_cast<const u32x2*>(row + pos(r, c0 + 2 * kg + 1) * 8 + 4 * half);
+        out.f[kg] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+      } else {
+        out.f[kg] = *reinterpret_cast<const u32x4*>(row + pos(r, c0 + 2 * kg + half) * 4);
+      }
+    }
+  }
+};
+
 // Cross-lane transpose through the matrix core.  A tile held as fragments with (lane <-> a, registers <-> b)
 // multiplied by the identity comes back as an accumulator with (lane <-> b, registers <-> a): C = X * I read as
 // A operand X[a][b].  Exact (products with 1.0, sums with 0).  Costs kGroups MFMA k-groups per 32x32 tile.
