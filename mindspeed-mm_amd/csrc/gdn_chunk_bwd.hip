@@ -389,13 +389,19 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     load16_to_lds(Ai + ch * 4096 + ((4 * j + wave) * 64 + lane) * VEC, TmF + (4 * j + wave) * 64 * VEC);
   issue(0, 0);
 
-  if (tid < 64) {
-    const float gv = G[ch * 64 + imin(tid, nvalid - 1)];
+  if (tid < 64) {   // the row vectors: all requests first, the same ones on every path
+    const int tc = imin(tid, nvalid - 1);
+    const float gv = G[ch * 64 + tc], bv = beta[(tok0 + tc) * Hv + h];
+    float rq1 = 1.f, rk1v = 1.f;
+    if (l2) {
+      rq1 = rstd_q[(tok0 + tc) * Hqk + hq];
+      rk1v = rstd_k[(tok0 + tc) * Hqk + hq];
+    }
     Gs[tid] = gv;
     egs[tid] = __expf(gv);
-    bs[tid] = tid < nvalid ? beta[(tok0 + tid) * Hv + h] : 0.f;
-    rsq[tid] = l2 ? rstd_q[(tok0 + imin(tid, nvalid - 1)) * Hqk + hq] : 1.f;
-    rsk[tid] = l2 ? rstd_k[(tok0 + imin(tid, nvalid - 1)) * Hqk + hq] : 1.f;
+    bs[tid] = tid < nvalid ? bv : 0.f;
+    rsq[tid] = rq1;
+    rsk[tid] = rk1v;
   }
   rq[tid] = 0.f; rk1[tid] = 0.f; rbk[tid] = 0.f; rf[tid] = 0.f; rv[tid] = 0.f;   // 256 threads, 256 entries each
   GDN_WAIT_VMEM();

@@ -569,27 +569,35 @@ template <typename T> struct Patch { static constexpr int kLd = 32 + 16 / (int)s
 template <typename T, bool ADD>
 __device__ __forceinline__ void acc_store_rows(const f32x16& acc, const IdentityFrag<T>& id, T* patch, T* g,
                                                int64_t row_stride, int rows_valid) {
-  constexpr int PLD = Patch<T>::kLd, V = Elem<T>::kVec, PPR = 32 / V;
+  constexpr int PLD = Patch<T>::kLd, V = Elem<T>::kVec, PPR = 32 / V, NP = 32 * PPR / 64;   // NP pieces per lane
   const int lane = threadIdx.x & 63;
+  if (rows_valid <= 0) return;   // wave-uniform
+  // ADD: what memory holds is requested for all of the lane's pieces before the tile is turned, so that the requests
+  // overlap each other and that work (rows past the end repeat the last valid one: the same loads on every path)
+  Vec16<T> y[NP];
+  if constexpr (ADD) {
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const int p = lane + 64 * i, row = imin(p / PPR, rows_valid - 1), cc = p % PPR;
+      y[i] = ld16(g + (int64_t)row * row_stride + cc * V);
+    }
+  }
   GDN_WAVE_LDS_SYNC();   // earlier readers of the patch are done
   acc_to_lds_rm(acc, id, patch, PLD, 0, 0);
   GDN_WAVE_LDS_SYNC();
 #pragma unroll
-  for (int p = lane; p < 32 * PPR; p += 64) {
-    const int row = p / PPR, cc = p % PPR;
-    if (row < rows_valid) {
-      Vec16<T> x = ld16(patch + row * PLD + cc * V);
-      if constexpr (ADD) {
-        const Vec16<T> y = ld16(g + (int64_t)row * row_stride + cc * V);
-        float fx[V], fy[V];
-        unpack16<T>(x, fx);
-        unpack16<T>(y, fy);
+  for (int i = 0; i < NP; ++i) {
+    const int p = lane + 64 * i, row = p / PPR, cc = p % PPR;
+    Vec16<T> x = ld16(patch + row * PLD + cc * V);
+    if constexpr (ADD) {
+      float fx[V], fy[V];
+      unpack16<T>(x, fx);
+      unpack16<T>(y[i], fy);
 #pragma unroll
-        for (int e = 0; e < V; ++e) fx[e] += fy[e];
-        x = pack16<T>(fx);
-      }
-      st16(g + (int64_t)row * row_stride + cc * V, x);
+      for (int e = 0; e < V; ++e) fx[e] += fy[e];
+      x = pack16<T>(fx);
     }
+    if (row < rows_valid) st16(g + (int64_t)row * row_stride + cc * V, x);
   }
   GDN_WAVE_LDS_SYNC();   // the patch may be overwritten (also by a direct global->LDS load) once every lane has read it
 }
