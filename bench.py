@@ -37,8 +37,8 @@ CFG = dict(B=2, T=8192, Hqk=16, Hv=32, K=128, V=128, C=64)
 # (rocprofv3 --pmc, one run per counter, each scaled by what the same counter reads for a 512 MiB copy): the figures
 # of profiles/chunk_fwd_bwd_B2_T8192_bf16_hbm_traffic.md.  Measured offline, reported beside the live timings.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "chunk_prep_kernel": 1114360545, "chunk_state_kernel": 749423797, "chunk_out_kernel": 672581114,
-    "chunk_state_bwd_kernel": 884322872, "chunk_bwd_local_kernel": 1174922825,
+    "chunk_prep_kernel": 1136386895, "chunk_state_kernel": 749425757, "chunk_out_kernel": 673376638,
+    "chunk_state_bwd_kernel": 884322839, "chunk_bwd_local_kernel": 1151905110,
 }
 
 
