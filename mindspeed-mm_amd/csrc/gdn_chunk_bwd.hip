@@ -590,6 +590,14 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     }
   }
   GDN_LDS_BARRIER();   // the ds tiles and the dW tiles are consumed
+  // later value heads of a group add to the dq, dk rows the earlier ones wrote: what memory holds is requested well
+  // ahead, dq here (no store is in flight), dk right behind the dq stores (three phases before it is needed)
+  RowPieces<T> held[2];
+  if (has_k && hh != 0) {
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri)
+      rows_request<T>(held[ri], dq + (tok0 + 32 * ri) * ts.dq + hq * DK + 32 * cj, ts.dq, nvalid - 32 * ri);
+  }
   if (lower) {  // <R_t, v_t> = sum_i Tm[i][t] (dV' V^T)[i][t]: column sums of Tm . a2, no second pass over V needed
     const f32x16 tmv = tm_t(tj, ti).unpack();   // Tm tile (ti, tj) with lane <-> column, registers <-> row
     float sv = 0.f;
@@ -619,7 +627,12 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       }
       T* dst = dq + (tok0 + 32 * ri) * ts.dq + hq * DK + 32 * cj;
       if (hh == 0) acc_store_rows<T, false>(dQi[ri], id, patch, dst, ts.dq, nvalid - 32 * ri);
-      else acc_store_rows<T, true>(dQi[ri], id, patch, dst, ts.dq, nvalid - 32 * ri);
+      else acc_store_rows<T, true>(dQi[ri], id, patch, dst, ts.dq, nvalid - 32 * ri, held[ri]);
+    }
+    if (hh != 0) {
+#pragma unroll
+      for (int ri = 0; ri < 2; ++ri)
+        rows_request<T>(held[ri], dk + (tok0 + 32 * ri) * ts.dk + hq * DK + 32 * cj, ts.dk, nvalid - 32 * ri);
     }
   }
   GDN_LDS_BARRIER();
@@ -692,7 +705,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       }
       T* dst = dk + (tok0 + 32 * ri) * ts.dk + hq * DK + 32 * cj;
       if (hh == 0) acc_store_rows<T, false>(dKi[ri], id, patch, dst, ts.dk, nvalid - 32 * ri);
-      else acc_store_rows<T, true>(dKi[ri], id, patch, dst, ts.dk, nvalid - 32 * ri);
+      else acc_store_rows<T, true>(dKi[ri], id, patch, dst, ts.dk, nvalid - 32 * ri, held[ri]);
     }
   }
   if (wave == 0) {   // d(cumulative G) -> d(g): suffix sum inside the chunk

@@ -565,23 +565,31 @@ __device__ __forceinline__ f32x16 rows_ld4(const float* arr, int i0) {
 // 16-byte pieces after a pass through a wave-private LDS patch of 32 x kPatchLd elements.  Element-wise stores of
 // an accumulator tile (2 bytes per lane, 16 instructions) are several times slower than these.
 template <typename T> struct Patch { static constexpr int kLd = 32 + 16 / (int)sizeof(T), kElems = 32 * kLd; };
-// ADD: the rows are added to what global memory already holds (written earlier by this very thread).
+// What global memory holds at the rows such a tile will be added to: requested by rows_request() well before
+// acc_store_rows() adds and writes back, so that the requests of several tiles are in flight together and none of
+// them is issued behind a store (loads and stores complete in one order: a load issued after a store is not seen
+// before that store has been acknowledged).  Rows past the end repeat the last valid one: the same loads on every path.
+template <typename T> struct RowPieces {
+  static constexpr int kN = 32 * (32 / Elem<T>::kVec) / 64;   // 16-byte pieces per lane
+  Vec16<T> y[kN];
+};
+template <typename T>
+__device__ __forceinline__ void rows_request(RowPieces<T>& r, const T* g, int64_t row_stride, int rows_valid) {
+  constexpr int V = Elem<T>::kVec, PPR = 32 / V;
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int i = 0; i < RowPieces<T>::kN; ++i) {
+    const int p = lane + 64 * i, row = imax(imin(p / PPR, rows_valid - 1), 0), cc = p % PPR;
+    r.y[i] = ld16(g + (int64_t)row * row_stride + cc * V);
+  }
+}
+// ADD: the rows are added to `held` (what memory held, see rows_request) before they are written.
 template <typename T, bool ADD>
 __device__ __forceinline__ void acc_store_rows(const f32x16& acc, const IdentityFrag<T>& id, T* patch, T* g,
-                                               int64_t row_stride, int rows_valid) {
-  constexpr int PLD = Patch<T>::kLd, V = Elem<T>::kVec, PPR = 32 / V, NP = 32 * PPR / 64;   // NP pieces per lane
+                                               int64_t row_stride, int rows_valid, const RowPieces<T>& held) {
+  constexpr int PLD = Patch<T>::kLd, V = Elem<T>::kVec, PPR = 32 / V, NP = RowPieces<T>::kN;
   const int lane = threadIdx.x & 63;
   if (rows_valid <= 0) return;   // wave-uniform
-  // ADD: what memory holds is requested for all of the lane's pieces before the tile is turned, so that the requests
-  // overlap each other and that work (rows past the end repeat the last valid one: the same loads on every path)
-  Vec16<T> y[NP];
-  if constexpr (ADD) {
-#pragma unroll
-    for (int i = 0; i < NP; ++i) {
-      const int p = lane + 64 * i, row = imin(p / PPR, rows_valid - 1), cc = p % PPR;
-      y[i] = ld16(g + (int64_t)row * row_stride + cc * V);
-    }
-  }
   GDN_WAVE_LDS_SYNC();   // earlier readers of the patch are done
   acc_to_lds_rm(acc, id, patch, PLD, 0, 0);
   GDN_WAVE_LDS_SYNC();
@@ -592,7 +600,7 @@ __device__ __forceinline__ void acc_store_rows(const f32x16& acc, const Identity
     if constexpr (ADD) {
       float fx[V], fy[V];
       unpack16<T>(x, fx);
-      unpack16<T>(y[i], fy);
+      unpack16<T>(held.y[i], fy);
 #pragma unroll
       for (int e = 0; e < V; ++e) fx[e] += fy[e];
       x = pack16<T>(fx);
@@ -600,6 +608,13 @@ __device__ __forceinline__ void acc_store_rows(const f32x16& acc, const Identity
     if (row < rows_valid) st16(g + (int64_t)row * row_stride + cc * V, x);
   }
   GDN_WAVE_LDS_SYNC();   // the patch may be overwritten (also by a direct global->LDS load) once every lane has read it
+}
+template <typename T, bool ADD>
+__device__ __forceinline__ void acc_store_rows(const f32x16& acc, const IdentityFrag<T>& id, T* patch, T* g,
+                                               int64_t row_stride, int rows_valid) {
+  static_assert(!ADD, "adding needs the rows requested beforehand");
+  RowPieces<T> none;
+  acc_store_rows<T, false>(acc, id, patch, g, row_stride, rows_valid, none);
 }
 
 // sum over the 32 lanes that share a half-wave (all columns of one accumulator row)
