@@ -31,7 +31,6 @@ struct ChunkDims {
 // Byte offsets into the workspace.  Everything the backward pass re-reads is written by the forward.
 struct ChunkWorkspace {
   int64_t chunk_offsets;  // int32 [N+1]      chunks before each packed sequence
-  int64_t qn;             // T [tokens,Hqk,K] l2-normalised q (only with use_qk_l2norm)
   int64_t rstd;           // f32 [2][tokens,Hqk] 1/|q|, 1/|k| of that normalisation
   int64_t G;              // f32 [chunks,Hv,64]      chunk-local cumulative log decay
   int64_t WAF;            // T [chunks,Hv,K/32,2]    -W as A operand: tile = (32 tokens) x (32 columns of K), fragment order
@@ -59,7 +58,6 @@ inline ChunkWorkspace chunk_workspace_layout(const ChunkDims& d, int elem_bytes)
   auto take = [&](int64_t bytes) { int64_t o = off; off += align256(bytes); return o; };
   const int64_t tok = d.tokens(), nc = d.max_chunks();
   w.chunk_offsets = take((int64_t)(d.N + 1) * 4);
-  w.qn = take(tok * d.Hqk * d.K * elem_bytes);
   w.rstd = take(2 * tok * d.Hqk * 4);
   w.G = take(nc * 64 * d.Hv * 4);
   w.WAF = take(nc * 64 * d.Hv * d.K * elem_bytes);

@@ -127,7 +127,7 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
     const float* __restrict__ beta, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets,
     float* __restrict__ G_out, T* __restrict__ Ai_out, T* __restrict__ W_out, T* __restrict__ U_out,
     T* __restrict__ Aq_out, T* __restrict__ KT_out, T* __restrict__ WF_out, T* __restrict__ KA_out,
-    T* __restrict__ QT_out, T* __restrict__ qn_out, float* __restrict__ rstd_q_out, float* __restrict__ rstd_k_out,
+    T* __restrict__ QT_out, float* __restrict__ rstd_q_out, float* __restrict__ rstd_k_out,
     int T_len, int N, int Hqk, int Hv, int V, float scale, int l2norm, TokenStrides ts) {
   using SM = PrepSmem<T, DK, BV>;
   constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64, VEC = Elem<T>::kVec;
@@ -167,12 +167,11 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
   }
   {
     // q and k arrive raw; with the in-kernel l2 norm they are normalised on the way into LDS.  The first value head
-    // of each q/k group also leaves the normalised q (for the output kernel and the backward pass) and 1/|q|, 1/|k|.
+    // of each q/k group also leaves 1/|q|, 1/|k| (for the output kernel, which scales q itself, and the backward pass).
     const bool keep = l2norm && (h % (Hv / Hqk)) == 0;
-    const int64_t off = (tok0 * Hqk + hq) * DK, roff = tok0 * Hqk + hq;
+    const int64_t roff = tok0 * Hqk + hq;
     tile_qk_finish<T, DK>(kt, Ks, LDK, nvalid, tid, l2norm != 0, nullptr, 0, keep ? rstd_k_out + roff : nullptr, Hqk);
-    tile_qk_finish<T, DK>(qt, Qs, LDK, nvalid, tid, l2norm != 0, keep ? qn_out + off : nullptr, (int64_t)Hqk * DK,
-                          keep ? rstd_q_out + roff : nullptr, Hqk);
+    tile_qk_finish<T, DK>(qt, Qs, LDK, nvalid, tid, l2norm != 0, nullptr, 0, keep ? rstd_q_out + roff : nullptr, Hqk);
   }
   GDN_LDS_BARRIER();
 
@@ -641,7 +640,7 @@ __global__ __launch_bounds__(64 * NW) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 2)
     const T* __restrict__ q, const T* __restrict__ aqf, const T* __restrict__ vf, const T* __restrict__ hf,
     const float* __restrict__ G, T* __restrict__ o, const int64_t* __restrict__ cu,
     const int* __restrict__ chunk_offsets, int T_len, int N, int Hqk, int Hv, int V, float scale, int64_t q_stride,
-    OutNorm<T, TW> nm) {
+    const float* __restrict__ rstd_q, OutNorm<T, TW> nm) {
   using SM = OutSmem<T, DK, NW>;
   constexpr int LDK = SM::LDK, NT = 64 * NW, VEC = Elem<T>::kVec, NKT = DK / 32;
   T* Qs = reinterpret_cast<T*>(gdn_smem + SM::off_qs);
@@ -665,10 +664,16 @@ __global__ __launch_bounds__(64 * NW) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 2)
   Af[0].load(aqf + (ch * 4 + 0) * 1024);   // tiles (0,0), (1,0), (1,1) of tril(Q K^T . Gam)
   Af[1].load(aqf + (ch * 4 + 2) * 1024);
   Af[2].load(aqf + (ch * 4 + 3) * 1024);
+  // q arrives raw; with the in-kernel l2 norm its rows are scaled by the 1/|q| the prep kernel left (the same fp32
+  // product and rounding it applied itself: no normalised copy of q is kept in memory)
   for (int c = tid; c < 64 * (DK / VEC); c += NT) {
     const int row = c / (DK / VEC), cc = c % (DK / VEC);
-    st16(Qs + row * LDK + cc * VEC,
-         row < nvalid ? ld16(q + (tok0 + row) * q_stride + hq * DK + cc * VEC) : zero16<T>());
+    Vec16<T> x = zero16<T>();
+    if (row < nvalid) {
+      x = ld16(q + (tok0 + row) * q_stride + hq * DK + cc * VEC);
+      if (rstd_q != nullptr) x = scale16<T>(x, rstd_q[(tok0 + row) * Hqk + hq]);
+    }
+    st16(Qs + row * LDK + cc * VEC, x);
   }
   if (tid < 64) Eg[tid] = scale * __expf(G[ch * 64 + imin(tid, nvalid - 1)]);
   IdentityFrag<T> id;
@@ -772,7 +777,6 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   const T* qq = (const T*)q;
   const T* kk = (const T*)k;
   if (cu != nullptr) GDN_LAUNCH(kKernChunkTable, st, chunk_table_kernel, dim3(1), dim3(kThreads), 0, st, cu, chunk_offsets, d.N);
-  T* qn = l2norm ? reinterpret_cast<T*>(ws + L.qn) : nullptr;   // normalised q, written by the prep kernel
   float* rstd = reinterpret_cast<float*>(ws + L.rstd);
   float* G = reinterpret_cast<float*>(ws + L.G);
   T* Ai = with_backward ? reinterpret_cast<T*>(ws + L.Ai) : nullptr;
@@ -790,7 +794,7 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     constexpr int smem = PrepSmem<T, DK, BVP>::bytes;
     if (int e = set_lds(kern, smem)) return e;
     GDN_LAUNCH(kKernPrep, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, (const T*)v, g, beta, cu,
-               (const int*)chunk_offsets, G, Ai, W, UF, AQ, KTF, WF, KAF, QTF, qn, rstd, rstd + tok * d.Hqk, d.T, d.N, d.Hqk,
+               (const int*)chunk_offsets, G, Ai, W, UF, AQ, KTF, WF, KAF, QTF, rstd, rstd + tok * d.Hqk, d.T, d.N, d.Hqk,
                d.Hv, d.V, scale, l2norm, d.strides());
   }
   {
@@ -804,9 +808,9 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   auto launch_out = [&](auto kern, auto nm) -> int {
     constexpr int smem = OutSmem<T, DK, NW>::bytes;
     if (int e = set_lds(kern, smem)) return e;
-    GDN_LAUNCH(kKernOut, st, kern, dim3(nc, d.Hv, d.V / (32 * NW)), dim3(64 * NW), smem, st, l2norm ? (const T*)qn : qq,
+    GDN_LAUNCH(kKernOut, st, kern, dim3(nc, d.Hv, d.V / (32 * NW)), dim3(64 * NW), smem, st, qq,
                (const T*)AQ, (const T*)VF, (const T*)HF, (const float*)G, (T*)o, cu, (const int*)chunk_offsets, d.T, d.N, d.Hqk,
-               d.Hv, d.V, scale, l2norm ? (int64_t)d.Hqk * d.K : d.strides().q, nm);
+               d.Hv, d.V, scale, d.strides().q, l2norm ? (const float*)rstd : (const float*)nullptr, nm);
     return 0;
   };
   if (fn.y == nullptr) {

@@ -577,9 +577,10 @@ template <typename T>
 __device__ __forceinline__ void rows_request(RowPieces<T>& r, const T* g, int64_t row_stride, int rows_valid) {
   constexpr int V = Elem<T>::kVec, PPR = 32 / V;
   const int lane = threadIdx.x & 63;
+  if (rows_valid <= 0) return;   // wave-uniform; no row of the tile exists (its first row may lie past the tensor's end)
 #pragma unroll
   for (int i = 0; i < RowPieces<T>::kN; ++i) {
-    const int p = lane + 64 * i, row = imax(imin(p / PPR, rows_valid - 1), 0), cc = p % PPR;
+    const int p = lane + 64 * i, row = imin(p / PPR, rows_valid - 1), cc = p % PPR;
     r.y[i] = ld16(g + (int64_t)row * row_stride + cc * V);
   }
 }

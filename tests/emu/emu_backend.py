@@ -2,6 +2,7 @@
 
 This exists so that kernel indexing, LDS use and barriers can be checked on a machine without a GPU, with
 guard pages instead of GPU faults.  The shipped package never imports this module."""
+import contextlib
 import ctypes
 import os
 import sys
@@ -46,3 +47,20 @@ def guarded(t: torch.Tensor, at_end: bool = True) -> torch.Tensor:
     out = raw[: t.numel() * t.element_size()].view(t.dtype).view(t.shape)
     out.copy_(t)
     return out
+
+
+@contextlib.contextmanager
+def guarded_outputs():
+    """While active, every CPU tensor made by torch.empty (the operators allocate their outputs, gradients and
+    workspaces with it) ends flush against an inaccessible page, so that a kernel reading or writing past the end of
+    an output is a SIGSEGV here."""
+    real = torch.empty
+
+    def empty(*size, **kw):
+        t = real(*size, **kw)
+        return guarded(t) if t.device.type == "cpu" and t.numel() > 0 and not kw.get("pin_memory") else t
+    torch.empty = empty
+    try:
+        yield
+    finally:
+        torch.empty = real

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from tests import parity as P
-from tests.emu.emu_backend import emu_ops, guarded
+from tests.emu.emu_backend import emu_ops, guarded, guarded_outputs
 
 BF, F32 = torch.bfloat16, torch.float32
 
@@ -140,3 +140,15 @@ def test_chunk_random_shapes(ops, seed):
     """Seeded random shapes: ragged lengths, packed sequences with empty and one-token members, grouped heads."""
     dtype, B, T, Hqk, Hv, K, V, l2, cu = _random_case(seed)
     P.check_chunk(ops, "cpu", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu, backward=True, wrap=guarded, h0_std=0.1, seed=seed)
+
+
+@pytest.mark.parametrize("dtype,B,T,Hqk,Hv,K,V,cu", [
+    (BF, 1, 70, 1, 2, 64, 64, None),               # last chunk of 6 tokens: its second 32-row half does not exist
+    (BF, 1, 200, 2, 4, 128, 128, None),
+    (F32, 1, 97, 1, 2, 64, 64, [0, 33, 97]),
+])
+def test_chunk_backward_stays_inside_its_outputs(ops, dtype, B, T, Hqk, Hv, K, V, cu):
+    """Grouped heads (later value heads add to the dq, dk rows of the first) with a short last chunk, outputs and
+    workspace against guard pages: no kernel may touch rows past the end of dq, dk, dv."""
+    with guarded_outputs():
+        P.check_chunk(ops, "cpu", B, T, Hqk, Hv, K, V, dtype, cu=cu, backward=True, wrap=guarded, h0_std=0.1)
