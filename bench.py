@@ -37,8 +37,8 @@ CFG = dict(B=2, T=8192, Hqk=16, Hv=32, K=128, V=128, C=64)
 # (rocprofv3 --pmc, one run per counter, each scaled by what the same counter reads for a 512 MiB copy): the figures
 # of profiles/chunk_fwd_bwd_B2_T8192_bf16_hbm_traffic.md.  Measured offline, reported beside the live timings.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "chunk_prep_kernel": 1136386895, "chunk_state_kernel": 749425757, "chunk_out_kernel": 673376638,
-    "chunk_state_bwd_kernel": 884322839, "chunk_bwd_local_kernel": 1151905110,
+    "chunk_prep_kernel": 1052614045, "chunk_state_kernel": 749425750, "chunk_out_kernel": 676335796,
+    "chunk_state_bwd_kernel": 884322942, "chunk_bwd_local_kernel": 1194691190,
 }
 
 
@@ -67,10 +67,10 @@ def kernel_algorithmic_bytes(K, V, grp, e=2, C=64):
     cc = [64,64] tile, row = 64 fp32 values."""
     tk, tv, st, cc, row = C * K * e, C * V * e, K * V * e, C * C * e, C * 4
     return {
-        # v, g, beta -> G, Tm, Aq, -W, U, -W^T tiles; once per q/k group: q, k -> K^T, K, Q^T tiles, normalised q, 1/|q|, 1/|k|
-        "chunk_prep_kernel": tv + 2 * row + row + 2 * cc + tk + tv + tk + (2 * tk + 4 * tk + 2 * row) // grp,
+        # v, g, beta -> G, Tm, Aq, -W, U, -W^T tiles; once per q/k group: q, k -> K^T, K, Q^T tiles, 1/|q|, 1/|k|
+        "chunk_prep_kernel": tv + 2 * row + row + 2 * cc + tk + tv + tk + (2 * tk + 3 * tk + 2 * row) // grp,
         "chunk_state_kernel": tk + tk // grp + tv + row + tv + st,   # -W, K^T (per group), U, G -> v_new, state before the chunk
-        "chunk_out_kernel": tk // grp + cc + tv + st + row + tv,     # normalised q (per group), Aq, v_new, state, G -> o
+        "chunk_out_kernel": (tk + row) // grp + cc + tv + st + row + tv,   # q, 1/|q| (per group), Aq, v_new, state, G -> o
         # K, Q^T (per group), -W^T, Aq, dO, G -> dv_new, dS
         "chunk_state_bwd_kernel": 2 * tk // grp + tk + cc + tv + row + tv + st,
         # v_new, dv_new, dO, S, dS, v, K, q, Tm, row vectors -> dv, dg, dbeta, dq/dk (written by the first head of a
