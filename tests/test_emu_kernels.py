@@ -17,6 +17,14 @@ def ops():
     return emu_ops()
 
 
+@pytest.fixture(autouse=True)
+def _outputs_against_guard_pages():
+    """Every test here also runs with what the operators allocate themselves (outputs, gradients, workspaces)
+    flush against guard pages, not only the inputs the test hands in."""
+    with guarded_outputs():
+        yield
+
+
 @pytest.mark.parametrize("dtype,B,T,Hqk,Hv,K,V", [
     (F32, 2, 3, 1, 2, 64, 64), (BF, 2, 2, 2, 4, 128, 128), (F32, 1, 1, 1, 1, 128, 192), (BF, 1, 4, 1, 2, 256, 128),
 ])
@@ -150,5 +158,4 @@ def test_chunk_random_shapes(ops, seed):
 def test_chunk_backward_stays_inside_its_outputs(ops, dtype, B, T, Hqk, Hv, K, V, cu):
     """Grouped heads (later value heads add to the dq, dk rows of the first) with a short last chunk, outputs and
     workspace against guard pages: no kernel may touch rows past the end of dq, dk, dv."""
-    with guarded_outputs():
-        P.check_chunk(ops, "cpu", B, T, Hqk, Hv, K, V, dtype, cu=cu, backward=True, wrap=guarded, h0_std=0.1)
+    P.check_chunk(ops, "cpu", B, T, Hqk, Hv, K, V, dtype, cu=cu, backward=True, wrap=guarded, h0_std=0.1)
