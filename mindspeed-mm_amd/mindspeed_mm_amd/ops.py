@@ -129,9 +129,15 @@ class GdnOps:
 
     def chunk_gated_delta_rule_qkv(self, mixed_qkv, g, beta, num_k_heads, num_v_heads, head_k_dim, head_v_dim,
                                    scale=None, initial_state=None, output_final_state=False,
-                                   use_qk_l2norm_in_kernel=False, cu_seqlens=None):
+                                   use_qk_l2norm_in_kernel=False, cu_seqlens=None, gate=None, norm_weight=None,
+                                   norm_eps=1e-6):
         """chunk_gated_delta_rule on the unsplit [B,T,2 Hqk K + Hv V] output of the convolution: equal to splitting it
-        into q, k, v as modeling_qwen3_5.py:818-831 does and calling chunk_gated_delta_rule, without the copies."""
+        into q, k, v as modeling_qwen3_5.py:818-831 does and calling chunk_gated_delta_rule, without the copies.
+        With gate (the layer's z) and norm_weight the gated RMSNorm of modeling_qwen3_5.py:897-900 is applied inside
+        the output kernel (see chunk_gated_delta_rule_norm); q, k, v are then read in place as well, and a backward
+        pass returns their gradients through the split's own backward."""
+        if (gate is None) != (norm_weight is None):
+            raise ValueError("gate and norm_weight go together")
         if mixed_qkv.dim() != 3 or mixed_qkv.shape[-1] < 2 * num_k_heads * head_k_dim + num_v_heads * head_v_dim:
             raise ValueError("expected mixed_qkv [B, T, D] with D >= 2 * num_k_heads * head_k_dim + num_v_heads * head_v_dim")
         if mixed_qkv.dtype not in (torch.float32, torch.bfloat16):
@@ -151,6 +157,14 @@ class GdnOps:
         if scale is None:
             scale = head_k_dim ** -0.5
         self._need(mixed_qkv, g, beta, initial_state, cu_seqlens)
+        if gate is not None:
+            B, T = mixed_qkv.shape[:2]
+            nq, nv = num_k_heads * head_k_dim, num_v_heads * head_v_dim
+            q, k, v = mixed_qkv[..., :nq], mixed_qkv[..., nq:2 * nq], mixed_qkv[..., 2 * nq:2 * nq + nv]
+            return self.chunk_gated_delta_rule_norm(
+                q.unflatten(-1, (num_k_heads, head_k_dim)), k.unflatten(-1, (num_k_heads, head_k_dim)),
+                v.unflatten(-1, (num_v_heads, head_v_dim)), g, beta, gate, norm_weight, norm_eps, scale, initial_state,
+                output_final_state, use_qk_l2norm_in_kernel, cu_seqlens)
         mixed_qkv, g, beta, initial_state = self._no_grad_views(mixed_qkv, g, beta, initial_state)
         return _ChunkGatedDeltaRuleQKV.apply(mixed_qkv, g, beta, int(num_k_heads), int(num_v_heads), int(head_k_dim),
                                              int(head_v_dim), float(scale), initial_state, bool(output_final_state),
@@ -681,10 +695,10 @@ def chunk_gated_delta_rule_norm(q, k, v, g, beta, gate, norm_weight, eps=1e-6, s
 
 def chunk_gated_delta_rule_qkv(mixed_qkv, g, beta, num_k_heads, num_v_heads, head_k_dim, head_v_dim, scale=None,
                                initial_state=None, output_final_state=False, use_qk_l2norm_in_kernel=False,
-                               cu_seqlens=None):
+                               cu_seqlens=None, gate=None, norm_weight=None, norm_eps=1e-6):
     return _default_ops().chunk_gated_delta_rule_qkv(mixed_qkv, g, beta, num_k_heads, num_v_heads, head_k_dim,
                                                      head_v_dim, scale, initial_state, output_final_state,
-                                                     use_qk_l2norm_in_kernel, cu_seqlens)
+                                                     use_qk_l2norm_in_kernel, cu_seqlens, gate, norm_weight, norm_eps)
 
 
 def gdn_gates(a, b, A_log, dt_bias):

@@ -247,6 +247,43 @@ def check_chunk_norm(ops, device, B, T, Hqk, Hv, K, V, dtype, l2=True, cu=None, 
     return errs
 
 
+def check_chunk_qkv_norm(ops, device, B, T, Hqk, Hv, K, V, dtype, l2=True, cu=None, backward=True, seed=0,
+                         wrap=lambda t: t, **recipe):
+    """The layer's sequence convolution output -> rule -> gated norm in one call on the unsplit tensor, bit for bit
+    against the rule on the unsplit tensor followed by the norm operator (each checked against the oracle on its own)."""
+    N = (len(cu) - 1) if cu is not None else B
+    x = gdn_inputs(B, T, Hqk, Hv, K, V, dtype, seed=seed, N=N, l2norm_in_kernel=l2, **recipe)
+    gen = torch.Generator().manual_seed(seed + 5)
+    nq, nv = Hqk * K, Hv * V
+    mixed = torch.cat([x["q"].reshape(B, T, nq), x["k"].reshape(B, T, nq), x["v"].reshape(B, T, nv)], dim=-1)
+    z = (1.5 * torch.randn(B, T, nv, generator=gen)).to(dtype)
+    w = (1.0 + 0.2 * torch.randn(V, generator=gen)).to(dtype)
+    dy = torch.randn(B, T, Hv, V, generator=gen).to(dtype)
+    cu_t = torch.tensor(cu, dtype=torch.int64, device=device) if cu is not None else None
+
+    def leaves():
+        L = dict(mx=wrap(mixed.to(device)).clone(), z=wrap(z.to(device)).clone(), w=wrap(w.to(device)).clone(),
+                 g=wrap(x["g"].to(device)).clone(), beta=wrap(x["beta"].to(device)).clone(),
+                 h0=wrap(x["h0"].to(device)).clone())
+        return {n: t.requires_grad_(backward) for n, t in L.items()}
+    A, Bc = leaves(), leaves()
+    y, ht = ops.chunk_gated_delta_rule_qkv(A["mx"], A["g"], A["beta"], Hqk, Hv, K, V, initial_state=A["h0"],
+                                           output_final_state=True, use_qk_l2norm_in_kernel=l2, cu_seqlens=cu_t,
+                                           gate=A["z"], norm_weight=A["w"])
+    o2, ht2 = ops.chunk_gated_delta_rule_qkv(Bc["mx"], Bc["g"], Bc["beta"], Hqk, Hv, K, V, initial_state=Bc["h0"],
+                                             output_final_state=True, use_qk_l2norm_in_kernel=l2, cu_seqlens=cu_t)
+    y2 = ops.rms_norm_gated(o2.reshape(-1, V), Bc["z"].reshape(-1, V), Bc["w"], 1e-6).view(B, T, Hv, V)
+    assert y.shape == (B, T, Hv, V) and torch.equal(y, y2) and torch.equal(ht, ht2)
+    if backward:
+        dyd = wrap(dy.to(device)).float()
+        (y.float() * dyd).sum().backward()
+        (y2.float() * dyd).sum().backward()
+        for n in A:
+            assert A[n].grad is not None and A[n].grad.shape == A[n].shape and A[n].grad.dtype == A[n].dtype, n
+            assert torch.equal(A[n].grad, Bc[n].grad), f"gradient of {n} differs from the two operators in sequence"
+    return {"y_max": y.detach().float().abs().max().item()}
+
+
 def check_gdn_gates(ops, device, shape, Hv, dtype, param_dtype=None, seed=0, backward=True, wrap=lambda t: t):
     """Gate recipe against the oracle on the same (dtype-valued) inputs.  g is fp32 on both sides (relative 1e-4 of
     the largest value, the fp32 bar); beta and the gradients in half precision carry one rounding to bf16."""

@@ -108,6 +108,14 @@ def test_chunk_with_fused_norm(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu, wdt, bwd
                        wrap=guarded, h0_std=0.1)
 
 
+@pytest.mark.parametrize("dtype,B,T,Hqk,Hv,K,V,l2,cu,bwd", [
+    (BF, 1, 100, 1, 2, 64, 128, True, None, True),
+    (BF, 1, 140, 2, 4, 64, 64, False, [0, 5, 70, 71, 140], False),
+])
+def test_chunk_on_unsplit_qkv_with_fused_norm(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu, bwd):
+    P.check_chunk_qkv_norm(ops, "cpu", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu, backward=bwd, wrap=guarded, h0_std=0.1)
+
+
 @pytest.mark.parametrize("dtype,shape,Hv,pdt", [
     (F32, (2, 37), 6, None), (BF, (1, 300), 32, None), (BF, (3, 5), 48, torch.float32), (F32, (1,), 256, None),
     (BF, (1100,), 4, None),

@@ -145,6 +145,16 @@ def test_chunk_with_fused_norm(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu, wdt, bwd
                        h0_std=0.1)
 
 
+@pytest.mark.parametrize("dtype,B,T,Hqk,Hv,K,V,l2,cu,bwd", [
+    (BF, 2, 200, 2, 4, 128, 128, True, None, True),
+    (BF, 1, 512, 4, 8, 128, 128, True, [0, 100, 101, 512], False),
+    (F32, 1, 100, 1, 2, 64, 64, True, None, True),
+])
+def test_chunk_on_unsplit_qkv_with_fused_norm(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu, bwd):
+    print(f"chunk qkv+norm {dtype} B{B} T{T} Hqk{Hqk} Hv{Hv} K{K} V{V} l2={l2} varlen={cu is not None} bwd={bwd}", flush=True)
+    P.check_chunk_qkv_norm(ops, "cuda", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu, backward=bwd, h0_std=0.1)
+
+
 def test_fused_norm_rejects_other_head_dims(ops):
     q = torch.randn(1, 64, 1, 64, device="cuda", dtype=BF)
     v = torch.randn(1, 64, 1, 256, device="cuda", dtype=BF)
