@@ -419,7 +419,7 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ?
   static_assert(64 * (DK / VEC) % NT == 0 && (NW * 2048 / VEC) % NT == 0, "tile chunks must divide over the loaders");
   static_assert(STAGES == 1 || STAGES == 2, "one or two LDS stages");
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31;
+  const int tid = threadIdx.x, wave = tid >> 6;
   const int nh = xcd_grouped_head(blockIdx.x, gridDim.x, Hv / Hqk), n = nh / Hv, h = nh % Hv;
   const int64_t bos = cu ? cu[n] : (int64_t)n * T_len;
   const int len = cu ? (int)(cu[n + 1] - bos) : T_len;
@@ -435,7 +435,6 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ?
     Vec16<T> pw[DEPTH][CW], pk[DEPTH][CW], pu[DEPTH][CUL];
     float glast[DEPTH], pdec[DEPTH];
     auto issue = [&](int c, int set) {      // global -> registers
-      const int64_t tok0 = bos + (int64_t)c * kChunk;
       const int nvalid = imin(kChunk, len - c * kChunk);
 #pragma unroll
       for (int i = 0; i < CW; ++i) {
