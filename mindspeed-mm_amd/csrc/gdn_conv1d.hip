@@ -181,16 +181,21 @@ __global__ __launch_bounds__(kConvThreads) void conv1d_bwd_kernel(
   // t runs W-1 steps past the last dyp so that the final dx of the tile are flushed.  W tokens per trip: the windows
   // win (x[t-(W-1)+j]) and dyw (dyp[s+u], s = t-(W-1)) are rings whose logical index j sits in slot (uu + j) % W at
   // the uu-th token of a trip, so sliding a window moves no register.
-  for (int64_t tb = t0; tb < t1 + (W - 1); tb += W) {
-    Vec16<T> xr[W], gr[W];
+  // The rows of a trip are requested one trip ahead (two register sets, the loop runs two trips per turn), the same
+  // loads on every path: rows past the end repeat the last one and are never used.
+  auto request = [&](Vec16<T> (&xr)[W], Vec16<T> (&gr)[W], int64_t tb) {
 #pragma unroll
     for (int u = 0; u < W; ++u) {
-      if (tb + u < tend) { xr[u] = ld16(x + (tb + u) * D + d0); gr[u] = ld16(dy + (tb + u) * D + d0); }
+      const int64_t row = tb + u < total ? tb + u : total - 1;
+      xr[u] = ld16(x + row * D + d0);
+      gr[u] = ld16(dy + row * D + d0);
     }
+  };
+  auto trip = [&](int64_t tb, const Vec16<T> (&xr)[W], const Vec16<T> (&gr)[W]) {
 #pragma unroll
     for (int uu = 0; uu < W; ++uu) {
       const int64_t t = tb + uu;
-      if (t >= t1 + (W - 1)) break;
+      if (t >= t1 + (W - 1)) return;
       constexpr int kNewest = W - 1;
       float* newest_x = win[(uu + kNewest) % W];
       float* newest_g = dyw[(uu + kNewest) % W];
@@ -248,6 +253,15 @@ __global__ __launch_bounds__(kConvThreads) void conv1d_bwd_kernel(
         store_chan(dx + s_ * D + d0, out);
       }
     }
+  };
+  Vec16<T> xa[W], ga[W], xb[W], gb[W];
+  request(xa, ga, t0);
+  for (int64_t tb = t0; tb < t1 + (W - 1); tb += 2 * W) {
+    request(xb, gb, tb + W);
+    trip(tb, xa, ga);
+    if (tb + W >= t1 + (W - 1)) break;
+    request(xa, ga, tb + 2 * W);
+    trip(tb + W, xb, gb);
   }
   float* pp = part + (int64_t)blockIdx.y * (W + 1) * D;
 #pragma unroll
