@@ -665,16 +665,25 @@ __global__ __launch_bounds__(64 * NW) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 2)
   Af[2].load(aqf + (ch * 4 + 3) * 1024);
   // q arrives raw; with the in-kernel l2 norm its rows are scaled by the 1/|q| the prep kernel left (the same fp32
   // product and rounding it applied itself: no normalised copy of q is kept in memory)
-  for (int c = tid; c < 64 * (DK / VEC); c += NT) {
-    const int row = c / (DK / VEC), cc = c % (DK / VEC);
+  constexpr int QPT = 64 * (DK / VEC) / NT;   // pieces of the Q tile per thread: all requested before the first is used
+  static_assert(64 * (DK / VEC) % NT == 0, "every thread takes the same number of pieces of the Q tile");
+  Vec16<T> qreg[QPT];
+  float qs[QPT];
+#pragma unroll
+  for (int i = 0; i < QPT; ++i) {
+    const int c = tid + i * NT, row = imin(c / (DK / VEC), nvalid - 1), cc = c % (DK / VEC);
+    qreg[i] = ld16(q + (tok0 + row) * q_stride + hq * DK + cc * VEC);
+    qs[i] = rstd_q != nullptr ? rstd_q[(tok0 + row) * Hqk + hq] : 1.f;
+  }
+  const float gval = G[ch * 64 + imin(tid & 63, nvalid - 1)];
+#pragma unroll
+  for (int i = 0; i < QPT; ++i) {
+    const int c = tid + i * NT, row = c / (DK / VEC), cc = c % (DK / VEC);
     Vec16<T> x = zero16<T>();
-    if (row < nvalid) {
-      x = ld16(q + (tok0 + row) * q_stride + hq * DK + cc * VEC);
-      if (rstd_q != nullptr) x = scale16<T>(x, rstd_q[(tok0 + row) * Hqk + hq]);
-    }
+    if (row < nvalid) x = rstd_q != nullptr ? scale16<T>(qreg[i], qs[i]) : qreg[i];
     st16(Qs + row * LDK + cc * VEC, x);
   }
-  if (tid < 64) Eg[tid] = scale * __expf(G[ch * 64 + imin(tid, nvalid - 1)]);
+  if (tid < 64) Eg[tid] = scale * __expf(gval);
   IdentityFrag<T> id;
   id.init();
 #pragma unroll
