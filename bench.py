@@ -37,8 +37,8 @@ CFG = dict(B=2, T=8192, Hqk=16, Hv=32, K=128, V=128, C=64)
 # (rocprofv3 --pmc, one run per counter, each scaled by what the same counter reads for a 512 MiB copy): the figures
 # of profiles/chunk_fwd_bwd_B2_T8192_bf16_hbm_traffic.md.  Measured offline, reported beside the live timings.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "chunk_prep_kernel": 1054227566, "chunk_state_kernel": 749425754, "chunk_out_kernel": 692627090,
-    "chunk_state_bwd_kernel": 884322953, "chunk_bwd_local_kernel": 1190265533,
+    "chunk_prep_kernel": 1042433488, "chunk_state_kernel": 749425775, "chunk_out_kernel": 682825408,
+    "chunk_state_bwd_kernel": 884322958, "chunk_bwd_local_kernel": 1156464169,
 }
 
 

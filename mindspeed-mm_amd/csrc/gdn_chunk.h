@@ -31,7 +31,7 @@ struct ChunkDims {
 // Byte offsets into the workspace.  Everything the backward pass re-reads is written by the forward.
 struct ChunkWorkspace {
   int64_t chunk_offsets;  // int32 [N+1]      chunks before each packed sequence
-  int64_t rstd;           // f32 [2][tokens,Hqk] 1/|q|, 1/|k| of that normalisation
+  int64_t rstd;           // f32 [2][chunks,Hqk,64] 1/|q|, 1/|k| of the in-kernel l2 norm, 64 contiguous values per chunk
   int64_t G;              // f32 [chunks,Hv,64]      chunk-local cumulative log decay
   int64_t WAF;            // T [chunks,Hv,K/32,2]    -W as A operand: tile = (32 tokens) x (32 columns of K), fragment order
   int64_t AQ;             // T [chunks,Hv,2,2]       scale tril(Q K^T . Gam), accumulator tiles: lane <-> column, registers <-> row
@@ -56,9 +56,9 @@ inline ChunkWorkspace chunk_workspace_layout(const ChunkDims& d, int elem_bytes)
   ChunkWorkspace w;
   int64_t off = 0;
   auto take = [&](int64_t bytes) { int64_t o = off; off += align256(bytes); return o; };
-  const int64_t tok = d.tokens(), nc = d.max_chunks();
+  const int64_t nc = d.max_chunks();
   w.chunk_offsets = take((int64_t)(d.N + 1) * 4);
-  w.rstd = take(2 * tok * d.Hqk * 4);
+  w.rstd = take(2 * nc * 64 * d.Hqk * 4);
   w.G = take(nc * 64 * d.Hv * 4);
   w.WAF = take(nc * 64 * d.Hv * d.K * elem_bytes);
   w.AQ = take(nc * 64 * d.Hv * 64 * elem_bytes);

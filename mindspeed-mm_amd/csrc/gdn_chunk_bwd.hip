@@ -394,8 +394,8 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     const float gv = G[ch * 64 + tc], bv = beta[(tok0 + tc) * Hv + h];
     float rq1 = 1.f, rk1v = 1.f;
     if (l2) {
-      rq1 = rstd_q[(tok0 + tc) * Hqk + hq];
-      rk1v = rstd_k[(tok0 + tc) * Hqk + hq];
+      rq1 = rstd_q[((int64_t)blockIdx.x * Hqk + hq) * 64 + tc];
+      rk1v = rstd_k[((int64_t)blockIdx.x * Hqk + hq) * 64 + tc];
     }
     Gs[tid] = gv;
     egs[tid] = __expf(gv);
@@ -737,7 +737,6 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
                             const float* beta, const int64_t* cu, const void* dO, const float* dht, void* dq, void* dk,
                             void* dv, float* dg, float* dbeta, float* dh0, unsigned char* ws, float scale, int l2norm,
                             hipStream_t st) {
-  const int64_t tok = d.tokens();
   const int nc = (int)d.max_chunks();
   const int* chunk_offsets = reinterpret_cast<const int*>(ws + L.chunk_offsets);
   (void)q; (void)k;   // q and k reach the backward kernels as the forward pass's fragment tiles
@@ -752,7 +751,7 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   T* DVF = reinterpret_cast<T*>(ws + L.DVF);
   T* DHF = reinterpret_cast<T*>(ws + L.DHF);
   const float* rstd_q = l2norm ? reinterpret_cast<const float*>(ws + L.rstd) : nullptr;
-  const float* rstd_k = l2norm ? rstd_q + tok * d.Hqk : nullptr;
+  const float* rstd_k = l2norm ? rstd_q + (int64_t)nc * 64 * d.Hqk : nullptr;
   {
     auto kern = chunk_state_bwd_kernel<T, DK, NWS, NLS, STAGES>;
     constexpr int smem = StateBwdSmem<T, DK, NWS, STAGES>::bytes;

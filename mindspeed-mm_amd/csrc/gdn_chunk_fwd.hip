@@ -169,9 +169,9 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
     // q and k arrive raw; with the in-kernel l2 norm they are normalised on the way into LDS.  The first value head
     // of each q/k group also leaves 1/|q|, 1/|k| (for the output kernel, which scales q itself, and the backward pass).
     const bool keep = l2norm && (h % (Hv / Hqk)) == 0;
-    const int64_t roff = tok0 * Hqk + hq;
-    tile_qk_finish<T, DK>(kt, Ks, LDK, nvalid, tid, l2norm != 0, nullptr, 0, keep ? rstd_k_out + roff : nullptr, Hqk);
-    tile_qk_finish<T, DK>(qt, Qs, LDK, nvalid, tid, l2norm != 0, nullptr, 0, keep ? rstd_q_out + roff : nullptr, Hqk);
+    const int64_t roff = ((int64_t)blockIdx.x * Hqk + hq) * 64;   // 64 contiguous values per chunk and q/k head
+    tile_qk_finish<T, DK>(kt, Ks, LDK, nvalid, tid, l2norm != 0, nullptr, 0, keep ? rstd_k_out + roff : nullptr, 1);
+    tile_qk_finish<T, DK>(qt, Qs, LDK, nvalid, tid, l2norm != 0, nullptr, 0, keep ? rstd_q_out + roff : nullptr, 1);
   }
   GDN_LDS_BARRIER();
 
@@ -673,7 +673,7 @@ __global__ __launch_bounds__(64 * NW) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 2)
   for (int i = 0; i < QPT; ++i) {
     const int c = tid + i * NT, row = imin(c / (DK / VEC), nvalid - 1), cc = c % (DK / VEC);
     qreg[i] = ld16(q + (tok0 + row) * q_stride + hq * DK + cc * VEC);
-    qs[i] = rstd_q != nullptr ? rstd_q[(tok0 + row) * Hqk + hq] : 1.f;
+    qs[i] = rstd_q != nullptr ? rstd_q[((int64_t)blockIdx.x * Hqk + hq) * 64 + row] : 1.f;
   }
   const float gval = G[ch * 64 + imin(tid & 63, nvalid - 1)];
 #pragma unroll
@@ -779,7 +779,6 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
                             const float* g, const float* beta, const float* h0, const int64_t* cu, void* o, float* ht,
                             unsigned char* ws, float scale, int l2norm, bool with_backward, const FwdNorm& fn,
                             hipStream_t st) {
-  const int64_t tok = d.tokens();
   const int nc = (int)d.max_chunks();
   int* chunk_offsets = reinterpret_cast<int*>(ws + L.chunk_offsets);
   const T* qq = (const T*)q;
@@ -802,7 +801,7 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     constexpr int smem = PrepSmem<T, DK, BVP>::bytes;
     if (int e = set_lds(kern, smem)) return e;
     GDN_LAUNCH(kKernPrep, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, (const T*)v, g, beta, cu,
-               (const int*)chunk_offsets, G, Ai, W, UF, AQ, KTF, WF, KAF, QTF, rstd, rstd + tok * d.Hqk, d.T, d.N, d.Hqk,
+               (const int*)chunk_offsets, G, Ai, W, UF, AQ, KTF, WF, KAF, QTF, rstd, rstd + (int64_t)nc * 64 * d.Hqk, d.T, d.N, d.Hqk,
                d.Hv, d.V, scale, l2norm, d.strides());
   }
   {
