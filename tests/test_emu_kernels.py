@@ -167,3 +167,25 @@ def test_chunk_backward_stays_inside_its_outputs(ops, dtype, B, T, Hqk, Hv, K, V
     """Grouped heads (later value heads add to the dq, dk rows of the first) with a short last chunk, outputs and
     workspace against guard pages: no kernel may touch rows past the end of dq, dk, dv."""
     P.check_chunk(ops, "cpu", B, T, Hqk, Hv, K, V, dtype, cu=cu, backward=True, wrap=guarded, h0_std=0.1)
+
+
+def _random_conv_case(seed):
+    import random
+    rng = random.Random(1000 + seed)
+    dtype = rng.choice([BF, F32, BF])
+    B, T, W = rng.choice([1, 1, 2, 3]), rng.randint(1, 300), rng.randint(1, 8)
+    D = rng.choice([8, 16, 64, 72, 256])
+    cu = None
+    if B == 1 and rng.random() < 0.6:
+        cuts = sorted(rng.sample(range(0, T + 1), min(T + 1, rng.randint(0, 5))))
+        cu = [0] + cuts + [T]
+    return dict(B=B, T=T, D=D, W=W, dtype=dtype, cu=cu, residual=rng.random() < 0.5, bias=rng.random() < 0.7,
+                state=rng.random() < 0.7, activation=rng.choice(["silu", None]), seed=seed)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_conv1d_random_shapes(ops, seed):
+    """Seeded random shapes of the convolution: widths 1..8, ragged and packed lengths, with and without bias,
+    residual, initial state and activation."""
+    c = _random_conv_case(seed)
+    P.check_conv(ops, "cpu", c.pop("B"), c.pop("T"), c.pop("D"), c.pop("W"), c.pop("dtype"), wrap=guarded, **c)

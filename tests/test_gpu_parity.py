@@ -301,3 +301,12 @@ def test_no_grad_forward_prepares_no_backward(ops):
                                             output_final_state=True, use_qk_l2norm_in_kernel=True)
     assert o1.requires_grad and not o2.requires_grad and o2.grad_fn is None
     assert torch.equal(o1, o2) and torch.equal(h1, h2)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_conv1d_random_shapes(ops, seed):
+    """The seeded random convolution shapes of the CPU emulation tests (and more seeds), on the device build."""
+    from tests.test_emu_kernels import _random_conv_case
+    c = _random_conv_case(seed)
+    print(f"conv random {seed}: {c}", flush=True)
+    P.check_conv(ops, "cuda", c.pop("B"), c.pop("T"), c.pop("D"), c.pop("W"), c.pop("dtype"), **c)
