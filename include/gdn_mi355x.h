@@ -150,6 +150,16 @@ int gdn_gate_bwd(const void* a, const void* b, const void* A_log, const void* dt
                  const void* dbeta, void* da, void* db, float* dA_log, float* ddt_bias, void* workspace,
                  int64_t workspace_bytes, int64_t tokens, int Hv, int dtype, int param_dtype, void* stream);
 
+/* gdn_gate_bwd without the workspace argument.  No counterpart in the reference: it exists for callers that cannot
+ * allocate device memory around the call (a step under HIP graph capture, a loop whose harness forbids hipMalloc).
+ * The per-workgroup partial sums live in a 1 MiB buffer inside the library (one per device, held until the process
+ * ends), which limits Hv to 128 (-3 beyond); any number of tokens is accepted.  Same kernels and same order of
+ * additions as gdn_gate_bwd: identical results.  Calls that overlap on one device (two streams) share that buffer and
+ * race; calls on one stream are ordered.  Nothing is allocated, freed or synchronised. */
+int gdn_gate_bwd_noalloc(const void* a, const void* b, const void* A_log, const void* dt_bias, const float* dg,
+                         const void* dbeta, void* da, void* db, float* dA_log, float* ddt_bias, int64_t tokens, int Hv,
+                         int dtype, int param_dtype, void* stream);
+
 /* -------- per-kernel timing ------------------------------------------------------------------------
  * op-level counterpart of the reference's step profiler (mindspeed_mm/fsdp/tools/profiler.py:32-147).
  * While enabled, every kernel launch of this library is bracketed by HIP events on its stream (this mode

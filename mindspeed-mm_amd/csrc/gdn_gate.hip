@@ -11,7 +11,15 @@
 #include "gdn_common.h"
 #include "gdn_profile.h"
 
+#include <mutex>
+
 namespace gdn {
+
+// Partial sums of gdn_gate_bwd_noalloc: [workgroups <= 1024][2][Hv <= kGateNoAllocMaxHv] fp32, 1 MiB per device, held
+// until the process ends.  Every slot a launch reads has been written by the same launch, so nothing needs clearing.
+constexpr int kGateNoAllocMaxHv = 128;
+constexpr int kGateMaxBlocks = 1024;
+static __device__ __align__(256) float gate_scratch[kGateMaxBlocks * 2 * kGateNoAllocMaxHv];
 
 template <typename T> __device__ __forceinline__ float gate_ld(const T* p, int64_t i) { return Elem<T>::to_f(p[i]); }
 __device__ __forceinline__ float gate_sigmoid(float x) { return 1.f / (1.f + expf(-x)); }
@@ -81,7 +89,7 @@ __global__ __launch_bounds__(kThreads) void gate_reduce_kernel(const float* __re
 static int gate_bwd_blocks(int64_t tokens, int Hv) {
   const int rows = kThreads / Hv;
   const int64_t need = (tokens + rows - 1) / rows;
-  return (int)(need < 1024 ? (need > 0 ? need : 1) : 1024);
+  return (int)(need < kGateMaxBlocks ? (need > 0 ? need : 1) : kGateMaxBlocks);
 }
 
 template <typename T, typename TP>
@@ -141,6 +149,45 @@ extern "C" int gdn_gate_bwd(const void* a, const void* b, const void* A_log, con
   if (workspace_bytes < gdn_gate_bwd_workspace_bytes(tokens, Hv)) return -5;
   hipStream_t st = (hipStream_t)stream;
   float* part = static_cast<float*>(workspace);
+  if (dtype == 0)
+    return gate_bwd_launch<float, float>(a, b, A_log, dt_bias, dg, dbeta, da, db, dA_log, ddt_bias, part, tokens, Hv, st);
+  if (param_dtype == 1)
+    return gate_bwd_launch<bf16_t, bf16_t>(a, b, A_log, dt_bias, dg, dbeta, da, db, dA_log, ddt_bias, part, tokens, Hv, st);
+  return gate_bwd_launch<bf16_t, float>(a, b, A_log, dt_bias, dg, dbeta, da, db, dA_log, ddt_bias, part, tokens, Hv, st);
+}
+
+namespace gdn {
+// Device address of gate_scratch on the current device.  In host code the array's name is only a handle: the address
+// a kernel may use comes from hipGetSymbolAddress, once per device (each device holds its own copy).
+static int gate_scratch_ptr(float** out) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static float* ptrs[kMaxDevices] = {};
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev)) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return -2;
+  std::lock_guard<std::mutex> lk(mu);
+  if (ptrs[dev] == nullptr) {
+    void* p = nullptr;
+    if (hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(gate_scratch))) return (int)e;
+    if (p == nullptr) return -1;
+    ptrs[dev] = static_cast<float*>(p);
+  }
+  *out = ptrs[dev];
+  return 0;
+}
+}  // namespace gdn
+
+extern "C" int gdn_gate_bwd_noalloc(const void* a, const void* b, const void* A_log, const void* dt_bias,
+                                    const float* dg, const void* dbeta, void* da, void* db, float* dA_log,
+                                    float* ddt_bias, int64_t tokens, int Hv, int dtype, int param_dtype, void* stream) {
+  using namespace gdn;
+  if (!a || !b || !A_log || !dt_bias || !dg || !dbeta || !da || !db || !dA_log || !ddt_bias) return -1;
+  if (int e = gate_check(tokens, Hv, dtype, param_dtype)) return e;
+  if (Hv > kGateNoAllocMaxHv) return -3;   // the partial sums would not fit the library's own buffer
+  float* part = nullptr;
+  if (int e = gate_scratch_ptr(&part)) return e;
+  hipStream_t st = (hipStream_t)stream;
   if (dtype == 0)
     return gate_bwd_launch<float, float>(a, b, A_log, dt_bias, dg, dbeta, da, db, dA_log, ddt_bias, part, tokens, Hv, st);
   if (param_dtype == 1)
