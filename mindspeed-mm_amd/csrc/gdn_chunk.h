@@ -29,22 +29,18 @@ struct ChunkDims {
 };
 
 // Byte offsets into the workspace.  Everything the backward pass re-reads is written by the forward.
+// Tiles exchanged between kernels are in fragment order (see AccB<>): 1024 elements per 32x32 tile.
 struct ChunkWorkspace {
   int64_t chunk_offsets;  // int32 [N+1]      chunks before each packed sequence
   int64_t rstd;           // f32 [2][chunks,Hqk,64] 1/|q|, 1/|k| of the in-kernel l2 norm, 64 contiguous values per chunk
   int64_t G;              // f32 [chunks,Hv,64]      chunk-local cumulative log decay
-  int64_t WAF;            // T [chunks,Hv,K/32,2]    -W as A operand: tile = (32 tokens) x (32 columns of K), fragment order
+  int64_t Ai;             // T [chunks,Hv,2,2]       Tm = (I + L)^-1 as A operand: tile = (32 rows) x (32 columns)
   int64_t AQ;             // T [chunks,Hv,2,2]       scale tril(Q K^T . Gam), accumulator tiles: lane <-> column, registers <-> row
-  // Tiles exchanged between kernels in fragment order (see AccB<>): 1024 elements per 32x32 tile.
-  int64_t KTF;            // T [chunks,Hqk,K/32,2]   K^T as A operand: tile = (32 columns of K) x (32 tokens)
-  int64_t UF;             // T [chunks,Hv,V/32,2]    U,            tile = (32-token block ri) x (32-column block)
-  int64_t VF;             // T [chunks,Hv,V/32,2]    v_new = U - W S
+  int64_t KAF;            // T [chunks,Hqk,K/32,2]   K as A operand: tile = (32 tokens) x (32 columns of K)
+  int64_t QTF;            // T [chunks,Hqk,K/32,2]   Q^T as A operand: tile = (32 columns of K) x (32 tokens)
+  int64_t VF;             // T [chunks,Hv,V/32,2]    v_new = Tm (beta v - beta e^G K S), tile = (32-column block) x (32-token block)
   int64_t HF;             // T [chunks,Hv,V/32,K/32] state BEFORE each chunk, tile = (32 rows of K) x (32 columns of V)
   int64_t fwd_bytes;
-  int64_t Ai;             // T [chunks,Hv,2,2]       (I + A)^-1 as A operand: tile = (32 rows) x (32 columns), fragment order
-  int64_t WF;             // T [chunks,Hv,K/32,2]    -W^T as A operand (written by the forward when a backward follows)
-  int64_t QTF;            // T [chunks,Hqk,K/32,2]   Q^T as A operand: tile = (32 columns of K) x (32 tokens)
-  int64_t KAF;            // T [chunks,Hqk,K/32,2]   K as A operand: tile = (32 tokens) x (32 columns of K)
   int64_t DVF;            // T [chunks,Hv,V/32,2]    d(v_new)
   int64_t DHF;            // T [chunks,Hv,V/32,K/32] gradient of the state AFTER each chunk
   int64_t total_bytes;
@@ -60,17 +56,13 @@ inline ChunkWorkspace chunk_workspace_layout(const ChunkDims& d, int elem_bytes)
   w.chunk_offsets = take((int64_t)(d.N + 1) * 4);
   w.rstd = take(2 * nc * 64 * d.Hqk * 4);
   w.G = take(nc * 64 * d.Hv * 4);
-  w.WAF = take(nc * 64 * d.Hv * d.K * elem_bytes);
+  w.Ai = take(nc * 64 * d.Hv * 64 * elem_bytes);
   w.AQ = take(nc * 64 * d.Hv * 64 * elem_bytes);
-  w.KTF = take(nc * 64 * d.Hqk * d.K * elem_bytes);
-  w.UF = take(nc * 64 * d.Hv * d.V * elem_bytes);
+  w.KAF = take(nc * 64 * d.Hqk * d.K * elem_bytes);
+  w.QTF = take(nc * 64 * d.Hqk * d.K * elem_bytes);
   w.VF = take(nc * 64 * d.Hv * d.V * elem_bytes);
   w.HF = take(nc * d.Hv * d.V * d.K * elem_bytes);
   w.fwd_bytes = off;
-  w.Ai = take(nc * 64 * d.Hv * 64 * elem_bytes);
-  w.WF = take(nc * 64 * d.Hv * d.K * elem_bytes);
-  w.QTF = take(nc * 64 * d.Hqk * d.K * elem_bytes);
-  w.KAF = take(nc * 64 * d.Hqk * d.K * elem_bytes);
   w.DVF = take(nc * 64 * d.Hv * d.V * elem_bytes);
   w.DHF = take(nc * d.Hv * d.V * d.K * elem_bytes);
   w.total_bytes = off;

@@ -24,112 +24,126 @@ namespace gdn {
 // ---------------------------------------------------------------------------------------------
 // chunk_state_bwd_kernel: the reverse recurrence, mirror of chunk_state_kernel.  One compute wave owns a 32-column
 // slab of dS[K, 32] in fp32 accumulators and per chunk (last to first) does
-//     dV' = (e^{G_last-G} . K) dS + dv_local          dS <- e^{G_last} dS + Q^T (scale e^G . dO) - W^T dV'
-// with dS and dV' used as B operands straight from accumulator registers.  dS (gradient of the state AFTER the
-// chunk) and dV' leave in fragment order.  Loader waves copy the A operands (K, Q^T, W^T: `big` stages) from
-// contiguous fragment-order blocks, and the `small` stage: the slab's dO rows as they lie in memory plus the
-// forward pass's tril(Q K^T . Gam) tiles, from which the compute waves form dv_local = scale Aq^T dO themselves.
+//     dV' = e^{G_last-G} . (K dS) + (scale Aq)^T dO
+//     R = Tm^T dV'        dS <- e^{G_last} dS + Q^T (scale e^G . dO) - K^T (beta e^G . R)
+// (the last term is W^T dV' with W = Tm (beta e^G K) never materialised), dS, dV', R and the scaled dO used as B
+// operands straight from registers.  dS (gradient of the state AFTER the chunk) and dV' leave in fragment order.
+// Loader waves copy the A operands from contiguous fragment-order blocks: K and Q^T per q/k group, Tm and Aq per value
+// head; K^T and Tm^T are the same images read with the transposing LDS read, and so are the slab's raw dO rows on
+// their way into the B-operand layout.
 // ---------------------------------------------------------------------------------------------
 template <typename T, int DK, int NW, int STAGES> struct StateBwdSmem {
-  static constexpr int big = 3 * 64 * DK * (int)sizeof(T) + 2 * 64 * 4 + 16;   // K, Q^T, W^T images, [64 unused], G_last, scale e^G [64]
-  static constexpr int off_small = STAGES * big;            // dO rows of the slab [64][32 NW] | tril(Q K^T . Gam) tiles [4]
-  static constexpr int small_elems = NW * 2048 + 4096;
-  // two small stages (and one barrier per step instead of two) where the CU's 160 KB of LDS allow it
-  static constexpr int small_stages = (STAGES == 2 && off_small + 2 * small_elems * (int)sizeof(T) <= 160 * 1024) ? 2 : 1;
-  static constexpr int bytes = off_small + small_stages * small_elems * (int)sizeof(T);
+  // one stage, in elements of T
+  static constexpr int off_k = 0;                        // K image [K/32][2] tiles
+  static constexpr int off_q = off_k + 64 * DK;          // Q^T image
+  static constexpr int off_tm = off_q + 64 * DK;         // Tm tiles (0,0), (1,0), (1,1)
+  static constexpr int off_aq = off_tm + 3 * 1024;       // Aq tiles (0,0), (1,0), (1,1)
+  static constexpr int off_do = off_aq + 3 * 1024;       // raw dO rows of the slabs [64][32 NW]
+  static constexpr int off_row = (off_do + 64 * 32 * NW) * (int)sizeof(T);   // bytes: float rows
+  // rows: e^{G_last-G} [64], beta e^G [64], scale e^G [64], G_last
+  static constexpr int stage = off_row + (3 * 64 + 4) * 4;
+  static constexpr int bytes = STAGES * stage;
+  static_assert(bytes <= 160 * 1024, "one CU's LDS");
 };
+
+template <int PIECES, int NT> struct DealB { static constexpr int kPer = (PIECES + NT - 1) / NT; };
 
 template <typename T, int DK, int NW, int NL, int STAGES>
 __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 && NL >= 4) ? 2 : 1) void chunk_state_bwd_kernel(
-    const T* __restrict__ kaf, const T* __restrict__ qtf, const T* __restrict__ wf, const T* __restrict__ aqf,
-    const T* __restrict__ dO, const float* __restrict__ G, const float* __restrict__ dht, float* __restrict__ dh0,
-    T* __restrict__ dvf, T* __restrict__ dhf, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets,
-    int T_len, int Hqk, int Hv, int V, float scale) {
+    const T* __restrict__ kaf, const T* __restrict__ qtf, const T* __restrict__ ai, const T* __restrict__ aqf,
+    const T* __restrict__ dO, const float* __restrict__ G, const float* __restrict__ beta, const float* __restrict__ dht,
+    float* __restrict__ dh0, T* __restrict__ dvf, T* __restrict__ dhf, const int64_t* __restrict__ cu,
+    const int* __restrict__ chunk_offsets, int T_len, int Hqk, int Hv, int V, float scale) {
   using SM = StateBwdSmem<T, DK, NW, STAGES>;
   constexpr int NT = 64 * NL, VEC = Elem<T>::kVec, NKT = DK / 32;   // NT loader threads
-  constexpr int CW = 64 * (DK / VEC) / NT, CUL = NW * 2048 / VEC / NT, CAQ = 4096 / VEC / NT, TILE = 64 * DK;
-  constexpr int PPR = 32 * NW / VEC;   // 16-byte pieces per dO row of the slab
-  static_assert(64 * (DK / VEC) % NT == 0 && (NW * 2048 / VEC) % NT == 0 && (4096 / VEC) % NT == 0,
-                "tile chunks must divide over the loaders");
-  static_assert(STAGES == 1 || STAGES == 2, "one or two big LDS stages");
+  constexpr int PK = 64 * DK / VEC, PTM = 3 * 1024 / VEC, PD = 64 * 32 * NW / VEC, DPR = 32 * NW / VEC;
+  constexpr int CK = DealB<PK, NT>::kPer, CTM = DealB<PTM, NT>::kPer, CD = DealB<PD, NT>::kPer;
+  static_assert(STAGES == 1 || STAGES == 2, "one or two LDS stages");
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, wave = tid >> 6;
   const int nh = xcd_grouped_head(blockIdx.x, gridDim.x, Hv / Hqk), n = nh / Hv, h = nh % Hv;
   const int64_t bos = cu ? cu[n] : (int64_t)n * T_len;
   const int len = cu ? (int)(cu[n + 1] - bos) : T_len;
   const int nchunks = (len + kChunk - 1) / kChunk;
   const int64_t chunk_base = cu ? chunk_offsets[n] : (int64_t)n * ((T_len + kChunk - 1) / kChunk);
-  T* small0 = reinterpret_cast<T*>(gdn_smem + SM::off_small);   // per stage: dO rows of the slab, row-major | Aq tiles
 
   // step s = 0 .. nchunks-1 handles chunk nchunks-1-s
   if (wave >= NW) {
     // ================= loader waves =================
     const int lt = tid - 64 * NW;
     constexpr int DEPTH = (STAGES == 2) ? 2 : 1;
-    Vec16<T> pk[DEPTH][CW], pq[DEPTH][CW], pw[DEPTH][CW], pa[DEPTH][CAQ], pd[DEPTH][CUL];
-    float pgt[DEPTH], pgl[DEPTH], pgk[DEPTH][2];
+    Vec16<T> pk[DEPTH][CK], pq[DEPTH][CK], ptm[DEPTH][CTM], pa[DEPTH][CTM], pd[DEPTH][CD];
+    float pgl[DEPTH], pg[DEPTH], pb[DEPTH];
+    int pnv[DEPTH];
+    auto tm_src = [&](int idc) {   // piece of the three kept tiles -> its place among the four stored ones
+      const int t = idc / (1024 / VEC);
+      return (t == 0 ? 0 : t + 1) * (1024 / VEC) + idc % (1024 / VEC);
+    };
     auto issue = [&](int st, int set) {
       const int c = nchunks - 1 - st;
       const int64_t tok0 = bos + (int64_t)c * kChunk;
       const int nvalid = imin(kChunk, len - c * kChunk);
       const int64_t ch = (chunk_base + c) * Hv + h, chq = (chunk_base + c) * Hqk + h / (Hv / Hqk);
 #pragma unroll
-      for (int i = 0; i < CW; ++i) {
-        const int id = lt + i * NT;
-        pk[set][i] = ld16(kaf + chq * TILE + id * VEC);
-        pq[set][i] = ld16(qtf + chq * TILE + id * VEC);
-        pw[set][i] = ld16(wf + ch * TILE + id * VEC);
+      for (int i = 0; i < CK; ++i) {
+        const int idc = imin(lt + i * NT, PK - 1);
+        pk[set][i] = ld16(kaf + chq * (64 * DK) + idc * VEC);
+        pq[set][i] = ld16(qtf + chq * (64 * DK) + idc * VEC);
       }
 #pragma unroll
-      for (int i = 0; i < CAQ; ++i) pa[set][i] = ld16(aqf + ch * 4096 + (lt + i * NT) * VEC);
+      for (int i = 0; i < CTM; ++i) {
+        const int src = tm_src(imin(lt + i * NT, PTM - 1));
+        ptm[set][i] = ld16(ai + ch * 4096 + src * VEC);
+        pa[set][i] = ld16(aqf + ch * 4096 + src * VEC);
+      }
 #pragma unroll
-      for (int i = 0; i < CUL; ++i) {   // dO rows of this slab, 16-byte pieces; rows past the end are zero
-        const int p = lt + i * NT, row = p / PPR, cc = p % PPR;
-        pd[set][i] = row < nvalid ? ld16(dO + ((tok0 + row) * Hv + h) * V + blockIdx.y * (32 * NW) + cc * VEC)
-                                  : zero16<T>();
+      for (int i = 0; i < CD; ++i) {   // dO rows of the slabs; rows past the end repeat the last one and are cleared below
+        const int idc = imin(lt + i * NT, PD - 1), row = imin(idc / DPR, nvalid - 1), cc = idc % DPR;
+        pd[set][i] = ld16(dO + ((tok0 + row) * Hv + h) * V + blockIdx.y * (32 * NW) + cc * VEC);
       }
       const float* gc = G + ch * 64;
+      const int t = lt & 63;
       // raw values only: arithmetic here would wait for every load issued so far.  The array repeats G_last past the
       // end of a short chunk.
       pgl[set] = gc[63];
-      pgt[set] = gc[lt & 63];
-      pgk[set][0] = gc[lt & 31];
-      pgk[set][1] = gc[32 + (lt & 31)];
+      pg[set] = gc[t];
+      pb[set] = beta[(tok0 + imin(t, nvalid - 1)) * Hv + h];
+      pnv[set] = nvalid;
     };
-    auto commit_big = [&](int set, int buf) {
-      unsigned char* base = gdn_smem + buf * SM::big;
-      T* Ka = reinterpret_cast<T*>(base);
-      T* Qa = Ka + TILE;
-      T* Wa = Qa + TILE;
-      float* dec = reinterpret_cast<float*>(Wa + TILE);
-      // K goes to LDS scaled by e^{G_last-G} of its token: in the A-operand tiles (rows = tokens) every 16-byte piece
-      // belongs to one token, 32 (tile & 1) + lane % 32.  The K tiles in memory are shared by the value heads of a
-      // q/k group, the decay is per value head.
-      const float kd[2] = {__expf(pgl[set] - pgk[set][0]), __expf(pgl[set] - pgk[set][1])};
+    auto commit = [&](int set, int buf) {
+      T* st = reinterpret_cast<T*>(gdn_smem + buf * SM::stage);
 #pragma unroll
-      for (int i = 0; i < CW; ++i) {
-        const int id = lt + i * NT;
-        st16(Ka + id * VEC, scale16<T>(pk[set][i], kd[(id / (1024 / VEC)) & 1]));
-        st16(Qa + id * VEC, pq[set][i]);
-        st16(Wa + id * VEC, pw[set][i]);
+      for (int i = 0; i < CK; ++i) {
+        const int idc = imin(lt + i * NT, PK - 1);
+        st16(st + SM::off_k + idc * VEC, pk[set][i]);
+        st16(st + SM::off_q + idc * VEC, pq[set][i]);
       }
-      if (lt < 64) dec[68 + lt] = scale * __expf(pgt[set]);
-      if (lt == 0) dec[64] = pgl[set];
-    };
-    auto commit_small = [&](int set, int buf) {
-      T* small = small0 + buf * SM::small_elems;
 #pragma unroll
-      for (int i = 0; i < CUL; ++i) st16(small + (lt + i * NT) * VEC, pd[set][i]);
+      for (int i = 0; i < CTM; ++i) {
+        const int idc = imin(lt + i * NT, PTM - 1);
+        st16(st + SM::off_tm + idc * VEC, ptm[set][i]);
+        st16(st + SM::off_aq + idc * VEC, pa[set][i]);
+      }
 #pragma unroll
-      for (int i = 0; i < CAQ; ++i) st16(small + NW * 2048 + (lt + i * NT) * VEC, pa[set][i]);
+      for (int i = 0; i < CD; ++i) {
+        const int idc = imin(lt + i * NT, PD - 1);
+        st16(st + SM::off_do + idc * VEC, idc / DPR < pnv[set] ? pd[set][i] : zero16<T>());
+      }
+      float* row = reinterpret_cast<float*>(gdn_smem + buf * SM::stage + SM::off_row);
+      if (lt < 64) {
+        const float b = lt < pnv[set] ? pb[set] : 0.f, eg = __expf(pg[set]);
+        row[lt] = __expf(pgl[set] - pg[set]);
+        row[64 + lt] = b * eg;
+        row[128 + lt] = scale * eg;
+      }
+      if (lt == 0) row[192] = pgl[set];
     };
+    if (nchunks == 0) return;
     if (STAGES == 2) {
       // Every path through this loop issues the same loads in the same order (steps past the end are clamped and
       // their data is never used), so that the number of loads in flight at each wait is a compile-time fact.
-      if (nchunks == 0) return;
       issue(0, 0);
-      commit_big(0, 0);
-      commit_small(0, 0);
+      commit(0, 0);
 #pragma unroll
       for (int j = 1; j <= DEPTH; ++j) issue(imin(j, nchunks - 1), j % DEPTH);
       for (int s0 = 0;; s0 += DEPTH) {
@@ -137,21 +151,17 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
         for (int u = 0; u < DEPTH; ++u) {
           const int st = s0 + u;
           if (st >= nchunks) return;
-          GDN_LDS_BARRIER();                // (A) step st staged; the other stages (step st-1) are free
-          if (SM::small_stages == 1) GDN_LDS_BARRIER();   // (B) the compute waves have taken the single small stage
-          commit_small((u + 1) % DEPTH, (st + 1) & (SM::small_stages - 1));
-          commit_big((u + 1) % DEPTH, (st + 1) & 1);
+          GDN_LDS_BARRIER();                // (A) step st staged; the other stage (step st-1) is free
+          commit((u + 1) % DEPTH, (st + 1) & 1);
           issue(imin(st + 1 + DEPTH, nchunks - 1), (u + 1) % DEPTH);
         }
       }
     } else {
       for (int st = 0; st < nchunks; ++st) {
-        if (st > 0) GDN_LDS_BARRIER();      // (C) the single big stage is free again
+        if (st > 0) GDN_LDS_BARRIER();      // (B) the single stage is free again
         issue(st, 0);
-        commit_big(0, 0);
-        commit_small(0, 0);
+        commit(0, 0);
         GDN_LDS_BARRIER();                  // (A)
-        GDN_LDS_BARRIER();                  // (B) the compute waves have taken their dO rows and the Aq tiles
       }
     }
     return;
@@ -159,8 +169,6 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
 
   // ================= compute waves =================
   const int vblk = blockIdx.y * NW + wave, v0 = 32 * vblk;
-  IdentityFrag<T> id;
-  id.init();
   f32x16 dS[NKT];
 #pragma unroll
   for (int kt = 0; kt < NKT; ++kt) {
@@ -180,40 +188,38 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
     const int c = nchunks - 1 - st;
     const int buf = (STAGES == 2) ? (st & 1) : 0;
     GDN_LDS_BARRIER();                      // (A)
-    // dO of this wave's 32 columns as B operand (lane <-> V column, registers <-> token), turned from the row-major
-    // rows through the matrix core; dv_local = (scale tril(Q K^T . Gam))^T dO from the forward pass's tiles
+    const T* sm = reinterpret_cast<const T*>(gdn_smem + buf * SM::stage);
+    const T* Ka = sm + SM::off_k;
+    const T* Qa = sm + SM::off_q;
+    const T* Tm = sm + SM::off_tm;
+    const T* Aq = sm + SM::off_aq;
+    const T* dOs = sm + SM::off_do;
+    const float* row = reinterpret_cast<const float*>(gdn_smem + buf * SM::stage + SM::off_row);
+    // dO of this wave's 32 columns as B operand (lane <-> V column, registers <-> token), and scaled by scale e^G of
+    // its token: the factor of the Q^T product rides on dO, so that the Q^T tiles are the same for every value head
+    // of a q/k group
     AccB<T> dob[2], dos[2], aq[3];
-    const T* small = small0 + (st & (SM::small_stages - 1)) * SM::small_elems;
-    frags_from_lds<T>(dob[0], small + (lane & 31) * (32 * NW) + 32 * wave);
-    frags_from_lds<T>(dob[1], small + (32 + (lane & 31)) * (32 * NW) + 32 * wave);
-    aq[0].load(small + NW * 2048);            // tiles (0,0), (1,0), (1,1)
-    aq[1].load(small + NW * 2048 + 2048);
-    aq[2].load(small + NW * 2048 + 3072);
-    if (SM::small_stages == 1) GDN_LDS_BARRIER();   // (B) the single small stage may be refilled
-    unsigned char* base = gdn_smem + buf * SM::big;
-    const T* Ka = reinterpret_cast<const T*>(base);
-    const T* Qa = Ka + TILE;
-    const T* Wa = Qa + TILE;
-    const float* dec = reinterpret_cast<const float*>(Wa + TILE);
-    const float eg = __expf(dec[64]);
+    dob[0].load_cols(dOs + 32 * wave, 32 * NW);
+    dob[1].load_cols(dOs + 32 * (32 * NW) + 32 * wave, 32 * NW);
+    aq[0].load(Aq);                           // tiles (0,0), (1,0), (1,1)
+    aq[1].load(Aq + 1024);
+    aq[2].load(Aq + 2048);
+    const float eg = __expf(row[192]);
     const int64_t tile0 = ((chunk_base + c) * Hv + h) * (V / 32) + vblk;
 #pragma unroll
     for (int kt = 0; kt < NKT; ++kt) dSb[kt].store_stream(dhf + (tile0 * NKT + kt) * 1024);
     {
-      // the per-token factor scale e^G of the Q^T product rides on dO, so that the Q^T tiles are the same for every
-      // value head of a q/k group
-      const f32x16 q0 = rows_ld(dec + 68, 0), q1 = rows_ld(dec + 68, 32);
-      f32x16 t0 = mfma_transpose<T>(dob[0], id), t1 = mfma_transpose<T>(dob[1], id);
-      dob[0].pack(t0);
-      dob[1].pack(t1);
+      const f32x16 q0 = rows_ld(row + 128, 0), q1 = rows_ld(row + 128, 32);
+      f32x16 t0 = dob[0].unpack(), t1 = dob[1].unpack();
 #pragma unroll
       for (int r = 0; r < 16; ++r) { t0[r] *= q0[r]; t1[r] *= q1[r]; }
       dos[0].pack(t0);
       dos[1].pack(t1);
     }
-    // dV' = (e^{G_last-G} . K) dS + dv_local, one accumulation chain per 32-token block.  The A-operand tiles come
-    // from LDS two tiles ahead of the matrix instructions that use them; the decay of dS rides in between.
-    f32x16 a0 = acc_zero(), a1 = acc_zero();
+    // dv_local = (scale tril(Q K^T . Gam))^T dO from the forward pass's tiles, and y = K dS, one accumulation chain per
+    // 32-token block each.  The A-operand tiles come from LDS two tiles ahead of the matrix instructions that use
+    // them; the decay of dS rides in between.
+    f32x16 a0 = acc_zero(), a1 = acc_zero(), y0 = acc_zero(), y1 = acc_zero();
     AccB<T> af[3];
     af[0].load(Ka);
     af[1].load(Ka + 1024);
@@ -224,33 +230,56 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
 #pragma unroll
     for (int i = 0; i < 2 * NKT; ++i) {       // tile i = (K tile i / 2, token block i % 2)
       if (i + 2 < 2 * NKT) af[(i + 2) % 3].load(Ka + (i + 2) * 1024);
-      mma32_ff<T>((i & 1) ? a1 : a0, af[i % 3], dSb[i / 2]);
+      mma32_ff<T>((i & 1) ? y1 : y0, af[i % 3], dSb[i / 2]);
 #pragma unroll
       for (int r = 0; r < 8; ++r) dS[i / 2][8 * (i & 1) + r] *= eg;
       GDN_SCHED_FENCE();
     }
-    // dS <- e^{G_last} dS + Q^T (scale e^G . dO) - W^T dV'  (the W^T tiles arrive negated); a finished tile of dS is
-    // packed for the next step while the matrix pipe works on the following one
-    auto tile_qw = [&](int i) {               // i = 4 kt + 2 tj + (0: Q^T, 1: W^T)
-      return ((i & 1) ? Wa : Qa) + ((i >> 2) * 2 + ((i >> 1) & 1)) * 1024;
-    };
-    af[0].load(tile_qw(0));
-    af[1].load(tile_qw(1));
-    AccB<T> dvb[2];
+    // dV' = e^{G_last-G} . y + dv_local
+    AccB<T> dvb[2], rb[2], tf[3];
+#pragma unroll
+    for (int t = 0; t < 3; ++t) tf[t].load_t(Tm + t * 1024);   // Tm^T tiles: (lane <-> column of Tm, registers <-> row)
+    {
+      const f32x16 d0 = rows_ld(row, 0), d1 = rows_ld(row, 32);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { a0[r] += d0[r] * y0[r]; a1[r] += d1[r] * y1[r]; }
+    }
     dvb[0].pack(a0);
     dvb[1].pack(a1);
     dvb[0].store_stream(dvf + (tile0 * 2 + 0) * 1024);
     dvb[1].store_stream(dvf + (tile0 * 2 + 1) * 1024);
+    // R = Tm^T dV' (upper triangular: R_0 = Tm00^T dV'_0 + Tm10^T dV'_1, R_1 = Tm11^T dV'_1), then -(beta e^G . R)
+    y0 = acc_zero();
+    y1 = acc_zero();
+    mma32_ff<T>(y0, tf[0], dvb[0]);
+    mma32_ff<T>(y1, tf[2], dvb[1]);
+    mma32_ff<T>(y0, tf[1], dvb[1]);
+    auto tile_qk = [&](int i) {               // i = 4 kt + 2 tj + (0: Q^T, 1: K^T)
+      return ((i & 1) ? Ka : Qa) + ((i >> 2) * 2 + ((i >> 1) & 1)) * 1024;
+    };
+    af[0].load(tile_qk(0));
+    af[1].load_t(tile_qk(1));
+    {
+      const f32x16 e0 = rows_ld(row + 64, 0), e1 = rows_ld(row + 64, 32);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { y0[r] *= -e0[r]; y1[r] *= -e1[r]; }
+      rb[0].pack(y0);
+      rb[1].pack(y1);
+    }
     GDN_SCHED_FENCE();
+    // dS <- e^{G_last} dS + Q^T (scale e^G . dO) - K^T (beta e^G . R); a finished tile of dS is packed for the next
+    // step while the matrix pipe works on the following one
 #pragma unroll
     for (int i = 0; i < 4 * NKT; ++i) {
-      if (i + 2 < 4 * NKT) af[(i + 2) % 3].load(tile_qw(i + 2));
-      mma32_ff<T>(dS[i >> 2], af[i % 3], (i & 1) ? dvb[(i >> 1) & 1] : dos[(i >> 1) & 1]);
+      if (i + 2 < 4 * NKT) {
+        if ((i + 2) & 1) af[(i + 2) % 3].load_t(tile_qk(i + 2)); else af[(i + 2) % 3].load(tile_qk(i + 2));
+      }
+      mma32_ff<T>(dS[i >> 2], af[i % 3], (i & 1) ? rb[(i >> 1) & 1] : dos[(i >> 1) & 1]);
       if ((i & 3) == 3 && i >= 4) dSb[(i >> 2) - 1].pack(dS[(i >> 2) - 1]);
       GDN_SCHED_FENCE();
     }
     dSb[NKT - 1].pack(dS[NKT - 1]);
-    if (STAGES == 1 && st + 1 < nchunks) GDN_LDS_BARRIER();   // (C)
+    if (STAGES == 1 && st + 1 < nchunks) GDN_LDS_BARRIER();   // (B)
   }
   if (dh0 != nullptr) {
 #pragma unroll
@@ -743,7 +772,6 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   const float* G = reinterpret_cast<const float*>(ws + L.G);
   const T* Ai = reinterpret_cast<const T*>(ws + L.Ai);
   const T* AQ = reinterpret_cast<const T*>(ws + L.AQ);
-  const T* WF = reinterpret_cast<const T*>(ws + L.WF);
   const T* VF = reinterpret_cast<const T*>(ws + L.VF);
   const T* HF = reinterpret_cast<const T*>(ws + L.HF);
   const T* QTF = reinterpret_cast<const T*>(ws + L.QTF);
@@ -757,7 +785,7 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     constexpr int smem = StateBwdSmem<T, DK, NWS, STAGES>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
     GDN_LAUNCH(kKernStateBwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NWS)), dim3(64 * (NWS + NLS)), smem, st, (const T*)KAF,
-               (const T*)QTF, WF, AQ, (const T*)dO, G, dht, dh0, DVF, DHF, cu, chunk_offsets, d.T, d.Hqk, d.Hv, d.V,
+               (const T*)QTF, Ai, AQ, (const T*)dO, G, beta, dht, dh0, DVF, DHF, cu, chunk_offsets, d.T, d.Hqk, d.Hv, d.V,
                scale);
   }
   {

@@ -98,49 +98,44 @@ __device__ __forceinline__ void tile_qk_finish(TileQK<T, DK>& t, T* lds, int ld,
 }
 
 // ---------------------------------------------------------------------------------------------
-// chunk_prep_kernel: everything that is independent across chunks.
-//   G (cumulative decay), Tm = (I+L)^-1, -W = -Tm (beta e^G K), U = Tm (beta V), Aq = scale tril(Q K^T . Gam),
-//   per q/k group the K^T, K and Q^T tiles of the recurrence kernels
-// U is written in fragment order (AccB<>): tile (32-token block ri) x (32-column block vb) at
-// U[chunk][head][vb][ri][1024], 16 bytes per lane per k-group -- the recurrence kernel copies it straight to LDS.
-// Three quarters of the kernel's traffic are stores, issued all along the way; its barriers order LDS traffic only
-// (GDN_LDS_BARRIER), because a __syncthreads() would also wait until every store issued so far has been acknowledged.
+// chunk_prep_kernel: what is independent across chunks and does not involve v.
+//   G (cumulative decay), Tm = (I+L)^-1, Aq = scale tril(Q K^T . Gam), and per q/k group the K and Q^T tiles, all in
+//   fragment order (AccB<>): 16 bytes per lane per k-group, copied straight to LDS by the recurrence kernels.
+// W = Tm (beta e^G K) and U = Tm (beta V) are never formed: the recurrence applies Tm to beta (v - e^G K S) itself.
+// Its barriers order LDS traffic only (GDN_LDS_BARRIER): a __syncthreads() would also wait until every store issued
+// so far has been acknowledged.
 // ---------------------------------------------------------------------------------------------
-template <typename T, int DK, int BV> struct PrepSmem {
-  static constexpr int LDK = lds_ld<T>(DK), LDV = lds_ld<T>(BV), L64 = lds_ld<T>(64);
+template <typename T, int DK> struct PrepSmem {
+  static constexpr int LDK = lds_ld<T>(DK), L64 = lds_ld<T>(64);
   static constexpr int cmax(int a, int b) { return a > b ? a : b; }
   // Two regions, each reused once its tenant is dead, so that four workgroups (bf16) fit a CU's LDS:
-  //   region 1: K tile -> Tm (fp32, solve output) -> beta e^G K (parked in registers during the solve) -> (beta V) tile
+  //   region 1: K tile -> Tm (fp32, solve output)
   //   region 2: Q tile -> A (fp32, solve input) -> Tm in T
   static constexpr int off_ks = 0;
-  static constexpr int r1_bytes = cmax(cmax(64 * LDK * (int)sizeof(T), 64 * kLF * 4), 64 * LDV * (int)sizeof(T));
+  static constexpr int r1_bytes = cmax(64 * LDK * (int)sizeof(T), 64 * kLF * 4);
   static constexpr int off_qs = off_ks + r1_bytes;
   static constexpr int qs_bytes = cmax(cmax(64 * LDK * (int)sizeof(T), 64 * kLF * 4), 64 * L64 * (int)sizeof(T));
   static constexpr int off_ti = off_ks;
   static constexpr int off_misc = off_qs + qs_bytes;
-  static constexpr int bytes = off_misc + 3 * 64 * 4;
+  static constexpr int bytes = off_misc + 2 * 64 * 4;
 };
 
-template <typename T, int DK, int BV>
+template <typename T, int DK>
 __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3) void chunk_prep_kernel(
-    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ g,
-    const float* __restrict__ beta, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets,
-    float* __restrict__ G_out, T* __restrict__ Ai_out, T* __restrict__ W_out, T* __restrict__ U_out,
-    T* __restrict__ Aq_out, T* __restrict__ KT_out, T* __restrict__ WF_out, T* __restrict__ KA_out,
-    T* __restrict__ QT_out, float* __restrict__ rstd_q_out, float* __restrict__ rstd_k_out,
-    int T_len, int N, int Hqk, int Hv, int V, float scale, int l2norm, TokenStrides ts) {
-  using SM = PrepSmem<T, DK, BV>;
-  constexpr int LDK = SM::LDK, LDV = SM::LDV, L64 = SM::L64, VEC = Elem<T>::kVec;
+    const T* __restrict__ q, const T* __restrict__ k, const float* __restrict__ g, const float* __restrict__ beta,
+    const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, float* __restrict__ G_out,
+    T* __restrict__ Ai_out, T* __restrict__ Aq_out, T* __restrict__ KA_out, T* __restrict__ QT_out,
+    float* __restrict__ rstd_q_out, float* __restrict__ rstd_k_out, int T_len, int N, int Hqk, int Hv, float scale,
+    int l2norm, TokenStrides ts) {
+  using SM = PrepSmem<T, DK>;
+  constexpr int LDK = SM::LDK, L64 = SM::L64, VEC = Elem<T>::kVec;
   T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
-  T* Kb = Ks;                                                     // after Tm (fp32)
   T* Qs = reinterpret_cast<T*>(gdn_smem + SM::off_qs);
   float* As = reinterpret_cast<float*>(gdn_smem + SM::off_qs);    // after Q
   T* Tms = reinterpret_cast<T*>(gdn_smem + SM::off_qs);          // after A
-  float* Ti = reinterpret_cast<float*>(gdn_smem + SM::off_ti);
-  T* Vb = reinterpret_cast<T*>(gdn_smem + SM::off_ti);           // after beta e^G K
+  float* Ti = reinterpret_cast<float*>(gdn_smem + SM::off_ti);   // after K
   float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_misc);
   float* bs = Gs + 64;
-  float* egs = bs + 64;
 
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
@@ -162,7 +157,6 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
     }
     Gs[lane] = x;
     bs[lane] = b;
-    egs[lane] = b * __expf(x);
     G_out[((int64_t)blockIdx.x * Hv + h) * 64 + lane] = x;   // 64 contiguous values per chunk and head
   }
   {
@@ -196,41 +190,23 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
       aq[r] *= gam * scale;
     }
     // scale tril(Q K^T . Gam) leaves as four 32x32 tiles in fragment order, packed as they sit in the accumulator
-    // (lane <-> column j, registers <-> row i): the A operand of Aq^T dO as is, of Aq V' after one turn
+    // (lane <-> column j, registers <-> row i): the A operand of Aq^T dO as is, of Aq V' read transposed
     AccB<T> af;
     af.pack(aq);
     af.store_stream(Aq_out + (((int64_t)blockIdx.x * Hv + h) * 4 + wave) * 1024);
   }
-  // K^T as A-operand fragments for the state update: K tile fragments (lane <-> token) turned through the matrix
-  // core into (lane <-> K column, registers <-> token), stored in fragment order (the decay is applied by the reader)
-  {
-    IdentityFrag<T> id;
-    id.init();
-    const bool group_first = (h % (Hv / Hqk)) == 0;   // K and Q^T tiles are shared by the value heads of a q/k group
+  // K (lane <-> token, registers <-> K column) and Q^T (lane <-> K column, registers <-> token) as A-operand fragments,
+  // once per q/k group; the recurrence kernels read each of them both as it lies and transposed
+  if ((h % (Hv / Hqk)) == 0) {
     for (int tt = wave; tt < 2 * (DK / 32); tt += 4) {
       const int tj = tt & 1, kt = tt >> 1;
       const int64_t gtile = ((((int64_t)blockIdx.x * Hqk + hq) * (DK / 32) + kt) * 2 + tj) * 1024;
       AccB<T> kf;
       frags_from_lds<T>(kf, Ks + (32 * tj + (lane & 31)) * LDK + 32 * kt);
-      if (KA_out != nullptr && group_first) kf.store_stream(KA_out + gtile);   // K as an A operand (lane <-> token)
-      if (group_first) {   // K^T as an A operand (lane <-> K column), for the state update
-        kf.pack(mfma_transpose<T>(kf, id));
-        kf.store_stream(KT_out + gtile);
-      }
-      if (QT_out != nullptr && group_first) {   // Q^T as an A operand (lane <-> K column), for the backward pass
-        frags_from_lds<T>(kf, Qs + (32 * tj + (lane & 31)) * LDK + 32 * kt);
-        kf.pack(mfma_transpose<T>(kf, id));
-        kf.store_stream(QT_out + gtile);
-      }
+      kf.store_stream(KA_out + gtile);
+      kf.load_cols(Qs + 32 * tj * LDK + 32 * kt, LDK);
+      kf.store_stream(QT_out + gtile);
     }
-  }
-  // beta e^G K, this thread's pieces of the K tile, parked in registers: the K tile's space takes the fp32 Tm first
-  constexpr int KPT = 64 * (DK / VEC) / kThreads;
-  Vec16<T> kreg[KPT];
-#pragma unroll
-  for (int i = 0; i < KPT; ++i) {
-    const int c = tid + i * kThreads, row = c / (DK / VEC), cc = c % (DK / VEC);
-    kreg[i] = scale16<T>(ld16(Ks + row * LDK + cc * VEC), egs[row]);
   }
   GDN_LDS_BARRIER();   // Q and K are consumed: their space takes A and Tm
 
@@ -240,15 +216,6 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
     for (int r = 0; r < 16; ++r) As[(32 * ti + acc_row(r)) * kLF + j] = a_tile[r];
   }
   for (int i = tid; i < 64 * kLF; i += kThreads) Ti[i] = 0.f;
-  // the first V block is requested now and parked in registers until the fp32 Tm has been consumed
-  const T* vg = v + tok0 * ts.v + h * V;
-  constexpr int VPT = 64 * (BV / VEC) / kThreads;   // 16-byte pieces of the V tile per thread
-  Vec16<T> vreg[VPT];
-#pragma unroll
-  for (int i = 0; i < VPT; ++i) {
-    const int c = tid + i * kThreads, row = c / (BV / VEC), cc = c % (BV / VEC);
-    vreg[i] = ld16(vg + imin(row, nvalid - 1) * ts.v + cc * VEC);   // rows past the end: beta = 0 will clear them
-  }
   GDN_LDS_BARRIER();
 
   // ---- phase 2a: invert the four 16x16 diagonal blocks by forward substitution (fp32) ----
@@ -313,7 +280,7 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
   }
   GDN_LDS_BARRIER();
 
-  // ---- phase 3: Tm in operand precision, kept for the backward pass ----
+  // ---- phase 3: Tm in operand precision, as four 32x32 A-operand tiles (lane <-> row, registers <-> column) ----
   {
     constexpr int CPR = 64 / VEC;
     for (int c = tid; c < 64 * CPR; c += kThreads) {
@@ -325,99 +292,62 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
     }
   }
   GDN_LDS_BARRIER();
-  // the fp32 Tm is consumed: its space takes the beta e^G K tile parked in registers
-#pragma unroll
-  for (int i = 0; i < KPT; ++i) {
-    const int c = tid + i * kThreads, row = c / (DK / VEC), cc = c % (DK / VEC);
-    st16(Kb + row * LDK + cc * VEC, kreg[i]);
-  }
-  // The V block requested above has long arrived.  Waiting for it here, before the stores of the next phases are
-  // issued, keeps its first use from waiting for those stores as well (loads and stores are counted in one order).
-  GDN_WAIT_VMEM();
-  if (Ai_out != nullptr) {  // the four 32x32 tiles of Tm as A operands (lane <-> row, registers <-> column), for the backward
+  {
     AccB<T> tf;
     frags_from_lds<T>(tf, Tms + (32 * (wave >> 1) + (lane & 31)) * L64 + 32 * (wave & 1));
     tf.store_stream(Ai_out + (((int64_t)blockIdx.x * Hv + h) * 4 + wave) * 1024);
   }
-  GDN_LDS_BARRIER();
-
-  // ---- phase 4: W = Tm (beta e^G K), handed on in fragment order only ----
-  {
-    IdentityFrag<T> id;
-    id.init();
-    for (int tt = wave; tt < 2 * (DK / 32); tt += 4) {
-      const int ri = tt & 1, cj = tt >> 1;
-      f32x16 acc = acc_zero();
-      mma32<T, 64, true, false>(acc, Tms + 32 * ri * L64, L64, Kb + 32 * cj, LDK);
-      const int64_t tile = (((int64_t)blockIdx.x * Hv + h) * (DK / 32) + cj) * 2 + ri;
-      AccB<T> wf;
-      wf.pack(acc);              // (lane <-> K column, registers <-> token): -W^T as an A operand, for the backward pass
-      wf.negate();               // both uses subtract the product (U - W S, dS - W^T dV')
-      if (WF_out != nullptr) wf.store_stream(WF_out + tile * 1024);
-      const f32x16 wt = mfma_transpose<T>(wf, id);
-      wf.pack(wt);               // (lane <-> token, registers <-> K column): -W as an A operand, for U - W S
-      wf.store_stream(W_out + tile * 1024);
-    }
-  }
-  // ---- phase 5: U = Tm (beta V), V block by V block, stored in fragment order ----
-  for (int vb = 0; vb < V / BV; ++vb) {
-    GDN_LDS_BARRIER();   // the tile in region 1 (beta e^G K, or the previous V block) is consumed
-    if (vb == 0) {     // the first (beta V) block was parked in registers
-#pragma unroll
-      for (int i = 0; i < VPT; ++i) {
-        const int c = tid + i * kThreads, row = c / (BV / VEC), cc = c % (BV / VEC);
-        st16(Vb + row * LDV + cc * VEC, scale16<T>(vreg[i], bs[row]));
-      }
-    } else {
-      load_tile_scaled<T, BV>(Vb, LDV, vg + vb * BV, ts.v, nvalid, bs, tid);
-    }
-    GDN_LDS_BARRIER();
-    for (int tt = wave; tt < 2 * (BV / 32); tt += 4) {
-      const int ri = tt & 1, cj = tt >> 1;
-      f32x16 acc = acc_zero();
-      mma32<T, 64, true, false>(acc, Tms + 32 * ri * L64, L64, Vb + 32 * cj, LDV);
-      const int vblk = vb * (BV / 32) + cj;
-      AccB<T> uf;
-      uf.pack(acc);
-      uf.store_stream(U_out + ((((int64_t)blockIdx.x * Hv + h) * (V / 32) + vblk) * 2 + ri) * 1024);
-    }
-  }
 }
 
 // ---------------------------------------------------------------------------------------------
-// chunk_state_kernel: the inter-chunk recurrence, kept as lean as possible because it is the only part of the
-// forward pass that is sequential in the chunks.  One compute wave owns a 32-column slab of the state S[K, 32] in
-// fp32 registers for the whole sequence and per chunk does
-//     V' = U - W S            S <- e^{G_last} S + K^T (e^{G_last-G} . V')
-// Both B operands (S, V') are taken straight from accumulator registers (frag_b_from_acc), so the chain
-// W S -> V' -> S never touches LDS and the compute waves of a workgroup never exchange data.  S (before the chunk)
-// and V' leave the kernel in fragment order, 16 bytes per lane per k-group, for chunk_out_kernel and the backward
-// pass.  The A operands (-W per value head, K^T per q/k group) and U arrive in fragment order, one contiguous 16 KB
-// block per chunk prepared by chunk_prep_kernel (token-major tiles would be 64 rows scattered 8 KB apart), and are
-// copied to LDS in 16-byte pieces by NL loader waves of the same workgroup, which run ahead of the NW compute
-// waves: loads for chunks c+2 and c+3 are in flight in registers while chunk c+1 sits in the other LDS stage; the
-// two roles meet at one barrier per chunk.
+// chunk_state_kernel: the inter-chunk recurrence, the only part of the forward pass that is sequential in the
+// chunks.  One compute wave owns a 32-column slab of the state S[K, 32] in fp32 registers for the whole sequence
+// and per chunk does
+//     y = K S     z = beta (v - e^G . y)     V' = Tm z     S <- e^{G_last} S + K^T (e^{G_last-G} . V')
+// which is V' = U - W S with W = Tm (beta e^G K), U = Tm (beta V) never materialised.  Every B operand (S, z, V')
+// comes straight from accumulator registers (frag_b_from_acc), so the chain never touches LDS.  The A operands are
+// fragment-order tiles prepared by chunk_prep_kernel (K per q/k group, Tm per value head), one contiguous block per
+// chunk; K^T is the same K image read with the transposing LDS read, and the slab's raw v rows are read the same way
+// into the accumulator layout.  NL loader waves of the workgroup copy the next chunks' operands global -> registers ->
+// LDS two chunks ahead (two LDS stages); the roles meet at one barrier per chunk.
+// OUT: a second wave per slab forms the output O = scale e^G . (Q S) + Aq V' of the same 32 columns from the state and
+// V' the compute wave leaves in LDS (Q read transposed from the Q^T image, Aq likewise), one step behind it, so that
+// neither S nor V' has to be re-read from memory; both are still stored when a backward pass will need them.
 // ---------------------------------------------------------------------------------------------
-template <typename T, int DK, int NW, int STAGES> struct StateSmem {
-  static constexpr int off_ws = 0;
-  static constexpr int off_kt = off_ws + 64 * DK * (int)sizeof(T);
-  static constexpr int off_uf = off_kt + DK * 64 * (int)sizeof(T);
-  static constexpr int off_gl = off_uf + NW * 2048 * (int)sizeof(T);   // e^{G_last - G_t} [64], G_last
-  static constexpr int stage = off_gl + 64 * 4 + 16;
-  static constexpr int bytes = STAGES * stage;
+template <typename T, int DK, int NW, int STAGES, bool OUT> struct StateSmem {
+  // one stage, in elements of T
+  static constexpr int off_k = 0;                                   // K image [K/32][2] tiles
+  static constexpr int off_tm = off_k + 64 * DK;                    // Tm tiles (0,0), (1,0), (1,1)
+  static constexpr int off_v = off_tm + 3 * 1024;                   // raw v rows of the slabs [64][32 NW]
+  static constexpr int off_q = off_v + 64 * 32 * NW;                // OUT: Q^T image
+  static constexpr int off_aq = off_q + (OUT ? 64 * DK : 0);        // OUT: Aq tiles (0,0), (1,0), (1,1)
+  static constexpr int off_row = (off_aq + (OUT ? 3 * 1024 : 0)) * (int)sizeof(T);   // bytes: float rows
+  // rows: e^{G_last-G} [64], beta e^G [64], beta [64], scale e^G [64], G_last
+  static constexpr int stage = off_row + (4 * 64 + 4) * 4;
+  static constexpr int off_x = STAGES * stage;                      // OUT: per slab S [2][DK*32], V' [2][2048], store patch
+  static constexpr int x_elems = 2 * DK * 32 + 2 * 2048 + Patch<T>::kElems;
+  static constexpr int bytes = off_x + (OUT ? NW * x_elems * (int)sizeof(T) : 0);
+  static_assert(bytes <= 160 * 1024, "one CU's LDS");
 };
 
-template <typename T, int DK, int NW, int NL, int STAGES>
-__global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 2 : 1) void chunk_state_kernel(
-    const T* __restrict__ ktf, const T* __restrict__ w, const T* __restrict__ uf, const float* __restrict__ G,
-    const float* __restrict__ h0, float* __restrict__ ht, T* __restrict__ vf, T* __restrict__ hf,
-    const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int Hqk, int Hv, int V) {
-  using SM = StateSmem<T, DK, NW, STAGES>;
-  constexpr int NT = 64 * NL, VEC = Elem<T>::kVec;   // loader threads
-  constexpr int NKT = DK / 32;
-  constexpr int CW = 64 * (DK / VEC) / NT, CUL = NW * 2048 / VEC / NT;
-  static_assert(64 * (DK / VEC) % NT == 0 && (NW * 2048 / VEC) % NT == 0, "tile chunks must divide over the loaders");
+// pieces [0, PIECES) of 16 bytes dealt to NT threads, the same number to each: indices past the end repeat the last
+// piece (the same loads on every path; the duplicate lands on the same LDS address with the same data)
+template <int PIECES, int NT> struct Deal { static constexpr int kPer = (PIECES + NT - 1) / NT; };
+
+template <typename T, int DK, int NW, int NL, int STAGES, bool OUT>
+__global__ __launch_bounds__(64 * (NW + (OUT ? NW : 0) + NL)) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 2 : 1)
+void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, const T* __restrict__ ai,
+                        const T* __restrict__ aqf, const T* __restrict__ v, const float* __restrict__ G,
+                        const float* __restrict__ beta, const float* __restrict__ h0, float* __restrict__ ht,
+                        T* __restrict__ vf, T* __restrict__ hf, T* __restrict__ o, const int64_t* __restrict__ cu,
+                        const int* __restrict__ chunk_offsets, int T_len, int Hqk, int Hv, int V, float scale,
+                        int64_t v_stride) {
+  using SM = StateSmem<T, DK, NW, STAGES, OUT>;
+  constexpr int NT = 64 * NL, VEC = Elem<T>::kVec, NKT = DK / 32, NWO = OUT ? NW : 0;
+  constexpr int PK = 64 * DK / VEC, PTM = 3 * 1024 / VEC, PV = 64 * 32 * NW / VEC, VPR = 32 * NW / VEC;
+  constexpr int CK = Deal<PK, NT>::kPer, CTM = Deal<PTM, NT>::kPer, CV = Deal<PV, NT>::kPer;
   static_assert(STAGES == 1 || STAGES == 2, "one or two LDS stages");
+  static_assert(!OUT || STAGES == 2, "the output waves read a stage while the next one is filled");
 
   const int tid = threadIdx.x, wave = tid >> 6;
   const int nh = xcd_grouped_head(blockIdx.x, gridDim.x, Hv / Hqk), n = nh / Hv, h = nh % Hv;
@@ -425,52 +355,93 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ?
   const int len = cu ? (int)(cu[n + 1] - bos) : T_len;
   const int nchunks = (len + kChunk - 1) / kChunk;
   const int64_t chunk_base = cu ? chunk_offsets[n] : (int64_t)n * ((T_len + kChunk - 1) / kChunk);
+  // number of barriers every wave passes: one per chunk, plus one that hands the last V' to the output waves
+  const int nsteps = nchunks + (OUT ? 1 : 0);
+  if (nchunks == 0) {   // an empty sequence: its final state is its initial state
+    if (wave < NW && ht != nullptr) {
+      const int v0 = 32 * (blockIdx.y * NW + wave);
+      for (int kt = 0; kt < NKT; ++kt)
+        for (int r = 0; r < 16; ++r) {
+          const int64_t at = (((int64_t)n * Hv + h) * DK + 32 * kt + acc_row(r)) * V + v0 + acc_col();
+          ht[at] = h0 != nullptr ? h0[at] : 0.f;
+        }
+    }
+    return;
+  }
 
-  if (wave >= NW) {
-    // ================= loader waves: straight 16-byte copies =================
-    const int lt = tid - 64 * NW;
+  if (wave >= NW + NWO) {
+    // ================= loader waves: 16-byte copies =================
+    const int lt = tid - 64 * (NW + NWO);
     // DEPTH register sets: chunk j sits in set j % DEPTH from the iteration that requests it (j - DEPTH - 1) to the
     // one that copies it to LDS (j - 1), so global loads have DEPTH chunk periods to arrive
     constexpr int DEPTH = (STAGES == 2) ? 2 : 1;
-    Vec16<T> pw[DEPTH][CW], pk[DEPTH][CW], pu[DEPTH][CUL];
-    float glast[DEPTH], pdec[DEPTH];
+    Vec16<T> pk[DEPTH][CK], ptm[DEPTH][CTM], pv[DEPTH][CV], pq[DEPTH][OUT ? CK : 1], pa[DEPTH][OUT ? CTM : 1];
+    float pgl[DEPTH], pg[DEPTH], pb[DEPTH];
+    int pnv[DEPTH];
+    auto tm_src = [&](int idc) {   // piece of the three kept tiles -> its place among the four stored ones
+      const int t = idc / (1024 / VEC);
+      return (t == 0 ? 0 : t + 1) * (1024 / VEC) + idc % (1024 / VEC);
+    };
     auto issue = [&](int c, int set) {      // global -> registers
       const int nvalid = imin(kChunk, len - c * kChunk);
+      const int64_t ch = (chunk_base + c) * Hv + h, chq = (chunk_base + c) * Hqk + h / (Hv / Hqk);
+      const int64_t tok0 = bos + (int64_t)c * kChunk;
 #pragma unroll
-      for (int i = 0; i < CW; ++i) {
-        const int id = lt + i * NT;
-        pw[set][i] = ld16(w + ((chunk_base + c) * Hv + h) * (64 * DK) + id * VEC);
-        pk[set][i] = ld16(ktf + ((chunk_base + c) * Hqk + h / (Hv / Hqk)) * (64 * DK) + id * VEC);   // shared by the group
+      for (int i = 0; i < CK; ++i) {
+        const int idc = imin(lt + i * NT, PK - 1);
+        pk[set][i] = ld16(kaf + chq * (64 * DK) + idc * VEC);   // shared by the value heads of the group
+        if constexpr (OUT) pq[set][i] = ld16(qtf + chq * (64 * DK) + idc * VEC);
       }
-      const T* ug = uf + (((chunk_base + c) * Hv + h) * (V / 32) + blockIdx.y * NW) * 2048;
 #pragma unroll
-      for (int i = 0; i < CUL; ++i) pu[set][i] = ld16(ug + (lt + i * NT) * VEC);
-      const float* gc = G + ((chunk_base + c) * Hv + h) * 64;
-      glast[set] = gc[nvalid - 1];          // raw values only: arithmetic here would wait for every load issued so far
-      pdec[set] = gc[imin(lt & 63, nvalid - 1)];
+      for (int i = 0; i < CTM; ++i) {
+        const int src = tm_src(imin(lt + i * NT, PTM - 1));
+        ptm[set][i] = ld16(ai + ch * 4096 + src * VEC);
+        if constexpr (OUT) pa[set][i] = ld16(aqf + ch * 4096 + src * VEC);
+      }
+#pragma unroll
+      for (int i = 0; i < CV; ++i) {   // rows past the end of the sequence repeat the last one (their beta is 0)
+        const int idc = imin(lt + i * NT, PV - 1), row = imin(idc / VPR, nvalid - 1), cc = idc % VPR;
+        pv[set][i] = ld16(v + (tok0 + row) * v_stride + (int64_t)h * V + blockIdx.y * (32 * NW) + cc * VEC);
+      }
+      const float* gc = G + ch * 64;
+      const int t = lt & 63;
+      // raw values only: arithmetic here would wait for every load issued so far.  G repeats G_last past the end of a
+      // short chunk.
+      pgl[set] = gc[63];
+      pg[set] = gc[t];
+      pb[set] = beta[(tok0 + imin(t, nvalid - 1)) * Hv + h];
+      pnv[set] = nvalid;
     };
     auto commit = [&](int set, int buf) {   // registers -> LDS stage
-      unsigned char* base = gdn_smem + buf * SM::stage;
-      T* Ws = reinterpret_cast<T*>(base + SM::off_ws);
-      T* KT = reinterpret_cast<T*>(base + SM::off_kt);
-      T* Uf = reinterpret_cast<T*>(base + SM::off_uf);
+      T* st = reinterpret_cast<T*>(gdn_smem + buf * SM::stage);
 #pragma unroll
-      for (int i = 0; i < CW; ++i) {
-        const int id = lt + i * NT;
-        st16(Ws + id * VEC, pw[set][i]);
-        st16(KT + id * VEC, pk[set][i]);
+      for (int i = 0; i < CK; ++i) {
+        const int idc = imin(lt + i * NT, PK - 1);
+        st16(st + SM::off_k + idc * VEC, pk[set][i]);
+        if constexpr (OUT) st16(st + SM::off_q + idc * VEC, pq[set][i]);
       }
 #pragma unroll
-      for (int i = 0; i < CUL; ++i) st16(Uf + (lt + i * NT) * VEC, pu[set][i]);
-      float* dec = reinterpret_cast<float*>(base + SM::off_gl);
-      if (lt < 64) dec[lt] = __expf(glast[set] - pdec[set]);
-      if (lt == 0) dec[64] = glast[set];
+      for (int i = 0; i < CTM; ++i) {
+        const int idc = imin(lt + i * NT, PTM - 1);
+        st16(st + SM::off_tm + idc * VEC, ptm[set][i]);
+        if constexpr (OUT) st16(st + SM::off_aq + idc * VEC, pa[set][i]);
+      }
+#pragma unroll
+      for (int i = 0; i < CV; ++i) st16(st + SM::off_v + imin(lt + i * NT, PV - 1) * VEC, pv[set][i]);
+      float* row = reinterpret_cast<float*>(gdn_smem + buf * SM::stage + SM::off_row);
+      if (lt < 64) {
+        const float b = lt < pnv[set] ? pb[set] : 0.f, eg = __expf(pg[set]);
+        row[lt] = __expf(pgl[set] - pg[set]);
+        row[64 + lt] = b * eg;
+        row[128 + lt] = b;
+        row[192 + lt] = scale * eg;
+      }
+      if (lt == 0) row[256] = pgl[set];
     };
     if (STAGES == 2) {
       // Every path through this loop issues the same loads in the same order (chunk indices past the end are clamped
       // and their data is never used), so that the number of loads in flight at each wait is a compile-time fact and
       // the waits before the LDS writes of one register set leave the younger sets in flight.
-      if (nchunks == 0) return;
       issue(0, 0);
       commit(0, 0);
 #pragma unroll
@@ -479,21 +450,78 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ?
 #pragma unroll
         for (int u = 0; u < DEPTH; ++u) {
           const int c = c0 + u;
-          if (c >= nchunks) return;
+          if (c >= nsteps) return;
           GDN_LDS_BARRIER();                // (A) chunk c staged; the other stage (chunk c-1) is free
           commit((u + 1) % DEPTH, (c + 1) & 1);
           issue(imin(c + 1 + DEPTH, nchunks - 1), (u + 1) % DEPTH);
         }
       }
     } else {
-      for (int c = 0; c < nchunks; ++c) {
+      for (int c = 0; c < nsteps; ++c) {
         if (c > 0) GDN_LDS_BARRIER();       // (B) the single stage is free again
-        issue(c, 0);
+        issue(imin(c, nchunks - 1), 0);
         commit(0, 0);
         GDN_LDS_BARRIER();                  // (A)
       }
     }
     return;
+  }
+
+  if constexpr (OUT) {
+    if (wave >= NW) {
+      // ================= output waves: O of the slab's 32 columns, one step behind the compute wave =================
+      const int w = wave - NW;
+      const int vblk = blockIdx.y * NW + w, v0 = 32 * vblk;
+      T* xs = reinterpret_cast<T*>(gdn_smem + SM::off_x) + w * SM::x_elems;
+      T* patch = xs + 2 * DK * 32 + 2 * 2048;
+      IdentityFrag<T> id;
+      id.init();
+      f32x16 oa[2];
+      AccB<T> Af[3];
+      for (int c = 0; c < nsteps; ++c) {
+        const int buf = (STAGES == 2) ? (c & 1) : 0;
+        GDN_LDS_BARRIER();                    // (A)
+        if (c > 0) {                          // finish chunk c-1: + Aq V', rows out
+          const T* vx = xs + 2 * DK * 32 + ((c - 1) & 1) * 2048;
+          AccB<T> Vb[2];
+          Vb[0].load(vx);
+          Vb[1].load(vx + 1024);
+          mma32_ff<T>(oa[0], Af[0], Vb[0]);
+          mma32_ff<T>(oa[1], Af[1], Vb[0]);
+          mma32_ff<T>(oa[1], Af[2], Vb[1]);
+          const int64_t tok0 = bos + (int64_t)(c - 1) * kChunk;
+          const int nvalid = imin(kChunk, len - (c - 1) * kChunk);
+          T* og = o + (tok0 * Hv + h) * V + v0;
+#pragma unroll
+          for (int ri = 0; ri < 2; ++ri)
+            acc_store_rows<T, false>(oa[ri], id, patch, og + (int64_t)32 * ri * Hv * V, (int64_t)Hv * V, nvalid - 32 * ri);
+        }
+        if (c < nchunks) {                    // start chunk c: scale e^G . (Q S), and its Aq tiles into registers
+          const T* st = reinterpret_cast<const T*>(gdn_smem + buf * SM::stage);
+          const float* row = reinterpret_cast<const float*>(gdn_smem + buf * SM::stage + SM::off_row);
+          const T* sx = xs + (c & 1) * (DK * 32);
+          oa[0] = acc_zero();
+          oa[1] = acc_zero();
+#pragma unroll
+          for (int kt = 0; kt < NKT; ++kt) {
+            AccB<T> Sb, Qf;
+            Sb.load(sx + kt * 1024);
+#pragma unroll
+            for (int ri = 0; ri < 2; ++ri) {
+              Qf.load_t(st + SM::off_q + (kt * 2 + ri) * 1024);   // Q tile (token block ri, K block kt)
+              mma32_ff<T>(oa[ri], Qf, Sb);
+            }
+          }
+          const f32x16 e0 = rows_ld(row + 192, 0), e1 = rows_ld(row + 192, 32);
+#pragma unroll
+          for (int r = 0; r < 16; ++r) { oa[0][r] *= e0[r]; oa[1][r] *= e1[r]; }
+#pragma unroll
+          for (int t = 0; t < 3; ++t) Af[t].load_t(st + SM::off_aq + t * 1024);   // (lane <-> row i, registers <-> column j)
+          if (STAGES == 1 && c + 1 < nsteps) GDN_LDS_BARRIER();   // (B)
+        }
+      }
+      return;
+    }
   }
 
   // ================= compute waves =================
@@ -510,71 +538,101 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ?
   }
   // The wave issues its instructions in order and a matrix instruction occupies the matrix pipe for 32 cycles, in
   // which eight vector instructions can issue: the loop body is written so that the vector work which does not
-  // depend on the running product (decay of S, packing S for the next chunk, unpacking U) sits between the matrix
-  // instructions instead of before or after them.
+  // depend on the running product (decay of S, packing S for the next chunk) sits between the matrix instructions
+  // instead of before or after them.
   AccB<T> Sb[NKT];
+  T* xs = reinterpret_cast<T*>(gdn_smem + SM::off_x) + wave * SM::x_elems;   // OUT only
 #pragma unroll
-  for (int kt = 0; kt < NKT; ++kt) Sb[kt].pack(S[kt]);
+  for (int kt = 0; kt < NKT; ++kt) {
+    Sb[kt].pack(S[kt]);
+    if constexpr (OUT) Sb[kt].store(xs + kt * 1024);
+  }
   for (int c = 0; c < nchunks; ++c) {
     const int buf = (STAGES == 2) ? (c & 1) : 0;
     GDN_LDS_BARRIER();                        // (A) stage `buf` holds chunk c
-    unsigned char* base = gdn_smem + buf * SM::stage;
-    const T* Ws = reinterpret_cast<const T*>(base + SM::off_ws);
-    const T* KT = reinterpret_cast<const T*>(base + SM::off_kt);
-    const T* Uf = reinterpret_cast<const T*>(base + SM::off_uf) + wave * 2048;
-    const float* dec = reinterpret_cast<const float*>(base + SM::off_gl);
+    const T* st = reinterpret_cast<const T*>(gdn_smem + buf * SM::stage);
+    const T* Ka = st + SM::off_k;
+    const T* Tm = st + SM::off_tm;
+    const T* Vs = st + SM::off_v;
+    const float* row = reinterpret_cast<const float*>(gdn_smem + buf * SM::stage + SM::off_row);
     const int64_t tile0 = ((chunk_base + c) * Hv + h) * (V / 32) + vblk;
 
     constexpr int NP = NKT / 2;             // K tiles are processed two at a time
-    AccB<T> Wf[2][2][2];                    // [buffer][32-token block][K tile of the pair]
-    AccB<T> Kf[2][2][2];                    // [buffer][K tile of the pair][32-token block]
-    auto load_w = [&](int b, int kp) {
+    AccB<T> Kf[2][2][2];                    // [buffer][32-token block][K tile of the pair]; later [buffer][K tile][token block]
+    auto load_k = [&](int b, int kp) {      // K as it lies: (lane <-> token, registers <-> K column)
 #pragma unroll
       for (int ri = 0; ri < 2; ++ri)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) Wf[b][ri][j].load(Ws + ((2 * kp + j) * 2 + ri) * 1024);
+        for (int j = 0; j < 2; ++j) Kf[b][ri][j].load(Ka + ((2 * kp + j) * 2 + ri) * 1024);
     };
-    auto load_k = [&](int b, int kp) {
+    auto load_kt = [&](int b, int kp) {     // K^T: (lane <-> K column, registers <-> token)
 #pragma unroll
       for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int tj = 0; tj < 2; ++tj) Kf[b][j][tj].load(KT + ((2 * kp + j) * 2 + tj) * 1024);
+        for (int tj = 0; tj < 2; ++tj) Kf[b][j][tj].load_t(Ka + ((2 * kp + j) * 2 + tj) * 1024);
     };
-    AccB<T> Vb[2];
-    Vb[0].load(Uf);
-    Vb[1].load(Uf + 1024);
-    load_w(0, 0);
-    if (NP > 1) load_w(1, 1);
-    const float eg = __expf(dec[64]);
+    AccB<T> Vb[2], Tf[3];
+    Vb[0].load_cols(Vs + 32 * wave, 32 * NW);                     // raw v, (lane <-> V column, registers <-> token)
+    Vb[1].load_cols(Vs + 32 * (32 * NW) + 32 * wave, 32 * NW);
+    load_k(0, 0);
+    if (NP > 1) load_k(1, 1);
+    const float eg = __expf(row[256]);
+    if (hf != nullptr) {
 #pragma unroll
-    for (int kt = 0; kt < NKT; ++kt) Sb[kt].store_stream(hf + (tile0 * NKT + kt) * 1024);
-    // V' = U - W S: the accumulators start from U and the W tiles arrive negated; the two 32-token blocks are
-    // independent accumulation chains.  The decay of S rides between the matrix instructions.
-    f32x16 p0 = Vb[0].unpack(), p1 = Vb[1].unpack();
+      for (int kt = 0; kt < NKT; ++kt) Sb[kt].store_stream(hf + (tile0 * NKT + kt) * 1024);
+    }
+    // y = K S, the two 32-token blocks are independent accumulation chains.  The decay of S rides between the matrix
+    // instructions.
+    f32x16 p0 = acc_zero(), p1 = acc_zero();
     GDN_SCHED_FENCE();
 #pragma unroll
     for (int kp = 0; kp < NP; ++kp) {
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        mma32_ff<T>(p0, Wf[kp & 1][0][j], Sb[2 * kp + j]);
-        mma32_ff<T>(p1, Wf[kp & 1][1][j], Sb[2 * kp + j]);
+        mma32_ff<T>(p0, Kf[kp & 1][0][j], Sb[2 * kp + j]);
+        mma32_ff<T>(p1, Kf[kp & 1][1][j], Sb[2 * kp + j]);
 #pragma unroll
         for (int r = 0; r < 16; ++r) S[2 * kp + j][r] *= eg;
         GDN_INTERLEAVE_MFMA_VALU(2 * AccK<T>::kGroups, 16 / (2 * AccK<T>::kGroups));
       }
       GDN_SCHED_FENCE();
-      if (kp + 2 < NP) load_w(kp & 1, kp + 2);
-      if (kp == (NP > 1 ? NP - 2 : 0)) load_k(0, 0);
-      if (kp == NP - 1 && NP > 1) load_k(1, 1);
+      if (kp + 2 < NP) load_k(kp & 1, kp + 2);
       GDN_SCHED_FENCE();
     }
-    const f32x16 d0 = rows_ld(dec, 0), d1 = rows_ld(dec, 32);
+#pragma unroll
+    for (int t = 0; t < 3; ++t) Tf[t].load(Tm + t * 1024);
+    {
+      // z = beta (v - e^G . y), the B operand of Tm z
+      const f32x16 b0 = rows_ld(row + 128, 0), b1 = rows_ld(row + 128, 32);
+      const f32x16 e0 = rows_ld(row + 64, 0), e1 = rows_ld(row + 64, 32);
+      const f32x16 x0 = Vb[0].unpack(), x1 = Vb[1].unpack();
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { p0[r] = b0[r] * x0[r] - e0[r] * p0[r]; p1[r] = b1[r] * x1[r] - e1[r] * p1[r]; }
+      Vb[0].pack(p0);
+      Vb[1].pack(p1);
+    }
+    load_kt(0, 0);
+    // V' = Tm z (Tm lower triangular: tiles (0,0), (1,0), (1,1))
+    p0 = acc_zero();
+    p1 = acc_zero();
+    mma32_ff<T>(p0, Tf[0], Vb[0]);
+    mma32_ff<T>(p1, Tf[1], Vb[0]);
+    mma32_ff<T>(p1, Tf[2], Vb[1]);
+    if (NP > 1) load_kt(1, 1);
+    const f32x16 d0 = rows_ld(row, 0), d1 = rows_ld(row, 32);
     Vb[0].pack(p0);
     Vb[1].pack(p1);
-    Vb[0].store_stream(vf + (tile0 * 2 + 0) * 1024);
-    Vb[1].store_stream(vf + (tile0 * 2 + 1) * 1024);
+    if (vf != nullptr) {
+      Vb[0].store_stream(vf + (tile0 * 2 + 0) * 1024);
+      Vb[1].store_stream(vf + (tile0 * 2 + 1) * 1024);
+    }
+    if constexpr (OUT) {
+      T* vx = xs + 2 * DK * 32 + (c & 1) * 2048;
+      Vb[0].store(vx);
+      Vb[1].store(vx + 1024);
+    }
     // the decay of the state update rides on V': (e^{G_last - G} . K)^T V' = K^T (e^{G_last - G} . V'), so that the
-    // K^T tiles are the same for every value head of a q/k group
+    // K tiles are the same for every value head of a q/k group
 #pragma unroll
     for (int r = 0; r < 16; ++r) { p0[r] *= d0[r]; p1[r] *= d1[r]; }
     Vb[0].pack(p0);
@@ -592,12 +650,17 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ?
         if (kt >= 2) Sb[kt - 2].pack(S[kt - 2]);
       }
       GDN_SCHED_FENCE();
-      if (kp + 2 < NP) { load_k(kp & 1, kp + 2); GDN_SCHED_FENCE(); }
+      if (kp + 2 < NP) { load_kt(kp & 1, kp + 2); GDN_SCHED_FENCE(); }
     }
 #pragma unroll
     for (int kt = (NKT >= 2 ? NKT - 2 : 0); kt < NKT; ++kt) Sb[kt].pack(S[kt]);
-    if (STAGES == 1 && c + 1 < nchunks) GDN_LDS_BARRIER();      // (B) done with the single stage
+    if constexpr (OUT) {   // the state before chunk c+1, for the output wave's next step
+#pragma unroll
+      for (int kt = 0; kt < NKT; ++kt) Sb[kt].store(xs + ((c + 1) & 1) * (DK * 32) + kt * 1024);
+    }
+    if (STAGES == 1 && c + 1 < nsteps) GDN_LDS_BARRIER();      // (B) done with the single stage
   }
+  if constexpr (OUT) GDN_LDS_BARRIER();       // (A) of the extra step: the last V' is in LDS for the output wave
   if (ht != nullptr) {
 #pragma unroll
     for (int kt = 0; kt < NKT; ++kt)
@@ -774,7 +837,9 @@ struct FwdNorm {
   bool weight_fp32;
 };
 
-template <typename T, int DK, int BVP, int NW, int NWS, int NLS, int STAGES>
+// NW: waves (32-column blocks) per workgroup of the stand-alone output kernel; NWS, NLS, STAGES: slabs, loader waves
+// and LDS stages of the recurrence kernel; FUSE: the recurrence kernel's own output waves write O (no norm, bf16)
+template <typename T, int DK, int NW, int NWS, int NLS, int STAGES, bool FUSE>
 static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const void* q, const void* k, const void* v,
                             const float* g, const float* beta, const float* h0, const int64_t* cu, void* o, float* ht,
                             unsigned char* ws, float scale, int l2norm, bool with_backward, const FwdNorm& fn,
@@ -786,38 +851,49 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   if (cu != nullptr) GDN_LAUNCH(kKernChunkTable, st, chunk_table_kernel, dim3(1), dim3(kThreads), 0, st, cu, chunk_offsets, d.N);
   float* rstd = reinterpret_cast<float*>(ws + L.rstd);
   float* G = reinterpret_cast<float*>(ws + L.G);
-  T* Ai = with_backward ? reinterpret_cast<T*>(ws + L.Ai) : nullptr;
-  T* W = reinterpret_cast<T*>(ws + L.WAF);
+  T* Ai = reinterpret_cast<T*>(ws + L.Ai);
   T* AQ = reinterpret_cast<T*>(ws + L.AQ);
-  T* UF = reinterpret_cast<T*>(ws + L.UF);
-  T* KTF = reinterpret_cast<T*>(ws + L.KTF);
-  T* WF = with_backward ? reinterpret_cast<T*>(ws + L.WF) : nullptr;
-  T* KAF = with_backward ? reinterpret_cast<T*>(ws + L.KAF) : nullptr;
-  T* QTF = with_backward ? reinterpret_cast<T*>(ws + L.QTF) : nullptr;
-  T* VF = reinterpret_cast<T*>(ws + L.VF);
-  T* HF = reinterpret_cast<T*>(ws + L.HF);
+  T* KAF = reinterpret_cast<T*>(ws + L.KAF);
+  T* QTF = reinterpret_cast<T*>(ws + L.QTF);
+  const bool fuse = FUSE && fn.y == nullptr;
+  // the per-chunk states and v_new leave the recurrence kernel only for a later reader: the backward pass or the
+  // stand-alone output kernel
+  const bool keep = with_backward || !fuse;
+  T* VF = keep ? reinterpret_cast<T*>(ws + L.VF) : nullptr;
+  T* HF = keep ? reinterpret_cast<T*>(ws + L.HF) : nullptr;
+  const TokenStrides ts = d.strides();
   {
-    auto kern = chunk_prep_kernel<T, DK, BVP>;
-    constexpr int smem = PrepSmem<T, DK, BVP>::bytes;
+    auto kern = chunk_prep_kernel<T, DK>;
+    constexpr int smem = PrepSmem<T, DK>::bytes;
     if (int e = set_lds(kern, smem)) return e;
-    GDN_LAUNCH(kKernPrep, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, (const T*)v, g, beta, cu,
-               (const int*)chunk_offsets, G, Ai, W, UF, AQ, KTF, WF, KAF, QTF, rstd, rstd + (int64_t)nc * 64 * d.Hqk, d.T, d.N, d.Hqk,
-               d.Hv, d.V, scale, l2norm, d.strides());
+    GDN_LAUNCH(kKernPrep, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, g, beta, cu,
+               (const int*)chunk_offsets, G, Ai, AQ, KAF, QTF, rstd, rstd + (int64_t)nc * 64 * d.Hqk, d.T, d.N, d.Hqk,
+               d.Hv, scale, l2norm, ts);
   }
-  {
-    auto kern = chunk_state_kernel<T, DK, NWS, NLS, STAGES>;
-    constexpr int smem = StateSmem<T, DK, NWS, STAGES>::bytes;
+  auto launch_state = [&](auto kern, int smem, int waves, T* op) -> int {
     if (int e = set_lds(kern, smem)) return e;
-    GDN_LAUNCH(kKernStateFwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NWS)), dim3(64 * (NWS + NLS)), smem, st,
-               (const T*)KTF, (const T*)W, (const T*)UF, (const float*)G, h0, ht, VF, HF, cu,
-               (const int*)chunk_offsets, d.T, d.Hqk, d.Hv, d.V);
+    GDN_LAUNCH(kKernStateFwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NWS)), dim3(64 * waves), smem, st, (const T*)KAF,
+               (const T*)QTF, (const T*)Ai, (const T*)AQ, (const T*)v, (const float*)G, beta, h0, ht, VF, HF, op, cu,
+               (const int*)chunk_offsets, d.T, d.Hqk, d.Hv, d.V, scale, ts.v);
+    return 0;
+  };
+  if constexpr (FUSE) {
+    if (fuse) {
+      if (int e = launch_state(chunk_state_kernel<T, DK, NWS, NLS, STAGES, true>, StateSmem<T, DK, NWS, STAGES, true>::bytes,
+                               2 * NWS + NLS, (T*)o))
+        return e;
+      return (int)hipGetLastError();
+    }
   }
+  if (int e = launch_state(chunk_state_kernel<T, DK, NWS, NLS, STAGES, false>, StateSmem<T, DK, NWS, STAGES, false>::bytes,
+                           NWS + NLS, (T*)nullptr))
+    return e;
   auto launch_out = [&](auto kern, auto nm) -> int {
     constexpr int smem = OutSmem<T, DK, NW>::bytes;
     if (int e = set_lds(kern, smem)) return e;
     GDN_LAUNCH(kKernOut, st, kern, dim3(nc, d.Hv, d.V / (32 * NW)), dim3(64 * NW), smem, st, qq,
                (const T*)AQ, (const T*)VF, (const T*)HF, (const float*)G, (T*)o, cu, (const int*)chunk_offsets, d.T, d.N, d.Hqk,
-               d.Hv, d.V, scale, d.strides().q, l2norm ? (const float*)rstd : (const float*)nullptr, nm);
+               d.Hv, d.V, scale, ts.q, l2norm ? (const float*)rstd : (const float*)nullptr, nm);
     return 0;
   };
   if (fn.y == nullptr) {
@@ -879,26 +955,26 @@ static int chunk_fwd_entry(const void* q, const void* k, const void* v, int64_t 
   dl.varlen = true;  // one layout for both modes (the packed bound is the larger)
   const ChunkWorkspace L = chunk_workspace_layout(dl, dtype == 0 ? 4 : 2);
   if (workspace_bytes < L.fwd_bytes) return -5;
-  const bool with_bwd = workspace_bytes >= L.total_bytes;   // a workspace sized for backward also receives W^T fragments
+  const bool with_bwd = workspace_bytes >= L.total_bytes;   // a workspace sized for backward: the per-chunk states and v_new are kept
   if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
   unsigned char* ws = static_cast<unsigned char*>(workspace);
   hipStream_t st = (hipStream_t)stream;
-#define GDN_FWD(T_, DK_, BVP_, NW_, NWS_, NLS_, ST_)                                                                        \
-  return chunk_fwd_launch<T_, DK_, BVP_, NW_, NWS_, NLS_, ST_>(d, L, q, k, v, g, beta, initial_state, cu_seqlens, o, final_state, \
+#define GDN_FWD(T_, DK_, NW_, NWS_, NLS_, ST_, FUSE_)                                                                       \
+  return chunk_fwd_launch<T_, DK_, NW_, NWS_, NLS_, ST_, FUSE_>(d, L, q, k, v, g, beta, initial_state, cu_seqlens, o, final_state, \
                                                    ws, scale, use_qk_l2norm, with_bwd, fn, st)
   const bool wide = (V % 128 == 0);
   const bool solo = one_slab_per_workgroup(d, device_compute_units());
   if (dtype == 1) {
-    if (K == 128 && wide && solo) GDN_FWD(bf16_t, 128, 128, 4, 1, 2, 2);
-    if (K == 128 && wide) GDN_FWD(bf16_t, 128, 128, 4, 2, 2, 2);
-    if (K == 128) GDN_FWD(bf16_t, 128, 64, 2, 2, 2, 2);
-    if (K == 64 && wide) GDN_FWD(bf16_t, 64, 128, 4, 2, 2, 2);
-    GDN_FWD(bf16_t, 64, 64, 2, 2, 2, 2);
+    if (K == 128 && wide && solo) GDN_FWD(bf16_t, 128, 4, 1, 4, 2, true);
+    if (K == 128 && wide) GDN_FWD(bf16_t, 128, 4, 2, 4, 2, true);
+    if (K == 128) GDN_FWD(bf16_t, 128, 2, 2, 4, 2, true);
+    if (K == 64 && wide) GDN_FWD(bf16_t, 64, 4, 2, 4, 2, true);
+    GDN_FWD(bf16_t, 64, 2, 2, 4, 2, true);
   } else {
-    if (K == 128 && wide) GDN_FWD(float, 128, 64, 4, 4, 4, 1);
-    if (K == 128) GDN_FWD(float, 128, 64, 2, 2, 2, 1);
-    if (wide) GDN_FWD(float, 64, 64, 4, 4, 4, 2);
-    GDN_FWD(float, 64, 64, 2, 2, 2, 2);
+    if (K == 128 && wide) GDN_FWD(float, 128, 4, 4, 4, 1, false);
+    if (K == 128) GDN_FWD(float, 128, 2, 2, 2, 1, false);
+    if (wide) GDN_FWD(float, 64, 4, 4, 4, 2, false);
+    GDN_FWD(float, 64, 2, 2, 2, 2, false);
   }
 #undef GDN_FWD
 }

@@ -317,6 +317,15 @@ template <typename T> __device__ __forceinline__ u32x4 frag_a_split(const T* p) 
     return *reinterpret_cast<const u32x4*>(p + 4 * half);
   }
 }
+// Transposing read from LDS (ds_read_b64_tr_b16): every lane names 8 bytes (4 16-bit elements); within each group of
+// 16 lanes, lane 4 a + b receives element b of the lanes 4 e + a, e = 0..3.  Read as a 4 x 16 block of elements whose
+// row e is held, 4 columns each, by the lanes 4 e .. 4 e + 3: lane n of the group gets column n, rows 0..3.
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x2 lds_read_tr16(const void* p) {
+  const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
+  return __builtin_bit_cast(u32x2, v);
+}
+
 // all k-groups of one 32x32 accumulator tile packed as operand fragments ("fragment order").  The same 1024
 // elements, stored as [k-group][lane][16 bytes], are also the on-memory format in which kernels hand tiles to
 // each other: a lane writes/reads 16 contiguous bytes per k-group and never goes through LDS.
@@ -372,6 +381,56 @@ template <typename T> struct AccB {
     const int lane = threadIdx.x & 63;
 #pragma unroll
     for (int g = 0; g < kG; ++g) f[g] = *reinterpret_cast<const u32x4*>(tile + (g * 64 + lane) * kVecElems);
+  }
+  // The fragments of X^T from a tile in LDS that holds X in fragment order: what load() followed by a turn through
+  // the matrix core and pack() gives, without either.  Element (lane a, register index b) of a fragment-order tile
+  // sits at [k-group of b][a][position of b]; a lane of the transposed set needs a run of consecutive a for one b,
+  // which is a column of 16-byte rows: 16-bit types read it with the transposing LDS read, four a at a time.
+  __device__ __forceinline__ void load_t(const T* tile) {
+    const int lane = threadIdx.x & 63;
+    if constexpr (sizeof(T) == 2) {
+      const int gr = lane >> 4, i = lane & 15, e = i >> 2, q = i & 3, hh = gr >> 1;
+      const T* base = tile + (((gr & 1) * 64 + 32 * (q & 1) + 4 * hh + e) * 8 + 4 * (q >> 1));
+#pragma unroll
+      for (int g = 0; g < 2; ++g)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          const u32x2 r = lds_read_tr16(base + (16 * g + 8 * t) * 8);
+          f[g][2 * t] = r[0];
+          f[g][2 * t + 1] = r[1];
+        }
+    } else {
+      const int m = lane & 31, h = lane >> 5;
+      const T* base = tile + (((m >> 3) * 64 + 32 * ((m & 7) >> 2) + 4 * h) * 4 + (m & 3));
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) f[g][e] = __float_as_uint(Elem<T>::to_f(base[(8 * g + e) * 4]));
+    }
+  }
+  // From a row-major tile in LDS (x = &X[first row][first column], rows ld elements apart, ld a multiple of 4):
+  // lane <-> column, registers <-> row, i.e. X as a B operand contracted over its rows, or, unpack()ed, X in the
+  // accumulator layout.
+  __device__ __forceinline__ void load_cols(const T* x, int ld) {
+    const int lane = threadIdx.x & 63;
+    if constexpr (sizeof(T) == 2) {
+      const int gr = lane >> 4, i = lane & 15, e = i >> 2, q = i & 3, hh = gr >> 1;
+      const T* base = x + (4 * hh + e) * ld + (gr & 1) * 16 + 4 * q;
+#pragma unroll
+      for (int g = 0; g < 2; ++g)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          const u32x2 r = lds_read_tr16(base + (16 * g + 8 * t) * ld);
+          f[g][2 * t] = r[0];
+          f[g][2 * t + 1] = r[1];
+        }
+    } else {
+      const int m = lane & 31, h = lane >> 5;
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) f[g][e] = __float_as_uint(Elem<T>::to_f(x[(8 * g + 4 * h + e) * ld + m]));
+    }
   }
 };
 // d(32x32) += A[32 rows][32 k] * B(32 k x 32) with B packed from an accumulator; arow = &A[row of this lane][k0]

@@ -134,6 +134,22 @@ template <class T> inline T shfl(T v, int src) {
   return o;
 }
 
+// ds_read_b64_tr_b16: within each group of 16 lanes, lane 4 a + b receives element b of the lanes 4 e + a, e = 0..3
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+inline s16x4_t ds_read_tr16(const void* p) {
+  uint64_t mine;
+  memcpy(&mine, p, 8);
+  auto s = wave_exchange(&mine, 8);
+  const int l = lane(), base = l & ~15, n = l & 15;
+  s16x4_t out;
+  for (int e = 0; e < 4; ++e) {
+    uint16_t h;
+    memcpy(&h, s[base + 4 * e + (n >> 2)] + 2 * (n & 3), 2);
+    out[e] = (short)h;
+  }
+  return out;
+}
+
 // rendezvous of the lanes of one wave (lanes run as cooperative fibers: a wave-private LDS hand-over needs one)
 inline void wave_sync() { char c = 0; (void)wave_exchange(&c, 1); }
 
@@ -255,6 +271,7 @@ static emu::GdimProxy gridDim;
 #define __builtin_amdgcn_wave_barrier() emu::wave_sync()
 #define __builtin_amdgcn_readfirstlane(x) (x)
 #define __builtin_amdgcn_s_waitcnt(x) ((void)0)
+#define __builtin_amdgcn_ds_read_tr16_b64_v4i16(p) emu::ds_read_tr16((const void*)(uintptr_t)(p))
 // direct global -> LDS load: lane l's `size` bytes land at dst + l*size (done at once: the emulator has no asynchrony)
 #define __builtin_amdgcn_global_load_lds(src, dst, size, off, aux) \
   memcpy((unsigned char*)(uintptr_t)(dst) + (off) + emu::lane() * (size), (const void*)(uintptr_t)(src), (size))
