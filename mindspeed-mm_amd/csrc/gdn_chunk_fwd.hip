@@ -486,6 +486,11 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
           AccB<T> Vb[2];
           Vb[0].load(vx);
           Vb[1].load(vx + 1024);
+          if (vf != nullptr) {   // v_new of chunk c-1, for the backward pass
+            const int64_t tile0 = ((chunk_base + c - 1) * Hv + h) * (V / 32) + vblk;
+            Vb[0].store_stream(vf + (tile0 * 2 + 0) * 1024);
+            Vb[1].store_stream(vf + (tile0 * 2 + 1) * 1024);
+          }
           mma32_ff<T>(oa[0], Af[0], Vb[0]);
           mma32_ff<T>(oa[1], Af[1], Vb[0]);
           mma32_ff<T>(oa[1], Af[2], Vb[1]);
@@ -506,6 +511,8 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
           for (int kt = 0; kt < NKT; ++kt) {
             AccB<T> Sb, Qf;
             Sb.load(sx + kt * 1024);
+            if (hf != nullptr)   // the state before chunk c, for the backward pass
+              Sb.store_stream(hf + ((((chunk_base + c) * Hv + h) * (V / 32) + vblk) * NKT + kt) * 1024);
 #pragma unroll
             for (int ri = 0; ri < 2; ++ri) {
               Qf.load_t(st + SM::off_q + (kt * 2 + ri) * 1024);   // Q tile (token block ri, K block kt)
@@ -577,7 +584,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
     load_k(0, 0);
     if (NP > 1) load_k(1, 1);
     const float eg = __expf(row[256]);
-    if (hf != nullptr) {
+    if (!OUT && hf != nullptr) {   // with output waves the stores are theirs: they hold S and V' too and have the time
 #pragma unroll
       for (int kt = 0; kt < NKT; ++kt) Sb[kt].store_stream(hf + (tile0 * NKT + kt) * 1024);
     }
@@ -622,7 +629,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
     const f32x16 d0 = rows_ld(row, 0), d1 = rows_ld(row, 32);
     Vb[0].pack(p0);
     Vb[1].pack(p1);
-    if (vf != nullptr) {
+    if (!OUT && vf != nullptr) {
       Vb[0].store_stream(vf + (tile0 * 2 + 0) * 1024);
       Vb[1].store_stream(vf + (tile0 * 2 + 1) * 1024);
     }
