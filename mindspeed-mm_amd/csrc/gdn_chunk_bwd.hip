@@ -30,18 +30,19 @@ namespace gdn {
 // operands straight from registers.  dS (gradient of the state AFTER the chunk) and dV' leave in fragment order.
 // Loader waves copy the A operands from contiguous fragment-order blocks: K and Q^T per q/k group, Tm and Aq per value
 // head; K^T and Tm^T are the same images read with the transposing LDS read, and so are the slab's raw dO rows on
-// their way into the B-operand layout.
+// their way into the B-operand layout.  The per-token factors never enter the compute wave's dependent chain: the
+// loaders write K twice, rows scaled by e^{G_last-G} (for K dS) and by -beta e^G (for the K^T product), and dO twice,
+// raw and with rows scaled by scale e^G.
 // ---------------------------------------------------------------------------------------------
 template <typename T, int DK, int NW, int STAGES> struct StateBwdSmem {
   // one stage, in elements of T
-  static constexpr int off_k = 0;                        // K image [K/32][2] tiles
-  static constexpr int off_q = off_k + 64 * DK;          // Q^T image
+  static constexpr int off_k = 0;                        // K images [2][K/32][2] tiles: rows x e^{G_last-G}, rows x -beta e^G
+  static constexpr int off_q = off_k + 2 * 64 * DK;      // Q^T image
   static constexpr int off_tm = off_q + 64 * DK;         // Tm tiles (0,0), (1,0), (1,1)
   static constexpr int off_aq = off_tm + 3 * 1024;       // Aq tiles (0,0), (1,0), (1,1)
-  static constexpr int off_do = off_aq + 3 * 1024;       // raw dO rows of the slabs [64][32 NW]
-  static constexpr int off_row = (off_do + 64 * 32 * NW) * (int)sizeof(T);   // bytes: float rows
-  // rows: e^{G_last-G} [64], beta e^G [64], scale e^G [64], G_last
-  static constexpr int stage = off_row + (3 * 64 + 4) * 4;
+  static constexpr int off_do = off_aq + 3 * 1024;       // dO rows of the slabs [2][64][32 NW]: raw, rows x scale e^G
+  static constexpr int off_row = (off_do + 2 * 64 * 32 * NW) * (int)sizeof(T);   // bytes: G_last
+  static constexpr int stage = off_row + 16;
   static constexpr int bytes = STAGES * stage;
   static_assert(bytes <= 160 * 1024, "one CU's LDS");
 };
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
     const int lt = tid - 64 * NW;
     constexpr int DEPTH = (STAGES == 2) ? 2 : 1;
     Vec16<T> pk[DEPTH][CK], pq[DEPTH][CK], ptm[DEPTH][CTM], pa[DEPTH][CTM], pd[DEPTH][CD];
-    float pgl[DEPTH], pg[DEPTH], pb[DEPTH];
+    float pgl[DEPTH], pgk[DEPTH][2], pbk[DEPTH][2], pgd[DEPTH][CD];
     int pnv[DEPTH];
     auto tm_src = [&](int idc) {   // piece of the three kept tiles -> its place among the four stored ones
       const int t = idc / (1024 / VEC);
@@ -100,22 +101,33 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
       for (int i = 0; i < CD; ++i) {   // dO rows of the slabs; rows past the end repeat the last one and are cleared below
         const int idc = imin(lt + i * NT, PD - 1), row = imin(idc / DPR, nvalid - 1), cc = idc % DPR;
         pd[set][i] = ld16(dO + ((tok0 + row) * Hv + h) * V + blockIdx.y * (32 * NW) + cc * VEC);
+        pgd[set][i] = G[ch * 64 + row];
       }
       const float* gc = G + ch * 64;
-      const int t = lt & 63;
       // raw values only: arithmetic here would wait for every load issued so far.  The array repeats G_last past the
-      // end of a short chunk.
+      // end of a short chunk.  In the K tiles every 16-byte piece belongs to one token, 32 (tile & 1) + lane % 32, and
+      // this thread's pieces all have lane % 32 = lt % 32: the gates of two tokens cover them.
       pgl[set] = gc[63];
-      pg[set] = gc[t];
-      pb[set] = beta[(tok0 + imin(t, nvalid - 1)) * Hv + h];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        pgk[set][j] = gc[32 * j + (lt & 31)];
+        pbk[set][j] = beta[(tok0 + imin(32 * j + (lt & 31), nvalid - 1)) * Hv + h];
+      }
       pnv[set] = nvalid;
     };
     auto commit = [&](int set, int buf) {
       T* st = reinterpret_cast<T*>(gdn_smem + buf * SM::stage);
+      float f1[2], f2[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        f1[j] = __expf(pgl[set] - pgk[set][j]);
+        f2[j] = (32 * j + (lt & 31) < pnv[set]) ? -pbk[set][j] * __expf(pgk[set][j]) : 0.f;
+      }
 #pragma unroll
       for (int i = 0; i < CK; ++i) {
-        const int idc = imin(lt + i * NT, PK - 1);
-        st16(st + SM::off_k + idc * VEC, pk[set][i]);
+        const int idc = imin(lt + i * NT, PK - 1), tj = (idc / (1024 / VEC)) & 1;
+        st16(st + SM::off_k + idc * VEC, scale16<T>(pk[set][i], f1[tj]));
+        st16(st + SM::off_k + 64 * DK + idc * VEC, scale16<T>(pk[set][i], f2[tj]));
         st16(st + SM::off_q + idc * VEC, pq[set][i]);
       }
 #pragma unroll
@@ -127,16 +139,12 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
 #pragma unroll
       for (int i = 0; i < CD; ++i) {
         const int idc = imin(lt + i * NT, PD - 1);
-        st16(st + SM::off_do + idc * VEC, idc / DPR < pnv[set] ? pd[set][i] : zero16<T>());
+        const Vec16<T> x = idc / DPR < pnv[set] ? pd[set][i] : zero16<T>();
+        st16(st + SM::off_do + idc * VEC, x);
+        st16(st + SM::off_do + 64 * 32 * NW + idc * VEC, scale16<T>(x, scale * __expf(pgd[set][i])));
       }
       float* row = reinterpret_cast<float*>(gdn_smem + buf * SM::stage + SM::off_row);
-      if (lt < 64) {
-        const float b = lt < pnv[set] ? pb[set] : 0.f, eg = __expf(pg[set]);
-        row[lt] = __expf(pgl[set] - pg[set]);
-        row[64 + lt] = b * eg;
-        row[128 + lt] = scale * eg;
-      }
-      if (lt == 0) row[192] = pgl[set];
+      if (lt == 0) row[0] = pgl[set];
     };
     if (nchunks == 0) return;
     if (STAGES == 2) {
@@ -189,37 +197,32 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
     const int buf = (STAGES == 2) ? (st & 1) : 0;
     GDN_LDS_BARRIER();                      // (A)
     const T* sm = reinterpret_cast<const T*>(gdn_smem + buf * SM::stage);
-    const T* Ka = sm + SM::off_k;
+    const T* Ka = sm + SM::off_k;              // rows x e^{G_last-G}
+    const T* Kn = Ka + 64 * DK;                // rows x -beta e^G
     const T* Qa = sm + SM::off_q;
     const T* Tm = sm + SM::off_tm;
     const T* Aq = sm + SM::off_aq;
     const T* dOs = sm + SM::off_do;
     const float* row = reinterpret_cast<const float*>(gdn_smem + buf * SM::stage + SM::off_row);
-    // dO of this wave's 32 columns as B operand (lane <-> V column, registers <-> token), and scaled by scale e^G of
-    // its token: the factor of the Q^T product rides on dO, so that the Q^T tiles are the same for every value head
+    // dO of this wave's 32 columns as B operand (lane <-> V column, registers <-> token), raw and scaled by scale e^G
+    // of its token: the factor of the Q^T product rides on dO, so that the Q^T tiles are the same for every value head
     // of a q/k group
     AccB<T> dob[2], dos[2], aq[3];
     dob[0].load_cols(dOs + 32 * wave, 32 * NW);
     dob[1].load_cols(dOs + 32 * (32 * NW) + 32 * wave, 32 * NW);
+    dos[0].load_cols(dOs + 64 * 32 * NW + 32 * wave, 32 * NW);
+    dos[1].load_cols(dOs + 64 * 32 * NW + 32 * (32 * NW) + 32 * wave, 32 * NW);
     aq[0].load(Aq);                           // tiles (0,0), (1,0), (1,1)
     aq[1].load(Aq + 1024);
     aq[2].load(Aq + 2048);
-    const float eg = __expf(row[192]);
+    const float eg = __expf(row[0]);
     const int64_t tile0 = ((chunk_base + c) * Hv + h) * (V / 32) + vblk;
 #pragma unroll
     for (int kt = 0; kt < NKT; ++kt) dSb[kt].store_stream(dhf + (tile0 * NKT + kt) * 1024);
-    {
-      const f32x16 q0 = rows_ld(row + 128, 0), q1 = rows_ld(row + 128, 32);
-      f32x16 t0 = dob[0].unpack(), t1 = dob[1].unpack();
-#pragma unroll
-      for (int r = 0; r < 16; ++r) { t0[r] *= q0[r]; t1[r] *= q1[r]; }
-      dos[0].pack(t0);
-      dos[1].pack(t1);
-    }
-    // dv_local = (scale tril(Q K^T . Gam))^T dO from the forward pass's tiles, and y = K dS, one accumulation chain per
-    // 32-token block each.  The A-operand tiles come from LDS two tiles ahead of the matrix instructions that use
+    // dV' = (scale tril(Q K^T . Gam))^T dO (from the forward pass's tiles) + (e^{G_last-G} . K) dS, one accumulation
+    // chain per 32-token block.  The A-operand tiles come from LDS two tiles ahead of the matrix instructions that use
     // them; the decay of dS rides in between.
-    f32x16 a0 = acc_zero(), a1 = acc_zero(), y0 = acc_zero(), y1 = acc_zero();
+    f32x16 a0 = acc_zero(), a1 = acc_zero();
     AccB<T> af[3];
     af[0].load(Ka);
     af[1].load(Ka + 1024);
@@ -230,44 +233,32 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
 #pragma unroll
     for (int i = 0; i < 2 * NKT; ++i) {       // tile i = (K tile i / 2, token block i % 2)
       if (i + 2 < 2 * NKT) af[(i + 2) % 3].load(Ka + (i + 2) * 1024);
-      mma32_ff<T>((i & 1) ? y1 : y0, af[i % 3], dSb[i / 2]);
+      mma32_ff<T>((i & 1) ? a1 : a0, af[i % 3], dSb[i / 2]);
 #pragma unroll
       for (int r = 0; r < 8; ++r) dS[i / 2][8 * (i & 1) + r] *= eg;
       GDN_SCHED_FENCE();
     }
-    // dV' = e^{G_last-G} . y + dv_local
     AccB<T> dvb[2], rb[2], tf[3];
 #pragma unroll
     for (int t = 0; t < 3; ++t) tf[t].load_t(Tm + t * 1024);   // Tm^T tiles: (lane <-> column of Tm, registers <-> row)
-    {
-      const f32x16 d0 = rows_ld(row, 0), d1 = rows_ld(row, 32);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) { a0[r] += d0[r] * y0[r]; a1[r] += d1[r] * y1[r]; }
-    }
     dvb[0].pack(a0);
     dvb[1].pack(a1);
     dvb[0].store_stream(dvf + (tile0 * 2 + 0) * 1024);
     dvb[1].store_stream(dvf + (tile0 * 2 + 1) * 1024);
-    // R = Tm^T dV' (upper triangular: R_0 = Tm00^T dV'_0 + Tm10^T dV'_1, R_1 = Tm11^T dV'_1), then -(beta e^G . R)
-    y0 = acc_zero();
-    y1 = acc_zero();
+    // R = Tm^T dV' (upper triangular: R_0 = Tm00^T dV'_0 + Tm10^T dV'_1, R_1 = Tm11^T dV'_1)
+    f32x16 y0 = acc_zero(), y1 = acc_zero();
     mma32_ff<T>(y0, tf[0], dvb[0]);
     mma32_ff<T>(y1, tf[2], dvb[1]);
     mma32_ff<T>(y0, tf[1], dvb[1]);
     auto tile_qk = [&](int i) {               // i = 4 kt + 2 tj + (0: Q^T, 1: K^T)
-      return ((i & 1) ? Ka : Qa) + ((i >> 2) * 2 + ((i >> 1) & 1)) * 1024;
+      return ((i & 1) ? Kn : Qa) + ((i >> 2) * 2 + ((i >> 1) & 1)) * 1024;
     };
     af[0].load(tile_qk(0));
     af[1].load_t(tile_qk(1));
-    {
-      const f32x16 e0 = rows_ld(row + 64, 0), e1 = rows_ld(row + 64, 32);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) { y0[r] *= -e0[r]; y1[r] *= -e1[r]; }
-      rb[0].pack(y0);
-      rb[1].pack(y1);
-    }
+    rb[0].pack(y0);
+    rb[1].pack(y1);
     GDN_SCHED_FENCE();
-    // dS <- e^{G_last} dS + Q^T (scale e^G . dO) - K^T (beta e^G . R); a finished tile of dS is packed for the next
+    // dS <- e^{G_last} dS + Q^T (scale e^G . dO) + (-beta e^G . K)^T R; a finished tile of dS is packed for the next
     // step while the matrix pipe works on the following one
 #pragma unroll
     for (int i = 0; i < 4 * NKT; ++i) {
@@ -837,7 +828,7 @@ extern "C" int gdn_chunk_bwd_strided(const void* q, const void* k, const void* v
     GDN_BWD(bf16_t, 64, 2, 2, 2, 2);
   } else {
     if (K == 128) GDN_BWD(float, 128, 2, 2, 2, 1);
-    GDN_BWD(float, 64, 2, 2, 2, 2);
+    GDN_BWD(float, 64, 2, 2, 2, 1);
   }
 #undef GDN_BWD
 }

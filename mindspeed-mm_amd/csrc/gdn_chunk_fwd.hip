@@ -309,23 +309,34 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
 // fragment-order tiles prepared by chunk_prep_kernel (K per q/k group, Tm per value head), one contiguous block per
 // chunk; K^T is the same K image read with the transposing LDS read, and the slab's raw v rows are read the same way
 // into the accumulator layout.  NL loader waves of the workgroup copy the next chunks' operands global -> registers ->
-// LDS two chunks ahead (two LDS stages); the roles meet at one barrier per chunk.
+// LDS two chunks ahead (two LDS stages); the roles meet at one barrier per chunk.  Where LDS allows (PRE) the loaders
+// write K twice, rows scaled by -beta e^G and by e^{G_last-G}, and v scaled by beta, so that the per-token factors
+// never enter the compute wave's dependent chain: z is the accumulator of (-beta e^G K) S started from beta v.
 // OUT: a second wave per slab forms the output O = scale e^G . (Q S) + Aq V' of the same 32 columns from the state and
 // V' the compute wave leaves in LDS (Q read transposed from the Q^T image, Aq likewise), one step behind it, so that
 // neither S nor V' has to be re-read from memory; both are still stored when a backward pass will need them.
 // ---------------------------------------------------------------------------------------------
-template <typename T, int DK, int NW, int STAGES, bool OUT> struct StateSmem {
+// PRE: two images of K, rows scaled by -beta e^G and by e^{G_last-G} on their way into LDS.  Whether they fit is
+// decided for the variant with output waves (FUSE), and the variant without them follows, so that both round alike.
+template <typename T, int DK, int NW, int STAGES, bool FUSE> struct StatePre {
+  static constexpr int x_elems = 2 * DK * 32 + 2 * 2048 + Patch<T>::kElems;
+  static constexpr bool value = STAGES * ((2 * 64 * DK + 3 * 1024 + 64 * 32 * NW + (FUSE ? 64 * DK + 3 * 1024 : 0)) * (int)sizeof(T) + 68 * 4) +
+                                    (FUSE ? NW * x_elems * (int)sizeof(T) : 0) <= 160 * 1024;
+};
+template <typename T, int DK, int NW, int STAGES, bool OUT, bool PRE_> struct StateSmem {
+  static constexpr int x_elems = 2 * DK * 32 + 2 * 2048 + Patch<T>::kElems;
+  static constexpr bool PRE = PRE_;
   // one stage, in elements of T
-  static constexpr int off_k = 0;                                   // K image [K/32][2] tiles
-  static constexpr int off_tm = off_k + 64 * DK;                    // Tm tiles (0,0), (1,0), (1,1)
+  static constexpr int off_k = 0;                                   // K image(s) [K/32][2] tiles
+  static constexpr int off_tm = off_k + (PRE ? 2 : 1) * 64 * DK;    // Tm tiles (0,0), (1,0), (1,1)
   static constexpr int off_v = off_tm + 3 * 1024;                   // raw v rows of the slabs [64][32 NW]
   static constexpr int off_q = off_v + 64 * 32 * NW;                // OUT: Q^T image
   static constexpr int off_aq = off_q + (OUT ? 64 * DK : 0);        // OUT: Aq tiles (0,0), (1,0), (1,1)
   static constexpr int off_row = (off_aq + (OUT ? 3 * 1024 : 0)) * (int)sizeof(T);   // bytes: float rows
-  // rows: e^{G_last-G} [64], beta e^G [64], beta [64], scale e^G [64], G_last
-  static constexpr int stage = off_row + (4 * 64 + 4) * 4;
+  // rows: scale e^G [64], G_last; without PRE also e^{G_last-G} [64], beta e^G [64], beta [64]
+  static constexpr int stage = off_row + (PRE ? 68 : 260) * 4;   // a multiple of 16 bytes, like the offset of every row vector
+  static_assert(stage % 16 == 0, "stages keep 16-byte alignment");
   static constexpr int off_x = STAGES * stage;                      // OUT: per slab S [2][DK*32], V' [2][2048], store patch
-  static constexpr int x_elems = 2 * DK * 32 + 2 * 2048 + Patch<T>::kElems;
   static constexpr int bytes = off_x + (OUT ? NW * x_elems * (int)sizeof(T) : 0);
   static_assert(bytes <= 160 * 1024, "one CU's LDS");
 };
@@ -334,7 +345,7 @@ template <typename T, int DK, int NW, int STAGES, bool OUT> struct StateSmem {
 // piece (the same loads on every path; the duplicate lands on the same LDS address with the same data)
 template <int PIECES, int NT> struct Deal { static constexpr int kPer = (PIECES + NT - 1) / NT; };
 
-template <typename T, int DK, int NW, int NL, int STAGES, bool OUT>
+template <typename T, int DK, int NW, int NL, int STAGES, bool OUT, bool PRE_>
 __global__ __launch_bounds__(64 * (NW + (OUT ? NW : 0) + NL)) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 2 : 1)
 void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, const T* __restrict__ ai,
                         const T* __restrict__ aqf, const T* __restrict__ v, const float* __restrict__ G,
@@ -342,7 +353,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
                         T* __restrict__ vf, T* __restrict__ hf, T* __restrict__ o, const int64_t* __restrict__ cu,
                         const int* __restrict__ chunk_offsets, int T_len, int Hqk, int Hv, int V, float scale,
                         int64_t v_stride) {
-  using SM = StateSmem<T, DK, NW, STAGES, OUT>;
+  using SM = StateSmem<T, DK, NW, STAGES, OUT, PRE_>;
   constexpr int NT = 64 * NL, VEC = Elem<T>::kVec, NKT = DK / 32, NWO = OUT ? NW : 0;
   constexpr int PK = 64 * DK / VEC, PTM = 3 * 1024 / VEC, PV = 64 * 32 * NW / VEC, VPR = 32 * NW / VEC;
   constexpr int CK = Deal<PK, NT>::kPer, CTM = Deal<PTM, NT>::kPer, CV = Deal<PV, NT>::kPer;
@@ -376,8 +387,9 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
     // one that copies it to LDS (j - 1), so global loads have DEPTH chunk periods to arrive
     constexpr int DEPTH = (STAGES == 2) ? 2 : 1;
     Vec16<T> pk[DEPTH][CK], ptm[DEPTH][CTM], pv[DEPTH][CV], pq[DEPTH][OUT ? CK : 1], pa[DEPTH][OUT ? CTM : 1];
-    float pgl[DEPTH], pg[DEPTH], pb[DEPTH];
+    float pgl[DEPTH], pg[DEPTH], pb[DEPTH], pgk[DEPTH][2], pbk[DEPTH][2], pbv[DEPTH][CV];
     int pnv[DEPTH];
+    constexpr bool PRE = SM::PRE;
     auto tm_src = [&](int idc) {   // piece of the three kept tiles -> its place among the four stored ones
       const int t = idc / (1024 / VEC);
       return (t == 0 ? 0 : t + 1) * (1024 / VEC) + idc % (1024 / VEC);
@@ -402,6 +414,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
       for (int i = 0; i < CV; ++i) {   // rows past the end of the sequence repeat the last one (their beta is 0)
         const int idc = imin(lt + i * NT, PV - 1), row = imin(idc / VPR, nvalid - 1), cc = idc % VPR;
         pv[set][i] = ld16(v + (tok0 + row) * v_stride + (int64_t)h * V + blockIdx.y * (32 * NW) + cc * VEC);
+        if constexpr (PRE) pbv[set][i] = beta[(tok0 + row) * Hv + h];
       }
       const float* gc = G + ch * 64;
       const int t = lt & 63;
@@ -411,13 +424,36 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
       pg[set] = gc[t];
       pb[set] = beta[(tok0 + imin(t, nvalid - 1)) * Hv + h];
       pnv[set] = nvalid;
+      if constexpr (PRE) {
+        // In the K tiles every 16-byte piece belongs to one token, 32 (tile & 1) + lane % 32, and this thread's pieces
+        // all have lane % 32 = lt % 32: the gates of two tokens cover them.
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          pgk[set][j] = gc[32 * j + (lt & 31)];
+          pbk[set][j] = beta[(tok0 + imin(32 * j + (lt & 31), nvalid - 1)) * Hv + h];
+        }
+      }
     };
     auto commit = [&](int set, int buf) {   // registers -> LDS stage
       T* st = reinterpret_cast<T*>(gdn_smem + buf * SM::stage);
+      float f1[2], f2[2];
+      if constexpr (PRE) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          f1[j] = (32 * j + (lt & 31) < pnv[set]) ? -pbk[set][j] * __expf(pgk[set][j]) : 0.f;
+          f2[j] = __expf(pgl[set] - pgk[set][j]);
+        }
+      }
 #pragma unroll
       for (int i = 0; i < CK; ++i) {
         const int idc = imin(lt + i * NT, PK - 1);
-        st16(st + SM::off_k + idc * VEC, pk[set][i]);
+        if constexpr (PRE) {
+          const int tj = (idc / (1024 / VEC)) & 1;
+          st16(st + SM::off_k + idc * VEC, scale16<T>(pk[set][i], f1[tj]));
+          st16(st + SM::off_k + 64 * DK + idc * VEC, scale16<T>(pk[set][i], f2[tj]));
+        } else {
+          st16(st + SM::off_k + idc * VEC, pk[set][i]);
+        }
         if constexpr (OUT) st16(st + SM::off_q + idc * VEC, pq[set][i]);
       }
 #pragma unroll
@@ -427,16 +463,22 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
         if constexpr (OUT) st16(st + SM::off_aq + idc * VEC, pa[set][i]);
       }
 #pragma unroll
-      for (int i = 0; i < CV; ++i) st16(st + SM::off_v + imin(lt + i * NT, PV - 1) * VEC, pv[set][i]);
+      for (int i = 0; i < CV; ++i) {
+        const int idc = imin(lt + i * NT, PV - 1);
+        if constexpr (PRE) st16(st + SM::off_v + idc * VEC, scale16<T>(pv[set][i], idc / VPR < pnv[set] ? pbv[set][i] : 0.f));
+        else st16(st + SM::off_v + idc * VEC, pv[set][i]);
+      }
       float* row = reinterpret_cast<float*>(gdn_smem + buf * SM::stage + SM::off_row);
       if (lt < 64) {
         const float b = lt < pnv[set] ? pb[set] : 0.f, eg = __expf(pg[set]);
-        row[lt] = __expf(pgl[set] - pg[set]);
-        row[64 + lt] = b * eg;
-        row[128 + lt] = b;
-        row[192 + lt] = scale * eg;
+        row[lt] = scale * eg;
+        if constexpr (!PRE) {
+          row[68 + lt] = __expf(pgl[set] - pg[set]);
+          row[132 + lt] = b * eg;
+          row[196 + lt] = b;
+        }
       }
-      if (lt == 0) row[256] = pgl[set];
+      if (lt == 0) row[64] = pgl[set];
     };
     if (STAGES == 2) {
       // Every path through this loop issues the same loads in the same order (chunk indices past the end are clamped
@@ -519,7 +561,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
               mma32_ff<T>(oa[ri], Qf, Sb);
             }
           }
-          const f32x16 e0 = rows_ld(row + 192, 0), e1 = rows_ld(row + 192, 32);
+          const f32x16 e0 = rows_ld(row, 0), e1 = rows_ld(row, 32);
 #pragma unroll
           for (int r = 0; r < 16; ++r) { oa[0][r] *= e0[r]; oa[1][r] *= e1[r]; }
 #pragma unroll
@@ -558,7 +600,9 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
     const int buf = (STAGES == 2) ? (c & 1) : 0;
     GDN_LDS_BARRIER();                        // (A) stage `buf` holds chunk c
     const T* st = reinterpret_cast<const T*>(gdn_smem + buf * SM::stage);
-    const T* Ka = st + SM::off_k;
+    constexpr bool PRE = SM::PRE;
+    const T* Ka = st + SM::off_k;                        // PRE: rows scaled by -beta e^G
+    const T* Kb = Ka + (PRE ? 64 * DK : 0);              // PRE: rows scaled by e^{G_last-G}
     const T* Tm = st + SM::off_tm;
     const T* Vs = st + SM::off_v;
     const float* row = reinterpret_cast<const float*>(gdn_smem + buf * SM::stage + SM::off_row);
@@ -576,21 +620,21 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
 #pragma unroll
       for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int tj = 0; tj < 2; ++tj) Kf[b][j][tj].load_t(Ka + ((2 * kp + j) * 2 + tj) * 1024);
+        for (int tj = 0; tj < 2; ++tj) Kf[b][j][tj].load_t(Kb + ((2 * kp + j) * 2 + tj) * 1024);
     };
     AccB<T> Vb[2], Tf[3];
     Vb[0].load_cols(Vs + 32 * wave, 32 * NW);                     // raw v, (lane <-> V column, registers <-> token)
     Vb[1].load_cols(Vs + 32 * (32 * NW) + 32 * wave, 32 * NW);
     load_k(0, 0);
     if (NP > 1) load_k(1, 1);
-    const float eg = __expf(row[256]);
+    const float eg = __expf(row[64]);
     if (!OUT && hf != nullptr) {   // with output waves the stores are theirs: they hold S and V' too and have the time
 #pragma unroll
       for (int kt = 0; kt < NKT; ++kt) Sb[kt].store_stream(hf + (tile0 * NKT + kt) * 1024);
     }
-    // y = K S, the two 32-token blocks are independent accumulation chains.  The decay of S rides between the matrix
-    // instructions.
-    f32x16 p0 = acc_zero(), p1 = acc_zero();
+    // y = K S (PRE: z = beta v - beta e^G . (K S) at once), the two 32-token blocks are independent accumulation
+    // chains.  The decay of S rides between the matrix instructions.
+    f32x16 p0 = PRE ? Vb[0].unpack() : acc_zero(), p1 = PRE ? Vb[1].unpack() : acc_zero();
     GDN_SCHED_FENCE();
 #pragma unroll
     for (int kp = 0; kp < NP; ++kp) {
@@ -608,16 +652,16 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
     }
 #pragma unroll
     for (int t = 0; t < 3; ++t) Tf[t].load(Tm + t * 1024);
-    {
+    if constexpr (!PRE) {
       // z = beta (v - e^G . y), the B operand of Tm z
-      const f32x16 b0 = rows_ld(row + 128, 0), b1 = rows_ld(row + 128, 32);
-      const f32x16 e0 = rows_ld(row + 64, 0), e1 = rows_ld(row + 64, 32);
+      const f32x16 b0 = rows_ld(row + 196, 0), b1 = rows_ld(row + 196, 32);
+      const f32x16 e0 = rows_ld(row + 132, 0), e1 = rows_ld(row + 132, 32);
       const f32x16 x0 = Vb[0].unpack(), x1 = Vb[1].unpack();
 #pragma unroll
       for (int r = 0; r < 16; ++r) { p0[r] = b0[r] * x0[r] - e0[r] * p0[r]; p1[r] = b1[r] * x1[r] - e1[r] * p1[r]; }
-      Vb[0].pack(p0);
-      Vb[1].pack(p1);
     }
+    Vb[0].pack(p0);
+    Vb[1].pack(p1);
     load_kt(0, 0);
     // V' = Tm z (Tm lower triangular: tiles (0,0), (1,0), (1,1))
     p0 = acc_zero();
@@ -626,7 +670,6 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
     mma32_ff<T>(p1, Tf[1], Vb[0]);
     mma32_ff<T>(p1, Tf[2], Vb[1]);
     if (NP > 1) load_kt(1, 1);
-    const f32x16 d0 = rows_ld(row, 0), d1 = rows_ld(row, 32);
     Vb[0].pack(p0);
     Vb[1].pack(p1);
     if (!OUT && vf != nullptr) {
@@ -638,12 +681,14 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
       Vb[0].store(vx);
       Vb[1].store(vx + 1024);
     }
-    // the decay of the state update rides on V': (e^{G_last - G} . K)^T V' = K^T (e^{G_last - G} . V'), so that the
-    // K tiles are the same for every value head of a q/k group
+    if constexpr (!PRE) {
+      // the decay of the state update rides on V': (e^{G_last - G} . K)^T V' = K^T (e^{G_last - G} . V')
+      const f32x16 d0 = rows_ld(row + 68, 0), d1 = rows_ld(row + 68, 32);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { p0[r] *= d0[r]; p1[r] *= d1[r]; }
-    Vb[0].pack(p0);
-    Vb[1].pack(p1);
+      for (int r = 0; r < 16; ++r) { p0[r] *= d0[r]; p1[r] *= d1[r]; }
+      Vb[0].pack(p0);
+      Vb[1].pack(p1);
+    }
     GDN_SCHED_FENCE();
     // S <- e^{G_last} S + K^T (e^{G_last - G} . V'); a finished tile of S is packed for the next chunk while the
     // matrix pipe works on the following ones
@@ -877,6 +922,7 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
                (const int*)chunk_offsets, G, Ai, AQ, KAF, QTF, rstd, rstd + (int64_t)nc * 64 * d.Hqk, d.T, d.N, d.Hqk,
                d.Hv, scale, l2norm, ts);
   }
+  constexpr bool PRE = StatePre<T, DK, NWS, STAGES, FUSE>::value;
   auto launch_state = [&](auto kern, int smem, int waves, T* op) -> int {
     if (int e = set_lds(kern, smem)) return e;
     GDN_LAUNCH(kKernStateFwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NWS)), dim3(64 * waves), smem, st, (const T*)KAF,
@@ -886,14 +932,14 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   };
   if constexpr (FUSE) {
     if (fuse) {
-      if (int e = launch_state(chunk_state_kernel<T, DK, NWS, NLS, STAGES, true>, StateSmem<T, DK, NWS, STAGES, true>::bytes,
-                               2 * NWS + NLS, (T*)o))
+      if (int e = launch_state(chunk_state_kernel<T, DK, NWS, NLS, STAGES, true, PRE>,
+                               StateSmem<T, DK, NWS, STAGES, true, PRE>::bytes, 2 * NWS + NLS, (T*)o))
         return e;
       return (int)hipGetLastError();
     }
   }
-  if (int e = launch_state(chunk_state_kernel<T, DK, NWS, NLS, STAGES, false>, StateSmem<T, DK, NWS, STAGES, false>::bytes,
-                           NWS + NLS, (T*)nullptr))
+  if (int e = launch_state(chunk_state_kernel<T, DK, NWS, NLS, STAGES, false, PRE>,
+                           StateSmem<T, DK, NWS, STAGES, false, PRE>::bytes, NWS + NLS, (T*)nullptr))
     return e;
   auto launch_out = [&](auto kern, auto nm) -> int {
     constexpr int smem = OutSmem<T, DK, NW>::bytes;
