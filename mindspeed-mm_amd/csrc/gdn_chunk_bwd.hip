@@ -76,6 +76,8 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
     Vec16<T> pk[DEPTH][CK], pq[DEPTH][CK], ptm[DEPTH][CTM], pa[DEPTH][CTM], pd[DEPTH][CD];
     float pgl[DEPTH], pgk[DEPTH][2], pbk[DEPTH][2], pgd[DEPTH][CD];
     int pnv[DEPTH];
+    static_assert(NT % (sizeof(T) == 2 ? 128 : 32) == 0, "a thread's pieces sit at one place of their tiles");
+    const int krow = frag_piece_row<T>(lt & 127);
     auto tm_src = [&](int idc) {   // piece of the three kept tiles -> its place among the four stored ones
       const int t = idc / (1024 / VEC);
       return (t == 0 ? 0 : t + 1) * (1024 / VEC) + idc % (1024 / VEC);
@@ -105,13 +107,13 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
       }
       const float* gc = G + ch * 64;
       // raw values only: arithmetic here would wait for every load issued so far.  The array repeats G_last past the
-      // end of a short chunk.  In the K tiles every 16-byte piece belongs to one token, 32 (tile & 1) + lane % 32, and
-      // this thread's pieces all have lane % 32 = lt % 32: the gates of two tokens cover them.
+      // end of a short chunk.  In the K tiles every 16-byte piece belongs to one token, 32 (tile & 1) + the row of its
+      // place, and this thread's pieces all sit at the same place of their tiles: the gates of two tokens cover them.
       pgl[set] = gc[63];
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        pgk[set][j] = gc[32 * j + (lt & 31)];
-        pbk[set][j] = beta[(tok0 + imin(32 * j + (lt & 31), nvalid - 1)) * Hv + h];
+        pgk[set][j] = gc[32 * j + krow];
+        pbk[set][j] = beta[(tok0 + imin(32 * j + krow, nvalid - 1)) * Hv + h];
       }
       pnv[set] = nvalid;
     };
@@ -121,7 +123,7 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         f1[j] = __expf(pgl[set] - pgk[set][j]);
-        f2[j] = (32 * j + (lt & 31) < pnv[set]) ? -pbk[set][j] * __expf(pgk[set][j]) : 0.f;
+        f2[j] = (32 * j + krow < pnv[set]) ? -pbk[set][j] * __expf(pgk[set][j]) : 0.f;
       }
 #pragma unroll
       for (int i = 0; i < CK; ++i) {

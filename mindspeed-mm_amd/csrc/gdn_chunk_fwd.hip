@@ -390,6 +390,8 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
     float pgl[DEPTH], pg[DEPTH], pb[DEPTH], pgk[DEPTH][2], pbk[DEPTH][2], pbv[DEPTH][CV];
     int pnv[DEPTH];
     constexpr bool PRE = SM::PRE;
+    static_assert(NT % (sizeof(T) == 2 ? 128 : 32) == 0, "a thread's pieces sit at one place of their tiles");
+    const int krow = frag_piece_row<T>(lt & 127);
     auto tm_src = [&](int idc) {   // piece of the three kept tiles -> its place among the four stored ones
       const int t = idc / (1024 / VEC);
       return (t == 0 ? 0 : t + 1) * (1024 / VEC) + idc % (1024 / VEC);
@@ -425,12 +427,12 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
       pb[set] = beta[(tok0 + imin(t, nvalid - 1)) * Hv + h];
       pnv[set] = nvalid;
       if constexpr (PRE) {
-        // In the K tiles every 16-byte piece belongs to one token, 32 (tile & 1) + lane % 32, and this thread's pieces
-        // all have lane % 32 = lt % 32: the gates of two tokens cover them.
+        // In the K tiles every 16-byte piece belongs to one token, 32 (tile & 1) + the row of its place, and this
+        // thread's pieces all sit at the same place of their tiles: the gates of two tokens cover them.
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-          pgk[set][j] = gc[32 * j + (lt & 31)];
-          pbk[set][j] = beta[(tok0 + imin(32 * j + (lt & 31), nvalid - 1)) * Hv + h];
+          pgk[set][j] = gc[32 * j + krow];
+          pbk[set][j] = beta[(tok0 + imin(32 * j + krow, nvalid - 1)) * Hv + h];
         }
       }
     };
@@ -440,7 +442,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
       if constexpr (PRE) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-          f1[j] = (32 * j + (lt & 31) < pnv[set]) ? -pbk[set][j] * __expf(pgk[set][j]) : 0.f;
+          f1[j] = (32 * j + krow < pnv[set]) ? -pbk[set][j] * __expf(pgk[set][j]) : 0.f;
           f2[j] = __expf(pgl[set] - pgk[set][j]);
         }
       }

@@ -329,6 +329,19 @@ __device__ __forceinline__ u32x2 lds_read_tr16(const void* p) {
 // all k-groups of one 32x32 accumulator tile packed as operand fragments ("fragment order").  The same 1024
 // elements, stored as [k-group][lane][16 bytes], are also the on-memory format in which kernels hand tiles to
 // each other: a lane writes/reads 16 contiguous bytes per k-group and never goes through LDS.
+// Place of a lane's 16-byte piece inside a stored tile, in pieces: [k-group][half-wave][32 places].  For 16-bit types
+// the pieces of block (g, h) are rotated by 4 (2 g + h) places, so that the transposing read, which visits the same
+// four rows in all four blocks at once, finds them on different LDS banks (without the rotation they are 512 bytes
+// apart: a four-way conflict); a plain load or store still touches every place of a block exactly once.
+template <typename T> __device__ __forceinline__ int frag_slot(int g, int lane) {
+  if constexpr (sizeof(T) == 2) return g * 64 + (lane & 32) + ((lane + 4 * (2 * g + (lane >> 5))) & 31);
+  else return g * 64 + lane;
+}
+// the tile row (lane % 32 of its owner) of the piece at place p of a stored tile
+template <typename T> __device__ __forceinline__ int frag_piece_row(int p) {
+  if constexpr (sizeof(T) == 2) return ((p & 31) - 4 * ((p >> 5) & 3)) & 31;
+  else return p & 31;
+}
 template <typename T> struct AccB {
   static constexpr int kG = AccK<T>::kGroups;
   static constexpr int kVecElems = 16 / (int)sizeof(T);   // elements per lane per k-group
@@ -367,7 +380,7 @@ template <typename T> struct AccB {
   __device__ __forceinline__ void store(T* tile) const {
     const int lane = threadIdx.x & 63;
 #pragma unroll
-    for (int g = 0; g < kG; ++g) *reinterpret_cast<u32x4*>(tile + (g * 64 + lane) * kVecElems) = f[g];
+    for (int g = 0; g < kG; ++g) *reinterpret_cast<u32x4*>(tile + frag_slot<T>(g, lane) * kVecElems) = f[g];
   }
   // streaming variant for global tiles that are read again only by a later kernel: the data goes to memory without
   // staying in the L2, which is left to the loads (measured gain on the kernels that stream many tiles: 7-10 %)
@@ -375,12 +388,12 @@ template <typename T> struct AccB {
     const int lane = threadIdx.x & 63;
 #pragma unroll
     for (int g = 0; g < kG; ++g)
-      __builtin_nontemporal_store(f[g], reinterpret_cast<u32x4*>(tile + (g * 64 + lane) * kVecElems));
+      __builtin_nontemporal_store(f[g], reinterpret_cast<u32x4*>(tile + frag_slot<T>(g, lane) * kVecElems));
   }
   __device__ __forceinline__ void load(const T* tile) {
     const int lane = threadIdx.x & 63;
 #pragma unroll
-    for (int g = 0; g < kG; ++g) f[g] = *reinterpret_cast<const u32x4*>(tile + (g * 64 + lane) * kVecElems);
+    for (int g = 0; g < kG; ++g) f[g] = *reinterpret_cast<const u32x4*>(tile + frag_slot<T>(g, lane) * kVecElems);
   }
   // The fragments of X^T from a tile in LDS that holds X in fragment order: what load() followed by a turn through
   // the matrix core and pack() gives, without either.  Element (lane a, register index b) of a fragment-order tile
@@ -390,12 +403,15 @@ template <typename T> struct AccB {
     const int lane = threadIdx.x & 63;
     if constexpr (sizeof(T) == 2) {
       const int gr = lane >> 4, i = lane & 15, e = i >> 2, q = i & 3, hh = gr >> 1;
-      const T* base = tile + (((gr & 1) * 64 + 32 * (q & 1) + 4 * hh + e) * 8 + 4 * (q >> 1));
+      // this lane fetches columns 4 (q >> 1) .. + 3 of rows 16 g + 8 t + 4 hh + e of the stored block (gr & 1, q & 1),
+      // which is rotated by 4 (2 (gr & 1) + (q & 1)) places
+      const int rot = 4 * hh + e + 4 * (2 * (gr & 1) + (q & 1));
+      const T* base = tile + (((gr & 1) * 64 + 32 * (q & 1)) * 8 + 4 * (q >> 1));
 #pragma unroll
       for (int g = 0; g < 2; ++g)
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-          const u32x2 r = lds_read_tr16(base + (16 * g + 8 * t) * 8);
+          const u32x2 r = lds_read_tr16(base + ((16 * g + 8 * t + rot) & 31) * 8);
           f[g][2 * t] = r[0];
           f[g][2 * t + 1] = r[1];
         }
