@@ -6,6 +6,8 @@
 A step is one chunked gated-delta-rule forward + backward over the configuration the metric is quoted on
 (BASELINE.json configs[1]: B=2, T=8192, H_qk=16, H_v=32, d_k=d_v=128, bf16, in-kernel q/k L2 norm, N(0,0.02)
 initial state, upstream grad ~ N(0,1)); inputs are synthetic and already resident in HBM.  Prints ONE JSON line.
+The step keeps the forward pass's workspace for the backward pass (skip_recompute=True); the operator's default,
+which keeps nothing and recomputes, is timed beside it under aux.
 
   value        tokens/s of fwd+bwd (B*T / step time), measured without per-kernel instrumentation
   roofline     the kernel with the largest share of the step: its algorithmic HBM bytes per launch divided by its
@@ -14,8 +16,12 @@ initial state, upstream grad ~ N(0,1)); inputs are synthetic and already residen
                bf16 MFMA peak (2.5 PFLOP/s) is given beside it
   cpu_baseline the CPU oracle (PyTorch fp32 restatement of the reference's torch path, autograd backward) timed on
                this box's host cores on a bounded sample of the same workload
-  aux          the whole path against the MFMA peak with the reference's FLOP formula, the per-kernel split,
-               and the HBM-bound siblings (batch-256 decode, the packed conv1d, the gated RMSNorm) with their achieved GB/s
+               roofline.path gives the whole step against the two machine peaks: the reference's FLOP formula
+               against the bf16 MFMA peak, and the minimal HBM bytes of the operator (inputs and outputs only)
+               against the HBM peak, with the traffic the kernels really move beside it
+  aux          the per-kernel split, the other BASELINE configurations (packed sequences, the long-context shape,
+               the CPU-runnable case) and the HBM-bound siblings (batch-256 decode, the packed conv1d, the gated
+               RMSNorm) with their achieved GB/s
 """
 import argparse
 import json
@@ -35,10 +41,11 @@ CFG = dict(B=2, T=8192, Hqk=16, Hv=32, K=128, V=128, C=64)
 
 # HBM bytes per launch of each kernel on CFG, read + written, from the hardware counters FETCH_SIZE and WRITE_SIZE
 # (rocprofv3 --pmc, one run per counter, each scaled by what the same counter reads for a 512 MiB copy): the figures
-# of profiles/chunk_fwd_bwd_B2_T8192_bf16_hbm_traffic.md.  Measured offline, reported beside the live timings.
+# of the file named below.  Measured offline on the kernels as they are in this tree, reported beside the live timings.
+TRAFFIC_SOURCE = "profiles/chunk_fwd_bwd_B2_T8192_bf16_hbm_traffic.md"
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "chunk_prep_kernel": 1042433488, "chunk_state_kernel": 749425775, "chunk_out_kernel": 682825408,
-    "chunk_state_bwd_kernel": 884322958, "chunk_bwd_local_kernel": 1156464169,
+    "chunk_prep_kernel": None, "chunk_state_kernel": None,
+    "chunk_state_bwd_kernel": None, "chunk_bwd_local_kernel": None,
 }
 
 
@@ -47,14 +54,24 @@ def ref_formula_flops(tokens, Hv, K, V, C=64):
     return 3 * 2 * tokens * Hv * (3 * V * C + 2 * K * C + 3 * K * V)
 
 
+def minimal_bytes(B, T, N, Hqk, Hv, K, V, e=2):
+    """HBM bytes the operator cannot avoid, fwd+bwd: every input read once and every output written once per pass
+    (q, k, v, o and their gradients in `e` bytes, g, beta and the states in fp32), grouped q/k heads read natively."""
+    tok = B * T
+    fwd = tok * (e * (2 * Hqk * K + 2 * Hv * V) + 8 * Hv) + 2 * 4 * N * Hv * K * V
+    bwd = tok * (e * (4 * Hqk * K + 3 * Hv * V) + 16 * Hv) + 2 * 4 * N * Hv * K * V
+    return fwd + bwd
+
+
 def kernel_matmul_flops(K, V, C=64):
     """Matmul FLOP each kernel performs per (chunk, value head): 2*M*N*K summed over its contractions."""
     g = lambda m, n, k: 2 * m * n * k
     return {
-        "chunk_prep_kernel": 2 * g(C, C, K) + g(C, K, C) + g(C, V, C),     # K K^T, Q K^T, Tm (b e^G K), Tm (b V)
-        "chunk_state_kernel": g(C, V, K) + g(K, V, C),                     # W S, (decayed K)^T V'
-        "chunk_out_kernel": g(C, V, K) + g(C, V, C),                       # Q S, Aq V'
-        "chunk_state_bwd_kernel": g(C, V, C) + g(C, V, K) + 2 * g(K, V, C),   # Aq^T dO, K dS, Q^T dO, W^T dV'
+        "chunk_prep_kernel": 2 * g(C, C, K),                               # K K^T, Q K^T (the solve is not counted)
+        # K S, Tm z, (decayed K)^T V', Q S, Aq V'
+        "chunk_state_kernel": g(C, V, K) + g(C, V, C) + g(K, V, C) + g(C, V, K) + g(C, V, C),
+        # Aq^T dO, K dS, Tm^T dV', Q^T dO, K^T R
+        "chunk_state_bwd_kernel": g(C, V, C) + g(C, V, K) + g(C, V, C) + 2 * g(K, V, C),
         # dO V'^T, dO S^T, V' dS^T, dV' S^T, ds K, ds^T Q | Tm^T dW, dW K^T, Tm^T dV', dV' V^T, dTm Tm^T, Tm^T X, dM K, dM^T K
         "chunk_bwd_local_kernel": g(C, C, V) + 3 * g(C, K, V) + 2 * g(C, K, C)
                                   + g(C, K, C) + g(C, C, K) + g(C, V, C) + g(C, C, V) + 2 * g(C, C, C) + 2 * g(C, K, C),
@@ -64,15 +81,16 @@ def kernel_matmul_flops(K, V, C=64):
 def kernel_algorithmic_bytes(K, V, grp, e=2, C=64):
     """HBM bytes each kernel has to move per (chunk, value head) given its interface: every input tile read once, every
     output tile written once (bf16 tiles, fp32 row vectors).  tk = [64,K] tile, tv = [64,V] tile, st = [K,V] state,
-    cc = [64,64] tile, row = 64 fp32 values."""
+    cc = [64,64] tile (three of its four 32x32 tiles where it is triangular), row = 64 fp32 values."""
     tk, tv, st, cc, row = C * K * e, C * V * e, K * V * e, C * C * e, C * 4
+    tri = 3 * cc // 4
     return {
-        # v, g, beta -> G, Tm, Aq, -W, U, -W^T tiles; once per q/k group: q, k -> K^T, K, Q^T tiles, 1/|q|, 1/|k|
-        "chunk_prep_kernel": tv + 2 * row + row + 2 * cc + tk + tv + tk + (2 * tk + 3 * tk + 2 * row) // grp,
-        "chunk_state_kernel": tk + tk // grp + tv + row + tv + st,   # -W, K^T (per group), U, G -> v_new, state before the chunk
-        "chunk_out_kernel": (tk + row) // grp + cc + tv + st + row + tv,   # q, 1/|q| (per group), Aq, v_new, state, G -> o
-        # K, Q^T (per group), -W^T, Aq, dO, G -> dv_new, dS
-        "chunk_state_bwd_kernel": 2 * tk // grp + tk + cc + tv + row + tv + st,
+        # g, beta -> G, Tm, Aq; once per q/k group: q, k -> K, Q^T tiles, 1/|q|, 1/|k|
+        "chunk_prep_kernel": 2 * row + row + 2 * cc + (2 * tk + 2 * tk + 2 * row) // grp,
+        # K, Q^T (per group), Tm, Aq, v, G, beta -> o, v_new, state before the chunk
+        "chunk_state_kernel": 2 * tk // grp + 2 * tri + tv + 2 * row + tv + tv + st,
+        # K, Q^T (per group), Tm, Aq, dO, G, beta -> dv_new, dS
+        "chunk_state_bwd_kernel": 2 * tk // grp + 2 * tri + tv + 2 * row + tv + st,
         # v_new, dv_new, dO, S, dS, v, K, q, Tm, row vectors -> dv, dg, dbeta, dq/dk (written by the first head of a
         # group, read and re-written by the others)
         "chunk_bwd_local_kernel": 3 * tv + 2 * st + tv + 2 * tk + cc + 5 * row + tv + 2 * row
@@ -113,9 +131,10 @@ def main():
     d = {n: t.to(dev) for n, t in x.items()}
     leaves = [d[n].requires_grad_(True) for n in ("q", "k", "v", "g", "beta", "h0")]
 
-    def step():
+    def step(skip_recompute=True):
         o, ht = ops.chunk_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], initial_state=d["h0"],
-                                           output_final_state=True, use_qk_l2norm_in_kernel=True)
+                                           output_final_state=True, use_qk_l2norm_in_kernel=True,
+                                           skip_recompute=skip_recompute)
         return torch.autograd.grad([o], leaves, [d["do"]])
 
     for _ in range(args.warmup):
@@ -171,14 +190,35 @@ def main():
     bytes_per_launch = abytes[dom] * nchunk_heads / launches
     dom_gbps = bytes_per_launch / (per_kernel[dom]["avg_ms"] * 1e-3) / 1e9
     dom_tflops = flops[dom] * nchunk_heads / (per_kernel[dom]["step_ms"] * 1e-3) / 1e12
+    path_tflops = ref_formula_flops(tokens, c["Hv"], c["K"], c["V"]) / (ms_per_step * 1e-3) / 1e12
+    min_bytes = minimal_bytes(c["B"], c["T"], c["B"], c["Hqk"], c["Hv"], c["K"], c["V"])
+    interface_total = sum(abytes[n] * nchunk_heads for n in per_kernel if n in abytes)
+    measured = [MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(n) for n in per_kernel if n in abytes]
+    traffic_total = None
+    if all(m is not None for m in measured):
+        traffic_total = sum(MEASURED_TRAFFIC_BYTES_PER_LAUNCH[n] * per_kernel[n]["launches_per_step"]
+                            for n in per_kernel if n in abytes)
+    # the whole step against both roofs: the operator's minimal bytes (inputs and outputs only) and the reference's
+    # FLOP count say what an ideal implementation would need; the kernels' own interfaces move more (intermediates
+    # between the launches), which is what the per-kernel figures above are measured against
+    path = {"ms_per_step": round(ms_per_step, 4),
+            "minimal_bytes_per_step": int(min_bytes),
+            "frac_hbm_minimal": round(min_bytes / (ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+            "flops_ref_formula_per_step": ref_formula_flops(tokens, c["Hv"], c["K"], c["V"]),
+            "tflops_ref_formula": round(path_tflops, 2),
+            "frac_mfma_ref_formula": round(path_tflops / PEAK_BF16_TFLOPS, 4),
+            "kernel_interface_bytes_per_step": int(interface_total),
+            "interface_over_minimal": round(interface_total / min_bytes, 2),
+            "traffic_per_step_total": None if traffic_total is None else int(traffic_total),
+            "traffic_over_minimal": None if traffic_total is None else round(traffic_total / min_bytes, 2)}
     roofline = {"kernel": dom, "bound": "hbm", "achieved": round(dom_gbps, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                 "frac": round(dom_gbps / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(dom),
+                "traffic_source": TRAFFIC_SOURCE + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, collected offline)",
                 "algorithmic_bytes_per_launch": int(bytes_per_launch), "launches_per_step": launches,
                 "avg_launch_ms": per_kernel[dom]["avg_ms"],
                 "flop_per_byte": round(flops[dom] / abytes[dom], 1), "tflops": round(dom_tflops, 1),
-                "frac_of_bf16_mfma_peak": round(dom_tflops / PEAK_BF16_TFLOPS, 4)}
+                "frac_of_bf16_mfma_peak": round(dom_tflops / PEAK_BF16_TFLOPS, 4), "path": path}
 
-    path_tflops = ref_formula_flops(tokens, c["Hv"], c["K"], c["V"]) / (ms_per_step * 1e-3) / 1e12
     aux = {"path_tflops_ref_formula": round(path_tflops, 2),
            "path_frac_of_bf16_mfma_peak": round(path_tflops / PEAK_BF16_TFLOPS, 4),
            "kernel_ms_sum": round(total_kernel_ms, 3), "step_time_spread": spread, "kernels": per_kernel}
@@ -333,6 +373,11 @@ def main():
                                            output_final_state=True, use_qk_l2norm_in_kernel=True)
         pf = wall_ms(prefill_step, 20)
         aux["forward_only"] = {"ms": round(pf, 4), "tokens_per_s": round(tokens / (pf * 1e-3), 1)}
+        rc = wall_ms(lambda: step(False), 20)
+        aux["default_mode_recompute_in_backward"] = {
+            "ms_per_step": round(rc, 4), "tokens_per_s": round(tokens / (rc * 1e-3), 1),
+            "note": "skip_recompute=False: only the inputs are kept between the passes, the backward pass refills a "
+                    "workspace (chunk-local kernel and recurrence) first"}
         zg = torch.randn(c["B"], c["T"], c["Hv"], c["V"], generator=gen).to(dev, torch.bfloat16)
         nw = torch.ones(c["V"], device=dev, dtype=torch.bfloat16)
 
@@ -340,7 +385,7 @@ def main():
             with torch.no_grad():
                 ops.chunk_gated_delta_rule_norm(d["q"], d["k"], d["v"], d["g"], d["beta"], zg, nw,
                                                 initial_state=d["h0"], output_final_state=True,
-                                                use_qk_l2norm_in_kernel=True)
+                                                use_qk_l2norm_in_kernel=True, in_output_kernel=True)
 
         def prefill_norm_separate():
             with torch.no_grad():
@@ -386,6 +431,48 @@ def main():
                         "fused_fwd_bwd_kernel_ms": round(kernel_sum_ms(gates_step, 20), 4),
                         "torch_elementwise_fwd_bwd_ms": round(wall_ms(gates_eager_step, 100), 4)}
 
+    if not args.no_aux:
+        # ---- the other BASELINE configurations (parity-tested at full size in tests/test_gpu_full_size.py) ----
+        def fwd_bwd_ms(dd, cu=None, n=5, warm=2, skip=True):
+            L = [dd[m].requires_grad_(True) for m in ("q", "k", "v", "g", "beta", "h0")]
+
+            def f():
+                o_, _ = ops.chunk_gated_delta_rule(dd["q"], dd["k"], dd["v"], dd["g"], dd["beta"], initial_state=dd["h0"],
+                                                   output_final_state=True, use_qk_l2norm_in_kernel=True, cu_seqlens=cu,
+                                                   skip_recompute=skip)
+                torch.autograd.grad([o_], L, [dd["do"]])
+            for _ in range(warm):
+                f()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n):
+                f()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / n * 1e3
+        del d, leaves
+        torch.cuda.empty_cache()
+        cu2 = packed_lengths()
+        x2 = gdn_inputs(1, cu2[-1], c["Hqk"], c["Hv"], c["K"], c["V"], torch.bfloat16, seed=2, N=len(cu2) - 1)
+        d2 = {n: t.to(dev) for n, t in x2.items()}
+        ms2 = fwd_bwd_ms(d2, torch.tensor(cu2, dtype=torch.int64, device=dev))
+        fl2 = ref_formula_flops(cu2[-1], c["Hv"], c["K"], c["V"])
+        aux["config2_packed_24_sequences_32768_tokens"] = {
+            "ms_per_step": round(ms2, 4), "tokens_per_s": round(cu2[-1] / (ms2 * 1e-3), 1),
+            "frac_mfma_ref_formula": round(fl2 / (ms2 * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}
+        del d2, x2
+        torch.cuda.empty_cache()
+        T4, Hv4, V4 = 65536, 64, 256
+        x4 = gdn_inputs(1, T4, c["Hqk"], Hv4, c["K"], V4, torch.bfloat16, seed=4, a_log=(0.5, 2.0), dt_bias=(-6.0, -4.0))
+        d4 = {n: t.to(dev) for n, t in x4.items()}
+        del x4
+        ms4 = fwd_bwd_ms(d4, n=3, warm=1)
+        fl4 = 3 * 2 * T4 * Hv4 * (3 * V4 * 64 + 2 * c["K"] * 64 + 3 * c["K"] * V4)
+        aux["config4_T65536_Hv64_dv256"] = {
+            "ms_per_step": round(ms4, 3), "tokens_per_s": round(T4 / (ms4 * 1e-3), 1),
+            "frac_mfma_ref_formula": round(fl4 / (ms4 * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}
+        del d4
+        torch.cuda.empty_cache()
+
     if args.calibrate_copy:
         src = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
@@ -397,6 +484,14 @@ def main():
     cpu = None
     if not args.no_cpu_baseline:
         from oracle import gdn_oracle as O
+        # BASELINE configs[0], the reference's own CPU-runnable case: forward only, fp32, B=1 T=512 H=4 d=64
+        x0 = gdn_inputs(1, 512, 4, 4, 64, 64, torch.float32, seed=0, l2norm_in_kernel=False)
+        t0 = time.perf_counter()
+        for _ in range(3):
+            O.chunk_gated_delta_rule_ref(x0["q"], x0["k"], x0["v"], x0["g"], x0["beta"], output_final_state=True)
+        dt0 = (time.perf_counter() - t0) / 3
+        aux["config0_cpu_forward_fp32"] = {"ms": round(dt0 * 1e3, 2), "tokens_per_s": round(512 / dt0, 1),
+                                           "cores": torch.get_num_threads()}
         Ts = 8192
         sample = {n: x[n][:1, :Ts] for n in ("q", "k", "v", "g", "beta", "do")}
         L = {n: sample[n].float().requires_grad_(True) for n in ("q", "k", "v", "g", "beta")}
@@ -416,7 +511,8 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "GDN chunk forward+backward, B=2 T=8192 H_qk=16 H_v=32 d_k=d_v=128 chunk=64, "
-                               "use_qk_l2norm_in_kernel, initial state N(0,0.02), native grouped q/k heads",
+                               "use_qk_l2norm_in_kernel, initial state N(0,0.02), native grouped q/k heads, "
+                               "skip_recompute=True (forward workspace kept for the backward pass)",
                    "global_batch": c["B"], "seq_len": c["T"], "parallelism": "single GPU"},
         "roofline": roofline, "cpu_baseline": cpu, "aux": aux,
     }

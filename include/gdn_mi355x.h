@@ -9,7 +9,8 @@
  *   - every pointer is device memory, tensors are dense (contiguous) in the stated layout unless an entry
  *     point takes strides;
  *   - dtype: 0 = fp32, 1 = bf16 (conv1d also 2 = fp16) and applies to q/k/v/o and their gradients;
- *     g, beta, states and their gradients are always fp32;
+ *     g, states and their gradients are always fp32; beta and its gradient are fp32 unless an entry point takes
+ *     beta_dtype (0 = fp32, or equal to dtype: the layer's beta = sigmoid(b) is bf16, modeling_qwen3_5.py:833);
  *   - `stream` is a hipStream_t; launches are asynchronous, nothing allocates or synchronises;
  *   - return 0 on success, <0 for an invalid argument (-1 null pointer, -2 bad shape, -3 unsupported
  *     size, -4 bad dtype, -5 workspace too small, -6 bad stride or a pointer not 16-byte aligned), >0 is a
@@ -29,9 +30,12 @@ extern "C" {
  * replaces chunk_gated_delta_rule_fwd / _bwd, mindspeed_mm/fsdp/ops/gdn/chunk_gated_delta_rule.py:30-174
  * (semantics of torch_chunk_gated_delta_rule, modeling_qwen3_5.py:398-475). K in {64,128}, V % 64 == 0.
  *
- * The workspace keeps what the backward pass needs (cumulative decay, WY factors, per-chunk states);
- * gdn_chunk_bwd must be given the workspace its forward call filled, unchanged, and that workspace
- * must have been sized with with_backward = 1.  The workspace must be 256-byte aligned.
+ * The workspace keeps what the backward pass needs (cumulative decay, Tm, per-chunk states, v_new);
+ * gdn_chunk_bwd must be given a workspace a forward call on the same inputs filled, unchanged, sized with
+ * with_backward = 1.  The workspace must be 256-byte aligned.  A forward call with o = NULL (and such a workspace)
+ * only fills the workspace and writes no output: it is the recomputation step of a backward pass whose forward pass
+ * kept nothing (chunk_gated_delta_rule.py:102-119 recomputes w, u, h, v_new the same way).  A forward call with a
+ * workspace sized with with_backward = 0 writes neither per-chunk states nor v_new to memory.
  */
 int64_t gdn_chunk_workspace_bytes(int B, int T, int N, int Hqk, int Hv, int K, int V, int dtype, int with_backward);
 
@@ -53,10 +57,10 @@ int gdn_chunk_bwd(const void* q, const void* k, const void* v, const float* g, c
  * The reference's Triton entry makes such views contiguous first (input_guard, triton/utils.py:210-239); reading
  * and writing them in place saves those copies and the concatenation of dq, dk, dv in the backward pass. */
 int gdn_chunk_fwd_strided(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
-                          int64_t v_stride, const float* g, const float* beta, const float* initial_state,
+                          int64_t v_stride, const float* g, const void* beta, const float* initial_state,
                           const int64_t* cu_seqlens, void* o, float* final_state, void* workspace,
                           int64_t workspace_bytes, int B, int T, int N, int Hqk, int Hv, int K, int V, float scale,
-                          int use_qk_l2norm, int dtype, void* stream);
+                          int use_qk_l2norm, int dtype, int beta_dtype, void* stream);
 
 /* gdn_chunk_fwd_strided followed, inside its output kernel, by the layer's gated RMSNorm over head_v_dim
  * (Qwen3_5RMSNormGated.forward, modeling_qwen3_5.py:330-349, applied to the rule's output at :897-900):
@@ -65,18 +69,19 @@ int gdn_chunk_fwd_strided(const void* q, const void* k, const void* v, int64_t q
  * output) and rstd [tokens * Hv] fp32 are written only if non-null: a caller without a backward pass saves one write
  * and one read of o.  V must be 64 or 128 (a workgroup of the output kernel then holds whole rows), else -3. */
 int gdn_chunk_fwd_norm_strided(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
-                               int64_t v_stride, const float* g, const float* beta, const float* initial_state,
+                               int64_t v_stride, const float* g, const void* beta, const float* initial_state,
                                const int64_t* cu_seqlens, const void* gate, const void* norm_weight, void* o, void* y,
                                float* rstd, float* final_state, void* workspace, int64_t workspace_bytes, int B,
                                int T, int N, int Hqk, int Hv, int K, int V, float scale, float eps,
-                               int use_qk_l2norm, int dtype, int weight_dtype, void* stream);
+                               int use_qk_l2norm, int dtype, int weight_dtype, int beta_dtype, void* stream);
 
 int gdn_chunk_bwd_strided(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
-                          int64_t v_stride, const float* g, const float* beta, const float* initial_state,
+                          int64_t v_stride, const float* g, const void* beta, const float* initial_state,
                           const int64_t* cu_seqlens, const void* d_o, const float* d_final_state, void* dq, void* dk,
-                          void* dv, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride, float* dg, float* dbeta,
+                          void* dv, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride, float* dg, void* dbeta,
                           float* d_initial_state, void* workspace, int64_t workspace_bytes, int B, int T, int N,
-                          int Hqk, int Hv, int K, int V, float scale, int use_qk_l2norm, int dtype, void* stream);
+                          int Hqk, int Hv, int K, int V, float scale, int use_qk_l2norm, int dtype, int beta_dtype,
+                          void* stream);
 
 /* -------- fused recurrent gated delta rule (decode) ------------------------------------------
  * replaces the `recurrent_gated_delta_rule` slot (third-party fla kernel or

@@ -52,7 +52,8 @@ template <int PIECES, int NT> struct DealB { static constexpr int kPer = (PIECES
 template <typename T, int DK, int NW, int NL, int STAGES>
 __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 && NL >= 4) ? 2 : 1) void chunk_state_bwd_kernel(
     const T* __restrict__ kaf, const T* __restrict__ qtf, const T* __restrict__ ai, const T* __restrict__ aqf,
-    const T* __restrict__ dO, const float* __restrict__ G, const float* __restrict__ beta, const float* __restrict__ dht,
+    const T* __restrict__ dO, const float* __restrict__ G, const void* __restrict__ beta, int beta_same,
+    const float* __restrict__ dht,
     float* __restrict__ dh0, T* __restrict__ dvf, T* __restrict__ dhf, const int64_t* __restrict__ cu,
     const int* __restrict__ chunk_offsets, int T_len, int Hqk, int Hv, int V, float scale) {
   using SM = StateBwdSmem<T, DK, NW, STAGES>;
@@ -74,7 +75,8 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
     const int lt = tid - 64 * NW;
     constexpr int DEPTH = (STAGES == 2) ? 2 : 1;
     Vec16<T> pk[DEPTH][CK], pq[DEPTH][CK], ptm[DEPTH][CTM], pa[DEPTH][CTM], pd[DEPTH][CD];
-    float pgl[DEPTH], pgk[DEPTH][2], pbk[DEPTH][2], pgd[DEPTH][CD];
+    float pgl[DEPTH], pgk[DEPTH][2], pgd[DEPTH][CD];
+    uint32_t pbk[DEPTH][2];   // beta as fetched
     int pnv[DEPTH];
     static_assert(NT % (sizeof(T) == 2 ? 128 : 32) == 0, "a thread's pieces sit at one place of their tiles");
     const int krow = frag_piece_row<T>(lt & 127);
@@ -113,7 +115,7 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         pgk[set][j] = gc[32 * j + krow];
-        pbk[set][j] = beta[(tok0 + imin(32 * j + krow, nvalid - 1)) * Hv + h];
+        pbk[set][j] = gate_raw<T>(beta, beta_same, (tok0 + imin(32 * j + krow, nvalid - 1)) * Hv + h);
       }
       pnv[set] = nvalid;
     };
@@ -123,7 +125,7 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         f1[j] = __expf(pgl[set] - pgk[set][j]);
-        f2[j] = (32 * j + krow < pnv[set]) ? -pbk[set][j] * __expf(pgk[set][j]) : 0.f;
+        f2[j] = (32 * j + krow < pnv[set]) ? -gate_val<T>(pbk[set][j], beta_same) * __expf(pgk[set][j]) : 0.f;
       }
 #pragma unroll
       for (int i = 0; i < CK; ++i) {
@@ -321,10 +323,10 @@ template <typename T, int DK> struct BwdLocalSmem {
 
 template <typename T, int DK>
 __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_local_kernel(
-    const T* __restrict__ qtf, const T* __restrict__ kaf, const T* __restrict__ v, const float* __restrict__ beta,
+    const T* __restrict__ qtf, const T* __restrict__ kaf, const T* __restrict__ v, const void* __restrict__ beta, int beta_same,
     const float* __restrict__ G, const T* __restrict__ Ai, const T* __restrict__ vf, const T* __restrict__ dvf,
     const T* __restrict__ dO, const T* __restrict__ hf, const T* __restrict__ dhf, const float* __restrict__ rstd_q,
-    const float* __restrict__ rstd_k, T* dq, T* dk, T* __restrict__ dv_out, float* __restrict__ dbeta,
+    const float* __restrict__ rstd_k, T* dq, T* dk, T* __restrict__ dv_out, void* __restrict__ dbeta,
     float* __restrict__ dg, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N,
     int Hqk, int Hv, int V, float scale, int hh, TokenStrides ts) {
   using SM = BwdLocalSmem<T, DK>;
@@ -413,7 +415,8 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
 
   if (tid < 64) {   // the row vectors: all requests first, the same ones on every path
     const int tc = imin(tid, nvalid - 1);
-    const float gv = G[ch * 64 + tc], bv = beta[(tok0 + tc) * Hv + h];
+    const float gv = G[ch * 64 + tc];
+    const uint32_t braw = gate_raw<T>(beta, beta_same, (tok0 + tc) * Hv + h);
     float rq1 = 1.f, rk1v = 1.f;
     if (l2) {
       rq1 = rstd_q[((int64_t)blockIdx.x * Hqk + hq) * 64 + tc];
@@ -421,7 +424,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     }
     Gs[tid] = gv;
     egs[tid] = __expf(gv);
-    bs[tid] = tid < nvalid ? bv : 0.f;
+    bs[tid] = tid < nvalid ? gate_val<T>(braw, beta_same) : 0.f;
     rsq[tid] = rq1;
     rsk[tid] = rk1v;
   }
@@ -743,7 +746,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     }
     if (lane < nvalid) {
       dg[(tok0 + lane) * Hv + h] = x;
-      dbeta[(tok0 + lane) * Hv + h] = sbk + slots(rv);
+      gate_st<T>(dbeta, beta_same, (tok0 + lane) * Hv + h, sbk + slots(rv));
     }
   }
 }
@@ -756,8 +759,8 @@ template <typename K> static int set_lds_b(K kernel, int bytes) {
 
 template <typename T, int DK, int NW, int NWS, int NLS, int STAGES>
 static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const void* q, const void* k, const void* v,
-                            const float* beta, const int64_t* cu, const void* dO, const float* dht, void* dq, void* dk,
-                            void* dv, float* dg, float* dbeta, float* dh0, unsigned char* ws, float scale, int l2norm,
+                            const void* beta, int beta_same, const int64_t* cu, const void* dO, const float* dht, void* dq,
+                            void* dk, void* dv, float* dg, void* dbeta, float* dh0, unsigned char* ws, float scale, int l2norm,
                             hipStream_t st) {
   const int nc = (int)d.max_chunks();
   const int* chunk_offsets = reinterpret_cast<const int*>(ws + L.chunk_offsets);
@@ -778,7 +781,7 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     constexpr int smem = StateBwdSmem<T, DK, NWS, STAGES>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
     GDN_LAUNCH(kKernStateBwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NWS)), dim3(64 * (NWS + NLS)), smem, st, (const T*)KAF,
-               (const T*)QTF, Ai, AQ, (const T*)dO, G, beta, dht, dh0, DVF, DHF, cu, chunk_offsets, d.T, d.Hqk, d.Hv, d.V,
+               (const T*)QTF, Ai, AQ, (const T*)dO, G, beta, beta_same, dht, dh0, DVF, DHF, cu, chunk_offsets, d.T, d.Hqk, d.Hv, d.V,
                scale);
   }
   {
@@ -787,7 +790,7 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     if (int e = set_lds_b(kern, smem)) return e;
     for (int hh = 0; hh < d.Hv / d.Hqk; ++hh)
       GDN_LAUNCH(kKernBwdLocal, st, kern, dim3(nc, d.Hqk), dim3(kThreads), smem, st, QTF, (const T*)KAF, (const T*)v,
-                 beta, G, Ai, VF, (const T*)DVF, (const T*)dO, HF, (const T*)DHF, rstd_q, rstd_k, (T*)dq, (T*)dk,
+                 beta, beta_same, G, Ai, VF, (const T*)DVF, (const T*)dO, HF, (const T*)DHF, rstd_q, rstd_k, (T*)dq, (T*)dk,
                  (T*)dv, dbeta, dg, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale, hh, d.strides());
   }
   return (int)hipGetLastError();
@@ -796,18 +799,20 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
 }  // namespace gdn
 
 extern "C" int gdn_chunk_bwd_strided(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
-                                     int64_t v_stride, const float* g, const float* beta, const float* initial_state,
+                                     int64_t v_stride, const float* g, const void* beta, const float* initial_state,
                                      const int64_t* cu_seqlens, const void* d_o, const float* d_final_state, void* dq,
                                      void* dk, void* dv, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride,
-                                     float* dg, float* dbeta, float* d_initial_state, void* workspace,
+                                     float* dg, void* dbeta, float* d_initial_state, void* workspace,
                                      int64_t workspace_bytes, int B, int T, int N, int Hqk, int Hv, int K, int V,
-                                     float scale, int use_qk_l2norm, int dtype, void* stream) {
+                                     float scale, int use_qk_l2norm, int dtype, int beta_dtype, void* stream) {
   using namespace gdn;
   (void)g; (void)initial_state;   // their effect is already in the workspace (G, per-chunk states)
   if (!q || !k || !v || !beta || !d_o || !dq || !dk || !dv || !dg || !dbeta || !workspace) return -1;
   ChunkDims d{B, T, N, Hqk, Hv, K, V, cu_seqlens != nullptr};
   d.ts = {q_stride, k_stride, v_stride, dq_stride, dk_stride, dv_stride};
   if (int e = chunk_check_dims(d, dtype)) return e;
+  if (beta_dtype != 0 && beta_dtype != dtype) return -4;
+  const int beta_same = beta_dtype != 0;
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)d_o | (uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv) & 15) return -6;
   ChunkDims dl = d;
   dl.varlen = true;
@@ -817,7 +822,7 @@ extern "C" int gdn_chunk_bwd_strided(const void* q, const void* k, const void* v
   unsigned char* ws = static_cast<unsigned char*>(workspace);
   hipStream_t st = (hipStream_t)stream;
 #define GDN_BWD(T_, DK_, NW_, NWS_, NLS_, ST_)                                                       \
-  return chunk_bwd_launch<T_, DK_, NW_, NWS_, NLS_, ST_>(d, L, q, k, v, beta, cu_seqlens, d_o, d_final_state, dq, \
+  return chunk_bwd_launch<T_, DK_, NW_, NWS_, NLS_, ST_>(d, L, q, k, v, beta, beta_same, cu_seqlens, d_o, d_final_state, dq, \
                                                           dk, dv, dg, dbeta, d_initial_state, ws, scale,         \
                                                           use_qk_l2norm, st)
   const bool wide = (V % 128 == 0);
@@ -842,5 +847,5 @@ extern "C" int gdn_chunk_bwd(const void* q, const void* k, const void* v, const 
                              int Hqk, int Hv, int K, int V, float scale, int use_qk_l2norm, int dtype, void* stream) {
   return gdn_chunk_bwd_strided(q, k, v, 0, 0, 0, g, beta, initial_state, cu_seqlens, d_o, d_final_state, dq, dk, dv, 0, 0,
                                0, dg, dbeta, d_initial_state, workspace, workspace_bytes, B, T, N, Hqk, Hv, K, V, scale,
-                               use_qk_l2norm, dtype, stream);
+                               use_qk_l2norm, dtype, 0, stream);
 }

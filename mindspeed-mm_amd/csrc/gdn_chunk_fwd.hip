@@ -122,8 +122,8 @@ template <typename T, int DK> struct PrepSmem {
 
 template <typename T, int DK>
 __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3) void chunk_prep_kernel(
-    const T* __restrict__ q, const T* __restrict__ k, const float* __restrict__ g, const float* __restrict__ beta,
-    const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, float* __restrict__ G_out,
+    const T* __restrict__ q, const T* __restrict__ k, const float* __restrict__ g, const void* __restrict__ beta,
+    int beta_same, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, float* __restrict__ G_out,
     T* __restrict__ Ai_out, T* __restrict__ Aq_out, T* __restrict__ KA_out, T* __restrict__ QT_out,
     float* __restrict__ rstd_q_out, float* __restrict__ rstd_k_out, int T_len, int N, int Hqk, int Hv, float scale,
     int l2norm, TokenStrides ts) {
@@ -149,7 +149,7 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
   tile_qk_request<T, DK>(qt, q + tok0 * ts.q + hq * DK, ts.q, nvalid, tid);
   if (wave == 0) {
     float x = lane < nvalid ? g[(tok0 + lane) * Hv + h] : 0.f;
-    const float b = lane < nvalid ? beta[(tok0 + lane) * Hv + h] : 0.f;
+    const float b = lane < nvalid ? gate_val<T>(gate_raw<T>(beta, beta_same, (tok0 + lane) * Hv + h), beta_same) : 0.f;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
       const float t = __shfl_up(x, d);
@@ -317,7 +317,8 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
 // neither S nor V' has to be re-read from memory; both are still stored when a backward pass will need them.
 // ---------------------------------------------------------------------------------------------
 // PRE: two images of K, rows scaled by -beta e^G and by e^{G_last-G} on their way into LDS.  Whether they fit is
-// decided for the variant with output waves (FUSE), and the variant without them follows, so that both round alike.
+// decided for the variant with output waves (FUSE) and two slabs per workgroup, and every other variant of the same
+// element type and key width follows, so that all of them round alike.
 template <typename T, int DK, int NW, int STAGES, bool FUSE> struct StatePre {
   static constexpr int x_elems = 2 * DK * 32 + 2 * 2048 + Patch<T>::kElems;
   static constexpr bool value = STAGES * ((2 * 64 * DK + 3 * 1024 + 64 * 32 * NW + (FUSE ? 64 * DK + 3 * 1024 : 0)) * (int)sizeof(T) + 68 * 4) +
@@ -349,7 +350,7 @@ template <typename T, int DK, int NW, int NL, int STAGES, bool OUT, bool PRE_>
 __global__ __launch_bounds__(64 * (NW + (OUT ? NW : 0) + NL)) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 2 : 1)
 void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, const T* __restrict__ ai,
                         const T* __restrict__ aqf, const T* __restrict__ v, const float* __restrict__ G,
-                        const float* __restrict__ beta, const float* __restrict__ h0, float* __restrict__ ht,
+                        const void* __restrict__ beta, int beta_same, const float* __restrict__ h0, float* __restrict__ ht,
                         T* __restrict__ vf, T* __restrict__ hf, T* __restrict__ o, const int64_t* __restrict__ cu,
                         const int* __restrict__ chunk_offsets, int T_len, int Hqk, int Hv, int V, float scale,
                         int64_t v_stride) {
@@ -387,7 +388,8 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
     // one that copies it to LDS (j - 1), so global loads have DEPTH chunk periods to arrive
     constexpr int DEPTH = (STAGES == 2) ? 2 : 1;
     Vec16<T> pk[DEPTH][CK], ptm[DEPTH][CTM], pv[DEPTH][CV], pq[DEPTH][OUT ? CK : 1], pa[DEPTH][OUT ? CTM : 1];
-    float pgl[DEPTH], pg[DEPTH], pb[DEPTH], pgk[DEPTH][2], pbk[DEPTH][2], pbv[DEPTH][CV];
+    float pgl[DEPTH], pg[DEPTH], pgk[DEPTH][2];
+    uint32_t pb[DEPTH], pbk[DEPTH][2], pbv[DEPTH][CV];   // beta as fetched
     int pnv[DEPTH];
     constexpr bool PRE = SM::PRE;
     static_assert(NT % (sizeof(T) == 2 ? 128 : 32) == 0, "a thread's pieces sit at one place of their tiles");
@@ -416,7 +418,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
       for (int i = 0; i < CV; ++i) {   // rows past the end of the sequence repeat the last one (their beta is 0)
         const int idc = imin(lt + i * NT, PV - 1), row = imin(idc / VPR, nvalid - 1), cc = idc % VPR;
         pv[set][i] = ld16(v + (tok0 + row) * v_stride + (int64_t)h * V + blockIdx.y * (32 * NW) + cc * VEC);
-        if constexpr (PRE) pbv[set][i] = beta[(tok0 + row) * Hv + h];
+        if constexpr (PRE) pbv[set][i] = gate_raw<T>(beta, beta_same, (tok0 + row) * Hv + h);
       }
       const float* gc = G + ch * 64;
       const int t = lt & 63;
@@ -424,7 +426,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
       // short chunk.
       pgl[set] = gc[63];
       pg[set] = gc[t];
-      pb[set] = beta[(tok0 + imin(t, nvalid - 1)) * Hv + h];
+      pb[set] = gate_raw<T>(beta, beta_same, (tok0 + imin(t, nvalid - 1)) * Hv + h);
       pnv[set] = nvalid;
       if constexpr (PRE) {
         // In the K tiles every 16-byte piece belongs to one token, 32 (tile & 1) + the row of its place, and this
@@ -432,7 +434,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
           pgk[set][j] = gc[32 * j + krow];
-          pbk[set][j] = beta[(tok0 + imin(32 * j + krow, nvalid - 1)) * Hv + h];
+          pbk[set][j] = gate_raw<T>(beta, beta_same, (tok0 + imin(32 * j + krow, nvalid - 1)) * Hv + h);
         }
       }
     };
@@ -442,7 +444,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
       if constexpr (PRE) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-          f1[j] = (32 * j + krow < pnv[set]) ? -pbk[set][j] * __expf(pgk[set][j]) : 0.f;
+          f1[j] = (32 * j + krow < pnv[set]) ? -gate_val<T>(pbk[set][j], beta_same) * __expf(pgk[set][j]) : 0.f;
           f2[j] = __expf(pgl[set] - pgk[set][j]);
         }
       }
@@ -467,12 +469,12 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
 #pragma unroll
       for (int i = 0; i < CV; ++i) {
         const int idc = imin(lt + i * NT, PV - 1);
-        if constexpr (PRE) st16(st + SM::off_v + idc * VEC, scale16<T>(pv[set][i], idc / VPR < pnv[set] ? pbv[set][i] : 0.f));
+        if constexpr (PRE) st16(st + SM::off_v + idc * VEC, scale16<T>(pv[set][i], idc / VPR < pnv[set] ? gate_val<T>(pbv[set][i], beta_same) : 0.f));
         else st16(st + SM::off_v + idc * VEC, pv[set][i]);
       }
       float* row = reinterpret_cast<float*>(gdn_smem + buf * SM::stage + SM::off_row);
       if (lt < 64) {
-        const float b = lt < pnv[set] ? pb[set] : 0.f, eg = __expf(pg[set]);
+        const float b = lt < pnv[set] ? gate_val<T>(pb[set], beta_same) : 0.f, eg = __expf(pg[set]);
         row[lt] = scale * eg;
         if constexpr (!PRE) {
           row[68 + lt] = __expf(pgl[set] - pg[set]);
@@ -895,8 +897,8 @@ struct FwdNorm {
 // and LDS stages of the recurrence kernel; FUSE: the recurrence kernel's own output waves write O (no norm, bf16)
 template <typename T, int DK, int NW, int NWS, int NLS, int STAGES, bool FUSE>
 static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const void* q, const void* k, const void* v,
-                            const float* g, const float* beta, const float* h0, const int64_t* cu, void* o, float* ht,
-                            unsigned char* ws, float scale, int l2norm, bool with_backward, const FwdNorm& fn,
+                            const float* g, const void* beta, int beta_same, const float* h0, const int64_t* cu, void* o,
+                            float* ht, unsigned char* ws, float scale, int l2norm, bool with_backward, const FwdNorm& fn,
                             hipStream_t st) {
   const int nc = (int)d.max_chunks();
   int* chunk_offsets = reinterpret_cast<int*>(ws + L.chunk_offsets);
@@ -909,7 +911,8 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   T* AQ = reinterpret_cast<T*>(ws + L.AQ);
   T* KAF = reinterpret_cast<T*>(ws + L.KAF);
   T* QTF = reinterpret_cast<T*>(ws + L.QTF);
-  const bool fuse = FUSE && fn.y == nullptr;
+  const bool fill_only = o == nullptr && fn.y == nullptr;   // refill the workspace for a backward pass, no output
+  const bool fuse = FUSE && fn.y == nullptr && !fill_only;
   // the per-chunk states and v_new leave the recurrence kernel only for a later reader: the backward pass or the
   // stand-alone output kernel
   const bool keep = with_backward || !fuse;
@@ -920,15 +923,17 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     auto kern = chunk_prep_kernel<T, DK>;
     constexpr int smem = PrepSmem<T, DK>::bytes;
     if (int e = set_lds(kern, smem)) return e;
-    GDN_LAUNCH(kKernPrep, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, g, beta, cu,
+    GDN_LAUNCH(kKernPrep, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, g, beta, beta_same, cu,
                (const int*)chunk_offsets, G, Ai, AQ, KAF, QTF, rstd, rstd + (int64_t)nc * 64 * d.Hqk, d.T, d.N, d.Hqk,
                d.Hv, scale, l2norm, ts);
   }
-  constexpr bool PRE = StatePre<T, DK, NWS, STAGES, FUSE>::value;
+  // decided for the two-slab variant, the largest one: results must not depend on how many slabs a launch happens
+  // to give a workgroup (a sequence computes the same bits alone and inside a packed batch)
+  constexpr bool PRE = StatePre<T, DK, 2, STAGES, FUSE>::value && StatePre<T, DK, NWS, STAGES, FUSE>::value;
   auto launch_state = [&](auto kern, int smem, int waves, T* op) -> int {
     if (int e = set_lds(kern, smem)) return e;
     GDN_LAUNCH(kKernStateFwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NWS)), dim3(64 * waves), smem, st, (const T*)KAF,
-               (const T*)QTF, (const T*)Ai, (const T*)AQ, (const T*)v, (const float*)G, beta, h0, ht, VF, HF, op, cu,
+               (const T*)QTF, (const T*)Ai, (const T*)AQ, (const T*)v, (const float*)G, beta, beta_same, h0, ht, VF, HF, op, cu,
                (const int*)chunk_offsets, d.T, d.Hqk, d.Hv, d.V, scale, ts.v);
     return 0;
   };
@@ -943,6 +948,7 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   if (int e = launch_state(chunk_state_kernel<T, DK, NWS, NLS, STAGES, false, PRE>,
                            StateSmem<T, DK, NWS, STAGES, false, PRE>::bytes, NWS + NLS, (T*)nullptr))
     return e;
+  if (fill_only) return (int)hipGetLastError();
   auto launch_out = [&](auto kern, auto nm) -> int {
     constexpr int smem = OutSmem<T, DK, NW>::bytes;
     if (int e = set_lds(kern, smem)) return e;
@@ -994,15 +1000,17 @@ extern "C" int64_t gdn_chunk_workspace_bytes(int B, int T, int N, int Hqk, int H
 
 namespace gdn {
 static int chunk_fwd_entry(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
-                           int64_t v_stride, const float* g, const float* beta, const float* initial_state,
+                           int64_t v_stride, const float* g, const void* beta, int beta_dtype, const float* initial_state,
                            const int64_t* cu_seqlens, void* o, float* final_state, void* workspace,
                            int64_t workspace_bytes, int B, int T, int N, int Hqk, int Hv, int K, int V, float scale,
                            int use_qk_l2norm, int dtype, const FwdNorm& fn, void* stream) {
   if (!q || !k || !v || !g || !beta || !workspace) return -1;
-  if (fn.y == nullptr ? !o : (!fn.gate || !fn.weight)) return -1;
+  if (fn.y != nullptr && (!fn.gate || !fn.weight)) return -1;
   ChunkDims d{B, T, N, Hqk, Hv, K, V, cu_seqlens != nullptr};
   d.ts = {q_stride, k_stride, v_stride, 0, 0, 0};
   if (int e = chunk_check_dims(d, dtype)) return e;
+  if (beta_dtype != 0 && beta_dtype != dtype) return -4;
+  const int beta_same = beta_dtype != 0;
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o | (uintptr_t)fn.y | (uintptr_t)fn.gate |
        (uintptr_t)fn.weight) & 15)
     return -6;
@@ -1010,12 +1018,13 @@ static int chunk_fwd_entry(const void* q, const void* k, const void* v, int64_t 
   dl.varlen = true;  // one layout for both modes (the packed bound is the larger)
   const ChunkWorkspace L = chunk_workspace_layout(dl, dtype == 0 ? 4 : 2);
   if (workspace_bytes < L.fwd_bytes) return -5;
-  const bool with_bwd = workspace_bytes >= L.total_bytes;   // a workspace sized for backward: the per-chunk states and v_new are kept
+  const bool with_bwd = workspace_bytes >= L.total_bytes;
+  if (!o && !fn.y && !with_bwd) return -1;   // without an output the call only makes sense as a refill   // a workspace sized for backward: the per-chunk states and v_new are kept
   if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
   unsigned char* ws = static_cast<unsigned char*>(workspace);
   hipStream_t st = (hipStream_t)stream;
 #define GDN_FWD(T_, DK_, NW_, NWS_, NLS_, ST_, FUSE_)                                                                       \
-  return chunk_fwd_launch<T_, DK_, NW_, NWS_, NLS_, ST_, FUSE_>(d, L, q, k, v, g, beta, initial_state, cu_seqlens, o, final_state, \
+  return chunk_fwd_launch<T_, DK_, NW_, NWS_, NLS_, ST_, FUSE_>(d, L, q, k, v, g, beta, beta_same, initial_state, cu_seqlens, o, final_state, \
                                                    ws, scale, use_qk_l2norm, with_bwd, fn, st)
   const bool wide = (V % 128 == 0);
   const bool solo = one_slab_per_workgroup(d, device_compute_units());
@@ -1036,26 +1045,26 @@ static int chunk_fwd_entry(const void* q, const void* k, const void* v, int64_t 
 }  // namespace gdn
 
 extern "C" int gdn_chunk_fwd_strided(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
-                                     int64_t v_stride, const float* g, const float* beta, const float* initial_state,
+                                     int64_t v_stride, const float* g, const void* beta, const float* initial_state,
                                      const int64_t* cu_seqlens, void* o, float* final_state, void* workspace,
                                      int64_t workspace_bytes, int B, int T, int N, int Hqk, int Hv, int K, int V,
-                                     float scale, int use_qk_l2norm, int dtype, void* stream) {
-  return gdn::chunk_fwd_entry(q, k, v, q_stride, k_stride, v_stride, g, beta, initial_state, cu_seqlens, o, final_state,
+                                     float scale, int use_qk_l2norm, int dtype, int beta_dtype, void* stream) {
+  return gdn::chunk_fwd_entry(q, k, v, q_stride, k_stride, v_stride, g, beta, beta_dtype, initial_state, cu_seqlens, o, final_state,
                               workspace, workspace_bytes, B, T, N, Hqk, Hv, K, V, scale, use_qk_l2norm, dtype,
                               gdn::FwdNorm{}, stream);
 }
 
 extern "C" int gdn_chunk_fwd_norm_strided(const void* q, const void* k, const void* v, int64_t q_stride,
-                                          int64_t k_stride, int64_t v_stride, const float* g, const float* beta,
+                                          int64_t k_stride, int64_t v_stride, const float* g, const void* beta,
                                           const float* initial_state, const int64_t* cu_seqlens, const void* gate,
                                           const void* norm_weight, void* o, void* y, float* rstd, float* final_state,
                                           void* workspace, int64_t workspace_bytes, int B, int T, int N, int Hqk,
                                           int Hv, int K, int V, float scale, float eps, int use_qk_l2norm, int dtype,
-                                          int weight_dtype, void* stream) {
+                                          int weight_dtype, int beta_dtype, void* stream) {
   if (!y) return -1;
   if (weight_dtype != 0 && weight_dtype != dtype) return -4;
   if (V != 64 && V != 128) return -3;
-  return gdn::chunk_fwd_entry(q, k, v, q_stride, k_stride, v_stride, g, beta, initial_state, cu_seqlens, o, final_state,
+  return gdn::chunk_fwd_entry(q, k, v, q_stride, k_stride, v_stride, g, beta, beta_dtype, initial_state, cu_seqlens, o, final_state,
                               workspace, workspace_bytes, B, T, N, Hqk, Hv, K, V, scale, use_qk_l2norm, dtype,
                               gdn::FwdNorm{gate, norm_weight, y, rstd, eps, weight_dtype == 0}, stream);
 }
@@ -1065,5 +1074,5 @@ extern "C" int gdn_chunk_fwd(const void* q, const void* k, const void* v, const 
                              void* workspace, int64_t workspace_bytes, int B, int T, int N, int Hqk, int Hv, int K,
                              int V, float scale, int use_qk_l2norm, int dtype, void* stream) {
   return gdn_chunk_fwd_strided(q, k, v, 0, 0, 0, g, beta, initial_state, cu_seqlens, o, final_state, workspace,
-                               workspace_bytes, B, T, N, Hqk, Hv, K, V, scale, use_qk_l2norm, dtype, stream);
+                               workspace_bytes, B, T, N, Hqk, Hv, K, V, scale, use_qk_l2norm, dtype, 0, stream);
 }

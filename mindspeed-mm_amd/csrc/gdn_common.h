@@ -121,6 +121,24 @@ template <typename T> __device__ __forceinline__ void load16_to_lds(const T* src
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                    (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
 }
+// beta (and its gradient) as the caller holds it: fp32, or, with `same` set, the 16-bit type T of q, k, v.  The value
+// is fetched raw and converted later, so that a loader can issue the fetch without waiting for it.
+template <typename T> __device__ __forceinline__ uint32_t gate_raw(const void* p, int same, int64_t i) {
+  if (sizeof(T) == 2 && same) return reinterpret_cast<const uint16_t*>(p)[i];
+  return reinterpret_cast<const uint32_t*>(p)[i];
+}
+template <typename T> __device__ __forceinline__ float gate_val(uint32_t raw, int same) {
+  if constexpr (sizeof(T) == 2) {
+    if (same) { T t; t.bits = (uint16_t)raw; return Elem<T>::to_f(t); }
+  }
+  return __uint_as_float(raw);
+}
+template <typename T> __device__ __forceinline__ void gate_st(void* p, int same, int64_t i, float x) {
+  if constexpr (sizeof(T) == 2) {
+    if (same) { reinterpret_cast<uint16_t*>(p)[i] = Elem<T>::from_f(x).bits; return; }
+  }
+  reinterpret_cast<float*>(p)[i] = x;
+}
 __device__ __forceinline__ int imin(int a, int b) { return a < b ? a : b; }
 __device__ __forceinline__ int imax(int a, int b) { return a > b ? a : b; }
 

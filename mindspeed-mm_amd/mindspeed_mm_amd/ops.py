@@ -15,12 +15,56 @@
 Everything here is host glue: validation, output/workspace allocation with torch, and one call into the
 C ABI per operator.  The kernels themselves are the HIP library; nothing in this file computes.
 """
+import functools
 import warnings
 from typing import Optional
 
 import torch
 
 from ._lib import DTYPE_CODE, GdnLibrary, default_library, ptr
+
+
+def _input_guard(fn):
+    """Runs an autograd function's forward / backward with the device of its first tensor argument current, as the
+    reference's input_guard does (mindspeed_mm/fsdp/ops/gdn/triton/utils.py:210-239): the backward pass is called
+    from the autograd engine's thread, where another device may be current."""
+    @functools.wraps(fn)
+    def wrapper(ctx, *args):
+        dev = next((a.device for a in args if isinstance(a, torch.Tensor)), None)
+        if dev is not None and dev.type == "cuda":
+            with torch.cuda.device(dev):
+                return fn(ctx, *args)
+        return fn(ctx, *args)
+    return wrapper
+
+
+# forward and backward keep the autocast state of the forward call (triton/utils.py:194-197)
+_custom_fwd = functools.partial(torch.amp.custom_fwd, device_type="cuda")
+_custom_bwd = functools.partial(torch.amp.custom_bwd, device_type="cuda")
+
+
+def _beta_arg(beta, act_dtype):
+    """beta as handed to the kernels: in place when it has the 16-bit dtype of q, k, v (the layer's beta = b.sigmoid()
+    is bf16, modeling_qwen3_5.py:833), else as float32.  Returns (tensor, dtype code)."""
+    if beta.dtype == act_dtype and act_dtype == torch.bfloat16:
+        return beta.detach().contiguous(), 1
+    return beta.detach().to(torch.float32).contiguous(), 0
+
+
+def _check_packed_length(cu_seqlens, tokens):
+    """The kernels visit the chunks of the listed sequences only: rows past cu_seqlens[-1] would be left unwritten.
+    Checked where it costs no device synchronisation (lists and host tensors); a device tensor must satisfy it too."""
+    if cu_seqlens is None:
+        return
+    if isinstance(cu_seqlens, torch.Tensor):
+        if cu_seqlens.device.type != "cpu" or cu_seqlens.numel() == 0:
+            return
+        first, last = int(cu_seqlens[0]), int(cu_seqlens[-1])
+    else:
+        first, last = int(cu_seqlens[0]), int(cu_seqlens[-1])
+    if first != 0 or last != tokens:
+        raise ValueError(f"cu_seqlens must start at 0 and end at the number of packed tokens ({tokens}), got "
+                         f"{first} ... {last}")
 
 
 def _act_code(activation):
@@ -64,16 +108,23 @@ class GdnOps:
         scale = self._check_chunk_args(q, k, v, g, beta, scale, initial_state, cu_seqlens, chunk_size, head_first)
         q, k, v, g, beta, initial_state = self._no_grad_views(q, k, v, g, beta, initial_state)
         return _ChunkGatedDeltaRule.apply(q, k, v, g, beta, float(scale), initial_state, bool(output_final_state),
-                                          cu_seqlens, bool(use_qk_l2norm_in_kernel), self)
+                                          cu_seqlens, bool(use_qk_l2norm_in_kernel), bool(skip_recompute), self)
 
     def chunk_gated_delta_rule_norm(self, q, k, v, g, beta, gate, norm_weight, eps=1e-6, scale=None,
                                     initial_state=None, output_final_state=False, use_qk_l2norm_in_kernel=False,
-                                    cu_seqlens=None):
+                                    cu_seqlens=None, in_output_kernel=False, skip_recompute=False):
         """The rule followed by the layer's gated RMSNorm over head_v_dim (modeling_qwen3_5.py:886-900:
-        `core_attn_out = self.norm(core_attn_out.reshape(-1, head_v_dim), z.reshape(-1, head_v_dim))`) in one pass:
-        the output kernel normalises and gates the rows before they leave, so `o` is neither written nor read again
-        when no gradient is needed.  Returns (y [B,T,Hv,V], final_state); same bits as the two operators in sequence.
-        head_v_dim must be 64 or 128."""
+        `core_attn_out = self.norm(core_attn_out.reshape(-1, head_v_dim), z.reshape(-1, head_v_dim))`).
+        Returns (y [B,T,Hv,V], final_state).  By default the two operators run in sequence (the rule's output comes
+        from the recurrence kernel itself, which is the faster arrangement); with in_output_kernel=True the stand-alone
+        output kernel forms it from the stored per-chunk states and normalises and gates the rows before they leave
+        (one launch less, head_v_dim 64 or 128).  Both give the same bits."""
+        if not in_output_kernel:
+            o, ht = self.chunk_gated_delta_rule(q, k, v, g, beta, scale, initial_state, output_final_state,
+                                                use_qk_l2norm_in_kernel, cu_seqlens, skip_recompute=skip_recompute)
+            V = v.shape[-1]
+            y = self.rms_norm_gated(o.reshape(-1, V), gate.reshape(-1, V).to(o.dtype), norm_weight, eps)
+            return y.view(o.shape), ht
         scale = self._check_chunk_args(q, k, v, g, beta, scale, initial_state, cu_seqlens, 64, False)
         V = v.shape[-1]
         if V not in (64, 128):
@@ -124,7 +175,9 @@ class GdnOps:
             raise ValueError("expected q,k [B,T,Hqk,K], v [B,T,Hv,V], g,beta [B,T,Hv] with Hv % Hqk == 0")
         if scale is None:
             scale = k.shape[-1] ** -0.5
-        self._need(q, k, v, g, beta, initial_state, cu_seqlens)
+        _check_packed_length(cu_seqlens, q.shape[1])
+        self._need(q, k, v, g, beta, initial_state, cu_seqlens if isinstance(cu_seqlens, torch.Tensor) and
+                   cu_seqlens.device.type != "cpu" else None)
         return scale
 
     def chunk_gated_delta_rule_qkv(self, mixed_qkv, g, beta, num_k_heads, num_v_heads, head_k_dim, head_v_dim,
@@ -133,9 +186,7 @@ class GdnOps:
                                    norm_eps=1e-6):
         """chunk_gated_delta_rule on the unsplit [B,T,2 Hqk K + Hv V] output of the convolution: equal to splitting it
         into q, k, v as modeling_qwen3_5.py:818-831 does and calling chunk_gated_delta_rule, without the copies.
-        With gate (the layer's z) and norm_weight the gated RMSNorm of modeling_qwen3_5.py:897-900 is applied inside
-        the output kernel (see chunk_gated_delta_rule_norm); q, k, v are then read in place as well, and a backward
-        pass returns their gradients through the split's own backward."""
+        With gate (the layer's z) and norm_weight the gated RMSNorm of modeling_qwen3_5.py:897-900 follows."""
         if (gate is None) != (norm_weight is None):
             raise ValueError("gate and norm_weight go together")
         if mixed_qkv.dim() != 3 or mixed_qkv.shape[-1] < 2 * num_k_heads * head_k_dim + num_v_heads * head_v_dim:
@@ -156,19 +207,18 @@ class GdnOps:
                     f"i.e., {len(cu_seqlens) - 1} rather than {initial_state.shape[0]}.")
         if scale is None:
             scale = head_k_dim ** -0.5
-        self._need(mixed_qkv, g, beta, initial_state, cu_seqlens)
-        if gate is not None:
-            B, T = mixed_qkv.shape[:2]
-            nq, nv = num_k_heads * head_k_dim, num_v_heads * head_v_dim
-            q, k, v = mixed_qkv[..., :nq], mixed_qkv[..., nq:2 * nq], mixed_qkv[..., 2 * nq:2 * nq + nv]
-            return self.chunk_gated_delta_rule_norm(
-                q.unflatten(-1, (num_k_heads, head_k_dim)), k.unflatten(-1, (num_k_heads, head_k_dim)),
-                v.unflatten(-1, (num_v_heads, head_v_dim)), g, beta, gate, norm_weight, norm_eps, scale, initial_state,
-                output_final_state, use_qk_l2norm_in_kernel, cu_seqlens)
+        _check_packed_length(cu_seqlens, mixed_qkv.shape[1])
+        self._need(mixed_qkv, g, beta, initial_state, cu_seqlens if isinstance(cu_seqlens, torch.Tensor) and
+                   cu_seqlens.device.type != "cpu" else None)
         mixed_qkv, g, beta, initial_state = self._no_grad_views(mixed_qkv, g, beta, initial_state)
-        return _ChunkGatedDeltaRuleQKV.apply(mixed_qkv, g, beta, int(num_k_heads), int(num_v_heads), int(head_k_dim),
-                                             int(head_v_dim), float(scale), initial_state, bool(output_final_state),
-                                             cu_seqlens, bool(use_qk_l2norm_in_kernel), self)
+        o, ht = _ChunkGatedDeltaRuleQKV.apply(mixed_qkv, g, beta, int(num_k_heads), int(num_v_heads), int(head_k_dim),
+                                              int(head_v_dim), float(scale), initial_state, bool(output_final_state),
+                                              cu_seqlens, bool(use_qk_l2norm_in_kernel), self)
+        if gate is None:
+            return o, ht
+        y = self.rms_norm_gated(o.reshape(-1, head_v_dim), gate.reshape(-1, head_v_dim).to(o.dtype), norm_weight,
+                                norm_eps)
+        return y.view(o.shape), ht
 
     def gdn_gates(self, a, b, A_log, dt_bias):
         """(g, beta) of the layer from its projections a, b [..., Hv] and parameters A_log, dt_bias [Hv]:
@@ -320,7 +370,7 @@ class GdnOps:
 def _i64(cu, ref):
     if cu is None:
         return None
-    return cu.to(device=ref.device, dtype=torch.int64).contiguous()
+    return torch.as_tensor(cu).to(device=ref.device, dtype=torch.int64).contiguous()
 
 
 def _token_view(x):
@@ -343,55 +393,73 @@ def _chunk_workspace(lib, device, B, T, N, Hqk, Hv, K, V, code, need_grad):
 
 
 class _ChunkGatedDeltaRule(torch.autograd.Function):
-    """Positional order as ChunkGatedDeltaRuleFunction.forward (chunk_gated_delta_rule.py:182-196)."""
+    """Positional order as ChunkGatedDeltaRuleFunction.forward (chunk_gated_delta_rule.py:182-196).
+
+    skip_recompute=False (the default, as in the reference, which saves q, k, v, g, beta, A, h0 and recomputes w, u, h
+    and v_new in its backward pass, chunk_gated_delta_rule.py:102-119, :264): nothing but the inputs is kept between
+    the passes; the backward pass refills a workspace (chunk-local kernel and recurrence, no output) before its own
+    kernels.  skip_recompute=True keeps the forward pass's workspace instead (per-chunk states, v_new, Tm, ...:
+    gdn_chunk_workspace_bytes with with_backward=1) and skips that work.  Both give the same gradients, bit for bit."""
 
     @staticmethod
+    @_input_guard
+    @_custom_fwd
     def forward(ctx, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens,
-                use_qk_l2norm_in_kernel, ops):
+                use_qk_l2norm_in_kernel, skip_recompute, ops):
         lib = ops.lib
         B, T, Hqk, K = q.shape
         Hv, V = v.shape[2], v.shape[3]
         N = (len(cu_seqlens) - 1) if cu_seqlens is not None else B
         need_grad = any(ctx.needs_input_grad[:5]) or (initial_state is not None and ctx.needs_input_grad[6])
+        keep = need_grad and skip_recompute
         (qc, sq), (kc, sk), (vc, sv) = _token_view(q), _token_view(k), _token_view(v)
-        g32, b32, h0 = ops._f32(g), ops._f32(beta), ops._f32(initial_state)
+        g32, h0 = ops._f32(g), ops._f32(initial_state)
+        bc, bcode = _beta_arg(beta, q.dtype)
         cu = _i64(cu_seqlens, q)
         code = DTYPE_CODE[q.dtype]
-        ws, nbytes = _chunk_workspace(lib, q.device, B, T, N, Hqk, Hv, K, V, code, need_grad)
+        ws, nbytes = _chunk_workspace(lib, q.device, B, T, N, Hqk, Hv, K, V, code, keep)
         o = torch.empty(B, T, Hv, V, dtype=v.dtype, device=v.device)
         ht = torch.empty(N, Hv, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
-        rc = lib.gdn_chunk_fwd_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(b32), ptr(h0), ptr(cu),
+        rc = lib.gdn_chunk_fwd_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(bc), ptr(h0), ptr(cu),
                                        ptr(o), ptr(ht), ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale,
-                                       int(use_qk_l2norm_in_kernel), code, lib.stream())
+                                       int(use_qk_l2norm_in_kernel), code, bcode, lib.stream())
         lib.check(rc, "gdn_chunk_fwd_strided")
         if need_grad:
-            ctx.save_for_backward(qc, kc, vc, g32, b32, h0, cu, ws)
+            ctx.save_for_backward(qc, kc, vc, g32, bc, h0, cu, ws if keep else None)
             ctx.meta = (B, T, N, Hqk, Hv, K, V, scale, int(use_qk_l2norm_in_kernel), code, nbytes,
-                        g.dtype, beta.dtype, None if initial_state is None else initial_state.dtype, sq, sk, sv)
+                        g.dtype, beta.dtype, None if initial_state is None else initial_state.dtype, sq, sk, sv, bcode)
             ctx.ops = ops
         return o, ht
 
     @staticmethod
+    @_input_guard
+    @_custom_bwd
     def backward(ctx, do, dht):
-        qc, kc, vc, g32, b32, h0, cu, ws = ctx.saved_tensors
-        B, T, N, Hqk, Hv, K, V, scale, l2, code, nbytes, g_dt, b_dt, h_dt, sq, sk, sv = ctx.meta
+        qc, kc, vc, g32, bc, h0, cu, ws = ctx.saved_tensors
+        B, T, N, Hqk, Hv, K, V, scale, l2, code, nbytes, g_dt, b_dt, h_dt, sq, sk, sv, bcode = ctx.meta
         lib = ctx.ops.lib
+        dev = qc.device
+        if ws is None:   # nothing was kept: refill a workspace (no output is written when o is null)
+            ws, nbytes = _chunk_workspace(lib, dev, B, T, N, Hqk, Hv, K, V, code, True)
+            rc = lib.gdn_chunk_fwd_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(bc), ptr(h0), ptr(cu),
+                                           None, None, ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale, l2, code, bcode,
+                                           lib.stream())
+            lib.check(rc, "gdn_chunk_fwd_strided (recompute)")
         do = do.contiguous()
         dht = ctx.ops._f32(dht)
-        dev = qc.device
         dq = torch.empty(B, T, Hqk, K, dtype=qc.dtype, device=dev)
         dk = torch.empty(B, T, Hqk, K, dtype=qc.dtype, device=dev)
         dv = torch.empty(B, T, Hv, V, dtype=qc.dtype, device=dev)
         dg = torch.empty(B, T, Hv, dtype=torch.float32, device=dev)
-        db = torch.empty(B, T, Hv, dtype=torch.float32, device=dev)
+        db = torch.empty(B, T, Hv, dtype=bc.dtype, device=dev)
         dh0 = torch.empty(N, Hv, K, V, dtype=torch.float32, device=dev) if h0 is not None else None
-        rc = lib.gdn_chunk_bwd_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(b32), ptr(h0), ptr(cu),
+        rc = lib.gdn_chunk_bwd_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(bc), ptr(h0), ptr(cu),
                                        ptr(do), ptr(dht), ptr(dq), ptr(dk), ptr(dv), 0, 0, 0, ptr(dg), ptr(db),
-                                       ptr(dh0), ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale, l2, code,
+                                       ptr(dh0), ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale, l2, code, bcode,
                                        lib.stream())
         lib.check(rc, "gdn_chunk_bwd_strided")
         return (dq, dk, dv, dg.to(g_dt), db.to(b_dt), None, None if dh0 is None else dh0.to(h_dt), None, None, None,
-                None)
+                None, None)
 
 
 class _ChunkGatedDeltaRuleNorm(torch.autograd.Function):
@@ -399,6 +467,8 @@ class _ChunkGatedDeltaRuleNorm(torch.autograd.Function):
     (the forward then also writes `o` and 1/rms, which they need)."""
 
     @staticmethod
+    @_input_guard
+    @_custom_fwd
     def forward(ctx, q, k, v, g, beta, gate, norm_weight, eps, scale, initial_state, output_final_state, cu_seqlens,
                 use_qk_l2norm_in_kernel, ops):
         lib = ops.lib
@@ -408,7 +478,8 @@ class _ChunkGatedDeltaRuleNorm(torch.autograd.Function):
         rule_grad = any(ctx.needs_input_grad[:5]) or (initial_state is not None and ctx.needs_input_grad[9])
         need_grad = rule_grad or ctx.needs_input_grad[5] or ctx.needs_input_grad[6]
         (qc, sq), (kc, sk), (vc, sv) = _token_view(q), _token_view(k), _token_view(v)
-        g32, b32, h0 = ops._f32(g), ops._f32(beta), ops._f32(initial_state)
+        g32, h0 = ops._f32(g), ops._f32(initial_state)
+        b32, bcode = _beta_arg(beta, q.dtype)
         cu = _i64(cu_seqlens, q)
         dt = q.dtype
         code = DTYPE_CODE[dt]
@@ -423,21 +494,23 @@ class _ChunkGatedDeltaRuleNorm(torch.autograd.Function):
         rc = lib.gdn_chunk_fwd_norm_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(b32), ptr(h0),
                                             ptr(cu), ptr(gc), ptr(wc), ptr(o), ptr(y), ptr(rstd), ptr(ht), ptr(ws),
                                             nbytes, B, T, N, Hqk, Hv, K, V, scale, eps,
-                                            int(use_qk_l2norm_in_kernel), code, DTYPE_CODE[w_dt], lib.stream())
+                                            int(use_qk_l2norm_in_kernel), code, DTYPE_CODE[w_dt], bcode, lib.stream())
         lib.check(rc, "gdn_chunk_fwd_norm_strided")
         if need_grad:
             ctx.save_for_backward(qc, kc, vc, g32, b32, h0, cu, ws if rule_grad else None, o, gc, wc, rstd)
             ctx.meta = (B, T, N, Hqk, Hv, K, V, scale, int(use_qk_l2norm_in_kernel), code, nbytes, g.dtype,
                         beta.dtype, None if initial_state is None else initial_state.dtype, sq, sk, sv, w_dt,
-                        norm_weight.dtype, gate.dtype, gate.shape, rule_grad)
+                        norm_weight.dtype, gate.dtype, gate.shape, rule_grad, bcode)
             ctx.ops = ops
         return y, ht
 
     @staticmethod
+    @_input_guard
+    @_custom_bwd
     def backward(ctx, dy, dht):
         qc, kc, vc, g32, b32, h0, cu, ws, o, gc, wc, rstd = ctx.saved_tensors
         (B, T, N, Hqk, Hv, K, V, scale, l2, code, nbytes, g_dt, b_dt, h_dt, sq, sk, sv, w_dt, weight_dt, gate_dt,
-         gate_shape, rule_grad) = ctx.meta
+         gate_shape, rule_grad, bcode) = ctx.meta
         lib = ctx.ops.lib
         dev, dt = qc.device, qc.dtype
         rows = B * T * Hv
@@ -457,12 +530,12 @@ class _ChunkGatedDeltaRuleNorm(torch.autograd.Function):
             dk = torch.empty(B, T, Hqk, K, dtype=dt, device=dev)
             dv = torch.empty(B, T, Hv, V, dtype=dt, device=dev)
             dg = torch.empty(B, T, Hv, dtype=torch.float32, device=dev)
-            db = torch.empty(B, T, Hv, dtype=torch.float32, device=dev)
+            db = torch.empty(B, T, Hv, dtype=b32.dtype, device=dev)
             dh0 = torch.empty(N, Hv, K, V, dtype=torch.float32, device=dev) if h0 is not None else None
             rc = lib.gdn_chunk_bwd_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(b32), ptr(h0),
                                            ptr(cu), ptr(do), ptr(dht), ptr(dq), ptr(dk), ptr(dv), 0, 0, 0, ptr(dg),
                                            ptr(db), ptr(dh0), ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale, l2,
-                                           code, lib.stream())
+                                           code, bcode, lib.stream())
             lib.check(rc, "gdn_chunk_bwd_strided")
             dg, db = dg.to(g_dt), db.to(b_dt)
             dh0 = None if dh0 is None else dh0.to(h_dt)
@@ -476,6 +549,8 @@ class _ChunkGatedDeltaRuleQKV(torch.autograd.Function):
     backward pass writes dq, dk, dv into one [B,T,D] gradient, so neither the split nor its backward copies."""
 
     @staticmethod
+    @_input_guard
+    @_custom_fwd
     def forward(ctx, qkv, g, beta, Hqk, Hv, K, V, scale, initial_state, output_final_state, cu_seqlens,
                 use_qk_l2norm_in_kernel, ops):
         lib = ops.lib
@@ -485,7 +560,8 @@ class _ChunkGatedDeltaRuleQKV(torch.autograd.Function):
         need_grad = any(ctx.needs_input_grad[:3]) or (initial_state is not None and ctx.needs_input_grad[8])
         vec = 16 // qkv.element_size()
         x = qkv if (qkv.is_contiguous() and D % vec == 0 and qkv.data_ptr() % 16 == 0) else qkv.contiguous()
-        g32, b32, h0 = ops._f32(g), ops._f32(beta), ops._f32(initial_state)
+        g32, h0 = ops._f32(g), ops._f32(initial_state)
+        b32, bcode = _beta_arg(beta, qkv.dtype)
         cu = _i64(cu_seqlens, qkv)
         code = DTYPE_CODE[qkv.dtype]
         es = x.element_size()
@@ -495,19 +571,21 @@ class _ChunkGatedDeltaRuleQKV(torch.autograd.Function):
         base = x.data_ptr()
         rc = lib.gdn_chunk_fwd_strided(base, base + nq * es, base + 2 * nq * es, D, D, D, ptr(g32), ptr(b32), ptr(h0),
                                        ptr(cu), ptr(o), ptr(ht), ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale,
-                                       int(use_qk_l2norm_in_kernel), code, lib.stream())
+                                       int(use_qk_l2norm_in_kernel), code, bcode, lib.stream())
         lib.check(rc, "gdn_chunk_fwd_strided")
         if need_grad:
             ctx.save_for_backward(x, g32, b32, h0, cu, ws)
             ctx.meta = (B, T, D, N, Hqk, Hv, K, V, scale, int(use_qk_l2norm_in_kernel), code, nbytes,
-                        g.dtype, beta.dtype, None if initial_state is None else initial_state.dtype)
+                        g.dtype, beta.dtype, None if initial_state is None else initial_state.dtype, bcode)
             ctx.ops = ops
         return o, ht
 
     @staticmethod
+    @_input_guard
+    @_custom_bwd
     def backward(ctx, do, dht):
         x, g32, b32, h0, cu, ws = ctx.saved_tensors
-        B, T, D, N, Hqk, Hv, K, V, scale, l2, code, nbytes, g_dt, b_dt, h_dt = ctx.meta
+        B, T, D, N, Hqk, Hv, K, V, scale, l2, code, nbytes, g_dt, b_dt, h_dt, bcode = ctx.meta
         lib = ctx.ops.lib
         nq, nv, es, dev = Hqk * K, Hv * V, x.element_size(), x.device
         do = do.contiguous()
@@ -515,13 +593,13 @@ class _ChunkGatedDeltaRuleQKV(torch.autograd.Function):
         # columns past q, k, v (none in the layer) receive no gradient
         dx = torch.empty_like(x) if D == 2 * nq + nv else torch.zeros_like(x)
         dg = torch.empty(B, T, Hv, dtype=torch.float32, device=dev)
-        db = torch.empty(B, T, Hv, dtype=torch.float32, device=dev)
+        db = torch.empty(B, T, Hv, dtype=b32.dtype, device=dev)
         dh0 = torch.empty(N, Hv, K, V, dtype=torch.float32, device=dev) if h0 is not None else None
         base, dbase = x.data_ptr(), dx.data_ptr()
         rc = lib.gdn_chunk_bwd_strided(base, base + nq * es, base + 2 * nq * es, D, D, D, ptr(g32), ptr(b32), ptr(h0),
                                        ptr(cu), ptr(do), ptr(dht), dbase, dbase + nq * es, dbase + 2 * nq * es, D, D,
                                        D, ptr(dg), ptr(db), ptr(dh0), ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale,
-                                       l2, code, lib.stream())
+                                       l2, code, bcode, lib.stream())
         lib.check(rc, "gdn_chunk_bwd_strided")
         return (dx, dg.to(g_dt), db.to(b_dt), None, None, None, None, None, None if dh0 is None else dh0.to(h_dt),
                 None, None, None, None)
@@ -531,6 +609,8 @@ class _GdnGates(torch.autograd.Function):
     """beta = sigmoid(b), g = -exp(A_log.float()) * softplus(a.float() + dt_bias), modeling_qwen3_5.py:833-841."""
 
     @staticmethod
+    @_input_guard
+    @_custom_fwd
     def forward(ctx, a, b, A_log, dt_bias, ops):
         lib = ops.lib
         Hv = a.shape[-1]
@@ -549,6 +629,8 @@ class _GdnGates(torch.autograd.Function):
         return g, beta
 
     @staticmethod
+    @_input_guard
+    @_custom_bwd
     def backward(ctx, dg, dbeta):
         ac, bc, Ac, dc = ctx.saved_tensors
         tokens, Hv, A_dt, d_dt = ctx.meta
@@ -571,6 +653,8 @@ class _CausalConv1d(torch.autograd.Function):
     """Argument order as CausalConv1dFunction.forward (models/qwen3_5/causal_conv1d.py:27-38)."""
 
     @staticmethod
+    @_input_guard
+    @_custom_fwd
     def forward(ctx, x, weight, bias, residual, initial_state, activation, cu_seqlens, output_final_state, ops):
         lib = ops.lib
         B, T, D = x.shape
@@ -596,6 +680,8 @@ class _CausalConv1d(torch.autograd.Function):
         return y, fs
 
     @staticmethod
+    @_input_guard
+    @_custom_bwd
     def backward(ctx, dy, dfs):
         xc, wc, bc, h0, cu = ctx.saved_tensors
         B, T, N, D, W, act, dt, w_dt, b_dt, has_res, r_dt, h_dt = ctx.meta
@@ -619,6 +705,8 @@ class _RMSNormGated(torch.autograd.Function):
     """y = (weight * rmsnorm(x)) * silu(gate) over the last axis."""
 
     @staticmethod
+    @_input_guard
+    @_custom_fwd
     def forward(ctx, x, gate, weight, eps, ops):
         lib = ops.lib
         dt = x.dtype
@@ -645,6 +733,8 @@ class _RMSNormGated(torch.autograd.Function):
         return y.view(x.shape)
 
     @staticmethod
+    @_input_guard
+    @_custom_bwd
     def backward(ctx, dy):
         xc, gc, wc, rstd = ctx.saved_tensors
         rows, N, dt, w_dt, weight_dt, gate_dt, shape = ctx.meta
@@ -680,7 +770,10 @@ def chunk_gated_delta_rule(q, k, v, g, beta, scale=None, initial_state=None, out
 
     q,k [B,T,Hqk,K]; v [B,T,Hv,V]; g,beta [B,T,Hv]; Hv may be a multiple of Hqk (grouped heads are read in
     place; dq/dk come back summed over each group).  float32 is accepted as well as bfloat16.
-    `skip_recompute` is accepted and ignored (all backward inputs are kept in the workspace)."""
+    skip_recompute=False (default, as in the reference): nothing but the inputs is kept for the backward pass, which
+    recomputes Tm, the per-chunk states and v_new; skip_recompute=True keeps the forward pass's workspace instead
+    (gdn_chunk_workspace_bytes with with_backward=1: 1.2 GB at B=2, T=8192, H_v=32, d=128) for a faster backward pass.
+    The gradients are the same bits either way."""
     return _default_ops().chunk_gated_delta_rule(q, k, v, g, beta, scale, initial_state, output_final_state,
                                                  use_qk_l2norm_in_kernel, cu_seqlens, chunk_size, head_first,
                                                  skip_recompute)
@@ -688,11 +781,14 @@ def chunk_gated_delta_rule(q, k, v, g, beta, scale=None, initial_state=None, out
 
 @torch.compiler.disable
 def chunk_gated_delta_rule_norm(q, k, v, g, beta, gate, norm_weight, eps=1e-6, scale=None, initial_state=None,
-                                output_final_state=False, use_qk_l2norm_in_kernel=False, cu_seqlens=None):
+                                output_final_state=False, use_qk_l2norm_in_kernel=False, cu_seqlens=None,
+                                in_output_kernel=False, skip_recompute=False):
     return _default_ops().chunk_gated_delta_rule_norm(q, k, v, g, beta, gate, norm_weight, eps, scale, initial_state,
-                                                      output_final_state, use_qk_l2norm_in_kernel, cu_seqlens)
+                                                      output_final_state, use_qk_l2norm_in_kernel, cu_seqlens,
+                                                      in_output_kernel, skip_recompute)
 
 
+@torch.compiler.disable
 def chunk_gated_delta_rule_qkv(mixed_qkv, g, beta, num_k_heads, num_v_heads, head_k_dim, head_v_dim, scale=None,
                                initial_state=None, output_final_state=False, use_qk_l2norm_in_kernel=False,
                                cu_seqlens=None, gate=None, norm_weight=None, norm_eps=1e-6):
@@ -701,10 +797,12 @@ def chunk_gated_delta_rule_qkv(mixed_qkv, g, beta, num_k_heads, num_v_heads, hea
                                                      use_qk_l2norm_in_kernel, cu_seqlens, gate, norm_weight, norm_eps)
 
 
+@torch.compiler.disable
 def gdn_gates(a, b, A_log, dt_bias):
     return _default_ops().gdn_gates(a, b, A_log, dt_bias)
 
 
+@torch.compiler.disable
 def fused_recurrent_gated_delta_rule(q, k, v, g, beta=None, scale=None, initial_state=None,
                                      output_final_state=False, cu_seqlens=None, use_qk_l2norm_in_kernel=False,
                                      inplace_state=False):
@@ -722,6 +820,7 @@ def fused_recurrent_gated_delta_rule_qkv(mixed_qkv, a, b, A_log, dt_bias, num_k_
         output_final_state, use_qk_l2norm_in_kernel, inplace_state)
 
 
+@torch.compiler.disable
 def decode_step(mixed_qkv, a, b, conv_state, recurrent_state, conv_weight, conv_bias, A_log, dt_bias, num_k_heads,
                 num_v_heads, head_k_dim, head_v_dim, activation="silu"):
     return _default_ops().decode_step(mixed_qkv, a, b, conv_state, recurrent_state, conv_weight, conv_bias, A_log,
@@ -758,6 +857,7 @@ class GdnDecodeCache:
                 self.recurrent_states[i] = self.recurrent_states[i].index_select(0, idx)
 
 
+@torch.compiler.disable
 def causal_conv1d(x, weight, bias=None, residual=None, initial_state=None, activation=None, cu_seqlens=None,
                   output_final_state=False):
     return _default_ops().causal_conv1d(x, weight, bias, residual, initial_state, activation, cu_seqlens,

@@ -32,7 +32,7 @@ def _err(name, got, ref, dtype, abs_tol, rtol=0.0):
 
 
 def check_chunk(ops, device, B, T, Hqk, Hv, K, V, dtype, l2=True, cu=None, backward=False, seed=0, with_h0=True,
-                scale=None, wrap=lambda t: t, **recipe):
+                scale=None, wrap=lambda t: t, skip_recompute=False, **recipe):
     N = (len(cu) - 1) if cu is not None else B
     x = gdn_inputs(B, T, Hqk, Hv, K, V, dtype, seed=seed, N=N, l2norm_in_kernel=l2, **recipe)
     dev = {n: wrap(t.to(device)) for n, t in x.items()}
@@ -41,7 +41,7 @@ def check_chunk(ops, device, B, T, Hqk, Hv, K, V, dtype, l2=True, cu=None, backw
     cu_t = torch.tensor(cu, dtype=torch.int64, device=device) if cu is not None else None
     o, ht = ops.chunk_gated_delta_rule(leaves["q"], leaves["k"], leaves["v"], leaves["g"], leaves["beta"],
                                        scale=scale, initial_state=h0, output_final_state=True,
-                                       use_qk_l2norm_in_kernel=l2, cu_seqlens=cu_t)
+                                       use_qk_l2norm_in_kernel=l2, cu_seqlens=cu_t, skip_recompute=skip_recompute)
     ref_leaves = {n: x[n].float().clone().requires_grad_(backward) for n in ("q", "k", "v", "g", "beta")}
     rh0 = x["h0"].clone().requires_grad_(backward) if with_h0 else None
     ro, rht = O.chunk_gated_delta_rule_ref(ref_leaves["q"], ref_leaves["k"], ref_leaves["v"], ref_leaves["g"],
@@ -58,6 +58,65 @@ def check_chunk(ops, device, B, T, Hqk, Hv, K, V, dtype, l2=True, cu=None, backw
         if with_h0:
             errs["dh0"] = _err("dh0", h0.grad, rh0.grad, dtype, BF16_ABS_GRAD)
     return errs
+
+
+def check_chunk_reference_recipe(ops, device, B, T, H, K, V, l2, cu=None, oracle_heads=2, seed=42):
+    """The reference's own test of the operator (tests/ut_fsdp/models/qwen3_5/test_chunk_gated_delta_rule.py:158-247):
+    bf16, q, k, v ~ N(0,1) (q, k l2-normalised beforehand when the kernel is not asked to), beta = sigmoid(U(0,1)),
+    g = logsigmoid(U(0,1)) in bf16, no initial state, loss = sum(o * do), seed 42.  All heads run on the device; the
+    oracle runs on the first `oracle_heads` heads (heads are independent), which keeps its CPU time bounded.
+    Checked against the task's bounds (2e-2 on o, 5e-2 on gradients, absolute) and against the reference test's own
+    allclose(rtol=1e-2, atol=1e-2)."""
+    dtype = torch.bfloat16
+    gen = torch.Generator().manual_seed(seed)
+    q, k = torch.randn(B, T, H, K, generator=gen), torch.randn(B, T, H, K, generator=gen)
+    if not l2:
+        q = q * torch.rsqrt((q * q).sum(-1, keepdim=True) + 1e-6)
+        k = k * torch.rsqrt((k * k).sum(-1, keepdim=True) + 1e-6)
+    v = torch.randn(B, T, H, V, generator=gen)
+    beta = torch.rand(B, T, H, generator=gen).to(dtype).sigmoid()
+    g = torch.nn.functional.logsigmoid(torch.rand(B, T, H, generator=gen).to(dtype))
+    do = torch.randn(B, T, H, V, generator=gen).to(dtype)
+    x = dict(q=q.to(dtype), k=k.to(dtype), v=v.to(dtype), g=g, beta=beta)
+    leaves = {n: t.to(device).requires_grad_(True) for n, t in x.items()}
+    cu_t = torch.tensor(cu, dtype=torch.int64, device=device) if cu is not None else None
+    o, _ = ops.chunk_gated_delta_rule(leaves["q"], leaves["k"], leaves["v"], leaves["g"], leaves["beta"],
+                                      use_qk_l2norm_in_kernel=l2, cu_seqlens=cu_t)
+    (o.float() * do.to(device).float()).sum().backward()
+    hs = min(oracle_heads, H)
+    ref = {n: t[:, :, :hs].float().clone().requires_grad_(True) for n, t in x.items()}
+    ro, _ = O.chunk_gated_delta_rule_ref(ref["q"], ref["k"], ref["v"], ref["g"], ref["beta"],
+                                         use_qk_l2norm_in_kernel=l2, cu_seqlens=cu)
+    (ro * do[:, :, :hs].float()).sum().backward()
+    assert o.dtype == dtype
+    errs = {"o": _err("o", o[:, :, :hs], ro, dtype, BF16_ABS_O)}
+    _err("o (reference test's allclose)", o[:, :, :hs], ro, dtype, 1e-2, 1e-2)
+    for n in ("q", "k", "v", "g", "beta"):
+        assert leaves[n].grad.dtype == leaves[n].dtype
+        errs["d" + n] = _err("d" + n, leaves[n].grad[:, :, :hs], ref[n].grad, dtype, BF16_ABS_GRAD)
+    return errs
+
+
+def check_chunk_recompute_equals_stored(ops, device, B, T, Hqk, Hv, K, V, dtype, l2=True, cu=None, seed=0,
+                                        wrap=lambda t: t, **recipe):
+    """skip_recompute=False (nothing kept, the backward pass refills a workspace) against skip_recompute=True (the
+    forward pass's workspace is kept): outputs and every gradient bit for bit."""
+    N = (len(cu) - 1) if cu is not None else B
+    x = gdn_inputs(B, T, Hqk, Hv, K, V, dtype, seed=seed, N=N, l2norm_in_kernel=l2, **recipe)
+    dev = {n: wrap(t.to(device)) for n, t in x.items()}
+    cu_t = torch.tensor(cu, dtype=torch.int64, device=device) if cu is not None else None
+    res = []
+    for skip in (False, True):
+        L = {n: dev[n].clone().requires_grad_(True) for n in ("q", "k", "v", "g", "beta", "h0")}
+        o, ht = ops.chunk_gated_delta_rule(L["q"], L["k"], L["v"], L["g"], L["beta"], initial_state=L["h0"],
+                                           output_final_state=True, use_qk_l2norm_in_kernel=l2, cu_seqlens=cu_t,
+                                           skip_recompute=skip)
+        ((o.float() * dev["do"].float()).sum() + (ht * dev["dht"]).sum()).backward()
+        res.append((o, ht, L))
+    (o1, h1, L1), (o2, h2, L2) = res
+    assert torch.equal(o1, o2) and torch.equal(h1, h2)
+    for n in L1:
+        assert torch.equal(L1[n].grad, L2[n].grad), f"gradient of {n} differs between the two modes"
 
 
 def check_recurrent(ops, device, B, T, Hqk, Hv, K, V, dtype, l2=True, seed=0, with_state=True, wrap=lambda t: t):
@@ -215,7 +274,7 @@ def check_chunk_norm(ops, device, B, T, Hqk, Hv, K, V, dtype, l2=True, cu=None, 
     A, Bc = leaves(), leaves()
     y, ht = ops.chunk_gated_delta_rule_norm(A["q"], A["k"], A["v"], A["g"], A["beta"], A["z"], A["w"], eps=1e-6,
                                             initial_state=A["h0"], output_final_state=True,
-                                            use_qk_l2norm_in_kernel=l2, cu_seqlens=cu_t)
+                                            use_qk_l2norm_in_kernel=l2, cu_seqlens=cu_t, in_output_kernel=True)
     o2, ht2 = ops.chunk_gated_delta_rule(Bc["q"], Bc["k"], Bc["v"], Bc["g"], Bc["beta"], initial_state=Bc["h0"],
                                          output_final_state=True, use_qk_l2norm_in_kernel=l2, cu_seqlens=cu_t)
     y2 = ops.rms_norm_gated(o2.reshape(-1, V), Bc["z"].reshape(-1, V), Bc["w"], 1e-6).view(B, T, Hv, V)
@@ -226,7 +285,7 @@ def check_chunk_norm(ops, device, B, T, Hqk, Hv, K, V, dtype, l2=True, cu=None, 
         with torch.no_grad():
             y3, _ = ops.chunk_gated_delta_rule_norm(dev["q"], dev["k"], dev["v"], dev["g"], dev["beta"],
                                                     wrap(z.to(device)), wrap(w.to(device)), initial_state=dev["h0"],
-                                                    use_qk_l2norm_in_kernel=l2, cu_seqlens=cu_t)
+                                                    use_qk_l2norm_in_kernel=l2, cu_seqlens=cu_t, in_output_kernel=True)
         assert torch.equal(y3, y)
     ro, rht = O.chunk_gated_delta_rule_ref(x["q"].float(), x["k"].float(), x["v"].float(), x["g"], x["beta"],
                                            initial_state=x["h0"], output_final_state=True,

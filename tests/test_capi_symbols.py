@@ -79,6 +79,31 @@ def test_validation_errors_match_reference():
         M.causal_conv1d(torch.randn(1, 8, 8), torch.randn(4, 16))
 
 
+def test_packed_lengths_must_cover_every_token():
+    """The kernels visit the chunks of the listed sequences only; a cu_seqlens list or host tensor that stops short
+    of the packed length would leave output rows unwritten, so it is refused (no device synchronisation needed)."""
+    import torch
+    import mindspeed_mm_amd as M
+    q = torch.randn(1, 100, 1, 64, dtype=torch.bfloat16)
+    g, b = torch.zeros(1, 100, 1), torch.ones(1, 100, 1)
+    with pytest.raises(ValueError, match="cu_seqlens must start at 0 and end"):
+        M.chunk_gated_delta_rule(q, q, q, g, b, cu_seqlens=torch.tensor([0, 30, 90]))
+    with pytest.raises(ValueError, match="cu_seqlens must start at 0 and end"):
+        M.chunk_gated_delta_rule(q, q, q, g, b, cu_seqlens=[5, 30, 100])
+    with pytest.raises(RuntimeError, match="no host fallback"):      # a complete list passes the check
+        M.chunk_gated_delta_rule(q, q, q, g, b, cu_seqlens=[0, 30, 100])
+
+
+def test_autograd_functions_carry_the_guards():
+    """Every autograd function runs with its tensors' device current and keeps the forward's autocast state in the
+    backward pass (the reference's input_guard and custom_fwd / custom_bwd)."""
+    from mindspeed_mm_amd import ops
+    for cls in (ops._ChunkGatedDeltaRule, ops._ChunkGatedDeltaRuleNorm, ops._ChunkGatedDeltaRuleQKV, ops._GdnGates,
+                ops._CausalConv1d, ops._RMSNormGated):
+        for fn in (cls.forward, cls.backward):
+            assert hasattr(fn, "__wrapped__"), (cls.__name__, fn.__name__)
+
+
 def test_validation_of_the_layer_level_entry_points():
     """Shape and dtype errors of the operators around the rule are raised before anything touches a device."""
     import torch

@@ -62,6 +62,13 @@ def test_chunk_packed_with_empty_sequences(ops, cu):
     P.check_chunk(ops, "cpu", 1, cu[-1], 1, 2, 64, 64, F32, cu=cu, backward=True, wrap=guarded, h0_std=0.1)
 
 
+@pytest.mark.parametrize("dtype,B,T,Hqk,Hv,K,V,cu", [
+    (BF, 1, 200, 1, 2, 128, 128, None), (F32, 1, 140, 1, 2, 64, 64, [0, 5, 70, 140]),
+])
+def test_chunk_backward_recompute_mode_equals_stored_mode(ops, dtype, B, T, Hqk, Hv, K, V, cu):
+    P.check_chunk_recompute_equals_stored(ops, "cpu", B, T, Hqk, Hv, K, V, dtype, cu=cu, wrap=guarded, h0_std=0.1)
+
+
 def test_chunk_backward_without_initial_state(ops):
     P.check_chunk(ops, "cpu", 1, 70, 1, 1, 64, 64, F32, backward=True, with_h0=False, wrap=guarded)
 

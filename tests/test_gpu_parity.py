@@ -63,6 +63,7 @@ CHUNK_CASES = [
     (BF, 2, 130, 4, 16, 128, 128, True, None),
     (BF, 1, 600, 1, 2, 64, 64, False, [0, 64, 65, 130, 258, 300, 450, 599, 600]),
     (F32, 8, 70, 1, 2, 64, 64, True, None),
+    (F32, 1, 1024, 2, 4, 128, 128, True, None),                  # fp32 with grouped heads over many chunks
 ]
 
 
@@ -80,6 +81,82 @@ def test_chunk_backward(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu):
 
 def test_chunk_backward_without_initial_state(ops):
     P.check_chunk(ops, "cuda", 1, 200, 2, 2, 128, 128, BF, backward=True, with_h0=False)
+
+
+def test_chunk_backward_wide_value_heads_group_of_four_slow_decay(ops):
+    """Head shape of BASELINE config 4 (d_k 128, d_v 256, four value heads per q/k head) with its decay recipe
+    (A_log ~ U(log 0.5, log 2), dt_bias ~ U(-6, -4): slow forgetting), forward and backward against the oracle."""
+    print("chunk bwd bf16 B1 T512 Hqk1 Hv4 K128 V256 slow decay", flush=True)
+    P.check_chunk(ops, "cuda", 1, 512, 1, 4, 128, 256, BF, backward=True, a_log=(0.5, 2.0), dt_bias=(-6.0, -4.0))
+
+
+@pytest.mark.parametrize("B,T,H,K,V,l2,cu,heads", [
+    # rows of the reference's own table (test_chunk_gated_delta_rule.py:116-140) with its input recipe (:158-175)
+    (1, 128, 8, 128, 128, False, None, 2),
+    (1, 1024, 64, 128, 128, True, None, 2),
+    (1, 1121, 16, 128, 128, True, [0, 112, 209, 240, 281, 489, 523, 566, 689, 721, 785, 837, 985, 1071, 1121], 2),
+    (21, 195, 32, 128, 128, True, None, 1),
+    (1, 160, 32, 128, 128, True, None, 2),
+    (1, 4608, 2, 128, 128, True, None, 2),
+    (1, 4608, 32, 128, 128, True, None, 1),
+    (1, 32832, 32, 128, 128, True, [0, 14012, 26600, 32766, 32832], 1),
+])
+def test_chunk_reference_test_table_and_recipe(ops, B, T, H, K, V, l2, cu, heads):
+    print(f"chunk reference recipe B{B} T{T} H{H} K{K} V{V} l2={l2} varlen={cu is not None}", flush=True)
+    P.check_chunk_reference_recipe(ops, "cuda", B, T, H, K, V, l2, cu=cu, oracle_heads=heads)
+
+
+@pytest.mark.parametrize("dtype,B,T,Hqk,Hv,K,V,l2,cu", [
+    (BF, 2, 300, 2, 4, 128, 128, True, None),
+    (BF, 1, 1121, 2, 2, 128, 128, True, [0, 112, 209, 240, 281, 489, 523, 566, 689, 721, 785, 837, 985, 1071, 1121]),
+    (BF, 1, 256, 1, 4, 128, 256, True, None),
+    (BF, 1, 200, 2, 2, 64, 64, False, None),
+    (F32, 1, 200, 1, 2, 128, 128, True, None),
+])
+def test_chunk_backward_recompute_mode_equals_stored_mode(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu):
+    print(f"chunk recompute vs stored {dtype} B{B} T{T} Hqk{Hqk} Hv{Hv} K{K} V{V}", flush=True)
+    P.check_chunk_recompute_equals_stored(ops, "cuda", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu)
+
+
+def test_chunk_backward_stored_mode_against_oracle(ops):
+    P.check_chunk(ops, "cuda", 2, 200, 2, 4, 128, 128, BF, backward=True, skip_recompute=True)
+
+
+def test_chunk_beta_in_float32_and_in_the_activation_dtype(ops):
+    """beta is read in its own dtype: bf16 in place (the layer's), anything else as float32; dbeta comes back in it."""
+    x = P.gdn_inputs(1, 200, 2, 4, 128, 128, BF, seed=5)
+    d = {n: t.cuda() for n, t in x.items()}
+    outs = []
+    for bdt in (BF, F32):
+        L = {n: d[n].clone().requires_grad_(True) for n in ("q", "k", "v", "g")}
+        beta = d["beta"].to(bdt).clone().detach().requires_grad_(True)
+        o, _ = ops.chunk_gated_delta_rule(L["q"], L["k"], L["v"], L["g"], beta, use_qk_l2norm_in_kernel=True)
+        (o.float() * d["do"].float()).sum().backward()
+        assert beta.grad.dtype == bdt
+        outs.append((o, beta.grad, L["q"].grad))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][2], outs[1][2])   # same values of beta
+    assert torch.equal(outs[0][1], outs[1][1].to(BF))
+
+
+def test_chunk_rejects_key_width_256(ops):
+    """The chunk kernels hold K in {64, 128} (the reference allows up to 256, chunk_delta_h.py:259): a clean error."""
+    q = torch.randn(1, 64, 1, 256, device="cuda", dtype=BF)
+    g, b = -torch.rand(1, 64, 1, device="cuda"), torch.rand(1, 64, 1, device="cuda")
+    with pytest.raises(ValueError, match="unsupported size"):
+        ops.chunk_gated_delta_rule(q, q, q, g, b)
+
+
+def test_chunk_under_autocast_keeps_dtypes(ops):
+    """custom_fwd / custom_bwd: under torch.autocast the operator still computes in the dtype of its inputs."""
+    x = P.gdn_inputs(1, 130, 1, 2, 64, 64, F32, seed=2)
+    d = {n: t.cuda() for n, t in x.items()}
+    L = {n: d[n].clone().requires_grad_(True) for n in ("q", "k", "v", "g", "beta")}
+    o0, _ = ops.chunk_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], use_qk_l2norm_in_kernel=True)
+    with torch.autocast("cuda", dtype=BF):
+        o, _ = ops.chunk_gated_delta_rule(L["q"], L["k"], L["v"], L["g"], L["beta"], use_qk_l2norm_in_kernel=True)
+        (o * d["do"]).sum().backward()
+    assert o.dtype == F32 and torch.equal(o, o0)
+    assert all(L[n].grad.dtype == F32 for n in L)
 
 
 @pytest.mark.parametrize("dtype,B,T,D,W,cu", [
@@ -160,7 +237,8 @@ def test_fused_norm_rejects_other_head_dims(ops):
     v = torch.randn(1, 64, 1, 256, device="cuda", dtype=BF)
     g, b = -torch.rand(1, 64, 1, device="cuda"), torch.rand(1, 64, 1, device="cuda")
     with pytest.raises(ValueError):
-        ops.chunk_gated_delta_rule_norm(q, q, v, g, b, torch.randn_like(v), torch.ones(256, device="cuda", dtype=BF))
+        ops.chunk_gated_delta_rule_norm(q, q, v, g, b, torch.randn_like(v), torch.ones(256, device="cuda", dtype=BF),
+                                        in_output_kernel=True)
 
 
 def test_chunk_rejects_bad_strides(ops):
@@ -178,7 +256,7 @@ def test_chunk_rejects_bad_strides(ops):
     rc = lib.gdn_chunk_fwd_strided(q.data_ptr(), k.data_ptr(), v.data_ptr(), 3 * K + 4, 3 * K + 4, 3 * K + 4,
                                    g.data_ptr(), beta.data_ptr(), None, None, o.data_ptr(), None,
                                    ws.data_ptr() + (-ws.data_ptr()) % 256, ws.numel() - 256, B, T, B, H, H, K, K, 0.125, 0,
-                                   1, lib.stream())
+                                   1, 0, lib.stream())
     assert rc == -6
 
 
