@@ -158,14 +158,25 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
       commit(0, 0);
 #pragma unroll
       for (int j = 1; j <= DEPTH; ++j) issue(imin(j, nchunks - 1), j % DEPTH);
-      for (int s0 = 0;; s0 += DEPTH) {
+      // The loop leaves only at the end of a whole round of register sets: an exit in the middle of the round would be
+      // one more way into the code that follows it, one on which fewer loads are in flight, and the waits before the
+      // LDS writes (counted by the compiler over all ways in) would then also wait for the younger set.
+      int s0 = 0;
+      for (; s0 + DEPTH <= nchunks; s0 += DEPTH) {
 #pragma unroll
         for (int u = 0; u < DEPTH; ++u) {
           const int st = s0 + u;
-          if (st >= nchunks) return;
           GDN_LDS_BARRIER();                // (A) step st staged; the other stage (step st-1) is free
           commit((u + 1) % DEPTH, (st + 1) & 1);
           issue(imin(st + 1 + DEPTH, nchunks - 1), (u + 1) % DEPTH);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < DEPTH - 1; ++u) {   // the steps left over: their barriers, and the stage the next one reads
+        const int st = s0 + u;
+        if (st < nchunks) {
+          GDN_LDS_BARRIER();
+          commit((u + 1) % DEPTH, (st + 1) & 1);
         }
       }
     } else {
@@ -307,18 +318,22 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
 //   dQ, dK, dv leave as 16-byte row pieces.
 // ---------------------------------------------------------------------------------------------
 template <typename T, int DK> struct BwdLocalSmem {
-  // one stage, in elements: [v_new x2 | dV' x2] shared tiles, raw dO [64][32], [S | dS'] per wave, raw V [64][32]
-  // (the raw blocks as SwizzledTile<T, 32>)
-  static constexpr int st_doraw = 4 * 1024, st_priv = 6 * 1024, st_vraw = st_priv + 4 * 2048, stage_elems = st_vraw + 64 * 32;
-  // epilogue, stage that idles during the last block: K tiles [K/32][2] | the Q^T tiles [2] of each wave
-  static constexpr int ea_q = 8 * 1024;
-  // epilogue, other stage: dW tiles [2][K/32] (later the store patches) | D-form tiles [4] | T-form tiles [4]
-  static constexpr int eb_d = 8 * 1024, eb_t = 12 * 1024;
-  static constexpr int off_tm = 2 * stage_elems * (int)sizeof(T);             // Tm tiles [2][2], whole kernel
+  // main loop, in elements:
+  //   sh   [2 stages][v_new x2 | dV' x2]      shared fragment tiles of one 32-column V block, one block ahead
+  //   raw  [2 buffers][dO [64][64] | V [64][64]]  raw rows of a PAIR of V blocks (SwizzledTile<T, 64>): 128-byte row
+  //        pieces, i.e. whole lines of dO and V (32-column blocks would use half of every line they touch and fetch
+  //        it twice), one pair ahead
+  //   priv [4 waves][S | dS']                 per wave, single: a wave takes its tiles into registers at the top of a
+  //        block and requests the next block's right behind
+  static constexpr int sh = 0, raw = 2 * 4096, raw_elems = 2 * 64 * 64, priv = raw + 2 * raw_elems, main_elems = priv + 4 * 2048;
+  // epilogue: K tiles [K/32][2] in the raw buffer that idles during the last block, the Q^T tiles [2] of each wave in
+  // its priv slot (later the (beta dM) D-form tiles); then dW tiles [2][K/32] (later the store patches) in the other raw
+  // buffer, D-form tiles [4] and T-form tiles [4] in the two shared stages
+  static constexpr int off_tm = main_elems * (int)sizeof(T);                 // Tm tiles [2][2], whole kernel
   static constexpr int off_row = off_tm + 4 * 1024 * (int)sizeof(T);
   static constexpr int bytes = off_row + (5 * 64 + 5 * 256 + 8) * 4;   // 5 row vectors, 5 per-wave row-sum arrays
-  static_assert(stage_elems == 16 * 1024, "the epilogue layout fills a stage exactly");
-  static_assert(Patch<T>::kElems <= 2048, "store patches fit");
+  static_assert(main_elems == 32 * 1024, "as large as two former stages");
+  static_assert(4 * Patch<T>::kElems <= raw_elems && 2 * (DK / 32) * 1024 <= raw_elems, "epilogue tenants fit");
 };
 
 template <typename T, int DK>
@@ -365,53 +380,61 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   const int h = hq * grp + hh;
   const int64_t ch = (int64_t)blockIdx.x * Hv + h;
 
-  // stage `buf` <- operands of V block `vblk`; every load moves 64 x 16 bytes, lane l's piece landing at +16 l
-  auto issue = [&](int vblk, int buf) {
-    T* st = stage0 + buf * SM::stage_elems;
+  // every load below moves 64 x 16 bytes, lane l's piece landing at +16 l
+  auto issue_shared = [&](int vblk) {                // v_new and dV' tiles of V block `vblk`
+    T* st = stage0 + SM::sh + (vblk & 1) * 4096;
     const int64_t t2 = (ch * nblk + vblk) * 2;
 #pragma unroll
-    for (int j = 0; j < 4 * KG / 4; ++j) {           // shared tiles: k-group pieces dealt round-robin to the waves
+    for (int j = 0; j < 4 * KG / 4; ++j) {           // k-group pieces dealt round-robin to the waves
       const int piece = 4 * j + wave, tile = piece / KG, g = piece % KG;
       const T* src = tile < 2 ? vf + (t2 + tile) * 1024 : dvf + (t2 + tile - 2) * 1024;
       load16_to_lds(src + (g * 64 + lane) * VEC, st + tile * 1024 + g * 64 * VEC);
     }
-#pragma unroll
-    for (int j = 0; j < (int)sizeof(T) / 2; ++j) {   // raw dO and V blocks [64][32], rows past the end repeat the last row
-      constexpr int LPR = 32 / VEC, RPP = 64 / LPR;  // lanes per row, rows per piece
-      const int piece = 4 * j + wave, row = piece * RPP + lane / LPR, cc = SwizzledTile<T, 32>::pos(row, lane % LPR);
-      const int64_t tok = tok0 + imin(row, nvalid - 1), col = (int64_t)h * V + 32 * vblk + cc * VEC;
-      load16_to_lds(dO + tok * Hv * V + col, st + SM::st_doraw + piece * 64 * VEC);
-      load16_to_lds(v + tok * ts.v + col, st + SM::st_vraw + piece * 64 * VEC);
-    }
+  };
+  auto issue_priv = [&](int vblk) {                  // this wave's S and dS' tiles of V block `vblk`
     if (has_k) {
+      T* pv = stage0 + SM::priv + wave * 2048;
       const int64_t tile = ((ch * nblk + vblk) * NKT + cj) * 1024;
 #pragma unroll
       for (int g = 0; g < KG; ++g) {
-        load16_to_lds(hf + tile + (g * 64 + lane) * VEC, st + SM::st_priv + wave * 2048 + g * 64 * VEC);
-        load16_to_lds(dhf + tile + (g * 64 + lane) * VEC, st + SM::st_priv + wave * 2048 + 1024 + g * 64 * VEC);
+        load16_to_lds(hf + tile + (g * 64 + lane) * VEC, pv + g * 64 * VEC);
+        load16_to_lds(dhf + tile + (g * 64 + lane) * VEC, pv + 1024 + g * 64 * VEC);
       }
     }
   };
-  // stage `buf` <- epilogue operands: all K tiles of the chunk, this wave's 32 columns of Q^T (both in fragment order)
-  auto issue_epilogue = [&](int buf) {
-    T* st = stage0 + buf * SM::stage_elems;
+  auto issue_raw = [&](int pair) {                   // dO and V rows of V blocks 2 pair, 2 pair + 1; rows past the end repeat the last
+    T* rb = stage0 + SM::raw + (pair & 1) * SM::raw_elems;
+    constexpr int LPR = 64 / VEC, RPP = 64 / LPR;    // lanes per row, rows per 64-lane piece
+#pragma unroll
+    for (int j = 0; j < 64 / RPP / 4; ++j) {
+      const int piece = 4 * j + wave, row = piece * RPP + lane / LPR, cc = SwizzledTile<T, 64>::pos(row, lane % LPR);
+      const int64_t tok = tok0 + imin(row, nvalid - 1), col = (int64_t)h * V + 64 * pair + cc * VEC;
+      load16_to_lds(dO + tok * Hv * V + col, rb + piece * 64 * VEC);
+      load16_to_lds(v + tok * ts.v + col, rb + 64 * 64 + piece * 64 * VEC);
+    }
+  };
+  // epilogue operands: all K tiles of the chunk into raw buffer `rbuf`, this wave's 32 columns of Q^T into its priv slot
+  auto issue_epilogue = [&](int rbuf) {
+    T* kt = stage0 + SM::raw + rbuf * SM::raw_elems;
 #pragma unroll
     for (int j = 0; j < 2 * NKT * KG / 4; ++j) {
       const int piece = 4 * j + wave;
       load16_to_lds(kaf + ((int64_t)blockIdx.x * Hqk + hq) * (NKT * 2048) + (piece * 64 + lane) * VEC,
-                    st + piece * 64 * VEC);
+                    kt + piece * 64 * VEC);
     }
     if (has_k) {
 #pragma unroll
       for (int piece = 0; piece < 2 * KG; ++piece)
         load16_to_lds(qtf + (((int64_t)blockIdx.x * Hqk + hq) * NKT + cj) * 2048 + (piece * 64 + lane) * VEC,
-                      st + SM::ea_q + wave * 2048 + piece * 64 * VEC);
+                      stage0 + SM::priv + wave * 2048 + piece * 64 * VEC);
     }
   };
 #pragma unroll
   for (int j = 0; j < KG; ++j)                        // Tm tiles, fragment order
     load16_to_lds(Ai + ch * 4096 + ((4 * j + wave) * 64 + lane) * VEC, TmF + (4 * j + wave) * 64 * VEC);
-  issue(0, 0);
+  issue_shared(0);
+  issue_priv(0);
+  issue_raw(0);
 
   if (tid < 64) {   // the row vectors: all requests first, the same ones on every path
     const int tc = imin(tid, nvalid - 1);
@@ -445,28 +468,37 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   float sds = 0.f;
 
   for (int vblk = 0; vblk < nblk; ++vblk) {
-    const T* st = stage0 + (vblk & 1) * SM::stage_elems;
+    const T* st = stage0 + SM::sh + (vblk & 1) * 4096;
+    const T* rb = stage0 + SM::raw + ((vblk >> 1) & 1) * SM::raw_elems;
+    const int rk0 = 32 * (vblk & 1);         // this block's columns inside the raw pair
     if (vblk > 0) {
-      GDN_WAIT_VMEM();       // this wave's share of the stage has landed ...
-      GDN_LDS_BARRIER();     // ... and so has everybody else's; the other stage is no longer read
+      GDN_WAIT_VMEM();       // this wave's share of the block's operands has landed ...
+      GDN_LDS_BARRIER();     // ... and so has everybody else's; the other stage and raw buffer are no longer read
     }
-    if (vblk + 1 < nblk) issue(vblk + 1, (vblk + 1) & 1); else issue_epilogue((vblk + 1) & 1);
     // Operands are taken one after the other so that few fragments are live at a time; tile indices that depend on
     // the wave are compared against loop constants (fragments indexed at run time would go to scratch).
     AccB<T> f, Sf, dSf, dOt[2];
     if (has_k) {                             // (lane <-> K column, registers <-> V)
-      f.load(st + SM::st_priv + wave * 2048);
+      f.load(stage0 + SM::priv + wave * 2048);
       const f32x16 sv = mfma_transpose<T>(f, id);
       Sf.pack(sv);
-      f.load(st + SM::st_priv + wave * 2048 + 1024);
+      f.load(stage0 + SM::priv + wave * 2048 + 1024);
       const f32x16 dsv = mfma_transpose<T>(f, id);
       dSf.pack(dsv);
 #pragma unroll
       for (int r = 0; r < 16; ++r) sds += sv[r] * dsv[r];
     }
+    GDN_WAVE_LDS_SYNC();     // the wave's priv slot is in registers: the next tenant may be requested
+    if (vblk + 1 < nblk) {
+      issue_shared(vblk + 1);
+      issue_priv(vblk + 1);
+      if ((vblk & 1) == 0 && vblk + 2 < nblk) issue_raw((vblk >> 1) + 1);   // its buffer was last read in block vblk - 1
+    } else {
+      issue_epilogue(((vblk >> 1) + 1) & 1);
+    }
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {         // (lane <-> token, registers <-> V) from here on; dO rows have it already
-      SwizzledTile<T, 32>::frags(dOt[ri], st + SM::st_doraw, 32 * ri + l32, 0);
+      SwizzledTile<T, 64>::frags(dOt[ri], rb, 32 * ri + l32, rk0);
       if (32 * ri + l32 >= nvalid) {
 #pragma unroll
         for (int g = 0; g < KG; ++g) dOt[ri].f[g] = u32x4{0u, 0u, 0u, 0u};
@@ -490,7 +522,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       dVt.pack(mfma_transpose<T>(f, id));
       if (has_k) mma32_ff<T>(dWa[ri], dVt, Sf);
       if (lower && ri == ti) {
-        SwizzledTile<T, 32>::frags(f, st + SM::st_vraw, 32 * tj + l32, 0);
+        SwizzledTile<T, 64>::frags(f, rb + 64 * 64, 32 * tj + l32, rk0);
         mma32_ff<T>(a2, dVt, f);
       }
     }
@@ -516,12 +548,13 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   }
   sds = wave_sum(sds);
   if (lane == 0) wsum[wave] = sds;
-  T* EA = stage0 + (nblk & 1) * SM::stage_elems;        // K tiles | Q columns; later (beta dM) D-form tiles over Q
-  T* EB = stage0 + ((nblk - 1) & 1) * SM::stage_elems;  // dW tiles | D-form tiles | T-form tiles
-  T* dWF = EB;
-  T* tileD = EB + SM::eb_d;
-  T* tileT = EB + SM::eb_t;
-  T* dMD = EA + SM::ea_q;
+  const int rlast = ((nblk - 1) >> 1) & 1;               // raw buffer of the last pair
+  T* EA = stage0 + SM::raw + (rlast ^ 1) * SM::raw_elems;   // K tiles
+  T* EQ = stage0 + SM::priv;                             // Q columns per wave; later (beta dM) D-form tiles
+  T* dWF = stage0 + SM::raw + rlast * SM::raw_elems;     // dW tiles, later the store patches
+  T* tileD = stage0 + SM::sh;
+  T* tileT = stage0 + SM::sh + 4096;
+  T* dMD = EQ;
   GDN_WAIT_VMEM();
   GDN_LDS_BARRIER();   // the epilogue operands have landed; the last block's stage is consumed
 
@@ -533,7 +566,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       AccB<T> f;
       f.load(EA + (2 * cj + t) * 1024);
       KTf[t].pack(mfma_transpose<T>(f, id));
-      QTf[t].load(EA + SM::ea_q + wave * 2048 + t * 1024);
+      QTf[t].load(EQ + wave * 2048 + t * 1024);
     }
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {         // dW = -(dV' S^T): B operand of P in registers, A operand of a1 to LDS

@@ -319,13 +319,15 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
 // PRE: two images of K, rows scaled by -beta e^G and by e^{G_last-G} on their way into LDS.  Whether they fit is
 // decided for the variant with output waves (FUSE) and two slabs per workgroup, and every other variant of the same
 // element type and key width follows, so that all of them round alike.
+// output waves per slab: a workgroup with a single slab has room for two, one per 32-token block of the chunk
+template <int NW> struct StateOutWaves { static constexpr int value = NW == 1 ? 2 : 1; };
 template <typename T, int DK, int NW, int STAGES, bool FUSE> struct StatePre {
-  static constexpr int x_elems = 2 * DK * 32 + 2 * 2048 + Patch<T>::kElems;
+  static constexpr int x_elems = 2 * DK * 32 + 2 * 2048 + StateOutWaves<NW>::value * Patch<T>::kElems;
   static constexpr bool value = STAGES * ((2 * 64 * DK + 3 * 1024 + 64 * 32 * NW + (FUSE ? 64 * DK + 3 * 1024 : 0)) * (int)sizeof(T) + 68 * 4) +
                                     (FUSE ? NW * x_elems * (int)sizeof(T) : 0) <= 160 * 1024;
 };
 template <typename T, int DK, int NW, int STAGES, bool OUT, bool PRE_> struct StateSmem {
-  static constexpr int x_elems = 2 * DK * 32 + 2 * 2048 + Patch<T>::kElems;
+  static constexpr int x_elems = 2 * DK * 32 + 2 * 2048 + StateOutWaves<NW>::value * Patch<T>::kElems;
   static constexpr bool PRE = PRE_;
   // one stage, in elements of T
   static constexpr int off_k = 0;                                   // K image(s) [K/32][2] tiles
@@ -337,7 +339,7 @@ template <typename T, int DK, int NW, int STAGES, bool OUT, bool PRE_> struct St
   // rows: scale e^G [64], G_last; without PRE also e^{G_last-G} [64], beta e^G [64], beta [64]
   static constexpr int stage = off_row + (PRE ? 68 : 260) * 4;   // a multiple of 16 bytes, like the offset of every row vector
   static_assert(stage % 16 == 0, "stages keep 16-byte alignment");
-  static constexpr int off_x = STAGES * stage;                      // OUT: per slab S [2][DK*32], V' [2][2048], store patch
+  static constexpr int off_x = STAGES * stage;                      // OUT: per slab S [2][DK*32], V' [2][2048], a store patch per output wave
   static constexpr int bytes = off_x + (OUT ? NW * x_elems * (int)sizeof(T) : 0);
   static_assert(bytes <= 160 * 1024, "one CU's LDS");
 };
@@ -347,7 +349,7 @@ template <typename T, int DK, int NW, int STAGES, bool OUT, bool PRE_> struct St
 template <int PIECES, int NT> struct Deal { static constexpr int kPer = (PIECES + NT - 1) / NT; };
 
 template <typename T, int DK, int NW, int NL, int STAGES, bool OUT, bool PRE_>
-__global__ __launch_bounds__(64 * (NW + (OUT ? NW : 0) + NL)) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 2 : 1)
+__global__ __launch_bounds__(64 * (NW + (OUT ? NW * StateOutWaves<NW>::value : 0) + NL)) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 2 : 1)
 void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, const T* __restrict__ ai,
                         const T* __restrict__ aqf, const T* __restrict__ v, const float* __restrict__ G,
                         const void* __restrict__ beta, int beta_same, const float* __restrict__ h0, float* __restrict__ ht,
@@ -355,7 +357,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
                         const int* __restrict__ chunk_offsets, int T_len, int Hqk, int Hv, int V, float scale,
                         int64_t v_stride) {
   using SM = StateSmem<T, DK, NW, STAGES, OUT, PRE_>;
-  constexpr int NT = 64 * NL, VEC = Elem<T>::kVec, NKT = DK / 32, NWO = OUT ? NW : 0;
+  constexpr int NT = 64 * NL, VEC = Elem<T>::kVec, NKT = DK / 32, OS = StateOutWaves<NW>::value, NWO = OUT ? NW * OS : 0;
   constexpr int PK = 64 * DK / VEC, PTM = 3 * 1024 / VEC, PV = 64 * 32 * NW / VEC, VPR = 32 * NW / VEC;
   constexpr int CK = Deal<PK, NT>::kPer, CTM = Deal<PTM, NT>::kPer, CV = Deal<PV, NT>::kPer;
   static_assert(STAGES == 1 || STAGES == 2, "one or two LDS stages");
@@ -492,14 +494,25 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
       commit(0, 0);
 #pragma unroll
       for (int j = 1; j <= DEPTH; ++j) issue(imin(j, nchunks - 1), j % DEPTH);
-      for (int c0 = 0;; c0 += DEPTH) {
+      // The loop leaves only at the end of a whole round of register sets: an exit in the middle of the round would be
+      // one more way into the code that follows it, one on which fewer loads are in flight, and the waits before the
+      // LDS writes (counted by the compiler over all ways in) would then also wait for the younger set.
+      int c0 = 0;
+      for (; c0 + DEPTH <= nsteps; c0 += DEPTH) {
 #pragma unroll
         for (int u = 0; u < DEPTH; ++u) {
           const int c = c0 + u;
-          if (c >= nsteps) return;
           GDN_LDS_BARRIER();                // (A) chunk c staged; the other stage (chunk c-1) is free
           commit((u + 1) % DEPTH, (c + 1) & 1);
           issue(imin(c + 1 + DEPTH, nchunks - 1), (u + 1) % DEPTH);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < DEPTH - 1; ++u) {   // the steps left over: their barriers, and the stage the next one reads
+        const int c = c0 + u;
+        if (c < nsteps) {
+          GDN_LDS_BARRIER();
+          commit((u + 1) % DEPTH, (c + 1) & 1);
         }
       }
     } else {
@@ -516,10 +529,13 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
   if constexpr (OUT) {
     if (wave >= NW) {
       // ================= output waves: O of the slab's 32 columns, one step behind the compute wave =================
-      const int w = wave - NW;
+      // OS == 2: wave `hw` of the slab's two owns the chunk's 32-token block hw (and that share of the stores for the
+      // backward pass); OS == 1: one wave does both blocks.  Either way every row is accumulated by the same
+      // instructions in the same order.
+      const int w = (wave - NW) / OS, hw = (wave - NW) % OS;
       const int vblk = blockIdx.y * NW + w, v0 = 32 * vblk;
       T* xs = reinterpret_cast<T*>(gdn_smem + SM::off_x) + w * SM::x_elems;
-      T* patch = xs + 2 * DK * 32 + 2 * 2048;
+      T* patch = xs + 2 * DK * 32 + 2 * 2048 + hw * Patch<T>::kElems;
       IdentityFrag<T> id;
       id.init();
       f32x16 oa[2];
@@ -529,23 +545,33 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
         GDN_LDS_BARRIER();                    // (A)
         if (c > 0) {                          // finish chunk c-1: + Aq V', rows out
           const T* vx = xs + 2 * DK * 32 + ((c - 1) & 1) * 2048;
-          AccB<T> Vb[2];
-          Vb[0].load(vx);
-          Vb[1].load(vx + 1024);
-          if (vf != nullptr) {   // v_new of chunk c-1, for the backward pass
-            const int64_t tile0 = ((chunk_base + c - 1) * Hv + h) * (V / 32) + vblk;
-            Vb[0].store_stream(vf + (tile0 * 2 + 0) * 1024);
-            Vb[1].store_stream(vf + (tile0 * 2 + 1) * 1024);
-          }
-          mma32_ff<T>(oa[0], Af[0], Vb[0]);
-          mma32_ff<T>(oa[1], Af[1], Vb[0]);
-          mma32_ff<T>(oa[1], Af[2], Vb[1]);
+          const int64_t tile0 = ((chunk_base + c - 1) * Hv + h) * (V / 32) + vblk;
           const int64_t tok0 = bos + (int64_t)(c - 1) * kChunk;
           const int nvalid = imin(kChunk, len - (c - 1) * kChunk);
           T* og = o + (tok0 * Hv + h) * V + v0;
+          AccB<T> Vb[2];
+          Vb[0].load(vx);
+          if (OS == 1 || hw == 1) Vb[1].load(vx + 1024);
+          if constexpr (OS == 2) {
+            if (vf != nullptr) {                          // v_new of chunk c-1, for the backward pass
+              if (hw == 0) Vb[0].store_stream(vf + (tile0 * 2 + 0) * 1024);
+              else Vb[1].store_stream(vf + (tile0 * 2 + 1) * 1024);
+            }
+            mma32_ff<T>(oa[0], Af[0], Vb[0]);            // hw == 0: Aq tile (0,0); hw == 1: tile (1,0) ...
+            if (hw == 1) mma32_ff<T>(oa[0], Af[1], Vb[1]);   // ... and (1,1)
+            acc_store_rows<T, false>(oa[0], id, patch, og + (int64_t)32 * hw * Hv * V, (int64_t)Hv * V, nvalid - 32 * hw);
+          } else {
+            if (vf != nullptr) {
+              Vb[0].store_stream(vf + (tile0 * 2 + 0) * 1024);
+              Vb[1].store_stream(vf + (tile0 * 2 + 1) * 1024);
+            }
+            mma32_ff<T>(oa[0], Af[0], Vb[0]);
+            mma32_ff<T>(oa[1], Af[1], Vb[0]);
+            mma32_ff<T>(oa[1], Af[2], Vb[1]);
 #pragma unroll
-          for (int ri = 0; ri < 2; ++ri)
-            acc_store_rows<T, false>(oa[ri], id, patch, og + (int64_t)32 * ri * Hv * V, (int64_t)Hv * V, nvalid - 32 * ri);
+            for (int ri = 0; ri < 2; ++ri)
+              acc_store_rows<T, false>(oa[ri], id, patch, og + (int64_t)32 * ri * Hv * V, (int64_t)Hv * V, nvalid - 32 * ri);
+          }
         }
         if (c < nchunks) {                    // start chunk c: scale e^G . (Q S), and its Aq tiles into registers
           const T* st = reinterpret_cast<const T*>(gdn_smem + buf * SM::stage);
@@ -557,19 +583,32 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
           for (int kt = 0; kt < NKT; ++kt) {
             AccB<T> Sb, Qf;
             Sb.load(sx + kt * 1024);
-            if (hf != nullptr)   // the state before chunk c, for the backward pass
+            if (hf != nullptr && (OS == 1 || (kt & 1) == hw))   // the state before chunk c, for the backward pass
               Sb.store_stream(hf + ((((chunk_base + c) * Hv + h) * (V / 32) + vblk) * NKT + kt) * 1024);
+            if constexpr (OS == 2) {
+              Qf.load_t(st + SM::off_q + (kt * 2 + hw) * 1024);   // Q tile (token block hw, K block kt)
+              mma32_ff<T>(oa[0], Qf, Sb);
+            } else {
 #pragma unroll
-            for (int ri = 0; ri < 2; ++ri) {
-              Qf.load_t(st + SM::off_q + (kt * 2 + ri) * 1024);   // Q tile (token block ri, K block kt)
-              mma32_ff<T>(oa[ri], Qf, Sb);
+              for (int ri = 0; ri < 2; ++ri) {
+                Qf.load_t(st + SM::off_q + (kt * 2 + ri) * 1024);   // Q tile (token block ri, K block kt)
+                mma32_ff<T>(oa[ri], Qf, Sb);
+              }
             }
           }
-          const f32x16 e0 = rows_ld(row, 0), e1 = rows_ld(row, 32);
+          if constexpr (OS == 2) {
+            const f32x16 e0 = rows_ld(row, 32 * hw);
 #pragma unroll
-          for (int r = 0; r < 16; ++r) { oa[0][r] *= e0[r]; oa[1][r] *= e1[r]; }
+            for (int r = 0; r < 16; ++r) oa[0][r] *= e0[r];
+            Af[0].load_t(st + SM::off_aq + hw * 1024);   // (lane <-> row i, registers <-> column j)
+            if (hw == 1) Af[1].load_t(st + SM::off_aq + 2 * 1024);
+          } else {
+            const f32x16 e0 = rows_ld(row, 0), e1 = rows_ld(row, 32);
 #pragma unroll
-          for (int t = 0; t < 3; ++t) Af[t].load_t(st + SM::off_aq + t * 1024);   // (lane <-> row i, registers <-> column j)
+            for (int r = 0; r < 16; ++r) { oa[0][r] *= e0[r]; oa[1][r] *= e1[r]; }
+#pragma unroll
+            for (int t = 0; t < 3; ++t) Af[t].load_t(st + SM::off_aq + t * 1024);   // (lane <-> row i, registers <-> column j)
+          }
           if (STAGES == 1 && c + 1 < nsteps) GDN_LDS_BARRIER();   // (B)
         }
       }
@@ -940,7 +979,7 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   if constexpr (FUSE) {
     if (fuse) {
       if (int e = launch_state(chunk_state_kernel<T, DK, NWS, NLS, STAGES, true, PRE>,
-                               StateSmem<T, DK, NWS, STAGES, true, PRE>::bytes, 2 * NWS + NLS, (T*)o))
+                               StateSmem<T, DK, NWS, STAGES, true, PRE>::bytes, NWS * (1 + StateOutWaves<NWS>::value) + NLS, (T*)o))
         return e;
       return (int)hipGetLastError();
     }
