@@ -47,3 +47,22 @@ def packed_lengths(n_seq=24, total=32768, lo=64, hi=4096, seed=0):
     for x in lens:
         cu.append(cu[-1] + x)
     return cu
+
+
+def kda_inputs(B, T, H, K, V, dtype, seed=0, N=None, a_log=(1.0, 16.0), dt_bias=(-4.0, -2.0), h0_std=0.02):
+    """Inputs of the KDA operator as its layer hands them over (mindspeed_mm/fsdp/models/kimi_k3/
+    modeling_kimi_linear.py:584-596, 665-671): q, k, v ~ N(0,1); the raw gate input g ~ N(0,1) per key channel with
+    A_log ~ U(log a0, log a1) per head and dt_bias ~ U(b0, b1) per head and channel; beta raw ~ N(0,1) (the
+    operator applies the sigmoid); h0, dht ~ N(0, h0_std) fp32 in [N,H,K,V]; do ~ N(0,1)."""
+    gen = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=gen)
+    q, k, v, g = r(B, T, H, K), r(B, T, H, K), r(B, T, H, V), r(B, T, H, K)
+    beta = r(B, T, H)
+    A_log = torch.empty(H).uniform_(math.log(a_log[0]), math.log(a_log[1]), generator=gen)
+    bias = torch.empty(H * K).uniform_(dt_bias[0], dt_bias[1], generator=gen)
+    n = N if N is not None else B
+    h0 = h0_std * r(n, H, K, V)
+    do = r(B, T, H, V)
+    dht = h0_std * r(n, H, K, V)
+    return dict(q=q.to(dtype), k=k.to(dtype), v=v.to(dtype), g=g.to(dtype), beta=beta.to(dtype), A_log=A_log,
+                dt_bias=bias, h0=h0, do=do.to(dtype), dht=dht)
