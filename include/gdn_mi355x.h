@@ -165,6 +165,27 @@ int gdn_gate_bwd_noalloc(const void* a, const void* b, const void* A_log, const 
                          const void* dbeta, void* da, void* db, float* dA_log, float* ddt_bias, int64_t tokens, int Hv,
                          int dtype, int param_dtype, void* stream);
 
+/* -------- KDA (Kimi delta attention): the delta rule with one decay per key channel ------------------
+ * replaces: chunk_kda (mindspeed_mm/fsdp/ops/kda/triton_ascend/chunk.py:215-407, the fused operator the layer calls at
+ * mindspeed_mm/fsdp/models/kimi_k3/modeling_kimi_linear.py:681-699) and its pure-PyTorch statement chunk_kda_naive
+ * (mindspeed_mm/fsdp/ops/kda/chunk_kda_naive.py:223-381; gate :76-104, chunk algebra :106-221).
+ * q, k, g [B,T,H,K], v, o [B,T,H,V], beta [B,T,H] (token-major, contiguous); q, k, v, o in `dtype` (0 fp32, 1 bf16),
+ * g in g_dtype and beta in beta_dtype (each 0 = fp32 or equal to dtype); A_log [H] and dt_bias [H*K] (or null) in fp32;
+ * initial_state, final_state [N,H,K,V] fp32 or null; cu_seqlens int64 [N+1] on the device or null (then N = B).
+ * use_gate: g is the raw gate input and the log decay is -e^{A_log} softplus(g + dt_bias), or, with has_lower_bound,
+ * lower_bound * sigmoid(e^{A_log} (g + dt_bias)); otherwise g is the log decay itself (<= 0).
+ * beta_sigmoid: beta <- sigmoid(beta), times 2 with allow_neg_eigval.  K in {64, 128}, V a multiple of 64.
+ * A workspace of gdn_kda_workspace_bytes(..., with_backward = 1, ...) bytes also keeps the chunk-local cumulative
+ * decay and 1/|q|, 1/|k|.  Returns 0, or -1 null argument, -2 shape, -3 unsupported K / V, -4 dtype, -5 workspace,
+ * -6 alignment. */
+int64_t gdn_kda_workspace_bytes(int B, int T, int N, int H, int K, int V, int with_backward, int dtype);
+
+int gdn_kda_fwd(const void* q, const void* k, const void* v, const void* g, const void* beta, const float* A_log,
+                const float* dt_bias, const float* initial_state, const int64_t* cu_seqlens, void* o,
+                float* final_state, void* workspace, int64_t workspace_bytes, int B, int T, int N, int H, int K, int V,
+                float scale, int use_qk_l2norm, int use_gate, int has_lower_bound, float lower_bound, int beta_sigmoid,
+                int allow_neg_eigval, int dtype, int g_dtype, int beta_dtype, void* stream);
+
 /* -------- per-kernel timing ------------------------------------------------------------------------
  * op-level counterpart of the reference's step profiler (mindspeed_mm/fsdp/tools/profiler.py:32-147).
  * While enabled, every kernel launch of this library is bracketed by HIP events on its stream (this mode

@@ -69,6 +69,48 @@ inline ChunkWorkspace chunk_workspace_layout(const ChunkDims& d, int elem_bytes)
   return w;
 }
 
+// KDA (one decay per key channel; q, k, v heads in equal number H): what its prep kernel leaves for the recurrence and
+// the output kernel.  The two K images carry the per-channel factors, so the recurrence itself only decays the rows
+// of the state by e^{G_last}.
+struct KdaWorkspace {
+  int64_t chunk_offsets;  // int32 [N+1]
+  int64_t rstd;           // f32 [2][chunks,H,64]   1/|q|, 1/|k| of the in-kernel l2 norm
+  int64_t bhat;           // f32 [tokens,H]         beta as the recurrence uses it (after the optional sigmoid)
+  int64_t dec;            // f32 [chunks,H,K]       e^{G_last}: decay of each key channel over the whole chunk
+  int64_t Ai;             // T [chunks,H,2,2]       Tm = (I + L)^-1 tiles
+  int64_t AQ;             // T [chunks,H,2,2]       scale tril(sum_d q_i k_j e^{G_i-G_j}) tiles
+  int64_t K1F;            // T [chunks,H,K/32,2]    rows -beta k . e^{G}
+  int64_t K2F;            // T [chunks,H,K/32,2]    rows k . e^{G_last-G}
+  int64_t QB;             // T [tokens,H,K]         rows scale q . e^{G}, row-major
+  int64_t VF;             // T [chunks,H,V/32,2]    v_new
+  int64_t HF;             // T [chunks,H,V/32,K/32] state before each chunk
+  int64_t fwd_bytes;
+  int64_t GC;             // f32 [chunks,H,64,K]    chunk-local cumulative log decay (kept for a backward pass)
+  int64_t total_bytes;
+};
+
+inline KdaWorkspace kda_workspace_layout(const ChunkDims& d, int elem_bytes) {
+  KdaWorkspace w;
+  int64_t off = 0;
+  auto take = [&](int64_t bytes) { int64_t o = off; off += align256(bytes); return o; };
+  const int64_t nc = d.max_chunks(), H = d.Hv;
+  w.chunk_offsets = take((int64_t)(d.N + 1) * 4);
+  w.rstd = take(2 * nc * 64 * H * 4);
+  w.bhat = take(d.tokens() * H * 4);
+  w.dec = take(nc * H * d.K * 4);
+  w.Ai = take(nc * 64 * H * 64 * elem_bytes);
+  w.AQ = take(nc * 64 * H * 64 * elem_bytes);
+  w.K1F = take(nc * 64 * H * d.K * elem_bytes);
+  w.K2F = take(nc * 64 * H * d.K * elem_bytes);
+  w.QB = take(d.tokens() * H * d.K * elem_bytes);
+  w.VF = take(nc * 64 * H * d.V * elem_bytes);
+  w.HF = take(nc * H * d.V * d.K * elem_bytes);
+  w.fwd_bytes = off;
+  w.GC = take(nc * 64 * H * d.K * 4);
+  w.total_bytes = off;
+  return w;
+}
+
 // The two sequential kernels give one compute wave a 32-column slab of the state.  What limits them is the rate at
 // which one CU gets its requests served (about 35 GB/s measured, loads and stores together), whatever the number of
 // slabs the workgroup serves, so when the whole problem has no more slabs than the device has CUs every slab gets a

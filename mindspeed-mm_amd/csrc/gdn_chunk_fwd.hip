@@ -97,6 +97,98 @@ __device__ __forceinline__ void tile_qk_finish(TileQK<T, DK>& t, T* lds, int ld,
   }
 }
 
+// (I + A)^-1 of a strictly lower triangular 64x64 matrix.  A arrives in As (fp32, leading dimension kLF; its upper
+// triangle is used as scratch), the inverse is left in Ti, which must arrive zeroed.  All four waves; the last thing
+// it does is a barrier.
+__device__ __forceinline__ void tril_inverse_64(float* As, float* Ti, int wave, int lane) {
+  // ---- phase 2a: invert the four 16x16 diagonal blocks by forward substitution (fp32) ----
+  if (lane < 16) {
+    const int o = 16 * wave, j = lane;
+    float tcol[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      float x = (i == j) ? 1.f : 0.f;
+#pragma unroll
+      for (int m = 0; m < i; ++m) x -= As[(o + i) * kLF + o + m] * tcol[m];
+      tcol[i] = x;
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) Ti[(o + i) * kLF + o + j] = tcol[i];
+  }
+  GDN_LDS_BARRIER();
+
+  // ---- phase 2b: 16 -> 32 merges  X = -T22 (A21 T11); the zero upper triangle of As is scratch ----
+  {
+    const int p = wave & 1;           // waves 0,1 write; 2,3 repeat the same values (benign)
+    const int C0 = 32 * p, R0 = C0 + 16;
+    const int li = lane & 15, lk = lane >> 4;
+    f32x4 y = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+      y = mfma16_f32(y, As[(R0 + li) * kLF + C0 + 4 * kk + lk], Ti[(C0 + 4 * kk + lk) * kLF + C0 + li]);
+    if (wave < 2) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) As[(C0 + 4 * lk + r) * kLF + R0 + li] = y[r];
+    }
+    GDN_LDS_BARRIER();
+    f32x4 x = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+      x = mfma16_f32(x, Ti[(R0 + li) * kLF + R0 + 4 * kk + lk], As[(C0 + 4 * kk + lk) * kLF + R0 + li]);
+    if (wave < 2) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) Ti[(R0 + 4 * lk + r) * kLF + C0 + li] = -x[r];
+    }
+  }
+  GDN_LDS_BARRIER();
+
+  // ---- phase 2c: 32 -> 64 merge, one 16x16 tile of the 32x32 block per wave ----
+  {
+    const int ta = wave >> 1, tb = wave & 1;
+    const int li = lane & 15, lk = lane >> 4;
+    f32x4 y = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk)
+      y = mfma16_f32(y, As[(32 + 16 * ta + li) * kLF + 4 * kk + lk], Ti[(4 * kk + lk) * kLF + 16 * tb + li]);
+    // scratch: upper-right 32x32 quadrant of As (never read as part of A)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) As[(16 * ta + 4 * lk + r) * kLF + 32 + 16 * tb + li] = y[r];
+    GDN_LDS_BARRIER();
+    f32x4 x = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk)
+      x = mfma16_f32(x, Ti[(32 + 16 * ta + li) * kLF + 32 + 4 * kk + lk], As[(4 * kk + lk) * kLF + 32 + 16 * tb + li]);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) Ti[(32 + 16 * ta + 4 * lk + r) * kLF + 16 * tb + li] = -x[r];
+  }
+  GDN_LDS_BARRIER();
+
+}
+
+// The inverse as four 32x32 A-operand tiles in operand precision (lane <-> row, registers <-> column), through the
+// row-major staging tile Tms [64][lds_ld<T>(64)].
+template <typename T>
+__device__ __forceinline__ void store_tm_tiles(const float* Ti, T* Tms, T* tiles_out, int tid, int wave, int lane) {
+  constexpr int L64 = lds_ld<T>(64), VEC = Elem<T>::kVec;
+  // ---- phase 3: Tm in operand precision, as four 32x32 A-operand tiles (lane <-> row, registers <-> column) ----
+  {
+    constexpr int CPR = 64 / VEC;
+    for (int c = tid; c < 64 * CPR; c += kThreads) {
+      const int row = c / CPR, cc = c % CPR;
+      float f[VEC];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) f[e] = Ti[row * kLF + cc * VEC + e];
+      st16(Tms + row * L64 + cc * VEC, pack16<T>(f));
+    }
+  }
+  GDN_LDS_BARRIER();
+  {
+    AccB<T> tf;
+    frags_from_lds<T>(tf, Tms + (32 * (wave >> 1) + (lane & 31)) * L64 + 32 * (wave & 1));
+    tf.store_stream(tiles_out + wave * 1024);
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // chunk_prep_kernel: what is independent across chunks and does not involve v.
 //   G (cumulative decay), Tm = (I+L)^-1, Aq = scale tril(Q K^T . Gam), and per q/k group the K and Q^T tiles, all in
@@ -218,85 +310,8 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
   for (int i = tid; i < 64 * kLF; i += kThreads) Ti[i] = 0.f;
   GDN_LDS_BARRIER();
 
-  // ---- phase 2a: invert the four 16x16 diagonal blocks by forward substitution (fp32) ----
-  if (lane < 16) {
-    const int o = 16 * wave, j = lane;
-    float tcol[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      float x = (i == j) ? 1.f : 0.f;
-#pragma unroll
-      for (int m = 0; m < i; ++m) x -= As[(o + i) * kLF + o + m] * tcol[m];
-      tcol[i] = x;
-    }
-#pragma unroll
-    for (int i = 0; i < 16; ++i) Ti[(o + i) * kLF + o + j] = tcol[i];
-  }
-  GDN_LDS_BARRIER();
-
-  // ---- phase 2b: 16 -> 32 merges  X = -T22 (A21 T11); the zero upper triangle of As is scratch ----
-  {
-    const int p = wave & 1;           // waves 0,1 write; 2,3 repeat the same values (benign)
-    const int C0 = 32 * p, R0 = C0 + 16;
-    const int li = lane & 15, lk = lane >> 4;
-    f32x4 y = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk)
-      y = mfma16_f32(y, As[(R0 + li) * kLF + C0 + 4 * kk + lk], Ti[(C0 + 4 * kk + lk) * kLF + C0 + li]);
-    if (wave < 2) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) As[(C0 + 4 * lk + r) * kLF + R0 + li] = y[r];
-    }
-    GDN_LDS_BARRIER();
-    f32x4 x = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk)
-      x = mfma16_f32(x, Ti[(R0 + li) * kLF + R0 + 4 * kk + lk], As[(C0 + 4 * kk + lk) * kLF + R0 + li]);
-    if (wave < 2) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) Ti[(R0 + 4 * lk + r) * kLF + C0 + li] = -x[r];
-    }
-  }
-  GDN_LDS_BARRIER();
-
-  // ---- phase 2c: 32 -> 64 merge, one 16x16 tile of the 32x32 block per wave ----
-  {
-    const int ta = wave >> 1, tb = wave & 1;
-    const int li = lane & 15, lk = lane >> 4;
-    f32x4 y = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int kk = 0; kk < 8; ++kk)
-      y = mfma16_f32(y, As[(32 + 16 * ta + li) * kLF + 4 * kk + lk], Ti[(4 * kk + lk) * kLF + 16 * tb + li]);
-    // scratch: upper-right 32x32 quadrant of As (never read as part of A)
-#pragma unroll
-    for (int r = 0; r < 4; ++r) As[(16 * ta + 4 * lk + r) * kLF + 32 + 16 * tb + li] = y[r];
-    GDN_LDS_BARRIER();
-    f32x4 x = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int kk = 0; kk < 8; ++kk)
-      x = mfma16_f32(x, Ti[(32 + 16 * ta + li) * kLF + 32 + 4 * kk + lk], As[(4 * kk + lk) * kLF + 32 + 16 * tb + li]);
-#pragma unroll
-    for (int r = 0; r < 4; ++r) Ti[(32 + 16 * ta + 4 * lk + r) * kLF + 16 * tb + li] = -x[r];
-  }
-  GDN_LDS_BARRIER();
-
-  // ---- phase 3: Tm in operand precision, as four 32x32 A-operand tiles (lane <-> row, registers <-> column) ----
-  {
-    constexpr int CPR = 64 / VEC;
-    for (int c = tid; c < 64 * CPR; c += kThreads) {
-      const int row = c / CPR, cc = c % CPR;
-      float f[VEC];
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) f[e] = Ti[row * kLF + cc * VEC + e];
-      st16(Tms + row * L64 + cc * VEC, pack16<T>(f));
-    }
-  }
-  GDN_LDS_BARRIER();
-  {
-    AccB<T> tf;
-    frags_from_lds<T>(tf, Tms + (32 * (wave >> 1) + (lane & 31)) * L64 + 32 * (wave & 1));
-    tf.store_stream(Ai_out + (((int64_t)blockIdx.x * Hv + h) * 4 + wave) * 1024);
-  }
+  tril_inverse_64(As, Ti, wave, lane);
+  store_tm_tiles<T>(Ti, Tms, Ai_out + ((int64_t)blockIdx.x * Hv + h) * 4096, tid, wave, lane);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -326,7 +341,7 @@ template <typename T, int DK, int NW, int STAGES, bool FUSE> struct StatePre {
   static constexpr bool value = STAGES * ((2 * 64 * DK + 3 * 1024 + 64 * 32 * NW + (FUSE ? 64 * DK + 3 * 1024 : 0)) * (int)sizeof(T) + 68 * 4) +
                                     (FUSE ? NW * x_elems * (int)sizeof(T) : 0) <= 160 * 1024;
 };
-template <typename T, int DK, int NW, int STAGES, bool OUT, bool PRE_> struct StateSmem {
+template <typename T, int DK, int NW, int STAGES, bool OUT, bool PRE_, bool KDA = false> struct StateSmem {
   static constexpr int x_elems = 2 * DK * 32 + 2 * 2048 + StateOutWaves<NW>::value * Patch<T>::kElems;
   static constexpr bool PRE = PRE_;
   // one stage, in elements of T
@@ -336,8 +351,10 @@ template <typename T, int DK, int NW, int STAGES, bool OUT, bool PRE_> struct St
   static constexpr int off_q = off_v + 64 * 32 * NW;                // OUT: Q^T image
   static constexpr int off_aq = off_q + (OUT ? 64 * DK : 0);        // OUT: Aq tiles (0,0), (1,0), (1,1)
   static constexpr int off_row = (off_aq + (OUT ? 3 * 1024 : 0)) * (int)sizeof(T);   // bytes: float rows
-  // rows: scale e^G [64], G_last; without PRE also e^{G_last-G} [64], beta e^G [64], beta [64]
-  static constexpr int stage = off_row + (PRE ? 68 : 260) * 4;   // a multiple of 16 bytes, like the offset of every row vector
+  // rows: scale e^G [64], G_last; without PRE also e^{G_last-G} [64], beta e^G [64], beta [64]; KDA: e^{G_last} per key
+  // channel [DK] at 68
+  static constexpr int stage = off_row + (PRE && !KDA ? 68 : 260) * 4;   // a multiple of 16 bytes, like the offset of every row vector
+  static_assert(!KDA || (PRE && !OUT && DK <= 128), "KDA: both K images arrive ready-made, the output is a kernel of its own");
   static_assert(stage % 16 == 0, "stages keep 16-byte alignment");
   static constexpr int off_x = STAGES * stage;                      // OUT: per slab S [2][DK*32], V' [2][2048], a store patch per output wave
   static constexpr int bytes = off_x + (OUT ? NW * x_elems * (int)sizeof(T) : 0);
@@ -348,7 +365,10 @@ template <typename T, int DK, int NW, int STAGES, bool OUT, bool PRE_> struct St
 // piece (the same loads on every path; the duplicate lands on the same LDS address with the same data)
 template <int PIECES, int NT> struct Deal { static constexpr int kPer = (PIECES + NT - 1) / NT; };
 
-template <typename T, int DK, int NW, int NL, int STAGES, bool OUT, bool PRE_>
+// KDA (one decay per key channel): kaf and qtf hold the two K images ready-made, rows scaled by -beta e^{G} and by
+// e^{G_last-G} channel by channel, G holds e^{G_last} [chunks,Hv,DK] and beta the transformed beta in fp32; the state's
+// rows decay each by their own factor.
+template <typename T, int DK, int NW, int NL, int STAGES, bool OUT, bool PRE_, bool KDA = false>
 __global__ __launch_bounds__(64 * (NW + (OUT ? NW * StateOutWaves<NW>::value : 0) + NL)) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 2 : 1)
 void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, const T* __restrict__ ai,
                         const T* __restrict__ aqf, const T* __restrict__ v, const float* __restrict__ G,
@@ -356,7 +376,8 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
                         T* __restrict__ vf, T* __restrict__ hf, T* __restrict__ o, const int64_t* __restrict__ cu,
                         const int* __restrict__ chunk_offsets, int T_len, int Hqk, int Hv, int V, float scale,
                         int64_t v_stride) {
-  using SM = StateSmem<T, DK, NW, STAGES, OUT, PRE_>;
+  using SM = StateSmem<T, DK, NW, STAGES, OUT, PRE_, KDA>;
+  static_assert(!KDA || 64 * NL >= DK, "a loader thread per key channel");
   constexpr int NT = 64 * NL, VEC = Elem<T>::kVec, NKT = DK / 32, OS = StateOutWaves<NW>::value, NWO = OUT ? NW * OS : 0;
   constexpr int PK = 64 * DK / VEC, PTM = 3 * 1024 / VEC, PV = 64 * 32 * NW / VEC, VPR = 32 * NW / VEC;
   constexpr int CK = Deal<PK, NT>::kPer, CTM = Deal<PTM, NT>::kPer, CV = Deal<PV, NT>::kPer;
@@ -389,7 +410,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
     // DEPTH register sets: chunk j sits in set j % DEPTH from the iteration that requests it (j - DEPTH - 1) to the
     // one that copies it to LDS (j - 1), so global loads have DEPTH chunk periods to arrive
     constexpr int DEPTH = (STAGES == 2) ? 2 : 1;
-    Vec16<T> pk[DEPTH][CK], ptm[DEPTH][CTM], pv[DEPTH][CV], pq[DEPTH][OUT ? CK : 1], pa[DEPTH][OUT ? CTM : 1];
+    Vec16<T> pk[DEPTH][CK], ptm[DEPTH][CTM], pv[DEPTH][CV], pq[DEPTH][OUT || KDA ? CK : 1], pa[DEPTH][OUT ? CTM : 1];   // KDA: pq = second K image
     float pgl[DEPTH], pg[DEPTH], pgk[DEPTH][2];
     uint32_t pb[DEPTH], pbk[DEPTH][2], pbv[DEPTH][CV];   // beta as fetched
     int pnv[DEPTH];
@@ -408,7 +429,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
       for (int i = 0; i < CK; ++i) {
         const int idc = imin(lt + i * NT, PK - 1);
         pk[set][i] = ld16(kaf + chq * (64 * DK) + idc * VEC);   // shared by the value heads of the group
-        if constexpr (OUT) pq[set][i] = ld16(qtf + chq * (64 * DK) + idc * VEC);
+        if constexpr (OUT || KDA) pq[set][i] = ld16(qtf + chq * (64 * DK) + idc * VEC);
       }
 #pragma unroll
       for (int i = 0; i < CTM; ++i) {
@@ -422,6 +443,11 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
         pv[set][i] = ld16(v + (tok0 + row) * v_stride + (int64_t)h * V + blockIdx.y * (32 * NW) + cc * VEC);
         if constexpr (PRE) pbv[set][i] = gate_raw<T>(beta, beta_same, (tok0 + row) * Hv + h);
       }
+      pnv[set] = nvalid;
+      if constexpr (KDA) {
+        pgl[set] = G[ch * DK + imin(lt, DK - 1)];   // e^{G_last} of this thread's key channel
+        return;
+      }
       const float* gc = G + ch * 64;
       const int t = lt & 63;
       // raw values only: arithmetic here would wait for every load issued so far.  G repeats G_last past the end of a
@@ -429,7 +455,6 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
       pgl[set] = gc[63];
       pg[set] = gc[t];
       pb[set] = gate_raw<T>(beta, beta_same, (tok0 + imin(t, nvalid - 1)) * Hv + h);
-      pnv[set] = nvalid;
       if constexpr (PRE) {
         // In the K tiles every 16-byte piece belongs to one token, 32 (tile & 1) + the row of its place, and this
         // thread's pieces all sit at the same place of their tiles: the gates of two tokens cover them.
@@ -443,7 +468,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
     auto commit = [&](int set, int buf) {   // registers -> LDS stage
       T* st = reinterpret_cast<T*>(gdn_smem + buf * SM::stage);
       float f1[2], f2[2];
-      if constexpr (PRE) {
+      if constexpr (PRE && !KDA) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
           f1[j] = (32 * j + krow < pnv[set]) ? -gate_val<T>(pbk[set][j], beta_same) * __expf(pgk[set][j]) : 0.f;
@@ -453,7 +478,10 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
 #pragma unroll
       for (int i = 0; i < CK; ++i) {
         const int idc = imin(lt + i * NT, PK - 1);
-        if constexpr (PRE) {
+        if constexpr (KDA) {
+          st16(st + SM::off_k + idc * VEC, pk[set][i]);
+          st16(st + SM::off_k + 64 * DK + idc * VEC, pq[set][i]);
+        } else if constexpr (PRE) {
           const int tj = (idc / (1024 / VEC)) & 1;
           st16(st + SM::off_k + idc * VEC, scale16<T>(pk[set][i], f1[tj]));
           st16(st + SM::off_k + 64 * DK + idc * VEC, scale16<T>(pk[set][i], f2[tj]));
@@ -475,6 +503,10 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
         else st16(st + SM::off_v + idc * VEC, pv[set][i]);
       }
       float* row = reinterpret_cast<float*>(gdn_smem + buf * SM::stage + SM::off_row);
+      if constexpr (KDA) {
+        if (lt < DK) row[68 + lt] = pgl[set];
+        return;
+      }
       if (lt < 64) {
         const float b = lt < pnv[set] ? gate_val<T>(pb[set], beta_same) : 0.f, eg = __expf(pg[set]);
         row[lt] = scale * eg;
@@ -670,7 +702,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
     Vb[1].load_cols(Vs + 32 * (32 * NW) + 32 * wave, 32 * NW);
     load_k(0, 0);
     if (NP > 1) load_k(1, 1);
-    const float eg = __expf(row[64]);
+    const float eg = KDA ? 1.f : __expf(row[64]);
     if (!OUT && hf != nullptr) {   // with output waves the stores are theirs: they hold S and V' too and have the time
 #pragma unroll
       for (int kt = 0; kt < NKT; ++kt) Sb[kt].store_stream(hf + (tile0 * NKT + kt) * 1024);
@@ -685,8 +717,14 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
       for (int j = 0; j < 2; ++j) {
         mma32_ff<T>(p0, Kf[kp & 1][0][j], Sb[2 * kp + j]);
         mma32_ff<T>(p1, Kf[kp & 1][1][j], Sb[2 * kp + j]);
+        if constexpr (KDA) {
+          const f32x16 dk = rows_ld(row + 68, 32 * (2 * kp + j));   // the decay of each of the tile's 32 key channels
 #pragma unroll
-        for (int r = 0; r < 16; ++r) S[2 * kp + j][r] *= eg;
+          for (int r = 0; r < 16; ++r) S[2 * kp + j][r] *= dk[r];
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) S[2 * kp + j][r] *= eg;
+        }
         GDN_INTERLEAVE_MFMA_VALU(2 * AccK<T>::kGroups, 16 / (2 * AccK<T>::kGroups));
       }
       GDN_SCHED_FENCE();
@@ -833,7 +871,8 @@ __global__ __launch_bounds__(64 * NW) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 2)
     qreg[i] = ld16(q + (tok0 + row) * q_stride + hq * DK + cc * VEC);
     qs[i] = rstd_q != nullptr ? rstd_q[((int64_t)blockIdx.x * Hqk + hq) * 64 + row] : 1.f;
   }
-  const float gval = G[ch * 64 + imin(tid & 63, nvalid - 1)];
+  // G null: the rows of q arrive with scale and decay already applied (KDA, one decay per key channel)
+  const float gval = G != nullptr ? G[ch * 64 + imin(tid & 63, nvalid - 1)] : 0.f;
 #pragma unroll
   for (int i = 0; i < QPT; ++i) {
     const int c = tid + i * NT, row = c / (DK / VEC), cc = c % (DK / VEC);
@@ -841,7 +880,7 @@ __global__ __launch_bounds__(64 * NW) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 2)
     if (row < nvalid) x = rstd_q != nullptr ? scale16<T>(qreg[i], qs[i]) : qreg[i];
     st16(Qs + row * LDK + cc * VEC, x);
   }
-  if (tid < 64) Eg[tid] = scale * __expf(gval);
+  if (tid < 64) Eg[tid] = G != nullptr ? scale * __expf(gval) : 1.f;
   IdentityFrag<T> id;
   id.init();
 #pragma unroll
@@ -1115,3 +1154,5 @@ extern "C" int gdn_chunk_fwd(const void* q, const void* k, const void* v, const 
   return gdn_chunk_fwd_strided(q, k, v, 0, 0, 0, g, beta, initial_state, cu_seqlens, o, final_state, workspace,
                                workspace_bytes, B, T, N, Hqk, Hv, K, V, scale, use_qk_l2norm, dtype, 0, stream);
 }
+
+#include "gdn_kda_fwd.h"

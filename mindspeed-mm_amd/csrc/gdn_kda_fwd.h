@@ -1,0 +1,386 @@
+// KDA (Kimi delta attention) forward: the gated delta rule with one decay per key channel,
+//     S <- diag(e^{g_t}) S;  S <- S + beta_t k_t (v_t - S^T k_t)^T;  o_t = scale S^T q_t
+// (reference: mindspeed_mm/fsdp/ops/kda/chunk_kda_naive.py:106-221, operator entry :223-381, gate :76-104).
+// Included at the end of gdn_chunk_fwd.hip: the recurrence and the output product are that file's kernels
+// (chunk_state_kernel in its KDA mode, chunk_out_kernel with rows of q that already carry scale and decay); this file
+// adds the chunk-local preparation, which is where the per-channel decay changes the algebra, and the entry points.
+//
+// Per chunk, with G the chunk-local cumulative log decay [64, K]:
+//     L_ij  = beta_i sum_d k_id k_jd e^{G_id - G_jd}   (i > j)       Tm = (I + L)^-1
+//     Aq_ij = scale sum_d q_id k_jd e^{G_id - G_jd}    (i >= j)
+//     V' = Tm beta (v - (k . e^G) S)      O = (scale q . e^G) S + Aq V'      S <- e^{G_last} . S + (k . e^{G_last-G})^T V'
+// e^{G_i - G_j} does not factor over a whole chunk without overflow (e^{-G_j} is unbounded), so the two 32x32 diagonal
+// blocks of L and Aq are summed channel by channel in fp32 with the exact exponent, and the off-diagonal block uses the
+// matrix cores on rows rescaled around the decay at the block boundary, k_i e^{G_i - G_31} (i >= 32) against
+// k_j e^{G_31 - G_j} (j < 32): both factors are at most 1.
+#pragma once
+
+namespace gdn {
+
+struct KdaFlags {
+  int l2norm, use_gate, has_lower_bound, beta_sigmoid, beta_x2, g_f32, beta_f32;
+  float lower_bound;
+};
+
+template <typename T, int DK> struct KdaPrepSmem {
+  static constexpr int LDK = lds_ld<T>(DK), LDG = DK + 4, L64 = lds_ld<T>(64);
+  static constexpr int tile = 64 * LDK * (int)sizeof(T), amat = 64 * kLF * 4;
+  static constexpr int off_ks = 0, off_qs = off_ks + tile, off_gs = off_qs + tile;   // k, q rows (T), G rows (fp32)
+  static constexpr int off_x1 = off_gs + 64 * LDG * 4;   // 64 rows of T: rescaled rows for the matrix cores, then staging
+  static constexpr int off_x2 = off_x1 + tile;           // 32 rows of T
+  static constexpr int off_misc = off_x2 + tile / 2;     // beta [64], partial totals of the cumulative sum [4][DK]
+  static constexpr int end0 = off_misc + (64 + 4 * DK) * 4;
+  // L, Aq (fp32), the inverse and its staging tile: for K = 128 they take the place of k, q, G and the staging rows,
+  // all dead by then; for K = 64 those are too small and there is room behind them
+  static constexpr bool alias = DK > 64;
+  static constexpr int off_as = alias ? off_ks : end0, off_aq = alias ? off_qs : end0 + amat;
+  static constexpr int off_ti = alias ? off_gs : end0 + 2 * amat, off_tm = alias ? off_x1 : end0 + 3 * amat;
+  static constexpr int bytes = alias ? end0 : end0 + 3 * amat + 64 * L64 * (int)sizeof(T);
+  static_assert(!alias || (amat <= tile && amat <= 64 * LDG * 4 && 64 * L64 * (int)sizeof(T) <= tile), "tenants fit");
+  static_assert(bytes <= 160 * 1024, "one CU's LDS");
+};
+
+__device__ __forceinline__ float kda_sigmoid(float x) { return 1.f / (1.f + __expf(-x)); }
+__device__ __forceinline__ float kda_softplus(float x) { return x > 20.f ? x : log1pf(__expf(x)); }
+
+// VEC consecutive fp32 values of an LDS row
+template <int VEC> __device__ __forceinline__ void ld_f32(const float* p, float* f) {
+#pragma unroll
+  for (int e = 0; e < VEC; e += 4) {
+    const f32x4 x = *reinterpret_cast<const f32x4*>(p + e);
+    f[e] = x[0]; f[e + 1] = x[1]; f[e + 2] = x[2]; f[e + 3] = x[3];
+  }
+}
+
+template <typename T, int DK>
+__global__ __launch_bounds__(kThreads) void kda_prep_kernel(
+    const T* __restrict__ q, const T* __restrict__ k, const void* __restrict__ g, const void* __restrict__ beta,
+    const float* __restrict__ A_log, const float* __restrict__ dt_bias, const int64_t* __restrict__ cu,
+    const int* __restrict__ chunk_offsets, float* __restrict__ bhat_out, float* __restrict__ dec_out,
+    float* __restrict__ G_out, T* __restrict__ Ai_out, T* __restrict__ Aq_out, T* __restrict__ K1_out,
+    T* __restrict__ K2_out, T* __restrict__ QB_out, float* __restrict__ rstd_q_out, float* __restrict__ rstd_k_out,
+    int T_len, int N, int H, float scale, KdaFlags fl) {
+  using SM = KdaPrepSmem<T, DK>;
+  constexpr int LDK = SM::LDK, LDG = SM::LDG, VEC = Elem<T>::kVec, CPR = DK / VEC;
+  T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
+  T* Qs = reinterpret_cast<T*>(gdn_smem + SM::off_qs);
+  float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_gs);
+  T* X1 = reinterpret_cast<T*>(gdn_smem + SM::off_x1);
+  T* X2 = reinterpret_cast<T*>(gdn_smem + SM::off_x2);
+  float* bs = reinterpret_cast<float*>(gdn_smem + SM::off_misc);
+  float* tot = bs + 64;
+  float* As = reinterpret_cast<float*>(gdn_smem + SM::off_as);
+  float* Aqs = reinterpret_cast<float*>(gdn_smem + SM::off_aq);
+  float* Ti = reinterpret_cast<float*>(gdn_smem + SM::off_ti);
+  T* Tms = reinterpret_cast<T*>(gdn_smem + SM::off_tm);
+
+  const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
+  if (s.nvalid <= 0) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int h = blockIdx.y, nvalid = s.nvalid;
+  const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk, hk = (int64_t)H * DK;
+  const int64_t ch = (int64_t)blockIdx.x * H + h;
+
+  // ---- phase 0: requests first: k, q rows, the gate input (4 channels per piece), beta ----
+  TileQK<T, DK> kt, qt;
+  tile_qk_request<T, DK>(kt, k + tok0 * hk + h * DK, hk, nvalid, tid);
+  tile_qk_request<T, DK>(qt, q + tok0 * hk + h * DK, hk, nvalid, tid);
+  constexpr int GP = 64 * (DK / 4) / kThreads;
+  const bool g32 = sizeof(T) == 4 || fl.g_f32;
+  float gx[GP][4];
+#pragma unroll
+  for (int i = 0; i < GP; ++i) {
+    const int c = tid + i * kThreads, row = imin(c / (DK / 4), nvalid - 1), c4 = c % (DK / 4);
+    const int64_t at = (tok0 + row) * hk + h * DK + 4 * c4;
+    if (g32) {
+      const f32x4 x = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(g) + at);
+      gx[i][0] = x[0]; gx[i][1] = x[1]; gx[i][2] = x[2]; gx[i][3] = x[3];
+    } else {
+      const u32x2 x = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(g) + at);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        T t;
+        if constexpr (sizeof(T) == 2) t.bits = (uint16_t)(x[e >> 1] >> (16 * (e & 1)));
+        gx[i][e] = Elem<T>::to_f(t);
+      }
+    }
+  }
+  if (wave == 0) {
+    const int64_t at = (tok0 + imin(lane, nvalid - 1)) * H + h;
+    float b;
+    if (sizeof(T) == 4 || fl.beta_f32) b = reinterpret_cast<const float*>(beta)[at];
+    else { T t; if constexpr (sizeof(T) == 2) t.bits = reinterpret_cast<const uint16_t*>(beta)[at]; b = Elem<T>::to_f(t); }
+    if (fl.beta_sigmoid) b = kda_sigmoid(b) * (fl.beta_x2 ? 2.f : 1.f);
+    bs[lane] = lane < nvalid ? b : 0.f;
+    if (lane < nvalid) bhat_out[at] = b;
+  }
+  // the gate: log decay of every token and channel, 0 on the rows past the end (they leave the cumulative sum alone)
+  {
+    const float a = fl.use_gate ? __expf(A_log[h]) : 0.f;
+#pragma unroll
+    for (int i = 0; i < GP; ++i) {
+      const int c = tid + i * kThreads, row = c / (DK / 4), c4 = c % (DK / 4);
+      f32x4 y;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float x = gx[i][e];
+        if (fl.use_gate) {
+          if (dt_bias != nullptr) x += dt_bias[h * DK + 4 * c4 + e];
+          x = fl.has_lower_bound ? fl.lower_bound * kda_sigmoid(a * x) : -a * kda_softplus(x);
+        }
+        y[e] = row < nvalid ? x : 0.f;
+      }
+      *reinterpret_cast<f32x4*>(Gs + row * LDG + 4 * c4) = y;
+    }
+  }
+  {
+    const int64_t roff = ch * 64;
+    tile_qk_finish<T, DK>(kt, Ks, LDK, nvalid, tid, fl.l2norm != 0, nullptr, 0, rstd_k_out ? rstd_k_out + roff : nullptr, 1);
+    tile_qk_finish<T, DK>(qt, Qs, LDK, nvalid, tid, fl.l2norm != 0, nullptr, 0, rstd_q_out ? rstd_q_out + roff : nullptr, 1);
+  }
+  GDN_LDS_BARRIER();
+  // cumulative sum down the tokens, a thread per channel and part of the chunk, then the totals of the parts before it
+  {
+    constexpr int PARTS = kThreads / DK, RPP = 64 / PARTS;
+    const int d = tid % DK, part = tid / DK;
+    float run = 0.f;
+#pragma unroll
+    for (int r = 0; r < RPP; ++r) {
+      run += Gs[(part * RPP + r) * LDG + d];
+      Gs[(part * RPP + r) * LDG + d] = run;
+    }
+    tot[part * DK + d] = run;
+    GDN_LDS_BARRIER();
+    float off = 0.f;
+#pragma unroll
+    for (int p = 0; p < PARTS - 1; ++p) off += p < part ? tot[p * DK + d] : 0.f;
+    if (part > 0) {
+#pragma unroll
+      for (int r = 0; r < RPP; ++r) Gs[(part * RPP + r) * LDG + d] += off;
+    }
+  }
+  GDN_LDS_BARRIER();
+
+  // ---- phase 1a: rows rescaled around the decay at the block boundary: X1 = [k_i ; q_i] e^{G_i-G_31} (i >= 32),
+  //      X2 = k_j e^{G_31-G_j} (j < 32) ----
+  for (int c = tid; c < 96 * CPR; c += kThreads) {
+    const int r = c / CPR, cc = c % CPR;
+    const int src = r < 32 ? 32 + r : (r < 64 ? r : r - 64);
+    const T* from = (r >= 32 && r < 64) ? Qs : Ks;
+    float f[VEC], gi[VEC], gr[VEC];
+    unpack16<T>(ld16(from + src * LDK + cc * VEC), f);
+    ld_f32<VEC>(Gs + src * LDG + cc * VEC, gi);
+    ld_f32<VEC>(Gs + 31 * LDG + cc * VEC, gr);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) f[e] *= __expf(r < 64 ? gi[e] - gr[e] : gr[e] - gi[e]);
+    T* to = r < 64 ? X1 + r * LDK : X2 + (r - 64) * LDK;
+    st16(to + cc * VEC, pack16<T>(f));
+  }
+  GDN_LDS_BARRIER();
+
+  // ---- phase 1b: the off-diagonal block on the matrix cores (wave 0: k k, wave 1: q k) ----
+  f32x16 acc = acc_zero();
+  if (wave < 2) mma32<T, DK, true, true>(acc, X1 + 32 * wave * LDK, LDK, X2, LDK);
+  // the two diagonal blocks, pair by pair with the exact exponent.  Rows i and 31-i of a block have 33 pairs
+  // between them: eight threads share them.
+  float akk[5], aqk[5];
+  const int blk = tid >> 7, rp = (tid & 127) >> 3, cg = tid & 7;
+#pragma unroll
+  for (int t = 0; t < 5; ++t) {
+    const int p = cg + 8 * t;
+    int i = p <= rp ? rp : 31 - rp, j = p <= rp ? p : p - rp - 1;
+    if (p >= 33) { i = 0; j = 0; }
+    i += 32 * blk; j += 32 * blk;
+    float s1 = 0.f, s2 = 0.f;
+    for (int cc = 0; cc < CPR; ++cc) {
+      float ki[VEC], qi[VEC], kj[VEC], gi[VEC], gj[VEC];
+      unpack16<T>(ld16(Ks + i * LDK + cc * VEC), ki);
+      unpack16<T>(ld16(Qs + i * LDK + cc * VEC), qi);
+      unpack16<T>(ld16(Ks + j * LDK + cc * VEC), kj);
+      ld_f32<VEC>(Gs + i * LDG + cc * VEC, gi);
+      ld_f32<VEC>(Gs + j * LDG + cc * VEC, gj);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const float x = __expf(gi[e] - gj[e]) * kj[e];
+        s1 += ki[e] * x;
+        s2 += qi[e] * x;
+      }
+    }
+    akk[t] = s1;
+    aqk[t] = s2;
+  }
+  GDN_LDS_BARRIER();   // X1, X2 are free
+
+  // ---- phase 1c: what the recurrence reads.  K images through the staging rows into fragment order ----
+  auto stage_k = [&](bool first) {
+    for (int c = tid; c < 64 * CPR; c += kThreads) {
+      const int row = c / CPR, cc = c % CPR;
+      float f[VEC], gi[VEC], gl[VEC];
+      unpack16<T>(ld16(Ks + row * LDK + cc * VEC), f);
+      ld_f32<VEC>(Gs + row * LDG + cc * VEC, gi);
+      ld_f32<VEC>(Gs + 63 * LDG + cc * VEC, gl);
+      const float nb = -bs[row];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) f[e] *= first ? nb * __expf(gi[e]) : __expf(gl[e] - gi[e]);
+      st16(X1 + row * LDK + cc * VEC, pack16<T>(f));
+    }
+  };
+  auto store_k = [&](T* out) {
+    for (int tt = wave; tt < 2 * (DK / 32); tt += 4) {
+      const int tj = tt & 1, kt2 = tt >> 1;
+      AccB<T> kf;
+      frags_from_lds<T>(kf, X1 + (32 * tj + (lane & 31)) * LDK + 32 * kt2);
+      kf.store_stream(out + ((ch * (DK / 32) + kt2) * 2 + tj) * 1024);
+    }
+  };
+  stage_k(true);
+  GDN_LDS_BARRIER();
+  store_k(K1_out);
+  GDN_LDS_BARRIER();
+  stage_k(false);
+  GDN_LDS_BARRIER();
+  store_k(K2_out);
+  // rows of q with scale and decay, the decay of the whole chunk per channel, the cumulative decay itself
+  for (int c = tid; c < 64 * CPR; c += kThreads) {
+    const int row = c / CPR, cc = c % CPR;
+    if (row < nvalid) {
+      float f[VEC], gi[VEC];
+      unpack16<T>(ld16(Qs + row * LDK + cc * VEC), f);
+      ld_f32<VEC>(Gs + row * LDG + cc * VEC, gi);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) f[e] *= scale * __expf(gi[e]);
+      st16(QB_out + (tok0 + row) * hk + h * DK + cc * VEC, pack16<T>(f));
+    }
+  }
+  if (tid < DK) dec_out[ch * DK + tid] = __expf(Gs[63 * LDG + tid]);
+  if (G_out != nullptr) {
+    for (int c = tid; c < 64 * (DK / 4); c += kThreads) {
+      const int row = c / (DK / 4), c4 = c % (DK / 4);
+      *reinterpret_cast<f32x4*>(G_out + (ch * 64 + row) * DK + 4 * c4) = *reinterpret_cast<const f32x4*>(Gs + row * LDG + 4 * c4);
+    }
+  }
+  GDN_LDS_BARRIER();   // k, q, G and the staging rows are dead
+
+  // ---- phase 1d: L and Aq as 64x64 fp32 matrices ----
+  for (int i = tid; i < 64 * kLF; i += kThreads) { As[i] = 0.f; Aqs[i] = 0.f; Ti[i] = 0.f; }
+  GDN_LDS_BARRIER();
+#pragma unroll
+  for (int t = 0; t < 5; ++t) {
+    const int p = cg + 8 * t;
+    if (p < 33) {
+      const int i = 32 * blk + (p <= rp ? rp : 31 - rp), j = 32 * blk + (p <= rp ? p : p - rp - 1);
+      As[i * kLF + j] = i > j ? bs[i] * akk[t] : 0.f;
+      Aqs[i * kLF + j] = scale * aqk[t];
+    }
+  }
+  if (wave < 2) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int i = 32 + acc_row(r), j = acc_col();
+      if (wave == 0) As[i * kLF + j] = bs[i] * acc[r]; else Aqs[i * kLF + j] = scale * acc[r];
+    }
+  }
+  GDN_LDS_BARRIER();
+  {  // Aq leaves as four tiles packed as they sit in an accumulator (lane <-> column j, registers <-> row i)
+    const int ti = wave >> 1, tj = wave & 1;
+    f32x16 aq;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) aq[r] = Aqs[(32 * ti + acc_row(r)) * kLF + 32 * tj + acc_col()];
+    AccB<T> af;
+    af.pack(aq);
+    af.store_stream(Aq_out + (ch * 4 + wave) * 1024);
+  }
+  tril_inverse_64(As, Ti, wave, lane);
+  store_tm_tiles<T>(Ti, Tms, Ai_out + ch * 4096, tid, wave, lane);
+}
+
+// NWO: waves of the output kernel's workgroup; NWS, NLS, STAGES: slabs, loader waves and LDS stages of the recurrence
+template <typename T, int DK, int NWO, int NWS, int NLS, int STAGES>
+static int kda_fwd_launch(const ChunkDims& d, const KdaWorkspace& L, const void* q, const void* k, const void* v,
+                          const void* g, const void* beta, const float* A_log, const float* dt_bias, const float* h0,
+                          const int64_t* cu, void* o, float* ht, unsigned char* ws, float scale, const KdaFlags& fl,
+                          bool with_backward, hipStream_t st) {
+  const int H = d.Hv;
+  const int nc = (int)d.max_chunks();
+  int* chunk_offsets = reinterpret_cast<int*>(ws + L.chunk_offsets);
+  float* rstd = reinterpret_cast<float*>(ws + L.rstd);
+  float* bhat = reinterpret_cast<float*>(ws + L.bhat);
+  float* dec = reinterpret_cast<float*>(ws + L.dec);
+  T* Ai = reinterpret_cast<T*>(ws + L.Ai);
+  T* AQ = reinterpret_cast<T*>(ws + L.AQ);
+  T* K1F = reinterpret_cast<T*>(ws + L.K1F);
+  T* K2F = reinterpret_cast<T*>(ws + L.K2F);
+  T* QB = reinterpret_cast<T*>(ws + L.QB);
+  T* VF = reinterpret_cast<T*>(ws + L.VF);
+  T* HF = reinterpret_cast<T*>(ws + L.HF);
+  float* GC = with_backward ? reinterpret_cast<float*>(ws + L.GC) : nullptr;
+  if (cu != nullptr) GDN_LAUNCH(kKernChunkTable, st, chunk_table_kernel, dim3(1), dim3(kThreads), 0, st, cu, chunk_offsets, d.N);
+  {
+    auto kern = kda_prep_kernel<T, DK>;
+    constexpr int smem = KdaPrepSmem<T, DK>::bytes;
+    if (int e = set_lds(kern, smem)) return e;
+    const bool keep = with_backward && fl.l2norm;
+    GDN_LAUNCH(kKernKdaPrep, st, kern, dim3(nc, H), dim3(kThreads), smem, st, (const T*)q, (const T*)k, g, beta, A_log,
+               dt_bias, cu, (const int*)chunk_offsets, bhat, dec, GC, Ai, AQ, K1F, K2F, QB, keep ? rstd : nullptr,
+               keep ? rstd + (int64_t)nc * 64 * H : nullptr, d.T, d.N, H, scale, fl);
+  }
+  {
+    auto kern = chunk_state_kernel<T, DK, NWS, NLS, STAGES, false, true, true>;
+    constexpr int smem = StateSmem<T, DK, NWS, STAGES, false, true, true>::bytes;
+    if (int e = set_lds(kern, smem)) return e;
+    GDN_LAUNCH(kKernStateFwd, st, kern, dim3(d.N * H, d.V / (32 * NWS)), dim3(64 * (NWS + NLS)), smem, st, (const T*)K1F,
+               (const T*)K2F, (const T*)Ai, (const T*)AQ, (const T*)v, (const float*)dec, (const void*)bhat, 0, h0, ht, VF, HF,
+               (T*)nullptr, cu, (const int*)chunk_offsets, d.T, H, H, d.V, scale, (int64_t)H * d.V);
+  }
+  {
+    auto kern = chunk_out_kernel<T, DK, NWO, false, T>;
+    constexpr int smem = OutSmem<T, DK, NWO>::bytes;
+    if (int e = set_lds(kern, smem)) return e;
+    GDN_LAUNCH(kKernOut, st, kern, dim3(nc, H, d.V / (32 * NWO)), dim3(64 * NWO), smem, st, (const T*)QB, (const T*)AQ,
+               (const T*)VF, (const T*)HF, (const float*)nullptr, (T*)o, cu, (const int*)chunk_offsets, d.T, d.N, H, H, d.V,
+               scale, (int64_t)H * DK, (const float*)nullptr, OutNorm<T, T>{});
+  }
+  return (int)hipGetLastError();
+}
+
+}  // namespace gdn
+
+extern "C" int64_t gdn_kda_workspace_bytes(int B, int T, int N, int H, int K, int V, int with_backward, int dtype) {
+  gdn::ChunkDims d{B, T, N, H, H, K, V, true};   // the packed bound is the larger
+  const gdn::KdaWorkspace w = gdn::kda_workspace_layout(d, dtype == 0 ? 4 : 2);
+  return with_backward ? w.total_bytes : w.fwd_bytes;
+}
+
+extern "C" int gdn_kda_fwd(const void* q, const void* k, const void* v, const void* g, const void* beta,
+                           const float* A_log, const float* dt_bias, const float* initial_state,
+                           const int64_t* cu_seqlens, void* o, float* final_state, void* workspace,
+                           int64_t workspace_bytes, int B, int T, int N, int H, int K, int V, float scale,
+                           int use_qk_l2norm, int use_gate, int has_lower_bound, float lower_bound, int beta_sigmoid,
+                           int allow_neg_eigval, int dtype, int g_dtype, int beta_dtype, void* stream) {
+  using namespace gdn;
+  if (!q || !k || !v || !g || !beta || !o || !workspace) return -1;
+  if (use_gate && !A_log) return -1;
+  ChunkDims d{B, T, N, H, H, K, V, cu_seqlens != nullptr};
+  if (int e = chunk_check_dims(d, dtype)) return e;
+  if ((g_dtype != 0 && g_dtype != dtype) || (beta_dtype != 0 && beta_dtype != dtype)) return -4;
+  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)g | (uintptr_t)o) & 15) return -6;
+  ChunkDims dl = d;
+  dl.varlen = true;
+  const KdaWorkspace L = kda_workspace_layout(dl, dtype == 0 ? 4 : 2);
+  if (workspace_bytes < L.fwd_bytes || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
+  const bool with_bwd = workspace_bytes >= L.total_bytes;
+  KdaFlags fl{use_qk_l2norm, use_gate, has_lower_bound, beta_sigmoid, allow_neg_eigval, g_dtype == 0, beta_dtype == 0, lower_bound};
+  unsigned char* ws = static_cast<unsigned char*>(workspace);
+  hipStream_t st = (hipStream_t)stream;
+#define GDN_KDA(T_, DK_, NWO_, NWS_, NLS_, ST_)                                                                          \
+  return kda_fwd_launch<T_, DK_, NWO_, NWS_, NLS_, ST_>(d, L, q, k, v, g, beta, A_log, dt_bias, initial_state, cu_seqlens, o, \
+                                                        final_state, ws, scale, fl, with_bwd, st)
+  if (dtype == 1) {
+    if (K == 128) GDN_KDA(bf16_t, 128, 2, 2, 4, 2);
+    GDN_KDA(bf16_t, 64, 2, 2, 4, 2);
+  } else {
+    if (K == 128) GDN_KDA(float, 128, 2, 2, 2, 1);
+    GDN_KDA(float, 64, 2, 2, 2, 2);
+  }
+#undef GDN_KDA
+}

@@ -33,6 +33,8 @@ SIGNATURES = {
     "gdn_gate_bwd_workspace_bytes": (L, [L, I]),
     "gdn_gate_bwd": (I, [P] * 11 + [L, L, I, I, I, P]),
     "gdn_gate_bwd_noalloc": (I, [P] * 10 + [L, I, I, I, P]),
+    "gdn_kda_workspace_bytes": (L, [I] * 8),
+    "gdn_kda_fwd": (I, [P] * 12 + [L] + [I] * 6 + [F, I, I, I, F, I, I, I, I, I, P]),
     "gdn_profile_enable": (I, [I]),
     "gdn_profile_kernel_count": (I, []),
     "gdn_profile_kernel_name": (ctypes.c_char_p, [I]),

@@ -8,6 +8,8 @@
     rms_norm_gated / RMSNormGated     Qwen3_5RMSNormGated, modeling_qwen3_5.py:330-349, called at :897-900
     gdn_gates                         g / beta recipe of the layer, modeling_qwen3_5.py:833-841
     chunk_gated_delta_rule_qkv        the rule on the unsplit convolution output (split at :818-831)
+    chunk_kda                         mindspeed_mm/fsdp/ops/kda/triton_ascend/chunk.py:215-407 (the fused operator),
+                                      mindspeed_mm/fsdp/ops/kda/chunk_kda_naive.py:223-381 (its pure-PyTorch statement)
     fused_recurrent_gated_delta_rule_qkv / decode_step / GdnDecodeCache
                                       the layer's decode branch (:738-744, :808-848, :877-890) and the
                                       linear-attention part of Qwen3_5DynamicCache (:134-221)
@@ -219,6 +221,62 @@ class GdnOps:
         y = self.rms_norm_gated(o.reshape(-1, head_v_dim), gate.reshape(-1, head_v_dim).to(o.dtype), norm_weight,
                                 norm_eps)
         return y.view(o.shape), ht
+
+    # ------------------------------------------------------------------ KDA
+    def chunk_kda(self, q, k, v, g, beta, scale=None, initial_state=None, output_final_state=False,
+                  use_qk_l2norm_in_kernel=False, use_gate_in_kernel=False, use_beta_sigmoid_in_kernel=False,
+                  allow_neg_eigval=False, cu_seqlens=None, cu_seqlens_cpu=None, safe_gate=False, lower_bound=None,
+                  disable_recompute=False, return_intermediate_states=False, transpose_state_layout=False,
+                  skip_recompute=False, chunk_size=64, **kwargs):
+        """Kimi delta attention, chunked: the delta rule with one decay per key channel.  Signature and argument
+        checks of chunk_kda (triton_ascend/chunk.py:215-407) and chunk_kda_naive (chunk_kda_naive.py:223-381):
+        q, k, g [B,T,H,K], v [B,T,H,V], beta [B,T,H]; A_log [H] and dt_bias [H*K] come as keyword arguments when
+        use_gate_in_kernel is set.  safe_gate, disable_recompute, skip_recompute and cu_seqlens_cpu are hints of the
+        reference's kernels without effect on the result and are accepted and ignored."""
+        A_log, dt_bias = kwargs.get("A_log"), kwargs.get("dt_bias")
+        if use_gate_in_kernel and A_log is None:
+            raise ValueError("A_log must be provided when use_gate_in_kernel=True.")
+        if allow_neg_eigval and not use_beta_sigmoid_in_kernel:
+            raise ValueError("`allow_neg_eigval=True` requires `use_beta_sigmoid_in_kernel=True`.")
+        if not (q.shape == k.shape == g.shape):
+            raise ValueError("q, k, g must have the same shape.")
+        if beta.shape != q.shape[:3]:
+            raise ValueError("beta must be of shape (batch size, seq len, num of head).")
+        if tuple(v.shape[:3]) != tuple(q.shape[:3]) or v.dim() != 4:
+            raise ValueError("v must be of shape (batch size, seq len, num of head, head dim).")
+        if q.dtype != k.dtype or k.dtype != v.dtype or q.dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"chunk_kda supports bfloat16 and float32 q, k, v of one dtype, got {q.dtype}, {k.dtype}, {v.dtype}")
+        if chunk_size != 64:
+            raise ValueError("only chunk_size=64 is supported")
+        if return_intermediate_states:
+            raise NotImplementedError("return_intermediate_states=True (the per-chunk states in [K,V] order for an "
+                                      "inference engine) is not provided: the states are kept in matrix-core tile order")
+        N = q.shape[0]
+        if cu_seqlens is not None:
+            if q.shape[0] != 1:
+                raise ValueError(
+                    f"The batch size is expected to be 1 rather than {q.shape[0]} when using `cu_seqlens`."
+                    f"Please flatten variable-length inputs before processing.")
+            N = len(cu_seqlens) - 1
+            if initial_state is not None and initial_state.shape[0] != N:
+                raise ValueError(
+                    f"The number of initial states is expected to be equal to the number of input sequences, "
+                    f"i.e., {N} rather than {initial_state.shape[0]}.")
+        if initial_state is not None and initial_state.dtype != torch.float32:
+            raise ValueError("initial_state must be in float32.")
+        if scale is None:
+            scale = k.shape[-1] ** -0.5
+        _check_packed_length(cu_seqlens, q.shape[1])
+        self._need(q, k, v, g, beta, initial_state, A_log, dt_bias)
+        q, k, v, g, beta, initial_state, A_log, dt_bias = self._no_grad_views(q, k, v, g, beta, initial_state, A_log, dt_bias)
+        if transpose_state_layout and initial_state is not None:
+            initial_state = initial_state.transpose(-1, -2)
+        o, ht = _ChunkKda.apply(q, k, v, g, beta, A_log, dt_bias, float(scale), initial_state, bool(output_final_state),
+                                bool(use_qk_l2norm_in_kernel), bool(use_gate_in_kernel), bool(use_beta_sigmoid_in_kernel),
+                                bool(allow_neg_eigval), cu_seqlens, lower_bound, self)
+        if ht is not None and transpose_state_layout:
+            ht = ht.transpose(-1, -2)
+        return o, ht
 
     def gdn_gates(self, a, b, A_log, dt_bias):
         """(g, beta) of the layer from its projections a, b [..., Hv] and parameters A_log, dt_bias [Hv]:
@@ -605,6 +663,44 @@ class _ChunkGatedDeltaRuleQKV(torch.autograd.Function):
                 None, None, None, None)
 
 
+class _ChunkKda(torch.autograd.Function):
+    """Forward pass of KDA in the HIP library (gdn_kda_fwd).  A backward pass of its own is not built: asking for
+    gradients raises."""
+
+    @staticmethod
+    @_input_guard
+    @_custom_fwd
+    def forward(ctx, q, k, v, g, beta, A_log, dt_bias, scale, initial_state, output_final_state, l2norm, use_gate,
+                beta_sigmoid, allow_neg, cu_seqlens, lower_bound, ops):
+        lib = ops.lib
+        B, T, H, K = q.shape
+        V = v.shape[3]
+        N = (len(cu_seqlens) - 1) if cu_seqlens is not None else B
+        code = DTYPE_CODE[q.dtype]
+        qc, kc, vc = q.detach().contiguous(), k.detach().contiguous(), v.detach().contiguous()
+        gc = g.detach().contiguous() if g.dtype == q.dtype else g.detach().to(torch.float32).contiguous()
+        gcode = code if g.dtype == q.dtype else 0
+        bc, bcode = _beta_arg(beta, q.dtype)
+        a32, d32, h0 = ops._f32(A_log), ops._f32(dt_bias), ops._f32(initial_state)
+        cu = _i64(cu_seqlens, q)
+        nbytes = lib.gdn_kda_workspace_bytes(B, T, N, H, K, V, 0, code)
+        ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=q.device)
+        off = (-ws.data_ptr()) % 256
+        ws = ws[off:off + nbytes]
+        o = torch.empty(B, T, H, V, dtype=v.dtype, device=v.device)
+        ht = torch.empty(N, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
+        rc = lib.gdn_kda_fwd(ptr(qc), ptr(kc), ptr(vc), ptr(gc), ptr(bc), ptr(a32), ptr(d32), ptr(h0), ptr(cu), ptr(o),
+                             ptr(ht), ptr(ws), nbytes, B, T, N, H, K, V, scale, int(l2norm), int(use_gate),
+                             int(lower_bound is not None), float(lower_bound if lower_bound is not None else 0.0),
+                             int(beta_sigmoid), int(allow_neg), code, gcode, bcode, lib.stream())
+        lib.check(rc, "gdn_kda_fwd")
+        return o, ht
+
+    @staticmethod
+    def backward(ctx, do, dht):
+        raise NotImplementedError("chunk_kda: the backward pass is not built; call it under torch.no_grad()")
+
+
 class _GdnGates(torch.autograd.Function):
     """beta = sigmoid(b), g = -exp(A_log.float()) * softplus(a.float() + dt_bias), modeling_qwen3_5.py:833-841."""
 
@@ -795,6 +891,11 @@ def chunk_gated_delta_rule_qkv(mixed_qkv, g, beta, num_k_heads, num_v_heads, hea
     return _default_ops().chunk_gated_delta_rule_qkv(mixed_qkv, g, beta, num_k_heads, num_v_heads, head_k_dim,
                                                      head_v_dim, scale, initial_state, output_final_state,
                                                      use_qk_l2norm_in_kernel, cu_seqlens, gate, norm_weight, norm_eps)
+
+
+@torch.compiler.disable
+def chunk_kda(q, k, v, g, beta, scale=None, initial_state=None, output_final_state=False, **kwargs):
+    return _default_ops().chunk_kda(q, k, v, g, beta, scale, initial_state, output_final_state, **kwargs)
 
 
 @torch.compiler.disable

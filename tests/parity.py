@@ -1,15 +1,16 @@
 """Parity checks shared by the GPU tests (HIP library on cuda:0) and the CPU kernel-emulation tests.
 
 Each check runs one operator of the package through the C ABI on seeded inputs and compares it with the
-CPU oracle (oracle/gdn_oracle.py).  Tolerances are the ones the task states:
+CPU oracle (oracle/gdn_oracle.py, oracle/kda_oracle.py).  Tolerances are the ones the task states:
     fp32: max relative error (max|x - ref| / max|ref|) <= 1e-4
     bf16 vs the fp32 oracle on the same (bf16-valued) inputs: max abs error <= 2e-2 on o,
           <= 5e-2 on dq/dk/dv/dg/dbeta (and on the states, whose magnitude is O(1)).
 """
 import torch
 
-from mindspeed_mm_amd.inputs import gdn_inputs
+from mindspeed_mm_amd.inputs import gdn_inputs, kda_inputs
 from oracle import gdn_oracle as O
+from oracle import kda_oracle as KO
 
 FP32_REL = 1e-4
 BF16_ABS_O = 2e-2
@@ -417,3 +418,34 @@ def check_decode_step(ops, device, B, steps, Hqk, Hv, K, V, W, dtype, param_dtyp
     errs["conv_state"] = _err("conv_state", conv1, rconv, dtype, 1e-2, 1e-2)
     errs["state"] = _err("recurrent_state", S1, rS, dtype, BF16_ABS_GRAD)
     return errs
+
+
+def check_kda(ops, device, B, T, H, K, V, dtype, cu=None, seed=0, with_h0=True, gate_in_kernel=True, lower_bound=None,
+              beta_sigmoid=True, allow_neg=False, l2=True, transpose_state=True, g_dtype=None, scale=None,
+              wrap=lambda t: t, **recipe):
+    """chunk_kda against the oracle's statement of chunk_kda_naive, with the options of the layer's call
+    (modeling_kimi_linear.py:681-699: raw gate and beta, l2 norm in the kernel, [N,H,V,K] states) or without them."""
+    N = (len(cu) - 1) if cu is not None else B
+    x = kda_inputs(B, T, H, K, V, dtype, seed=seed, N=N, **recipe)
+    if not gate_in_kernel:   # the caller hands over the log decay itself
+        x["g"] = KO.kda_gate_ref(x["g"], x["A_log"], x["dt_bias"], lower_bound)
+    if g_dtype is not None:
+        x["g"] = x["g"].to(g_dtype)
+    if not beta_sigmoid:
+        x["beta"] = torch.sigmoid(x["beta"].float()).to(x["beta"].dtype)
+    if not l2:
+        x["q"], x["k"] = (KO._l2norm_rounded(t) for t in (x["q"], x["k"]))
+    if transpose_state:
+        x["h0"] = x["h0"].transpose(-1, -2).contiguous()
+    dev = {n: wrap(t.to(device)) for n, t in x.items()}
+    cu_t = torch.tensor(cu, dtype=torch.int64, device=device) if cu is not None else None
+    kw = dict(scale=scale, output_final_state=True, use_qk_l2norm_in_kernel=l2, use_gate_in_kernel=gate_in_kernel,
+              use_beta_sigmoid_in_kernel=beta_sigmoid, allow_neg_eigval=allow_neg, lower_bound=lower_bound if gate_in_kernel else None,
+              transpose_state_layout=transpose_state)
+    with torch.no_grad():
+        o, ht = ops.chunk_kda(dev["q"], dev["k"], dev["v"], dev["g"], dev["beta"], initial_state=dev["h0"] if with_h0 else None,
+                              cu_seqlens=cu_t, safe_gate=lower_bound is not None, A_log=dev["A_log"], dt_bias=dev["dt_bias"], **kw)
+    ro, rht = KO.chunk_kda_ref(x["q"], x["k"], x["v"], x["g"], x["beta"], initial_state=x["h0"] if with_h0 else None,
+                               cu_seqlens=cu, A_log=x["A_log"], dt_bias=x["dt_bias"], round_output=False, **kw)
+    assert o.dtype == dtype and ht.dtype == torch.float32 and ht.shape == rht.shape
+    return {"o": _err("o", o, ro, dtype, BF16_ABS_O), "ht": _err("final_state", ht, rht, dtype, BF16_ABS_GRAD)}

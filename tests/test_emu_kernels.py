@@ -196,3 +196,15 @@ def test_conv1d_random_shapes(ops, seed):
     residual, initial state and activation."""
     c = _random_conv_case(seed)
     P.check_conv(ops, "cpu", c.pop("B"), c.pop("T"), c.pop("D"), c.pop("W"), c.pop("dtype"), wrap=guarded, **c)
+
+
+@pytest.mark.parametrize("dtype,B,T,H,K,V,cu,kw", [
+    (F32, 1, 64, 1, 64, 64, None, {}),
+    (F32, 2, 100, 2, 128, 128, None, {}),
+    (BF, 1, 200, 2, 128, 128, None, {}),
+    (BF, 1, 140, 2, 64, 64, [0, 5, 70, 71, 140], dict(lower_bound=-5.0)),
+    (F32, 1, 96, 1, 128, 192, [0, 1, 38, 96], dict(gate_in_kernel=False, beta_sigmoid=False, l2=False, transpose_state=False)),
+    (BF, 1, 130, 1, 128, 64, None, dict(allow_neg=True, with_h0=False, g_dtype=torch.float32)),
+])
+def test_kda_forward(ops, dtype, B, T, H, K, V, cu, kw):
+    P.check_kda(ops, "cpu", B, T, H, K, V, dtype, cu=cu, wrap=guarded, h0_std=0.1, **kw)

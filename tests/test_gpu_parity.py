@@ -388,3 +388,44 @@ def test_conv1d_random_shapes(ops, seed):
     c = _random_conv_case(seed)
     print(f"conv random {seed}: {c}", flush=True)
     P.check_conv(ops, "cuda", c.pop("B"), c.pop("T"), c.pop("D"), c.pop("W"), c.pop("dtype"), **c)
+
+
+# ---- KDA (one decay per key channel) ------------------------------------------------------------------------------
+
+KDA_CASES = [
+    # dtype, B, T, H, K, V, cu, options
+    (F32, 1, 64, 1, 64, 64, None, {}),
+    (F32, 2, 100, 2, 128, 128, None, {}),
+    (F32, 1, 1024, 2, 128, 128, None, dict(a_log=(0.5, 2.0), dt_bias=(-6.0, -4.0))),          # slow decay, long memory
+    (BF, 1, 200, 2, 128, 128, None, {}),
+    (BF, 2, 512, 4, 128, 128, None, dict(a_log=(0.5, 2.0), dt_bias=(-6.0, -4.0))),
+    (BF, 1, 140, 2, 64, 64, [0, 5, 70, 71, 140], dict(lower_bound=-5.0)),
+    (BF, 1, 1121, 2, 128, 128, [0, 112, 209, 240, 281, 489, 523, 566, 689, 721, 785, 837, 985, 1071, 1121],
+     dict(lower_bound=-5.0)),
+    (F32, 1, 96, 1, 128, 192, [0, 1, 38, 96], dict(gate_in_kernel=False, beta_sigmoid=False, l2=False, transpose_state=False)),
+    (BF, 1, 130, 1, 128, 64, None, dict(allow_neg=True, with_h0=False, g_dtype=torch.float32)),
+    (BF, 1, 300, 3, 128, 256, [0, 0, 300], dict(gate_in_kernel=False)),                      # an empty sequence
+    (BF, 1, 2048, 4, 128, 128, None, {}),                                                     # the layer's head shape
+]
+
+
+@pytest.mark.parametrize("dtype,B,T,H,K,V,cu,kw", KDA_CASES)
+def test_kda_forward(ops, dtype, B, T, H, K, V, cu, kw):
+    print(f"kda {dtype} B{B} T{T} H{H} K{K} V{V} cu={'yes' if cu else 'no'} {kw}", flush=True)
+    errs = P.check_kda(ops, "cuda", B, T, H, K, V, dtype, cu=cu, **kw)
+    print("   ", {n: f"{e:.2e}" for n, e in errs.items()}, flush=True)
+
+
+def test_kda_argument_checks(ops):
+    x = P.kda_inputs(1, 64, 2, 64, 64, BF)
+    d = {n: t.cuda() for n, t in x.items()}
+    with pytest.raises(ValueError):
+        ops.chunk_kda(d["q"], d["k"], d["v"], d["g"], d["beta"], use_gate_in_kernel=True)               # no A_log
+    with pytest.raises(ValueError):
+        ops.chunk_kda(d["q"], d["k"], d["v"], d["g"], d["beta"], allow_neg_eigval=True)
+    with pytest.raises(ValueError):
+        ops.chunk_kda(d["q"], d["k"], d["v"], d["g"][..., :32], d["beta"])
+    with pytest.raises(ValueError):
+        ops.chunk_kda(d["q"], d["k"], d["v"], d["g"], d["beta"], initial_state=d["h0"].bfloat16())
+    with pytest.raises(NotImplementedError):
+        ops.chunk_kda(d["q"], d["k"], d["v"], d["g"], d["beta"], return_intermediate_states=True)
