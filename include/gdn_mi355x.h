@@ -186,6 +186,21 @@ int gdn_kda_fwd(const void* q, const void* k, const void* v, const void* g, cons
                 float scale, int use_qk_l2norm, int use_gate, int has_lower_bound, float lower_bound, int beta_sigmoid,
                 int allow_neg_eigval, int dtype, int g_dtype, int beta_dtype, void* stream);
 
+/* Backward pass of gdn_kda_fwd: needs the workspace that call filled when it was sized with with_backward = 1, and the
+ * same q, k, v, g, A_log, dt_bias, cu_seqlens and options.  The reference has no hand-written counterpart in its tree
+ * (it differentiates chunk_kda_naive.py:106-221 with autograd; the fused operator's backward,
+ * triton_ascend/chunk.py:172-213, calls kernels of a package that is not part of it).  d_o [B,T,H,V] in `dtype`;
+ * d_final_state [N,H,K,V] fp32 or null.  Written: dq, dk [B,T,H,K] and dv [B,T,H,V] in `dtype`, dg [B,T,H,K] in g_dtype
+ * (gradient of the raw gate input when use_gate is set, of the log decay otherwise), dbeta [B,T,H] in beta_dtype
+ * (gradient of beta as handed in, i.e. before the sigmoid when beta_sigmoid is set), dA_log [H] and ddt_bias [H*K]
+ * fp32 (each may be null; written only with use_gate), d_initial_state [N,H,K,V] fp32 or null. */
+int gdn_kda_bwd(const void* q, const void* k, const void* v, const void* g, const float* A_log, const float* dt_bias,
+                const int64_t* cu_seqlens, const void* d_o, const float* d_final_state, void* dq, void* dk, void* dv,
+                void* dg, void* dbeta, float* dA_log, float* ddt_bias, float* d_initial_state, void* workspace,
+                int64_t workspace_bytes, int B, int T, int N, int H, int K, int V, float scale, int use_qk_l2norm,
+                int use_gate, int has_lower_bound, float lower_bound, int beta_sigmoid, int allow_neg_eigval, int dtype,
+                int g_dtype, int beta_dtype, void* stream);
+
 /* -------- per-kernel timing ------------------------------------------------------------------------
  * op-level counterpart of the reference's step profiler (mindspeed_mm/fsdp/tools/profiler.py:32-147).
  * While enabled, every kernel launch of this library is bracketed by HIP events on its stream (this mode

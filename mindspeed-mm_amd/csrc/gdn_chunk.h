@@ -85,8 +85,16 @@ struct KdaWorkspace {
   int64_t VF;             // T [chunks,H,V/32,2]    v_new
   int64_t HF;             // T [chunks,H,V/32,K/32] state before each chunk
   int64_t fwd_bytes;
-  int64_t GC;             // f32 [chunks,H,64,K]    chunk-local cumulative log decay (kept for a backward pass)
+  // kept for a backward pass
+  int64_t GC;             // f32 [chunks,H,64,K]    chunk-local cumulative log decay
+  int64_t TMR;            // T [chunks,H,64,64]     Tm row-major, as rounded for the tiles
+  int64_t QBT;            // T [chunks,H,K/32,2]    (scale q . e^{G})^T as A operand: tile = (32 columns of K) x (32 tokens)
+  int64_t DVF;            // T [chunks,H,V/32,2]    d(v_new)
+  int64_t DHF;            // T [chunks,H,V/32,K/32] gradient of the state AFTER each chunk
+  int64_t DUMP;           // f32 [chunks,H][dQb | dK2 | P : 64,K each][dAq | a2 : 64,64 each][dD : K]  sums over V of the chunk-local pass
+  int64_t PART;           // f32 [chunks,H][1 + K]  partial sums of dA_log and d(dt_bias)
   int64_t total_bytes;
+  static int64_t dump_floats(int K) { return 3 * 64 * (int64_t)K + 2 * 64 * 64 + K; }
 };
 
 inline KdaWorkspace kda_workspace_layout(const ChunkDims& d, int elem_bytes) {
@@ -107,6 +115,12 @@ inline KdaWorkspace kda_workspace_layout(const ChunkDims& d, int elem_bytes) {
   w.HF = take(nc * H * d.V * d.K * elem_bytes);
   w.fwd_bytes = off;
   w.GC = take(nc * 64 * H * d.K * 4);
+  w.TMR = take(nc * H * 64 * 64 * elem_bytes);
+  w.QBT = take(nc * 64 * H * d.K * elem_bytes);
+  w.DVF = take(nc * 64 * H * d.V * elem_bytes);
+  w.DHF = take(nc * H * d.V * d.K * elem_bytes);
+  w.DUMP = take(nc * H * KdaWorkspace::dump_floats(d.K) * 4);
+  w.PART = take(nc * H * (1 + d.K) * 4);
   w.total_bytes = off;
   return w;
 }

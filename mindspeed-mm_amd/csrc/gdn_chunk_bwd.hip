@@ -34,29 +34,33 @@ namespace gdn {
 // loaders write K twice, rows scaled by e^{G_last-G} (for K dS) and by -beta e^G (for the K^T product), and dO twice,
 // raw and with rows scaled by scale e^G.
 // ---------------------------------------------------------------------------------------------
-template <typename T, int DK, int NW, int STAGES> struct StateBwdSmem {
+template <typename T, int DK, int NW, int STAGES, bool KDA = false> struct StateBwdSmem {
   // one stage, in elements of T
   static constexpr int off_k = 0;                        // K images [2][K/32][2] tiles: rows x e^{G_last-G}, rows x -beta e^G
   static constexpr int off_q = off_k + 2 * 64 * DK;      // Q^T image
   static constexpr int off_tm = off_q + 64 * DK;         // Tm tiles (0,0), (1,0), (1,1)
   static constexpr int off_aq = off_tm + 3 * 1024;       // Aq tiles (0,0), (1,0), (1,1)
   static constexpr int off_do = off_aq + 3 * 1024;       // dO rows of the slabs [2][64][32 NW]: raw, rows x scale e^G
-  static constexpr int off_row = (off_do + 2 * 64 * 32 * NW) * (int)sizeof(T);   // bytes: G_last
-  static constexpr int stage = off_row + 16;
+  static constexpr int off_row = (off_do + 2 * 64 * 32 * NW) * (int)sizeof(T);   // bytes: G_last; KDA: e^{G_last} per key channel [DK]
+  static constexpr int stage = off_row + (KDA ? DK * 4 : 16);
   static constexpr int bytes = STAGES * stage;
   static_assert(bytes <= 160 * 1024, "one CU's LDS");
 };
 
 template <int PIECES, int NT> struct DealB { static constexpr int kPer = (PIECES + NT - 1) / NT; };
 
-template <typename T, int DK, int NW, int NL, int STAGES>
+// KDA (one decay per key channel): kaf and kaf2 hold the two K images ready-made (rows x e^{G_last-G} and rows x
+// -beta e^{G}, channel by channel), qtf the transposed rows of q with scale and decay already applied (so dO is used
+// as it is), G holds e^{G_last} [chunks,Hv,DK]; the rows of dS decay each by their own factor.
+template <typename T, int DK, int NW, int NL, int STAGES, bool KDA = false>
 __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 && NL >= 4) ? 2 : 1) void chunk_state_bwd_kernel(
-    const T* __restrict__ kaf, const T* __restrict__ qtf, const T* __restrict__ ai, const T* __restrict__ aqf,
+    const T* __restrict__ kaf, const T* __restrict__ kaf2, const T* __restrict__ qtf, const T* __restrict__ ai, const T* __restrict__ aqf,
     const T* __restrict__ dO, const float* __restrict__ G, const void* __restrict__ beta, int beta_same,
     const float* __restrict__ dht,
     float* __restrict__ dh0, T* __restrict__ dvf, T* __restrict__ dhf, const int64_t* __restrict__ cu,
     const int* __restrict__ chunk_offsets, int T_len, int Hqk, int Hv, int V, float scale) {
-  using SM = StateBwdSmem<T, DK, NW, STAGES>;
+  using SM = StateBwdSmem<T, DK, NW, STAGES, KDA>;
+  static_assert(!KDA || 64 * NL >= DK, "a loader thread per key channel");
   constexpr int NT = 64 * NL, VEC = Elem<T>::kVec, NKT = DK / 32;   // NT loader threads
   constexpr int PK = 64 * DK / VEC, PTM = 3 * 1024 / VEC, PD = 64 * 32 * NW / VEC, DPR = 32 * NW / VEC;
   constexpr int CK = DealB<PK, NT>::kPer, CTM = DealB<PTM, NT>::kPer, CD = DealB<PD, NT>::kPer;
@@ -74,7 +78,7 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
     // ================= loader waves =================
     const int lt = tid - 64 * NW;
     constexpr int DEPTH = (STAGES == 2) ? 2 : 1;
-    Vec16<T> pk[DEPTH][CK], pq[DEPTH][CK], ptm[DEPTH][CTM], pa[DEPTH][CTM], pd[DEPTH][CD];
+    Vec16<T> pk[DEPTH][CK], pk2[DEPTH][KDA ? CK : 1], pq[DEPTH][CK], ptm[DEPTH][CTM], pa[DEPTH][CTM], pd[DEPTH][CD];
     float pgl[DEPTH], pgk[DEPTH][2], pgd[DEPTH][CD];
     uint32_t pbk[DEPTH][2];   // beta as fetched
     int pnv[DEPTH];
@@ -93,6 +97,7 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
       for (int i = 0; i < CK; ++i) {
         const int idc = imin(lt + i * NT, PK - 1);
         pk[set][i] = ld16(kaf + chq * (64 * DK) + idc * VEC);
+        if constexpr (KDA) pk2[set][i] = ld16(kaf2 + chq * (64 * DK) + idc * VEC);
         pq[set][i] = ld16(qtf + chq * (64 * DK) + idc * VEC);
       }
 #pragma unroll
@@ -105,7 +110,12 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
       for (int i = 0; i < CD; ++i) {   // dO rows of the slabs; rows past the end repeat the last one and are cleared below
         const int idc = imin(lt + i * NT, PD - 1), row = imin(idc / DPR, nvalid - 1), cc = idc % DPR;
         pd[set][i] = ld16(dO + ((tok0 + row) * Hv + h) * V + blockIdx.y * (32 * NW) + cc * VEC);
-        pgd[set][i] = G[ch * 64 + row];
+        if constexpr (!KDA) pgd[set][i] = G[ch * 64 + row];
+      }
+      pnv[set] = nvalid;
+      if constexpr (KDA) {
+        pgl[set] = G[ch * DK + imin(lt, DK - 1)];   // e^{G_last} of this thread's key channel
+        return;
       }
       const float* gc = G + ch * 64;
       // raw values only: arithmetic here would wait for every load issued so far.  The array repeats G_last past the
@@ -117,21 +127,27 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
         pgk[set][j] = gc[32 * j + krow];
         pbk[set][j] = gate_raw<T>(beta, beta_same, (tok0 + imin(32 * j + krow, nvalid - 1)) * Hv + h);
       }
-      pnv[set] = nvalid;
     };
     auto commit = [&](int set, int buf) {
       T* st = reinterpret_cast<T*>(gdn_smem + buf * SM::stage);
       float f1[2], f2[2];
+      if constexpr (!KDA) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        f1[j] = __expf(pgl[set] - pgk[set][j]);
-        f2[j] = (32 * j + krow < pnv[set]) ? -gate_val<T>(pbk[set][j], beta_same) * __expf(pgk[set][j]) : 0.f;
+        for (int j = 0; j < 2; ++j) {
+          f1[j] = __expf(pgl[set] - pgk[set][j]);
+          f2[j] = (32 * j + krow < pnv[set]) ? -gate_val<T>(pbk[set][j], beta_same) * __expf(pgk[set][j]) : 0.f;
+        }
       }
 #pragma unroll
       for (int i = 0; i < CK; ++i) {
         const int idc = imin(lt + i * NT, PK - 1), tj = (idc / (1024 / VEC)) & 1;
-        st16(st + SM::off_k + idc * VEC, scale16<T>(pk[set][i], f1[tj]));
-        st16(st + SM::off_k + 64 * DK + idc * VEC, scale16<T>(pk[set][i], f2[tj]));
+        if constexpr (KDA) {
+          st16(st + SM::off_k + idc * VEC, pk[set][i]);
+          st16(st + SM::off_k + 64 * DK + idc * VEC, pk2[set][i]);
+        } else {
+          st16(st + SM::off_k + idc * VEC, scale16<T>(pk[set][i], f1[tj]));
+          st16(st + SM::off_k + 64 * DK + idc * VEC, scale16<T>(pk[set][i], f2[tj]));
+        }
         st16(st + SM::off_q + idc * VEC, pq[set][i]);
       }
 #pragma unroll
@@ -145,9 +161,14 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
         const int idc = imin(lt + i * NT, PD - 1);
         const Vec16<T> x = idc / DPR < pnv[set] ? pd[set][i] : zero16<T>();
         st16(st + SM::off_do + idc * VEC, x);
-        st16(st + SM::off_do + 64 * 32 * NW + idc * VEC, scale16<T>(x, scale * __expf(pgd[set][i])));
+        if constexpr (KDA) st16(st + SM::off_do + 64 * 32 * NW + idc * VEC, x);
+        else st16(st + SM::off_do + 64 * 32 * NW + idc * VEC, scale16<T>(x, scale * __expf(pgd[set][i])));
       }
       float* row = reinterpret_cast<float*>(gdn_smem + buf * SM::stage + SM::off_row);
+      if constexpr (KDA) {
+        if (lt < DK) row[lt] = pgl[set];
+        return;
+      }
       if (lt == 0) row[0] = pgl[set];
     };
     if (nchunks == 0) return;
@@ -230,7 +251,7 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
     aq[0].load(Aq);                           // tiles (0,0), (1,0), (1,1)
     aq[1].load(Aq + 1024);
     aq[2].load(Aq + 2048);
-    const float eg = __expf(row[0]);
+    const float eg = KDA ? 1.f : __expf(row[0]);
     const int64_t tile0 = ((chunk_base + c) * Hv + h) * (V / 32) + vblk;
 #pragma unroll
     for (int kt = 0; kt < NKT; ++kt) dSb[kt].store_stream(dhf + (tile0 * NKT + kt) * 1024);
@@ -249,8 +270,14 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
     for (int i = 0; i < 2 * NKT; ++i) {       // tile i = (K tile i / 2, token block i % 2)
       if (i + 2 < 2 * NKT) af[(i + 2) % 3].load(Ka + (i + 2) * 1024);
       mma32_ff<T>((i & 1) ? a1 : a0, af[i % 3], dSb[i / 2]);
+      if constexpr (KDA) {
+        const f32x16 dk = rows_ld(row, 32 * (i / 2));   // the decay of each of the tile's 32 key channels
 #pragma unroll
-      for (int r = 0; r < 8; ++r) dS[i / 2][8 * (i & 1) + r] *= eg;
+        for (int r = 0; r < 8; ++r) dS[i / 2][8 * (i & 1) + r] *= dk[8 * (i & 1) + r];
+      } else {
+#pragma unroll
+        for (int r = 0; r < 8; ++r) dS[i / 2][8 * (i & 1) + r] *= eg;
+      }
       GDN_SCHED_FENCE();
     }
     AccB<T> dvb[2], rb[2], tf[3];
@@ -336,14 +363,19 @@ template <typename T, int DK> struct BwdLocalSmem {
   static_assert(4 * Patch<T>::kElems <= raw_elems && 2 * (DK / 32) * 1024 <= raw_elems, "epilogue tenants fit");
 };
 
-template <typename T, int DK>
+// KDA (one decay per key channel): the sums over V are the same, what follows them is not.  The kernel then stops after
+// its main loop (dv is written there) and leaves the sums in kda_dump, per chunk and head
+//   [dQb = dO S^T | dK2 = V' dS'^T | P = dV' S^T : 64 x DK each][dAq = dO V'^T | a2 = dV' V^T : 64 x 64 each, lower tiles]
+//   [dD = sum_v dS' . S : DK]    (fp32)
+// for kda_bwd_finish_kernel; G is not read and beta is the transformed beta in fp32.
+template <typename T, int DK, bool KDA = false>
 __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_local_kernel(
     const T* __restrict__ qtf, const T* __restrict__ kaf, const T* __restrict__ v, const void* __restrict__ beta, int beta_same,
     const float* __restrict__ G, const T* __restrict__ Ai, const T* __restrict__ vf, const T* __restrict__ dvf,
     const T* __restrict__ dO, const T* __restrict__ hf, const T* __restrict__ dhf, const float* __restrict__ rstd_q,
     const float* __restrict__ rstd_k, T* dq, T* dk, T* __restrict__ dv_out, void* __restrict__ dbeta,
     float* __restrict__ dg, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N,
-    int Hqk, int Hv, int V, float scale, int hh, TokenStrides ts) {
+    int Hqk, int Hv, int V, float scale, int hh, TokenStrides ts, float* __restrict__ kda_dump) {
   using SM = BwdLocalSmem<T, DK>;
   constexpr int NKT = DK / 32, VEC = Elem<T>::kVec, KG = AccK<T>::kGroups;
   static_assert(NKT <= 4, "one 32-column block of K per wave");
@@ -438,7 +470,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
 
   if (tid < 64) {   // the row vectors: all requests first, the same ones on every path
     const int tc = imin(tid, nvalid - 1);
-    const float gv = G[ch * 64 + tc];
+    const float gv = KDA ? 0.f : G[ch * 64 + tc];
     const uint32_t braw = gate_raw<T>(beta, beta_same, (tok0 + tc) * Hv + h);
     float rq1 = 1.f, rk1v = 1.f;
     if (l2) {
@@ -493,7 +525,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       issue_shared(vblk + 1);
       issue_priv(vblk + 1);
       if ((vblk & 1) == 0 && vblk + 2 < nblk) issue_raw((vblk >> 1) + 1);   // its buffer was last read in block vblk - 1
-    } else {
+    } else if constexpr (!KDA) {
       issue_epilogue(((vblk >> 1) + 1) & 1);
     }
 #pragma unroll
@@ -545,6 +577,32 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       if (32 * rj + l32 < nvalid)
         acc_to_lds_t<T>(Rt, dv_out + (tok0 + 32 * rj + l32) * ts.dv + h * V + 32 * vblk, 0, 0, 0);
     }
+  }
+  if constexpr (KDA) {
+    constexpr int64_t kDumpFloats = 3 * 64 * DK + 2 * 64 * 64 + DK;
+    float* dump = kda_dump + ch * kDumpFloats;
+    if (has_k) {
+#pragma unroll
+      for (int ri = 0; ri < 2; ++ri)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int at = (32 * ri + acc_row(r)) * DK + 32 * cj + l32;
+          dump[at] = dQi[ri][r];
+          dump[64 * DK + at] = dKi[ri][r];
+          dump[2 * 64 * DK + at] = dWa[ri][r];
+        }
+      sds += __shfl_xor(sds, 32);   // the other half of the V block's rows
+      if (lane < 32) dump[3 * 64 * DK + 2 * 64 * 64 + 32 * cj + lane] = sds;
+    }
+    if (lower) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int at = (32 * ti + acc_row(r)) * 64 + 32 * tj + l32;
+        dump[3 * 64 * DK + at] = ds[r];
+        dump[3 * 64 * DK + 64 * 64 + at] = a2[r];
+      }
+    }
+    return;
   }
   sds = wave_sum(sds);
   if (lane == 0) wsum[wave] = sds;
@@ -814,7 +872,7 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     constexpr int smem = StateBwdSmem<T, DK, NWS, STAGES>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
     GDN_LAUNCH(kKernStateBwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NWS)), dim3(64 * (NWS + NLS)), smem, st, (const T*)KAF,
-               (const T*)QTF, Ai, AQ, (const T*)dO, G, beta, beta_same, dht, dh0, DVF, DHF, cu, chunk_offsets, d.T, d.Hqk, d.Hv, d.V,
+               (const T*)nullptr, (const T*)QTF, Ai, AQ, (const T*)dO, G, beta, beta_same, dht, dh0, DVF, DHF, cu, chunk_offsets, d.T, d.Hqk, d.Hv, d.V,
                scale);
   }
   {
@@ -824,7 +882,7 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     for (int hh = 0; hh < d.Hv / d.Hqk; ++hh)
       GDN_LAUNCH(kKernBwdLocal, st, kern, dim3(nc, d.Hqk), dim3(kThreads), smem, st, QTF, (const T*)KAF, (const T*)v,
                  beta, beta_same, G, Ai, VF, (const T*)DVF, (const T*)dO, HF, (const T*)DHF, rstd_q, rstd_k, (T*)dq, (T*)dk,
-                 (T*)dv, dbeta, dg, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale, hh, d.strides());
+                 (T*)dv, dbeta, dg, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale, hh, d.strides(), (float*)nullptr);
   }
   return (int)hipGetLastError();
 }
@@ -882,3 +940,5 @@ extern "C" int gdn_chunk_bwd(const void* q, const void* k, const void* v, const 
                                0, dg, dbeta, d_initial_state, workspace, workspace_bytes, B, T, N, Hqk, Hv, K, V, scale,
                                use_qk_l2norm, dtype, 0, stream);
 }
+
+#include "gdn_kda_bwd.h"

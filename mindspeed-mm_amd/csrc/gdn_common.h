@@ -725,6 +725,52 @@ __device__ __forceinline__ float wave_sum(float v) {
   return half_wave_sum(v);
 }
 
+// A [64, DK] q or k tile on its way into LDS, in two steps so that the requests of both tiles (and of the gates) are
+// in flight together instead of one 16-byte piece at a time: tile_qk_request() issues this thread's loads (rows past
+// the end of the sequence are zero), tile_qk_finish() applies the optional l2 norm (y = x rsqrt(sum x^2 + 1e-6) over
+// the row, modeling_qwen3_5.py:392-395; fp32 arithmetic, result rounded to T; a row sits on DK/VEC neighbouring lanes
+// that combine their partial sums with data-parallel-primitive moves), writes the tile to
+// LDS and, on request, the normalised rows (row stride y_stride) and 1/|x| (stride rstd_stride) to global memory.
+template <typename T, int DK> struct TileQK {
+  static constexpr int V = Elem<T>::kVec, CPR = DK / V, PT = 64 * CPR / kThreads;   // lanes per row; pieces per thread
+  static_assert((64 * CPR) % kThreads == 0, "every thread takes the same number of pieces");
+  Vec16<T> x[PT];
+};
+template <typename T, int DK>
+__device__ __forceinline__ void tile_qk_request(TileQK<T, DK>& t, const T* g, int64_t row_stride, int nvalid, int tid) {
+  constexpr int V = TileQK<T, DK>::V, CPR = TileQK<T, DK>::CPR;
+#pragma unroll
+  for (int i = 0; i < TileQK<T, DK>::PT; ++i) {
+    const int c = tid + i * kThreads, row = c / CPR, cc = c % CPR;
+    t.x[i] = ld16(g + (int64_t)imin(row, nvalid - 1) * row_stride + cc * V);   // the same load on every path
+  }
+}
+template <typename T, int DK>
+__device__ __forceinline__ void tile_qk_finish(TileQK<T, DK>& t, T* lds, int ld, int nvalid, int tid, bool l2norm,
+                                               T* y_out, int64_t y_stride, float* rstd_out, int64_t rstd_stride) {
+  constexpr int V = TileQK<T, DK>::V, CPR = TileQK<T, DK>::CPR;
+#pragma unroll
+  for (int i = 0; i < TileQK<T, DK>::PT; ++i) {
+    const int c = tid + i * kThreads, row = c / CPR, cc = c % CPR;
+    const bool ok = row < nvalid;
+    Vec16<T> x = ok ? t.x[i] : zero16<T>();
+    if (l2norm) {   // uniform: every lane takes part in the shuffles
+      float f[V], ss = 0.f;
+      unpack16<T>(x, f);
+#pragma unroll
+      for (int e = 0; e < V; ++e) ss += f[e] * f[e];
+      ss = lane_group_sum<CPR>(ss);
+      const float r = rsqrtf(ss + 1e-6f);
+#pragma unroll
+      for (int e = 0; e < V; ++e) f[e] *= r;
+      x = pack16<T>(f);
+      if (ok && y_out != nullptr) st16(y_out + (int64_t)row * y_stride + cc * V, x);
+      if (ok && rstd_out != nullptr && cc == 0) rstd_out[(int64_t)row * rstd_stride] = r;
+    }
+    st16(lds + row * ld + cc * V, x);
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // Packed-sequence bookkeeping.  chunk_offsets[n] = number of 64-token chunks before sequence n
 // (chunk_offsets[N] = total); built on the device by gdn_chunk_table_kernel so that no host sync is

@@ -1,0 +1,504 @@
+// KDA (Kimi delta attention) backward.  Included at the end of gdn_chunk_bwd.hip: the reverse recurrence and the sums
+// over V of the chunk-local pass are that file's kernels in their KDA modes (chunk_state_bwd_kernel,
+// chunk_bwd_local_kernel, which also writes dv); this file turns those sums into the gradients of q, k, the gate input
+// and beta, which is where the decay per key channel changes the algebra.  The reference differentiates its pure
+// PyTorch statement with autograd (mindspeed_mm/fsdp/ops/kda/chunk_kda_naive.py:106-221); the equations below are the
+// hand-derived backward of that statement.
+//
+// Forward, per chunk (G cumulative log decay [64,K], b = transformed beta, S the state before the chunk):
+//   Kp = k . e^{G}   K1 = -b Kp   K2 = k . e^{G_last-G}   Qb = scale q . e^{G}
+//   L_ij = b_i sum_d k_id k_jd e^{G_id-G_jd} (i>j)   Tm = (I+L)^-1   Aq_ij = scale sum_d q_id k_jd e^{G_id-G_jd} (i>=j)
+//   z = b v + K1 S    V' = Tm z    O = Qb S + Aq V'    S' = e^{G_last} . S + K2^T V'
+// What arrives (sums over V, fp32): dQb = dO S^T, dK2 = V' dS'^T, P = dV' S^T, dAq = tril(dO V'^T), a2 = dV' V^T,
+// dD = sum_v dS' . S.  Then
+//   dTm = stril(b_j (a2 - P Kp^T))    dL = -stril(Tm^T dTm Tm^T)    dK1 = Tm^T P    <R_t, v_t> = sum_i Tm_it a2_it
+//   U_i  = sum_{j<i}  dL_ij        k_j . e^{G_i-G_j}          Uq_i = sum_{j<=i} scale dAq_ij k_j . e^{G_i-G_j}
+//   W_j  = sum_{i>=j} (dL_ij b_i k_i + scale dAq_ij q_i) . e^{G_i-G_j}
+//   dq^ = scale e^{G} . dQb + Uq
+//   dk^ = -b e^{G} . dK1 + e^{G_last-G} . dK2 + b U + W
+//   dG  = q^ . dq^ + k^ . (-b e^{G} . dK1 + b U - e^{G_last-G} . dK2 - W)         per token and channel
+//   dG_last = sum_i k^_i . e^{G_last-G_i} . dK2_i + dD . e^{G_last}               per channel
+//   db_i = <R_i, v_i> + sum_d k^_id (U_id - e^{G_id} dK1_id)
+//   dg_t = sum_{i>=t} dG_i + dG_last, then back through the gate, the l2 norm and the sigmoid of beta.
+// The decay-weighted sums over a chunk use the split of the forward pass: within the two 32-token blocks term by term in
+// fp32 with the exact exponent, between the blocks on the matrix cores with rows rescaled at the block boundary (for
+// fp32 operands, whose tiles would not fit LDS beside everything else, every pair is summed term by term).
+#pragma once
+#include "gdn_kda_common.h"
+
+namespace gdn {
+
+template <typename T, int DK> struct KdaBwdSmem {
+  static constexpr int LDK = lds_ld<T>(DK), LDG = DK + 4, L64 = lds_ld<T>(64);
+  static constexpr bool FULL = sizeof(T) == 4;   // no rescaled images: every pair term by term
+  static constexpr int tile = 64 * LDK * (int)sizeof(T), gmat = 64 * LDG * 4, mat = 64 * L64 * (int)sizeof(T);
+  static constexpr int off_ks = 0;                   // k^ rows
+  static constexpr int off_qs = off_ks + tile;       // first P as T, then q^ rows
+  static constexpr int off_gs = off_qs + tile;       // first Kp as T (64 rows), then G rows (fp32)
+  static constexpr int off_tm = off_gs + gmat;       // Tm row-major; later, with the next two, the store patches
+  static constexpr int off_m1 = off_tm + mat;        // dTm, then dL
+  static constexpr int off_m2 = off_m1 + mat;        // X = Tm^T dTm, then scale dAq
+  static constexpr int off_xi = off_m2 + mat;        // rescaled rows [b k ; q] of tokens 32..63 (not FULL)
+  static constexpr int off_xr = off_xi + (FULL ? 0 : tile);       // rescaled rows k of tokens 0..31
+  static constexpr int off_row = off_xr + (FULL ? 0 : tile / 2);
+  // beta, 1/|q|, 1/|k| [64 each]; per-wave row sums <q^,dq^>, <k^,dk^>, db, <R,v> [256 each]; 8 scalars
+  static constexpr int bytes = off_row + (3 * 64 + 4 * 256 + 8) * 4;
+  static_assert(tile <= gmat, "Kp fits where G will be");
+  static_assert(4 * Patch<T>::kElems * (int)sizeof(T) <= 3 * mat, "store patches fit");
+  static_assert(bytes <= 160 * 1024, "one CU's LDS");
+};
+
+template <typename T, int DK>
+__global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
+    const T* __restrict__ q, const T* __restrict__ k, const void* __restrict__ g, const float* __restrict__ A_log,
+    const float* __restrict__ dt_bias, const float* __restrict__ bhat, const float* __restrict__ GC,
+    const T* __restrict__ TMR, const float* __restrict__ dumps, const int64_t* __restrict__ cu,
+    const int* __restrict__ chunk_offsets, T* __restrict__ dq, T* __restrict__ dk, void* __restrict__ dg,
+    void* __restrict__ dbeta, float* __restrict__ part, int T_len, int N, int H, float scale, KdaFlags fl) {
+  using SM = KdaBwdSmem<T, DK>;
+  constexpr int LDK = SM::LDK, LDG = SM::LDG, L64 = SM::L64, VEC = Elem<T>::kVec, CPR = DK / VEC, NKT = DK / 32;
+  constexpr bool FULL = SM::FULL;
+  T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
+  T* Qs = reinterpret_cast<T*>(gdn_smem + SM::off_qs);
+  T* Pt = Qs;
+  float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_gs);
+  T* Kp = reinterpret_cast<T*>(gdn_smem + SM::off_gs);
+  T* TmT = reinterpret_cast<T*>(gdn_smem + SM::off_tm);
+  T* M1 = reinterpret_cast<T*>(gdn_smem + SM::off_m1);
+  T* M2 = reinterpret_cast<T*>(gdn_smem + SM::off_m2);
+  T* XI = reinterpret_cast<T*>(gdn_smem + SM::off_xi);
+  T* XR = reinterpret_cast<T*>(gdn_smem + SM::off_xr);
+  float* bs = reinterpret_cast<float*>(gdn_smem + SM::off_row);
+  float* rsq = bs + 64;
+  float* rsk = rsq + 64;
+  float* rq = rsk + 64;     // per-wave row sums (rows_add / rows_ld4)
+  float* rk = rq + 256;
+  float* rb = rk + 256;
+  float* rv = rb + 256;
+  float* wsum = rv + 256;
+
+  const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
+  if (s.nvalid <= 0) return;
+  const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, wave = tid >> 6;
+  const int h = blockIdx.y, nvalid = s.nvalid;
+  const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk, hk = (int64_t)H * DK;
+  const int64_t ch = (int64_t)blockIdx.x * H + h;
+  const int ti = wave >> 1, tj = wave & 1, cj = wave;
+  const bool lower = tj <= ti, has_k = wave < NKT;
+  const float* dump = dumps + ch * (3 * 64 * DK + 2 * 64 * 64 + DK);
+  const float* dQb = dump, *dK2 = dump + 64 * DK, *Pm = dump + 2 * 64 * DK;
+  const float* dAq = dump + 3 * 64 * DK, *a2m = dAq + 64 * 64, *dD = a2m + 64 * 64;
+  const float* Gc = GC + ch * 64 * DK;
+
+  // ---- phase A0: k^ rows; P and Tm as operands; beta ----
+  TileQK<T, DK> kt;
+  tile_qk_request<T, DK>(kt, k + tok0 * hk + h * DK, hk, nvalid, tid);
+  if (tid < 64) {
+    bs[tid] = tid < nvalid ? bhat[(tok0 + tid) * H + h] : 0.f;
+    rsq[tid] = 1.f;
+    rsk[tid] = 1.f;
+  }
+  rq[tid] = 0.f; rk[tid] = 0.f; rb[tid] = 0.f; rv[tid] = 0.f;
+  for (int c = tid; c < 64 * CPR; c += kThreads) {
+    const int row = c / CPR, cc = c % CPR;
+    float f[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) f[e] = Pm[row * DK + cc * VEC + e];
+    st16(Pt + row * LDK + cc * VEC, pack16<T>(f));
+  }
+  {
+    constexpr int C64 = 64 / VEC;
+    for (int c = tid; c < 64 * C64; c += kThreads)
+      st16(TmT + (c / C64) * L64 + (c % C64) * VEC, ld16(TMR + ch * 4096 + (c / C64) * 64 + (c % C64) * VEC));
+  }
+  GDN_LDS_BARRIER();   // the row vectors are initialised before the norm below writes 1/|k| over its entries
+  tile_qk_finish<T, DK>(kt, Ks, LDK, nvalid, tid, fl.l2norm != 0, nullptr, 0, rsk, 1);
+  GDN_LDS_BARRIER();
+  for (int c = tid; c < 64 * CPR; c += kThreads) {   // Kp = k^ . e^{G}
+    const int row = c / CPR, cc = c % CPR;
+    float f[VEC];
+    unpack16<T>(ld16(Ks + row * LDK + cc * VEC), f);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) f[e] *= __expf(Gc[row * DK + cc * VEC + e]);
+    st16(Kp + row * LDK + cc * VEC, pack16<T>(f));
+  }
+  GDN_LDS_BARRIER();
+
+  // ---- phase A1: dTm = stril(b_j (a2 - P Kp^T)), one 32x32 tile per wave; <R_t, v_t> from Tm and a2 ----
+  {
+    f32x16 x = acc_zero();
+    if (lower) mma32<T, DK, true, true>(x, Pt + 32 * ti * LDK, LDK, Kp + 32 * tj * LDK, LDK);
+    const int j = 32 * tj + l32;
+    const float bj = bs[j];
+    float sv = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int i = 32 * ti + acc_row(r);
+      const float a2v = lower ? a2m[i * 64 + j] : 0.f;
+      sv += a2v * Elem<T>::to_f(TmT[i * L64 + j]);
+      M1[i * L64 + j] = Elem<T>::from_f(i > j ? bj * (a2v - x[r]) : 0.f);
+    }
+    sv += __shfl_xor(sv, 32);
+    if (lane < 32) rv[wave * 64 + 32 * tj + lane] = sv;
+  }
+  GDN_LDS_BARRIER();
+  // ---- phase A2: X = Tm^T dTm (the tiles dL needs: a >= the column block) ----
+  {
+    f32x16 x = acc_zero();
+    if (lower) mma32<T, 64, false, false>(x, TmT + 32 * ti, L64, M1 + 32 * tj, L64);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) M2[(32 * ti + acc_row(r)) * L64 + 32 * tj + l32] = Elem<T>::from_f(x[r]);
+  }
+  GDN_LDS_BARRIER();
+  // ---- phase A3: dL = -stril(X Tm^T); dK1 = Tm^T P for this wave's 32 key channels; scale dAq ----
+  f32x16 dK1[2];
+  dK1[0] = acc_zero();
+  dK1[1] = acc_zero();
+  f32x16 dl = acc_zero(), sa;
+  if (lower) mma32<T, 64, true, true>(dl, M2 + 32 * ti * L64, L64, TmT + 32 * tj * L64, L64);
+  if (has_k) {
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri) mma32<T, 64, false, false>(dK1[ri], TmT + 32 * ri, L64, Pt + 32 * cj, LDK);
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int i = 32 * ti + acc_row(r), j = 32 * tj + l32;
+    dl[r] = i > j ? -dl[r] : 0.f;
+    sa[r] = (lower && i >= j) ? scale * dAq[i * 64 + j] : 0.f;
+  }
+  GDN_LDS_BARRIER();   // dTm, X, P, Kp are consumed
+  // ---- phase A4: the coefficient matrices in place of dTm and X; q^ rows and G in place of P and Kp ----
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int at = (32 * ti + acc_row(r)) * L64 + 32 * tj + l32;
+    M1[at] = Elem<T>::from_f(dl[r]);
+    M2[at] = Elem<T>::from_f(sa[r]);
+  }
+  {
+    TileQK<T, DK> qt;
+    tile_qk_request<T, DK>(qt, q + tok0 * hk + h * DK, hk, nvalid, tid);
+    tile_qk_finish<T, DK>(qt, Qs, LDK, nvalid, tid, fl.l2norm != 0, nullptr, 0, rsq, 1);
+  }
+  for (int c = tid; c < 64 * (DK / 4); c += kThreads) {
+    const int row = c / (DK / 4), c4 = c % (DK / 4);
+    *reinterpret_cast<f32x4*>(Gs + row * LDG + 4 * c4) = *reinterpret_cast<const f32x4*>(Gc + row * DK + 4 * c4);
+  }
+  GDN_LDS_BARRIER();
+
+  // ---- phase B: the decay-weighted sums.  A wave owns 32 key channels, a lane one of them and, per 32-token block,
+  //      the 16 rows of its accumulator registers ----
+  const int d = 32 * cj + l32;
+  float Gi[2][16], ki[2][16], qi[2][16], U[2][16], Uq[2][16], W[2][16];
+  if (has_k) {
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int i = 32 * ri + acc_row(r);
+        Gi[ri][r] = Gs[i * LDG + d];
+        ki[ri][r] = Elem<T>::to_f(Ks[i * LDK + d]);
+        qi[ri][r] = Elem<T>::to_f(Qs[i * LDK + d]);
+        U[ri][r] = 0.f; Uq[ri][r] = 0.f; W[ri][r] = 0.f;
+      }
+  }
+  if constexpr (!FULL) {
+    // between the blocks: rows rescaled around the decay at the boundary, [b k ; q]_i e^{G_i-G_31} and k_j e^{G_31-G_j}
+    for (int c = tid; c < 96 * CPR; c += kThreads) {
+      const int r = c / CPR, cc = c % CPR;
+      const int src = r < 32 ? 32 + r : (r < 64 ? r : r - 64);
+      const T* from = (r >= 32 && r < 64) ? Qs : Ks;
+      float f[VEC], gi[VEC], gr[VEC];
+      unpack16<T>(ld16(from + src * LDK + cc * VEC), f);
+      ld_f32<VEC>(Gs + src * LDG + cc * VEC, gi);
+      ld_f32<VEC>(Gs + 31 * LDG + cc * VEC, gr);
+      const float b = r < 32 ? bs[src] : 1.f;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) f[e] *= b * __expf(r < 64 ? gi[e] - gr[e] : gr[e] - gi[e]);
+      T* to = r < 64 ? XI + r * LDK : XR + (r - 64) * LDK;
+      st16(to + cc * VEC, pack16<T>(f));
+    }
+    GDN_LDS_BARRIER();
+    if (has_k) {
+      const float g31 = Gs[31 * LDG + d];
+      f32x16 u = acc_zero(), uq = acc_zero(), w = acc_zero();
+      mma32<T, 32, true, false>(u, M1 + 32 * L64, L64, XR + 32 * cj, LDK);     // sum_j dL[32+i][j] KR[j][d]
+      mma32<T, 32, true, false>(uq, M2 + 32 * L64, L64, XR + 32 * cj, LDK);
+      mma32<T, 32, false, false>(w, M1 + 32 * L64, L64, XI + 32 * cj, LDK);    // sum_i dL[32+i][j] (b k)_i[d]
+      mma32<T, 32, false, false>(w, M2 + 32 * L64, L64, XI + 32 * LDK + 32 * cj, LDK);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float e1 = __expf(Gi[1][r] - g31);
+        U[1][r] = u[r] * e1;
+        Uq[1][r] = uq[r] * e1;
+        W[0][r] = w[r] * __expf(g31 - Gi[0][r]);
+      }
+    }
+  }
+  if (has_k) {
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri) {
+      // rows i of this lane against the earlier rows j of the block (of the chunk when FULL)
+      for (int jj = FULL ? 0 : 32 * ri; jj <= 32 * ri + 31; ++jj) {
+        const float gj = Gs[jj * LDG + d], kj = Elem<T>::to_f(Ks[jj * LDK + d]);
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+          if (32 * ri + 8 * qd + 7 < jj) continue;   // none of the group's rows reaches jj (same for every lane)
+#pragma unroll
+          for (int m = 0; m < 4; ++m) {
+            const int r = 4 * qd + m, i = 32 * ri + acc_row(r);
+            const float t = kj * __expf(i >= jj ? Gi[ri][r] - gj : 0.f);
+            U[ri][r] += Elem<T>::to_f(M1[i * L64 + jj]) * t;    // coefficients are zero where i < jj
+            Uq[ri][r] += Elem<T>::to_f(M2[i * L64 + jj]) * t;
+          }
+        }
+      }
+      // rows j of this lane against the later rows i
+      for (int ii = 32 * ri; ii <= (FULL ? 63 : 32 * ri + 31); ++ii) {
+        const float gi = Gs[ii * LDG + d], kb = bs[ii] * Elem<T>::to_f(Ks[ii * LDK + d]), qv = Elem<T>::to_f(Qs[ii * LDK + d]);
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+          if (32 * ri + 8 * qd > ii) continue;
+#pragma unroll
+          for (int m = 0; m < 4; ++m) {
+            const int r = 4 * qd + m, j = 32 * ri + acc_row(r);
+            const float e = __expf(ii >= j ? gi - Gi[ri][r] : 0.f);
+            W[ri][r] += (Elem<T>::to_f(M1[ii * L64 + j]) * kb + Elem<T>::to_f(M2[ii * L64 + j]) * qv) * e;
+          }
+        }
+      }
+    }
+  }
+  // ---- phase B3: the gradients of q^, k^, G per token and channel; row sums for beta and the l2 norm ----
+  f32x16 dqh[2], dkh[2], dGv[2];
+  float gl_sum = 0.f;
+  if (has_k) {
+    const float glast = Gs[63 * LDG + d];
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri) {
+      f32x16 pq, pk, pb;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int i = 32 * ri + acc_row(r);
+        const float eG = __expf(Gi[ri][r]), b = bs[i];
+        const float t1 = -b * eG * dK1[ri][r];
+        const float t2 = __expf(glast - Gi[ri][r]) * dK2[i * DK + d];
+        dqh[ri][r] = scale * eG * dQb[i * DK + d] + Uq[ri][r];
+        dkh[ri][r] = t1 + t2 + b * U[ri][r] + W[ri][r];
+        dGv[ri][r] = qi[ri][r] * dqh[ri][r] + ki[ri][r] * (t1 + b * U[ri][r] - t2 - W[ri][r]);
+        gl_sum += ki[ri][r] * t2;
+        pq[r] = qi[ri][r] * dqh[ri][r];
+        pk[r] = ki[ri][r] * dkh[ri][r];
+        pb[r] = ki[ri][r] * (U[ri][r] - eG * dK1[ri][r]);
+      }
+      rows_add(pq, rq, 32 * ri);
+      rows_add(pk, rk, 32 * ri);
+      rows_add(pb, rb, 32 * ri);
+    }
+  }
+  GDN_LDS_BARRIER();   // row sums are complete; the matrices are dead: their place takes the store patches
+
+  // ---- phase B4: l2 norm backward, dq and dk out; dg by a reverse cumulative sum, back through the gate ----
+  IdentityFrag<T> id;
+  id.init();
+  T* patch = TmT + wave * Patch<T>::kElems;
+  float da_sum = 0.f;
+  if (has_k) {
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri) {
+      if (fl.l2norm) {
+        const f32x16 dotq = rows_ld4(rq, 32 * ri), dotk = rows_ld4(rk, 32 * ri);
+        const f32x16 sq = rows_ld(rsq, 32 * ri), sk = rows_ld(rsk, 32 * ri);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          dqh[ri][r] = (dqh[ri][r] - dotq[r] * qi[ri][r]) * sq[r];
+          dkh[ri][r] = (dkh[ri][r] - dotk[r] * ki[ri][r]) * sk[r];
+        }
+      }
+      const int64_t at = (tok0 + 32 * ri) * hk + h * DK + 32 * cj;
+      acc_store_rows<T, false>(dqh[ri], id, patch, dq + at, hk, nvalid - 32 * ri);
+      acc_store_rows<T, false>(dkh[ri], id, patch, dk + at, hk, nvalid - 32 * ri);
+    }
+    // dG_last: column sum over all rows of this channel, plus the decay of the state
+    gl_sum += __shfl_xor(gl_sum, 32);
+    const float dglast = gl_sum + dD[d] * __expf(Gs[63 * LDG + d]);
+    // suffix sums down the tokens.  Rows of a block in token order: group qd = 0..3, half-wave 0 then 1, m = 0..3
+    float so[2][4], sx[2][4], blk[2];
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri) {
+      blk[ri] = 0.f;
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        so[ri][qd] = dGv[ri][4 * qd] + dGv[ri][4 * qd + 1] + dGv[ri][4 * qd + 2] + dGv[ri][4 * qd + 3];
+        sx[ri][qd] = __shfl_xor(so[ri][qd], 32);
+        blk[ri] += so[ri][qd] + sx[ri][qd];
+      }
+    }
+    const bool first_half = lane < 32;
+    const float a = fl.use_gate ? __expf(A_log[h]) : 0.f;
+    const float bias = (fl.use_gate && dt_bias != nullptr) ? dt_bias[h * DK + d] : 0.f;
+    const bool g32 = sizeof(T) == 4 || fl.g_f32;
+    float dt_sum = 0.f;
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri) {
+      f32x16 dgr;
+      float later = ri == 0 ? blk[1] : 0.f;     // everything after the group being handled
+#pragma unroll
+      for (int qd = 3; qd >= 0; --qd) {
+        float run = later + (first_half ? sx[ri][qd] : 0.f);
+#pragma unroll
+        for (int m = 3; m >= 0; --m) {
+          const int r = 4 * qd + m, i = 32 * ri + acc_row(r);
+          run += dGv[ri][r];
+          float x = run + dglast;     // d(log decay of token i, channel d)
+          if (fl.use_gate) {
+            const int64_t gat = (tok0 + imin(i, nvalid - 1)) * hk + h * DK + d;
+            float raw;
+            if (g32) raw = reinterpret_cast<const float*>(g)[gat];
+            else { T t; if constexpr (sizeof(T) == 2) t.bits = reinterpret_cast<const uint16_t*>(g)[gat]; raw = Elem<T>::to_f(t); }
+            raw += bias;
+            if (fl.has_lower_bound) {
+              const float sg = kda_sigmoid(a * raw), ds_ = fl.lower_bound * sg * (1.f - sg);
+              if (i < nvalid) da_sum += x * ds_ * a * raw;
+              x *= ds_ * a;
+            } else {
+              if (i < nvalid) da_sum += x * (-a * kda_softplus(raw));
+              x *= -a * kda_sigmoid(raw);
+            }
+          }
+          if (i >= nvalid) x = 0.f;
+          dt_sum += x;
+          dgr[r] = x;
+        }
+        later += so[ri][qd] + sx[ri][qd];
+      }
+      if (g32) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int i = 32 * ri + acc_row(r);
+          if (i < nvalid) reinterpret_cast<float*>(dg)[(tok0 + i) * hk + h * DK + d] = dgr[r];
+        }
+      } else {
+        acc_store_rows<T, false>(dgr, id, patch, reinterpret_cast<T*>(dg) + (tok0 + 32 * ri) * hk + h * DK + 32 * cj, hk,
+                                 nvalid - 32 * ri);
+      }
+    }
+    dt_sum += __shfl_xor(dt_sum, 32);
+    if (lane < 32) part[ch * (1 + DK) + 1 + d] = dt_sum;
+    da_sum = wave_sum(da_sum);
+  }
+  if (lane == 0) wsum[wave] = has_k ? da_sum : 0.f;
+  GDN_LDS_BARRIER();
+  if (tid == 0) part[ch * (1 + DK)] = wsum[0] + wsum[1] + wsum[2] + wsum[3];
+  if (tid < 64 && tid < nvalid) {
+    float x = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) x += rb[w * 64 + tid] + rv[w * 64 + tid];
+    if (fl.beta_sigmoid) { const float b = bs[tid]; x *= b * (1.f - (fl.beta_x2 ? 0.5f * b : b)); }
+    gate_st<T>(dbeta, fl.beta_f32 ? 0 : 1, (tok0 + tid) * H + h, x);
+  }
+}
+
+// dA_log [H] and d(dt_bias) [H*K] from the per-chunk partial sums
+__global__ __launch_bounds__(kThreads) void kda_bwd_reduce_kernel(const float* __restrict__ part, const int64_t* cu,
+                                                                 const int* __restrict__ chunk_offsets, int N, int nc,
+                                                                 int H, int K, float* __restrict__ dA_log,
+                                                                 float* __restrict__ ddt_bias) {
+  const int h = blockIdx.x, t = threadIdx.x;
+  const int n = cu != nullptr ? chunk_offsets[N] : nc;
+  if (t > K) return;
+  float x = 0.f;
+  for (int c = 0; c < n; ++c) x += part[((int64_t)c * H + h) * (1 + K) + t];
+  if (t == 0) { if (dA_log != nullptr) dA_log[h] = x; }
+  else if (ddt_bias != nullptr) ddt_bias[h * K + t - 1] = x;
+}
+
+template <typename T, int DK, int NWS, int NLS, int STAGES>
+static int kda_bwd_launch(const ChunkDims& d, const KdaWorkspace& L, const void* q, const void* k, const void* v,
+                          const void* g, const float* A_log, const float* dt_bias, const int64_t* cu, const void* dO,
+                          const float* dht, void* dq, void* dk, void* dv, void* dg, void* dbeta, float* dA_log,
+                          float* ddt_bias, float* dh0, unsigned char* ws, float scale, const KdaFlags& fl, hipStream_t st) {
+  const int H = d.Hv;
+  const int nc = (int)d.max_chunks();
+  const int* chunk_offsets = reinterpret_cast<const int*>(ws + L.chunk_offsets);
+  const float* bhat = reinterpret_cast<const float*>(ws + L.bhat);
+  const float* dec = reinterpret_cast<const float*>(ws + L.dec);
+  const T* Ai = reinterpret_cast<const T*>(ws + L.Ai);
+  const T* AQ = reinterpret_cast<const T*>(ws + L.AQ);
+  const T* K1F = reinterpret_cast<const T*>(ws + L.K1F);
+  const T* K2F = reinterpret_cast<const T*>(ws + L.K2F);
+  const T* VF = reinterpret_cast<const T*>(ws + L.VF);
+  const T* HF = reinterpret_cast<const T*>(ws + L.HF);
+  const float* GC = reinterpret_cast<const float*>(ws + L.GC);
+  const T* TMR = reinterpret_cast<const T*>(ws + L.TMR);
+  const T* QBT = reinterpret_cast<const T*>(ws + L.QBT);
+  T* DVF = reinterpret_cast<T*>(ws + L.DVF);
+  T* DHF = reinterpret_cast<T*>(ws + L.DHF);
+  float* DUMP = reinterpret_cast<float*>(ws + L.DUMP);
+  float* PART = reinterpret_cast<float*>(ws + L.PART);
+  {
+    auto kern = chunk_state_bwd_kernel<T, DK, NWS, NLS, STAGES, true>;
+    constexpr int smem = StateBwdSmem<T, DK, NWS, STAGES, true>::bytes;
+    if (int e = set_lds_b(kern, smem)) return e;
+    GDN_LAUNCH(kKernStateBwd, st, kern, dim3(d.N * H, d.V / (32 * NWS)), dim3(64 * (NWS + NLS)), smem, st, K2F, K1F, QBT,
+               Ai, AQ, (const T*)dO, dec, (const void*)bhat, 0, dht, dh0, DVF, DHF, cu, chunk_offsets, d.T, H, H, d.V, scale);
+  }
+  {
+    auto kern = chunk_bwd_local_kernel<T, DK, true>;
+    constexpr int smem = BwdLocalSmem<T, DK>::bytes;
+    if (int e = set_lds_b(kern, smem)) return e;
+    TokenStrides ts = d.strides();
+    GDN_LAUNCH(kKernBwdLocal, st, kern, dim3(nc, H), dim3(kThreads), smem, st, QBT, K1F, (const T*)v, (const void*)bhat, 0,
+               (const float*)nullptr, Ai, VF, (const T*)DVF, (const T*)dO, HF, (const T*)DHF, (const float*)nullptr,
+               (const float*)nullptr, (T*)nullptr, (T*)nullptr, (T*)dv, (void*)nullptr, (float*)nullptr, cu, chunk_offsets, d.T,
+               d.N, H, H, d.V, scale, 0, ts, DUMP);
+  }
+  {
+    auto kern = kda_bwd_finish_kernel<T, DK>;
+    constexpr int smem = KdaBwdSmem<T, DK>::bytes;
+    if (int e = set_lds_b(kern, smem)) return e;
+    GDN_LAUNCH(kKernKdaBwdFinish, st, kern, dim3(nc, H), dim3(kThreads), smem, st, (const T*)q, (const T*)k, g, A_log, dt_bias,
+               bhat, GC, TMR, (const float*)DUMP, cu, chunk_offsets, (T*)dq, (T*)dk, dg, dbeta, PART, d.T, d.N, H, scale, fl);
+  }
+  if (fl.use_gate && (dA_log != nullptr || ddt_bias != nullptr))
+    GDN_LAUNCH(kKernKdaBwdFinish, st, kda_bwd_reduce_kernel, dim3(H), dim3(kThreads), 0, st, (const float*)PART, cu,
+               chunk_offsets, d.N, nc, H, d.K, dA_log, ddt_bias);
+  return (int)hipGetLastError();
+}
+
+}  // namespace gdn
+
+extern "C" int gdn_kda_bwd(const void* q, const void* k, const void* v, const void* g, const float* A_log,
+                           const float* dt_bias, const int64_t* cu_seqlens, const void* d_o, const float* d_final_state,
+                           void* dq, void* dk, void* dv, void* dg, void* dbeta, float* dA_log, float* ddt_bias,
+                           float* d_initial_state, void* workspace, int64_t workspace_bytes, int B, int T, int N, int H,
+                           int K, int V, float scale, int use_qk_l2norm, int use_gate, int has_lower_bound,
+                           float lower_bound, int beta_sigmoid, int allow_neg_eigval, int dtype, int g_dtype,
+                           int beta_dtype, void* stream) {
+  using namespace gdn;
+  if (!q || !k || !v || !g || !d_o || !dq || !dk || !dv || !dg || !dbeta || !workspace) return -1;
+  if (use_gate && !A_log) return -1;
+  ChunkDims d{B, T, N, H, H, K, V, cu_seqlens != nullptr};
+  if (int e = chunk_check_dims(d, dtype)) return e;
+  if ((g_dtype != 0 && g_dtype != dtype) || (beta_dtype != 0 && beta_dtype != dtype)) return -4;
+  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)g | (uintptr_t)d_o | (uintptr_t)dq | (uintptr_t)dk |
+       (uintptr_t)dv | (uintptr_t)dg) & 15)
+    return -6;
+  ChunkDims dl = d;
+  dl.varlen = true;
+  const KdaWorkspace L = kda_workspace_layout(dl, dtype == 0 ? 4 : 2);
+  if (workspace_bytes < L.total_bytes || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
+  KdaFlags fl{use_qk_l2norm, use_gate, has_lower_bound, beta_sigmoid, allow_neg_eigval, g_dtype == 0, beta_dtype == 0, lower_bound};
+  unsigned char* ws = static_cast<unsigned char*>(workspace);
+  hipStream_t st = (hipStream_t)stream;
+#define GDN_KDAB(T_, DK_, NWS_, NLS_, ST_)                                                                              \
+  return kda_bwd_launch<T_, DK_, NWS_, NLS_, ST_>(d, L, q, k, v, g, A_log, dt_bias, cu_seqlens, d_o, d_final_state, dq, dk, dv, \
+                                                  dg, dbeta, dA_log, ddt_bias, d_initial_state, ws, scale, fl, st)
+  if (dtype == 1) {
+    if (K == 128) GDN_KDAB(bf16_t, 128, 2, 4, 2);
+    GDN_KDAB(bf16_t, 64, 2, 2, 2);
+  } else {
+    if (K == 128) GDN_KDAB(float, 128, 2, 2, 1);
+    GDN_KDAB(float, 64, 2, 2, 1);
+  }
+#undef GDN_KDAB
+}

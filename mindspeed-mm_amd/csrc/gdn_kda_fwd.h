@@ -14,13 +14,9 @@
 // matrix cores on rows rescaled around the decay at the block boundary, k_i e^{G_i - G_31} (i >= 32) against
 // k_j e^{G_31 - G_j} (j < 32): both factors are at most 1.
 #pragma once
+#include "gdn_kda_common.h"
 
 namespace gdn {
-
-struct KdaFlags {
-  int l2norm, use_gate, has_lower_bound, beta_sigmoid, beta_x2, g_f32, beta_f32;
-  float lower_bound;
-};
 
 template <typename T, int DK> struct KdaPrepSmem {
   static constexpr int LDK = lds_ld<T>(DK), LDG = DK + 4, L64 = lds_ld<T>(64);
@@ -40,25 +36,14 @@ template <typename T, int DK> struct KdaPrepSmem {
   static_assert(bytes <= 160 * 1024, "one CU's LDS");
 };
 
-__device__ __forceinline__ float kda_sigmoid(float x) { return 1.f / (1.f + __expf(-x)); }
-__device__ __forceinline__ float kda_softplus(float x) { return x > 20.f ? x : log1pf(__expf(x)); }
-
-// VEC consecutive fp32 values of an LDS row
-template <int VEC> __device__ __forceinline__ void ld_f32(const float* p, float* f) {
-#pragma unroll
-  for (int e = 0; e < VEC; e += 4) {
-    const f32x4 x = *reinterpret_cast<const f32x4*>(p + e);
-    f[e] = x[0]; f[e + 1] = x[1]; f[e + 2] = x[2]; f[e + 3] = x[3];
-  }
-}
-
 template <typename T, int DK>
 __global__ __launch_bounds__(kThreads) void kda_prep_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const void* __restrict__ g, const void* __restrict__ beta,
     const float* __restrict__ A_log, const float* __restrict__ dt_bias, const int64_t* __restrict__ cu,
     const int* __restrict__ chunk_offsets, float* __restrict__ bhat_out, float* __restrict__ dec_out,
     float* __restrict__ G_out, T* __restrict__ Ai_out, T* __restrict__ Aq_out, T* __restrict__ K1_out,
-    T* __restrict__ K2_out, T* __restrict__ QB_out, float* __restrict__ rstd_q_out, float* __restrict__ rstd_k_out,
+    T* __restrict__ K2_out, T* __restrict__ QB_out, T* __restrict__ QBT_out, T* __restrict__ TMR_out,
+    float* __restrict__ rstd_q_out, float* __restrict__ rstd_k_out,
     int T_len, int N, int H, float scale, KdaFlags fl) {
   using SM = KdaPrepSmem<T, DK>;
   constexpr int LDK = SM::LDK, LDG = SM::LDG, VEC = Elem<T>::kVec, CPR = DK / VEC;
@@ -240,16 +225,27 @@ __global__ __launch_bounds__(kThreads) void kda_prep_kernel(
   stage_k(false);
   GDN_LDS_BARRIER();
   store_k(K2_out);
-  // rows of q with scale and decay, the decay of the whole chunk per channel, the cumulative decay itself
+  GDN_LDS_BARRIER();
+  // rows of q with scale and decay (row-major for the output kernel; transposed tiles for a backward pass), the decay
+  // of the whole chunk per channel, the cumulative decay itself
   for (int c = tid; c < 64 * CPR; c += kThreads) {
     const int row = c / CPR, cc = c % CPR;
-    if (row < nvalid) {
-      float f[VEC], gi[VEC];
-      unpack16<T>(ld16(Qs + row * LDK + cc * VEC), f);
-      ld_f32<VEC>(Gs + row * LDG + cc * VEC, gi);
+    float f[VEC], gi[VEC];
+    unpack16<T>(ld16(Qs + row * LDK + cc * VEC), f);
+    ld_f32<VEC>(Gs + row * LDG + cc * VEC, gi);
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) f[e] *= scale * __expf(gi[e]);
-      st16(QB_out + (tok0 + row) * hk + h * DK + cc * VEC, pack16<T>(f));
+    for (int e = 0; e < VEC; ++e) f[e] *= scale * __expf(gi[e]);
+    const Vec16<T> x = pack16<T>(f);
+    if (row < nvalid) st16(QB_out + (tok0 + row) * hk + h * DK + cc * VEC, x);
+    st16(X1 + row * LDK + cc * VEC, x);
+  }
+  if (QBT_out != nullptr) {
+    GDN_LDS_BARRIER();
+    for (int tt = wave; tt < 2 * (DK / 32); tt += 4) {
+      const int tj = tt & 1, kt2 = tt >> 1;
+      AccB<T> kf;
+      kf.load_cols(X1 + 32 * tj * LDK + 32 * kt2, LDK);
+      kf.store_stream(QBT_out + ((ch * (DK / 32) + kt2) * 2 + tj) * 1024);
     }
   }
   if (tid < DK) dec_out[ch * DK + tid] = __expf(Gs[63 * LDG + tid]);
@@ -292,6 +288,11 @@ __global__ __launch_bounds__(kThreads) void kda_prep_kernel(
   }
   tril_inverse_64(As, Ti, wave, lane);
   store_tm_tiles<T>(Ti, Tms, Ai_out + ch * 4096, tid, wave, lane);
+  if (TMR_out != nullptr) {   // the staging tile holds Tm row-major in operand precision
+    constexpr int C64 = 64 / VEC;
+    for (int c = tid; c < 64 * C64; c += kThreads)
+      st16(TMR_out + ch * 4096 + (c / C64) * 64 + (c % C64) * VEC, ld16(Tms + (c / C64) * SM::L64 + (c % C64) * VEC));
+  }
 }
 
 // NWO: waves of the output kernel's workgroup; NWS, NLS, STAGES: slabs, loader waves and LDS stages of the recurrence
@@ -314,6 +315,8 @@ static int kda_fwd_launch(const ChunkDims& d, const KdaWorkspace& L, const void*
   T* VF = reinterpret_cast<T*>(ws + L.VF);
   T* HF = reinterpret_cast<T*>(ws + L.HF);
   float* GC = with_backward ? reinterpret_cast<float*>(ws + L.GC) : nullptr;
+  T* QBT = with_backward ? reinterpret_cast<T*>(ws + L.QBT) : nullptr;
+  T* TMR = with_backward ? reinterpret_cast<T*>(ws + L.TMR) : nullptr;
   if (cu != nullptr) GDN_LAUNCH(kKernChunkTable, st, chunk_table_kernel, dim3(1), dim3(kThreads), 0, st, cu, chunk_offsets, d.N);
   {
     auto kern = kda_prep_kernel<T, DK>;
@@ -321,7 +324,7 @@ static int kda_fwd_launch(const ChunkDims& d, const KdaWorkspace& L, const void*
     if (int e = set_lds(kern, smem)) return e;
     const bool keep = with_backward && fl.l2norm;
     GDN_LAUNCH(kKernKdaPrep, st, kern, dim3(nc, H), dim3(kThreads), smem, st, (const T*)q, (const T*)k, g, beta, A_log,
-               dt_bias, cu, (const int*)chunk_offsets, bhat, dec, GC, Ai, AQ, K1F, K2F, QB, keep ? rstd : nullptr,
+               dt_bias, cu, (const int*)chunk_offsets, bhat, dec, GC, Ai, AQ, K1F, K2F, QB, QBT, TMR, keep ? rstd : nullptr,
                keep ? rstd + (int64_t)nc * 64 * H : nullptr, d.T, d.N, H, scale, fl);
   }
   {

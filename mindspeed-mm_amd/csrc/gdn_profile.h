@@ -9,7 +9,7 @@ enum KernelId {
   kKernChunkTable = 0, kKernPrep, kKernStateFwd, kKernOut, kKernStateBwd, kKernBwdLocal,
   kKernRecurrent, kKernConvFwd, kKernConvState, kKernConvBwd, kKernConvReduce,
   kKernConvDh0, kKernConvUpdate, kKernRmsNormFwd, kKernRmsNormBwd, kKernRmsNormReduce,
-  kKernGateFwd, kKernGateBwd, kKernGateReduce, kKernKdaPrep, kKernCount
+  kKernGateFwd, kKernGateBwd, kKernGateReduce, kKernKdaPrep, kKernKdaBwdFinish, kKernCount
 };
 
 bool profile_on();

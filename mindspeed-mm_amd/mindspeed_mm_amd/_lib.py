@@ -35,6 +35,7 @@ SIGNATURES = {
     "gdn_gate_bwd_noalloc": (I, [P] * 10 + [L, I, I, I, P]),
     "gdn_kda_workspace_bytes": (L, [I] * 8),
     "gdn_kda_fwd": (I, [P] * 12 + [L] + [I] * 6 + [F, I, I, I, F, I, I, I, I, I, P]),
+    "gdn_kda_bwd": (I, [P] * 18 + [L] + [I] * 6 + [F, I, I, I, F, I, I, I, I, I, P]),
     "gdn_profile_enable": (I, [I]),
     "gdn_profile_kernel_count": (I, []),
     "gdn_profile_kernel_name": (ctypes.c_char_p, [I]),

@@ -664,8 +664,8 @@ class _ChunkGatedDeltaRuleQKV(torch.autograd.Function):
 
 
 class _ChunkKda(torch.autograd.Function):
-    """Forward pass of KDA in the HIP library (gdn_kda_fwd).  A backward pass of its own is not built: asking for
-    gradients raises."""
+    """KDA through the HIP library: gdn_kda_fwd, and gdn_kda_bwd on the workspace the forward call filled (it is kept
+    between the passes when a gradient is asked for)."""
 
     @staticmethod
     @_input_guard
@@ -677,28 +677,55 @@ class _ChunkKda(torch.autograd.Function):
         V = v.shape[3]
         N = (len(cu_seqlens) - 1) if cu_seqlens is not None else B
         code = DTYPE_CODE[q.dtype]
+        need_grad = any(ctx.needs_input_grad[:7]) or (initial_state is not None and ctx.needs_input_grad[8])
         qc, kc, vc = q.detach().contiguous(), k.detach().contiguous(), v.detach().contiguous()
         gc = g.detach().contiguous() if g.dtype == q.dtype else g.detach().to(torch.float32).contiguous()
         gcode = code if g.dtype == q.dtype else 0
         bc, bcode = _beta_arg(beta, q.dtype)
         a32, d32, h0 = ops._f32(A_log), ops._f32(dt_bias), ops._f32(initial_state)
         cu = _i64(cu_seqlens, q)
-        nbytes = lib.gdn_kda_workspace_bytes(B, T, N, H, K, V, 0, code)
+        nbytes = lib.gdn_kda_workspace_bytes(B, T, N, H, K, V, int(need_grad), code)
         ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=q.device)
         off = (-ws.data_ptr()) % 256
         ws = ws[off:off + nbytes]
         o = torch.empty(B, T, H, V, dtype=v.dtype, device=v.device)
         ht = torch.empty(N, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
+        opts = (int(l2norm), int(use_gate), int(lower_bound is not None),
+                float(lower_bound if lower_bound is not None else 0.0), int(beta_sigmoid), int(allow_neg), code, gcode, bcode)
         rc = lib.gdn_kda_fwd(ptr(qc), ptr(kc), ptr(vc), ptr(gc), ptr(bc), ptr(a32), ptr(d32), ptr(h0), ptr(cu), ptr(o),
-                             ptr(ht), ptr(ws), nbytes, B, T, N, H, K, V, scale, int(l2norm), int(use_gate),
-                             int(lower_bound is not None), float(lower_bound if lower_bound is not None else 0.0),
-                             int(beta_sigmoid), int(allow_neg), code, gcode, bcode, lib.stream())
+                             ptr(ht), ptr(ws), nbytes, B, T, N, H, K, V, scale, *opts, lib.stream())
         lib.check(rc, "gdn_kda_fwd")
+        if need_grad:
+            ctx.save_for_backward(qc, kc, vc, gc, a32, d32, cu, ws)
+            ctx.meta = (B, T, N, H, K, V, scale, opts, nbytes, g.dtype, beta.dtype, bc.dtype,
+                        None if A_log is None else A_log.dtype, None if dt_bias is None else (dt_bias.dtype, dt_bias.shape),
+                        None if initial_state is None else initial_state.dtype)
+            ctx.ops = ops
         return o, ht
 
     @staticmethod
+    @_input_guard
+    @_custom_bwd
     def backward(ctx, do, dht):
-        raise NotImplementedError("chunk_kda: the backward pass is not built; call it under torch.no_grad()")
+        qc, kc, vc, gc, a32, d32, cu, ws = ctx.saved_tensors
+        B, T, N, H, K, V, scale, opts, nbytes, g_dt, b_dt, bc_dt, a_dt, d_dt, h_dt = ctx.meta
+        lib = ctx.ops.lib
+        dev = qc.device
+        do = do.contiguous()
+        dht = ctx.ops._f32(dht)
+        dq, dk, dv, dg = torch.empty_like(qc), torch.empty_like(kc), torch.empty_like(vc), torch.empty_like(gc)
+        db = torch.empty(B, T, H, dtype=bc_dt, device=dev)
+        use_gate = bool(opts[1])
+        dA = torch.empty(H, dtype=torch.float32, device=dev) if (use_gate and a32 is not None) else None
+        dD = torch.empty(H * K, dtype=torch.float32, device=dev) if (use_gate and d32 is not None) else None
+        dh0 = torch.empty(N, H, K, V, dtype=torch.float32, device=dev) if h_dt is not None else None
+        rc = lib.gdn_kda_bwd(ptr(qc), ptr(kc), ptr(vc), ptr(gc), ptr(a32), ptr(d32), ptr(cu), ptr(do), ptr(dht), ptr(dq),
+                             ptr(dk), ptr(dv), ptr(dg), ptr(db), ptr(dA), ptr(dD), ptr(dh0), ptr(ws), nbytes, B, T, N, H, K,
+                             V, scale, *opts, lib.stream())
+        lib.check(rc, "gdn_kda_bwd")
+        return (dq, dk, dv, dg.to(g_dt), db.to(b_dt), None if dA is None else dA.to(a_dt),
+                None if dD is None else dD.to(d_dt[0]).reshape(d_dt[1]), None, None if dh0 is None else dh0.to(h_dt),
+                None, None, None, None, None, None, None, None)
 
 
 class _GdnGates(torch.autograd.Function):

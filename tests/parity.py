@@ -15,6 +15,8 @@ from oracle import kda_oracle as KO
 FP32_REL = 1e-4
 BF16_ABS_O = 2e-2
 BF16_ABS_GRAD = 5e-2
+# dA_log and d(dt_bias) are sums over every token of the batch: their error bound grows with their size
+KDA_PARAM_RTOL = 2e-2
 
 
 def _err(name, got, ref, dtype, abs_tol, rtol=0.0):
@@ -421,10 +423,11 @@ def check_decode_step(ops, device, B, steps, Hqk, Hv, K, V, W, dtype, param_dtyp
 
 
 def check_kda(ops, device, B, T, H, K, V, dtype, cu=None, seed=0, with_h0=True, gate_in_kernel=True, lower_bound=None,
-              beta_sigmoid=True, allow_neg=False, l2=True, transpose_state=True, g_dtype=None, scale=None,
+              beta_sigmoid=True, allow_neg=False, l2=True, transpose_state=True, g_dtype=None, scale=None, backward=False,
               wrap=lambda t: t, **recipe):
     """chunk_kda against the oracle's statement of chunk_kda_naive, with the options of the layer's call
-    (modeling_kimi_linear.py:681-699: raw gate and beta, l2 norm in the kernel, [N,H,V,K] states) or without them."""
+    (modeling_kimi_linear.py:681-699: raw gate and beta, l2 norm in the kernel, [N,H,V,K] states) or without them.
+    backward: every gradient against autograd through the oracle (loss = <o, do> + <final state, dht>)."""
     N = (len(cu) - 1) if cu is not None else B
     x = kda_inputs(B, T, H, K, V, dtype, seed=seed, N=N, **recipe)
     if not gate_in_kernel:   # the caller hands over the log decay itself
@@ -436,16 +439,30 @@ def check_kda(ops, device, B, T, H, K, V, dtype, cu=None, seed=0, with_h0=True, 
     if not l2:
         x["q"], x["k"] = (KO._l2norm_rounded(t) for t in (x["q"], x["k"]))
     if transpose_state:
-        x["h0"] = x["h0"].transpose(-1, -2).contiguous()
+        x["h0"], x["dht"] = (x[n].transpose(-1, -2).contiguous() for n in ("h0", "dht"))
+    names = ("q", "k", "v", "g", "beta", "h0", "A_log", "dt_bias")
     dev = {n: wrap(t.to(device)) for n, t in x.items()}
+    leaves = {n: dev[n].clone().requires_grad_(backward) for n in names}
+    ref = {n: x[n].clone().requires_grad_(backward) for n in names}
     cu_t = torch.tensor(cu, dtype=torch.int64, device=device) if cu is not None else None
     kw = dict(scale=scale, output_final_state=True, use_qk_l2norm_in_kernel=l2, use_gate_in_kernel=gate_in_kernel,
               use_beta_sigmoid_in_kernel=beta_sigmoid, allow_neg_eigval=allow_neg, lower_bound=lower_bound if gate_in_kernel else None,
               transpose_state_layout=transpose_state)
-    with torch.no_grad():
-        o, ht = ops.chunk_kda(dev["q"], dev["k"], dev["v"], dev["g"], dev["beta"], initial_state=dev["h0"] if with_h0 else None,
-                              cu_seqlens=cu_t, safe_gate=lower_bound is not None, A_log=dev["A_log"], dt_bias=dev["dt_bias"], **kw)
-    ro, rht = KO.chunk_kda_ref(x["q"], x["k"], x["v"], x["g"], x["beta"], initial_state=x["h0"] if with_h0 else None,
-                               cu_seqlens=cu, A_log=x["A_log"], dt_bias=x["dt_bias"], round_output=False, **kw)
+    with torch.set_grad_enabled(backward):
+        o, ht = ops.chunk_kda(leaves["q"], leaves["k"], leaves["v"], leaves["g"], leaves["beta"],
+                              initial_state=leaves["h0"] if with_h0 else None, cu_seqlens=cu_t,
+                              safe_gate=lower_bound is not None, A_log=leaves["A_log"], dt_bias=leaves["dt_bias"], **kw)
+        ro, rht = KO.chunk_kda_ref(ref["q"], ref["k"], ref["v"], ref["g"], ref["beta"], initial_state=ref["h0"] if with_h0 else None,
+                                   cu_seqlens=cu, A_log=ref["A_log"], dt_bias=ref["dt_bias"], round_output=False, **kw)
     assert o.dtype == dtype and ht.dtype == torch.float32 and ht.shape == rht.shape
-    return {"o": _err("o", o, ro, dtype, BF16_ABS_O), "ht": _err("final_state", ht, rht, dtype, BF16_ABS_GRAD)}
+    errs = {"o": _err("o", o, ro, dtype, BF16_ABS_O), "ht": _err("final_state", ht, rht, dtype, BF16_ABS_GRAD)}
+    if backward:
+        ((o.float() * dev["do"].float()).sum() + (ht * dev["dht"]).sum()).backward()
+        ((ro * x["do"].float()).sum() + (rht * x["dht"]).sum()).backward()
+        for n in names:
+            if (n == "h0" and not with_h0) or (n in ("A_log", "dt_bias") and not gate_in_kernel):
+                continue
+            assert leaves[n].grad is not None, n
+            assert leaves[n].grad.dtype == leaves[n].dtype and leaves[n].grad.shape == leaves[n].shape
+            errs["d" + n] = _err("d" + n, leaves[n].grad, ref[n].grad, dtype, BF16_ABS_GRAD, rtol=KDA_PARAM_RTOL if n in ("A_log", "dt_bias") else 0.0)
+    return errs

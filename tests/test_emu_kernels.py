@@ -208,3 +208,16 @@ def test_conv1d_random_shapes(ops, seed):
 ])
 def test_kda_forward(ops, dtype, B, T, H, K, V, cu, kw):
     P.check_kda(ops, "cpu", B, T, H, K, V, dtype, cu=cu, wrap=guarded, h0_std=0.1, **kw)
+
+
+@pytest.mark.parametrize("dtype,B,T,H,K,V,cu,kw", [
+    (F32, 1, 64, 1, 64, 64, None, {}),
+    (F32, 1, 100, 2, 128, 128, None, {}),
+    (BF, 1, 200, 2, 128, 128, None, {}),
+    (BF, 1, 140, 2, 64, 64, [0, 5, 70, 71, 140], dict(lower_bound=-5.0)),
+    (F32, 1, 96, 1, 128, 64, [0, 1, 38, 96], dict(gate_in_kernel=False, beta_sigmoid=False, l2=False, transpose_state=False)),
+    (BF, 1, 130, 1, 128, 64, None, dict(allow_neg=True, with_h0=False, g_dtype=torch.float32)),
+])
+def test_kda_backward(ops, dtype, B, T, H, K, V, cu, kw):
+    errs = P.check_kda(ops, "cpu", B, T, H, K, V, dtype, cu=cu, backward=True, wrap=guarded, h0_std=0.1, **kw)
+    print({n: f"{e:.2e}" for n, e in errs.items()})

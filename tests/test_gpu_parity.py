@@ -416,6 +416,13 @@ def test_kda_forward(ops, dtype, B, T, H, K, V, cu, kw):
     print("   ", {n: f"{e:.2e}" for n, e in errs.items()}, flush=True)
 
 
+@pytest.mark.parametrize("dtype,B,T,H,K,V,cu,kw", KDA_CASES)
+def test_kda_backward(ops, dtype, B, T, H, K, V, cu, kw):
+    print(f"kda backward {dtype} B{B} T{T} H{H} K{K} V{V} cu={'yes' if cu else 'no'} {kw}", flush=True)
+    errs = P.check_kda(ops, "cuda", B, T, H, K, V, dtype, cu=cu, backward=True, **kw)
+    print("   ", {n: f"{e:.2e}" for n, e in errs.items()}, flush=True)
+
+
 def test_kda_argument_checks(ops):
     x = P.kda_inputs(1, 64, 2, 64, 64, BF)
     d = {n: t.cuda() for n, t in x.items()}
