@@ -472,6 +472,39 @@ def main():
             "frac_mfma_ref_formula": round(fl4 / (ms4 * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}
         del d4
         torch.cuda.empty_cache()
+        # KDA (one decay per key channel) at the benchmark's token count and the Kimi linear-attention head shape
+        # (mindspeed_mm/fsdp/models/kimi_k3/modeling_kimi_linear.py:549-596: 32 heads of 128), with the layer's
+        # options: raw gate and beta, l2 norm in the kernel, [N,H,V,K] states
+        from mindspeed_mm_amd.inputs import kda_inputs
+        Hk = c["Hv"]
+        xk = kda_inputs(c["B"], c["T"], Hk, c["K"], c["V"], torch.bfloat16, seed=5)
+        dk_ = {n: t.to(dev) for n, t in xk.items()}
+        del xk
+        kl = {n: dk_[n].clone().requires_grad_(True) for n in ("q", "k", "v", "g", "beta", "A_log", "dt_bias")}
+        kh0 = dk_["h0"].transpose(-1, -2).contiguous().requires_grad_(True)
+        kda_kw = dict(initial_state=kh0, output_final_state=True, use_qk_l2norm_in_kernel=True, use_gate_in_kernel=True,
+                      use_beta_sigmoid_in_kernel=True, transpose_state_layout=True, A_log=kl["A_log"], dt_bias=kl["dt_bias"])
+
+        def kda_step():
+            o_, _ = ops.chunk_kda(kl["q"], kl["k"], kl["v"], kl["g"], kl["beta"], **kda_kw)
+            torch.autograd.grad([o_], list(kl.values()) + [kh0], [dk_["do"]])
+
+        def kda_prefill():
+            with torch.no_grad():
+                ops.chunk_kda(kl["q"], kl["k"], kl["v"], kl["g"], kl["beta"], **kda_kw)
+        kms, kpf = wall_ms(kda_step, 10, 3), wall_ms(kda_prefill, 10, 3)
+        torch.cuda.synchronize()
+        lib.gdn_profile_enable(1)
+        for _ in range(5):
+            kda_step()
+        torch.cuda.synchronize()
+        ktm = _lib.kernel_timings(lib)
+        lib.gdn_profile_enable(0)
+        aux["kda_B2_T8192_H32_d128"] = {
+            "fwd_bwd_ms": round(kms, 4), "tokens_per_s": round(tokens / (kms * 1e-3), 1), "forward_only_ms": round(kpf, 4),
+            "kernels_ms_per_step": {n: round(ms / 5, 4) for n, (ms, _) in ktm.items()}}
+        del dk_, kl, kh0
+        torch.cuda.empty_cache()
 
     if args.calibrate_copy:
         src = torch.empty(512 << 20, dtype=torch.uint8, device=dev)

@@ -35,16 +35,20 @@ template <typename T, int DK> struct KdaBwdSmem {
   static constexpr int off_ks = 0;                   // k^ rows
   static constexpr int off_qs = off_ks + tile;       // first P as T, then q^ rows
   static constexpr int off_gs = off_qs + tile;       // first Kp as T (64 rows), then G rows (fp32)
-  static constexpr int off_tm = off_gs + gmat;       // Tm row-major; later, with the next two, the store patches
-  static constexpr int off_m1 = off_tm + mat;        // dTm, then dL
+  static constexpr int off_m1 = off_gs + gmat;       // dTm, then dL; later, with the next one, the store patches
   static constexpr int off_m2 = off_m1 + mat;        // X = Tm^T dTm, then scale dAq
-  static constexpr int off_xi = off_m2 + mat;        // rescaled rows [b k ; q] of tokens 32..63 (not FULL)
+  static constexpr int off_tm = off_m2 + mat;        // Tm row-major
+  static constexpr int off_xi = off_tm + mat;        // rescaled rows [b k ; q] of tokens 32..63 (not FULL)
   static constexpr int off_xr = off_xi + (FULL ? 0 : tile);       // rescaled rows k of tokens 0..31
-  static constexpr int off_row = off_xr + (FULL ? 0 : tile / 2);
+  // 16-bit operands: once Tm and the rescaled rows are consumed their place takes the two coefficients of every pair
+  // packed into one word, (dL_ij | scale dAq_ij << 16), row-major [i][j] and transposed [j][i] (uint32 [64][kLC] each)
+  static constexpr int kLC = 68, off_mc = off_tm, off_mct = off_mc + 64 * kLC * 4;
+  static constexpr int cmax(int a, int b) { return a > b ? a : b; }
+  static constexpr int off_row = FULL ? off_xr : cmax(off_xr + tile / 2, off_mct + 64 * kLC * 4);
   // beta, 1/|q|, 1/|k| [64 each]; per-wave row sums <q^,dq^>, <k^,dk^>, db, <R,v> [256 each]; 8 scalars
   static constexpr int bytes = off_row + (3 * 64 + 4 * 256 + 8) * 4;
   static_assert(tile <= gmat, "Kp fits where G will be");
-  static_assert(4 * Patch<T>::kElems * (int)sizeof(T) <= 3 * mat, "store patches fit");
+  static_assert(4 * Patch<T>::kElems * (int)sizeof(T) <= 2 * mat, "store patches fit");
   static_assert(bytes <= 160 * 1024, "one CU's LDS");
 };
 
@@ -68,6 +72,9 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
   T* M2 = reinterpret_cast<T*>(gdn_smem + SM::off_m2);
   T* XI = reinterpret_cast<T*>(gdn_smem + SM::off_xi);
   T* XR = reinterpret_cast<T*>(gdn_smem + SM::off_xr);
+  uint32_t* MC = reinterpret_cast<uint32_t*>(gdn_smem + SM::off_mc);
+  uint32_t* MCt = reinterpret_cast<uint32_t*>(gdn_smem + SM::off_mct);
+  constexpr int kLC = SM::kLC;
   float* bs = reinterpret_cast<float*>(gdn_smem + SM::off_row);
   float* rsq = bs + 64;
   float* rsk = rsq + 64;
@@ -90,9 +97,16 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
   const float* dAq = dump + 3 * 64 * DK, *a2m = dAq + 64 * 64, *dD = a2m + 64 * 64;
   const float* Gc = GC + ch * 64 * DK;
 
-  // ---- phase A0: k^ rows; P and Tm as operands; beta ----
+  // ---- phase A0: k^ rows; P and Tm as operands; beta.  This wave's tiles of a2 and dAq are requested now ----
   TileQK<T, DK> kt;
   tile_qk_request<T, DK>(kt, k + tok0 * hk + h * DK, hk, nvalid, tid);
+  f32x16 a2t, dat;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int at = (32 * ti + acc_row(r)) * 64 + 32 * tj + l32;
+    a2t[r] = lower ? a2m[at] : 0.f;
+    dat[r] = lower ? dAq[at] : 0.f;
+  }
   if (tid < 64) {
     bs[tid] = tid < nvalid ? bhat[(tok0 + tid) * H + h] : 0.f;
     rsq[tid] = 1.f;
@@ -134,7 +148,7 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int i = 32 * ti + acc_row(r);
-      const float a2v = lower ? a2m[i * 64 + j] : 0.f;
+      const float a2v = a2t[r];
       sv += a2v * Elem<T>::to_f(TmT[i * L64 + j]);
       M1[i * L64 + j] = Elem<T>::from_f(i > j ? bj * (a2v - x[r]) : 0.f);
     }
@@ -164,7 +178,7 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
   for (int r = 0; r < 16; ++r) {
     const int i = 32 * ti + acc_row(r), j = 32 * tj + l32;
     dl[r] = i > j ? -dl[r] : 0.f;
-    sa[r] = (lower && i >= j) ? scale * dAq[i * 64 + j] : 0.f;
+    sa[r] = i >= j ? scale * dat[r] : 0.f;
   }
   GDN_LDS_BARRIER();   // dTm, X, P, Kp are consumed
   // ---- phase A4: the coefficient matrices in place of dTm and X; q^ rows and G in place of P and Kp ----
@@ -233,6 +247,15 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
         W[0][r] = w[r] * __expf(g31 - Gi[0][r]);
       }
     }
+    GDN_LDS_BARRIER();   // Tm and the rescaled rows are consumed
+    for (int c = tid; c < 64 * 64; c += kThreads) {
+      const int i = c >> 6, j = c & 63;
+      uint32_t w = 0;
+      if constexpr (sizeof(T) == 2) w = (uint32_t)M1[i * L64 + j].bits | ((uint32_t)M2[i * L64 + j].bits << 16);
+      MC[i * kLC + j] = w;
+      MCt[j * kLC + i] = w;
+    }
+    GDN_LDS_BARRIER();
   }
   if (has_k) {
 #pragma unroll
@@ -243,12 +266,17 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
 #pragma unroll
         for (int qd = 0; qd < 4; ++qd) {
           if (32 * ri + 8 * qd + 7 < jj) continue;   // none of the group's rows reaches jj (same for every lane)
+          u32x4 cw = {0u, 0u, 0u, 0u};
+          if constexpr (!FULL) cw = *reinterpret_cast<const u32x4*>(MCt + jj * kLC + 32 * ri + acc_row(4 * qd));
 #pragma unroll
           for (int m = 0; m < 4; ++m) {
             const int r = 4 * qd + m, i = 32 * ri + acc_row(r);
             const float t = kj * __expf(i >= jj ? Gi[ri][r] - gj : 0.f);
-            U[ri][r] += Elem<T>::to_f(M1[i * L64 + jj]) * t;    // coefficients are zero where i < jj
-            Uq[ri][r] += Elem<T>::to_f(M2[i * L64 + jj]) * t;
+            float cl, cq;   // coefficients are zero where i < jj
+            if constexpr (FULL) { cl = Elem<T>::to_f(M1[i * L64 + jj]); cq = Elem<T>::to_f(M2[i * L64 + jj]); }
+            else { cl = __uint_as_float(cw[m] << 16); cq = __uint_as_float(cw[m] & 0xffff0000u); }
+            U[ri][r] += cl * t;
+            Uq[ri][r] += cq * t;
           }
         }
       }
@@ -258,11 +286,16 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
 #pragma unroll
         for (int qd = 0; qd < 4; ++qd) {
           if (32 * ri + 8 * qd > ii) continue;
+          u32x4 cw = {0u, 0u, 0u, 0u};
+          if constexpr (!FULL) cw = *reinterpret_cast<const u32x4*>(MC + ii * kLC + 32 * ri + acc_row(4 * qd));
 #pragma unroll
           for (int m = 0; m < 4; ++m) {
             const int r = 4 * qd + m, j = 32 * ri + acc_row(r);
             const float e = __expf(ii >= j ? gi - Gi[ri][r] : 0.f);
-            W[ri][r] += (Elem<T>::to_f(M1[ii * L64 + j]) * kb + Elem<T>::to_f(M2[ii * L64 + j]) * qv) * e;
+            float cl, cq;
+            if constexpr (FULL) { cl = Elem<T>::to_f(M1[ii * L64 + j]); cq = Elem<T>::to_f(M2[ii * L64 + j]); }
+            else { cl = __uint_as_float(cw[m] << 16); cq = __uint_as_float(cw[m] & 0xffff0000u); }
+            W[ri][r] += (cl * kb + cq * qv) * e;
           }
         }
       }
@@ -300,9 +333,22 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
   // ---- phase B4: l2 norm backward, dq and dk out; dg by a reverse cumulative sum, back through the gate ----
   IdentityFrag<T> id;
   id.init();
-  T* patch = TmT + wave * Patch<T>::kElems;
+  T* patch = M1 + wave * Patch<T>::kElems;
   float da_sum = 0.f;
   if (has_k) {
+    // the raw gate input of this lane's rows, requested before the stores below
+    const bool g32 = sizeof(T) == 4 || fl.g_f32;
+    float raws[2][16];
+    if (fl.use_gate) {
+#pragma unroll
+      for (int ri = 0; ri < 2; ++ri)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int64_t gat = (tok0 + imin(32 * ri + acc_row(r), nvalid - 1)) * hk + h * DK + d;
+          if (g32) raws[ri][r] = reinterpret_cast<const float*>(g)[gat];
+          else { T t; if constexpr (sizeof(T) == 2) t.bits = reinterpret_cast<const uint16_t*>(g)[gat]; raws[ri][r] = Elem<T>::to_f(t); }
+        }
+    }
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {
       if (fl.l2norm) {
@@ -336,7 +382,6 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
     const bool first_half = lane < 32;
     const float a = fl.use_gate ? __expf(A_log[h]) : 0.f;
     const float bias = (fl.use_gate && dt_bias != nullptr) ? dt_bias[h * DK + d] : 0.f;
-    const bool g32 = sizeof(T) == 4 || fl.g_f32;
     float dt_sum = 0.f;
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {
@@ -351,11 +396,7 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
           run += dGv[ri][r];
           float x = run + dglast;     // d(log decay of token i, channel d)
           if (fl.use_gate) {
-            const int64_t gat = (tok0 + imin(i, nvalid - 1)) * hk + h * DK + d;
-            float raw;
-            if (g32) raw = reinterpret_cast<const float*>(g)[gat];
-            else { T t; if constexpr (sizeof(T) == 2) t.bits = reinterpret_cast<const uint16_t*>(g)[gat]; raw = Elem<T>::to_f(t); }
-            raw += bias;
+            const float raw = raws[ri][r] + bias;
             if (fl.has_lower_bound) {
               const float sg = kda_sigmoid(a * raw), ds_ = fl.lower_bound * sg * (1.f - sg);
               if (i < nvalid) da_sum += x * ds_ * a * raw;
@@ -460,7 +501,7 @@ static int kda_bwd_launch(const ChunkDims& d, const KdaWorkspace& L, const void*
                bhat, GC, TMR, (const float*)DUMP, cu, chunk_offsets, (T*)dq, (T*)dk, dg, dbeta, PART, d.T, d.N, H, scale, fl);
   }
   if (fl.use_gate && (dA_log != nullptr || ddt_bias != nullptr))
-    GDN_LAUNCH(kKernKdaBwdFinish, st, kda_bwd_reduce_kernel, dim3(H), dim3(kThreads), 0, st, (const float*)PART, cu,
+    GDN_LAUNCH(kKernKdaBwdReduce, st, kda_bwd_reduce_kernel, dim3(H), dim3(kThreads), 0, st, (const float*)PART, cu,
                chunk_offsets, d.N, nc, H, d.K, dA_log, ddt_bias);
   return (int)hipGetLastError();
 }

@@ -10,7 +10,9 @@ struct KdaFlags {
 };
 
 __device__ __forceinline__ float kda_sigmoid(float x) { return 1.f / (1.f + __expf(-x)); }
-__device__ __forceinline__ float kda_softplus(float x) { return x > 20.f ? x : log1pf(__expf(x)); }
+// log(1 + e^x) = max(x, 0) + log(1 + e^{-|x|}) with the hardware exponential and logarithm: absolute error of the
+// order of 1e-7 everywhere (the argument of the logarithm lies in (1, 2])
+__device__ __forceinline__ float kda_softplus(float x) { return fmaxf(x, 0.f) + __logf(1.f + __expf(-fabsf(x))); }
 
 // VEC consecutive fp32 values of an LDS row
 template <int VEC> __device__ __forceinline__ void ld_f32(const float* p, float* f) {

@@ -9,10 +9,13 @@
 //     L_ij  = beta_i sum_d k_id k_jd e^{G_id - G_jd}   (i > j)       Tm = (I + L)^-1
 //     Aq_ij = scale sum_d q_id k_jd e^{G_id - G_jd}    (i >= j)
 //     V' = Tm beta (v - (k . e^G) S)      O = (scale q . e^G) S + Aq V'      S <- e^{G_last} . S + (k . e^{G_last-G})^T V'
-// e^{G_i - G_j} does not factor over a whole chunk without overflow (e^{-G_j} is unbounded), so the two 32x32 diagonal
-// blocks of L and Aq are summed channel by channel in fp32 with the exact exponent, and the off-diagonal block uses the
-// matrix cores on rows rescaled around the decay at the block boundary, k_i e^{G_i - G_31} (i >= 32) against
-// k_j e^{G_31 - G_j} (j < 32): both factors are at most 1.
+// e^{G_i - G_j} does not factor over a whole chunk without overflow (e^{-G_j} is unbounded).  It does factor safely
+// for a pair (i, j) that straddles a point m, j < m <= i: e^{G_i-G_m} e^{G_m-G_j}, both factors at most 1.  Halving the
+// chunk recursively (blocks of 64, 32, ..., 2 tokens, m the middle of the block) puts every pair i > j into exactly one
+// such block at one level, where i lies in the second half and j in the first.  So per level every row is rescaled
+// once, x_r e^{-|G_r - G_m|} with m the middle of its block, the 32x32 tile products run on the matrix cores, and of
+// each product only the entries of that level are kept; the diagonal i = j needs no decay at all.  The rescaled rows
+// are built in registers, straight into the operand layout, so nothing but k, q and G occupies LDS.
 #pragma once
 #include "gdn_kda_common.h"
 
@@ -20,19 +23,19 @@ namespace gdn {
 
 template <typename T, int DK> struct KdaPrepSmem {
   static constexpr int LDK = lds_ld<T>(DK), LDG = DK + 4, L64 = lds_ld<T>(64);
-  static constexpr int tile = 64 * LDK * (int)sizeof(T), amat = 64 * kLF * 4;
+  static constexpr int tile = 64 * LDK * (int)sizeof(T), gmat = 64 * LDG * 4, amat = 64 * kLF * 4;
   static constexpr int off_ks = 0, off_qs = off_ks + tile, off_gs = off_qs + tile;   // k, q rows (T), G rows (fp32)
-  static constexpr int off_x1 = off_gs + 64 * LDG * 4;   // 64 rows of T: rescaled rows for the matrix cores, then staging
-  static constexpr int off_x2 = off_x1 + tile;           // 32 rows of T
-  static constexpr int off_misc = off_x2 + tile / 2;     // beta [64], partial totals of the cumulative sum [4][DK]
-  static constexpr int end0 = off_misc + (64 + 4 * DK) * 4;
-  // L, Aq (fp32), the inverse and its staging tile: for K = 128 they take the place of k, q, G and the staging rows,
-  // all dead by then; for K = 64 those are too small and there is room behind them
-  static constexpr bool alias = DK > 64;
-  static constexpr int off_as = alias ? off_ks : end0, off_aq = alias ? off_qs : end0 + amat;
-  static constexpr int off_ti = alias ? off_gs : end0 + 2 * amat, off_tm = alias ? off_x1 : end0 + 3 * amat;
-  static constexpr int bytes = alias ? end0 : end0 + 3 * amat + 64 * L64 * (int)sizeof(T);
-  static_assert(!alias || (amat <= tile && amat <= 64 * LDG * 4 && 64 * L64 * (int)sizeof(T) <= tile), "tenants fit");
+  static constexpr int off_misc = off_gs + gmat;         // beta [64], partial totals of the cumulative sum [4][DK]
+  static constexpr int off_tm = off_misc + (64 + 4 * DK) * 4;   // the inverse in operand precision, row-major
+  static constexpr int end0 = off_tm + 64 * L64 * (int)sizeof(T);
+  // L, Aq and the inverse (fp32 64 x kLF each) take the place of k, q and G once those are dead; where a region is too
+  // small for its tenant the tenant moves behind everything else
+  static constexpr bool wide = tile >= amat;             // K = 128
+  static constexpr int off_as = off_ks;                                  // K = 64: spans the k and q rows
+  static constexpr int off_aq = wide ? off_qs : off_gs;
+  static constexpr int off_ti = wide ? off_gs : end0;
+  static constexpr int bytes = wide ? end0 : end0 + amat;
+  static_assert(wide ? gmat >= amat : (2 * tile >= amat && gmat >= amat), "tenants fit");
   static_assert(bytes <= 160 * 1024, "one CU's LDS");
 };
 
@@ -50,8 +53,6 @@ __global__ __launch_bounds__(kThreads) void kda_prep_kernel(
   T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
   T* Qs = reinterpret_cast<T*>(gdn_smem + SM::off_qs);
   float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_gs);
-  T* X1 = reinterpret_cast<T*>(gdn_smem + SM::off_x1);
-  T* X2 = reinterpret_cast<T*>(gdn_smem + SM::off_x2);
   float* bs = reinterpret_cast<float*>(gdn_smem + SM::off_misc);
   float* tot = bs + 64;
   float* As = reinterpret_cast<float*>(gdn_smem + SM::off_as);
@@ -146,57 +147,87 @@ __global__ __launch_bounds__(kThreads) void kda_prep_kernel(
   }
   GDN_LDS_BARRIER();
 
-  // ---- phase 1a: rows rescaled around the decay at the block boundary: X1 = [k_i ; q_i] e^{G_i-G_31} (i >= 32),
-  //      X2 = k_j e^{G_31-G_j} (j < 32) ----
-  for (int c = tid; c < 96 * CPR; c += kThreads) {
-    const int r = c / CPR, cc = c % CPR;
-    const int src = r < 32 ? 32 + r : (r < 64 ? r : r - 64);
-    const T* from = (r >= 32 && r < 64) ? Qs : Ks;
-    float f[VEC], gi[VEC], gr[VEC];
-    unpack16<T>(ld16(from + src * LDK + cc * VEC), f);
-    ld_f32<VEC>(Gs + src * LDG + cc * VEC, gi);
-    ld_f32<VEC>(Gs + 31 * LDG + cc * VEC, gr);
+  // ---- phase 1: L and Aq level by level on the matrix cores.  Wave w: matrix w & 1 (0: k k^T, 1: q k^T), diagonal
+  //      tile w >> 1; the tile below the diagonal (level 64) goes to waves 0 and 1 ----
+  const int mat = wave & 1, td = wave >> 1, l32 = lane & 31, half = lane >> 5;
+  constexpr int KGL = KGroup<T>::kLen, NKG = DK / KGL;
+  // one product X_A[rows ra] X_K[rows rb]^T over all channels, rows rescaled around row ma / mb of G (negative: as they are)
+  auto level_product = [&](int ra, int ma, int rb, int mb) {
+    f32x16 acc = acc_zero();
+    const T* arow = (mat ? Qs : Ks) + ra * LDK;
+    const T* brow = Ks + rb * LDK;
+#pragma unroll 2
+    for (int kg = 0; kg < NKG; ++kg) {
+      const int c0 = kg * KGL + half * VEC;
+      float fa[VEC], fb[VEC], ga[VEC], gm[VEC];
+      unpack16<T>(ld16(arow + c0), fa);
+      if (ma >= 0) {
+        ld_f32<VEC>(Gs + ra * LDG + c0, ga);
+        ld_f32<VEC>(Gs + ma * LDG + c0, gm);
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) f[e] *= __expf(r < 64 ? gi[e] - gr[e] : gr[e] - gi[e]);
-    T* to = r < 64 ? X1 + r * LDK : X2 + (r - 64) * LDK;
-    st16(to + cc * VEC, pack16<T>(f));
-  }
-  GDN_LDS_BARRIER();
-
-  // ---- phase 1b: the off-diagonal block on the matrix cores (wave 0: k k, wave 1: q k) ----
-  f32x16 acc = acc_zero();
-  if (wave < 2) mma32<T, DK, true, true>(acc, X1 + 32 * wave * LDK, LDK, X2, LDK);
-  // the two diagonal blocks, pair by pair with the exact exponent.  Rows i and 31-i of a block have 33 pairs
-  // between them: eight threads share them.
-  float akk[5], aqk[5];
-  const int blk = tid >> 7, rp = (tid & 127) >> 3, cg = tid & 7;
+        for (int e = 0; e < VEC; ++e) fa[e] *= __expf(-fabsf(ga[e] - gm[e]));
+      }
+      u32x4 bfrag;
+      if (mat == 0 && ra == rb) {
+        bfrag = pack16<T>(fa).raw;   // k k^T on a diagonal tile: both operands are the same rows
+      } else {
+        unpack16<T>(ld16(brow + c0), fb);
+        if (mb >= 0) {
+          ld_f32<VEC>(Gs + rb * LDG + c0, ga);
+          ld_f32<VEC>(Gs + mb * LDG + c0, gm);
 #pragma unroll
-  for (int t = 0; t < 5; ++t) {
-    const int p = cg + 8 * t;
-    int i = p <= rp ? rp : 31 - rp, j = p <= rp ? p : p - rp - 1;
-    if (p >= 33) { i = 0; j = 0; }
-    i += 32 * blk; j += 32 * blk;
-    float s1 = 0.f, s2 = 0.f;
-    for (int cc = 0; cc < CPR; ++cc) {
-      float ki[VEC], qi[VEC], kj[VEC], gi[VEC], gj[VEC];
-      unpack16<T>(ld16(Ks + i * LDK + cc * VEC), ki);
-      unpack16<T>(ld16(Qs + i * LDK + cc * VEC), qi);
-      unpack16<T>(ld16(Ks + j * LDK + cc * VEC), kj);
-      ld_f32<VEC>(Gs + i * LDG + cc * VEC, gi);
-      ld_f32<VEC>(Gs + j * LDG + cc * VEC, gj);
+          for (int e = 0; e < VEC; ++e) fb[e] *= __expf(-fabsf(ga[e] - gm[e]));
+        }
+        bfrag = pack16<T>(fb).raw;
+      }
+      mfma_kgroup<T>(acc, pack16<T>(fa).raw, bfrag);
+    }
+    return acc;
+  };
+  f32x16 a_diag = acc_zero(), a_low = acc_zero();
+  {
+    const int R = 32 * td + l32;
+    if (mat == 1) {   // the diagonal of q k^T: no decay
+      const f32x16 x = level_product(R, -1, R, -1);
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        const float x = __expf(gi[e] - gj[e]) * kj[e];
-        s1 += ki[e] * x;
-        s2 += qi[e] * x;
+      for (int r = 0; r < 16; ++r) a_diag[r] = acc_row(r) == l32 ? x[r] : 0.f;
+    }
+    for (int n = 2; n <= 32; n <<= 1) {   // blocks of n tokens: rows of the second half against rows of the first
+      const int m = (R / n) * n + n / 2;
+      const f32x16 x = level_product(R, m, R, m);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int i = acc_row(r), j = l32;
+        const bool keep = (i / n == j / n) && (i % n >= n / 2) && (j % n < n / 2);
+        a_diag[r] += keep ? x[r] : 0.f;
       }
     }
-    akk[t] = s1;
-    aqk[t] = s2;
+    if (wave < 2) a_low = level_product(32 + l32, 32, l32, 32);   // level 64: tokens 32..63 against 0..31, all kept
   }
-  GDN_LDS_BARRIER();   // X1, X2 are free
+  GDN_LDS_BARRIER();   // every wave is done with q as it lies: its place becomes the staging tile
 
-  // ---- phase 1c: what the recurrence reads.  K images through the staging rows into fragment order ----
+  // ---- phase 1c: what the recurrence reads, through a row-major staging tile (the q rows' place) into fragment order:
+  //      rows of q with scale and decay first (in place), then the two K images ----
+  for (int c = tid; c < 64 * CPR; c += kThreads) {
+    const int row = c / CPR, cc = c % CPR;
+    float f[VEC], gi[VEC];
+    unpack16<T>(ld16(Qs + row * LDK + cc * VEC), f);
+    ld_f32<VEC>(Gs + row * LDG + cc * VEC, gi);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) f[e] *= scale * __expf(gi[e]);
+    const Vec16<T> x = pack16<T>(f);
+    if (row < nvalid) st16(QB_out + (tok0 + row) * hk + h * DK + cc * VEC, x);   // row-major for the output kernel
+    st16(Qs + row * LDK + cc * VEC, x);
+  }
+  if (QBT_out != nullptr) {   // transposed tiles for a backward pass
+    GDN_LDS_BARRIER();
+    for (int tt = wave; tt < 2 * (DK / 32); tt += 4) {
+      const int tj = tt & 1, kt2 = tt >> 1;
+      AccB<T> kf;
+      kf.load_cols(Qs + 32 * tj * LDK + 32 * kt2, LDK);
+      kf.store_stream(QBT_out + ((ch * (DK / 32) + kt2) * 2 + tj) * 1024);
+    }
+  }
   auto stage_k = [&](bool first) {
     for (int c = tid; c < 64 * CPR; c += kThreads) {
       const int row = c / CPR, cc = c % CPR;
@@ -207,17 +238,18 @@ __global__ __launch_bounds__(kThreads) void kda_prep_kernel(
       const float nb = -bs[row];
 #pragma unroll
       for (int e = 0; e < VEC; ++e) f[e] *= first ? nb * __expf(gi[e]) : __expf(gl[e] - gi[e]);
-      st16(X1 + row * LDK + cc * VEC, pack16<T>(f));
+      st16(Qs + row * LDK + cc * VEC, pack16<T>(f));
     }
   };
   auto store_k = [&](T* out) {
     for (int tt = wave; tt < 2 * (DK / 32); tt += 4) {
       const int tj = tt & 1, kt2 = tt >> 1;
       AccB<T> kf;
-      frags_from_lds<T>(kf, X1 + (32 * tj + (lane & 31)) * LDK + 32 * kt2);
+      frags_from_lds<T>(kf, Qs + (32 * tj + (lane & 31)) * LDK + 32 * kt2);
       kf.store_stream(out + ((ch * (DK / 32) + kt2) * 2 + tj) * 1024);
     }
   };
+  GDN_LDS_BARRIER();
   stage_k(true);
   GDN_LDS_BARRIER();
   store_k(K1_out);
@@ -225,29 +257,7 @@ __global__ __launch_bounds__(kThreads) void kda_prep_kernel(
   stage_k(false);
   GDN_LDS_BARRIER();
   store_k(K2_out);
-  GDN_LDS_BARRIER();
-  // rows of q with scale and decay (row-major for the output kernel; transposed tiles for a backward pass), the decay
-  // of the whole chunk per channel, the cumulative decay itself
-  for (int c = tid; c < 64 * CPR; c += kThreads) {
-    const int row = c / CPR, cc = c % CPR;
-    float f[VEC], gi[VEC];
-    unpack16<T>(ld16(Qs + row * LDK + cc * VEC), f);
-    ld_f32<VEC>(Gs + row * LDG + cc * VEC, gi);
-#pragma unroll
-    for (int e = 0; e < VEC; ++e) f[e] *= scale * __expf(gi[e]);
-    const Vec16<T> x = pack16<T>(f);
-    if (row < nvalid) st16(QB_out + (tok0 + row) * hk + h * DK + cc * VEC, x);
-    st16(X1 + row * LDK + cc * VEC, x);
-  }
-  if (QBT_out != nullptr) {
-    GDN_LDS_BARRIER();
-    for (int tt = wave; tt < 2 * (DK / 32); tt += 4) {
-      const int tj = tt & 1, kt2 = tt >> 1;
-      AccB<T> kf;
-      kf.load_cols(X1 + 32 * tj * LDK + 32 * kt2, LDK);
-      kf.store_stream(QBT_out + ((ch * (DK / 32) + kt2) * 2 + tj) * 1024);
-    }
-  }
+  // the decay of the whole chunk per channel, the cumulative decay itself
   if (tid < DK) dec_out[ch * DK + tid] = __expf(Gs[63 * LDG + tid]);
   if (G_out != nullptr) {
     for (int c = tid; c < 64 * (DK / 4); c += kThreads) {
@@ -255,25 +265,19 @@ __global__ __launch_bounds__(kThreads) void kda_prep_kernel(
       *reinterpret_cast<f32x4*>(G_out + (ch * 64 + row) * DK + 4 * c4) = *reinterpret_cast<const f32x4*>(Gs + row * LDG + 4 * c4);
     }
   }
-  GDN_LDS_BARRIER();   // k, q, G and the staging rows are dead
+  GDN_LDS_BARRIER();   // k, the staging tile and G are dead
 
   // ---- phase 1d: L and Aq as 64x64 fp32 matrices ----
   for (int i = tid; i < 64 * kLF; i += kThreads) { As[i] = 0.f; Aqs[i] = 0.f; Ti[i] = 0.f; }
   GDN_LDS_BARRIER();
 #pragma unroll
-  for (int t = 0; t < 5; ++t) {
-    const int p = cg + 8 * t;
-    if (p < 33) {
-      const int i = 32 * blk + (p <= rp ? rp : 31 - rp), j = 32 * blk + (p <= rp ? p : p - rp - 1);
-      As[i * kLF + j] = i > j ? bs[i] * akk[t] : 0.f;
-      Aqs[i * kLF + j] = scale * aqk[t];
-    }
-  }
-  if (wave < 2) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int i = 32 + acc_row(r), j = acc_col();
-      if (wave == 0) As[i * kLF + j] = bs[i] * acc[r]; else Aqs[i * kLF + j] = scale * acc[r];
+  for (int r = 0; r < 16; ++r) {
+    const int i = 32 * td + acc_row(r), j = 32 * td + l32;
+    if (mat == 0) As[i * kLF + j] = i > j ? bs[i] * a_diag[r] : 0.f;
+    else Aqs[i * kLF + j] = i >= j ? scale * a_diag[r] : 0.f;
+    if (wave < 2) {
+      const int i2 = 32 + acc_row(r);
+      if (mat == 0) As[i2 * kLF + l32] = bs[i2] * a_low[r]; else Aqs[i2 * kLF + l32] = scale * a_low[r];
     }
   }
   GDN_LDS_BARRIER();

@@ -9,7 +9,7 @@ enum KernelId {
   kKernChunkTable = 0, kKernPrep, kKernStateFwd, kKernOut, kKernStateBwd, kKernBwdLocal,
   kKernRecurrent, kKernConvFwd, kKernConvState, kKernConvBwd, kKernConvReduce,
   kKernConvDh0, kKernConvUpdate, kKernRmsNormFwd, kKernRmsNormBwd, kKernRmsNormReduce,
-  kKernGateFwd, kKernGateBwd, kKernGateReduce, kKernKdaPrep, kKernKdaBwdFinish, kKernCount
+  kKernGateFwd, kKernGateBwd, kKernGateReduce, kKernKdaPrep, kKernKdaBwdFinish, kKernKdaBwdReduce, kKernCount
 };
 
 bool profile_on();

@@ -14,7 +14,7 @@ static const char* const kNames[kKernCount] = {
     "recurrent_kernel", "conv1d_fwd_kernel", "conv1d_final_state_kernel",
     "conv1d_bwd_kernel", "conv1d_reduce_kernel", "conv1d_dh0_kernel", "conv1d_update_kernel",
     "rmsnorm_gated_fwd_kernel", "rmsnorm_gated_bwd_kernel", "rmsnorm_gated_dw_reduce_kernel",
-    "gate_fwd_kernel", "gate_bwd_kernel", "gate_reduce_kernel", "kda_prep_kernel", "kda_bwd_finish_kernel"};
+    "gate_fwd_kernel", "gate_bwd_kernel", "gate_reduce_kernel", "kda_prep_kernel", "kda_bwd_finish_kernel", "kda_bwd_reduce_kernel"};
 
 struct Pending { int id; hipEvent_t a, b; };
 static bool g_on = false;

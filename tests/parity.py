@@ -15,7 +15,9 @@ from oracle import kda_oracle as KO
 FP32_REL = 1e-4
 BF16_ABS_O = 2e-2
 BF16_ABS_GRAD = 5e-2
-# dA_log and d(dt_bias) are sums over every token of the batch: their error bound grows with their size
+# dA_log and d(dt_bias) are sums over every token of the batch (dA_log over the channels too) of terms of both signs,
+# each within the bound above: the error of the sum grows like a random walk, with the square root of the number of
+# chunks, while the sum itself may cancel; 2 % of the reference on top
 KDA_PARAM_RTOL = 2e-2
 
 
@@ -464,5 +466,8 @@ def check_kda(ops, device, B, T, H, K, V, dtype, cu=None, seed=0, with_h0=True, 
                 continue
             assert leaves[n].grad is not None, n
             assert leaves[n].grad.dtype == leaves[n].dtype and leaves[n].grad.shape == leaves[n].shape
-            errs["d" + n] = _err("d" + n, leaves[n].grad, ref[n].grad, dtype, BF16_ABS_GRAD, rtol=KDA_PARAM_RTOL if n in ("A_log", "dt_bias") else 0.0)
+            param = n in ("A_log", "dt_bias")
+            errs["d" + n] = _err("d" + n, leaves[n].grad, ref[n].grad, dtype,
+                                 BF16_ABS_GRAD * (max(1.0, B * T / 64.0) ** 0.5 if param else 1.0),
+                                 rtol=KDA_PARAM_RTOL if param else 0.0)
     return errs
