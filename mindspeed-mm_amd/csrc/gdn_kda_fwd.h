@@ -40,7 +40,7 @@ template <typename T, int DK> struct KdaPrepSmem {
 };
 
 template <typename T, int DK>
-__global__ __launch_bounds__(kThreads) void kda_prep_kernel(
+__global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const void* __restrict__ g, const void* __restrict__ beta,
     const float* __restrict__ A_log, const float* __restrict__ dt_bias, const int64_t* __restrict__ cu,
     const int* __restrict__ chunk_offsets, float* __restrict__ bhat_out, float* __restrict__ dec_out,
@@ -151,58 +151,62 @@ __global__ __launch_bounds__(kThreads) void kda_prep_kernel(
   //      tile w >> 1; the tile below the diagonal (level 64) goes to waves 0 and 1 ----
   const int mat = wave & 1, td = wave >> 1, l32 = lane & 31, half = lane >> 5;
   constexpr int KGL = KGroup<T>::kLen, NKG = DK / KGL;
-  // one product X_A[rows ra] X_K[rows rb]^T over all channels, rows rescaled around row ma / mb of G (negative: as they are)
-  auto level_product = [&](int ra, int ma, int rb, int mb) {
-    f32x16 acc = acc_zero();
-    const T* arow = (mat ? Qs : Ks) + ra * LDK;
-    const T* brow = Ks + rb * LDK;
-#pragma unroll 2
-    for (int kg = 0; kg < NKG; ++kg) {
-      const int c0 = kg * KGL + half * VEC;
-      float fa[VEC], fb[VEC], ga[VEC], gm[VEC];
-      unpack16<T>(ld16(arow + c0), fa);
-      if (ma >= 0) {
-        ld_f32<VEC>(Gs + ra * LDG + c0, ga);
-        ld_f32<VEC>(Gs + ma * LDG + c0, gm);
+  // All levels advance together through the channels: the rows of k, q and G are read once per group of channels and
+  // only the reference row of G differs from level to level; the products of the levels are independent chains.
+  f32x16 lv[5], a_dg = acc_zero(), a_low = acc_zero();
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) fa[e] *= __expf(-fabsf(ga[e] - gm[e]));
-      }
-      u32x4 bfrag;
-      if (mat == 0 && ra == rb) {
-        bfrag = pack16<T>(fa).raw;   // k k^T on a diagonal tile: both operands are the same rows
-      } else {
-        unpack16<T>(ld16(brow + c0), fb);
-        if (mb >= 0) {
-          ld_f32<VEC>(Gs + rb * LDG + c0, ga);
-          ld_f32<VEC>(Gs + mb * LDG + c0, gm);
+  for (int i = 0; i < 5; ++i) lv[i] = acc_zero();
+  const int R = 32 * td + l32;
+#pragma unroll 1
+  for (int kg = 0; kg < NKG; ++kg) {
+    const int c0 = kg * KGL + half * VEC;
+    float fk[VEC], fa[VEC], gR[VEC];
+    unpack16<T>(ld16(Ks + R * LDK + c0), fk);
+    if (mat) unpack16<T>(ld16(Qs + R * LDK + c0), fa);
+    else {
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) fb[e] *= __expf(-fabsf(ga[e] - gm[e]));
-        }
-        bfrag = pack16<T>(fb).raw;
-      }
-      mfma_kgroup<T>(acc, pack16<T>(fa).raw, bfrag);
+      for (int e = 0; e < VEC; ++e) fa[e] = fk[e];
     }
-    return acc;
-  };
-  f32x16 a_diag = acc_zero(), a_low = acc_zero();
-  {
-    const int R = 32 * td + l32;
-    if (mat == 1) {   // the diagonal of q k^T: no decay
-      const f32x16 x = level_product(R, -1, R, -1);
+    ld_f32<VEC>(Gs + R * LDG + c0, gR);
+    if (mat) mfma_kgroup<T>(a_dg, pack16<T>(fa).raw, pack16<T>(fk).raw);   // the diagonal of q k^T: no decay
 #pragma unroll
-      for (int r = 0; r < 16; ++r) a_diag[r] = acc_row(r) == l32 ? x[r] : 0.f;
-    }
-    for (int n = 2; n <= 32; n <<= 1) {   // blocks of n tokens: rows of the second half against rows of the first
-      const int m = (R / n) * n + n / 2;
-      const f32x16 x = level_product(R, m, R, m);
+    for (int i = 0; i < 5; ++i) {   // blocks of n = 2 << i tokens: rows of the second half against rows of the first
+      const int n = 2 << i, m = (R / n) * n + n / 2;
+      float gm[VEC], xa[VEC], xb[VEC];
+      ld_f32<VEC>(Gs + m * LDG + c0, gm);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int i = acc_row(r), j = l32;
-        const bool keep = (i / n == j / n) && (i % n >= n / 2) && (j % n < n / 2);
-        a_diag[r] += keep ? x[r] : 0.f;
+      for (int e = 0; e < VEC; ++e) {
+        const float f = __expf(-fabsf(gR[e] - gm[e]));
+        xa[e] = fa[e] * f;
+        xb[e] = fk[e] * f;
       }
+      const u32x4 afrag = pack16<T>(xa).raw;
+      mfma_kgroup<T>(lv[i], afrag, mat ? pack16<T>(xb).raw : afrag);
     }
-    if (wave < 2) a_low = level_product(32 + l32, 32, l32, 32);   // level 64: tokens 32..63 against 0..31, all kept
+    if (wave < 2) {   // level 64: tokens 32..63 against 0..31 (these waves' rows R), all entries kept
+      float gm[VEC], ga[VEC], xa[VEC], xb[VEC];
+      ld_f32<VEC>(Gs + 32 * LDG + c0, gm);
+      ld_f32<VEC>(Gs + (32 + l32) * LDG + c0, ga);
+      unpack16<T>(ld16((mat ? Qs : Ks) + (32 + l32) * LDK + c0), xa);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        xa[e] *= __expf(-fabsf(ga[e] - gm[e]));
+        xb[e] = fk[e] * __expf(-fabsf(gR[e] - gm[e]));
+      }
+      mfma_kgroup<T>(a_low, pack16<T>(xa).raw, pack16<T>(xb).raw);
+    }
+  }
+  f32x16 a_diag;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int i = acc_row(r), j = l32;
+    float x = (mat == 1 && i == j) ? a_dg[r] : 0.f;
+#pragma unroll
+    for (int q2 = 0; q2 < 5; ++q2) {
+      const int n = 2 << q2;
+      x += ((i / n == j / n) && (i % n >= n / 2) && (j % n < n / 2)) ? lv[q2][r] : 0.f;
+    }
+    a_diag[r] = x;
   }
   GDN_LDS_BARRIER();   // every wave is done with q as it lies: its place becomes the staging tile
 
