@@ -20,9 +20,12 @@
 //   dG_last = sum_i k^_i . e^{G_last-G_i} . dK2_i + dD . e^{G_last}               per channel
 //   db_i = <R_i, v_i> + sum_d k^_id (U_id - e^{G_id} dK1_id)
 //   dg_t = sum_{i>=t} dG_i + dG_last, then back through the gate, the l2 norm and the sigmoid of beta.
-// The decay-weighted sums over a chunk use the split of the forward pass: within the two 32-token blocks term by term in
-// fp32 with the exact exponent, between the blocks on the matrix cores with rows rescaled at the block boundary (for
-// fp32 operands, whose tiles would not fit LDS beside everything else, every pair is summed term by term).
+// The decay-weighted sums over a chunk use the recursive halving of the forward pass: a pair i > j belongs to one block
+// of one level (64, 32, ..., 2 tokens), in which i lies in the second half and j in the first, and there
+// e^{G_i-G_j} = e^{G_i-G_m} e^{G_m-G_j} with m the middle of the block, both factors at most 1.  Per level the
+// coefficients outside that level's pairs are masked away, the partner rows are rescaled in registers straight into
+// the B-operand layout, the products run on the matrix cores and the rows of the result are scaled by their own
+// factor.  (For fp32 operands every pair is summed term by term in fp32 instead.)
 #pragma once
 #include "gdn_kda_common.h"
 
@@ -37,14 +40,9 @@ template <typename T, int DK> struct KdaBwdSmem {
   static constexpr int off_gs = off_qs + tile;       // first Kp as T (64 rows), then G rows (fp32)
   static constexpr int off_m1 = off_gs + gmat;       // dTm, then dL; later, with the next one, the store patches
   static constexpr int off_m2 = off_m1 + mat;        // X = Tm^T dTm, then scale dAq
-  static constexpr int off_tm = off_m2 + mat;        // Tm row-major
-  static constexpr int off_xi = off_tm + mat;        // rescaled rows [b k ; q] of tokens 32..63 (not FULL)
-  static constexpr int off_xr = off_xi + (FULL ? 0 : tile);       // rescaled rows k of tokens 0..31
-  // 16-bit operands: once Tm and the rescaled rows are consumed their place takes the two coefficients of every pair
-  // packed into one word, (dL_ij | scale dAq_ij << 16), row-major [i][j] and transposed [j][i] (uint32 [64][kLC] each)
-  static constexpr int kLC = 68, off_mc = off_tm, off_mct = off_mc + 64 * kLC * 4;
-  static constexpr int cmax(int a, int b) { return a > b ? a : b; }
-  static constexpr int off_row = FULL ? off_xr : cmax(off_xr + tile / 2, off_mct + 64 * kLC * 4);
+  static constexpr int off_tm = off_m2 + mat;        // Tm row-major, then dL transposed
+  static constexpr int off_m2t = off_tm + mat;       // scale dAq transposed (not FULL)
+  static constexpr int off_row = off_m2t + (FULL ? 0 : mat);
   // beta, 1/|q|, 1/|k| [64 each]; per-wave row sums <q^,dq^>, <k^,dk^>, db, <R,v> [256 each]; 8 scalars
   static constexpr int bytes = off_row + (3 * 64 + 4 * 256 + 8) * 4;
   static_assert(tile <= gmat, "Kp fits where G will be");
@@ -70,11 +68,8 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
   T* TmT = reinterpret_cast<T*>(gdn_smem + SM::off_tm);
   T* M1 = reinterpret_cast<T*>(gdn_smem + SM::off_m1);
   T* M2 = reinterpret_cast<T*>(gdn_smem + SM::off_m2);
-  T* XI = reinterpret_cast<T*>(gdn_smem + SM::off_xi);
-  T* XR = reinterpret_cast<T*>(gdn_smem + SM::off_xr);
-  uint32_t* MC = reinterpret_cast<uint32_t*>(gdn_smem + SM::off_mc);
-  uint32_t* MCt = reinterpret_cast<uint32_t*>(gdn_smem + SM::off_mct);
-  constexpr int kLC = SM::kLC;
+  T* M1t = TmT;
+  T* M2t = reinterpret_cast<T*>(gdn_smem + SM::off_m2t);
   float* bs = reinterpret_cast<float*>(gdn_smem + SM::off_row);
   float* rsq = bs + 64;
   float* rsk = rsq + 64;
@@ -187,6 +182,11 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
     const int at = (32 * ti + acc_row(r)) * L64 + 32 * tj + l32;
     M1[at] = Elem<T>::from_f(dl[r]);
     M2[at] = Elem<T>::from_f(sa[r]);
+    if constexpr (!FULL) {
+      const int att = (32 * tj + l32) * L64 + 32 * ti + acc_row(r);
+      M1t[att] = Elem<T>::from_f(dl[r]);
+      M2t[att] = Elem<T>::from_f(sa[r]);
+    }
   }
   {
     TileQK<T, DK> qt;
@@ -216,86 +216,134 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
       }
   }
   if constexpr (!FULL) {
-    // between the blocks: rows rescaled around the decay at the boundary, [b k ; q]_i e^{G_i-G_31} and k_j e^{G_31-G_j}
-    for (int c = tid; c < 96 * CPR; c += kThreads) {
-      const int r = c / CPR, cc = c % CPR;
-      const int src = r < 32 ? 32 + r : (r < 64 ? r : r - 64);
-      const T* from = (r >= 32 && r < 64) ? Qs : Ks;
-      float f[VEC], gi[VEC], gr[VEC];
-      unpack16<T>(ld16(from + src * LDK + cc * VEC), f);
-      ld_f32<VEC>(Gs + src * LDG + cc * VEC, gi);
-      ld_f32<VEC>(Gs + 31 * LDG + cc * VEC, gr);
-      const float b = r < 32 ? bs[src] : 1.f;
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) f[e] *= b * __expf(r < 64 ? gi[e] - gr[e] : gr[e] - gi[e]);
-      T* to = r < 64 ? XI + r * LDK : XR + (r - 64) * LDK;
-      st16(to + cc * VEC, pack16<T>(f));
-    }
-    GDN_LDS_BARRIER();
     if (has_k) {
-      const float g31 = Gs[31 * LDG + d];
-      f32x16 u = acc_zero(), uq = acc_zero(), w = acc_zero();
-      mma32<T, 32, true, false>(u, M1 + 32 * L64, L64, XR + 32 * cj, LDK);     // sum_j dL[32+i][j] KR[j][d]
-      mma32<T, 32, true, false>(uq, M2 + 32 * L64, L64, XR + 32 * cj, LDK);
-      mma32<T, 32, false, false>(w, M1 + 32 * L64, L64, XI + 32 * cj, LDK);    // sum_i dL[32+i][j] (b k)_i[d]
-      mma32<T, 32, false, false>(w, M2 + 32 * L64, L64, XI + 32 * LDK + 32 * cj, LDK);
+      const int half = lane >> 5;
+      // fragment of a coefficient matrix: row `row`, 8 consecutive columns from `col0`, of which only those of the
+      // level's pairs are kept.  second: the row index is the later token i (kept when i is in the second half of its
+      // block and the column j in the first), else the row index is the earlier token j.
+      auto coef = [&](const T* M, int row, int col0, int a, int b0, int lg, bool second) {
+        u32x4 w = ld16(M + row * L64 + col0).raw;
+        const int n2 = (1 << lg) >> 1, nm = (1 << lg) - 1;
+        const bool rok = second ? ((a & nm) >= n2) : ((a & nm) < n2);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float e1 = __expf(Gi[1][r] - g31);
-        U[1][r] = u[r] * e1;
-        Uq[1][r] = uq[r] * e1;
-        W[0][r] = w[r] * __expf(g31 - Gi[0][r]);
+        for (int e = 0; e < 4; ++e) {
+          const int b1 = b0 + 2 * e, b2 = b1 + 1;
+          const bool k1 = rok && (a >> lg) == (b1 >> lg) && (second ? ((b1 & nm) < n2) : ((b1 & nm) >= n2));
+          const bool k2 = rok && (a >> lg) == (b2 >> lg) && (second ? ((b2 & nm) < n2) : ((b2 & nm) >= n2));
+          w[e] &= (k1 ? 0xffffu : 0u) | (k2 ? 0xffff0000u : 0u);
+        }
+        return w;
+      };
+#pragma unroll
+      for (int ri = 0; ri < 2; ++ri) {
+        // the partner rows this lane supplies as B operand, channel d: tokens 32 ri + 16 kg + 8 half + e
+        float kj[2][8], bk[2][8], qj[2][8], gj[2][8];
+#pragma unroll
+        for (int kg = 0; kg < 2; ++kg)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const int x = 32 * ri + 16 * kg + 8 * half + e;
+            gj[kg][e] = Gs[x * LDG + d];
+            kj[kg][e] = Elem<T>::to_f(Ks[x * LDK + d]);
+            bk[kg][e] = bs[x] * kj[kg][e];
+            qj[kg][e] = Elem<T>::to_f(Qs[x * LDK + d]);
+          }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {   // the pair i = j: no decay (dL has no diagonal)
+          const int i = 32 * ri + acc_row(r);
+          const float c = Elem<T>::to_f(M2[i * L64 + i]);
+          Uq[ri][r] += c * ki[ri][r];
+          W[ri][r] += c * qi[ri][r];
+        }
+#pragma unroll 1
+        for (int lg = 1; lg <= 5; ++lg) {   // blocks of n = 2^lg tokens inside the 32-token block
+          const int n = 1 << lg;
+          f32x16 cu = acc_zero(), cq = acc_zero(), cw = acc_zero();
+#pragma unroll
+          for (int kg = 0; kg < 2; ++kg) {
+            float xk[8], xb[8], xq[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const int x = 32 * ri + 16 * kg + 8 * half + e, m = ((x >> lg) << lg) + (n >> 1);
+              const float f = __expf(-fabsf(gj[kg][e] - Gs[m * LDG + d]));
+              xk[e] = kj[kg][e] * f; xb[e] = bk[kg][e] * f; xq[e] = qj[kg][e] * f;
+            }
+            const u32x4 bK = pack16<T>(xk).raw, bB = pack16<T>(xb).raw, bQ = pack16<T>(xq).raw;
+            const int row = 32 * ri + l32, col0 = 32 * ri + 16 * kg + 8 * half, b0 = 16 * kg + 8 * half;
+            mfma_kgroup<T>(cu, coef(M1, row, col0, l32, b0, lg, true), bK);     // sum_j dL_ij (k_j f_j)
+            mfma_kgroup<T>(cq, coef(M2, row, col0, l32, b0, lg, true), bK);
+            mfma_kgroup<T>(cw, coef(M1t, row, col0, l32, b0, lg, false), bB);   // sum_i dL_ij (b_i k_i f_i)
+            mfma_kgroup<T>(cw, coef(M2t, row, col0, l32, b0, lg, false), bQ);
+          }
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {   // every row by its own factor
+            const int i = 32 * ri + acc_row(r), m = ((i >> lg) << lg) + (n >> 1);
+            const float f = __expf(-fabsf(Gi[ri][r] - Gs[m * LDG + d]));
+            U[ri][r] += f * cu[r];
+            Uq[ri][r] += f * cq[r];
+            W[ri][r] += f * cw[r];
+          }
+        }
+      }
+      {   // the level of the whole chunk: tokens 32..63 against tokens 0..31, m = 32, every pair kept
+        const float g32v = Gs[32 * LDG + d];
+        f32x16 cu = acc_zero(), cq = acc_zero(), cw = acc_zero();
+#pragma unroll
+        for (int kg = 0; kg < 2; ++kg) {
+          float xk[8], xb[8], xq[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const int j = 16 * kg + 8 * half + e, i = 32 + j;
+            xk[e] = Elem<T>::to_f(Ks[j * LDK + d]) * __expf(-fabsf(Gs[j * LDG + d] - g32v));
+            const float f = __expf(-fabsf(Gs[i * LDG + d] - g32v));
+            xb[e] = bs[i] * Elem<T>::to_f(Ks[i * LDK + d]) * f;
+            xq[e] = Elem<T>::to_f(Qs[i * LDK + d]) * f;
+          }
+          const int c0 = 16 * kg + 8 * half;
+          mfma_kgroup<T>(cu, ld16(M1 + (32 + l32) * L64 + c0).raw, pack16<T>(xk).raw);
+          mfma_kgroup<T>(cq, ld16(M2 + (32 + l32) * L64 + c0).raw, pack16<T>(xk).raw);
+          mfma_kgroup<T>(cw, ld16(M1t + l32 * L64 + 32 + c0).raw, pack16<T>(xb).raw);
+          mfma_kgroup<T>(cw, ld16(M2t + l32 * L64 + 32 + c0).raw, pack16<T>(xq).raw);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float f1 = __expf(-fabsf(Gi[1][r] - g32v)), f0 = __expf(-fabsf(Gi[0][r] - g32v));
+          U[1][r] += f1 * cu[r];
+          Uq[1][r] += f1 * cq[r];
+          W[0][r] += f0 * cw[r];
+        }
       }
     }
-    GDN_LDS_BARRIER();   // Tm and the rescaled rows are consumed
-    for (int c = tid; c < 64 * 64; c += kThreads) {
-      const int i = c >> 6, j = c & 63;
-      uint32_t w = 0;
-      if constexpr (sizeof(T) == 2) w = (uint32_t)M1[i * L64 + j].bits | ((uint32_t)M2[i * L64 + j].bits << 16);
-      MC[i * kLC + j] = w;
-      MCt[j * kLC + i] = w;
-    }
-    GDN_LDS_BARRIER();
   }
-  if (has_k) {
+  if (FULL && has_k) {
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {
-      // rows i of this lane against the earlier rows j of the block (of the chunk when FULL)
-      for (int jj = FULL ? 0 : 32 * ri; jj <= 32 * ri + 31; ++jj) {
+      // rows i of this lane against the earlier rows j of the chunk
+      for (int jj = 0; jj <= 32 * ri + 31; ++jj) {
         const float gj = Gs[jj * LDG + d], kj = Elem<T>::to_f(Ks[jj * LDK + d]);
 #pragma unroll
         for (int qd = 0; qd < 4; ++qd) {
           if (32 * ri + 8 * qd + 7 < jj) continue;   // none of the group's rows reaches jj (same for every lane)
-          u32x4 cw = {0u, 0u, 0u, 0u};
-          if constexpr (!FULL) cw = *reinterpret_cast<const u32x4*>(MCt + jj * kLC + 32 * ri + acc_row(4 * qd));
 #pragma unroll
           for (int m = 0; m < 4; ++m) {
             const int r = 4 * qd + m, i = 32 * ri + acc_row(r);
             const float t = kj * __expf(i >= jj ? Gi[ri][r] - gj : 0.f);
-            float cl, cq;   // coefficients are zero where i < jj
-            if constexpr (FULL) { cl = Elem<T>::to_f(M1[i * L64 + jj]); cq = Elem<T>::to_f(M2[i * L64 + jj]); }
-            else { cl = __uint_as_float(cw[m] << 16); cq = __uint_as_float(cw[m] & 0xffff0000u); }
-            U[ri][r] += cl * t;
-            Uq[ri][r] += cq * t;
+            U[ri][r] += Elem<T>::to_f(M1[i * L64 + jj]) * t;    // coefficients are zero where i < jj
+            Uq[ri][r] += Elem<T>::to_f(M2[i * L64 + jj]) * t;
           }
         }
       }
       // rows j of this lane against the later rows i
-      for (int ii = 32 * ri; ii <= (FULL ? 63 : 32 * ri + 31); ++ii) {
+      for (int ii = 32 * ri; ii <= 63; ++ii) {
         const float gi = Gs[ii * LDG + d], kb = bs[ii] * Elem<T>::to_f(Ks[ii * LDK + d]), qv = Elem<T>::to_f(Qs[ii * LDK + d]);
 #pragma unroll
         for (int qd = 0; qd < 4; ++qd) {
           if (32 * ri + 8 * qd > ii) continue;
-          u32x4 cw = {0u, 0u, 0u, 0u};
-          if constexpr (!FULL) cw = *reinterpret_cast<const u32x4*>(MC + ii * kLC + 32 * ri + acc_row(4 * qd));
 #pragma unroll
           for (int m = 0; m < 4; ++m) {
             const int r = 4 * qd + m, j = 32 * ri + acc_row(r);
             const float e = __expf(ii >= j ? gi - Gi[ri][r] : 0.f);
-            float cl, cq;
-            if constexpr (FULL) { cl = Elem<T>::to_f(M1[ii * L64 + j]); cq = Elem<T>::to_f(M2[ii * L64 + j]); }
-            else { cl = __uint_as_float(cw[m] << 16); cq = __uint_as_float(cw[m] & 0xffff0000u); }
-            W[ri][r] += (cl * kb + cq * qv) * e;
+            W[ri][r] += (Elem<T>::to_f(M1[ii * L64 + j]) * kb + Elem<T>::to_f(M2[ii * L64 + j]) * qv) * e;
           }
         }
       }
