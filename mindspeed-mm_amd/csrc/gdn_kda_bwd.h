@@ -108,27 +108,50 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
     rsk[tid] = 1.f;
   }
   rq[tid] = 0.f; rk[tid] = 0.f; rb[tid] = 0.f; rv[tid] = 0.f;
-  for (int c = tid; c < 64 * CPR; c += kThreads) {
-    const int row = c / CPR, cc = c % CPR;
+  // this thread's pieces of P and G (VEC consecutive channels of a row each), all requested before the first wait
+  constexpr int NIT = 64 * CPR / kThreads, C64 = 64 / VEC, NTM = 64 * C64 / kThreads;
+  static_assert(64 * CPR % kThreads == 0 && 64 * C64 % kThreads == 0 && VEC % 4 == 0, "whole rounds of 16-byte pieces");
+  f32x4 pf[NIT][VEC / 4], gk[NIT][VEC / 4];
+  Vec16<T> tmv[NTM];
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int c = tid + it * kThreads, at = (c / CPR) * DK + (c % CPR) * VEC;
+#pragma unroll
+    for (int e = 0; e < VEC / 4; ++e) {
+      pf[it][e] = *reinterpret_cast<const f32x4*>(Pm + at + 4 * e);
+      gk[it][e] = *reinterpret_cast<const f32x4*>(Gc + at + 4 * e);
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < NTM; ++it) {
+    const int c = tid + it * kThreads;
+    tmv[it] = ld16(TMR + ch * 4096 + (c / C64) * 64 + (c % C64) * VEC);
+  }
+  TileQK<T, DK> qt;
+  tile_qk_request<T, DK>(qt, q + tok0 * hk + h * DK, hk, nvalid, tid);
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int c = tid + it * kThreads;
     float f[VEC];
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) f[e] = Pm[row * DK + cc * VEC + e];
-    st16(Pt + row * LDK + cc * VEC, pack16<T>(f));
+    for (int e = 0; e < VEC; ++e) f[e] = pf[it][e / 4][e % 4];
+    st16(Pt + (c / CPR) * LDK + (c % CPR) * VEC, pack16<T>(f));
   }
-  {
-    constexpr int C64 = 64 / VEC;
-    for (int c = tid; c < 64 * C64; c += kThreads)
-      st16(TmT + (c / C64) * L64 + (c % C64) * VEC, ld16(TMR + ch * 4096 + (c / C64) * 64 + (c % C64) * VEC));
+#pragma unroll
+  for (int it = 0; it < NTM; ++it) {
+    const int c = tid + it * kThreads;
+    st16(TmT + (c / C64) * L64 + (c % C64) * VEC, tmv[it]);
   }
   GDN_LDS_BARRIER();   // the row vectors are initialised before the norm below writes 1/|k| over its entries
   tile_qk_finish<T, DK>(kt, Ks, LDK, nvalid, tid, fl.l2norm != 0, nullptr, 0, rsk, 1);
   GDN_LDS_BARRIER();
-  for (int c = tid; c < 64 * CPR; c += kThreads) {   // Kp = k^ . e^{G}
-    const int row = c / CPR, cc = c % CPR;
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {   // Kp = k^ . e^{G}
+    const int c = tid + it * kThreads, row = c / CPR, cc = c % CPR;
     float f[VEC];
     unpack16<T>(ld16(Ks + row * LDK + cc * VEC), f);
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) f[e] *= __expf(Gc[row * DK + cc * VEC + e]);
+    for (int e = 0; e < VEC; ++e) f[e] *= __expf(gk[it][e / 4][e % 4]);
     st16(Kp + row * LDK + cc * VEC, pack16<T>(f));
   }
   GDN_LDS_BARRIER();
@@ -188,14 +211,13 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
       M2t[att] = Elem<T>::from_f(sa[r]);
     }
   }
-  {
-    TileQK<T, DK> qt;
-    tile_qk_request<T, DK>(qt, q + tok0 * hk + h * DK, hk, nvalid, tid);
-    tile_qk_finish<T, DK>(qt, Qs, LDK, nvalid, tid, fl.l2norm != 0, nullptr, 0, rsq, 1);
-  }
-  for (int c = tid; c < 64 * (DK / 4); c += kThreads) {
-    const int row = c / (DK / 4), c4 = c % (DK / 4);
-    *reinterpret_cast<f32x4*>(Gs + row * LDG + 4 * c4) = *reinterpret_cast<const f32x4*>(Gc + row * DK + 4 * c4);
+  tile_qk_finish<T, DK>(qt, Qs, LDK, nvalid, tid, fl.l2norm != 0, nullptr, 0, rsq, 1);
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int c = tid + it * kThreads;
+#pragma unroll
+    for (int e = 0; e < VEC / 4; ++e)
+      *reinterpret_cast<f32x4*>(Gs + (c / CPR) * LDG + (c % CPR) * VEC + 4 * e) = gk[it][e];
   }
   GDN_LDS_BARRIER();
 
@@ -386,17 +408,24 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
   if (has_k) {
     // the raw gate input of this lane's rows, requested before the stores below
     const bool g32 = sizeof(T) == 4 || fl.g_f32;
-    float raws[2][16];
+    // (as bits, widened after the loop: a conversion inside it would make every load wait for the one before)
+    uint32_t raws[2][16];
     if (fl.use_gate) {
+      if (g32) {
 #pragma unroll
-      for (int ri = 0; ri < 2; ++ri)
+        for (int ri = 0; ri < 2; ++ri)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int64_t gat = (tok0 + imin(32 * ri + acc_row(r), nvalid - 1)) * hk + h * DK + d;
-          if (g32) raws[ri][r] = reinterpret_cast<const float*>(g)[gat];
-          else { T t; if constexpr (sizeof(T) == 2) t.bits = reinterpret_cast<const uint16_t*>(g)[gat]; raws[ri][r] = Elem<T>::to_f(t); }
-        }
+          for (int r = 0; r < 16; ++r)
+            raws[ri][r] = reinterpret_cast<const uint32_t*>(g)[(tok0 + imin(32 * ri + acc_row(r), nvalid - 1)) * hk + h * DK + d];
+      } else {
+#pragma unroll
+        for (int ri = 0; ri < 2; ++ri)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            raws[ri][r] = reinterpret_cast<const uint16_t*>(g)[(tok0 + imin(32 * ri + acc_row(r), nvalid - 1)) * hk + h * DK + d];
+      }
     }
+    const int raw_shift = g32 ? 0 : 16;
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {
       if (fl.l2norm) {
@@ -431,46 +460,55 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
     const float a = fl.use_gate ? __expf(A_log[h]) : 0.f;
     const float bias = (fl.use_gate && dt_bias != nullptr) ? dt_bias[h * DK + d] : 0.f;
     float dt_sum = 0.f;
+    // MODE 0: g is the log decay itself; 1: -e^{A_log} softplus(g + bias); 2: lower_bound sigmoid(e^{A_log} (g + bias)).
+    // One copy of the loop per mode: a test of the options per element would cost as much as the gate.
+    auto gate_back = [&](auto mode) {
+      constexpr int MODE = decltype(mode)::value;
 #pragma unroll
-    for (int ri = 0; ri < 2; ++ri) {
-      f32x16 dgr;
-      float later = ri == 0 ? blk[1] : 0.f;     // everything after the group being handled
+      for (int ri = 0; ri < 2; ++ri) {
+        f32x16 dgr;
+        float later = ri == 0 ? blk[1] : 0.f;     // everything after the group being handled
 #pragma unroll
-      for (int qd = 3; qd >= 0; --qd) {
-        float run = later + (first_half ? sx[ri][qd] : 0.f);
+        for (int qd = 3; qd >= 0; --qd) {
+          float run = later + (first_half ? sx[ri][qd] : 0.f);
 #pragma unroll
-        for (int m = 3; m >= 0; --m) {
-          const int r = 4 * qd + m, i = 32 * ri + acc_row(r);
-          run += dGv[ri][r];
-          float x = run + dglast;     // d(log decay of token i, channel d)
-          if (fl.use_gate) {
-            const float raw = raws[ri][r] + bias;
-            if (fl.has_lower_bound) {
-              const float sg = kda_sigmoid(a * raw), ds_ = fl.lower_bound * sg * (1.f - sg);
-              if (i < nvalid) da_sum += x * ds_ * a * raw;
-              x *= ds_ * a;
-            } else {
-              if (i < nvalid) da_sum += x * (-a * kda_softplus(raw));
-              x *= -a * kda_sigmoid(raw);
+          for (int m = 3; m >= 0; --m) {
+            const int r = 4 * qd + m, i = 32 * ri + acc_row(r);
+            run += dGv[ri][r];
+            float x = i < nvalid ? run + dglast : 0.f;     // d(log decay of token i, channel d)
+            if (MODE != 0) {
+              const float raw = __uint_as_float(raws[ri][r] << raw_shift) + bias;
+              if (MODE == 2) {
+                const float sg = kda_sigmoid(a * raw), ds_ = fl.lower_bound * sg * (1.f - sg);
+                da_sum += x * ds_ * a * raw;
+                x *= ds_ * a;
+              } else {
+                float sp, sg;
+                kda_softplus_sigmoid(raw, sp, sg);
+                da_sum -= x * a * sp;
+                x *= -a * sg;
+              }
             }
+            dt_sum += x;
+            dgr[r] = x;
           }
-          if (i >= nvalid) x = 0.f;
-          dt_sum += x;
-          dgr[r] = x;
+          later += so[ri][qd] + sx[ri][qd];
         }
-        later += so[ri][qd] + sx[ri][qd];
-      }
-      if (g32) {
+        if (g32) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int i = 32 * ri + acc_row(r);
-          if (i < nvalid) reinterpret_cast<float*>(dg)[(tok0 + i) * hk + h * DK + d] = dgr[r];
+          for (int r = 0; r < 16; ++r) {
+            const int i = 32 * ri + acc_row(r);
+            if (i < nvalid) reinterpret_cast<float*>(dg)[(tok0 + i) * hk + h * DK + d] = dgr[r];
+          }
+        } else {
+          acc_store_rows<T, false>(dgr, id, patch, reinterpret_cast<T*>(dg) + (tok0 + 32 * ri) * hk + h * DK + 32 * cj, hk,
+                                   nvalid - 32 * ri);
         }
-      } else {
-        acc_store_rows<T, false>(dgr, id, patch, reinterpret_cast<T*>(dg) + (tok0 + 32 * ri) * hk + h * DK + 32 * cj, hk,
-                                 nvalid - 32 * ri);
       }
-    }
+    };
+    if (!fl.use_gate) gate_back(IntConst<0>());
+    else if (!fl.has_lower_bound) gate_back(IntConst<1>());
+    else gate_back(IntConst<2>());
     dt_sum += __shfl_xor(dt_sum, 32);
     if (lane < 32) part[ch * (1 + DK) + 1 + d] = dt_sum;
     da_sum = wave_sum(da_sum);

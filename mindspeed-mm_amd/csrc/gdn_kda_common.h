@@ -9,10 +9,24 @@ struct KdaFlags {
   float lower_bound;
 };
 
-__device__ __forceinline__ float kda_sigmoid(float x) { return 1.f / (1.f + __expf(-x)); }
-// log(1 + e^x) = max(x, 0) + log(1 + e^{-|x|}) with the hardware exponential and logarithm: absolute error of the
-// order of 1e-7 everywhere (the argument of the logarithm lies in (1, 2])
-__device__ __forceinline__ float kda_softplus(float x) { return fmaxf(x, 0.f) + __logf(1.f + __expf(-fabsf(x))); }
+// A compile-time integer as a function argument: lets one generic lambda be stamped out once per mode.
+template <int V> struct IntConst { static constexpr int value = V; };
+
+// The hardware reciprocal and base-2 logarithm, one instruction each (1 ulp), in place of the IEEE division and the
+// range-checked logarithm: a gate costs a few instructions per element, and the kernels evaluate one per token and
+// key channel.
+__device__ __forceinline__ float kda_sigmoid(float x) { return __builtin_amdgcn_rcpf(1.f + __expf(-x)); }
+// log(1 + e^x) = max(x, 0) + log(1 + e^{-|x|}): the argument of the logarithm lies in (1, 2], absolute error of the
+// order of 1e-7 everywhere
+__device__ __forceinline__ float kda_softplus(float x) {
+  return fmaxf(x, 0.f) + 0.69314718f * __builtin_amdgcn_logf(1.f + __expf(-fabsf(x)));
+}
+// softplus and its derivative, the sigmoid, from one exponential
+__device__ __forceinline__ void kda_softplus_sigmoid(float x, float& sp, float& sg) {
+  const float t = __expf(-fabsf(x)), r = __builtin_amdgcn_rcpf(1.f + t);
+  sp = fmaxf(x, 0.f) + 0.69314718f * __builtin_amdgcn_logf(1.f + t);
+  sg = x >= 0.f ? r : t * r;
+}
 
 // VEC consecutive fp32 values of an LDS row
 template <int VEC> __device__ __forceinline__ void ld_f32(const float* p, float* f) {

@@ -73,23 +73,30 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
   tile_qk_request<T, DK>(qt, q + tok0 * hk + h * DK, hk, nvalid, tid);
   constexpr int GP = 64 * (DK / 4) / kThreads;
   const bool g32 = sizeof(T) == 4 || fl.g_f32;
-  float gx[GP][4];
+  // as bits, and with one branch around each whole round of requests: a conversion or a test between two loads would
+  // make each of them wait for the one before
+  u32x4 gw[GP];
+  f32x4 bv[GP];
+  if (g32) {
 #pragma unroll
-  for (int i = 0; i < GP; ++i) {
-    const int c = tid + i * kThreads, row = imin(c / (DK / 4), nvalid - 1), c4 = c % (DK / 4);
-    const int64_t at = (tok0 + row) * hk + h * DK + 4 * c4;
-    if (g32) {
-      const f32x4 x = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(g) + at);
-      gx[i][0] = x[0]; gx[i][1] = x[1]; gx[i][2] = x[2]; gx[i][3] = x[3];
-    } else {
-      const u32x2 x = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(g) + at);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        T t;
-        if constexpr (sizeof(T) == 2) t.bits = (uint16_t)(x[e >> 1] >> (16 * (e & 1)));
-        gx[i][e] = Elem<T>::to_f(t);
-      }
+    for (int i = 0; i < GP; ++i) {
+      const int c = tid + i * kThreads, row = imin(c / (DK / 4), nvalid - 1), c4 = c % (DK / 4);
+      gw[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint32_t*>(g) + (tok0 + row) * hk + h * DK + 4 * c4);
     }
+  } else {
+#pragma unroll
+    for (int i = 0; i < GP; ++i) {
+      const int c = tid + i * kThreads, row = imin(c / (DK / 4), nvalid - 1), c4 = c % (DK / 4);
+      const u32x2 x = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(g) + (tok0 + row) * hk + h * DK + 4 * c4);
+      gw[i][0] = x[0]; gw[i][1] = x[1]; gw[i][2] = 0; gw[i][3] = 0;
+    }
+  }
+  if (fl.use_gate && dt_bias != nullptr) {
+#pragma unroll
+    for (int i = 0; i < GP; ++i) bv[i] = *reinterpret_cast<const f32x4*>(dt_bias + h * DK + 4 * ((tid + i * kThreads) % (DK / 4)));
+  } else {
+#pragma unroll
+    for (int i = 0; i < GP; ++i) { bv[i][0] = 0.f; bv[i][1] = 0.f; bv[i][2] = 0.f; bv[i][3] = 0.f; }
   }
   if (wave == 0) {
     const int64_t at = (tok0 + imin(lane, nvalid - 1)) * H + h;
@@ -103,21 +110,27 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
   // the gate: log decay of every token and channel, 0 on the rows past the end (they leave the cumulative sum alone)
   {
     const float a = fl.use_gate ? __expf(A_log[h]) : 0.f;
+    // MODE 0: g is the log decay itself; 1: -e^{A_log} softplus(g + bias); 2: lower_bound sigmoid(e^{A_log} (g + bias)).
+    // One copy of the loop per mode: a test of the options per element would cost as much as the gate.
+    auto gate_rows = [&](auto mode) {
+      constexpr int MODE = decltype(mode)::value;
 #pragma unroll
-    for (int i = 0; i < GP; ++i) {
-      const int c = tid + i * kThreads, row = c / (DK / 4), c4 = c % (DK / 4);
-      f32x4 y;
+      for (int i = 0; i < GP; ++i) {
+        const int c = tid + i * kThreads, row = c / (DK / 4), c4 = c % (DK / 4);
+        f32x4 y;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        float x = gx[i][e];
-        if (fl.use_gate) {
-          if (dt_bias != nullptr) x += dt_bias[h * DK + 4 * c4 + e];
-          x = fl.has_lower_bound ? fl.lower_bound * kda_sigmoid(a * x) : -a * kda_softplus(x);
+        for (int e = 0; e < 4; ++e) {
+          float x = __uint_as_float(g32 ? gw[i][e] : (gw[i][e >> 1] >> (16 * (e & 1))) << 16);
+          if (MODE == 1) x = -a * kda_softplus(x + bv[i][e]);
+          if (MODE == 2) x = fl.lower_bound * kda_sigmoid(a * (x + bv[i][e]));
+          y[e] = row < nvalid ? x : 0.f;
         }
-        y[e] = row < nvalid ? x : 0.f;
+        *reinterpret_cast<f32x4*>(Gs + row * LDG + 4 * c4) = y;
       }
-      *reinterpret_cast<f32x4*>(Gs + row * LDG + 4 * c4) = y;
-    }
+    };
+    if (!fl.use_gate) gate_rows(IntConst<0>());
+    else if (!fl.has_lower_bound) gate_rows(IntConst<1>());
+    else gate_rows(IntConst<2>());
   }
   {
     const int64_t roff = ch * 64;

@@ -266,9 +266,11 @@ static emu::GdimProxy gridDim;
 #define __builtin_amdgcn_fence(...) ((void)0)
 #define __builtin_amdgcn_sched_barrier(x) ((void)0)
 #define __builtin_amdgcn_rcpf(x) (1.0f / (x))
+#define __builtin_amdgcn_logf(x) log2f(x)
 #define GDN_WAVES_PER_SIMD(n)
 #define __builtin_amdgcn_sched_group_barrier(m, n, s) ((void)0)
 #define __builtin_amdgcn_wave_barrier() emu::wave_sync()
+#define __builtin_amdgcn_s_sleep(x) emu::yield()
 #define __builtin_amdgcn_readfirstlane(x) (x)
 #define __builtin_amdgcn_s_waitcnt(x) ((void)0)
 #define __builtin_amdgcn_ds_read_tr16_b64_v4i16(p) emu::ds_read_tr16((const void*)(uintptr_t)(p))
