@@ -36,22 +36,40 @@ template <typename T, int DK> struct KdaBwdSmem {
   static constexpr bool FULL = sizeof(T) == 4;   // no rescaled images: every pair term by term
   static constexpr int tile = 64 * LDK * (int)sizeof(T), gmat = 64 * LDG * 4, mat = 64 * L64 * (int)sizeof(T);
   static constexpr int off_ks = 0;                   // k^ rows
-  static constexpr int off_qs = off_ks + tile;       // first P as T, then q^ rows
+  static constexpr int off_qs = off_ks + tile;       // P as T; FULL: then q^ rows
   static constexpr int off_gs = off_qs + tile;       // first Kp as T (64 rows), then G rows (fp32)
   static constexpr int off_m1 = off_gs + gmat;       // dTm, then dL; later, with the next one, the store patches
   static constexpr int off_m2 = off_m1 + mat;        // X = Tm^T dTm, then scale dAq
-  static constexpr int off_tm = off_m2 + mat;        // Tm row-major, then dL transposed
+  static constexpr int off_tm = off_m2 + mat;        // Tm row-major
   static constexpr int off_m2t = off_tm + mat;       // scale dAq transposed (not FULL)
-  static constexpr int off_row = off_m2t + (FULL ? 0 : mat);
-  // beta, 1/|q|, 1/|k| [64 each]; per-wave row sums <q^,dq^>, <k^,dk^>, db, <R,v> [256 each]; 8 scalars
-  static constexpr int bytes = off_row + (3 * 64 + 4 * 256 + 8) * 4;
+  // not FULL: q^ rows and dL transposed get places of their own, so that P and Tm live until dK1 = Tm^T P is formed
+  // where it is used, after the decay-weighted sums, instead of occupying registers through them
+  static constexpr int off_q2 = off_m2t + (FULL ? 0 : mat);
+  static constexpr int off_m1t = off_q2 + (FULL ? 0 : tile);
+  static constexpr int off_row = off_m1t + (FULL ? 0 : mat);
+  // beta, 1/|q|, 1/|k| [64 each]; row sums <q^,dq^>, <k^,dk^>, db, <R,v> [256 each]; per-wave scalars [8]; what the
+  // two waves of a channel block exchange: parts of dG_last and d(dt_bias) [8][32 each], sum of dG over tokens 32.. [4][32]
+  static constexpr int bytes = off_row + (3 * 64 + 4 * 256 + 8 + 2 * 256 + 128) * 4;
   static_assert(tile <= gmat, "Kp fits where G will be");
-  static_assert(4 * Patch<T>::kElems * (int)sizeof(T) <= 2 * mat, "store patches fit");
+  static_assert(8 * Patch<T>::kElems * (int)sizeof(T) <= 3 * mat, "store patches fit");
   static_assert(bytes <= 160 * 1024, "one CU's LDS");
 };
 
+// Eight waves, two per SIMD: the kernel is a chain of short dependent steps (LDS reads, exponentials, small matrix
+// products), and a second wave on the SIMD fills the waits of the first.  Waves 0..3 each own a 32x32 tile of the 64x64
+// matrices of phases A1..A4; in phase B wave w owns key channels 32 (w >> 1).. and tokens 32 (w & 1).. of the chunk.
+constexpr int kFinThreads = 512;
+
+// rowacc[i0 + i] += sum_j x[i][j] for the 32 rows of an accumulator tile (see rows_add; the caller picks the slot)
+__device__ __forceinline__ void rows_add_at(const f32x16& x, float* rowacc, int i0) {
+  float s = rows16_partial(x);
+  s += __shfl_xor(s, 16);
+  const int lane = threadIdx.x & 63;
+  if ((lane & 16) == 0) rowacc[i0 + acc_row(lane & 15)] += s;
+}
+
 template <typename T, int DK>
-__global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
+__global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const void* __restrict__ g, const float* __restrict__ A_log,
     const float* __restrict__ dt_bias, const float* __restrict__ bhat, const float* __restrict__ GC,
     const T* __restrict__ TMR, const float* __restrict__ dumps, const int64_t* __restrict__ cu,
@@ -61,23 +79,26 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
   constexpr int LDK = SM::LDK, LDG = SM::LDG, L64 = SM::L64, VEC = Elem<T>::kVec, CPR = DK / VEC, NKT = DK / 32;
   constexpr bool FULL = SM::FULL;
   T* Ks = reinterpret_cast<T*>(gdn_smem + SM::off_ks);
-  T* Qs = reinterpret_cast<T*>(gdn_smem + SM::off_qs);
-  T* Pt = Qs;
+  T* Pt = reinterpret_cast<T*>(gdn_smem + SM::off_qs);
+  T* Qs = FULL ? Pt : reinterpret_cast<T*>(gdn_smem + SM::off_q2);
   float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_gs);
   T* Kp = reinterpret_cast<T*>(gdn_smem + SM::off_gs);
   T* TmT = reinterpret_cast<T*>(gdn_smem + SM::off_tm);
   T* M1 = reinterpret_cast<T*>(gdn_smem + SM::off_m1);
   T* M2 = reinterpret_cast<T*>(gdn_smem + SM::off_m2);
-  T* M1t = TmT;
+  T* M1t = reinterpret_cast<T*>(gdn_smem + SM::off_m1t);
   T* M2t = reinterpret_cast<T*>(gdn_smem + SM::off_m2t);
   float* bs = reinterpret_cast<float*>(gdn_smem + SM::off_row);
   float* rsq = bs + 64;
   float* rsk = rsq + 64;
-  float* rq = rsk + 64;     // per-wave row sums (rows_add / rows_ld4)
+  float* rq = rsk + 64;     // row sums, a slot of 64 rows per block of 32 key channels (rows_add_at / rows_ld4)
   float* rk = rq + 256;
   float* rb = rk + 256;
-  float* rv = rb + 256;
-  float* wsum = rv + 256;
+  float* rv = rb + 256;     // <R_t, v_t>, a slot per tile wave
+  float* wsum = rv + 256;   // [8]   per wave: its part of dA_log
+  float* xgl = wsum + 8;    // [8][32] per wave and channel: its part of dG_last
+  float* xdt = xgl + 256;   // [8][32] per wave and channel: its part of d(dt_bias)
+  float* xblk = xdt + 256;  // [4][32] per channel: sum of dG over tokens 32..63
 
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
@@ -85,16 +106,18 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
   const int h = blockIdx.y, nvalid = s.nvalid;
   const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk, hk = (int64_t)H * DK;
   const int64_t ch = (int64_t)blockIdx.x * H + h;
-  const int ti = wave >> 1, tj = wave & 1, cj = wave;
-  const bool lower = tj <= ti, has_k = wave < NKT;
+  const int ti = (wave >> 1) & 1, tj = wave & 1;
+  const bool tile_wave = wave < 4, lower = tile_wave && tj <= ti;
+  const int cj = wave >> 1, ri = wave & 1;
+  const bool has_k = cj < NKT;
   const float* dump = dumps + ch * (3 * 64 * DK + 2 * 64 * 64 + DK);
   const float* dQb = dump, *dK2 = dump + 64 * DK, *Pm = dump + 2 * 64 * DK;
   const float* dAq = dump + 3 * 64 * DK, *a2m = dAq + 64 * 64, *dD = a2m + 64 * 64;
   const float* Gc = GC + ch * 64 * DK;
 
-  // ---- phase A0: k^ rows; P and Tm as operands; beta.  This wave's tiles of a2 and dAq are requested now ----
-  TileQK<T, DK> kt;
-  tile_qk_request<T, DK>(kt, k + tok0 * hk + h * DK, hk, nvalid, tid);
+  // ---- phase A0: k^ rows; P and Tm as operands; beta.  The tile waves request their tiles of a2 and dAq now ----
+  TileQK<T, DK> kt, qt;     // moved by the first kThreads threads
+  if (tile_wave) tile_qk_request<T, DK>(kt, k + tok0 * hk + h * DK, hk, nvalid, tid);
   f32x16 a2t, dat;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
@@ -107,15 +130,15 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
     rsq[tid] = 1.f;
     rsk[tid] = 1.f;
   }
-  rq[tid] = 0.f; rk[tid] = 0.f; rb[tid] = 0.f; rv[tid] = 0.f;
+  if (tid < 256) { rq[tid] = 0.f; rk[tid] = 0.f; rb[tid] = 0.f; rv[tid] = 0.f; }
   // this thread's pieces of P and G (VEC consecutive channels of a row each), all requested before the first wait
-  constexpr int NIT = 64 * CPR / kThreads, C64 = 64 / VEC, NTM = 64 * C64 / kThreads;
-  static_assert(64 * CPR % kThreads == 0 && 64 * C64 % kThreads == 0 && VEC % 4 == 0, "whole rounds of 16-byte pieces");
+  constexpr int NIT = 64 * CPR / kFinThreads, C64 = 64 / VEC, NTM = 64 * C64 / kFinThreads;
+  static_assert(64 * CPR % kFinThreads == 0 && 64 * C64 % kFinThreads == 0 && VEC % 4 == 0, "whole rounds of 16-byte pieces");
   f32x4 pf[NIT][VEC / 4], gk[NIT][VEC / 4];
   Vec16<T> tmv[NTM];
 #pragma unroll
   for (int it = 0; it < NIT; ++it) {
-    const int c = tid + it * kThreads, at = (c / CPR) * DK + (c % CPR) * VEC;
+    const int c = tid + it * kFinThreads, at = (c / CPR) * DK + (c % CPR) * VEC;
 #pragma unroll
     for (int e = 0; e < VEC / 4; ++e) {
       pf[it][e] = *reinterpret_cast<const f32x4*>(Pm + at + 4 * e);
@@ -124,14 +147,13 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
   }
 #pragma unroll
   for (int it = 0; it < NTM; ++it) {
-    const int c = tid + it * kThreads;
+    const int c = tid + it * kFinThreads;
     tmv[it] = ld16(TMR + ch * 4096 + (c / C64) * 64 + (c % C64) * VEC);
   }
-  TileQK<T, DK> qt;
-  tile_qk_request<T, DK>(qt, q + tok0 * hk + h * DK, hk, nvalid, tid);
+  if (tile_wave) tile_qk_request<T, DK>(qt, q + tok0 * hk + h * DK, hk, nvalid, tid);
 #pragma unroll
   for (int it = 0; it < NIT; ++it) {
-    const int c = tid + it * kThreads;
+    const int c = tid + it * kFinThreads;
     float f[VEC];
 #pragma unroll
     for (int e = 0; e < VEC; ++e) f[e] = pf[it][e / 4][e % 4];
@@ -139,15 +161,15 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
   }
 #pragma unroll
   for (int it = 0; it < NTM; ++it) {
-    const int c = tid + it * kThreads;
+    const int c = tid + it * kFinThreads;
     st16(TmT + (c / C64) * L64 + (c % C64) * VEC, tmv[it]);
   }
   GDN_LDS_BARRIER();   // the row vectors are initialised before the norm below writes 1/|k| over its entries
-  tile_qk_finish<T, DK>(kt, Ks, LDK, nvalid, tid, fl.l2norm != 0, nullptr, 0, rsk, 1);
+  if (tile_wave) tile_qk_finish<T, DK>(kt, Ks, LDK, nvalid, tid, fl.l2norm != 0, nullptr, 0, rsk, 1);
   GDN_LDS_BARRIER();
 #pragma unroll
   for (int it = 0; it < NIT; ++it) {   // Kp = k^ . e^{G}
-    const int c = tid + it * kThreads, row = c / CPR, cc = c % CPR;
+    const int c = tid + it * kFinThreads, row = c / CPR, cc = c % CPR;
     float f[VEC];
     unpack16<T>(ld16(Ks + row * LDK + cc * VEC), f);
 #pragma unroll
@@ -156,8 +178,8 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
   }
   GDN_LDS_BARRIER();
 
-  // ---- phase A1: dTm = stril(b_j (a2 - P Kp^T)), one 32x32 tile per wave; <R_t, v_t> from Tm and a2 ----
-  {
+  // ---- phase A1: dTm = stril(b_j (a2 - P Kp^T)), one 32x32 tile per tile wave; <R_t, v_t> from Tm and a2 ----
+  if (tile_wave) {
     f32x16 x = acc_zero();
     if (lower) mma32<T, DK, true, true>(x, Pt + 32 * ti * LDK, LDK, Kp + 32 * tj * LDK, LDK);
     const int j = 32 * tj + l32;
@@ -175,67 +197,58 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
   }
   GDN_LDS_BARRIER();
   // ---- phase A2: X = Tm^T dTm (the tiles dL needs: a >= the column block) ----
-  {
+  if (tile_wave) {
     f32x16 x = acc_zero();
     if (lower) mma32<T, 64, false, false>(x, TmT + 32 * ti, L64, M1 + 32 * tj, L64);
 #pragma unroll
     for (int r = 0; r < 16; ++r) M2[(32 * ti + acc_row(r)) * L64 + 32 * tj + l32] = Elem<T>::from_f(x[r]);
   }
   GDN_LDS_BARRIER();
-  // ---- phase A3: dL = -stril(X Tm^T); dK1 = Tm^T P for this wave's 32 key channels; scale dAq ----
-  f32x16 dK1[2];
-  dK1[0] = acc_zero();
-  dK1[1] = acc_zero();
-  f32x16 dl = acc_zero(), sa;
+  // ---- phase A3: dL = -stril(X Tm^T); dK1 = Tm^T P for this wave's tokens and key channels; scale dAq ----
+  f32x16 dK1 = acc_zero(), dl = acc_zero(), sa;
   if (lower) mma32<T, 64, true, true>(dl, M2 + 32 * ti * L64, L64, TmT + 32 * tj * L64, L64);
-  if (has_k) {
-#pragma unroll
-    for (int ri = 0; ri < 2; ++ri) mma32<T, 64, false, false>(dK1[ri], TmT + 32 * ri, L64, Pt + 32 * cj, LDK);
-  }
+  if (FULL && has_k) mma32<T, 64, false, false>(dK1, TmT + 32 * ri, L64, Pt + 32 * cj, LDK);
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int i = 32 * ti + acc_row(r), j = 32 * tj + l32;
     dl[r] = i > j ? -dl[r] : 0.f;
     sa[r] = i >= j ? scale * dat[r] : 0.f;
   }
-  GDN_LDS_BARRIER();   // dTm, X, P, Kp are consumed
-  // ---- phase A4: the coefficient matrices in place of dTm and X; q^ rows and G in place of P and Kp ----
+  GDN_LDS_BARRIER();   // dTm, X, Kp are consumed (FULL: P too)
+  // ---- phase A4: the coefficient matrices in place of dTm and X; G in place of Kp; q^ rows (FULL: in place of P) ----
+  if (tile_wave) {
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int at = (32 * ti + acc_row(r)) * L64 + 32 * tj + l32;
-    M1[at] = Elem<T>::from_f(dl[r]);
-    M2[at] = Elem<T>::from_f(sa[r]);
-    if constexpr (!FULL) {
-      const int att = (32 * tj + l32) * L64 + 32 * ti + acc_row(r);
-      M1t[att] = Elem<T>::from_f(dl[r]);
-      M2t[att] = Elem<T>::from_f(sa[r]);
+    for (int r = 0; r < 16; ++r) {
+      const int at = (32 * ti + acc_row(r)) * L64 + 32 * tj + l32;
+      M1[at] = Elem<T>::from_f(dl[r]);
+      M2[at] = Elem<T>::from_f(sa[r]);
+      if constexpr (!FULL) {
+        const int att = (32 * tj + l32) * L64 + 32 * ti + acc_row(r);
+        M1t[att] = Elem<T>::from_f(dl[r]);
+        M2t[att] = Elem<T>::from_f(sa[r]);
+      }
     }
+    tile_qk_finish<T, DK>(qt, Qs, LDK, nvalid, tid, fl.l2norm != 0, nullptr, 0, rsq, 1);
   }
-  tile_qk_finish<T, DK>(qt, Qs, LDK, nvalid, tid, fl.l2norm != 0, nullptr, 0, rsq, 1);
 #pragma unroll
   for (int it = 0; it < NIT; ++it) {
-    const int c = tid + it * kThreads;
+    const int c = tid + it * kFinThreads;
 #pragma unroll
     for (int e = 0; e < VEC / 4; ++e)
       *reinterpret_cast<f32x4*>(Gs + (c / CPR) * LDG + (c % CPR) * VEC + 4 * e) = gk[it][e];
   }
   GDN_LDS_BARRIER();
 
-  // ---- phase B: the decay-weighted sums.  A wave owns 32 key channels, a lane one of them and, per 32-token block,
-  //      the 16 rows of its accumulator registers ----
+  // ---- phase B: the decay-weighted sums.  A lane has one key channel and the 16 rows of its accumulator registers
+  //      in the wave's 32-token block ----
   const int d = 32 * cj + l32;
-  float Gi[2][16], ki[2][16], qi[2][16], U[2][16], Uq[2][16], W[2][16];
+  float Gi[16], U[16], Uq[16], W[16];
   if (has_k) {
 #pragma unroll
-    for (int ri = 0; ri < 2; ++ri)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int i = 32 * ri + acc_row(r);
-        Gi[ri][r] = Gs[i * LDG + d];
-        ki[ri][r] = Elem<T>::to_f(Ks[i * LDK + d]);
-        qi[ri][r] = Elem<T>::to_f(Qs[i * LDK + d]);
-        U[ri][r] = 0.f; Uq[ri][r] = 0.f; W[ri][r] = 0.f;
-      }
+    for (int r = 0; r < 16; ++r) {
+      Gi[r] = Gs[(32 * ri + acc_row(r)) * LDG + d];
+      U[r] = 0.f; Uq[r] = 0.f; W[r] = 0.f;
+    }
   }
   if constexpr (!FULL) {
     if (has_k) {
@@ -256,39 +269,31 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
         }
         return w;
       };
-#pragma unroll
-      for (int ri = 0; ri < 2; ++ri) {
-        // the partner rows this lane supplies as B operand, channel d: tokens 32 ri + 16 kg + 8 half + e
-        float kj[2][8], bk[2][8], qj[2][8], gj[2][8];
-#pragma unroll
-        for (int kg = 0; kg < 2; ++kg)
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const int x = 32 * ri + 16 * kg + 8 * half + e;
-            gj[kg][e] = Gs[x * LDG + d];
-            kj[kg][e] = Elem<T>::to_f(Ks[x * LDK + d]);
-            bk[kg][e] = bs[x] * kj[kg][e];
-            qj[kg][e] = Elem<T>::to_f(Qs[x * LDK + d]);
-          }
+      {
+        // The partner rows this lane supplies as B operand, channel d, are tokens 32 ri + 16 kg + 8 half + e.  They
+        // are read again at every level: held in registers through the levels they would push other values out to
+        // scratch memory, which costs more than the reads.
 #pragma unroll
         for (int r = 0; r < 16; ++r) {   // the pair i = j: no decay (dL has no diagonal)
           const int i = 32 * ri + acc_row(r);
           const float c = Elem<T>::to_f(M2[i * L64 + i]);
-          Uq[ri][r] += c * ki[ri][r];
-          W[ri][r] += c * qi[ri][r];
+          Uq[r] += c * Elem<T>::to_f(Ks[i * LDK + d]);
+          W[r] += c * Elem<T>::to_f(Qs[i * LDK + d]);
         }
 #pragma unroll 1
         for (int lg = 1; lg <= 5; ++lg) {   // blocks of n = 2^lg tokens inside the 32-token block
           const int n = 1 << lg;
+          asm volatile("" ::: "memory");   // the reads of a level stay inside it
           f32x16 cu = acc_zero(), cq = acc_zero(), cw = acc_zero();
 #pragma unroll
           for (int kg = 0; kg < 2; ++kg) {
-            float xk[8], xb[8], xq[8];
+            float xk[8], xb[8], xq[8], bx[8];
+            ld_f32<8>(bs + 32 * ri + 16 * kg + 8 * half, bx);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
               const int x = 32 * ri + 16 * kg + 8 * half + e, m = ((x >> lg) << lg) + (n >> 1);
-              const float f = __expf(-fabsf(gj[kg][e] - Gs[m * LDG + d]));
-              xk[e] = kj[kg][e] * f; xb[e] = bk[kg][e] * f; xq[e] = qj[kg][e] * f;
+              const float f = __expf(-fabsf(Gs[x * LDG + d] - Gs[m * LDG + d]));
+              xk[e] = Elem<T>::to_f(Ks[x * LDK + d]) * f; xb[e] = bx[e] * xk[e]; xq[e] = Elem<T>::to_f(Qs[x * LDK + d]) * f;
             }
             const u32x4 bK = pack16<T>(xk).raw, bB = pack16<T>(xb).raw, bQ = pack16<T>(xq).raw;
             const int row = 32 * ri + l32, col0 = 32 * ri + 16 * kg + 8 * half, b0 = 16 * kg + 8 * half;
@@ -300,102 +305,147 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
 #pragma unroll
           for (int r = 0; r < 16; ++r) {   // every row by its own factor
             const int i = 32 * ri + acc_row(r), m = ((i >> lg) << lg) + (n >> 1);
-            const float f = __expf(-fabsf(Gi[ri][r] - Gs[m * LDG + d]));
-            U[ri][r] += f * cu[r];
-            Uq[ri][r] += f * cq[r];
-            W[ri][r] += f * cw[r];
+            const float f = __expf(-fabsf(Gi[r] - Gs[m * LDG + d]));
+            U[r] += f * cu[r];
+            Uq[r] += f * cq[r];
+            W[r] += f * cw[r];
           }
         }
       }
-      {   // the level of the whole chunk: tokens 32..63 against tokens 0..31, m = 32, every pair kept
+      {   // the level of the whole chunk: tokens 32..63 against tokens 0..31, m = 32, every pair kept.  The wave of the
+          // later tokens takes the sums over j (U, Uq), the wave of the earlier ones the sum over i (W)
         const float g32v = Gs[32 * LDG + d];
-        f32x16 cu = acc_zero(), cq = acc_zero(), cw = acc_zero();
+        f32x16 c1 = acc_zero(), c2 = acc_zero();
 #pragma unroll
         for (int kg = 0; kg < 2; ++kg) {
-          float xk[8], xb[8], xq[8];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const int j = 16 * kg + 8 * half + e, i = 32 + j;
-            xk[e] = Elem<T>::to_f(Ks[j * LDK + d]) * __expf(-fabsf(Gs[j * LDG + d] - g32v));
-            const float f = __expf(-fabsf(Gs[i * LDG + d] - g32v));
-            xb[e] = bs[i] * Elem<T>::to_f(Ks[i * LDK + d]) * f;
-            xq[e] = Elem<T>::to_f(Qs[i * LDK + d]) * f;
-          }
           const int c0 = 16 * kg + 8 * half;
-          mfma_kgroup<T>(cu, ld16(M1 + (32 + l32) * L64 + c0).raw, pack16<T>(xk).raw);
-          mfma_kgroup<T>(cq, ld16(M2 + (32 + l32) * L64 + c0).raw, pack16<T>(xk).raw);
-          mfma_kgroup<T>(cw, ld16(M1t + l32 * L64 + 32 + c0).raw, pack16<T>(xb).raw);
-          mfma_kgroup<T>(cw, ld16(M2t + l32 * L64 + 32 + c0).raw, pack16<T>(xq).raw);
+          if (ri == 1) {
+            float xk[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const int j = c0 + e;
+              xk[e] = Elem<T>::to_f(Ks[j * LDK + d]) * __expf(-fabsf(Gs[j * LDG + d] - g32v));
+            }
+            const u32x4 bK = pack16<T>(xk).raw;
+            mfma_kgroup<T>(c1, ld16(M1 + (32 + l32) * L64 + c0).raw, bK);
+            mfma_kgroup<T>(c2, ld16(M2 + (32 + l32) * L64 + c0).raw, bK);
+          } else {
+            float xb[8], xq[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const int i = 32 + c0 + e;
+              const float f = __expf(-fabsf(Gs[i * LDG + d] - g32v));
+              xb[e] = bs[i] * Elem<T>::to_f(Ks[i * LDK + d]) * f;
+              xq[e] = Elem<T>::to_f(Qs[i * LDK + d]) * f;
+            }
+            mfma_kgroup<T>(c1, ld16(M1t + l32 * L64 + 32 + c0).raw, pack16<T>(xb).raw);
+            mfma_kgroup<T>(c1, ld16(M2t + l32 * L64 + 32 + c0).raw, pack16<T>(xq).raw);
+          }
         }
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const float f1 = __expf(-fabsf(Gi[1][r] - g32v)), f0 = __expf(-fabsf(Gi[0][r] - g32v));
-          U[1][r] += f1 * cu[r];
-          Uq[1][r] += f1 * cq[r];
-          W[0][r] += f0 * cw[r];
+          const float f = __expf(-fabsf(Gi[r] - g32v));
+          if (ri == 1) { U[r] += f * c1[r]; Uq[r] += f * c2[r]; }
+          else W[r] += f * c1[r];
         }
       }
     }
   }
   if (FULL && has_k) {
+    // rows i of this lane against the earlier rows j of the chunk
+    for (int jj = 0; jj <= 32 * ri + 31; ++jj) {
+      const float gj = Gs[jj * LDG + d], kj = Elem<T>::to_f(Ks[jj * LDK + d]);
 #pragma unroll
-    for (int ri = 0; ri < 2; ++ri) {
-      // rows i of this lane against the earlier rows j of the chunk
-      for (int jj = 0; jj <= 32 * ri + 31; ++jj) {
-        const float gj = Gs[jj * LDG + d], kj = Elem<T>::to_f(Ks[jj * LDK + d]);
+      for (int qd = 0; qd < 4; ++qd) {
+        if (32 * ri + 8 * qd + 7 < jj) continue;   // none of the group's rows reaches jj (same for every lane)
 #pragma unroll
-        for (int qd = 0; qd < 4; ++qd) {
-          if (32 * ri + 8 * qd + 7 < jj) continue;   // none of the group's rows reaches jj (same for every lane)
-#pragma unroll
-          for (int m = 0; m < 4; ++m) {
-            const int r = 4 * qd + m, i = 32 * ri + acc_row(r);
-            const float t = kj * __expf(i >= jj ? Gi[ri][r] - gj : 0.f);
-            U[ri][r] += Elem<T>::to_f(M1[i * L64 + jj]) * t;    // coefficients are zero where i < jj
-            Uq[ri][r] += Elem<T>::to_f(M2[i * L64 + jj]) * t;
-          }
+        for (int m = 0; m < 4; ++m) {
+          const int r = 4 * qd + m, i = 32 * ri + acc_row(r);
+          const float t = kj * __expf(i >= jj ? Gi[r] - gj : 0.f);
+          U[r] += Elem<T>::to_f(M1[i * L64 + jj]) * t;    // coefficients are zero where i < jj
+          Uq[r] += Elem<T>::to_f(M2[i * L64 + jj]) * t;
         }
       }
-      // rows j of this lane against the later rows i
-      for (int ii = 32 * ri; ii <= 63; ++ii) {
-        const float gi = Gs[ii * LDG + d], kb = bs[ii] * Elem<T>::to_f(Ks[ii * LDK + d]), qv = Elem<T>::to_f(Qs[ii * LDK + d]);
+    }
+    // rows j of this lane against the later rows i
+    for (int ii = 32 * ri; ii <= 63; ++ii) {
+      const float gi = Gs[ii * LDG + d], kb = bs[ii] * Elem<T>::to_f(Ks[ii * LDK + d]), qv = Elem<T>::to_f(Qs[ii * LDK + d]);
 #pragma unroll
-        for (int qd = 0; qd < 4; ++qd) {
-          if (32 * ri + 8 * qd > ii) continue;
+      for (int qd = 0; qd < 4; ++qd) {
+        if (32 * ri + 8 * qd > ii) continue;
 #pragma unroll
-          for (int m = 0; m < 4; ++m) {
-            const int r = 4 * qd + m, j = 32 * ri + acc_row(r);
-            const float e = __expf(ii >= j ? gi - Gi[ri][r] : 0.f);
-            W[ri][r] += (Elem<T>::to_f(M1[ii * L64 + j]) * kb + Elem<T>::to_f(M2[ii * L64 + j]) * qv) * e;
-          }
+        for (int m = 0; m < 4; ++m) {
+          const int r = 4 * qd + m, j = 32 * ri + acc_row(r);
+          const float e = __expf(ii >= j ? gi - Gi[r] : 0.f);
+          W[r] += (Elem<T>::to_f(M1[ii * L64 + j]) * kb + Elem<T>::to_f(M2[ii * L64 + j]) * qv) * e;
         }
       }
     }
   }
   // ---- phase B3: the gradients of q^, k^, G per token and channel; row sums for beta and the l2 norm ----
-  f32x16 dqh[2], dkh[2], dGv[2];
-  float gl_sum = 0.f;
+  // (the loads below stay below: moved above the sums, which leave no register free, their results would be spilled)
+  asm volatile("" ::: "memory");
+  f32x16 dqh, dkh, dGv;
+  float ki[16], qi[16];
+  // suffix sums down the tokens come later.  Rows of a block in token order: group qd = 0..3, half-wave 0 then 1,
+  // m = 0..3; so[qd] is this lane's sum of a group, sx[qd] that of the other half-wave
+  float so[4], sx[4];
   if (has_k) {
     const float glast = Gs[63 * LDG + d];
+    float gl_sum = 0.f, blk = 0.f;
+    // the sums over V of this lane's rows: all requested before the first is used, and used in two passes so that few
+    // intermediate rows are alive at a time (a schedule that runs out of registers waits after every load)
+    float lq[16], lk[16];
 #pragma unroll
-    for (int ri = 0; ri < 2; ++ri) {
-      f32x16 pq, pk, pb;
+    for (int r = 0; r < 16; ++r) {
+      const int i = 32 * ri + acc_row(r);
+      lq[r] = dQb[i * DK + d];
+      lk[r] = dK2[i * DK + d];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (!FULL) mma32<T, 64, false, false>(dK1, TmT + 32 * ri, L64, Pt + 32 * cj, LDK);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int i = 32 * ri + acc_row(r);
+      ki[r] = Elem<T>::to_f(Ks[i * LDK + d]);
+      qi[r] = Elem<T>::to_f(Qs[i * LDK + d]);
+    }
+    {
+      f32x16 pq;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int i = 32 * ri + acc_row(r);
-        const float eG = __expf(Gi[ri][r]), b = bs[i];
-        const float t1 = -b * eG * dK1[ri][r];
-        const float t2 = __expf(glast - Gi[ri][r]) * dK2[i * DK + d];
-        dqh[ri][r] = scale * eG * dQb[i * DK + d] + Uq[ri][r];
-        dkh[ri][r] = t1 + t2 + b * U[ri][r] + W[ri][r];
-        dGv[ri][r] = qi[ri][r] * dqh[ri][r] + ki[ri][r] * (t1 + b * U[ri][r] - t2 - W[ri][r]);
-        gl_sum += ki[ri][r] * t2;
-        pq[r] = qi[ri][r] * dqh[ri][r];
-        pk[r] = ki[ri][r] * dkh[ri][r];
-        pb[r] = ki[ri][r] * (U[ri][r] - eG * dK1[ri][r]);
+        dqh[r] = scale * __expf(Gi[r]) * lq[r] + Uq[r];
+        pq[r] = qi[r] * dqh[r];
+        dGv[r] = pq[r];
       }
-      rows_add(pq, rq, 32 * ri);
-      rows_add(pk, rk, 32 * ri);
-      rows_add(pb, rb, 32 * ri);
+      rows_add_at(pq, rq + 64 * cj, 32 * ri);
+    }
+    {
+      f32x16 pk, pb;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float eG = __expf(Gi[r]), b = bs[32 * ri + acc_row(r)];
+        const float t1 = -b * eG * dK1[r];
+        const float t2 = __expf(glast - Gi[r]) * lk[r];
+        dkh[r] = t1 + t2 + b * U[r] + W[r];
+        dGv[r] += ki[r] * (t1 + b * U[r] - t2 - W[r]);
+        gl_sum += ki[r] * t2;
+        pk[r] = ki[r] * dkh[r];
+        pb[r] = ki[r] * (U[r] - eG * dK1[r]);
+      }
+      rows_add_at(pk, rk + 64 * cj, 32 * ri);
+      rows_add_at(pb, rb + 64 * cj, 32 * ri);
+    }
+#pragma unroll
+    for (int qd = 0; qd < 4; ++qd) {
+      so[qd] = dGv[4 * qd] + dGv[4 * qd + 1] + dGv[4 * qd + 2] + dGv[4 * qd + 3];
+      sx[qd] = __shfl_xor(so[qd], 32);
+      blk += so[qd] + sx[qd];
+    }
+    gl_sum += __shfl_xor(gl_sum, 32);
+    if (lane < 32) {
+      xgl[wave * 32 + lane] = gl_sum;
+      if (ri == 1) xblk[cj * 32 + lane] = blk;
     }
   }
   GDN_LDS_BARRIER();   // row sums are complete; the matrices are dead: their place takes the store patches
@@ -409,53 +459,33 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
     // the raw gate input of this lane's rows, requested before the stores below
     const bool g32 = sizeof(T) == 4 || fl.g_f32;
     // (as bits, widened after the loop: a conversion inside it would make every load wait for the one before)
-    uint32_t raws[2][16];
+    uint32_t raws[16];
     if (fl.use_gate) {
       if (g32) {
 #pragma unroll
-        for (int ri = 0; ri < 2; ++ri)
-#pragma unroll
-          for (int r = 0; r < 16; ++r)
-            raws[ri][r] = reinterpret_cast<const uint32_t*>(g)[(tok0 + imin(32 * ri + acc_row(r), nvalid - 1)) * hk + h * DK + d];
+        for (int r = 0; r < 16; ++r)
+          raws[r] = reinterpret_cast<const uint32_t*>(g)[(tok0 + imin(32 * ri + acc_row(r), nvalid - 1)) * hk + h * DK + d];
       } else {
 #pragma unroll
-        for (int ri = 0; ri < 2; ++ri)
-#pragma unroll
-          for (int r = 0; r < 16; ++r)
-            raws[ri][r] = reinterpret_cast<const uint16_t*>(g)[(tok0 + imin(32 * ri + acc_row(r), nvalid - 1)) * hk + h * DK + d];
+        for (int r = 0; r < 16; ++r)
+          raws[r] = reinterpret_cast<const uint16_t*>(g)[(tok0 + imin(32 * ri + acc_row(r), nvalid - 1)) * hk + h * DK + d];
       }
     }
     const int raw_shift = g32 ? 0 : 16;
+    if (fl.l2norm) {
+      const f32x16 dotq = rows_ld4(rq, 32 * ri), dotk = rows_ld4(rk, 32 * ri);
+      const f32x16 sq = rows_ld(rsq, 32 * ri), sk = rows_ld(rsk, 32 * ri);
 #pragma unroll
-    for (int ri = 0; ri < 2; ++ri) {
-      if (fl.l2norm) {
-        const f32x16 dotq = rows_ld4(rq, 32 * ri), dotk = rows_ld4(rk, 32 * ri);
-        const f32x16 sq = rows_ld(rsq, 32 * ri), sk = rows_ld(rsk, 32 * ri);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          dqh[ri][r] = (dqh[ri][r] - dotq[r] * qi[ri][r]) * sq[r];
-          dkh[ri][r] = (dkh[ri][r] - dotk[r] * ki[ri][r]) * sk[r];
-        }
+      for (int r = 0; r < 16; ++r) {
+        dqh[r] = (dqh[r] - dotq[r] * qi[r]) * sq[r];
+        dkh[r] = (dkh[r] - dotk[r] * ki[r]) * sk[r];
       }
-      const int64_t at = (tok0 + 32 * ri) * hk + h * DK + 32 * cj;
-      acc_store_rows<T, false>(dqh[ri], id, patch, dq + at, hk, nvalid - 32 * ri);
-      acc_store_rows<T, false>(dkh[ri], id, patch, dk + at, hk, nvalid - 32 * ri);
     }
+    const int64_t at = (tok0 + 32 * ri) * hk + h * DK + 32 * cj;
+    acc_store_rows<T, false>(dqh, id, patch, dq + at, hk, nvalid - 32 * ri);
+    acc_store_rows<T, false>(dkh, id, patch, dk + at, hk, nvalid - 32 * ri);
     // dG_last: column sum over all rows of this channel, plus the decay of the state
-    gl_sum += __shfl_xor(gl_sum, 32);
-    const float dglast = gl_sum + dD[d] * __expf(Gs[63 * LDG + d]);
-    // suffix sums down the tokens.  Rows of a block in token order: group qd = 0..3, half-wave 0 then 1, m = 0..3
-    float so[2][4], sx[2][4], blk[2];
-#pragma unroll
-    for (int ri = 0; ri < 2; ++ri) {
-      blk[ri] = 0.f;
-#pragma unroll
-      for (int qd = 0; qd < 4; ++qd) {
-        so[ri][qd] = dGv[ri][4 * qd] + dGv[ri][4 * qd + 1] + dGv[ri][4 * qd + 2] + dGv[ri][4 * qd + 3];
-        sx[ri][qd] = __shfl_xor(so[ri][qd], 32);
-        blk[ri] += so[ri][qd] + sx[ri][qd];
-      }
-    }
+    const float dglast = xgl[2 * cj * 32 + l32] + xgl[(2 * cj + 1) * 32 + l32] + dD[d] * __expf(Gs[63 * LDG + d]);
     const bool first_half = lane < 32;
     const float a = fl.use_gate ? __expf(A_log[h]) : 0.f;
     const float bias = (fl.use_gate && dt_bias != nullptr) ? dt_bias[h * DK + d] : 0.f;
@@ -464,58 +494,61 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
     // One copy of the loop per mode: a test of the options per element would cost as much as the gate.
     auto gate_back = [&](auto mode) {
       constexpr int MODE = decltype(mode)::value;
+      f32x16 dgr;
+      float later = ri == 0 ? xblk[cj * 32 + l32] : 0.f;     // everything after the group being handled
 #pragma unroll
-      for (int ri = 0; ri < 2; ++ri) {
-        f32x16 dgr;
-        float later = ri == 0 ? blk[1] : 0.f;     // everything after the group being handled
+      for (int qd = 3; qd >= 0; --qd) {
+        float run = later + (first_half ? sx[qd] : 0.f);
 #pragma unroll
-        for (int qd = 3; qd >= 0; --qd) {
-          float run = later + (first_half ? sx[ri][qd] : 0.f);
-#pragma unroll
-          for (int m = 3; m >= 0; --m) {
-            const int r = 4 * qd + m, i = 32 * ri + acc_row(r);
-            run += dGv[ri][r];
-            float x = i < nvalid ? run + dglast : 0.f;     // d(log decay of token i, channel d)
-            if (MODE != 0) {
-              const float raw = __uint_as_float(raws[ri][r] << raw_shift) + bias;
-              if (MODE == 2) {
-                const float sg = kda_sigmoid(a * raw), ds_ = fl.lower_bound * sg * (1.f - sg);
-                da_sum += x * ds_ * a * raw;
-                x *= ds_ * a;
-              } else {
-                float sp, sg;
-                kda_softplus_sigmoid(raw, sp, sg);
-                da_sum -= x * a * sp;
-                x *= -a * sg;
-              }
+        for (int m = 3; m >= 0; --m) {
+          const int r = 4 * qd + m, i = 32 * ri + acc_row(r);
+          run += dGv[r];
+          float x = i < nvalid ? run + dglast : 0.f;     // d(log decay of token i, channel d)
+          if (MODE != 0) {
+            const float raw = __uint_as_float(raws[r] << raw_shift) + bias;
+            if (MODE == 2) {
+              const float sg = kda_sigmoid(a * raw), ds_ = fl.lower_bound * sg * (1.f - sg);
+              da_sum += x * ds_ * a * raw;
+              x *= ds_ * a;
+            } else {
+              float sp, sg;
+              kda_softplus_sigmoid(raw, sp, sg);
+              da_sum -= x * a * sp;
+              x *= -a * sg;
             }
-            dt_sum += x;
-            dgr[r] = x;
           }
-          later += so[ri][qd] + sx[ri][qd];
+          dt_sum += x;
+          dgr[r] = x;
         }
-        if (g32) {
+        later += so[qd] + sx[qd];
+      }
+      if (g32) {
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int i = 32 * ri + acc_row(r);
-            if (i < nvalid) reinterpret_cast<float*>(dg)[(tok0 + i) * hk + h * DK + d] = dgr[r];
-          }
-        } else {
-          acc_store_rows<T, false>(dgr, id, patch, reinterpret_cast<T*>(dg) + (tok0 + 32 * ri) * hk + h * DK + 32 * cj, hk,
-                                   nvalid - 32 * ri);
+        for (int r = 0; r < 16; ++r) {
+          const int i = 32 * ri + acc_row(r);
+          if (i < nvalid) reinterpret_cast<float*>(dg)[(tok0 + i) * hk + h * DK + d] = dgr[r];
         }
+      } else {
+        acc_store_rows<T, false>(dgr, id, patch, reinterpret_cast<T*>(dg) + (tok0 + 32 * ri) * hk + h * DK + 32 * cj, hk,
+                                 nvalid - 32 * ri);
       }
     };
     if (!fl.use_gate) gate_back(IntConst<0>());
     else if (!fl.has_lower_bound) gate_back(IntConst<1>());
     else gate_back(IntConst<2>());
     dt_sum += __shfl_xor(dt_sum, 32);
-    if (lane < 32) part[ch * (1 + DK) + 1 + d] = dt_sum;
+    if (lane < 32) xdt[wave * 32 + lane] = dt_sum;
     da_sum = wave_sum(da_sum);
   }
   if (lane == 0) wsum[wave] = has_k ? da_sum : 0.f;
   GDN_LDS_BARRIER();
-  if (tid == 0) part[ch * (1 + DK)] = wsum[0] + wsum[1] + wsum[2] + wsum[3];
+  if (tid == 0) {
+    float x = 0.f;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) x += wsum[w];
+    part[ch * (1 + DK)] = x;
+  }
+  if (tid < DK) part[ch * (1 + DK) + 1 + tid] = xdt[2 * (tid >> 5) * 32 + (tid & 31)] + xdt[(2 * (tid >> 5) + 1) * 32 + (tid & 31)];
   if (tid < 64 && tid < nvalid) {
     float x = 0.f;
 #pragma unroll
@@ -525,18 +558,27 @@ __global__ __launch_bounds__(kThreads) void kda_bwd_finish_kernel(
   }
 }
 
-// dA_log [H] and d(dt_bias) [H*K] from the per-chunk partial sums
+// dA_log [H] and d(dt_bias) [H*K] from the per-chunk partial sums.  A workgroup sums 32 of the 1 + K columns of one
+// head: 8 threads per column take every 8th chunk, and their sums are added in a fixed order.
 __global__ __launch_bounds__(kThreads) void kda_bwd_reduce_kernel(const float* __restrict__ part, const int64_t* cu,
                                                                  const int* __restrict__ chunk_offsets, int N, int nc,
                                                                  int H, int K, float* __restrict__ dA_log,
                                                                  float* __restrict__ ddt_bias) {
-  const int h = blockIdx.x, t = threadIdx.x;
+  __shared__ float seg_sum[8][32];
+  const int h = blockIdx.x, col = 32 * blockIdx.y + (threadIdx.x & 31), seg = threadIdx.x >> 5;
   const int n = cu != nullptr ? chunk_offsets[N] : nc;
-  if (t > K) return;
   float x = 0.f;
-  for (int c = 0; c < n; ++c) x += part[((int64_t)c * H + h) * (1 + K) + t];
-  if (t == 0) { if (dA_log != nullptr) dA_log[h] = x; }
-  else if (ddt_bias != nullptr) ddt_bias[h * K + t - 1] = x;
+  if (col <= K) {
+#pragma unroll 4
+    for (int c = seg; c < n; c += 8) x += part[((int64_t)c * H + h) * (1 + K) + col];
+  }
+  seg_sum[seg][threadIdx.x & 31] = x;
+  __syncthreads();
+  if (seg != 0 || col > K) return;
+#pragma unroll
+  for (int i = 1; i < 8; ++i) x += seg_sum[i][threadIdx.x];
+  if (col == 0) { if (dA_log != nullptr) dA_log[h] = x; }
+  else if (ddt_bias != nullptr) ddt_bias[h * K + col - 1] = x;
 }
 
 template <typename T, int DK, int NWS, int NLS, int STAGES>
@@ -583,11 +625,11 @@ static int kda_bwd_launch(const ChunkDims& d, const KdaWorkspace& L, const void*
     auto kern = kda_bwd_finish_kernel<T, DK>;
     constexpr int smem = KdaBwdSmem<T, DK>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
-    GDN_LAUNCH(kKernKdaBwdFinish, st, kern, dim3(nc, H), dim3(kThreads), smem, st, (const T*)q, (const T*)k, g, A_log, dt_bias,
+    GDN_LAUNCH(kKernKdaBwdFinish, st, kern, dim3(nc, H), dim3(kFinThreads), smem, st, (const T*)q, (const T*)k, g, A_log, dt_bias,
                bhat, GC, TMR, (const float*)DUMP, cu, chunk_offsets, (T*)dq, (T*)dk, dg, dbeta, PART, d.T, d.N, H, scale, fl);
   }
   if (fl.use_gate && (dA_log != nullptr || ddt_bias != nullptr))
-    GDN_LAUNCH(kKernKdaBwdReduce, st, kda_bwd_reduce_kernel, dim3(H), dim3(kThreads), 0, st, (const float*)PART, cu,
+    GDN_LAUNCH(kKernKdaBwdReduce, st, kda_bwd_reduce_kernel, dim3(H, (d.K + 32) / 32), dim3(kThreads), 0, st, (const float*)PART, cu,
                chunk_offsets, d.N, nc, H, d.K, dA_log, ddt_bias);
   return (int)hipGetLastError();
 }
