@@ -91,10 +91,11 @@ struct KdaWorkspace {
   int64_t QBT;            // T [chunks,H,K/32,2]    (scale q . e^{G})^T as A operand: tile = (32 columns of K) x (32 tokens)
   int64_t DVF;            // T [chunks,H,V/32,2]    d(v_new)
   int64_t DHF;            // T [chunks,H,V/32,K/32] gradient of the state AFTER each chunk
-  int64_t DUMP;           // f32 [chunks,H][dQb | dK2 | P : 64,K each][dAq | a2 : 64,64 each][dD : K]  sums over V of the chunk-local pass
+  int64_t DUMP;           // T [chunks,H][dQb | dK2 | P : 64,K each][dAq | a2 : 64,64 each]  sums over V of the chunk-local pass
+  int64_t DD;             // f32 [chunks,H,K]       sum over V of dS' . S: the gradient of the chunk's decay per channel
   int64_t PART;           // f32 [chunks,H][1 + K]  partial sums of dA_log and d(dt_bias)
   int64_t total_bytes;
-  static int64_t dump_floats(int K) { return 3 * 64 * (int64_t)K + 2 * 64 * 64 + K; }
+  static int64_t dump_elems(int K) { return 3 * 64 * (int64_t)K + 2 * 64 * 64; }
 };
 
 inline KdaWorkspace kda_workspace_layout(const ChunkDims& d, int elem_bytes) {
@@ -119,7 +120,8 @@ inline KdaWorkspace kda_workspace_layout(const ChunkDims& d, int elem_bytes) {
   w.QBT = take(nc * 64 * H * d.K * elem_bytes);
   w.DVF = take(nc * 64 * H * d.V * elem_bytes);
   w.DHF = take(nc * H * d.V * d.K * elem_bytes);
-  w.DUMP = take(nc * H * KdaWorkspace::dump_floats(d.K) * 4);
+  w.DUMP = take(nc * H * KdaWorkspace::dump_elems(d.K) * elem_bytes);
+  w.DD = take(nc * H * d.K * 4);
   w.PART = take(nc * H * (1 + d.K) * 4);
   w.total_bytes = off;
   return w;

@@ -366,7 +366,8 @@ template <typename T, int DK> struct BwdLocalSmem {
 // KDA (one decay per key channel): the sums over V are the same, what follows them is not.  The kernel then stops after
 // its main loop (dv is written there) and leaves the sums in kda_dump, per chunk and head
 //   [dQb = dO S^T | dK2 = V' dS'^T | P = dV' S^T : 64 x DK each][dAq = dO V'^T | a2 = dV' V^T : 64 x 64 each, lower tiles]
-//   [dD = sum_v dS' . S : DK]    (fp32)
+// rounded to T like every other tensor that passes between two kernels (they are the largest of them: in fp32 they made
+// up half of what the backward pass moved), and dD = sum_v dS' . S [DK] in kda_dd, in fp32,
 // for kda_bwd_finish_kernel; G is not read and beta is the transformed beta in fp32.
 template <typename T, int DK, bool KDA = false>
 __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_local_kernel(
@@ -375,7 +376,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     const T* __restrict__ dO, const T* __restrict__ hf, const T* __restrict__ dhf, const float* __restrict__ rstd_q,
     const float* __restrict__ rstd_k, T* dq, T* dk, T* __restrict__ dv_out, void* __restrict__ dbeta,
     float* __restrict__ dg, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N,
-    int Hqk, int Hv, int V, float scale, int hh, TokenStrides ts, float* __restrict__ kda_dump) {
+    int Hqk, int Hv, int V, float scale, int hh, TokenStrides ts, T* __restrict__ kda_dump, float* __restrict__ kda_dd) {
   using SM = BwdLocalSmem<T, DK>;
   constexpr int NKT = DK / 32, VEC = Elem<T>::kVec, KG = AccK<T>::kGroups;
   static_assert(NKT <= 4, "one 32-column block of K per wave");
@@ -579,28 +580,26 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     }
   }
   if constexpr (KDA) {
-    constexpr int64_t kDumpFloats = 3 * 64 * DK + 2 * 64 * 64 + DK;
-    float* dump = kda_dump + ch * kDumpFloats;
+    constexpr int64_t kDumpElems = 3 * 64 * DK + 2 * 64 * 64;
+    T* dump = kda_dump + ch * kDumpElems;
+    GDN_WAIT_VMEM();
+    GDN_LDS_BARRIER();   // the last block's stage is consumed: its place takes the store patches
+    T* patch = stage0 + SM::sh + wave * Patch<T>::kElems;
     if (has_k) {
 #pragma unroll
-      for (int ri = 0; ri < 2; ++ri)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int at = (32 * ri + acc_row(r)) * DK + 32 * cj + l32;
-          dump[at] = dQi[ri][r];
-          dump[64 * DK + at] = dKi[ri][r];
-          dump[2 * 64 * DK + at] = dWa[ri][r];
-        }
+      for (int ri = 0; ri < 2; ++ri) {
+        T* at = dump + 32 * ri * DK + 32 * cj;
+        acc_store_rows<T, false>(dQi[ri], id, patch, at, DK, 32);
+        acc_store_rows<T, false>(dKi[ri], id, patch, at + 64 * DK, DK, 32);
+        acc_store_rows<T, false>(dWa[ri], id, patch, at + 2 * 64 * DK, DK, 32);
+      }
       sds += __shfl_xor(sds, 32);   // the other half of the V block's rows
-      if (lane < 32) dump[3 * 64 * DK + 2 * 64 * 64 + 32 * cj + lane] = sds;
+      if (lane < 32) kda_dd[ch * DK + 32 * cj + lane] = sds;
     }
     if (lower) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int at = (32 * ti + acc_row(r)) * 64 + 32 * tj + l32;
-        dump[3 * 64 * DK + at] = ds[r];
-        dump[3 * 64 * DK + 64 * 64 + at] = a2[r];
-      }
+      T* at = dump + 3 * 64 * DK + 32 * ti * 64 + 32 * tj;
+      acc_store_rows<T, false>(ds, id, patch, at, 64, 32);
+      acc_store_rows<T, false>(a2, id, patch, at + 64 * 64, 64, 32);
     }
     return;
   }
@@ -882,7 +881,7 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     for (int hh = 0; hh < d.Hv / d.Hqk; ++hh)
       GDN_LAUNCH(kKernBwdLocal, st, kern, dim3(nc, d.Hqk), dim3(kThreads), smem, st, QTF, (const T*)KAF, (const T*)v,
                  beta, beta_same, G, Ai, VF, (const T*)DVF, (const T*)dO, HF, (const T*)DHF, rstd_q, rstd_k, (T*)dq, (T*)dk,
-                 (T*)dv, dbeta, dg, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale, hh, d.strides(), (float*)nullptr);
+                 (T*)dv, dbeta, dg, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale, hh, d.strides(), (T*)nullptr, (float*)nullptr);
   }
   return (int)hipGetLastError();
 }

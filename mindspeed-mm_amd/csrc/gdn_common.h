@@ -95,6 +95,12 @@ __device__ __forceinline__ int xcd_grouped_head(int b, int total, int grp) {
 #ifndef GDN_WAVES_PER_SIMD
 #define GDN_WAVES_PER_SIMD(n) __attribute__((amdgpu_waves_per_eu(n, n)))
 #endif
+// Pins a register value to this point of the program: the compiler can neither compute what follows from it earlier
+// nor sink what precedes it.  Used where a cheap operation on a loaded value would otherwise be moved up to right
+// behind the load and make the wave wait for it there, before the loads that follow have been issued.
+#ifndef GDN_KEEP_HERE
+#define GDN_KEEP_HERE(x) asm volatile("" : "+v"(x))
+#endif
 // Asks the scheduler for the pattern (1 matrix instruction, nvalu vector instructions) x nmfma in the current
 // scheduling region.
 #define GDN_INTERLEAVE_MFMA_VALU(nmfma, nvalu)                        \

@@ -78,9 +78,12 @@ __global__ __launch_bounds__(kConvThreads) GDN_WAVES_PER_SIMD(W <= 4 ? 4 : 2) vo
     const T* __restrict__ init, const int64_t* __restrict__ cu, T* __restrict__ y, int64_t total, int T_len, int N,
     int D, int tile, int silu) {
   constexpr int V = Elem<T>::kVec;
-  const int d0 = (blockIdx.x * kConvThreads + threadIdx.x) * V;
+  // one linear grid, channel blocks fastest: the number of token tiles is not bounded by the y dimension's 65535
+  const int nbd = (D / V + kConvThreads - 1) / kConvThreads, bx = blockIdx.x % nbd;
+  const int64_t by = blockIdx.x / nbd;
+  const int d0 = (bx * kConvThreads + threadIdx.x) * V;
   if (d0 >= D) return;
-  const int64_t t0 = (int64_t)blockIdx.y * tile;
+  const int64_t t0 = by * tile;
   const int64_t t1 = t0 + tile < total ? t0 + tile : total;
   float wgt[W][V], bs[V], win[W][V];
 #pragma unroll
@@ -158,9 +161,12 @@ __global__ __launch_bounds__(kConvThreads) void conv1d_bwd_kernel(
     const T* __restrict__ init, const T* __restrict__ dht, const int64_t* __restrict__ cu, T* __restrict__ dx,
     float* __restrict__ part, int64_t total, int T_len, int N, int D, int tile, int silu) {
   constexpr int V = Elem<T>::kVec;
-  const int d0 = (blockIdx.x * kConvThreads + threadIdx.x) * V;
+  // one linear grid, channel blocks fastest: the number of token tiles is not bounded by the y dimension's 65535
+  const int nbd = (D / V + kConvThreads - 1) / kConvThreads, bx = blockIdx.x % nbd;
+  const int64_t by = blockIdx.x / nbd;
+  const int d0 = (bx * kConvThreads + threadIdx.x) * V;
   if (d0 >= D) return;
-  const int64_t t0 = (int64_t)blockIdx.y * tile;
+  const int64_t t0 = by * tile;
   const int64_t t1 = t0 + tile < total ? t0 + tile : total;
   const int64_t tend = t1 + (W - 1) < total ? t1 + (W - 1) : total;  // halo: dyp of later tokens feeds dx
   float wgt[W][V], bs[V], win[W][V], dyw[W][V], dwa[W][V], dba[V];
@@ -263,7 +269,7 @@ __global__ __launch_bounds__(kConvThreads) void conv1d_bwd_kernel(
     request(xa, ga, tb + 2 * W);
     trip(tb + W, xb, gb);
   }
-  float* pp = part + (int64_t)blockIdx.y * (W + 1) * D;
+  float* pp = part + by * (W + 1) * D;
 #pragma unroll
   for (int w = 0; w < W; ++w)
 #pragma unroll
@@ -379,7 +385,9 @@ template <typename T> struct ConvLaunch {
     constexpr int V = Elem<T>::kVec;
     const int64_t total = (int64_t)B * T_len;
     const int tile = 64;
-    dim3 grid((D / V + kConvThreads - 1) / kConvThreads, (unsigned)((total + tile - 1) / tile));
+    const int64_t nblocks = (int64_t)((D / V + kConvThreads - 1) / kConvThreads) * ((total + tile - 1) / tile);
+    if (nblocks > 0x7fffffffLL) return -3;
+    dim3 grid((unsigned)nblocks);
     if (total > 0) {
       switch (W) {
 #define GDN_CASE(W_)                                                                                              \
@@ -407,7 +415,9 @@ template <typename T> struct ConvLaunch {
     const int64_t total = (int64_t)B * T_len;
     const int tile = 256;
     const int ntiles = (int)((total + tile - 1) / tile);
-    dim3 grid((D / V + kConvThreads - 1) / kConvThreads, (unsigned)ntiles);
+    const int64_t nblocks = (int64_t)((D / V + kConvThreads - 1) / kConvThreads) * ntiles;
+    if (nblocks > 0x7fffffffLL) return -3;
+    dim3 grid((unsigned)nblocks);
     if (total > 0) {
       switch (W) {
 #define GDN_CASE(W_)                                                                                              \

@@ -9,7 +9,7 @@
 //   Kp = k . e^{G}   K1 = -b Kp   K2 = k . e^{G_last-G}   Qb = scale q . e^{G}
 //   L_ij = b_i sum_d k_id k_jd e^{G_id-G_jd} (i>j)   Tm = (I+L)^-1   Aq_ij = scale sum_d q_id k_jd e^{G_id-G_jd} (i>=j)
 //   z = b v + K1 S    V' = Tm z    O = Qb S + Aq V'    S' = e^{G_last} . S + K2^T V'
-// What arrives (sums over V, fp32): dQb = dO S^T, dK2 = V' dS'^T, P = dV' S^T, dAq = tril(dO V'^T), a2 = dV' V^T,
+// What arrives (sums over V, rounded to T; dD in fp32): dQb = dO S^T, dK2 = V' dS'^T, P = dV' S^T, dAq = tril(dO V'^T), a2 = dV' V^T,
 // dD = sum_v dS' . S.  Then
 //   dTm = stril(b_j (a2 - P Kp^T))    dL = -stril(Tm^T dTm Tm^T)    dK1 = Tm^T P    <R_t, v_t> = sum_i Tm_it a2_it
 //   U_i  = sum_{j<i}  dL_ij        k_j . e^{G_i-G_j}          Uq_i = sum_{j<=i} scale dAq_ij k_j . e^{G_i-G_j}
@@ -72,7 +72,7 @@ template <typename T, int DK>
 __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const void* __restrict__ g, const float* __restrict__ A_log,
     const float* __restrict__ dt_bias, const float* __restrict__ bhat, const float* __restrict__ GC,
-    const T* __restrict__ TMR, const float* __restrict__ dumps, const int64_t* __restrict__ cu,
+    const T* __restrict__ TMR, const T* __restrict__ dumps, const float* __restrict__ dd, const int64_t* __restrict__ cu,
     const int* __restrict__ chunk_offsets, T* __restrict__ dq, T* __restrict__ dk, void* __restrict__ dg,
     void* __restrict__ dbeta, float* __restrict__ part, int T_len, int N, int H, float scale, KdaFlags fl) {
   using SM = KdaBwdSmem<T, DK>;
@@ -110,40 +110,39 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
   const bool tile_wave = wave < 4, lower = tile_wave && tj <= ti;
   const int cj = wave >> 1, ri = wave & 1;
   const bool has_k = cj < NKT;
-  const float* dump = dumps + ch * (3 * 64 * DK + 2 * 64 * 64 + DK);
-  const float* dQb = dump, *dK2 = dump + 64 * DK, *Pm = dump + 2 * 64 * DK;
-  const float* dAq = dump + 3 * 64 * DK, *a2m = dAq + 64 * 64, *dD = a2m + 64 * 64;
+  const T* dump = dumps + ch * (3 * 64 * DK + 2 * 64 * 64);
+  const T* dQb = dump, *dK2 = dump + 64 * DK, *Pm = dump + 2 * 64 * DK;
+  const T* dAq = dump + 3 * 64 * DK, *a2m = dAq + 64 * 64;
+  const float* dD = dd + ch * DK;
   const float* Gc = GC + ch * 64 * DK;
 
   // ---- phase A0: k^ rows; P and Tm as operands; beta.  The tile waves request their tiles of a2 and dAq now ----
   TileQK<T, DK> kt, qt;     // moved by the first kThreads threads
   if (tile_wave) tile_qk_request<T, DK>(kt, k + tok0 * hk + h * DK, hk, nvalid, tid);
-  f32x16 a2t, dat;
+  // (every tile wave loads, also the one of the upper tile, which nobody wrote: a test per load would make each of
+  // them wait for the one before; what it reads is dropped below)
+  // (as bits in a register each, widened where they are used: anything done to a value here waits for its load)
+  uint32_t a2r[16], dar[16];
+  if (tile_wave) {
+    using Bits = typename std::conditional<sizeof(T) == 2, uint16_t, uint32_t>::type;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int at = (32 * ti + acc_row(r)) * 64 + 32 * tj + l32;
-    a2t[r] = lower ? a2m[at] : 0.f;
-    dat[r] = lower ? dAq[at] : 0.f;
+    for (int r = 0; r < 16; ++r) {
+      const int at = (32 * ti + acc_row(r)) * 64 + 32 * tj + l32;
+      a2r[r] = reinterpret_cast<const Bits*>(a2m)[at];
+      dar[r] = reinterpret_cast<const Bits*>(dAq)[at];
+    }
   }
-  if (tid < 64) {
-    bs[tid] = tid < nvalid ? bhat[(tok0 + tid) * H + h] : 0.f;
-    rsq[tid] = 1.f;
-    rsk[tid] = 1.f;
-  }
-  if (tid < 256) { rq[tid] = 0.f; rk[tid] = 0.f; rb[tid] = 0.f; rv[tid] = 0.f; }
   // this thread's pieces of P and G (VEC consecutive channels of a row each), all requested before the first wait
   constexpr int NIT = 64 * CPR / kFinThreads, C64 = 64 / VEC, NTM = 64 * C64 / kFinThreads;
   static_assert(64 * CPR % kFinThreads == 0 && 64 * C64 % kFinThreads == 0 && VEC % 4 == 0, "whole rounds of 16-byte pieces");
-  f32x4 pf[NIT][VEC / 4], gk[NIT][VEC / 4];
-  Vec16<T> tmv[NTM];
+  f32x4 gk[NIT][VEC / 4];
+  Vec16<T> pf[NIT], tmv[NTM];
 #pragma unroll
   for (int it = 0; it < NIT; ++it) {
     const int c = tid + it * kFinThreads, at = (c / CPR) * DK + (c % CPR) * VEC;
+    pf[it] = ld16(Pm + at);
 #pragma unroll
-    for (int e = 0; e < VEC / 4; ++e) {
-      pf[it][e] = *reinterpret_cast<const f32x4*>(Pm + at + 4 * e);
-      gk[it][e] = *reinterpret_cast<const f32x4*>(Gc + at + 4 * e);
-    }
+    for (int e = 0; e < VEC / 4; ++e) gk[it][e] = *reinterpret_cast<const f32x4*>(Gc + at + 4 * e);
   }
 #pragma unroll
   for (int it = 0; it < NTM; ++it) {
@@ -151,13 +150,16 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     tmv[it] = ld16(TMR + ch * 4096 + (c / C64) * 64 + (c % C64) * VEC);
   }
   if (tile_wave) tile_qk_request<T, DK>(qt, q + tok0 * hk + h * DK, hk, nvalid, tid);
+  if (tid < 64) {
+    bs[tid] = tid < nvalid ? bhat[(tok0 + tid) * H + h] : 0.f;
+    rsq[tid] = 1.f;
+    rsk[tid] = 1.f;
+  }
+  if (tid < 256) { rq[tid] = 0.f; rk[tid] = 0.f; rb[tid] = 0.f; rv[tid] = 0.f; }
 #pragma unroll
   for (int it = 0; it < NIT; ++it) {
     const int c = tid + it * kFinThreads;
-    float f[VEC];
-#pragma unroll
-    for (int e = 0; e < VEC; ++e) f[e] = pf[it][e / 4][e % 4];
-    st16(Pt + (c / CPR) * LDK + (c % CPR) * VEC, pack16<T>(f));
+    st16(Pt + (c / CPR) * LDK + (c % CPR) * VEC, pf[it]);
   }
 #pragma unroll
   for (int it = 0; it < NTM; ++it) {
@@ -179,6 +181,16 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
   GDN_LDS_BARRIER();
 
   // ---- phase A1: dTm = stril(b_j (a2 - P Kp^T)), one 32x32 tile per tile wave; <R_t, v_t> from Tm and a2 ----
+  f32x16 a2t = acc_zero(), dat = acc_zero();
+  if (lower) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      GDN_KEEP_HERE(a2r[r]);
+      GDN_KEEP_HERE(dar[r]);
+      a2t[r] = __uint_as_float(a2r[r] << (sizeof(T) == 2 ? 16 : 0));
+      dat[r] = __uint_as_float(dar[r] << (sizeof(T) == 2 ? 16 : 0));
+    }
+  }
   if (tile_wave) {
     f32x16 x = acc_zero();
     if (lower) mma32<T, DK, true, true>(x, Pt + 32 * ti * LDK, LDK, Kp + 32 * tj * LDK, LDK);
@@ -399,8 +411,8 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int i = 32 * ri + acc_row(r);
-      lq[r] = dQb[i * DK + d];
-      lk[r] = dK2[i * DK + d];
+      lq[r] = Elem<T>::to_f(dQb[i * DK + d]);
+      lk[r] = Elem<T>::to_f(dK2[i * DK + d]);
     }
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (!FULL) mma32<T, 64, false, false>(dK1, TmT + 32 * ri, L64, Pt + 32 * cj, LDK);
@@ -602,7 +614,8 @@ static int kda_bwd_launch(const ChunkDims& d, const KdaWorkspace& L, const void*
   const T* QBT = reinterpret_cast<const T*>(ws + L.QBT);
   T* DVF = reinterpret_cast<T*>(ws + L.DVF);
   T* DHF = reinterpret_cast<T*>(ws + L.DHF);
-  float* DUMP = reinterpret_cast<float*>(ws + L.DUMP);
+  T* DUMP = reinterpret_cast<T*>(ws + L.DUMP);
+  float* DD = reinterpret_cast<float*>(ws + L.DD);
   float* PART = reinterpret_cast<float*>(ws + L.PART);
   {
     auto kern = chunk_state_bwd_kernel<T, DK, NWS, NLS, STAGES, true>;
@@ -619,14 +632,14 @@ static int kda_bwd_launch(const ChunkDims& d, const KdaWorkspace& L, const void*
     GDN_LAUNCH(kKernBwdLocal, st, kern, dim3(nc, H), dim3(kThreads), smem, st, QBT, K1F, (const T*)v, (const void*)bhat, 0,
                (const float*)nullptr, Ai, VF, (const T*)DVF, (const T*)dO, HF, (const T*)DHF, (const float*)nullptr,
                (const float*)nullptr, (T*)nullptr, (T*)nullptr, (T*)dv, (void*)nullptr, (float*)nullptr, cu, chunk_offsets, d.T,
-               d.N, H, H, d.V, scale, 0, ts, DUMP);
+               d.N, H, H, d.V, scale, 0, ts, DUMP, DD);
   }
   {
     auto kern = kda_bwd_finish_kernel<T, DK>;
     constexpr int smem = KdaBwdSmem<T, DK>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
     GDN_LAUNCH(kKernKdaBwdFinish, st, kern, dim3(nc, H), dim3(kFinThreads), smem, st, (const T*)q, (const T*)k, g, A_log, dt_bias,
-               bhat, GC, TMR, (const float*)DUMP, cu, chunk_offsets, (T*)dq, (T*)dk, dg, dbeta, PART, d.T, d.N, H, scale, fl);
+               bhat, GC, TMR, (const T*)DUMP, (const float*)DD, cu, chunk_offsets, (T*)dq, (T*)dk, dg, dbeta, PART, d.T, d.N, H, scale, fl);
   }
   if (fl.use_gate && (dA_log != nullptr || ddt_bias != nullptr))
     GDN_LAUNCH(kKernKdaBwdReduce, st, kda_bwd_reduce_kernel, dim3(H, (d.K + 32) / 32), dim3(kThreads), 0, st, (const float*)PART, cu,

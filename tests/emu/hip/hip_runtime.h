@@ -268,6 +268,7 @@ static emu::GdimProxy gridDim;
 #define __builtin_amdgcn_rcpf(x) (1.0f / (x))
 #define __builtin_amdgcn_logf(x) log2f(x)
 #define GDN_WAVES_PER_SIMD(n)
+#define GDN_KEEP_HERE(x) ((void)0)
 #define __builtin_amdgcn_sched_group_barrier(m, n, s) ((void)0)
 #define __builtin_amdgcn_wave_barrier() emu::wave_sync()
 #define __builtin_amdgcn_s_sleep(x) emu::yield()
