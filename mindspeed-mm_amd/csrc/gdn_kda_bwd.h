@@ -46,7 +46,10 @@ template <typename T, int DK> struct KdaBwdSmem {
   // where it is used, after the decay-weighted sums, instead of occupying registers through them
   static constexpr int off_q2 = off_m2t + (FULL ? 0 : mat);
   static constexpr int off_m1t = off_q2 + (FULL ? 0 : tile);
-  static constexpr int off_row = off_m1t + (FULL ? 0 : mat);
+  // not FULL: which entries of a coefficient fragment belong to a level's pairs: [5 levels][2 halves of the 32 columns]
+  // [row = earlier | later token][64 lanes] masks of 16 bytes.  They depend on nothing but the lane.
+  static constexpr int off_keep = off_m1t + (FULL ? 0 : mat);
+  static constexpr int off_row = off_keep + (FULL ? 0 : 5 * 2 * 2 * 64 * 16);
   // beta, 1/|q|, 1/|k| [64 each]; row sums <q^,dq^>, <k^,dk^>, db, <R,v> [256 each]; per-wave scalars [8]; what the
   // two waves of a channel block exchange: parts of dG_last and d(dt_bias) [8][32 each], sum of dG over tokens 32.. [4][32]
   static constexpr int bytes = off_row + (3 * 64 + 4 * 256 + 8 + 2 * 256 + 128) * 4;
@@ -130,6 +133,27 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
       const int at = (32 * ti + acc_row(r)) * 64 + 32 * tj + l32;
       a2r[r] = reinterpret_cast<const Bits*>(a2m)[at];
       dar[r] = reinterpret_cast<const Bits*>(dAq)[at];
+    }
+  }
+  u32x4* keepT = reinterpret_cast<u32x4*>(gdn_smem + SM::off_keep);
+  if constexpr (!FULL) {
+    // Which of 8 consecutive entries of a coefficient row belong to a level's pairs, as a mask over the fragment (two
+    // 16-bit entries per register).  a: the row's token within the 32-token block, b: that of a column.  second: the
+    // row index is the later token i (kept when i is in the second half of its block of 2^lg tokens and the column j
+    // in the first half of the same block), else the row index is the earlier token j.
+    for (int idx = tid; idx < 5 * 2 * 2 * 64; idx += kFinThreads) {
+      const int ln = idx & 63, second = (idx >> 6) & 1, kg = (idx >> 7) & 1, lg = (idx >> 8) + 1;
+      const int a = ln & 31, b0 = 16 * kg + 8 * (ln >> 5), n2 = (1 << lg) >> 1, nm = (1 << lg) - 1;
+      const bool rok = second ? ((a & nm) >= n2) : ((a & nm) < n2);
+      u32x4 w;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int b1 = b0 + 2 * e, b2 = b1 + 1;
+        const bool k1 = rok && (a >> lg) == (b1 >> lg) && (second ? ((b1 & nm) < n2) : ((b1 & nm) >= n2));
+        const bool k2 = rok && (a >> lg) == (b2 >> lg) && (second ? ((b2 & nm) < n2) : ((b2 & nm) >= n2));
+        w[e] = (k1 ? 0xffffu : 0u) | (k2 ? 0xffff0000u : 0u);
+      }
+      keepT[idx] = w;
     }
   }
   // this thread's pieces of P and G (VEC consecutive channels of a row each), all requested before the first wait
@@ -265,22 +289,6 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
   if constexpr (!FULL) {
     if (has_k) {
       const int half = lane >> 5;
-      // fragment of a coefficient matrix: row `row`, 8 consecutive columns from `col0`, of which only those of the
-      // level's pairs are kept.  second: the row index is the later token i (kept when i is in the second half of its
-      // block and the column j in the first), else the row index is the earlier token j.
-      auto coef = [&](const T* M, int row, int col0, int a, int b0, int lg, bool second) {
-        u32x4 w = ld16(M + row * L64 + col0).raw;
-        const int n2 = (1 << lg) >> 1, nm = (1 << lg) - 1;
-        const bool rok = second ? ((a & nm) >= n2) : ((a & nm) < n2);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int b1 = b0 + 2 * e, b2 = b1 + 1;
-          const bool k1 = rok && (a >> lg) == (b1 >> lg) && (second ? ((b1 & nm) < n2) : ((b1 & nm) >= n2));
-          const bool k2 = rok && (a >> lg) == (b2 >> lg) && (second ? ((b2 & nm) < n2) : ((b2 & nm) >= n2));
-          w[e] &= (k1 ? 0xffffu : 0u) | (k2 ? 0xffff0000u : 0u);
-        }
-        return w;
-      };
       {
         // The partner rows this lane supplies as B operand, channel d, are tokens 32 ri + 16 kg + 8 half + e.  They
         // are read again at every level: held in registers through the levels they would push other values out to
@@ -294,8 +302,15 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
         }
 #pragma unroll 1
         for (int lg = 1; lg <= 5; ++lg) {   // blocks of n = 2^lg tokens inside the 32-token block
-          const int n = 1 << lg;
+          const int n2 = (1 << lg) >> 1;
           asm volatile("" ::: "memory");   // the reads of a level stay inside it
+          // The reference row of a token is the middle of its block of 2^lg tokens.  For the lane's 8 partner rows of a
+          // group (and for the rows of its accumulator registers) it is a row that depends on the lane only through the
+          // half-wave, and that only while the block is no larger than the group of rows the half-wave holds, plus an
+          // offset that is the same for every lane: one addition per address instead of a shift, a mask and a product.
+          const float* Gpm = Gs + (32 * ri + (lg <= 3 ? 8 * half : 0)) * LDG + d;
+          const float* Gom = Gs + (32 * ri + (lg <= 2 ? 4 * half : 0)) * LDG + d;
+          const u32x4* keepL = keepT + (lg - 1) * 4 * 64 + lane;
           f32x16 cu = acc_zero(), cq = acc_zero(), cw = acc_zero();
 #pragma unroll
           for (int kg = 0; kg < 2; ++kg) {
@@ -303,21 +318,22 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
             ld_f32<8>(bs + 32 * ri + 16 * kg + 8 * half, bx);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-              const int x = 32 * ri + 16 * kg + 8 * half + e, m = ((x >> lg) << lg) + (n >> 1);
-              const float f = __expf(-fabsf(Gs[x * LDG + d] - Gs[m * LDG + d]));
+              const int x = 32 * ri + 16 * kg + 8 * half + e, sm = (((16 * kg + e) >> lg) << lg) + n2;
+              const float f = __expf(-fabsf(Gs[x * LDG + d] - Gpm[sm * LDG]));
               xk[e] = Elem<T>::to_f(Ks[x * LDK + d]) * f; xb[e] = bx[e] * xk[e]; xq[e] = Elem<T>::to_f(Qs[x * LDK + d]) * f;
             }
             const u32x4 bK = pack16<T>(xk).raw, bB = pack16<T>(xb).raw, bQ = pack16<T>(xq).raw;
-            const int row = 32 * ri + l32, col0 = 32 * ri + 16 * kg + 8 * half, b0 = 16 * kg + 8 * half;
-            mfma_kgroup<T>(cu, coef(M1, row, col0, l32, b0, lg, true), bK);     // sum_j dL_ij (k_j f_j)
-            mfma_kgroup<T>(cq, coef(M2, row, col0, l32, b0, lg, true), bK);
-            mfma_kgroup<T>(cw, coef(M1t, row, col0, l32, b0, lg, false), bB);   // sum_i dL_ij (b_i k_i f_i)
-            mfma_kgroup<T>(cw, coef(M2t, row, col0, l32, b0, lg, false), bQ);
+            const int row = 32 * ri + l32, col0 = 32 * ri + 16 * kg + 8 * half;
+            const u32x4 keep1 = keepL[2 * kg * 64], keep2 = keepL[(2 * kg + 1) * 64];
+            mfma_kgroup<T>(cu, ld16(M1 + row * L64 + col0).raw & keep2, bK);     // sum_j dL_ij (k_j f_j)
+            mfma_kgroup<T>(cq, ld16(M2 + row * L64 + col0).raw & keep2, bK);
+            mfma_kgroup<T>(cw, ld16(M1t + row * L64 + col0).raw & keep1, bB);   // sum_i dL_ij (b_i k_i f_i)
+            mfma_kgroup<T>(cw, ld16(M2t + row * L64 + col0).raw & keep1, bQ);
           }
 #pragma unroll
           for (int r = 0; r < 16; ++r) {   // every row by its own factor
-            const int i = 32 * ri + acc_row(r), m = ((i >> lg) << lg) + (n >> 1);
-            const float f = __expf(-fabsf(Gi[r] - Gs[m * LDG + d]));
+            const int sm = (((8 * (r / 4) + r % 4) >> lg) << lg) + n2;
+            const float f = __expf(-fabsf(Gi[r] - Gom[sm * LDG]));
             U[r] += f * cu[r];
             Uq[r] += f * cq[r];
             W[r] += f * cw[r];
