@@ -395,6 +395,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   float* rv = rf + 256;    // <R_i, v_i>, taken as the column sums of Tm . (dV' V^T)
   float* wsum = rv + 256;  // per wave: <S,dS'> [0..3], sum_i <k_i, dK_inter_i> [4..7]
 
+  stagger_second_resident<127>(3, 8 * kStaggerCUs);
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31;
