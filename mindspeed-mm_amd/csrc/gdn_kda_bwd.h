@@ -692,8 +692,12 @@ extern "C" int gdn_kda_bwd(const void* q, const void* k, const void* v, const vo
 #define GDN_KDAB(T_, DK_, NWS_, NLS_, ST_)                                                                              \
   return kda_bwd_launch<T_, DK_, NWS_, NLS_, ST_>(d, L, q, k, v, g, A_log, dt_bias, cu_seqlens, d_o, d_final_state, dq, dk, dv, \
                                                   dg, dbeta, dA_log, ddt_bias, d_initial_state, ws, scale, fl, st)
+  const bool one_slab = one_slab_per_workgroup(d, device_compute_units());
   if (dtype == 1) {
-    if (K == 128) GDN_KDAB(bf16_t, 128, 2, 4, 2);
+    if (K == 128) {
+      if (one_slab) GDN_KDAB(bf16_t, 128, 1, 4, 2);
+      GDN_KDAB(bf16_t, 128, 2, 4, 2);
+    }
     GDN_KDAB(bf16_t, 64, 2, 2, 2);
   } else {
     if (K == 128) GDN_KDAB(float, 128, 2, 2, 1);

@@ -400,8 +400,13 @@ extern "C" int gdn_kda_fwd(const void* q, const void* k, const void* v, const vo
 #define GDN_KDA(T_, DK_, NWO_, NWS_, NLS_, ST_)                                                                          \
   return kda_fwd_launch<T_, DK_, NWO_, NWS_, NLS_, ST_>(d, L, q, k, v, g, beta, A_log, dt_bias, initial_state, cu_seqlens, o, \
                                                         final_state, ws, scale, fl, with_bwd, st)
+  // a CU per 32-column slab of the state while there are no more slabs than CUs (see one_slab_per_workgroup)
+  const bool one_slab = one_slab_per_workgroup(d, device_compute_units());
   if (dtype == 1) {
-    if (K == 128) GDN_KDA(bf16_t, 128, 2, 2, 4, 2);
+    if (K == 128) {
+      if (one_slab) GDN_KDA(bf16_t, 128, 2, 1, 4, 2);
+      GDN_KDA(bf16_t, 128, 2, 2, 4, 2);
+    }
     GDN_KDA(bf16_t, 64, 2, 2, 4, 2);
   } else {
     if (K == 128) GDN_KDA(float, 128, 2, 2, 2, 1);

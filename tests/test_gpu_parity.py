@@ -406,6 +406,7 @@ KDA_CASES = [
     (BF, 1, 130, 1, 128, 64, None, dict(allow_neg=True, with_h0=False, g_dtype=torch.float32)),
     (BF, 1, 300, 3, 128, 256, [0, 0, 300], dict(gate_in_kernel=False)),                      # an empty sequence
     (BF, 1, 2048, 4, 128, 128, None, {}),                                                     # the layer's head shape
+    (BF, 4, 130, 24, 128, 128, None, {}),                          # more 32-column slabs of the state than CUs: two per workgroup
 ]
 
 
