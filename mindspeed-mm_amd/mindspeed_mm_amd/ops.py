@@ -1015,3 +1015,58 @@ class RMSNormGated(torch.nn.Module):
     def forward(self, hidden_states, gate=None):
         return rms_norm_gated(hidden_states, gate, self.weight, self.variance_epsilon)
 
+
+class ShortConvolution(torch.nn.Conv1d):
+    """Drop-in for the KDA layer's ShortConvolution (mindspeed_mm/fsdp/ops/kda/short_conv.py:18-218): the same
+    constructor, parameters (a depthwise nn.Conv1d weight [D, 1, W], optional bias) and forward, over causal_conv1d /
+    causal_conv1d_update of this package.  `backend` is accepted and reported as 'mi355x'."""
+
+    def __init__(self, hidden_size, kernel_size, bias=False, activation="silu", backend="triton", device=None,
+                 dtype=None, **kwargs):
+        super().__init__(in_channels=hidden_size, out_channels=hidden_size, kernel_size=kernel_size,
+                         groups=hidden_size, bias=bias, padding=kernel_size - 1, device=device, dtype=dtype)
+        self.hidden_size = hidden_size
+        self.activation = None
+        if activation is not None:
+            if activation not in ("silu", "swish"):
+                raise AssertionError(f"Activation `{activation}` not supported yet.")   # short_conv.py:72
+            self.activation = activation
+        self.backend = "mi355x"
+
+    def extra_repr(self):
+        return (f"{self.in_channels}, {self.out_channels}, kernel_size={self.kernel_size}, groups={self.groups}, "
+                f"bias={self.bias is not None}, activation={self.activation}, backend={self.backend}")
+
+    def forward(self, x, residual=None, mask=None, cache=None, output_final_state=False, cu_seqlens=None,
+                chunk_indices=None, **kwargs):
+        """x [B, T, D] (B = 1 with cu_seqlens); cache [N, D, W], updated in place in the decoding case (one token per
+        sequence, short_conv.py:145-154); returns (y [B, T, D], final state [N, D, W] or None)."""
+        B, T = x.shape[0], x.shape[1]
+        N = B if cu_seqlens is None else len(cu_seqlens) - 1
+        if mask is not None:
+            if cu_seqlens is not None:
+                raise ValueError("`mask` and `cu_seqlens` cannot be provided at the same time")
+            x = x.mul_(mask.unsqueeze(-1))     # in place, as the reference does (short_conv.py:143)
+        if B * T == N:
+            return self.step(x, residual, cache, output_final_state, cu_seqlens)
+        weight = self.weight.squeeze(1).transpose(0, 1).contiguous()      # [D, 1, W] -> [W, D]
+        return causal_conv1d(x=x, weight=weight, bias=self.bias, residual=residual, initial_state=cache,
+                             output_final_state=output_final_state, activation=self.activation,
+                             cu_seqlens=cu_seqlens, **kwargs)
+
+    def step(self, x, residual, cache, output_final_state=False, cu_seqlens=None):
+        """One token per sequence: the cache rolls by one and takes the token (short_conv.py:185-213)."""
+        D, W = x.shape[-1], self.kernel_size[0]
+        N = x.shape[0] if cu_seqlens is None else len(cu_seqlens) - 1
+        if cache is None:
+            cache = x.new_zeros(N, D, W)
+        y = causal_conv1d_update(x.reshape(N, 1, D), cache, self.weight.squeeze(1), self.bias, self.activation)
+        y = y.reshape(x.shape)
+        if residual is not None:
+            y = y + residual
+        return y, (cache if output_final_state else None)
+
+    @property
+    def state_size(self):
+        return self.hidden_size * self.kernel_size[0]
+

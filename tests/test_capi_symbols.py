@@ -143,3 +143,25 @@ def test_decode_cache_bookkeeping():
     c.reorder_cache(torch.tensor([1, 1, 0]))
     assert torch.equal(c.conv_states[1], conv[[1, 1, 0]]) and torch.equal(c.recurrent_states[1], rec[[1, 1, 0]])
     assert c.conv_states[0] is None and c.recurrent_states[2] is None
+
+
+def test_short_convolution_module_host_side():
+    """Constructor, parameters and argument checks of the KDA layer's convolution module (short_conv.py:46-81,
+    137-143), none of which touches a device; a host tensor then meets the operator's refusal."""
+    import torch
+    import mindspeed_mm_amd as M
+    conv = M.ShortConvolution(32, 4, bias=True, activation="silu", backend="cuda", dtype=torch.bfloat16)
+    assert isinstance(conv, torch.nn.Conv1d) and conv.groups == 32 and conv.padding == (3,)
+    assert tuple(conv.weight.shape) == (32, 1, 4) and conv.weight.dtype == torch.bfloat16 and tuple(conv.bias.shape) == (32,)
+    assert M.ShortConvolution(8, 2).bias is None and M.ShortConvolution(8, 2, activation=None).activation is None
+    assert conv.state_size == 32 * 4 and "activation=silu" in repr(conv)
+    with pytest.raises(AssertionError):
+        M.ShortConvolution(8, 4, activation="relu")
+    x = torch.randn(1, 10, 32, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="cannot be provided at the same time"):
+        conv(x, mask=torch.ones(1, 10), cu_seqlens=torch.tensor([0, 4, 10]))
+    with pytest.raises(RuntimeError, match="no host fallback"):
+        conv(x)
+    with pytest.raises(RuntimeError, match="no host fallback"):
+        conv(x[:, :1])     # one token per sequence: the decoding call
+

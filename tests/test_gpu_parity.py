@@ -437,3 +437,54 @@ def test_kda_argument_checks(ops):
         ops.chunk_kda(d["q"], d["k"], d["v"], d["g"], d["beta"], initial_state=d["h0"].bfloat16())
     with pytest.raises(NotImplementedError):
         ops.chunk_kda(d["q"], d["k"], d["v"], d["g"], d["beta"], return_intermediate_states=True)
+
+
+@pytest.mark.parametrize("dtype,B,T,D,W,cu", [(F32, 2, 37, 16, 4, None), (BF, 1, 300, 64, 4, [0, 1, 3, 130, 131, 300])])
+def test_short_convolution_module(ops, dtype, B, T, D, W, cu):
+    """The KDA layer's convolution module (short_conv.py:18-218) over this package's operators: the prefill call with
+    a cache, a residual and the final state, its gradients down to the nn.Conv1d parameters, then the decoding call
+    (one token per sequence) on the cache it returned, against the convolution oracle."""
+    import mindspeed_mm_amd as M
+    from oracle import gdn_oracle as O
+    print(f"short convolution {dtype} B{B} T{T} D{D} W{W} varlen={cu is not None}", flush=True)
+    gen = torch.Generator().manual_seed(3)
+    r = lambda *s: torch.randn(*s, generator=gen)
+    N = B if cu is None else len(cu) - 1
+    conv = M.ShortConvolution(D, W, bias=True, activation="silu", device="cuda", dtype=dtype)
+    assert tuple(conv.weight.shape) == (D, 1, W) and tuple(conv.bias.shape) == (D,)
+    w0, b0 = (r(D, 1, W) / 2).to(dtype), r(D).to(dtype)
+    with torch.no_grad():
+        conv.weight.copy_(w0)
+        conv.bias.copy_(b0)
+    x, res, cache, dy = r(B, T, D).to(dtype), r(B, T, D).to(dtype), r(N, D, W).to(dtype), r(B, T, D).to(dtype)
+    cu_t = None if cu is None else torch.tensor(cu, dtype=torch.int64, device="cuda")
+    xd = x.cuda().requires_grad_(True)
+    y, fs = conv(xd, residual=res.cuda(), cache=cache.cuda(), output_final_state=True, cu_seqlens=cu_t)
+    R = dict(x=x.float().requires_grad_(True), w=w0.float().squeeze(1).t().contiguous().requires_grad_(True),
+             b=b0.float().requires_grad_(True))
+    ry, rfs = O.causal_conv1d_ref(R["x"], R["w"], R["b"], res.float(), cache.float(), "silu", cu, True)
+    P._err("y", y, ry, dtype, 1e-2, 1e-2)
+    P._err("final_state", fs, rfs, dtype, 1e-2, 1e-2)
+    y.backward(dy.cuda())
+    ry.backward(dy.float())
+    tol = 5e-2 * max(1.0, B * T / 256)
+    P._err("dx", xd.grad, R["x"].grad, dtype, 5e-2, 1e-2)
+    P._err("dweight", conv.weight.grad.squeeze(1).t(), R["w"].grad, dtype, tol, 1e-2)
+    P._err("dbias", conv.bias.grad, R["b"].grad, dtype, tol, 1e-2)
+    # decoding: one token per sequence; the cache is rolled in place and handed back
+    x1, res1 = r(N, 1, D).to(dtype), r(N, 1, D).to(dtype)
+    if cu is not None:       # packed: [1, N, D] with one token per sequence
+        x1, res1 = x1.transpose(0, 1).contiguous(), res1.transpose(0, 1).contiguous()
+    step_cache = fs.detach().clone()
+    cu1 = None if cu is None else torch.arange(N + 1, dtype=torch.int64, device="cuda")
+    with torch.no_grad():
+        y1, c1 = conv(x1.cuda(), residual=res1.cuda(), cache=step_cache, output_final_state=True, cu_seqlens=cu1)
+    assert c1 is step_cache and y1.shape == x1.shape
+    ref_state = rfs.detach().clone()
+    ry1 = O.causal_conv1d_update_ref(x1.float().reshape(N, 1, D), ref_state, w0.float().squeeze(1), b0.float(), "silu")
+    P._err("step y", y1.reshape(N, 1, D), ry1 + res1.float().reshape(N, 1, D), dtype, 1e-2, 1e-2)
+    P._err("step cache", step_cache, ref_state, dtype, 1e-2, 1e-2)
+    with torch.no_grad():    # without a cache the step starts from zeros and returns none unless asked
+        y2, c2 = conv(x1.cuda(), cu_seqlens=cu1)
+    assert c2 is None and y2.shape == x1.shape
+
