@@ -131,15 +131,19 @@ int gdn_conv1d_update(const void* hidden, void* conv_state, const void* weight, 
  * :897-900): y = (weight * (x * rsqrt(mean(x^2) + eps))) * silu(gate), intermediate casts to the input dtype as
  * in the reference.  x, gate, y, dy, dx, dgate [rows, N]; weight [N] in the input dtype (weight_dtype = dtype) or
  * fp32 (weight_dtype = 0); rstd [rows] fp32 is written by the forward and read by the backward; dweight [N] fp32.
- * N * element size / 16 must be 4, 8, 16, 32 or 64 (bf16: N = 32 ... 512; fp32: N = 16 ... 256). */
+ * N * element size / 16 must be 4, 8, 16, 32 or 64 (bf16: N = 32 ... 512; fp32: N = 16 ... 256).
+ * gate_activation = 1 replaces KimiK_3_MoeRMSNormGated.forward of the KDA layer instead,
+ * mindspeed_mm/fsdp/models/kimi_k3/modeling_kimi_linear.py:75-96 (called at :741 on rows of head_dim elements):
+ * y = (weight * (x * rsqrt(mean(x^2) + eps))) * sigmoid(gate), the sigmoid cast to the input dtype before the
+ * product; the result is in the input dtype. */
 int gdn_rmsnorm_gated_fwd(const void* x, const void* gate, const void* weight, void* y, float* rstd, int64_t rows,
-                          int N, float eps, int dtype, int weight_dtype, void* stream);
+                          int N, float eps, int dtype, int weight_dtype, int gate_activation, void* stream);
 
 int64_t gdn_rmsnorm_gated_bwd_workspace_bytes(int64_t rows, int N);
 
 int gdn_rmsnorm_gated_bwd(const void* x, const void* gate, const void* weight, const float* rstd, const void* dy,
                           void* dx, void* dgate, float* dweight, void* workspace, int64_t workspace_bytes,
-                          int64_t rows, int N, int dtype, int weight_dtype, void* stream);
+                          int64_t rows, int N, int dtype, int weight_dtype, int gate_activation, void* stream);
 
 /* -------- gates of the rule from the layer's projections -------------------------------------------------
  * replaces the elementwise chain in Qwen3_5GatedDeltaNet.forward, modeling_qwen3_5.py:833-841:

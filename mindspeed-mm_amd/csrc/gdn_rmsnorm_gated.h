@@ -4,6 +4,10 @@
 // for bit.
 //     xn = x * rsqrt(mean(x^2) + eps)        (fp32, then cast to the input dtype)
 //     y  = (weight * xn) * silu(gate)        (gate in fp32; result cast to the input dtype)
+// ACT = 1 is the norm of the KDA layer (KimiK_3_MoeRMSNormGated.forward,
+// mindspeed_mm/fsdp/models/kimi_k3/modeling_kimi_linear.py:83-96): the gate passes through a sigmoid that is cast to
+// the input dtype before the product,
+//     y  = (weight * xn) * cast(sigmoid(gate))
 #pragma once
 #include "gdn_common.h"
 
@@ -35,7 +39,7 @@ template <typename T> __device__ __forceinline__ float piece_sumsq(const Vec16<T
 }
 
 // TW = T: weight in the input dtype, weight * xn is rounded to T as in the reference; TW = float: kept in fp32
-template <typename T, typename TW>
+template <typename T, typename TW, int ACT = 0>
 __device__ __forceinline__ Vec16<T> rmsnorm_gated_piece(const Vec16<T>& xv, const Vec16<T>& gv, const float* w, float rstd) {
   Vec16<T> out = zero16<T>();
 #pragma unroll
@@ -43,7 +47,7 @@ __device__ __forceinline__ Vec16<T> rmsnorm_gated_piece(const Vec16<T>& xv, cons
     const float xn = round_to<T>(xv.get(e) * rstd);
     const float t = sizeof(TW) == sizeof(T) ? round_to<T>(w[e] * xn) : w[e] * xn;
     const float gf = gv.get(e);
-    out.set(e, t * (gf * sigmoid_(gf)));
+    out.set(e, ACT == 0 ? t * (gf * sigmoid_(gf)) : t * round_to<T>(sigmoid_(gf)));
   }
   return out;
 }

@@ -5,8 +5,10 @@
 //     y  = (weight * xn) * silu(gate)        (gate in fp32; result cast to the input dtype)
 // Row-wise and bandwidth-bound: forward reads x, gate and writes y; backward reads x, gate, dy and writes dx, dgate.
 // A row of N elements is held by N/VEC neighbouring lanes (16 bytes each); row sums use data-parallel-primitive moves.
-// Backward, with t = weight * xn, s = silu(gate), xh = x * rstd in fp32:
-//     dgate = dy t silu'(gate)     dt = dy s     dweight = sum_rows dt xn     dxn = dt weight
+// With gate_activation = 1 the gate passes through a sigmoid instead (the KDA layer's norm, KimiK_3_MoeRMSNormGated,
+// mindspeed_mm/fsdp/models/kimi_k3/modeling_kimi_linear.py:75-96): s = cast(sigmoid(gate)).
+// Backward, with t = weight * xn, s = silu(gate) or sigmoid(gate), xh = x * rstd in fp32:
+//     dgate = dy t s'(gate)     dt = dy s     dweight = sum_rows dt xn     dxn = dt weight
 //     dx = rstd (dxn - xh mean(dxn xh))
 // dweight is accumulated per thread over the rows it visits, reduced inside the workgroup through LDS and written as one
 // partial row per workgroup; rmsnorm_gated_dw_reduce_kernel adds the partials in a fixed order (bitwise reproducible).
@@ -26,7 +28,7 @@ template <int LPR> __device__ __forceinline__ float row_lanes_sum(float v) {
 }
 
 // TW = T: weight in the input dtype, weight * xn is rounded to T as in the reference; TW = float: kept in fp32
-template <typename T, typename TW, int LPR>
+template <typename T, typename TW, int LPR, int ACT>
 __global__ __launch_bounds__(kThreads) void rmsnorm_gated_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gate,
                                                                      const TW* __restrict__ weight, T* __restrict__ y,
                                                                      float* __restrict__ rstd_out, int64_t rows,
@@ -42,7 +44,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_gated_fwd_kernel(const T* __
     const Vec16<T> gv = ok ? ld16(gate + row * N + c * V) : zero16<T>();
     const float ss = row_lanes_sum<LPR>(piece_sumsq<T>(xv));
     const float rstd = rsqrtf(ss * (1.f / N) + eps);
-    const Vec16<T> out = rmsnorm_gated_piece<T, TW>(xv, gv, w, rstd);
+    const Vec16<T> out = rmsnorm_gated_piece<T, TW, ACT>(xv, gv, w, rstd);
     if (ok) {
       __builtin_nontemporal_store(out.raw, reinterpret_cast<u32x4*>(y + row * N + c * V));
       if (c == 0) rstd_out[row] = rstd;
@@ -50,7 +52,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_gated_fwd_kernel(const T* __
   }
 }
 
-template <typename T, typename TW, int LPR>
+template <typename T, typename TW, int LPR, int ACT>
 __global__ __launch_bounds__(kThreads) void rmsnorm_gated_bwd_kernel(
     const T* __restrict__ x, const T* __restrict__ gate, const TW* __restrict__ weight,
     const float* __restrict__ rstd_in, const T* __restrict__ dy, T* __restrict__ dx, T* __restrict__ dgate,
@@ -77,8 +79,8 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_gated_bwd_kernel(
       const float xn = round_to<T>(xh[e]);
       const float t = sizeof(TW) == sizeof(T) ? round_to<T>(w[e] * xn) : w[e] * xn;
       const float gf = gv.get(e), sg = sigmoid_(gf), d = dv.get(e);
-      dgo.set(e, d * t * sg * (1.f + gf * (1.f - sg)));
-      const float dt = d * gf * sg;
+      dgo.set(e, ACT == 0 ? d * t * sg * (1.f + gf * (1.f - sg)) : d * t * sg * (1.f - sg));
+      const float dt = ACT == 0 ? d * gf * sg : d * round_to<T>(sg);
       dwa[e] += dt * xn;
       dxn[e] = dt * w[e];
       dot += dxn[e] * xh[e];
@@ -126,19 +128,28 @@ static int rmsnorm_blocks(int64_t rows, int rpb) {
 
 template <typename T, typename TW, int LPR>
 static int rmsnorm_fwd_launch(const void* x, const void* gate, const void* weight, void* y, float* rstd, int64_t rows,
-                              float eps, hipStream_t st) {
-  GDN_LAUNCH(kKernRmsNormFwd, st, (rmsnorm_gated_fwd_kernel<T, TW, LPR>), dim3(rmsnorm_blocks(rows, kThreads / LPR)),
-             dim3(kThreads), 0, st, (const T*)x, (const T*)gate, (const TW*)weight, (T*)y, rstd, rows, eps);
+                              float eps, int act, hipStream_t st) {
+  const dim3 grid(rmsnorm_blocks(rows, kThreads / LPR));
+  if (act == 0)
+    GDN_LAUNCH(kKernRmsNormFwd, st, (rmsnorm_gated_fwd_kernel<T, TW, LPR, 0>), grid, dim3(kThreads), 0, st, (const T*)x,
+               (const T*)gate, (const TW*)weight, (T*)y, rstd, rows, eps);
+  else
+    GDN_LAUNCH(kKernRmsNormFwd, st, (rmsnorm_gated_fwd_kernel<T, TW, LPR, 1>), grid, dim3(kThreads), 0, st, (const T*)x,
+               (const T*)gate, (const TW*)weight, (T*)y, rstd, rows, eps);
   return (int)hipGetLastError();
 }
 
 template <typename T, typename TW, int LPR>
 static int rmsnorm_bwd_launch(const void* x, const void* gate, const void* weight, const float* rstd, const void* dy,
-                              void* dx, void* dgate, float* dw, float* part, int64_t rows, hipStream_t st) {
+                              void* dx, void* dgate, float* dw, float* part, int64_t rows, int act, hipStream_t st) {
   constexpr int N = LPR * Elem<T>::kVec;
   const int nb = rmsnorm_blocks(rows, kThreads / LPR);
-  GDN_LAUNCH(kKernRmsNormBwd, st, (rmsnorm_gated_bwd_kernel<T, TW, LPR>), dim3(nb), dim3(kThreads), 0, st, (const T*)x,
-             (const T*)gate, (const TW*)weight, rstd, (const T*)dy, (T*)dx, (T*)dgate, part, rows);
+  if (act == 0)
+    GDN_LAUNCH(kKernRmsNormBwd, st, (rmsnorm_gated_bwd_kernel<T, TW, LPR, 0>), dim3(nb), dim3(kThreads), 0, st, (const T*)x,
+               (const T*)gate, (const TW*)weight, rstd, (const T*)dy, (T*)dx, (T*)dgate, part, rows);
+  else
+    GDN_LAUNCH(kKernRmsNormBwd, st, (rmsnorm_gated_bwd_kernel<T, TW, LPR, 1>), dim3(nb), dim3(kThreads), 0, st, (const T*)x,
+               (const T*)gate, (const TW*)weight, rstd, (const T*)dy, (T*)dx, (T*)dgate, part, rows);
   GDN_LAUNCH(kKernRmsNormReduce, st, rmsnorm_gated_dw_reduce_kernel, dim3(N), dim3(kThreads), 0, st,
              (const float*)part, dw, nb, N);
   return (int)hipGetLastError();
@@ -164,26 +175,28 @@ static int rmsnorm_lpr(int N, int elem) {
   }
 
 extern "C" int gdn_rmsnorm_gated_fwd(const void* x, const void* gate, const void* weight, void* y, float* rstd,
-                                     int64_t rows, int N, float eps, int dtype, int weight_dtype, void* stream) {
+                                     int64_t rows, int N, float eps, int dtype, int weight_dtype, int gate_activation,
+                                     void* stream) {
   using namespace gdn;
   if (!x || !gate || !weight || !y || !rstd) return -1;
   if (rows < 0) return -2;
   if (dtype != 0 && dtype != 1) return -4;
   if (weight_dtype != 0 && weight_dtype != dtype) return -4;
+  if (gate_activation != 0 && gate_activation != 1) return -4;
   const int lpr = rmsnorm_lpr(N, dtype == 0 ? 4 : 2);
   if (lpr == 0) return -3;
   if (rows == 0) return 0;
   hipStream_t st = (hipStream_t)stream;
   if (dtype == 0) {
-#define CALL(L_) rmsnorm_fwd_launch<float, float, L_>(x, gate, weight, y, rstd, rows, eps, st)
+#define CALL(L_) rmsnorm_fwd_launch<float, float, L_>(x, gate, weight, y, rstd, rows, eps, gate_activation, st)
     GDN_RMS_DISPATCH(CALL)
 #undef CALL
   } else if (weight_dtype == 1) {
-#define CALL(L_) rmsnorm_fwd_launch<bf16_t, bf16_t, L_>(x, gate, weight, y, rstd, rows, eps, st)
+#define CALL(L_) rmsnorm_fwd_launch<bf16_t, bf16_t, L_>(x, gate, weight, y, rstd, rows, eps, gate_activation, st)
     GDN_RMS_DISPATCH(CALL)
 #undef CALL
   } else {
-#define CALL(L_) rmsnorm_fwd_launch<bf16_t, float, L_>(x, gate, weight, y, rstd, rows, eps, st)
+#define CALL(L_) rmsnorm_fwd_launch<bf16_t, float, L_>(x, gate, weight, y, rstd, rows, eps, gate_activation, st)
     GDN_RMS_DISPATCH(CALL)
 #undef CALL
   }
@@ -197,12 +210,13 @@ extern "C" int64_t gdn_rmsnorm_gated_bwd_workspace_bytes(int64_t rows, int N) {
 extern "C" int gdn_rmsnorm_gated_bwd(const void* x, const void* gate, const void* weight, const float* rstd,
                                      const void* dy, void* dx, void* dgate, float* dweight, void* workspace,
                                      int64_t workspace_bytes, int64_t rows, int N, int dtype, int weight_dtype,
-                                     void* stream) {
+                                     int gate_activation, void* stream) {
   using namespace gdn;
   if (!x || !gate || !weight || !rstd || !dy || !dx || !dgate || !dweight || !workspace) return -1;
   if (rows < 0) return -2;
   if (dtype != 0 && dtype != 1) return -4;
   if (weight_dtype != 0 && weight_dtype != dtype) return -4;
+  if (gate_activation != 0 && gate_activation != 1) return -4;
   const int lpr = rmsnorm_lpr(N, dtype == 0 ? 4 : 2);
   if (lpr == 0) return -3;
   if (workspace_bytes < gdn_rmsnorm_gated_bwd_workspace_bytes(rows, N)) return -5;
@@ -214,15 +228,15 @@ extern "C" int gdn_rmsnorm_gated_bwd(const void* x, const void* gate, const void
     return (int)hipGetLastError();
   }
   if (dtype == 0) {
-#define CALL(L_) rmsnorm_bwd_launch<float, float, L_>(x, gate, weight, rstd, dy, dx, dgate, dweight, part, rows, st)
+#define CALL(L_) rmsnorm_bwd_launch<float, float, L_>(x, gate, weight, rstd, dy, dx, dgate, dweight, part, rows, gate_activation, st)
     GDN_RMS_DISPATCH(CALL)
 #undef CALL
   } else if (weight_dtype == 1) {
-#define CALL(L_) rmsnorm_bwd_launch<bf16_t, bf16_t, L_>(x, gate, weight, rstd, dy, dx, dgate, dweight, part, rows, st)
+#define CALL(L_) rmsnorm_bwd_launch<bf16_t, bf16_t, L_>(x, gate, weight, rstd, dy, dx, dgate, dweight, part, rows, gate_activation, st)
     GDN_RMS_DISPATCH(CALL)
 #undef CALL
   } else {
-#define CALL(L_) rmsnorm_bwd_launch<bf16_t, float, L_>(x, gate, weight, rstd, dy, dx, dgate, dweight, part, rows, st)
+#define CALL(L_) rmsnorm_bwd_launch<bf16_t, float, L_>(x, gate, weight, rstd, dy, dx, dgate, dweight, part, rows, gate_activation, st)
     GDN_RMS_DISPATCH(CALL)
 #undef CALL
   }

@@ -26,9 +26,9 @@ SIGNATURES = {
     "gdn_conv1d_bwd_workspace_bytes": (L, [I] * 4),
     "gdn_conv1d_bwd": (I, [P] * 12 + [L] + [I] * 7 + [P]),
     "gdn_conv1d_update": (I, [P] * 5 + [I] * 7 + [P]),
-    "gdn_rmsnorm_gated_fwd": (I, [P] * 5 + [L, I, F, I, I, P]),
+    "gdn_rmsnorm_gated_fwd": (I, [P] * 5 + [L, I, F, I, I, I, P]),
     "gdn_rmsnorm_gated_bwd_workspace_bytes": (L, [L, I]),
-    "gdn_rmsnorm_gated_bwd": (I, [P] * 9 + [L, L, I, I, I, P]),
+    "gdn_rmsnorm_gated_bwd": (I, [P] * 9 + [L, L, I, I, I, I, P]),
     "gdn_gate_fwd": (I, [P] * 6 + [L, I, I, I, P]),
     "gdn_gate_bwd_workspace_bytes": (L, [L, I]),
     "gdn_gate_bwd": (I, [P] * 11 + [L, L, I, I, I, P]),

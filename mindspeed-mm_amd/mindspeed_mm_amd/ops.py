@@ -418,11 +418,13 @@ class GdnOps:
         return out
 
     # ------------------------------------------------------------------ gated RMSNorm
-    def rms_norm_gated(self, hidden_states, gate, weight, eps=1e-6):
+    def rms_norm_gated(self, hidden_states, gate, weight, eps=1e-6, activation="silu"):
         if gate is None:
             raise ValueError("rms_norm_gated needs a gate (the reference layer always passes one)")
+        if activation not in _GATE_ACTIVATION:
+            raise ValueError(f"gate activation {activation!r}: 'silu' (Qwen3_5RMSNormGated) or 'sigmoid' (KimiK_3_MoeRMSNormGated)")
         self._need(hidden_states, gate, weight)
-        return _RMSNormGated.apply(hidden_states, gate, weight, eps, self)
+        return _RMSNormGated.apply(hidden_states, gate, weight, eps, self, _GATE_ACTIVATION[activation])
 
 
 def _i64(cu, ref):
@@ -579,7 +581,7 @@ class _ChunkGatedDeltaRuleNorm(torch.autograd.Function):
         nb = lib.gdn_rmsnorm_gated_bwd_workspace_bytes(rows, V)
         nws = torch.empty(nb, dtype=torch.uint8, device=dev)
         rc = lib.gdn_rmsnorm_gated_bwd(ptr(o), ptr(gc), ptr(wc), ptr(rstd), ptr(dyc), ptr(do), ptr(dgate), ptr(dw),
-                                       ptr(nws), nb, rows, V, code, DTYPE_CODE[w_dt], lib.stream())
+                                       ptr(nws), nb, rows, V, code, DTYPE_CODE[w_dt], 0, lib.stream())
         lib.check(rc, "gdn_rmsnorm_gated_bwd")
         dq = dk = dv = dg = db = dh0 = None
         if rule_grad:
@@ -824,13 +826,16 @@ class _CausalConv1d(torch.autograd.Function):
                 None if dh0 is None else dh0.to(h_dt), None, None, None, None)
 
 
+_GATE_ACTIVATION = {"silu": 0, "swish": 0, "sigmoid": 1}
+
+
 class _RMSNormGated(torch.autograd.Function):
-    """y = (weight * rmsnorm(x)) * silu(gate) over the last axis."""
+    """y = (weight * rmsnorm(x)) * act(gate) over the last axis, act = silu (code 0) or sigmoid (code 1)."""
 
     @staticmethod
     @_input_guard
     @_custom_fwd
-    def forward(ctx, x, gate, weight, eps, ops):
+    def forward(ctx, x, gate, weight, eps, ops, act=0):
         lib = ops.lib
         dt = x.dtype
         if dt not in (torch.float32, torch.bfloat16):
@@ -848,10 +853,10 @@ class _RMSNormGated(torch.autograd.Function):
         y = torch.empty_like(xc)
         rstd = torch.empty(rows, dtype=torch.float32, device=x.device)
         code = lib.gdn_rmsnorm_gated_fwd(ptr(xc), ptr(gc), ptr(wc), ptr(y), ptr(rstd), rows, N, float(eps),
-                                         DTYPE_CODE[dt], DTYPE_CODE[w_dt], lib.stream())
+                                         DTYPE_CODE[dt], DTYPE_CODE[w_dt], act, lib.stream())
         lib.check(code, "gdn_rmsnorm_gated_fwd")
         ctx.save_for_backward(xc, gc, wc, rstd)
-        ctx.meta = (rows, N, dt, w_dt, weight.dtype, gate.dtype, x.shape)
+        ctx.meta = (rows, N, dt, w_dt, weight.dtype, gate.dtype, x.shape, act)
         ctx.ops = ops
         return y.view(x.shape)
 
@@ -860,7 +865,7 @@ class _RMSNormGated(torch.autograd.Function):
     @_custom_bwd
     def backward(ctx, dy):
         xc, gc, wc, rstd = ctx.saved_tensors
-        rows, N, dt, w_dt, weight_dt, gate_dt, shape = ctx.meta
+        rows, N, dt, w_dt, weight_dt, gate_dt, shape, act = ctx.meta
         lib = ctx.ops.lib
         dyc = dy.to(dt).contiguous().view(-1, N)
         dx = torch.empty_like(xc)
@@ -869,9 +874,9 @@ class _RMSNormGated(torch.autograd.Function):
         nbytes = lib.gdn_rmsnorm_gated_bwd_workspace_bytes(rows, N)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=xc.device)
         code = lib.gdn_rmsnorm_gated_bwd(ptr(xc), ptr(gc), ptr(wc), ptr(rstd), ptr(dyc), ptr(dx), ptr(dg), ptr(dw),
-                                         ptr(ws), nbytes, rows, N, DTYPE_CODE[dt], DTYPE_CODE[w_dt], lib.stream())
+                                         ptr(ws), nbytes, rows, N, DTYPE_CODE[dt], DTYPE_CODE[w_dt], act, lib.stream())
         lib.check(code, "gdn_rmsnorm_gated_bwd")
-        return dx.view(shape), dg.view(shape).to(gate_dt), dw.to(weight_dt), None, None
+        return dx.view(shape), dg.view(shape).to(gate_dt), dw.to(weight_dt), None, None, None
 
 
 # ---------------------------------------------------------------------- module-level entry points
@@ -998,22 +1003,28 @@ def causal_conv1d_update(hidden_states, conv_state, weight, bias=None, activatio
 
 
 @torch.compiler.disable
-def rms_norm_gated(hidden_states, gate, weight, eps=1e-6):
+def rms_norm_gated(hidden_states, gate, weight, eps=1e-6, activation="silu"):
     """Functional form of Qwen3_5RMSNormGated.forward (modeling_qwen3_5.py:341-349):
-    (weight * rmsnorm(hidden_states)) * silu(gate) over the last axis, in the input dtype."""
-    return _default_ops().rms_norm_gated(hidden_states, gate, weight, eps)
+    (weight * rmsnorm(hidden_states)) * silu(gate) over the last axis, in the input dtype; with activation="sigmoid"
+    that of KimiK_3_MoeRMSNormGated.forward (modeling_kimi_linear.py:83-96), whose gate passes through a sigmoid."""
+    return _default_ops().rms_norm_gated(hidden_states, gate, weight, eps, activation)
 
 
 class RMSNormGated(torch.nn.Module):
-    """Drop-in for Qwen3_5RMSNormGated (modeling_qwen3_5.py:330-349): same constructor, parameter and forward."""
+    """Drop-in for Qwen3_5RMSNormGated (modeling_qwen3_5.py:330-349) and, constructed with activation="sigmoid" as the
+    KDA layer constructs its norm (modeling_kimi_linear.py:603-604), for KimiK_3_MoeRMSNormGated (:75-96): same
+    constructor, parameter and forward."""
 
-    def __init__(self, hidden_size, eps=1e-6, **kwargs):
+    def __init__(self, hidden_size, eps=1e-6, activation="silu", **kwargs):
         super().__init__()
+        if activation not in _GATE_ACTIVATION:
+            raise ValueError(f"gate activation {activation!r}: 'silu' or 'sigmoid'")
         self.weight = torch.nn.Parameter(torch.ones(hidden_size))
         self.variance_epsilon = eps
+        self.activation = activation
 
     def forward(self, hidden_states, gate=None):
-        return rms_norm_gated(hidden_states, gate, self.weight, self.variance_epsilon)
+        return rms_norm_gated(hidden_states, gate, self.weight, self.variance_epsilon, self.activation)
 
 
 class ShortConvolution(torch.nn.Conv1d):

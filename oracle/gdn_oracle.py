@@ -340,6 +340,21 @@ def rms_norm_gated_ref(hidden_states: torch.Tensor, gate: torch.Tensor, weight: 
     return x.to(input_dtype)
 
 
+def rms_norm_sigmoid_gated_ref(hidden_states: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor,
+                               eps: float = 1e-6) -> torch.Tensor:
+    """KimiK_3_MoeRMSNormGated.forward, the branch without NPU operators (mindspeed_mm/fsdp/models/kimi_k3/
+    modeling_kimi_linear.py:89-94): normalise in fp32, cast back to the input dtype, scale by ``weight``, multiply with
+    ``sigmoid(gate)`` taken in fp32 and cast to the input dtype.  The reference leaves the product in the promoted dtype
+    of weight and input; the operator returns the input dtype, so does this.  Differentiable."""
+    input_dtype = hidden_states.dtype
+    x = hidden_states.to(torch.float32)
+    variance = x.pow(2).mean(-1, keepdim=True)
+    x = x * torch.rsqrt(variance + eps)
+    x = weight * x.to(input_dtype)
+    x = x * torch.sigmoid(gate.to(torch.float32)).to(input_dtype)
+    return x.to(input_dtype)
+
+
 def gdn_gates_ref(a: torch.Tensor, b: torch.Tensor, A_log: torch.Tensor,
                   dt_bias: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """(g, beta) as Qwen3_5GatedDeltaNet.forward forms them (modeling_qwen3_5.py:833-841, the branch without sequence

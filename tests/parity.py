@@ -177,7 +177,8 @@ def check_conv_update(ops, device, B, T, D, W, dtype, seed=0, wrap=lambda t: t, 
     return {"y": _err("y", y, ry, dtype, 1e-2, 1e-2), "state": _err("state", st_dev, st_ref, dtype, 1e-2, 1e-2)}
 
 
-def check_rms_norm_gated(ops, device, rows_shape, N, dtype, weight_dtype=None, seed=0, backward=True, wrap=lambda t: t):
+def check_rms_norm_gated(ops, device, rows_shape, N, dtype, weight_dtype=None, seed=0, backward=True, wrap=lambda t: t,
+                         activation="silu"):
     """Gated RMSNorm against the oracle on the same (dtype-valued) inputs.  Half precision: the outputs are O(1)
     products of values rounded to bf16 several times on both sides, compared with |err| <= atol + rtol |ref|."""
     gen = torch.Generator().manual_seed(seed)
@@ -187,16 +188,17 @@ def check_rms_norm_gated(ops, device, rows_shape, N, dtype, weight_dtype=None, s
              w=(1.0 + 0.2 * r(N)).to(weight_dtype), dy=r(*rows_shape, N).to(dtype))
     dev = {n: wrap(t.to(device)) for n, t in x.items()}
     L = {n: dev[n].clone().requires_grad_(backward) for n in ("x", "g", "w")}
-    y = ops.rms_norm_gated(L["x"], L["g"], L["w"], 1e-6)
+    ref = O.rms_norm_gated_ref if activation == "silu" else O.rms_norm_sigmoid_gated_ref
+    y = ops.rms_norm_gated(L["x"], L["g"], L["w"], 1e-6, activation)
     R = {n: x[n].clone().requires_grad_(backward) for n in ("x", "g", "w")}
-    ry = O.rms_norm_gated_ref(R["x"], R["g"], R["w"], 1e-6)
+    ry = ref(R["x"], R["g"], R["w"], 1e-6)
     assert y.shape == ry.shape and y.dtype == dtype
     errs = {"y": _err("y", y, ry, dtype, 2e-2, rtol=1e-2)}
     if backward:
         y.backward(dev["dy"])
         # the oracle's own autograd in half precision rounds every intermediate; differentiate its fp32 form instead
         R32 = {n: x[n].float().clone().requires_grad_(True) for n in ("x", "g", "w")}
-        O.rms_norm_gated_ref(R32["x"], R32["g"], R32["w"], 1e-6).backward(x["dy"].float())
+        ref(R32["x"], R32["g"], R32["w"], 1e-6).backward(x["dy"].float())
         for n, m in (("x", "dx"), ("g", "dgate")):
             assert L[n].grad.dtype == dtype
             errs[m] = _err(m, L[n].grad, R32[n].grad, dtype, 5e-2, rtol=2e-2)

@@ -95,6 +95,11 @@ def test_rms_norm_gated(ops, dtype, shape, N, wdt):
     P.check_rms_norm_gated(ops, "cpu", shape, N, dtype, weight_dtype=wdt, wrap=guarded)
 
 
+@pytest.mark.parametrize("dtype,shape,N,wdt", [(F32, (3, 5), 64, None), (BF, (70,), 128, None), (BF, (2, 9), 128, torch.float32)])
+def test_rms_norm_sigmoid_gated(ops, dtype, shape, N, wdt):
+    P.check_rms_norm_gated(ops, "cpu", shape, N, dtype, weight_dtype=wdt, wrap=guarded, activation="sigmoid")
+
+
 @pytest.mark.parametrize("dtype,B,T,Hqk,Hv,K,V,l2,cu,pad", [
     (F32, 1, 100, 1, 2, 64, 64, True, None, 0),
     (BF, 2, 70, 2, 4, 128, 128, True, None, 0),

@@ -183,6 +183,17 @@ def test_rms_norm_gated(ops, dtype, shape, N, wdt):
     P.check_rms_norm_gated(ops, "cuda", shape, N, dtype, weight_dtype=wdt)
 
 
+@pytest.mark.parametrize("dtype,shape,N,wdt", [(F32, (3, 5), 64, None), (BF, (2, 70, 3), 128, None), (BF, (9,), 128, torch.float32)])
+def test_rms_norm_sigmoid_gated(ops, dtype, shape, N, wdt):
+    """The KDA layer's norm (KimiK_3_MoeRMSNormGated, modeling_kimi_linear.py:75-96), forward and backward."""
+    errs = P.check_rms_norm_gated(ops, "cuda", shape, N, dtype, weight_dtype=wdt, activation="sigmoid")
+    print("   ", {n: f"{e:.2e}" for n, e in errs.items()}, flush=True)
+    import mindspeed_mm_amd as M
+    norm = M.RMSNormGated(N, eps=1e-6, activation="sigmoid").cuda()        # as the layer constructs it (:603-604)
+    x, g = torch.randn(4, N, device="cuda", dtype=dtype), torch.randn(4, N, device="cuda", dtype=dtype)
+    assert torch.equal(norm(x, g), ops.rms_norm_gated(x, g, norm.weight, 1e-6, "sigmoid"))
+
+
 def test_rms_norm_gated_module_matches_functional(ops):
     from mindspeed_mm_amd import RMSNormGated
     m = RMSNormGated(128).to("cuda", BF)

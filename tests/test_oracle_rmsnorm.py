@@ -68,3 +68,43 @@ def test_gradcheck_float64():
     fn(*args).backward(dy.double())
     for p, q in zip(a32, args):
         assert torch.allclose(p.grad.double(), q.grad, rtol=1e-4, atol=1e-5)
+
+
+# ---- the KDA layer's norm: sigmoid gate (KimiK_3_MoeRMSNormGated.forward, modeling_kimi_linear.py:89-94)
+def test_sigmoid_gated_matches_library_rms_norm_times_sigmoid():
+    x, g, w = _inputs(37, 128)
+    ref = F.rms_norm(x, (128,), w, eps=1e-6) * torch.special.expit(g)
+    got = O.rms_norm_sigmoid_gated_ref(x.float(), g.float(), w.float()).double()
+    assert torch.allclose(got, ref, rtol=2e-6, atol=2e-6)
+
+
+def test_sigmoid_gated_limits_of_the_gate():
+    # gate = 0 halves the normalised row; a wide open gate (sigmoid -> 1) leaves it; a closed one removes it
+    x, _, w = _inputs(6, 64, torch.float32, seed=2)
+    plain = F.rms_norm(x, (64,), w, eps=1e-6)
+    assert torch.allclose(O.rms_norm_sigmoid_gated_ref(x, torch.zeros_like(x), w), 0.5 * plain, rtol=1e-6, atol=1e-7)
+    assert torch.allclose(O.rms_norm_sigmoid_gated_ref(x, torch.full_like(x, 40.0), w), plain, rtol=1e-6, atol=1e-7)
+    assert O.rms_norm_sigmoid_gated_ref(x, torch.full_like(x, -120.0), w).abs().max() == 0
+    # and the two gated norms differ by exactly the factor gate: silu(g) = g sigmoid(g)
+    g = torch.linspace(-3, 3, 64).expand(6, 64)
+    assert torch.allclose(O.rms_norm_gated_ref(x, g, w), g * O.rms_norm_sigmoid_gated_ref(x, g, w), rtol=1e-5, atol=1e-6)
+
+
+def test_sigmoid_gated_half_precision_casts_follow_the_reference_order():
+    # bf16: normalised row rounded, weighted row rounded (weight in bf16), the sigmoid rounded to bf16 before the product
+    x, g, w = _inputs(5, 128, torch.bfloat16, seed=3)
+    xn = (x.float() * torch.rsqrt(x.float().pow(2).mean(-1, keepdim=True) + 1e-6)).to(torch.bfloat16)
+    expect = (w * xn) * torch.sigmoid(g.float()).to(torch.bfloat16)
+    assert expect.dtype == torch.bfloat16 and torch.equal(O.rms_norm_sigmoid_gated_ref(x, g, w), expect)
+
+
+def test_sigmoid_gated_gradient_against_the_silu_form():
+    # d/dg of t sigmoid(g) from the pinned silu form: t silu(g) = g (t sigmoid(g))  =>  d(silu form)/dg = y + g dy/dg
+    x, g, w = _inputs(4, 32, torch.float32, seed=5)
+    g1 = g.clone().requires_grad_(True)
+    y = O.rms_norm_sigmoid_gated_ref(x, g1, w)
+    dy_dg, = torch.autograd.grad(y.sum(), g1)
+    g2 = g.clone().requires_grad_(True)
+    ds_dg, = torch.autograd.grad(O.rms_norm_gated_ref(x, g2, w).sum(), g2)
+    assert torch.allclose(ds_dg, y.detach() + g * dy_dg, rtol=1e-5, atol=1e-6)
+
