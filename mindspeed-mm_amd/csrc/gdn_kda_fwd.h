@@ -161,67 +161,82 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
   }
   GDN_LDS_BARRIER();
 
-  // ---- phase 1: L and Aq level by level on the matrix cores.  Wave w: matrix w & 1 (0: k k^T, 1: q k^T), diagonal
-  //      tile w >> 1; the tile below the diagonal (level 64) goes to waves 0 and 1 ----
-  const int mat = wave & 1, td = wave >> 1, l32 = lane & 31, half = lane >> 5;
-  constexpr int KGL = KGroup<T>::kLen, NKG = DK / KGL;
-  // All levels advance together through the channels: the rows of k, q and G are read once per group of channels and
-  // only the reference row of G differs from level to level; the products of the levels are independent chains.
-  f32x16 lv[5], a_dg = acc_zero(), a_low = acc_zero();
-#pragma unroll
-  for (int i = 0; i < 5; ++i) lv[i] = acc_zero();
+  // ---- phase 1: L and Aq level by level on the matrix cores.  Wave w: diagonal tile w >> 1 of both matrices (k k^T and
+  //      q k^T share every rescaling factor, the costly part) over half w & 1 of the channel groups; the tile below
+  //      the diagonal (level 64) goes to waves 0 and 1.  The halves are added in phase 1d. ----
+  const int kh = wave & 1, td = wave >> 1, l32 = lane & 31, half = lane >> 5;
+  constexpr int KGL = KGroup<T>::kLen, NKG = DK / KGL, NKH = NKG / 2;
+  static_assert(NKG % 2 == 0, "two halves of the channel groups");
   const int R = 32 * td + l32;
+  // the levels' entries, each kept where its level owns the pair: tile (td, td) of k k^T and of q k^T, and the tile below
+  f32x16 dgk = acc_zero(), dgq = acc_zero(), lowk = acc_zero(), lowq = acc_zero();
+  // One pass over this wave's channel groups for the levels [I0, I0 + NI) (blocks of 2 << level tokens), all of them
+  // advancing together: the rows of k, q and G are read once per group and only the reference row of G differs from
+  // level to level; the products of the levels are independent chains.  Two passes (three levels and the undecayed
+  // diagonal of q k^T, then two levels and level 64): the accumulators of all levels of both matrices at once would
+  // not fit the registers that two workgroups per CU leave a wave.
+  auto level_pass = [&](auto i0_c, auto ni_c, auto diag_c, auto low_c) {
+    constexpr int I0 = decltype(i0_c)::value, NI = decltype(ni_c)::value;
+    constexpr bool DIAG = decltype(diag_c)::value != 0, LOW = decltype(low_c)::value != 0;
+    f32x16 ak[NI], aq[NI], adg = acc_zero();
+#pragma unroll
+    for (int i = 0; i < NI; ++i) { ak[i] = acc_zero(); aq[i] = acc_zero(); }
 #pragma unroll 1
-  for (int kg = 0; kg < NKG; ++kg) {
-    const int c0 = kg * KGL + half * VEC;
-    float fk[VEC], fa[VEC], gR[VEC];
-    unpack16<T>(ld16(Ks + R * LDK + c0), fk);
-    if (mat) unpack16<T>(ld16(Qs + R * LDK + c0), fa);
-    else {
+    for (int kg = kh * NKH; kg < (kh + 1) * NKH; ++kg) {
+      const int c0 = kg * KGL + half * VEC;
+      float fk[VEC], fq[VEC], gR[VEC];
+      unpack16<T>(ld16(Ks + R * LDK + c0), fk);
+      unpack16<T>(ld16(Qs + R * LDK + c0), fq);
+      ld_f32<VEC>(Gs + R * LDG + c0, gR);
+      if (DIAG) mfma_kgroup<T>(adg, pack16<T>(fq).raw, pack16<T>(fk).raw);   // the diagonal of q k^T: no decay
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) fa[e] = fk[e];
-    }
-    ld_f32<VEC>(Gs + R * LDG + c0, gR);
-    if (mat) mfma_kgroup<T>(a_dg, pack16<T>(fa).raw, pack16<T>(fk).raw);   // the diagonal of q k^T: no decay
+      for (int i = 0; i < NI; ++i) {   // rows of the second half of a block against rows of its first half
+        const int n = 2 << (I0 + i), m = (R / n) * n + n / 2;
+        float gm[VEC], xq[VEC], xk[VEC];
+        ld_f32<VEC>(Gs + m * LDG + c0, gm);
 #pragma unroll
-    for (int i = 0; i < 5; ++i) {   // blocks of n = 2 << i tokens: rows of the second half against rows of the first
-      const int n = 2 << i, m = (R / n) * n + n / 2;
-      float gm[VEC], xa[VEC], xb[VEC];
-      ld_f32<VEC>(Gs + m * LDG + c0, gm);
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        const float f = __expf(-fabsf(gR[e] - gm[e]));
-        xa[e] = fa[e] * f;
-        xb[e] = fk[e] * f;
+        for (int e = 0; e < VEC; ++e) {
+          const float f = __expf(-fabsf(gR[e] - gm[e]));
+          xq[e] = fq[e] * f;
+          xk[e] = fk[e] * f;
+        }
+        const u32x4 bK = pack16<T>(xk).raw;
+        mfma_kgroup<T>(ak[i], bK, bK);
+        mfma_kgroup<T>(aq[i], pack16<T>(xq).raw, bK);
       }
-      const u32x4 afrag = pack16<T>(xa).raw;
-      mfma_kgroup<T>(lv[i], afrag, mat ? pack16<T>(xb).raw : afrag);
-    }
-    if (wave < 2) {   // level 64: tokens 32..63 against 0..31 (these waves' rows R), all entries kept
-      float gm[VEC], ga[VEC], xa[VEC], xb[VEC];
-      ld_f32<VEC>(Gs + 32 * LDG + c0, gm);
-      ld_f32<VEC>(Gs + (32 + l32) * LDG + c0, ga);
-      unpack16<T>(ld16((mat ? Qs : Ks) + (32 + l32) * LDK + c0), xa);
+      if (LOW && wave < 2) {   // level 64: tokens 32..63 against 0..31 (these waves' rows R), all entries kept
+        float gm[VEC], ga[VEC], xk2[VEC], xq2[VEC], xb[VEC];
+        ld_f32<VEC>(Gs + 32 * LDG + c0, gm);
+        ld_f32<VEC>(Gs + (32 + l32) * LDG + c0, ga);
+        unpack16<T>(ld16(Ks + (32 + l32) * LDK + c0), xk2);
+        unpack16<T>(ld16(Qs + (32 + l32) * LDK + c0), xq2);
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        xa[e] *= __expf(-fabsf(ga[e] - gm[e]));
-        xb[e] = fk[e] * __expf(-fabsf(gR[e] - gm[e]));
+        for (int e = 0; e < VEC; ++e) {
+          const float fa = __expf(-fabsf(ga[e] - gm[e]));
+          xk2[e] *= fa;
+          xq2[e] *= fa;
+          xb[e] = fk[e] * __expf(-fabsf(gR[e] - gm[e]));
+        }
+        const u32x4 bK = pack16<T>(xb).raw;
+        mfma_kgroup<T>(lowk, pack16<T>(xk2).raw, bK);
+        mfma_kgroup<T>(lowq, pack16<T>(xq2).raw, bK);
       }
-      mfma_kgroup<T>(a_low, pack16<T>(xa).raw, pack16<T>(xb).raw);
     }
-  }
-  f32x16 a_diag;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int i = acc_row(r), j = l32;
-    float x = (mat == 1 && i == j) ? a_dg[r] : 0.f;
+    for (int r = 0; r < 16; ++r) {
+      const int i = acc_row(r), j = l32;
 #pragma unroll
-    for (int q2 = 0; q2 < 5; ++q2) {
-      const int n = 2 << q2;
-      x += ((i / n == j / n) && (i % n >= n / 2) && (j % n < n / 2)) ? lv[q2][r] : 0.f;
+      for (int q2 = 0; q2 < NI; ++q2) {
+        const int n = 2 << (I0 + q2);
+        const bool keep = (i / n == j / n) && (i % n >= n / 2) && (j % n < n / 2);
+        dgk[r] += keep ? ak[q2][r] : 0.f;
+        dgq[r] += keep ? aq[q2][r] : 0.f;
+      }
+      if (DIAG) dgq[r] += i == j ? adg[r] : 0.f;
     }
-    a_diag[r] = x;
-  }
+  };
+  level_pass(IntConst<0>(), IntConst<3>(), IntConst<1>(), IntConst<0>());
+  level_pass(IntConst<3>(), IntConst<2>(), IntConst<0>(), IntConst<1>());
   GDN_LDS_BARRIER();   // every wave is done with q as it lies: its place becomes the staging tile
 
   // ---- phase 1c: what the recurrence reads, through a row-major staging tile (the q rows' place) into fragment order:
@@ -288,17 +303,24 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
   // ---- phase 1d: L and Aq as 64x64 fp32 matrices ----
   for (int i = tid; i < 64 * kLF; i += kThreads) { As[i] = 0.f; Aqs[i] = 0.f; Ti[i] = 0.f; }
   GDN_LDS_BARRIER();
+  // each entry is the sum of the two waves that share a tile (one per half of the channels): they add one after the other
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int i = 32 * td + acc_row(r), j = 32 * td + l32;
-    if (mat == 0) As[i * kLF + j] = i > j ? bs[i] * a_diag[r] : 0.f;
-    else Aqs[i * kLF + j] = i >= j ? scale * a_diag[r] : 0.f;
-    if (wave < 2) {
-      const int i2 = 32 + acc_row(r);
-      if (mat == 0) As[i2 * kLF + l32] = bs[i2] * a_low[r]; else Aqs[i2 * kLF + l32] = scale * a_low[r];
+  for (int turn = 0; turn < 2; ++turn) {
+    if (kh == turn) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int i = 32 * td + acc_row(r), j = 32 * td + l32;
+        As[i * kLF + j] += i > j ? bs[i] * dgk[r] : 0.f;
+        Aqs[i * kLF + j] += i >= j ? scale * dgq[r] : 0.f;
+        if (wave < 2) {
+          const int i2 = 32 + acc_row(r);
+          As[i2 * kLF + l32] += bs[i2] * lowk[r];
+          Aqs[i2 * kLF + l32] += scale * lowq[r];
+        }
+      }
     }
+    GDN_LDS_BARRIER();
   }
-  GDN_LDS_BARRIER();
   {  // Aq leaves as four tiles packed as they sit in an accumulator (lane <-> column j, registers <-> row i)
     const int ti = wave >> 1, tj = wave & 1;
     f32x16 aq;
