@@ -234,3 +234,69 @@ def test_config4_long_sequence_wide_heads(ops):
                                                use_qk_l2norm_in_kernel=True)
     _err("o", o[:, :, hs], ro, BF, BF16_ABS_O)
     _err("final_state", ht[:, hs], rht, BF, BF16_ABS_GRAD)
+
+
+def test_kda_full_size(ops):
+    """The KDA benchmark shape (B=2, T=8192, H=32, d=128, bf16, the layer's options) forward and backward: split-run
+    continuity, exact linearity, and the oracle on one head (heads are independent; the gradients of A_log and dt_bias of
+    a head sum over the batch rows, which the slice keeps both of)."""
+    from mindspeed_mm_amd.inputs import kda_inputs
+    from oracle import kda_oracle as KO
+    from parity import KDA_PARAM_RTOL
+    B, T, H, K, V = 2, 8192, 32, 128, 128
+    x = kda_inputs(B, T, H, K, V, BF, seed=11)
+    x["h0"], x["dht"] = (x[n].transpose(-1, -2).contiguous() for n in ("h0", "dht"))     # [N,H,V,K] as the layer keeps them
+    d = {n: t.cuda() for n, t in x.items()}
+    names = ("q", "k", "v", "g", "beta", "A_log", "dt_bias", "h0")
+    kw = dict(output_final_state=True, use_qk_l2norm_in_kernel=True, use_gate_in_kernel=True,
+              use_beta_sigmoid_in_kernel=True, transpose_state_layout=True)
+
+    def run(t, h0, backward=False, do=None, dht=None):
+        L = {n: t[n].clone().requires_grad_(backward) for n in names[:-1]}
+        h = h0.clone().requires_grad_(backward)
+        with torch.set_grad_enabled(backward):
+            o, ht = ops.chunk_kda(L["q"], L["k"], L["v"], L["g"], L["beta"], initial_state=h, A_log=L["A_log"],
+                                  dt_bias=L["dt_bias"], **kw)
+        if not backward:
+            return o, ht
+        grads = torch.autograd.grad([o, ht], [L[n] for n in names[:-1]] + [h], [do, dht])
+        return o, ht, dict(zip(names, grads))
+
+    o, ht, gr = run(d, d["h0"], True, d["do"], d["dht"])
+    assert torch.isfinite(o.float()).all() and torch.isfinite(ht).all()
+    assert all(torch.isfinite(g.float()).all() for g in gr.values())
+
+    # split-run continuity at a chunk boundary: every chunk sees the same operands
+    tok = ("q", "k", "v", "g", "beta")
+    half = dict(d, **{n: d[n][:, :T // 2].contiguous() for n in tok})
+    rest = dict(d, **{n: d[n][:, T // 2:].contiguous() for n in tok})
+    o1, s1 = run(half, d["h0"])
+    o2, s2 = run(rest, s1)
+    assert torch.equal(torch.cat([o1, o2], 1), o) and torch.equal(s2, ht)
+
+    # linear in (v, h0) forward and in (dO, dht) backward: a factor of two is exact
+    o_2, ht_2 = run(dict(d, v=d["v"] * 2), d["h0"] * 2)
+    assert torch.equal(o_2, o * 2) and torch.equal(ht_2, ht * 2)
+    _, _, gr2 = run(d, d["h0"], True, d["do"] * 2, d["dht"] * 2)
+    for n in gr:
+        assert torch.equal(gr2[n], gr[n] * 2), n
+
+    # the oracle on head hs of both batch rows, all 128 chunks
+    hs = 7
+    R = {n: x[n][:, :, hs:hs + 1].clone().requires_grad_(True) for n in tok}
+    R["A_log"] = x["A_log"][hs:hs + 1].clone().requires_grad_(True)
+    R["dt_bias"] = x["dt_bias"][hs * K:(hs + 1) * K].clone().requires_grad_(True)
+    R["h0"] = x["h0"][:, hs:hs + 1].clone().requires_grad_(True)
+    ro, rht = KO.chunk_kda_ref(R["q"], R["k"], R["v"], R["g"], R["beta"], initial_state=R["h0"], A_log=R["A_log"],
+                               dt_bias=R["dt_bias"], round_output=False, **kw)
+    rg = torch.autograd.grad([ro, rht], [R[n] for n in names], [x["do"][:, :, hs:hs + 1].float(), x["dht"][:, hs:hs + 1]])
+    rg = dict(zip(names, rg))
+    _err("o", o[:, :, hs:hs + 1], ro, BF, BF16_ABS_O)
+    _err("final_state", ht[:, hs:hs + 1], rht, BF, BF16_ABS_GRAD)
+    for n in tok:
+        _err("d" + n, gr[n][:, :, hs:hs + 1], rg[n], BF, BF16_ABS_GRAD)
+    _err("dh0", gr["h0"][:, hs:hs + 1], rg["h0"], BF, BF16_ABS_GRAD)
+    ptol = BF16_ABS_GRAD * (B * T / 64.0) ** 0.5
+    _err("dA_log", gr["A_log"][hs:hs + 1], rg["A_log"], BF, ptol, rtol=KDA_PARAM_RTOL)
+    _err("ddt_bias", gr["dt_bias"][hs * K:(hs + 1) * K], rg["dt_bias"], BF, ptol, rtol=KDA_PARAM_RTOL)
+
