@@ -17,8 +17,17 @@ BF16_ABS_O = 2e-2
 BF16_ABS_GRAD = 5e-2
 # dA_log and d(dt_bias) are sums over every token of the batch (dA_log over the channels too) of terms of both signs,
 # each within the bound above: the error of the sum grows like a random walk, with the square root of the number of
-# chunks, while the sum itself may cancel; 2 % of the reference on top
+# chunks, while the sum itself may cancel; 2 % on top, of the largest entry of the reference (the heads and channels
+# draw their terms from one distribution, so the largest sum stands for the size of the terms also where an entry's own
+# sum has cancelled)
 KDA_PARAM_RTOL = 2e-2
+
+
+def kda_param_tol(ref_grad, tokens):
+    """Absolute bound for an entry of dA_log or d(dt_bias) in half precision.  Twice the per-entry bound per square root
+    of the number of chunks: the oracle itself, evaluated in bf16 instead of fp32 on the seeded random cases of
+    test_kda_random_shapes, moves dA_log by up to 0.2 at 400 tokens (the kernels by 0.02-0.2 on the same cases)."""
+    return 2.0 * BF16_ABS_GRAD * max(1.0, tokens / 64.0) ** 0.5 + KDA_PARAM_RTOL * ref_grad.abs().max().item()
 
 
 def _err(name, got, ref, dtype, abs_tol, rtol=0.0):
@@ -470,6 +479,5 @@ def check_kda(ops, device, B, T, H, K, V, dtype, cu=None, seed=0, with_h0=True, 
             assert leaves[n].grad.dtype == leaves[n].dtype and leaves[n].grad.shape == leaves[n].shape
             param = n in ("A_log", "dt_bias")
             errs["d" + n] = _err("d" + n, leaves[n].grad, ref[n].grad, dtype,
-                                 BF16_ABS_GRAD * (max(1.0, B * T / 64.0) ** 0.5 if param else 1.0),
-                                 rtol=KDA_PARAM_RTOL if param else 0.0)
+                                 kda_param_tol(ref[n].grad, B * T) if param else BF16_ABS_GRAD)
     return errs

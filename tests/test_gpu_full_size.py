@@ -242,7 +242,7 @@ def test_kda_full_size(ops):
     a head sum over the batch rows, which the slice keeps both of)."""
     from mindspeed_mm_amd.inputs import kda_inputs
     from oracle import kda_oracle as KO
-    from parity import KDA_PARAM_RTOL
+    from parity import kda_param_tol
     B, T, H, K, V = 2, 8192, 32, 128, 128
     x = kda_inputs(B, T, H, K, V, BF, seed=11)
     x["h0"], x["dht"] = (x[n].transpose(-1, -2).contiguous() for n in ("h0", "dht"))     # [N,H,V,K] as the layer keeps them
@@ -296,7 +296,6 @@ def test_kda_full_size(ops):
     for n in tok:
         _err("d" + n, gr[n][:, :, hs:hs + 1], rg[n], BF, BF16_ABS_GRAD)
     _err("dh0", gr["h0"][:, hs:hs + 1], rg["h0"], BF, BF16_ABS_GRAD)
-    ptol = BF16_ABS_GRAD * (B * T / 64.0) ** 0.5
-    _err("dA_log", gr["A_log"][hs:hs + 1], rg["A_log"], BF, ptol, rtol=KDA_PARAM_RTOL)
-    _err("ddt_bias", gr["dt_bias"][hs * K:(hs + 1) * K], rg["dt_bias"], BF, ptol, rtol=KDA_PARAM_RTOL)
+    _err("dA_log", gr["A_log"][hs:hs + 1], rg["A_log"], BF, kda_param_tol(rg["A_log"], B * T))
+    _err("ddt_bias", gr["dt_bias"][hs * K:(hs + 1) * K], rg["dt_bias"], BF, kda_param_tol(rg["dt_bias"], B * T))
 

@@ -499,3 +499,40 @@ def test_short_convolution_module(ops, dtype, B, T, D, W, cu):
         y2, c2 = conv(x1.cuda(), cu_seqlens=cu1)
     assert c2 is None and y2.shape == x1.shape
 
+
+def _random_kda_case(seed):
+    """A seeded random KDA problem: shape, packing and every option of the operator."""
+    import random
+    rnd = random.Random(1000 + seed)
+    dtype = rnd.choice([BF, BF, BF, F32])
+    K, V = rnd.choice([64, 128]), rnd.choice([64, 128, 192, 256])
+    H = rnd.choice([1, 2, 3, 5])
+    if rnd.random() < 0.5:
+        B, T, cu = rnd.choice([1, 2, 3]), rnd.choice([1, 17, 64, 65, 130, 200, 333]), None
+    else:
+        n = rnd.choice([1, 2, 4, 7])
+        lens = [rnd.choice([0, 1, 5, 63, 64, 65, 100, 129, 200]) for _ in range(n)]
+        if sum(lens) == 0:
+            lens[-1] = 70
+        cu = [0]
+        for x in lens:
+            cu.append(cu[-1] + x)
+        B, T = 1, cu[-1]
+    kw = dict(gate_in_kernel=rnd.random() < 0.7, beta_sigmoid=rnd.random() < 0.7, l2=rnd.random() < 0.7,
+              transpose_state=rnd.random() < 0.5, with_h0=rnd.random() < 0.7)
+    if kw["gate_in_kernel"] and rnd.random() < 0.5:
+        kw["lower_bound"] = -5.0
+    if kw["beta_sigmoid"] and rnd.random() < 0.3:
+        kw["allow_neg"] = True
+    if dtype == BF and rnd.random() < 0.3:
+        kw["g_dtype"] = torch.float32
+    return dtype, B, T, H, K, V, cu, kw
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_kda_random_shapes(ops, seed):
+    dtype, B, T, H, K, V, cu, kw = _random_kda_case(seed)
+    print(f"kda random {seed}: {dtype} B{B} T{T} H{H} K{K} V{V} cu={cu} {kw}", flush=True)
+    errs = P.check_kda(ops, "cuda", B, T, H, K, V, dtype, cu=cu, backward=True, seed=seed, **kw)
+    print("   ", {n: f"{e:.2e}" for n, e in errs.items()}, flush=True)
+
