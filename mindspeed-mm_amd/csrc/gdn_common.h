@@ -102,26 +102,19 @@ __device__ __forceinline__ int xcd_grouped_head(int b, int total, int grp) {
 #define GDN_KEEP_HERE(x) asm volatile("" : "+v"(x))
 #endif
 // The workgroups of a launch start together and, doing equal work, stay in step: they all load at the same time and
-// all compute at the same time, and the workgroups that share a CU do not fill each other's waits.  Holding back part
-// of the first resident set once shifts those workgroups, and every workgroup that later takes over one of their
-// places, for the rest of the launch.  Measured on MI355X (256 CUs; workgroup ids are handed out breadth first, so
-// ids 256..511 are the second workgroup of each CU): 3 % on the chunk-local backward kernel, 6-7 % on the KDA
-// preparation and finishing kernels, where loads and arithmetic are further apart.  The wait costs its own length once,
-// at the end of the launch, so launches of fewer than `min_groups` workgroups skip it.
-// units: 64 clock cycles (the argument of s_sleep is an immediate, at most 127).
-template <int UNITS> __device__ __forceinline__ void stagger_sleep(int times) {
-  for (int i = 0; i < times; ++i) __builtin_amdgcn_s_sleep(UNITS);
-}
+// all compute at the same time, and the two workgroups that share a CU do not fill each other's waits.  Holding back
+// the second workgroup of each CU once (workgroup ids are handed out breadth first, so on the 256 CUs of an MI355X
+// these are ids 256..511) shifts it, and every workgroup that later takes over its place, for the rest of the launch.
+// Worth 2 % on the chunk-local backward kernel, measured in alternation with the same build without the wait; nothing
+// on kernels whose phases are shorter or that run one workgroup per CU.  The wait costs its own length once, at the
+// end of the launch, so launches of fewer than `min_groups` workgroups skip it.
+// UNITS: 64 clock cycles each (the argument of s_sleep is an immediate, at most 127).
 constexpr int kStaggerCUs = 256;
-// the second workgroup of each CU waits `times` x UNITS x 64 cycles
 template <int UNITS> __device__ __forceinline__ void stagger_second_resident(int times, int min_groups) {
   const int lin = blockIdx.x + gridDim.x * blockIdx.y;
-  if ((int)(gridDim.x * gridDim.y) >= min_groups && lin >= kStaggerCUs && lin < 2 * kStaggerCUs) stagger_sleep<UNITS>(times);
-}
-// one workgroup per CU: each of the first set waits 0..15 x UNITS x 64 cycles
-template <int UNITS> __device__ __forceinline__ void stagger_first_resident(int min_groups) {
-  const int lin = blockIdx.x + gridDim.x * blockIdx.y;
-  if ((int)(gridDim.x * gridDim.y) >= min_groups && lin < kStaggerCUs) stagger_sleep<UNITS>((lin * 5) & 15);
+  if ((int)(gridDim.x * gridDim.y) >= min_groups && lin >= kStaggerCUs && lin < 2 * kStaggerCUs) {
+    for (int i = 0; i < times; ++i) __builtin_amdgcn_s_sleep(UNITS);
+  }
 }
 // Asks the scheduler for the pattern (1 matrix instruction, nvalu vector instructions) x nmfma in the current
 // scheduling region.

@@ -103,7 +103,6 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
   float* xdt = xgl + 256;   // [8][32] per wave and channel: its part of d(dt_bias)
   float* xblk = xdt + 256;  // [4][32] per channel: sum of dG over tokens 32..63
 
-  stagger_first_resident<35>(8 * kStaggerCUs);
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, wave = tid >> 6;

@@ -60,7 +60,6 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
   float* Ti = reinterpret_cast<float*>(gdn_smem + SM::off_ti);
   T* Tms = reinterpret_cast<T*>(gdn_smem + SM::off_tm);
 
-  stagger_second_resident<127>(4, 8 * kStaggerCUs);
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
