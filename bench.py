@@ -49,6 +49,9 @@ MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
 }
 
 
+CLOCK_RAMP_S = 0.5   # untimed run of the benchmark step before the warm-up steps (see main)
+
+
 def ref_formula_flops(tokens, Hv, K, V, C=64):
     """fwd+bwd FLOP of the reference's own counter (mindspeed_mm/fsdp/tools/flops_tool/flops_qwen3_5.py:170-204)."""
     return 3 * 2 * tokens * Hv * (3 * V * C + 2 * K * C + 3 * K * V)
@@ -137,6 +140,14 @@ def main():
                                            skip_recompute=skip_recompute)
         return torch.autograd.grad([o], leaves, [d["do"]])
 
+    # The GPU raises its clocks over the first half second of work of a process: steps timed right after start-up run
+    # about 3 % slower than the same steps a second later.  The figure reported is the steady state, so the same step
+    # runs untimed for CLOCK_RAMP_S before the W warm-up steps and the K timed ones.
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < CLOCK_RAMP_S:
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -221,7 +232,8 @@ def main():
 
     aux = {"path_tflops_ref_formula": round(path_tflops, 2),
            "path_frac_of_bf16_mfma_peak": round(path_tflops / PEAK_BF16_TFLOPS, 4),
-           "kernel_ms_sum": round(total_kernel_ms, 3), "step_time_spread": spread, "kernels": per_kernel}
+           "kernel_ms_sum": round(total_kernel_ms, 3), "step_time_spread": spread, "kernels": per_kernel,
+           "clock_ramp_before_warmup_s": CLOCK_RAMP_S}
 
     if not args.no_aux:
         # ---- decode: batch 256, 64 consecutive steps, state updated in place (BASELINE.json configs[3]) ----
