@@ -358,7 +358,7 @@ template <typename T, int DK> struct BwdLocalSmem {
   // buffer, D-form tiles [4] and T-form tiles [4] in the two shared stages
   static constexpr int off_tm = main_elems * (int)sizeof(T);                 // Tm tiles [2][2], whole kernel
   static constexpr int off_row = off_tm + 4 * 1024 * (int)sizeof(T);
-  static constexpr int bytes = off_row + (5 * 64 + 5 * 256 + 8) * 4;   // 5 row vectors, 5 per-wave row-sum arrays
+  static constexpr int bytes = off_row + (6 * 64 + 5 * 256 + 8) * 4;   // 6 row vectors, 5 per-wave row-sum arrays
   static_assert(main_elems == 32 * 1024, "as large as two former stages");
   static_assert(4 * Patch<T>::kElems <= raw_elems && 2 * (DK / 32) * 1024 <= raw_elems, "epilogue tenants fit");
 };
@@ -394,6 +394,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   float* rf = rbk + 256;   // <F_i, k_i>
   float* rv = rf + 256;    // <R_i, v_i>, taken as the column sums of Tm . (dV' V^T)
   float* wsum = rv + 256;  // per wave: <S,dS'> [0..3], sum_i <k_i, dK_inter_i> [4..7]
+  float* rqc = wsum + 8;   // <q_i, dQ_i> summed over the waves' slots
 
   stagger_second_resident<127>(3, 8 * kStaggerCUs);
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
@@ -732,12 +733,16 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     t.pack(mfma_transpose<T>(d, id));
     t.store(tileT + wave * 1024);
   }
+  // <q_i, dQ_i> once per row, for the l2-norm backward of dq behind the next barrier (instead of every lane adding
+  // up the four slots for each of its sixteen rows)
+  if (l2 && wave == 3) rqc[lane] = (rq[lane] + rq[64 + lane]) + (rq[128 + lane] + rq[192 + lane]);
+  GDN_LDS_BARRIER();
   T* patch = dWF + wave * Patch<T>::kElems;
   if (has_k) {
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {
       if (l2) {
-        const f32x16 qq = QTf[ri].unpack(), dot = rows_ld4(rq, 32 * ri), rs = rows_ld(rsq, 32 * ri);
+        const f32x16 qq = QTf[ri].unpack(), dot = rows_ld(rqc, 32 * ri), rs = rows_ld(rsq, 32 * ri);
 #pragma unroll
         for (int r = 0; r < 16; ++r) dQi[ri][r] = (dQi[ri][r] - dot[r] * qq[r]) * rs[r];
       }
@@ -751,7 +756,6 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
         rows_request<T>(held[ri], dk + (tok0 + 32 * ri) * ts.dk + hq * DK + 32 * cj, ts.dk, nvalid - 32 * ri);
     }
   }
-  GDN_LDS_BARRIER();
   {  // X = dTm Tm^T, handed on in D form
     f32x16 x = acc_zero();
     AccB<T> a, b;
@@ -809,15 +813,20 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     }
   }
   GDN_LDS_BARRIER();   // the row sums are complete
+  auto slots = [&](const float* a) { return (a[lane] + a[64 + lane]) + (a[128 + lane] + a[192 + lane]); };
+  if (l2) {
+    // <k_i, dK_i> = <k,dK1> + beta (e^G <P,k> + <E,k>) + <F,k>, once per row (e^G has served: its place takes it) instead
+    // of the four slots of three arrays being added up by every lane for each of its sixteen rows
+    if (wave == 1) egs[lane] = slots(rk1) + bs[lane] * slots(rbk) + slots(rf);
+    GDN_LDS_BARRIER();
+  }
   if (has_k) {
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {
-      if (l2) {          // <k_i, dK_i> = <k,dK1> + beta (e^G <P,k> + <E,k>) + <F,k>
-        const f32x16 kk = KTf[ri].unpack(), d1 = rows_ld4(rk1, 32 * ri), db = rows_ld4(rbk, 32 * ri),
-                     df = rows_ld4(rf, 32 * ri), br = rows_ld(bs, 32 * ri), rs = rows_ld(rsk, 32 * ri);
+      if (l2) {
+        const f32x16 kk = KTf[ri].unpack(), dot = rows_ld(egs, 32 * ri), rs = rows_ld(rsk, 32 * ri);
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          dKi[ri][r] = (dKi[ri][r] - (d1[r] + br[r] * db[r] + df[r]) * kk[r]) * rs[r];
+        for (int r = 0; r < 16; ++r) dKi[ri][r] = (dKi[ri][r] - dot[r] * kk[r]) * rs[r];
       }
       T* dst = dk + (tok0 + 32 * ri) * ts.dk + hq * DK + 32 * cj;
       if (hh == 0) acc_store_rows<T, false>(dKi[ri], id, patch, dst, ts.dk, nvalid - 32 * ri);
@@ -825,7 +834,6 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     }
   }
   if (wave == 0) {   // d(cumulative G) -> d(g): suffix sum inside the chunk
-    auto slots = [&](const float* a) { return (a[lane] + a[64 + lane]) + (a[128 + lane] + a[192 + lane]); };
     const float sbk = slots(rbk);
     float x = slots(rq) - slots(rk1) + bs[lane] * sbk - slots(rf);
     if (lane == nvalid - 1)
