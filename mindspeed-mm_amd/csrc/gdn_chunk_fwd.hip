@@ -620,6 +620,15 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
   // instead of before or after them.
   AccB<T> Sb[NKT];
   T* xs = reinterpret_cast<T*>(gdn_smem + SM::off_x) + wave * SM::x_elems;   // OUT only
+  // Two tile products into two accumulators, the matrix instructions of one alternating with those of the other: back
+  // to back on one accumulator a matrix instruction costs half as much again (49 cycles against 34, measured).
+  auto mma2 = [](f32x16& x0, const AccB<T>& a0, const AccB<T>& b0, f32x16& x1, const AccB<T>& a1, const AccB<T>& b1) {
+#pragma unroll
+    for (int kg = 0; kg < AccK<T>::kGroups; ++kg) {
+      mfma_kgroup<T>(x0, a0.f[kg], b0.f[kg]);
+      mfma_kgroup<T>(x1, a1.f[kg], b1.f[kg]);
+    }
+  };
 #pragma unroll
   for (int kt = 0; kt < NKT; ++kt) {
     Sb[kt].pack(S[kt]);
@@ -669,8 +678,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
     for (int kp = 0; kp < NP; ++kp) {
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        mma32_ff<T>(p0, Kf[kp & 1][0][j], Sb[2 * kp + j]);
-        mma32_ff<T>(p1, Kf[kp & 1][1][j], Sb[2 * kp + j]);
+        mma2(p0, Kf[kp & 1][0][j], Sb[2 * kp + j], p1, Kf[kp & 1][1][j], Sb[2 * kp + j]);
         if constexpr (KDA) {
           const f32x16 dk = rows_ld(row + 68, 32 * (2 * kp + j));   // the decay of each of the tile's 32 key channels
 #pragma unroll
@@ -701,8 +709,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
     // V' = Tm z (Tm lower triangular: tiles (0,0), (1,0), (1,1))
     p0 = acc_zero();
     p1 = acc_zero();
-    mma32_ff<T>(p0, Tf[0], Vb[0]);
-    mma32_ff<T>(p1, Tf[1], Vb[0]);
+    mma2(p0, Tf[0], Vb[0], p1, Tf[1], Vb[0]);
     mma32_ff<T>(p1, Tf[2], Vb[1]);
     if (NP > 1) load_kt(1, 1);
     Vb[0].pack(p0);
@@ -730,11 +737,9 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
 #pragma unroll
     for (int kp = 0; kp < NP; ++kp) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int kt = 2 * kp + j;
-        mma32_ff<T>(S[kt], Kf[kp & 1][j][0], Vb[0]);
-        mma32_ff<T>(S[kt], Kf[kp & 1][j][1], Vb[1]);
-        if (kt >= 2) Sb[kt - 2].pack(S[kt - 2]);
+      for (int tj = 0; tj < 2; ++tj) {   // the pair's two tiles of S take turns
+        mma2(S[2 * kp], Kf[kp & 1][0][tj], Vb[tj], S[2 * kp + 1], Kf[kp & 1][1][tj], Vb[tj]);
+        if (kp >= 1) Sb[2 * kp - 2 + tj].pack(S[2 * kp - 2 + tj]);
       }
       GDN_SCHED_FENCE();
       if (kp + 2 < NP) { load_kt(kp & 1, kp + 2); GDN_SCHED_FENCE(); }
