@@ -36,6 +36,13 @@ extern "C" {
  * only fills the workspace and writes no output: it is the recomputation step of a backward pass whose forward pass
  * kept nothing (chunk_gated_delta_rule.py:102-119 recomputes w, u, h, v_new the same way).  A forward call with a
  * workspace sized with with_backward = 0 writes neither per-chunk states nor v_new to memory.
+ *
+ * The workspace has two parts.  The prep part (with_backward = 2) holds what depends on q, k, g, beta only: the
+ * cumulative decay, Tm, the intra-chunk Q K^T tiles and the K / Q^T tile images; the state part (with_backward = 3)
+ * holds the per-chunk states, v_new and room for their gradients.  with_backward = 1 is both, contiguous.  A forward
+ * call in a 16-bit dtype that writes o (and no fused norm) needs the prep part only.  gdn_chunk_bwd_parts takes the
+ * two parts as separate buffers, so that a caller can keep the prep part of its forward call (0.28 GB at B=2, T=8192,
+ * Hqk=16, Hv=32, d=128 in bf16, against 1.2 GB for both) and have the backward pass rebuild the state part.
  */
 int64_t gdn_chunk_workspace_bytes(int B, int T, int N, int Hqk, int Hv, int K, int V, int dtype, int with_backward);
 
@@ -82,6 +89,26 @@ int gdn_chunk_bwd_strided(const void* q, const void* k, const void* v, int64_t q
                           float* d_initial_state, void* workspace, int64_t workspace_bytes, int B, int T, int N,
                           int Hqk, int Hv, int K, int V, float scale, int use_qk_l2norm, int dtype, int beta_dtype,
                           void* stream);
+
+/* The backward pass in phases, on a workspace given in two buffers (see gdn_chunk_workspace_bytes): any combination of
+ *   1  refill the state part (forward recurrence without output; chunk_prep_kernel first unless prep_valid != 0,
+ *      i.e. unless workspace_prep still holds what a forward call on the same inputs left there)
+ *   2  the reverse recurrence
+ *   4  the chunk-local kernels (dq, dk, dv, dg, dbeta); needs phases 1 and 2 of the same inputs done
+ * Phases 1 and 2 do not depend on each other: a caller may launch them on two streams and join both before phase 4.
+ * Each of them is a latency-bound kernel with one workgroup per compute unit at most; for shapes whose slabs would fill
+ * more than half of the device they are launched with two slabs per workgroup here, so that the two fit side by side
+ * (same results, bit for bit).  Counterpart in the reference: the recomputation inside chunk_gated_delta_rule_bwd,
+ * chunk_gated_delta_rule.py:102-119, followed by its stages :120-174.  Arguments a phase does not use may be NULL
+ * (g for 2 and 4; d_o for 1; the gradient outputs for 1 and 2). */
+int gdn_chunk_bwd_parts(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
+                        int64_t v_stride, const float* g, const void* beta, const float* initial_state,
+                        const int64_t* cu_seqlens, const void* d_o, const float* d_final_state, void* dq, void* dk,
+                        void* dv, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride, float* dg, void* dbeta,
+                        float* d_initial_state, void* workspace_prep, int64_t workspace_prep_bytes,
+                        void* workspace_state, int64_t workspace_state_bytes, int phases, int prep_valid, int B, int T,
+                        int N, int Hqk, int Hv, int K, int V, float scale, int use_qk_l2norm, int dtype, int beta_dtype,
+                        void* stream);
 
 /* -------- fused recurrent gated delta rule (decode) ------------------------------------------
  * replaces the `recurrent_gated_delta_rule` slot (third-party fla kernel or

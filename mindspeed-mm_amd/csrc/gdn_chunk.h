@@ -38,6 +38,8 @@ struct ChunkWorkspace {
   int64_t AQ;             // T [chunks,Hv,2,2]       scale tril(Q K^T . Gam), accumulator tiles: lane <-> column, registers <-> row
   int64_t KAF;            // T [chunks,Hqk,K/32,2]   K as A operand: tile = (32 tokens) x (32 columns of K)
   int64_t QTF;            // T [chunks,Hqk,K/32,2]   Q^T as A operand: tile = (32 columns of K) x (32 tokens)
+  int64_t prep_bytes;     // everything above: what chunk_prep_kernel leaves (no v, no state in it).  What follows, the "state
+                          // part", may live in a second buffer: the kernels take a base pointer for each part.
   int64_t VF;             // T [chunks,Hv,V/32,2]    v_new = Tm (beta v - beta e^G K S), tile = (32-column block) x (32-token block)
   int64_t HF;             // T [chunks,Hv,V/32,K/32] state BEFORE each chunk, tile = (32 rows of K) x (32 columns of V)
   int64_t fwd_bytes;
@@ -60,6 +62,7 @@ inline ChunkWorkspace chunk_workspace_layout(const ChunkDims& d, int elem_bytes)
   w.AQ = take(nc * 64 * d.Hv * 64 * elem_bytes);
   w.KAF = take(nc * 64 * d.Hqk * d.K * elem_bytes);
   w.QTF = take(nc * 64 * d.Hqk * d.K * elem_bytes);
+  w.prep_bytes = off;
   w.VF = take(nc * 64 * d.Hv * d.V * elem_bytes);
   w.HF = take(nc * d.Hv * d.V * d.K * elem_bytes);
   w.fwd_bytes = off;
@@ -136,6 +139,34 @@ int device_compute_units();   // defined with the forward launcher
 inline bool one_slab_per_workgroup(const ChunkDims& d, int compute_units) {
   return (int64_t)d.N * d.Hv * (d.V / 32) <= compute_units;
 }
+// Two recurrences at once (a backward pass that refills the forward states on a second stream while the reverse
+// recurrence runs): with two slabs per workgroup each of them is as fast as with one and needs half of the compute
+// units, so both fit the device side by side.  Only needed where one slab per workgroup would take more than half.
+inline bool two_slabs_to_share_device(const ChunkDims& d, int compute_units) {
+  const int64_t slabs = (int64_t)d.N * d.Hv * (d.V / 32);
+  return slabs <= compute_units && 2 * slabs > compute_units;
+}
+
+// the gated RMSNorm applied by the output kernel (null y: none); weight in fp32 or in the rule's dtype
+struct FwdNorm {
+  const void* gate;
+  const void* weight;
+  void* y;
+  float* rstd;
+  float eps;
+  bool weight_fp32;
+};
+
+// The forward pass behind gdn_chunk_fwd_strided / gdn_chunk_fwd_norm_strided (defined with the forward kernels).
+// workspace_state non-null: the workspace comes in two buffers, `workspace` holding the prep part and workspace_state
+// the state part; skip_prep: the prep part already holds this input's tiles and is not computed again; share_device:
+// the recurrence leaves half of the compute units to another one that runs beside it (two_slabs_to_share_device).
+int chunk_fwd_entry(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride, int64_t v_stride,
+                    const float* g, const void* beta, int beta_dtype, const float* initial_state,
+                    const int64_t* cu_seqlens, void* o, float* final_state, void* workspace, int64_t workspace_bytes,
+                    int B, int T, int N, int Hqk, int Hv, int K, int V, float scale, int use_qk_l2norm, int dtype,
+                    const FwdNorm& fn, void* stream, void* workspace_state = nullptr, int64_t workspace_state_bytes = 0,
+                    bool skip_prep = false, bool share_device = false);
 
 inline int chunk_check_dims(const ChunkDims& d, int dtype) {
   if (d.B <= 0 || d.T <= 0 || d.N <= 0 || d.Hqk <= 0 || d.Hv <= 0 || d.Hv % d.Hqk != 0) return -2;

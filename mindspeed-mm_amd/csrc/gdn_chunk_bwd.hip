@@ -880,23 +880,25 @@ template <typename K> static int set_lds_b(K kernel, int bytes) {
 template <typename T, int DK, int NW, int NWS, int NLS, int STAGES>
 static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const void* q, const void* k, const void* v,
                             const void* beta, int beta_same, const int64_t* cu, const void* dO, const float* dht, void* dq,
-                            void* dk, void* dv, float* dg, void* dbeta, float* dh0, unsigned char* ws, float scale, int l2norm,
-                            hipStream_t st) {
+                            void* dk, void* dv, float* dg, void* dbeta, float* dh0, unsigned char* ws, unsigned char* ws_state,
+                            int phases, float scale, int l2norm, hipStream_t st) {
+  // ws, ws_state: bases of the workspace's prep part and state part (see ChunkWorkspace); phases: 2 = the reverse
+  // recurrence, 4 = the chunk-local kernels
   const int nc = (int)d.max_chunks();
   const int* chunk_offsets = reinterpret_cast<const int*>(ws + L.chunk_offsets);
   (void)q; (void)k;   // q and k reach the backward kernels as the forward pass's fragment tiles
   const float* G = reinterpret_cast<const float*>(ws + L.G);
   const T* Ai = reinterpret_cast<const T*>(ws + L.Ai);
   const T* AQ = reinterpret_cast<const T*>(ws + L.AQ);
-  const T* VF = reinterpret_cast<const T*>(ws + L.VF);
-  const T* HF = reinterpret_cast<const T*>(ws + L.HF);
+  const T* VF = reinterpret_cast<const T*>(ws_state + L.VF);
+  const T* HF = reinterpret_cast<const T*>(ws_state + L.HF);
   const T* QTF = reinterpret_cast<const T*>(ws + L.QTF);
   const T* KAF = reinterpret_cast<const T*>(ws + L.KAF);
-  T* DVF = reinterpret_cast<T*>(ws + L.DVF);
-  T* DHF = reinterpret_cast<T*>(ws + L.DHF);
+  T* DVF = reinterpret_cast<T*>(ws_state + L.DVF);
+  T* DHF = reinterpret_cast<T*>(ws_state + L.DHF);
   const float* rstd_q = l2norm ? reinterpret_cast<const float*>(ws + L.rstd) : nullptr;
   const float* rstd_k = l2norm ? rstd_q + (int64_t)nc * 64 * d.Hqk : nullptr;
-  {
+  if (phases & 2) {
     auto kern = chunk_state_bwd_kernel<T, DK, NWS, NLS, STAGES>;
     constexpr int smem = StateBwdSmem<T, DK, NWS, STAGES>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
@@ -904,7 +906,7 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
                (const T*)nullptr, (const T*)QTF, Ai, AQ, (const T*)dO, G, beta, beta_same, dht, dh0, DVF, DHF, cu, chunk_offsets, d.T, d.Hqk, d.Hv, d.V,
                scale);
   }
-  {
+  if (phases & 4) {
     auto kern = chunk_bwd_local_kernel<T, DK>;
     constexpr int smem = BwdLocalSmem<T, DK>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
@@ -918,16 +920,20 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
 
 }  // namespace gdn
 
-extern "C" int gdn_chunk_bwd_strided(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
-                                     int64_t v_stride, const float* g, const void* beta, const float* initial_state,
-                                     const int64_t* cu_seqlens, const void* d_o, const float* d_final_state, void* dq,
-                                     void* dk, void* dv, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride,
-                                     float* dg, void* dbeta, float* d_initial_state, void* workspace,
-                                     int64_t workspace_bytes, int B, int T, int N, int Hqk, int Hv, int K, int V,
-                                     float scale, int use_qk_l2norm, int dtype, int beta_dtype, void* stream) {
-  using namespace gdn;
-  (void)g; (void)initial_state;   // their effect is already in the workspace (G, per-chunk states)
-  if (!q || !k || !v || !beta || !d_o || !dq || !dk || !dv || !dg || !dbeta || !workspace) return -1;
+namespace gdn {
+// phases: 1 = refill the state part from the prep part (prep itself first unless prep_valid), 2 = the reverse recurrence,
+// 4 = the chunk-local kernels.  workspace_state null: one buffer holds both parts.
+static int chunk_bwd_entry(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride, int64_t v_stride,
+                           const float* g, const void* beta, const float* initial_state, const int64_t* cu_seqlens,
+                           const void* d_o, const float* d_final_state, void* dq, void* dk, void* dv, int64_t dq_stride,
+                           int64_t dk_stride, int64_t dv_stride, float* dg, void* dbeta, float* d_initial_state,
+                           void* workspace, int64_t workspace_bytes, void* workspace_state, int64_t workspace_state_bytes,
+                           int phases, int prep_valid, bool share_device, int B, int T, int N, int Hqk, int Hv, int K, int V,
+                           float scale, int use_qk_l2norm, int dtype, int beta_dtype, void* stream) {
+  if (!q || !k || !v || !beta || !workspace) return -1;
+  if ((phases & 6) && !d_o) return -1;
+  if ((phases & 4) && (!dq || !dk || !dv || !dg || !dbeta)) return -1;
+  if ((phases & ~7) || phases == 0) return -2;
   ChunkDims d{B, T, N, Hqk, Hv, K, V, cu_seqlens != nullptr};
   d.ts = {q_stride, k_stride, v_stride, dq_stride, dk_stride, dv_stride};
   if (int e = chunk_check_dims(d, dtype)) return e;
@@ -937,16 +943,33 @@ extern "C" int gdn_chunk_bwd_strided(const void* q, const void* k, const void* v
   ChunkDims dl = d;
   dl.varlen = true;
   const ChunkWorkspace L = chunk_workspace_layout(dl, dtype == 0 ? 4 : 2);
-  if (workspace_bytes < L.total_bytes) return -5;
-  if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
   unsigned char* ws = static_cast<unsigned char*>(workspace);
+  unsigned char* ws_state = ws;
+  if (workspace_state != nullptr) {
+    if (workspace_bytes < L.prep_bytes || workspace_state_bytes < L.total_bytes - L.prep_bytes) return -5;
+    if ((reinterpret_cast<uintptr_t>(workspace_state) & 255) != 0) return -5;
+    ws_state = static_cast<unsigned char*>(workspace_state) - L.prep_bytes;
+  } else if (workspace_bytes < L.total_bytes) {
+    return -5;
+  }
+  if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
   hipStream_t st = (hipStream_t)stream;
+  if (phases & 1) {
+    if (!g) return -1;
+    if (workspace_state == nullptr && prep_valid) return -1;   // one buffer is always refilled whole
+    if (int e = chunk_fwd_entry(q, k, v, q_stride, k_stride, v_stride, g, beta, beta_dtype, initial_state, cu_seqlens, nullptr,
+                                nullptr, workspace, workspace_bytes, B, T, N, Hqk, Hv, K, V, scale, use_qk_l2norm, dtype,
+                                FwdNorm{}, stream, workspace_state, workspace_state_bytes, prep_valid != 0, share_device))
+      return e;
+    if (!(phases & 6)) return 0;
+  }
 #define GDN_BWD(T_, DK_, NW_, NWS_, NLS_, ST_)                                                       \
   return chunk_bwd_launch<T_, DK_, NW_, NWS_, NLS_, ST_>(d, L, q, k, v, beta, beta_same, cu_seqlens, d_o, d_final_state, dq, \
-                                                          dk, dv, dg, dbeta, d_initial_state, ws, scale,         \
+                                                          dk, dv, dg, dbeta, d_initial_state, ws, ws_state, phases, scale, \
                                                           use_qk_l2norm, st)
   const bool wide = (V % 128 == 0);
-  const bool solo = one_slab_per_workgroup(d, device_compute_units());
+  const bool solo = one_slab_per_workgroup(d, device_compute_units()) &&
+                    !(share_device && two_slabs_to_share_device(d, device_compute_units()));
   if (dtype == 1) {
     if (K == 128 && wide && solo) GDN_BWD(bf16_t, 128, 4, 1, 4, 2);
     if (K == 128 && wide) GDN_BWD(bf16_t, 128, 4, 2, 4, 2);
@@ -958,6 +981,36 @@ extern "C" int gdn_chunk_bwd_strided(const void* q, const void* k, const void* v
     GDN_BWD(float, 64, 2, 2, 2, 1);
   }
 #undef GDN_BWD
+}
+}  // namespace gdn
+
+extern "C" int gdn_chunk_bwd_strided(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
+                                     int64_t v_stride, const float* g, const void* beta, const float* initial_state,
+                                     const int64_t* cu_seqlens, const void* d_o, const float* d_final_state, void* dq,
+                                     void* dk, void* dv, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride,
+                                     float* dg, void* dbeta, float* d_initial_state, void* workspace,
+                                     int64_t workspace_bytes, int B, int T, int N, int Hqk, int Hv, int K, int V,
+                                     float scale, int use_qk_l2norm, int dtype, int beta_dtype, void* stream) {
+  (void)g; (void)initial_state;   // their effect is already in the workspace (G, per-chunk states)
+  return gdn::chunk_bwd_entry(q, k, v, q_stride, k_stride, v_stride, g, beta, initial_state, cu_seqlens, d_o, d_final_state,
+                              dq, dk, dv, dq_stride, dk_stride, dv_stride, dg, dbeta, d_initial_state, workspace,
+                              workspace_bytes, nullptr, 0, 6, 1, false, B, T, N, Hqk, Hv, K, V, scale, use_qk_l2norm, dtype,
+                              beta_dtype, stream);
+}
+
+extern "C" int gdn_chunk_bwd_parts(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
+                                   int64_t v_stride, const float* g, const void* beta, const float* initial_state,
+                                   const int64_t* cu_seqlens, const void* d_o, const float* d_final_state, void* dq,
+                                   void* dk, void* dv, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride, float* dg,
+                                   void* dbeta, float* d_initial_state, void* workspace_prep, int64_t workspace_prep_bytes,
+                                   void* workspace_state, int64_t workspace_state_bytes, int phases, int prep_valid, int B,
+                                   int T, int N, int Hqk, int Hv, int K, int V, float scale, int use_qk_l2norm, int dtype,
+                                   int beta_dtype, void* stream) {
+  if (!workspace_state) return -1;
+  return gdn::chunk_bwd_entry(q, k, v, q_stride, k_stride, v_stride, g, beta, initial_state, cu_seqlens, d_o, d_final_state,
+                              dq, dk, dv, dq_stride, dk_stride, dv_stride, dg, dbeta, d_initial_state, workspace_prep,
+                              workspace_prep_bytes, workspace_state, workspace_state_bytes, phases, prep_valid, true, B, T, N,
+                              Hqk, Hv, K, V, scale, use_qk_l2norm, dtype, beta_dtype, stream);
 }
 
 extern "C" int gdn_chunk_bwd(const void* q, const void* k, const void* v, const float* g, const float* beta,

@@ -920,28 +920,20 @@ template <typename K> static int set_lds(K kernel, int bytes) {
                                   bytes);
 }
 
-// the gated RMSNorm applied by the output kernel (null y: none); weight in fp32 or in the rule's dtype
-struct FwdNorm {
-  const void* gate;
-  const void* weight;
-  void* y;
-  float* rstd;
-  float eps;
-  bool weight_fp32;
-};
-
 // NW: waves (32-column blocks) per workgroup of the stand-alone output kernel; NWS, NLS, STAGES: slabs, loader waves
 // and LDS stages of the recurrence kernel; FUSE: the recurrence kernel's own output waves write O (no norm, bf16)
 template <typename T, int DK, int NW, int NWS, int NLS, int STAGES, bool FUSE>
 static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const void* q, const void* k, const void* v,
                             const float* g, const void* beta, int beta_same, const float* h0, const int64_t* cu, void* o,
-                            float* ht, unsigned char* ws, float scale, int l2norm, bool with_backward, const FwdNorm& fn,
-                            hipStream_t st) {
+                            float* ht, unsigned char* ws, unsigned char* ws_state, bool skip_prep, float scale, int l2norm,
+                            bool with_backward, const FwdNorm& fn, hipStream_t st) {
+  // ws: base of the workspace's prep part; ws_state: base such that ws_state + L.VF, + L.HF are the state part (equal to
+  // ws when the workspace is one buffer).  skip_prep: the prep part already holds this input's tiles.
   const int nc = (int)d.max_chunks();
   int* chunk_offsets = reinterpret_cast<int*>(ws + L.chunk_offsets);
   const T* qq = (const T*)q;
   const T* kk = (const T*)k;
-  if (cu != nullptr) GDN_LAUNCH(kKernChunkTable, st, chunk_table_kernel, dim3(1), dim3(kThreads), 0, st, cu, chunk_offsets, d.N);
+  if (cu != nullptr && !skip_prep) GDN_LAUNCH(kKernChunkTable, st, chunk_table_kernel, dim3(1), dim3(kThreads), 0, st, cu, chunk_offsets, d.N);
   float* rstd = reinterpret_cast<float*>(ws + L.rstd);
   float* G = reinterpret_cast<float*>(ws + L.G);
   T* Ai = reinterpret_cast<T*>(ws + L.Ai);
@@ -953,10 +945,10 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   // the per-chunk states and v_new leave the recurrence kernel only for a later reader: the backward pass or the
   // stand-alone output kernel
   const bool keep = with_backward || !fuse;
-  T* VF = keep ? reinterpret_cast<T*>(ws + L.VF) : nullptr;
-  T* HF = keep ? reinterpret_cast<T*>(ws + L.HF) : nullptr;
+  T* VF = keep ? reinterpret_cast<T*>(ws_state + L.VF) : nullptr;
+  T* HF = keep ? reinterpret_cast<T*>(ws_state + L.HF) : nullptr;
   const TokenStrides ts = d.strides();
-  {
+  if (!skip_prep) {
     auto kern = chunk_prep_kernel<T, DK>;
     constexpr int smem = PrepSmem<T, DK>::bytes;
     if (int e = set_lds(kern, smem)) return e;
@@ -1032,15 +1024,18 @@ extern "C" int64_t gdn_chunk_workspace_bytes(int B, int T, int N, int Hqk, int H
   // one layout for padded and packed input: the packed chunk bound is the larger of the two
   gdn::ChunkDims d{B, T, N, Hqk, Hv, K, V, true};
   const gdn::ChunkWorkspace w = gdn::chunk_workspace_layout(d, dtype == 0 ? 4 : 2);
+  if (with_backward == 2) return w.prep_bytes;                    // the prep part alone
+  if (with_backward == 3) return w.total_bytes - w.prep_bytes;    // the state part alone
   return with_backward ? w.total_bytes : w.fwd_bytes;
 }
 
 namespace gdn {
-static int chunk_fwd_entry(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
+int chunk_fwd_entry(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
                            int64_t v_stride, const float* g, const void* beta, int beta_dtype, const float* initial_state,
                            const int64_t* cu_seqlens, void* o, float* final_state, void* workspace,
                            int64_t workspace_bytes, int B, int T, int N, int Hqk, int Hv, int K, int V, float scale,
-                           int use_qk_l2norm, int dtype, const FwdNorm& fn, void* stream) {
+                           int use_qk_l2norm, int dtype, const FwdNorm& fn, void* stream, void* workspace_state,
+                           int64_t workspace_state_bytes, bool skip_prep, bool share_device) {
   if (!q || !k || !v || !g || !beta || !workspace) return -1;
   if (fn.y != nullptr && (!fn.gate || !fn.weight)) return -1;
   ChunkDims d{B, T, N, Hqk, Hv, K, V, cu_seqlens != nullptr};
@@ -1054,17 +1049,32 @@ static int chunk_fwd_entry(const void* q, const void* k, const void* v, int64_t 
   ChunkDims dl = d;
   dl.varlen = true;  // one layout for both modes (the packed bound is the larger)
   const ChunkWorkspace L = chunk_workspace_layout(dl, dtype == 0 ? 4 : 2);
-  if (workspace_bytes < L.fwd_bytes) return -5;
-  const bool with_bwd = workspace_bytes >= L.total_bytes;
-  if (!o && !fn.y && !with_bwd) return -1;   // without an output the call only makes sense as a refill   // a workspace sized for backward: the per-chunk states and v_new are kept
-  if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
+  // One buffer: sized for backward (states and v_new are kept), for forward only, or -- where the recurrence writes the
+  // output itself and nothing reads states or v_new from memory (16-bit types, no fused norm) -- just the prep part.
+  // Two buffers: the prep part and the state part (forward states, v_new, and room for their gradients).
+  const bool fused_out = dtype == 1 && fn.y == nullptr && o != nullptr;
+  bool with_bwd;
   unsigned char* ws = static_cast<unsigned char*>(workspace);
+  unsigned char* ws_state = ws;
+  if (workspace_state != nullptr) {
+    if (workspace_bytes < L.prep_bytes || workspace_state_bytes < L.total_bytes - L.prep_bytes) return -5;
+    if ((reinterpret_cast<uintptr_t>(workspace_state) & 255) != 0) return -5;
+    ws_state = static_cast<unsigned char*>(workspace_state) - L.prep_bytes;
+    with_bwd = true;
+  } else {
+    if (workspace_bytes < (fused_out ? L.prep_bytes : L.fwd_bytes)) return -5;
+    with_bwd = workspace_bytes >= L.total_bytes;
+    if (skip_prep) return -1;
+  }
+  if (!o && !fn.y && !with_bwd) return -1;   // without an output the call only makes sense as a refill
+  if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
   hipStream_t st = (hipStream_t)stream;
 #define GDN_FWD(T_, DK_, NW_, NWS_, NLS_, ST_, FUSE_)                                                                       \
   return chunk_fwd_launch<T_, DK_, NW_, NWS_, NLS_, ST_, FUSE_>(d, L, q, k, v, g, beta, beta_same, initial_state, cu_seqlens, o, final_state, \
-                                                   ws, scale, use_qk_l2norm, with_bwd, fn, st)
+                                                   ws, ws_state, skip_prep, scale, use_qk_l2norm, with_bwd, fn, st)
   const bool wide = (V % 128 == 0);
-  const bool solo = one_slab_per_workgroup(d, device_compute_units());
+  const bool solo = one_slab_per_workgroup(d, device_compute_units()) &&
+                    !(share_device && two_slabs_to_share_device(d, device_compute_units()));
   if (dtype == 1) {
     if (K == 128 && wide && solo) GDN_FWD(bf16_t, 128, 4, 1, 4, 2, true);
     if (K == 128 && wide) GDN_FWD(bf16_t, 128, 4, 2, 4, 2, true);

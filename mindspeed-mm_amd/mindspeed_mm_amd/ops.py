@@ -18,6 +18,7 @@ Everything here is host glue: validation, output/workspace allocation with torch
 C ABI per operator.  The kernels themselves are the HIP library; nothing in this file computes.
 """
 import functools
+import os
 import warnings
 from typing import Optional
 
@@ -82,6 +83,21 @@ class GdnOps:
 
     def __init__(self, lib: GdnLibrary):
         self.lib = lib
+        self._helpers = {}
+        # False: the backward pass of the chunked rule runs its two recurrences one after the other on the caller's stream
+        self.two_stream_backward = os.environ.get("GDN_TWO_STREAM_BACKWARD", "1") != "0"
+
+    def helper_stream(self, device):
+        """A second stream on `device` (default priority, made once) for work that may run beside the caller's stream;
+        None where there are no streams (the host build of the kernels) or two_stream_backward is off."""
+        if self.lib.device_type != "cuda" or not self.two_stream_backward:
+            return None
+        key = torch.device(device).index
+        if key is None:
+            key = torch.cuda.current_device()
+        if key not in self._helpers:
+            self._helpers[key] = torch.cuda.Stream(device=key)
+        return self._helpers[key]
 
     # ------------------------------------------------------------------ helpers
     def _need(self, *tensors):
@@ -446,6 +462,8 @@ def _token_view(x):
 
 
 def _chunk_workspace(lib, device, B, T, N, Hqk, Hv, K, V, code, need_grad):
+    """A 256-byte aligned workspace; need_grad: False / True for a forward-only or a forward + backward workspace,
+    2 / 3 for its prep part / state part alone (gdn_chunk_workspace_bytes)."""
     nbytes = lib.gdn_chunk_workspace_bytes(B, T, N, Hqk, Hv, K, V, code, int(need_grad))
     ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=device)
     off = (-ws.data_ptr()) % 256
@@ -455,11 +473,14 @@ def _chunk_workspace(lib, device, B, T, N, Hqk, Hv, K, V, code, need_grad):
 class _ChunkGatedDeltaRule(torch.autograd.Function):
     """Positional order as ChunkGatedDeltaRuleFunction.forward (chunk_gated_delta_rule.py:182-196).
 
-    skip_recompute=False (the default, as in the reference, which saves q, k, v, g, beta, A, h0 and recomputes w, u, h
-    and v_new in its backward pass, chunk_gated_delta_rule.py:102-119, :264): nothing but the inputs is kept between
-    the passes; the backward pass refills a workspace (chunk-local kernel and recurrence, no output) before its own
-    kernels.  skip_recompute=True keeps the forward pass's workspace instead (per-chunk states, v_new, Tm, ...:
-    gdn_chunk_workspace_bytes with with_backward=1) and skips that work.  Both give the same gradients, bit for bit."""
+    skip_recompute=False (the default, as in the reference, which saves q, k, v, g_cum, beta, Ai, h0 and recomputes w,
+    u, h and v_new in its backward pass, chunk_gated_delta_rule.py:102-119, :264): in the 16-bit dtypes the forward pass
+    keeps the prep part of its workspace (cumulative decay, Tm, the intra-chunk tiles and the K / Q^T images: everything
+    that does not depend on v or on the state) and the backward pass rebuilds the per-chunk states and v_new with the
+    forward recurrence on a second stream while the reverse recurrence runs on the caller's; both are latency-bound and
+    fit the device side by side.  In fp32 nothing but the inputs is kept and the backward pass refills the whole
+    workspace first.  skip_recompute=True keeps the whole forward workspace instead (per-chunk states and v_new too:
+    gdn_chunk_workspace_bytes with with_backward=1) and skips that work.  All give the same gradients, bit for bit."""
 
     @staticmethod
     @_input_guard
@@ -472,12 +493,13 @@ class _ChunkGatedDeltaRule(torch.autograd.Function):
         N = (len(cu_seqlens) - 1) if cu_seqlens is not None else B
         need_grad = any(ctx.needs_input_grad[:5]) or (initial_state is not None and ctx.needs_input_grad[6])
         keep = need_grad and skip_recompute
+        prep_only = q.dtype != torch.float32 and not keep   # the recurrence writes o itself: no state leaves it
         (qc, sq), (kc, sk), (vc, sv) = _token_view(q), _token_view(k), _token_view(v)
         g32, h0 = ops._f32(g), ops._f32(initial_state)
         bc, bcode = _beta_arg(beta, q.dtype)
         cu = _i64(cu_seqlens, q)
         code = DTYPE_CODE[q.dtype]
-        ws, nbytes = _chunk_workspace(lib, q.device, B, T, N, Hqk, Hv, K, V, code, keep)
+        ws, nbytes = _chunk_workspace(lib, q.device, B, T, N, Hqk, Hv, K, V, code, 2 if prep_only else keep)
         o = torch.empty(B, T, Hv, V, dtype=v.dtype, device=v.device)
         ht = torch.empty(N, Hv, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
         rc = lib.gdn_chunk_fwd_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(bc), ptr(h0), ptr(cu),
@@ -485,7 +507,8 @@ class _ChunkGatedDeltaRule(torch.autograd.Function):
                                        int(use_qk_l2norm_in_kernel), code, bcode, lib.stream())
         lib.check(rc, "gdn_chunk_fwd_strided")
         if need_grad:
-            ctx.save_for_backward(qc, kc, vc, g32, bc, h0, cu, ws if keep else None)
+            ctx.save_for_backward(qc, kc, vc, g32, bc, h0, cu, ws if (keep or prep_only) else None)
+            ctx.prep_only = prep_only
             ctx.meta = (B, T, N, Hqk, Hv, K, V, scale, int(use_qk_l2norm_in_kernel), code, nbytes,
                         g.dtype, beta.dtype, None if initial_state is None else initial_state.dtype, sq, sk, sv, bcode)
             ctx.ops = ops
@@ -499,12 +522,6 @@ class _ChunkGatedDeltaRule(torch.autograd.Function):
         B, T, N, Hqk, Hv, K, V, scale, l2, code, nbytes, g_dt, b_dt, h_dt, sq, sk, sv, bcode = ctx.meta
         lib = ctx.ops.lib
         dev = qc.device
-        if ws is None:   # nothing was kept: refill a workspace (no output is written when o is null)
-            ws, nbytes = _chunk_workspace(lib, dev, B, T, N, Hqk, Hv, K, V, code, True)
-            rc = lib.gdn_chunk_fwd_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(bc), ptr(h0), ptr(cu),
-                                           None, None, ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale, l2, code, bcode,
-                                           lib.stream())
-            lib.check(rc, "gdn_chunk_fwd_strided (recompute)")
         do = do.contiguous()
         dht = ctx.ops._f32(dht)
         dq = torch.empty(B, T, Hqk, K, dtype=qc.dtype, device=dev)
@@ -513,6 +530,35 @@ class _ChunkGatedDeltaRule(torch.autograd.Function):
         dg = torch.empty(B, T, Hv, dtype=torch.float32, device=dev)
         db = torch.empty(B, T, Hv, dtype=bc.dtype, device=dev)
         dh0 = torch.empty(N, Hv, K, V, dtype=torch.float32, device=dev) if h0 is not None else None
+        if ws is not None and ctx.prep_only:
+            # the prep part was kept: the state part is rebuilt beside the reverse recurrence, then the chunk-local kernels
+            ws_state, nstate = _chunk_workspace(lib, dev, B, T, N, Hqk, Hv, K, V, code, 3)
+
+            def phase(ph):
+                rc = lib.gdn_chunk_bwd_parts(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(bc), ptr(h0), ptr(cu),
+                                             ptr(do), ptr(dht), ptr(dq), ptr(dk), ptr(dv), 0, 0, 0, ptr(dg), ptr(db),
+                                             ptr(dh0), ptr(ws), nbytes, ptr(ws_state), nstate, ph, 1, B, T, N, Hqk, Hv, K,
+                                             V, scale, l2, code, bcode, lib.stream())
+                lib.check(rc, "gdn_chunk_bwd_parts")
+            helper = ctx.ops.helper_stream(dev)
+            if helper is None:
+                phase(7)
+            else:
+                main = torch.cuda.current_stream(dev)
+                helper.wait_stream(main)
+                with torch.cuda.stream(helper):
+                    phase(1)
+                phase(2)
+                main.wait_stream(helper)
+                phase(4)
+            return (dq, dk, dv, dg.to(g_dt), db.to(b_dt), None, None if dh0 is None else dh0.to(h_dt), None, None,
+                    None, None, None)
+        if ws is None:   # nothing was kept: refill a workspace (no output is written when o is null)
+            ws, nbytes = _chunk_workspace(lib, dev, B, T, N, Hqk, Hv, K, V, code, True)
+            rc = lib.gdn_chunk_fwd_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(bc), ptr(h0), ptr(cu),
+                                           None, None, ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale, l2, code, bcode,
+                                           lib.stream())
+            lib.check(rc, "gdn_chunk_fwd_strided (recompute)")
         rc = lib.gdn_chunk_bwd_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(bc), ptr(h0), ptr(cu),
                                        ptr(do), ptr(dht), ptr(dq), ptr(dk), ptr(dv), 0, 0, 0, ptr(dg), ptr(db),
                                        ptr(dh0), ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale, l2, code, bcode,
