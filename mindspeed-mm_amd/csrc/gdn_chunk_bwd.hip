@@ -397,7 +397,8 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     const T* __restrict__ dO, const T* __restrict__ hf, const T* __restrict__ dhf, const float* __restrict__ rstd_q,
     const float* __restrict__ rstd_k, T* dq, T* dk, T* __restrict__ dv_out, void* __restrict__ dbeta,
     float* __restrict__ dg, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N,
-    int Hqk, int Hv, int V, float scale, int hh, TokenStrides ts, T* __restrict__ kda_dump, float* __restrict__ kda_dd) {
+    int Hqk, int Hv, int V, float scale, int hh, TokenStrides ts, T* __restrict__ kda_dump, float* __restrict__ kda_dd,
+    int cus) {
   using SM = BwdLocalSmem<T, DK>;
   constexpr int NKT = DK / 32, VEC = Elem<T>::kVec, KG = AccK<T>::kGroups;
   static_assert(NKT <= 4, "one 32-column block of K per wave");
@@ -417,7 +418,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   float* wsum = rv + 256;  // per wave: <S,dS'> [0..3], sum_i <k_i, dK_inter_i> [4..7]
   float* rqc = wsum + 8;   // <q_i, dQ_i> summed over the waves' slots
 
-  stagger_second_resident<127>(3, 8 * kStaggerCUs);
+  stagger_second_resident<127>(3, 8 * cus, cus);
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31;
@@ -907,13 +908,19 @@ static int chunk_bwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
                scale);
   }
   if (phases & 4) {
+    const TokenStrides gs = d.strides();
+    const int es = (int)sizeof(T), bb = beta_same ? es : 4;
+    TailRows tail{{dq, dk, dv, dg, dbeta}, {gs.dq * es, gs.dk * es, gs.dv * es, (int64_t)d.Hv * 4, (int64_t)d.Hv * bb},
+                  {d.Hqk * DK * es, d.Hqk * DK * es, d.Hv * d.V * es, d.Hv * 4, d.Hv * bb}};
+    launch_zero_tail_rows(cu, d.N, d.tokens(), tail, st);
     auto kern = chunk_bwd_local_kernel<T, DK>;
     constexpr int smem = BwdLocalSmem<T, DK>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
     for (int hh = 0; hh < d.Hv / d.Hqk; ++hh)
       GDN_LAUNCH(kKernBwdLocal, st, kern, dim3(nc, d.Hqk), dim3(kThreads), smem, st, QTF, (const T*)KAF, (const T*)v,
                  beta, beta_same, G, Ai, VF, (const T*)DVF, (const T*)dO, HF, (const T*)DHF, rstd_q, rstd_k, (T*)dq, (T*)dk,
-                 (T*)dv, dbeta, dg, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale, hh, d.strides(), (T*)nullptr, (float*)nullptr);
+                 (T*)dv, dbeta, dg, cu, chunk_offsets, d.T, d.N, d.Hqk, d.Hv, d.V, scale, hh, d.strides(), (T*)nullptr, (float*)nullptr,
+                 device_compute_units());
   }
   return (int)hipGetLastError();
 }

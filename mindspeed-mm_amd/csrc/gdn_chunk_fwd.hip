@@ -948,6 +948,11 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   T* VF = keep ? reinterpret_cast<T*>(ws_state + L.VF) : nullptr;
   T* HF = keep ? reinterpret_cast<T*>(ws_state + L.HF) : nullptr;
   const TokenStrides ts = d.strides();
+  {
+    const int64_t ob = (int64_t)d.Hv * d.V * (int)sizeof(T);
+    TailRows tail{{o, fn.y, fn.y != nullptr ? (void*)fn.rstd : nullptr}, {ob, ob, (int64_t)d.Hv * 4}, {(int)ob, (int)ob, d.Hv * 4}};
+    launch_zero_tail_rows(cu, d.N, d.tokens(), tail, st);
+  }
   if (!skip_prep) {
     auto kern = chunk_prep_kernel<T, DK>;
     constexpr int smem = PrepSmem<T, DK>::bytes;

@@ -103,16 +103,15 @@ __device__ __forceinline__ int xcd_grouped_head(int b, int total, int grp) {
 #endif
 // The workgroups of a launch start together and, doing equal work, stay in step: they all load at the same time and
 // all compute at the same time, and the two workgroups that share a CU do not fill each other's waits.  Holding back
-// the second workgroup of each CU once (workgroup ids are handed out breadth first, so on the 256 CUs of an MI355X
-// these are ids 256..511) shifts it, and every workgroup that later takes over its place, for the rest of the launch.
+// the second workgroup of each CU once (workgroup ids are handed out breadth first, so with `cus` compute units these
+// are ids cus .. 2 cus - 1) shifts it, and every workgroup that later takes over its place, for the rest of the launch.
 // Worth 2 % on the chunk-local backward kernel, measured in alternation with the same build without the wait; nothing
 // on kernels whose phases are shorter or that run one workgroup per CU.  The wait costs its own length once, at the
 // end of the launch, so launches of fewer than `min_groups` workgroups skip it.
 // UNITS: 64 clock cycles each (the argument of s_sleep is an immediate, at most 127).
-constexpr int kStaggerCUs = 256;
-template <int UNITS> __device__ __forceinline__ void stagger_second_resident(int times, int min_groups) {
+template <int UNITS> __device__ __forceinline__ void stagger_second_resident(int times, int min_groups, int cus) {
   const int lin = blockIdx.x + gridDim.x * blockIdx.y;
-  if ((int)(gridDim.x * gridDim.y) >= min_groups && lin >= kStaggerCUs && lin < 2 * kStaggerCUs) {
+  if ((int)(gridDim.x * gridDim.y) >= min_groups && lin >= cus && lin < 2 * cus) {
     for (int i = 0; i < times; ++i) __builtin_amdgcn_s_sleep(UNITS);
   }
 }
@@ -829,6 +828,37 @@ __device__ __forceinline__ SeqInfo locate_chunk(int gchunk, const int64_t* cu_se
   s.chunk = gchunk - chunk_offsets[lo];
   s.nvalid = imin(kChunk, s.len - s.chunk * kChunk);
   return s;
+}
+
+// Rows of packed outputs that belong to no sequence: with cu_seqlens on the device the host cannot check that the last
+// entry equals the number of tokens, and the kernels visit listed chunks only, so rows past cu_seqlens[N] would keep
+// whatever the allocation held.  One workgroup per 64 rows; those before the end of the last sequence leave at once.
+struct TailRows {
+  void* base[6];              // null entries are skipped
+  int64_t row_stride[6];      // bytes between consecutive tokens
+  int row_bytes[6];           // bytes to clear per token (a multiple of 2)
+};
+static __global__ void zero_tail_rows_kernel(const int64_t* __restrict__ cu, int N, int64_t tokens, TailRows t) {
+  const int64_t covered = cu[N], lo = (int64_t)blockIdx.x * 64, hi = lo + 64 < tokens ? lo + 64 : tokens;
+  if (hi <= covered) return;
+  const int64_t first = lo > covered ? lo : covered;
+  for (int a = 0; a < 6; ++a) {
+    if (t.base[a] == nullptr) continue;
+    unsigned char* b = static_cast<unsigned char*>(t.base[a]);
+    if (t.row_bytes[a] % 4 == 0 && t.row_stride[a] % 4 == 0) {
+      const int words = t.row_bytes[a] / 4;
+      for (int64_t i = threadIdx.x; i < (hi - first) * words; i += blockDim.x)
+        reinterpret_cast<uint32_t*>(b + (first + i / words) * t.row_stride[a])[i % words] = 0u;
+    } else {   // rows of an odd number of 16-bit values
+      const int halves = t.row_bytes[a] / 2;
+      for (int64_t i = threadIdx.x; i < (hi - first) * halves; i += blockDim.x)
+        reinterpret_cast<uint16_t*>(b + (first + i / halves) * t.row_stride[a])[i % halves] = 0;
+    }
+  }
+}
+static inline void launch_zero_tail_rows(const int64_t* cu, int N, int64_t tokens, const TailRows& t, hipStream_t st) {
+  if (cu == nullptr || tokens <= 0) return;
+  hipLaunchKernelGGL(zero_tail_rows_kernel, dim3((unsigned)((tokens + 63) / 64)), dim3(256), 0, st, cu, N, tokens, t);
 }
 
 }  // namespace gdn

@@ -648,7 +648,14 @@ static int kda_bwd_launch(const ChunkDims& d, const KdaWorkspace& L, const void*
     GDN_LAUNCH(kKernBwdLocal, st, kern, dim3(nc, H), dim3(kThreads), smem, st, QBT, K1F, (const T*)v, (const void*)bhat, 0,
                (const float*)nullptr, Ai, VF, (const T*)DVF, (const T*)dO, HF, (const T*)DHF, (const float*)nullptr,
                (const float*)nullptr, (T*)nullptr, (T*)nullptr, (T*)dv, (void*)nullptr, (float*)nullptr, cu, chunk_offsets, d.T,
-               d.N, H, H, d.V, scale, 0, ts, DUMP, DD);
+               d.N, H, H, d.V, scale, 0, ts, DUMP, DD, device_compute_units());
+  }
+  {
+    const int es = (int)sizeof(T), ge = fl.g_f32 ? 4 : es, be = fl.beta_f32 ? 4 : es;
+    const int64_t kb = (int64_t)H * DK, vb = (int64_t)H * d.V;
+    TailRows tail{{dq, dk, dv, dg, dbeta}, {kb * es, kb * es, vb * es, kb * ge, (int64_t)H * be},
+                  {(int)(kb * es), (int)(kb * es), (int)(vb * es), (int)(kb * ge), H * be}};
+    launch_zero_tail_rows(cu, d.N, d.tokens(), tail, st);
   }
   {
     auto kern = kda_bwd_finish_kernel<T, DK>;

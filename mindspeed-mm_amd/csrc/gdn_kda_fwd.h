@@ -362,6 +362,11 @@ static int kda_fwd_launch(const ChunkDims& d, const KdaWorkspace& L, const void*
   T* TMR = with_backward ? reinterpret_cast<T*>(ws + L.TMR) : nullptr;
   if (cu != nullptr) GDN_LAUNCH(kKernChunkTable, st, chunk_table_kernel, dim3(1), dim3(kThreads), 0, st, cu, chunk_offsets, d.N);
   {
+    const int64_t ob = (int64_t)H * d.V * (int)sizeof(T);
+    TailRows tail{{o}, {ob}, {(int)ob}};
+    launch_zero_tail_rows(cu, d.N, d.tokens(), tail, st);
+  }
+  {
     auto kern = kda_prep_kernel<T, DK>;
     constexpr int smem = KdaPrepSmem<T, DK>::bytes;
     if (int e = set_lds(kern, smem)) return e;

@@ -124,6 +124,13 @@ class GdnOps:
                                use_qk_l2norm_in_kernel=False, cu_seqlens=None, chunk_size=64, head_first=False,
                                skip_recompute=False):
         scale = self._check_chunk_args(q, k, v, g, beta, scale, initial_state, cu_seqlens, chunk_size, head_first)
+        if q.dtype == torch.float16:
+            # float16 (which the reference's entry accepts, chunk_gated_delta_rule.py:379-386) runs on the float32
+            # kernels: q, k, v are widened, o comes back in float16, and autograd carries the casts
+            o, ht = self.chunk_gated_delta_rule(q.float(), k.float(), v.float(), g, beta, scale, initial_state,
+                                                output_final_state, use_qk_l2norm_in_kernel, cu_seqlens, chunk_size,
+                                                False, skip_recompute)
+            return o.to(torch.float16), ht
         q, k, v, g, beta, initial_state = self._no_grad_views(q, k, v, g, beta, initial_state)
         return _ChunkGatedDeltaRule.apply(q, k, v, g, beta, float(scale), initial_state, bool(output_final_state),
                                           cu_seqlens, bool(use_qk_l2norm_in_kernel), bool(skip_recompute), self)
@@ -164,18 +171,19 @@ class GdnOps:
             raise ValueError(
                 f"q current type is {q.dtype} , k current type is {k.dtype} ,v current type is {v.dtype} , "
                 "they should are equal")
-        if q.dtype not in (torch.float32, torch.bfloat16):
-            raise ValueError(f"chunk_gated_delta_rule supports bfloat16 and float32, got {q.dtype}")
+        if q.dtype not in (torch.float32, torch.bfloat16, torch.float16):
+            raise ValueError(f"chunk_gated_delta_rule supports bfloat16, float16 and float32, got {q.dtype}")
         if len(beta.shape) != 3:
             raise ValueError(
                 f"beta current shape len is {len(beta.shape)}, beta must be of shape [B, T, H] if head_first=False, "
                 "or [B, H, T] otherwise.")
-        if head_first:
-            raise ValueError("head_first=True is deprecated in the reference and not supported here; "
-                             "pass [B, T, H, ...] tensors")
+        if head_first:   # as the reference: a warning, and the tensors are taken as [B, T, H, ...] all the same
+            warnings.warn(
+                "head_first is deprecated and will be removed in a future version. "
+                "Please use head_first=False for now instead.")
         if chunk_size != 64:
             raise ValueError("only chunk_size=64 is supported")
-        if q.shape[1] < q.shape[2]:
+        if not head_first and q.shape[1] < q.shape[2]:
             warnings.warn(
                 f"Input tensor shape suggests potential format mismatch: seq_len ({q.shape[1]}) < num_heads "
                 f"({q.shape[2]}). Please verify your input tensor format matches the expected shape [B, T, H, ...].")
@@ -264,6 +272,11 @@ class GdnOps:
             raise ValueError(f"chunk_kda supports bfloat16 and float32 q, k, v of one dtype, got {q.dtype}, {k.dtype}, {v.dtype}")
         if chunk_size != 64:
             raise ValueError("only chunk_size=64 is supported")
+        if safe_gate and use_gate_in_kernel:   # triton_ascend/chunk.py:373-377
+            if lower_bound is None:
+                raise ValueError("`lower_bound` must be specified when `safe_gate=True` and `use_gate_in_kernel=True`.")
+            if not (-5 <= lower_bound < 0):
+                raise ValueError(f"`lower_bound` must be in the safe range [-5, 0), got {lower_bound}.")
         if return_intermediate_states:
             raise NotImplementedError("return_intermediate_states=True (the per-chunk states in [K,V] order for an "
                                       "inference engine) is not provided: the states are kept in matrix-core tile order")
@@ -1107,9 +1120,10 @@ class ShortConvolution(torch.nn.Conv1d):
         if B * T == N:
             return self.step(x, residual, cache, output_final_state, cu_seqlens)
         weight = self.weight.squeeze(1).transpose(0, 1).contiguous()      # [D, 1, W] -> [W, D]
+        # further keywords (the reference hands them to a kernel that ignores them, short_conv.py:155-166) are dropped
         return causal_conv1d(x=x, weight=weight, bias=self.bias, residual=residual, initial_state=cache,
                              output_final_state=output_final_state, activation=self.activation,
-                             cu_seqlens=cu_seqlens, **kwargs)
+                             cu_seqlens=cu_seqlens)
 
     def step(self, x, residual, cache, output_final_state=False, cu_seqlens=None):
         """One token per sequence: the cache rolls by one and takes the token (short_conv.py:185-213)."""

@@ -2,9 +2,13 @@
 
 Each check runs one operator of the package through the C ABI on seeded inputs and compares it with the
 CPU oracle (oracle/gdn_oracle.py, oracle/kda_oracle.py).  Tolerances are the ones the task states:
-    fp32: max relative error (max|x - ref| / max|ref|) <= 1e-4
-    bf16 vs the fp32 oracle on the same (bf16-valued) inputs: max abs error <= 2e-2 on o,
-          <= 5e-2 on dq/dk/dv/dg/dbeta (and on the states, whose magnitude is O(1)).
+    fp32: "max relative error <= 1e-4", checked in two readings at once:
+          normalised   max|x - ref| <= 1e-4 max|ref|
+          elementwise  |x - ref| <= 1e-4 |ref| + 1e-5 max|ref|   (the floor stands for entries that are themselves the
+                       rounding residue of sums of terms of size max|ref|; an entry a hundred times smaller than the
+                       largest is thereby held to 1e-3 of its own size, one ten thousand times smaller to 1e-1)
+    bf16 vs the fp32 oracle on the same (bf16-valued) inputs: max abs error <= 2e-2 on o and on the final state,
+          <= 5e-2 on dq/dk/dv/dg/dbeta (and on the gradient of the initial state).
 """
 import torch
 
@@ -13,6 +17,7 @@ from oracle import gdn_oracle as O
 from oracle import kda_oracle as KO
 
 FP32_REL = 1e-4
+FP32_FLOOR = 1e-5
 BF16_ABS_O = 2e-2
 BF16_ABS_GRAD = 5e-2
 # dA_log and d(dt_bias) are sums over every token of the batch (dA_log over the channels too) of terms of both signs,
@@ -31,7 +36,8 @@ def kda_param_tol(ref_grad, tokens):
 
 
 def _err(name, got, ref, dtype, abs_tol, rtol=0.0):
-    """fp32: max|x-ref| <= 1e-4 max|ref|.  Half precision: |x-ref| <= abs_tol + rtol |ref| elementwise."""
+    """fp32: max|x-ref| <= 1e-4 max|ref| and |x-ref| <= 1e-4 |ref| + 1e-5 max|ref| elementwise.  Half precision:
+    |x-ref| <= abs_tol + rtol |ref| elementwise."""
     got, ref = got.detach().float().cpu(), ref.detach().float().cpu()
     assert got.shape == ref.shape, f"{name}: shape {tuple(got.shape)} vs {tuple(ref.shape)}"
     assert torch.isfinite(got).all(), f"{name}: non-finite values"
@@ -39,6 +45,10 @@ def _err(name, got, ref, dtype, abs_tol, rtol=0.0):
     scale = ref.abs().max().item() if got.numel() else 0.0
     if dtype == torch.float32:
         assert diff <= FP32_REL * max(scale, 1e-30), f"{name}: max rel err {diff / max(scale, 1e-30):.3e} > {FP32_REL}"
+        if got.numel():
+            over = ((got - ref).abs() - FP32_REL * ref.abs()).max().item()
+            assert over <= FP32_FLOOR * scale, (f"{name}: an entry is off by {over / max(scale, 1e-30):.3e} max|ref| beyond "
+                                                f"{FP32_REL} of its own size (floor {FP32_FLOOR})")
     else:
         excess = ((got - ref).abs() - rtol * ref.abs()).max().item() if got.numel() else 0.0
         assert excess <= abs_tol, f"{name}: max abs err {diff:.3e} > {abs_tol} + {rtol}|ref| (ref max {scale:.3f})"
@@ -46,7 +56,9 @@ def _err(name, got, ref, dtype, abs_tol, rtol=0.0):
 
 
 def check_chunk(ops, device, B, T, Hqk, Hv, K, V, dtype, l2=True, cu=None, backward=False, seed=0, with_h0=True,
-                scale=None, wrap=lambda t: t, skip_recompute=False, **recipe):
+                scale=None, wrap=lambda t: t, skip_recompute=False, grad_rtol=0.0, **recipe):
+    """grad_rtol: half precision only: the gradients are held to 5e-2 + grad_rtol |ref| instead of 5e-2 (for recipes whose
+    gradients grow far beyond 1, where 5e-2 is below the resolution of the 16-bit operands)."""
     N = (len(cu) - 1) if cu is not None else B
     x = gdn_inputs(B, T, Hqk, Hv, K, V, dtype, seed=seed, N=N, l2norm_in_kernel=l2, **recipe)
     dev = {n: wrap(t.to(device)) for n, t in x.items()}
@@ -62,15 +74,15 @@ def check_chunk(ops, device, B, T, Hqk, Hv, K, V, dtype, l2=True, cu=None, backw
                                            ref_leaves["beta"], scale=scale, initial_state=rh0,
                                            output_final_state=True, use_qk_l2norm_in_kernel=l2, cu_seqlens=cu)
     assert o.dtype == dtype and ht.dtype == torch.float32
-    errs = {"o": _err("o", o, ro, dtype, BF16_ABS_O), "ht": _err("final_state", ht, rht, dtype, BF16_ABS_GRAD)}
+    errs = {"o": _err("o", o, ro, dtype, BF16_ABS_O), "ht": _err("final_state", ht, rht, dtype, BF16_ABS_O)}
     if backward:
         ((o.float() * dev["do"].float()).sum() + (ht * dev["dht"]).sum()).backward()
         ((ro * x["do"].float()).sum() + (rht * x["dht"]).sum()).backward()
         for n in ("q", "k", "v", "g", "beta"):
             assert leaves[n].grad.dtype == leaves[n].dtype
-            errs["d" + n] = _err("d" + n, leaves[n].grad, ref_leaves[n].grad, dtype, BF16_ABS_GRAD)
+            errs["d" + n] = _err("d" + n, leaves[n].grad, ref_leaves[n].grad, dtype, BF16_ABS_GRAD, grad_rtol)
         if with_h0:
-            errs["dh0"] = _err("dh0", h0.grad, rh0.grad, dtype, BF16_ABS_GRAD)
+            errs["dh0"] = _err("dh0", h0.grad, rh0.grad, dtype, BF16_ABS_GRAD, grad_rtol)
     return errs
 
 
@@ -244,7 +256,7 @@ def check_chunk_qkv(ops, device, B, T, Hqk, Hv, K, V, dtype, l2=True, cu=None, b
     rh0 = x["h0"].clone().requires_grad_(backward)
     ro, rht = O.chunk_gated_delta_rule_ref(ref["q"], ref["k"], ref["v"], ref["g"], ref["beta"], initial_state=rh0,
                                            output_final_state=True, use_qk_l2norm_in_kernel=l2, cu_seqlens=cu)
-    errs = {"o": _err("o", o, ro, dtype, BF16_ABS_O), "ht": _err("final_state", ht, rht, dtype, BF16_ABS_GRAD)}
+    errs = {"o": _err("o", o, ro, dtype, BF16_ABS_O), "ht": _err("final_state", ht, rht, dtype, BF16_ABS_O)}
     if backward:
         ((o.float() * dev["do"].float()).sum() + (ht * dev["dht"]).sum()).backward()
         ((o2.float() * dev["do"].float()).sum() + (ht2 * dev["dht"]).sum()).backward()
@@ -468,7 +480,7 @@ def check_kda(ops, device, B, T, H, K, V, dtype, cu=None, seed=0, with_h0=True, 
         ro, rht = KO.chunk_kda_ref(ref["q"], ref["k"], ref["v"], ref["g"], ref["beta"], initial_state=ref["h0"] if with_h0 else None,
                                    cu_seqlens=cu, A_log=ref["A_log"], dt_bias=ref["dt_bias"], round_output=False, **kw)
     assert o.dtype == dtype and ht.dtype == torch.float32 and ht.shape == rht.shape
-    errs = {"o": _err("o", o, ro, dtype, BF16_ABS_O), "ht": _err("final_state", ht, rht, dtype, BF16_ABS_GRAD)}
+    errs = {"o": _err("o", o, ro, dtype, BF16_ABS_O), "ht": _err("final_state", ht, rht, dtype, BF16_ABS_O)}
     if backward:
         ((o.float() * dev["do"].float()).sum() + (ht * dev["dht"]).sum()).backward()
         ((ro * x["do"].float()).sum() + (rht * x["dht"]).sum()).backward()

@@ -146,6 +146,63 @@ def test_chunk_rejects_key_width_256(ops):
         ops.chunk_gated_delta_rule(q, q, q, g, b)
 
 
+def test_chunk_rows_past_the_last_sequence_are_cleared(ops):
+    """cu_seqlens on the device cannot be checked against the number of tokens without a synchronisation: rows after
+    the last listed sequence belong to no chunk, and every output row there is written as zero (forward and
+    backward), the rows before it as in a call on the covered tokens alone."""
+    T, Tc, cu = 100, 90, [0, 30, 90]
+    x = P.gdn_inputs(1, T, 1, 2, 64, 64, BF, seed=5, N=2)
+    d = {n: t.cuda() for n, t in x.items()}
+    cu_t = torch.tensor(cu, dtype=torch.int64, device="cuda")
+    outs = []
+    for t_len in (T, Tc):
+        L = {n: d[n][:, :t_len].clone().requires_grad_(True) for n in ("q", "k", "v", "g", "beta")}
+        o, ht = ops.chunk_gated_delta_rule(L["q"], L["k"], L["v"], L["g"], L["beta"], initial_state=d["h0"],
+                                           output_final_state=True, use_qk_l2norm_in_kernel=True, cu_seqlens=cu_t)
+        (o.float() * d["do"][:, :t_len].float()).sum().backward()
+        outs.append((o, ht, {n: L[n].grad for n in L}))
+    (o, ht, gr), (oc, htc, grc) = outs
+    assert torch.equal(o[:, :Tc], oc) and torch.equal(ht, htc) and not o[:, Tc:].any()
+    for n in gr:
+        assert torch.equal(gr[n][:, :Tc], grc[n]), n
+        assert not gr[n][:, Tc:].any(), n
+
+
+def test_chunk_float16(ops):
+    """float16 q, k, v (accepted by the reference's entry, chunk_gated_delta_rule.py:379-386) run through the float32
+    kernels: the output and the gradients come back in float16 and meet the half-precision bounds against the oracle
+    on the same float16-valued inputs."""
+    H16 = torch.float16
+    x = P.gdn_inputs(1, 200, 1, 2, 64, 64, F32, seed=9)
+    x = {n: (t.to(H16) if n in ("q", "k", "v", "do") else t) for n, t in x.items()}
+    d = {n: t.cuda() for n, t in x.items()}
+    L = {n: d[n].clone().requires_grad_(True) for n in ("q", "k", "v", "g", "beta")}
+    R = {n: x[n].float().clone().requires_grad_(True) for n in ("q", "k", "v", "g", "beta")}
+    o, ht = ops.chunk_gated_delta_rule(L["q"], L["k"], L["v"], L["g"], L["beta"], initial_state=d["h0"],
+                                       output_final_state=True, use_qk_l2norm_in_kernel=True)
+    ro, rht = P.O.chunk_gated_delta_rule_ref(R["q"], R["k"], R["v"], R["g"], R["beta"], initial_state=x["h0"],
+                                             output_final_state=True, use_qk_l2norm_in_kernel=True)
+    assert o.dtype == H16 and ht.dtype == F32
+    (o.float() * d["do"].float()).sum().backward()
+    (ro * x["do"].float()).sum().backward()
+    P._err("o", o, ro, H16, P.BF16_ABS_O)
+    P._err("final_state", ht, rht, H16, P.BF16_ABS_O)
+    for n in L:
+        assert L[n].grad.dtype == L[n].dtype
+        P._err("d" + n, L[n].grad, R[n].grad, H16, P.BF16_ABS_GRAD)
+
+
+def test_chunk_head_first_warns_and_proceeds(ops):
+    """head_first=True is deprecated in the reference, which warns and then treats the tensors as [B, T, H, ...]
+    all the same (chunk_gated_delta_rule.py:392-396)."""
+    x = P.gdn_inputs(1, 70, 1, 1, 64, 64, BF, seed=3)
+    d = {n: t.cuda() for n, t in x.items()}
+    with pytest.warns(UserWarning, match="head_first is deprecated"):
+        o1, _ = ops.chunk_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], head_first=True)
+    o2, _ = ops.chunk_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"])
+    assert torch.equal(o1, o2)
+
+
 def test_chunk_under_autocast_keeps_dtypes(ops):
     """custom_fwd / custom_bwd: under torch.autocast the operator still computes in the dtype of its inputs."""
     x = P.gdn_inputs(1, 130, 1, 2, 64, 64, F32, seed=2)
@@ -448,6 +505,18 @@ def test_kda_argument_checks(ops):
         ops.chunk_kda(d["q"], d["k"], d["v"], d["g"], d["beta"], initial_state=d["h0"].bfloat16())
     with pytest.raises(NotImplementedError):
         ops.chunk_kda(d["q"], d["k"], d["v"], d["g"], d["beta"], return_intermediate_states=True)
+    # the safe gate needs its bound, inside [-5, 0) (triton_ascend/chunk.py:373-377)
+    gate = dict(use_gate_in_kernel=True, A_log=d["A_log"], dt_bias=d["dt_bias"], safe_gate=True)
+    with pytest.raises(ValueError, match="must be specified"):
+        ops.chunk_kda(d["q"], d["k"], d["v"], d["g"], d["beta"], **gate)
+    with pytest.raises(ValueError, match="safe range"):
+        ops.chunk_kda(d["q"], d["k"], d["v"], d["g"], d["beta"], lower_bound=-6.0, **gate)
+
+
+def test_kda_log_decay_in_half_precision(ops):
+    """The caller hands over the log decay itself (use_gate_in_kernel=False) in the dtype of q, k, v."""
+    errs = P.check_kda(ops, "cuda", 1, 200, 2, 128, 128, BF, gate_in_kernel=False, g_dtype=BF, backward=True, seed=6)
+    print({n: f"{e:.2e}" for n, e in errs.items()})
 
 
 @pytest.mark.parametrize("dtype,B,T,D,W,cu", [(F32, 2, 37, 16, 4, None), (BF, 1, 300, 64, 4, [0, 1, 3, 130, 131, 300])])
