@@ -191,7 +191,9 @@ int gdn_gate_bwd(const void* a, const void* b, const void* A_log, const void* dt
  * The per-workgroup partial sums live in a 1 MiB buffer inside the library (one per device, held until the process
  * ends), which limits Hv to 128 (-3 beyond); any number of tokens is accepted.  Same kernels and same order of
  * additions as gdn_gate_bwd: identical results.  Calls that overlap on one device (two streams) share that buffer and
- * race; calls on one stream are ordered.  Nothing is allocated, freed or synchronised. */
+ * race; calls on one stream are ordered.  Nothing is allocated, freed or synchronised.  The first call on each device
+ * looks the buffer's address up (hipGetSymbolAddress, which may load the code object): make that one call, with any
+ * small input, before a capture begins or a no-allocation region is entered; every later call only launches kernels. */
 int gdn_gate_bwd_noalloc(const void* a, const void* b, const void* A_log, const void* dt_bias, const float* dg,
                          const void* dbeta, void* da, void* db, float* dA_log, float* ddt_bias, int64_t tokens, int Hv,
                          int dtype, int param_dtype, void* stream);

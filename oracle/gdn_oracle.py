@@ -114,6 +114,9 @@ def naive_gated_delta_rule(
     """
     B, T, Hv, V = v.shape
     K = k.shape[-1]
+    # The reference normalises before its cast to fp32 (:410-415), i.e. in the input dtype; here the cast comes first,
+    # so that a 16-bit input is normalised without an extra rounding (the kernels do the same, in fp32 registers).
+    # For fp32 / fp64 inputs, which the oracle tests use, the two orders coincide.
     q, k, v, g, beta = (x.to(dtype) for x in (q, k, v, g, beta))
     if use_qk_l2norm_in_kernel:
         q, k = l2norm(q), l2norm(k)
@@ -203,6 +206,9 @@ def chunk_gated_delta_rule_ref(
     docstring.  Returns o [B,T,Hv,V] in ``dtype`` and the state in ``dtype``."""
     B, T, Hv, V = v.shape
     K = k.shape[-1]
+    # The reference normalises before its cast to fp32 (:410-415), i.e. in the input dtype; here the cast comes first,
+    # so that a 16-bit input is normalised without an extra rounding (the kernels do the same, in fp32 registers).
+    # For fp32 / fp64 inputs, which the oracle tests use, the two orders coincide.
     q, k, v, g, beta = (x.to(dtype) for x in (q, k, v, g, beta))
     if use_qk_l2norm_in_kernel:
         q, k = l2norm(q), l2norm(k)
@@ -239,6 +245,9 @@ def recurrent_gated_delta_rule_ref(
     scale = K**-0.5 unless given, new state tensor returned."""
     B, T, Hv, V = v.shape
     K = k.shape[-1]
+    # The reference normalises before its cast to fp32 (:410-415), i.e. in the input dtype; here the cast comes first,
+    # so that a 16-bit input is normalised without an extra rounding (the kernels do the same, in fp32 registers).
+    # For fp32 / fp64 inputs, which the oracle tests use, the two orders coincide.
     q, k, v, g, beta = (x.to(dtype) for x in (q, k, v, g, beta))
     if use_qk_l2norm_in_kernel:
         q, k = l2norm(q), l2norm(k)
