@@ -6,8 +6,10 @@
 A step is one chunked gated-delta-rule forward + backward over the configuration the metric is quoted on
 (BASELINE.json configs[1]: B=2, T=8192, H_qk=16, H_v=32, d_k=d_v=128, bf16, in-kernel q/k L2 norm, N(0,0.02)
 initial state, upstream grad ~ N(0,1)); inputs are synthetic and already resident in HBM.  Prints ONE JSON line.
-The step keeps the forward pass's workspace for the backward pass (skip_recompute=True); the operator's default,
-which keeps nothing and recomputes, is timed beside it under aux.
+The step keeps the forward pass's workspace for the backward pass (skip_recompute=True, an option the reference's
+operator has as well); the operator's default call (skip_recompute=False: the input-only part of the workspace is
+kept, states and corrected values are rebuilt in the backward pass) is timed right after it, same K and W, and
+reported beside it in roofline.path.default_mode.
 
   value        tokens/s of fwd+bwd (B*T / step time), measured without per-kernel instrumentation
   roofline     the kernel with the largest share of the step: its algorithmic HBM bytes per launch divided by its
@@ -40,13 +42,31 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 CFG = dict(B=2, T=8192, Hqk=16, Hv=32, K=128, V=128, C=64)
 
 # HBM bytes per launch of each kernel on CFG, read + written, from the hardware counters FETCH_SIZE and WRITE_SIZE
-# (rocprofv3 --pmc, one run per counter, each scaled by what the same counter reads for a 512 MiB copy): the figures
-# of the file named below.  Measured offline on the kernels as they are in this tree, reported beside the live timings.
+# (rocprofv3 --pmc, one run per counter, each scaled by what the same counter reads for a 512 MiB copy).  They are
+# collected offline and live in the tracked summary named below, which is the only place they are written down:
+# this script reads its table of the benchmark shape and reports the figures beside the live timings.
 TRAFFIC_SOURCE = "profiles/chunk_fwd_bwd_B2_T8192_bf16_hbm_traffic.md"
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "chunk_prep_kernel": 413194211, "chunk_state_kernel": 926225572,
-    "chunk_state_bwd_kernel": 791955313, "chunk_bwd_local_kernel": 1070646198,
-}
+
+
+def measured_traffic_bytes_per_launch():
+    """{kernel: bytes per launch} from the first table of TRAFFIC_SOURCE (rows `| kernel<...> | ... | bytes |`, the last
+    column being bytes per launch); empty when the file is missing, and the traffic fields are then null."""
+    out, in_main = {}, False
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_SOURCE)) as f:
+            lines = f.read().splitlines()
+    except OSError:
+        return out
+    for ln in lines:
+        if ln.startswith("## "):
+            in_main = ln.startswith("## Chunk fwd+bwd at the benchmark shape")
+        elif in_main and ln.startswith("| chunk_"):
+            cells = [c.strip() for c in ln.strip().strip("|").split("|")]
+            try:
+                out[cells[0].split("<")[0]] = int(cells[-1])
+            except ValueError:
+                pass
+    return out
 
 
 CLOCK_RAMP_S = 0.5   # untimed run of the benchmark step before the warm-up steps (see main)
@@ -157,6 +177,15 @@ def main():
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     value = tokens / (ms_per_step * 1e-3)
+    # the operator's default call, timed the same way
+    for _ in range(args.warmup):
+        step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(False)
+    torch.cuda.synchronize()
+    ms_default = (time.perf_counter() - t0) * 1e3 / args.steps
 
     # ---- spread of the step time: each of max(steps, 50) further steps bracketed by events on the launch stream ----
     nspread = max(args.steps, 50)
@@ -204,11 +233,10 @@ def main():
     path_tflops = ref_formula_flops(tokens, c["Hv"], c["K"], c["V"]) / (ms_per_step * 1e-3) / 1e12
     min_bytes = minimal_bytes(c["B"], c["T"], c["B"], c["Hqk"], c["Hv"], c["K"], c["V"])
     interface_total = sum(abytes[n] * nchunk_heads for n in per_kernel if n in abytes)
-    measured = [MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(n) for n in per_kernel if n in abytes]
+    traffic_table = measured_traffic_bytes_per_launch()
     traffic_total = None
-    if all(m is not None for m in measured):
-        traffic_total = sum(MEASURED_TRAFFIC_BYTES_PER_LAUNCH[n] * per_kernel[n]["launches_per_step"]
-                            for n in per_kernel if n in abytes)
+    if all(n in traffic_table for n in per_kernel if n in abytes):
+        traffic_total = sum(traffic_table[n] * per_kernel[n]["launches_per_step"] for n in per_kernel if n in abytes)
     # the whole step against both roofs: the operator's minimal bytes (inputs and outputs only) and the reference's
     # FLOP count say what an ideal implementation would need; the kernels' own interfaces move more (intermediates
     # between the launches), which is what the per-kernel figures above are measured against
@@ -221,9 +249,18 @@ def main():
             "kernel_interface_bytes_per_step": int(interface_total),
             "interface_over_minimal": round(interface_total / min_bytes, 2),
             "traffic_per_step_total": None if traffic_total is None else int(traffic_total),
-            "traffic_over_minimal": None if traffic_total is None else round(traffic_total / min_bytes, 2)}
+            "traffic_over_minimal": None if traffic_total is None else round(traffic_total / min_bytes, 2),
+            # skip_recompute=False, the call a user of the reference makes without changing anything
+            "default_mode": {"ms_per_step": round(ms_default, 4), "tokens_per_s": round(tokens / (ms_default * 1e-3), 1),
+                             "tflops_ref_formula": round(path_tflops * ms_per_step / ms_default, 2),
+                             "frac_mfma_ref_formula": round(path_tflops * ms_per_step / ms_default / PEAK_BF16_TFLOPS, 4),
+                             "frac_hbm_minimal": round(min_bytes / (ms_default * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                             "kept_between_passes_bytes": int(lib.gdn_chunk_workspace_bytes(
+                                 c["B"], c["T"], c["B"], c["Hqk"], c["Hv"], c["K"], c["V"], 1, 2)),
+                             "stored_mode_kept_bytes": int(lib.gdn_chunk_workspace_bytes(
+                                 c["B"], c["T"], c["B"], c["Hqk"], c["Hv"], c["K"], c["V"], 1, 1))}}
     roofline = {"kernel": dom, "bound": "hbm", "achieved": round(dom_gbps, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                "frac": round(dom_gbps / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(dom),
+                "frac": round(dom_gbps / PEAK_HBM_GBS, 4), "traffic": traffic_table.get(dom),
                 "traffic_source": TRAFFIC_SOURCE + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, collected offline)",
                 "algorithmic_bytes_per_launch": int(bytes_per_launch), "launches_per_step": launches,
                 "avg_launch_ms": per_kernel[dom]["avg_ms"],
@@ -385,11 +422,14 @@ def main():
                                            output_final_state=True, use_qk_l2norm_in_kernel=True)
         pf = wall_ms(prefill_step, 20)
         aux["forward_only"] = {"ms": round(pf, 4), "tokens_per_s": round(tokens / (pf * 1e-3), 1)}
+        two_streams = ops.two_stream_backward
+        ops.two_stream_backward = False
         rc = wall_ms(lambda: step(False), 20)
-        aux["default_mode_recompute_in_backward"] = {
+        ops.two_stream_backward = two_streams
+        aux["default_mode_on_one_stream"] = {
             "ms_per_step": round(rc, 4), "tokens_per_s": round(tokens / (rc * 1e-3), 1),
-            "note": "skip_recompute=False: only the inputs are kept between the passes, the backward pass refills a "
-                    "workspace (chunk-local kernel and recurrence) first"}
+            "note": "skip_recompute=False with the backward pass's rebuild of states and corrected values queued in "
+                    "front of the reverse recurrence instead of beside it on a second stream"}
         zg = torch.randn(c["B"], c["T"], c["Hv"], c["V"], generator=gen).to(dev, torch.bfloat16)
         nw = torch.ones(c["V"], device=dev, dtype=torch.bfloat16)
 
@@ -557,7 +597,8 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "GDN chunk forward+backward, B=2 T=8192 H_qk=16 H_v=32 d_k=d_v=128 chunk=64, "
                                "use_qk_l2norm_in_kernel, initial state N(0,0.02), native grouped q/k heads, "
-                               "skip_recompute=True (forward workspace kept for the backward pass)",
+                               "skip_recompute=True (forward workspace kept for the backward pass); the default call "
+                               "(skip_recompute=False) is timed beside it: roofline.path.default_mode",
                    "global_batch": c["B"], "seq_len": c["T"], "parallelism": "single GPU"},
         "roofline": roofline, "cpu_baseline": cpu, "aux": aux,
     }
