@@ -219,6 +219,15 @@ int gdn_kda_fwd(const void* q, const void* k, const void* v, const void* g, cons
                 float scale, int use_qk_l2norm, int use_gate, int has_lower_bound, float lower_bound, int beta_sigmoid,
                 int allow_neg_eigval, int dtype, int g_dtype, int beta_dtype, void* stream);
 
+/* chunk_kda(..., return_intermediate_states=True) (chunk_kda_naive.py:287-303, :375-380; triton_ascend/chunk.py:149-151,
+ * an inference-time option): the state at the entry of every chunk of 64 tokens, from the workspace a gdn_kda_fwd call
+ * with the same B, T, N, H, K, V, dtype and cu_seqlens filled.  h_out [h_chunks, H, K, V], or [h_chunks, H, V, K] with
+ * transpose_state_layout, in `dtype`; chunk c of batch row b is row b * ceil(T/64) + c, packed input lists the chunks
+ * of its sequences in order (h_chunks = sum of ceil(len/64); chunks past h_chunks are not written). */
+int gdn_kda_intermediate_states(const void* workspace, int64_t workspace_bytes, const int64_t* cu_seqlens, void* h_out,
+                                int64_t h_chunks, int B, int T, int N, int H, int K, int V, int transpose_state_layout,
+                                int dtype, void* stream);
+
 /* Backward pass of gdn_kda_fwd: needs the workspace that call filled when it was sized with with_backward = 1, and the
  * same q, k, v, g, A_log, dt_bias, cu_seqlens and options.  The reference has no hand-written counterpart in its tree
  * (it differentiates chunk_kda_naive.py:106-221 with autograd; the fused operator's backward,

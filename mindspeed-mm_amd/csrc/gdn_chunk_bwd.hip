@@ -265,8 +265,8 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
 #pragma unroll
     for (int kt = 0; kt < NKT; ++kt) dSb[kt].store_stream(dhf + (tile0 * NKT + kt) * 1024);
     // dV' = (scale tril(Q K^T . Gam))^T dO (from the forward pass's tiles) + (e^{G_last-G} . K) dS, one accumulation
-    // chain per 32-token block.  The A-operand tiles come from LDS two tiles ahead of the matrix instructions that use
-    // them; the decay of dS rides in between.
+    // chain per 32-token block.  The pair of A-operand tiles of K tile kt + 1 is requested from LDS before the matrix
+    // instructions of K tile kt are issued (two register buffers); the decay of dS rides in between.
     f32x16 a0 = acc_zero(), a1 = acc_zero();
     AccB<T> af[2][2];                         // [buffer][tile of the pair]
     af[0][0].load(Ka);

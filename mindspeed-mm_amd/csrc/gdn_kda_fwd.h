@@ -396,6 +396,66 @@ static int kda_fwd_launch(const ChunkDims& d, const KdaWorkspace& L, const void*
 
 }  // namespace gdn
 
+namespace gdn {
+// chunk_kda(..., return_intermediate_states=True) (chunk_kda_naive.py:287-303, :375-380): the state at the entry of
+// every chunk.  The recurrence left it in the workspace as fragment-order tiles (lane <-> V column, registers <-> K
+// row, tile (V block, K block) of chunk and head at ((ch * V/32 + vb) * K/32 + kt) * 1024); here it is written out as
+// [chunks, H, K, V] or, transposed, [chunks, H, V, K] in the operand type.  One workgroup per (chunk, head), the tiles
+// dealt to its four waves.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void kda_states_out_kernel(const T* __restrict__ hf, T* __restrict__ out,
+                                                                 const int64_t* __restrict__ cu,
+                                                                 const int* __restrict__ chunk_offsets, int N, int T_len,
+                                                                 int H, int K, int V, int transposed, int64_t out_chunks) {
+  const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
+  if (s.nvalid <= 0 || (int64_t)blockIdx.x >= out_chunks) return;
+  const int wave = threadIdx.x >> 6, nkt = K / 32, nvb = V / 32;
+  const int64_t ch = (int64_t)blockIdx.x * H + blockIdx.y;
+  T* dst = out + ch * K * V;
+  IdentityFrag<T> id;
+  id.init();
+  T* patch = reinterpret_cast<T*>(gdn_smem) + wave * Patch<T>::kElems;
+  for (int t = wave; t < nkt * nvb; t += kThreads / 64) {
+    const int vb = t / nkt, kt = t % nkt;
+    AccB<T> f;
+    f.load(hf + (ch * nvb * nkt + t) * 1024);
+    const f32x16 c = f.unpack();
+    if (transposed) acc_to_lds_t<T>(c, dst, K, 32 * kt, 32 * vb);
+    else acc_store_rows<T, false>(c, id, patch, dst + (int64_t)32 * kt * V + 32 * vb, V, 32);
+  }
+}
+
+template <typename T>
+static int kda_states_out_launch(const ChunkDims& d, const KdaWorkspace& L, const unsigned char* ws, const int64_t* cu,
+                                 void* out, int64_t out_chunks, int transposed, hipStream_t st) {
+  const int smem = 4 * Patch<T>::kElems * (int)sizeof(T);
+  hipLaunchKernelGGL(kda_states_out_kernel<T>, dim3((unsigned)d.max_chunks(), d.Hv), dim3(kThreads), smem, st,
+                     reinterpret_cast<const T*>(ws + L.HF), static_cast<T*>(out), cu,
+                     reinterpret_cast<const int*>(ws + L.chunk_offsets), d.N, d.T, d.Hv, d.K, d.V, transposed, out_chunks);
+  return (int)hipGetLastError();
+}
+}  // namespace gdn
+
+extern "C" int gdn_kda_intermediate_states(const void* workspace, int64_t workspace_bytes, const int64_t* cu_seqlens,
+                                           void* h_out, int64_t h_chunks, int B, int T, int N, int H, int K, int V,
+                                           int transpose_state_layout, int dtype, void* stream) {
+  using namespace gdn;
+  if (!workspace || !h_out) return -1;
+  ChunkDims d{B, T, N, H, H, K, V, cu_seqlens != nullptr};
+  if (int e = chunk_check_dims(d, dtype)) return e;
+  if (h_chunks < 0) return -2;
+  if ((uintptr_t)h_out & 15) return -6;
+  ChunkDims dl = d;
+  dl.varlen = true;
+  const KdaWorkspace L = kda_workspace_layout(dl, dtype == 0 ? 4 : 2);
+  if (workspace_bytes < L.fwd_bytes || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
+  if (h_chunks == 0) return 0;
+  const unsigned char* ws = static_cast<const unsigned char*>(workspace);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == 1) return kda_states_out_launch<bf16_t>(d, L, ws, cu_seqlens, h_out, h_chunks, transpose_state_layout, st);
+  return kda_states_out_launch<float>(d, L, ws, cu_seqlens, h_out, h_chunks, transpose_state_layout, st);
+}
+
 extern "C" int64_t gdn_kda_workspace_bytes(int B, int T, int N, int H, int K, int V, int with_backward, int dtype) {
   gdn::ChunkDims d{B, T, N, H, H, K, V, true};   // the packed bound is the larger
   const gdn::KdaWorkspace w = gdn::kda_workspace_layout(d, dtype == 0 ? 4 : 2);

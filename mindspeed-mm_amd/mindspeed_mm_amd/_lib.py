@@ -36,6 +36,7 @@ SIGNATURES = {
     "gdn_gate_bwd_noalloc": (I, [P] * 10 + [L, I, I, I, P]),
     "gdn_kda_workspace_bytes": (L, [I] * 8),
     "gdn_kda_fwd": (I, [P] * 12 + [L] + [I] * 6 + [F, I, I, I, F, I, I, I, I, I, P]),
+    "gdn_kda_intermediate_states": (I, [P, L, P, P, L] + [I] * 8 + [P]),
     "gdn_kda_bwd": (I, [P] * 18 + [L] + [I] * 6 + [F, I, I, I, F, I, I, I, I, I, P]),
     "gdn_profile_enable": (I, [I]),
     "gdn_profile_kernel_count": (I, []),

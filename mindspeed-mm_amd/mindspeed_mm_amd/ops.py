@@ -256,7 +256,10 @@ class GdnOps:
         checks of chunk_kda (triton_ascend/chunk.py:215-407) and chunk_kda_naive (chunk_kda_naive.py:223-381):
         q, k, g [B,T,H,K], v [B,T,H,V], beta [B,T,H]; A_log [H] and dt_bias [H*K] come as keyword arguments when
         use_gate_in_kernel is set.  safe_gate, disable_recompute, skip_recompute and cu_seqlens_cpu are hints of the
-        reference's kernels without effect on the result and are accepted and ignored."""
+        reference's kernels without effect on the result and are accepted and ignored.
+        return_intermediate_states=True adds a third result: the state at the entry of every chunk of 64 tokens,
+        [B, NT, H, K, V] ([B, NT, H, V, K] with transpose_state_layout) in the dtype of q; packed input: B = 1 and NT
+        counts the chunks of all sequences (chunk_kda_naive.py:287-303).  It carries no gradient."""
         A_log, dt_bias = kwargs.get("A_log"), kwargs.get("dt_bias")
         if use_gate_in_kernel and A_log is None:
             raise ValueError("A_log must be provided when use_gate_in_kernel=True.")
@@ -277,9 +280,6 @@ class GdnOps:
                 raise ValueError("`lower_bound` must be specified when `safe_gate=True` and `use_gate_in_kernel=True`.")
             if not (-5 <= lower_bound < 0):
                 raise ValueError(f"`lower_bound` must be in the safe range [-5, 0), got {lower_bound}.")
-        if return_intermediate_states:
-            raise NotImplementedError("return_intermediate_states=True (the per-chunk states in [K,V] order for an "
-                                      "inference engine) is not provided: the states are kept in matrix-core tile order")
         N = q.shape[0]
         if cu_seqlens is not None:
             if q.shape[0] != 1:
@@ -300,11 +300,14 @@ class GdnOps:
         q, k, v, g, beta, initial_state, A_log, dt_bias = self._no_grad_views(q, k, v, g, beta, initial_state, A_log, dt_bias)
         if transpose_state_layout and initial_state is not None:
             initial_state = initial_state.transpose(-1, -2)
-        o, ht = _ChunkKda.apply(q, k, v, g, beta, A_log, dt_bias, float(scale), initial_state, bool(output_final_state),
-                                bool(use_qk_l2norm_in_kernel), bool(use_gate_in_kernel), bool(use_beta_sigmoid_in_kernel),
-                                bool(allow_neg_eigval), cu_seqlens, lower_bound, self)
+        o, ht, hs = _ChunkKda.apply(q, k, v, g, beta, A_log, dt_bias, float(scale), initial_state,
+                                    bool(output_final_state), bool(use_qk_l2norm_in_kernel), bool(use_gate_in_kernel),
+                                    bool(use_beta_sigmoid_in_kernel), bool(allow_neg_eigval), cu_seqlens, lower_bound,
+                                    bool(return_intermediate_states), bool(transpose_state_layout), self)
         if ht is not None and transpose_state_layout:
             ht = ht.transpose(-1, -2)
+        if return_intermediate_states:
+            return o, ht, hs
         return o, ht
 
     def gdn_gates(self, a, b, A_log, dt_bias):
@@ -732,7 +735,7 @@ class _ChunkKda(torch.autograd.Function):
     @_input_guard
     @_custom_fwd
     def forward(ctx, q, k, v, g, beta, A_log, dt_bias, scale, initial_state, output_final_state, l2norm, use_gate,
-                beta_sigmoid, allow_neg, cu_seqlens, lower_bound, ops):
+                beta_sigmoid, allow_neg, cu_seqlens, lower_bound, want_states, transposed_states, ops):
         lib = ops.lib
         B, T, H, K = q.shape
         V = v.shape[3]
@@ -756,18 +759,32 @@ class _ChunkKda(torch.autograd.Function):
         rc = lib.gdn_kda_fwd(ptr(qc), ptr(kc), ptr(vc), ptr(gc), ptr(bc), ptr(a32), ptr(d32), ptr(h0), ptr(cu), ptr(o),
                              ptr(ht), ptr(ws), nbytes, B, T, N, H, K, V, scale, *opts, lib.stream())
         lib.check(rc, "gdn_kda_fwd")
+        hs = None
+        if want_states:
+            # the states at chunk entries, from the tiles the recurrence left in the workspace; the number of chunks of a
+            # packed batch needs the sequence lengths on the host (the reference reads them there as well)
+            if cu_seqlens is None:
+                rows, nt = B, (T + 63) // 64
+            else:
+                c = cu_seqlens.tolist() if torch.is_tensor(cu_seqlens) else list(cu_seqlens)
+                rows, nt = 1, sum((int(b) - int(a) + 63) // 64 for a, b in zip(c[:-1], c[1:]))
+            hs = torch.empty((rows, nt, H, V, K) if transposed_states else (rows, nt, H, K, V), dtype=q.dtype, device=q.device)
+            rc = lib.gdn_kda_intermediate_states(ptr(ws), nbytes, ptr(cu), ptr(hs), rows * nt, B, T, N, H, K, V,
+                                                 int(transposed_states), code, lib.stream())
+            lib.check(rc, "gdn_kda_intermediate_states")
+            ctx.mark_non_differentiable(hs)
         if need_grad:
             ctx.save_for_backward(qc, kc, vc, gc, a32, d32, cu, ws)
             ctx.meta = (B, T, N, H, K, V, scale, opts, nbytes, g.dtype, beta.dtype, bc.dtype,
                         None if A_log is None else A_log.dtype, None if dt_bias is None else (dt_bias.dtype, dt_bias.shape),
                         None if initial_state is None else initial_state.dtype)
             ctx.ops = ops
-        return o, ht
+        return o, ht, hs
 
     @staticmethod
     @_input_guard
     @_custom_bwd
-    def backward(ctx, do, dht):
+    def backward(ctx, do, dht, _dhs=None):
         qc, kc, vc, gc, a32, d32, cu, ws = ctx.saved_tensors
         B, T, N, H, K, V, scale, opts, nbytes, g_dt, b_dt, bc_dt, a_dt, d_dt, h_dt = ctx.meta
         lib = ctx.ops.lib
@@ -786,7 +803,7 @@ class _ChunkKda(torch.autograd.Function):
         lib.check(rc, "gdn_kda_bwd")
         return (dq, dk, dv, dg.to(g_dt), db.to(b_dt), None if dA is None else dA.to(a_dt),
                 None if dD is None else dD.to(d_dt[0]).reshape(d_dt[1]), None, None if dh0 is None else dh0.to(h_dt),
-                None, None, None, None, None, None, None, None)
+                None, None, None, None, None, None, None, None, None, None)
 
 
 class _GdnGates(torch.autograd.Function):

@@ -97,7 +97,8 @@ def naive_kda_recurrence(q, k, v, g, beta, scale: Optional[float] = None,
 
 def _kda_chunks(q, k, v, g, beta, scale, S0, chunk: int):
     """One sequence, all heads: q,k,g [T,H,K], v [T,H,V], beta [T,H] in the compute type; S0 [H,K,V].
-    Returns o [T,H,V] and the final state (chunk_kda_naive.py:139-216)."""
+    Returns o [T,H,V], the final state and the state at the entry of every chunk [nc,H,K,V]
+    (chunk_kda_naive.py:139-216)."""
     T, H, K = k.shape
     V = v.shape[-1]
     dt = k.dtype
@@ -132,14 +133,15 @@ def _kda_chunks(q, k, v, g, beta, scale, S0, chunk: int):
     W = Tm @ (beta[..., None] * k * G.exp())                     # [H, nc, C, K]
     Aq = scale * qk * lower
     S = S0
-    outs = []
+    outs, entries = [], []
     for c in range(nc):
+        entries.append(S)
         vn = U[:, c] - W[:, c] @ S                               # what the chunk writes, net of what the state holds
         outs.append(scale * (q[:, c] * G[:, c].exp()) @ S + Aq[:, c] @ vn)
         glast = G[:, c, -1]                                      # [H, K]
         S = glast.exp()[:, :, None] * S + (k[:, c] * (glast[:, None, :] - G[:, c]).exp()).transpose(-1, -2) @ vn
     o = torch.stack(outs, dim=1).reshape(H, nc * chunk, V)[:, :T].permute(1, 0, 2)
-    return o, S
+    return o, S, torch.stack(entries)
 
 
 def chunk_kda_ref(q, k, v, g, beta, scale: Optional[float] = None, initial_state: Optional[torch.Tensor] = None,
@@ -148,10 +150,14 @@ def chunk_kda_ref(q, k, v, g, beta, scale: Optional[float] = None, initial_state
                   allow_neg_eigval: bool = False, cu_seqlens=None, lower_bound: Optional[float] = None,
                   transpose_state_layout: bool = False, A_log: Optional[torch.Tensor] = None,
                   dt_bias: Optional[torch.Tensor] = None, chunk_size: int = 64,
-                  compute_dtype: torch.dtype = torch.float32, round_output: bool = True
-                  ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+                  compute_dtype: torch.dtype = torch.float32, round_output: bool = True,
+                  return_intermediate_states: bool = False):
     """The operator as the reference states it (chunk_kda_naive.py:223-381).  ``compute_dtype`` float64 and
-    ``round_output=False`` turn it into a differentiable high-precision version of the same algebra."""
+    ``round_output=False`` turn it into a differentiable high-precision version of the same algebra.
+    ``return_intermediate_states`` adds a third result, the state at the entry of every chunk, [B, NT, H, K, V]
+    ([.., V, K] with the transposed layout) in the input type, packed input: B = 1 and the chunks of all sequences in
+    order, as the reference documents it (:287-303, :375-380).  (Its own loop stores them with ``h[:, :, i] = S`` into
+    a [B, NT, H, K, V] buffer, :196-203, which only runs where NT == H; the documented meaning is what is stated here.)"""
     B, T, H, K = k.shape
     if allow_neg_eigval and not use_beta_sigmoid_in_kernel:
         raise ValueError("allow_neg_eigval needs use_beta_sigmoid_in_kernel")
@@ -174,12 +180,13 @@ def chunk_kda_ref(q, k, v, g, beta, scale: Optional[float] = None, initial_state
     V = v.shape[-1]
     o = torch.zeros(B, T, H, V, dtype=compute_dtype)
     pieces = [[] for _ in range(B)]
-    finals = []
+    finals, entries = [], [[] for _ in range(B)]
     for n, (b, s, e) in enumerate(_seqs(cu_seqlens, B, T)):
         S0 = torch.zeros(H, K, V, dtype=compute_dtype) if h0 is None else h0[n].to(compute_dtype)
         if e > s:
-            on, S0 = _kda_chunks(q[b, s:e], k[b, s:e], v[b, s:e], gl[b, s:e], beta[b, s:e], scale, S0, chunk_size)
+            on, S0, hs = _kda_chunks(q[b, s:e], k[b, s:e], v[b, s:e], gl[b, s:e], beta[b, s:e], scale, S0, chunk_size)
             pieces[b].append((s, e, on))
+            entries[b].append(hs)
         finals.append(S0)
     rows = []
     for b in range(B):
@@ -200,4 +207,9 @@ def chunk_kda_ref(q, k, v, g, beta, scale: Optional[float] = None, initial_state
         ht = torch.stack(finals)
         if transpose_state_layout:
             ht = ht.transpose(-1, -2)
+    if return_intermediate_states:
+        h = torch.stack([torch.cat(e) if e else o.new_zeros(0, H, K, V) for e in entries])
+        if transpose_state_layout:
+            h = h.transpose(-1, -2)
+        return o, ht, (h.to(in_dtype) if round_output else h)
     return o, ht

@@ -449,10 +449,11 @@ def check_decode_step(ops, device, B, steps, Hqk, Hv, K, V, W, dtype, param_dtyp
 
 def check_kda(ops, device, B, T, H, K, V, dtype, cu=None, seed=0, with_h0=True, gate_in_kernel=True, lower_bound=None,
               beta_sigmoid=True, allow_neg=False, l2=True, transpose_state=True, g_dtype=None, scale=None, backward=False,
-              wrap=lambda t: t, **recipe):
+              wrap=lambda t: t, states=False, **recipe):
     """chunk_kda against the oracle's statement of chunk_kda_naive, with the options of the layer's call
     (modeling_kimi_linear.py:681-699: raw gate and beta, l2 norm in the kernel, [N,H,V,K] states) or without them.
-    backward: every gradient against autograd through the oracle (loss = <o, do> + <final state, dht>)."""
+    backward: every gradient against autograd through the oracle (loss = <o, do> + <final state, dht>).
+    states: also return_intermediate_states=True, the state at every chunk entry against the oracle's."""
     N = (len(cu) - 1) if cu is not None else B
     x = kda_inputs(B, T, H, K, V, dtype, seed=seed, N=N, **recipe)
     if not gate_in_kernel:   # the caller hands over the log decay itself
@@ -472,15 +473,18 @@ def check_kda(ops, device, B, T, H, K, V, dtype, cu=None, seed=0, with_h0=True, 
     cu_t = torch.tensor(cu, dtype=torch.int64, device=device) if cu is not None else None
     kw = dict(scale=scale, output_final_state=True, use_qk_l2norm_in_kernel=l2, use_gate_in_kernel=gate_in_kernel,
               use_beta_sigmoid_in_kernel=beta_sigmoid, allow_neg_eigval=allow_neg, lower_bound=lower_bound if gate_in_kernel else None,
-              transpose_state_layout=transpose_state)
+              transpose_state_layout=transpose_state, return_intermediate_states=states)
     with torch.set_grad_enabled(backward):
-        o, ht = ops.chunk_kda(leaves["q"], leaves["k"], leaves["v"], leaves["g"], leaves["beta"],
+        o, ht, *hs = ops.chunk_kda(leaves["q"], leaves["k"], leaves["v"], leaves["g"], leaves["beta"],
                               initial_state=leaves["h0"] if with_h0 else None, cu_seqlens=cu_t,
                               safe_gate=lower_bound is not None, A_log=leaves["A_log"], dt_bias=leaves["dt_bias"], **kw)
-        ro, rht = KO.chunk_kda_ref(ref["q"], ref["k"], ref["v"], ref["g"], ref["beta"], initial_state=ref["h0"] if with_h0 else None,
+        ro, rht, *rhs = KO.chunk_kda_ref(ref["q"], ref["k"], ref["v"], ref["g"], ref["beta"], initial_state=ref["h0"] if with_h0 else None,
                                    cu_seqlens=cu, A_log=ref["A_log"], dt_bias=ref["dt_bias"], round_output=False, **kw)
     assert o.dtype == dtype and ht.dtype == torch.float32 and ht.shape == rht.shape
     errs = {"o": _err("o", o, ro, dtype, BF16_ABS_O), "ht": _err("final_state", ht, rht, dtype, BF16_ABS_O)}
+    if states:
+        assert len(hs) == 1 and hs[0].dtype == dtype and not hs[0].requires_grad
+        errs["h"] = _err("intermediate states", hs[0], rhs[0], dtype, BF16_ABS_O)
     if backward:
         ((o.float() * dev["do"].float()).sum() + (ht * dev["dht"]).sum()).backward()
         ((ro * x["do"].float()).sum() + (rht * x["dht"]).sum()).backward()

@@ -226,3 +226,14 @@ def test_kda_forward(ops, dtype, B, T, H, K, V, cu, kw):
 def test_kda_backward(ops, dtype, B, T, H, K, V, cu, kw):
     errs = P.check_kda(ops, "cpu", B, T, H, K, V, dtype, cu=cu, backward=True, wrap=guarded, h0_std=0.1, **kw)
     print({n: f"{e:.2e}" for n, e in errs.items()})
+
+
+@pytest.mark.parametrize("dtype,B,T,H,K,V,cu,kw", [
+    (F32, 2, 100, 2, 128, 64, None, {}),
+    (BF, 1, 200, 2, 64, 128, [0, 70, 70, 200], dict(transpose_state=False)),
+    (BF, 1, 130, 1, 128, 128, None, dict(with_h0=False)),
+])
+def test_kda_intermediate_states(ops, dtype, B, T, H, K, V, cu, kw):
+    """The states at chunk entries, written out from the workspace's tiles in both layouts."""
+    errs = P.check_kda(ops, "cpu", B, T, H, K, V, dtype, cu=cu, wrap=guarded, h0_std=0.1, states=True, **kw)
+    assert "h" in errs

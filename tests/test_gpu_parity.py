@@ -492,6 +492,22 @@ def test_kda_backward(ops, dtype, B, T, H, K, V, cu, kw):
     print("   ", {n: f"{e:.2e}" for n, e in errs.items()}, flush=True)
 
 
+@pytest.mark.parametrize("dtype", [BF, torch.float32])
+@pytest.mark.parametrize("B,T,H,K,V,cu,transposed", [
+    (2, 150, 2, 128, 128, None, True),              # dense batch, a partial last chunk
+    (1, 200, 3, 64, 128, [0, 70, 70, 200], False),  # packed, an empty sequence, [K,V] layout, K != V
+    (1, 64, 1, 128, 64, None, False),               # one chunk: the state at its entry is the initial state
+])
+def test_kda_intermediate_states(ops, dtype, B, T, H, K, V, cu, transposed):
+    """return_intermediate_states=True: the state at every chunk entry, [B, NT, H, K, V] or [.., V, K] in the input
+    type (chunk_kda_naive.py:287-303), against the oracle; nothing else about the call changes."""
+    e = P.check_kda(ops, "cuda", B, T, H, K, V, dtype, cu=cu, transpose_state=transposed, states=True, seed=21)
+    assert "h" in e
+    # under autograd the states come back without a gradient and the other results keep theirs
+    e = P.check_kda(ops, "cuda", B, T, H, K, V, dtype, cu=cu, transpose_state=transposed, states=True, backward=True, seed=22)
+    assert "dq" in e and "h" in e
+
+
 def test_kda_argument_checks(ops):
     x = P.kda_inputs(1, 64, 2, 64, 64, BF)
     d = {n: t.cuda() for n, t in x.items()}
@@ -503,8 +519,6 @@ def test_kda_argument_checks(ops):
         ops.chunk_kda(d["q"], d["k"], d["v"], d["g"][..., :32], d["beta"])
     with pytest.raises(ValueError):
         ops.chunk_kda(d["q"], d["k"], d["v"], d["g"], d["beta"], initial_state=d["h0"].bfloat16())
-    with pytest.raises(NotImplementedError):
-        ops.chunk_kda(d["q"], d["k"], d["v"], d["g"], d["beta"], return_intermediate_states=True)
     # the safe gate needs its bound, inside [-5, 0) (triton_ascend/chunk.py:373-377)
     gate = dict(use_gate_in_kernel=True, A_log=d["A_log"], dt_bias=d["dt_bias"], safe_gate=True)
     with pytest.raises(ValueError, match="must be specified"):

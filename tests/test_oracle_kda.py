@@ -196,3 +196,41 @@ def test_golden_vectors():
     ((o * t["do"]).sum() + (ht * t["dht"]).sum()).backward()
     for n, leaf in zip(("dq", "dk", "dv", "dg", "dbeta", "dh0", "dA_log", "ddt_bias"), leaves):
         torch.testing.assert_close(leaf.grad, t[n], rtol=1e-7, atol=1e-9)
+
+
+def test_intermediate_states_are_the_recurrence_states_at_chunk_entries():
+    """h[:, c] is the state the per-token recurrence holds after 64 c tokens of the sequence (chunk_kda_naive.py:287-303):
+    dense batches, packed sequences (chunks of all sequences in order; an empty sequence contributes none), the
+    transposed layout, the cast to the input type."""
+    q, k, v, g, beta, h0 = make(2, 150, 2, 8, 12, seed=11)
+    o, s, h = ref64(q, k, v, g, beta, h0, return_intermediate_states=True)
+    assert h.shape == (2, 3, 2, 8, 12)
+    for c in range(3):
+        if c == 0:
+            want = h0
+        else:
+            _, want = KO.naive_kda_recurrence(q[:, :64 * c], k[:, :64 * c], v[:, :64 * c], g[:, :64 * c], beta[:, :64 * c],
+                                              initial_state=h0, output_final_state=True)
+        torch.testing.assert_close(h[:, c], want, rtol=1e-9, atol=1e-11)
+    cu = [0, 1, 1, 70, 150]
+    h4 = 0.5 * torch.randn(4, 2, 8, 12, dtype=F64, generator=torch.Generator().manual_seed(12))
+    _, _, hp = ref64(q[:1], k[:1], v[:1], g[:1], beta[:1], h4, cu_seqlens=cu, return_intermediate_states=True)
+    assert hp.shape == (1, 1 + 0 + 2 + 2, 2, 8, 12)
+    at = 0
+    for n in range(4):
+        a, b = cu[n], cu[n + 1]
+        for c in range((b - a + 63) // 64):
+            if c == 0:
+                want = h4[n:n + 1]
+            else:
+                _, want = KO.naive_kda_recurrence(q[:1, a:a + 64 * c], k[:1, a:a + 64 * c], v[:1, a:a + 64 * c],
+                                                  g[:1, a:a + 64 * c], beta[:1, a:a + 64 * c], initial_state=h4[n:n + 1],
+                                                  output_final_state=True)
+            torch.testing.assert_close(hp[:, at], want, rtol=1e-9, atol=1e-11)
+            at += 1
+    _, _, ht = ref64(q[:1], k[:1], v[:1], g[:1], beta[:1], h4.transpose(-1, -2).contiguous(), cu_seqlens=cu,
+                     transpose_state_layout=True, return_intermediate_states=True)
+    torch.testing.assert_close(ht, hp.transpose(-1, -2))
+    qb, kb, vb = q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16)
+    _, _, hb = KO.chunk_kda_ref(qb, kb, vb, g.float(), beta.float(), initial_state=h0.float(), return_intermediate_states=True)
+    assert hb.dtype == torch.bfloat16 and hb.shape == h.shape
