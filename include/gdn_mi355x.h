@@ -120,6 +120,15 @@ int gdn_recurrent_fwd(const void* q, const void* k, const void* v, const float* 
                       const float* state_in, float* state_out, void* o, int B, int T, int Hqk, int Hv, int K,
                       int V, float scale, int use_qk_l2norm, int dtype, void* stream);
 
+/* The same rule on packed sequences: q, k, v, g, beta, o hold one batch row of T tokens, cu_seqlens int64 [N+1] on the
+ * device lists the N sequences, state_in / state_out are [N,Hv,K,V]; every sequence runs on its own from its own
+ * state.  Counterpart: the `cu_seqlens` argument of the kernel bound in the same slot (third-party fla, un-vendored;
+ * the in-tree torch fallback has none), with the meaning packed input has at the chunk entry
+ * (chunk_gated_delta_rule.py:297-311).  Tokens outside every listed sequence are not written. */
+int gdn_recurrent_fwd_packed(const void* q, const void* k, const void* v, const float* g, const float* beta,
+                             const float* state_in, float* state_out, void* o, const int64_t* cu_seqlens, int N, int T,
+                             int Hqk, int Hv, int K, int V, float scale, int use_qk_l2norm, int dtype, void* stream);
+
 /* The same step reading q, k, v in place from the [tokens, D] output of the convolution (column ranges [0, Hqk K),
  * [Hqk K, 2 Hqk K), [2 Hqk K, 2 Hqk K + Hv V); token_stride >= that width, in elements, a multiple of 16 bytes) and
  * forming the gates from the layer's projections a, b [tokens, Hv] and parameters A_log, dt_bias [Hv] (in `dtype`

@@ -30,8 +30,8 @@ struct RecurrentGates {   // either g, beta (fp32 [tokens,Hv]) or the projection
 template <typename T, typename TP, int DK, int BV>
 __global__ __launch_bounds__(256) void recurrent_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, int64_t sq, int64_t sk, int64_t sv,
-    RecurrentGates gates, const float* state_in, float* state_out, T* __restrict__ o, int B, int T_len,
-    int Hqk, int Hv, int V, float scale, int use_l2norm) {
+    RecurrentGates gates, const float* state_in, float* state_out, T* __restrict__ o, const int64_t* __restrict__ cu,
+    int B, int T_len, int Hqk, int Hv, int V, float scale, int use_l2norm) {
   constexpr int CG = BV / 4;            // column groups (4 fp32 = 16 bytes each)
   constexpr int NRG = kThreads / CG;    // row groups
   constexpr int RPT = DK / NRG;         // state rows held by a thread
@@ -57,8 +57,11 @@ __global__ __launch_bounds__(256) void recurrent_kernel(
     }
   }
 
-  for (int t = 0; t < T_len; ++t) {
-    const int64_t tok = (int64_t)b * T_len + t;
+  // packed input (cu given): "sequence" b owns the tokens cu[b] .. cu[b+1] of the one batch row
+  const int64_t tok0 = cu != nullptr ? cu[b] : (int64_t)b * T_len;
+  const int ntok = cu != nullptr ? (int)(cu[b + 1] - cu[b]) : T_len;
+  for (int t = 0; t < ntok; ++t) {
+    const int64_t tok = tok0 + t;
     // ---- q, k of this token: optional l2 norm, q pre-scaled ----
     float kv_ = 0.f, qv_ = 0.f;
     if (tid < DK) {
@@ -160,11 +163,12 @@ __global__ __launch_bounds__(256) void recurrent_kernel(
 template <typename T, typename TP>
 static int launch_recurrent(const void* q, const void* k, const void* v, int64_t sq, int64_t sk, int64_t sv,
                             const RecurrentGates& gates, const float* state_in, float* state_out, void* o, int B,
-                            int T_len, int Hqk, int Hv, int K, int V, float scale, int use_l2norm, hipStream_t stream) {
+                            int T_len, int Hqk, int Hv, int K, int V, float scale, int use_l2norm, hipStream_t stream,
+                            const int64_t* cu = nullptr) {
 #define GDN_REC(DK_, BV_)                                                                                          \
   GDN_LAUNCH(kKernRecurrent, stream, (recurrent_kernel<T, TP, DK_, BV_>), dim3(B * Hv, V / BV_), dim3(kThreads), 0, \
-             stream, (const T*)q, (const T*)k, (const T*)v, sq, sk, sv, gates, state_in, state_out, (T*)o, B, T_len,  \
-             Hqk, Hv, V, scale, use_l2norm)
+             stream, (const T*)q, (const T*)k, (const T*)v, sq, sk, sv, gates, state_in, state_out, (T*)o, cu, B,     \
+             T_len, Hqk, Hv, V, scale, use_l2norm)
   const bool wide = (V % 128 == 0);
   if (K == 64 && wide) GDN_REC(64, 128);
   else if (K == 64) GDN_REC(64, 64);
@@ -201,6 +205,25 @@ extern "C" int gdn_recurrent_fwd(const void* q, const void* k, const void* v, co
   if (dtype == 1)
     return launch_recurrent<bf16_t, float>(q, k, v, nq, nq, nv, gates, state_in, state_out, o, B, T, Hqk, Hv, K, V, scale,
                                            use_qk_l2norm, s);
+  return -4;
+}
+
+extern "C" int gdn_recurrent_fwd_packed(const void* q, const void* k, const void* v, const float* g, const float* beta,
+                                        const float* state_in, float* state_out, void* o, const int64_t* cu_seqlens,
+                                        int N, int T, int Hqk, int Hv, int K, int V, float scale, int use_qk_l2norm,
+                                        int dtype, void* stream) {
+  using namespace gdn;
+  if (!q || !k || !v || !g || !beta || !o || !cu_seqlens) return -1;
+  if (int e = recurrent_check(N, T, Hqk, Hv, V)) return e;
+  hipStream_t s = (hipStream_t)stream;
+  const RecurrentGates gates{g, beta, nullptr, nullptr, nullptr, nullptr};
+  const int64_t nq = (int64_t)Hqk * K, nv = (int64_t)Hv * V;
+  if (dtype == 0)
+    return launch_recurrent<float, float>(q, k, v, nq, nq, nv, gates, state_in, state_out, o, N, T, Hqk, Hv, K, V, scale,
+                                          use_qk_l2norm, s, cu_seqlens);
+  if (dtype == 1)
+    return launch_recurrent<bf16_t, float>(q, k, v, nq, nq, nv, gates, state_in, state_out, o, N, T, Hqk, Hv, K, V, scale,
+                                           use_qk_l2norm, s, cu_seqlens);
   return -4;
 }
 

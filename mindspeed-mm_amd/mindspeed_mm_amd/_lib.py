@@ -22,6 +22,7 @@ SIGNATURES = {
     "gdn_chunk_bwd_strided": (I, [P] * 3 + [L] * 3 + [P] * 9 + [L] * 3 + [P] * 4 + [L] + [I] * 7 + [F, I, I, I, P]),
     "gdn_chunk_bwd_parts": (I, [P] * 3 + [L] * 3 + [P] * 9 + [L] * 3 + [P] * 4 + [L, P, L] + [I] * 9 + [F, I, I, I, P]),
     "gdn_recurrent_fwd": (I, [P] * 8 + [I] * 6 + [F, I, I, P]),
+    "gdn_recurrent_fwd_packed": (I, [P] * 9 + [I] * 6 + [F, I, I, P]),
     "gdn_recurrent_fwd_qkv": (I, [P, L] + [P] * 7 + [I] * 6 + [F, I, I, I, P]),
     "gdn_conv1d_fwd": (I, [P] * 8 + [I] * 7 + [P]),
     "gdn_conv1d_bwd_workspace_bytes": (L, [I] * 4),

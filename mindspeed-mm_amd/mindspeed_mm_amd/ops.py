@@ -55,19 +55,20 @@ def _beta_arg(beta, act_dtype):
 
 
 def _check_packed_length(cu_seqlens, tokens):
-    """The kernels visit the chunks of the listed sequences only: rows past cu_seqlens[-1] would be left unwritten.
-    Checked where it costs no device synchronisation (lists and host tensors); a device tensor must satisfy it too."""
+    """cu_seqlens must start at 0, not decrease and stay within the packed tokens; rows past cu_seqlens[-1] (a padded
+    batch) are cleared by the kernels.  Checked where it costs no device synchronisation (lists and host tensors); a
+    device tensor must satisfy it too."""
     if cu_seqlens is None:
         return
     if isinstance(cu_seqlens, torch.Tensor):
         if cu_seqlens.device.type != "cpu" or cu_seqlens.numel() == 0:
             return
-        first, last = int(cu_seqlens[0]), int(cu_seqlens[-1])
+        cu = [int(c) for c in cu_seqlens.tolist()]
     else:
-        first, last = int(cu_seqlens[0]), int(cu_seqlens[-1])
-    if first != 0 or last != tokens:
-        raise ValueError(f"cu_seqlens must start at 0 and end at the number of packed tokens ({tokens}), got "
-                         f"{first} ... {last}")
+        cu = [int(c) for c in cu_seqlens]
+    if cu[0] != 0 or cu[-1] > tokens or any(b < a for a, b in zip(cu[:-1], cu[1:])):
+        raise ValueError(f"cu_seqlens must start at 0, not decrease and end at or before the number of packed tokens "
+                         f"({tokens}), got {cu[0]} ... {cu[-1]}")
 
 
 def _act_code(activation):
@@ -325,20 +326,33 @@ class GdnOps:
                                          output_final_state=False, cu_seqlens=None, use_qk_l2norm_in_kernel=False,
                                          inplace_state=False):
         """One or more decode tokens per sequence.  Returns (o, final_state); final_state is a new fp32 tensor
-        unless inplace_state=True, in which case initial_state (fp32, contiguous) is updated and returned."""
-        if cu_seqlens is not None:
-            raise NotImplementedError("cu_seqlens is not supported by the decode kernel")
+        unless inplace_state=True, in which case initial_state (fp32, contiguous) is updated and returned.
+        cu_seqlens (list or int64 tensor [N+1]): the batch is one row of packed sequences, each run from its own
+        state [N,Hv,K,V], as at the chunk entry (chunk_gated_delta_rule.py:297-311, :398-411)."""
         if q.dtype != k.dtype or k.dtype != v.dtype or q.dtype not in (torch.float32, torch.bfloat16):
             raise ValueError("q, k, v must share a dtype, bfloat16 or float32")
         B, T, Hqk, K = q.shape
         Hv, V = v.shape[2], v.shape[3]
+        N = B
+        if cu_seqlens is not None:
+            if B != 1:
+                raise ValueError(
+                    f"The batch size is expected to be 1 rather than {B} when using `cu_seqlens`."
+                    f"Please flatten variable-length inputs before processing.")
+            N = len(cu_seqlens) - 1
+            if initial_state is not None and initial_state.shape[0] != N:
+                raise ValueError(
+                    f"The number of initial states is expected to be equal to the number of input sequences, "
+                    f"i.e., {N} rather than {initial_state.shape[0]}.")
+            _check_packed_length(cu_seqlens, T)
         if beta is None:
             beta = torch.ones(B, T, Hv, dtype=torch.float32, device=q.device)
         self._need(q, k, v, g, beta, initial_state)
         if scale is None:
             scale = K ** -0.5
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-        o = torch.empty_like(v)
+        # rows outside every listed sequence (a padded packed batch) are not visited by the kernel
+        o = torch.zeros_like(v) if cu_seqlens is not None else torch.empty_like(v)
         s_in = None
         if initial_state is not None:
             if inplace_state:
@@ -350,8 +364,15 @@ class GdnOps:
         s_out = None
         if output_final_state or inplace_state:
             s_out = s_in if (inplace_state and s_in is not None) else \
-                torch.empty(B, Hv, K, V, dtype=torch.float32, device=q.device)
+                torch.empty(N, Hv, K, V, dtype=torch.float32, device=q.device)
         g32, b32 = self._f32(g), self._f32(beta)   # named: temporaries must outlive the launch
+        if cu_seqlens is not None:
+            cu = _i64(cu_seqlens, q)
+            code = self.lib.gdn_recurrent_fwd_packed(ptr(q), ptr(k), ptr(v), ptr(g32), ptr(b32), ptr(s_in), ptr(s_out),
+                                                     ptr(o), ptr(cu), N, T, Hqk, Hv, K, V, float(scale),
+                                                     int(use_qk_l2norm_in_kernel), DTYPE_CODE[q.dtype], self.lib.stream())
+            self.lib.check(code, "gdn_recurrent_fwd_packed")
+            return o, (s_out if output_final_state else None)
         code = self.lib.gdn_recurrent_fwd(ptr(q), ptr(k), ptr(v), ptr(g32), ptr(b32), ptr(s_in),
                                           ptr(s_out), ptr(o), B, T, Hqk, Hv, K, V, float(scale),
                                           int(use_qk_l2norm_in_kernel), DTYPE_CODE[q.dtype], self.lib.stream())

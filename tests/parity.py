@@ -156,6 +156,31 @@ def check_recurrent(ops, device, B, T, Hqk, Hv, K, V, dtype, l2=True, seed=0, wi
     return {"o": _err("o", o, ro, dtype, BF16_ABS_O), "state": _err("state", s, rs, torch.float32, 0)}
 
 
+def check_recurrent_packed(ops, device, T, cu, Hqk, Hv, K, V, dtype, l2=True, seed=0, with_state=True, wrap=lambda t: t):
+    """The decode rule on one row of packed sequences against the oracle run sequence by sequence, each from its own
+    state; tokens outside every listed sequence come back as zeros."""
+    N = len(cu) - 1
+    x = gdn_inputs(1, T, Hqk, Hv, K, V, dtype, seed=seed, N=N, l2norm_in_kernel=l2)
+    dev = {n: wrap(t.to(device)) for n, t in x.items()}
+    o, s = ops.fused_recurrent_gated_delta_rule(dev["q"], dev["k"], dev["v"], dev["g"], dev["beta"],
+                                                initial_state=dev["h0"] if with_state else None, output_final_state=True,
+                                                use_qk_l2norm_in_kernel=l2,
+                                                cu_seqlens=torch.tensor(cu, dtype=torch.int64, device=device))
+    ro = torch.zeros(1, T, Hv, V)
+    rs = torch.zeros(N, Hv, K, V)
+    for n in range(N):
+        a, b = cu[n], cu[n + 1]
+        h0 = x["h0"][n:n + 1] if with_state else None
+        if b > a:
+            ro[:, a:b], rs[n:n + 1] = O.recurrent_gated_delta_rule_ref(
+                x["q"][:, a:b].float(), x["k"][:, a:b].float(), x["v"][:, a:b].float(), x["g"][:, a:b],
+                x["beta"][:, a:b].float(), h0, True, l2)
+        elif with_state:
+            rs[n] = x["h0"][n]
+    assert s.shape == rs.shape
+    return {"o": _err("o", o, ro, dtype, BF16_ABS_O), "state": _err("state", s, rs, torch.float32, 0)}
+
+
 def check_conv(ops, device, B, T, D, W, dtype, activation="silu", cu=None, bias=True, residual=False, state=True,
                backward=True, seed=0, wrap=lambda t: t):
     gen = torch.Generator().manual_seed(seed)

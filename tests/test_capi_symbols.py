@@ -79,19 +79,22 @@ def test_validation_errors_match_reference():
         M.causal_conv1d(torch.randn(1, 8, 8), torch.randn(4, 16))
 
 
-def test_packed_lengths_must_cover_every_token():
-    """The kernels visit the chunks of the listed sequences only; a cu_seqlens list or host tensor that stops short
-    of the packed length would leave output rows unwritten, so it is refused (no device synchronisation needed)."""
+def test_packed_lengths_are_checked_on_the_host():
+    """A cu_seqlens list or host tensor must start at 0, not decrease and stay within the packed tokens (no device
+    synchronisation needed for the check); one that stops short of the packed length is a padded batch and passes:
+    the kernels clear the rows behind it."""
     import torch
     import mindspeed_mm_amd as M
     q = torch.randn(1, 100, 1, 64, dtype=torch.bfloat16)
     g, b = torch.zeros(1, 100, 1), torch.ones(1, 100, 1)
-    with pytest.raises(ValueError, match="cu_seqlens must start at 0 and end"):
-        M.chunk_gated_delta_rule(q, q, q, g, b, cu_seqlens=torch.tensor([0, 30, 90]))
-    with pytest.raises(ValueError, match="cu_seqlens must start at 0 and end"):
-        M.chunk_gated_delta_rule(q, q, q, g, b, cu_seqlens=[5, 30, 100])
-    with pytest.raises(RuntimeError, match="no host fallback"):      # a complete list passes the check
-        M.chunk_gated_delta_rule(q, q, q, g, b, cu_seqlens=[0, 30, 100])
+    for bad in ([5, 30, 100], [0, 60, 30, 100], [0, 30, 101]):
+        with pytest.raises(ValueError, match="cu_seqlens must start at 0, not decrease and end at or before"):
+            M.chunk_gated_delta_rule(q, q, q, g, b, cu_seqlens=bad)
+    with pytest.raises(ValueError, match="cu_seqlens must start at 0"):
+        M.chunk_gated_delta_rule(q, q, q, g, b, cu_seqlens=torch.tensor([0, 30, 120]))
+    for good in ([0, 30, 100], torch.tensor([0, 30, 90])):
+        with pytest.raises(RuntimeError, match="no host fallback"):      # passes the check, then needs the GPU
+            M.chunk_gated_delta_rule(q, q, q, g, b, cu_seqlens=good)
 
 
 def test_autograd_functions_carry_the_guards():

@@ -33,6 +33,14 @@ def test_recurrent(ops, dtype, B, T, Hqk, Hv, K, V):
     P.check_recurrent(ops, "cpu", B, T, Hqk, Hv, K, V, dtype, l2=False, with_state=False, wrap=guarded)
 
 
+@pytest.mark.parametrize("dtype,T,cu,Hqk,Hv,K,V", [
+    (F32, 12, [0, 3, 3, 8, 12], 1, 2, 64, 64), (BF, 9, [0, 1, 6], 1, 2, 128, 64),
+])
+def test_recurrent_packed_sequences(ops, dtype, T, cu, Hqk, Hv, K, V):
+    P.check_recurrent_packed(ops, "cpu", T, cu, Hqk, Hv, K, V, dtype, wrap=guarded)
+    P.check_recurrent_packed(ops, "cpu", T, cu, Hqk, Hv, K, V, dtype, l2=False, with_state=False, wrap=guarded)
+
+
 @pytest.mark.parametrize("dtype,B,T,Hqk,Hv,K,V,l2,cu", [
     (F32, 1, 64, 1, 1, 64, 64, False, None),
     (F32, 2, 100, 2, 4, 128, 128, True, None),

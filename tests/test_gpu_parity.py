@@ -30,6 +30,22 @@ def test_recurrent(ops, dtype, B, T, Hqk, Hv, K, V):
     P.check_recurrent(ops, "cuda", B, T, Hqk, Hv, K, V, dtype, l2=False, with_state=False)
 
 
+@pytest.mark.parametrize("dtype,T,cu,Hqk,Hv,K,V", [
+    (F32, 20, [0, 3, 3, 9, 20], 1, 2, 64, 64),       # an empty sequence
+    (BF, 70, [0, 1, 40, 70], 2, 4, 128, 128),
+    (BF, 12, [0, 5, 9], 1, 2, 128, 64),              # a padded batch: tokens 9..11 belong to no sequence
+])
+def test_recurrent_packed_sequences(ops, dtype, T, cu, Hqk, Hv, K, V):
+    """cu_seqlens at the decode entry: every listed sequence runs on its own from its own state."""
+    print(f"recurrent packed {dtype} T{T} cu{cu} Hqk{Hqk} Hv{Hv} K{K} V{V}", flush=True)
+    P.check_recurrent_packed(ops, "cuda", T, cu, Hqk, Hv, K, V, dtype)
+    P.check_recurrent_packed(ops, "cuda", T, cu, Hqk, Hv, K, V, dtype, l2=False, with_state=False)
+    x = P.gdn_inputs(2, 4, Hqk, Hv, K, V, dtype)
+    d = {n: t.cuda() for n, t in x.items()}
+    with pytest.raises(ValueError, match="batch size is expected to be 1"):
+        ops.fused_recurrent_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], cu_seqlens=[0, 2, 4])
+
+
 def test_recurrent_inplace_state(ops):
     x = P.gdn_inputs(2, 1, 2, 4, 128, 128, BF, seed=3)
     d = {n: t.cuda() for n, t in x.items()}
