@@ -6,6 +6,8 @@ from .ops import (GdnDecodeCache, GdnOps, RMSNormGated, ShortConvolution, causal
                   chunk_gated_delta_rule_norm, chunk_gated_delta_rule_qkv, chunk_kda, decode_step, fused_recurrent_gated_delta_rule,
                   fused_recurrent_gated_delta_rule_qkv, gdn_gates, rms_norm_gated)
 
+from . import library   # registers torch.ops.mindspeed_mm_amd.* (the same entry points as torch.library operators)
+
 __all__ = ["GdnDecodeCache", "GdnOps", "RMSNormGated", "ShortConvolution", "causal_conv1d", "causal_conv1d_update",
            "chunk_gated_delta_rule", "chunk_gated_delta_rule_norm", "chunk_gated_delta_rule_qkv", "chunk_kda", "decode_step", "fused_recurrent_gated_delta_rule",
-           "fused_recurrent_gated_delta_rule_qkv", "gdn_gates", "rms_norm_gated"]
+           "fused_recurrent_gated_delta_rule_qkv", "gdn_gates", "library", "rms_norm_gated"]

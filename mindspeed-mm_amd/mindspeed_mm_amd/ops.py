@@ -103,7 +103,9 @@ class GdnOps:
     # ------------------------------------------------------------------ helpers
     def _need(self, *tensors):
         for t in tensors:
-            if t is not None and t.device.type != self.lib.device_type:
+            if not isinstance(t, torch.Tensor):   # None, or cu_seqlens given as a list
+                continue
+            if t.device.type != self.lib.device_type:
                 raise RuntimeError(
                     f"tensor on {t.device}; these operators run only on {self.lib.device_type} tensors "
                     "(there is no host fallback)")
@@ -446,7 +448,7 @@ class GdnOps:
         if cu_seqlens is not None and x.shape[0] != 1:
             raise ValueError("cu_seqlens needs batch size 1 (packed input)")
         _act_code(activation)
-        self._need(x, weight, bias, residual, initial_state, cu_seqlens)
+        self._need(x, weight, bias, residual, initial_state)   # cu_seqlens: a list or a tensor on any device
         return _CausalConv1d.apply(x, weight, bias, residual, initial_state, activation, cu_seqlens,
                                    bool(output_final_state), self)
 
@@ -507,6 +509,85 @@ def _chunk_workspace(lib, device, B, T, N, Hqk, Hv, K, V, code, need_grad):
     return ws[off:off + nbytes], nbytes
 
 
+def _chunk_forward_call(ops, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens,
+                        use_qk_l2norm_in_kernel, need_grad, skip_recompute):
+    """One forward call of the chunk rule through the C ABI.  Returns (o, final_state or None, the tensors a backward
+    call needs, their description); shared by the autograd function and the torch.library operator."""
+    lib = ops.lib
+    B, T, Hqk, K = q.shape
+    Hv, V = v.shape[2], v.shape[3]
+    N = (len(cu_seqlens) - 1) if cu_seqlens is not None else B
+    keep = need_grad and skip_recompute
+    prep_only = q.dtype != torch.float32 and not keep   # the recurrence writes o itself: no state leaves it
+    (qc, sq), (kc, sk), (vc, sv) = _token_view(q), _token_view(k), _token_view(v)
+    g32, h0 = ops._f32(g), ops._f32(initial_state)
+    bc, bcode = _beta_arg(beta, q.dtype)
+    cu = _i64(cu_seqlens, q)
+    code = DTYPE_CODE[q.dtype]
+    ws, nbytes = _chunk_workspace(lib, q.device, B, T, N, Hqk, Hv, K, V, code, 2 if prep_only else keep)
+    o = torch.empty(B, T, Hv, V, dtype=v.dtype, device=v.device)
+    ht = torch.empty(N, Hv, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
+    rc = lib.gdn_chunk_fwd_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(bc), ptr(h0), ptr(cu),
+                                   ptr(o), ptr(ht), ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale,
+                                   int(use_qk_l2norm_in_kernel), code, bcode, lib.stream())
+    lib.check(rc, "gdn_chunk_fwd_strided")
+    saved = (qc, kc, vc, g32, bc, h0, cu, ws if (keep or prep_only) else None)
+    meta = (B, T, N, Hqk, Hv, K, V, scale, int(use_qk_l2norm_in_kernel), code, nbytes,
+            g.dtype, beta.dtype, None if initial_state is None else initial_state.dtype, sq, sk, sv, bcode, prep_only)
+    return o, ht, saved, meta
+
+
+def _chunk_backward_call(ops, saved, meta, do, dht):
+    """The backward pass for a forward call described by (saved, meta) of _chunk_forward_call.
+    Returns (dq, dk, dv, dg, dbeta, d initial_state or None) in the dtypes of the forward call's arguments."""
+    qc, kc, vc, g32, bc, h0, cu, ws = saved
+    B, T, N, Hqk, Hv, K, V, scale, l2, code, nbytes, g_dt, b_dt, h_dt, sq, sk, sv, bcode, prep_only = meta
+    lib = ops.lib
+    dev = qc.device
+    do = do.contiguous()
+    dht = ops._f32(dht)
+    dq = torch.empty(B, T, Hqk, K, dtype=qc.dtype, device=dev)
+    dk = torch.empty(B, T, Hqk, K, dtype=qc.dtype, device=dev)
+    dv = torch.empty(B, T, Hv, V, dtype=qc.dtype, device=dev)
+    dg = torch.empty(B, T, Hv, dtype=torch.float32, device=dev)
+    db = torch.empty(B, T, Hv, dtype=bc.dtype, device=dev)
+    dh0 = torch.empty(N, Hv, K, V, dtype=torch.float32, device=dev) if h0 is not None else None
+    if ws is not None and prep_only:
+        # the prep part was kept: the state part is rebuilt beside the reverse recurrence, then the chunk-local kernels
+        ws_state, nstate = _chunk_workspace(lib, dev, B, T, N, Hqk, Hv, K, V, code, 3)
+
+        def phase(ph):
+            rc = lib.gdn_chunk_bwd_parts(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(bc), ptr(h0), ptr(cu),
+                                         ptr(do), ptr(dht), ptr(dq), ptr(dk), ptr(dv), 0, 0, 0, ptr(dg), ptr(db),
+                                         ptr(dh0), ptr(ws), nbytes, ptr(ws_state), nstate, ph, 1, B, T, N, Hqk, Hv, K,
+                                         V, scale, l2, code, bcode, lib.stream())
+            lib.check(rc, "gdn_chunk_bwd_parts")
+        helper = ops.helper_stream(dev)
+        if helper is None:
+            phase(7)
+        else:
+            main = torch.cuda.current_stream(dev)
+            helper.wait_stream(main)
+            with torch.cuda.stream(helper):
+                phase(1)
+            phase(2)
+            main.wait_stream(helper)
+            phase(4)
+        return dq, dk, dv, dg.to(g_dt), db.to(b_dt), None if dh0 is None else dh0.to(h_dt)
+    if ws is None:   # nothing was kept: refill a workspace (no output is written when o is null)
+        ws, nbytes = _chunk_workspace(lib, dev, B, T, N, Hqk, Hv, K, V, code, True)
+        rc = lib.gdn_chunk_fwd_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(bc), ptr(h0), ptr(cu),
+                                       None, None, ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale, l2, code, bcode,
+                                       lib.stream())
+        lib.check(rc, "gdn_chunk_fwd_strided (recompute)")
+    rc = lib.gdn_chunk_bwd_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(bc), ptr(h0), ptr(cu),
+                                   ptr(do), ptr(dht), ptr(dq), ptr(dk), ptr(dv), 0, 0, 0, ptr(dg), ptr(db),
+                                   ptr(dh0), ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale, l2, code, bcode,
+                                   lib.stream())
+    lib.check(rc, "gdn_chunk_bwd_strided")
+    return dq, dk, dv, dg.to(g_dt), db.to(b_dt), None if dh0 is None else dh0.to(h_dt)
+
+
 class _ChunkGatedDeltaRule(torch.autograd.Function):
     """Positional order as ChunkGatedDeltaRuleFunction.forward (chunk_gated_delta_rule.py:182-196).
 
@@ -524,30 +605,12 @@ class _ChunkGatedDeltaRule(torch.autograd.Function):
     @_custom_fwd
     def forward(ctx, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens,
                 use_qk_l2norm_in_kernel, skip_recompute, ops):
-        lib = ops.lib
-        B, T, Hqk, K = q.shape
-        Hv, V = v.shape[2], v.shape[3]
-        N = (len(cu_seqlens) - 1) if cu_seqlens is not None else B
         need_grad = any(ctx.needs_input_grad[:5]) or (initial_state is not None and ctx.needs_input_grad[6])
-        keep = need_grad and skip_recompute
-        prep_only = q.dtype != torch.float32 and not keep   # the recurrence writes o itself: no state leaves it
-        (qc, sq), (kc, sk), (vc, sv) = _token_view(q), _token_view(k), _token_view(v)
-        g32, h0 = ops._f32(g), ops._f32(initial_state)
-        bc, bcode = _beta_arg(beta, q.dtype)
-        cu = _i64(cu_seqlens, q)
-        code = DTYPE_CODE[q.dtype]
-        ws, nbytes = _chunk_workspace(lib, q.device, B, T, N, Hqk, Hv, K, V, code, 2 if prep_only else keep)
-        o = torch.empty(B, T, Hv, V, dtype=v.dtype, device=v.device)
-        ht = torch.empty(N, Hv, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
-        rc = lib.gdn_chunk_fwd_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(bc), ptr(h0), ptr(cu),
-                                       ptr(o), ptr(ht), ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale,
-                                       int(use_qk_l2norm_in_kernel), code, bcode, lib.stream())
-        lib.check(rc, "gdn_chunk_fwd_strided")
+        o, ht, saved, meta = _chunk_forward_call(ops, q, k, v, g, beta, scale, initial_state, output_final_state,
+                                                 cu_seqlens, use_qk_l2norm_in_kernel, need_grad, skip_recompute)
         if need_grad:
-            ctx.save_for_backward(qc, kc, vc, g32, bc, h0, cu, ws if (keep or prep_only) else None)
-            ctx.prep_only = prep_only
-            ctx.meta = (B, T, N, Hqk, Hv, K, V, scale, int(use_qk_l2norm_in_kernel), code, nbytes,
-                        g.dtype, beta.dtype, None if initial_state is None else initial_state.dtype, sq, sk, sv, bcode)
+            ctx.save_for_backward(*saved)
+            ctx.meta = meta
             ctx.ops = ops
         return o, ht
 
@@ -555,54 +618,8 @@ class _ChunkGatedDeltaRule(torch.autograd.Function):
     @_input_guard
     @_custom_bwd
     def backward(ctx, do, dht):
-        qc, kc, vc, g32, bc, h0, cu, ws = ctx.saved_tensors
-        B, T, N, Hqk, Hv, K, V, scale, l2, code, nbytes, g_dt, b_dt, h_dt, sq, sk, sv, bcode = ctx.meta
-        lib = ctx.ops.lib
-        dev = qc.device
-        do = do.contiguous()
-        dht = ctx.ops._f32(dht)
-        dq = torch.empty(B, T, Hqk, K, dtype=qc.dtype, device=dev)
-        dk = torch.empty(B, T, Hqk, K, dtype=qc.dtype, device=dev)
-        dv = torch.empty(B, T, Hv, V, dtype=qc.dtype, device=dev)
-        dg = torch.empty(B, T, Hv, dtype=torch.float32, device=dev)
-        db = torch.empty(B, T, Hv, dtype=bc.dtype, device=dev)
-        dh0 = torch.empty(N, Hv, K, V, dtype=torch.float32, device=dev) if h0 is not None else None
-        if ws is not None and ctx.prep_only:
-            # the prep part was kept: the state part is rebuilt beside the reverse recurrence, then the chunk-local kernels
-            ws_state, nstate = _chunk_workspace(lib, dev, B, T, N, Hqk, Hv, K, V, code, 3)
-
-            def phase(ph):
-                rc = lib.gdn_chunk_bwd_parts(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(bc), ptr(h0), ptr(cu),
-                                             ptr(do), ptr(dht), ptr(dq), ptr(dk), ptr(dv), 0, 0, 0, ptr(dg), ptr(db),
-                                             ptr(dh0), ptr(ws), nbytes, ptr(ws_state), nstate, ph, 1, B, T, N, Hqk, Hv, K,
-                                             V, scale, l2, code, bcode, lib.stream())
-                lib.check(rc, "gdn_chunk_bwd_parts")
-            helper = ctx.ops.helper_stream(dev)
-            if helper is None:
-                phase(7)
-            else:
-                main = torch.cuda.current_stream(dev)
-                helper.wait_stream(main)
-                with torch.cuda.stream(helper):
-                    phase(1)
-                phase(2)
-                main.wait_stream(helper)
-                phase(4)
-            return (dq, dk, dv, dg.to(g_dt), db.to(b_dt), None, None if dh0 is None else dh0.to(h_dt), None, None,
-                    None, None, None)
-        if ws is None:   # nothing was kept: refill a workspace (no output is written when o is null)
-            ws, nbytes = _chunk_workspace(lib, dev, B, T, N, Hqk, Hv, K, V, code, True)
-            rc = lib.gdn_chunk_fwd_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(bc), ptr(h0), ptr(cu),
-                                           None, None, ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale, l2, code, bcode,
-                                           lib.stream())
-            lib.check(rc, "gdn_chunk_fwd_strided (recompute)")
-        rc = lib.gdn_chunk_bwd_strided(ptr(qc), ptr(kc), ptr(vc), sq, sk, sv, ptr(g32), ptr(bc), ptr(h0), ptr(cu),
-                                       ptr(do), ptr(dht), ptr(dq), ptr(dk), ptr(dv), 0, 0, 0, ptr(dg), ptr(db),
-                                       ptr(dh0), ptr(ws), nbytes, B, T, N, Hqk, Hv, K, V, scale, l2, code, bcode,
-                                       lib.stream())
-        lib.check(rc, "gdn_chunk_bwd_strided")
-        return (dq, dk, dv, dg.to(g_dt), db.to(b_dt), None, None if dh0 is None else dh0.to(h_dt), None, None, None,
-                None, None)
+        dq, dk, dv, dg, db, dh0 = _chunk_backward_call(ctx.ops, ctx.saved_tensors, ctx.meta, do, dht)
+        return dq, dk, dv, dg, db, None, dh0, None, None, None, None, None
 
 
 class _ChunkGatedDeltaRuleNorm(torch.autograd.Function):
