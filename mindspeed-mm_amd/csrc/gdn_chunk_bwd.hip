@@ -678,41 +678,42 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   if (has_k) {
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {
-      const f32x16 kk = KTf[ri].unpack(), qq = QTf[ri].unpack();
-      const f32x16 gi = rows_ld(Gs, 32 * ri);
+      // the dQ half and the dK half one after the other: each unpacks its own partner rows, so that the two sets of
+      // sixteen values are not alive together
+      {
+        const f32x16 gi = rows_ld(Gs, 32 * ri);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        dQi[ri][r] *= scale * __expf(gi[r]);
-        dKi[ri][r] *= __expf(glast - gi[r]);
-        ski += dKi[ri][r] * kk[r];           // still only the inter-chunk part
+        for (int r = 0; r < 16; ++r) dQi[ri][r] *= scale * __expf(gi[r]);
+        AccB<T> a;
+#pragma unroll
+        for (int t = 0; t <= ri; ++t) { a.load(tileT + (2 * ri + t) * 1024); mma32_ff<T>(dQi[ri], a, KTf[t]); }
+        const f32x16 qq = QTf[ri].unpack();
+        f32x16 p;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) p[r] = dQi[ri][r] * qq[r];
+        rows_add(p, rq, 32 * ri);
       }
-      AccB<T> a;
+      GDN_SCHED_FENCE();
+      {
+        const f32x16 gi = rows_ld(Gs, 32 * ri), kk = KTf[ri].unpack();
 #pragma unroll
-      for (int t = 0; t <= ri; ++t) { a.load(tileT + (2 * ri + t) * 1024); mma32_ff<T>(dQi[ri], a, KTf[t]); }
+        for (int r = 0; r < 16; ++r) {
+          dKi[ri][r] *= __expf(glast - gi[r]);
+          ski += dKi[ri][r] * kk[r];           // still only the inter-chunk part
+        }
+        AccB<T> a;
 #pragma unroll
-      for (int t = ri; t < 2; ++t) { a.load(tileD + (2 * t + ri) * 1024); mma32_ff<T>(dKi[ri], a, QTf[t]); }
-      f32x16 p;
+        for (int t = ri; t < 2; ++t) { a.load(tileD + (2 * t + ri) * 1024); mma32_ff<T>(dKi[ri], a, QTf[t]); }
+        f32x16 p;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) p[r] = dQi[ri][r] * qq[r];
-      rows_add(p, rq, 32 * ri);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) p[r] = dKi[ri][r] * kk[r];
-      rows_add(p, rk1, 32 * ri);
+        for (int r = 0; r < 16; ++r) p[r] = dKi[ri][r] * kk[r];
+        rows_add(p, rk1, 32 * ri);
+      }
+      GDN_SCHED_FENCE();
     }
   }
   ski = wave_sum(ski);
   if (lane == 0) wsum[4 + wave] = ski;
-  // dTm pieces (lower tiles only): a1 = dW K^T over all of K, a2 = dV' V^T from the main loop
-  f32x16 a1 = acc_zero();
-  if (lower) {
-#pragma unroll
-    for (int kt = 0; kt < NKT; ++kt) {
-      AccB<T> a, b;
-      a.load(dWF + (ti * NKT + kt) * 1024);
-      b.load(EA + (2 * kt + tj) * 1024);
-      mma32_ff<T>(a1, a, b);
-    }
-  }
   if (has_k) {       // P = Tm^T dW; dK += beta e^G P; e^G <P,k> joins the dbeta / dG row sums
 #pragma unroll
     for (int rj = 0; rj < 2; ++rj) {
@@ -728,9 +729,9 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       }
     }
   }
-  GDN_LDS_BARRIER();   // the ds tiles and the dW tiles are consumed
+  GDN_LDS_BARRIER();   // the ds tiles are consumed
   // later value heads of a group add to the dq, dk rows the earlier ones wrote: what memory holds is requested well
-  // ahead, dq here (no store is in flight), dk right behind the dq stores (three phases before it is needed)
+  // ahead, dq here (no store is in flight), dk two phases before it is needed
   RowPieces<T> held[2];
   if (has_k && hh != 0) {
 #pragma unroll
@@ -745,7 +746,18 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     sv += __shfl_xor(sv, 32);
     if (lane < 32) rv[wave * 64 + 32 * tj + lane] += sv;
   }
-  {  // dTm[i][j] = beta_j (e^{G_j} a1 + a2), i > j, handed on in T form
+  {  // dTm[i][j] = beta_j (e^{G_j} a1 + a2), i > j, handed on in T form; a1 = dW K^T over all of K (the dW tiles stay
+     // in place until the store patches take their buffer behind the next barrier), a2 = dV' V^T from the main loop
+    f32x16 a1 = acc_zero();
+    if (lower) {
+#pragma unroll
+      for (int kt = 0; kt < NKT; ++kt) {
+        AccB<T> a, b;
+        a.load(dWF + (ti * NKT + kt) * 1024);
+        b.load(EA + (2 * kt + tj) * 1024);
+        mma32_ff<T>(a1, a, b);
+      }
+    }
     const int j = 32 * tj + acc_col();
     const float bj = bs[j], ej = egs[j];
 #pragma unroll
@@ -772,11 +784,6 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       if (hh == 0) acc_store_rows<T, false>(dQi[ri], id, patch, dst, ts.dq, nvalid - 32 * ri);
       else acc_store_rows<T, true>(dQi[ri], id, patch, dst, ts.dq, nvalid - 32 * ri, held[ri]);
     }
-    if (hh != 0) {
-#pragma unroll
-      for (int ri = 0; ri < 2; ++ri)
-        rows_request<T>(held[ri], dk + (tok0 + 32 * ri) * ts.dk + hq * DK + 32 * cj, ts.dk, nvalid - 32 * ri);
-    }
   }
   {  // X = dTm Tm^T, handed on in D form
     f32x16 x = acc_zero();
@@ -797,7 +804,9 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       b.load(tileD + (2 * m + tj) * 1024);
       mma32_ff<T>(y, tm_t(ti, m), b);
     }
-    const int j = 32 * tj + acc_col();
+    int j = 32 * tj + acc_col();
+    GDN_KEEP_HERE(j);   // recomputed here: the address of G_j from the first use, far above, would sit in a register (or in
+                        // scratch memory) through the phases between
     const float gj = Gs[j];
     const f32x16 gi = rows_ld(Gs, 32 * ti), br = rows_ld(bs, 32 * ti);
     f32x16 yb;
@@ -814,6 +823,11 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     d.store(dMD + wave * 1024);
   }
   GDN_LDS_BARRIER();
+  if (has_k && hh != 0) {   // the dk rows the earlier heads wrote, two phases before they are added to
+#pragma unroll
+    for (int ri = 0; ri < 2; ++ri)
+      rows_request<T>(held[ri], dk + (tok0 + 32 * ri) * ts.dk + hq * DK + 32 * cj, ts.dk, nvalid - 32 * ri);
+  }
   if (has_k) {       // E = dM K, F = dM^T (beta K): dK += beta E + F; <E,k> and <F,k> complete the row sums
 #pragma unroll
     for (int ri = 0; ri < 2; ++ri) {
