@@ -379,7 +379,7 @@ template <typename T, int DK> struct BwdLocalSmem {
   // buffer, D-form tiles [4] and T-form tiles [4] in the two shared stages
   static constexpr int off_tm = main_elems * (int)sizeof(T);                 // Tm tiles [2][2], whole kernel
   static constexpr int off_row = off_tm + 4 * 1024 * (int)sizeof(T);
-  static constexpr int bytes = off_row + (6 * 64 + 5 * 256 + 8) * 4;   // 6 row vectors, 5 per-wave row-sum arrays
+  static constexpr int bytes = off_row + (8 * 64 + 5 * 256 + 8) * 4;   // 8 row vectors, 5 per-wave row-sum arrays
   static_assert(main_elems == 32 * 1024, "as large as two former stages");
   static_assert(4 * Patch<T>::kElems <= raw_elems && 2 * (DK / 32) * 1024 <= raw_elems, "epilogue tenants fit");
 };
@@ -417,6 +417,8 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   float* rv = rf + 256;    // <R_i, v_i>, taken as the column sums of Tm . (dV' V^T)
   float* wsum = rv + 256;  // per wave: <S,dS'> [0..3], sum_i <k_i, dK_inter_i> [4..7]
   float* rqc = wsum + 8;   // <q_i, dQ_i> summed over the waves' slots
+  float* sgs = rqc + 64;   // scale e^{G_i}: the row factor of the inter-chunk part of dQ
+  float* egl = sgs + 64;   // e^{G_last - G_i}: that of dK (one exponential per row here instead of one per element there)
 
   stagger_second_resident<127>(3, 8 * cus, cus);
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
@@ -495,7 +497,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
 
   if (tid < 64) {   // the row vectors: all requests first, the same ones on every path
     const int tc = imin(tid, nvalid - 1);
-    const float gv = KDA ? 0.f : G[ch * 64 + tc];
+    const float gv = KDA ? 0.f : G[ch * 64 + tc], gl = KDA ? 0.f : G[ch * 64 + nvalid - 1];
     const uint32_t braw = gate_raw<T>(beta, beta_same, (tok0 + tc) * Hv + h);
     float rq1 = 1.f, rk1v = 1.f;
     if (l2) {
@@ -504,6 +506,8 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     }
     Gs[tid] = gv;
     egs[tid] = __expf(gv);
+    sgs[tid] = scale * __expf(gv);
+    egl[tid] = __expf(gl - gv);
     bs[tid] = tid < nvalid ? gate_val<T>(braw, beta_same) : 0.f;
     rsq[tid] = rq1;
     rsk[tid] = rk1v;
@@ -681,9 +685,9 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       // the dQ half and the dK half one after the other: each unpacks its own partner rows, so that the two sets of
       // sixteen values are not alive together
       {
-        const f32x16 gi = rows_ld(Gs, 32 * ri);
+        const f32x16 fq = rows_ld(sgs, 32 * ri);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) dQi[ri][r] *= scale * __expf(gi[r]);
+        for (int r = 0; r < 16; ++r) dQi[ri][r] *= fq[r];
         AccB<T> a;
 #pragma unroll
         for (int t = 0; t <= ri; ++t) { a.load(tileT + (2 * ri + t) * 1024); mma32_ff<T>(dQi[ri], a, KTf[t]); }
@@ -695,10 +699,10 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       }
       GDN_SCHED_FENCE();
       {
-        const f32x16 gi = rows_ld(Gs, 32 * ri), kk = KTf[ri].unpack();
+        const f32x16 fk = rows_ld(egl, 32 * ri), kk = KTf[ri].unpack();
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          dKi[ri][r] *= __expf(glast - gi[r]);
+          dKi[ri][r] *= fk[r];
           ski += dKi[ri][r] * kk[r];           // still only the inter-chunk part
         }
         AccB<T> a;
