@@ -489,8 +489,10 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     }
   };
 #pragma unroll
-  for (int j = 0; j < KG; ++j)                        // Tm tiles, fragment order
-    load16_to_lds(Ai + ch * 4096 + ((4 * j + wave) * 64 + lane) * VEC, TmF + (4 * j + wave) * 64 * VEC);
+  for (int j = 0; j < KG; ++j) {                      // Tm tiles, fragment order; tile (0,1) is zero, unused and not stored
+    const int piece = 4 * j + wave;
+    if (piece / KG != 1) load16_to_lds(Ai + ch * 4096 + (piece * 64 + lane) * VEC, TmF + piece * 64 * VEC);
+  }
   issue_shared(0);
   issue_priv(0);
   issue_raw(0);

@@ -137,9 +137,12 @@ __device__ __forceinline__ void store_tm_tiles(const float* Ti, T* Tms, T* tiles
   }
   GDN_LDS_BARRIER();
   {
-    AccB<T> tf;
-    frags_from_lds<T>(tf, Tms + (32 * (wave >> 1) + (lane & 31)) * L64 + 32 * (wave & 1));
-    tf.store_stream(tiles_out + wave * 1024);
+    // tile (0,1) of a lower triangular matrix is zero: no kernel reads it, and it is not written
+    if (wave != 1) {
+      AccB<T> tf;
+      frags_from_lds<T>(tf, Tms + (32 * (wave >> 1) + (lane & 31)) * L64 + 32 * (wave & 1));
+      tf.store_stream(tiles_out + wave * 1024);
+    }
   }
 }
 
@@ -237,9 +240,12 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
     }
     // scale tril(Q K^T . Gam) leaves as four 32x32 tiles in fragment order, packed as they sit in the accumulator
     // (lane <-> column j, registers <-> row i): the A operand of Aq^T dO as is, of Aq V' read transposed
-    AccB<T> af;
-    af.pack(aq);
-    af.store_stream(Aq_out + (((int64_t)blockIdx.x * Hv + h) * 4 + wave) * 1024);
+    // (tile (0,1) is zero, is read by no kernel and is not written)
+    if (wave != 1) {
+      AccB<T> af;
+      af.pack(aq);
+      af.store_stream(Aq_out + (((int64_t)blockIdx.x * Hv + h) * 4 + wave) * 1024);
+    }
   }
   // K (lane <-> token, registers <-> K column) and Q^T (lane <-> K column, registers <-> token) as A-operand fragments,
   // once per q/k group; the recurrence kernels read each of them both as it lies and transposed

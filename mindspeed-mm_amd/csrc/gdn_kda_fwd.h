@@ -320,7 +320,8 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
     }
     GDN_LDS_BARRIER();
   }
-  {  // Aq leaves as four tiles packed as they sit in an accumulator (lane <-> column j, registers <-> row i)
+  if (wave != 1) {  // Aq leaves as tiles packed as they sit in an accumulator (lane <-> column j, registers <-> row i);
+                    // tile (0,1) is zero, is read by no kernel and is not written
     const int ti = wave >> 1, tj = wave & 1;
     f32x16 aq;
 #pragma unroll
