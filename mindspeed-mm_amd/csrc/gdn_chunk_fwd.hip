@@ -166,7 +166,8 @@ template <typename T, int DK> struct PrepSmem {
   static constexpr int qs_bytes = cmax(cmax(64 * LDK * (int)sizeof(T), 64 * kLF * 4), 64 * L64 * (int)sizeof(T));
   static constexpr int off_ti = off_ks;
   static constexpr int off_misc = off_qs + qs_bytes;
-  static constexpr int bytes = off_misc + 2 * 64 * 4;
+  static constexpr int bytes = off_misc + 2 * 64 * 4;            // plus as much per further value head of the group
+  static int launch_bytes(int heads_per_group) { return bytes + (heads_per_group - 1) * 2 * 64 * 4; }
 };
 
 template <typename T, int DK>
@@ -183,20 +184,21 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
   float* As = reinterpret_cast<float*>(gdn_smem + SM::off_qs);    // after Q
   T* Tms = reinterpret_cast<T*>(gdn_smem + SM::off_qs);          // after A
   float* Ti = reinterpret_cast<float*>(gdn_smem + SM::off_ti);   // after K
-  float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_misc);
-  float* bs = Gs + 64;
+  float* Gs = reinterpret_cast<float*>(gdn_smem + SM::off_misc);   // per value head of the group: G [64], beta [64]
 
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int h = blockIdx.y, hq = h / (Hv / Hqk), nvalid = s.nvalid;
+  const int hq = blockIdx.y, grp = Hv / Hqk, nvalid = s.nvalid;
   const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk;
 
-  // ---- phase 0: cumulative decay (one lane per token), beta; K and Q tiles.  All requests first. ----
+  // ---- phase 0: K and Q tiles of the q/k group; cumulative decay (one lane per token) and beta of each of its value
+  //      heads, a wave per head.  All requests first. ----
   TileQK<T, DK> kt, qt;
   tile_qk_request<T, DK>(kt, k + tok0 * ts.k + hq * DK, ts.k, nvalid, tid);
   tile_qk_request<T, DK>(qt, q + tok0 * ts.q + hq * DK, ts.q, nvalid, tid);
-  if (wave == 0) {
+  for (int hh = wave; hh < grp; hh += 4) {
+    const int h = hq * grp + hh;
     float x = lane < nvalid ? g[(tok0 + lane) * Hv + h] : 0.f;
     const float b = lane < nvalid ? gate_val<T>(gate_raw<T>(beta, beta_same, (tok0 + lane) * Hv + h), beta_same) : 0.f;
 #pragma unroll
@@ -204,74 +206,75 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
       const float t = __shfl_up(x, d);
       if (lane >= d) x += t;
     }
-    Gs[lane] = x;
-    bs[lane] = b;
+    Gs[hh * 128 + lane] = x;
+    Gs[hh * 128 + 64 + lane] = b;
     G_out[((int64_t)blockIdx.x * Hv + h) * 64 + lane] = x;   // 64 contiguous values per chunk and head
   }
   {
-    // q and k arrive raw; with the in-kernel l2 norm they are normalised on the way into LDS.  The first value head
-    // of each q/k group also leaves 1/|q|, 1/|k| (for the output kernel, which scales q itself, and the backward pass).
-    const bool keep = l2norm && (h % (Hv / Hqk)) == 0;
+    // q and k arrive raw; with the in-kernel l2 norm they are normalised on the way into LDS, and 1/|q|, 1/|k| are left
+    // for the output kernel, which scales q itself, and the backward pass
     const int64_t roff = ((int64_t)blockIdx.x * Hqk + hq) * 64;   // 64 contiguous values per chunk and q/k head
-    tile_qk_finish<T, DK>(kt, Ks, LDK, nvalid, tid, l2norm != 0, nullptr, 0, keep ? rstd_k_out + roff : nullptr, 1);
-    tile_qk_finish<T, DK>(qt, Qs, LDK, nvalid, tid, l2norm != 0, nullptr, 0, keep ? rstd_q_out + roff : nullptr, 1);
+    tile_qk_finish<T, DK>(kt, Ks, LDK, nvalid, tid, l2norm != 0, nullptr, 0, l2norm ? rstd_k_out + roff : nullptr, 1);
+    tile_qk_finish<T, DK>(qt, Qs, LDK, nvalid, tid, l2norm != 0, nullptr, 0, l2norm ? rstd_q_out + roff : nullptr, 1);
   }
   GDN_LDS_BARRIER();
 
-  // ---- phase 1: A = strict_tril(beta_i k_i.k_j Gam_ij) and Aq = tril(q_i.k_j Gam_ij), one 32x32 tile per wave ----
-  f32x16 a_tile = acc_zero();   // goes to LDS (over the Q tile) once every wave is done with Q
-  {
-    const int ti = wave >> 1, tj = wave & 1;
-    f32x16 aq = acc_zero();
-    if (tj <= ti) {
-      mma32<T, DK, true, true>(a_tile, Ks + 32 * ti * LDK, LDK, Ks + 32 * tj * LDK, LDK);
-      mma32<T, DK, true, true>(aq, Qs + 32 * ti * LDK, LDK, Ks + 32 * tj * LDK, LDK);
-    }
-    const int j = 32 * tj + acc_col();
-    const float gj = Gs[j];
-    const f32x16 gi = rows_ld(Gs, 32 * ti), bi = rows_ld(bs, 32 * ti);
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {   // branch-free: where the mask discards the value the exponent is set to 0 first
-      const int i = 32 * ti + acc_row(r);
-      const float e = __expf(i >= j ? gi[r] - gj : 0.f);
-      const float gam = i >= j ? e : 0.f;
-      a_tile[r] = i > j ? bi[r] * a_tile[r] * gam : 0.f;
-      aq[r] *= gam * scale;
-    }
-    // scale tril(Q K^T . Gam) leaves as four 32x32 tiles in fragment order, packed as they sit in the accumulator
-    // (lane <-> column j, registers <-> row i): the A operand of Aq^T dO as is, of Aq V' read transposed
-    // (tile (0,1) is zero, is read by no kernel and is not written)
-    if (wave != 1) {
-      AccB<T> af;
-      af.pack(aq);
-      af.store_stream(Aq_out + (((int64_t)blockIdx.x * Hv + h) * 4 + wave) * 1024);
-    }
+  // ---- phase 1: the products k_i.k_j and q_i.k_j, one 32x32 tile per wave, once for the group: the value heads
+  //      differ in decay and beta only ----
+  const int ti = wave >> 1, tj = wave & 1;
+  f32x16 kk_raw = acc_zero(), qk_raw = acc_zero();
+  if (tj <= ti) {
+    mma32<T, DK, true, true>(kk_raw, Ks + 32 * ti * LDK, LDK, Ks + 32 * tj * LDK, LDK);
+    mma32<T, DK, true, true>(qk_raw, Qs + 32 * ti * LDK, LDK, Ks + 32 * tj * LDK, LDK);
   }
   // K (lane <-> token, registers <-> K column) and Q^T (lane <-> K column, registers <-> token) as A-operand fragments,
   // once per q/k group; the recurrence kernels read each of them both as it lies and transposed
-  if ((h % (Hv / Hqk)) == 0) {
-    for (int tt = wave; tt < 2 * (DK / 32); tt += 4) {
-      const int tj = tt & 1, kt = tt >> 1;
-      const int64_t gtile = ((((int64_t)blockIdx.x * Hqk + hq) * (DK / 32) + kt) * 2 + tj) * 1024;
-      AccB<T> kf;
-      frags_from_lds<T>(kf, Ks + (32 * tj + (lane & 31)) * LDK + 32 * kt);
-      kf.store_stream(KA_out + gtile);
-      kf.load_cols(Qs + 32 * tj * LDK + 32 * kt, LDK);
-      kf.store_stream(QT_out + gtile);
-    }
+  for (int tt = wave; tt < 2 * (DK / 32); tt += 4) {
+    const int tjj = tt & 1, ktt = tt >> 1;
+    const int64_t gtile = ((((int64_t)blockIdx.x * Hqk + hq) * (DK / 32) + ktt) * 2 + tjj) * 1024;
+    AccB<T> kf;
+    frags_from_lds<T>(kf, Ks + (32 * tjj + (lane & 31)) * LDK + 32 * ktt);
+    kf.store_stream(KA_out + gtile);
+    kf.load_cols(Qs + 32 * tjj * LDK + 32 * ktt, LDK);
+    kf.store_stream(QT_out + gtile);
   }
   GDN_LDS_BARRIER();   // Q and K are consumed: their space takes A and Tm
 
-  {
-    const int ti = wave >> 1, tj = wave & 1, j = 32 * tj + acc_col();
+  // ---- per value head: A = strict_tril(beta_i k_i.k_j Gam_ij), Aq = scale tril(q_i.k_j Gam_ij), Tm = (I + A)^-1 ----
+#pragma clang loop unroll(disable)
+  for (int hh = 0; hh < grp; ++hh) {
+    const int h = hq * grp + hh;
+    const float* Gh = Gs + hh * 128;
+    const float* bh = Gh + 64;
+    {
+      const int j = 32 * tj + acc_col();
+      const float gj = Gh[j];
+      const f32x16 gi = rows_ld(Gh, 32 * ti), bi = rows_ld(bh, 32 * ti);
+      f32x16 aq;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) As[(32 * ti + acc_row(r)) * kLF + j] = a_tile[r];
-  }
-  for (int i = tid; i < 64 * kLF; i += kThreads) Ti[i] = 0.f;
-  GDN_LDS_BARRIER();
+      for (int r = 0; r < 16; ++r) {   // branch-free: where the mask discards the value the exponent is set to 0 first
+        const int i = 32 * ti + acc_row(r);
+        const float e = __expf(i >= j ? gi[r] - gj : 0.f);
+        const float gam = i >= j ? e : 0.f;
+        As[i * kLF + j] = i > j ? bi[r] * kk_raw[r] * gam : 0.f;
+        aq[r] = qk_raw[r] * (gam * scale);
+      }
+      // scale tril(Q K^T . Gam) leaves as 32x32 tiles in fragment order, packed as they sit in the accumulator
+      // (lane <-> column j, registers <-> row i): the A operand of Aq^T dO as is, of Aq V' read transposed
+      // (tile (0,1) is zero, is read by no kernel and is not written)
+      if (wave != 1) {
+        AccB<T> af;
+        af.pack(aq);
+        af.store_stream(Aq_out + (((int64_t)blockIdx.x * Hv + h) * 4 + wave) * 1024);
+      }
+    }
+    for (int i = tid; i < 64 * kLF; i += kThreads) Ti[i] = 0.f;
+    GDN_LDS_BARRIER();
 
-  tril_inverse_64(As, Ti, wave, lane);
-  store_tm_tiles<T>(Ti, Tms, Ai_out + ((int64_t)blockIdx.x * Hv + h) * 4096, tid, wave, lane);
+    tril_inverse_64(As, Ti, wave, lane);
+    store_tm_tiles<T>(Ti, Tms, Ai_out + ((int64_t)blockIdx.x * Hv + h) * 4096, tid, wave, lane);
+    GDN_LDS_BARRIER();   // the staging tile (where the next head's A goes) and Tm are consumed
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -961,9 +964,9 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
   }
   if (!skip_prep) {
     auto kern = chunk_prep_kernel<T, DK>;
-    constexpr int smem = PrepSmem<T, DK>::bytes;
+    const int smem = PrepSmem<T, DK>::launch_bytes(d.Hv / d.Hqk);
     if (int e = set_lds(kern, smem)) return e;
-    GDN_LAUNCH(kKernPrep, st, kern, dim3(nc, d.Hv), dim3(kThreads), smem, st, qq, kk, g, beta, beta_same, cu,
+    GDN_LAUNCH(kKernPrep, st, kern, dim3(nc, d.Hqk), dim3(kThreads), smem, st, qq, kk, g, beta, beta_same, cu,
                (const int*)chunk_offsets, G, Ai, AQ, KAF, QTF, rstd, rstd + (int64_t)nc * 64 * d.Hqk, d.T, d.N, d.Hqk,
                d.Hv, scale, l2norm, ts);
   }
