@@ -575,7 +575,14 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       Vt.pack(mfma_transpose<T>(f, id));
       if (has_k) mma32_ff<T>(dKi[ri], Vt, dSf);
       if (lower && ri == tj) {
-        if (ti == 0) mma32_ff<T>(ds, dOt[0], Vt); else mma32_ff<T>(ds, dOt[1], Vt);
+        // the dO fragments of this wave's token block, picked register by register (an indexed fragment would go to
+        // scratch memory, a branch per block makes the compiler copy the accumulator between two places)
+        AccB<T> dsel;
+#pragma unroll
+        for (int g = 0; g < KG; ++g)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) dsel.f[g][e] = ti == 0 ? dOt[0].f[g][e] : dOt[1].f[g][e];
+        mma32_ff<T>(ds, dsel, Vt);
       }
     }
 #pragma unroll
