@@ -420,7 +420,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   float* sgs = rqc + 64;   // scale e^{G_i}: the row factor of the inter-chunk part of dQ
   float* egl = sgs + 64;   // e^{G_last - G_i}: that of dK (one exponential per row here instead of one per element there)
 
-  stagger_second_resident<127>(3, 8 * cus, cus);
+  stagger_second_resident<127>(KDA ? 3 : 4, 8 * cus, cus);   // about half of a workgroup's duration
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31;
