@@ -134,6 +134,98 @@ def test_chunk_backward_recompute_mode_equals_stored_mode(ops, dtype, B, T, Hqk,
     P.check_chunk_recompute_equals_stored(ops, "cuda", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu)
 
 
+@pytest.mark.parametrize("dtype,B,T,Hqk,Hv,K,V,cu", [
+    (BF, 2, 300, 2, 4, 128, 128, None),
+    (BF, 1, 333, 1, 2, 64, 128, [0, 70, 70, 333]),
+    (F32, 1, 130, 1, 2, 128, 64, None),
+])
+def test_chunk_backward_in_phases_through_the_c_abi(ops, dtype, B, T, Hqk, Hv, K, V, cu):
+    """gdn_chunk_bwd_parts on a two-part workspace against gdn_chunk_bwd_strided on one full workspace, bit for bit:
+    all phases in one call; refill / reverse recurrence / chunk-local in three calls; with the prep part rebuilt as
+    well (prep_valid = 0); a state part that is too small is refused."""
+    from mindspeed_mm_amd._lib import DTYPE_CODE, ptr
+    lib = ops.lib
+    N = (len(cu) - 1) if cu is not None else B
+    x = P.gdn_inputs(B, T, Hqk, Hv, K, V, dtype, seed=41, N=N)
+    d = {n: t.cuda() for n, t in x.items()}
+    q, k, v, g, do = d["q"], d["k"], d["v"], d["g"], d["do"]
+    beta = d["beta"].float()
+    h0, dht = d["h0"], d["dht"]
+    cu_t = torch.tensor(cu, dtype=torch.int64, device="cuda") if cu is not None else None
+    code, scale = DTYPE_CODE[dtype], K ** -0.5
+    dims = (B, T, N, Hqk, Hv, K, V)
+
+    def buf(mode):
+        n = lib.gdn_chunk_workspace_bytes(*dims, code, mode)
+        t = torch.empty(n + 256, dtype=torch.uint8, device="cuda")
+        off = (-t.data_ptr()) % 256
+        return t[off:off + n], n
+
+    def grads():
+        return [torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), torch.empty_like(g), torch.empty_like(beta),
+                torch.empty_like(h0)]
+
+    def fwd(ws, n, o):
+        rc = lib.gdn_chunk_fwd_strided(ptr(q), ptr(k), ptr(v), 0, 0, 0, ptr(g), ptr(beta), ptr(h0), ptr(cu_t), ptr(o), None,
+                                       ptr(ws), n, *dims, scale, 1, code, 0, lib.stream())
+        assert rc == 0, rc
+
+    def parts(G, wp, np_, wst, ns, phases, prep_valid):
+        return lib.gdn_chunk_bwd_parts(ptr(q), ptr(k), ptr(v), 0, 0, 0, ptr(g), ptr(beta), ptr(h0), ptr(cu_t), ptr(do),
+                                       ptr(dht), ptr(G[0]), ptr(G[1]), ptr(G[2]), 0, 0, 0, ptr(G[3]), ptr(G[4]), ptr(G[5]),
+                                       ptr(wp), np_, ptr(wst), ns, phases, prep_valid, *dims, scale, 1, code, 0, lib.stream())
+
+    o = torch.empty_like(v)
+    full, nfull = buf(1)
+    fwd(full, nfull, o)
+    want = grads()
+    rc = lib.gdn_chunk_bwd_strided(ptr(q), ptr(k), ptr(v), 0, 0, 0, ptr(g), ptr(beta), ptr(h0), ptr(cu_t), ptr(do), ptr(dht),
+                                   ptr(want[0]), ptr(want[1]), ptr(want[2]), 0, 0, 0, ptr(want[3]), ptr(want[4]),
+                                   ptr(want[5]), ptr(full), nfull, *dims, scale, 1, code, 0, lib.stream())
+    assert rc == 0, rc
+    prep, nprep = buf(2)
+    state, nstate = buf(3)
+    assert nprep + nstate >= nfull > nstate > 0 and nprep > 0
+    if dtype == BF:
+        fwd(prep, nprep, o)            # a 16-bit forward call that writes o needs the prep part only
+        cases = [("one call", (7,), 1), ("three calls", (1, 2, 4), 1), ("prep rebuilt too", (7,), 0)]
+    else:
+        cases = [("prep rebuilt too", (7,), 0), ("three calls, prep rebuilt by the first", (1, 2, 4), 0)]
+    for name, phases, prep_valid in cases:
+        state.zero_()
+        if not prep_valid:
+            prep.zero_()
+        got = grads()
+        for ph in phases:
+            rc = parts(got, prep, nprep, state, nstate, ph, prep_valid or ph != phases[0])
+            assert rc == 0, (name, ph, rc)
+        torch.cuda.synchronize()
+        for w, g_, nm in zip(want, got, ("dq", "dk", "dv", "dg", "dbeta", "dh0")):
+            assert torch.equal(w, g_), (name, nm)
+    assert parts(grads(), prep, nprep, state, nstate - 256, 7, 1) == -5
+
+
+def test_chunk_default_mode_on_one_stream_equals_two_streams(ops):
+    """The default mode's backward pass rebuilds states and corrected values on a second stream beside the reverse
+    recurrence; with that switched off (everything on the caller's stream) the gradients are the same bits."""
+    x = P.gdn_inputs(2, 500, 2, 4, 128, 128, BF, seed=42)
+    d = {n: t.cuda() for n, t in x.items()}
+    outs = []
+    was = ops.two_stream_backward
+    try:
+        for two in (True, False):
+            ops.two_stream_backward = two
+            L = {n: d[n].clone().requires_grad_(True) for n in ("q", "k", "v", "g", "beta", "h0")}
+            o, ht = ops.chunk_gated_delta_rule(L["q"], L["k"], L["v"], L["g"], L["beta"], initial_state=L["h0"],
+                                               output_final_state=True, use_qk_l2norm_in_kernel=True)
+            ((o.float() * d["do"].float()).sum() + (ht * d["dht"]).sum()).backward()
+            outs.append([o, ht] + [L[n].grad for n in L])
+    finally:
+        ops.two_stream_backward = was
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+
+
 def test_chunk_backward_stored_mode_against_oracle(ops):
     P.check_chunk(ops, "cuda", 2, 200, 2, 4, 128, 128, BF, backward=True, skip_recompute=True)
 
