@@ -151,6 +151,9 @@ __device__ __forceinline__ void store_tm_tiles(const float* Ti, T* Tms, T* tiles
 //   G (cumulative decay), Tm = (I+L)^-1, Aq = scale tril(Q K^T . Gam), and per q/k group the K and Q^T tiles, all in
 //   fragment order (AccB<>): 16 bytes per lane per k-group, copied straight to LDS by the recurrence kernels.
 // W = Tm (beta e^G K) and U = Tm (beta V) are never formed: the recurrence applies Tm to beta (v - e^G K S) itself.
+// One workgroup per (chunk, q/k group): q and k are loaded and normalised, and the products k.k and q.k formed, once
+// for the group; its value heads, which differ in decay and beta only, follow one after the other (mask, Aq tiles,
+// the 64x64 inverse).
 // Its barriers order LDS traffic only (GDN_LDS_BARRIER): a __syncthreads() would also wait until every store issued
 // so far has been acknowledged.
 // ---------------------------------------------------------------------------------------------
