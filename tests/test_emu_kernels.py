@@ -59,6 +59,8 @@ def test_chunk_forward(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu):
     (BF, 1, 200, 1, 2, 128, 128, True, None),
     (BF, 1, 140, 2, 2, 64, 64, False, [0, 5, 70, 71, 140]),
     (F32, 1, 96, 1, 1, 128, 192, True, [0, 1, 38, 96]),
+    (BF, 1, 100, 1, 6, 64, 64, True, None),          # more value heads per group than the prep kernel has waves
+    (F32, 1, 70, 1, 3, 64, 64, True, [0, 3, 70]),
 ])
 def test_chunk_backward(ops, dtype, B, T, Hqk, Hv, K, V, l2, cu):
     P.check_chunk(ops, "cpu", B, T, Hqk, Hv, K, V, dtype, l2=l2, cu=cu, backward=True, wrap=guarded, h0_std=0.1)

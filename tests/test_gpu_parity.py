@@ -80,6 +80,10 @@ CHUNK_CASES = [
     (BF, 1, 600, 1, 2, 64, 64, False, [0, 64, 65, 130, 258, 300, 450, 599, 600]),
     (F32, 8, 70, 1, 2, 64, 64, True, None),
     (F32, 1, 1024, 2, 4, 128, 128, True, None),                  # fp32 with grouped heads over many chunks
+    # value heads per q/k group other than 1, 2, 4: the prep kernel deals a group's heads to its four waves
+    (BF, 1, 200, 1, 3, 128, 128, True, None),
+    (BF, 1, 140, 2, 12, 64, 64, True, [0, 5, 70, 71, 140]),
+    (F32, 1, 100, 1, 5, 64, 64, False, None),
 ]
 
 
