@@ -230,7 +230,8 @@ int gdn_kda_fwd(const void* q, const void* k, const void* v, const void* g, cons
 
 /* chunk_kda(..., return_intermediate_states=True) (chunk_kda_naive.py:287-303, :375-380; triton_ascend/chunk.py:149-151,
  * an inference-time option): the state at the entry of every chunk of 64 tokens, from the workspace a gdn_kda_fwd call
- * with the same B, T, N, H, K, V, dtype and cu_seqlens filled.  h_out [h_chunks, H, K, V], or [h_chunks, H, V, K] with
+ * with the same B, T, N, H, K, V, dtype and cu_seqlens filled; that workspace must have the size
+ * gdn_kda_workspace_bytes gives with with_backward = 1 (a forward-only workspace does not keep the states: -5).  h_out [h_chunks, H, K, V], or [h_chunks, H, V, K] with
  * transpose_state_layout, in `dtype`; chunk c of batch row b is row b * ceil(T/64) + c, packed input lists the chunks
  * of its sequences in order (h_chunks = sum of ceil(len/64); chunks past h_chunks are not written). */
 int gdn_kda_intermediate_states(const void* workspace, int64_t workspace_bytes, const int64_t* cu_seqlens, void* h_out,

@@ -84,14 +84,15 @@ struct KdaWorkspace {
   int64_t AQ;             // T [chunks,H,2,2]       scale tril(sum_d q_i k_j e^{G_i-G_j}) tiles
   int64_t K1F;            // T [chunks,H,K/32,2]    rows -beta k . e^{G}
   int64_t K2F;            // T [chunks,H,K/32,2]    rows k . e^{G_last-G}
-  int64_t QB;             // T [tokens,H,K]         rows scale q . e^{G}, row-major
+  int64_t QB;             // T [tokens,H,K]         rows scale q . e^{G}, row-major: written for the stand-alone output kernel only
+  int64_t QBT;            // T [chunks,H,K/32,2]    (scale q . e^{G})^T as A operand: tile = (32 columns of K) x (32 tokens);
+                          //                        written when the recurrence forms the output itself or a backward pass follows
   int64_t VF;             // T [chunks,H,V/32,2]    v_new
   int64_t HF;             // T [chunks,H,V/32,K/32] state before each chunk
   int64_t fwd_bytes;
   // kept for a backward pass
   int64_t GC;             // f32 [chunks,H,64,K]    chunk-local cumulative log decay
   int64_t TMR;            // T [chunks,H,64,64]     Tm row-major, as rounded for the tiles
-  int64_t QBT;            // T [chunks,H,K/32,2]    (scale q . e^{G})^T as A operand: tile = (32 columns of K) x (32 tokens)
   int64_t DVF;            // T [chunks,H,V/32,2]    d(v_new)
   int64_t DHF;            // T [chunks,H,V/32,K/32] gradient of the state AFTER each chunk
   int64_t DUMP;           // T [chunks,H][dQb | dK2 | P : 64,K each][dAq | a2 : 64,64 each]  sums over V of the chunk-local pass
@@ -115,12 +116,12 @@ inline KdaWorkspace kda_workspace_layout(const ChunkDims& d, int elem_bytes) {
   w.K1F = take(nc * 64 * H * d.K * elem_bytes);
   w.K2F = take(nc * 64 * H * d.K * elem_bytes);
   w.QB = take(d.tokens() * H * d.K * elem_bytes);
+  w.QBT = take(nc * 64 * H * d.K * elem_bytes);
   w.VF = take(nc * 64 * H * d.V * elem_bytes);
   w.HF = take(nc * H * d.V * d.K * elem_bytes);
   w.fwd_bytes = off;
   w.GC = take(nc * 64 * H * d.K * 4);
   w.TMR = take(nc * H * 64 * 64 * elem_bytes);
-  w.QBT = take(nc * 64 * H * d.K * elem_bytes);
   w.DVF = take(nc * 64 * H * d.V * elem_bytes);
   w.DHF = take(nc * H * d.V * d.K * elem_bytes);
   w.DUMP = take(nc * H * KdaWorkspace::dump_elems(d.K) * elem_bytes);

@@ -320,7 +320,7 @@ template <typename T, int DK, int NW, int STAGES, bool OUT, bool PRE_, bool KDA 
   // rows: scale e^G [64], G_last; without PRE also e^{G_last-G} [64], beta e^G [64], beta [64]; KDA: e^{G_last} per key
   // channel [DK] at 68
   static constexpr int stage = off_row + (PRE && !KDA ? 68 : 260) * 4;   // a multiple of 16 bytes, like the offset of every row vector
-  static_assert(!KDA || (PRE && !OUT && DK <= 128), "KDA: both K images arrive ready-made, the output is a kernel of its own");
+  static_assert(!KDA || (PRE && DK <= 128), "KDA: both K images arrive ready-made");
   static_assert(stage % 16 == 0, "stages keep 16-byte alignment");
   static constexpr int off_x = STAGES * stage;                      // OUT: per slab S [2][DK*32], V' [2][2048], a store patch per output wave
   static constexpr int bytes = off_x + (OUT ? NW * x_elems * (int)sizeof(T) : 0);
@@ -333,7 +333,8 @@ template <int PIECES, int NT> struct Deal { static constexpr int kPer = (PIECES 
 
 // KDA (one decay per key channel): kaf and qtf hold the two K images ready-made, rows scaled by -beta e^{G} and by
 // e^{G_last-G} channel by channel, G holds e^{G_last} [chunks,Hv,DK] and beta the transformed beta in fp32; the state's
-// rows decay each by their own factor.
+// rows decay each by their own factor.  With OUT the output waves take (scale q . e^{G})^T from a third image, qim,
+// whose rows carry every factor of the output's first term (the other modes read their Q^T image through qtf).
 template <typename T, int DK, int NW, int NL, int STAGES, bool OUT, bool PRE_, bool KDA = false>
 __global__ __launch_bounds__(64 * (NW + (OUT ? NW * StateOutWaves<NW>::value : 0) + NL)) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 2 : 1)
 void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, const T* __restrict__ ai,
@@ -341,7 +342,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
                         const void* __restrict__ beta, int beta_same, const float* __restrict__ h0, float* __restrict__ ht,
                         T* __restrict__ vf, T* __restrict__ hf, T* __restrict__ o, const int64_t* __restrict__ cu,
                         const int* __restrict__ chunk_offsets, int T_len, int Hqk, int Hv, int V, float scale,
-                        int64_t v_stride) {
+                        int64_t v_stride, const T* __restrict__ qim) {
   using SM = StateSmem<T, DK, NW, STAGES, OUT, PRE_, KDA>;
   static_assert(!KDA || 64 * NL >= DK, "a loader thread per key channel");
   constexpr int NT = 64 * NL, VEC = Elem<T>::kVec, NKT = DK / 32, OS = StateOutWaves<NW>::value, NWO = OUT ? NW * OS : 0;
@@ -377,6 +378,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
     // one that copies it to LDS (j - 1), so global loads have DEPTH chunk periods to arrive
     constexpr int DEPTH = (STAGES == 2) ? 2 : 1;
     Vec16<T> pk[DEPTH][CK], ptm[DEPTH][CTM], pv[DEPTH][CV], pq[DEPTH][OUT || KDA ? CK : 1], pa[DEPTH][OUT ? CTM : 1];   // KDA: pq = second K image
+    Vec16<T> pq2[DEPTH][OUT && KDA ? CK : 1];   // KDA with output waves: the Q^T image
     float pgl[DEPTH], pg[DEPTH], pgk[DEPTH][2];
     uint32_t pb[DEPTH], pbk[DEPTH][2], pbv[DEPTH][CV];   // beta as fetched
     int pnv[DEPTH];
@@ -396,6 +398,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
         const int idc = imin(lt + i * NT, PK - 1);
         pk[set][i] = ld16(kaf + chq * (64 * DK) + idc * VEC);   // shared by the value heads of the group
         if constexpr (OUT || KDA) pq[set][i] = ld16(qtf + chq * (64 * DK) + idc * VEC);
+        if constexpr (OUT && KDA) pq2[set][i] = ld16(qim + chq * (64 * DK) + idc * VEC);
       }
 #pragma unroll
       for (int i = 0; i < CTM; ++i) {
@@ -454,7 +457,7 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
         } else {
           st16(st + SM::off_k + idc * VEC, pk[set][i]);
         }
-        if constexpr (OUT) st16(st + SM::off_q + idc * VEC, pq[set][i]);
+        if constexpr (OUT) st16(st + SM::off_q + idc * VEC, KDA ? pq2[set][i] : pq[set][i]);
       }
 #pragma unroll
       for (int i = 0; i < CTM; ++i) {
@@ -595,15 +598,19 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
             }
           }
           if constexpr (OS == 2) {
-            const f32x16 e0 = rows_ld(row, 32 * hw);
+            if constexpr (!KDA) {   // KDA: the rows of the Q image carry scale and decay
+              const f32x16 e0 = rows_ld(row, 32 * hw);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) oa[0][r] *= e0[r];
+              for (int r = 0; r < 16; ++r) oa[0][r] *= e0[r];
+            }
             Af[0].load_t(st + SM::off_aq + hw * 1024);   // (lane <-> row i, registers <-> column j)
             if (hw == 1) Af[1].load_t(st + SM::off_aq + 2 * 1024);
           } else {
-            const f32x16 e0 = rows_ld(row, 0), e1 = rows_ld(row, 32);
+            if constexpr (!KDA) {
+              const f32x16 e0 = rows_ld(row, 0), e1 = rows_ld(row, 32);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) { oa[0][r] *= e0[r]; oa[1][r] *= e1[r]; }
+              for (int r = 0; r < 16; ++r) { oa[0][r] *= e0[r]; oa[1][r] *= e1[r]; }
+            }
 #pragma unroll
             for (int t = 0; t < 3; ++t) Af[t].load_t(st + SM::off_aq + t * 1024);   // (lane <-> row i, registers <-> column j)
           }
@@ -980,7 +987,7 @@ static int chunk_fwd_launch(const ChunkDims& d, const ChunkWorkspace& L, const v
     if (int e = set_lds(kern, smem)) return e;
     GDN_LAUNCH(kKernStateFwd, st, kern, dim3(d.N * d.Hv, d.V / (32 * NWS)), dim3(64 * waves), smem, st, (const T*)KAF,
                (const T*)QTF, (const T*)Ai, (const T*)AQ, (const T*)v, (const float*)G, beta, beta_same, h0, ht, VF, HF, op, cu,
-               (const int*)chunk_offsets, d.T, d.Hqk, d.Hv, d.V, scale, ts.v);
+               (const int*)chunk_offsets, d.T, d.Hqk, d.Hv, d.V, scale, ts.v, (const T*)nullptr);
     return 0;
   };
   if constexpr (FUSE) {

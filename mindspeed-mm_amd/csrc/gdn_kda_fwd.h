@@ -2,8 +2,10 @@
 //     S <- diag(e^{g_t}) S;  S <- S + beta_t k_t (v_t - S^T k_t)^T;  o_t = scale S^T q_t
 // (reference: mindspeed_mm/fsdp/ops/kda/chunk_kda_naive.py:106-221, operator entry :223-381, gate :76-104).
 // Included at the end of gdn_chunk_fwd.hip: the recurrence and the output product are that file's kernels
-// (chunk_state_kernel in its KDA mode, chunk_out_kernel with rows of q that already carry scale and decay); this file
-// adds the chunk-local preparation, which is where the per-channel decay changes the algebra, and the entry points.
+// (chunk_state_kernel in its KDA mode, whose output waves form O from an image of q that already carries scale and
+// decay; where a workgroup serves two slabs of the state, or in fp32, chunk_out_kernel forms O from the stored states
+// instead); this file adds the chunk-local preparation, which is where the per-channel decay changes the algebra, and
+// the entry points.
 //
 // Per chunk, with G the chunk-local cumulative log decay [64, K]:
 //     L_ij  = beta_i sum_d k_id k_jd e^{G_id - G_jd}   (i > j)       Tm = (I + L)^-1
@@ -248,10 +250,10 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
 #pragma unroll
     for (int e = 0; e < VEC; ++e) f[e] *= scale * __expf(gi[e]);
     const Vec16<T> x = pack16<T>(f);
-    if (row < nvalid) st16(QB_out + (tok0 + row) * hk + h * DK + cc * VEC, x);   // row-major for the output kernel
+    if (QB_out != nullptr && row < nvalid) st16(QB_out + (tok0 + row) * hk + h * DK + cc * VEC, x);   // row-major for the output kernel
     st16(Qs + row * LDK + cc * VEC, x);
   }
-  if (QBT_out != nullptr) {   // transposed tiles for a backward pass
+  if (QBT_out != nullptr) {   // transposed tiles for the recurrence's output waves and for a backward pass
     GDN_LDS_BARRIER();
     for (int tt = wave; tt < 2 * (DK / 32); tt += 4) {
       const int tj = tt & 1, kt2 = tt >> 1;
@@ -355,11 +357,14 @@ static int kda_fwd_launch(const ChunkDims& d, const KdaWorkspace& L, const void*
   T* AQ = reinterpret_cast<T*>(ws + L.AQ);
   T* K1F = reinterpret_cast<T*>(ws + L.K1F);
   T* K2F = reinterpret_cast<T*>(ws + L.K2F);
-  T* QB = reinterpret_cast<T*>(ws + L.QB);
+  // Where one slab per workgroup is the choice and the K, Q and Aq images of two stages fit the LDS beside the slab's
+  // state, the recurrence kernel's own output waves write O and the stand-alone output kernel is not launched.
+  constexpr bool FUSE = NWS == 1 && STAGES == 2 && sizeof(T) == 2;
+  T* QB = FUSE ? nullptr : reinterpret_cast<T*>(ws + L.QB);
   T* VF = reinterpret_cast<T*>(ws + L.VF);
   T* HF = reinterpret_cast<T*>(ws + L.HF);
   float* GC = with_backward ? reinterpret_cast<float*>(ws + L.GC) : nullptr;
-  T* QBT = with_backward ? reinterpret_cast<T*>(ws + L.QBT) : nullptr;
+  T* QBT = (with_backward || FUSE) ? reinterpret_cast<T*>(ws + L.QBT) : nullptr;
   T* TMR = with_backward ? reinterpret_cast<T*>(ws + L.TMR) : nullptr;
   if (cu != nullptr) GDN_LAUNCH(kKernChunkTable, st, chunk_table_kernel, dim3(1), dim3(kThreads), 0, st, cu, chunk_offsets, d.N);
   {
@@ -376,13 +381,24 @@ static int kda_fwd_launch(const ChunkDims& d, const KdaWorkspace& L, const void*
                dt_bias, cu, (const int*)chunk_offsets, bhat, dec, GC, Ai, AQ, K1F, K2F, QB, QBT, TMR, keep ? rstd : nullptr,
                keep ? rstd + (int64_t)nc * 64 * H : nullptr, d.T, d.N, H, scale, fl);
   }
+  if constexpr (FUSE) {
+    auto kern = chunk_state_kernel<T, DK, NWS, NLS, STAGES, true, true, true>;
+    constexpr int smem = StateSmem<T, DK, NWS, STAGES, true, true, true>::bytes;
+    if (int e = set_lds(kern, smem)) return e;
+    // the per-chunk states and v_new leave the kernel only for a backward pass
+    GDN_LAUNCH(kKernStateFwd, st, kern, dim3(d.N * H, d.V / (32 * NWS)), dim3(64 * (NWS * (1 + StateOutWaves<NWS>::value) + NLS)),
+               smem, st, (const T*)K1F, (const T*)K2F, (const T*)Ai, (const T*)AQ, (const T*)v, (const float*)dec,
+               (const void*)bhat, 0, h0, ht, with_backward ? VF : (T*)nullptr, with_backward ? HF : (T*)nullptr, (T*)o, cu,
+               (const int*)chunk_offsets, d.T, H, H, d.V, scale, (int64_t)H * d.V, (const T*)QBT);
+    return (int)hipGetLastError();
+  }
   {
     auto kern = chunk_state_kernel<T, DK, NWS, NLS, STAGES, false, true, true>;
     constexpr int smem = StateSmem<T, DK, NWS, STAGES, false, true, true>::bytes;
     if (int e = set_lds(kern, smem)) return e;
     GDN_LAUNCH(kKernStateFwd, st, kern, dim3(d.N * H, d.V / (32 * NWS)), dim3(64 * (NWS + NLS)), smem, st, (const T*)K1F,
                (const T*)K2F, (const T*)Ai, (const T*)AQ, (const T*)v, (const float*)dec, (const void*)bhat, 0, h0, ht, VF, HF,
-               (T*)nullptr, cu, (const int*)chunk_offsets, d.T, H, H, d.V, scale, (int64_t)H * d.V);
+               (T*)nullptr, cu, (const int*)chunk_offsets, d.T, H, H, d.V, scale, (int64_t)H * d.V, (const T*)nullptr);
   }
   {
     auto kern = chunk_out_kernel<T, DK, NWO, false, T>;
@@ -449,7 +465,8 @@ extern "C" int gdn_kda_intermediate_states(const void* workspace, int64_t worksp
   ChunkDims dl = d;
   dl.varlen = true;
   const KdaWorkspace L = kda_workspace_layout(dl, dtype == 0 ? 4 : 2);
-  if (workspace_bytes < L.fwd_bytes || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
+  // the recurrence keeps the per-chunk states only in a workspace of the size that serves a backward pass
+  if (workspace_bytes < L.total_bytes || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return -5;
   if (h_chunks == 0) return 0;
   const unsigned char* ws = static_cast<const unsigned char*>(workspace);
   hipStream_t st = (hipStream_t)stream;

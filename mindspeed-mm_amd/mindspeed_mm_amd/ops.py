@@ -786,7 +786,8 @@ class _ChunkKda(torch.autograd.Function):
         bc, bcode = _beta_arg(beta, q.dtype)
         a32, d32, h0 = ops._f32(A_log), ops._f32(dt_bias), ops._f32(initial_state)
         cu = _i64(cu_seqlens, q)
-        nbytes = lib.gdn_kda_workspace_bytes(B, T, N, H, K, V, int(need_grad), code)
+        # the per-chunk states stay in the workspace only when it has the size that serves a backward pass
+        nbytes = lib.gdn_kda_workspace_bytes(B, T, N, H, K, V, int(need_grad or want_states), code)
         ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=q.device)
         off = (-ws.data_ptr()) % 256
         ws = ws[off:off + nbytes]

@@ -620,6 +620,21 @@ def test_kda_intermediate_states(ops, dtype, B, T, H, K, V, cu, transposed):
     assert "dq" in e and "h" in e
 
 
+def test_kda_output_from_the_recurrence_equals_the_output_kernel(ops):
+    """With one 32-column slab of the state per workgroup the 16-bit recurrence writes the output itself; with more
+    slabs than compute units it leaves states and v_new to the stand-alone output kernel.  Both accumulate a row in the
+    same order: batch row 0 alone (the first way) and inside a batch of four (the second way) give the same bits."""
+    B, T, H, K, V = 4, 200, 24, 128, 128
+    d = {n: t.cuda() for n, t in P.kda_inputs(B, T, H, K, V, BF, seed=3).items()}
+    kw = dict(output_final_state=True, use_qk_l2norm_in_kernel=True, use_gate_in_kernel=True,
+              use_beta_sigmoid_in_kernel=True, A_log=d["A_log"], dt_bias=d["dt_bias"])
+    with torch.no_grad():
+        o, ht = ops.chunk_kda(d["q"], d["k"], d["v"], d["g"], d["beta"], initial_state=d["h0"], **kw)
+        o1, ht1 = ops.chunk_kda(d["q"][:1], d["k"][:1], d["v"][:1], d["g"][:1], d["beta"][:1],
+                                initial_state=d["h0"][:1], **kw)
+    assert torch.equal(o[:1], o1) and torch.equal(ht[:1], ht1)
+
+
 def test_kda_argument_checks(ops):
     x = P.kda_inputs(1, 64, 2, 64, 64, BF)
     d = {n: t.cuda() for n, t in x.items()}
