@@ -105,7 +105,8 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
 
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
-  const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: branches and offsets from it are scalar
   const int h = blockIdx.y, nvalid = s.nvalid;
   const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk, hk = (int64_t)H * DK;
   const int64_t ch = (int64_t)blockIdx.x * H + h;

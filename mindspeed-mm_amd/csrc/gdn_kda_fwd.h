@@ -64,7 +64,8 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
 
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: branches and offsets from it are scalar
   const int h = blockIdx.y, nvalid = s.nvalid;
   const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk, hk = (int64_t)H * DK;
   const int64_t ch = (int64_t)blockIdx.x * H + h;
@@ -304,19 +305,41 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
   // ---- phase 1d: L and Aq as 64x64 fp32 matrices ----
   for (int i = tid; i < 64 * kLF; i += kThreads) { As[i] = 0.f; Aqs[i] = 0.f; Ti[i] = 0.f; }
   GDN_LDS_BARRIER();
-  // each entry is the sum of the two waves that share a tile (one per half of the channels): they add one after the other
+  // each entry is the sum of the two waves that share a tile (one per half of the channels): they add one after the
+  // other.  A wave reads all of its entries, then adds, then writes: entry by entry each read would wait for the write
+  // before it (the compiler must assume that the two matrices overlap).
 #pragma unroll
   for (int turn = 0; turn < 2; ++turn) {
     if (kh == turn) {
+      float ca[16], cq[16], bi[16];
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int i = 32 * td + acc_row(r), j = 32 * td + l32;
-        As[i * kLF + j] += i > j ? bs[i] * dgk[r] : 0.f;
-        Aqs[i * kLF + j] += i >= j ? scale * dgq[r] : 0.f;
-        if (wave < 2) {
+        ca[r] = As[i * kLF + j];
+        cq[r] = Aqs[i * kLF + j];
+        bi[r] = bs[i];
+      }
+      GDN_SCHED_FENCE();
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int i = 32 * td + acc_row(r), j = 32 * td + l32;
+        As[i * kLF + j] = ca[r] + (i > j ? bi[r] * dgk[r] : 0.f);
+        Aqs[i * kLF + j] = cq[r] + (i >= j ? scale * dgq[r] : 0.f);
+      }
+      if (wave < 2) {   // the tile below the diagonal
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
           const int i2 = 32 + acc_row(r);
-          As[i2 * kLF + l32] += bs[i2] * lowk[r];
-          Aqs[i2 * kLF + l32] += scale * lowq[r];
+          ca[r] = As[i2 * kLF + l32];
+          cq[r] = Aqs[i2 * kLF + l32];
+          bi[r] = bs[i2];
+        }
+        GDN_SCHED_FENCE();
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int i2 = 32 + acc_row(r);
+          As[i2 * kLF + l32] = ca[r] + bi[r] * lowk[r];
+          Aqs[i2 * kLF + l32] = cq[r] + scale * lowq[r];
         }
       }
     }
