@@ -66,7 +66,8 @@ __global__ __launch_bounds__(64 * (NW + NL)) GDN_WAVES_PER_SIMD((sizeof(T) == 2 
   constexpr int CK = DealB<PK, NT>::kPer, CTM = DealB<PTM, NT>::kPer, CD = DealB<PD, NT>::kPer;
   static_assert(STAGES == 1 || STAGES == 2, "one or two LDS stages");
 
-  const int tid = threadIdx.x, wave = tid >> 6;
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: the roles branch on a scalar
   const int nh = xcd_grouped_head(blockIdx.x, gridDim.x, Hv / Hqk), n = nh / Hv, h = nh % Hv;
   const int64_t bos = cu ? cu[n] : (int64_t)n * T_len;
   const int len = cu ? (int)(cu[n + 1] - bos) : T_len;

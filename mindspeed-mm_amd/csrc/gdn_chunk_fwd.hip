@@ -191,7 +191,8 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
 
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: branches and offsets from it are scalar
   const int hq = blockIdx.y, grp = Hv / Hqk, nvalid = s.nvalid;
   const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk;
 
@@ -351,7 +352,8 @@ void chunk_state_kernel(const T* __restrict__ kaf, const T* __restrict__ qtf, co
   static_assert(STAGES == 1 || STAGES == 2, "one or two LDS stages");
   static_assert(!OUT || STAGES == 2, "the output waves read a stage while the next one is filled");
 
-  const int tid = threadIdx.x, wave = tid >> 6;
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: the roles branch on a scalar
   const int nh = xcd_grouped_head(blockIdx.x, gridDim.x, Hv / Hqk), n = nh / Hv, h = nh % Hv;
   const int64_t bos = cu ? cu[n] : (int64_t)n * T_len;
   const int len = cu ? (int)(cu[n + 1] - bos) : T_len;
