@@ -142,17 +142,20 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     // 16-bit entries per register).  a: the row's token within the 32-token block, b: that of a column.  second: the
     // row index is the later token i (kept when i is in the second half of its block of 2^lg tokens and the column j
     // in the first half of the same block), else the row index is the earlier token j.
+    // In terms of bits: i and j share the block and sit in different halves of it when (i ^ j) >> (lg - 1) == 1, and
+    // the row's own half is bit lg - 1 of its index.  (Plain bit arithmetic: written with comparisons of the halves
+    // the compiler turns every entry into a branch.)
     for (int idx = tid; idx < 5 * 2 * 2 * 64; idx += kFinThreads) {
-      const int ln = idx & 63, second = (idx >> 6) & 1, kg = (idx >> 7) & 1, lg = (idx >> 8) + 1;
-      const int a = ln & 31, b0 = 16 * kg + 8 * (ln >> 5), n2 = (1 << lg) >> 1, nm = (1 << lg) - 1;
-      const bool rok = second ? ((a & nm) >= n2) : ((a & nm) < n2);
+      const int ln = idx & 63, second = (idx >> 6) & 1, kg = (idx >> 7) & 1, sh = idx >> 8;   // sh = lg - 1
+      const int a = ln & 31, b0 = 16 * kg + 8 * (ln >> 5);
+      const uint32_t rok = ((a >> sh) & 1) == second ? 0xffffffffu : 0u;
       u32x4 w;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int b1 = b0 + 2 * e, b2 = b1 + 1;
-        const bool k1 = rok && (a >> lg) == (b1 >> lg) && (second ? ((b1 & nm) < n2) : ((b1 & nm) >= n2));
-        const bool k2 = rok && (a >> lg) == (b2 >> lg) && (second ? ((b2 & nm) < n2) : ((b2 & nm) >= n2));
-        w[e] = (k1 ? 0xffffu : 0u) | (k2 ? 0xffff0000u : 0u);
+        const uint32_t k1 = ((a ^ b1) >> sh) == 1 ? 0xffffu : 0u;
+        const uint32_t k2 = ((a ^ b2) >> sh) == 1 ? 0xffff0000u : 0u;
+        w[e] = (k1 | k2) & rok;
       }
       keepT[idx] = w;
     }
