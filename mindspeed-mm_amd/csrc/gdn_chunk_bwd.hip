@@ -676,8 +676,16 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     const int j = 32 * tj + acc_col();
     const float gj = Gs[j];
     const f32x16 gi = rows_ld(Gs, 32 * ti);
+    // (every exponential first, then the selection: written as one conditional expression per entry the compiler
+    // branches around each exponential and the sixteen chains run one after the other)
+    float eg[16];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) ds[r] = (32 * ti + acc_row(r) >= j) ? scale * ds[r] * __expf(gi[r] - gj) : 0.f;
+    for (int r = 0; r < 16; ++r) {
+      eg[r] = __expf(fminf(gi[r] - gj, 0.f));
+      GDN_KEEP_HERE(eg[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) ds[r] = (32 * ti + acc_row(r) >= j) ? scale * ds[r] * eg[r] : 0.f;
     AccB<T> d, t;
     d.pack(ds);
     d.store(tileD + wave * 1024);
