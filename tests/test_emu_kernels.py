@@ -238,6 +238,34 @@ def test_kda_backward(ops, dtype, B, T, H, K, V, cu, kw):
     print({n: f"{e:.2e}" for n, e in errs.items()})
 
 
+def _random_kda_case(seed):
+    import random
+    rng = random.Random(1000 + seed)
+    B = rng.choice([1, 1, 2])
+    T = rng.randint(1, 200)
+    H = rng.choice([1, 2, 3])
+    K, V = rng.choice([64, 128]), rng.choice([64, 128, 192])
+    cu = None
+    if B == 1 and rng.random() < 0.6:
+        cuts = sorted(rng.sample(range(0, T + 1), min(T + 1, rng.randint(0, 4))))
+        cu = [0] + cuts + [T]
+    kw = dict(gate_in_kernel=rng.random() < 0.7, beta_sigmoid=rng.random() < 0.7, l2=rng.random() < 0.7,
+              transpose_state=rng.random() < 0.5, with_h0=rng.random() < 0.7, allow_neg=rng.random() < 0.3)
+    if kw["gate_in_kernel"] and rng.random() < 0.4:
+        kw["lower_bound"] = -5.0
+    if not kw["beta_sigmoid"]:
+        kw["allow_neg"] = False   # the doubled beta is an option of the in-kernel sigmoid
+    return (BF if seed % 2 else F32), B, T, H, K, V, cu, kw
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_kda_random_shapes(ops, seed):
+    """Seeded random shapes and options of chunk_kda, forward and backward: ragged and packed lengths with empty
+    members, both state layouts, with and without the in-kernel gate, sigmoid and norm."""
+    dtype, B, T, H, K, V, cu, kw = _random_kda_case(seed)
+    P.check_kda(ops, "cpu", B, T, H, K, V, dtype, cu=cu, backward=True, wrap=guarded, h0_std=0.1, seed=seed, **kw)
+
+
 @pytest.mark.parametrize("dtype,B,T,H,K,V,cu,kw", [
     (F32, 2, 100, 2, 128, 64, None, {}),
     (BF, 1, 200, 2, 64, 128, [0, 70, 70, 200], dict(transpose_state=False)),
