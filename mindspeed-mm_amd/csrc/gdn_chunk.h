@@ -91,7 +91,7 @@ struct KdaWorkspace {
   int64_t HF;             // T [chunks,H,V/32,K/32] state before each chunk
   int64_t fwd_bytes;
   // kept for a backward pass
-  int64_t GC;             // f32 [chunks,H,64,K]    chunk-local cumulative log decay
+  int64_t GC;             // f32 [chunks,H,64,K]    chunk-local cumulative log decay (16-bit kernels: times log2 e, see KdaDecay)
   int64_t TMR;            // T [chunks,H,64,64]     Tm row-major, as rounded for the tiles
   int64_t DVF;            // T [chunks,H,V/32,2]    d(v_new)
   int64_t DHF;            // T [chunks,H,V/32,K/32] gradient of the state AFTER each chunk

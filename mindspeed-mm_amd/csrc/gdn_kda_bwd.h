@@ -225,7 +225,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     float f[VEC];
     unpack16<T>(ld16(Ks + row * LDK + cc * VEC), f);
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) f[e] *= __expf(gk[it][e / 4][e % 4]);
+    for (int e = 0; e < VEC; ++e) f[e] *= KdaDecay<T>::exp(gk[it][e / 4][e % 4]);
     st16(Kp + row * LDK + cc * VEC, pack16<T>(f));
   }
   GDN_LDS_BARRIER();
@@ -358,7 +358,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
               const int x = 32 * ri + 16 * kg + 8 * half + e, sm = (((16 * kg + e) >> lg) << lg) + n2;
-              const float f = __expf(-fabsf(Gs[x * LDG + d] - Gpm[sm * LDG]));
+              const float f = KdaDecay<T>::exp(-fabsf(Gs[x * LDG + d] - Gpm[sm * LDG]));
               xk[e] = Elem<T>::to_f(Ks[x * LDK + d]) * f; xb[e] = bx[e] * xk[e]; xq[e] = Elem<T>::to_f(Qs[x * LDK + d]) * f;
             }
             const u32x4 bK = pack16<T>(xk).raw, bB = pack16<T>(xb).raw, bQ = pack16<T>(xq).raw;
@@ -372,7 +372,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
 #pragma unroll
           for (int r = 0; r < 16; ++r) {   // every row by its own factor
             const int sm = (((8 * (r / 4) + r % 4) >> lg) << lg) + n2;
-            const float f = __expf(-fabsf(Gi[r] - Gom[sm * LDG]));
+            const float f = KdaDecay<T>::exp(-fabsf(Gi[r] - Gom[sm * LDG]));
             U[r] += f * cu[r];
             Uq[r] += f * cq[r];
             W[r] += f * cw[r];
@@ -391,7 +391,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
               const int j = c0 + e;
-              xk[e] = Elem<T>::to_f(Ks[j * LDK + d]) * __expf(-fabsf(Gs[j * LDG + d] - g32v));
+              xk[e] = Elem<T>::to_f(Ks[j * LDK + d]) * KdaDecay<T>::exp(-fabsf(Gs[j * LDG + d] - g32v));
             }
             const u32x4 bK = pack16<T>(xk).raw;
             mfma_kgroup<T>(c1, ld16(M1 + (32 + l32) * L64 + c0).raw, bK);
@@ -401,7 +401,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
               const int i = 32 + c0 + e;
-              const float f = __expf(-fabsf(Gs[i * LDG + d] - g32v));
+              const float f = KdaDecay<T>::exp(-fabsf(Gs[i * LDG + d] - g32v));
               xb[e] = bs[i] * Elem<T>::to_f(Ks[i * LDK + d]) * f;
               xq[e] = Elem<T>::to_f(Qs[i * LDK + d]) * f;
             }
@@ -411,7 +411,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
         }
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const float f = __expf(-fabsf(Gi[r] - g32v));
+          const float f = KdaDecay<T>::exp(-fabsf(Gi[r] - g32v));
           if (ri == 1) { U[r] += f * c1[r]; Uq[r] += f * c2[r]; }
           else W[r] += f * c1[r];
         }
@@ -428,7 +428,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
 #pragma unroll
         for (int m = 0; m < 4; ++m) {
           const int r = 4 * qd + m, i = 32 * ri + acc_row(r);
-          const float t = kj * __expf(i >= jj ? Gi[r] - gj : 0.f);
+          const float t = kj * KdaDecay<T>::exp(i >= jj ? Gi[r] - gj : 0.f);
           U[r] += Elem<T>::to_f(M1[i * L64 + jj]) * t;    // coefficients are zero where i < jj
           Uq[r] += Elem<T>::to_f(M2[i * L64 + jj]) * t;
         }
@@ -443,7 +443,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
 #pragma unroll
         for (int m = 0; m < 4; ++m) {
           const int r = 4 * qd + m, j = 32 * ri + acc_row(r);
-          const float e = __expf(ii >= j ? gi - Gi[r] : 0.f);
+          const float e = KdaDecay<T>::exp(ii >= j ? gi - Gi[r] : 0.f);
           W[r] += (Elem<T>::to_f(M1[ii * L64 + j]) * kb + Elem<T>::to_f(M2[ii * L64 + j]) * qv) * e;
         }
       }
@@ -481,7 +481,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
       f32x16 pq;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        dqh[r] = scale * __expf(Gi[r]) * lq[r] + Uq[r];
+        dqh[r] = scale * KdaDecay<T>::exp(Gi[r]) * lq[r] + Uq[r];
         pq[r] = qi[r] * dqh[r];
         dGv[r] = pq[r];
       }
@@ -491,9 +491,9 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
       f32x16 pk, pb;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float eG = __expf(Gi[r]), b = bs[32 * ri + acc_row(r)];
+        const float eG = KdaDecay<T>::exp(Gi[r]), b = bs[32 * ri + acc_row(r)];
         const float t1 = -b * eG * dK1[r];
-        const float t2 = __expf(glast - Gi[r]) * lk[r];
+        const float t2 = KdaDecay<T>::exp(glast - Gi[r]) * lk[r];
         dkh[r] = t1 + t2 + b * U[r] + W[r];
         dGv[r] += ki[r] * (t1 + b * U[r] - t2 - W[r]);
         gl_sum += ki[r] * t2;
@@ -552,7 +552,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     acc_store_rows<T, false>(dqh, id, patch, dq + at, hk, nvalid - 32 * ri);
     acc_store_rows<T, false>(dkh, id, patch, dk + at, hk, nvalid - 32 * ri);
     // dG_last: column sum over all rows of this channel, plus the decay of the state
-    const float dglast = xgl[2 * cj * 32 + l32] + xgl[(2 * cj + 1) * 32 + l32] + dD[d] * __expf(Gs[63 * LDG + d]);
+    const float dglast = xgl[2 * cj * 32 + l32] + xgl[(2 * cj + 1) * 32 + l32] + dD[d] * KdaDecay<T>::exp(Gs[63 * LDG + d]);
     const bool first_half = lane < 32;
     const float a = fl.use_gate ? __expf(A_log[h]) : 0.f;
     const float bias = (fl.use_gate && dt_bias != nullptr) ? dt_bias[h * DK + d] : 0.f;

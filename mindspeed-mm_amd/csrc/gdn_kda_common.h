@@ -28,6 +28,20 @@ __device__ __forceinline__ void kda_softplus_sigmoid(float x, float& sp, float& 
   sg = x >= 0.f ? r : t * r;
 }
 
+// The cumulative log decay G enters the kernels only through e^{G}, e^{G_i - G_j}.  The 16-bit kernels keep it in units
+// of log 2 (G log2 e, applied once where the gate leaves its values), so that each of the many exponentials is the
+// hardware's base-2 instruction alone, without the multiplication in front of it; the workspace's GC then holds
+// G log2 e as well.  The fp32 kernels (the parity path) keep natural units: a difference of pre-scaled values carries
+// the rounding of both, which grows with |G| instead of with the difference.
+template <typename T> struct KdaDecay {
+  static constexpr bool kBase2 = sizeof(T) == 2;
+  static constexpr float kUnit = kBase2 ? 1.4426950408889634f : 1.f;   // G as stored = G * kUnit
+  static __device__ __forceinline__ float exp(float x) {
+    if constexpr (kBase2) return __builtin_amdgcn_exp2f(x);
+    else return __expf(x);
+  }
+};
+
 // VEC consecutive fp32 values of an LDS row
 template <int VEC> __device__ __forceinline__ void ld_f32(const float* p, float* f) {
 #pragma unroll

@@ -113,6 +113,7 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
   // the gate: log decay of every token and channel, 0 on the rows past the end (they leave the cumulative sum alone)
   {
     const float a = fl.use_gate ? __expf(A_log[h]) : 0.f;
+    const float au = a * KdaDecay<T>::kUnit, lbu = fl.lower_bound * KdaDecay<T>::kUnit;   // in the units G is kept in
     // MODE 0: g is the log decay itself; 1: -e^{A_log} softplus(g + bias); 2: lower_bound sigmoid(e^{A_log} (g + bias)).
     // One copy of the loop per mode: a test of the options per element would cost as much as the gate.
     auto gate_rows = [&](auto mode) {
@@ -124,8 +125,9 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           float x = __uint_as_float(g32 ? gw[i][e] : (gw[i][e >> 1] >> (16 * (e & 1))) << 16);
-          if (MODE == 1) x = -a * kda_softplus(x + bv[i][e]);
-          if (MODE == 2) x = fl.lower_bound * kda_sigmoid(a * (x + bv[i][e]));
+          if (MODE == 0) x *= KdaDecay<T>::kUnit;
+          if (MODE == 1) x = -au * kda_softplus(x + bv[i][e]);
+          if (MODE == 2) x = lbu * kda_sigmoid(a * (x + bv[i][e]));
           y[e] = row < nvalid ? x : 0.f;
         }
         *reinterpret_cast<f32x4*>(Gs + row * LDG + 4 * c4) = y;
@@ -198,7 +200,7 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
         ld_f32<VEC>(Gs + m * LDG + c0, gm);
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
-          const float f = __expf(-fabsf(gR[e] - gm[e]));
+          const float f = KdaDecay<T>::exp(-fabsf(gR[e] - gm[e]));
           xq[e] = fq[e] * f;
           xk[e] = fk[e] * f;
         }
@@ -214,10 +216,10 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
         unpack16<T>(ld16(Qs + (32 + l32) * LDK + c0), xq2);
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
-          const float fa = __expf(-fabsf(ga[e] - gm[e]));
+          const float fa = KdaDecay<T>::exp(-fabsf(ga[e] - gm[e]));
           xk2[e] *= fa;
           xq2[e] *= fa;
-          xb[e] = fk[e] * __expf(-fabsf(gR[e] - gm[e]));
+          xb[e] = fk[e] * KdaDecay<T>::exp(-fabsf(gR[e] - gm[e]));
         }
         const u32x4 bK = pack16<T>(xb).raw;
         mfma_kgroup<T>(lowk, pack16<T>(xk2).raw, bK);
@@ -249,7 +251,7 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
     unpack16<T>(ld16(Qs + row * LDK + cc * VEC), f);
     ld_f32<VEC>(Gs + row * LDG + cc * VEC, gi);
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) f[e] *= scale * __expf(gi[e]);
+    for (int e = 0; e < VEC; ++e) f[e] *= scale * KdaDecay<T>::exp(gi[e]);
     const Vec16<T> x = pack16<T>(f);
     if (QB_out != nullptr && row < nvalid) st16(QB_out + (tok0 + row) * hk + h * DK + cc * VEC, x);   // row-major for the output kernel
     st16(Qs + row * LDK + cc * VEC, x);
@@ -272,7 +274,7 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
       ld_f32<VEC>(Gs + 63 * LDG + cc * VEC, gl);
       const float nb = -bs[row];
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) f[e] *= first ? nb * __expf(gi[e]) : __expf(gl[e] - gi[e]);
+      for (int e = 0; e < VEC; ++e) f[e] *= first ? nb * KdaDecay<T>::exp(gi[e]) : KdaDecay<T>::exp(gl[e] - gi[e]);
       st16(Qs + row * LDK + cc * VEC, pack16<T>(f));
     }
   };
@@ -293,7 +295,7 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
   GDN_LDS_BARRIER();
   store_k(K2_out);
   // the decay of the whole chunk per channel, the cumulative decay itself
-  if (tid < DK) dec_out[ch * DK + tid] = __expf(Gs[63 * LDG + tid]);
+  if (tid < DK) dec_out[ch * DK + tid] = KdaDecay<T>::exp(Gs[63 * LDG + tid]);
   if (G_out != nullptr) {
     for (int c = tid; c < 64 * (DK / 4); c += kThreads) {
       const int row = c / (DK / 4), c4 = c % (DK / 4);

@@ -307,6 +307,7 @@ inline int emu_update_dpp(int /*old*/, int src, int ctrl) {
 #define __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, x, y, z) emu::mfma_16x16x4_f32(a, b, c)
 
 #define __expf(x) expf(x)
+#define __builtin_amdgcn_exp2f(x) exp2f(x)
 #define __logf(x) logf(x)
 static inline float __frsqrt_rn(float x) { return 1.0f / sqrtf(x); }
 static inline float rsqrtf(float x) { return 1.0f / sqrtf(x); }
