@@ -339,8 +339,11 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
           Uq[r] += c * Elem<T>::to_f(Ks[i * LDK + d]);
           W[r] += c * Elem<T>::to_f(Qs[i * LDK + d]);
         }
-#pragma unroll 1
-        for (int lg = 1; lg <= 5; ++lg) {   // blocks of n = 2^lg tokens inside the 32-token block
+        // One level: blocks of n = 2^lg tokens inside the 32-token block.  WIDE (lg >= 3): a block is at least as long as
+        // the 8 partner rows a half-wave holds per group and as the 8 rows that two of its accumulator groups span, so
+        // those rows share their reference row: one read of it instead of eight (or four).
+        auto level = [&](int lg, auto wide_c) {
+          constexpr bool WIDE = decltype(wide_c)::value != 0;
           const int n2 = (1 << lg) >> 1;
           asm volatile("" ::: "memory");   // the reads of a level stay inside it
           // The reference row of a token is the middle of its block of 2^lg tokens.  For the lane's 8 partner rows of a
@@ -355,10 +358,11 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
           for (int kg = 0; kg < 2; ++kg) {
             float xk[8], xb[8], xq[8], bx[8];
             ld_f32<8>(bs + 32 * ri + 16 * kg + 8 * half, bx);
+            const float gmid = WIDE ? Gpm[((((16 * kg) >> lg) << lg) + n2) * LDG] : 0.f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
               const int x = 32 * ri + 16 * kg + 8 * half + e, sm = (((16 * kg + e) >> lg) << lg) + n2;
-              const float f = KdaDecay<T>::exp(-fabsf(Gs[x * LDG + d] - Gpm[sm * LDG]));
+              const float f = KdaDecay<T>::exp(-fabsf(Gs[x * LDG + d] - (WIDE ? gmid : Gpm[sm * LDG])));
               xk[e] = Elem<T>::to_f(Ks[x * LDK + d]) * f; xb[e] = bx[e] * xk[e]; xq[e] = Elem<T>::to_f(Qs[x * LDK + d]) * f;
             }
             const u32x4 bK = pack16<T>(xk).raw, bB = pack16<T>(xb).raw, bQ = pack16<T>(xq).raw;
@@ -370,14 +374,22 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
             mfma_kgroup<T>(cw, ld16(M2t + row * L64 + col0).raw & keep1, bQ);
           }
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {   // every row by its own factor
-            const int sm = (((8 * (r / 4) + r % 4) >> lg) << lg) + n2;
-            const float f = KdaDecay<T>::exp(-fabsf(Gi[r] - Gom[sm * LDG]));
-            U[r] += f * cu[r];
-            Uq[r] += f * cq[r];
-            W[r] += f * cw[r];
+          for (int qd = 0; qd < 4; ++qd) {   // every row by its own factor
+            const float gq = WIDE ? Gom[((((8 * qd) >> lg) << lg) + n2) * LDG] : 0.f;
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+              const int r = 4 * qd + m, sm = (((8 * qd + m) >> lg) << lg) + n2;
+              const float f = KdaDecay<T>::exp(-fabsf(Gi[r] - (WIDE ? gq : Gom[sm * LDG])));
+              U[r] += f * cu[r];
+              Uq[r] += f * cq[r];
+              W[r] += f * cw[r];
+            }
           }
-        }
+        };
+#pragma unroll 1
+        for (int lg = 1; lg <= 2; ++lg) level(lg, IntConst<0>());
+#pragma unroll 1
+        for (int lg = 3; lg <= 5; ++lg) level(lg, IntConst<1>());
       }
       {   // the level of the whole chunk: tokens 32..63 against tokens 0..31, m = 32, every pair kept.  The wave of the
           // later tokens takes the sums over j (U, Uq), the wave of the earlier ones the sum over i (W)
