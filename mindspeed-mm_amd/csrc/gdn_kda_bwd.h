@@ -332,12 +332,20 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
         // The partner rows this lane supplies as B operand, channel d, are tokens 32 ri + 16 kg + 8 half + e.  They
         // are read again at every level: held in registers through the levels they would push other values out to
         // scratch memory, which costs more than the reads.
+        {   // the pair i = j: no decay (dL has no diagonal).  This lane's rows of k^ and q^, channel d: four transposing
+            // reads per tile instead of a two-byte read per row
+          AccB<T> t;
+          t.load_cols(Ks + 32 * ri * LDK + 32 * cj, LDK);
+          const f32x16 kd = t.unpack();
+          t.load_cols(Qs + 32 * ri * LDK + 32 * cj, LDK);
+          const f32x16 qd = t.unpack();
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {   // the pair i = j: no decay (dL has no diagonal)
-          const int i = 32 * ri + acc_row(r);
-          const float c = Elem<T>::to_f(M2[i * L64 + i]);
-          Uq[r] += c * Elem<T>::to_f(Ks[i * LDK + d]);
-          W[r] += c * Elem<T>::to_f(Qs[i * LDK + d]);
+          for (int r = 0; r < 16; ++r) {
+            const int i = 32 * ri + acc_row(r);
+            const float c = Elem<T>::to_f(M2[i * L64 + i]);
+            Uq[r] += c * kd[r];
+            W[r] += c * qd[r];
+          }
         }
         // One level: blocks of n = 2^lg tokens inside the 32-token block.  WIDE (lg >= 3): a block is at least as long as
         // the 8 partner rows a half-wave holds per group and as the 8 rows that two of its accumulator groups span, so
@@ -483,11 +491,21 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     }
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (!FULL) mma32<T, 64, false, false>(dK1, TmT + 32 * ri, L64, Pt + 32 * cj, LDK);
+    if constexpr (FULL) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int i = 32 * ri + acc_row(r);
-      ki[r] = Elem<T>::to_f(Ks[i * LDK + d]);
-      qi[r] = Elem<T>::to_f(Qs[i * LDK + d]);
+      for (int r = 0; r < 16; ++r) {
+        const int i = 32 * ri + acc_row(r);
+        ki[r] = Ks[i * LDK + d];
+        qi[r] = Qs[i * LDK + d];
+      }
+    } else {
+      AccB<T> t;
+      t.load_cols(Ks + 32 * ri * LDK + 32 * cj, LDK);
+      const f32x16 kd = t.unpack();
+      t.load_cols(Qs + 32 * ri * LDK + 32 * cj, LDK);
+      const f32x16 qd = t.unpack();
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { ki[r] = kd[r]; qi[r] = qd[r]; }
     }
     {
       f32x16 pq;
