@@ -486,6 +486,22 @@ template <typename T> struct AccB {
         for (int e = 0; e < 4; ++e) f[g][e] = __float_as_uint(Elem<T>::to_f(x[(8 * g + 4 * h + e) * ld + m]));
     }
   }
+  // As load_cols for 16-bit types, but the 8 rows a lane holds of k-group g are consecutive, 16 g + 8 (lane >> 5) + 0..7:
+  // the k order of an A operand that is read with one 16-byte read per k-group straight from a row-major tile.
+  __device__ __forceinline__ void load_cols_consecutive(const T* x, int ld) {
+    static_assert(sizeof(T) == 2, "16-bit types");
+    const int lane = threadIdx.x & 63;
+    const int gr = lane >> 4, i = lane & 15, e = i >> 2, q = i & 3, hh = gr >> 1;
+    const T* base = x + (8 * hh + e) * ld + (gr & 1) * 16 + 4 * q;
+#pragma unroll
+    for (int g = 0; g < 2; ++g)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const u32x2 r = lds_read_tr16(base + (16 * g + 4 * t) * ld);
+        f[g][2 * t] = r[0];
+        f[g][2 * t + 1] = r[1];
+      }
+  }
 };
 // d(32x32) += A[32 rows][32 k] * B(32 k x 32) with B packed from an accumulator; arow = &A[row of this lane][k0]
 template <typename T> __device__ __forceinline__ void mma32_accb(f32x16& d, const T* arow, const AccB<T>& b) {

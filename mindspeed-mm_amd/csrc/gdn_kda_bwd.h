@@ -362,16 +362,21 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
           const float* Gom = Gs + (32 * ri + (lg <= 2 ? 4 * half : 0)) * LDG + d;
           const u32x4* keepL = keepT + (lg - 1) * 4 * 64 + lane;
           f32x16 cu = acc_zero(), cq = acc_zero(), cw = acc_zero();
+          // the partner rows of k^ and q^, channel d, as they lie (16 kg + 8 half + e): four transposing reads per tile
+          AccB<T> kpart, qpart;
+          kpart.load_cols_consecutive(Ks + 32 * ri * LDK + 32 * cj, LDK);
+          qpart.load_cols_consecutive(Qs + 32 * ri * LDK + 32 * cj, LDK);
 #pragma unroll
           for (int kg = 0; kg < 2; ++kg) {
-            float xk[8], xb[8], xq[8], bx[8];
+            float xk[8], xb[8], xq[8], bx[8], kx[8], qx[8];
             ld_f32<8>(bs + 32 * ri + 16 * kg + 8 * half, bx);
+            { Vec16<T> v; v.raw = kpart.f[kg]; unpack16<T>(v, kx); v.raw = qpart.f[kg]; unpack16<T>(v, qx); }
             const float gmid = WIDE ? Gpm[((((16 * kg) >> lg) << lg) + n2) * LDG] : 0.f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
               const int x = 32 * ri + 16 * kg + 8 * half + e, sm = (((16 * kg + e) >> lg) << lg) + n2;
               const float f = KdaDecay<T>::exp(-fabsf(Gs[x * LDG + d] - (WIDE ? gmid : Gpm[sm * LDG])));
-              xk[e] = Elem<T>::to_f(Ks[x * LDK + d]) * f; xb[e] = bx[e] * xk[e]; xq[e] = Elem<T>::to_f(Qs[x * LDK + d]) * f;
+              xk[e] = kx[e] * f; xb[e] = bx[e] * xk[e]; xq[e] = qx[e] * f;
             }
             const u32x4 bK = pack16<T>(xk).raw, bB = pack16<T>(xb).raw, bQ = pack16<T>(xq).raw;
             const int row = 32 * ri + l32, col0 = 32 * ri + 16 * kg + 8 * half;
