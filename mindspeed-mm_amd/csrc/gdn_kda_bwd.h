@@ -408,27 +408,34 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
           // later tokens takes the sums over j (U, Uq), the wave of the earlier ones the sum over i (W)
         const float g32v = Gs[32 * LDG + d];
         f32x16 c1 = acc_zero(), c2 = acc_zero();
+        // the rows of the other 32-token block, channel d, as they lie (transposing reads)
+        AccB<T> kpart, qpart;
+        kpart.load_cols_consecutive(Ks + 32 * (1 - ri) * LDK + 32 * cj, LDK);
+        if (ri == 0) qpart.load_cols_consecutive(Qs + 32 * LDK + 32 * cj, LDK);
 #pragma unroll
         for (int kg = 0; kg < 2; ++kg) {
           const int c0 = 16 * kg + 8 * half;
+          float kx[8];
+          { Vec16<T> v; v.raw = kpart.f[kg]; unpack16<T>(v, kx); }
           if (ri == 1) {
             float xk[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
               const int j = c0 + e;
-              xk[e] = Elem<T>::to_f(Ks[j * LDK + d]) * KdaDecay<T>::exp(-fabsf(Gs[j * LDG + d] - g32v));
+              xk[e] = kx[e] * KdaDecay<T>::exp(-fabsf(Gs[j * LDG + d] - g32v));
             }
             const u32x4 bK = pack16<T>(xk).raw;
             mfma_kgroup<T>(c1, ld16(M1 + (32 + l32) * L64 + c0).raw, bK);
             mfma_kgroup<T>(c2, ld16(M2 + (32 + l32) * L64 + c0).raw, bK);
           } else {
-            float xb[8], xq[8];
+            float xb[8], xq[8], qx[8];
+            { Vec16<T> v; v.raw = qpart.f[kg]; unpack16<T>(v, qx); }
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
               const int i = 32 + c0 + e;
               const float f = KdaDecay<T>::exp(-fabsf(Gs[i * LDG + d] - g32v));
-              xb[e] = bs[i] * Elem<T>::to_f(Ks[i * LDK + d]) * f;
-              xq[e] = Elem<T>::to_f(Qs[i * LDK + d]) * f;
+              xb[e] = bs[i] * kx[e] * f;
+              xq[e] = qx[e] * f;
             }
             mfma_kgroup<T>(c1, ld16(M1t + l32 * L64 + 32 + c0).raw, pack16<T>(xb).raw);
             mfma_kgroup<T>(c1, ld16(M2t + l32 * L64 + 32 + c0).raw, pack16<T>(xq).raw);
