@@ -350,6 +350,11 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
         // One level: blocks of n = 2^lg tokens inside the 32-token block.  WIDE (lg >= 3): a block is at least as long as
         // the 8 partner rows a half-wave holds per group and as the 8 rows that two of its accumulator groups span, so
         // those rows share their reference row: one read of it instead of eight (or four).
+        // the partner rows of k^ and q^, channel d, as they lie (16 kg + 8 half + e): four transposing reads per tile,
+        // packed pairs held through the levels
+        AccB<T> kpart, qpart;
+        kpart.load_cols_consecutive(Ks + 32 * ri * LDK + 32 * cj, LDK);
+        qpart.load_cols_consecutive(Qs + 32 * ri * LDK + 32 * cj, LDK);
         auto level = [&](int lg, auto wide_c) {
           constexpr bool WIDE = decltype(wide_c)::value != 0;
           const int n2 = (1 << lg) >> 1;
@@ -362,10 +367,6 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
           const float* Gom = Gs + (32 * ri + (lg <= 2 ? 4 * half : 0)) * LDG + d;
           const u32x4* keepL = keepT + (lg - 1) * 4 * 64 + lane;
           f32x16 cu = acc_zero(), cq = acc_zero(), cw = acc_zero();
-          // the partner rows of k^ and q^, channel d, as they lie (16 kg + 8 half + e): four transposing reads per tile
-          AccB<T> kpart, qpart;
-          kpart.load_cols_consecutive(Ks + 32 * ri * LDK + 32 * cj, LDK);
-          qpart.load_cols_consecutive(Qs + 32 * ri * LDK + 32 * cj, LDK);
 #pragma unroll
           for (int kg = 0; kg < 2; ++kg) {
             float xk[8], xb[8], xq[8], bx[8], kx[8], qx[8];
