@@ -355,6 +355,11 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
         AccB<T> kpart, qpart;
         kpart.load_cols_consecutive(Ks + 32 * ri * LDK + 32 * cj, LDK);
         qpart.load_cols_consecutive(Qs + 32 * ri * LDK + 32 * cj, LDK);
+        float gpart[2][8];   // and their cumulative decays
+#pragma unroll
+        for (int kg = 0; kg < 2; ++kg)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) gpart[kg][e] = Gs[(32 * ri + 16 * kg + 8 * half + e) * LDG + d];
         auto level = [&](int lg, auto wide_c) {
           constexpr bool WIDE = decltype(wide_c)::value != 0;
           const int n2 = (1 << lg) >> 1;
@@ -375,8 +380,8 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
             const float gmid = WIDE ? Gpm[((((16 * kg) >> lg) << lg) + n2) * LDG] : 0.f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-              const int x = 32 * ri + 16 * kg + 8 * half + e, sm = (((16 * kg + e) >> lg) << lg) + n2;
-              const float f = KdaDecay<T>::exp(-fabsf(Gs[x * LDG + d] - (WIDE ? gmid : Gpm[sm * LDG])));
+              const int sm = (((16 * kg + e) >> lg) << lg) + n2;
+              const float f = KdaDecay<T>::exp(-fabsf(gpart[kg][e] - (WIDE ? gmid : Gpm[sm * LDG])));
               xk[e] = kx[e] * f; xb[e] = bx[e] * xk[e]; xq[e] = qx[e] * f;
             }
             const u32x4 bK = pack16<T>(xk).raw, bB = pack16<T>(xb).raw, bQ = pack16<T>(xq).raw;
