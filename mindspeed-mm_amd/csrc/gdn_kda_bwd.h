@@ -292,6 +292,9 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
   GDN_LDS_BARRIER();   // dTm, X, Kp are consumed (FULL: P too)
   // ---- phase A4: the coefficient matrices in place of dTm and X; G in place of Kp; q^ rows (FULL: in place of P) ----
   if (tile_wave) {
+    // the transposed dL carries the beta of its later token (its row in dL): the sum over i of dL_ij b_i k_i f_i then
+    // takes the same rescaled rows k_i f_i as the sum over j
+    const f32x16 bi = rows_ld(bs, 32 * ti);
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int at = (32 * ti + acc_row(r)) * L64 + 32 * tj + l32;
@@ -299,7 +302,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
       M2[at] = Elem<T>::from_f(sa[r]);
       if constexpr (!FULL) {
         const int att = (32 * tj + l32) * L64 + 32 * ti + acc_row(r);
-        M1t[att] = Elem<T>::from_f(dl[r]);
+        M1t[att] = Elem<T>::from_f(dl[r] * bi[r]);
         M2t[att] = Elem<T>::from_f(sa[r]);
       }
     }
@@ -374,22 +377,21 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
           f32x16 cu = acc_zero(), cq = acc_zero(), cw = acc_zero();
 #pragma unroll
           for (int kg = 0; kg < 2; ++kg) {
-            float xk[8], xb[8], xq[8], bx[8], kx[8], qx[8];
-            ld_f32<8>(bs + 32 * ri + 16 * kg + 8 * half, bx);
+            float xk[8], xq[8], kx[8], qx[8];
             { Vec16<T> v; v.raw = kpart.f[kg]; unpack16<T>(v, kx); v.raw = qpart.f[kg]; unpack16<T>(v, qx); }
             const float gmid = WIDE ? Gpm[((((16 * kg) >> lg) << lg) + n2) * LDG] : 0.f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
               const int sm = (((16 * kg + e) >> lg) << lg) + n2;
               const float f = KdaDecay<T>::exp(-fabsf(gpart[kg][e] - (WIDE ? gmid : Gpm[sm * LDG])));
-              xk[e] = kx[e] * f; xb[e] = bx[e] * xk[e]; xq[e] = qx[e] * f;
+              xk[e] = kx[e] * f; xq[e] = qx[e] * f;
             }
-            const u32x4 bK = pack16<T>(xk).raw, bB = pack16<T>(xb).raw, bQ = pack16<T>(xq).raw;
+            const u32x4 bK = pack16<T>(xk).raw, bQ = pack16<T>(xq).raw;
             const int row = 32 * ri + l32, col0 = 32 * ri + 16 * kg + 8 * half;
             const u32x4 keep1 = keepL[2 * kg * 64], keep2 = keepL[(2 * kg + 1) * 64];
             mfma_kgroup<T>(cu, ld16(M1 + row * L64 + col0).raw & keep2, bK);     // sum_j dL_ij (k_j f_j)
             mfma_kgroup<T>(cq, ld16(M2 + row * L64 + col0).raw & keep2, bK);
-            mfma_kgroup<T>(cw, ld16(M1t + row * L64 + col0).raw & keep1, bB);   // sum_i dL_ij (b_i k_i f_i)
+            mfma_kgroup<T>(cw, ld16(M1t + row * L64 + col0).raw & keep1, bK);   // sum_i (dL_ij b_i) (k_i f_i)
             mfma_kgroup<T>(cw, ld16(M2t + row * L64 + col0).raw & keep1, bQ);
           }
 #pragma unroll
@@ -440,7 +442,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
             for (int e = 0; e < 8; ++e) {
               const int i = 32 + c0 + e;
               const float f = KdaDecay<T>::exp(-fabsf(Gs[i * LDG + d] - g32v));
-              xb[e] = bs[i] * kx[e] * f;
+              xb[e] = kx[e] * f;
               xq[e] = qx[e] * f;
             }
             mfma_kgroup<T>(c1, ld16(M1t + l32 * L64 + 32 + c0).raw, pack16<T>(xb).raw);
