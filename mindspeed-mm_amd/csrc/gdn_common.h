@@ -272,6 +272,15 @@ __device__ __forceinline__ void load_tile_scaled(T* lds, int ld, const T* g, int
 // (bf16: 8 k values -> one 32x32x16 instruction; fp32: 4 k values -> four 32x32x2 instructions).
 template <typename T> struct KGroup { static constexpr int kLen = (sizeof(T) == 2) ? 16 : 8; };
 
+// Transposing read from LDS (ds_read_b64_tr_b16): every lane names 8 bytes (4 16-bit elements); within each group of
+// 16 lanes, lane 4 a + b receives element b of the lanes 4 e + a, e = 0..3.  Read as a 4 x 16 block of elements whose
+// row e is held, 4 columns each, by the lanes 4 e .. 4 e + 3: lane n of the group gets column n, rows 0..3.
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x2 lds_read_tr16(const void* p) {
+  const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
+  return __builtin_bit_cast(u32x2, v);
+}
+
 // contiguous: p points at element [row][k0]; the lane reads kVec consecutive k
 template <typename T> __device__ __forceinline__ u32x4 frag_contig(const T* p) {
   return *reinterpret_cast<const u32x4*>(p);
@@ -290,6 +299,18 @@ template <typename T> __device__ __forceinline__ u32x4 frag_strided(const T* p, 
     }
   }
   return r;
+}
+
+// strided, 16-bit types: tile points at element [k0][first of the wave's 32 columns] of a [k][ld] array in LDS; the lane
+// receives its 8 consecutive k (k0 + 8 (lane >> 5) ..) of column lane & 31 from two transposing reads instead of
+// gathering eight two-byte elements
+template <typename T> __device__ __forceinline__ u32x4 frag_strided_tr(const T* tile, int ld) {
+  static_assert(sizeof(T) == 2, "16-bit types");
+  const int lane = threadIdx.x & 63;
+  const int gr = lane >> 4, i = lane & 15, e = i >> 2, q = i & 3, hh = gr >> 1;
+  const T* base = tile + (8 * hh + e) * ld + (gr & 1) * 16 + 4 * q;
+  const u32x2 r0 = lds_read_tr16(base), r1 = lds_read_tr16(base + 4 * ld);
+  return u32x4{r0[0], r0[1], r1[0], r1[1]};
 }
 
 template <typename T> __device__ __forceinline__ void mfma_kgroup(f32x16& acc, u32x4 a, u32x4 b) {
@@ -317,8 +338,12 @@ __device__ __forceinline__ void mma32(f32x16& acc, const T* A, int lda, const T*
   for (int kg = 0; kg < KLEN / G; ++kg) {
     const int k = kg * G + half * V;
     u32x4 a, b;
-    if constexpr (A_KC) a = frag_contig(A + r32 * lda + k); else a = frag_strided(A + k * lda + r32, lda);
-    if constexpr (B_KC) b = frag_contig(B + r32 * ldb + k); else b = frag_strided(B + k * ldb + r32, ldb);
+    if constexpr (A_KC) a = frag_contig(A + r32 * lda + k);
+    else if constexpr (sizeof(T) == 2) a = frag_strided_tr(A + kg * G * lda, lda);
+    else a = frag_strided(A + k * lda + r32, lda);
+    if constexpr (B_KC) b = frag_contig(B + r32 * ldb + k);
+    else if constexpr (sizeof(T) == 2) b = frag_strided_tr(B + kg * G * ldb, ldb);
+    else b = frag_strided(B + k * ldb + r32, ldb);
     mfma_kgroup<T>(acc, a, b);
   }
 }
@@ -355,15 +380,6 @@ template <typename T> __device__ __forceinline__ u32x4 frag_a_split(const T* p) 
     return *reinterpret_cast<const u32x4*>(p + 4 * half);
   }
 }
-// Transposing read from LDS (ds_read_b64_tr_b16): every lane names 8 bytes (4 16-bit elements); within each group of
-// 16 lanes, lane 4 a + b receives element b of the lanes 4 e + a, e = 0..3.  Read as a 4 x 16 block of elements whose
-// row e is held, 4 columns each, by the lanes 4 e .. 4 e + 3: lane n of the group gets column n, rows 0..3.
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ u32x2 lds_read_tr16(const void* p) {
-  const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
-  return __builtin_bit_cast(u32x2, v);
-}
-
 // all k-groups of one 32x32 accumulator tile packed as operand fragments ("fragment order").  The same 1024
 // elements, stored as [k-group][lane][16 bytes], are also the on-memory format in which kernels hand tiles to
 // each other: a lane writes/reads 16 contiguous bytes per k-group and never goes through LDS.
