@@ -52,7 +52,8 @@ template <typename T, int DK> struct KdaBwdSmem {
   static constexpr int off_row = off_keep + (FULL ? 0 : 5 * 2 * 2 * 64 * 16);
   // beta, 1/|q|, 1/|k| [64 each]; row sums <q^,dq^>, <k^,dk^>, db, <R,v> [256 each]; per-wave scalars [8]; what the
   // two waves of a channel block exchange: parts of dG_last and d(dt_bias) [8][32 each], sum of dG over tokens 32.. [4][32]
-  static constexpr int bytes = off_row + (3 * 64 + 4 * 256 + 8 + 2 * 256 + 128) * 4;
+  // ... and the diagonal of scale dAq [64]
+  static constexpr int bytes = off_row + (3 * 64 + 4 * 256 + 8 + 2 * 256 + 128 + 64) * 4;
   static_assert(tile <= gmat, "Kp fits where G will be");
   static_assert(8 * Patch<T>::kElems * (int)sizeof(T) <= 3 * mat, "store patches fit");
   static_assert(bytes <= 160 * 1024, "one CU's LDS");
@@ -102,6 +103,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
   float* xgl = wsum + 8;    // [8][32] per wave and channel: its part of dG_last
   float* xdt = xgl + 256;   // [8][32] per wave and channel: its part of d(dt_bias)
   float* xblk = xdt + 256;  // [4][32] per channel: sum of dG over tokens 32..63
+  float* dgq = xblk + 128;  // [64] scale dAq_ii: the pair i = j of the decay-weighted sums
 
   const SeqInfo s = locate_chunk(blockIdx.x, cu, chunk_offsets, N, T_len);
   if (s.nvalid <= 0) return;
@@ -253,11 +255,20 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     const int j = 32 * tj + l32;
     const float bj = bs[j];
     float sv = 0.f;
+    f32x16 tmt;   // this wave's tile of Tm as the accumulator holds a tile
+    if constexpr (FULL) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) tmt[r] = TmT[(32 * ti + acc_row(r)) * L64 + j];
+    } else {
+      AccB<T> t;
+      t.load_cols(TmT + 32 * ti * L64 + 32 * tj, L64);
+      tmt = t.unpack();
+    }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int i = 32 * ti + acc_row(r);
       const float a2v = a2t[r];
-      sv += a2v * Elem<T>::to_f(TmT[i * L64 + j]);
+      sv += a2v * tmt[r];
       M1[i * L64 + j] = Elem<T>::from_f(i > j ? bj * (a2v - x[r]) : 0.f);
     }
     sv += __shfl_xor(sv, 32);
@@ -301,9 +312,22 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
       M1[at] = Elem<T>::from_f(dl[r]);
       M2[at] = Elem<T>::from_f(sa[r]);
       if constexpr (!FULL) {
-        const int att = (32 * tj + l32) * L64 + 32 * ti + acc_row(r);
-        M1t[att] = Elem<T>::from_f(dl[r] * bi[r]);
-        M2t[att] = Elem<T>::from_f(sa[r]);
+        if (ti == tj && acc_row(r) == l32) dgq[32 * ti + l32] = Elem<T>::to_f(Elem<T>::from_f(sa[r]));
+      }
+    }
+    if constexpr (!FULL) {   // the transposed copies: a lane's four consecutive rows of a group are four consecutive columns there
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        const int att = (32 * tj + l32) * L64 + 32 * ti + acc_row(4 * qd);
+        u32x2 w1, w2;
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+          const int r = 4 * qd + 2 * m;
+          w1[m] = f32x2_to_bf16x2(dl[r] * bi[r], dl[r + 1] * bi[r + 1]);
+          w2[m] = f32x2_to_bf16x2(sa[r], sa[r + 1]);
+        }
+        *reinterpret_cast<u32x2*>(M1t + att) = w1;
+        *reinterpret_cast<u32x2*>(M2t + att) = w2;
       }
     }
     tile_qk_finish<T, DK>(qt, Qs, LDK, nvalid, tid, fl.l2norm != 0, nullptr, 0, rsq, 1);
@@ -342,12 +366,11 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
           const f32x16 kd = t.unpack();
           t.load_cols(Qs + 32 * ri * LDK + 32 * cj, LDK);
           const f32x16 qd = t.unpack();
+          const f32x16 c = rows_ld(dgq, 32 * ri);
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const int i = 32 * ri + acc_row(r);
-            const float c = Elem<T>::to_f(M2[i * L64 + i]);
-            Uq[r] += c * kd[r];
-            W[r] += c * qd[r];
+            Uq[r] += c[r] * kd[r];
+            W[r] += c[r] * qd[r];
           }
         }
         // One level: blocks of n = 2^lg tokens inside the 32-token block.  WIDE (lg >= 3): a block is at least as long as
