@@ -95,7 +95,8 @@ struct KdaWorkspace {
   int64_t TMR;            // T [chunks,H,64,64]     Tm row-major, as rounded for the tiles
   int64_t DVF;            // T [chunks,H,V/32,2]    d(v_new)
   int64_t DHF;            // T [chunks,H,V/32,K/32] gradient of the state AFTER each chunk
-  int64_t DUMP;           // T [chunks,H][dQb | dK2 | P : 64,K each][dAq | a2 : 64,64 each]  sums over V of the chunk-local pass
+  int64_t DUMP;           // T [chunks,H][dQb | dK2 | P : 64,K each][dAq | a2 : 64,64 each]  sums over V of the chunk-local pass;
+                          //   P as rows, the others as 32x32 tiles in fragment order: (token block, channel block), (row block, column block)
   int64_t DD;             // f32 [chunks,H,K]       sum over V of dS' . S: the gradient of the chunk's decay per channel
   int64_t PART;           // f32 [chunks,H][1 + K]  partial sums of dA_log and d(dt_bias)
   int64_t total_bytes;

@@ -623,21 +623,28 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     GDN_WAIT_VMEM();
     GDN_LDS_BARRIER();   // the last block's stage is consumed: its place takes the store patches
     T* patch = stage0 + SM::sh + wave * Patch<T>::kElems;
+    // dQb, dK2 and the two 64x64 sums leave as tiles in fragment order (the finish kernel wants them element by
+    // element in the accumulator layout): tile (token block, channel block) resp. (row block, column block); P, which
+    // it feeds to the matrix cores from LDS, as rows
     if (has_k) {
 #pragma unroll
       for (int ri = 0; ri < 2; ++ri) {
-        T* at = dump + 32 * ri * DK + 32 * cj;
-        acc_store_rows<T, false>(dQi[ri], id, patch, at, DK, 32);
-        acc_store_rows<T, false>(dKi[ri], id, patch, at + 64 * DK, DK, 32);
-        acc_store_rows<T, false>(dWa[ri], id, patch, at + 2 * 64 * DK, DK, 32);
+        AccB<T> f;
+        f.pack(dQi[ri]);
+        f.store_stream(dump + (ri * NKT + cj) * 1024);
+        f.pack(dKi[ri]);
+        f.store_stream(dump + 64 * DK + (ri * NKT + cj) * 1024);
+        acc_store_rows<T, false>(dWa[ri], id, patch, dump + 2 * 64 * DK + 32 * ri * DK + 32 * cj, DK, 32);
       }
       sds += __shfl_xor(sds, 32);   // the other half of the V block's rows
       if (lane < 32) kda_dd[ch * DK + 32 * cj + lane] = sds;
     }
     if (lower) {
-      T* at = dump + 3 * 64 * DK + 32 * ti * 64 + 32 * tj;
-      acc_store_rows<T, false>(ds, id, patch, at, 64, 32);
-      acc_store_rows<T, false>(a2, id, patch, at + 64 * 64, 64, 32);
+      AccB<T> f;
+      f.pack(ds);
+      f.store_stream(dump + 3 * 64 * DK + (2 * ti + tj) * 1024);
+      f.pack(a2);
+      f.store_stream(dump + 3 * 64 * DK + 64 * 64 + (2 * ti + tj) * 1024);
     }
     return;
   }

@@ -125,32 +125,12 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
   // ---- phase A0: k^ rows; P and Tm as operands; beta.  The tile waves request their tiles of a2 and dAq now ----
   TileQK<T, DK> kt, qt;     // moved by the first kThreads threads
   if (tile_wave) tile_qk_request<T, DK>(kt, k + tok0 * hk + h * DK, hk, nvalid, tid);
-  // FULL: element by element into registers (every tile wave loads, also the one of the upper tile, which nobody wrote:
-  // a test per load would make each of them wait for the one before; what it reads is dropped below), as bits, widened
-  // where they are used: anything done to a value here waits for its load.
-  // Not FULL: the whole workgroup moves both matrices in 16-byte pieces to the places of the transposed coefficient
-  // matrices (free until phase A4), where the tile waves pick their tiles up with four transposing reads each: an
-  // eighth of the load instructions, and no registers held from here to phases A1 and A3.
-  uint32_t a2r[FULL ? 16 : 1], dar[FULL ? 16 : 1];
-  constexpr int NA2 = FULL ? 1 : 64 * (64 / VEC) / kFinThreads;
-  static_assert(FULL || 64 * (64 / VEC) % kFinThreads == 0, "whole rounds of 16-byte pieces");
-  Vec16<T> a2v[NA2], dav[NA2];
-  if constexpr (FULL) {
-    if (tile_wave) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int at = (32 * ti + acc_row(r)) * 64 + 32 * tj + l32;
-        a2r[r] = reinterpret_cast<const uint32_t*>(a2m)[at];
-        dar[r] = reinterpret_cast<const uint32_t*>(dAq)[at];
-      }
-    }
-  } else {
-#pragma unroll
-    for (int it = 0; it < NA2; ++it) {
-      const int c = tid + it * kFinThreads;
-      a2v[it] = ld16(a2m + c * VEC);
-      dav[it] = ld16(dAq + c * VEC);
-    }
+  // a2 and dAq arrive as tiles in fragment order: a tile wave takes its own (every tile wave loads, also the one of the
+  // upper tile, which nobody wrote: what it reads is dropped below)
+  AccB<T> a2f, daf;
+  if (tile_wave) {
+    a2f.load(a2m + (2 * ti + tj) * 1024);
+    daf.load(dAq + (2 * ti + tj) * 1024);
   }
   u32x4* keepT = reinterpret_cast<u32x4*>(gdn_smem + SM::off_keep);
   if constexpr (!FULL) {
@@ -210,14 +190,6 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     const int c = tid + it * kFinThreads;
     st16(TmT + (c / C64) * L64 + (c % C64) * VEC, tmv[it]);
   }
-  if constexpr (!FULL) {
-#pragma unroll
-    for (int it = 0; it < NA2; ++it) {
-      const int c = tid + it * kFinThreads;
-      st16(M1t + (c / C64) * L64 + (c % C64) * VEC, a2v[it]);
-      st16(M2t + (c / C64) * L64 + (c % C64) * VEC, dav[it]);
-    }
-  }
   GDN_LDS_BARRIER();   // the row vectors are initialised before the norm below writes 1/|k| over its entries
   if (tile_wave) tile_qk_finish<T, DK>(kt, Ks, LDK, nvalid, tid, fl.l2norm != 0, nullptr, 0, rsk, 1);
   GDN_LDS_BARRIER();
@@ -234,21 +206,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
 
   // ---- phase A1: dTm = stril(b_j (a2 - P Kp^T)), one 32x32 tile per tile wave; <R_t, v_t> from Tm and a2 ----
   f32x16 a2t = acc_zero(), dat = acc_zero();
-  if (lower) {
-    if constexpr (FULL) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        GDN_KEEP_HERE(a2r[r]);
-        GDN_KEEP_HERE(dar[r]);
-        a2t[r] = __uint_as_float(a2r[r]);
-        dat[r] = __uint_as_float(dar[r]);
-      }
-    } else {
-      AccB<T> t;
-      t.load_cols(M1t + 32 * ti * L64 + 32 * tj, L64);
-      a2t = t.unpack();
-    }
-  }
+  if (lower) a2t = a2f.unpack();
   if (tile_wave) {
     f32x16 x = acc_zero();
     if (lower) mma32<T, DK, true, true>(x, Pt + 32 * ti * LDK, LDK, Kp + 32 * tj * LDK, LDK);
@@ -287,13 +245,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
   f32x16 dK1 = acc_zero(), dl = acc_zero(), sa;
   if (lower) mma32<T, 64, true, true>(dl, M2 + 32 * ti * L64, L64, TmT + 32 * tj * L64, L64);
   if (FULL && has_k) mma32<T, 64, false, false>(dK1, TmT + 32 * ri, L64, Pt + 32 * cj, LDK);
-  if constexpr (!FULL) {
-    if (lower) {   // dAq from its staging place, which the next phase overwrites
-      AccB<T> t;
-      t.load_cols(M2t + 32 * ti * L64 + 32 * tj, L64);
-      dat = t.unpack();
-    }
-  }
+  if (lower) dat = daf.unpack();
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int i = 32 * ti + acc_row(r), j = 32 * tj + l32;
@@ -525,13 +477,10 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     float gl_sum = 0.f, blk = 0.f;
     // the sums over V of this lane's rows: all requested before the first is used, and used in two passes so that few
     // intermediate rows are alive at a time (a schedule that runs out of registers waits after every load)
-    float lq[16], lk[16];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int i = 32 * ri + acc_row(r);
-      lq[r] = Elem<T>::to_f(dQb[i * DK + d]);
-      lk[r] = Elem<T>::to_f(dK2[i * DK + d]);
-    }
+    // (tiles in fragment order: token block ri, channel block cj)
+    AccB<T> lqf, lkf;
+    lqf.load(dQb + (ri * NKT + cj) * 1024);
+    lkf.load(dK2 + (ri * NKT + cj) * 1024);
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (!FULL) mma32<T, 64, false, false>(dK1, TmT + 32 * ri, L64, Pt + 32 * cj, LDK);
     if constexpr (FULL) {
@@ -550,6 +499,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) { ki[r] = kd[r]; qi[r] = qd[r]; }
     }
+    const f32x16 lq = lqf.unpack(), lk = lkf.unpack();
     {
       f32x16 pq;
 #pragma unroll
