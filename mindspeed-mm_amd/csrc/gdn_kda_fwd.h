@@ -70,10 +70,9 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
   const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk, hk = (int64_t)H * DK;
   const int64_t ch = (int64_t)blockIdx.x * H + h;
 
-  // ---- phase 0: requests first: k, q rows, the gate input (4 channels per piece), beta ----
+  // ---- phase 0: requests first: the gate input (4 channels per piece; loads arrive in the order of their requests
+  //      and the gate is what the workgroup computes first), then k and q rows, beta ----
   TileQK<T, DK> kt, qt;
-  tile_qk_request<T, DK>(kt, k + tok0 * hk + h * DK, hk, nvalid, tid);
-  tile_qk_request<T, DK>(qt, q + tok0 * hk + h * DK, hk, nvalid, tid);
   constexpr int GP = 64 * (DK / 4) / kThreads;
   const bool g32 = sizeof(T) == 4 || fl.g_f32;
   // as bits, and with one branch around each whole round of requests: a conversion or a test between two loads would
@@ -101,6 +100,8 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
 #pragma unroll
     for (int i = 0; i < GP; ++i) { bv[i][0] = 0.f; bv[i][1] = 0.f; bv[i][2] = 0.f; bv[i][3] = 0.f; }
   }
+  tile_qk_request<T, DK>(kt, k + tok0 * hk + h * DK, hk, nvalid, tid);
+  tile_qk_request<T, DK>(qt, q + tok0 * hk + h * DK, hk, nvalid, tid);
   if (wave == 0) {
     const int64_t at = (tok0 + imin(lane, nvalid - 1)) * H + h;
     float b;
