@@ -125,13 +125,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
   // ---- phase A0: k^ rows; P and Tm as operands; beta.  The tile waves request their tiles of a2 and dAq now ----
   TileQK<T, DK> kt, qt;     // moved by the first kThreads threads
   if (tile_wave) tile_qk_request<T, DK>(kt, k + tok0 * hk + h * DK, hk, nvalid, tid);
-  // a2 and dAq arrive as tiles in fragment order: a tile wave takes its own (every tile wave loads, also the one of the
-  // upper tile, which nobody wrote: what it reads is dropped below)
   AccB<T> a2f, daf;
-  if (tile_wave) {
-    a2f.load(a2m + (2 * ti + tj) * 1024);
-    daf.load(dAq + (2 * ti + tj) * 1024);
-  }
   u32x4* keepT = reinterpret_cast<u32x4*>(gdn_smem + SM::off_keep);
   if constexpr (!FULL) {
     // Which of 8 consecutive entries of a coefficient row belong to a level's pairs, as a mask over the fragment (two
@@ -172,6 +166,12 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
   for (int it = 0; it < NTM; ++it) {
     const int c = tid + it * kFinThreads;
     tmv[it] = ld16(TMR + ch * 4096 + (c / C64) * 64 + (c % C64) * VEC);
+  }
+  // a2 and dAq arrive as tiles in fragment order: a tile wave takes its own (every tile wave loads, also the one of the
+  // upper tile, which nobody wrote: what it reads is dropped below).  Requested behind what the first barrier waits for.
+  if (tile_wave) {
+    a2f.load(a2m + (2 * ti + tj) * 1024);
+    daf.load(dAq + (2 * ti + tj) * 1024);
   }
   if (tile_wave) tile_qk_request<T, DK>(qt, q + tok0 * hk + h * DK, hk, nvalid, tid);
   if (tid < 64) {
