@@ -173,7 +173,11 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     a2f.load(a2m + (2 * ti + tj) * 1024);
     daf.load(dAq + (2 * ti + tj) * 1024);
   }
-  if (tile_wave) tile_qk_request<T, DK>(qt, q + tok0 * hk + h * DK, hk, nvalid, tid);
+  // q^ rows: in the 16-bit kernel they have a place of their own, and the waves that own no tile of the 64x64 phases
+  // normalise them during those phases
+  constexpr bool Q_BY_OTHERS = !FULL;
+  const bool q_wave = Q_BY_OTHERS ? !tile_wave : tile_wave;
+  if (q_wave) tile_qk_request<T, DK>(qt, q + tok0 * hk + h * DK, hk, nvalid, tid & (kThreads - 1));
   if (tid < 64) {
     bs[tid] = tid < nvalid ? bhat[(tok0 + tid) * H + h] : 0.f;
     rsq[tid] = 1.f;
@@ -204,6 +208,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
   }
   GDN_LDS_BARRIER();
 
+  if (Q_BY_OTHERS && q_wave) tile_qk_finish<T, DK>(qt, Qs, LDK, nvalid, tid & (kThreads - 1), fl.l2norm != 0, nullptr, 0, rsq, 1);
   // ---- phase A1: dTm = stril(b_j (a2 - P Kp^T)), one 32x32 tile per tile wave; <R_t, v_t> from Tm and a2 ----
   f32x16 a2t = acc_zero(), dat = acc_zero();
   if (lower) a2t = a2f.unpack();
@@ -282,7 +287,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
         *reinterpret_cast<u32x2*>(M2t + att) = w2;
       }
     }
-    tile_qk_finish<T, DK>(qt, Qs, LDK, nvalid, tid, fl.l2norm != 0, nullptr, 0, rsq, 1);
+    if constexpr (!Q_BY_OTHERS) tile_qk_finish<T, DK>(qt, Qs, LDK, nvalid, tid, fl.l2norm != 0, nullptr, 0, rsq, 1);
   }
 #pragma unroll
   for (int it = 0; it < NIT; ++it) {
