@@ -783,27 +783,28 @@ __device__ __forceinline__ float wave_sum(float v) {
 // the row, modeling_qwen3_5.py:392-395; fp32 arithmetic, result rounded to T; a row sits on DK/VEC neighbouring lanes
 // that combine their partial sums with data-parallel-primitive moves), writes the tile to
 // LDS and, on request, the normalised rows (row stride y_stride) and 1/|x| (stride rstd_stride) to global memory.
-template <typename T, int DK> struct TileQK {
-  static constexpr int V = Elem<T>::kVec, CPR = DK / V, PT = 64 * CPR / kThreads;   // lanes per row; pieces per thread
-  static_assert((64 * CPR) % kThreads == 0, "every thread takes the same number of pieces");
+// NT: the threads that move the tile (tid = 0 .. NT - 1).
+template <typename T, int DK, int NT = kThreads> struct TileQK {
+  static constexpr int V = Elem<T>::kVec, CPR = DK / V, PT = 64 * CPR / NT;   // lanes per row; pieces per thread
+  static_assert((64 * CPR) % NT == 0, "every thread takes the same number of pieces");
   Vec16<T> x[PT];
 };
-template <typename T, int DK>
-__device__ __forceinline__ void tile_qk_request(TileQK<T, DK>& t, const T* g, int64_t row_stride, int nvalid, int tid) {
-  constexpr int V = TileQK<T, DK>::V, CPR = TileQK<T, DK>::CPR;
+template <typename T, int DK, int NT>
+__device__ __forceinline__ void tile_qk_request(TileQK<T, DK, NT>& t, const T* g, int64_t row_stride, int nvalid, int tid) {
+  constexpr int V = TileQK<T, DK, NT>::V, CPR = TileQK<T, DK, NT>::CPR;
 #pragma unroll
-  for (int i = 0; i < TileQK<T, DK>::PT; ++i) {
-    const int c = tid + i * kThreads, row = c / CPR, cc = c % CPR;
+  for (int i = 0; i < TileQK<T, DK, NT>::PT; ++i) {
+    const int c = tid + i * NT, row = c / CPR, cc = c % CPR;
     t.x[i] = ld16(g + (int64_t)imin(row, nvalid - 1) * row_stride + cc * V);   // the same load on every path
   }
 }
-template <typename T, int DK>
-__device__ __forceinline__ void tile_qk_finish(TileQK<T, DK>& t, T* lds, int ld, int nvalid, int tid, bool l2norm,
+template <typename T, int DK, int NT>
+__device__ __forceinline__ void tile_qk_finish(TileQK<T, DK, NT>& t, T* lds, int ld, int nvalid, int tid, bool l2norm,
                                                T* y_out, int64_t y_stride, float* rstd_out, int64_t rstd_stride) {
-  constexpr int V = TileQK<T, DK>::V, CPR = TileQK<T, DK>::CPR;
+  constexpr int V = TileQK<T, DK, NT>::V, CPR = TileQK<T, DK, NT>::CPR;
 #pragma unroll
-  for (int i = 0; i < TileQK<T, DK>::PT; ++i) {
-    const int c = tid + i * kThreads, row = c / CPR, cc = c % CPR;
+  for (int i = 0; i < TileQK<T, DK, NT>::PT; ++i) {
+    const int c = tid + i * NT, row = c / CPR, cc = c % CPR;
     const bool ok = row < nvalid;
     Vec16<T> x = ok ? t.x[i] : zero16<T>();
     if (l2norm) {   // uniform: every lane takes part in the shuffles

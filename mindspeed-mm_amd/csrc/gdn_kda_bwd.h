@@ -123,8 +123,9 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
   const float* Gc = GC + ch * 64 * DK;
 
   // ---- phase A0: k^ rows; P and Tm as operands; beta.  The tile waves request their tiles of a2 and dAq now ----
-  TileQK<T, DK> kt, qt;     // moved by the first kThreads threads
-  if (tile_wave) tile_qk_request<T, DK>(kt, k + tok0 * hk + h * DK, hk, nvalid, tid);
+  TileQK<T, DK, kFinThreads> kt;   // moved by every thread
+  TileQK<T, DK> qt;                // moved by kThreads threads, see below
+  tile_qk_request<T, DK>(kt, k + tok0 * hk + h * DK, hk, nvalid, tid);
   AccB<T> a2f, daf;
   u32x4* keepT = reinterpret_cast<u32x4*>(gdn_smem + SM::off_keep);
   if constexpr (!FULL) {
@@ -195,7 +196,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     st16(TmT + (c / C64) * L64 + (c % C64) * VEC, tmv[it]);
   }
   GDN_LDS_BARRIER();   // the row vectors are initialised before the norm below writes 1/|k| over its entries
-  if (tile_wave) tile_qk_finish<T, DK>(kt, Ks, LDK, nvalid, tid, fl.l2norm != 0, nullptr, 0, rsk, 1);
+  tile_qk_finish<T, DK>(kt, Ks, LDK, nvalid, tid, fl.l2norm != 0, nullptr, 0, rsk, 1);
   GDN_LDS_BARRIER();
 #pragma unroll
   for (int it = 0; it < NIT; ++it) {   // Kp = k^ . e^{G}
