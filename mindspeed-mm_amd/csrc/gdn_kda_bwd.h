@@ -136,7 +136,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     // In terms of bits: i and j share the block and sit in different halves of it when (i ^ j) >> (lg - 1) == 1, and
     // the row's own half is bit lg - 1 of its index.  (Plain bit arithmetic: written with comparisons of the halves
     // the compiler turns every entry into a branch.)
-    for (int idx = tid; idx < 5 * 2 * 2 * 64; idx += kFinThreads) {
+    for (int idx = 2 * 2 * 2 * 64 + tid; idx < 5 * 2 * 2 * 64; idx += kFinThreads) {   // levels of 8, 16, 32 tokens
       const int ln = idx & 63, second = (idx >> 6) & 1, kg = (idx >> 7) & 1, sh = idx >> 8;   // sh = lg - 1
       const int a = ln & 31, b0 = 16 * kg + 8 * (ln >> 5);
       const uint32_t rok = ((a >> sh) & 1) == second ? 0xffffffffu : 0u;
@@ -330,10 +330,50 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
             Uq[r] += c[r] * kd[r];
             W[r] += c[r] * qd[r];
           }
+          // The levels of 2 and 4 tokens inside the lane: the four rows of an accumulator group, tokens t0 .. t0 + 3, are
+          // one block of 4, and every pair of these two levels has both of its rows there.  Level 2: pairs (1,0), (3,2),
+          // reference row = the later token; level 4: i in {2,3}, j in {0,1}, reference row 2.  Coefficients: rows 1..3
+          // of the block's 4x4 diagonal piece of dL and of scale dAq, 8 bytes each, the same for every lane of a
+          // half-wave.  One exponential per pair member instead of one per row and level, and no matrix products.
+          const f32x16 bo = rows_ld(bs, 32 * ri);
+#pragma unroll
+          for (int g4 = 0; g4 < 4; ++g4) {
+            const int t0 = 32 * ri + 8 * g4 + 4 * half, r0 = 4 * g4;
+            f32x4 cl[3], ca[3];
+#pragma unroll
+            for (int m = 1; m < 4; ++m) {
+              const u32x2 wl = *reinterpret_cast<const u32x2*>(M1 + (t0 + m) * L64 + t0);
+              const u32x2 wa = *reinterpret_cast<const u32x2*>(M2 + (t0 + m) * L64 + t0);
+              cl[m - 1] = f32x4{__uint_as_float(wl[0] << 16), __uint_as_float(wl[0] & 0xffff0000u),
+                                __uint_as_float(wl[1] << 16), __uint_as_float(wl[1] & 0xffff0000u)};
+              ca[m - 1] = f32x4{__uint_as_float(wa[0] << 16), __uint_as_float(wa[0] & 0xffff0000u),
+                                __uint_as_float(wa[1] << 16), __uint_as_float(wa[1] & 0xffff0000u)};
+            }
+            float bk[4];
+#pragma unroll
+            for (int m = 0; m < 4; ++m) bk[m] = bo[r0 + m] * kd[r0 + m];
+            // rows t0 + i > t0 + j of the block, decay factor w = e^{G_i - G_j}
+#define GDN_KDA_PAIR(i, j, w)                                                              \
+            do {                                                                           \
+              const float dl_ = cl[(i) - 1][j], sa_ = ca[(i) - 1][j], w_ = (w), kjw_ = kd[r0 + (j)] * w_; \
+              U[r0 + (i)] += dl_ * kjw_;                                                   \
+              Uq[r0 + (i)] += sa_ * kjw_;                                                  \
+              W[r0 + (j)] += (dl_ * bk[i] + sa_ * qd[r0 + (i)]) * w_;                      \
+            } while (0)
+            GDN_KDA_PAIR(1, 0, KdaDecay<T>::exp(Gi[r0 + 1] - Gi[r0]));
+            const float f3 = KdaDecay<T>::exp(Gi[r0 + 3] - Gi[r0 + 2]);
+            GDN_KDA_PAIR(3, 2, f3);
+            const float g0 = KdaDecay<T>::exp(Gi[r0 + 2] - Gi[r0]), g1 = KdaDecay<T>::exp(Gi[r0 + 2] - Gi[r0 + 1]);
+            GDN_KDA_PAIR(2, 0, g0);
+            GDN_KDA_PAIR(2, 1, g1);
+            GDN_KDA_PAIR(3, 0, f3 * g0);
+            GDN_KDA_PAIR(3, 1, f3 * g1);
+#undef GDN_KDA_PAIR
+          }
         }
-        // One level: blocks of n = 2^lg tokens inside the 32-token block.  WIDE (lg >= 3): a block is at least as long as
-        // the 8 partner rows a half-wave holds per group and as the 8 rows that two of its accumulator groups span, so
-        // those rows share their reference row: one read of it instead of eight (or four).
+        // The levels of 8, 16 and 32 tokens on the matrix cores.  A block is at least as long as the 8 partner rows a
+        // half-wave holds per group and as the 8 rows that two of its accumulator groups span, so those rows share their
+        // reference row: one read of it instead of eight (or four).
         // the partner rows of k^ and q^, channel d, as they lie (16 kg + 8 half + e): four transposing reads per tile,
         // packed pairs held through the levels
         AccB<T> kpart, qpart;
@@ -388,8 +428,6 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
             }
           }
         };
-#pragma unroll 1
-        for (int lg = 1; lg <= 2; ++lg) level(lg, IntConst<0>());
 #pragma unroll 1
         for (int lg = 3; lg <= 5; ++lg) level(lg, IntConst<1>());
       }
