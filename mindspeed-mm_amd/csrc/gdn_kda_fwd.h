@@ -244,57 +244,122 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
   level_pass(IntConst<3>(), IntConst<2>(), IntConst<0>(), IntConst<1>());
   GDN_LDS_BARRIER();   // every wave is done with q as it lies: its place becomes the staging tile
 
-  // ---- phase 1c: what the recurrence reads, through a row-major staging tile (the q rows' place) into fragment order:
-  //      rows of q with scale and decay first (in place), then the two K images ----
-  for (int c = tid; c < 64 * CPR; c += kThreads) {
-    const int row = c / CPR, cc = c % CPR;
-    float f[VEC], gi[VEC];
-    unpack16<T>(ld16(Qs + row * LDK + cc * VEC), f);
-    ld_f32<VEC>(Gs + row * LDG + cc * VEC, gi);
-#pragma unroll
-    for (int e = 0; e < VEC; ++e) f[e] *= scale * KdaDecay<T>::exp(gi[e]);
-    const Vec16<T> x = pack16<T>(f);
-    if (QB_out != nullptr && row < nvalid) st16(QB_out + (tok0 + row) * hk + h * DK + cc * VEC, x);   // row-major for the output kernel
-    st16(Qs + row * LDK + cc * VEC, x);
-  }
-  if (QBT_out != nullptr) {   // transposed tiles for the recurrence's output waves and for a backward pass
-    GDN_LDS_BARRIER();
+  // ---- phase 1c: what the recurrence reads, in fragment order: the two K images and (scale q . e^{G})^T ----
+  if (QB_out == nullptr) {
+    // Straight from the rows in LDS into the registers of an A operand (lane <-> token, 4 consecutive channels per
+    // piece, frag_a_split's order): e^{G} serves q and the first K image, nothing is staged and no barrier is needed.
+    // The q tiles are turned by a pass through the matrix core (exact) into (lane <-> channel, registers <-> token).
+    constexpr int KG = AccK<T>::kGroups, GL = KGroup<T>::kLen, NP = sizeof(T) == 2 ? 2 : 1;
+    IdentityFrag<T> id;
+    id.init();
     for (int tt = wave; tt < 2 * (DK / 32); tt += 4) {
-      const int tj = tt & 1, kt2 = tt >> 1;
-      AccB<T> kf;
-      kf.load_cols(Qs + 32 * tj * LDK + 32 * kt2, LDK);
-      kf.store_stream(QBT_out + ((ch * (DK / 32) + kt2) * 2 + tj) * 1024);
+      const int tj = tt & 1, kt2 = tt >> 1, row = 32 * tj + l32;
+      const float nb = -bs[row];
+      AccB<T> f1, f2, fq;
+#pragma unroll
+      for (int kg = 0; kg < KG; ++kg) {
+        float x1[4 * NP], x2[4 * NP], xq[4 * NP];
+#pragma unroll
+        for (int pc = 0; pc < NP; ++pc) {
+          const int c = 32 * kt2 + GL * kg + 4 * half + 8 * pc;
+          float k4[4], q4[4];
+          if constexpr (sizeof(T) == 2) {
+            const u32x2 kw = *reinterpret_cast<const u32x2*>(Ks + row * LDK + c), qw = *reinterpret_cast<const u32x2*>(Qs + row * LDK + c);
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+              k4[2 * e] = __uint_as_float(kw[e] << 16); k4[2 * e + 1] = __uint_as_float(kw[e] & 0xffff0000u);
+              q4[2 * e] = __uint_as_float(qw[e] << 16); q4[2 * e + 1] = __uint_as_float(qw[e] & 0xffff0000u);
+            }
+          } else {
+            const f32x4 kw = *reinterpret_cast<const f32x4*>(Ks + row * LDK + c), qw = *reinterpret_cast<const f32x4*>(Qs + row * LDK + c);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { k4[e] = kw[e]; q4[e] = qw[e]; }
+          }
+          const f32x4 g4 = *reinterpret_cast<const f32x4*>(Gs + row * LDG + c), gl4 = *reinterpret_cast<const f32x4*>(Gs + 63 * LDG + c);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float eg = KdaDecay<T>::exp(g4[e]);
+            x1[4 * pc + e] = k4[e] * (nb * eg);      // the products in the order of the staged path below: same bits
+            x2[4 * pc + e] = k4[e] * KdaDecay<T>::exp(gl4[e] - g4[e]);
+            xq[4 * pc + e] = q4[e] * (scale * eg);
+          }
+        }
+        if constexpr (sizeof(T) == 2) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            f1.f[kg][e] = f32x2_to_bf16x2(x1[2 * e], x1[2 * e + 1]);
+            f2.f[kg][e] = f32x2_to_bf16x2(x2[2 * e], x2[2 * e + 1]);
+            fq.f[kg][e] = f32x2_to_bf16x2(xq[2 * e], xq[2 * e + 1]);
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            f1.f[kg][e] = __float_as_uint(x1[e]); f2.f[kg][e] = __float_as_uint(x2[e]); fq.f[kg][e] = __float_as_uint(xq[e]);
+          }
+        }
+      }
+      const int64_t tile = ((ch * (DK / 32) + kt2) * 2 + tj) * 1024;
+      f1.store_stream(K1_out + tile);
+      f2.store_stream(K2_out + tile);
+      if (QBT_out != nullptr) {
+        AccB<T> qt2;
+        qt2.pack(mfma_transpose<T>(fq, id));
+        qt2.store_stream(QBT_out + tile);
+      }
     }
-  }
-  auto stage_k = [&](bool first) {
+  } else {
+    // with the rows of q also wanted as rows (the stand-alone output kernel): through a row-major staging tile (the q
+    // rows' place): rows of q with scale and decay first (in place), then the two K images
     for (int c = tid; c < 64 * CPR; c += kThreads) {
       const int row = c / CPR, cc = c % CPR;
-      float f[VEC], gi[VEC], gl[VEC];
-      unpack16<T>(ld16(Ks + row * LDK + cc * VEC), f);
+      float f[VEC], gi[VEC];
+      unpack16<T>(ld16(Qs + row * LDK + cc * VEC), f);
       ld_f32<VEC>(Gs + row * LDG + cc * VEC, gi);
-      ld_f32<VEC>(Gs + 63 * LDG + cc * VEC, gl);
-      const float nb = -bs[row];
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) f[e] *= first ? nb * KdaDecay<T>::exp(gi[e]) : KdaDecay<T>::exp(gl[e] - gi[e]);
-      st16(Qs + row * LDK + cc * VEC, pack16<T>(f));
+      for (int e = 0; e < VEC; ++e) f[e] *= scale * KdaDecay<T>::exp(gi[e]);
+      const Vec16<T> x = pack16<T>(f);
+      if (row < nvalid) st16(QB_out + (tok0 + row) * hk + h * DK + cc * VEC, x);   // row-major for the output kernel
+      st16(Qs + row * LDK + cc * VEC, x);
     }
-  };
-  auto store_k = [&](T* out) {
-    for (int tt = wave; tt < 2 * (DK / 32); tt += 4) {
-      const int tj = tt & 1, kt2 = tt >> 1;
-      AccB<T> kf;
-      frags_from_lds<T>(kf, Qs + (32 * tj + (lane & 31)) * LDK + 32 * kt2);
-      kf.store_stream(out + ((ch * (DK / 32) + kt2) * 2 + tj) * 1024);
+    if (QBT_out != nullptr) {   // transposed tiles for a backward pass
+      GDN_LDS_BARRIER();
+      for (int tt = wave; tt < 2 * (DK / 32); tt += 4) {
+        const int tj = tt & 1, kt2 = tt >> 1;
+        AccB<T> kf;
+        kf.load_cols(Qs + 32 * tj * LDK + 32 * kt2, LDK);
+        kf.store_stream(QBT_out + ((ch * (DK / 32) + kt2) * 2 + tj) * 1024);
+      }
     }
-  };
-  GDN_LDS_BARRIER();
-  stage_k(true);
-  GDN_LDS_BARRIER();
-  store_k(K1_out);
-  GDN_LDS_BARRIER();
-  stage_k(false);
-  GDN_LDS_BARRIER();
-  store_k(K2_out);
+    auto stage_k = [&](bool first) {
+      for (int c = tid; c < 64 * CPR; c += kThreads) {
+        const int row = c / CPR, cc = c % CPR;
+        float f[VEC], gi[VEC], gl[VEC];
+        unpack16<T>(ld16(Ks + row * LDK + cc * VEC), f);
+        ld_f32<VEC>(Gs + row * LDG + cc * VEC, gi);
+        ld_f32<VEC>(Gs + 63 * LDG + cc * VEC, gl);
+        const float nb = -bs[row];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) f[e] *= first ? nb * KdaDecay<T>::exp(gi[e]) : KdaDecay<T>::exp(gl[e] - gi[e]);
+        st16(Qs + row * LDK + cc * VEC, pack16<T>(f));
+      }
+    };
+    auto store_k = [&](T* out) {
+      for (int tt = wave; tt < 2 * (DK / 32); tt += 4) {
+        const int tj = tt & 1, kt2 = tt >> 1;
+        AccB<T> kf;
+        frags_from_lds<T>(kf, Qs + (32 * tj + (lane & 31)) * LDK + 32 * kt2);
+        kf.store_stream(out + ((ch * (DK / 32) + kt2) * 2 + tj) * 1024);
+      }
+    };
+    GDN_LDS_BARRIER();
+    stage_k(true);
+    GDN_LDS_BARRIER();
+    store_k(K1_out);
+    GDN_LDS_BARRIER();
+    stage_k(false);
+    GDN_LDS_BARRIER();
+    store_k(K2_out);
+  }
   // the decay of the whole chunk per channel, the cumulative decay itself
   if (tid < DK) dec_out[ch * DK + tid] = KdaDecay<T>::exp(Gs[63 * LDG + tid]);
   if (G_out != nullptr) {
