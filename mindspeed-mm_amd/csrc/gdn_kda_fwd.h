@@ -371,48 +371,70 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
   GDN_LDS_BARRIER();   // k, the staging tile and G are dead
 
   // ---- phase 1d: L and Aq as 64x64 fp32 matrices ----
-  for (int i = tid; i < 64 * kLF; i += kThreads) { As[i] = 0.f; Aqs[i] = 0.f; Ti[i] = 0.f; }
-  GDN_LDS_BARRIER();
-  // each entry is the sum of the two waves that share a tile (one per half of the channels): they add one after the
-  // other.  A wave reads all of its entries, then adds, then writes: entry by entry each read would wait for the write
-  // before it (the compiler must assume that the two matrices overlap).
+  // Zeroed: the place of the inverse, and the tile above the diagonal of both matrices; every other entry is written by
+  // the first of the two waves that share a tile (one per half of the channels), then the second adds its half.  A wave
+  // reads all of its entries, then adds, then writes: entry by entry each read would wait for the write before it (the
+  // compiler must assume that the two matrices overlap).
+  static_assert(kLF % 4 == 0, "rows of the fp32 matrices are whole 16-byte pieces");
+  for (int i = tid; i < 64 * kLF / 4; i += kThreads) reinterpret_cast<f32x4*>(Ti)[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int i = tid; i < 32 * 8; i += kThreads) {
+    const int at = (i >> 3) * kLF + 32 + 4 * (i & 7);
+    *reinterpret_cast<f32x4*>(As + at) = f32x4{0.f, 0.f, 0.f, 0.f};
+    *reinterpret_cast<f32x4*>(Aqs + at) = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  if (kh == 0) {
+    const f32x16 bi = rows_ld(bs, 32 * td);
 #pragma unroll
-  for (int turn = 0; turn < 2; ++turn) {
-    if (kh == turn) {
-      float ca[16], cq[16], bi[16];
+    for (int r = 0; r < 16; ++r) {
+      const int i = 32 * td + acc_row(r), j = 32 * td + l32;
+      As[i * kLF + j] = i > j ? bi[r] * dgk[r] : 0.f;
+      Aqs[i * kLF + j] = i >= j ? scale * dgq[r] : 0.f;
+    }
+    if (wave < 2) {   // the tile below the diagonal
+      const f32x16 bl = rows_ld(bs, 32);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int i = 32 * td + acc_row(r), j = 32 * td + l32;
-        ca[r] = As[i * kLF + j];
-        cq[r] = Aqs[i * kLF + j];
-        bi[r] = bs[i];
+        const int i2 = 32 + acc_row(r);
+        As[i2 * kLF + l32] = bl[r] * lowk[r];
+        Aqs[i2 * kLF + l32] = scale * lowq[r];
+      }
+    }
+  }
+  GDN_LDS_BARRIER();
+  if (kh == 1) {
+    float ca[16], cq[16];
+    const f32x16 bi = rows_ld(bs, 32 * td);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int i = 32 * td + acc_row(r), j = 32 * td + l32;
+      ca[r] = As[i * kLF + j];
+      cq[r] = Aqs[i * kLF + j];
+    }
+    GDN_SCHED_FENCE();
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int i = 32 * td + acc_row(r), j = 32 * td + l32;
+      As[i * kLF + j] = ca[r] + (i > j ? bi[r] * dgk[r] : 0.f);
+      Aqs[i * kLF + j] = cq[r] + (i >= j ? scale * dgq[r] : 0.f);
+    }
+    if (wave < 2) {   // the tile below the diagonal
+      const f32x16 bl = rows_ld(bs, 32);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int i2 = 32 + acc_row(r);
+        ca[r] = As[i2 * kLF + l32];
+        cq[r] = Aqs[i2 * kLF + l32];
       }
       GDN_SCHED_FENCE();
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int i = 32 * td + acc_row(r), j = 32 * td + l32;
-        As[i * kLF + j] = ca[r] + (i > j ? bi[r] * dgk[r] : 0.f);
-        Aqs[i * kLF + j] = cq[r] + (i >= j ? scale * dgq[r] : 0.f);
-      }
-      if (wave < 2) {   // the tile below the diagonal
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int i2 = 32 + acc_row(r);
-          ca[r] = As[i2 * kLF + l32];
-          cq[r] = Aqs[i2 * kLF + l32];
-          bi[r] = bs[i2];
-        }
-        GDN_SCHED_FENCE();
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int i2 = 32 + acc_row(r);
-          As[i2 * kLF + l32] = ca[r] + bi[r] * lowk[r];
-          Aqs[i2 * kLF + l32] = cq[r] + scale * lowq[r];
-        }
+        const int i2 = 32 + acc_row(r);
+        As[i2 * kLF + l32] = ca[r] + bl[r] * lowk[r];
+        Aqs[i2 * kLF + l32] = cq[r] + scale * lowq[r];
       }
     }
-    GDN_LDS_BARRIER();
   }
+  GDN_LDS_BARRIER();
   if (wave != 1) {  // Aq leaves as tiles packed as they sit in an accumulator (lane <-> column j, registers <-> row i);
                     // tile (0,1) is zero, is read by no kernel and is not written
     const int ti = wave >> 1, tj = wave & 1;
