@@ -272,7 +272,8 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
         af.store_stream(Aq_out + (((int64_t)blockIdx.x * Hv + h) * 4 + wave) * 1024);
       }
     }
-    for (int i = tid; i < 64 * kLF; i += kThreads) Ti[i] = 0.f;
+    static_assert(kLF % 4 == 0, "rows of the fp32 matrices are whole 16-byte pieces");
+    for (int i = tid; i < 64 * kLF / 4; i += kThreads) reinterpret_cast<f32x4*>(Ti)[i] = f32x4{0.f, 0.f, 0.f, 0.f};
     GDN_LDS_BARRIER();
 
     tril_inverse_64(As, Ti, wave, lane);
