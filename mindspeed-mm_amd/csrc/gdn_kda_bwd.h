@@ -303,6 +303,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
   //      in the wave's 32-token block ----
   const int d = 32 * cj + l32;
   float Gi[16], U[16], Uq[16], W[16];
+  AccB<T> lqf, lkf;   // the sums over V of this lane's rows (dQb, dK2) for phase B3
   if (has_k) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -431,6 +432,9 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
 #pragma unroll 1
         for (int lg = 3; lg <= 5; ++lg) level(lg, IntConst<1>());
       }
+      // (the registers of the levels are free again: phase B3's tiles are requested here, a level ahead of their use)
+      lqf.load(dQb + (ri * NKT + cj) * 1024);
+      lkf.load(dK2 + (ri * NKT + cj) * 1024);
       {   // the level of the whole chunk: tokens 32..63 against tokens 0..31, m = 32, every pair kept.  The wave of the
           // later tokens takes the sums over j (U, Uq), the wave of the earlier ones the sum over i (W)
         const float g32v = Gs[32 * LDG + d];
@@ -521,10 +525,10 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     float gl_sum = 0.f, blk = 0.f;
     // the sums over V of this lane's rows: all requested before the first is used, and used in two passes so that few
     // intermediate rows are alive at a time (a schedule that runs out of registers waits after every load)
-    // (tiles in fragment order: token block ri, channel block cj)
-    AccB<T> lqf, lkf;
-    lqf.load(dQb + (ri * NKT + cj) * 1024);
-    lkf.load(dK2 + (ri * NKT + cj) * 1024);
+    if constexpr (FULL) {   // (tiles in fragment order: token block ri, channel block cj)
+      lqf.load(dQb + (ri * NKT + cj) * 1024);
+      lkf.load(dK2 + (ri * NKT + cj) * 1024);
+    }
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (!FULL) mma32<T, 64, false, false>(dK1, TmT + 32 * ri, L64, Pt + 32 * cj, LDK);
     if constexpr (FULL) {
