@@ -429,12 +429,12 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
             }
           }
         };
+        // (phase B3's tiles are requested here, four levels ahead of their use: 16 registers)
+        lqf.load(dQb + (ri * NKT + cj) * 1024);
+        lkf.load(dK2 + (ri * NKT + cj) * 1024);
 #pragma unroll 1
         for (int lg = 3; lg <= 5; ++lg) level(lg, IntConst<1>());
       }
-      // (the registers of the levels are free again: phase B3's tiles are requested here, a level ahead of their use)
-      lqf.load(dQb + (ri * NKT + cj) * 1024);
-      lkf.load(dK2 + (ri * NKT + cj) * 1024);
       {   // the level of the whole chunk: tokens 32..63 against tokens 0..31, m = 32, every pair kept.  The wave of the
           // later tokens takes the sums over j (U, Uq), the wave of the earlier ones the sum over i (W)
         const float g32v = Gs[32 * LDG + d];
