@@ -22,10 +22,14 @@
 //   dg_t = sum_{i>=t} dG_i + dG_last, then back through the gate, the l2 norm and the sigmoid of beta.
 // The decay-weighted sums over a chunk use the recursive halving of the forward pass: a pair i > j belongs to one block
 // of one level (64, 32, ..., 2 tokens), in which i lies in the second half and j in the first, and there
-// e^{G_i-G_j} = e^{G_i-G_m} e^{G_m-G_j} with m the middle of the block, both factors at most 1.  Per level the
-// coefficients outside that level's pairs are masked away, the partner rows are rescaled in registers straight into
-// the B-operand layout, the products run on the matrix cores and the rows of the result are scaled by their own
-// factor.  (For fp32 operands every pair is summed term by term in fp32 instead.)
+// e^{G_i-G_j} = e^{G_i-G_m} e^{G_m-G_j} with m the middle of the block, both factors at most 1.  For the levels of 8
+// to 64 tokens the coefficients outside that level's pairs are masked away, the partner rows are rescaled in
+// registers straight into the B-operand layout, the products run on the matrix cores and the rows of the result are
+// scaled by their own factor.  The levels of 2 and 4 tokens stay inside a lane: a lane has one key channel and, per
+// accumulator group, four consecutive tokens, which are one block of 4.  (For fp32 operands every pair is summed term
+// by term in fp32 instead.)
+// What the chunk-local kernel leaves (the workspace's DUMP): P as rows, dQb, dK2, dAq and a2 as 32x32 tiles in
+// fragment order, which is how both kernels hold them in registers.
 #pragma once
 #include "gdn_kda_common.h"
 
@@ -47,7 +51,8 @@ template <typename T, int DK> struct KdaBwdSmem {
   static constexpr int off_q2 = off_m2t + (FULL ? 0 : mat);
   static constexpr int off_m1t = off_q2 + (FULL ? 0 : tile);
   // not FULL: which entries of a coefficient fragment belong to a level's pairs: [5 levels][2 halves of the 32 columns]
-  // [row = earlier | later token][64 lanes] masks of 16 bytes.  They depend on nothing but the lane.
+  // [row = earlier | later token][64 lanes] masks of 16 bytes (only the levels of 8, 16 and 32 tokens are filled and
+  // used).  They depend on nothing but the lane.
   static constexpr int off_keep = off_m1t + (FULL ? 0 : mat);
   static constexpr int off_row = off_keep + (FULL ? 0 : 5 * 2 * 2 * 64 * 16);
   // beta, 1/|q|, 1/|k| [64 each]; row sums <q^,dq^>, <k^,dk^>, db, <R,v> [256 each]; per-wave scalars [8]; what the
@@ -315,9 +320,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     if (has_k) {
       const int half = lane >> 5;
       {
-        // The partner rows this lane supplies as B operand, channel d, are tokens 32 ri + 16 kg + 8 half + e.  They
-        // are read again at every level: held in registers through the levels they would push other values out to
-        // scratch memory, which costs more than the reads.
+        // The partner rows this lane supplies as B operand, channel d, are tokens 32 ri + 16 kg + 8 half + e.
         {   // the pair i = j: no decay (dL has no diagonal).  This lane's rows of k^ and q^, channel d: four transposing
             // reads per tile instead of a two-byte read per row
           AccB<T> t;
