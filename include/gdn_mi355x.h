@@ -94,7 +94,9 @@ int gdn_chunk_bwd_strided(const void* q, const void* k, const void* v, int64_t q
  *   1  refill the state part (forward recurrence without output; chunk_prep_kernel first unless prep_valid != 0,
  *      i.e. unless workspace_prep still holds what a forward call on the same inputs left there)
  *   2  the reverse recurrence
- *   4  the chunk-local kernels (dq, dk, dv, dg, dbeta); needs phases 1 and 2 of the same inputs done
+ *   4  the chunk-local kernels (dq, dk, dv, dg, dbeta); needs phases 1 and 2 of the same inputs done, and uses up what
+ *      phase 2 left: with several value heads per q/k head it reuses the place of the state gradients it has read, so a
+ *      second run of phase 4 needs phase 2 again
  * Phases 1 and 2 do not depend on each other: a caller may launch them on two streams and join both before phase 4.
  * Each of them is a latency-bound kernel with one workgroup per compute unit at most; for shapes whose slabs would fill
  * more than half of the device they are launched with two slabs per workgroup here, so that the two fit side by side

@@ -44,7 +44,8 @@ struct ChunkWorkspace {
   int64_t HF;             // T [chunks,Hv,V/32,K/32] state BEFORE each chunk, tile = (32 rows of K) x (32 columns of V)
   int64_t fwd_bytes;
   int64_t DVF;            // T [chunks,Hv,V/32,2]    d(v_new)
-  int64_t DHF;            // T [chunks,Hv,V/32,K/32] gradient of the state AFTER each chunk
+  int64_t DHF;            // T [chunks,Hv,V/32,K/32] gradient of the state AFTER each chunk; once the chunk-local kernel of a
+                          //   head has read its part it may leave the group's dq, dk sums there for the next head's launch
   int64_t total_bytes;
 };
 

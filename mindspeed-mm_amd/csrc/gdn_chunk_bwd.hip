@@ -395,7 +395,7 @@ template <typename T, int DK, bool KDA = false>
 __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_local_kernel(
     const T* __restrict__ qtf, const T* __restrict__ kaf, const T* __restrict__ v, const void* __restrict__ beta, int beta_same,
     const float* __restrict__ G, const T* __restrict__ Ai, const T* __restrict__ vf, const T* __restrict__ dvf,
-    const T* __restrict__ dO, const T* __restrict__ hf, const T* __restrict__ dhf, const float* __restrict__ rstd_q,
+    const T* __restrict__ dO, const T* __restrict__ hf, const T* dhf_in, const float* __restrict__ rstd_q,
     const float* __restrict__ rstd_k, T* dq, T* dk, T* __restrict__ dv_out, void* __restrict__ dbeta,
     float* __restrict__ dg, const int64_t* __restrict__ cu, const int* __restrict__ chunk_offsets, int T_len, int N,
     int Hqk, int Hv, int V, float scale, int hh, TokenStrides ts, T* __restrict__ kda_dump, float* __restrict__ kda_dd,
@@ -458,7 +458,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
 #pragma unroll
       for (int g = 0; g < KG; ++g) {
         load16_to_lds(hf + tile + (g * 64 + lane) * VEC, pv + g * 64 * VEC);
-        load16_to_lds(dhf + tile + (g * 64 + lane) * VEC, pv + 1024 + g * 64 * VEC);
+        load16_to_lds(dhf_in + tile + (g * 64 + lane) * VEC, pv + 1024 + g * 64 * VEC);
       }
     }
   };
@@ -759,11 +759,24 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   GDN_LDS_BARRIER();   // the ds tiles are consumed
   // later value heads of a group add to the dq, dk rows the earlier ones wrote: what memory holds is requested well
   // ahead, dq here (no store is in flight), dk two phases before it is needed
+  // Where the state gradient of a (chunk, head) has room for them (V >= 128: V K elements against 2 x 64 K), the sums
+  // travel from one head's launch to the next as fragment-order tiles in that place, which this launch has finished
+  // reading (the reverse recurrence rewrites it in every backward pass): no pass through rows, and only the group's
+  // last head writes dq and dk.  Tiles: dq (token block, channel block), then dk likewise.
+  const bool frag_sums = V >= 128 && grp > 1, last_head = hh == grp - 1;
+  T* sums_out = const_cast<T*>(dhf_in) + ch * (int64_t)(V / 32) * NKT * 1024;
+  const T* sums_in = sums_out - (int64_t)(V / 32) * NKT * 1024;   // the head before this one
   RowPieces<T> held[2];
+  AccB<T> heldf[2];
   if (has_k && hh != 0) {
+    if (frag_sums) {
 #pragma unroll
-    for (int ri = 0; ri < 2; ++ri)
-      rows_request<T>(held[ri], dq + (tok0 + 32 * ri) * ts.dq + hq * DK + 32 * cj, ts.dq, nvalid - 32 * ri);
+      for (int ri = 0; ri < 2; ++ri) heldf[ri].load(sums_in + (ri * NKT + cj) * 1024);
+    } else {
+#pragma unroll
+      for (int ri = 0; ri < 2; ++ri)
+        rows_request<T>(held[ri], dq + (tok0 + 32 * ri) * ts.dq + hq * DK + 32 * cj, ts.dq, nvalid - 32 * ri);
+    }
   }
   if (lower) {  // <R_t, v_t> = sum_i Tm[i][t] (dV' V^T)[i][t]: column sums of Tm . a2, no second pass over V needed
     const f32x16 tmv = tm_t(tj, ti).unpack();   // Tm tile (ti, tj) with lane <-> column, registers <-> row
@@ -808,8 +821,24 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
         for (int r = 0; r < 16; ++r) dQi[ri][r] = (dQi[ri][r] - dot[r] * qq[r]) * rs[r];
       }
       T* dst = dq + (tok0 + 32 * ri) * ts.dq + hq * DK + 32 * cj;
-      if (hh == 0) acc_store_rows<T, false>(dQi[ri], id, patch, dst, ts.dq, nvalid - 32 * ri);
-      else acc_store_rows<T, true>(dQi[ri], id, patch, dst, ts.dq, nvalid - 32 * ri, held[ri]);
+      if (frag_sums) {
+        if (hh != 0) {
+          const f32x16 prev = heldf[ri].unpack();
+#pragma unroll
+          for (int r = 0; r < 16; ++r) dQi[ri][r] += prev[r];
+        }
+        if (last_head) {
+          acc_store_rows<T, false>(dQi[ri], id, patch, dst, ts.dq, nvalid - 32 * ri);
+        } else {
+          AccB<T> f;
+          f.pack(dQi[ri]);
+          f.store_stream(sums_out + (ri * NKT + cj) * 1024);
+        }
+      } else if (hh == 0) {
+        acc_store_rows<T, false>(dQi[ri], id, patch, dst, ts.dq, nvalid - 32 * ri);
+      } else {
+        acc_store_rows<T, true>(dQi[ri], id, patch, dst, ts.dq, nvalid - 32 * ri, held[ri]);
+      }
     }
   }
   {  // X = dTm Tm^T, handed on in D form
@@ -850,10 +879,15 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
     d.store(dMD + wave * 1024);
   }
   GDN_LDS_BARRIER();
-  if (has_k && hh != 0) {   // the dk rows the earlier heads wrote, two phases before they are added to
+  if (has_k && hh != 0) {   // the dk sums of the earlier heads, two phases before they are added to
+    if (frag_sums) {
 #pragma unroll
-    for (int ri = 0; ri < 2; ++ri)
-      rows_request<T>(held[ri], dk + (tok0 + 32 * ri) * ts.dk + hq * DK + 32 * cj, ts.dk, nvalid - 32 * ri);
+      for (int ri = 0; ri < 2; ++ri) heldf[ri].load(sums_in + ((2 + ri) * NKT + cj) * 1024);
+    } else {
+#pragma unroll
+      for (int ri = 0; ri < 2; ++ri)
+        rows_request<T>(held[ri], dk + (tok0 + 32 * ri) * ts.dk + hq * DK + 32 * cj, ts.dk, nvalid - 32 * ri);
+    }
   }
   if (has_k) {       // E = dM K, F = dM^T (beta K): dK += beta E + F; <E,k> and <F,k> complete the row sums
 #pragma unroll
@@ -892,8 +926,24 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
         for (int r = 0; r < 16; ++r) dKi[ri][r] = (dKi[ri][r] - dot[r] * kk[r]) * rs[r];
       }
       T* dst = dk + (tok0 + 32 * ri) * ts.dk + hq * DK + 32 * cj;
-      if (hh == 0) acc_store_rows<T, false>(dKi[ri], id, patch, dst, ts.dk, nvalid - 32 * ri);
-      else acc_store_rows<T, true>(dKi[ri], id, patch, dst, ts.dk, nvalid - 32 * ri, held[ri]);
+      if (frag_sums) {
+        if (hh != 0) {
+          const f32x16 prev = heldf[ri].unpack();
+#pragma unroll
+          for (int r = 0; r < 16; ++r) dKi[ri][r] += prev[r];
+        }
+        if (last_head) {
+          acc_store_rows<T, false>(dKi[ri], id, patch, dst, ts.dk, nvalid - 32 * ri);
+        } else {
+          AccB<T> f;
+          f.pack(dKi[ri]);
+          f.store_stream(sums_out + ((2 + ri) * NKT + cj) * 1024);
+        }
+      } else if (hh == 0) {
+        acc_store_rows<T, false>(dKi[ri], id, patch, dst, ts.dk, nvalid - 32 * ri);
+      } else {
+        acc_store_rows<T, true>(dKi[ri], id, patch, dst, ts.dk, nvalid - 32 * ri, held[ri]);
+      }
     }
   }
   if (wave == 0) {   // d(cumulative G) -> d(g): suffix sum inside the chunk
