@@ -46,6 +46,15 @@ _custom_fwd = functools.partial(torch.amp.custom_fwd, device_type="cuda")
 _custom_bwd = functools.partial(torch.amp.custom_bwd, device_type="cuda")
 
 
+def _out_grad(grad, like):
+    """The gradient of the main output, for autograd functions that ask for undefined gradients to stay None (the final
+    state is rarely used: its zero gradient is then neither filled nor read): zeros only when the output itself went
+    unused while the final state was used.  `like` = (shape, dtype, device) of that output."""
+    if grad is not None:
+        return grad.contiguous()
+    return torch.zeros(like[0], dtype=like[1], device=like[2])
+
+
 def _beta_arg(beta, act_dtype):
     """beta as handed to the kernels: in place when it has the 16-bit dtype of q, k, v (the layer's beta = b.sigmoid()
     is bf16, modeling_qwen3_5.py:833), else as float32.  Returns (tensor, dtype code)."""
@@ -612,12 +621,15 @@ class _ChunkGatedDeltaRule(torch.autograd.Function):
             ctx.save_for_backward(*saved)
             ctx.meta = meta
             ctx.ops = ops
+            ctx.set_materialize_grads(False)
+            ctx.o_like = (o.shape, o.dtype, o.device)
         return o, ht
 
     @staticmethod
     @_input_guard
     @_custom_bwd
     def backward(ctx, do, dht):
+        do = _out_grad(do, ctx.o_like)
         dq, dk, dv, dg, db, dh0 = _chunk_backward_call(ctx.ops, ctx.saved_tensors, ctx.meta, do, dht)
         return dq, dk, dv, dg, db, None, dh0, None, None, None, None, None
 
@@ -662,6 +674,8 @@ class _ChunkGatedDeltaRuleNorm(torch.autograd.Function):
                         beta.dtype, None if initial_state is None else initial_state.dtype, sq, sk, sv, w_dt,
                         norm_weight.dtype, gate.dtype, gate.shape, rule_grad, bcode)
             ctx.ops = ops
+            ctx.set_materialize_grads(False)
+            ctx.o_like = (y.shape, y.dtype, y.device)
         return y, ht
 
     @staticmethod
@@ -674,7 +688,7 @@ class _ChunkGatedDeltaRuleNorm(torch.autograd.Function):
         lib = ctx.ops.lib
         dev, dt = qc.device, qc.dtype
         rows = B * T * Hv
-        dyc = dy.to(dt).contiguous()
+        dyc = _out_grad(dy, ctx.o_like).to(dt).contiguous()
         do = torch.empty_like(o)
         dgate = torch.empty_like(o)
         dw = torch.empty(V, dtype=torch.float32, device=dev)
@@ -738,6 +752,8 @@ class _ChunkGatedDeltaRuleQKV(torch.autograd.Function):
             ctx.meta = (B, T, D, N, Hqk, Hv, K, V, scale, int(use_qk_l2norm_in_kernel), code, nbytes,
                         g.dtype, beta.dtype, None if initial_state is None else initial_state.dtype, bcode)
             ctx.ops = ops
+            ctx.set_materialize_grads(False)
+            ctx.o_like = (o.shape, o.dtype, o.device)
         return o, ht
 
     @staticmethod
@@ -748,7 +764,7 @@ class _ChunkGatedDeltaRuleQKV(torch.autograd.Function):
         B, T, D, N, Hqk, Hv, K, V, scale, l2, code, nbytes, g_dt, b_dt, h_dt, bcode = ctx.meta
         lib = ctx.ops.lib
         nq, nv, es, dev = Hqk * K, Hv * V, x.element_size(), x.device
-        do = do.contiguous()
+        do = _out_grad(do, ctx.o_like)
         dht = ctx.ops._f32(dht)
         # columns past q, k, v (none in the layer) receive no gradient
         dx = torch.empty_like(x) if D == 2 * nq + nv else torch.zeros_like(x)
@@ -818,6 +834,8 @@ class _ChunkKda(torch.autograd.Function):
                         None if A_log is None else A_log.dtype, None if dt_bias is None else (dt_bias.dtype, dt_bias.shape),
                         None if initial_state is None else initial_state.dtype)
             ctx.ops = ops
+            ctx.set_materialize_grads(False)
+            ctx.o_like = (o.shape, o.dtype, o.device)
         return o, ht, hs
 
     @staticmethod
@@ -828,7 +846,7 @@ class _ChunkKda(torch.autograd.Function):
         B, T, N, H, K, V, scale, opts, nbytes, g_dt, b_dt, bc_dt, a_dt, d_dt, h_dt = ctx.meta
         lib = ctx.ops.lib
         dev = qc.device
-        do = do.contiguous()
+        do = _out_grad(do, ctx.o_like)
         dht = ctx.ops._f32(dht)
         dq, dk, dv, dg = torch.empty_like(qc), torch.empty_like(kc), torch.empty_like(vc), torch.empty_like(gc)
         db = torch.empty(B, T, H, dtype=bc_dt, device=dev)

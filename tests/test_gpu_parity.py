@@ -209,6 +209,52 @@ def test_chunk_backward_in_phases_through_the_c_abi(ops, dtype, B, T, Hqk, Hv, K
     assert parts(grads(), prep, nprep, state, nstate - 256, 7, 1) == -5
 
 
+def _one_output_gradients(ops, device, kda):
+    """A loss that uses only one of the two outputs reaches the backward pass with the other gradient undefined (the
+    functions ask autograd not to fill it with zeros): the gradients from o alone and from the final state alone add up
+    to those of the loss over both (linearity), in fp32."""
+    import tests.parity as P
+    B, T, H, K, V = 1, 130, 2, 64, 128
+    if kda:
+        x = P.kda_inputs(B, T, H, K, V, torch.float32, seed=7)
+        names = ("q", "k", "v", "g", "beta", "h0", "A_log", "dt_bias")
+    else:
+        x = P.gdn_inputs(B, T, H, 2 * H, K, V, torch.float32, seed=7)
+        names = ("q", "k", "v", "g", "beta", "h0")
+    d = {n: t.to(device) for n, t in x.items()}
+
+    def grads(use_o, use_ht):
+        leaves = {n: d[n].clone().requires_grad_(True) for n in names}
+        if kda:
+            o, ht = ops.chunk_kda(leaves["q"], leaves["k"], leaves["v"], leaves["g"], leaves["beta"],
+                                  initial_state=leaves["h0"], output_final_state=True, use_qk_l2norm_in_kernel=True,
+                                  use_gate_in_kernel=True, use_beta_sigmoid_in_kernel=True, A_log=leaves["A_log"],
+                                  dt_bias=leaves["dt_bias"])
+        else:
+            o, ht = ops.chunk_gated_delta_rule(leaves["q"], leaves["k"], leaves["v"], leaves["g"], leaves["beta"],
+                                               initial_state=leaves["h0"], output_final_state=True,
+                                               use_qk_l2norm_in_kernel=True)
+        loss = 0
+        if use_o:
+            loss = loss + (o * d["do"]).sum()
+        if use_ht:
+            loss = loss + (ht * d["dht"]).sum()
+        return torch.autograd.grad(loss, list(leaves.values()))
+    both, only_o, only_ht = grads(True, True), grads(True, False), grads(False, True)
+    for n, a, b, c in zip(names, both, only_o, only_ht):
+        scale = max(a.abs().max().item(), 1e-6)
+        assert ((b + c) - a).abs().max().item() <= 2e-5 * scale + 1e-6, n
+        if n in ("k", "v", "h0"):   # the final state does not depend on q
+            assert c.abs().max().item() > 0, n
+        if n == "q":
+            assert c.abs().max().item() == 0
+
+
+@pytest.mark.parametrize("kda", [False, True])
+def test_gradient_from_one_output_only(ops, kda):
+    _one_output_gradients(ops, "cuda", kda)
+
+
 def test_chunk_default_mode_on_one_stream_equals_two_streams(ops):
     """The default mode's backward pass rebuilds states and corrected values on a second stream beside the reverse
     recurrence; with that switched off (everything on the caller's stream) the gradients are the same bits."""
