@@ -613,8 +613,16 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       const float bj = bs[32 * rj + l32];
 #pragma unroll
       for (int r = 0; r < 16; ++r) Rt[r] *= bj;
-      if (32 * rj + l32 < nvalid)
-        acc_to_lds_t<T>(Rt, dv_out + (tok0 + 32 * rj + l32) * ts.dv + h * V + 32 * vblk, 0, 0, 0);
+      // (rows past the end repeat the last valid one: the half-waves trade pieces, so every lane takes part)
+      T* dvrow = dv_out + (tok0 + imin(32 * rj + l32, nvalid - 1)) * ts.dv + h * V + 32 * vblk;
+      if constexpr (sizeof(T) == 2) {
+        if (32 * rj < nvalid) {   // wave-uniform
+          const bool live = 32 * rj + l32 < nvalid;
+          acc_store_t_rows16<T>(Rt, dvrow, live);
+        }
+      } else {
+        if (32 * rj + l32 < nvalid) acc_to_lds_t<T>(Rt, dvrow, 0, 0, 0);
+      }
     }
   }
   if constexpr (KDA) {

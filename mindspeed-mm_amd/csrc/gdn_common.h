@@ -623,6 +623,29 @@ template <typename T> __device__ __forceinline__ void acc_to_lds_t(const f32x16&
     }
   }
 }
+// accumulator tile -> global memory, transposed, for 16-bit types: `row` is this lane's own row of the destination
+// (column acc_col() of the tile) at the tile's first column.  acc_to_lds_t with ld = 0 writes it in 8-byte pieces: the
+// lower half-wave has columns 8g..8g+3 of a row, the upper one 8g+4..8g+7.  Here the half-waves trade pieces first
+// (v_permlane32_swap: the upper half of the first register with the lower half of the second), so that the lower one
+// holds columns 16p..16p+7 and the upper one 16p+8..16p+15: two 16-byte stores per lane instead of four of 8 bytes.
+// Every lane of the wave must call it (the trade); `live` says whether this lane's row exists.
+template <typename T> __device__ __forceinline__ void acc_store_t_rows16(const f32x16& acc, T* row, bool live) {
+  static_assert(sizeof(T) == 2, "16-bit types");
+  const int half = (threadIdx.x & 63) >> 5;
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    u32x4 w;
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const uint32_t x = f32x2_to_bf16x2(acc[8 * p + 2 * e], acc[8 * p + 2 * e + 1]);          // group 2p
+      const uint32_t y = f32x2_to_bf16x2(acc[8 * p + 4 + 2 * e], acc[8 * p + 4 + 2 * e + 1]);  // group 2p + 1
+      const auto r = __builtin_amdgcn_permlane32_swap(x, y, false, false);
+      w[e] = r[0];
+      w[2 + e] = r[1];
+    }
+    if (live) *reinterpret_cast<u32x4*>(row + 16 * p + 8 * half) = w;   // every lane trades, lanes of rows past the end do not store
+  }
+}
 // accumulator tile -> LDS, row-major, by way of the matrix core: the tile is rounded to T, transposed (exact) and
 // then written like a transposed tile, four contiguous elements per lane and store instead of one.
 template <typename T>

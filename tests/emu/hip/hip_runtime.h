@@ -278,6 +278,17 @@ static emu::GdimProxy gridDim;
 // direct global -> LDS load: lane l's `size` bytes land at dst + l*size (done at once: the emulator has no asynchrony)
 #define __builtin_amdgcn_global_load_lds(src, dst, size, off, aux) \
   memcpy((unsigned char*)(uintptr_t)(dst) + (off) + emu::lane() * (size), (const void*)(uintptr_t)(src), (size))
+// v_permlane32_swap: the upper 32 lanes of the first operand trade places with the lower 32 lanes of the second;
+// returns (new first, new second)
+struct emu_u32x2 { unsigned v[2]; unsigned operator[](int i) const { return v[i]; } };
+inline emu_u32x2 __builtin_amdgcn_permlane32_swap(unsigned a, unsigned b, bool, bool) {
+  const int l = emu::lane();
+  const unsigned a_other = emu::shfl(a, l ^ 32), b_other = emu::shfl(b, l ^ 32);
+  emu_u32x2 r;
+  r.v[0] = l < 32 ? a : b_other;   // first: lower half keeps its own, upper half receives the second's lower half
+  r.v[1] = l < 32 ? a_other : b;   // second: lower half receives the first's upper half, upper half keeps its own
+  return r;
+}
 template <class T> inline T __shfl(T v, int src, int = 64) { return emu::shfl(v, src); }
 template <class T> inline T __shfl_xor(T v, int m, int = 64) { return emu::shfl(v, emu::lane() ^ m); }
 template <class T> inline T __shfl_up(T v, unsigned d, int = 64) {
