@@ -544,7 +544,7 @@ def main():
         def kda_prefill():
             with torch.no_grad():
                 ops.chunk_kda(kl["q"], kl["k"], kl["v"], kl["g"], kl["beta"], **kda_kw)
-        kms, kpf = wall_ms(kda_step, 10, 3), wall_ms(kda_prefill, 10, 3)
+        kms, kpf = wall_ms(kda_step, 30, 5), wall_ms(kda_prefill, 30, 5)
         torch.cuda.synchronize()
         lib.gdn_profile_enable(1)
         for _ in range(5):

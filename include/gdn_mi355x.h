@@ -219,8 +219,9 @@ int gdn_gate_bwd_noalloc(const void* a, const void* b, const void* A_log, const 
  * use_gate: g is the raw gate input and the log decay is -e^{A_log} softplus(g + dt_bias), or, with has_lower_bound,
  * lower_bound * sigmoid(e^{A_log} (g + dt_bias)); otherwise g is the log decay itself (<= 0).
  * beta_sigmoid: beta <- sigmoid(beta), times 2 with allow_neg_eigval.  K in {64, 128}, V a multiple of 64.
- * A workspace of gdn_kda_workspace_bytes(..., with_backward = 1, ...) bytes also keeps the chunk-local cumulative
- * decay and 1/|q|, 1/|k|.  Returns 0, or -1 null argument, -2 shape, -3 unsupported K / V, -4 dtype, -5 workspace,
+ * A workspace of gdn_kda_workspace_bytes(..., with_backward = 1, ...) bytes also keeps Tm as rows, 1/|q|, 1/|k| and
+ * the places of the backward pass's intermediates (the cumulative decay is not kept: gdn_kda_bwd rebuilds it from g,
+ * A_log and dt_bias).  Returns 0, or -1 null argument, -2 shape, -3 unsupported K / V, -4 dtype, -5 workspace,
  * -6 alignment. */
 int64_t gdn_kda_workspace_bytes(int B, int T, int N, int H, int K, int V, int with_backward, int dtype);
 

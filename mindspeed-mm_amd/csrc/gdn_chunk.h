@@ -92,7 +92,6 @@ struct KdaWorkspace {
   int64_t HF;             // T [chunks,H,V/32,K/32] state before each chunk
   int64_t fwd_bytes;
   // kept for a backward pass
-  int64_t GC;             // f32 [chunks,H,64,K]    chunk-local cumulative log decay (16-bit kernels: times log2 e, see KdaDecay)
   int64_t TMR;            // T [chunks,H,64,64]     Tm row-major, as rounded for the tiles
   int64_t DVF;            // T [chunks,H,V/32,2]    d(v_new)
   int64_t DHF;            // T [chunks,H,V/32,K/32] gradient of the state AFTER each chunk
@@ -122,7 +121,6 @@ inline KdaWorkspace kda_workspace_layout(const ChunkDims& d, int elem_bytes) {
   w.VF = take(nc * 64 * H * d.V * elem_bytes);
   w.HF = take(nc * H * d.V * d.K * elem_bytes);
   w.fwd_bytes = off;
-  w.GC = take(nc * 64 * H * d.K * 4);
   w.TMR = take(nc * H * 64 * 64 * elem_bytes);
   w.DVF = take(nc * 64 * H * d.V * elem_bytes);
   w.DHF = take(nc * H * d.V * d.K * elem_bytes);

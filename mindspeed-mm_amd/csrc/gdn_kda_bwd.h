@@ -80,7 +80,7 @@ __device__ __forceinline__ void rows_add_at(const f32x16& x, float* rowacc, int 
 template <typename T, int DK>
 __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const void* __restrict__ g, const float* __restrict__ A_log,
-    const float* __restrict__ dt_bias, const float* __restrict__ bhat, const float* __restrict__ GC,
+    const float* __restrict__ dt_bias, const float* __restrict__ bhat,
     const T* __restrict__ TMR, const T* __restrict__ dumps, const float* __restrict__ dd, const int64_t* __restrict__ cu,
     const int* __restrict__ chunk_offsets, T* __restrict__ dq, T* __restrict__ dk, void* __restrict__ dg,
     void* __restrict__ dbeta, float* __restrict__ part, int T_len, int N, int H, float scale, KdaFlags fl) {
@@ -125,9 +125,48 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
   const T* dQb = dump, *dK2 = dump + 64 * DK, *Pm = dump + 2 * 64 * DK;
   const T* dAq = dump + 3 * 64 * DK, *a2m = dAq + 64 * 64;
   const float* dD = dd + ch * DK;
-  const float* Gc = GC + ch * 64 * DK;
 
-  // ---- phase A0: k^ rows; P and Tm as operands; beta.  The tile waves request their tiles of a2 and dAq now ----
+  // ---- phase A0: G from the gate input; k^ rows; P and Tm as operands; beta.  The tile waves request their tiles of
+  //      a2 and dAq now ----
+  // This thread's pieces of the 64 x DK operands: VEC consecutive channels of a row each.  The gate input goes first
+  // (loads arrive in the order of their requests): the cumulative decay is rebuilt from it, with the forward pass's own
+  // operations, while the other operands are on their way.  (As bits, one branch around the whole round of requests.)
+  constexpr int NIT = 64 * CPR / kFinThreads, C64 = 64 / VEC, NTM = 64 * C64 / kFinThreads;
+  static_assert(64 * CPR % kFinThreads == 0 && 64 * C64 % kFinThreads == 0 && VEC % 4 == 0, "whole rounds of 16-byte pieces");
+  static_assert(kFinThreads % CPR == 0, "a thread's pieces share their channels");
+  const bool g32 = sizeof(T) == 4 || fl.g_f32;
+  u32x4 gw[NIT][VEC / 4];
+  f32x4 bv[VEC / 4];
+  if (g32) {
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int c = tid + it * kFinThreads, row = imin(c / CPR, nvalid - 1);
+#pragma unroll
+      for (int e = 0; e < VEC / 4; ++e)
+        gw[it][e] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint32_t*>(g) + (tok0 + row) * hk + h * DK +
+                                                    (c % CPR) * VEC + 4 * e);
+    }
+  } else {
+    if constexpr (sizeof(T) == 2) {   // VEC = 8 two-byte values: one 16-byte piece
+#pragma unroll
+      for (int it = 0; it < NIT; ++it) {
+        const int c = tid + it * kFinThreads, row = imin(c / CPR, nvalid - 1);
+        gw[it][0] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(g) + (tok0 + row) * hk + h * DK +
+                                                    (c % CPR) * VEC);
+      }
+    }
+  }
+  {
+    // without a branch around the request (the compiler would wait for it at the join): with no bias the pieces come
+    // from a place that is always there and are dropped
+    const bool has_bias = fl.use_gate && dt_bias != nullptr;
+    const float* bp = (has_bias ? dt_bias + h * DK : dD) + (tid % CPR) * VEC;
+#pragma unroll
+    for (int e = 0; e < VEC / 4; ++e) {
+      const f32x4 x = *reinterpret_cast<const f32x4*>(bp + 4 * e);
+      bv[e] = has_bias ? x : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+  }
   TileQK<T, DK, kFinThreads> kt;   // moved by every thread
   TileQK<T, DK> qt;                // moved by kThreads threads, see below
   tile_qk_request<T, DK>(kt, k + tok0 * hk + h * DK, hk, nvalid, tid);
@@ -156,25 +195,51 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
       keepT[idx] = w;
     }
   }
-  // this thread's pieces of P and G (VEC consecutive channels of a row each), all requested before the first wait
-  constexpr int NIT = 64 * CPR / kFinThreads, C64 = 64 / VEC, NTM = 64 * C64 / kFinThreads;
-  static_assert(64 * CPR % kFinThreads == 0 && 64 * C64 % kFinThreads == 0 && VEC % 4 == 0, "whole rounds of 16-byte pieces");
+  // this thread's pieces of P and Tm, all requested before the first wait
   f32x4 gk[NIT][VEC / 4];
   Vec16<T> pf[NIT], tmv[NTM];
 #pragma unroll
   for (int it = 0; it < NIT; ++it) {
-    const int c = tid + it * kFinThreads, at = (c / CPR) * DK + (c % CPR) * VEC;
-    pf[it] = ld16(Pm + at);
-#pragma unroll
-    for (int e = 0; e < VEC / 4; ++e) gk[it][e] = *reinterpret_cast<const f32x4*>(Gc + at + 4 * e);
+    const int c = tid + it * kFinThreads;
+    pf[it] = ld16(Pm + (c / CPR) * DK + (c % CPR) * VEC);
   }
 #pragma unroll
   for (int it = 0; it < NTM; ++it) {
     const int c = tid + it * kFinThreads;
     tmv[it] = ld16(TMR + ch * 4096 + (c / C64) * 64 + (c % C64) * VEC);
   }
+  // G: the gate's log decay of every token and channel (0 on the rows past the end) into the place Kp will take,
+  // summed down the tokens there, and back into this thread's registers until Kp is consumed
+  {
+    const float a = fl.use_gate ? __expf(A_log[h]) : 0.f;
+    const float au = a * KdaDecay<T>::kUnit, lbu = fl.lower_bound * KdaDecay<T>::kUnit;
+    auto gate_rows = [&](auto mode) {   // one copy of the loop per mode, as in the forward pass
+      constexpr int MODE = decltype(mode)::value;
+#pragma unroll
+      for (int it = 0; it < NIT; ++it) {
+        const int c = tid + it * kFinThreads, row = c / CPR, cc = c % CPR;
+#pragma unroll
+        for (int e4 = 0; e4 < VEC / 4; ++e4) {
+          f32x4 y;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int idx = 4 * e4 + e;
+            const float x = __uint_as_float(g32 ? gw[it][e4][e] : (gw[it][0][(idx >> 1) & 3] >> (16 * (idx & 1))) << 16);
+            y[e] = row < nvalid ? kda_gate<T, MODE>(x, bv[e4][e], a, au, lbu) : 0.f;
+          }
+          *reinterpret_cast<f32x4*>(Gs + row * LDG + cc * VEC + 4 * e4) = y;
+        }
+      }
+    };
+    if (!fl.use_gate) gate_rows(IntConst<0>());
+    else if (!fl.has_lower_bound) gate_rows(IntConst<1>());
+    else gate_rows(IntConst<2>());
+    GDN_LDS_BARRIER();
+  }
   // a2 and dAq arrive as tiles in fragment order: a tile wave takes its own (every tile wave loads, also the one of the
-  // upper tile, which nobody wrote: what it reads is dropped below).  Requested behind what the first barrier waits for.
+  // upper tile, which nobody wrote: what it reads is dropped below).  These requests and the two after them come behind
+  // the gate: none of them is needed before phase A1, and requested ahead of the gate their branches made every wave
+  // wait for all of its earlier requests first.
   if (tile_wave) {
     a2f.load(a2m + (2 * ti + tj) * 1024);
     daf.load(dAq + (2 * ti + tj) * 1024);
@@ -184,8 +249,27 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
   constexpr bool Q_BY_OTHERS = !FULL;
   const bool q_wave = Q_BY_OTHERS ? !tile_wave : tile_wave;
   if (q_wave) tile_qk_request<T, DK>(qt, q + tok0 * hk + h * DK, hk, nvalid, tid & (kThreads - 1));
+  // beta: requested by every wave alike, stored with the other row vectors below
+  const float bh = bhat[(tok0 + imin(lane, nvalid - 1)) * H + h];
+  {
+    constexpr int PARTS = kThreads / DK;   // the forward pass's split of the chunk, for the same rounding
+    float* tot = xgl;                      // [PARTS][DK]: free until phase B
+    static_assert(PARTS * DK <= 256, "the totals fit the vector they borrow");
+    if (tid < kThreads) kda_cumsum_part<DK, LDG, PARTS>(Gs, tot, tid);
+    GDN_LDS_BARRIER();
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int c = tid + it * kFinThreads, row = c / CPR, cc = c % CPR, part = row / (64 / PARTS);
+#pragma unroll
+      for (int e4 = 0; e4 < VEC / 4; ++e4) {
+        gk[it][e4] = *reinterpret_cast<const f32x4*>(Gs + row * LDG + cc * VEC + 4 * e4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) gk[it][e4][e] += kda_cumsum_before<DK, PARTS>(tot, part, cc * VEC + 4 * e4 + e);
+      }
+    }
+  }
   if (tid < 64) {
-    bs[tid] = tid < nvalid ? bhat[(tok0 + tid) * H + h] : 0.f;
+    bs[tid] = tid < nvalid ? bh : 0.f;
     rsq[tid] = 1.f;
     rsk[tid] = 1.f;
   }
@@ -200,7 +284,7 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     const int c = tid + it * kFinThreads;
     st16(TmT + (c / C64) * L64 + (c % C64) * VEC, tmv[it]);
   }
-  GDN_LDS_BARRIER();   // the row vectors are initialised before the norm below writes 1/|k| over its entries
+  GDN_LDS_BARRIER();   // the row vectors are initialised before the norm below writes 1/|k| over its entries; G is in registers
   tile_qk_finish<T, DK>(kt, Ks, LDK, nvalid, tid, fl.l2norm != 0, nullptr, 0, rsk, 1);
   GDN_LDS_BARRIER();
 #pragma unroll
@@ -598,7 +682,6 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
   float da_sum = 0.f;
   if (has_k) {
     // the raw gate input of this lane's rows, requested before the stores below
-    const bool g32 = sizeof(T) == 4 || fl.g_f32;
     // (as bits, widened after the loop: a conversion inside it would make every load wait for the one before)
     uint32_t raws[16];
     if (fl.use_gate) {
@@ -738,7 +821,6 @@ static int kda_bwd_launch(const ChunkDims& d, const KdaWorkspace& L, const void*
   const T* K2F = reinterpret_cast<const T*>(ws + L.K2F);
   const T* VF = reinterpret_cast<const T*>(ws + L.VF);
   const T* HF = reinterpret_cast<const T*>(ws + L.HF);
-  const float* GC = reinterpret_cast<const float*>(ws + L.GC);
   const T* TMR = reinterpret_cast<const T*>(ws + L.TMR);
   const T* QBT = reinterpret_cast<const T*>(ws + L.QBT);
   T* DVF = reinterpret_cast<T*>(ws + L.DVF);
@@ -775,7 +857,7 @@ static int kda_bwd_launch(const ChunkDims& d, const KdaWorkspace& L, const void*
     constexpr int smem = KdaBwdSmem<T, DK>::bytes;
     if (int e = set_lds_b(kern, smem)) return e;
     GDN_LAUNCH(kKernKdaBwdFinish, st, kern, dim3(nc, H), dim3(kFinThreads), smem, st, (const T*)q, (const T*)k, g, A_log, dt_bias,
-               bhat, GC, TMR, (const T*)DUMP, (const float*)DD, cu, chunk_offsets, (T*)dq, (T*)dk, dg, dbeta, PART, d.T, d.N, H, scale, fl);
+               bhat, TMR, (const T*)DUMP, (const float*)DD, cu, chunk_offsets, (T*)dq, (T*)dk, dg, dbeta, PART, d.T, d.N, H, scale, fl);
   }
   if (fl.use_gate && (dA_log != nullptr || ddt_bias != nullptr))
     GDN_LAUNCH(kKernKdaBwdReduce, st, kda_bwd_reduce_kernel, dim3(H, (d.K + 32) / 32), dim3(kThreads), 0, st, (const float*)PART, cu,

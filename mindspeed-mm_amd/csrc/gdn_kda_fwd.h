@@ -46,7 +46,7 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
     const T* __restrict__ q, const T* __restrict__ k, const void* __restrict__ g, const void* __restrict__ beta,
     const float* __restrict__ A_log, const float* __restrict__ dt_bias, const int64_t* __restrict__ cu,
     const int* __restrict__ chunk_offsets, float* __restrict__ bhat_out, float* __restrict__ dec_out,
-    float* __restrict__ G_out, T* __restrict__ Ai_out, T* __restrict__ Aq_out, T* __restrict__ K1_out,
+    T* __restrict__ Ai_out, T* __restrict__ Aq_out, T* __restrict__ K1_out,
     T* __restrict__ K2_out, T* __restrict__ QB_out, T* __restrict__ QBT_out, T* __restrict__ TMR_out,
     float* __restrict__ rstd_q_out, float* __restrict__ rstd_k_out,
     int T_len, int N, int H, float scale, KdaFlags fl) {
@@ -125,11 +125,8 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
         f32x4 y;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          float x = __uint_as_float(g32 ? gw[i][e] : (gw[i][e >> 1] >> (16 * (e & 1))) << 16);
-          if (MODE == 0) x *= KdaDecay<T>::kUnit;
-          if (MODE == 1) x = -au * kda_softplus(x + bv[i][e]);
-          if (MODE == 2) x = lbu * kda_sigmoid(a * (x + bv[i][e]));
-          y[e] = row < nvalid ? x : 0.f;
+          const float x = __uint_as_float(g32 ? gw[i][e] : (gw[i][e >> 1] >> (16 * (e & 1))) << 16);
+          y[e] = row < nvalid ? kda_gate<T, MODE>(x, bv[i][e], a, au, lbu) : 0.f;
         }
         *reinterpret_cast<f32x4*>(Gs + row * LDG + 4 * c4) = y;
       }
@@ -148,17 +145,9 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
   {
     constexpr int PARTS = kThreads / DK, RPP = 64 / PARTS;
     const int d = tid % DK, part = tid / DK;
-    float run = 0.f;
-#pragma unroll
-    for (int r = 0; r < RPP; ++r) {
-      run += Gs[(part * RPP + r) * LDG + d];
-      Gs[(part * RPP + r) * LDG + d] = run;
-    }
-    tot[part * DK + d] = run;
+    kda_cumsum_part<DK, LDG, PARTS>(Gs, tot, tid);
     GDN_LDS_BARRIER();
-    float off = 0.f;
-#pragma unroll
-    for (int p = 0; p < PARTS - 1; ++p) off += p < part ? tot[p * DK + d] : 0.f;
+    const float off = kda_cumsum_before<DK, PARTS>(tot, part, d);
     if (part > 0) {
 #pragma unroll
       for (int r = 0; r < RPP; ++r) Gs[(part * RPP + r) * LDG + d] += off;
@@ -360,14 +349,9 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
     GDN_LDS_BARRIER();
     store_k(K2_out);
   }
-  // the decay of the whole chunk per channel, the cumulative decay itself
+  // the decay of the whole chunk per channel (the cumulative decay itself is not kept: the backward pass rebuilds it
+  // from the gate input, which it reads anyway)
   if (tid < DK) dec_out[ch * DK + tid] = KdaDecay<T>::exp(Gs[63 * LDG + tid]);
-  if (G_out != nullptr) {
-    for (int c = tid; c < 64 * (DK / 4); c += kThreads) {
-      const int row = c / (DK / 4), c4 = c % (DK / 4);
-      *reinterpret_cast<f32x4*>(G_out + (ch * 64 + row) * DK + 4 * c4) = *reinterpret_cast<const f32x4*>(Gs + row * LDG + 4 * c4);
-    }
-  }
   GDN_LDS_BARRIER();   // k, the staging tile and G are dead
 
   // ---- phase 1d: L and Aq as 64x64 fp32 matrices ----
@@ -476,7 +460,6 @@ static int kda_fwd_launch(const ChunkDims& d, const KdaWorkspace& L, const void*
   T* QB = FUSE ? nullptr : reinterpret_cast<T*>(ws + L.QB);
   T* VF = reinterpret_cast<T*>(ws + L.VF);
   T* HF = reinterpret_cast<T*>(ws + L.HF);
-  float* GC = with_backward ? reinterpret_cast<float*>(ws + L.GC) : nullptr;
   T* QBT = (with_backward || FUSE) ? reinterpret_cast<T*>(ws + L.QBT) : nullptr;
   T* TMR = with_backward ? reinterpret_cast<T*>(ws + L.TMR) : nullptr;
   if (cu != nullptr) GDN_LAUNCH(kKernChunkTable, st, chunk_table_kernel, dim3(1), dim3(kThreads), 0, st, cu, chunk_offsets, d.N);
@@ -491,7 +474,7 @@ static int kda_fwd_launch(const ChunkDims& d, const KdaWorkspace& L, const void*
     if (int e = set_lds(kern, smem)) return e;
     const bool keep = with_backward && fl.l2norm;
     GDN_LAUNCH(kKernKdaPrep, st, kern, dim3(nc, H), dim3(kThreads), smem, st, (const T*)q, (const T*)k, g, beta, A_log,
-               dt_bias, cu, (const int*)chunk_offsets, bhat, dec, GC, Ai, AQ, K1F, K2F, QB, QBT, TMR, keep ? rstd : nullptr,
+               dt_bias, cu, (const int*)chunk_offsets, bhat, dec, Ai, AQ, K1F, K2F, QB, QBT, TMR, keep ? rstd : nullptr,
                keep ? rstd + (int64_t)nc * 64 * H : nullptr, d.T, d.N, H, scale, fl);
   }
   if constexpr (FUSE) {
