@@ -236,11 +236,11 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     else gate_rows(IntConst<2>());
     GDN_LDS_BARRIER();
   }
-  // a2 and dAq arrive as tiles in fragment order: a tile wave takes its own (every tile wave loads, also the one of the
-  // upper tile, which nobody wrote: what it reads is dropped below).  These requests and the two after them come behind
-  // the gate: none of them is needed before phase A1, and requested ahead of the gate their branches made every wave
-  // wait for all of its earlier requests first.
-  if (tile_wave) {
+  // a2 and dAq arrive as tiles in fragment order: a tile wave takes its own (nobody wrote the tile above the diagonal,
+  // and its wave asks for nothing).  These requests and the two after them come behind the gate: none of them is needed
+  // before phase A1, and requested ahead of the gate their branches made every wave wait for all of its earlier
+  // requests first.
+  if (lower) {
     a2f.load(a2m + (2 * ti + tj) * 1024);
     daf.load(dAq + (2 * ti + tj) * 1024);
   }
@@ -683,8 +683,10 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
   if (has_k) {
     // the raw gate input of this lane's rows, requested before the stores below
     // (as bits, widened after the loop: a conversion inside it would make every load wait for the one before)
+    // (The 16-bit kernels need none for the softplus gate: there the gate's value and slope follow from G itself, below.)
+    constexpr bool FROM_G = KdaDecay<T>::kBase2;
     uint32_t raws[16];
-    if (fl.use_gate) {
+    if (fl.use_gate && !(FROM_G && !fl.has_lower_bound)) {
       if (g32) {
 #pragma unroll
         for (int r = 0; r < 16; ++r)
@@ -716,6 +718,11 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     float dt_sum = 0.f;
     // MODE 0: g is the log decay itself; 1: -e^{A_log} softplus(g + bias); 2: lower_bound sigmoid(e^{A_log} (g + bias)).
     // One copy of the loop per mode: a test of the options per element would cost as much as the gate.
+    // MODE 1 in the 16-bit kernels: the token's own log decay is the difference of two rows of G (exact to half an ulp
+    // of G: G_i was formed as the rounded sum of G_{i-1} and it), -e^{A_log} log2(e) softplus(raw), and the slope of the
+    // softplus is 1 - e^{-softplus} = 1 - 2^{G_tok / e^{A_log}}: one exponential per element, and no second pass over
+    // the gate input.
+    const float inv_a = __builtin_amdgcn_rcpf(a);
     auto gate_back = [&](auto mode) {
       constexpr int MODE = decltype(mode)::value;
       f32x16 dgr;
@@ -723,12 +730,21 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
 #pragma unroll
       for (int qd = 3; qd >= 0; --qd) {
         float run = later + (first_half ? sx[qd] : 0.f);
+        float gprev = 0.f;   // G of the row before this group of four
+        if (MODE == 1 && FROM_G) {
+          const int i0 = 32 * ri + acc_row(4 * qd);
+          gprev = i0 > 0 ? Gs[(i0 - 1) * LDG + d] : 0.f;
+        }
 #pragma unroll
         for (int m = 3; m >= 0; --m) {
           const int r = 4 * qd + m, i = 32 * ri + acc_row(r);
           run += dGv[r];
           float x = i < nvalid ? run + dglast : 0.f;     // d(log decay of token i, channel d)
-          if (MODE != 0) {
+          if (MODE == 1 && FROM_G) {
+            const float gt = Gi[r] - (m > 0 ? Gi[r - 1] : gprev);
+            da_sum += x * gt * (1.f / KdaDecay<T>::kUnit);
+            x *= a * (__builtin_amdgcn_exp2f(gt * inv_a) - 1.f);
+          } else if (MODE != 0) {
             const float raw = __uint_as_float(raws[r] << raw_shift) + bias;
             if (MODE == 2) {
               const float sg = kda_sigmoid(a * raw), ds_ = fl.lower_bound * sg * (1.f - sg);

@@ -90,7 +90,8 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
     for (int i = 0; i < GP; ++i) {
       const int c = tid + i * kThreads, row = imin(c / (DK / 4), nvalid - 1), c4 = c % (DK / 4);
       const u32x2 x = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(g) + (tok0 + row) * hk + h * DK + 4 * c4);
-      gw[i][0] = x[0]; gw[i][1] = x[1]; gw[i][2] = 0; gw[i][3] = 0;
+      gw[i][0] = x[0]; gw[i][1] = x[1];   // the other two stay unset: unread on this path, and zeros here made the
+                                          // fp32 path wait at the join for its requests
     }
   }
   if (fl.use_gate && dt_bias != nullptr) {
@@ -102,15 +103,12 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
   }
   tile_qk_request<T, DK>(kt, k + tok0 * hk + h * DK, hk, nvalid, tid);
   tile_qk_request<T, DK>(qt, q + tok0 * hk + h * DK, hk, nvalid, tid);
-  if (wave == 0) {
-    const int64_t at = (tok0 + imin(lane, nvalid - 1)) * H + h;
-    float b;
-    if (sizeof(T) == 4 || fl.beta_f32) b = reinterpret_cast<const float*>(beta)[at];
-    else { T t; if constexpr (sizeof(T) == 2) t.bits = reinterpret_cast<const uint16_t*>(beta)[at]; b = Elem<T>::to_f(t); }
-    if (fl.beta_sigmoid) b = kda_sigmoid(b) * (fl.beta_x2 ? 2.f : 1.f);
-    bs[lane] = lane < nvalid ? b : 0.f;
-    if (lane < nvalid) bhat_out[at] = b;
-  }
+  // beta: requested by every wave alike (a branch around the request would make its wave wait at the join for all of
+  // the requests above), as bits; used behind the gate
+  const int64_t beta_at = (tok0 + imin(lane, nvalid - 1)) * H + h;
+  uint32_t beta_bits;
+  if (sizeof(T) == 4 || fl.beta_f32) beta_bits = reinterpret_cast<const uint32_t*>(beta)[beta_at];
+  else beta_bits = reinterpret_cast<const uint16_t*>(beta)[beta_at];
   // the gate: log decay of every token and channel, 0 on the rows past the end (they leave the cumulative sum alone)
   {
     const float a = fl.use_gate ? __expf(A_log[h]) : 0.f;
@@ -134,6 +132,15 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(2) void kda_prep_kerne
     if (!fl.use_gate) gate_rows(IntConst<0>());
     else if (!fl.has_lower_bound) gate_rows(IntConst<1>());
     else gate_rows(IntConst<2>());
+  }
+  if (wave == 0) {
+    float b = __uint_as_float(beta_bits);
+    if constexpr (sizeof(T) == 2) {
+      if (!fl.beta_f32) { T t; t.bits = (uint16_t)beta_bits; b = Elem<T>::to_f(t); }
+    }
+    if (fl.beta_sigmoid) b = kda_sigmoid(b) * (fl.beta_x2 ? 2.f : 1.f);
+    bs[lane] = lane < nvalid ? b : 0.f;
+    if (lane < nvalid) bhat_out[beta_at] = b;
   }
   {
     const int64_t roff = ch * 64;
