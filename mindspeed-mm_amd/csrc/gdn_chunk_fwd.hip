@@ -197,14 +197,20 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
   const int64_t tok0 = s.bos + (int64_t)s.chunk * kChunk;
 
   // ---- phase 0: K and Q tiles of the q/k group; cumulative decay (one lane per token) and beta of each of its value
-  //      heads, a wave per head.  All requests first. ----
+  //      heads, a wave per head.  All requests first: the gate values of the wave's first head (every wave and lane
+  //      asks alike, for a place that exists; inside the loop over heads the request would come behind a wait for the
+  //      tiles), then the tiles. ----
+  const int64_t tokl = tok0 + imin(lane, nvalid - 1);
+  const int64_t at0 = tokl * Hv + hq * grp + imin(wave, grp - 1);
+  const float g_first = g[at0];
+  const uint32_t b_first = gate_raw<T>(beta, beta_same, at0);
   TileQK<T, DK> kt, qt;
   tile_qk_request<T, DK>(kt, k + tok0 * ts.k + hq * DK, ts.k, nvalid, tid);
   tile_qk_request<T, DK>(qt, q + tok0 * ts.q + hq * DK, ts.q, nvalid, tid);
-  for (int hh = wave; hh < grp; hh += 4) {
+  auto head_gates = [&](int hh, float graw, uint32_t braw) {
     const int h = hq * grp + hh;
-    float x = lane < nvalid ? g[(tok0 + lane) * Hv + h] : 0.f;
-    const float b = lane < nvalid ? gate_val<T>(gate_raw<T>(beta, beta_same, (tok0 + lane) * Hv + h), beta_same) : 0.f;
+    float x = lane < nvalid ? graw : 0.f;
+    const float b = lane < nvalid ? gate_val<T>(braw, beta_same) : 0.f;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
       const float t = __shfl_up(x, d);
@@ -213,6 +219,12 @@ __global__ __launch_bounds__(kThreads) GDN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3
     Gs[hh * 128 + lane] = x;
     Gs[hh * 128 + 64 + lane] = b;
     G_out[((int64_t)blockIdx.x * Hv + h) * 64 + lane] = x;   // 64 contiguous values per chunk and head
+  };
+  if (wave < grp) head_gates(wave, g_first, b_first);
+  for (int hh = wave + 4; hh < grp; hh += 4) {
+    const int64_t at = tokl * Hv + hq * grp + hh;
+    const float graw = g[at];
+    head_gates(hh, graw, gate_raw<T>(beta, beta_same, at));
   }
   {
     // q and k arrive raw; with the in-kernel l2 norm they are normalised on the way into LDS, and 1/|q|, 1/|k| are left

@@ -698,6 +698,9 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
       }
     }
     const int raw_shift = g32 ? 0 : 16;
+    // ... and so are the two per-channel values of the gate's backward
+    const float dDd = dD[d];
+    const float bias = (fl.use_gate && dt_bias != nullptr) ? dt_bias[h * DK + d] : 0.f;
     if (fl.l2norm) {
       const f32x16 dotq = rows_ld4(rq, 32 * ri), dotk = rows_ld4(rk, 32 * ri);
       const f32x16 sq = rows_ld(rsq, 32 * ri), sk = rows_ld(rsk, 32 * ri);
@@ -711,10 +714,9 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     acc_store_rows<T, false>(dqh, id, patch, dq + at, hk, nvalid - 32 * ri);
     acc_store_rows<T, false>(dkh, id, patch, dk + at, hk, nvalid - 32 * ri);
     // dG_last: column sum over all rows of this channel, plus the decay of the state
-    const float dglast = xgl[2 * cj * 32 + l32] + xgl[(2 * cj + 1) * 32 + l32] + dD[d] * KdaDecay<T>::exp(Gs[63 * LDG + d]);
+    const float dglast = xgl[2 * cj * 32 + l32] + xgl[(2 * cj + 1) * 32 + l32] + dDd * KdaDecay<T>::exp(Gs[63 * LDG + d]);
     const bool first_half = lane < 32;
     const float a = fl.use_gate ? __expf(A_log[h]) : 0.f;
-    const float bias = (fl.use_gate && dt_bias != nullptr) ? dt_bias[h * DK + d] : 0.f;
     float dt_sum = 0.f;
     // MODE 0: g is the log decay itself; 1: -e^{A_log} softplus(g + bias); 2: lower_bound sigmoid(e^{A_log} (g + bias)).
     // One copy of the loop per mode: a test of the options per element would cost as much as the gate.
