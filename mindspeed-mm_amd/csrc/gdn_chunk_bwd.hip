@@ -774,17 +774,12 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   const bool frag_sums = V >= 128 && grp > 1, last_head = hh == grp - 1;
   T* sums_out = const_cast<T*>(dhf_in) + ch * (int64_t)(V / 32) * NKT * 1024;
   const T* sums_in = sums_out - (int64_t)(V / 32) * NKT * 1024;   // the head before this one
-  RowPieces<T> held[2];
-  AccB<T> heldf[2];
+  RowPieces<T> held[2];   // rows, or a tile in fragment order: one set of requests either way (rows_or_tile_request)
   if (has_k && hh != 0) {
-    if (frag_sums) {
 #pragma unroll
-      for (int ri = 0; ri < 2; ++ri) heldf[ri].load(sums_in + (ri * NKT + cj) * 1024);
-    } else {
-#pragma unroll
-      for (int ri = 0; ri < 2; ++ri)
-        rows_request<T>(held[ri], dq + (tok0 + 32 * ri) * ts.dq + hq * DK + 32 * cj, ts.dq, nvalid - 32 * ri);
-    }
+    for (int ri = 0; ri < 2; ++ri)
+      rows_or_tile_request<T>(held[ri], frag_sums, sums_in + (ri * NKT + cj) * 1024,
+                              dq + (tok0 + 32 * ri) * ts.dq + hq * DK + 32 * cj, ts.dq, nvalid - 32 * ri);
   }
   if (lower) {  // <R_t, v_t> = sum_i Tm[i][t] (dV' V^T)[i][t]: column sums of Tm . a2, no second pass over V needed
     const f32x16 tmv = tm_t(tj, ti).unpack();   // Tm tile (ti, tj) with lane <-> column, registers <-> row
@@ -831,7 +826,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       T* dst = dq + (tok0 + 32 * ri) * ts.dq + hq * DK + 32 * cj;
       if (frag_sums) {
         if (hh != 0) {
-          const f32x16 prev = heldf[ri].unpack();
+          const f32x16 prev = as_frag<T>(held[ri]).unpack();
 #pragma unroll
           for (int r = 0; r < 16; ++r) dQi[ri][r] += prev[r];
         }
@@ -888,14 +883,10 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
   }
   GDN_LDS_BARRIER();
   if (has_k && hh != 0) {   // the dk sums of the earlier heads, two phases before they are added to
-    if (frag_sums) {
 #pragma unroll
-      for (int ri = 0; ri < 2; ++ri) heldf[ri].load(sums_in + ((2 + ri) * NKT + cj) * 1024);
-    } else {
-#pragma unroll
-      for (int ri = 0; ri < 2; ++ri)
-        rows_request<T>(held[ri], dk + (tok0 + 32 * ri) * ts.dk + hq * DK + 32 * cj, ts.dk, nvalid - 32 * ri);
-    }
+    for (int ri = 0; ri < 2; ++ri)
+      rows_or_tile_request<T>(held[ri], frag_sums, sums_in + ((2 + ri) * NKT + cj) * 1024,
+                              dk + (tok0 + 32 * ri) * ts.dk + hq * DK + 32 * cj, ts.dk, nvalid - 32 * ri);
   }
   if (has_k) {       // E = dM K, F = dM^T (beta K): dK += beta E + F; <E,k> and <F,k> complete the row sums
 #pragma unroll
@@ -936,7 +927,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void chunk_bwd_lo
       T* dst = dk + (tok0 + 32 * ri) * ts.dk + hq * DK + 32 * cj;
       if (frag_sums) {
         if (hh != 0) {
-          const f32x16 prev = heldf[ri].unpack();
+          const f32x16 prev = as_frag<T>(held[ri]).unpack();
 #pragma unroll
           for (int r = 0; r < 16; ++r) dKi[ri][r] += prev[r];
         }

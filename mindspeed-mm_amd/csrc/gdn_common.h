@@ -752,6 +752,33 @@ __device__ __forceinline__ void rows_request(RowPieces<T>& r, const T* g, int64_
     r.y[i] = ld16(g + (int64_t)row * row_stride + cc * V);
   }
 }
+// The same requests for either of two sources, chosen by the wave-uniform `frag` on the addresses: the rows of
+// rows_request, or a 32x32 tile in fragment order (what AccB::load reads; as_frag() gives it that type).  A branch
+// between the two kinds of request would join with loaded registers, and the compiler waits for them there.  Unlike
+// rows_request this asks also when the tile has no valid row: `g` must then point 32 rows past a block whose rows
+// exist (rows_valid >= -31: the row index goes back into that block).
+template <typename T>
+__device__ __forceinline__ void rows_or_tile_request(RowPieces<T>& r, bool frag, const T* tile, const T* g,
+                                                     int64_t row_stride, int rows_valid) {
+  constexpr int V = Elem<T>::kVec, PPR = 32 / V;
+  static_assert(RowPieces<T>::kN == AccB<T>::kG, "a lane holds as many 16-byte pieces of a tile either way");
+  const int lane = threadIdx.x & 63;
+  // a uniform base and one 32-bit offset per piece (never negative: the rows are counted from 32 rows before g)
+  const T* base = frag ? tile : g - 32 * row_stride;
+#pragma unroll
+  for (int i = 0; i < RowPieces<T>::kN; ++i) {
+    const int p = lane + 64 * i, row = imin(p / PPR, rows_valid - 1), cc = p % PPR;
+    const uint32_t off = frag ? (uint32_t)(frag_slot<T>(i, lane) * AccB<T>::kVecElems)
+                              : (uint32_t)((row + 32) * (int)row_stride + cc * V);
+    r.y[i] = ld16(base + off);
+  }
+}
+template <typename T> __device__ __forceinline__ AccB<T> as_frag(const RowPieces<T>& r) {
+  AccB<T> f;
+#pragma unroll
+  for (int i = 0; i < AccB<T>::kG; ++i) f.f[i] = r.y[i].raw;
+  return f;
+}
 // ADD: the rows are added to `held` (what memory held, see rows_request) before they are written.
 template <typename T, bool ADD>
 __device__ __forceinline__ void acc_store_rows(const f32x16& acc, const IdentityFrag<T>& id, T* patch, T* g,
