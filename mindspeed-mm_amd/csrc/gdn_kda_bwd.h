@@ -208,6 +208,9 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     const int c = tid + it * kFinThreads;
     tmv[it] = ld16(TMR + ch * 4096 + (c / C64) * 64 + (c % C64) * VEC);
   }
+  // beta: requested by every wave alike and with the early group (loads arrive in the order of their requests: the
+  // store of the row vectors below then waits for P and Tm, not for the requests made behind the gate)
+  const float bh = bhat[(tok0 + imin(lane, nvalid - 1)) * H + h];
   // G: the gate's log decay of every token and channel (0 on the rows past the end) into the place Kp will take,
   // summed down the tokens there, and back into this thread's registers until Kp is consumed
   {
@@ -236,21 +239,45 @@ __global__ __launch_bounds__(kFinThreads) void kda_bwd_finish_kernel(
     else gate_rows(IntConst<2>());
     GDN_LDS_BARRIER();
   }
-  // a2 and dAq arrive as tiles in fragment order: a tile wave takes its own (nobody wrote the tile above the diagonal,
-  // and its wave asks for nothing).  These requests and the two after them come behind the gate: none of them is needed
-  // before phase A1, and requested ahead of the gate their branches made every wave wait for all of its earlier
-  // requests first.
-  if (lower) {
-    a2f.load(a2m + (2 * ti + tj) * 1024);
-    daf.load(dAq + (2 * ti + tj) * 1024);
-  }
+  // a2 and dAq arrive as tiles in fragment order: a tile wave takes its own.  These requests come behind the gate: none
+  // of them is needed before phase A1, and requested ahead of the gate their branches made every wave wait for all of
+  // its earlier requests first.
   // q^ rows: in the 16-bit kernel they have a place of their own, and the waves that own no tile of the 64x64 phases
-  // normalise them during those phases
+  // normalise them during those phases.
+  // Every wave makes the same number of requests here (K = 128: four): the waits further down can then leave exactly
+  // these in flight.  The wave of the tile above the diagonal, which nobody wrote, asks for tile (0,0) again (cached)
+  // and drops it.
   constexpr bool Q_BY_OTHERS = !FULL;
   const bool q_wave = Q_BY_OTHERS ? !tile_wave : tile_wave;
-  if (q_wave) tile_qk_request<T, DK>(qt, q + tok0 * hk + h * DK, hk, nvalid, tid & (kThreads - 1));
-  // beta: requested by every wave alike, stored with the other row vectors below
-  const float bh = bhat[(tok0 + imin(lane, nvalid - 1)) * H + h];
+  const int tile_at = lower ? (2 * ti + tj) * 1024 : 0;
+  constexpr bool SAME_REQUESTS = Q_BY_OTHERS && TileQK<T, DK>::PT == 2 * AccB<T>::kG;
+  if constexpr (SAME_REQUESTS) {
+    // one set of requests, the choice made on the addresses (a branch with two arms does not survive the compiler as
+    // such, and behind two separate branches it assumes the fewest requests in flight)
+    const int t = tid & (kThreads - 1);
+#pragma unroll
+    for (int i = 0; i < TileQK<T, DK>::PT; ++i) {
+      const int c = t + i * kThreads, row = imin(c / CPR, nvalid - 1), cc = c % CPR;
+      const T* qa = q + (tok0 + row) * hk + h * DK + cc * VEC;
+      const T* ta = (i < AccB<T>::kG ? a2m : dAq) + tile_at + frag_slot<T>(i % AccB<T>::kG, lane) * AccB<T>::kVecElems;
+      qt.x[i] = ld16(tile_wave ? ta : qa);
+    }
+#pragma unroll
+    for (int g = 0; g < AccB<T>::kG; ++g) { a2f.f[g] = qt.x[g].raw; daf.f[g] = qt.x[AccB<T>::kG + g].raw; }
+  } else if constexpr (Q_BY_OTHERS) {
+    if (tile_wave) {
+      a2f.load(a2m + tile_at);
+      daf.load(dAq + tile_at);
+    } else {
+      tile_qk_request<T, DK>(qt, q + tok0 * hk + h * DK, hk, nvalid, tid & (kThreads - 1));
+    }
+  } else {
+    if (tile_wave) {
+      a2f.load(a2m + tile_at);
+      daf.load(dAq + tile_at);
+      tile_qk_request<T, DK>(qt, q + tok0 * hk + h * DK, hk, nvalid, tid & (kThreads - 1));
+    }
+  }
   {
     constexpr int PARTS = kThreads / DK;   // the forward pass's split of the chunk, for the same rounding
     float* tot = xgl;                      // [PARTS][DK]: free until phase B
