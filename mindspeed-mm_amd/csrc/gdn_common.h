@@ -863,7 +863,7 @@ __device__ __forceinline__ void tile_qk_finish(TileQK<T, DK, NT>& t, T* lds, int
 #pragma unroll
       for (int e = 0; e < V; ++e) ss += f[e] * f[e];
       ss = lane_group_sum<CPR>(ss);
-      const float r = rsqrtf(ss + 1e-6f);
+      const float r = __builtin_amdgcn_rsqf(ss + 1e-6f);   // the instruction alone: its argument is never subnormal
 #pragma unroll
       for (int e = 0; e < V; ++e) f[e] *= r;
       x = pack16<T>(f);

@@ -266,6 +266,7 @@ static emu::GdimProxy gridDim;
 #define __builtin_amdgcn_fence(...) ((void)0)
 #define __builtin_amdgcn_sched_barrier(x) ((void)0)
 #define __builtin_amdgcn_rcpf(x) (1.0f / (x))
+#define __builtin_amdgcn_rsqf(x) (1.0f / sqrtf(x))
 #define __builtin_amdgcn_logf(x) log2f(x)
 #define GDN_WAVES_PER_SIMD(n)
 #define GDN_KEEP_HERE(x) ((void)0)
