@@ -762,7 +762,9 @@ __device__ __forceinline__ void rows_or_tile_request(RowPieces<T>& r, bool frag,
                                                      int64_t row_stride, int rows_valid) {
   constexpr int V = Elem<T>::kVec, PPR = 32 / V;
   static_assert(RowPieces<T>::kN == AccB<T>::kG, "a lane holds as many 16-byte pieces of a tile either way");
-  const int lane = threadIdx.x & 63;
+  int lane = threadIdx.x & 63;
+  GDN_KEEP_HERE(lane);   // the offsets are formed here: shared with an equal expression far above they would sit in a
+                         // register (or in scratch memory) through the phases between
   // a uniform base and one 32-bit offset per piece (never negative: the rows are counted from 32 rows before g)
   const T* base = frag ? tile : g - 32 * row_stride;
 #pragma unroll
