@@ -517,7 +517,7 @@ def main():
         x4 = gdn_inputs(1, T4, c["Hqk"], Hv4, c["K"], V4, torch.bfloat16, seed=4, a_log=(0.5, 2.0), dt_bias=(-6.0, -4.0))
         d4 = {n: t.to(dev) for n, t in x4.items()}
         del x4
-        ms4 = fwd_bwd_ms(d4, n=3, warm=1)
+        ms4 = fwd_bwd_ms(d4)
         fl4 = 3 * 2 * T4 * Hv4 * (3 * V4 * 64 + 2 * c["K"] * 64 + 3 * c["K"] * V4)
         aux["config4_T65536_Hv64_dv256"] = {
             "ms_per_step": round(ms4, 3), "tokens_per_s": round(T4 / (ms4 * 1e-3), 1),
